@@ -1,0 +1,174 @@
+/*
+ * jetfire_amd.h — C ABI of the MI355X (gfx950) implementation of JetFire's GPU
+ * approximate-attention decode path.
+ *
+ * Every entry point takes plain device/host pointers, sizes and a HIP stream
+ * (passed as void*; NULL = the default stream).  Kernels are enqueued
+ * asynchronously on that stream.  Return value: 0 on success, a negative
+ * JF_ERR_* code otherwise; jf_last_error() returns the message for the calling
+ * thread (the reference raises RuntimeError through TORCH_CHECK at the same
+ * places).
+ *
+ * Layouts are the reference's (jetfire_vllm/adapter/cache_store.py:240-284):
+ *   K/V data   (H_kv, num_slots, P)  uint8, P = 32 (INT2) / 48 (INT3 planar) / 64 (INT4)
+ *   K/V scales (H_kv, num_slots, NG) bf16,  NG = 128 / group_size
+ *   block_table (B, max_blocks) int64, seq_lens (B,) int32, block size 16
+ *   slot = block_table[b, pos / 16] * 16 + pos % 16
+ * bf16 values are passed as uint16_t bit patterns.  head_dim is 128 throughout.
+ */
+#ifndef JETFIRE_AMD_H
+#define JETFIRE_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define JF_OK 0
+#define JF_ERR_ARG (-1)      /* unsupported shape / argument (reference: TORCH_CHECK) */
+#define JF_ERR_HIP (-2)      /* HIP runtime error */
+#define JF_ERR_STATE (-3)    /* bad handle / wrong call order */
+#define JF_ERR_TIMEOUT (-4)  /* CPU correction did not finish in time */
+
+#define JF_SCHEME_K3V2 32    /* INT3 keys, INT2 values  (SymInt3K_SymInt2V) */
+#define JF_SCHEME_K4V4 44    /* INT4 keys, INT4 values  (SymInt4K_SymInt4V) */
+
+const char* jf_last_error(void);
+const char* jf_version(void);
+
+/* ------------------------------------------------------------------ piece 1: quantise-on-append
+ * Replaces fused_quant_write_int{2,3,4}_sym (jetfire_vllm/kernels/fused_quant_write.py:242-270,
+ * 337-369, 746-781): per (token, kv-head) and per group: scale = bf16(max(amax/qmax, 1e-8)),
+ * code = clamp(rint(x / f32(scale)), +-qmax) + 2^(nbits-1), packed in the reference wire format and
+ * scattered to out_data[h, slots[t], :], out_scale[h, slots[t], g].  slots[t] < 0 skips the token.
+ * x is (T, H_kv, 128) bf16 with element strides x_stride_t / x_stride_h (last dim contiguous).
+ * Data strides are in bytes, scale strides in bf16 elements.  nbits in {2,3,4};
+ * group_size in {32, 64, 128}. */
+int jf_quant_write_sym(const uint16_t* x, int64_t x_stride_t, int64_t x_stride_h,
+                       const int64_t* slots, int64_t T, int H_kv,
+                       uint8_t* out_data, int64_t data_stride_h, int64_t data_stride_slot,
+                       uint16_t* out_scale, int64_t scale_stride_h, int64_t scale_stride_slot,
+                       int64_t num_slots, int group_size, int nbits, void* stream);
+
+/* K and V of an INT4/INT4 cache in one launch.  Replaces fused_quant_write_int4_sym_kv
+ * (jetfire_vllm/kernels/fused_quant_write.py:552-617). */
+int jf_quant_write_int4_sym_kv(const uint16_t* key, int64_t k_stride_t, int64_t k_stride_h,
+                               const uint16_t* value, int64_t v_stride_t, int64_t v_stride_h,
+                               const int64_t* slots, int64_t T, int H_kv,
+                               uint8_t* k_data, int64_t k_data_stride_h, int64_t k_data_stride_slot,
+                               uint16_t* k_scale, int64_t k_scale_stride_h, int64_t k_scale_stride_slot,
+                               uint8_t* v_data, int64_t v_data_stride_h, int64_t v_data_stride_slot,
+                               uint16_t* v_scale, int64_t v_scale_stride_h, int64_t v_scale_stride_slot,
+                               int64_t num_slots, int group_size, void* stream);
+
+/* ------------------------------------------------------------------ Stage A (split form)
+ * scores[b, hq, s] for s < seq_len, -inf for seq_len <= s < max_S.
+ * jf_int3_qk_scores replaces int3_qk_scores (jetfire_vllm/csrc/int3_qk_scores.cu:318-390):
+ *   bf16 q times bf16-rounded dequantised INT3 keys, fp32 accumulate, times attn_scale.
+ *   n_scale_groups in {1, 2}.
+ * jf_int8tc_qk_scores replaces int8tc_qk_scores (jetfire_vllm/csrc/int8tc_qk_scores.cu:1263-1331):
+ *   q quantised to int8 per (row, 32 channels), exact INT4 key codes, int32 accumulate,
+ *   fp32 rescale  s = fma(a3,qs3, fma(a2,qs2, fma(a1,qs1, a0*qs0))); score = (s*ks)*attn_scale. */
+int jf_int3_qk_scores(const uint16_t* q, const uint8_t* k_data, const uint16_t* k_scales,
+                      const int64_t* block_table, const int32_t* seq_lens,
+                      int B, int H_q, int H_kv, int max_S, int max_blocks, int64_t num_slots,
+                      int n_scale_groups, int block_size, float attn_scale,
+                      float* scores, void* stream);
+int jf_int8tc_qk_scores(const uint16_t* q, const uint8_t* k_data, const uint16_t* k_scales,
+                        const int64_t* block_table, const int32_t* seq_lens,
+                        int B, int H_q, int H_kv, int max_S, int max_blocks, int64_t num_slots,
+                        int block_size, float attn_scale,
+                        float* scores, void* stream);
+
+/* Exact top-k per (b, query head) over scores[b, hq, :min(max_S, seq_len)] by radix select on the
+ * order-preserving key of the fp32 score; ties at the threshold go to the lower position; winners
+ * are written in ascending position, the rest of the K lanes are -1; topk_slots is the paged slot of
+ * each winner.  Replaces topk_slots_kernel_v5 (jetfire_vllm/csrc/int3_qk_scores.cu:426-554), whose
+ * emission order and tie choice are arbitrary.  If softmax_m / softmax_inv_z are non-NULL they
+ * receive the row max (0 if not finite) and 1/sum(exp(s-m)) (0 if the sum is not positive), as
+ * topk_slots_stats_kernel_v5 does (jetfire_vllm/csrc/int8tc_qk_scores.cu:1678-1823).
+ * top_k must be a power of two in [32, 8192]; max_S <= 262144. */
+int jf_topk_slots(const float* scores, const int32_t* seq_lens, const int64_t* block_table,
+                  int B, int H_q, int max_S, int max_blocks, int block_size, int top_k,
+                  int64_t* topk_idx, int64_t* topk_slots,
+                  float* softmax_m, float* softmax_inv_z, void* stream);
+
+/* ------------------------------------------------------------------ Stage B (split form)
+ * o_hat = sum_s p_s Vhat_s, o_old_unnorm = sum_{s in topk} p_s Vhat_s, W = sum_{s in topk} p_s with
+ * p = exp(score - m) * inv_z and Vhat = (code - offset) * f32(scale) (no bf16 rounding).
+ * Replaces int2_softmax_v_with_pre_corr_wvs2 (jetfire_vllm/csrc/int2_softmax_v.cu:792-901) for
+ * v_nbits == 2 and int4_softmax_v_with_pre_corr_wvs2_scores (jetfire_vllm/csrc/int4_softmax_v.cu:
+ * 2203-2235) for v_nbits == 4.  softmax_m / softmax_inv_z may be NULL (computed internally), or the
+ * Stage-A statistics (then this is int8tc_softmax_v_with_pre_corr_reg_stats' contract with exact fp32
+ * weights, jetfire_vllm/csrc/int8tc_softmax_v_fused.cu:1591-1734).  topk_idx may be NULL (o_hat only).
+ * Split partials are reduced in a fixed order, so the result is run-to-run deterministic.
+ * workspace: jf_softmax_v_workspace_bytes() bytes of device memory. */
+size_t jf_softmax_v_workspace_bytes(int B, int H_q, int max_S);
+int jf_softmax_v_pre_corr(const float* scores, const float* softmax_m, const float* softmax_inv_z,
+                          const uint8_t* v_data, const uint16_t* v_scales,
+                          const int64_t* block_table, const int32_t* seq_lens, const int64_t* topk_idx,
+                          int B, int H_q, int H_kv, int max_S, int max_blocks, int64_t num_slots,
+                          int block_size, int top_k, int v_nbits, int n_scale_groups,
+                          float* o_hat, float* o_old_unnorm, float* W,
+                          void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------ pieces 2+3: fused decode scan + top-k
+ * One pass over the packed K and V of every (sequence, kv-head): Q.K^T for the GQA group, softmax
+ * statistics, P.V, and exact top-k, without a (B, H_q, max_S) score tensor in HBM.  Produces what the
+ * reference's Stage A + Stage B pair produces (jetfire_vllm/adapter/decode_path.py:2081-2131,
+ * 2785-2935): topk_idx, topk_slots, o_hat, o_old_unnorm, W, and optionally softmax_m / softmax_inv_z.
+ * The reference's own single-call form of this contract is int2_fused_attn_topk
+ * (jetfire_vllm/kernels/int2_fused_attn_topk.py:5-10).  scheme: JF_SCHEME_K3V2 (group 64 or 128) or
+ * JF_SCHEME_K4V4 (group 128).  If scores is non-NULL the fp32 scores are also written (validation).
+ * workspace: jf_fused_workspace_bytes() bytes of device memory. */
+size_t jf_fused_workspace_bytes(int scheme, int B, int H_q, int H_kv, int max_S, int top_k);
+int jf_fused_scan_topk(int scheme, int group_size,
+                       const uint16_t* q, const uint8_t* k_data, const uint16_t* k_scales,
+                       const uint8_t* v_data, const uint16_t* v_scales,
+                       const int64_t* block_table, const int32_t* seq_lens,
+                       int B, int H_q, int H_kv, int max_S, int max_blocks, int64_t num_slots,
+                       int block_size, float attn_scale, int top_k,
+                       int64_t* topk_idx, int64_t* topk_slots,
+                       float* o_hat, float* o_old_unnorm, float* W,
+                       float* softmax_m, float* softmax_inv_z, float* scores,
+                       void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------ piece 4: merge
+ * out = bf16_rne(fma(W, f32(o_new), o_hat) - o_old_unnorm).  Replaces blend_unnorm_into
+ * (jetfire_vllm/csrc/blend.cu:202-290).  o_new / out are (B, H_q, D) bf16. */
+int jf_blend_unnorm(const float* o_hat, const float* o_old_unnorm, const float* W,
+                    const uint16_t* o_new, uint16_t* out, int B, int H_q, int D, void* stream);
+
+/* ------------------------------------------------------------------ piece 4: CPU correction + hand-off
+ * Exact softmax attention over the top-k slots from the host bf16 shadow.  Replaces cpu_topk_attn
+ * (jetfire_vllm/csrc/cpu_topk_attn.cpp:854-956; row kernel :602-690): invalid slots (<0 or
+ * >= num_slots) score -inf, a row without a valid slot gives zeros, output rounded to bf16.
+ * All pointers are host memory.  done_flag (nullable) is set to 1 after the outputs are visible. */
+int jf_cpu_topk_attn(const uint16_t* q, const uint16_t* k_shadow, const uint16_t* v_shadow,
+                     const int64_t* head_map, const int64_t* ts_buf, uint16_t* o_new,
+                     int B, int H_q, int K, int H_kv, int64_t num_slots, float scale,
+                     int64_t* done_flag);
+int jf_set_cpu_attn_threads(int n);   /* set_cpu_attn_threads (cpu_topk_attn.cpp:2509-2530) */
+int jf_get_cpu_attn_threads(void);
+
+/* Pinned hand-off context: replaces create_cpu_topk_submit_ctx / stream_submit_cpu_topk_attn /
+ * stream_wait_cpu_topk_attn (jetfire_vllm/csrc/cpu_topk_attn.cpp:2054-2163, 2239, 2302) and the
+ * pinned copies around them (jetfire_vllm/adapter/decode_path.py:2243-2267, 3107-3114).
+ * submit: async D2H of q and topk_slots into pinned buffers, then a stream-ordered host function that
+ *         starts the CPU correction on the worker pool and returns.
+ * wait:   a stream-ordered host function that joins the CPU job, then async H2D of o_new into
+ *         o_new_dev.  Only one job per context may be in flight. */
+typedef struct jf_handoff jf_handoff;
+jf_handoff* jf_handoff_create(int B, int H_q, int H_kv, int K, int64_t num_slots,
+                              const uint16_t* k_shadow_host, const uint16_t* v_shadow_host, float scale);
+int jf_handoff_submit(jf_handoff* h, const uint16_t* q_dev, const int64_t* topk_slots_dev, void* stream);
+int jf_handoff_wait(jf_handoff* h, uint16_t* o_new_dev, void* stream);
+int64_t jf_handoff_submit_count(const jf_handoff* h);
+void jf_handoff_destroy(jf_handoff* h);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* JETFIRE_AMD_H */

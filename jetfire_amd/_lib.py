@@ -1,0 +1,68 @@
+"""ctypes binding of libjetfire_amd.so (the C ABI declared in include/jetfire_amd.h).
+
+The library is loaded from the package directory; if it is missing this module raises — there is
+no CPU fallback for any operator.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, "libjetfire_amd.so")
+
+P = C.c_void_p
+I = C.c_int
+L = C.c_int64
+F = C.c_float
+Z = C.c_size_t
+
+# name -> (restype, argtypes); must list every symbol of include/jetfire_amd.h
+SIGNATURES = {
+    "jf_last_error": (C.c_char_p, []),
+    "jf_version": (C.c_char_p, []),
+    "jf_quant_write_sym": (I, [P, L, L, P, L, I, P, L, L, P, L, L, L, I, I, P]),
+    "jf_quant_write_int4_sym_kv": (I, [P, L, L, P, L, L, P, L, I, P, L, L, P, L, L, P, L, L, P, L, L, L, I, P]),
+    "jf_int3_qk_scores": (I, [P, P, P, P, P, I, I, I, I, I, L, I, I, F, P, P]),
+    "jf_int8tc_qk_scores": (I, [P, P, P, P, P, I, I, I, I, I, L, I, F, P, P]),
+    "jf_topk_slots": (I, [P, P, P, I, I, I, I, I, I, P, P, P, P, P]),
+    "jf_softmax_v_workspace_bytes": (Z, [I, I, I]),
+    "jf_softmax_v_pre_corr": (I, [P, P, P, P, P, P, P, P, I, I, I, I, I, L, I, I, I, I, P, P, P, P, Z, P]),
+    "jf_fused_workspace_bytes": (Z, [I, I, I, I, I, I]),
+    "jf_fused_scan_topk": (I, [I, I, P, P, P, P, P, P, P, I, I, I, I, I, L, I, F, I, P, P, P, P, P, P, P, P, P, Z, P]),
+    "jf_blend_unnorm": (I, [P, P, P, P, P, I, I, I, P]),
+    "jf_cpu_topk_attn": (I, [P, P, P, P, P, P, I, I, I, I, L, F, P]),
+    "jf_set_cpu_attn_threads": (I, [I]),
+    "jf_get_cpu_attn_threads": (I, []),
+    "jf_handoff_create": (P, [I, I, I, I, L, P, P, F]),
+    "jf_handoff_submit": (I, [P, P, P, P]),
+    "jf_handoff_wait": (I, [P, P, P]),
+    "jf_handoff_submit_count": (L, [P]),
+    "jf_handoff_destroy": (None, [P]),
+}
+
+_lib = None
+
+
+def load() -> C.CDLL:
+    """Load the shared library (once) and attach the signatures."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `python -m jetfire_amd.build` "
+            "(the HIP library is the only implementation; there is no fallback)")
+    lib = C.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(rc: int) -> None:
+    if rc != 0:
+        msg = load().jf_last_error().decode("utf-8", "replace")
+        raise RuntimeError(msg or f"jetfire_amd call failed with status {rc}")

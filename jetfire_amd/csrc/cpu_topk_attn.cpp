@@ -1,0 +1,379 @@
+// Host side of the hand-off: exact softmax attention over the top-k slots from the bf16 shadow
+// (restates the contract of jetfire_vllm/csrc/cpu_topk_attn.cpp:602-690,854-956), a persistent
+// worker pool (spin, then sleep on a condition variable), and the stream-ordered pinned hand-off
+// (submit: D2H q + slots -> host function starts the CPU job; wait: host function joins -> H2D o_new).
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <chrono>
+#include <cmath>
+#include <condition_variable>
+#include <cstdlib>
+#include <cstring>
+#include <functional>
+#include <mutex>
+#include <thread>
+#include <vector>
+
+#if defined(__x86_64__)
+#include <immintrin.h>
+#endif
+
+#include "common.h"
+
+namespace jf {
+
+// ------------------------------------------------------------------ error string
+static thread_local char g_err[512] = "";
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+// ------------------------------------------------------------------ worker pool
+// One job at a time (like the reference's single-flight pool, jetfire_pool.h:270-305).  A job is a
+// range [0, n) of rows cut into contiguous shares, one per worker; the submitting thread either
+// blocks in run() or returns immediately from start() and later calls join().
+class Pool {
+ public:
+  static Pool& instance() {
+    static Pool p;
+    return p;
+  }
+  int threads() {
+    std::lock_guard<std::mutex> g(cfg_mu_);
+    return resolve_threads();
+  }
+  void set_threads(int n) {
+    std::lock_guard<std::mutex> g(cfg_mu_);
+    override_ = n;
+  }
+  // Start fn(begin, end) over [0, n) asynchronously.  Returns false if a job is already in flight.
+  bool start(int64_t n, std::function<void(int64_t, int64_t)> fn) {
+    ensure_workers();
+    std::unique_lock<std::mutex> lk(mu_);
+    if (busy_) return false;
+    busy_ = true;
+    fn_ = std::move(fn);
+    n_ = n;
+    const int w = (int)workers_.size();
+    active_ = w;
+    remaining_.store(w, std::memory_order_release);
+    epoch_.fetch_add(1, std::memory_order_acq_rel);
+    lk.unlock();
+    cv_work_.notify_all();
+    return true;
+  }
+  // Wait for the job started with start().  timeout_s <= 0: wait forever.
+  bool join(double timeout_s) {
+    const auto t0 = std::chrono::steady_clock::now();
+    for (int spin = 0; spin < 20000; ++spin) {
+      if (remaining_.load(std::memory_order_acquire) == 0) break;
+#if defined(__x86_64__)
+      _mm_pause();
+#endif
+    }
+    std::unique_lock<std::mutex> lk(mu_);
+    while (remaining_.load(std::memory_order_acquire) != 0) {
+      if (timeout_s > 0) {
+        const double el = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+        if (el > timeout_s) return false;
+        cv_done_.wait_for(lk, std::chrono::milliseconds(1));
+      } else {
+        cv_done_.wait_for(lk, std::chrono::milliseconds(1));
+      }
+    }
+    busy_ = false;
+    fn_ = nullptr;
+    return true;
+  }
+  bool run(int64_t n, std::function<void(int64_t, int64_t)> fn) {
+    while (!start(n, fn)) std::this_thread::yield();
+    return join(0);
+  }
+
+ private:
+  Pool() = default;
+  ~Pool() {
+    {
+      std::lock_guard<std::mutex> g(mu_);
+      stop_ = true;
+      epoch_.fetch_add(1, std::memory_order_acq_rel);
+    }
+    cv_work_.notify_all();
+    for (auto& t : workers_) t.join();
+  }
+  int resolve_threads() {
+    if (override_ > 0) return override_;
+    if (const char* e = std::getenv("JETFIRE_CPU_ATTN_THREADS")) {
+      const int n = std::atoi(e);
+      if (n > 0) return n;
+    }
+    unsigned hc = std::thread::hardware_concurrency();
+    if (hc == 0) hc = 1;
+    return (int)(hc < 64 ? hc : 64);
+  }
+  void ensure_workers() {
+    int want;
+    {
+      std::lock_guard<std::mutex> g(cfg_mu_);
+      want = resolve_threads();
+    }
+    std::unique_lock<std::mutex> lk(mu_);
+    if ((int)workers_.size() == want || busy_) return;
+    // resize: stop the old set, start a new one
+    if (!workers_.empty()) {
+      stop_ = true;
+      epoch_.fetch_add(1, std::memory_order_acq_rel);
+      lk.unlock();
+      cv_work_.notify_all();
+      for (auto& t : workers_) t.join();
+      lk.lock();
+      workers_.clear();
+      stop_ = false;
+    }
+    const uint64_t e0 = epoch_.load(std::memory_order_acquire);
+    for (int i = 0; i < want; ++i) workers_.emplace_back([this, i, e0] { worker(i, e0); });
+  }
+  void worker(int id, uint64_t seen) {
+    for (;;) {
+      // spin briefly for the next epoch, then sleep
+      bool got = false;
+      for (int spin = 0; spin < 4000; ++spin) {
+        if (epoch_.load(std::memory_order_acquire) != seen) { got = true; break; }
+#if defined(__x86_64__)
+        _mm_pause();
+#endif
+      }
+      if (!got) {
+        std::unique_lock<std::mutex> lk(mu_);
+        cv_work_.wait(lk, [&] { return epoch_.load(std::memory_order_acquire) != seen; });
+      }
+      std::function<void(int64_t, int64_t)> fn;
+      int64_t n;
+      int w;
+      {
+        std::lock_guard<std::mutex> g(mu_);
+        seen = epoch_.load(std::memory_order_acquire);
+        if (stop_) return;
+        fn = fn_;
+        n = n_;
+        w = active_;
+      }
+      if (fn && id < w) {
+        const int64_t per = (n + w - 1) / w;
+        const int64_t b = (int64_t)id * per, e = std::min<int64_t>(n, b + per);
+        if (b < e) fn(b, e);
+        if (remaining_.fetch_sub(1, std::memory_order_acq_rel) == 1) {
+          std::lock_guard<std::mutex> g(mu_);
+          cv_done_.notify_all();
+        }
+      }
+    }
+  }
+
+  std::mutex mu_, cfg_mu_;
+  std::condition_variable cv_work_, cv_done_;
+  std::vector<std::thread> workers_;
+  std::function<void(int64_t, int64_t)> fn_;
+  int64_t n_ = 0;
+  int active_ = 0;
+  int override_ = 0;
+  bool busy_ = false, stop_ = false;
+  std::atomic<uint64_t> epoch_{0};
+  std::atomic<int> remaining_{0};
+};
+
+// ------------------------------------------------------------------ row kernel
+static inline float bf(uint16_t b) { return bf16_to_f32(b); }
+
+// One (sequence, query head) row.  fp32 accumulation in ascending channel / slot order.
+static void topk_attn_row(const uint16_t* q, const uint16_t* k_shadow, const uint16_t* v_shadow, int64_t num_slots,
+                          const int64_t* head_map, const int64_t* slots, int K, int H_kv, float scale, uint16_t* out,
+                          float* score_buf) {
+  float qf[D];
+  for (int i = 0; i < D; ++i) qf[i] = bf(q[i]);
+  float mx = -INFINITY;
+  bool any = false;
+  for (int k = 0; k < K; ++k) {
+    const int64_t s = slots[k], h = head_map[k];
+    if (s < 0 || s >= num_slots || h < 0 || h >= H_kv) {
+      score_buf[k] = -INFINITY;
+      continue;
+    }
+    any = true;
+    const uint16_t* kr = k_shadow + ((size_t)h * num_slots + s) * D;
+    float lanes[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int i = 0; i < D; i += 8)
+      for (int j = 0; j < 8; ++j) lanes[j] += qf[i + j] * bf(kr[i + j]);
+    const float dot = ((lanes[0] + lanes[4]) + (lanes[2] + lanes[6])) + ((lanes[1] + lanes[5]) + (lanes[3] + lanes[7]));
+    const float sc = dot * scale;
+    score_buf[k] = sc;
+    if (sc > mx) mx = sc;
+  }
+  if (!any) {
+    memset(out, 0, D * sizeof(uint16_t));
+    return;
+  }
+  float den = 0.0f;
+  for (int k = 0; k < K; ++k) {
+    score_buf[k] = std::exp(score_buf[k] - mx);
+    den += score_buf[k];
+  }
+  if (!(den > 0.0f) || !std::isfinite(den)) {
+    memset(out, 0, D * sizeof(uint16_t));
+    return;
+  }
+  const float inv = 1.0f / den;
+  float o[D];
+  for (int i = 0; i < D; ++i) o[i] = 0.0f;
+  for (int k = 0; k < K; ++k) {
+    const int64_t s = slots[k], h = head_map[k];
+    if (s < 0 || s >= num_slots || h < 0 || h >= H_kv) continue;
+    const uint16_t* vr = v_shadow + ((size_t)h * num_slots + s) * D;
+    const float w = score_buf[k] * inv;
+    for (int i = 0; i < D; ++i) o[i] += w * bf(vr[i]);
+  }
+  for (int i = 0; i < D; ++i) out[i] = f32_to_bf16(o[i]);
+}
+
+struct CpuJob {
+  const uint16_t *q, *k_shadow, *v_shadow;
+  const int64_t *head_map, *ts_buf;
+  uint16_t* o_new;
+  int B, H_q, K, H_kv;
+  int64_t num_slots;
+  float scale;
+};
+
+static void run_rows(const CpuJob& j, int64_t b, int64_t e) {
+  std::vector<float> buf((size_t)j.K);
+  for (int64_t r = b; r < e; ++r)
+    topk_attn_row(j.q + r * D, j.k_shadow, j.v_shadow, j.num_slots, j.head_map + r * j.K, j.ts_buf + r * j.K, j.K, j.H_kv,
+                  j.scale, j.o_new + r * D, buf.data());
+}
+
+}  // namespace jf
+
+using namespace jf;
+
+extern "C" const char* jf_last_error(void) { return g_err; }
+extern "C" const char* jf_version(void) { return "jetfire_amd 0.1 (gfx950)"; }
+
+extern "C" int jf_set_cpu_attn_threads(int n) {
+  Pool::instance().set_threads(n);
+  return JF_OK;
+}
+extern "C" int jf_get_cpu_attn_threads(void) { return Pool::instance().threads(); }
+
+extern "C" int jf_cpu_topk_attn(const uint16_t* q, const uint16_t* k_shadow, const uint16_t* v_shadow,
+                                const int64_t* head_map, const int64_t* ts_buf, uint16_t* o_new, int B, int H_q, int K,
+                                int H_kv, int64_t num_slots, float scale, int64_t* done_flag) {
+  JF_CHECK_ARG(B >= 0 && H_q > 0 && K > 0 && H_kv > 0 && num_slots > 0, "cpu_topk_attn: bad shape");
+  if (B > 0) {
+    JF_CHECK_ARG(q && k_shadow && v_shadow && head_map && ts_buf && o_new, "cpu_topk_attn: null pointer");
+    CpuJob j{q, k_shadow, v_shadow, head_map, ts_buf, o_new, B, H_q, K, H_kv, num_slots, scale};
+    Pool::instance().run((int64_t)B * H_q, [j](int64_t b, int64_t e) { run_rows(j, b, e); });
+  }
+  std::atomic_thread_fence(std::memory_order_release);
+  if (done_flag) reinterpret_cast<std::atomic<int64_t>*>(done_flag)->store(1, std::memory_order_release);
+  return JF_OK;
+}
+
+// ------------------------------------------------------------------ pinned hand-off
+struct jf_handoff {
+  int B, H_q, H_kv, K;
+  int64_t num_slots;
+  const uint16_t *k_shadow, *v_shadow;
+  float scale;
+  uint16_t* q_pin = nullptr;       // (B, H_q, D) bf16
+  int64_t* ts_pin = nullptr;       // (B, H_q, K)
+  uint16_t* o_pin = nullptr;       // (B, H_q, D) bf16
+  std::vector<int64_t> head_map;   // (B, H_q, K)
+  std::atomic<int64_t> submits{0};
+  std::atomic<int> in_flight{0};
+  std::atomic<int> failed{0};
+  double timeout_s = 30.0;         // JETFIRE_CPU_FUTURE_TIMEOUT_S in the reference (decode_path.py:3082-3098)
+};
+
+static void handoff_submit_cb(void* p) {
+  jf_handoff* h = static_cast<jf_handoff*>(p);
+  CpuJob j{h->q_pin, h->k_shadow, h->v_shadow, h->head_map.data(), h->ts_pin, h->o_pin,
+           h->B, h->H_q, h->K, h->H_kv, h->num_slots, h->scale};
+  // Never block inside a stream callback for long: the pool is single-flight, so wait our turn briefly.
+  int tries = 0;
+  while (!Pool::instance().start((int64_t)h->B * h->H_q, [j](int64_t b, int64_t e) { run_rows(j, b, e); })) {
+    std::this_thread::yield();
+    if (++tries > 1000000) { h->failed.store(1); return; }
+  }
+  h->submits.fetch_add(1, std::memory_order_relaxed);
+  h->in_flight.store(1, std::memory_order_release);
+}
+
+static void handoff_wait_cb(void* p) {
+  jf_handoff* h = static_cast<jf_handoff*>(p);
+  if (h->in_flight.load(std::memory_order_acquire) == 0) return;
+  if (!Pool::instance().join(h->timeout_s)) h->failed.store(1);
+  h->in_flight.store(0, std::memory_order_release);
+}
+
+extern "C" jf_handoff* jf_handoff_create(int B, int H_q, int H_kv, int K, int64_t num_slots,
+                                         const uint16_t* k_shadow_host, const uint16_t* v_shadow_host, float scale) {
+  if (B <= 0 || H_q <= 0 || H_kv <= 0 || K <= 0 || num_slots <= 0 || H_q % H_kv != 0 || !k_shadow_host || !v_shadow_host) {
+    set_error("handoff_create: bad arguments");
+    return nullptr;
+  }
+  jf_handoff* h = new jf_handoff();
+  h->B = B; h->H_q = H_q; h->H_kv = H_kv; h->K = K; h->num_slots = num_slots;
+  h->k_shadow = k_shadow_host; h->v_shadow = v_shadow_host; h->scale = scale;
+  if (const char* e = std::getenv("JETFIRE_CPU_FUTURE_TIMEOUT_S")) {
+    const double t = std::atof(e);
+    if (t > 0) h->timeout_s = t;
+  }
+  const size_t nq = (size_t)B * H_q * D * sizeof(uint16_t), nt = (size_t)B * H_q * K * sizeof(int64_t);
+  if (hipHostMalloc((void**)&h->q_pin, nq, hipHostMallocDefault) != hipSuccess ||
+      hipHostMalloc((void**)&h->ts_pin, nt, hipHostMallocDefault) != hipSuccess ||
+      hipHostMalloc((void**)&h->o_pin, nq, hipHostMallocDefault) != hipSuccess) {
+    set_error("handoff_create: hipHostMalloc failed");
+    jf_handoff_destroy(h);
+    return nullptr;
+  }
+  const int G = H_q / H_kv;
+  h->head_map.resize((size_t)B * H_q * K);
+  for (int b = 0; b < B; ++b)
+    for (int hq = 0; hq < H_q; ++hq)
+      for (int k = 0; k < K; ++k) h->head_map[((size_t)b * H_q + hq) * K + k] = hq / G;  // decode_path.py:400-408
+  return h;
+}
+
+extern "C" int jf_handoff_submit(jf_handoff* h, const uint16_t* q_dev, const int64_t* topk_slots_dev, void* stream) {
+  JF_CHECK_ARG(h && q_dev && topk_slots_dev, "handoff_submit: null argument");
+  if (h->failed.load()) { set_error("handoff: an earlier CPU correction job failed or timed out"); return JF_ERR_TIMEOUT; }
+  hipStream_t st = (hipStream_t)stream;
+  JF_CHECK_HIP(hipMemcpyAsync(h->q_pin, q_dev, (size_t)h->B * h->H_q * D * sizeof(uint16_t), hipMemcpyDeviceToHost, st));
+  JF_CHECK_HIP(hipMemcpyAsync(h->ts_pin, topk_slots_dev, (size_t)h->B * h->H_q * h->K * sizeof(int64_t), hipMemcpyDeviceToHost, st));
+  JF_CHECK_HIP(hipLaunchHostFunc(st, handoff_submit_cb, h));
+  return JF_OK;
+}
+
+extern "C" int jf_handoff_wait(jf_handoff* h, uint16_t* o_new_dev, void* stream) {
+  JF_CHECK_ARG(h && o_new_dev, "handoff_wait: null argument");
+  hipStream_t st = (hipStream_t)stream;
+  JF_CHECK_HIP(hipLaunchHostFunc(st, handoff_wait_cb, h));
+  JF_CHECK_HIP(hipMemcpyAsync(o_new_dev, h->o_pin, (size_t)h->B * h->H_q * D * sizeof(uint16_t), hipMemcpyHostToDevice, st));
+  if (h->failed.load()) { set_error("handoff: CPU correction job failed or timed out"); return JF_ERR_TIMEOUT; }
+  return JF_OK;
+}
+
+extern "C" int64_t jf_handoff_submit_count(const jf_handoff* h) { return h ? h->submits.load() : -1; }
+
+extern "C" void jf_handoff_destroy(jf_handoff* h) {
+  if (!h) return;
+  if (h->in_flight.load(std::memory_order_acquire)) Pool::instance().join(h->timeout_s);
+  if (h->q_pin) (void)hipHostFree(h->q_pin);
+  if (h->ts_pin) (void)hipHostFree(h->ts_pin);
+  if (h->o_pin) (void)hipHostFree(h->o_pin);
+  delete h;
+}

@@ -1,0 +1,256 @@
+// Stage B in its split form: consumes an fp32 score tensor and produces o_hat, o_old_unnorm, W.
+//
+//   w_s   = exp(score_s - m) * inv_z                (jetfire_vllm/csrc/int4_softmax_v.cu:162-176)
+//   ws    = w_s * f32(v_scale[s, group(d)])         (jetfire_vllm/csrc/int2_softmax_v.cu:681-694)
+//   o_hat[d] = sum_s fma(ws, code[s, d] - offset)   (:696-706), positions in ascending order
+//   o_old_unnorm / W: the same sums over the top-k positions only (:738-788)
+//
+// Three launches: row statistics (only when the caller has none), a split-S weighted-V pass in which
+// one workgroup owns a (sequence, kv-head, S-range) and serves all G query heads from one read of V,
+// and a combine pass that adds the split partials in ascending order (deterministic, no atomics) and
+// does the top-k pre-correction.
+#include "common.h"
+
+namespace jf {
+namespace {
+
+constexpr int SV_THREADS = 128;
+
+__device__ inline float block_max_128(float v, float* red) {
+  v = wave_max(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return fmaxf(red[0], red[1]);
+}
+__device__ inline float block_sum_128(float v, float* red) {
+  v = wave_sum(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return red[0] + red[1];
+}
+
+__global__ __launch_bounds__(SV_THREADS) void softmax_stats_kernel(const float* __restrict__ scores,
+                                                                   const int32_t* __restrict__ seq_lens,
+                                                                   float* __restrict__ m_out, float* __restrict__ iz_out,
+                                                                   int max_S, int H_q) {
+  __shared__ float red[2];
+  const int b = blockIdx.x, hq = blockIdx.y, tid = threadIdx.x;
+  const size_t bh = (size_t)b * H_q + hq;
+  const int n = max(0, min(max_S, seq_lens[b]));
+  const float* row = scores + bh * (size_t)max_S;
+  float lm = -INFINITY;
+  for (int i = tid; i < n; i += SV_THREADS) lm = fmaxf(lm, row[i]);
+  float m = block_max_128(lm, red);
+  if (!isfinite(m)) m = 0.0f;
+  float ls = 0.0f;
+  for (int i = tid; i < n; i += SV_THREADS) ls += __expf(row[i] - m);
+  const float z = block_sum_128(ls, red);
+  if (tid == 0) {
+    m_out[bh] = m;
+    iz_out[bh] = (z > 0.0f) ? (1.0f / z) : 0.0f;
+  }
+}
+
+template <int NBITS>
+__device__ inline int v_code(const uint8_t* row, int d) {
+  if (NBITS == 2) return (int)((row[d >> 2] >> ((3 - (d & 3)) * 2)) & 3) - 2;
+  return (int)((row[d >> 1] >> ((1 - (d & 1)) * 4)) & 15) - 8;
+}
+
+// grid (n_splits, H_kv, B); thread = output channel d; acc[g] for the G query heads of this kv-head.
+template <int NBITS, int G, int NG>
+__global__ __launch_bounds__(SV_THREADS) void weighted_v_split_kernel(
+    const float* __restrict__ scores, const float* __restrict__ softmax_m, const float* __restrict__ softmax_inv_z,
+    const uint8_t* __restrict__ v_data, const uint16_t* __restrict__ v_scales, const int64_t* __restrict__ block_table,
+    const int32_t* __restrict__ seq_lens, float* __restrict__ partial, int H_q, int H_kv, int max_S, int max_blocks,
+    int64_t num_slots, int chunk, int n_splits) {
+  constexpr int P = D * NBITS / 8;
+  __shared__ __align__(16) uint8_t vbuf[BS * P];
+  __shared__ float wsbuf[G][BS][NG];
+  const int split = blockIdx.x, hkv = blockIdx.y, b = blockIdx.z, tid = threadIdx.x;
+  const int S = max(0, min(max_S, seq_lens[b]));
+  const int s0 = split * chunk, s1 = min(s0 + chunk, S);
+  float acc[G];
+#pragma unroll
+  for (int g = 0; g < G; ++g) acc[g] = 0.0f;
+  const int grp = (NG == 1) ? 0 : (tid / (D / NG));
+  const uint8_t* vbase = v_data + (size_t)hkv * num_slots * P;
+  const uint16_t* sbase = v_scales + (size_t)hkv * num_slots * NG;
+  const int64_t* bt = block_table + (size_t)b * max_blocks;
+  for (int p0 = s0; p0 < s1; p0 += BS) {  // chunk is a multiple of BS, so pages are aligned
+    const int64_t base_slot = bt[p0 / BS] * BS;
+    __syncthreads();
+    {
+      constexpr int DW = BS * P / 4 / SV_THREADS;  // dwords per thread
+      const uint32_t* src = reinterpret_cast<const uint32_t*>(vbase + base_slot * P);
+#pragma unroll
+      for (int i = 0; i < DW; ++i) reinterpret_cast<uint32_t*>(vbuf)[tid + i * SV_THREADS] = src[tid + i * SV_THREADS];
+    }
+    for (int i = tid; i < G * BS; i += SV_THREADS) {
+      const int g = i / BS, j = i % BS;
+      const int p = p0 + j;
+      const size_t bh = (size_t)b * H_q + (size_t)hkv * G + g;
+      float w = 0.0f;
+      if (p < s1) w = __expf(scores[bh * (size_t)max_S + p] - softmax_m[bh]) * softmax_inv_z[bh];
+#pragma unroll
+      for (int k = 0; k < NG; ++k)
+        wsbuf[g][j][k] = (p < s1) ? w * bf16_to_f32(sbase[(size_t)(base_slot + j) * NG + k]) : 0.0f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < BS; ++j) {
+      const float c = (float)v_code<NBITS>(vbuf + j * P, tid);
+#pragma unroll
+      for (int g = 0; g < G; ++g) acc[g] = __builtin_fmaf(wsbuf[g][j][grp], c, acc[g]);
+    }
+  }
+#pragma unroll
+  for (int g = 0; g < G; ++g)
+    partial[(((size_t)b * H_q + (size_t)hkv * G + g) * n_splits + split) * D + tid] = acc[g];
+}
+
+// grid (B, H_q); adds split partials in order, then the top-k pre-correction.
+template <int NBITS, int NG>
+__global__ __launch_bounds__(SV_THREADS) void combine_precorr_kernel(
+    const float* __restrict__ partial, const float* __restrict__ scores, const float* __restrict__ softmax_m,
+    const float* __restrict__ softmax_inv_z, const uint8_t* __restrict__ v_data, const uint16_t* __restrict__ v_scales,
+    const int64_t* __restrict__ block_table, const int32_t* __restrict__ seq_lens, const int64_t* __restrict__ topk_idx,
+    float* __restrict__ o_hat, float* __restrict__ o_old, float* __restrict__ W_out, int H_q, int H_kv, int max_S,
+    int max_blocks, int64_t num_slots, int n_splits, int K) {
+  constexpr int P = D * NBITS / 8;
+  constexpr int STEP = 128;
+  __shared__ int64_t slot_buf[STEP];
+  __shared__ float ws_buf[STEP][NG];
+  __shared__ float w_buf[STEP];
+  const int b = blockIdx.x, hq = blockIdx.y, tid = threadIdx.x;
+  const size_t bh = (size_t)b * H_q + hq;
+  const int hkv = hq / (H_q / H_kv);
+  float acc = 0.0f;
+  for (int s = 0; s < n_splits; ++s) acc += partial[(bh * n_splits + s) * D + tid];
+  o_hat[bh * D + tid] = acc;
+  if (topk_idx == nullptr) return;
+  const int S = max(0, min(max_S, seq_lens[b]));
+  const int grp = (NG == 1) ? 0 : (tid / (D / NG));
+  const uint8_t* vbase = v_data + (size_t)hkv * num_slots * P;
+  const uint16_t* sbase = v_scales + (size_t)hkv * num_slots * NG;
+  const int64_t* bt = block_table + (size_t)b * max_blocks;
+  const float m = softmax_m[bh], iz = softmax_inv_z[bh];
+  float acc_old = 0.0f, acc_w = 0.0f;
+  for (int k0 = 0; k0 < K; k0 += STEP) {
+    __syncthreads();
+    {
+      const int kk = k0 + tid;
+      int64_t slot = -1;
+      float w = 0.0f;
+      if (kk < K) {
+        const int64_t pos = topk_idx[bh * (size_t)K + kk];
+        if (pos >= 0 && pos < S) {
+          const int64_t blk = bt[pos / BS];
+          if (blk >= 0) {
+            slot = blk * BS + pos % BS;
+            w = __expf(scores[bh * (size_t)max_S + pos] - m) * iz;
+          }
+        }
+      }
+      slot_buf[tid] = slot;
+      w_buf[tid] = w;
+#pragma unroll
+      for (int g = 0; g < NG; ++g) ws_buf[tid][g] = (slot >= 0) ? w * bf16_to_f32(sbase[(size_t)slot * NG + g]) : 0.0f;
+    }
+    __syncthreads();
+    const int kend = min(STEP, K - k0);
+    for (int j = 0; j < kend; ++j) {
+      const int64_t slot = slot_buf[j];
+      if (slot < 0) continue;
+      const float c = (float)v_code<NBITS>(vbase + slot * P, tid);
+      acc_old = __builtin_fmaf(ws_buf[j][grp], c, acc_old);
+      acc_w += w_buf[j];
+    }
+  }
+  o_old[bh * D + tid] = acc_old;
+  if (tid == 0) W_out[bh] = acc_w;
+}
+
+inline int sv_splits(int B, int H_kv, int max_S) {
+  const int units = B * H_kv;
+  int want = (2048 + units - 1) / units;
+  const int max_by_len = (max_S + 63) / 64;
+  want = want < 1 ? 1 : want;
+  want = want > max_by_len ? max_by_len : want;
+  return want < 1 ? 1 : want;
+}
+
+}  // namespace
+}  // namespace jf
+
+using namespace jf;
+
+extern "C" size_t jf_softmax_v_workspace_bytes(int B, int H_q, int max_S) {
+  if (B <= 0 || H_q <= 0) return 256;
+  // partials for the largest split count any H_kv can produce, plus the two statistics rows
+  const size_t max_splits = (size_t)((max_S + 63) / 64 < 2048 ? (max_S + 63) / 64 : 2048);
+  return ((size_t)B * H_q * (max_splits > 0 ? max_splits : 1) * D + 2 * (size_t)B * H_q) * sizeof(float) + 256;
+}
+
+extern "C" int jf_softmax_v_pre_corr(const float* scores, const float* softmax_m, const float* softmax_inv_z,
+                                     const uint8_t* v_data, const uint16_t* v_scales, const int64_t* block_table,
+                                     const int32_t* seq_lens, const int64_t* topk_idx, int B, int H_q, int H_kv,
+                                     int max_S, int max_blocks, int64_t num_slots, int block_size, int top_k,
+                                     int v_nbits, int n_scale_groups, float* o_hat, float* o_old_unnorm, float* W,
+                                     void* workspace, size_t workspace_bytes, void* stream) {
+  JF_CHECK_ARG(B >= 0 && H_q > 0 && H_kv > 0 && max_S >= 0 && H_q % H_kv == 0, "softmax_v: bad shape");
+  const int G = H_q / H_kv;
+  JF_CHECK_ARG(G == 1 || G == 2 || G == 4 || G == 8 || G == 16, "softmax_v: GQA group %d not in {1,2,4,8,16}", G);
+  JF_CHECK_ARG(block_size == 16, "wvs2 only supports block_size=16");
+  JF_CHECK_ARG(v_nbits == 2 || v_nbits == 4, "softmax_v: v_nbits must be 2 or 4 (got %d)", v_nbits);
+  JF_CHECK_ARG(n_scale_groups == 1 || n_scale_groups == 2, "wvs2 requires num_groups=1 or 2 (got %d)", n_scale_groups);
+  JF_CHECK_ARG((int64_t)max_blocks * block_size >= max_S, "softmax_v: block_table does not cover max_S");
+  JF_CHECK_ARG((softmax_m == nullptr) == (softmax_inv_z == nullptr), "softmax_v: softmax_m and softmax_inv_z go together");
+  JF_CHECK_ARG(topk_idx == nullptr || top_k > 0, "softmax_v: top_k must be positive");
+  if (B == 0) return JF_OK;
+  JF_CHECK_ARG(scores && v_data && v_scales && block_table && seq_lens && o_hat, "softmax_v: null pointer");
+  JF_CHECK_ARG(topk_idx == nullptr || (o_old_unnorm && W), "softmax_v: o_old_unnorm / W required with topk_idx");
+  JF_CHECK_ARG(workspace && workspace_bytes >= jf_softmax_v_workspace_bytes(B, H_q, max_S),
+               "softmax_v: workspace too small (%zu < %zu)", workspace_bytes, jf_softmax_v_workspace_bytes(B, H_q, max_S));
+  hipStream_t st = (hipStream_t)stream;
+  const int n_splits = sv_splits(B, H_kv, max_S);
+  int chunk = (max_S + n_splits - 1) / n_splits;
+  chunk = (chunk + BS - 1) / BS * BS;
+  if (chunk < BS) chunk = BS;
+  float* partial = reinterpret_cast<float*>(workspace);
+  float* m_ws = partial + (size_t)B * H_q * n_splits * D;
+  float* iz_ws = m_ws + (size_t)B * H_q;
+  if (softmax_m == nullptr) {
+    hipLaunchKernelGGL(softmax_stats_kernel, dim3(B, H_q), dim3(SV_THREADS), 0, st, scores, seq_lens, m_ws, iz_ws, max_S, H_q);
+    JF_CHECK_LAUNCH();
+    softmax_m = m_ws;
+    softmax_inv_z = iz_ws;
+  }
+  dim3 grid(n_splits, H_kv, B), block(SV_THREADS);
+#define JF_SV_LAUNCH(NB, NGC)                                                                                           \
+  JF_DISPATCH_G2(G, {                                                                                                    \
+    hipLaunchKernelGGL((weighted_v_split_kernel<NB, GG, NGC>), grid, block, 0, st, scores, softmax_m, softmax_inv_z,     \
+                       v_data, v_scales, block_table, seq_lens, partial, H_q, H_kv, max_S, max_blocks, num_slots, chunk, \
+                       n_splits);                                                                                        \
+  });                                                                                                                    \
+  JF_CHECK_LAUNCH();                                                                                                     \
+  hipLaunchKernelGGL((combine_precorr_kernel<NB, NGC>), dim3(B, H_q), block, 0, st, partial, scores, softmax_m,          \
+                     softmax_inv_z, v_data, v_scales, block_table, seq_lens, topk_idx, o_hat, o_old_unnorm, W, H_q, H_kv, \
+                     max_S, max_blocks, num_slots, n_splits, top_k);                                                     \
+  JF_CHECK_LAUNCH();
+#define JF_DISPATCH_G2(G, ...)                               \
+  switch (G) {                                               \
+    case 1: { constexpr int GG = 1; __VA_ARGS__; } break;    \
+    case 2: { constexpr int GG = 2; __VA_ARGS__; } break;    \
+    case 4: { constexpr int GG = 4; __VA_ARGS__; } break;    \
+    case 8: { constexpr int GG = 8; __VA_ARGS__; } break;    \
+    default: { constexpr int GG = 16; __VA_ARGS__; } break;  \
+  }
+  if (v_nbits == 2 && n_scale_groups == 1) { JF_SV_LAUNCH(2, 1) }
+  else if (v_nbits == 2) { JF_SV_LAUNCH(2, 2) }
+  else if (n_scale_groups == 1) { JF_SV_LAUNCH(4, 1) }
+  else { JF_SV_LAUNCH(4, 2) }
+  return JF_OK;
+}

@@ -1,0 +1,475 @@
+"""Torch-facing operators over the C ABI.
+
+Function names, positional argument order, dtypes, return values and error behaviour follow the
+reference's extension modules (jetfire_vllm/csrc/*.cu pybind blocks and
+jetfire_vllm/kernels/fused_quant_write.py), so an adapter written for those calls these unchanged.
+Tensors are only used for device memory and the current stream; all arithmetic is in the HIP library.
+"""
+from __future__ import annotations
+
+from typing import List, Optional
+
+import torch
+
+from . import _lib
+
+HEAD_DIM = 128
+SUPPORTED_TOP_K = (32, 64, 128, 256, 512, 1024, 2048, 4096, 8192)
+
+_workspaces: dict = {}
+
+
+def _check(cond: bool, msg: str) -> None:
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _workspace(device: torch.device, nbytes: int, tag: str) -> torch.Tensor:
+    """Per-(device, stream, tag) scratch buffer that only grows; safe under stream ordering."""
+    key = (device, torch.cuda.current_stream(device).cuda_stream, tag)
+    buf = _workspaces.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
+        _workspaces[key] = buf
+    return buf
+
+
+def _gpu(*ts: torch.Tensor) -> None:
+    for t in ts:
+        _check(t.is_cuda, "all inputs must be on the GPU")
+
+
+# --------------------------------------------------------------------------- quantise-on-append
+
+
+def _quant_write(x, slots, out_data, out_scale, group_size: int, nbits: int) -> None:
+    lib = _lib.load()
+    _check(x.is_cuda and x.dtype == torch.bfloat16, "key/value tokens must be bf16 on the GPU")
+    _check(x.dim() == 3 and x.shape[2] == HEAD_DIM, "tokens must be (T, H_kv, 128)")
+    _check(x.stride(2) == 1, "tokens must be contiguous in the last dimension")
+    _check(slots.is_cuda and slots.dtype == torch.int64 and slots.dim() == 1 and slots.shape[0] == x.shape[0],
+           "slots must be (T,) int64 on the token device")
+    T, H_kv, D = x.shape
+    _check(D % group_size == 0, f"D={D} not divisible by gs={group_size}")
+    if out_scale.dim() == 2:
+        out_scale = out_scale.unsqueeze(-1)
+    _check(out_data.dtype == torch.uint8 and out_scale.dtype == torch.bfloat16, "cache must be uint8 data + bf16 scales")
+    _check(out_data.shape[0] == H_kv and out_data.shape[2] == D * nbits // 8 and out_data.stride(2) == 1,
+           f"cache data must be (H_kv, num_slots, {D * nbits // 8})")
+    _check(out_scale.shape[0] == H_kv and out_scale.shape[2] == D // group_size and out_scale.stride(2) == 1,
+           "cache scales must be (H_kv, num_slots, D/group_size)")
+    slots = slots.contiguous()
+    _lib.check(lib.jf_quant_write_sym(
+        x.data_ptr(), x.stride(0), x.stride(1), slots.data_ptr(), T, H_kv,
+        out_data.data_ptr(), out_data.stride(0), out_data.stride(1),
+        out_scale.data_ptr(), out_scale.stride(0), out_scale.stride(1),
+        out_data.shape[1], int(group_size), nbits, _stream(x)))
+
+
+def fused_quant_write_int2_sym(val_tok, slots, out_data, out_scale, group_size: int) -> None:
+    """fused_quant_write.py:242-270"""
+    _quant_write(val_tok, slots, out_data, out_scale, group_size, 2)
+
+
+def fused_quant_write_int3_sym(value_tok, slot_idx, v_data, v_scales, group_size: int) -> None:
+    """fused_quant_write.py:746-781"""
+    _quant_write(value_tok, slot_idx, v_data, v_scales, group_size, 3)
+
+
+def fused_quant_write_int4_sym(value_tok, slot_idx, v_data, v_scales, group_size: int) -> None:
+    """fused_quant_write.py:337-369"""
+    _quant_write(value_tok, slot_idx, v_data, v_scales, group_size, 4)
+
+
+def fused_quant_write_int4_sym_kv(key_tok, value_tok, slot_idx, k_data, k_scales, v_data, v_scales,
+                                  group_size: int) -> None:
+    """fused_quant_write.py:552-617 (K and V in one launch)."""
+    lib = _lib.load()
+    _check(key_tok.is_cuda and value_tok.is_cuda, "tokens must be on the GPU")
+    _check(key_tok.dtype == torch.bfloat16 and value_tok.dtype == torch.bfloat16, "tokens must be bf16")
+    _check(value_tok.shape == key_tok.shape and key_tok.dim() == 3 and key_tok.shape[2] == HEAD_DIM,
+           "key/value tokens must both be (T, H_kv, 128)")
+    _check(key_tok.stride(2) == 1 and value_tok.stride(2) == 1, "tokens must be contiguous in the last dimension")
+    T, H_kv, D = key_tok.shape
+    _check(D % group_size == 0, f"D={D} not divisible by gs={group_size}")
+    if k_scales.dim() == 2:
+        k_scales = k_scales.unsqueeze(-1)
+    if v_scales.dim() == 2:
+        v_scales = v_scales.unsqueeze(-1)
+    for d, s in ((k_data, k_scales), (v_data, v_scales)):
+        _check(d.dtype == torch.uint8 and s.dtype == torch.bfloat16, "cache must be uint8 data + bf16 scales")
+        _check(d.shape[0] == H_kv and d.shape[2] == D // 2 and d.stride(2) == 1, "cache data must be (H_kv, num_slots, 64)")
+        _check(s.shape[0] == H_kv and s.shape[2] == D // group_size and s.stride(2) == 1, "bad cache scales shape")
+    _check(slot_idx.is_cuda and slot_idx.dtype == torch.int64 and slot_idx.shape == (T,), "slots must be (T,) int64")
+    slot_idx = slot_idx.contiguous()
+    _lib.check(lib.jf_quant_write_int4_sym_kv(
+        key_tok.data_ptr(), key_tok.stride(0), key_tok.stride(1),
+        value_tok.data_ptr(), value_tok.stride(0), value_tok.stride(1),
+        slot_idx.data_ptr(), T, H_kv,
+        k_data.data_ptr(), k_data.stride(0), k_data.stride(1), k_scales.data_ptr(), k_scales.stride(0), k_scales.stride(1),
+        v_data.data_ptr(), v_data.stride(0), v_data.stride(1), v_scales.data_ptr(), v_scales.stride(0), v_scales.stride(1),
+        k_data.shape[1], int(group_size), _stream(key_tok)))
+
+
+# --------------------------------------------------------------------------- Stage A
+
+
+def _stage_a_args(q, k_data, k_scales, block_table, seq_lens, H_q, H_kv, packed):
+    _gpu(q, k_data, k_scales, block_table, seq_lens)
+    _check(q.dtype == torch.bfloat16, "q must be bf16")
+    _check(k_data.dtype == torch.uint8, "k_data must be uint8")
+    _check(k_scales.dtype == torch.bfloat16, "k_scales must be bf16")
+    _check(block_table.dtype == torch.int64, "block_table must be int64")
+    _check(seq_lens.dtype == torch.int32, "seq_lens must be int32")
+    _check(q.dim() == 3 and q.size(2) == HEAD_DIM, "q must be (B, H_q, 128)")
+    _check(q.size(1) == H_q, "q.size(1) must equal H_q")
+    _check(H_q % H_kv == 0, "H_q must be divisible by H_kv")
+    _check(k_data.dim() == 3 and k_data.size(-1) == packed, f"k_data last dim must be {packed}")
+    _check(k_data.size(0) == H_kv, "k_data.size(0) must equal H_kv")
+    _check(block_table.dim() == 2 and block_table.size(0) == q.size(0), "block_table must be (B, max_blocks)")
+    _check(seq_lens.numel() == q.size(0), "seq_lens must be (B,)")
+    ks = k_scales.unsqueeze(-1) if k_scales.dim() == 2 else k_scales
+    return q.contiguous(), k_data.contiguous(), ks.contiguous(), block_table.contiguous(), seq_lens.contiguous()
+
+
+def int3_qk_scores(q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_kv, block_size, attn_scale):
+    """int3_qk_scores.cu:318-390 -> scores (B, H_q, max_S) fp32."""
+    lib = _lib.load()
+    q, kd, ks, bt, sl = _stage_a_args(q, k_data, k_scales, block_table, seq_lens, H_q, H_kv, 48)
+    ng = ks.size(2)
+    _check(ng in (1, 2), f"int3_qk_scores currently supports K quant groups 1 or 2, got {ng}")
+    B = q.size(0)
+    scores = torch.empty((B, H_q, max_S), dtype=torch.float32, device=q.device)
+    _lib.check(lib.jf_int3_qk_scores(q.data_ptr(), kd.data_ptr(), ks.data_ptr(), bt.data_ptr(), sl.data_ptr(),
+                                     B, H_q, H_kv, int(max_S), bt.size(1), kd.size(1), ng, int(block_size),
+                                     float(attn_scale), scores.data_ptr(), _stream(q)))
+    return scores
+
+
+def int8tc_qk_scores(q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_kv, block_size, attn_scale):
+    """int8tc_qk_scores.cu:1263-1331 -> scores (B, H_q, max_S) fp32."""
+    lib = _lib.load()
+    if k_scales.dim() == 3:
+        _check(k_scales.size(2) == 1, "int8tc_qk_scores needs one K scale per token (group 128)")
+    q, kd, ks, bt, sl = _stage_a_args(q, k_data, k_scales, block_table, seq_lens, H_q, H_kv, 64)
+    B = q.size(0)
+    scores = torch.empty((B, H_q, max_S), dtype=torch.float32, device=q.device)
+    _lib.check(lib.jf_int8tc_qk_scores(q.data_ptr(), kd.data_ptr(), ks.data_ptr(), bt.data_ptr(), sl.data_ptr(),
+                                       B, H_q, H_kv, int(max_S), bt.size(1), kd.size(1), int(block_size),
+                                       float(attn_scale), scores.data_ptr(), _stream(q)))
+    return scores
+
+
+def _topk(scores, block_table, seq_lens, max_S, H_q, block_size, top_k, stats: bool, name: str, minimum: int = 32):
+    lib = _lib.load()
+    _check(int(top_k) in SUPPORTED_TOP_K and int(top_k) >= minimum,
+           f"{name}: unsupported radix-select top_k={top_k} (supported: "
+           f"{','.join(str(k) for k in SUPPORTED_TOP_K if k >= minimum)})")
+    _check(max_S <= 262144, f"{name}: max_S={max_S} exceeds supported limit (262144).")
+    B = scores.size(0)
+    bt, sl = block_table.contiguous(), seq_lens.contiguous()
+    idx = torch.empty((B, H_q, top_k), dtype=torch.int64, device=scores.device)
+    slots = torch.empty((B, H_q, top_k), dtype=torch.int64, device=scores.device)
+    m = iz = None
+    if stats:
+        m = torch.empty((B, H_q), dtype=torch.float32, device=scores.device)
+        iz = torch.empty((B, H_q), dtype=torch.float32, device=scores.device)
+    _lib.check(lib.jf_topk_slots(scores.data_ptr(), sl.data_ptr(), bt.data_ptr(), B, H_q, int(max_S), bt.size(1),
+                                 int(block_size), int(top_k), idx.data_ptr(), slots.data_ptr(), _ptr(m), _ptr(iz),
+                                 _stream(scores)))
+    return idx, slots, m, iz
+
+
+def int3_qk_scores_topk(q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_kv, block_size, attn_scale,
+                        top_k) -> List[torch.Tensor]:
+    """int3_qk_scores.cu:562-633 -> [scores, topk_idx, topk_slots]."""
+    scores = int3_qk_scores(q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_kv, block_size, attn_scale)
+    idx, slots, _, _ = _topk(scores, block_table, seq_lens, max_S, H_q, block_size, top_k, False, "int3_qk_scores_topk")
+    return [scores, idx, slots]
+
+
+def int8tc_qk_scores_topk(q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_kv, block_size, attn_scale,
+                          top_k) -> List[torch.Tensor]:
+    """int8tc_qk_scores.cu:2345-2424 -> [scores, topk_idx, topk_slots]."""
+    scores = int8tc_qk_scores(q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_kv, block_size, attn_scale)
+    idx, slots, _, _ = _topk(scores, block_table, seq_lens, max_S, H_q, block_size, top_k, False, "int8tc_qk_scores_topk")
+    return [scores, idx, slots]
+
+
+def int8tc_qk_scores_topk_stats(q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_kv, block_size, attn_scale,
+                                top_k) -> List[torch.Tensor]:
+    """int8tc_qk_scores.cu:2426-2482 -> [scores, topk_idx, topk_slots, softmax_m, softmax_inv_z]."""
+    scores = int8tc_qk_scores(q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_kv, block_size, attn_scale)
+    idx, slots, m, iz = _topk(scores, block_table, seq_lens, max_S, H_q, block_size, top_k, True,
+                              "int8tc_qk_scores_topk_stats", minimum=64)
+    return [scores, idx, slots, m, iz]
+
+
+# --------------------------------------------------------------------------- Stage B
+
+
+def _softmax_v(scores, m, iz, v_data, v_scales, block_table, seq_lens, topk_idx, max_S, H_q, H_kv, block_size, top_k,
+               nbits: int, outs=None):
+    lib = _lib.load()
+    _gpu(scores, v_data, v_scales, block_table, seq_lens)
+    _check(scores.dtype == torch.float32 and scores.dim() == 3, "scores must be (B, H_q, max_S) fp32")
+    _check(v_data.dtype == torch.uint8 and v_scales.dtype == torch.bfloat16, "v_data uint8 / v_scales bf16")
+    _check(block_table.dtype == torch.int64 and seq_lens.dtype == torch.int32, "block_table int64 / seq_lens int32")
+    _check(v_data.dim() == 3 and v_data.size(2) == HEAD_DIM * nbits // 8, f"v_data last dim must be {HEAD_DIM * nbits // 8}")
+    _check(H_q % H_kv == 0, "H_q must be divisible by H_kv")
+    _check(int(block_size) == 16, "wvs2 only supports block_size=16")
+    _check(scores.size(2) == max_S and scores.size(1) == H_q, "scores must be (B, H_q, max_S)")
+    if topk_idx is not None:
+        _check(topk_idx.is_cuda and topk_idx.dtype == torch.int64 and topk_idx.dim() == 3 and topk_idx.size(2) == top_k,
+               "topk_idx must be (B, H_q, top_k) int64")
+        topk_idx = topk_idx.contiguous()
+    vs = v_scales.unsqueeze(-1) if v_scales.dim() == 2 else v_scales
+    ng = vs.size(2)
+    _check(ng in (1, 2), f"wvs2 requires num_groups=1 or 2 (got {ng})")
+    sc, vd, vs = scores.contiguous(), v_data.contiguous(), vs.contiguous()
+    bt, sl = block_table.contiguous(), seq_lens.contiguous()
+    B = sc.size(0)
+    dev = sc.device
+    if outs is None:
+        o_hat = torch.empty((B, H_q, HEAD_DIM), dtype=torch.float32, device=dev)
+        o_old = torch.zeros((B, H_q, HEAD_DIM), dtype=torch.float32, device=dev)
+        W = torch.zeros((B, H_q), dtype=torch.float32, device=dev)
+    else:
+        o_hat, o_old, W = outs
+        for t in outs:
+            _check(t.is_cuda and t.dtype == torch.float32 and t.is_contiguous(), "output buffers must be contiguous fp32")
+    need = lib.jf_softmax_v_workspace_bytes(B, H_q, int(max_S))
+    ws = _workspace(dev, need, "softmax_v")
+    if m is not None:
+        m, iz = m.contiguous(), iz.contiguous()
+    _lib.check(lib.jf_softmax_v_pre_corr(
+        sc.data_ptr(), _ptr(m), _ptr(iz), vd.data_ptr(), vs.data_ptr(), bt.data_ptr(), sl.data_ptr(), _ptr(topk_idx),
+        B, H_q, H_kv, int(max_S), bt.size(1), vd.size(1), int(block_size), int(top_k), nbits, ng,
+        o_hat.data_ptr(), o_old.data_ptr(), W.data_ptr(), ws.data_ptr(), ws.numel(), _stream(sc)))
+    return [o_hat, o_old, W]
+
+
+def int2_softmax_v_with_pre_corr_wvs2(scores, v_data, v_scales, block_table, seq_lens, topk_idx, max_S, H_q, H_kv,
+                                      block_size, top_k) -> List[torch.Tensor]:
+    """int2_softmax_v.cu:792-901 -> [o_hat, o_old_unnorm, W]."""
+    return _softmax_v(scores, None, None, v_data, v_scales, block_table, seq_lens, topk_idx, max_S, H_q, H_kv,
+                      block_size, top_k, 2)
+
+
+def int2_softmax_v_with_pre_corr_wvs2_inplace(scores, v_data, v_scales, block_table, seq_lens, topk_idx, weights,
+                                              o_hat, o_old_unnorm, W_out, max_S, H_q, H_kv, block_size, top_k) -> None:
+    """int2_softmax_v.cu:903-1010: caller-owned outputs (graph capture). `weights` is accepted and unused:
+    this implementation never materialises the softmax weights."""
+    _softmax_v(scores, None, None, v_data, v_scales, block_table, seq_lens, topk_idx, max_S, H_q, H_kv, block_size,
+               top_k, 2, outs=(o_hat, o_old_unnorm, W_out))
+
+
+def int2_softmax_v_with_pre_corr(scores, v_data, v_scales, block_table, seq_lens, topk_idx, max_S, H_q, H_kv,
+                                 block_size, top_k) -> List[torch.Tensor]:
+    return int2_softmax_v_with_pre_corr_wvs2(scores, v_data, v_scales, block_table, seq_lens, topk_idx, max_S, H_q,
+                                             H_kv, block_size, top_k)
+
+
+def int2_softmax_v(scores, v_data, v_scales, block_table, seq_lens, max_S, H_q, H_kv, block_size) -> torch.Tensor:
+    return _softmax_v(scores, None, None, v_data, v_scales, block_table, seq_lens, None, max_S, H_q, H_kv, block_size,
+                      32, 2)[0]
+
+
+def int4_softmax_v_with_pre_corr_wvs2_scores(scores, v_data, v_scales, block_table, seq_lens, topk_idx, max_S, H_q,
+                                             H_kv, block_size, top_k) -> List[torch.Tensor]:
+    """int4_softmax_v.cu:2203-2235 -> [o_hat, o_old_unnorm, W]."""
+    return _softmax_v(scores, None, None, v_data, v_scales, block_table, seq_lens, topk_idx, max_S, H_q, H_kv,
+                      block_size, top_k, 4)
+
+
+def int4_softmax_v_with_pre_corr_wvs2(scores, v_data, v_scales, block_table, seq_lens, topk_idx, max_S, H_q, H_kv,
+                                      block_size, top_k) -> List[torch.Tensor]:
+    return int4_softmax_v_with_pre_corr_wvs2_scores(scores, v_data, v_scales, block_table, seq_lens, topk_idx, max_S,
+                                                    H_q, H_kv, block_size, top_k)
+
+
+def int8tc_softmax_v_with_pre_corr_reg_stats(scores, softmax_m, softmax_inv_z, v_data, v_scales, block_table, seq_lens,
+                                             topk_idx, max_S, H_q, H_kv, block_size, top_k) -> List[torch.Tensor]:
+    """int8tc_softmax_v_fused.cu:1591-1734 -> [o_hat, o_old_unnorm, W].
+
+    The reference quantises P*v_scale to int8 per 32-token tile (an extra approximation it tolerates at 3e-3,
+    scripts/validate_runtime.py:173-176); this implementation keeps the weights in fp32, i.e. it returns the dense
+    quantity that approximation targets, and uses the Stage-A statistics it is handed."""
+    _check(softmax_m.dtype == torch.float32 and softmax_inv_z.dtype == torch.float32, "softmax stats must be fp32")
+    vs = v_scales.unsqueeze(-1) if v_scales.dim() == 2 else v_scales
+    _check(vs.size(2) == 1, "int8tc_softmax_v requires one V scale per token (group 128)")
+    _check(H_q // H_kv <= 16, "int8tc_softmax_v requires H_q/H_kv <= 16")
+    return _softmax_v(scores, softmax_m, softmax_inv_z, v_data, v_scales, block_table, seq_lens, topk_idx, max_S, H_q,
+                      H_kv, block_size, top_k, 4)
+
+
+# --------------------------------------------------------------------------- fused scan
+
+
+def fused_attn_topk(scheme: str, q, k_data, k_scales, v_data, v_scales, block_table, seq_lens, max_S, H_q, H_kv,
+                    block_size, top_k, attn_scale, group_size: Optional[int] = None, return_scores: bool = False,
+                    return_stats: bool = False):
+    """One fused pass: -> (o_hat, topk_slots, o_old_unnorm, W, topk_idx[, softmax_m, softmax_inv_z][, scores]).
+
+    The single-call contract is the one of the reference's int2_fused_attn_topk
+    (jetfire_vllm/kernels/int2_fused_attn_topk.py:5-10) extended to the K3V2 / K4V4 schemes."""
+    lib = _lib.load()
+    scheme_id = {"k3v2": 32, "k4v4": 44}.get(scheme)
+    _check(scheme_id is not None, f"unknown scheme {scheme!r} (k3v2, k4v4)")
+    kp, vp = (48, 32) if scheme == "k3v2" else (64, 64)
+    q, kd, ks, bt, sl = _stage_a_args(q, k_data, k_scales, block_table, seq_lens, H_q, H_kv, kp)
+    _gpu(v_data, v_scales)
+    _check(v_data.dtype == torch.uint8 and v_data.dim() == 3 and v_data.size(2) == vp, f"v_data last dim must be {vp}")
+    _check(v_scales.dtype == torch.bfloat16, "v_scales must be bf16")
+    vs = (v_scales.unsqueeze(-1) if v_scales.dim() == 2 else v_scales).contiguous()
+    vd = v_data.contiguous()
+    _check(ks.size(2) == vs.size(2), "K and V must use the same group size")
+    gs = HEAD_DIM // ks.size(2)
+    if group_size is not None:
+        _check(int(group_size) == gs, f"group_size={group_size} does not match the scale tensors ({gs})")
+    _check(int(top_k) in SUPPORTED_TOP_K, f"unsupported top_k={top_k}")
+    _check(kd.size(1) == vd.size(1), "K and V caches must have the same number of slots")
+    B = q.size(0)
+    dev = q.device
+    idx = torch.empty((B, H_q, top_k), dtype=torch.int64, device=dev)
+    slots = torch.empty((B, H_q, top_k), dtype=torch.int64, device=dev)
+    o_hat = torch.empty((B, H_q, HEAD_DIM), dtype=torch.float32, device=dev)
+    o_old = torch.empty((B, H_q, HEAD_DIM), dtype=torch.float32, device=dev)
+    W = torch.empty((B, H_q), dtype=torch.float32, device=dev)
+    m = torch.empty((B, H_q), dtype=torch.float32, device=dev) if return_stats else None
+    iz = torch.empty((B, H_q), dtype=torch.float32, device=dev) if return_stats else None
+    scores = torch.empty((B, H_q, max_S), dtype=torch.float32, device=dev) if return_scores else None
+    need = lib.jf_fused_workspace_bytes(scheme_id, B, H_q, H_kv, int(max_S), int(top_k))
+    ws = _workspace(dev, need, "fused")
+    _lib.check(lib.jf_fused_scan_topk(
+        scheme_id, gs, q.data_ptr(), kd.data_ptr(), ks.data_ptr(), vd.data_ptr(), vs.data_ptr(), bt.data_ptr(),
+        sl.data_ptr(), B, H_q, H_kv, int(max_S), bt.size(1), kd.size(1), int(block_size), float(attn_scale), int(top_k),
+        idx.data_ptr(), slots.data_ptr(), o_hat.data_ptr(), o_old.data_ptr(), W.data_ptr(), _ptr(m), _ptr(iz),
+        _ptr(scores), ws.data_ptr(), ws.numel(), _stream(q)))
+    out = [o_hat, slots, o_old, W, idx]
+    if return_stats:
+        out += [m, iz]
+    if return_scores:
+        out.append(scores)
+    return tuple(out)
+
+
+# --------------------------------------------------------------------------- merge
+
+
+def blend_unnorm_into(o_hat, o_old_unnorm, W, o_new, out) -> None:
+    """blend.cu:229-290"""
+    lib = _lib.load()
+    _check(o_hat.is_cuda and o_old_unnorm.is_cuda and W.is_cuda and o_new.is_cuda and out.is_cuda,
+           "blend_unnorm_into: all tensors must be on the GPU")
+    _check(o_hat.dtype == torch.float32 and o_old_unnorm.dtype == torch.float32 and W.dtype == torch.float32,
+           "o_hat / o_old_unnorm / W must be fp32")
+    _check(o_new.dtype == torch.bfloat16 and out.dtype == torch.bfloat16, "o_new / out must be bf16")
+    _check(o_hat.dim() == 3 and o_old_unnorm.dim() == 3 and o_new.dim() == 3 and out.dim() == 3, "tensors must be 3D")
+    _check(W.dim() == 2, "W must be 2D")
+    _check(out.is_contiguous(), "out must be contiguous")
+    hc, oc, wc, nc = o_hat.contiguous(), o_old_unnorm.contiguous(), W.contiguous(), o_new.contiguous()
+    _check(oc.shape == hc.shape and nc.shape == hc.shape and out.shape == hc.shape, "shape mismatch")
+    _check(wc.shape == hc.shape[:2], "W must be (B, H_q)")
+    B, H_q, D = hc.shape
+    _lib.check(lib.jf_blend_unnorm(hc.data_ptr(), oc.data_ptr(), wc.data_ptr(), nc.data_ptr(), out.data_ptr(), B, H_q, D,
+                                   _stream(out)))
+
+
+def blend_unnorm(o_hat, o_old_unnorm, W, o_new) -> torch.Tensor:
+    out = torch.empty_like(o_new)
+    blend_unnorm_into(o_hat, o_old_unnorm, W, o_new, out)
+    return out
+
+
+# --------------------------------------------------------------------------- CPU correction
+
+
+def cpu_topk_attn(q, k_shadow, v_shadow, head_map, ts_buf, o_new, scale, done_flag=None) -> None:
+    """cpu_topk_attn.cpp:854-956: all CPU tensors; synchronous on the calling thread."""
+    lib = _lib.load()
+    for t in (q, k_shadow, v_shadow, head_map, ts_buf, o_new):
+        _check(not t.is_cuda, "cpu_topk_attn: all tensors must be CPU")
+    _check(q.dtype == torch.bfloat16 and k_shadow.dtype == torch.bfloat16 and v_shadow.dtype == torch.bfloat16
+           and o_new.dtype == torch.bfloat16, "q / shadows / o_new must be bf16")
+    _check(head_map.dtype == torch.int64 and ts_buf.dtype == torch.int64, "head_map / ts_buf must be int64")
+    _check(q.dim() == 3 and q.size(2) == HEAD_DIM and k_shadow.dim() == 3 and k_shadow.size(2) == HEAD_DIM,
+           "q must be (B, H_q, 128) and shadows (H_kv, num_slots, 128)")
+    _check(v_shadow.shape == k_shadow.shape, "k_shadow / v_shadow shape mismatch")
+    _check(head_map.shape == ts_buf.shape and ts_buf.dim() == 3 and ts_buf.shape[:2] == q.shape[:2],
+           "head_map / ts_buf must be (B, H_q, K)")
+    _check(o_new.shape == q.shape and o_new.is_contiguous(), "o_new must be contiguous (B, H_q, 128)")
+    for t in (q, k_shadow, v_shadow, head_map, ts_buf):
+        _check(t.is_contiguous(), "cpu_topk_attn: inputs must be contiguous")
+    if done_flag is not None:
+        _check(done_flag.dtype == torch.int64 and done_flag.numel() == 1 and not done_flag.is_cuda,
+               "done_flag must be a 1-element int64 CPU tensor")
+    B, H_q, _ = q.shape
+    _lib.check(lib.jf_cpu_topk_attn(q.data_ptr(), k_shadow.data_ptr(), v_shadow.data_ptr(), head_map.data_ptr(),
+                                    ts_buf.data_ptr(), o_new.data_ptr(), B, H_q, ts_buf.size(2), k_shadow.size(0),
+                                    k_shadow.size(1), float(scale), _ptr(done_flag)))
+
+
+def set_cpu_attn_threads(n: int) -> None:
+    _lib.check(_lib.load().jf_set_cpu_attn_threads(int(n)))
+
+
+def get_cpu_attn_threads() -> int:
+    return int(_lib.load().jf_get_cpu_attn_threads())
+
+
+class CpuTopkHandoff:
+    """Pinned hand-off context (create_cpu_topk_submit_ctx / stream_submit_cpu_topk_attn /
+    stream_wait_cpu_topk_attn in cpu_topk_attn.cpp:2054-2163,2239,2302).  The shadows must stay alive
+    and unmoved for the life of the context."""
+
+    def __init__(self, B, H_q, H_kv, K, k_shadow, v_shadow, scale):
+        lib = _lib.load()
+        _check(not k_shadow.is_cuda and not v_shadow.is_cuda and k_shadow.is_contiguous() and v_shadow.is_contiguous(),
+               "shadows must be contiguous CPU tensors")
+        _check(k_shadow.dtype == torch.bfloat16 and v_shadow.dtype == torch.bfloat16, "shadows must be bf16")
+        _check(k_shadow.shape == v_shadow.shape and k_shadow.size(0) == H_kv and k_shadow.size(2) == HEAD_DIM,
+               "shadows must be (H_kv, num_slots, 128)")
+        self._keep = (k_shadow, v_shadow)
+        self.shape = (B, H_q, K)
+        self._h = lib.jf_handoff_create(B, H_q, H_kv, K, k_shadow.size(1), k_shadow.data_ptr(), v_shadow.data_ptr(),
+                                        float(scale))
+        if not self._h:
+            raise RuntimeError(lib.jf_last_error().decode())
+
+    def submit(self, q, topk_slots) -> None:
+        B, H_q, K = self.shape
+        _check(q.is_cuda and q.dtype == torch.bfloat16 and q.is_contiguous() and q.shape == (B, H_q, HEAD_DIM),
+               "q must be contiguous (B, H_q, 128) bf16 on the GPU")
+        _check(topk_slots.is_cuda and topk_slots.dtype == torch.int64 and topk_slots.is_contiguous()
+               and topk_slots.shape == (B, H_q, K), "topk_slots must be contiguous (B, H_q, K) int64 on the GPU")
+        _lib.check(_lib.load().jf_handoff_submit(self._h, q.data_ptr(), topk_slots.data_ptr(), _stream(q)))
+
+    def wait(self, o_new) -> None:
+        B, H_q, _ = self.shape
+        _check(o_new.is_cuda and o_new.dtype == torch.bfloat16 and o_new.is_contiguous()
+               and o_new.shape == (B, H_q, HEAD_DIM), "o_new must be contiguous (B, H_q, 128) bf16 on the GPU")
+        _lib.check(_lib.load().jf_handoff_wait(self._h, o_new.data_ptr(), _stream(o_new)))
+
+    @property
+    def submit_count(self) -> int:
+        return int(_lib.load().jf_handoff_submit_count(self._h))
+
+    def close(self) -> None:
+        if self._h:
+            _lib.load().jf_handoff_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

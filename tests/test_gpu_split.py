@@ -1,0 +1,280 @@
+"""GPU parity of the split-form operators (pack, Stage A, top-k, Stage B, merge, hand-off) against the
+CPU oracle.  Bit-exact for packed bytes, scale bits, INT4-key scores, top-k indices/slots and the merge;
+fp32 accumulation-order tolerances (the reference's own, scripts/validate_runtime.py:147-195) elsewhere."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import jetfire_oracle as O
+from tests.helpers import bf16_tensor, bf16_to_bits, bf16_to_f32, bits_to_bf16, make_case, to_device
+
+pytestmark = pytest.mark.gpu
+
+GOLD = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_wire_vectors.json")))
+
+
+def ops():
+    from jetfire_amd import ops as _ops
+    return _ops
+
+
+# ------------------------------------------------------------------ pack
+
+
+@pytest.mark.parametrize("gs", GOLD["group_sizes"])
+@pytest.mark.parametrize("vec", GOLD["vectors"], ids=lambda v: f"int{v['bits']}")
+def test_pack_reference_wire_vectors(vec, gs):
+    bits, values, planes = vec["bits"], vec["values"], vec["planes"]
+    x = torch.tensor(values, dtype=torch.bfloat16).repeat(128 // len(values)).view(1, 1, 128).cuda()
+    P = 128 * bits // 8
+    data = torch.zeros(1, 4, P, dtype=torch.uint8, device="cuda")
+    scales = torch.zeros(1, 4, 128 // gs, dtype=torch.bfloat16, device="cuda")
+    getattr(ops(), f"fused_quant_write_int{bits}_sym")(x, torch.tensor([2], device="cuda"), data, scales, gs)
+    repeats = 128 // (8 if bits == 3 else 8 // bits)
+    expected = torch.tensor([b for b in planes for _ in range(repeats)], dtype=torch.uint8)
+    assert torch.equal(data[0, 2].cpu(), expected)
+    assert torch.equal(scales[0, 2].cpu(), torch.ones(128 // gs, dtype=torch.bfloat16))
+    assert int(data[0, [0, 1, 3]].abs().sum()) == 0
+
+
+@pytest.mark.parametrize("bits", (2, 3, 4))
+@pytest.mark.parametrize("gs", (32, 64, 128))
+def test_pack_bit_exact_scatter_masked_and_strided(bits, gs):
+    rng = np.random.default_rng(100 * bits + gs)
+    T, H = 257, 3
+    xn = O.bf16_round((rng.standard_normal((T, H, 128)) * 10 ** rng.uniform(-3, 2, (T, H, 1))).astype(np.float32))
+    xn[..., rng.permutation(128)[:4]] *= 8
+    xn[5] = 0.0                                                   # all-zero rows: scale clamps at 1e-8
+    xn[7, 0, :64] = np.array([0.5, 1.5, 2.5, -0.5] * 16)          # exact ties
+    xn = O.bf16_round(xn)
+    big = torch.zeros(T + 1, H + 1, 256, dtype=torch.bfloat16)
+    big[:T, :H, :128] = bf16_tensor(xn)
+    big[T, :H, :128] = bf16_tensor(xn[0])
+    x = big.cuda()[:, :H, :128]                                   # strided view, last dim contiguous
+    slots_np = np.concatenate([rng.permutation(T), [-1]]).astype(np.int64)
+    P = 128 * bits // 8
+    data = torch.full((H, T + 1, P), 0xA5, dtype=torch.uint8, device="cuda")
+    scales = torch.zeros(H, T + 1, 128 // gs, dtype=torch.bfloat16, device="cuda")
+    getattr(ops(), f"fused_quant_write_int{bits}_sym")(x, torch.from_numpy(slots_np).cuda(), data, scales, gs)
+    ref_d, ref_s = O.quantize_and_pack(xn, gs, bits)              # (T, H, ...)
+    got_d = data.cpu().numpy()[:, slots_np[:T]].transpose(1, 0, 2)
+    got_s = bf16_to_bits(scales)[:, slots_np[:T]].transpose(1, 0, 2)
+    assert np.array_equal(got_s, ref_s)
+    assert np.array_equal(got_d, ref_d)
+    assert bool((data[:, T] == 0xA5).all())                       # the masked token wrote nothing
+
+
+def test_pack_int4_kv_single_launch_matches_two_launches():
+    rng = np.random.default_rng(7)
+    T, H = 70, 8
+    k = bf16_tensor(O.bf16_round(rng.standard_normal((T, H, 128)).astype(np.float32))).cuda()
+    v = bf16_tensor(O.bf16_round(rng.standard_normal((T, H, 128)).astype(np.float32))).cuda()
+    slots = torch.from_numpy(rng.permutation(T + 9)[:T].astype(np.int64)).cuda()
+    mk = lambda: (torch.zeros(H, T + 9, 64, dtype=torch.uint8, device="cuda"),
+                  torch.zeros(H, T + 9, 1, dtype=torch.bfloat16, device="cuda"))
+    kd, ks = mk(); vd, vs = mk(); kd2, ks2 = mk(); vd2, vs2 = mk()
+    ops().fused_quant_write_int4_sym_kv(k, v, slots, kd, ks, vd, vs, 128)
+    ops().fused_quant_write_int4_sym(k, slots, kd2, ks2, 128)
+    ops().fused_quant_write_int4_sym(v, slots, vd2, vs2, 128)
+    assert torch.equal(kd, kd2) and torch.equal(vd, vd2) and torch.equal(ks, ks2) and torch.equal(vs, vs2)
+    ref_d, ref_s = O.quantize_and_pack(bf16_to_f32(v), 128, 4)
+    assert np.array_equal(vd.cpu().numpy()[:, slots.cpu().numpy()].transpose(1, 0, 2), ref_d)
+
+
+def test_pack_rejects_bad_arguments():
+    x = torch.zeros(2, 2, 128, dtype=torch.float16, device="cuda")
+    d = torch.zeros(2, 4, 48, dtype=torch.uint8, device="cuda")
+    s = torch.zeros(2, 4, 2, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(RuntimeError):
+        ops().fused_quant_write_int3_sym(x, torch.zeros(2, dtype=torch.int64, device="cuda"), d, s, 64)
+    with pytest.raises(RuntimeError):
+        ops().fused_quant_write_int3_sym(x.bfloat16(), torch.zeros(2, dtype=torch.int64, device="cuda"), d, s, 48)
+
+
+# ------------------------------------------------------------------ Stage A + top-k
+
+
+CASES_A = [  # (B, Hq, Hkv, S)
+    (2, 8, 2, 512), (3, 32, 8, 300), (2, 32, 4, 272), (1, 8, 2, 17),
+]
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,S", CASES_A)
+@pytest.mark.parametrize("gs", (64, 128))
+def test_int3_scores_and_topk(B, Hq, Hkv, S, gs):
+    c = make_case(11 + S + gs, B, Hq, Hkv, S, 3, 2, gs)
+    d = to_device(c)
+    scale = 128 ** -0.5
+    K = 32 if S < 64 else 64
+    scores, idx, slots = ops().int3_qk_scores_topk(d["q"], d["kd"], d["ks"], d["bt"], d["lens"], S, Hq, Hkv, 16, scale, K)
+    ref = O.scores_bf16_model(c["q"], c["kd"], c["ks"], c["bt"], c["lens"], S, Hq, Hkv, 16, scale, 3, gs)
+    got = scores.cpu().numpy()
+    valid = np.isfinite(ref)
+    assert np.array_equal(np.isneginf(got), ~valid)               # -inf exactly on the padding
+    np.testing.assert_allclose(got[valid], ref[valid], atol=2e-5, rtol=2e-5)   # validate_runtime.py:147-148
+    # top-k is exact on the scores the GPU itself produced, ties to the lower position, ascending order
+    ridx, rslots = O.topk_select(got, c["lens"], c["bt"], S, K)
+    assert np.array_equal(idx.cpu().numpy(), ridx)
+    assert np.array_equal(slots.cpu().numpy(), rslots)
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,S", CASES_A)
+def test_int8tc_scores_bit_exact_topk_and_stats(B, Hq, Hkv, S):
+    c = make_case(21 + S, B, Hq, Hkv, S, 4, 4, 128)
+    d = to_device(c)
+    scale = 128 ** -0.5
+    K = 64
+    scores, idx, slots, m, iz = ops().int8tc_qk_scores_topk_stats(
+        d["q"], d["kd"], d["ks"], d["bt"], d["lens"], S, Hq, Hkv, 16, scale, K)
+    ref = O.scores_int8_model(c["q"], c["kd"], c["ks"], c["bt"], c["lens"], S, Hq, Hkv, 16, scale)
+    got = scores.cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), ref.view(np.uint32))          # integer model: bit-exact
+    ridx, rslots = O.topk_select(ref, c["lens"], c["bt"], S, K)
+    assert np.array_equal(idx.cpu().numpy(), ridx)
+    assert np.array_equal(slots.cpu().numpy(), rslots)
+    rm, riz = O.softmax_stats(ref, c["lens"], S)
+    np.testing.assert_allclose(m.cpu().numpy(), rm, atol=0, rtol=0)
+    np.testing.assert_allclose(iz.cpu().numpy(), riz, rtol=1e-5)
+
+
+def test_topk_ties_short_rows_and_zero_length():
+    rng = np.random.default_rng(3)
+    B, Hq, S, K = 4, 4, 96, 32
+    sc = rng.integers(-2, 3, size=(B, Hq, S)).astype(np.float32)            # heavy ties
+    sc[0, 0, 5], sc[0, 0, 6] = -0.0, 0.0
+    lens = np.array([96, 0, 1, 31], dtype=np.int32)
+    bt = rng.permutation(B * 6).reshape(B, 6).astype(np.int64)
+    from jetfire_amd import _lib
+    lib = _lib.load()
+    t, lens_t, bt_t = torch.from_numpy(sc).cuda(), torch.from_numpy(lens).cuda(), torch.from_numpy(bt).cuda()
+    idx = torch.empty(B, Hq, K, dtype=torch.int64, device="cuda")
+    slots = torch.empty_like(idx)
+    torch.cuda.synchronize()
+    _lib.check(lib.jf_topk_slots(t.data_ptr(), lens_t.data_ptr(), bt_t.data_ptr(), B, Hq, S, 6, 16, K,
+                                 idx.data_ptr(), slots.data_ptr(), None, None, None))   # raw C ABI, default stream
+    torch.cuda.synchronize()
+    ridx, rslots = O.topk_select(sc, lens, bt, S, K)
+    assert np.array_equal(idx.cpu().numpy(), ridx)
+    assert np.array_equal(slots.cpu().numpy(), rslots)
+
+
+def test_topk_large_row_and_k():
+    rng = np.random.default_rng(4)
+    B, Hq, S, K = 1, 2, 40000, 512
+    sc = (rng.standard_normal((B, Hq, S)) * 0.15).astype(np.float32)
+    sc[0, 1, ::3] = np.float32(0.25)                                          # a tie class straddling the cut
+    lens = np.array([39990], dtype=np.int32)
+    bt = rng.permutation(2500).reshape(1, 2500).astype(np.int64)
+    o = ops()
+    idx, slots, _, _ = o._topk(torch.from_numpy(sc).cuda(), torch.from_numpy(bt).cuda(), torch.from_numpy(lens).cuda(),
+                               S, Hq, 16, K, False, "t")
+    ridx, rslots = O.topk_select(sc, lens, bt, S, K)
+    assert np.array_equal(idx.cpu().numpy(), ridx)
+    assert np.array_equal(slots.cpu().numpy(), rslots)
+
+
+def test_unsupported_top_k_raises():
+    c = make_case(1, 1, 8, 2, 64, 3, 2, 64)
+    d = to_device(c)
+    with pytest.raises(RuntimeError, match="unsupported radix-select top_k"):
+        ops().int3_qk_scores_topk(d["q"], d["kd"], d["ks"], d["bt"], d["lens"], 64, 8, 2, 16, 0.1, 48)
+    with pytest.raises(RuntimeError):
+        ops().int3_qk_scores(d["q"].float(), d["kd"], d["ks"], d["bt"], d["lens"], 64, 8, 2, 16, 0.1)
+
+
+# ------------------------------------------------------------------ Stage B + merge
+
+
+@pytest.mark.parametrize("scheme", ("k3v2", "k4v4", "k3v2_g128"))
+@pytest.mark.parametrize("B,Hq,Hkv,lens", [(2, 8, 2, None), (3, 32, 4, [17, 257, 512]), (4, 8, 2, [0, 1, 9, 17])])
+def test_stage_b_outputs(scheme, B, Hq, Hkv, lens):
+    kb, vb, gs = {"k3v2": (3, 2, 64), "k4v4": (4, 4, 128), "k3v2_g128": (3, 2, 128)}[scheme]
+    S = 512 if lens is None or max(lens) > 32 else 32
+    c = make_case(31 + B, B, Hq, Hkv, S, kb, vb, gs, lens=lens)
+    d = to_device(c)
+    scale = 128 ** -0.5
+    K = 64
+    o = ops()
+    if kb == 3:
+        ref_sc = O.scores_bf16_model(c["q"], c["kd"], c["ks"], c["bt"], c["lens"], S, Hq, Hkv, 16, scale, 3, gs)
+    else:
+        ref_sc = O.scores_int8_model(c["q"], c["kd"], c["ks"], c["bt"], c["lens"], S, Hq, Hkv, 16, scale)
+    ridx, _ = O.topk_select(ref_sc, c["lens"], c["bt"], S, K)
+    sc_t, idx_t = torch.from_numpy(ref_sc).cuda(), torch.from_numpy(ridx).cuda()
+    fn = o.int2_softmax_v_with_pre_corr_wvs2 if vb == 2 else o.int4_softmax_v_with_pre_corr_wvs2_scores
+    o_hat, o_old, W = fn(sc_t, d["vd"], d["vs"], d["bt"], d["lens"], idx_t, S, Hq, Hkv, 16, K)
+    r_hat, r_old, r_W = O.softmax_v(ref_sc, c["vd"], c["vs"], c["bt"], c["lens"], ridx, S, Hq, Hkv, 16, vb, gs)
+    np.testing.assert_allclose(o_hat.cpu().numpy(), r_hat, atol=3e-6, rtol=3e-6)     # validate_runtime.py:173-177
+    np.testing.assert_allclose(o_old.cpu().numpy(), r_old, atol=3e-6, rtol=3e-6)
+    np.testing.assert_allclose(W.cpu().numpy(), r_W, atol=3e-6, rtol=3e-6)
+    if vb == 4:                                                   # the variant that is handed Stage-A statistics
+        m, iz = O.softmax_stats(ref_sc, c["lens"], S)
+        o2 = o.int8tc_softmax_v_with_pre_corr_reg_stats(sc_t, torch.from_numpy(m).cuda(), torch.from_numpy(iz).cuda(),
+                                                        d["vd"], d["vs"], d["bt"], d["lens"], idx_t, S, Hq, Hkv, 16, K)
+        np.testing.assert_allclose(o2[0].cpu().numpy(), r_hat, atol=3e-6, rtol=3e-6)
+        if lens is None:   # long rows: within the reference's own int8-P tolerance (validate_runtime.py:173-176);
+            # on short peaked rows the int8-P approximation itself strays further (validate_runtime_edges.py:146-152)
+            t_hat, _, _ = O.softmax_v_int8_tiles(ref_sc, m, iz, c["vd"], c["vs"], c["bt"], c["lens"], ridx, S, Hq, Hkv, 16)
+            np.testing.assert_allclose(o2[0].cpu().numpy(), t_hat, atol=3e-3)
+
+
+def test_blend_bit_exact():
+    rng = np.random.default_rng(8)
+    hat = rng.standard_normal((3, 8, 128)).astype(np.float32)
+    old = (rng.standard_normal((3, 8, 128)) * 0.3).astype(np.float32)
+    W = rng.uniform(0, 1, (3, 8)).astype(np.float32)
+    new = O.bf16_round(rng.standard_normal((3, 8, 128)).astype(np.float32))
+    out = torch.empty(3, 8, 128, dtype=torch.bfloat16, device="cuda")
+    ops().blend_unnorm_into(torch.from_numpy(hat).cuda(), torch.from_numpy(old).cuda(), torch.from_numpy(W).cuda(),
+                            bf16_tensor(new).cuda(), out)
+    ref = O.blend_unnorm(hat, old, W, new)
+    assert np.array_equal(bf16_to_bits(out), O.f32_to_bf16_bits(ref))
+
+
+# ------------------------------------------------------------------ end-to-end split pipeline with the pinned hand-off
+
+
+@pytest.mark.parametrize("scheme,B,Hq,Hkv,lens,K", [
+    ("k3v2", 2, 8, 2, None, 256), ("k4v4", 2, 8, 2, None, 256),
+    ("k3v2", 3, 32, 4, [17, 257, 512], 256), ("k4v4", 4, 8, 2, [0, 1, 9, 17], 64),
+])
+def test_split_pipeline_with_handoff(scheme, B, Hq, Hkv, lens, K):
+    kb, vb, gs = (3, 2, 64) if scheme == "k3v2" else (4, 4, 128)
+    S = 512 if lens is None or max(lens) > 32 else 32
+    c = make_case(41 + B, B, Hq, Hkv, S, kb, vb, gs, lens=lens)
+    d = to_device(c)
+    o = ops()
+    scale = 128 ** -0.5
+    ksh, vsh = bf16_tensor(c["K"]), bf16_tensor(c["V"])
+    o.set_cpu_attn_threads(4)
+    h = o.CpuTopkHandoff(B, Hq, Hkv, K, ksh, vsh, scale)
+    out = torch.empty(B, Hq, 128, dtype=torch.bfloat16, device="cuda")
+    o_new = torch.empty_like(out)
+    for rep in range(2):                                          # the context is reusable
+        if scheme == "k3v2":
+            scores, idx, slots = o.int3_qk_scores_topk(d["q"], d["kd"], d["ks"], d["bt"], d["lens"], S, Hq, Hkv, 16, scale, K)
+        else:
+            scores, idx, slots, m, iz = o.int8tc_qk_scores_topk_stats(d["q"], d["kd"], d["ks"], d["bt"], d["lens"], S,
+                                                                      Hq, Hkv, 16, scale, K)
+        h.submit(d["q"], slots)
+        if scheme == "k3v2":
+            o_hat, o_old, W = o.int2_softmax_v_with_pre_corr_wvs2(scores, d["vd"], d["vs"], d["bt"], d["lens"], idx, S,
+                                                                  Hq, Hkv, 16, K)
+        else:
+            o_hat, o_old, W = o.int4_softmax_v_with_pre_corr_wvs2_scores(scores, d["vd"], d["vs"], d["bt"], d["lens"],
+                                                                         idx, S, Hq, Hkv, 16, K)
+        h.wait(o_new)
+        o.blend_unnorm_into(o_hat, o_old, W, o_new, out)
+        torch.cuda.synchronize()
+    assert h.submit_count == 2
+    r = O.decode_reference(c["q"], c["kd"], c["ks"], c["vd"], c["vs"], c["bt"], c["lens"], S, Hq, Hkv, 16, scale, K,
+                           scheme, c["K"], c["V"])
+    np.testing.assert_allclose(bf16_to_f32(o_new), r["o_new"], atol=2e-3, rtol=6e-3)          # validate_runtime.py:191
+    got = bf16_to_f32(out)
+    np.testing.assert_allclose(got, r["out"], atol=6e-3, rtol=1.5e-2)                         # validate_runtime.py:195
+    err = np.abs(got - r["out"])
+    assert err.max() <= 2e-2 and err.mean() <= 1e-3               # the acceptance bar for attention outputs
+    h.close()
