@@ -1,0 +1,155 @@
+"""GPU parity of the fused decode scan + top-k (and of the whole fused decode step with the CPU
+correction hand-off and the merge) against the CPU oracle, through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import jetfire_oracle as O
+from tests.helpers import bf16_tensor, bf16_to_f32, make_case, to_device
+
+pytestmark = pytest.mark.gpu
+
+SCALE = 128 ** -0.5
+
+
+def ops():
+    from jetfire_amd import ops as _ops
+    return _ops
+
+
+def run_fused(scheme, c, d, S, K):
+    o = ops()
+    return o.fused_attn_topk(scheme.split("_")[0], d["q"], d["kd"], d["ks"], d["vd"], d["vs"], d["bt"], d["lens"], S,
+                             c["Hq"], c["Hkv"], 16, K, SCALE, return_scores=True, return_stats=True)
+
+
+def check_against_oracle(scheme, c, S, K, out):
+    o_hat, slots, o_old, W, idx, m, iz, scores = [t.cpu().numpy() for t in out]
+    kb, vb, gs = c["kbits"], c["vbits"], c["gs"]
+    Hq, Hkv = c["Hq"], c["Hkv"]
+    if kb == 3:
+        ref_sc = O.scores_bf16_model(c["q"], c["kd"], c["ks"], c["bt"], c["lens"], S, Hq, Hkv, 16, SCALE, 3, gs)
+        valid = np.isfinite(ref_sc)
+        assert np.array_equal(np.isneginf(scores), ~valid)
+        np.testing.assert_allclose(scores[valid], ref_sc[valid], atol=2e-5, rtol=2e-5)
+    else:
+        ref_sc = O.scores_int8_model(c["q"], c["kd"], c["ks"], c["bt"], c["lens"], S, Hq, Hkv, 16, SCALE)
+        assert np.array_equal(scores.view(np.uint32), ref_sc.view(np.uint32))
+    # top-k: exact on the kernel's own scores (and therefore on the oracle's when those are bit-equal)
+    ridx, rslots = O.topk_select(scores, c["lens"], c["bt"], S, K)
+    assert np.array_equal(idx, ridx)
+    assert np.array_equal(slots, rslots)
+    # every oracle winner whose margin to the cut exceeds the score tolerance must be selected
+    oidx, _ = O.topk_select(ref_sc, c["lens"], c["bt"], S, K)
+    for b in range(c["B"]):
+        n = min(S, int(c["lens"][b]))
+        if n <= K:
+            continue
+        for h in range(Hq):
+            cut = np.sort(ref_sc[b, h, :n])[-K]
+            clear = [i for i in oidx[b, h] if ref_sc[b, h, i] > cut + 5e-5]
+            assert set(clear) <= set(idx[b, h].tolist())
+    rm, riz = O.softmax_stats(scores, c["lens"], S)
+    np.testing.assert_allclose(m, rm, atol=1e-7)
+    np.testing.assert_allclose(iz, riz, rtol=2e-5)
+    r_hat, r_old, r_W = O.softmax_v(scores, c["vd"], c["vs"], c["bt"], c["lens"], idx, S, Hq, Hkv, 16, vb, gs)
+    np.testing.assert_allclose(o_hat, r_hat, atol=3e-6, rtol=2e-5)
+    np.testing.assert_allclose(o_old, r_old, atol=3e-6, rtol=2e-5)
+    np.testing.assert_allclose(W, r_W, atol=3e-6, rtol=2e-5)
+    return ref_sc
+
+
+CASES = [
+    # scheme, B, Hq, Hkv, S, lens, K
+    ("k3v2", 2, 8, 2, 512, None, 64),
+    ("k4v4", 2, 8, 2, 512, None, 64),
+    ("k3v2", 3, 32, 4, 512, [17, 257, 512], 256),          # G=8, short rows (reference edge geometry)
+    ("k4v4", 3, 32, 4, 512, [17, 257, 512], 256),
+    ("k3v2", 4, 8, 2, 32, [0, 1, 9, 17], 32),             # S < K, zero-length row
+    ("k4v4", 4, 8, 2, 32, [0, 1, 9, 17], 64),
+    ("k3v2", 1, 8, 2, 5000, [4987], 256),                 # many splits, ragged tail
+    ("k4v4", 1, 8, 2, 5000, [4987], 512),
+    ("k3v2_g128", 2, 8, 2, 700, None, 128),               # INT3/INT2 with one scale group
+    ("k3v2", 1, 4, 4, 300, None, 32),                     # G=1
+    ("k4v4", 1, 4, 2, 300, None, 64),                     # G=2
+    ("k3v2", 1, 16, 1, 600, None, 64),                    # G=16
+    ("k4v4", 1, 16, 1, 600, None, 64),
+]
+
+
+@pytest.mark.parametrize("scheme,B,Hq,Hkv,S,lens,K", CASES)
+def test_fused_scan_matches_oracle(scheme, B, Hq, Hkv, S, lens, K):
+    kb, vb, gs = {"k3v2": (3, 2, 64), "k4v4": (4, 4, 128), "k3v2_g128": (3, 2, 128)}[scheme]
+    c = make_case(70 + S + Hq, B, Hq, Hkv, S, kb, vb, gs, lens=lens, extra_blocks=3)
+    d = to_device(c)
+    out = run_fused(scheme, c, d, S, K)
+    check_against_oracle(scheme, c, S, K, out)
+
+
+def test_fused_scan_ties_go_to_the_lower_position():
+    # identical keys in every slot -> every score of a head is equal: winners are positions 0..K-1
+    c = make_case(5, 1, 8, 2, 600, 3, 2, 64, ragged=False, shuffle=True)
+    c["kd"][:] = c["kd"][:, :1]
+    c["ks"][:] = c["ks"][:, :1]
+    d = to_device(c)
+    out = run_fused("k3v2", c, d, 600, 64)
+    idx = out[4].cpu().numpy()
+    assert (idx == np.arange(64)[None, None, :]).all()
+
+
+def test_fused_scan_is_deterministic_and_matches_split_path():
+    c = make_case(6, 2, 32, 8, 2048, 3, 2, 64)
+    d = to_device(c)
+    o = ops()
+    a = run_fused("k3v2", c, d, 2048, 256)
+    b2 = run_fused("k3v2", c, d, 2048, 256)
+    for x, y in zip(a, b2):
+        assert torch.equal(x, y)
+    scores, idx, slots = o.int3_qk_scores_topk(d["q"], d["kd"], d["ks"], d["bt"], d["lens"], 2048, 32, 8, 16, SCALE, 256)
+    o_hat, o_old, W = o.int2_softmax_v_with_pre_corr_wvs2(scores, d["vd"], d["vs"], d["bt"], d["lens"], idx, 2048, 32, 8, 16, 256)
+    np.testing.assert_allclose(a[7].cpu().numpy(), scores.cpu().numpy(), atol=2e-5, rtol=2e-5)
+    np.testing.assert_allclose(a[0].cpu().numpy(), o_hat.cpu().numpy(), atol=3e-6, rtol=2e-5)
+
+
+@pytest.mark.parametrize("scheme,B,Hq,Hkv,S,lens,K", [
+    ("k3v2", 2, 32, 8, 1024, None, 256),
+    ("k4v4", 2, 32, 8, 1024, None, 256),
+    ("k3v2", 2, 32, 4, 768, [700, 768], 256),             # the TP2 70B local-head geometry
+    ("k4v4", 4, 8, 2, 32, [0, 1, 9, 17], 64),
+])
+def test_fused_decode_step_end_to_end(scheme, B, Hq, Hkv, S, lens, K):
+    """scan+top-k -> pinned hand-off -> CPU correction -> merge, checked against the oracle's whole step and the
+    acceptance bar for attention outputs (max-abs 2e-2, mean-abs 1e-3 in bf16)."""
+    kb, vb, gs = (3, 2, 64) if scheme == "k3v2" else (4, 4, 128)
+    c = make_case(80 + B + Hq, B, Hq, Hkv, S, kb, vb, gs, lens=lens)
+    d = to_device(c)
+    o = ops()
+    o.set_cpu_attn_threads(4)
+    h = o.CpuTopkHandoff(B, Hq, Hkv, K, bf16_tensor(c["K"]), bf16_tensor(c["V"]), SCALE)
+    out = torch.empty(B, Hq, 128, dtype=torch.bfloat16, device="cuda")
+    o_new = torch.empty_like(out)
+    o_hat, slots, o_old, W, idx = o.fused_attn_topk(scheme, d["q"], d["kd"], d["ks"], d["vd"], d["vs"], d["bt"],
+                                                    d["lens"], S, Hq, Hkv, 16, K, SCALE)
+    h.submit(d["q"], slots)
+    h.wait(o_new)
+    o.blend_unnorm_into(o_hat, o_old, W, o_new, out)
+    torch.cuda.synchronize()
+    r = O.decode_reference(c["q"], c["kd"], c["ks"], c["vd"], c["vs"], c["bt"], c["lens"], S, Hq, Hkv, 16, SCALE, K,
+                           scheme, c["K"], c["V"])
+    got = bf16_to_f32(out)
+    np.testing.assert_allclose(got, r["out"], atol=6e-3, rtol=1.5e-2)
+    err = np.abs(got - r["out"])
+    assert err.max() <= 2e-2 and err.mean() <= 1e-3
+    h.close()
+
+
+def test_fused_scan_rejects_unsupported_arguments():
+    c = make_case(9, 1, 8, 2, 64, 3, 2, 64)
+    d = to_device(c)
+    o = ops()
+    with pytest.raises(RuntimeError):
+        o.fused_attn_topk("k3v2", d["q"], d["kd"], d["ks"], d["vd"], d["vs"], d["bt"], d["lens"], 64, 8, 2, 16, 48, SCALE)
+    with pytest.raises(RuntimeError):
+        o.fused_attn_topk("k3v2", d["q"], d["kd"], d["ks"], d["vd"], d["vs"], d["bt"], d["lens"], 64, 8, 2, 32, 64, SCALE)
+    with pytest.raises(RuntimeError):
+        o.fused_attn_topk("k9", d["q"], d["kd"], d["ks"], d["vd"], d["vs"], d["bt"], d["lens"], 64, 8, 2, 16, 64, SCALE)
