@@ -1,0 +1,173 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused decode scan + top-k on one MI355X.
+
+A step is one decode step of the attention path over all layers of the workload: per layer the fused
+scan (packed K and V streamed once from HBM), the top-k merge kernel and the GPU-side blend, on distinct
+per-layer caches that are resident in HBM before the timed region (together far larger than the caches,
+so no layer is served from L2 / Infinity Cache left by the previous step).
+
+Prints ONE JSON line (see --help for the workload choices).  `value` is packed KV bytes per second over
+the whole step; `roofline` is for the dominant kernel (fused_scan_kernel), its device time measured with
+HIP events recorded around every launch inside the timed region; `cpu_baseline` is the reference's
+PyTorch CPU path (unpack + dequant + attention + top-k) restated in oracle/torch_cpu_path.py, timed on
+this box's host cores on a bounded sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def cpu_baseline(w, budget_s: float = 20.0):
+    """Time the torch CPU path on sequence 0 / layer 0 of the workload (all kv heads, full context)."""
+    import torch
+    from oracle import torch_cpu_path as T
+    S, Hkv, gs = w.S, w.H_kv, w.group
+    kb, vb = (3, 2) if w.scheme == "k3v2" else (4, 4)
+    lay = w.layers[0]
+    # sequence 0 occupies slots [0, S) with the identity block table
+    kd = lay.k_data[:, :S].cpu().unsqueeze(0)
+    ks = lay.k_scales[:, :S].cpu().unsqueeze(0)
+    vd = lay.v_data[:, :S].cpu().unsqueeze(0)
+    vs = lay.v_scales[:, :S].cpu().unsqueeze(0)
+    q = w.q[:1].cpu()
+    threads = torch.get_num_threads()
+    T.decode_path(q, kd, ks, vd, vs, gs, kb, vb, w.top_k)                 # warm-up
+    times = []
+    t_start = time.perf_counter()
+    while len(times) < 5 and (time.perf_counter() - t_start) < budget_s:
+        t0 = time.perf_counter()
+        T.decode_path(q, kd, ks, vd, vs, gs, kb, vb, w.top_k)
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    sample_bytes = Hkv * S * (w.packed_bytes_per_layer // (w.B * w.H_kv * w.S))
+    return {
+        "value": round(sample_bytes / med / 1e9, 4), "unit": "GB/s", "cores": threads, "kind": "port",
+        "sample": f"1 of {w.B} sequences x {Hkv} kv-heads x {S} positions of one layer ({sample_bytes / 1e6:.1f} MB packed), "
+                  f"median of {len(times)} runs, {med * 1e3:.1f} ms per run",
+        "ms_per_layer_equiv": round(med * w.B * 1e3, 2),
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4", "c5"],
+                    help="c2: Llama-3.1-8B B4 S32768 K3V2 k256 x32 layers (the headline); c3: B1 S131072 K4V4 k512; "
+                         "c4: Qwen3-30B-A3B B4 GQA8 K3V2 x48; c5: Llama-3.3-70B TP2 shard B2 S65536 K3V2 x80")
+    ap.add_argument("--layers", type=int, default=None, help="override the number of distinct layer caches")
+    ap.add_argument("--paged", action="store_true", help="random block table instead of the identity mapping")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--graph", action="store_true", help="replay the step from a HIP graph (roofline timing stays eager)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this path runs on ONE GPU (no sharding, no collectives); --gpus must be 1", file=sys.stderr)
+        return 2
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 2
+    from jetfire_amd import _lib, ops, workloads
+
+    lib = _lib.load()
+    torch.cuda.set_device(0)
+    w = workloads.build(args.workload, n_layers=args.layers)
+    n_layers = len(w.layers)
+    o_new = torch.zeros(w.B, w.H_q, 128, dtype=torch.bfloat16, device="cuda")
+    out = torch.empty_like(o_new)
+
+    def step():
+        for lay in w.layers:
+            o_hat, slots, o_old, W, idx = ops.fused_attn_topk(
+                w.scheme, w.q, lay.k_data, lay.k_scales, lay.v_data, lay.v_scales, w.block_table, w.seq_lens,
+                w.S, w.H_q, w.H_kv, 16, w.top_k, w.attn_scale)
+            ops.blend_unnorm_into(o_hat, o_old, W, o_new, out)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+
+    graph = None
+    if args.graph:
+        graph = torch.cuda.CUDAGraph()
+        s = torch.cuda.Stream()
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            step()
+        torch.cuda.current_stream().wait_stream(s)
+        with torch.cuda.graph(graph, stream=s):
+            step()
+        graph.replay()
+        torch.cuda.synchronize()
+
+    # ---- timed region (whole-job throughput), with HIP events around every scan-kernel launch when eager
+    total_ms = ctypes.c_double(0.0)
+    launches = ctypes.c_int(0)
+    if graph is None:
+        _lib.check(lib.jf_profile_scan_begin(args.steps * n_layers))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        if graph is not None:
+            graph.replay()
+        else:
+            step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    if graph is None:
+        _lib.check(lib.jf_profile_scan_end(ctypes.byref(total_ms), ctypes.byref(launches)))
+    else:   # kernel time from a separate eager pass
+        _lib.check(lib.jf_profile_scan_begin(n_layers * 3))
+        for _ in range(3):
+            step()
+        torch.cuda.synchronize()
+        _lib.check(lib.jf_profile_scan_end(ctypes.byref(total_ms), ctypes.byref(launches)))
+
+    ms_per_step = elapsed / args.steps * 1e3
+    bytes_layer = w.packed_bytes_per_layer
+    value = bytes_layer * n_layers / (ms_per_step * 1e-3) / 1e9
+    scan_us = total_ms.value / max(1, launches.value) * 1e3
+    achieved = bytes_layer / (scan_us * 1e-6) / 1e9 if scan_us > 0 else 0.0
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", f"fused_scan_{w.scheme}_{args.workload}_traffic.json")
+    if os.path.exists(tpath):
+        try:
+            traffic = json.load(open(tpath)).get("traffic_bytes_per_launch")
+        except Exception:
+            traffic = None
+
+    res = {
+        "metric": "decode-scan HBM GB/s on packed KV (fused scan + top-k + merge, all layers of one decode step)",
+        "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "us_per_layer": round(ms_per_step * 1e3 / n_layers, 2),
+        "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u8 codes; int8/bf16 MFMA, fp32 softmax", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: B{w.B} Hq{w.H_q} Hkv{w.H_kv} D128 S{w.S} {w.scheme} g{w.group} "
+                               f"top_k{w.top_k} x{n_layers} layers, {'paged (random)' if args.paged else 'identity'} block table",
+                   "packed_bytes_per_layer": bytes_layer, "launch": "hip-graph" if graph is not None else "eager"},
+        "roofline": {"bound": "hbm", "kernel": "fused_scan_kernel", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
+                     "kernel_us": round(scan_us, 2), "launches_timed": launches.value},
+    }
+    if not args.no_cpu_baseline:
+        res["cpu_baseline"] = cpu_baseline(w)
+    print(json.dumps(res))
+    return 0
+
+
+if __name__ == "__main__":
+    raise SystemExit(main())

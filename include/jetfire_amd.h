@@ -135,6 +135,12 @@ int jf_fused_scan_topk(int scheme, int group_size,
                        float* softmax_m, float* softmax_inv_z, float* scores,
                        void* workspace, size_t workspace_bytes, void* stream);
 
+/* Measurement aid with no counterpart in the reference: between begin and end, every launch of the fused
+ * scan kernel is bracketed by a pair of HIP events recorded on the launch stream (at most max_launches
+ * launches); end synchronises them and returns the summed device time and the number of launches. */
+int jf_profile_scan_begin(int max_launches);
+int jf_profile_scan_end(double* total_ms, int* launches);
+
 /* ------------------------------------------------------------------ piece 4: merge
  * out = bf16_rne(fma(W, f32(o_new), o_hat) - o_old_unnorm).  Replaces blend_unnorm_into
  * (jetfire_vllm/csrc/blend.cu:202-290).  o_new / out are (B, H_q, D) bf16. */

@@ -7,8 +7,8 @@
 //            INT3 keys: K-hat = bf16((code-4)*scale) built in registers, v_mfma_f32_16x16x32_bf16 with the
 //                       tokens on the N side; the four 16-token tiles of a wavefront land one per
 //                       16-lane group, so lane l ends up holding the G scores of token l.
-//            INT4 keys: int8-quantised Q, exact nibble codes, v_dot4_i32_i8, fp32 rescale (bit-exact
-//                       with the split-form kernel and the CPU oracle).
+//            INT4 keys: int8-quantised Q, exact nibble codes, v_dot4_i32_i8, fp32 rescale (every step
+//                       is exactly reproducible, so it is bit-equal to the split-form kernel).
 //   phase B  P.V on v_mfma_i32_16x16x64_i8.  p = exp(s - m_split) is known exactly because phase A is
 //            complete, so w = p * v_scale is converted to 22-bit fixed point once (fma with 2^23), its
 //            three bytes are the A-operand rows (limb, head), and the int32 accumulators live for the whole
@@ -23,6 +23,8 @@
 // (the split-KV combine of jetfire_vllm/csrc/fused_decode_wmma.cu:1226-1253), and computes the
 // pre-correction terms o_old_unnorm, W over the winners (jetfire_vllm/csrc/int2_softmax_v.cu:738-788).
 #include "common.h"
+
+#include <vector>
 
 namespace jf {
 namespace {
@@ -766,6 +768,15 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   if (tid == 0) p.W[bh] = comb[2 * D] + comb[2 * D + 1];
 }
 
+// Optional measurement hook: when armed, every fused_scan_kernel launch is bracketed by a pair of HIP
+// events on its own stream, so a benchmark can read the kernel's device time without a profiler.
+struct ScanProfile {
+  std::vector<hipEvent_t> ev;
+  int used = 0;
+  bool armed = false;
+};
+ScanProfile g_prof;
+
 inline int lmax_for_group(int G) { return G <= 4 ? 2048 : (G <= 8 ? 1024 : 512); }
 
 inline void fused_plan(int B, int H_q, int H_kv, int max_S, int top_k, int* L_out, int* ns_out, int* kc_out) {
@@ -815,9 +826,19 @@ int launch_scan(const FusedParams& p, hipStream_t st) {
   if (!K3 && qsz > stage) stage = qsz;
   const size_t smem = (size_t)G * p.L * sizeof(float) + stage;
   auto kern = fused_scan_kernel<SCHEME, G, NG>;
-  JF_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+  static size_t attr_smem = 0;  // per instantiation: raise the dynamic-LDS limit only when it grows
+  if (smem > attr_smem) {
+    JF_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    attr_smem = smem;
+  }
+  const bool prof = g_prof.armed && g_prof.used + 2 <= (int)g_prof.ev.size();
+  if (prof) JF_CHECK_HIP(hipEventRecord(g_prof.ev[g_prof.used], st));
   hipLaunchKernelGGL(kern, dim3(p.n_splits, p.H_kv, p.B), dim3(FS_THREADS), smem, st, p);
   JF_CHECK_LAUNCH();
+  if (prof) {
+    JF_CHECK_HIP(hipEventRecord(g_prof.ev[g_prof.used + 1], st));
+    g_prof.used += 2;
+  }
   return JF_OK;
 }
 
@@ -917,5 +938,33 @@ extern "C" int jf_fused_scan_topk(int scheme, int group_size, const uint16_t* q,
     hipLaunchKernelGGL((fused_merge_kernel<4, 1>), mgrid, mblock, 0, st, p);
   }
   JF_CHECK_LAUNCH();
+  return JF_OK;
+}
+
+extern "C" int jf_profile_scan_begin(int max_launches) {
+  JF_CHECK_ARG(max_launches > 0 && max_launches <= (1 << 20), "profile_scan_begin: bad max_launches=%d", max_launches);
+  for (hipEvent_t e : g_prof.ev) (void)hipEventDestroy(e);
+  g_prof.ev.assign((size_t)max_launches * 2, nullptr);
+  for (auto& e : g_prof.ev) JF_CHECK_HIP(hipEventCreate(&e));
+  g_prof.used = 0;
+  g_prof.armed = true;
+  return JF_OK;
+}
+
+extern "C" int jf_profile_scan_end(double* total_ms, int* launches) {
+  JF_CHECK_ARG(total_ms && launches, "profile_scan_end: null output");
+  g_prof.armed = false;
+  double tot = 0.0;
+  for (int i = 0; i + 1 < g_prof.used; i += 2) {
+    JF_CHECK_HIP(hipEventSynchronize(g_prof.ev[i + 1]));
+    float ms = 0.f;
+    JF_CHECK_HIP(hipEventElapsedTime(&ms, g_prof.ev[i], g_prof.ev[i + 1]));
+    tot += ms;
+  }
+  *total_ms = tot;
+  *launches = g_prof.used / 2;
+  for (hipEvent_t e : g_prof.ev) (void)hipEventDestroy(e);
+  g_prof.ev.clear();
+  g_prof.used = 0;
   return JF_OK;
 }

@@ -1,0 +1,103 @@
+"""Synthetic decode workloads at the benchmark shapes: seeded K/V (bf16 N(0,1), four key channels
+scaled x8 as outliers), q ~ N(0,1)/sqrt(128), quantised on the GPU with the library's own
+quantise-on-append kernels into the reference cache layout, one cache per layer."""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import List
+
+import torch
+
+from . import ops
+
+HEAD_DIM = 128
+BLOCK = 16
+
+# name: (B, H_q, H_kv, S, scheme, group, top_k, layers)
+CONFIGS = {
+    "c1": (1, 32, 8, 4096, "k4v4", 128, 64, 1),
+    "c2": (4, 32, 8, 32768, "k3v2", 64, 256, 32),
+    "c3": (1, 32, 8, 131072, "k4v4", 128, 512, 32),
+    "c4": (4, 32, 4, 32768, "k3v2", 64, 256, 48),
+    "c5": (2, 32, 4, 65536, "k3v2", 64, 512, 80),
+}
+BYTES_PER_TOKEN_HEAD = {"k3v2": {64: 88, 128: 84}, "k4v4": {128: 132, 64: 136}}
+
+
+@dataclass
+class LayerCache:
+    k_data: torch.Tensor
+    k_scales: torch.Tensor
+    v_data: torch.Tensor
+    v_scales: torch.Tensor
+
+
+@dataclass
+class Workload:
+    name: str
+    B: int
+    H_q: int
+    H_kv: int
+    S: int
+    scheme: str
+    group: int
+    top_k: int
+    layers: List[LayerCache]
+    q: torch.Tensor
+    block_table: torch.Tensor
+    seq_lens: torch.Tensor
+    attn_scale: float
+
+    @property
+    def packed_bytes_per_layer(self) -> int:
+        return self.B * self.H_kv * self.S * BYTES_PER_TOKEN_HEAD[self.scheme][self.group]
+
+
+def build(name: str, n_layers: int | None = None, seed: int = 0, paged: bool = False, device: str = "cuda",
+          keep_shadow: bool = False) -> Workload:
+    B, Hq, Hkv, S, scheme, gs, top_k, layers = CONFIGS[name]
+    if n_layers is not None:
+        layers = n_layers
+    dev = torch.device(device)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(seed)
+    cpu_gen = torch.Generator().manual_seed(seed)
+    outliers = torch.randperm(HEAD_DIM, generator=cpu_gen)[:4].to(dev)
+    T = B * S
+    nblk = T // BLOCK
+    if paged:
+        perm = torch.randperm(nblk, generator=cpu_gen)
+    else:
+        perm = torch.arange(nblk)
+    block_table = perm.reshape(B, S // BLOCK).to(torch.int64).to(dev)
+    pos = torch.arange(S, device=dev)
+    slots = (block_table[:, pos // BLOCK] * BLOCK + pos % BLOCK).reshape(-1)      # token t = b*S + pos
+    kb, vb = (3, 2) if scheme == "k3v2" else (4, 4)
+    caches = []
+    shadows = []
+    for _ in range(layers):
+        k = torch.randn(T, Hkv, HEAD_DIM, generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16)
+        k[..., outliers] *= 8
+        v = torch.randn(T, Hkv, HEAD_DIM, generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16)
+        kd = torch.empty(Hkv, T, HEAD_DIM * kb // 8, dtype=torch.uint8, device=dev)
+        ks = torch.empty(Hkv, T, HEAD_DIM // gs, dtype=torch.bfloat16, device=dev)
+        vd = torch.empty(Hkv, T, HEAD_DIM * vb // 8, dtype=torch.uint8, device=dev)
+        vs = torch.empty(Hkv, T, HEAD_DIM // gs, dtype=torch.bfloat16, device=dev)
+        if scheme == "k3v2":
+            ops.fused_quant_write_int3_sym(k, slots, kd, ks, gs)
+            ops.fused_quant_write_int2_sym(v, slots, vd, vs, gs)
+        else:
+            ops.fused_quant_write_int4_sym_kv(k, v, slots, kd, ks, vd, vs, gs)
+        caches.append(LayerCache(kd, ks, vd, vs))
+        if keep_shadow:
+            ksh = torch.empty(Hkv, T, HEAD_DIM, dtype=torch.bfloat16)
+            vsh = torch.empty(Hkv, T, HEAD_DIM, dtype=torch.bfloat16)
+            ksh[:, slots.cpu()] = k.permute(1, 0, 2).cpu()
+            vsh[:, slots.cpu()] = v.permute(1, 0, 2).cpu()
+            shadows.append((ksh, vsh))
+        del k, v
+    q = (torch.randn(B, Hq, HEAD_DIM, generator=gen, device=dev, dtype=torch.float32) / HEAD_DIM ** 0.5).to(torch.bfloat16)
+    seq_lens = torch.full((B,), S, dtype=torch.int32, device=dev)
+    w = Workload(name, B, Hq, Hkv, S, scheme, gs, top_k, caches, q, block_table, seq_lens, HEAD_DIM ** -0.5)
+    w.shadows = shadows
+    return w
