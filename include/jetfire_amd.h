@@ -140,6 +140,10 @@ int jf_fused_scan_topk(int scheme, int group_size,
  * launches); end synchronises them and returns the summed device time and the number of launches. */
 int jf_profile_scan_begin(int max_launches);
 int jf_profile_scan_end(double* total_ms, int* launches);
+/* Measurement aid: if device_buffer is non-NULL, every fused-scan workgroup stores six s_memtime stamps
+ * (start, after Q.K^T, after the V-scale pass, after P.V, after the partial reduction, end) at
+ * device_buffer[((b * H_kv + hkv) * n_splits + split) * 6 ...] as int64.  NULL switches it off. */
+int jf_debug_phase_clock(void* device_buffer);
 
 /* ------------------------------------------------------------------ piece 4: merge
  * out = bf16_rne(fma(W, f32(o_new), o_hat) - o_old_unnorm).  Replaces blend_unnorm_into

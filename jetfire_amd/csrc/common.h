@@ -56,19 +56,52 @@ __device__ __host__ inline uint32_t score_key(float f) {
   return (v.u & 0x80000000u) ? ~v.u : (v.u | 0x80000000u);
 }
 
+// Wavefront-wide reductions and scans on the DPP network (row shifts inside 16-lane rows, then the two
+// row broadcasts), no LDS traffic.  After the sequence lane 63 holds the reduction over all 64 lanes.
+template <int CTRL, int ROW_MASK>
+__device__ inline int dpp_mov(int old, int v) {
+  return __builtin_amdgcn_update_dpp(old, v, CTRL, ROW_MASK, 0xf, false);
+}
+#define JF_DPP_REDUCE(v, OP, T, IDENT)                                                               \
+  do {                                                                                               \
+    v = OP(v, __builtin_bit_cast(T, dpp_mov<0x111, 0xf>(__builtin_bit_cast(int, (T)(IDENT)), __builtin_bit_cast(int, v)))); \
+    v = OP(v, __builtin_bit_cast(T, dpp_mov<0x112, 0xf>(__builtin_bit_cast(int, (T)(IDENT)), __builtin_bit_cast(int, v)))); \
+    v = OP(v, __builtin_bit_cast(T, dpp_mov<0x114, 0xf>(__builtin_bit_cast(int, (T)(IDENT)), __builtin_bit_cast(int, v)))); \
+    v = OP(v, __builtin_bit_cast(T, dpp_mov<0x118, 0xf>(__builtin_bit_cast(int, (T)(IDENT)), __builtin_bit_cast(int, v)))); \
+    v = OP(v, __builtin_bit_cast(T, dpp_mov<0x142, 0xa>(__builtin_bit_cast(int, (T)(IDENT)), __builtin_bit_cast(int, v)))); \
+    v = OP(v, __builtin_bit_cast(T, dpp_mov<0x143, 0xc>(__builtin_bit_cast(int, (T)(IDENT)), __builtin_bit_cast(int, v)))); \
+  } while (0)
+
+__device__ inline float op_fmax(float a, float b) { return fmaxf(a, b); }
+__device__ inline float op_fadd(float a, float b) { return a + b; }
+__device__ inline int op_iadd(int a, int b) { return a + b; }
+__device__ inline uint32_t op_umax(uint32_t a, uint32_t b) { return a > b ? a : b; }
+__device__ inline uint32_t op_umin(uint32_t a, uint32_t b) { return a < b ? a : b; }
+
+// result broadcast to every lane
 __device__ inline float wave_max(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
-  return v;
+  JF_DPP_REDUCE(v, op_fmax, float, -INFINITY);
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 __device__ inline float wave_sum(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
-  return v;
+  JF_DPP_REDUCE(v, op_fadd, float, 0.0f);
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 __device__ inline int wave_sum_i(int v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+  JF_DPP_REDUCE(v, op_iadd, int, 0);
+  return __builtin_amdgcn_readlane(v, 63);
+}
+__device__ inline uint32_t wave_max_u(uint32_t v) {
+  JF_DPP_REDUCE(v, op_umax, uint32_t, 0u);
+  return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
+}
+__device__ inline uint32_t wave_min_u(uint32_t v) {
+  JF_DPP_REDUCE(v, op_umin, uint32_t, 0xffffffffu);
+  return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
+}
+// inclusive prefix sum over lanes 0..l
+__device__ inline int wave_incl_scan_i(int v) {
+  JF_DPP_REDUCE(v, op_iadd, int, 0);
   return v;
 }
 

@@ -1,22 +1,24 @@
 // Fused decode scan + top-k for gfx950: one pass over the packed K and V of every (sequence, kv-head),
 // no (B, H_q, S) score tensor in HBM.
 //
-// Launch 1, fused_scan_kernel, grid (n_splits, H_kv, B), 256 threads.  A workgroup owns L consecutive
-// positions of one (sequence, kv-head) and all G query heads of that kv-head:
-//   phase A  Q.K^T            scores[G][L] -> LDS (fp32), running max per head
+// Launch 1, fused_scan_kernel, grid (n_splits, H_kv, B), 512 threads (8 wavefronts).  A workgroup owns L
+// consecutive positions of one (sequence, kv-head) and all G query heads of that kv-head.  The page
+// table of the split is read once into LDS; every wavefront then streams 64-token chunks with the loads
+// of its next chunk in flight while it works on the current one (no workgroup barrier inside a phase):
+//   phase A  Q.K^T            scores[G][L] -> LDS (fp32), running max per head, V scales -> LDS
 //            INT3 keys: K-hat = bf16((code-4)*scale) built in registers, v_mfma_f32_16x16x32_bf16 with the
-//                       tokens on the N side; the four 16-token tiles of a wavefront land one per
-//                       16-lane group, so lane l ends up holding the G scores of token l.
+//                       tokens on the N side; the four 16-token tiles of a chunk land one per 16-lane
+//                       group, so lane l ends up holding the G scores of token l.
 //            INT4 keys: int8-quantised Q, exact nibble codes, v_dot4_i32_i8, fp32 rescale (every step
 //                       is exactly reproducible, so it is bit-equal to the split-form kernel).
 //   phase B  P.V on v_mfma_i32_16x16x64_i8.  p = exp(s - m_split) is known exactly because phase A is
 //            complete, so w = p * v_scale is converted to 22-bit fixed point once (fma with 2^23), its
 //            three bytes are the A-operand rows (limb, head), and the int32 accumulators live for the whole
-//            split: every product is exact.  V codes are staged packed in LDS and transposed by
-//            ds_read_b64_tr_b4 (16 tokens of one channel per lane), then nibble-spread to bytes.
+//            split: every product is exact.  V codes are staged packed in wavefront-private LDS and
+//            transposed by ds_read_b64_tr_b4 (16 tokens of one channel per lane), then nibble-spread.
 //            sum_t w_t*(code - off) = sum_t w_t*code - off * sum_t w_t; a constant-ones row gives sum_t code.
-//   phase C  per-head radix select over the LDS scores: the split's top-min(K, n) candidates
-//            (key, position), ascending position.
+//   phase C  per-head radix select with the keys held in registers (bits shared by all keys of the split
+//            are skipped): the split's top-min(K, n) candidates (key, position), ascending position.
 // Launch 2, fused_merge_kernel, grid (B, H_q): selects the global top-k among the candidates (ties to
 // the lower position, ascending output), merges the split partials
 //   M = max m_i, l = sum l_i e^{m_i-M}, o_hat = sum o_i e^{m_i-M} / l
@@ -36,8 +38,12 @@ typedef float v2f __attribute__((ext_vector_type(2)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
 
-constexpr int FS_THREADS = 256;
-constexpr int FS_WAVES = 4;
+constexpr int FS_THREADS = 512;
+constexpr int FS_WAVES = 8;
+constexpr int FS_LMAX = 2048;          // positions per split (register-resident keys in phase C: 32 per lane)
+constexpr int FS_MAXCH = FS_LMAX / 64;
+constexpr int FS_MAX_TOPK = 1024;      // winners cached in LDS by the merge kernel
+constexpr int FS_CAND_SLACK = 256;     // extra candidate slots per (row, split)
 
 struct FusedParams {
   const uint16_t* q;
@@ -67,6 +73,32 @@ struct FusedParams {
   float* W;
   float* softmax_m;
   float* softmax_inv_z;
+  long long* phase_clock;  // optional: 6 s_memtime stamps per scan workgroup (measurement aid)
+};
+
+// LDS carve-up shared by the kernel and its launcher.
+template <int SCHEME, int G, int NG>
+struct ScanLds {
+  static constexpr bool K3 = (SCHEME == JF_SCHEME_K3V2);
+  static constexpr int NSET = (G + 3) / 4;
+  static constexpr int VP = K3 ? 32 : 64;
+  static constexpr int VROW = VP + 8;  // 16 consecutive rows hit 16 distinct bank pairs
+  static constexpr int VST = 64 * VROW;
+  static constexpr int WL = NG * NSET * 12 * 64;
+  static constexpr int WAVE_STAGE = VST + WL;
+  static constexpr int RED = NSET * 8 * 13 * 16 * 4;
+  static constexpr int QSZ = G * (16 + 16 + 4 + 4 + 4) * 4;
+  static constexpr int K3SZ = NSET * 16 * 4 * 2 * 16 + NSET * 4 * 2 * 4 * 3 + 128 * 4;
+  __host__ __device__ static constexpr int stage_bytes() {
+    int s = FS_WAVES * WAVE_STAGE;
+    if (RED > s) s = RED;
+    if (QSZ > s) s = QSZ;
+    if (K3SZ > s) s = K3SZ;
+    if (FS_WAVES * 264 * 4 > s) s = FS_WAVES * 264 * 4;
+    return (s + 15) & ~15;
+  }
+  __host__ __device__ static constexpr size_t per_position() { return (size_t)G * 4 + NG * 2; }
+  __host__ __device__ static size_t total(int L) { return per_position() * L + (size_t)(L / 16) * 4 + stage_bytes() + 64; }
 };
 
 __device__ inline uint32_t pack_bf16x2(float a, float b) {
@@ -84,33 +116,54 @@ __device__ inline float key_to_score(uint32_t key) {
 // transposed V dword yields tokens 0,2,4,6 | 1,3,5,7 | 8,10,12,14 | 9,11,13,15.
 __device__ inline int token_byte_pos(int r) { return (r & 8) | ((r & 1) << 2) | ((r >> 1) & 3); }
 
+// Orders this wavefront's earlier LDS writes before its later LDS reads (the LDS pipe executes one
+// wavefront's instructions in order; this only stops the compiler from moving them).
+__device__ inline void wave_lds_fence() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Phase-A constants of the INT3 path, built once per workgroup in LDS.
+template <int NSET>
+struct K3Prep {
+  int8_t aop[NSET][16][4][2][16];  // A operand bytes: [set][row = 4*head + limb][k-block][half][byte]
+  int sq4[NSET * 4][2];            // 4 * sum of the fixed-point query over the scale group
+  float qsc[NSET * 4][2];          // 2^(e-22) * attn_scale of the (head, group)
+  float eps[128];                  // 256 * (bf16(3s) - 3s) / s for s = 1 + m/128
+  int qexp[NSET * 4][2];
+};
+
 template <int G>
 struct QInt8F {
   int qe[G][16];
   int qo[G][16];
   float qs[G][4];
   int sum8[G][4];
+  float inv[G][4];
 };
 
 // ---------------------------------------------------------------------------------------------------
 template <int SCHEME, int G, int NG>
 __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
-  constexpr bool K3 = (SCHEME == JF_SCHEME_K3V2);
-  constexpr int NSET = (G + 3) / 4;
+  using Lds = ScanLds<SCHEME, G, NG>;
+  constexpr bool K3 = Lds::K3;
+  constexpr int NSET = Lds::NSET;
   constexpr int KP = K3 ? 48 : 64;
-  constexpr int VP = K3 ? 32 : 64;
-  constexpr int VROW = VP + 8;          // LDS row stride: 16 consecutive rows hit 16 distinct bank pairs
-  constexpr int VOFF = K3 ? 2 : 8;      // code offset of the V format
-  constexpr int NTILE = 8;              // 8 MFMA column tiles of 16 channels
-  constexpr int WL_WAVE = NG * NSET * 16 * 64;  // bytes of limb rows per wavefront
+  constexpr int VP = Lds::VP;
+  constexpr int VROW = Lds::VROW;
+  constexpr int VOFF = K3 ? 2 : 8;  // code offset of the V format
+  constexpr int NTILE = 8;          // 8 MFMA column tiles of 16 channels
 
   extern __shared__ __align__(16) uint8_t smem[];
   const int L = p.L;
-  float* sc = reinterpret_cast<float*>(smem);                 // [G][L]
-  uint8_t* stage = smem + (size_t)G * L * sizeof(float);      // staging, reused between phases
+  float* sc = reinterpret_cast<float*>(smem);                                   // [G][L]
+  int* sbase = reinterpret_cast<int*>(smem + (size_t)G * L * 4);                // [L/16] first slot of each page
+  uint16_t* vsl = reinterpret_cast<uint16_t*>(smem + (size_t)G * L * 4 + (size_t)(L / 16) * 4);  // [L][NG]
+  uint8_t* stage = smem + (((size_t)G * L * 4 + (size_t)(L / 16) * 4 + (size_t)L * NG * 2 + 15) & ~(size_t)15);
   __shared__ float red_f[FS_WAVES][16];
+  __shared__ float red_v[FS_WAVES][2];
   __shared__ float m_sh[16];
-  __shared__ float vmax_sh[FS_WAVES][2];
   __shared__ int e_sh[2];
   __shared__ unsigned long long wsum_sh[16][2];
 
@@ -121,91 +174,76 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
   const int s1 = min(s0 + L, S);
   const int n = max(0, s1 - s0);
   const int s_cover = min(s0 + L, p.max_S);
+  const int n_cover = max(0, s_cover - s0);
   const int64_t* bt = p.block_table + (size_t)b * p.max_blocks;
   const size_t head0 = (size_t)b * p.H_q + (size_t)hkv * G;
+  const size_t part_base = head0 * p.n_splits + split;  // + h * n_splits
   const uint8_t* kbase = p.k_data + (size_t)hkv * p.num_slots * KP;
+  const uint8_t* vbase = p.v_data + (size_t)hkv * p.num_slots * VP;
+  const uint16_t* vsbase = p.v_scales + (size_t)hkv * p.num_slots * NG;
 
-  float mx[G];
-#pragma unroll
-  for (int h = 0; h < G; ++h) mx[h] = -INFINITY;
+  long long* clk = p.phase_clock ? p.phase_clock + (((size_t)b * p.H_kv + hkv) * p.n_splits + split) * 10 : nullptr;
+  if (clk && tid == 0) clk[0] = clock64();
 
-  // ------------------------------------------------------------------ phase A
+  if (n == 0) {  // nothing valid in this split: padding scores, empty partials
+    if (p.scores)
+      for (int i = tid; i < G * n_cover; i += FS_THREADS)
+        p.scores[(head0 + i / n_cover) * (size_t)p.max_S + s0 + (i % n_cover)] = -INFINITY;
+    for (int i = tid; i < G * D; i += FS_THREADS) p.part_o[(part_base + (size_t)(i / D) * p.n_splits) * D + (i % D)] = 0.f;
+    if (tid < G) {
+      p.part_m[part_base + (size_t)tid * p.n_splits] = -INFINITY;
+      p.part_l[part_base + (size_t)tid * p.n_splits] = 0.f;
+      p.cand_cnt[part_base + (size_t)tid * p.n_splits] = 0;
+    }
+    return;
+  }
+
+  for (int i = tid; i < (n + 15) / 16; i += FS_THREADS) sbase[i] = (int)(bt[(s0 >> 4) + i] * BS);
+  if (tid < 32) wsum_sh[tid >> 1][tid & 1] = 0ull;
   if (K3) {
-    const int r = lane & 15, kb = lane >> 4;
-    v8bf qA[NSET][4];
-#pragma unroll
-    for (int set = 0; set < NSET; ++set) {
-      const int h = set * 4 + (r & 3);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        uint4 v = make_uint4(0, 0, 0, 0);
-        if (h < G) v = *reinterpret_cast<const uint4*>(p.q + (head0 + h) * D + 32 * kb + 8 * i);
-        qA[set][i] = __builtin_bit_cast(v8bf, v);
+    K3Prep<NSET>* prep = reinterpret_cast<K3Prep<NSET>*>(stage);
+    constexpr int GS = D / NG;
+    for (int i = tid; i < NSET * 16 * 4 * 2 * 16 / 4; i += FS_THREADS) reinterpret_cast<int*>(&prep->aop[0][0][0][0][0])[i] = 0;
+    if (tid < 128) {
+      const float sm = 1.0f + (float)tid * (1.0f / 128.0f);
+      const float t3 = 3.0f * sm;  // exact in fp32
+      prep->eps[tid] = 256.0f * ((bf16_to_f32(f32_to_bf16(t3)) - t3) / sm);
+    }
+    for (int i = tid; i < NSET * 4 * NG; i += FS_THREADS) {
+      const int h = i / NG, g = i % NG;
+      int e = 0;
+      long sum = 0;
+      if (h < G) {
+        const uint16_t* qr = p.q + (head0 + h) * D + g * GS;
+        float amax = 0.f;
+        for (int d = 0; d < GS; ++d) amax = fmaxf(amax, fabsf(bf16_to_f32(qr[d])));
+        if (amax > 0.f && isfinite(amax)) (void)frexpf(amax, &e);  // amax = f * 2^e, f in [0.5, 1)
+        for (int d = 0; d < GS; ++d) sum += (long)rintf(ldexpf(bf16_to_f32(qr[d]), 22 - e));
+      }
+      prep->qexp[h][g] = e;
+      prep->sq4[h][g] = (int)(4 * sum);
+      prep->qsc[h][g] = ldexpf(p.attn_scale, e - 22);
+    }
+    __syncthreads();
+    for (int i = tid; i < NSET * 4 * D; i += FS_THREADS) {
+      const int h = i / D, d = i % D;
+      if (h < G) {
+        const int g = d / GS;
+        const int qf = (int)rintf(ldexpf(bf16_to_f32(p.q[(head0 + h) * D + d]), 22 - prep->qexp[h][g]));
+        const int l0 = (int)(int8_t)(qf & 255);
+        const int r1 = (qf - l0) >> 8;
+        const int l1 = (int)(int8_t)(r1 & 255);
+        const int l2 = (r1 - l1) >> 8;
+        const int set = h >> 2, hh = h & 3;
+        const int kbk = d >> 5, j = (d >> 3) & 3, u = (d >> 2) & 1, ip = d & 3;
+        prep->aop[set][4 * hh + 0][kbk][u][4 * ip + j] = (int8_t)l0;
+        prep->aop[set][4 * hh + 1][kbk][u][4 * ip + j] = (int8_t)l1;
+        prep->aop[set][4 * hh + 2][kbk][u][4 * ip + j] = (int8_t)l2;
       }
     }
-    const uint16_t* ksbase = p.k_scales + (size_t)hkv * p.num_slots * NG;
-    const int kgrp = (NG == 1) ? 0 : (kb >> 1);
-    const int cover_end = s0 + ((max(s_cover - s0, 0) + 63) & ~63);
-    for (int c0 = s0 + wave * 64; c0 < cover_end; c0 += FS_THREADS) {
-      v4f Dt[NSET][4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-#pragma unroll
-        for (int set = 0; set < NSET; ++set) Dt[set][j] = (v4f){0.f, 0.f, 0.f, 0.f};
-        const int t0 = c0 + 16 * j;
-        uint32_t P0 = 0, P1 = 0, P2 = 0;
-        float s = 0.f;
-        if (t0 + r < s1) {
-          const int64_t slot = bt[t0 >> 4] * BS + r;
-          const uint32_t* row = reinterpret_cast<const uint32_t*>(kbase + slot * KP);
-          P0 = row[kb];
-          P1 = row[4 + kb];
-          P2 = row[8 + kb];
-          s = bf16_to_f32(ksbase[slot * NG + kgrp]);
-        }
-        if (t0 < s1) {  // wavefront-uniform: skip tiles with no valid token
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const uint32_t w = (((P0 >> (8 * i)) & 255u) << 16) | (((P1 >> (8 * i)) & 255u) << 8) | ((P2 >> (8 * i)) & 255u);
-            uint4 kv;
-            uint32_t* kvp = reinterpret_cast<uint32_t*>(&kv);
-#pragma unroll
-            for (int jj = 0; jj < 4; ++jj) {
-              const int ca = (int)((w >> (21 - 6 * jj)) & 7u) - 4;
-              const int cb = (int)((w >> (18 - 6 * jj)) & 7u) - 4;
-              kvp[jj] = pack_bf16x2((float)ca * s, (float)cb * s);
-            }
-            const v8bf kB = __builtin_bit_cast(v8bf, kv);
-#pragma unroll
-            for (int set = 0; set < NSET; ++set)
-              Dt[set][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qA[set][i], kB, Dt[set][j], 0, 0, 0);
-          }
-        }
-      }
-      // lane group g keeps tile g: lane l <-> token c0 + l, register <-> head
-      const int pos = c0 + lane;
-      const bool valid = pos < s1;
-#pragma unroll
-      for (int set = 0; set < NSET; ++set) {
-#pragma unroll
-        for (int rr = 0; rr < 4; ++rr) {
-          const int h = set * 4 + rr;
-          if (h < G) {
-            const float a = (kb == 0) ? Dt[set][0][rr] : (kb == 1) ? Dt[set][1][rr] : (kb == 2) ? Dt[set][2][rr] : Dt[set][3][rr];
-            const float sv = valid ? a * p.attn_scale : -INFINITY;
-            if (pos < s_cover) {
-              sc[h * L + (pos - s0)] = sv;
-              if (p.scores) p.scores[(head0 + h) * (size_t)p.max_S + pos] = sv;
-            }
-            mx[h] = fmaxf(mx[h], sv);
-          }
-        }
-      }
-    }
-  } else {
-    // INT4 keys, int8-Q model: lane = token
+  }
+  if (!K3) {  // int8 quantisation of the G query rows (int8tc_qk_scores.cu:250-290)
     QInt8F<G>* qsh = reinterpret_cast<QInt8F<G>*>(stage);
-    float* scratch = reinterpret_cast<float*>(stage + sizeof(QInt8F<G>));
     const uint16_t* qrow0 = p.q + head0 * D;
     for (int i = tid; i < G * 4; i += FS_THREADS) {
       const int g = i >> 2, kk = i & 3;
@@ -213,12 +251,12 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
       for (int d = 0; d < 32; ++d) amax = fmaxf(amax, fabsf(bf16_to_f32(qrow0[(size_t)g * D + kk * 32 + d])));
       const float s = fmaxf(amax / 127.0f, 1e-12f);
       qsh->qs[g][kk] = s;
-      scratch[i] = 1.0f / s;
+      qsh->inv[g][kk] = 1.0f / s;
     }
     __syncthreads();
     for (int i = tid; i < G * 16; i += FS_THREADS) {
       const int g = i >> 4, j = i & 15, kk = j >> 2;
-      const float inv = scratch[g * 4 + kk];
+      const float inv = qsh->inv[g][kk];
       int v[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) v[e] = max(-128, min(127, (int)rintf(bf16_to_f32(qrow0[(size_t)g * D + 8 * j + e]) * inv)));
@@ -236,25 +274,207 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
       }
       qsh->sum8[g][kk] = 8 * sum;
     }
-    __syncthreads();
-    const uint16_t* ksbase = p.k_scales + (size_t)hkv * p.num_slots;
-    for (int pos = s0 + tid; pos < s_cover; pos += FS_THREADS) {
-      const bool valid = pos < s1;
-      uint32_t pk[16];
-      float ks = 0.f;
-      if (valid) {
-        const int64_t slot = bt[pos >> 4] * BS + (pos & 15);
-        const uint4* row = reinterpret_cast<const uint4*>(kbase + slot * KP);
+  }
+  __syncthreads();
+
+  // ------------------------------------------------------------------ phase A
+  float mx[G];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const uint4 v = row[i];
-          pk[4 * i] = v.x; pk[4 * i + 1] = v.y; pk[4 * i + 2] = v.z; pk[4 * i + 3] = v.w;
-        }
-        ks = bf16_to_f32(ksbase[slot]);
-      } else {
+  for (int h = 0; h < G; ++h) mx[h] = -INFINITY;
+  float vmax[NG];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) pk[i] = 0;
+  for (int g = 0; g < NG; ++g) vmax[g] = 0.f;
+  const int nch_cover = (n_cover + 63) >> 6;
+
+  // per-lane V scale word of token t (clamped into the valid range)
+  auto load_vs = [&](int t) -> uint32_t {
+    const int tc = min(t, n - 1);
+    const int64_t slot = (int64_t)sbase[tc >> 4] + (tc & 15);
+    if (NG == 2) return *reinterpret_cast<const uint32_t*>(vsbase + slot * 2);
+    return (uint32_t)vsbase[slot];
+  };
+  auto finish_token = [&](int t, const float (&a)[G], uint32_t vsw) {
+    // a[h]: score of token t for head h (already scaled).  Writes LDS / optional HBM, tracks maxima.
+    const bool valid = t < n;
+    if (t < n_cover) {
+#pragma unroll
+      for (int h = 0; h < G; ++h) {
+        const float sv = valid ? a[h] : -INFINITY;
+        sc[h * L + t] = sv;
+        if (p.scores) p.scores[(head0 + h) * (size_t)p.max_S + s0 + t] = sv;
+        mx[h] = fmaxf(mx[h], sv);
       }
+      if (NG == 2) *reinterpret_cast<uint32_t*>(vsl + 2 * t) = vsw;
+      else vsl[t] = (uint16_t)vsw;
+      if (valid) {
+        vmax[0] = fmaxf(vmax[0], fabsf(bf16_to_f32((uint16_t)(vsw & 0xffffu))));
+        if (NG == 2) vmax[NG - 1] = fmaxf(vmax[NG - 1], fabsf(bf16_to_f32((uint16_t)(vsw >> 16))));
+      }
+    }
+  };
+
+  if (K3) {
+    // INT3 keys on v_mfma_i32_16x16x64_i8.  The bf16 query row is held exactly as a 23-bit fixed-point number
+    // per (head, scale group), split into three balanced int8 limbs that sit in different A-operand rows
+    // (row = 4*head + limb), so one MFMA chain yields the three integer partial sums of a (token, head) in the
+    // registers of one lane.  K codes are spread from the three byte planes to one byte per code with
+    // shift/mask on whole dwords (4 codes per VALU operation) and used unsigned; the -4 offset is removed with
+    // the per-row constant 4*sum(q).  The reference rounds every dequantised key to bf16
+    // (int3_qk_scores.cu:90-99); only codes +-3 are inexact, so that rounding is reproduced by a second
+    // contraction with the indicator (+1 for code 7, -1 for code 1, byte LUT through v_perm_b32) weighted by
+    // eps = (bf16(3s) - 3s) / s, which depends on the 7 mantissa bits of the scale only (128-entry table).
+    const K3Prep<NSET>* prep = reinterpret_cast<const K3Prep<NSET>*>(stage);
+    const int t16 = lane & 15, lg = lane >> 4;  // B operand: column (token), k-block; D: column, head
+    const int kgrp_of_lane = (NG == 1) ? 0 : (lg >> 1);
+    v4i Aop[NSET][NG][2];
+    int sq4[NSET][NG];
+    float qsc[NSET][NG];
+#pragma unroll
+    for (int set = 0; set < NSET; ++set) {
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const v4i raw = *reinterpret_cast<const v4i*>(&prep->aop[set][t16][lg][u][0]);
+#pragma unroll
+        for (int g = 0; g < NG; ++g) Aop[set][g][u] = (kgrp_of_lane == g) ? raw : (v4i){0, 0, 0, 0};
+      }
+#pragma unroll
+      for (int g = 0; g < NG; ++g) {
+        sq4[set][g] = prep->sq4[set * 4 + lg][g];
+        qsc[set][g] = prep->qsc[set * 4 + lg][g];
+      }
+    }
+    const uint16_t* ksbase = p.k_scales + (size_t)hkv * p.num_slots * NG;
+    uint32_t Pc[4][3], Pn[4][3];
+    uint32_t Sc[4], Sn[4], Vc[4], Vn[4];
+    auto issue = [&](int chunk, uint32_t (&P)[4][3], uint32_t (&Sx)[4], uint32_t (&Vx)[4]) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int tc = min(chunk * 64 + 16 * j + t16, n - 1);
+        const int64_t slot = (int64_t)sbase[tc >> 4] + (tc & 15);
+        const uint32_t* row = reinterpret_cast<const uint32_t*>(kbase + slot * KP);
+        P[j][0] = row[lg];
+        P[j][1] = row[4 + lg];
+        P[j][2] = row[8 + lg];
+        if (NG == 2) {
+          Sx[j] = *reinterpret_cast<const uint32_t*>(ksbase + slot * 2);
+          Vx[j] = *reinterpret_cast<const uint32_t*>(vsbase + slot * 2);
+        } else {
+          Sx[j] = ksbase[slot];
+          Vx[j] = vsbase[slot];
+        }
+      }
+    };
+    float mxl[NSET];
+#pragma unroll
+    for (int set = 0; set < NSET; ++set) mxl[set] = -INFINITY;
+    int chunk = wave;
+    if (chunk < nch_cover) issue(chunk, Pc, Sc, Vc);
+    for (; chunk < nch_cover; chunk += FS_WAVES) {
+      if (chunk + FS_WAVES < nch_cover) issue(chunk + FS_WAVES, Pn, Sn, Vn);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t P0 = Pc[j][0], P1 = Pc[j][1], P2 = Pc[j][2];
+        v4i Bc[2], Br[2];
+        Bc[0][0] = (int)((P0 >> 5) & 0x07070707u);
+        Bc[0][1] = (int)((P0 >> 2) & 0x07070707u);
+        Bc[0][2] = (int)(((P0 << 1) & 0x06060606u) | ((P1 >> 7) & 0x01010101u));
+        Bc[0][3] = (int)((P1 >> 4) & 0x07070707u);
+        Bc[1][0] = (int)((P1 >> 1) & 0x07070707u);
+        Bc[1][1] = (int)(((P1 << 2) & 0x04040404u) | ((P2 >> 6) & 0x03030303u));
+        Bc[1][2] = (int)((P2 >> 3) & 0x07070707u);
+        Bc[1][3] = (int)(P2 & 0x07070707u);
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            Br[u][e] = (int)__builtin_amdgcn_perm(0x01000000u, 0x0000ff00u, (uint32_t)Bc[u][e]);
+        // per-token scales (both groups) and the rounding coefficient
+        float sg[NG], eg[NG];
+        {
+          const uint32_t sw = Sc[j];
+          sg[0] = bf16_to_f32((uint16_t)(sw & 0xffffu));
+          eg[0] = prep->eps[sw & 0x7fu];
+          if (NG == 2) {
+            sg[NG - 1] = bf16_to_f32((uint16_t)(sw >> 16));
+            eg[NG - 1] = prep->eps[(sw >> 16) & 0x7fu];
+          }
+        }
+        const int tok = chunk * 64 + 16 * j + t16;
+        const bool valid = tok < n;
+#pragma unroll
+        for (int set = 0; set < NSET; ++set) {
+          float score = 0.f;
+#pragma unroll
+          for (int g = 0; g < NG; ++g) {
+            v4i Dc = {0, 0, 0, 0}, Dr = {0, 0, 0, 0};
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+              Dc = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][g][u], Bc[u], Dc, 0, 0, 0);
+              Dr = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][g][u], Br[u], Dr, 0, 0, 0);
+            }
+            const int xc = (((Dc[2] << 8) + Dc[1]) << 8) + Dc[0] - sq4[set][g];
+            const int xr = (Dr[2] << 8) + Dr[1];
+            const float v = __builtin_fmaf(eg[g], (float)xr, (float)xc);
+            score = __builtin_fmaf(v, sg[g] * qsc[set][g], score);
+          }
+          const int h = set * 4 + lg;
+          if (h < G && tok < n_cover) {
+            const float sv = valid ? score : -INFINITY;
+            sc[h * L + tok] = sv;
+            if (p.scores) p.scores[(head0 + h) * (size_t)p.max_S + s0 + tok] = sv;
+            mxl[set] = fmaxf(mxl[set], sv);
+          }
+        }
+        if (lg == 0 && tok < n_cover) {
+          const uint32_t vsw = Vc[j];
+          if (NG == 2) *reinterpret_cast<uint32_t*>(vsl + 2 * tok) = vsw;
+          else vsl[tok] = (uint16_t)vsw;
+          if (valid) {
+            vmax[0] = fmaxf(vmax[0], fabsf(bf16_to_f32((uint16_t)(vsw & 0xffffu))));
+            if (NG == 2) vmax[NG - 1] = fmaxf(vmax[NG - 1], fabsf(bf16_to_f32((uint16_t)(vsw >> 16))));
+          }
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        Pc[j][0] = Pn[j][0]; Pc[j][1] = Pn[j][1]; Pc[j][2] = Pn[j][2];
+        Sc[j] = Sn[j];
+        Vc[j] = Vn[j];
+      }
+    }
+    // lanes of 16-lane row lg hold the running maxima of head set*4 + lg: spread them into mx[] so the common
+    // reduction below applies (every other entry stays -inf)
+#pragma unroll
+    for (int set = 0; set < NSET; ++set)
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr)
+        if (set * 4 + rr < G) mx[set * 4 + rr] = (lg == rr) ? mxl[set] : -INFINITY;
+  } else {
+    // INT4 keys, int8-Q model: lane = token
+    const QInt8F<G>* qsh = reinterpret_cast<const QInt8F<G>*>(stage);
+    const uint16_t* ksbase = p.k_scales + (size_t)hkv * p.num_slots;
+    uint4 Rc[4], Rn[4];
+    uint32_t Kc_s = 0, Kn_s = 0, Vc = 0, Vn = 0;
+    auto issue = [&](int chunk, uint4 (&R)[4], uint32_t& ksw, uint32_t& vsw) {
+      const int tc = min(chunk * 64 + lane, n - 1);
+      const int64_t slot = (int64_t)sbase[tc >> 4] + (tc & 15);
+      const uint4* row = reinterpret_cast<const uint4*>(kbase + slot * KP);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) R[i] = row[i];
+      ksw = ksbase[slot];
+      vsw = load_vs(chunk * 64 + lane);
+    };
+    int chunk = wave;
+    if (chunk < nch_cover) issue(chunk, Rc, Kc_s, Vc);
+    for (; chunk < nch_cover; chunk += FS_WAVES) {
+      if (chunk + FS_WAVES < nch_cover) issue(chunk + FS_WAVES, Rn, Kn_s, Vn);
+      uint32_t pk[16];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        pk[4 * i] = Rc[i].x; pk[4 * i + 1] = Rc[i].y; pk[4 * i + 2] = Rc[i].z; pk[4 * i + 3] = Rc[i].w;
+      }
+      const float ks = bf16_to_f32((uint16_t)Kc_s);
+      float a[G];
 #pragma unroll
       for (int g = 0; g < G; ++g) {
         float sacc = 0.0f;
@@ -269,68 +489,54 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
           acc -= qsh->sum8[g][kk];
           sacc = (kk == 0) ? ((float)acc * qsh->qs[g][0]) : __builtin_fmaf((float)acc, qsh->qs[g][kk], sacc);
         }
-        const float sv = valid ? __fmul_rn(__fmul_rn(sacc, ks), p.attn_scale) : -INFINITY;
-        sc[g * L + (pos - s0)] = sv;
-        if (p.scores) p.scores[(head0 + g) * (size_t)p.max_S + pos] = sv;
-        mx[g] = fmaxf(mx[g], sv);
+        a[g] = __fmul_rn(__fmul_rn(sacc, ks), p.attn_scale);
       }
+      finish_token(chunk * 64 + lane, a, Vc);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) Rc[i] = Rn[i];
+      Kc_s = Kn_s;
+      Vc = Vn;
     }
   }
 
-  // split max per head
+  // split max per head, V-scale maxima
 #pragma unroll
   for (int h = 0; h < G; ++h) {
     const float v = wave_max(mx[h]);
     if (lane == 0) red_f[wave][h] = v;
   }
-  __syncthreads();
-  if (tid < G) m_sh[tid] = fmaxf(fmaxf(red_f[0][tid], red_f[1][tid]), fmaxf(red_f[2][tid], red_f[3][tid]));
-  if (tid < 16 * 2) wsum_sh[tid >> 1][tid & 1] = 0ull;
-  __syncthreads();
-
-  const size_t part_base = head0 * p.n_splits + split;  // + h * n_splits
-  if (n == 0) {
-    for (int i = tid; i < G * D; i += FS_THREADS) p.part_o[(part_base + (size_t)(i / D) * p.n_splits) * D + (i % D)] = 0.f;
-    if (tid < G) {
-      p.part_m[part_base + (size_t)tid * p.n_splits] = -INFINITY;
-      p.part_l[part_base + (size_t)tid * p.n_splits] = 0.f;
-      p.cand_cnt[part_base + (size_t)tid * p.n_splits] = 0;
-    }
-    return;
+#pragma unroll
+  for (int g = 0; g < NG; ++g) {
+    const float v = wave_max(vmax[g]);
+    if (lane == 0) red_v[wave][g] = v;
   }
+  __syncthreads();
+  if (tid < G) {
+    float m = red_f[0][tid];
+#pragma unroll
+    for (int w = 1; w < FS_WAVES; ++w) m = fmaxf(m, red_f[w][tid]);
+    m_sh[tid] = m;
+  }
+  if (tid >= 64 && tid < 64 + NG) {
+    const int g = tid - 64;
+    float v = red_v[0][g];
+#pragma unroll
+    for (int w = 1; w < FS_WAVES; ++w) v = fmaxf(v, red_v[w][g]);
+    int e = 0;
+    if (v > 0.f && isfinite(v)) (void)frexpf(v, &e);  // v = f * 2^e, f in [0.5, 1)
+    e_sh[g] = 22 - e;                                 // v * 2^E in [2^21, 2^22)
+  }
+  __syncthreads();
+  if (clk && tid == 0) clk[1] = clock64();
 
   // ------------------------------------------------------------------ phase B
-  const uint8_t* vbase = p.v_data + (size_t)hkv * p.num_slots * VP;
-  const uint16_t* vsbase = p.v_scales + (size_t)hkv * p.num_slots * NG;
-  {
-    float vm[NG];
-#pragma unroll
-    for (int g = 0; g < NG; ++g) vm[g] = 0.f;
-    for (int pos = s0 + tid; pos < s1; pos += FS_THREADS) {
-      const int64_t slot = bt[pos >> 4] * BS + (pos & 15);
-#pragma unroll
-      for (int g = 0; g < NG; ++g) vm[g] = fmaxf(vm[g], fabsf(bf16_to_f32(vsbase[slot * NG + g])));
-    }
-#pragma unroll
-    for (int g = 0; g < NG; ++g) {
-      const float v = wave_max(vm[g]);
-      if (lane == 0) vmax_sh[wave][g] = v;
-    }
-    __syncthreads();
-    if (tid < NG) {
-      float v = fmaxf(fmaxf(vmax_sh[0][tid], vmax_sh[1][tid]), fmaxf(vmax_sh[2][tid], vmax_sh[3][tid]));
-      int e = 0;
-      if (v > 0.f && isfinite(v)) (void)frexpf(v, &e);  // v = f * 2^e, f in [0.5, 1)
-      e_sh[tid] = 22 - e;                               // v * 2^E in [2^21, 2^22)
-    }
-    __syncthreads();
-  }
   int E[NG];
 #pragma unroll
   for (int g = 0; g < NG; ++g) E[g] = e_sh[g];
+  if (clk && tid == 0) clk[2] = clock64();
 
-  uint8_t* vst = stage;                                   // [256][VROW]
-  uint8_t* wl = stage + FS_THREADS * VROW;                // [4 waves][NG][NSET][16][64]
+  uint8_t* vst = stage + wave * Lds::WAVE_STAGE;  // [64][VROW], this wavefront only
+  uint8_t* wl = vst + Lds::VST;                   // [NG][NSET][12][64]
   v4i acc[NSET][NTILE];
 #pragma unroll
   for (int set = 0; set < NSET; ++set)
@@ -349,70 +555,71 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
   for (int h = 0; h < G; ++h) mh[h] = m_sh[h];
   const int r16 = lane & 15, kb4 = lane >> 4;
   const int bytepos = (kb4 << 4) | token_byte_pos(r16);
-  uint8_t* wl_w = wl + wave * WL_WAVE;
-
-  for (int base = s0; base < s1; base += FS_THREADS) {
-    __syncthreads();
-    const int pos = base + tid;
-    const bool valid = pos < s1;
-    float vsf[NG];
-    {
-      uint2* dst = reinterpret_cast<uint2*>(vst + tid * VROW);
-      if (valid) {
-        const int64_t slot = bt[pos >> 4] * BS + (pos & 15);
-        const uint4* src = reinterpret_cast<const uint4*>(vbase + slot * VP);
+  const int nch = (n + 63) >> 6;
+  {
+    uint4 Vc[VP / 16], Vn[VP / 16];
+    auto issue_v = [&](int chunk, uint4 (&R)[VP / 16]) {
+      const int tc = min(chunk * 64 + lane, n - 1);
+      const int64_t slot = (int64_t)sbase[tc >> 4] + (tc & 15);
+      const uint4* src = reinterpret_cast<const uint4*>(vbase + slot * VP);
+#pragma unroll
+      for (int i = 0; i < VP / 16; ++i) R[i] = src[i];
+    };
+    int chunk = wave;
+    if (chunk < nch) issue_v(chunk, Vc);
+    for (; chunk < nch; chunk += FS_WAVES) {
+      if (chunk + FS_WAVES < nch) issue_v(chunk + FS_WAVES, Vn);
+      const int t = chunk * 64 + lane;
+      const bool valid = t < n;
+      {
+        uint2* dst = reinterpret_cast<uint2*>(vst + lane * VROW);
 #pragma unroll
         for (int i = 0; i < VP / 16; ++i) {
-          const uint4 v = src[i];
-          dst[2 * i] = make_uint2(v.x, v.y);
-          dst[2 * i + 1] = make_uint2(v.z, v.w);
+          dst[2 * i] = valid ? make_uint2(Vc[i].x, Vc[i].y) : make_uint2(0u, 0u);
+          dst[2 * i + 1] = valid ? make_uint2(Vc[i].z, Vc[i].w) : make_uint2(0u, 0u);
         }
-#pragma unroll
-        for (int g = 0; g < NG; ++g) vsf[g] = ldexpf(bf16_to_f32(vsbase[slot * NG + g]), E[g]);
-      } else {
-#pragma unroll
-        for (int i = 0; i < VP / 8; ++i) dst[i] = make_uint2(0u, 0u);
-#pragma unroll
-        for (int g = 0; g < NG; ++g) vsf[g] = 0.f;
       }
-    }
-#pragma unroll
-    for (int h = 0; h < G; ++h) {
-      const float pw = valid ? __expf(sc[h * L + (pos - s0)] - mh[h]) : 0.f;
-      lsum[h] += pw;
-      const int set = h >> 2, hh = h & 3;
-#pragma unroll
-      for (int g = 0; g < NG; ++g) {
-        const uint32_t bits = __builtin_bit_cast(uint32_t, __builtin_fmaf(pw, vsf[g], 8388608.0f));
-        wsum[h][g] += bits & 0x7fffffu;
-        const uint32_t lim = bits ^ 0x00008080u;
-        uint8_t* rowp = wl_w + ((g * NSET + set) * 16) * 64 + bytepos;
-        rowp[(0 * 4 + hh) * 64] = (uint8_t)(lim & 255u);
-        rowp[(1 * 4 + hh) * 64] = (uint8_t)((lim >> 8) & 255u);
-        rowp[(2 * 4 + hh) * 64] = (uint8_t)((lim >> 16) & 255u);
+      float vsf[NG];
+      {
+        const uint32_t vsw = (NG == 2) ? *reinterpret_cast<const uint32_t*>(vsl + 2 * t) : (uint32_t)vsl[t];
+        vsf[0] = valid ? ldexpf(bf16_to_f32((uint16_t)(vsw & 0xffffu)), E[0]) : 0.f;
+        if (NG == 2) vsf[NG - 1] = valid ? ldexpf(bf16_to_f32((uint16_t)(vsw >> 16)), E[NG - 1]) : 0.f;
       }
-    }
-    __syncthreads();
-    if (base + wave * 64 < s1) {  // this wavefront's 64-token chunk holds at least one valid token
+#pragma unroll
+      for (int h = 0; h < G; ++h) {
+        const float pw = valid ? __expf(sc[h * L + t] - mh[h]) : 0.f;
+        lsum[h] += pw;
+        const int set = h >> 2, hh = h & 3;
+#pragma unroll
+        for (int g = 0; g < NG; ++g) {
+          const uint32_t bits = __builtin_bit_cast(uint32_t, __builtin_fmaf(pw, vsf[g], 8388608.0f));
+          wsum[h][g] += bits & 0x7fffffu;
+          const uint32_t lim = bits ^ 0x00008080u;
+          uint8_t* rowp = wl + ((g * NSET + set) * 12) * 64 + bytepos;
+          rowp[(0 * 4 + hh) * 64] = (uint8_t)(lim & 255u);
+          rowp[(1 * 4 + hh) * 64] = (uint8_t)((lim >> 8) & 255u);
+          rowp[(2 * 4 + hh) * 64] = (uint8_t)((lim >> 16) & 255u);
+        }
+      }
+      wave_lds_fence();
       v4i A[NG][NSET];
 #pragma unroll
       for (int g = 0; g < NG; ++g)
 #pragma unroll
         for (int set = 0; set < NSET; ++set) {
           if (r16 < 12) {
-            A[g][set] = *reinterpret_cast<const v4i*>(wl_w + ((g * NSET + set) * 16 + r16) * 64 + kb4 * 16);
+            A[g][set] = *reinterpret_cast<const v4i*>(wl + ((g * NSET + set) * 12 + r16) * 64 + kb4 * 16);
           } else if (r16 == 12) {
             A[g][set] = (v4i){0x01010101, 0x01010101, 0x01010101, 0x01010101};
           } else {
             A[g][set] = (v4i){0, 0, 0, 0};
           }
         }
-      const uint8_t* vrow = vst + (wave * 64 + lane) * VROW;
+      const uint8_t* vrow = vst + lane * VROW;
       if (K3) {
 #pragma unroll
         for (int qc = 0; qc < 4; ++qc) {
-          const v2i x = __builtin_amdgcn_ds_read_tr4_b64_v2i32(
-              (__attribute__((address_space(3))) v2i*)(vrow + 8 * qc));
+          const v2i x = __builtin_amdgcn_ds_read_tr4_b64_v2i32((__attribute__((address_space(3))) v2i*)(vrow + 8 * qc));
           const uint32_t x0 = (uint32_t)x[0], x1 = (uint32_t)x[1];
           const v4i Ba = {(int)((x0 >> 2) & 0x03030303u), (int)((x0 >> 6) & 0x03030303u),
                           (int)((x1 >> 2) & 0x03030303u), (int)((x1 >> 6) & 0x03030303u)};
@@ -428,8 +635,7 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
       } else {
 #pragma unroll
         for (int qc = 0; qc < 8; ++qc) {
-          const v2i x = __builtin_amdgcn_ds_read_tr4_b64_v2i32(
-              (__attribute__((address_space(3))) v2i*)(vrow + 8 * qc));
+          const v2i x = __builtin_amdgcn_ds_read_tr4_b64_v2i32((__attribute__((address_space(3))) v2i*)(vrow + 8 * qc));
           const uint32_t x0 = (uint32_t)x[0], x1 = (uint32_t)x[1];
           const v4i Bv = {(int)(x0 & 0x0f0f0f0fu), (int)((x0 >> 4) & 0x0f0f0f0fu),
                           (int)(x1 & 0x0f0f0f0fu), (int)((x1 >> 4) & 0x0f0f0f0fu)};
@@ -439,13 +645,17 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
             acc[set][qc] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[g][set], Bv, acc[set][qc], 0, 0, 0);
         }
       }
+      wave_lds_fence();
+#pragma unroll
+      for (int i = 0; i < VP / 16; ++i) Vc[i] = Vn[i];
     }
   }
   __syncthreads();
+  if (clk && tid == 0) clk[3] = clock64();
 
-  // reduce the four wavefronts' integer accumulators in LDS: red_i[set][tile][row][col]
+  // reduce the wavefronts' integer accumulators in LDS: red_i[set][tile][row 0..12][col]
   int* red_i = reinterpret_cast<int*>(stage);
-  for (int i = tid; i < NSET * NTILE * 256; i += FS_THREADS) red_i[i] = 0;
+  for (int i = tid; i < NSET * NTILE * 13 * 16; i += FS_THREADS) red_i[i] = 0;
   __syncthreads();
 #pragma unroll
   for (int set = 0; set < NSET; ++set)
@@ -454,7 +664,7 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
 #pragma unroll
       for (int rr = 0; rr < 4; ++rr) {
         const int row = 4 * kb4 + rr;
-        if (row <= 12) atomicAdd(&red_i[((set * NTILE + t) * 16 + row) * 16 + r16], acc[set][t][rr]);
+        if (row <= 12) atomicAdd(&red_i[((set * NTILE + t) * 13 + row) * 16 + r16], acc[set][t][rr]);
       }
 #pragma unroll
   for (int h = 0; h < G; ++h) {
@@ -462,10 +672,9 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
     if (lane == 0) red_f[wave][h] = ls;  // summed in wavefront order below: run-to-run deterministic
 #pragma unroll
     for (int g = 0; g < NG; ++g) {
-      unsigned long long wv = wsum[h][g];
-#pragma unroll
-      for (int off = 32; off > 0; off >>= 1) wv += __shfl_xor(wv, off);
-      if (lane == 0) atomicAdd(&wsum_sh[h][g], wv);
+      // per-lane sums stay below 2^27; add their 16-bit halves separately so the wavefront sums fit in 32 bits
+      const int lo = wave_sum_i((int)(wsum[h][g] & 0xffffu)), hi = wave_sum_i((int)(wsum[h][g] >> 16));
+      if (lane == 0) atomicAdd(&wsum_sh[h][g], (unsigned long long)(uint32_t)lo + ((unsigned long long)(uint32_t)hi << 16));
     }
   }
   __syncthreads();
@@ -483,108 +692,199 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
       tile = qc;
     }
     const int g = (NG == 1) ? 0 : (d / (D / NG));
-    const int* tb = red_i + (set * NTILE + tile) * 256;
+    const int* tb = red_i + (set * NTILE + tile) * 13 * 16;
     const long long i0 = tb[(0 * 4 + hh) * 16 + col], i1 = tb[(1 * 4 + hh) * 16 + col], i2 = tb[(2 * 4 + hh) * 16 + col];
     const long long cs = tb[12 * 16 + col];
     const long long tot = i2 * 65536ll + i1 * 256ll + i0 + 32896ll * cs - (long long)VOFF * (long long)wsum_sh[h][g];
     p.part_o[(part_base + (size_t)h * p.n_splits) * D + d] = (float)ldexp((double)tot, -E[g]);
   }
   if (tid < G) {
+    float l = red_f[0][tid];
+#pragma unroll
+    for (int w = 1; w < FS_WAVES; ++w) l += red_f[w][tid];
     p.part_m[part_base + (size_t)tid * p.n_splits] = m_sh[tid];
-    p.part_l[part_base + (size_t)tid * p.n_splits] = ((red_f[0][tid] + red_f[1][tid]) + red_f[2][tid]) + red_f[3][tid];
+    p.part_l[part_base + (size_t)tid * p.n_splits] = l;
   }
   __syncthreads();
+  if (clk && tid == 0) clk[4] = clock64();
 
   // ------------------------------------------------------------------ phase C: per-head radix select
-  int* hist = reinterpret_cast<int*>(stage) + wave * 256;
-  const int Kc = p.Kc;
+  // One wavefront per head, keys in registers.  Bits shared by every key of the split are skipped; each
+  // 8-bit level builds a histogram (LDS atomics, bin 256 swallows keys outside the current prefix) and
+  // finds the bin holding the Kt-th largest key.  As soon as "everything from that bin upwards" fits in
+  // the candidate buffer the search stops and all keys >= that bound are emitted (a superset of the
+  // split's top Kt, which is all the merge needs); otherwise it refines down to the exact key and emits
+  // the lowest-position ties that fill the quota.  Emission is an ordered ballot compaction.
+  int* hist = reinterpret_cast<int*>(stage) + wave * 264;
+  const int Kcap = p.Kc;
+  const int Kt = min(p.top_k, n);
   for (int h = wave; h < G; h += FS_WAVES) {
-    const float* row = sc + h * L;
-    uint32_t* ck = p.cand_key + (part_base + (size_t)h * p.n_splits) * Kc;
-    int32_t* ci = p.cand_idx + (part_base + (size_t)h * p.n_splits) * Kc;
-    uint32_t tau = 0;
-    int quota = 0;
-    const bool take_all = (n <= Kc);
-    if (!take_all) {
-      uint32_t prefix = 0;
-      int k_rem = Kc;
-      for (int level = 0; level < 4; ++level) {
-        for (int i = lane; i < 256; i += 64) hist[i] = 0;
-        const int shift = 24 - 8 * level;
-        for (int i = lane; i < n; i += 64) {
-          const uint32_t key = score_key(row[i]);
-          if (level == 0 || (key >> (shift + 8)) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1);
-        }
-        // suffix scan over 256 bins, 4 bins per lane (lane owns bins 4*lane .. 4*lane+3)
-        const int c0 = hist[4 * lane], c1 = hist[4 * lane + 1], c2 = hist[4 * lane + 2], c3 = hist[4 * lane + 3];
-        const int mine = c0 + c1 + c2 + c3;
-        int incl = mine;
+    uint32_t* krow = reinterpret_cast<uint32_t*>(sc + h * L);  // scores are rewritten in place as keys
+    uint32_t* ck = p.cand_key + (part_base + (size_t)h * p.n_splits) * Kcap;
+    int32_t* ci = p.cand_idx + (part_base + (size_t)h * p.n_splits) * Kcap;
+    uint32_t kmin = 0xffffffffu, kmax = 0u;
+    for (int t0 = 0; t0 < n; t0 += 512) {
+      uint32_t kk[8];
 #pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-          const int o = __shfl_down(incl, off);
-          if (lane + off < 64) incl += o;
-        }
-        const int above_lane = incl - mine;  // keys in bins of higher lanes
-        int cut = -1, above = 0;
-        const int s3 = above_lane, s2 = s3 + c3, s1x = s2 + c2, s0x = s1x + c1;
-        if (s3 < k_rem && k_rem <= s3 + c3) { cut = 4 * lane + 3; above = s3; }
-        else if (s2 < k_rem && k_rem <= s2 + c2) { cut = 4 * lane + 2; above = s2; }
-        else if (s1x < k_rem && k_rem <= s1x + c1) { cut = 4 * lane + 1; above = s1x; }
-        else if (s0x < k_rem && k_rem <= s0x + c0) { cut = 4 * lane; above = s0x; }
-        const unsigned long long who = __ballot(cut >= 0);
-        const int src = __ffsll((long long)who) - 1;
-        cut = __shfl(cut, src);
-        above = __shfl(above, src);
-        prefix = (prefix << 8) | (uint32_t)cut;
-        k_rem -= above;
+      for (int u = 0; u < 8; ++u) {
+        const int t = t0 + 64 * u + lane;
+        kk[u] = (t < n) ? krow[t] : 0u;
       }
-      tau = prefix;
-      quota = k_rem;
-    }
-    int base_above = 0, base_tie = 0;
-    for (int i0 = 0; i0 < n; i0 += 64) {
-      const int i = i0 + lane;
-      bool above = false, tie = false;
-      uint32_t key = 0;
-      if (i < n) {
-        key = score_key(row[i]);
-        if (take_all) above = true;
-        else { above = key > tau; tie = key == tau; }
-      }
-      const unsigned long long ma = __ballot(above), mt = __ballot(tie);
-      const unsigned long long lt = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
-      const int pa = base_above + __popcll(ma & lt), pt = base_tie + __popcll(mt & lt);
-      if (above || (tie && pt < quota)) {
-        const int pos = pa + min(pt, quota);
-        if (pos < Kc) {
-          ck[pos] = key;
-          ci[pos] = s0 + i;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int t = t0 + 64 * u + lane;
+        if (t < n) {
+          const uint32_t k = score_key(__builtin_bit_cast(float, kk[u]));
+          krow[t] = k;
+          kmin = min(kmin, k);
+          kmax = max(kmax, k);
         }
       }
-      base_above += __popcll(ma);
-      base_tie += __popcll(mt);
     }
-    if (lane == 0) p.cand_cnt[part_base + (size_t)h * p.n_splits] = min(Kc, base_above + min(base_tie, quota));
+    if (clk && tid == 0) clk[6] = clock64();
+    uint32_t T = 0;        // emit key > T (exact mode) or key >= T (bound mode)
+    int quota = 0;         // exact mode: ties to take
+    bool ge_mode = true;   // T = 0, ge: take everything (n <= Kcap)
+    if (n > Kcap) {
+      kmin = wave_min_u(kmin);
+      kmax = wave_max_u(kmax);
+      const uint32_t diff = kmin ^ kmax;
+      if (diff == 0u) {  // every key equal: the lowest positions win
+        T = kmax;
+        quota = Kt;
+        ge_mode = false;
+      } else {
+        int bits_left = 32 - __clz((int)diff);  // number of low bits that vary
+        uint32_t prefix = (bits_left == 32) ? 0u : (kmax >> bits_left);
+        int k_rem = Kt;
+        ge_mode = false;
+        while (bits_left > 0) {
+          const int nb = min(8, bits_left);
+          const int shift = bits_left - nb;
+          const uint32_t dmask = (1u << nb) - 1u;
+          for (int i = lane; i < 264; i += 64) hist[i] = 0;
+          const bool first = (bits_left == 32);
+          const int hi_shift = first ? 0 : bits_left;
+          for (int t0 = 0; t0 < n; t0 += 512) {
+            uint32_t kk[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+              const int t = t0 + 64 * u + lane;
+              kk[u] = (t < n) ? krow[t] : 0u;
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+              const int t = t0 + 64 * u + lane;
+              const bool inpre = (t < n) && (first || ((kk[u] >> hi_shift) == prefix));
+              atomicAdd(&hist[inpre ? (int)((kk[u] >> shift) & dmask) : 256], 1);
+            }
+          }
+          // lane l owns bins 255-4l .. 252-4l (descending), so a prefix scan over lanes counts the bins above
+          const int c3 = hist[255 - 4 * lane], c2 = hist[254 - 4 * lane], c1 = hist[253 - 4 * lane], c0 = hist[252 - 4 * lane];
+          const int mine = c0 + c1 + c2 + c3;
+          const int e3 = wave_incl_scan_i(mine) - mine;  // keys in bins above 255-4l
+          const int e2 = e3 + c3, e1 = e2 + c2, e0 = e1 + c1;
+          int cut = -1, above = 0, ccut = 0;
+          if (e3 < k_rem && k_rem <= e3 + c3) { cut = 255 - 4 * lane; above = e3; ccut = c3; }
+          else if (e2 < k_rem && k_rem <= e2 + c2) { cut = 254 - 4 * lane; above = e2; ccut = c2; }
+          else if (e1 < k_rem && k_rem <= e1 + c1) { cut = 253 - 4 * lane; above = e1; ccut = c1; }
+          else if (e0 < k_rem && k_rem <= e0 + c0) { cut = 252 - 4 * lane; above = e0; ccut = c0; }
+          const unsigned long long who = __ballot(cut >= 0);
+          const int src = __ffsll((long long)who) - 1;
+          cut = __builtin_amdgcn_readlane(cut, src);
+          above = __builtin_amdgcn_readlane(above, src);
+          ccut = __builtin_amdgcn_readlane(ccut, src);
+          prefix = (prefix << nb) | (uint32_t)cut;
+          k_rem -= above;
+          bits_left = shift;
+          if ((Kt - k_rem) + ccut <= Kcap) {  // the whole cut bin fits: stop here
+            ge_mode = true;
+            T = (bits_left == 0) ? prefix : (prefix << bits_left);
+            break;
+          }
+        }
+        if (!ge_mode) {
+          T = prefix;
+          quota = k_rem;
+        }
+      }
+    }
+    if (clk && tid == 0) { clk[7] = clock64(); clk[9] = ge_mode ? 1 : 0; }
+    int count = 0;
+    if (ge_mode) {
+      for (int t0 = 0; t0 < n; t0 += 512) {
+        uint32_t kk[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int t = t0 + 64 * u + lane;
+          kk[u] = (t < n) ? krow[t] : 0u;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int t = t0 + 64 * u + lane;
+          const bool above = (t < n) && (kk[u] >= T);
+          const unsigned long long ma = __ballot(above);
+          const int pos = count + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(ma >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)ma, 0u));
+          if (above && pos < Kcap) {
+            ck[pos] = kk[u];
+            ci[pos] = s0 + t;
+          }
+          count += __popcll(ma);
+        }
+      }
+    } else {
+      int base_tie = 0;
+      for (int t0 = 0; t0 < n; t0 += 64) {
+        const int t = t0 + lane;
+        const uint32_t k = (t < n) ? krow[t] : 0u;
+        const bool above = (t < n) && (k > T), tie = (t < n) && (k == T);
+        const unsigned long long ma = __ballot(above), mt = __ballot(tie);
+        const int pa = count + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(ma >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)ma, 0u));
+        const int pt = base_tie + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(mt >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mt, 0u));
+        if (above || (tie && pt < quota)) {
+          const int pos = pa + min(pt, quota);
+          if (pos < Kcap) {
+            ck[pos] = k;
+            ci[pos] = s0 + t;
+          }
+        }
+        count += __popcll(ma);
+        base_tie += __popcll(mt);
+      }
+      count += min(base_tie, quota);
+    }
+    if (clk && tid == 0) clk[8] = clock64();
+    if (lane == 0) p.cand_cnt[part_base + (size_t)h * p.n_splits] = min(Kcap, count);
   }
+  if (clk && tid == 0) clk[5] = clock64();
 }
 
 // ---------------------------------------------------------------------------------------------------
-constexpr int MG_THREADS = 256;
+constexpr int MG_THREADS = 1024;
 constexpr int MG_WAVES = MG_THREADS / 64;
+constexpr int MG_HIST = MG_WAVES / 2;
+constexpr int MG_MAX_SPLITS = 256;
+constexpr int MG_LDS_KEYS = 8192;  // candidate keys cached in LDS when they fit
 
 template <int VBITS, int NG>
 __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) {
   constexpr int VP = D * VBITS / 8;
   constexpr int VOFF = 1 << (VBITS - 1);
-  __shared__ int hist[MG_WAVES][256];
+  constexpr int DW = VP / 4;            // dwords per V row
+  constexpr int CPD = 32 / VBITS;       // codes per dword
+  constexpr int WPI = 64 / DW;          // winners per wavefront instruction
+  __shared__ uint32_t keys_sh[MG_LDS_KEYS];
+  __shared__ int hist[MG_HIST][256];  // one histogram per pair of wavefronts
   __shared__ int suffix_wave[4];
   __shared__ int cut_bin_sh, above_sh;
   __shared__ int wave_above[MG_WAVES], wave_tie[MG_WAVES];
-  __shared__ float coef_sh[1024];
+  __shared__ float coef_sh[MG_MAX_SPLITS];
   __shared__ float stat_sh[2];
-  __shared__ int64_t slot_buf[128];
-  __shared__ float ws_buf[128][NG];
-  __shared__ float w_buf[128];
+  __shared__ int cnt_sh[MG_MAX_SPLITS];
+  __shared__ int win_slot[FS_MAX_TOPK];
+  __shared__ float win_w[FS_MAX_TOPK];
+  __shared__ float old_sh[MG_WAVES][D];
+  __shared__ float w_sh[MG_WAVES];
 
   const int b = blockIdx.x, hq = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const size_t bh = (size_t)b * p.H_q + hq;
@@ -597,23 +897,26 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   int64_t* out_idx = p.topk_idx + bh * (size_t)K;
   int64_t* out_slot = p.topk_slots + bh * (size_t)K;
 
-  // ---- split statistics: M, l, coefficients
+  long long* mclk = p.phase_clock ? p.phase_clock + (size_t)p.B * p.H_kv * p.n_splits * 10 + bh * 8 : nullptr;
+  if (mclk && tid == 0) mclk[0] = clock64();
+  // ---- split statistics: M, coefficients e^{m_i - M}, l
   float mloc = -INFINITY;
   for (int s = tid; s < NS; s += MG_THREADS) mloc = fmaxf(mloc, p.part_m[bh * NS + s]);
   mloc = wave_max(mloc);
-  if (lane == 0) coef_sh[wave] = mloc;
+  if (lane == 0) hist[0][wave] = __builtin_bit_cast(int, mloc);
   __syncthreads();
-  float M = fmaxf(fmaxf(coef_sh[0], coef_sh[1]), fmaxf(coef_sh[2], coef_sh[3]));
+  float M = -INFINITY;
+#pragma unroll
+  for (int w = 0; w < MG_WAVES; ++w) M = fmaxf(M, __builtin_bit_cast(float, hist[0][w]));
   if (!isfinite(M)) M = 0.f;
+  for (int s = tid; s < NS; s += MG_THREADS) {
+    const float ms = p.part_m[bh * NS + s];
+    coef_sh[s] = (ms == -INFINITY) ? 0.f : __expf(ms - M);
+  }
   __syncthreads();
   if (tid == 0) {
     float l = 0.f;
-    for (int s = 0; s < NS; ++s) {  // fixed order: deterministic
-      const float ms = p.part_m[bh * NS + s];
-      const float c = (ms == -INFINITY) ? 0.f : __expf(ms - M);
-      if (s < 1024) coef_sh[s] = c;
-      l += p.part_l[bh * NS + s] * c;
-    }
+    for (int s = 0; s < NS; ++s) l = __builtin_fmaf(p.part_l[bh * NS + s], coef_sh[s], l);  // fixed order
     stat_sh[0] = l;
     stat_sh[1] = (l > 0.f) ? 1.0f / l : 0.f;
   }
@@ -629,143 +932,288 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
     p.softmax_inv_z[bh] = inv_z;
   }
 
-  // ---- global top-k among the candidates
-  int total = 0;
-  for (int s = 0; s < NS; ++s) total += cc[s];  // uniform scalar loop (NS <= 1024)
+  if (mclk && tid == 0) mclk[1] = clock64();
+  // ---- global top-k among the candidates (flat index f = split * Kc + j, valid when j < cnt[split])
   const int flat = NS * Kc;
+  const bool in_lds = flat <= MG_LDS_KEYS;
+  for (int s2 = tid; s2 < NS; s2 += MG_THREADS) cnt_sh[s2] = cc[s2];
+  __syncthreads();
+  int total = 0;
+  for (int s2 = 0; s2 < NS; ++s2) total += cnt_sh[s2];
+  if (in_lds) {  // unused slots become key 0, which no finite score maps to
+    for (int f0 = 0; f0 < flat; f0 += 4 * MG_THREADS) {
+      uint32_t kv[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int f = f0 + u * MG_THREADS + tid;
+        kv[u] = 0u;
+        if (f < flat) {
+          const int s2 = f / Kc;
+          if (f - s2 * Kc < cnt_sh[s2]) kv[u] = ck[f];
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int f = f0 + u * MG_THREADS + tid;
+        if (f < flat) keys_sh[f] = kv[u];
+      }
+    }
+  }
+  __syncthreads();
+  auto cand_key = [&](int f, bool& ok) -> uint32_t {
+    if (in_lds) {
+      const uint32_t k = keys_sh[f];
+      ok = k != 0u;
+      return k;
+    }
+    const int s2 = f / Kc;
+    ok = (f - s2 * Kc) < cnt_sh[s2];
+    return ok ? ck[f] : 0u;
+  };
+  if (mclk && tid == 0) mclk[2] = clock64();
   uint32_t tau = 0;
   int quota = 0;
   const bool take_all = (total <= K);
   if (!take_all) {
-    uint32_t prefix = 0;
+    // bits shared by every candidate key are skipped (the candidates are the upper tail of the row, so sign and
+    // exponent usually agree); the remaining bits are resolved 8 at a time
+    uint32_t kmin = 0xffffffffu, kmax = 0u;
+    for (int f = tid; f < flat; f += MG_THREADS) {
+      bool ok;
+      const uint32_t key = cand_key(f, ok);
+      if (ok) { kmin = min(kmin, key); kmax = max(kmax, key); }
+    }
+    kmin = wave_min_u(kmin);
+    kmax = wave_max_u(kmax);
+    if (lane == 0) { hist[0][wave] = (int)kmin; hist[1][wave] = (int)kmax; }
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < MG_WAVES; ++w) { kmin = min(kmin, (uint32_t)hist[0][w]); kmax = max(kmax, (uint32_t)hist[1][w]); }
+    __syncthreads();
+    const uint32_t diff = kmin ^ kmax;
+    int bits_left = (diff == 0u) ? 0 : 32 - __clz((int)diff);
+    uint32_t prefix = (bits_left == 32) ? 0u : (kmax >> bits_left);
     int k_rem = K;
-    for (int level = 0; level < 4; ++level) {
-      for (int i = tid; i < MG_WAVES * 256; i += MG_THREADS) (&hist[0][0])[i] = 0;
+    while (bits_left > 0) {
+      const int nb = min(8, bits_left);
+      const int shift = bits_left - nb;
+      const uint32_t dmask = (1u << nb) - 1u;
+      const bool first = (bits_left == 32);
+      const int hi_shift = first ? 0 : bits_left;
+      for (int i = tid; i < MG_HIST * 256; i += MG_THREADS) (&hist[0][0])[i] = 0;
       __syncthreads();
-      const int shift = 24 - 8 * level;
       for (int f = tid; f < flat; f += MG_THREADS) {
-        if ((f % Kc) < cc[f / Kc]) {
-          const uint32_t key = ck[f];
-          if (level == 0 || (key >> (shift + 8)) == prefix) atomicAdd(&hist[wave][(key >> shift) & 255u], 1);
+        bool ok;
+        const uint32_t key = cand_key(f, ok);
+        if (ok && (first || (key >> hi_shift) == prefix)) atomicAdd(&hist[wave >> 1][(key >> shift) & dmask], 1);
+      }
+      __syncthreads();
+      if (tid < 256) {
+        // thread tid covers bin 255 - tid, so an inclusive scan over threads counts the keys in bins >= it
+        const int bin = 255 - tid;
+        int rcnt = 0;
+#pragma unroll
+        for (int w = 0; w < MG_HIST; ++w) rcnt += hist[w][bin];
+        const int incl_r = wave_incl_scan_i(rcnt);
+        if (lane == 63) suffix_wave[wave] = incl_r;
+        hist[0][bin] = rcnt;      // own bin only: keep the totals for the second step
+        hist[1][bin] = incl_r;
+      }
+      __syncthreads();
+      if (tid < 256) {
+        const int bin = 255 - tid;
+        int before = 0;
+        for (int w = 0; w < wave; ++w) before += suffix_wave[w];
+        const int s_incl = hist[1][bin] + before, s_excl = s_incl - hist[0][bin];
+        if (s_excl < k_rem && k_rem <= s_incl) {
+          cut_bin_sh = bin;
+          above_sh = s_excl;
         }
       }
       __syncthreads();
-      int cnt = hist[0][tid] + hist[1][tid] + hist[2][tid] + hist[3][tid];  // MG_THREADS == 256 bins
-      int incl = cnt;
-#pragma unroll
-      for (int off = 1; off < 64; off <<= 1) {
-        const int o = __shfl_down(incl, off);
-        if (lane + off < 64) incl += o;
-      }
-      if (lane == 0) suffix_wave[wave] = incl;
-      __syncthreads();
-      int higher = 0;
-      for (int w = wave + 1; w < 4; ++w) higher += suffix_wave[w];
-      const int s_incl = incl + higher, s_excl = s_incl - cnt;
-      if (s_excl < k_rem && k_rem <= s_incl) {
-        cut_bin_sh = tid;
-        above_sh = s_excl;
-      }
-      __syncthreads();
-      prefix = (prefix << 8) | (uint32_t)cut_bin_sh;
+      prefix = (prefix << nb) | (uint32_t)cut_bin_sh;
       k_rem -= above_sh;
+      bits_left = shift;
       __syncthreads();
     }
     tau = prefix;
     quota = k_rem;
   }
+  if (mclk && tid == 0) mclk[3] = clock64();
+  // ordered compaction: winners' candidate ids go to LDS in ascending position order.  Pass 1 stores every
+  // (round, wavefront) count, one thread-block scan turns them into offsets, pass 2 places the winners:
+  // two barriers instead of two per round.
+  constexpr int MAX_ROUNDS = MG_LDS_KEYS / MG_THREADS;  // rounds handled by the batched path
+  const int rounds = (flat + MG_THREADS - 1) / MG_THREADS;
   int base_above = 0, base_tie = 0;
-  const int flat_round = (flat + MG_THREADS - 1) / MG_THREADS * MG_THREADS;
-  for (int f0 = 0; f0 < flat_round; f0 += MG_THREADS) {
-    const int f = f0 + tid;
-    bool above = false, tie = false;
-    if (f < flat && (f % Kc) < cc[f / Kc]) {
-      if (take_all) above = true;
-      else {
-        const uint32_t key = ck[f];
-        above = key > tau;
-        tie = key == tau;
-      }
-    }
-    const unsigned long long ma = __ballot(above), mt = __ballot(tie);
-    const unsigned long long lt = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
-    if (lane == 0) {
-      wave_above[wave] = __popcll(ma);
-      wave_tie[wave] = __popcll(mt);
-    }
-    __syncthreads();
-    int pa = base_above + __popcll(ma & lt), pt = base_tie + __popcll(mt & lt);
-    int tot_a = 0, tot_t = 0;
+  if (rounds <= MAX_ROUNDS) {
+    int* cnt_a = &hist[0][0];                 // [rounds][MG_WAVES]
+    int* cnt_t = &hist[0][0] + MAX_ROUNDS * MG_WAVES;
+    unsigned long long ma_r[MAX_ROUNDS], mt_r[MAX_ROUNDS];
 #pragma unroll
-    for (int w = 0; w < MG_WAVES; ++w) {
-      if (w < wave) { pa += wave_above[w]; pt += wave_tie[w]; }
-      tot_a += wave_above[w];
-      tot_t += wave_tie[w];
-    }
-    if (above || (tie && pt < quota)) {
-      const int pos = pa + min(pt, quota);
-      if (pos < K) out_idx[pos] = ((int64_t)f << 32) | (uint32_t)ci[f];  // provisional: candidate id + position
-    }
-    base_above += tot_a;
-    base_tie += tot_t;
-    __syncthreads();
-  }
-  const int n_out = min(K, base_above + min(base_tie, quota));
-  __syncthreads();
-
-  // ---- winners: finalise indices/slots and the pre-correction terms
-  const int grp = (NG == 1) ? 0 : ((tid & (D - 1)) / (D / NG));
-  const uint8_t* vbase = p.v_data + (size_t)hkv * p.num_slots * VP;
-  const uint16_t* vsbase = p.v_scales + (size_t)hkv * p.num_slots * NG;
-  const int dch = tid & (D - 1), half = tid >> 7;  // two halves of the 256 threads split the winners
-  float acc_old = 0.f, acc_w = 0.f;
-  for (int k0 = 0; k0 < K; k0 += 128) {
-    __syncthreads();
-    if (tid < 128) {
-      const int kk = k0 + tid;
-      int64_t slot = -1;
-      float w = 0.f;
-      if (kk < K) {
-        if (kk < n_out) {
-          const int64_t packed = out_idx[kk];
-          const int f = (int)(packed >> 32);
-          const int pos = (int)(packed & 0xffffffffll);
-          const int blk = pos / BS;
-          slot = (blk < p.max_blocks) ? bt[blk] * BS + (pos % BS) : -1;
-          out_idx[kk] = pos;
-          out_slot[kk] = slot;
-          if (slot >= 0) w = __expf(key_to_score(ck[f]) - M) * inv_z;
-        } else {
-          out_idx[kk] = -1;
-          out_slot[kk] = -1;
+    for (int r = 0; r < MAX_ROUNDS; ++r) {
+      ma_r[r] = 0ull; mt_r[r] = 0ull;
+      if (r < rounds) {
+        const int f = r * MG_THREADS + tid;
+        bool above = false, tie = false;
+        if (f < flat) {
+          bool ok;
+          const uint32_t key = cand_key(f, ok);
+          if (ok) {
+            if (take_all) above = true;
+            else { above = key > tau; tie = key == tau; }
+          }
+        }
+        ma_r[r] = __ballot(above);
+        mt_r[r] = __ballot(tie);
+        if (lane == 0) {
+          cnt_a[r * MG_WAVES + wave] = __popcll(ma_r[r]);
+          cnt_t[r * MG_WAVES + wave] = __popcll(mt_r[r]);
         }
       }
-      slot_buf[tid] = slot;
-      w_buf[tid] = w;
-#pragma unroll
-      for (int g = 0; g < NG; ++g) ws_buf[tid][g] = (slot >= 0) ? w * bf16_to_f32(vsbase[slot * NG + g]) : 0.f;
     }
     __syncthreads();
-    const int kend = min(128, K - k0);
-    for (int j = half; j < kend; j += 2) {
-      const int64_t slot = slot_buf[j];
-      if (slot < 0) continue;
-      const uint8_t* vr = vbase + slot * VP;
-      int c;
-      if (VBITS == 2) c = (int)((vr[dch >> 2] >> ((3 - (dch & 3)) * 2)) & 3) - VOFF;
-      else c = (int)((vr[dch >> 1] >> ((1 - (dch & 1)) * 4)) & 15) - VOFF;
-      acc_old = __builtin_fmaf(ws_buf[j][grp], (float)c, acc_old);
-      acc_w += w_buf[j];
+    if (wave == 0) {  // exclusive scan of the (round, wave) counts, 2 entries per lane (MAX_ROUNDS*MG_WAVES == 128)
+      const int n_ent = rounds * MG_WAVES;
+      const int i0 = 2 * lane, i1 = 2 * lane + 1;
+      const int a0 = (i0 < n_ent) ? cnt_a[i0] : 0, a1 = (i1 < n_ent) ? cnt_a[i1] : 0;
+      const int t0 = (i0 < n_ent) ? cnt_t[i0] : 0, t1 = (i1 < n_ent) ? cnt_t[i1] : 0;
+      const int ia = wave_incl_scan_i(a0 + a1), it = wave_incl_scan_i(t0 + t1);
+      if (i0 < n_ent) { cnt_a[i0] = ia - a0 - a1; cnt_t[i0] = it - t0 - t1; }
+      if (i1 < n_ent) { cnt_a[i1] = ia - a1; cnt_t[i1] = it - t1; }
+      if (lane == 63) { cut_bin_sh = ia; above_sh = it; }  // totals
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < MAX_ROUNDS; ++r) {
+      if (r < rounds) {
+        const int f = r * MG_THREADS + tid;
+        const unsigned long long ma = ma_r[r], mt = mt_r[r];
+        const bool above = (ma >> lane) & 1ull, tie = (mt >> lane) & 1ull;
+        const int pa = cnt_a[r * MG_WAVES + wave] + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(ma >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)ma, 0u));
+        const int pt = cnt_t[r * MG_WAVES + wave] + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(mt >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mt, 0u));
+        if (above || (tie && pt < quota)) {
+          const int pos = pa + min(pt, quota);
+          if (pos < K) win_slot[pos] = f;  // candidate id for now
+        }
+      }
+    }
+    base_above = cut_bin_sh;
+    base_tie = above_sh;
+    __syncthreads();
+  } else {
+    for (int r = 0; r < rounds; ++r) {
+      const int f = r * MG_THREADS + tid;
+      bool above = false, tie = false;
+      if (f < flat) {
+        bool ok;
+        const uint32_t key = cand_key(f, ok);
+        if (ok) {
+          if (take_all) above = true;
+          else { above = key > tau; tie = key == tau; }
+        }
+      }
+      const unsigned long long ma = __ballot(above), mt = __ballot(tie);
+      if (lane == 0) {
+        wave_above[wave] = __popcll(ma);
+        wave_tie[wave] = __popcll(mt);
+      }
+      __syncthreads();
+      int pa = base_above + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(ma >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)ma, 0u));
+      int pt = base_tie + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(mt >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mt, 0u));
+      int tot_a = 0, tot_t = 0;
+#pragma unroll
+      for (int w = 0; w < MG_WAVES; ++w) {
+        if (w < wave) { pa += wave_above[w]; pt += wave_tie[w]; }
+        tot_a += wave_above[w];
+        tot_t += wave_tie[w];
+      }
+      if (above || (tie && pt < quota)) {
+        const int pos = pa + min(pt, quota);
+        if (pos < K) win_slot[pos] = f;
+      }
+      base_above += tot_a;
+      base_tie += tot_t;
+      __syncthreads();
     }
   }
-  // combine the two halves (fixed order)
+  const int n_out = min(K, base_above + min(base_tie, quota));
+  // one thread per winner: position, paged slot, softmax weight (all loads independent); entry r of
+  // win_slot is read and rewritten by thread r only
+  for (int r = tid; r < K; r += MG_THREADS) {
+    int64_t position = -1, slot = -1;
+    int wslot = -1;
+    float ww = 0.f;
+    if (r < n_out) {
+      const int f = win_slot[r];
+      position = ci[f];
+      const int blk = (int)(position / BS);
+      slot = (blk < p.max_blocks) ? bt[blk] * BS + (position % BS) : -1;
+      wslot = (slot >= 0 && slot < p.num_slots) ? (int)slot : -1;
+      ww = __expf(key_to_score(ck[f]) - M) * inv_z;
+    }
+    out_idx[r] = position;
+    out_slot[r] = slot;
+    win_slot[r] = wslot;
+    win_w[r] = ww;
+  }
   __syncthreads();
-  float* comb = coef_sh;  // reuse: [2][D] + [2]
-  comb[half * D + dch] = acc_old;
-  if (dch == 0) comb[2 * D + half] = acc_w;
+
+  if (mclk && tid == 0) mclk[4] = clock64();
+  // ---- pre-correction over the winners.  One winner row per DW lanes: lane (w_in, dwi) holds dword dwi of
+  // the winner's packed V row (CPD codes) and accumulates its CPD channels; winners are visited in a fixed
+  // order, so the sums are run-to-run deterministic.
+  const uint8_t* vbase = p.v_data + (size_t)hkv * p.num_slots * VP;
+  const uint16_t* vsbase = p.v_scales + (size_t)hkv * p.num_slots * NG;
+  const int dwi = lane % DW, w_in = lane / DW;
+  float acc[CPD];
+#pragma unroll
+  for (int c = 0; c < CPD; ++c) acc[c] = 0.f;
+  float accw = 0.f;
+  for (int k0 = wave * WPI; k0 < n_out; k0 += MG_WAVES * WPI) {
+    const int k = k0 + w_in;
+    const int slot = (k < n_out) ? win_slot[k] : -1;
+    if (slot >= 0) {
+      const float w = win_w[k];
+      const uint32_t word = reinterpret_cast<const uint32_t*>(vbase + (size_t)slot * VP)[dwi];
+      const int g = (NG == 1) ? 0 : ((dwi * CPD) / (D / NG));
+      const float ws = w * bf16_to_f32(vsbase[(size_t)slot * NG + g]);
+      // byte `byte` of the dword holds its codes MSB first; channel of code c in the dword = dwi*CPD + c
+#pragma unroll
+      for (int c = 0; c < CPD; ++c) {
+        const int byte = c / (8 / VBITS), inb = c % (8 / VBITS);
+        const int code = (int)((word >> (8 * byte + (8 - VBITS * (inb + 1)))) & ((1u << VBITS) - 1u)) - VOFF;
+        acc[c] = __builtin_fmaf(ws, (float)code, acc[c]);
+      }
+      if (dwi == 0) accw += w;
+    }
+  }
+  // reduce over the WPI winners of a wavefront instruction (lanes with equal dwi), then over wavefronts
+#pragma unroll
+  for (int off = DW; off < 64; off <<= 1) {
+#pragma unroll
+    for (int c = 0; c < CPD; ++c) acc[c] += __shfl_xor(acc[c], off);
+    accw += __shfl_xor(accw, off);
+  }
+  if (w_in == 0) {
+#pragma unroll
+    for (int c = 0; c < CPD; ++c) old_sh[wave][dwi * CPD + c] = acc[c];
+    if (dwi == 0) w_sh[wave] = accw;
+  }
   __syncthreads();
-  if (tid < D) p.o_old[bh * D + tid] = comb[tid] + comb[D + tid];
-  if (tid == 0) p.W[bh] = comb[2 * D] + comb[2 * D + 1];
+  if (tid < D) {
+    float o = 0.f;
+#pragma unroll
+    for (int w = 0; w < MG_WAVES; ++w) o += old_sh[w][tid];  // fixed order
+    p.o_old[bh * D + tid] = o;
+  }
+  if (tid == 0) {
+    float o = 0.f;
+#pragma unroll
+    for (int w = 0; w < MG_WAVES; ++w) o += w_sh[w];
+    p.W[bh] = o;
+  }
+  if (mclk && tid == 0) mclk[5] = clock64();
 }
 
 // Optional measurement hook: when armed, every fused_scan_kernel launch is bracketed by a pair of HIP
@@ -776,24 +1224,53 @@ struct ScanProfile {
   bool armed = false;
 };
 ScanProfile g_prof;
+long long* g_phase_clock = nullptr;
 
-inline int lmax_for_group(int G) { return G <= 4 ? 2048 : (G <= 8 ? 1024 : 512); }
+constexpr size_t LDS_BUDGET_2WG = 79 * 1024;    // two workgroups per CU (160 KB LDS)
+constexpr size_t LDS_BUDGET_1WG = 158 * 1024;
 
-inline void fused_plan(int B, int H_q, int H_kv, int max_S, int top_k, int* L_out, int* ns_out, int* kc_out) {
+template <int SCHEME, int G, int NG>
+int lmax_for() {
+  using Lds = ScanLds<SCHEME, G, NG>;
+  const size_t budget = (G <= 4) ? LDS_BUDGET_2WG : LDS_BUDGET_1WG;
+  const size_t fixed = Lds::stage_bytes() + 64 + 1024;  // + static LDS of the kernel
+  long lm = (long)((budget - fixed) / (Lds::per_position() + 1));  // +1: page table (4 bytes per 16 positions)
+  lm = lm / 256 * 256;
+  if (lm > FS_LMAX) lm = FS_LMAX;
+  if (lm < 256) lm = 256;
+  return (int)lm;
+}
+
+inline int lmax_dispatch(int scheme, int G, int NG) {
+#define JF_LMAX_CASE(SCH, GG, NGG) if (scheme == SCH && G == GG && NG == NGG) return lmax_for<SCH, GG, NGG>()
+  JF_LMAX_CASE(JF_SCHEME_K3V2, 1, 1); JF_LMAX_CASE(JF_SCHEME_K3V2, 2, 1); JF_LMAX_CASE(JF_SCHEME_K3V2, 4, 1);
+  JF_LMAX_CASE(JF_SCHEME_K3V2, 8, 1); JF_LMAX_CASE(JF_SCHEME_K3V2, 16, 1);
+  JF_LMAX_CASE(JF_SCHEME_K3V2, 1, 2); JF_LMAX_CASE(JF_SCHEME_K3V2, 2, 2); JF_LMAX_CASE(JF_SCHEME_K3V2, 4, 2);
+  JF_LMAX_CASE(JF_SCHEME_K3V2, 8, 2); JF_LMAX_CASE(JF_SCHEME_K3V2, 16, 2);
+  JF_LMAX_CASE(JF_SCHEME_K4V4, 1, 1); JF_LMAX_CASE(JF_SCHEME_K4V4, 2, 1); JF_LMAX_CASE(JF_SCHEME_K4V4, 4, 1);
+  JF_LMAX_CASE(JF_SCHEME_K4V4, 8, 1); JF_LMAX_CASE(JF_SCHEME_K4V4, 16, 1);
+#undef JF_LMAX_CASE
+  return 256;
+}
+
+inline void fused_plan(int scheme, int NG, int B, int H_q, int H_kv, int max_S, int top_k, int* L_out, int* ns_out,
+                       int* kc_out) {
   const int G = H_q / H_kv;
   const int units = B * H_kv > 0 ? B * H_kv : 1;
-  int target = 512 / units;
+  const int wg_target = (G <= 4) ? 512 : 256;  // two (one) resident workgroups per CU on 256 CUs
+  int target = wg_target / units;
   if (target < 1) target = 1;
   int L = (max_S + target - 1) / target;
   L = (L + 255) / 256 * 256;
-  const int lmax = lmax_for_group(G);
+  const int lmax = lmax_dispatch(scheme, G, NG);
   if (L > lmax) L = lmax;
   if (L < 256) L = 256;
   int ns = (max_S + L - 1) / L;
   if (ns < 1) ns = 1;
   *L_out = L;
   *ns_out = ns;
-  *kc_out = top_k < L ? top_k : L;
+  const int cap = top_k + FS_CAND_SLACK;  // the split may emit a superset of its top-k (see phase C)
+  *kc_out = cap < L ? cap : L;
 }
 
 struct WsLayout {
@@ -816,15 +1293,7 @@ inline WsLayout ws_layout(int B, int H_q, int ns, int kc) {
 
 template <int SCHEME, int G, int NG>
 int launch_scan(const FusedParams& p, hipStream_t st) {
-  constexpr bool K3 = (SCHEME == JF_SCHEME_K3V2);
-  constexpr int NSET = (G + 3) / 4;
-  constexpr int VROW = (K3 ? 32 : 64) + 8;
-  size_t stage = (size_t)FS_THREADS * VROW + (size_t)FS_WAVES * NG * NSET * 16 * 64;
-  const size_t red = (size_t)NSET * 8 * 256 * 4;
-  if (red > stage) stage = red;
-  const size_t qsz = sizeof(QInt8F<G>) + G * 4 * sizeof(float);
-  if (!K3 && qsz > stage) stage = qsz;
-  const size_t smem = (size_t)G * p.L * sizeof(float) + stage;
+  const size_t smem = ScanLds<SCHEME, G, NG>::total(p.L);
   auto kern = fused_scan_kernel<SCHEME, G, NG>;
   static size_t attr_smem = 0;  // per instantiation: raise the dynamic-LDS limit only when it grows
   if (smem > attr_smem) {
@@ -842,17 +1311,24 @@ int launch_scan(const FusedParams& p, hipStream_t st) {
   return JF_OK;
 }
 
+inline int scheme_ng(int scheme, int group_size) { return (scheme == JF_SCHEME_K4V4) ? 1 : D / group_size; }
+
 }  // namespace
 }  // namespace jf
 
 using namespace jf;
 
 extern "C" size_t jf_fused_workspace_bytes(int scheme, int B, int H_q, int H_kv, int max_S, int top_k) {
-  (void)scheme;
   if (B <= 0 || H_q <= 0 || H_kv <= 0 || H_q % H_kv != 0 || max_S < 0 || top_k <= 0) return 256;
-  int L, ns, kc;
-  fused_plan(B, H_q, H_kv, max_S, top_k, &L, &ns, &kc);
-  return ws_layout(B, H_q, ns, kc).total;
+  // the split length depends on the group size only through the LDS budget; size for the worst case
+  size_t worst = 0;
+  for (int ng = 1; ng <= 2; ++ng) {
+    int L, ns, kc;
+    fused_plan(scheme, ng, B, H_q, H_kv, max_S, top_k, &L, &ns, &kc);
+    const size_t t = ws_layout(B, H_q, ns, kc).total;
+    if (t > worst) worst = t;
+  }
+  return worst;
 }
 
 extern "C" int jf_fused_scan_topk(int scheme, int group_size, const uint16_t* q, const uint8_t* k_data,
@@ -869,22 +1345,26 @@ extern "C" int jf_fused_scan_topk(int scheme, int group_size, const uint16_t* q,
   JF_CHECK_ARG(block_size == 16, "fused_scan only supports block_size=16");
   JF_CHECK_ARG(group_size == 64 || group_size == 128, "fused_scan: group_size must be 64 or 128 (got %d)", group_size);
   JF_CHECK_ARG(scheme != JF_SCHEME_K4V4 || group_size == 128, "fused_scan: the INT4 int8-Q path needs group_size 128");
-  JF_CHECK_ARG(is_pow2(top_k) && top_k >= 32 && top_k <= 8192, "fused_scan: unsupported top_k=%d", top_k);
+  JF_CHECK_ARG(is_pow2(top_k) && top_k >= 32 && top_k <= FS_MAX_TOPK,
+               "fused_scan: unsupported top_k=%d (supported: 32,64,128,256,512,1024; larger widths use the split-form operators)", top_k);
   JF_CHECK_ARG(max_S <= 262144, "fused_scan: max_S=%d exceeds supported limit (262144)", max_S);
   JF_CHECK_ARG((int64_t)max_blocks * block_size >= max_S, "fused_scan: block_table does not cover max_S");
+  JF_CHECK_ARG(num_slots > 0 && num_slots < (1ll << 31), "fused_scan: num_slots out of range");
   JF_CHECK_ARG((softmax_m == nullptr) == (softmax_inv_z == nullptr), "fused_scan: softmax_m and softmax_inv_z go together");
   if (B == 0) return JF_OK;
   JF_CHECK_ARG(q && k_data && k_scales && v_data && v_scales && block_table && seq_lens, "fused_scan: null input");
   JF_CHECK_ARG(topk_idx && topk_slots && o_hat && o_old_unnorm && W, "fused_scan: null output");
-  JF_CHECK_ARG(((uintptr_t)k_data & 15) == 0 && ((uintptr_t)v_data & 15) == 0 && ((uintptr_t)q & 15) == 0,
-               "fused_scan: q, k_data and v_data must be 16-byte aligned");
+  JF_CHECK_ARG(((uintptr_t)k_data & 15) == 0 && ((uintptr_t)v_data & 15) == 0 && ((uintptr_t)q & 15) == 0 &&
+                   ((uintptr_t)v_scales & 3) == 0,
+               "fused_scan: q, k_data and v_data must be 16-byte aligned, v_scales 4-byte aligned");
+  const int NGv = scheme_ng(scheme, group_size);
   FusedParams p;
   p.q = q; p.k_data = k_data; p.k_scales = k_scales; p.v_data = v_data; p.v_scales = v_scales;
   p.block_table = block_table; p.seq_lens = seq_lens;
   p.B = B; p.H_q = H_q; p.H_kv = H_kv; p.max_S = max_S; p.max_blocks = max_blocks; p.num_slots = num_slots;
   p.attn_scale = attn_scale; p.top_k = top_k;
-  fused_plan(B, H_q, H_kv, max_S, top_k, &p.L, &p.n_splits, &p.Kc);
-  JF_CHECK_ARG(p.n_splits <= 1024, "fused_scan: too many splits (%d)", p.n_splits);
+  fused_plan(scheme, NGv, B, H_q, H_kv, max_S, top_k, &p.L, &p.n_splits, &p.Kc);
+  JF_CHECK_ARG(p.n_splits <= MG_MAX_SPLITS, "fused_scan: too many splits (%d > %d)", p.n_splits, MG_MAX_SPLITS);
   const WsLayout wl = ws_layout(B, H_q, p.n_splits, p.Kc);
   JF_CHECK_ARG(workspace && workspace_bytes >= wl.total, "fused_scan: workspace too small (%zu < %zu)", workspace_bytes, wl.total);
   JF_CHECK_ARG(((uintptr_t)workspace & 255) == 0, "fused_scan: workspace must be 256-byte aligned");
@@ -898,8 +1378,8 @@ extern "C" int jf_fused_scan_topk(int scheme, int group_size, const uint16_t* q,
   p.cand_cnt = reinterpret_cast<int32_t*>(ws + wl.off_cnt);
   p.topk_idx = topk_idx; p.topk_slots = topk_slots; p.o_hat = o_hat; p.o_old = o_old_unnorm; p.W = W;
   p.softmax_m = softmax_m; p.softmax_inv_z = softmax_inv_z;
+  p.phase_clock = g_phase_clock;
   hipStream_t st = (hipStream_t)stream;
-  const int NGv = D / group_size;
   int rc = JF_OK;
 #define JF_FUSED_CASE(SCH, GG, NGG) rc = launch_scan<SCH, GG, NGG>(p, st)
   if (scheme == JF_SCHEME_K3V2) {
@@ -966,5 +1446,10 @@ extern "C" int jf_profile_scan_end(double* total_ms, int* launches) {
   for (hipEvent_t e : g_prof.ev) (void)hipEventDestroy(e);
   g_prof.ev.clear();
   g_prof.used = 0;
+  return JF_OK;
+}
+
+extern "C" int jf_debug_phase_clock(void* device_buffer) {
+  g_phase_clock = reinterpret_cast<long long*>(device_buffer);
   return JF_OK;
 }
