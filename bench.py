@@ -71,6 +71,8 @@ def main() -> int:
     ap.add_argument("--paged", action="store_true", help="random block table instead of the identity mapping")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--graph", action="store_true", help="replay the step from a HIP graph (roofline timing stays eager)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run a plain 1 GiB device copy 10 times and exit (reference for the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path runs on ONE GPU (no sharding, no collectives); --gpus must be 1", file=sys.stderr)
@@ -84,6 +86,14 @@ def main() -> int:
 
     lib = _lib.load()
     torch.cuda.set_device(0)
+    if args.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(10):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibrate_copy_bytes_read": 1 << 30, "calibrate_copy_bytes_written": 1 << 30, "launches": 10}))
+        return 0
     w = workloads.build(args.workload, n_layers=args.layers)
     n_layers = len(w.layers)
     o_new = torch.zeros(w.B, w.H_q, 128, dtype=torch.bfloat16, device="cuda")
