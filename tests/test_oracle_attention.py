@@ -200,3 +200,35 @@ def test_reference_select_top_k_table_and_head_map():
     assert hm.shape == (2, 32, 256) and hm.flags["C_CONTIGUOUS"]
     for h in range(32):
         assert (hm[:, h] == h // 8).all()
+
+
+@pytest.mark.parametrize("kbits,vbits,gs", [(3, 2, 64), (4, 4, 128)])
+def test_torch_cpu_path_agrees_with_the_numpy_oracle(kbits, vbits, gs):
+    """The torch restatement timed as the CPU baseline: its unpack is bit-equal to the oracle's bf16
+    dequant, and its dense attention + top-k agree with the oracle's bf16-dequant model."""
+    import torch
+    from oracle import torch_cpu_path as T
+    from tests.helpers import bf16_tensor, bits_to_bf16, bf16_to_bits
+    B, Hq, Hkv, S, K = 1, 8, 2, 160, 32
+    c = make_case(21, B, Hq, Hkv, S, kbits, vbits, gs, ragged=False, shuffle=False)
+    kd, vd = torch.from_numpy(c["kd"]), torch.from_numpy(c["vd"])
+    ks, vs = bits_to_bf16(c["ks"]), bits_to_bf16(c["vs"])
+    for data, sc, nb, npd, nps in ((kd, ks, kbits, c["kd"], c["ks"]), (vd, vs, vbits, c["vd"], c["vs"])):
+        got = bf16_to_bits(T.unpack(data, sc, gs, nb))
+        want = O.f32_to_bf16_bits(O.dequant(npd, nps, nb, gs, bf16=True))
+        assert np.array_equal(got, want)
+    o_hat, idx = T.decode_path(bf16_tensor(c["q"]), kd[None, :, :S], ks[None, :, :S], vd[None, :, :S], vs[None, :, :S],
+                               gs, kbits, vbits, K)
+    ref_sc = O.scores_bf16_model(c["q"], c["kd"], c["ks"], c["bt"], c["lens"], S, Hq, Hkv, 16, 128 ** -0.5, kbits, gs)
+    ridx, _ = O.topk_select(ref_sc, c["lens"], c["bt"], S, K)
+    # same winners unless a margin is inside fp32 accumulation noise
+    for h in range(Hq):
+        cut = np.sort(ref_sc[0, h])[-K]
+        clear = [i for i in ridx[0, h] if ref_sc[0, h, i] > cut + 1e-5]
+        assert set(clear) <= set(idx[0, h].tolist())
+    # o_hat: the oracle's Stage B dequantises V without the bf16 rounding; compare against the bf16-rounded V
+    vhat = O.dequant(c["vd"], c["vs"], vbits, gs, bf16=True)
+    p = np.exp(ref_sc[0].astype(np.float64) - ref_sc[0].max(-1, keepdims=True))
+    p /= p.sum(-1, keepdims=True)
+    want = np.einsum("hs,hsd->hd", p, vhat[np.arange(Hq) // (Hq // Hkv)][:, :S].astype(np.float64))
+    np.testing.assert_allclose(o_hat[0].numpy(), want, atol=2e-5, rtol=1e-4)
