@@ -53,7 +53,7 @@ __device__ __host__ inline uint16_t f32_to_bf16(float f) {
 __device__ __host__ inline uint32_t score_key(float f) {
   union { uint32_t u; float f; } v;
   v.f = f;
-  return (v.u & 0x80000000u) ? ~v.u : (v.u | 0x80000000u);
+  return v.u ^ ((uint32_t)((int32_t)v.u >> 31) | 0x80000000u);  // negative: all bits flipped; else: sign bit set
 }
 
 // Wavefront-wide reductions and scans on the DPP network (row shifts inside 16-lane rows, then the two
@@ -70,6 +70,15 @@ __device__ inline int dpp_mov(int old, int v) {
     v = OP(v, __builtin_bit_cast(T, dpp_mov<0x118, 0xf>(__builtin_bit_cast(int, (T)(IDENT)), __builtin_bit_cast(int, v)))); \
     v = OP(v, __builtin_bit_cast(T, dpp_mov<0x142, 0xa>(__builtin_bit_cast(int, (T)(IDENT)), __builtin_bit_cast(int, v)))); \
     v = OP(v, __builtin_bit_cast(T, dpp_mov<0x143, 0xc>(__builtin_bit_cast(int, (T)(IDENT)), __builtin_bit_cast(int, v)))); \
+  } while (0)
+
+// reduction inside each 16-lane row only: lane 15 of a row holds the row's result
+#define JF_DPP_ROW_REDUCE(v, OP, T, IDENT)                                                           \
+  do {                                                                                               \
+    v = OP(v, __builtin_bit_cast(T, dpp_mov<0x111, 0xf>(__builtin_bit_cast(int, (T)(IDENT)), __builtin_bit_cast(int, v)))); \
+    v = OP(v, __builtin_bit_cast(T, dpp_mov<0x112, 0xf>(__builtin_bit_cast(int, (T)(IDENT)), __builtin_bit_cast(int, v)))); \
+    v = OP(v, __builtin_bit_cast(T, dpp_mov<0x114, 0xf>(__builtin_bit_cast(int, (T)(IDENT)), __builtin_bit_cast(int, v)))); \
+    v = OP(v, __builtin_bit_cast(T, dpp_mov<0x118, 0xf>(__builtin_bit_cast(int, (T)(IDENT)), __builtin_bit_cast(int, v)))); \
   } while (0)
 
 __device__ inline float op_fmax(float a, float b) { return fmaxf(a, b); }

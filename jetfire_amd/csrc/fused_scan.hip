@@ -32,6 +32,8 @@ namespace jf {
 namespace {
 
 typedef int v2i __attribute__((ext_vector_type(2)));
+typedef unsigned v2u __attribute__((ext_vector_type(2)));
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef float v2f __attribute__((ext_vector_type(2)));
@@ -97,44 +99,44 @@ struct QInt8F {
 };
 
 // LDS carve-up shared by the kernel and its launcher.
+//   sc     [G][L] fp32 scores of the split
+//   sbase  [L/16] first slot of every 16-position page
+//   aux    phase A: query constants (K3Prep / QInt8F); afterwards: selection histograms [G][SEG][256]
+//   stage  one private staging area per wavefront: key rows in phase A, V rows + weight rows in phase B
+// After the selection the whole block is reused for the exchange of the P.V accumulators.
 template <int SCHEME, int G, int NG>
 struct ScanLds {
   static constexpr bool K3 = (SCHEME == JF_SCHEME_K3V2);
   static constexpr int NSET = (G + 3) / 4;
+  static constexpr int SEG = (G <= 4) ? 2 : 1;  // emission segments per head (one wavefront each)
+  static constexpr int KP = K3 ? 48 : 64;
+  static constexpr int KROW = K3 ? 48 : 80;     // LDS pitch of a staged key row (INT4: padded against bank conflicts)
   static constexpr int VP = K3 ? 32 : 64;
   static constexpr int VROW = VP + 8;  // 16 consecutive rows hit 16 distinct bank pairs
   static constexpr int VST = 64 * VROW;
   static constexpr int WL = NG * NSET * 64 * 16;  // per (group, set): one 16-byte weight row per token
-  static constexpr int WAVE_STAGE = VST + WL;
+  static constexpr int KST = 64 * KROW;
+  static constexpr int WAVE_STAGE = (VST + WL > KST) ? (VST + WL) : KST;
   static constexpr int ACC_REGS = 8 + NG;                   // v4i accumulators per set: 8 channel tiles + NG weight sums
-  static constexpr int RED = (4 + NSET) * ACC_REGS * 1024;  // four exchange slots + the final sums of every set
+  static constexpr int SPR = NSET < 2 ? NSET : 2;           // sets exchanged per round
+  static constexpr int XWAVE = ACC_REGS * (48 * 16 + 16 * 4);  // bytes one wavefront writes per set (rows 0..12 only)
+  static constexpr int RED = FS_WAVES * SPR * XWAVE;
   static constexpr int PREP = K3 ? (int)sizeof(K3Prep<NSET>) : (int)sizeof(QInt8F<G>);
-  __host__ __device__ static constexpr int stage_bytes() {
-    int s = FS_WAVES * WAVE_STAGE;
-    if (PREP > s) s = PREP;
-    return (s + 15) & ~15;
-  }
-  __host__ __device__ static constexpr size_t per_position() { return (size_t)G * 4 + NG * 2; }
+  static constexpr int HIST = G * SEG * 256 * 4;
+  static constexpr int AUX = ((PREP > HIST ? PREP : HIST) + 15) & ~15;
+  __host__ __device__ static constexpr int stage_bytes() { return FS_WAVES * WAVE_STAGE; }
+  __host__ __device__ static constexpr size_t per_position() { return (size_t)G * 4; }
+  __host__ __device__ static size_t aux_offset(int L) { return (per_position() * L + (size_t)(L / 16) * 4 + 15) & ~(size_t)15; }
   __host__ __device__ static size_t total(int L) {
-    const size_t t = per_position() * L + (size_t)(L / 16) * 4 + stage_bytes() + 64;
+    const size_t t = aux_offset(L) + AUX + stage_bytes() + 64;
     return t > (size_t)RED + 64 ? t : (size_t)RED + 64;
   }
 };
-
-__device__ inline uint32_t pack_bf16x2(float a, float b) {
-  v2f f = {a, b};
-  v2bf h = __builtin_convertvector(f, v2bf);  // v_cvt_pk_bf16_f32, round-to-nearest-even
-  return __builtin_bit_cast(uint32_t, h);
-}
 
 __device__ inline float key_to_score(uint32_t key) {
   const uint32_t u = (key & 0x80000000u) ? (key & 0x7fffffffu) : ~key;
   return __builtin_bit_cast(float, u);
 }
-
-// position of token r (0..15) of a 16-token block inside the 16-byte MFMA K-run: the nibble spread of a
-// transposed V dword yields tokens 0,2,4,6 | 1,3,5,7 | 8,10,12,14 | 9,11,13,15.
-__device__ inline int token_byte_pos(int r) { return (r & 8) | ((r & 1) << 2) | ((r >> 1) & 3); }
 
 // Orders this wavefront's earlier LDS writes before its later LDS reads (the LDS pipe executes one
 // wavefront's instructions in order; this only stops the compiler from moving them).
@@ -144,36 +146,49 @@ __device__ inline void wave_lds_fence() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// Workgroup barrier that orders LDS traffic only: unlike __syncthreads() it does not wait for global loads
+// that are still in flight (the prefetched key / value rows), which no other wavefront consumes.
+__device__ inline void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+__device__ inline float uniform_f(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, v)));
+}
+
 // ---------------------------------------------------------------------------------------------------
 template <int SCHEME, int G, int NG>
 __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
   using Lds = ScanLds<SCHEME, G, NG>;
   constexpr bool K3 = Lds::K3;
   constexpr int NSET = Lds::NSET;
-  constexpr int KP = K3 ? 48 : 64;
+  constexpr int SEG = Lds::SEG;
+  constexpr int KP = Lds::KP;
+  constexpr int KROW = Lds::KROW;
   constexpr int VP = Lds::VP;
   constexpr int VROW = Lds::VROW;
   constexpr int VOFF = K3 ? 2 : 8;  // code offset of the V format
   constexpr int NTILE = 8;          // 8 MFMA column tiles of 16 channels
   constexpr int AR = Lds::ACC_REGS;
-  constexpr int CW = G < 4 ? G : 4;  // wavefronts that run the candidate selection before joining phase B
   constexpr float LOG2E = 1.44269504088896340736f;
+  constexpr int MAXIT = FS_LMAX / 64 / FS_WAVES;  // chunks per wavefront
 
   extern __shared__ __align__(16) uint8_t smem[];
   const int L = p.L;
-  float* sc = reinterpret_cast<float*>(smem);                                   // [G][L]
-  int* sbase = reinterpret_cast<int*>(smem + (size_t)G * L * 4);                // [L/16] first slot of each page
-  uint16_t* vsl = reinterpret_cast<uint16_t*>(smem + (size_t)G * L * 4 + (size_t)(L / 16) * 4);  // [L][NG]
-  uint8_t* stage = smem + (((size_t)G * L * 4 + (size_t)(L / 16) * 4 + (size_t)L * NG * 2 + 15) & ~(size_t)15);
-  __shared__ float red_f[FS_WAVES][G];
+  float* sc = reinterpret_cast<float*>(smem);                     // [G][L]
+  int* sbase = reinterpret_cast<int*>(smem + (size_t)G * L * 4);  // [L/16] first slot of each page
+  uint8_t* aux = smem + Lds::aux_offset(L);
+  uint8_t* stage = aux + Lds::AUX;
+  int* hist = reinterpret_cast<int*>(aux);  // [G][SEG][256], valid after phase A
+  __shared__ float red_f[FS_WAVES][2 * G];
   __shared__ uint32_t vmax_sh[FS_WAVES][2];
-  __shared__ float m_sh[G];
+  __shared__ float m_sh[G], bin_a_sh[G], bin_b_sh[G], lsum_sh[FS_WAVES][G];
   __shared__ int e_sh[2];
-  __shared__ long long lsum_sh[FS_WAVES][G];
-  __shared__ int bq_sh;  // next unclaimed phase-B chunk
+  __shared__ int cut_sh[G], cnt0_sh[G], exact_sh[G];
+  __shared__ unsigned long long tmax_sh;
+  if (threadIdx.x == 0) tmax_sh = 0ull;
 
   const int split = blockIdx.x, hkv = blockIdx.y, b = blockIdx.z;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: keeps wave-derived addresses in SGPRs
   const int S = max(0, min(p.max_S, p.seq_lens[b]));
   const int s0 = split * L;
   const int s1 = min(s0 + L, S);
@@ -185,7 +200,7 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
   const size_t part_base = head0 * p.n_splits + split;  // + h * n_splits
   const uint8_t* kbase = p.k_data + (size_t)hkv * p.num_slots * KP;
   const uint8_t* vbase = p.v_data + (size_t)hkv * p.num_slots * VP;
-  const uint16_t* vsbase = p.v_scales + (size_t)hkv * p.num_slots * NG;
+  const uint8_t* vsbase = reinterpret_cast<const uint8_t*>(p.v_scales + (size_t)hkv * p.num_slots * NG);
 
   long long* clk = p.phase_clock ? p.phase_clock + (((size_t)b * p.H_kv + hkv) * p.n_splits + split) * 10 : nullptr;
   if (clk && tid == 0) clk[0] = clock64();
@@ -212,10 +227,65 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
     const int last_page = (n - 1) >> 4;
     for (int i = tid; i < nch_cover * 4; i += FS_THREADS) sbase[i] = (int)(bt[(s0 >> 4) + min(i, last_page)] * BS);
   }
-  if (tid == 0) bq_sh = 0;
-  __syncthreads();
+  // query elements of this thread (in flight while the page table arrives)
+  constexpr int QPT = (G * D + FS_THREADS - 1) / FS_THREADS;
+  static_assert(QPT == NSET, "one query element per thread and head set");
+  float qv[QPT];
+#pragma unroll
+  for (int it = 0; it < QPT; ++it) {
+    const int i = it * FS_THREADS + tid;
+    qv[it] = (i < G * D) ? bf16_to_f32(p.q[head0 * D + i]) : 0.f;
+  }
+  lds_barrier();
 
-  // V scales of the split: loaded now (in flight during the query set-up), kept in LDS for phase B
+  // ---- key stream, set-up.  A chunk is 64 consecutive positions = 4 pages; its rows are fetched with
+  // 16-byte loads whose lane addresses are consecutive inside a page, staged in this wavefront's LDS area
+  // in position order, and read back in the layout the arithmetic wants.
+  uint8_t* kst = stage + wave * Lds::WAVE_STAGE;
+  constexpr int KLD = KP / 16;  // 16-byte loads per lane and chunk
+  uint32_t kl_page[KLD], kl_off[KLD], kl_lds[KLD];
+#pragma unroll
+  for (int i = 0; i < KLD; ++i) {
+    const int o = 1024 * i + 16 * lane;  // byte offset inside the chunk's 64 rows
+    kl_page[i] = (uint32_t)(o / (16 * KP));
+    kl_off[i] = (uint32_t)(o % (16 * KP));
+    kl_lds[i] = (uint32_t)((o / KP) * KROW + (o % KP));
+  }
+  const uint8_t* ksb = reinterpret_cast<const uint8_t*>(p.k_scales + (size_t)hkv * p.num_slots * (K3 ? NG : 1));
+  struct KBuf {
+    v4u r[KLD];
+    uint32_t s[K3 ? 4 : 1];
+  };
+  const int t16 = lane & 15, lg = lane >> 4;
+  auto issue_k = [&](int chunk) -> KBuf {
+    KBuf kbuf;
+#pragma unroll
+    for (int i = 0; i < KLD; ++i) {
+      const uint32_t sb = (uint32_t)sbase[chunk * 4 + kl_page[i]];
+      kbuf.r[i] = *reinterpret_cast<const v4u*>(kbase + (size_t)(sb * (uint32_t)KP + kl_off[i]));
+    }
+    if constexpr (K3) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int sb = __builtin_amdgcn_readfirstlane(sbase[chunk * 4 + j]);  // first slot of the page (uniform)
+        const uint8_t* srow = ksb + (size_t)sb * (NG * 2) + t16 * (NG * 2);
+        if (NG == 2) kbuf.s[j] = *reinterpret_cast<const uint32_t*>(srow);
+        else kbuf.s[j] = *reinterpret_cast<const uint16_t*>(srow);
+      }
+    } else {
+      const int t = chunk * 64 + lane;
+      const uint32_t slot = (uint32_t)(sbase[t >> 4] + (t & 15));
+      kbuf.s[0] = *reinterpret_cast<const uint16_t*>(ksb + (size_t)(slot * 2u));
+    }
+    return kbuf;
+  };
+  auto stash_k = [&](const KBuf& kbuf) {
+#pragma unroll
+    for (int i = 0; i < KLD; ++i) *reinterpret_cast<v4u*>(kst + kl_lds[i]) = kbuf.r[i];
+  };
+  // first two chunks of this wavefront and the V scales of the split start now, before the query set-up
+  KBuf Ka = {}, Kb = {};
+  if (wave < nch_cover) Ka = issue_k(wave);
   constexpr int VSPT = FS_LMAX / FS_THREADS;
   uint32_t vsw[VSPT];
 #pragma unroll
@@ -224,37 +294,36 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
     vsw[i] = 0u;
     if (t < n) {
       const uint32_t slot = (uint32_t)(sbase[t >> 4] + (t & 15));
-      if (NG == 2) vsw[i] = *reinterpret_cast<const uint32_t*>(vsbase + (size_t)(slot * 2u));
-      else vsw[i] = (uint32_t)vsbase[slot];
+      if (NG == 2) vsw[i] = *reinterpret_cast<const uint32_t*>(vsbase + (size_t)(slot * 4u));
+      else vsw[i] = (uint32_t) * reinterpret_cast<const uint16_t*>(vsbase + (size_t)(slot * 2u));
     }
   }
 
-  if (K3) {
+  if constexpr (K3) {
     // Query rows -> 23-bit fixed point per (head, scale group), three balanced int8 limbs, written in the
     // byte order of the MFMA A operand.  One element per thread; group statistics by wavefront reductions.
-    K3Prep<NSET>* prep = reinterpret_cast<K3Prep<NSET>*>(stage);
-    float qv[NSET];
-#pragma unroll
-    for (int it = 0; it < NSET; ++it) {
-      const int i = it * FS_THREADS + tid, h = i >> 7, d = i & 127;
-      qv[it] = (h < G) ? bf16_to_f32(p.q[(head0 + h) * D + d]) : 0.f;
-      const float am = wave_max(fabsf(qv[it]));
-      if (lane == 0) prep->amax_w[it * FS_WAVES + wave] = am;
-    }
+    K3Prep<NSET>* prep = reinterpret_cast<K3Prep<NSET>*>(aux);
     if (tid < 128) {
       const float sm = 1.0f + (float)tid * (1.0f / 128.0f);
       const float t3 = 3.0f * sm;  // exact in fp32
       prep->eps[tid] = 256.0f * ((bf16_to_f32(f32_to_bf16(t3)) - t3) / sm);
     }
-    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < NSET; ++it) {
+      const float x = qv[it];
+      const float am = wave_max(fabsf(x));
+      if (lane == 0) prep->amax_w[it * FS_WAVES + wave] = am;
+    }
+    lds_barrier();
 #pragma unroll
     for (int it = 0; it < NSET; ++it) {
       const int i = it * FS_THREADS + tid, h = i >> 7, d = i & 127;
+      const float x = qv[it];
       const int c = it * FS_WAVES + wave;  // 64-channel half row of this wavefront
       const float amax = (NG == 2) ? prep->amax_w[c] : fmaxf(prep->amax_w[c & ~1], prep->amax_w[c | 1]);
       int e = 0;
       if (amax > 0.f && isfinite(amax)) (void)frexpf(amax, &e);  // amax = f * 2^e, f in [0.5, 1)
-      const int qf = (int)rintf(ldexpf(qv[it], 22 - e));
+      const int qf = (int)rintf(ldexpf(x, 22 - e));
       const int s = wave_sum_i(qf);
       if (lane == 0) {
         prep->sum_w[c] = s;
@@ -275,7 +344,7 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
       prep->aop[set][4 * hh + 2][kb][mi][by] = (int8_t)l2;
       prep->aop[set][4 * hh + 3][kb][mi][by] = 0;
     }
-    __syncthreads();
+    lds_barrier();
     if (tid < NSET * 4 * NG) {
       const int h = tid / NG, g = tid % NG;
       const int sum = (NG == 2) ? prep->sum_w[2 * h + g] : prep->sum_w[2 * h] + prep->sum_w[2 * h + 1];
@@ -285,55 +354,45 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
     }
   } else {
     // int8 quantisation of the G query rows per 32 channels (int8tc_qk_scores.cu:250-290), one element per thread
-    QInt8F<G>* qsh = reinterpret_cast<QInt8F<G>*>(stage);
-    for (int i = tid; i < G * D; i += FS_THREADS) {
-      const int g = i >> 7, d = i & 127, kk = d >> 5;
-      const float x = bf16_to_f32(p.q[(head0 + g) * D + d]);
-      float a = fabsf(x);
+    QInt8F<G>* qsh = reinterpret_cast<QInt8F<G>*>(aux);
 #pragma unroll
-      for (int off = 16; off >= 1; off >>= 1) a = fmaxf(a, __shfl_xor(a, off));
-      const float s = fmaxf(a / 127.0f, 1e-12f);
-      const float inv = 1.0f / s;
-      const int v = max(-128, min(127, (int)rintf(x * inv)));
-      int sv = v;
+    for (int it = 0; it < QPT; ++it) {
+      const int i = it * FS_THREADS + tid;
+      if (i < G * D) {  // uniform per wavefront: G * D is a multiple of 64
+        const int g = i >> 7, d = i & 127, kk = d >> 5;
+        const float x = qv[it];
+        float a = fabsf(x);
 #pragma unroll
-      for (int off = 16; off >= 1; off >>= 1) sv += __shfl_xor(sv, off);
-      const int j = d >> 3, e = d & 7;
-      int8_t* dst = (e & 1) ? reinterpret_cast<int8_t*>(&qsh->qo[g][j]) : reinterpret_cast<int8_t*>(&qsh->qe[g][j]);
-      dst[e >> 1] = (int8_t)v;
-      if ((lane & 31) == 0) {
-        qsh->qs[g][kk] = s;
-        qsh->sum8[g][kk] = 8 * sv;
+        for (int off = 16; off >= 1; off >>= 1) a = fmaxf(a, __shfl_xor(a, off));
+        const float s = fmaxf(a / 127.0f, 1e-12f);
+        const float inv = 1.0f / s;
+        const int v = max(-128, min(127, (int)rintf(x * inv)));
+        int sv = v;
+#pragma unroll
+        for (int off = 16; off >= 1; off >>= 1) sv += __shfl_xor(sv, off);
+        const int j = d >> 3, e = d & 7;
+        int8_t* dst = (e & 1) ? reinterpret_cast<int8_t*>(&qsh->qo[g][j]) : reinterpret_cast<int8_t*>(&qsh->qe[g][j]);
+        dst[e >> 1] = (int8_t)v;
+        if ((lane & 31) == 0) {
+          qsh->qs[g][kk] = s;
+          qsh->sum8[g][kk] = 8 * sv;
+        }
       }
     }
   }
-  {
-    uint32_t vm0 = 0u, vm1 = 0u;
-#pragma unroll
-    for (int i = 0; i < VSPT; ++i) {
-      const int t = tid + i * FS_THREADS;
-      if (t < nch_cover * 64) {
-        if (NG == 2) *reinterpret_cast<uint32_t*>(vsl + 2 * t) = vsw[i];
-        else vsl[t] = (uint16_t)vsw[i];
-      }
-      vm0 = max(vm0, vsw[i] & 0x7fffu);
-      vm1 = max(vm1, (vsw[i] >> 16) & 0x7fffu);
-    }
-    vm0 = wave_max_u(vm0);
-    vm1 = wave_max_u(vm1);
-    if (lane == 0) {
-      vmax_sh[wave][0] = vm0;
-      vmax_sh[wave][1] = vm1;
-    }
-  }
-  __syncthreads();
+  lds_barrier();
+  if (wave + FS_WAVES < nch_cover) Kb = issue_k(wave + FS_WAVES);
+  if (clk && tid == 0) clk[7] = clock64();
 
   // ------------------------------------------------------------------ phase A
-  float mx[G];
+  float mx[G], mn[G];
 #pragma unroll
-  for (int h = 0; h < G; ++h) mx[h] = -INFINITY;
+  for (int h = 0; h < G; ++h) {
+    mx[h] = -INFINITY;
+    mn[h] = INFINITY;
+  }
 
-  if (K3) {
+  if constexpr (K3) {
     // INT3 keys on v_mfma_i32_16x16x64_i8.  The bf16 query row is held exactly as a 23-bit fixed-point number
     // per (head, scale group), split into three balanced int8 limbs that sit in different A-operand rows
     // (row = 4*head + limb), so one MFMA yields the three integer partial sums of a (token, head) in the
@@ -345,8 +404,7 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
     // (int3_qk_scores.cu:90-99); only codes +-3 are inexact, so that rounding is reproduced by a second
     // contraction with the indicator (+1 for code 7, -1 for code 1, byte LUT through v_perm_b32) weighted by
     // eps = (bf16(3s) - 3s) / s, which depends on the 7 mantissa bits of the scale only (128-entry table).
-    const K3Prep<NSET>* prep = reinterpret_cast<const K3Prep<NSET>*>(stage);
-    const int t16 = lane & 15, lg = lane >> 4;  // B operand: column (token), k-block; D: column, head
+    const K3Prep<NSET>* prep = reinterpret_cast<const K3Prep<NSET>*>(aux);
     v4i Aop[NSET][2];
     int sq4[NSET][NG];
     float qsc[NSET][NG];
@@ -360,30 +418,35 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
         qsc[set][g] = prep->qsc[set * 4 + lg][g];
       }
     }
-    const uint8_t* ksb = reinterpret_cast<const uint8_t*>(p.k_scales + (size_t)hkv * p.num_slots * NG);
-    const uint32_t lane_koff = (uint32_t)(t16 * KP + lg * 4);
-    const uint32_t lane_soff = (uint32_t)(t16 * NG * 2);
-    uint32_t Pa[4][3], Pb[4][3], Sa[4], Sb[4];
-    auto issue = [&](int chunk, uint32_t (&P)[4][3], uint32_t (&Sx)[4]) {
+    const uint8_t* krd = kst + t16 * KROW + lg * 4;  // this lane's plane dwords of token t16 of a page
+    float mxl[NSET], mnl[NSET];
+#pragma unroll
+    for (int set = 0; set < NSET; ++set) {
+      mxl[set] = -INFINITY;
+      mnl[set] = INFINITY;
+    }
+    auto body = [&](int chunk, const uint32_t (&Sx)[4]) {
+      // all LDS reads of the chunk first (plane dwords of the four pages, rounding coefficients), then arithmetic
+      uint32_t Pj[4][3];
+      float sgj[4][NG], egj[4][NG];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const int sb = __builtin_amdgcn_readfirstlane(sbase[chunk * 4 + j]);  // first slot of the page (uniform)
-        const uint8_t* rowb = kbase + (size_t)sb * KP;
-        P[j][0] = *reinterpret_cast<const uint32_t*>(rowb + lane_koff);
-        P[j][1] = *reinterpret_cast<const uint32_t*>(rowb + lane_koff + 16);
-        P[j][2] = *reinterpret_cast<const uint32_t*>(rowb + lane_koff + 32);
-        const uint8_t* srow = ksb + (size_t)sb * (NG * 2);
-        if (NG == 2) Sx[j] = *reinterpret_cast<const uint32_t*>(srow + lane_soff);
-        else Sx[j] = *reinterpret_cast<const uint16_t*>(srow + lane_soff);
+        const uint8_t* rp = krd + j * 16 * KROW;
+        Pj[j][0] = *reinterpret_cast<const uint32_t*>(rp);
+        Pj[j][1] = *reinterpret_cast<const uint32_t*>(rp + 16);
+        Pj[j][2] = *reinterpret_cast<const uint32_t*>(rp + 32);
+        const uint32_t sw = Sx[j];
+        sgj[j][0] = bf16_to_f32((uint16_t)(sw & 0xffffu));
+        egj[j][0] = prep->eps[sw & 0x7fu];
+        if (NG == 2) {
+          sgj[j][NG - 1] = bf16_to_f32((uint16_t)(sw >> 16));
+          egj[j][NG - 1] = prep->eps[(sw >> 16) & 0x7fu];
+        }
       }
-    };
-    float mxl[NSET];
-#pragma unroll
-    for (int set = 0; set < NSET; ++set) mxl[set] = -INFINITY;
-    auto body = [&](int chunk, const uint32_t (&P)[4][3], const uint32_t (&Sx)[4]) {
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const uint32_t P0 = P[j][0], P1 = P[j][1], P2 = P[j][2];
+        const uint32_t P0 = Pj[j][0], P1 = Pj[j][1], P2 = Pj[j][2];
         v4i Bc[2], Br[2];
         Bc[0][0] = (int)((P0 >> 5) & 0x07070707u);
         Bc[0][1] = (int)((P0 >> 2) & 0x07070707u);
@@ -410,14 +473,10 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
             Br[u][e] = (int)__builtin_amdgcn_perm(0x01000000u, 0x0000ff00u, (uint32_t)Bc[u][e]);
         // per-token scales (both groups) and the rounding coefficient
         float sg[NG], eg[NG];
-        {
-          const uint32_t sw = Sx[j];
-          sg[0] = bf16_to_f32((uint16_t)(sw & 0xffffu));
-          eg[0] = prep->eps[sw & 0x7fu];
-          if (NG == 2) {
-            sg[NG - 1] = bf16_to_f32((uint16_t)(sw >> 16));
-            eg[NG - 1] = prep->eps[(sw >> 16) & 0x7fu];
-          }
+#pragma unroll
+        for (int g = 0; g < NG; ++g) {
+          sg[g] = sgj[j][g];
+          eg[g] = egj[j][g];
         }
         const int tok = chunk * 64 + 16 * j + t16;
         const bool valid = tok < n;
@@ -447,51 +506,52 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
           }
           const int h = set * 4 + lg;
           if ((G % 4 == 0) || h < G) {
-            const float sv = valid ? score : -INFINITY;
-            sc[h * L + tok] = sv;
-            if (p.scores && tok < n_cover) p.scores[(head0 + h) * (size_t)p.max_S + s0 + tok] = sv;
-            mxl[set] = fmaxf(mxl[set], sv);
+            sc[h * L + tok] = valid ? score : -INFINITY;
+            mxl[set] = fmaxf(mxl[set], valid ? score : -INFINITY);
+            mnl[set] = fminf(mnl[set], valid ? score : INFINITY);
           }
         }
       }
     };
-    int chunk = wave;
-    if (chunk < nch_cover) issue(chunk, Pa, Sa);
-    while (chunk < nch_cover) {
-      if (chunk + FS_WAVES < nch_cover) issue(chunk + FS_WAVES, Pb, Sb);
-      body(chunk, Pa, Sa);
-      chunk += FS_WAVES;
-      if (chunk >= nch_cover) break;
-      if (chunk + FS_WAVES < nch_cover) issue(chunk + FS_WAVES, Pa, Sa);
-      body(chunk, Pb, Sb);
-      chunk += FS_WAVES;
+    // at most FS_LMAX / 64 / FS_WAVES chunks per wavefront: straight-line code, so that the wait for a chunk's
+    // loads leaves the loads of the following chunks in flight
+#pragma unroll
+    for (int it = 0; it < MAXIT; ++it) {
+      const int chunk = wave + it * FS_WAVES;
+      if (chunk < nch_cover) {
+        KBuf& cur = (it & 1) ? Kb : Ka;
+        stash_k(cur);
+        wave_lds_fence();
+        uint32_t Sc[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) Sc[j] = cur.s[j];
+        if (it + 2 < MAXIT && chunk + 2 * FS_WAVES < nch_cover) cur = issue_k(chunk + 2 * FS_WAVES);
+        body(chunk, Sc);
+        wave_lds_fence();
+      }
     }
-    // lanes of 16-lane row lg hold the running maxima of head set*4 + lg: spread them into mx[] so the common
-    // reduction below applies (every other entry stays -inf)
+    // lanes of 16-lane row lg hold the running extrema of head set*4 + lg: reduce inside the rows (lane 15 of
+    // a row ends up with the row's result) and publish them
 #pragma unroll
-    for (int set = 0; set < NSET; ++set)
-#pragma unroll
-      for (int rr = 0; rr < 4; ++rr)
-        if (set * 4 + rr < G) mx[set * 4 + rr] = (lg == rr) ? mxl[set] : -INFINITY;
+    for (int set = 0; set < NSET; ++set) {
+      float a = mxl[set], c = -mnl[set];
+      JF_DPP_ROW_REDUCE(a, op_fmax, float, -INFINITY);
+      JF_DPP_ROW_REDUCE(c, op_fmax, float, -INFINITY);
+      const int h = set * 4 + lg;
+      if (t16 == 15 && h < G) {
+        red_f[wave][h] = a;
+        red_f[wave][G + h] = -c;
+      }
+    }
   } else {
-    // INT4 keys, int8-Q model: lane = token
-    const QInt8F<G>* qsh = reinterpret_cast<const QInt8F<G>*>(stage);
-    const uint16_t* ksbase = p.k_scales + (size_t)hkv * p.num_slots;
-    uint4 Ra[4], Rb[4];
-    uint32_t Ka = 0, Kb = 0;
-    auto issue = [&](int chunk, uint4 (&R)[4], uint32_t& ksw) {
-      const int t = chunk * 64 + lane;
-      const uint32_t slot = (uint32_t)(sbase[t >> 4] + (t & 15));
-      const uint4* row = reinterpret_cast<const uint4*>(kbase + (size_t)(slot * (uint32_t)KP));
-#pragma unroll
-      for (int i = 0; i < 4; ++i) R[i] = row[i];
-      ksw = ksbase[slot];
-    };
-    auto body = [&](int chunk, const uint4 (&R)[4], uint32_t ksw) {
+    // INT4 keys, int8-Q model: lane = token, row read back from the staged chunk
+    const QInt8F<G>* qsh = reinterpret_cast<const QInt8F<G>*>(aux);
+    auto body = [&](int chunk, uint32_t ksw) {
       uint32_t pk[16];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        pk[4 * i] = R[i].x; pk[4 * i + 1] = R[i].y; pk[4 * i + 2] = R[i].z; pk[4 * i + 3] = R[i].w;
+        const v4u r = *reinterpret_cast<const v4u*>(kst + lane * KROW + 16 * i);
+        pk[4 * i] = r[0]; pk[4 * i + 1] = r[1]; pk[4 * i + 2] = r[2]; pk[4 * i + 3] = r[3];
       }
       const float ks = bf16_to_f32((uint16_t)ksw);
       const int tok = chunk * 64 + lane;
@@ -511,37 +571,108 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
           sacc = (kk == 0) ? ((float)acc * qsh->qs[g][0]) : __builtin_fmaf((float)acc, qsh->qs[g][kk], sacc);
         }
         const float a = __fmul_rn(__fmul_rn(sacc, ks), p.attn_scale);
-        const float sv = valid ? a : -INFINITY;
-        sc[g * L + tok] = sv;
-        if (p.scores && tok < n_cover) p.scores[(head0 + g) * (size_t)p.max_S + s0 + tok] = sv;
-        mx[g] = fmaxf(mx[g], sv);
+        sc[g * L + tok] = valid ? a : -INFINITY;
+        mx[g] = fmaxf(mx[g], valid ? a : -INFINITY);
+        mn[g] = fminf(mn[g], valid ? a : INFINITY);
       }
     };
-    int chunk = wave;
-    if (chunk < nch_cover) issue(chunk, Ra, Ka);
-    while (chunk < nch_cover) {
-      if (chunk + FS_WAVES < nch_cover) issue(chunk + FS_WAVES, Rb, Kb);
-      body(chunk, Ra, Ka);
-      chunk += FS_WAVES;
-      if (chunk >= nch_cover) break;
-      if (chunk + FS_WAVES < nch_cover) issue(chunk + FS_WAVES, Ra, Ka);
-      body(chunk, Rb, Kb);
-      chunk += FS_WAVES;
+#pragma unroll
+    for (int it = 0; it < MAXIT; ++it) {
+      const int chunk = wave + it * FS_WAVES;
+      if (chunk < nch_cover) {
+        KBuf& cur = (it & 1) ? Kb : Ka;
+        stash_k(cur);
+        wave_lds_fence();
+        const uint32_t ksw = cur.s[0];
+        if (it + 2 < MAXIT && chunk + 2 * FS_WAVES < nch_cover) cur = issue_k(chunk + 2 * FS_WAVES);
+        body(chunk, ksw);
+        wave_lds_fence();
+      }
     }
   }
 
-  // split max per head; fixed-point exponent of the V scales
+  // ---- V stream, set-up (same scheme as the key stream); its first two chunks start before the barrier
+  uint8_t* vst = stage + wave * Lds::WAVE_STAGE;  // [64][VROW], this wavefront only
+  uint8_t* wl = vst + Lds::VST;                   // [NG][NSET][64 tokens][16]
+  constexpr int VLD = VP / 16;
+  uint32_t vl_page[VLD], vl_off[VLD], vl_lds[VLD];
 #pragma unroll
-  for (int h = 0; h < G; ++h) {
-    const float v = wave_max(mx[h]);
-    if (lane == 0) red_f[wave][h] = v;
+  for (int i = 0; i < VLD; ++i) {
+    const int o = 1024 * i + 16 * lane;
+    vl_page[i] = (uint32_t)(o / (16 * VP));
+    vl_off[i] = (uint32_t)(o % (16 * VP));
+    vl_lds[i] = (uint32_t)((o / VP) * VROW + (o % VP));
   }
-  __syncthreads();
-  if (tid < G) {
-    float m = red_f[0][tid];
+  struct VBuf {
+    v4u r[VLD];
+    uint32_t w;
+  };
+  auto issue_v = [&](int chunk) -> VBuf {
+    VBuf vbuf;
 #pragma unroll
-    for (int w = 1; w < FS_WAVES; ++w) m = fmaxf(m, red_f[w][tid]);
+    for (int i = 0; i < VLD; ++i) {
+      const uint32_t sb = (uint32_t)sbase[chunk * 4 + vl_page[i]];
+      vbuf.r[i] = *reinterpret_cast<const v4u*>(vbase + (size_t)(sb * (uint32_t)VP + vl_off[i]));
+    }
+    const int t = chunk * 64 + lane;
+    const uint32_t slot = (uint32_t)(sbase[t >> 4] + (t & 15));
+    if (NG == 2) vbuf.w = *reinterpret_cast<const uint32_t*>(vsbase + (size_t)(slot * 4u));
+    else vbuf.w = (uint32_t) * reinterpret_cast<const uint16_t*>(vsbase + (size_t)(slot * 2u));
+    return vbuf;
+  };
+  VBuf Va = {}, Vb = {};
+  if (wave < nch) Va = issue_v(wave);
+  if (wave + FS_WAVES < nch) Vb = issue_v(wave + FS_WAVES);
+
+  if (clk && tid == 0) clk[9] = clock64();  // wavefront 0 finished its chunks
+  if (clk && lane == 0) atomicMax(&tmax_sh, (unsigned long long)clock64());
+  // split extrema per head; fixed-point exponent of the V scales; selection buckets
+  {
+    uint32_t vm0 = 0u, vm1 = 0u;
+#pragma unroll
+    for (int i = 0; i < VSPT; ++i) {
+      vm0 = max(vm0, vsw[i] & 0x7fffu);
+      vm1 = max(vm1, (vsw[i] >> 16) & 0x7fffu);
+    }
+    vm0 = wave_max_u(vm0);
+    vm1 = wave_max_u(vm1);
+    if (lane == 0) {
+      vmax_sh[wave][0] = vm0;
+      vmax_sh[wave][1] = vm1;
+    }
+  }
+  if constexpr (!K3) {
+#pragma unroll
+    for (int h = 0; h < G; ++h) {
+      const float v = wave_max(mx[h]);
+      const float u = -wave_max(-mn[h]);
+      if (lane == 0) {
+        red_f[wave][h] = v;
+        red_f[wave][G + h] = u;
+      }
+    }
+  }
+  lds_barrier();  // phase A complete: the query constants are dead, their space becomes the histograms
+  if (clk && tid == 0) { clk[8] = clock64(); clk[5] = (long long)tmax_sh; }
+  if (p.scores)  // validation output
+    for (int i = tid; i < G * n_cover; i += FS_THREADS) {
+      const int h = i / n_cover, t = i - h * n_cover;
+      p.scores[(head0 + h) * (size_t)p.max_S + s0 + t] = sc[h * L + t];
+    }
+  for (int i = tid; i < G * SEG * 256; i += FS_THREADS) hist[i] = 0;
+  if (tid < G) {
+    float m = red_f[0][tid], lo = red_f[0][G + tid];
+#pragma unroll
+    for (int w = 1; w < FS_WAVES; ++w) {
+      m = fmaxf(m, red_f[w][tid]);
+      lo = fminf(lo, red_f[w][G + tid]);
+    }
     m_sh[tid] = m;
+    // bucket of a score: min(255, (m - s) * 255 / (m - lo)), bucket 0 = largest; monotone in s
+    const float range = m - lo;
+    const float iw = (range > 0.f && isfinite(range)) ? 254.99f / range : 0.f;
+    bin_a_sh[tid] = -iw;
+    bin_b_sh[tid] = isfinite(m) ? m * iw : 0.f;
   }
   if (tid >= 64 && tid < 64 + NG) {
     const int g = tid - 64;
@@ -553,165 +684,8 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
     if (v > 0.f && isfinite(v)) (void)frexpf(v, &e);  // v = f * 2^e, f in [0.5, 1)
     e_sh[g] = 22 - e;                                 // v * 2^E in [2^21, 2^22)
   }
-  __syncthreads();
+  lds_barrier();
   if (clk && tid == 0) clk[1] = clock64();
-
-  // ------------------------------------------------------------------ phase C: per-head radix select
-  // Wavefronts 0..CW-1 take the heads first and join phase B afterwards; the other wavefronts start phase B
-  // at once (chunks are claimed from a queue), so the selection's dependent LDS round trips overlap the V
-  // stream.  Scores are read in place and turned into order-preserving keys on the fly.  Bits shared by
-  // every key of the split are skipped; each 8-bit level builds a histogram (LDS atomics, bin 256 swallows
-  // keys outside the current prefix) and finds the bin holding the Kt-th largest key.  As soon as
-  // "everything from that bin upwards" fits in the candidate buffer the search stops and all keys >= that
-  // bound are emitted (a superset of the split's top Kt, which is all the merge needs); otherwise it refines
-  // down to the exact key and emits the lowest-position ties that fill the quota.  Emission is an ordered
-  // ballot compaction.
-  if (wave < CW) {
-    int* hist = reinterpret_cast<int*>(stage + wave * Lds::WAVE_STAGE);
-    const int Kcap = p.Kc;
-    const int Kt = min(p.top_k, n);
-    for (int h = wave; h < G; h += CW) {
-      const float* srow = sc + h * L;
-      uint32_t* ck = p.cand_key + (part_base + (size_t)h * p.n_splits) * Kcap;
-      int32_t* ci = p.cand_idx + (part_base + (size_t)h * p.n_splits) * Kcap;
-      uint32_t T = 0;        // emit key > T (exact mode) or key >= T (bound mode)
-      int quota = 0;         // exact mode: ties to take
-      bool ge_mode = true;   // T = 0, ge: take everything (n <= Kcap)
-      if (n > Kcap) {
-        uint32_t kmin = 0xffffffffu, kmax = 0u;
-        for (int t0 = 0; t0 < n; t0 += 512) {
-          float kk[8];
-#pragma unroll
-          for (int u = 0; u < 8; ++u) {
-            const int t = t0 + 64 * u + lane;
-            kk[u] = (t < n) ? srow[t] : 0.f;
-          }
-#pragma unroll
-          for (int u = 0; u < 8; ++u) {
-            const int t = t0 + 64 * u + lane;
-            if (t < n) {
-              const uint32_t k = score_key(kk[u]);
-              kmin = min(kmin, k);
-              kmax = max(kmax, k);
-            }
-          }
-        }
-        kmin = wave_min_u(kmin);
-        kmax = wave_max_u(kmax);
-        if (clk && tid == 0) clk[6] = clock64();
-        const uint32_t diff = kmin ^ kmax;
-        if (diff == 0u) {  // every key equal: the lowest positions win
-          T = kmax;
-          quota = Kt;
-          ge_mode = false;
-        } else {
-          int bits_left = 32 - __clz((int)diff);  // number of low bits that vary
-          uint32_t prefix = (bits_left == 32) ? 0u : (kmax >> bits_left);
-          int k_rem = Kt;
-          ge_mode = false;
-          while (bits_left > 0) {
-            if (clk && tid == 0) clk[9] += 1;
-            const int nb = min(8, bits_left);
-            const int shift = bits_left - nb;
-            const uint32_t dmask = (1u << nb) - 1u;
-            for (int i = lane; i < 264; i += 64) hist[i] = 0;
-            const bool first = (bits_left == 32);
-            const int hi_shift = first ? 0 : bits_left;
-            for (int t0 = 0; t0 < n; t0 += 512) {
-              float kk[8];
-#pragma unroll
-              for (int u = 0; u < 8; ++u) {
-                const int t = t0 + 64 * u + lane;
-                kk[u] = (t < n) ? srow[t] : 0.f;
-              }
-#pragma unroll
-              for (int u = 0; u < 8; ++u) {
-                const int t = t0 + 64 * u + lane;
-                const uint32_t k = score_key(kk[u]);
-                const bool inpre = (t < n) && (first || ((k >> hi_shift) == prefix));
-                if (inpre) atomicAdd(&hist[(int)((k >> shift) & dmask)], 1);
-              }
-            }
-            // lane l owns bins 255-4l .. 252-4l (descending), so a prefix scan over lanes counts the bins above
-            const int c3 = hist[255 - 4 * lane], c2 = hist[254 - 4 * lane], c1 = hist[253 - 4 * lane], c0 = hist[252 - 4 * lane];
-            const int mine = c0 + c1 + c2 + c3;
-            const int e3 = wave_incl_scan_i(mine) - mine;  // keys in bins above 255-4l
-            const int e2 = e3 + c3, e1 = e2 + c2, e0 = e1 + c1;
-            int cut = -1, above = 0, ccut = 0;
-            if (e3 < k_rem && k_rem <= e3 + c3) { cut = 255 - 4 * lane; above = e3; ccut = c3; }
-            else if (e2 < k_rem && k_rem <= e2 + c2) { cut = 254 - 4 * lane; above = e2; ccut = c2; }
-            else if (e1 < k_rem && k_rem <= e1 + c1) { cut = 253 - 4 * lane; above = e1; ccut = c1; }
-            else if (e0 < k_rem && k_rem <= e0 + c0) { cut = 252 - 4 * lane; above = e0; ccut = c0; }
-            const unsigned long long who = __ballot(cut >= 0);
-            const int src = __ffsll((long long)who) - 1;
-            cut = __builtin_amdgcn_readlane(cut, src);
-            above = __builtin_amdgcn_readlane(above, src);
-            ccut = __builtin_amdgcn_readlane(ccut, src);
-            prefix = (prefix << nb) | (uint32_t)cut;
-            k_rem -= above;
-            bits_left = shift;
-            if ((Kt - k_rem) + ccut <= Kcap) {  // the whole cut bin fits: stop here
-              ge_mode = true;
-              T = (bits_left == 0) ? prefix : (prefix << bits_left);
-              break;
-            }
-          }
-          if (!ge_mode) {
-            T = prefix;
-            quota = k_rem;
-          }
-        }
-      }
-      if (clk && tid == 0) clk[7] = clock64();
-      int count = 0;
-      if (ge_mode) {
-        for (int t0 = 0; t0 < n; t0 += 512) {
-          float kk[8];
-#pragma unroll
-          for (int u = 0; u < 8; ++u) {
-            const int t = t0 + 64 * u + lane;
-            kk[u] = (t < n) ? srow[t] : 0.f;
-          }
-#pragma unroll
-          for (int u = 0; u < 8; ++u) {
-            const int t = t0 + 64 * u + lane;
-            const uint32_t k = score_key(kk[u]);
-            const bool above = (t < n) && (k >= T);
-            const unsigned long long ma = __ballot(above);
-            const int pos = count + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(ma >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)ma, 0u));
-            if (above && pos < Kcap) {
-              ck[pos] = k;
-              ci[pos] = s0 + t;
-            }
-            count += __popcll(ma);
-          }
-        }
-      } else {
-        int base_tie = 0;
-        for (int t0 = 0; t0 < n; t0 += 64) {
-          const int t = t0 + lane;
-          const uint32_t k = (t < n) ? score_key(srow[t]) : 0u;
-          const bool above = (t < n) && (k > T), tie = (t < n) && (k == T);
-          const unsigned long long ma = __ballot(above), mt = __ballot(tie);
-          const int pa = count + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(ma >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)ma, 0u));
-          const int pt = base_tie + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(mt >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mt, 0u));
-          if (above || (tie && pt < quota)) {
-            const int pos = pa + min(pt, quota);
-            if (pos < Kcap) {
-              ck[pos] = k;
-              ci[pos] = s0 + t;
-            }
-          }
-          count += __popcll(ma);
-          base_tie += __popcll(mt);
-        }
-        count += min(base_tie, quota);
-      }
-      if (lane == 0) p.cand_cnt[part_base + (size_t)h * p.n_splits] = min(Kcap, count);
-    }
-    wave_lds_fence();
-    if (clk && tid == 0) clk[2] = clock64();
-  }
 
   // ------------------------------------------------------------------ phase B: P.V on v_mfma_i32_16x16x64_i8
   // p = exp(s - m_split) is known exactly because phase A is complete, so w = p * v_scale is converted to
@@ -721,12 +695,11 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
   // wants.  V codes are staged packed in wavefront-private LDS and transposed by ds_read_b64_tr_b4 (16
   // tokens of one channel pair per lane), then spread.  sum_t w_t*(code - off) = sum_t w_t*code - off*sum_t w_t:
   // the ones row gives sum_t code (needed because the limbs are balanced), a ones B tile gives sum_t w_t.
-  // Every accumulation is an exact integer, so the result does not depend on which wavefront took which chunk.
+  // Every accumulation is an exact integer.  The same pass drops every score into one of 256 linear buckets
+  // per (head, half of the split) for the candidate selection.
   int E[NG];
 #pragma unroll
-  for (int g = 0; g < NG; ++g) E[g] = e_sh[g];
-  uint8_t* vst = stage + wave * Lds::WAVE_STAGE;  // [64][VROW], this wavefront only
-  uint8_t* wl = vst + Lds::VST;                   // [NG][NSET][64 tokens][16]
+  for (int g = 0; g < NG; ++g) E[g] = __builtin_amdgcn_readfirstlane(e_sh[g]);
   v4i acc[NSET][NTILE], accw[NSET][NG];
 #pragma unroll
   for (int set = 0; set < NSET; ++set) {
@@ -735,58 +708,40 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
 #pragma unroll
     for (int g = 0; g < NG; ++g) accw[set][g] = (v4i){0, 0, 0, 0};
   }
-  uint32_t li[G];
-  float nml[G];
+  float lsum[G], nml[G], bin_a[G], bin_b[G];
 #pragma unroll
   for (int h = 0; h < G; ++h) {
-    li[h] = 0u;
-    nml[h] = -(m_sh[h] * LOG2E);
+    lsum[h] = 0.f;
+    nml[h] = uniform_f(-(m_sh[h] * LOG2E));
+    bin_a[h] = uniform_f(bin_a_sh[h]);
+    bin_b[h] = uniform_f(bin_b_sh[h]);
   }
-  int my_chunks = 0;
   const int r16 = lane & 15, kb4 = lane >> 4;
   // transposed weight read: 16-lane group kb4 fetches the rows of tokens 16*kb4 .. +15; the lane pair (2j, 2j+1)
-  // supplies the two halves of the row that must land in byte j, i.e. of the token whose token_byte_pos is j
+  // supplies the two halves of the row that must land in byte j, i.e. of the token whose byte position in the
+  // V operand (see below) is j
   const int tr_tok = (((r16 >> 1) & 3) << 1) | ((r16 >> 3) & 1);
   const uint8_t* wrow = wl + (kb4 * 16 + tr_tok) * 16 + (r16 & 1) * 8;
-  uint4 Va[VP / 16], Vb[VP / 16];
-  auto grab = [&]() -> int {
-    int c = 0;
-    if (lane == 0) c = atomicAdd(&bq_sh, 1);
-    return __builtin_amdgcn_readfirstlane(c);
-  };
-  auto issue_v = [&](int chunk, uint4 (&R)[VP / 16]) {
+  const int seg_chunk = L / 128;  // first chunk of the second half of the split
+  auto body_v = [&](int chunk, uint32_t vsw) {
     const int t = chunk * 64 + lane;
-    const uint32_t slot = (uint32_t)(sbase[t >> 4] + (t & 15));
-    const uint4* src = reinterpret_cast<const uint4*>(vbase + (size_t)(slot * (uint32_t)VP));
-#pragma unroll
-    for (int i = 0; i < VP / 16; ++i) R[i] = src[i];
-  };
-  auto body_v = [&](int chunk, const uint4 (&R)[VP / 16]) {
-    ++my_chunks;
-    const int t = chunk * 64 + lane;
-    {
-      uint2* dst = reinterpret_cast<uint2*>(vst + lane * VROW);
-#pragma unroll
-      for (int i = 0; i < VP / 16; ++i) {
-        dst[2 * i] = make_uint2(R[i].x, R[i].y);
-        dst[2 * i + 1] = make_uint2(R[i].z, R[i].w);
-      }
-    }
     float vsf[NG];
-    {
-      const uint32_t w = (NG == 2) ? *reinterpret_cast<const uint32_t*>(vsl + 2 * t) : (uint32_t)vsl[t];
-      vsf[0] = ldexpf(bf16_to_f32((uint16_t)(w & 0xffffu)), E[0]);
-      if (NG == 2) vsf[NG - 1] = ldexpf(bf16_to_f32((uint16_t)(w >> 16)), E[NG - 1]);
-    }
+    vsf[0] = ldexpf(bf16_to_f32((uint16_t)(vsw & 0xffffu)), E[0]);
+    if (NG == 2) vsf[NG - 1] = ldexpf(bf16_to_f32((uint16_t)(vsw >> 16)), E[NG - 1]);
+    int* hb = hist + ((SEG == 2 && chunk >= seg_chunk) ? 256 : 0);
+    const bool tv = t < n;
     uint32_t bits[NSET * 4][NG];
 #pragma unroll
     for (int h = 0; h < NSET * 4; ++h) {
       if (h < G) {
+        const float s = sc[h * L + t];
         // masked positions hold -inf: their weight is exactly zero
-        const float pw = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[h * L + t], LOG2E, nml[h]));
-        li[h] += __builtin_bit_cast(uint32_t, __builtin_fmaf(pw, 4194304.0f, 8388608.0f));
+        const float pw = __builtin_amdgcn_exp2f(__builtin_fmaf(s, LOG2E, nml[h]));
+        lsum[h] += pw;
 #pragma unroll
         for (int g = 0; g < NG; ++g) bits[h][g] = __builtin_bit_cast(uint32_t, __builtin_fmaf(pw, vsf[g], 8388608.0f));
+        const uint32_t bin = (uint32_t)__builtin_amdgcn_fmed3f(__builtin_fmaf(s, bin_a[h], bin_b[h]), 0.f, 255.f);
+        if (tv) atomicAdd(hb + h * (SEG * 256) + (int)bin, 1);
       } else {
 #pragma unroll
         for (int g = 0; g < NG; ++g) bits[h][g] = 0x4b000000u;
@@ -825,6 +780,8 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
 #pragma unroll
       for (int set = 0; set < NSET; ++set)
         accw[set][g] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[g][set], ones, accw[set][g], 0, 0, 0);
+    // the nibble spread of a transposed V dword yields tokens 0,2,4,6 | 1,3,5,7 | 8,10,12,14 | 9,11,13,15 of the
+    // lane group's 16 tokens: token r sits in byte (r&8) | ((r&1)<<2) | ((r>>1)&3)
     const uint8_t* vrow = vst + lane * VROW;
     if (K3) {
 #pragma unroll
@@ -857,97 +814,270 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
     }
     wave_lds_fence();
   };
-  {
-    int cur = grab();
-    if (cur < nch) issue_v(cur, Va);
-    while (cur < nch) {
-      int nxt = grab();
-      if (nxt < nch) issue_v(nxt, Vb);
-      body_v(cur, Va);
-      cur = nxt;
-      if (cur >= nch) break;
-      nxt = grab();
-      if (nxt < nch) issue_v(nxt, Va);
-      body_v(cur, Vb);
-      cur = nxt;
+  auto stash_v = [&](const VBuf& vbuf) {
+#pragma unroll
+    for (int i = 0; i < VLD; ++i) {
+      v2u* dst = reinterpret_cast<v2u*>(vst + vl_lds[i]);
+      dst[0] = (v2u){vbuf.r[i][0], vbuf.r[i][1]};
+      dst[1] = (v2u){vbuf.r[i][2], vbuf.r[i][3]};
+    }
+  };
+#pragma unroll
+  for (int it = 0; it < MAXIT; ++it) {
+    const int chunk = wave + it * FS_WAVES;
+    if (chunk < nch) {
+      VBuf& cur = (it & 1) ? Vb : Va;
+      stash_v(cur);
+      const uint32_t vw = cur.w;
+      if (it + 2 < MAXIT && chunk + 2 * FS_WAVES < nch) cur = issue_v(chunk + 2 * FS_WAVES);
+      body_v(chunk, vw);
     }
   }
-  // softmax denominators: every term added 0x4b000000 + round(p * 2^22); exact integer sums
 #pragma unroll
   for (int h = 0; h < G; ++h) {
-    const uint32_t v = li[h] - (uint32_t)my_chunks * 0x4b000000u;  // < 2^28 per lane
-    const int lo = wave_sum_i((int)(v & 0xffffu)), hi = wave_sum_i((int)(v >> 16));
-    if (lane == 0) lsum_sh[wave][h] = (long long)(uint32_t)lo + ((long long)(uint32_t)hi << 16);
+    const float ls = wave_sum(lsum[h]);
+    if (lane == 0) lsum_sh[wave][h] = ls;  // summed in wavefront order below: run-to-run deterministic
   }
-  __syncthreads();
+  lds_barrier();
+  if (clk && tid == 0) clk[2] = clock64();
+
+  // ------------------------------------------------------------------ phase C: candidates of the split
+  // The merge kernel needs a superset of the split's top Kt = min(top_k, n) scores per head that fits the
+  // candidate buffer (Kcap entries), in ascending position.  From the histograms: the smallest bucket index
+  // `cut` with count(bucket <= cut) >= Kt.  If that count fits, every position whose bucket is <= cut is
+  // emitted, one wavefront per (head, half of the split), the second half starting where the first one's count
+  // ends.  Otherwise (heavily tied scores) one wavefront falls back to an exact radix select over the keys.
+  const int Kcap = p.Kc;
+  const int Kt = min(p.top_k, n);
+  for (int h = wave; h < G; h += FS_WAVES) {
+    const int* h0 = hist + h * (SEG * 256);
+    // lane l owns buckets 4l .. 4l+3 (ascending bucket = descending score)
+    int c[4], c0sum = 0, mine = 0;
+    int a0[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      a0[u] = h0[4 * lane + u];
+      c[u] = a0[u] + ((SEG == 2) ? h0[256 + 4 * lane + u] : 0);
+      mine += c[u];
+      c0sum += a0[u];
+    }
+    const int incl = wave_incl_scan_i(mine);
+    const int incl0 = wave_incl_scan_i(c0sum);
+    int run = incl - mine, run0 = incl0 - c0sum;
+    int cut = -1, tot = 0, tot0 = 0;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int before = run;
+      run += c[u];
+      run0 += a0[u];
+      if (cut < 0 && before < Kt && run >= Kt) {
+        cut = 4 * lane + u;
+        tot = run;
+        tot0 = run0;
+      }
+    }
+    const unsigned long long who = __ballot(cut >= 0);
+    if (lane == 0) {
+      cut_sh[h] = 255;
+      cnt0_sh[h] = 0;
+      exact_sh[h] = 1;
+    }
+    if (who != 0ull) {
+      const int src = __ffsll((long long)who) - 1;
+      cut = __builtin_amdgcn_readlane(cut, src);
+      tot = __builtin_amdgcn_readlane(tot, src);
+      tot0 = __builtin_amdgcn_readlane(tot0, src);
+      if (lane == 0 && tot <= Kcap) {
+        cut_sh[h] = cut;
+        cnt0_sh[h] = tot0;
+        exact_sh[h] = 0;
+      }
+    }
+  }
+  lds_barrier();
+  if (clk && tid == 0) clk[6] = clock64();
+  for (int hs = wave; hs < G * SEG; hs += FS_WAVES) {
+    const int h = (SEG == 2) ? (hs >> 1) : hs, seg = (SEG == 2) ? (hs & 1) : 0;
+    const float* srow = sc + h * L;
+    uint32_t* ck = p.cand_key + (part_base + (size_t)h * p.n_splits) * Kcap;
+    int32_t* ci = p.cand_idx + (part_base + (size_t)h * p.n_splits) * Kcap;
+    if (!exact_sh[h]) {
+      const uint32_t cut = (uint32_t)cut_sh[h];
+      const float ba = bin_a_sh[h], bb = bin_b_sh[h];
+      const int tb = (SEG == 2) ? seg * (L / 2) : 0;
+      const int te = (SEG == 2) ? min(n, (seg + 1) * (L / 2)) : n;
+      // the emitted total is at most Kcap by construction of the cut
+      int count = __builtin_amdgcn_readfirstlane((seg == 1) ? cnt0_sh[h] : 0);
+      uint8_t* ckb = reinterpret_cast<uint8_t*>(ck);
+      uint8_t* cib = reinterpret_cast<uint8_t*>(ci);
+      for (int t0 = tb; t0 < te; t0 += 512) {
+        float kk[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int t = t0 + 64 * u + lane;
+          kk[u] = (t < te) ? srow[t] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int t = t0 + 64 * u + lane;
+          const uint32_t bin = (uint32_t)__builtin_amdgcn_fmed3f(__builtin_fmaf(kk[u], ba, bb), 0.f, 255.f);
+          const bool above = (t < te) && (bin <= cut);
+          const unsigned long long ma = __builtin_amdgcn_ballot_w64(above);
+          const uint32_t pos = (uint32_t)count + __builtin_amdgcn_mbcnt_hi((uint32_t)(ma >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)ma, 0u));
+          if (above) {
+            *reinterpret_cast<uint32_t*>(ckb + (size_t)(pos * 4u)) = score_key(kk[u]);
+            *reinterpret_cast<int32_t*>(cib + (size_t)(pos * 4u)) = s0 + t;
+          }
+          count += __popcll(ma);
+        }
+      }
+      if (lane == 0 && seg == SEG - 1) p.cand_cnt[part_base + (size_t)h * p.n_splits] = count;
+    } else if (seg == 0) {
+      // exact fallback: 8-bit radix select over the order-preserving keys (bits shared by every key skipped),
+      // then the keys above the K-th and the lowest-position ties that fill the quota
+      int* rh = reinterpret_cast<int*>(stage + wave * Lds::WAVE_STAGE);
+      uint32_t T = 0;
+      int quota = 0;
+      uint32_t kmin = 0xffffffffu, kmax = 0u;
+      for (int t = lane; t < n; t += 64) {
+        const uint32_t k = score_key(srow[t]);
+        kmin = min(kmin, k);
+        kmax = max(kmax, k);
+      }
+      kmin = wave_min_u(kmin);
+      kmax = wave_max_u(kmax);
+      const uint32_t diff = kmin ^ kmax;
+      if (diff == 0u) {  // every key equal: the lowest positions win
+        T = kmax;
+        quota = Kt;
+      } else {
+        int bits_left = 32 - __clz((int)diff);  // number of low bits that vary
+        uint32_t prefix = (bits_left == 32) ? 0u : (kmax >> bits_left);
+        int k_rem = Kt;
+        while (bits_left > 0) {
+          const int nb = min(8, bits_left);
+          const int shift = bits_left - nb;
+          const uint32_t dmask = (1u << nb) - 1u;
+          for (int i = lane; i < 256; i += 64) rh[i] = 0;
+          const bool first = (bits_left == 32);
+          const int hi_shift = first ? 0 : bits_left;
+          for (int t0 = 0; t0 < n; t0 += 64) {
+            const int t = t0 + lane;
+            const uint32_t k = (t < n) ? score_key(srow[t]) : 0u;
+            const bool inpre = (t < n) && (first || ((k >> hi_shift) == prefix));
+            if (inpre) atomicAdd(&rh[(int)((k >> shift) & dmask)], 1);
+          }
+          // lane l owns bins 255-4l .. 252-4l (descending), so a prefix scan over lanes counts the bins above
+          const int c3 = rh[255 - 4 * lane], c2 = rh[254 - 4 * lane], c1 = rh[253 - 4 * lane], c0 = rh[252 - 4 * lane];
+          const int mine = c0 + c1 + c2 + c3;
+          const int e3 = wave_incl_scan_i(mine) - mine;  // keys in bins above 255-4l
+          const int e2 = e3 + c3, e1 = e2 + c2, e0 = e1 + c1;
+          int cut = -1, above = 0;
+          if (e3 < k_rem && k_rem <= e3 + c3) { cut = 255 - 4 * lane; above = e3; }
+          else if (e2 < k_rem && k_rem <= e2 + c2) { cut = 254 - 4 * lane; above = e2; }
+          else if (e1 < k_rem && k_rem <= e1 + c1) { cut = 253 - 4 * lane; above = e1; }
+          else if (e0 < k_rem && k_rem <= e0 + c0) { cut = 252 - 4 * lane; above = e0; }
+          const unsigned long long who = __ballot(cut >= 0);
+          const int src = __ffsll((long long)who) - 1;
+          cut = __builtin_amdgcn_readlane(cut, src);
+          above = __builtin_amdgcn_readlane(above, src);
+          prefix = (prefix << nb) | (uint32_t)cut;
+          k_rem -= above;
+          bits_left = shift;
+        }
+        T = prefix;
+        quota = k_rem;
+      }
+      int count = 0, base_tie = 0;
+      for (int t0 = 0; t0 < n; t0 += 64) {
+        const int t = t0 + lane;
+        const uint32_t k = (t < n) ? score_key(srow[t]) : 0u;
+        const bool above = (t < n) && (k > T), tie = (t < n) && (k == T);
+        const unsigned long long ma = __ballot(above), mt = __ballot(tie);
+        const int pa = count + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(ma >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)ma, 0u));
+        const int pt = base_tie + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(mt >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mt, 0u));
+        if (above || (tie && pt < quota)) {
+          const int pos = pa + min(pt, quota);
+          if (pos < Kcap) {
+            ck[pos] = k;
+            ci[pos] = s0 + t;
+          }
+        }
+        count += __popcll(ma);
+        base_tie += __popcll(mt);
+      }
+      count += min(base_tie, quota);
+      if (lane == 0) p.cand_cnt[part_base + (size_t)h * p.n_splits] = min(Kcap, count);
+    }
+  }
+  lds_barrier();
   if (clk && tid == 0) clk[3] = clock64();
 
-  // Reduce the wavefronts' integer accumulators pairwise through LDS (the score rows are dead by now): in
-  // each round the upper half of the remaining wavefronts writes, the lower half adds.
-  v4i* slots = reinterpret_cast<v4i*>(smem);         // [4][AR][64]
-  v4i* fin = slots + 4 * AR * 64;                    // [NSET][AR][64]
+  // ---- exchange of the integer accumulators (the score rows are dead by now): every wavefront stores the
+  // rows that are used (0..12 of 16: lanes 0-47 whole registers, lanes 48-63 the first component), then each
+  // output element sums its eight partials.  D layout: row r of a tile sits in lane 16*(r>>2) + column,
+  // register r&3; rows are (limb, head), row 12 is the ones row.
+  constexpr int SPR = Lds::SPR;
+  v4i* xa = reinterpret_cast<v4i*>(smem);                                            // [wave][SPR][AR][48]
+  int* xb = reinterpret_cast<int*>(smem + (size_t)FS_WAVES * SPR * AR * 48 * 16);   // [wave][SPR][AR][16]
+  float lfin = 0.f;
+  if (tid < G) {
 #pragma unroll
-  for (int set = 0; set < NSET; ++set) {
-#pragma unroll
-    for (int stride = 4; stride >= 1; stride >>= 1) {
-      if (wave >= stride && wave < 2 * stride) {
-        v4i* dst = slots + (size_t)(wave - stride) * AR * 64 + lane;
-#pragma unroll
-        for (int t = 0; t < NTILE; ++t) dst[t * 64] = acc[set][t];
-#pragma unroll
-        for (int g = 0; g < NG; ++g) dst[(NTILE + g) * 64] = accw[set][g];
-      }
-      __syncthreads();
-      if (wave < stride) {
-        const v4i* src = slots + (size_t)wave * AR * 64 + lane;
-#pragma unroll
-        for (int t = 0; t < NTILE; ++t) acc[set][t] += src[t * 64];
-#pragma unroll
-        for (int g = 0; g < NG; ++g) accw[set][g] += src[(NTILE + g) * 64];
-      }
-      __syncthreads();
-    }
-    if (wave == 0) {
-      v4i* dst = fin + (size_t)set * AR * 64 + lane;
-#pragma unroll
-      for (int t = 0; t < NTILE; ++t) dst[t * 64] = acc[set][t];
-#pragma unroll
-      for (int g = 0; g < NG; ++g) dst[(NTILE + g) * 64] = accw[set][g];
-    }
+    for (int w = 0; w < FS_WAVES; ++w) lfin += lsum_sh[w][tid];
   }
-  __syncthreads();
-  // D layout: row r of a tile sits in lane 16*(r>>2) + column, register r&3; rows are (limb, head)
-  for (int i = tid; i < G * D; i += FS_THREADS) {
-    const int h = i / D, d = i % D;
-    const int set = h >> 2, hh = h & 3;
-    int tile, col;
-    if (K3) {
-      const int qc = d >> 5, rem = d & 31, kbyte = rem >> 2, e = rem & 3;
-      col = 2 * kbyte + ((e < 2) ? 1 : 0);
-      tile = 2 * qc + (e & 1);
-    } else {
-      const int qc = d >> 4, rem = d & 15, kbyte = rem >> 1;
-      col = 2 * kbyte + ((rem & 1) ? 0 : 1);
-      tile = qc;
+#pragma unroll
+  for (int round = 0; round < NSET / SPR; ++round) {
+    if (round > 0) lds_barrier();
+#pragma unroll
+    for (int sl = 0; sl < SPR; ++sl) {
+      const int set = round * SPR + sl;
+#pragma unroll
+      for (int r = 0; r < AR; ++r) {
+        const v4i v = (r < NTILE) ? acc[set][r < NTILE ? r : 0] : accw[set][r >= NTILE ? r - NTILE : 0];
+        if (lane < 48) xa[((size_t)(wave * SPR + sl) * AR + r) * 48 + lane] = v;
+        else xb[((wave * SPR + sl) * AR + r) * 16 + (lane - 48)] = v[0];
+      }
     }
-    const int g = (NG == 1) ? 0 : (d / (D / NG));
-    const v4i* tb = fin + ((size_t)set * AR + tile) * 64;
-    const long long i0 = tb[col][hh], i1 = tb[16 + col][hh], i2 = tb[32 + col][hh];
-    const long long cs = tb[48 + col][0];
-    const v4i* wb = fin + ((size_t)set * AR + NTILE + g) * 64;
-    const long long wsum = (long long)wb[32][hh] * 65536ll + (long long)wb[16][hh] * 256ll + (long long)wb[0][hh] +
-                           32896ll * 64ll * (long long)nch;
-    const long long tot = i2 * 65536ll + i1 * 256ll + i0 + 32896ll * cs - (long long)VOFF * wsum;
-    p.part_o[(part_base + (size_t)h * p.n_splits) * D + d] = (float)ldexp((double)tot, -E[g]);
+    lds_barrier();
+    for (int i = tid; i < SPR * 4 * D; i += FS_THREADS) {
+      const int hl = i / D, d = i % D;
+      const int sl = hl >> 2, hh = hl & 3;
+      const int set = round * SPR + sl, h = set * 4 + hh;
+      if (h >= G) continue;
+      int tile, col;
+      if (K3) {
+        const int qc = d >> 5, rem = d & 31, kbyte = rem >> 2, e = rem & 3;
+        col = 2 * kbyte + ((e < 2) ? 1 : 0);
+        tile = 2 * qc + (e & 1);
+      } else {
+        const int qc = d >> 4, rem = d & 15, kbyte = rem >> 1;
+        col = 2 * kbyte + ((rem & 1) ? 0 : 1);
+        tile = qc;
+      }
+      const int g = (NG == 1) ? 0 : (d / (D / NG));
+      int i0 = 0, i1 = 0, i2 = 0, cs = 0, w0 = 0, w1 = 0, w2 = 0;  // |partial| < 2^22 per wavefront: no overflow
+#pragma unroll
+      for (int w = 0; w < FS_WAVES; ++w) {
+        const v4i* ta = xa + ((size_t)(w * SPR + sl) * AR + tile) * 48;
+        i0 += ta[col][hh];
+        i1 += ta[16 + col][hh];
+        i2 += ta[32 + col][hh];
+        cs += xb[((w * SPR + sl) * AR + tile) * 16 + col];
+        const v4i* wa = xa + ((size_t)(w * SPR + sl) * AR + NTILE + g) * 48;
+        w0 += wa[0][hh];
+        w1 += wa[16][hh];
+        w2 += wa[32][hh];
+      }
+      const long long wsum = (long long)w2 * 65536ll + (long long)w1 * 256ll + (long long)w0 + 32896ll * 64ll * (long long)nch;
+      const long long tot = (long long)i2 * 65536ll + (long long)i1 * 256ll + (long long)i0 + 32896ll * (long long)cs - (long long)VOFF * wsum;
+      p.part_o[(part_base + (size_t)h * p.n_splits) * D + d] = (float)ldexp((double)tot, -E[g]);
+    }
   }
   if (tid < G) {
-    long long l = 0;
-#pragma unroll
-    for (int w = 0; w < FS_WAVES; ++w) l += lsum_sh[w][tid];
     p.part_m[part_base + (size_t)tid * p.n_splits] = m_sh[tid];
-    p.part_l[part_base + (size_t)tid * p.n_splits] = (float)ldexp((double)l, -22);
+    p.part_l[part_base + (size_t)tid * p.n_splits] = lfin;
   }
-  if (clk && tid == 0) { clk[4] = clock64(); clk[5] = clk[4]; }
+  if (clk && tid == 0) clk[4] = clock64();
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -1324,7 +1454,7 @@ template <int SCHEME, int G, int NG>
 int lmax_for() {
   using Lds = ScanLds<SCHEME, G, NG>;
   const size_t budget = (G <= 4) ? LDS_BUDGET_2WG : LDS_BUDGET_1WG;
-  const size_t fixed = Lds::stage_bytes() + 64 + 768;  // + static LDS of the kernel
+  const size_t fixed = Lds::AUX + Lds::stage_bytes() + 64 + 832;  // + static LDS of the kernel
   long lm = (long)((budget - fixed) / (Lds::per_position() + 1));  // +1: page table (4 bytes per 16 positions)
   lm = lm / 256 * 256;
   if (lm > FS_LMAX) lm = FS_LMAX;
