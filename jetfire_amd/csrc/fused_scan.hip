@@ -40,10 +40,6 @@ typedef float v2f __attribute__((ext_vector_type(2)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
 
-constexpr int FS_THREADS = 512;
-constexpr int FS_WAVES = 8;
-constexpr int FS_LMAX = 2048;          // positions per split (register-resident keys in phase C: 32 per lane)
-constexpr int FS_MAXCH = FS_LMAX / 64;
 constexpr int FS_MAX_TOPK = 1024;      // winners cached in LDS by the merge kernel
 constexpr int FS_CAND_SLACK = 256;     // extra candidate slots per (row, split)
 
@@ -60,6 +56,7 @@ struct FusedParams {
   float attn_scale;
   int top_k;
   int L, n_splits, Kc;
+  uint32_t kc_magic;  // ceil(2^32 / Kc)
   float* scores;  // optional (B, H_q, max_S)
   float* part_m;  // (B, H_q, NS)
   float* part_l;  // (B, H_q, NS)
@@ -108,7 +105,12 @@ template <int SCHEME, int G, int NG>
 struct ScanLds {
   static constexpr bool K3 = (SCHEME == JF_SCHEME_K3V2);
   static constexpr int NSET = (G + 3) / 4;
-  static constexpr int SEG = (G <= 4) ? 2 : 1;  // emission segments per head (one wavefront each)
+  // wavefronts per workgroup: sixteen where the register budget allows (128 VGPRs at 1024 threads), else eight
+  static constexpr int NW = (K3 && G <= 4) ? 16 : 8;
+  static constexpr int NT = NW * 64;
+  static constexpr int LMAX = NW * 256;  // four 64-position chunks per wavefront
+  // emission segments per head (one wavefront each)
+  static constexpr int SEG = (NW / G >= 4) ? 4 : ((NW / G >= 2) ? 2 : 1);
   static constexpr int KP = K3 ? 48 : 64;
   static constexpr int KROW = K3 ? 48 : 80;     // LDS pitch of a staged key row (INT4: padded against bank conflicts)
   static constexpr int VP = K3 ? 32 : 64;
@@ -118,13 +120,13 @@ struct ScanLds {
   static constexpr int KST = 64 * KROW;
   static constexpr int WAVE_STAGE = (VST + WL > KST) ? (VST + WL) : KST;
   static constexpr int ACC_REGS = 8 + NG;                   // v4i accumulators per set: 8 channel tiles + NG weight sums
-  static constexpr int SPR = NSET < 2 ? NSET : 2;           // sets exchanged per round
+  static constexpr int SPR = 1;                             // sets exchanged per round
   static constexpr int XWAVE = ACC_REGS * (48 * 16 + 16 * 4);  // bytes one wavefront writes per set (rows 0..12 only)
-  static constexpr int RED = FS_WAVES * SPR * XWAVE;
+  static constexpr int RED = NW * SPR * XWAVE;
   static constexpr int PREP = K3 ? (int)sizeof(K3Prep<NSET>) : (int)sizeof(QInt8F<G>);
   static constexpr int HIST = G * SEG * 256 * 4;
   static constexpr int AUX = ((PREP > HIST ? PREP : HIST) + 15) & ~15;
-  __host__ __device__ static constexpr int stage_bytes() { return FS_WAVES * WAVE_STAGE; }
+  __host__ __device__ static constexpr int stage_bytes() { return NW * WAVE_STAGE; }
   __host__ __device__ static constexpr size_t per_position() { return (size_t)G * 4; }
   __host__ __device__ static size_t aux_offset(int L) { return (per_position() * L + (size_t)(L / 16) * 4 + 15) & ~(size_t)15; }
   __host__ __device__ static size_t total(int L) {
@@ -156,7 +158,7 @@ __device__ inline float uniform_f(float v) {
 
 // ---------------------------------------------------------------------------------------------------
 template <int SCHEME, int G, int NG>
-__global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
+__global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kernel(FusedParams p) {
   using Lds = ScanLds<SCHEME, G, NG>;
   constexpr bool K3 = Lds::K3;
   constexpr int NSET = Lds::NSET;
@@ -169,7 +171,8 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
   constexpr int NTILE = 8;          // 8 MFMA column tiles of 16 channels
   constexpr int AR = Lds::ACC_REGS;
   constexpr float LOG2E = 1.44269504088896340736f;
-  constexpr int MAXIT = FS_LMAX / 64 / FS_WAVES;  // chunks per wavefront
+  constexpr int NW = Lds::NW, NT = Lds::NT;
+  constexpr int MAXIT = Lds::LMAX / 64 / NW;  // chunks per wavefront
 
   extern __shared__ __align__(16) uint8_t smem[];
   const int L = p.L;
@@ -178,11 +181,11 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
   uint8_t* aux = smem + Lds::aux_offset(L);
   uint8_t* stage = aux + Lds::AUX;
   int* hist = reinterpret_cast<int*>(aux);  // [G][SEG][256], valid after phase A
-  __shared__ float red_f[FS_WAVES][2 * G];
-  __shared__ uint32_t vmax_sh[FS_WAVES][2];
-  __shared__ float m_sh[G], bin_a_sh[G], bin_b_sh[G], lsum_sh[FS_WAVES][G];
+  __shared__ float red_f[NW][2 * G];
+  __shared__ uint32_t vmax_sh[NW][2];
+  __shared__ float m_sh[G], bin_a_sh[G], bin_b_sh[G], lsum_sh[NW][G];
   __shared__ int e_sh[2];
-  __shared__ int cut_sh[G], cnt0_sh[G], exact_sh[G];
+  __shared__ int cut_sh[G], segoff_sh[G][SEG + 1], exact_sh[G];
   __shared__ unsigned long long tmax_sh;
   if (threadIdx.x == 0) tmax_sh = 0ull;
 
@@ -207,9 +210,9 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
 
   if (n == 0) {  // nothing valid in this split: padding scores, empty partials
     if (p.scores)
-      for (int i = tid; i < G * n_cover; i += FS_THREADS)
+      for (int i = tid; i < G * n_cover; i += NT)
         p.scores[(head0 + i / n_cover) * (size_t)p.max_S + s0 + (i % n_cover)] = -INFINITY;
-    for (int i = tid; i < G * D; i += FS_THREADS) p.part_o[(part_base + (size_t)(i / D) * p.n_splits) * D + (i % D)] = 0.f;
+    for (int i = tid; i < G * D; i += NT) p.part_o[(part_base + (size_t)(i / D) * p.n_splits) * D + (i % D)] = 0.f;
     if (tid < G) {
       p.part_m[part_base + (size_t)tid * p.n_splits] = -INFINITY;
       p.part_l[part_base + (size_t)tid * p.n_splits] = 0.f;
@@ -225,15 +228,15 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
   const int nch = (n + 63) >> 6;
   {
     const int last_page = (n - 1) >> 4;
-    for (int i = tid; i < nch_cover * 4; i += FS_THREADS) sbase[i] = (int)(bt[(s0 >> 4) + min(i, last_page)] * BS);
+    for (int i = tid; i < nch_cover * 4; i += NT) sbase[i] = (int)(bt[(s0 >> 4) + min(i, last_page)] * BS);
   }
   // query elements of this thread (in flight while the page table arrives)
-  constexpr int QPT = (G * D + FS_THREADS - 1) / FS_THREADS;
-  static_assert(QPT == NSET, "one query element per thread and head set");
+  constexpr int QN = NSET * 4 * D;               // elements of the padded query block (whole head sets)
+  constexpr int QPT = (QN + NT - 1) / NT;
   float qv[QPT];
 #pragma unroll
   for (int it = 0; it < QPT; ++it) {
-    const int i = it * FS_THREADS + tid;
+    const int i = it * NT + tid;
     qv[it] = (i < G * D) ? bf16_to_f32(p.q[head0 * D + i]) : 0.f;
   }
   lds_barrier();
@@ -286,11 +289,11 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
   // first two chunks of this wavefront and the V scales of the split start now, before the query set-up
   KBuf Ka = {}, Kb = {};
   if (wave < nch_cover) Ka = issue_k(wave);
-  constexpr int VSPT = FS_LMAX / FS_THREADS;
+  constexpr int VSPT = Lds::LMAX / NT;
   uint32_t vsw[VSPT];
 #pragma unroll
   for (int i = 0; i < VSPT; ++i) {
-    const int t = tid + i * FS_THREADS;
+    const int t = tid + i * NT;
     vsw[i] = 0u;
     if (t < n) {
       const uint32_t slot = (uint32_t)(sbase[t >> 4] + (t & 15));
@@ -309,17 +312,20 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
       prep->eps[tid] = 256.0f * ((bf16_to_f32(f32_to_bf16(t3)) - t3) / sm);
     }
 #pragma unroll
-    for (int it = 0; it < NSET; ++it) {
-      const float x = qv[it];
-      const float am = wave_max(fabsf(x));
-      if (lane == 0) prep->amax_w[it * FS_WAVES + wave] = am;
+    for (int it = 0; it < QPT; ++it) {
+      const int c = it * NW + wave;  // 64-channel half row of this wavefront
+      if (c * 64 < QN) {             // uniform per wavefront
+        const float am = wave_max(fabsf(qv[it]));
+        if (lane == 0) prep->amax_w[c] = am;
+      }
     }
     lds_barrier();
 #pragma unroll
-    for (int it = 0; it < NSET; ++it) {
-      const int i = it * FS_THREADS + tid, h = i >> 7, d = i & 127;
+    for (int it = 0; it < QPT; ++it) {
+      const int i = it * NT + tid, h = i >> 7, d = i & 127;
       const float x = qv[it];
-      const int c = it * FS_WAVES + wave;  // 64-channel half row of this wavefront
+      const int c = it * NW + wave;
+      if (c * 64 >= QN) continue;
       const float amax = (NG == 2) ? prep->amax_w[c] : fmaxf(prep->amax_w[c & ~1], prep->amax_w[c | 1]);
       int e = 0;
       if (amax > 0.f && isfinite(amax)) (void)frexpf(amax, &e);  // amax = f * 2^e, f in [0.5, 1)
@@ -357,7 +363,7 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
     QInt8F<G>* qsh = reinterpret_cast<QInt8F<G>*>(aux);
 #pragma unroll
     for (int it = 0; it < QPT; ++it) {
-      const int i = it * FS_THREADS + tid;
+      const int i = it * NT + tid;
       if (i < G * D) {  // uniform per wavefront: G * D is a multiple of 64
         const int g = i >> 7, d = i & 127, kk = d >> 5;
         const float x = qv[it];
@@ -381,7 +387,7 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
     }
   }
   lds_barrier();
-  if (wave + FS_WAVES < nch_cover) Kb = issue_k(wave + FS_WAVES);
+  if (wave + NW < nch_cover) Kb = issue_k(wave + NW);
   if (clk && tid == 0) clk[7] = clock64();
 
   // ------------------------------------------------------------------ phase A
@@ -513,19 +519,20 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
         }
       }
     };
-    // at most FS_LMAX / 64 / FS_WAVES chunks per wavefront: straight-line code, so that the wait for a chunk's
+    // at most Lds::LMAX / 64 / NW chunks per wavefront: straight-line code, so that the wait for a chunk's
     // loads leaves the loads of the following chunks in flight
 #pragma unroll
     for (int it = 0; it < MAXIT; ++it) {
-      const int chunk = wave + it * FS_WAVES;
+      const int chunk = wave + it * NW;
       if (chunk < nch_cover) {
+        __builtin_amdgcn_s_setprio(3 - it);  // wavefronts that are behind get the issue slots first
         KBuf& cur = (it & 1) ? Kb : Ka;
         stash_k(cur);
         wave_lds_fence();
         uint32_t Sc[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) Sc[j] = cur.s[j];
-        if (it + 2 < MAXIT && chunk + 2 * FS_WAVES < nch_cover) cur = issue_k(chunk + 2 * FS_WAVES);
+        if (it + 2 < MAXIT && chunk + 2 * NW < nch_cover) cur = issue_k(chunk + 2 * NW);
         body(chunk, Sc);
         wave_lds_fence();
       }
@@ -578,13 +585,13 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
     };
 #pragma unroll
     for (int it = 0; it < MAXIT; ++it) {
-      const int chunk = wave + it * FS_WAVES;
+      const int chunk = wave + it * NW;
       if (chunk < nch_cover) {
         KBuf& cur = (it & 1) ? Kb : Ka;
         stash_k(cur);
         wave_lds_fence();
         const uint32_t ksw = cur.s[0];
-        if (it + 2 < MAXIT && chunk + 2 * FS_WAVES < nch_cover) cur = issue_k(chunk + 2 * FS_WAVES);
+        if (it + 2 < MAXIT && chunk + 2 * NW < nch_cover) cur = issue_k(chunk + 2 * NW);
         body(chunk, ksw);
         wave_lds_fence();
       }
@@ -622,10 +629,11 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
   };
   VBuf Va = {}, Vb = {};
   if (wave < nch) Va = issue_v(wave);
-  if (wave + FS_WAVES < nch) Vb = issue_v(wave + FS_WAVES);
+  if (wave + NW < nch) Vb = issue_v(wave + NW);
 
   if (clk && tid == 0) clk[9] = clock64();  // wavefront 0 finished its chunks
   if (clk && lane == 0) atomicMax(&tmax_sh, (unsigned long long)clock64());
+  __builtin_amdgcn_s_setprio(0);
   // split extrema per head; fixed-point exponent of the V scales; selection buckets
   {
     uint32_t vm0 = 0u, vm1 = 0u;
@@ -655,15 +663,15 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
   lds_barrier();  // phase A complete: the query constants are dead, their space becomes the histograms
   if (clk && tid == 0) { clk[8] = clock64(); clk[5] = (long long)tmax_sh; }
   if (p.scores)  // validation output
-    for (int i = tid; i < G * n_cover; i += FS_THREADS) {
+    for (int i = tid; i < G * n_cover; i += NT) {
       const int h = i / n_cover, t = i - h * n_cover;
       p.scores[(head0 + h) * (size_t)p.max_S + s0 + t] = sc[h * L + t];
     }
-  for (int i = tid; i < G * SEG * 256; i += FS_THREADS) hist[i] = 0;
+  for (int i = tid; i < G * SEG * 256; i += NT) hist[i] = 0;
   if (tid < G) {
     float m = red_f[0][tid], lo = red_f[0][G + tid];
 #pragma unroll
-    for (int w = 1; w < FS_WAVES; ++w) {
+    for (int w = 1; w < NW; ++w) {
       m = fmaxf(m, red_f[w][tid]);
       lo = fminf(lo, red_f[w][G + tid]);
     }
@@ -678,7 +686,7 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
     const int g = tid - 64;
     uint32_t vb = vmax_sh[0][g];
 #pragma unroll
-    for (int w = 1; w < FS_WAVES; ++w) vb = max(vb, vmax_sh[w][g]);
+    for (int w = 1; w < NW; ++w) vb = max(vb, vmax_sh[w][g]);
     const float v = bf16_to_f32((uint16_t)vb);
     int e = 0;
     if (v > 0.f && isfinite(v)) (void)frexpf(v, &e);  // v = f * 2^e, f in [0.5, 1)
@@ -722,13 +730,13 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
   // V operand (see below) is j
   const int tr_tok = (((r16 >> 1) & 3) << 1) | ((r16 >> 3) & 1);
   const uint8_t* wrow = wl + (kb4 * 16 + tr_tok) * 16 + (r16 & 1) * 8;
-  const int seg_chunk = L / 128;  // first chunk of the second half of the split
+  const int seg_chunks = L / 64 / SEG;  // chunks per emission segment
   auto body_v = [&](int chunk, uint32_t vsw) {
     const int t = chunk * 64 + lane;
     float vsf[NG];
     vsf[0] = ldexpf(bf16_to_f32((uint16_t)(vsw & 0xffffu)), E[0]);
     if (NG == 2) vsf[NG - 1] = ldexpf(bf16_to_f32((uint16_t)(vsw >> 16)), E[NG - 1]);
-    int* hb = hist + ((SEG == 2 && chunk >= seg_chunk) ? 256 : 0);
+    int* hb = hist + ((SEG == 1) ? 0 : (chunk / seg_chunks) * 256);
     const bool tv = t < n;
     uint32_t bits[NSET * 4][NG];
 #pragma unroll
@@ -824,15 +832,17 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
   };
 #pragma unroll
   for (int it = 0; it < MAXIT; ++it) {
-    const int chunk = wave + it * FS_WAVES;
+    const int chunk = wave + it * NW;
     if (chunk < nch) {
+      __builtin_amdgcn_s_setprio(3 - it);
       VBuf& cur = (it & 1) ? Vb : Va;
       stash_v(cur);
       const uint32_t vw = cur.w;
-      if (it + 2 < MAXIT && chunk + 2 * FS_WAVES < nch) cur = issue_v(chunk + 2 * FS_WAVES);
+      if (it + 2 < MAXIT && chunk + 2 * NW < nch) cur = issue_v(chunk + 2 * NW);
       body_v(chunk, vw);
     }
   }
+  __builtin_amdgcn_s_setprio(0);
 #pragma unroll
   for (int h = 0; h < G; ++h) {
     const float ls = wave_sum(lsum[h]);
@@ -849,65 +859,72 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
   // ends.  Otherwise (heavily tied scores) one wavefront falls back to an exact radix select over the keys.
   const int Kcap = p.Kc;
   const int Kt = min(p.top_k, n);
-  for (int h = wave; h < G; h += FS_WAVES) {
+  for (int h = wave; h < G; h += NW) {
     const int* h0 = hist + h * (SEG * 256);
-    // lane l owns buckets 4l .. 4l+3 (ascending bucket = descending score)
-    int c[4], c0sum = 0, mine = 0;
-    int a0[4];
+    // lane l owns buckets 4l .. 4l+3 (ascending bucket = descending score) of every segment's histogram
+    int cs[SEG][4], c[4], mine = 0;
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-      a0[u] = h0[4 * lane + u];
-      c[u] = a0[u] + ((SEG == 2) ? h0[256 + 4 * lane + u] : 0);
+      c[u] = 0;
+#pragma unroll
+      for (int sg = 0; sg < SEG; ++sg) {
+        cs[sg][u] = h0[sg * 256 + 4 * lane + u];
+        c[u] += cs[sg][u];
+      }
       mine += c[u];
-      c0sum += a0[u];
     }
     const int incl = wave_incl_scan_i(mine);
-    const int incl0 = wave_incl_scan_i(c0sum);
-    int run = incl - mine, run0 = incl0 - c0sum;
-    int cut = -1, tot = 0, tot0 = 0;
+    int run = incl - mine;
+    int cut = -1, tot = 0;
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int before = run;
       run += c[u];
-      run0 += a0[u];
       if (cut < 0 && before < Kt && run >= Kt) {
         cut = 4 * lane + u;
         tot = run;
-        tot0 = run0;
       }
     }
     const unsigned long long who = __ballot(cut >= 0);
-    if (lane == 0) {
-      cut_sh[h] = 255;
-      cnt0_sh[h] = 0;
-      exact_sh[h] = 1;
-    }
+    bool ok = false;
     if (who != 0ull) {
       const int src = __ffsll((long long)who) - 1;
       cut = __builtin_amdgcn_readlane(cut, src);
       tot = __builtin_amdgcn_readlane(tot, src);
-      tot0 = __builtin_amdgcn_readlane(tot0, src);
-      if (lane == 0 && tot <= Kcap) {
-        cut_sh[h] = cut;
-        cnt0_sh[h] = tot0;
-        exact_sh[h] = 0;
-      }
+      ok = tot <= Kcap;
+    }
+    if (!ok) cut = 255;
+    // entries every segment emits: its histogram summed over the buckets <= cut
+    int off = 0;
+#pragma unroll
+    for (int sg = 0; sg < SEG; ++sg) {
+      int part = 0;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) part += (4 * lane + u <= cut) ? cs[sg][u] : 0;
+      part = wave_sum_i(part);
+      if (lane == 0) segoff_sh[h][sg] = off;
+      off += part;
+    }
+    if (lane == 0) {
+      segoff_sh[h][SEG] = off;
+      cut_sh[h] = cut;
+      exact_sh[h] = ok ? 0 : 1;
     }
   }
   lds_barrier();
   if (clk && tid == 0) clk[6] = clock64();
-  for (int hs = wave; hs < G * SEG; hs += FS_WAVES) {
-    const int h = (SEG == 2) ? (hs >> 1) : hs, seg = (SEG == 2) ? (hs & 1) : 0;
+  for (int hs = wave; hs < G * SEG; hs += NW) {
+    const int h = hs / SEG, seg = hs % SEG;
     const float* srow = sc + h * L;
     uint32_t* ck = p.cand_key + (part_base + (size_t)h * p.n_splits) * Kcap;
     int32_t* ci = p.cand_idx + (part_base + (size_t)h * p.n_splits) * Kcap;
     if (!exact_sh[h]) {
       const uint32_t cut = (uint32_t)cut_sh[h];
       const float ba = bin_a_sh[h], bb = bin_b_sh[h];
-      const int tb = (SEG == 2) ? seg * (L / 2) : 0;
-      const int te = (SEG == 2) ? min(n, (seg + 1) * (L / 2)) : n;
+      const int tb = seg * (L / SEG);
+      const int te = min(n, (seg + 1) * (L / SEG));
       // the emitted total is at most Kcap by construction of the cut
-      int count = __builtin_amdgcn_readfirstlane((seg == 1) ? cnt0_sh[h] : 0);
+      int count = __builtin_amdgcn_readfirstlane(segoff_sh[h][seg]);
       uint8_t* ckb = reinterpret_cast<uint8_t*>(ck);
       uint8_t* cib = reinterpret_cast<uint8_t*>(ci);
       for (int t0 = tb; t0 < te; t0 += 512) {
@@ -1019,11 +1036,11 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
   // register r&3; rows are (limb, head), row 12 is the ones row.
   constexpr int SPR = Lds::SPR;
   v4i* xa = reinterpret_cast<v4i*>(smem);                                            // [wave][SPR][AR][48]
-  int* xb = reinterpret_cast<int*>(smem + (size_t)FS_WAVES * SPR * AR * 48 * 16);   // [wave][SPR][AR][16]
+  int* xb = reinterpret_cast<int*>(smem + (size_t)NW * SPR * AR * 48 * 16);   // [wave][SPR][AR][16]
   float lfin = 0.f;
   if (tid < G) {
 #pragma unroll
-    for (int w = 0; w < FS_WAVES; ++w) lfin += lsum_sh[w][tid];
+    for (int w = 0; w < NW; ++w) lfin += lsum_sh[w][tid];
   }
 #pragma unroll
   for (int round = 0; round < NSET / SPR; ++round) {
@@ -1039,7 +1056,7 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
       }
     }
     lds_barrier();
-    for (int i = tid; i < SPR * 4 * D; i += FS_THREADS) {
+    for (int i = tid; i < SPR * 4 * D; i += NT) {
       const int hl = i / D, d = i % D;
       const int sl = hl >> 2, hh = hl & 3;
       const int set = round * SPR + sl, h = set * 4 + hh;
@@ -1057,7 +1074,7 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
       const int g = (NG == 1) ? 0 : (d / (D / NG));
       int i0 = 0, i1 = 0, i2 = 0, cs = 0, w0 = 0, w1 = 0, w2 = 0;  // |partial| < 2^22 per wavefront: no overflow
 #pragma unroll
-      for (int w = 0; w < FS_WAVES; ++w) {
+      for (int w = 0; w < NW; ++w) {
         const v4i* ta = xa + ((size_t)(w * SPR + sl) * AR + tile) * 48;
         i0 += ta[col][hh];
         i1 += ta[16 + col][hh];
@@ -1081,12 +1098,25 @@ __global__ __launch_bounds__(FS_THREADS) void fused_scan_kernel(FusedParams p) {
 }
 
 // ---------------------------------------------------------------------------------------------------
-constexpr int MG_THREADS = 1024;
+constexpr int MG_THREADS = 512;
 constexpr int MG_WAVES = MG_THREADS / 64;
-constexpr int MG_HIST = MG_WAVES / 2;
 constexpr int MG_MAX_SPLITS = 256;
-constexpr int MG_LDS_KEYS = 8192;  // candidate keys cached in LDS when they fit
+constexpr int MG_REGK = 16;        // candidate (key, position) pairs a thread keeps in registers
+constexpr int MG_BINS = 1024;      // linear score buckets of the threshold search
+constexpr int MG_LIST = 1024;      // members of the cut bucket resolved by rank counting
+constexpr int MG_BT_LDS = 4096;    // block-table entries cached in LDS (65536 positions)
 
+// Launch 2: one workgroup per (sequence, query head).
+//   1. split statistics -> M, l, o_hat
+//   2. the K-th largest candidate key tau (and how many keys equal to tau still belong to the top K): the
+//      candidates are dropped into MG_BINS linear score buckets between the smallest candidate and M, a scan
+//      finds the bucket that holds the K-th largest, and the few members of that bucket are ranked against
+//      each other (a bisection over the key range covers the case of more than MG_LIST members)
+//   3. ordered compaction of the winners (key > tau, or key == tau while the quota lasts; candidates are stored
+//      in position order, so ties resolve to the lower position and the output is ascending)
+//   4. slots, softmax weights, and the pre-correction terms over the winners' V rows.
+// The first MG_REGK * MG_THREADS candidates stay in registers from a single load; anything beyond that is
+// re-read from global memory in every pass.
 template <int VBITS, int NG>
 __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) {
   constexpr int VP = D * VBITS / 8;
@@ -1094,20 +1124,27 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   constexpr int DW = VP / 4;            // dwords per V row
   constexpr int CPD = 32 / VBITS;       // codes per dword
   constexpr int WPI = 64 / DW;          // winners per wavefront instruction
-  __shared__ uint32_t keys_sh[MG_LDS_KEYS];
-  __shared__ int hist[MG_HIST][256];  // one histogram per pair of wavefronts
-  __shared__ int suffix_wave[4];
-  __shared__ int cut_bin_sh, above_sh;
-  __shared__ int wave_above[MG_WAVES], wave_tie[MG_WAVES];
+  __shared__ int hist[MG_BINS];
+  __shared__ uint32_t lkey[MG_LIST];
   __shared__ float coef_sh[MG_MAX_SPLITS];
-  __shared__ float stat_sh[2];
   __shared__ int cnt_sh[MG_MAX_SPLITS];
+  __shared__ int bt_sh[MG_BT_LDS];
+  __shared__ uint32_t win_key[FS_MAX_TOPK];
+  __shared__ int win_idx[FS_MAX_TOPK];
   __shared__ int win_slot[FS_MAX_TOPK];
   __shared__ float win_w[FS_MAX_TOPK];
+  __shared__ int cnt_a[MG_REGK * MG_WAVES], cnt_t[MG_REGK * MG_WAVES];
+  __shared__ float red_sh[4][D];
   __shared__ float old_sh[MG_WAVES][D];
   __shared__ float w_sh[MG_WAVES];
+  __shared__ float wred_f[MG_WAVES];
+  __shared__ uint32_t wred_u[MG_WAVES];
+  __shared__ int wred_i[MG_WAVES], wred_j[MG_WAVES];
+  __shared__ int lcount_sh, cut_sh, above_sh, quota_sh, tot_a_sh, tot_t_sh;
+  __shared__ uint32_t tau_sh;
 
-  const int b = blockIdx.x, hq = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int b = blockIdx.x, hq = blockIdx.y, tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const size_t bh = (size_t)b * p.H_q + hq;
   const int NS = p.n_splits, Kc = p.Kc, K = p.top_k;
   const int hkv = hq / (p.H_q / p.H_kv);
@@ -1117,296 +1154,352 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   const int64_t* bt = p.block_table + (size_t)b * p.max_blocks;
   int64_t* out_idx = p.topk_idx + bh * (size_t)K;
   int64_t* out_slot = p.topk_slots + bh * (size_t)K;
+  const int flat = NS * Kc;
+  const int rounds = (flat + MG_THREADS - 1) / MG_THREADS;
+  const int nblk_lds = min(p.max_blocks, MG_BT_LDS);
 
   long long* mclk = p.phase_clock ? p.phase_clock + (size_t)p.B * p.H_kv * p.n_splits * 10 + bh * 8 : nullptr;
   if (mclk && tid == 0) mclk[0] = clock64();
-  // ---- split statistics: M, coefficients e^{m_i - M}, l
-  float mloc = -INFINITY;
-  for (int s = tid; s < NS; s += MG_THREADS) mloc = fmaxf(mloc, p.part_m[bh * NS + s]);
-  mloc = wave_max(mloc);
-  if (lane == 0) hist[0][wave] = __builtin_bit_cast(int, mloc);
-  __syncthreads();
+
+  // ---- everything that does not depend on anything else is requested first, in the order of its use
+  float pm = -INFINITY, pl = 0.f;
+  int my_cnt = 0;
+  if (tid < NS) {
+    pm = p.part_m[bh * NS + tid];
+    pl = p.part_l[bh * NS + tid];
+    my_cnt = cc[tid];
+  }
+  uint32_t kreg[MG_REGK];
+  int ireg[MG_REGK];
+#pragma unroll
+  for (int r = 0; r < MG_REGK; ++r) {
+    const int f = r * MG_THREADS + tid;
+    kreg[r] = (f < flat) ? ck[f] : 0u;
+  }
+#pragma unroll
+  for (int r = 0; r < MG_REGK; ++r) {
+    const int f = r * MG_THREADS + tid;
+    ireg[r] = (f < flat) ? ci[f] : 0;
+  }
+  if (tid < NS) cnt_sh[tid] = my_cnt;
+  // o_hat: four thread groups take every fourth split (first four terms requested now)
+  constexpr int PO_PRE = 4;
+  float po[PO_PRE];
+  {
+    const int d = tid & (D - 1), q4 = tid >> 7;
+#pragma unroll
+    for (int i = 0; i < PO_PRE; ++i) {
+      const int sp = q4 + 4 * i;
+      po[i] = (sp < NS) ? p.part_o[(bh * NS + sp) * D + d] : 0.f;
+    }
+  }
+  for (int i = tid; i < nblk_lds; i += MG_THREADS) bt_sh[i] = (int)bt[i];
+  for (int i = tid; i < MG_BINS; i += MG_THREADS) hist[i] = 0;
+  if (tid == 0) lcount_sh = 0;
+
+  // ---- split statistics: M, coefficients e^{m_i - M}, l, o_hat
+  {
+    const float v = wave_max(pm);
+    if (lane == 0) wred_f[wave] = v;
+  }
+  lds_barrier();
+  if (mclk && tid == 0) mclk[6] = clock64();
   float M = -INFINITY;
 #pragma unroll
-  for (int w = 0; w < MG_WAVES; ++w) M = fmaxf(M, __builtin_bit_cast(float, hist[0][w]));
+  for (int w = 0; w < MG_WAVES; ++w) M = fmaxf(M, wred_f[w]);
   if (!isfinite(M)) M = 0.f;
-  for (int s = tid; s < NS; s += MG_THREADS) {
-    const float ms = p.part_m[bh * NS + s];
-    coef_sh[s] = (ms == -INFINITY) ? 0.f : __expf(ms - M);
+  const float coef = (pm == -INFINITY) ? 0.f : __expf(pm - M);
+  if (tid < NS) coef_sh[tid] = coef;
+  {
+    const float v = wave_sum(pl * coef);  // fixed reduction tree: deterministic
+    lds_barrier();                      // wred_f was read above
+    if (lane == 0) wred_f[wave] = v;
   }
-  __syncthreads();
-  if (tid == 0) {
-    float l = 0.f;
-    for (int s = 0; s < NS; ++s) l = __builtin_fmaf(p.part_l[bh * NS + s], coef_sh[s], l);  // fixed order
-    stat_sh[0] = l;
-    stat_sh[1] = (l > 0.f) ? 1.0f / l : 0.f;
-  }
-  __syncthreads();
-  const float inv_z = stat_sh[1];
-  if (tid < D) {
+  // candidates outside their list's count are not candidates: key 0 (no finite score maps to it)
+  int total = 0;
+  for (int s2 = 0; s2 < NS; ++s2) total += cnt_sh[s2];
+  auto valid_f = [&](int f) -> bool {
+    const int s2 = (int)__umulhi((uint32_t)f, p.kc_magic);  // f / Kc, exact for f < 2^21
+    return f < flat && (f - s2 * Kc) < cnt_sh[s2];
+  };
+#pragma unroll
+  for (int r = 0; r < MG_REGK; ++r)
+    if (!valid_f(r * MG_THREADS + tid)) kreg[r] = 0u;
+  lds_barrier();
+  if (mclk && tid == 0) mclk[7] = clock64();
+  float lsum = 0.f;
+#pragma unroll
+  for (int w = 0; w < MG_WAVES; ++w) lsum += wred_f[w];
+  const float inv_z = (lsum > 0.f) ? 1.0f / lsum : 0.f;
+  {
+    // o_hat: four thread groups take every fourth split, then a fixed-order sum
+    const int d = tid & (D - 1), q4 = tid >> 7;
     float o = 0.f;
-    for (int s = 0; s < NS; ++s) o = __builtin_fmaf(p.part_o[(bh * NS + s) * D + tid], coef_sh[s], o);
-    p.o_hat[bh * D + tid] = o * inv_z;
+#pragma unroll
+    for (int i = 0; i < PO_PRE; ++i) {
+      const int sp = q4 + 4 * i;
+      if (sp < NS) o = __builtin_fmaf(po[i], coef_sh[sp], o);
+    }
+    for (int sp = q4 + 4 * PO_PRE; sp < NS; sp += 4) o = __builtin_fmaf(p.part_o[(bh * NS + sp) * D + d], coef_sh[sp], o);
+    red_sh[q4][d] = o;
   }
+  lds_barrier();
+  if (tid < D) p.o_hat[bh * D + tid] = (((red_sh[0][tid] + red_sh[1][tid]) + red_sh[2][tid]) + red_sh[3][tid]) * inv_z;
   if (tid == 0 && p.softmax_m) {
     p.softmax_m[bh] = M;
     p.softmax_inv_z[bh] = inv_z;
   }
-
   if (mclk && tid == 0) mclk[1] = clock64();
-  // ---- global top-k among the candidates (flat index f = split * Kc + j, valid when j < cnt[split])
-  const int flat = NS * Kc;
-  const bool in_lds = flat <= MG_LDS_KEYS;
-  for (int s2 = tid; s2 < NS; s2 += MG_THREADS) cnt_sh[s2] = cc[s2];
-  __syncthreads();
-  int total = 0;
-  for (int s2 = 0; s2 < NS; ++s2) total += cnt_sh[s2];
-  if (in_lds) {  // unused slots become key 0, which no finite score maps to
-    for (int f0 = 0; f0 < flat; f0 += 4 * MG_THREADS) {
-      uint32_t kv[4];
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int f = f0 + u * MG_THREADS + tid;
-        kv[u] = 0u;
-        if (f < flat) {
-          const int s2 = f / Kc;
-          if (f - s2 * Kc < cnt_sh[s2]) kv[u] = ck[f];
-        }
-      }
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int f = f0 + u * MG_THREADS + tid;
-        if (f < flat) keys_sh[f] = kv[u];
-      }
-    }
-  }
-  __syncthreads();
-  auto cand_key = [&](int f, bool& ok) -> uint32_t {
-    if (in_lds) {
-      const uint32_t k = keys_sh[f];
-      ok = k != 0u;
-      return k;
-    }
-    const int s2 = f / Kc;
-    ok = (f - s2 * Kc) < cnt_sh[s2];
-    return ok ? ck[f] : 0u;
+
+  // key of candidate f in pass-over-all-candidates loops: registers first, global memory beyond
+  auto key_of = [&](int r) -> uint32_t {
+    const int f = r * MG_THREADS + tid;
+    return valid_f(f) ? ck[f] : 0u;
   };
-  if (mclk && tid == 0) mclk[2] = clock64();
+  // number of candidates with key >= x (x > 0), identical in every thread
+  auto count_ge = [&](uint32_t x) -> int {
+    int c = 0;
+#pragma unroll
+    for (int r = 0; r < MG_REGK; ++r) c += __popcll(__builtin_amdgcn_ballot_w64(kreg[r] >= x));
+    for (int r = MG_REGK; r < rounds; ++r) c += __popcll(__builtin_amdgcn_ballot_w64(key_of(r) >= x));
+    lds_barrier();
+    if (lane == 0) wred_i[wave] = c;
+    lds_barrier();
+    int t = 0;
+#pragma unroll
+    for (int w = 0; w < MG_WAVES; ++w) t += wred_i[w];
+    return t;
+  };
+
   uint32_t tau = 0;
   int quota = 0;
   const bool take_all = (total <= K);
   if (!take_all) {
-    // bits shared by every candidate key are skipped (the candidates are the upper tail of the row, so sign and
-    // exponent usually agree); the remaining bits are resolved 8 at a time
+    // range of the candidate keys
     uint32_t kmin = 0xffffffffu, kmax = 0u;
-    for (int f = tid; f < flat; f += MG_THREADS) {
-      bool ok;
-      const uint32_t key = cand_key(f, ok);
-      if (ok) { kmin = min(kmin, key); kmax = max(kmax, key); }
+#pragma unroll
+    for (int r = 0; r < MG_REGK; ++r)
+      if (kreg[r] != 0u) { kmin = min(kmin, kreg[r]); kmax = max(kmax, kreg[r]); }
+    for (int r = MG_REGK; r < rounds; ++r) {
+      const uint32_t k = key_of(r);
+      if (k != 0u) { kmin = min(kmin, k); kmax = max(kmax, k); }
     }
     kmin = wave_min_u(kmin);
     kmax = wave_max_u(kmax);
-    if (lane == 0) { hist[0][wave] = (int)kmin; hist[1][wave] = (int)kmax; }
-    __syncthreads();
+    if (lane == 0) { wred_u[wave] = kmin; wred_i[wave] = (int)kmax; }
+    lds_barrier();
 #pragma unroll
-    for (int w = 0; w < MG_WAVES; ++w) { kmin = min(kmin, (uint32_t)hist[0][w]); kmax = max(kmax, (uint32_t)hist[1][w]); }
-    __syncthreads();
-    const uint32_t diff = kmin ^ kmax;
-    int bits_left = (diff == 0u) ? 0 : 32 - __clz((int)diff);
-    uint32_t prefix = (bits_left == 32) ? 0u : (kmax >> bits_left);
-    int k_rem = K;
-    while (bits_left > 0) {
-      const int nb = min(8, bits_left);
-      const int shift = bits_left - nb;
-      const uint32_t dmask = (1u << nb) - 1u;
-      const bool first = (bits_left == 32);
-      const int hi_shift = first ? 0 : bits_left;
-      for (int i = tid; i < MG_HIST * 256; i += MG_THREADS) (&hist[0][0])[i] = 0;
-      __syncthreads();
-      for (int f = tid; f < flat; f += MG_THREADS) {
-        bool ok;
-        const uint32_t key = cand_key(f, ok);
-        if (ok && (first || (key >> hi_shift) == prefix)) atomicAdd(&hist[wave >> 1][(key >> shift) & dmask], 1);
-      }
-      __syncthreads();
-      if (tid < 256) {
-        // thread tid covers bin 255 - tid, so an inclusive scan over threads counts the keys in bins >= it
-        const int bin = 255 - tid;
-        int rcnt = 0;
+    for (int w = 0; w < MG_WAVES; ++w) { kmin = min(kmin, wred_u[w]); kmax = max(kmax, (uint32_t)wred_i[w]); }
+    const float hi = key_to_score(kmax), lo = key_to_score(kmin);
+    const float range = hi - lo;
+    const float iw = (range > 0.f && isfinite(range)) ? ((float)MG_BINS - 0.01f) / range : 0.f;
+    const float ba = -iw, bb = isfinite(hi) ? hi * iw : 0.f;
+    auto bin_of = [&](uint32_t k) -> int {
+      return (int)__builtin_amdgcn_fmed3f(__builtin_fmaf(key_to_score(k), ba, bb), 0.f, (float)(MG_BINS - 1));
+    };
 #pragma unroll
-        for (int w = 0; w < MG_HIST; ++w) rcnt += hist[w][bin];
-        const int incl_r = wave_incl_scan_i(rcnt);
-        if (lane == 63) suffix_wave[wave] = incl_r;
-        hist[0][bin] = rcnt;      // own bin only: keep the totals for the second step
-        hist[1][bin] = incl_r;
+    for (int r = 0; r < MG_REGK; ++r)
+      if (kreg[r] != 0u) atomicAdd(&hist[bin_of(kreg[r])], 1);
+    for (int r = MG_REGK; r < rounds; ++r) {
+      const uint32_t k = key_of(r);
+      if (k != 0u) atomicAdd(&hist[bin_of(k)], 1);
+    }
+    lds_barrier();
+    {
+      // thread t owns buckets 2t, 2t+1 (bucket 0 = largest scores): which bucket holds the K-th largest
+      const int c0 = hist[2 * tid], c1 = hist[2 * tid + 1];
+      const int incl = wave_incl_scan_i(c0 + c1);
+      if (lane == 63) wred_j[wave] = incl;
+      lds_barrier();
+      int before = 0;
+      for (int w = 0; w < wave; ++w) before += wred_j[w];
+      const int e0 = before + incl - c0 - c1, e1 = e0 + c0, e2 = e1 + c1;
+      if (e0 < K && K <= e1) { cut_sh = 2 * tid; above_sh = e0; }
+      else if (e1 < K && K <= e2) { cut_sh = 2 * tid + 1; above_sh = e1; }
+    }
+    lds_barrier();
+    const int cut = cut_sh, need = K - above_sh;  // `need` of the cut bucket's members belong to the top K
+#pragma unroll
+    for (int r = 0; r < MG_REGK; ++r)
+      if (kreg[r] != 0u && bin_of(kreg[r]) == cut) {
+        const int i = atomicAdd(&lcount_sh, 1);
+        if (i < MG_LIST) lkey[i] = kreg[r];
       }
-      __syncthreads();
-      if (tid < 256) {
-        const int bin = 255 - tid;
-        int before = 0;
-        for (int w = 0; w < wave; ++w) before += suffix_wave[w];
-        const int s_incl = hist[1][bin] + before, s_excl = s_incl - hist[0][bin];
-        if (s_excl < k_rem && k_rem <= s_incl) {
-          cut_bin_sh = bin;
-          above_sh = s_excl;
+    for (int r = MG_REGK; r < rounds; ++r) {
+      const uint32_t k = key_of(r);
+      if (k != 0u && bin_of(k) == cut) {
+        const int i = atomicAdd(&lcount_sh, 1);
+        if (i < MG_LIST) lkey[i] = k;
+      }
+    }
+    lds_barrier();
+    const int m = lcount_sh;
+    if (m <= MG_LIST) {
+      // rank counting: the member with fewer than `need` larger members and at least `need` members >= it
+      for (int i = tid; i < m; i += MG_THREADS) {
+        const uint32_t k = lkey[i];
+        int gt = 0, ge = 0;
+        for (int j = 0; j < m; ++j) {
+          const uint32_t o = lkey[j];
+          gt += (o > k) ? 1 : 0;
+          ge += (o >= k) ? 1 : 0;
+        }
+        if (gt < need && need <= ge) {  // every thread that gets here writes the same pair
+          tau_sh = k;
+          quota_sh = need - gt;
         }
       }
-      __syncthreads();
-      prefix = (prefix << nb) | (uint32_t)cut_bin_sh;
-      k_rem -= above_sh;
-      bits_left = shift;
-      __syncthreads();
+      lds_barrier();
+      tau = tau_sh;
+      quota = quota_sh;
+    } else {
+      // bisection over the key range: largest x with count(key >= x) >= K
+      uint32_t lo_k = kmin, hi_k = kmax;  // invariant: count_ge(lo_k) >= K
+      while (lo_k < hi_k) {
+        const uint32_t mid = lo_k + (hi_k - lo_k + 1u) / 2u;
+        if (count_ge(mid) >= K) lo_k = mid;
+        else hi_k = mid - 1u;
+      }
+      tau = lo_k;
+      quota = K - ((tau == 0xffffffffu) ? 0 : count_ge(tau + 1u));
     }
-    tau = prefix;
-    quota = k_rem;
   }
-  if (mclk && tid == 0) mclk[3] = clock64();
-  // ordered compaction: winners' candidate ids go to LDS in ascending position order.  Pass 1 stores every
-  // (round, wavefront) count, one thread-block scan turns them into offsets, pass 2 places the winners:
-  // two barriers instead of two per round.
-  constexpr int MAX_ROUNDS = MG_LDS_KEYS / MG_THREADS;  // rounds handled by the batched path
-  const int rounds = (flat + MG_THREADS - 1) / MG_THREADS;
+  if (mclk && tid == 0) mclk[2] = clock64();
+
+  // ---- ordered compaction: pass 1 stores every (round, wavefront) count, one scan turns them into offsets,
+  // pass 2 places the winners; the owner of a winner stores its key and position
   int base_above = 0, base_tie = 0;
-  if (rounds <= MAX_ROUNDS) {
-    int* cnt_a = &hist[0][0];                 // [rounds][MG_WAVES]
-    int* cnt_t = &hist[0][0] + MAX_ROUNDS * MG_WAVES;
-    unsigned long long ma_r[MAX_ROUNDS], mt_r[MAX_ROUNDS];
+  {
+    unsigned long long ma_r[MG_REGK], mt_r[MG_REGK];
 #pragma unroll
-    for (int r = 0; r < MAX_ROUNDS; ++r) {
-      ma_r[r] = 0ull; mt_r[r] = 0ull;
-      if (r < rounds) {
-        const int f = r * MG_THREADS + tid;
-        bool above = false, tie = false;
-        if (f < flat) {
-          bool ok;
-          const uint32_t key = cand_key(f, ok);
-          if (ok) {
-            if (take_all) above = true;
-            else { above = key > tau; tie = key == tau; }
-          }
-        }
-        ma_r[r] = __ballot(above);
-        mt_r[r] = __ballot(tie);
-        if (lane == 0) {
-          cnt_a[r * MG_WAVES + wave] = __popcll(ma_r[r]);
-          cnt_t[r * MG_WAVES + wave] = __popcll(mt_r[r]);
-        }
-      }
-    }
-    __syncthreads();
-    if (wave == 0) {  // exclusive scan of the (round, wave) counts, 2 entries per lane (MAX_ROUNDS*MG_WAVES == 128)
-      const int n_ent = rounds * MG_WAVES;
-      const int i0 = 2 * lane, i1 = 2 * lane + 1;
-      const int a0 = (i0 < n_ent) ? cnt_a[i0] : 0, a1 = (i1 < n_ent) ? cnt_a[i1] : 0;
-      const int t0 = (i0 < n_ent) ? cnt_t[i0] : 0, t1 = (i1 < n_ent) ? cnt_t[i1] : 0;
-      const int ia = wave_incl_scan_i(a0 + a1), it = wave_incl_scan_i(t0 + t1);
-      if (i0 < n_ent) { cnt_a[i0] = ia - a0 - a1; cnt_t[i0] = it - t0 - t1; }
-      if (i1 < n_ent) { cnt_a[i1] = ia - a1; cnt_t[i1] = it - t1; }
-      if (lane == 63) { cut_bin_sh = ia; above_sh = it; }  // totals
-    }
-    __syncthreads();
-#pragma unroll
-    for (int r = 0; r < MAX_ROUNDS; ++r) {
-      if (r < rounds) {
-        const int f = r * MG_THREADS + tid;
-        const unsigned long long ma = ma_r[r], mt = mt_r[r];
-        const bool above = (ma >> lane) & 1ull, tie = (mt >> lane) & 1ull;
-        const int pa = cnt_a[r * MG_WAVES + wave] + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(ma >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)ma, 0u));
-        const int pt = cnt_t[r * MG_WAVES + wave] + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(mt >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mt, 0u));
-        if (above || (tie && pt < quota)) {
-          const int pos = pa + min(pt, quota);
-          if (pos < K) win_slot[pos] = f;  // candidate id for now
-        }
-      }
-    }
-    base_above = cut_bin_sh;
-    base_tie = above_sh;
-    __syncthreads();
-  } else {
-    for (int r = 0; r < rounds; ++r) {
-      const int f = r * MG_THREADS + tid;
-      bool above = false, tie = false;
-      if (f < flat) {
-        bool ok;
-        const uint32_t key = cand_key(f, ok);
-        if (ok) {
-          if (take_all) above = true;
-          else { above = key > tau; tie = key == tau; }
-        }
-      }
-      const unsigned long long ma = __ballot(above), mt = __ballot(tie);
+    for (int r = 0; r < MG_REGK; ++r) {
+      const uint32_t key = kreg[r];
+      const bool above = (key != 0u) && (take_all || key > tau), tie = (key != 0u) && !take_all && key == tau;
+      ma_r[r] = __builtin_amdgcn_ballot_w64(above);
+      mt_r[r] = __builtin_amdgcn_ballot_w64(tie);
       if (lane == 0) {
-        wave_above[wave] = __popcll(ma);
-        wave_tie[wave] = __popcll(mt);
+        cnt_a[r * MG_WAVES + wave] = __popcll(ma_r[r]);
+        cnt_t[r * MG_WAVES + wave] = __popcll(mt_r[r]);
       }
-      __syncthreads();
-      int pa = base_above + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(ma >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)ma, 0u));
-      int pt = base_tie + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(mt >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mt, 0u));
-      int tot_a = 0, tot_t = 0;
+    }
+    lds_barrier();
+    if (wave == 0) {  // exclusive scan of the (round, wave) counts, 2 entries per lane
+      static_assert(MG_REGK * MG_WAVES == 128, "two entries per lane");
+      const int i0 = 2 * lane, i1 = 2 * lane + 1;
+      const int a0 = cnt_a[i0], a1 = cnt_a[i1], t0 = cnt_t[i0], t1 = cnt_t[i1];
+      const int ia = wave_incl_scan_i(a0 + a1), it = wave_incl_scan_i(t0 + t1);
+      cnt_a[i0] = ia - a0 - a1; cnt_t[i0] = it - t0 - t1;
+      cnt_a[i1] = ia - a1; cnt_t[i1] = it - t1;
+      if (lane == 63) { tot_a_sh = ia; tot_t_sh = it; }
+    }
+    lds_barrier();
 #pragma unroll
-      for (int w = 0; w < MG_WAVES; ++w) {
-        if (w < wave) { pa += wave_above[w]; pt += wave_tie[w]; }
-        tot_a += wave_above[w];
-        tot_t += wave_tie[w];
-      }
+    for (int r = 0; r < MG_REGK; ++r) {
+      const unsigned long long ma = ma_r[r], mt = mt_r[r];
+      const bool above = (ma >> lane) & 1ull, tie = (mt >> lane) & 1ull;
+      const int pa = cnt_a[r * MG_WAVES + wave] + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(ma >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)ma, 0u));
+      const int pt = cnt_t[r * MG_WAVES + wave] + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(mt >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mt, 0u));
       if (above || (tie && pt < quota)) {
         const int pos = pa + min(pt, quota);
-        if (pos < K) win_slot[pos] = f;
+        if (pos < K) {
+          win_key[pos] = kreg[r];
+          win_idx[pos] = ireg[r];
+        }
       }
-      base_above += tot_a;
-      base_tie += tot_t;
-      __syncthreads();
     }
+    base_above = tot_a_sh;
+    base_tie = tot_t_sh;
+    lds_barrier();
+  }
+  for (int r = MG_REGK; r < rounds; ++r) {  // candidates beyond the register-resident ones, one round at a time
+    const int f = r * MG_THREADS + tid;
+    const uint32_t key = key_of(r);
+    const bool above = (key != 0u) && (take_all || key > tau), tie = (key != 0u) && !take_all && key == tau;
+    const unsigned long long ma = __builtin_amdgcn_ballot_w64(above), mt = __builtin_amdgcn_ballot_w64(tie);
+    if (lane == 0) {
+      wred_i[wave] = __popcll(ma);
+      wred_j[wave] = __popcll(mt);
+    }
+    lds_barrier();
+    int pa = base_above + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(ma >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)ma, 0u));
+    int pt = base_tie + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(mt >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mt, 0u));
+    int tot_a = 0, tot_t = 0;
+#pragma unroll
+    for (int w = 0; w < MG_WAVES; ++w) {
+      if (w < wave) { pa += wred_i[w]; pt += wred_j[w]; }
+      tot_a += wred_i[w];
+      tot_t += wred_j[w];
+    }
+    if (above || (tie && pt < quota)) {
+      const int pos = pa + min(pt, quota);
+      if (pos < K) {
+        win_key[pos] = key;
+        win_idx[pos] = ci[f];
+      }
+    }
+    base_above += tot_a;
+    base_tie += tot_t;
+    lds_barrier();
   }
   const int n_out = min(K, base_above + min(base_tie, quota));
-  // one thread per winner: position, paged slot, softmax weight (all loads independent); entry r of
-  // win_slot is read and rewritten by thread r only
+  if (mclk && tid == 0) mclk[3] = clock64();
+
+  // one thread per winner: position, paged slot, softmax weight
   for (int r = tid; r < K; r += MG_THREADS) {
     int64_t position = -1, slot = -1;
     int wslot = -1;
     float ww = 0.f;
     if (r < n_out) {
-      const int f = win_slot[r];
-      position = ci[f];
+      position = win_idx[r];
       const int blk = (int)(position / BS);
-      slot = (blk < p.max_blocks) ? bt[blk] * BS + (position % BS) : -1;
+      if (blk < p.max_blocks) slot = (int64_t)((blk < nblk_lds) ? (int64_t)bt_sh[blk] : bt[blk]) * BS + (position % BS);
       wslot = (slot >= 0 && slot < p.num_slots) ? (int)slot : -1;
-      ww = __expf(key_to_score(ck[f]) - M) * inv_z;
+      ww = __expf(key_to_score(win_key[r]) - M) * inv_z;
     }
     out_idx[r] = position;
     out_slot[r] = slot;
     win_slot[r] = wslot;
     win_w[r] = ww;
   }
-  __syncthreads();
-
+  lds_barrier();
   if (mclk && tid == 0) mclk[4] = clock64();
+
   // ---- pre-correction over the winners.  One winner row per DW lanes: lane (w_in, dwi) holds dword dwi of
   // the winner's packed V row (CPD codes) and accumulates its CPD channels; winners are visited in a fixed
-  // order, so the sums are run-to-run deterministic.
+  // order, so the sums are run-to-run deterministic.  Four rows per lane are requested before any is used.
   const uint8_t* vbase = p.v_data + (size_t)hkv * p.num_slots * VP;
-  const uint16_t* vsbase = p.v_scales + (size_t)hkv * p.num_slots * NG;
+  const uint8_t* vsbase = reinterpret_cast<const uint8_t*>(p.v_scales + (size_t)hkv * p.num_slots * NG);
   const int dwi = lane % DW, w_in = lane / DW;
+  const int g_of_lane = (NG == 1) ? 0 : ((dwi * CPD) / (D / NG));
   float acc[CPD];
 #pragma unroll
   for (int c = 0; c < CPD; ++c) acc[c] = 0.f;
   float accw = 0.f;
-  for (int k0 = wave * WPI; k0 < n_out; k0 += MG_WAVES * WPI) {
-    const int k = k0 + w_in;
-    const int slot = (k < n_out) ? win_slot[k] : -1;
-    if (slot >= 0) {
-      const float w = win_w[k];
-      const uint32_t word = reinterpret_cast<const uint32_t*>(vbase + (size_t)slot * VP)[dwi];
-      const int g = (NG == 1) ? 0 : ((dwi * CPD) / (D / NG));
-      const float ws = w * bf16_to_f32(vsbase[(size_t)slot * NG + g]);
+  constexpr int UNR = 4;
+  for (int k0 = wave * WPI; k0 < n_out; k0 += UNR * MG_WAVES * WPI) {
+    uint32_t word[UNR];
+    uint16_t sbits[UNR];
+    float wv[UNR];
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      const int k = k0 + u * MG_WAVES * WPI + w_in;
+      const int slot = (k < n_out) ? win_slot[k] : -1;
+      wv[u] = (slot >= 0) ? win_w[k] : 0.f;
+      const uint32_t sl = (uint32_t)max(slot, 0);
+      word[u] = *reinterpret_cast<const uint32_t*>(vbase + (size_t)(sl * (uint32_t)VP) + dwi * 4);
+      sbits[u] = *reinterpret_cast<const uint16_t*>(vsbase + (size_t)(sl * (uint32_t)(NG * 2)) + g_of_lane * 2);
+    }
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      const float ws = wv[u] * bf16_to_f32(sbits[u]);  // zero for padding rows
       // byte `byte` of the dword holds its codes MSB first; channel of code c in the dword = dwi*CPD + c
 #pragma unroll
       for (int c = 0; c < CPD; ++c) {
         const int byte = c / (8 / VBITS), inb = c % (8 / VBITS);
-        const int code = (int)((word >> (8 * byte + (8 - VBITS * (inb + 1)))) & ((1u << VBITS) - 1u)) - VOFF;
+        const int code = (int)((word[u] >> (8 * byte + (8 - VBITS * (inb + 1)))) & ((1u << VBITS) - 1u)) - VOFF;
         acc[c] = __builtin_fmaf(ws, (float)code, acc[c]);
       }
-      if (dwi == 0) accw += w;
+      if (dwi == 0) accw += wv[u];
     }
   }
   // reduce over the WPI winners of a wavefront instruction (lanes with equal dwi), then over wavefronts
@@ -1421,7 +1514,7 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
     for (int c = 0; c < CPD; ++c) old_sh[wave][dwi * CPD + c] = acc[c];
     if (dwi == 0) w_sh[wave] = accw;
   }
-  __syncthreads();
+  lds_barrier();
   if (tid < D) {
     float o = 0.f;
 #pragma unroll
@@ -1453,11 +1546,11 @@ constexpr size_t LDS_BUDGET_1WG = 160 * 1024 - 1024;
 template <int SCHEME, int G, int NG>
 int lmax_for() {
   using Lds = ScanLds<SCHEME, G, NG>;
-  const size_t budget = (G <= 4) ? LDS_BUDGET_2WG : LDS_BUDGET_1WG;
+  const size_t budget = (G <= 4 && Lds::NW == 8) ? LDS_BUDGET_2WG : LDS_BUDGET_1WG;
   const size_t fixed = Lds::AUX + Lds::stage_bytes() + 64 + 832;  // + static LDS of the kernel
   long lm = (long)((budget - fixed) / (Lds::per_position() + 1));  // +1: page table (4 bytes per 16 positions)
   lm = lm / 256 * 256;
-  if (lm > FS_LMAX) lm = FS_LMAX;
+  if (lm > Lds::LMAX) lm = Lds::LMAX;
   if (lm < 256) lm = 256;
   return (int)lm;
 }
@@ -1478,7 +1571,9 @@ inline void fused_plan(int scheme, int NG, int B, int H_q, int H_kv, int max_S, 
                        int* kc_out) {
   const int G = H_q / H_kv;
   const int units = B * H_kv > 0 ? B * H_kv : 1;
-  const int wg_target = (G <= 4) ? 512 : 256;  // two (one) resident workgroups per CU on 256 CUs
+  // two resident workgroups per CU on 256 CUs where a workgroup has eight wavefronts and a small score block,
+  // one otherwise
+  const int wg_target = (G <= 4 && scheme != JF_SCHEME_K3V2) ? 512 : 256;
   int target = wg_target / units;
   if (target < 1) target = 1;
   int L = (max_S + target - 1) / target;
@@ -1523,7 +1618,7 @@ int launch_scan(const FusedParams& p, hipStream_t st) {
   }
   const bool prof = g_prof.armed && g_prof.used + 2 <= (int)g_prof.ev.size();
   if (prof) JF_CHECK_HIP(hipEventRecord(g_prof.ev[g_prof.used], st));
-  hipLaunchKernelGGL(kern, dim3(p.n_splits, p.H_kv, p.B), dim3(FS_THREADS), smem, st, p);
+  hipLaunchKernelGGL(kern, dim3(p.n_splits, p.H_kv, p.B), dim3(ScanLds<SCHEME, G, NG>::NT), smem, st, p);
   JF_CHECK_LAUNCH();
   if (prof) {
     JF_CHECK_HIP(hipEventRecord(g_prof.ev[g_prof.used + 1], st));
@@ -1585,6 +1680,7 @@ extern "C" int jf_fused_scan_topk(int scheme, int group_size, const uint16_t* q,
   p.B = B; p.H_q = H_q; p.H_kv = H_kv; p.max_S = max_S; p.max_blocks = max_blocks; p.num_slots = num_slots;
   p.attn_scale = attn_scale; p.top_k = top_k;
   fused_plan(scheme, NGv, B, H_q, H_kv, max_S, top_k, &p.L, &p.n_splits, &p.Kc);
+  p.kc_magic = (uint32_t)((0x100000000ull + (uint64_t)p.Kc - 1) / (uint64_t)p.Kc);
   JF_CHECK_ARG(p.n_splits <= MG_MAX_SPLITS, "fused_scan: too many splits (%d > %d)", p.n_splits, MG_MAX_SPLITS);
   const WsLayout wl = ws_layout(B, H_q, p.n_splits, p.Kc);
   JF_CHECK_ARG(workspace && workspace_bytes >= wl.total, "fused_scan: workspace too small (%zu < %zu)", workspace_bytes, wl.total);
