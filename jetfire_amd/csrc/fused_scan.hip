@@ -152,6 +152,14 @@ __device__ inline void wave_lds_fence() {
 // that are still in flight (the prefetched key / value rows), which no other wavefront consumes.
 __device__ inline void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
+// s_setprio takes an immediate; `p` is a compile-time constant after unrolling
+__device__ inline void set_wave_prio(int p) {
+  if (p >= 3) __builtin_amdgcn_s_setprio(3);
+  else if (p == 2) __builtin_amdgcn_s_setprio(2);
+  else if (p == 1) __builtin_amdgcn_s_setprio(1);
+  else __builtin_amdgcn_s_setprio(0);
+}
+
 __device__ inline float uniform_f(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, v)));
 }
@@ -525,7 +533,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     for (int it = 0; it < MAXIT; ++it) {
       const int chunk = wave + it * NW;
       if (chunk < nch_cover) {
-        __builtin_amdgcn_s_setprio(3 - it);  // wavefronts that are behind get the issue slots first
+        set_wave_prio(3 - it);  // wavefronts that are behind get the issue slots first
         KBuf& cur = (it & 1) ? Kb : Ka;
         stash_k(cur);
         wave_lds_fence();
@@ -834,7 +842,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   for (int it = 0; it < MAXIT; ++it) {
     const int chunk = wave + it * NW;
     if (chunk < nch) {
-      __builtin_amdgcn_s_setprio(3 - it);
+      set_wave_prio(3 - it);
       VBuf& cur = (it & 1) ? Vb : Va;
       stash_v(cur);
       const uint32_t vw = cur.w;

@@ -83,6 +83,85 @@ __device__ inline void quant_row(const uint16_t* __restrict__ xrow, uint8_t* __r
   }
 }
 
+// Fast path (16-byte aligned rows): sixteen lanes own one row, lane l holds channels 8l .. 8l+7 (one 16-byte
+// load), group maxima are DPP reductions inside the 16-lane row, and the packed row leaves as dword stores
+// that are contiguous across the lanes of a row.  A wavefront converts four rows at a time.
+template <int CTRL>
+__device__ inline uint32_t dpp_u32(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, true);
+}
+template <int CTRL>
+__device__ inline float dpp_f32(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+
+template <int NBITS>
+__global__ __launch_bounds__(256) void quant_write16_kernel(RowSrc s0, RowDst d0, RowSrc s1, RowDst d1,
+                                                            const int64_t* __restrict__ slots, int64_t T,
+                                                            int H_kv, int n_tensors, int group_size) {
+  constexpr int QMAX = (1 << (NBITS - 1)) - 1;
+  constexpr int OFF = 1 << (NBITS - 1);
+  const int l16 = threadIdx.x & 15;
+  const int64_t unit = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+  const int64_t total = T * H_kv * n_tensors;
+  // rows past the end and masked rows still take part in the cross-lane steps (with zeros)
+  bool live = unit < total;
+  const int64_t uc = live ? unit : 0;
+  const int which = (int)(uc / (T * H_kv));
+  const int64_t rem = uc - (int64_t)which * T * H_kv;
+  const int64_t t = rem / H_kv;
+  const int h = (int)(rem - t * H_kv);
+  const int64_t slot = slots[t];
+  live = live && slot >= 0;
+  const RowSrc& s = which ? s1 : s0;
+  const RowDst& d = which ? d1 : d0;
+  const uint16_t* xrow = s.x + t * s.stride_t + (int64_t)h * s.stride_h;
+  uint4 raw = make_uint4(0u, 0u, 0u, 0u);
+  if (live) raw = reinterpret_cast<const uint4*>(xrow)[l16];
+  float x[8];
+  x[0] = bf16_to_f32((uint16_t)(raw.x & 0xffffu)); x[1] = bf16_to_f32((uint16_t)(raw.x >> 16));
+  x[2] = bf16_to_f32((uint16_t)(raw.y & 0xffffu)); x[3] = bf16_to_f32((uint16_t)(raw.y >> 16));
+  x[4] = bf16_to_f32((uint16_t)(raw.z & 0xffffu)); x[5] = bf16_to_f32((uint16_t)(raw.z >> 16));
+  x[6] = bf16_to_f32((uint16_t)(raw.w & 0xffffu)); x[7] = bf16_to_f32((uint16_t)(raw.w >> 16));
+  float amax = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(x[i]));
+  // all-reduce over the lanes of one scale group: 4, 8 or 16 lanes
+  amax = fmaxf(amax, dpp_f32<0xB1>(amax));   // quad_perm [1,0,3,2]
+  amax = fmaxf(amax, dpp_f32<0x4E>(amax));   // quad_perm [2,3,0,1]
+  if (group_size >= 64) amax = fmaxf(amax, dpp_f32<0x141>(amax));   // row_half_mirror: lane i <-> 7 - i
+  if (group_size >= 128) amax = fmaxf(amax, dpp_f32<0x140>(amax));  // row_mirror: lane i <-> 15 - i
+  const float sraw = fmaxf(amax / (float)QMAX, 1e-8f);
+  const uint16_t sb = f32_to_bf16(sraw);
+  const float sf = bf16_to_f32(sb);
+  uint32_t c[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) c[i] = (uint32_t)((int)fminf(fmaxf(rintf(x[i] / sf), (float)-QMAX), (float)QMAX) + OFF);
+  uint8_t* drow = d.data + (int64_t)h * d.data_stride_h + slot * d.data_stride_slot;
+  uint16_t* srow = d.scale + (int64_t)h * d.scale_stride_h + slot * d.scale_stride_slot;
+  const int lpg = group_size >> 3;  // lanes per scale group
+  if (live && (l16 & (lpg - 1)) == 0) srow[l16 / lpg] = sb;
+  if (NBITS == 4) {
+    // byte j of the lane's dword = (c[2j] << 4) | c[2j+1]
+    const uint32_t v = ((c[0] << 4) | c[1]) | (((c[2] << 4) | c[3]) << 8) | (((c[4] << 4) | c[5]) << 16) | (((c[6] << 4) | c[7]) << 24);
+    if (live) reinterpret_cast<uint32_t*>(drow)[l16] = v;
+  } else if (NBITS == 2) {
+    // the lane's 8 codes are two bytes, four codes each MSB first; lane pairs share a dword
+    const uint32_t hw = ((c[0] << 6) | (c[1] << 4) | (c[2] << 2) | c[3]) | (((c[4] << 6) | (c[5] << 4) | (c[6] << 2) | c[7]) << 8);
+    const uint32_t nb = dpp_u32<0xB1>(hw);  // neighbour inside the lane pair
+    if (live && (l16 & 1) == 0) reinterpret_cast<uint32_t*>(drow)[l16 >> 1] = hw | (nb << 16);
+  } else {
+    // INT3 planar: the lane's 8 codes are the 24-bit word l16, MSB first; plane p holds byte p of every word.
+    // Lane (4j + p), p < 3, assembles dword j of plane p from the four words of its quad.
+    const uint32_t w = (c[0] << 21) | (c[1] << 18) | (c[2] << 15) | (c[3] << 12) | (c[4] << 9) | (c[5] << 6) | (c[6] << 3) | c[7];
+    const uint32_t w0 = dpp_u32<0x00>(w), w1 = dpp_u32<0x55>(w), w2 = dpp_u32<0xAA>(w), w3 = dpp_u32<0xFF>(w);  // quad broadcasts
+    const int pl = l16 & 3;
+    const int sh = 16 - 8 * pl;
+    const uint32_t v = ((w0 >> sh) & 255u) | (((w1 >> sh) & 255u) << 8) | (((w2 >> sh) & 255u) << 16) | (((w3 >> sh) & 255u) << 24);
+    if (live && pl < 3) reinterpret_cast<uint32_t*>(drow)[4 * pl + (l16 >> 2)] = v;
+  }
+}
+
 // units = T * H_kv * n_tensors (n_tensors = 2 for the fused K+V INT4 launch)
 template <int NBITS>
 __global__ __launch_bounds__(256) void quant_write_kernel(RowSrc s0, RowDst d0, RowSrc s1, RowDst d1,
@@ -104,6 +183,10 @@ __global__ __launch_bounds__(256) void quant_write_kernel(RowSrc s0, RowDst d0, 
   uint8_t* drow = d.data + (int64_t)h * d.data_stride_h + slot * d.data_stride_slot;
   uint16_t* srow = d.scale + (int64_t)h * d.scale_stride_h + slot * d.scale_stride_slot;
   quant_row<NBITS>(xrow, drow, srow, group_size, lane);
+}
+
+inline bool rows_16b_aligned(const void* x, int64_t stride_t, int64_t stride_h) {
+  return ((uintptr_t)x & 15) == 0 && stride_t % 8 == 0 && stride_h % 8 == 0;
 }
 
 int check_common(const void* x, const int64_t* slots, int64_t T, int H_kv, int group_size,
@@ -137,8 +220,16 @@ extern "C" int jf_quant_write_sym(const uint16_t* x, int64_t x_stride_t, int64_t
   RowSrc s{x, x_stride_t, x_stride_h};
   RowDst d{out_data, data_stride_h, data_stride_slot, out_scale, scale_stride_h, scale_stride_slot};
   const int64_t units = T * H_kv;
-  dim3 grid((unsigned)((units + 3) / 4)), block(256);
   hipStream_t st = (hipStream_t)stream;
+  if (rows_16b_aligned(x, x_stride_t, x_stride_h)) {
+    dim3 grid16((unsigned)((units + 15) / 16)), block16(256);
+    if (nbits == 2) hipLaunchKernelGGL(quant_write16_kernel<2>, grid16, block16, 0, st, s, d, s, d, slots, T, H_kv, 1, group_size);
+    else if (nbits == 3) hipLaunchKernelGGL(quant_write16_kernel<3>, grid16, block16, 0, st, s, d, s, d, slots, T, H_kv, 1, group_size);
+    else hipLaunchKernelGGL(quant_write16_kernel<4>, grid16, block16, 0, st, s, d, s, d, slots, T, H_kv, 1, group_size);
+    JF_CHECK_LAUNCH();
+    return JF_OK;
+  }
+  dim3 grid((unsigned)((units + 3) / 4)), block(256);
   if (nbits == 2) hipLaunchKernelGGL(quant_write_kernel<2>, grid, block, 0, st, s, d, s, d, slots, T, H_kv, 1, group_size);
   else if (nbits == 3) hipLaunchKernelGGL(quant_write_kernel<3>, grid, block, 0, st, s, d, s, d, slots, T, H_kv, 1, group_size);
   else hipLaunchKernelGGL(quant_write_kernel<4>, grid, block, 0, st, s, d, s, d, slots, T, H_kv, 1, group_size);
@@ -164,6 +255,12 @@ extern "C" int jf_quant_write_int4_sym_kv(const uint16_t* key, int64_t k_stride_
   RowDst d0{k_data, k_data_stride_h, k_data_stride_slot, k_scale, k_scale_stride_h, k_scale_stride_slot};
   RowDst d1{v_data, v_data_stride_h, v_data_stride_slot, v_scale, v_scale_stride_h, v_scale_stride_slot};
   const int64_t units = T * H_kv * 2;
+  if (rows_16b_aligned(key, k_stride_t, k_stride_h) && rows_16b_aligned(value, v_stride_t, v_stride_h)) {
+    dim3 grid16((unsigned)((units + 15) / 16)), block16(256);
+    hipLaunchKernelGGL(quant_write16_kernel<4>, grid16, block16, 0, (hipStream_t)stream, s0, d0, s1, d1, slots, T, H_kv, 2, group_size);
+    JF_CHECK_LAUNCH();
+    return JF_OK;
+  }
   dim3 grid((unsigned)((units + 3) / 4)), block(256);
   hipLaunchKernelGGL(quant_write_kernel<4>, grid, block, 0, (hipStream_t)stream, s0, d0, s1, d1, slots, T, H_kv, 2, group_size);
   JF_CHECK_LAUNCH();
