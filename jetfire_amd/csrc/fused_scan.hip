@@ -106,7 +106,7 @@ struct ScanLds {
   static constexpr bool K3 = (SCHEME == JF_SCHEME_K3V2);
   static constexpr int NSET = (G + 3) / 4;
   // wavefronts per workgroup: sixteen where the register budget allows (128 VGPRs at 1024 threads), else eight
-  static constexpr int NW = (K3 && G <= 4) ? 16 : 8;
+  static constexpr int NW = (G <= 4) ? 16 : 8;
   static constexpr int NT = NW * 64;
   static constexpr int LMAX = NW * 256;  // four 64-position chunks per wavefront
   // emission segments per head (one wavefront each)
@@ -1106,10 +1106,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
 }
 
 // ---------------------------------------------------------------------------------------------------
-constexpr int MG_THREADS = 512;
-constexpr int MG_WAVES = MG_THREADS / 64;
 constexpr int MG_MAX_SPLITS = 256;
-constexpr int MG_REGK = 16;        // candidate (key, position) pairs a thread keeps in registers
 constexpr int MG_BINS = 1024;      // linear score buckets of the threshold search
 constexpr int MG_LIST = 1024;      // members of the cut bucket resolved by rank counting
 constexpr int MG_BT_LDS = 4096;    // block-table entries cached in LDS (65536 positions)
@@ -1125,8 +1122,11 @@ constexpr int MG_BT_LDS = 4096;    // block-table entries cached in LDS (65536 p
 //   4. slots, softmax weights, and the pre-correction terms over the winners' V rows.
 // The first MG_REGK * MG_THREADS candidates stay in registers from a single load; anything beyond that is
 // re-read from global memory in every pass.
-template <int VBITS, int NG>
+// Two shapes: 512 threads x 16 register-resident candidates each (up to 8192 candidates, the common case)
+// and 1024 x 32 for long contexts with wide top-k.
+template <int VBITS, int NG, int MG_THREADS, int MG_REGK>
 __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) {
+  constexpr int MG_WAVES = MG_THREADS / 64;
   constexpr int VP = D * VBITS / 8;
   constexpr int VOFF = 1 << (VBITS - 1);
   constexpr int DW = VP / 4;            // dwords per V row
@@ -1142,7 +1142,7 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   __shared__ int win_slot[FS_MAX_TOPK];
   __shared__ float win_w[FS_MAX_TOPK];
   __shared__ int cnt_a[MG_REGK * MG_WAVES], cnt_t[MG_REGK * MG_WAVES];
-  __shared__ float red_sh[4][D];
+  __shared__ float red_sh[MG_THREADS / D][D];
   __shared__ float old_sh[MG_WAVES][D];
   __shared__ float w_sh[MG_WAVES];
   __shared__ float wred_f[MG_WAVES];
@@ -1177,27 +1177,28 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
     pl = p.part_l[bh * NS + tid];
     my_cnt = cc[tid];
   }
+  const int rreg = min(rounds, MG_REGK);  // rounds whose candidates live in registers (uniform)
   uint32_t kreg[MG_REGK];
   int ireg[MG_REGK];
 #pragma unroll
   for (int r = 0; r < MG_REGK; ++r) {
     const int f = r * MG_THREADS + tid;
-    kreg[r] = (f < flat) ? ck[f] : 0u;
+    kreg[r] = (r < rreg && f < flat) ? ck[f] : 0u;
   }
 #pragma unroll
   for (int r = 0; r < MG_REGK; ++r) {
     const int f = r * MG_THREADS + tid;
-    ireg[r] = (f < flat) ? ci[f] : 0;
+    ireg[r] = (r < rreg && f < flat) ? ci[f] : 0;
   }
   if (tid < NS) cnt_sh[tid] = my_cnt;
-  // o_hat: four thread groups take every fourth split (first four terms requested now)
-  constexpr int PO_PRE = 4;
+  // o_hat: the thread groups of 128 take the splits round-robin (first terms requested now)
+  constexpr int PO_PRE = 2, PO_GRP = MG_THREADS / D;
   float po[PO_PRE];
   {
     const int d = tid & (D - 1), q4 = tid >> 7;
 #pragma unroll
     for (int i = 0; i < PO_PRE; ++i) {
-      const int sp = q4 + 4 * i;
+      const int sp = q4 + PO_GRP * i;
       po[i] = (sp < NS) ? p.part_o[(bh * NS + sp) * D + d] : 0.f;
     }
   }
@@ -1232,7 +1233,7 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   };
 #pragma unroll
   for (int r = 0; r < MG_REGK; ++r)
-    if (!valid_f(r * MG_THREADS + tid)) kreg[r] = 0u;
+    if (r < rreg && !valid_f(r * MG_THREADS + tid)) kreg[r] = 0u;
   lds_barrier();
   if (mclk && tid == 0) mclk[7] = clock64();
   float lsum = 0.f;
@@ -1245,14 +1246,19 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
     float o = 0.f;
 #pragma unroll
     for (int i = 0; i < PO_PRE; ++i) {
-      const int sp = q4 + 4 * i;
+      const int sp = q4 + PO_GRP * i;
       if (sp < NS) o = __builtin_fmaf(po[i], coef_sh[sp], o);
     }
-    for (int sp = q4 + 4 * PO_PRE; sp < NS; sp += 4) o = __builtin_fmaf(p.part_o[(bh * NS + sp) * D + d], coef_sh[sp], o);
+    for (int sp = q4 + PO_GRP * PO_PRE; sp < NS; sp += PO_GRP) o = __builtin_fmaf(p.part_o[(bh * NS + sp) * D + d], coef_sh[sp], o);
     red_sh[q4][d] = o;
   }
   lds_barrier();
-  if (tid < D) p.o_hat[bh * D + tid] = (((red_sh[0][tid] + red_sh[1][tid]) + red_sh[2][tid]) + red_sh[3][tid]) * inv_z;
+  if (tid < D) {
+    float o = red_sh[0][tid];
+#pragma unroll
+    for (int q = 1; q < PO_GRP; ++q) o += red_sh[q][tid];  // fixed order
+    p.o_hat[bh * D + tid] = o * inv_z;
+  }
   if (tid == 0 && p.softmax_m) {
     p.softmax_m[bh] = M;
     p.softmax_inv_z[bh] = inv_z;
@@ -1268,7 +1274,8 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   auto count_ge = [&](uint32_t x) -> int {
     int c = 0;
 #pragma unroll
-    for (int r = 0; r < MG_REGK; ++r) c += __popcll(__builtin_amdgcn_ballot_w64(kreg[r] >= x));
+    for (int r = 0; r < MG_REGK; ++r)
+      if (r < rreg) c += __popcll(__builtin_amdgcn_ballot_w64(kreg[r] >= x));
     for (int r = MG_REGK; r < rounds; ++r) c += __popcll(__builtin_amdgcn_ballot_w64(key_of(r) >= x));
     lds_barrier();
     if (lane == 0) wred_i[wave] = c;
@@ -1287,7 +1294,7 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
     uint32_t kmin = 0xffffffffu, kmax = 0u;
 #pragma unroll
     for (int r = 0; r < MG_REGK; ++r)
-      if (kreg[r] != 0u) { kmin = min(kmin, kreg[r]); kmax = max(kmax, kreg[r]); }
+      if (r < rreg && kreg[r] != 0u) { kmin = min(kmin, kreg[r]); kmax = max(kmax, kreg[r]); }
     for (int r = MG_REGK; r < rounds; ++r) {
       const uint32_t k = key_of(r);
       if (k != 0u) { kmin = min(kmin, k); kmax = max(kmax, k); }
@@ -1307,29 +1314,37 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
     };
 #pragma unroll
     for (int r = 0; r < MG_REGK; ++r)
-      if (kreg[r] != 0u) atomicAdd(&hist[bin_of(kreg[r])], 1);
+      if (r < rreg && kreg[r] != 0u) atomicAdd(&hist[bin_of(kreg[r])], 1);
     for (int r = MG_REGK; r < rounds; ++r) {
       const uint32_t k = key_of(r);
       if (k != 0u) atomicAdd(&hist[bin_of(k)], 1);
     }
     lds_barrier();
     {
-      // thread t owns buckets 2t, 2t+1 (bucket 0 = largest scores): which bucket holds the K-th largest
-      const int c0 = hist[2 * tid], c1 = hist[2 * tid + 1];
-      const int incl = wave_incl_scan_i(c0 + c1);
+      // thread t owns buckets BPT*t .. BPT*t + BPT-1 (bucket 0 = largest scores): which bucket holds the K-th largest
+      constexpr int BPT = MG_BINS / MG_THREADS;
+      int cb[BPT], mine = 0;
+#pragma unroll
+      for (int u = 0; u < BPT; ++u) {
+        cb[u] = hist[BPT * tid + u];
+        mine += cb[u];
+      }
+      const int incl = wave_incl_scan_i(mine);
       if (lane == 63) wred_j[wave] = incl;
       lds_barrier();
-      int before = 0;
-      for (int w = 0; w < wave; ++w) before += wred_j[w];
-      const int e0 = before + incl - c0 - c1, e1 = e0 + c0, e2 = e1 + c1;
-      if (e0 < K && K <= e1) { cut_sh = 2 * tid; above_sh = e0; }
-      else if (e1 < K && K <= e2) { cut_sh = 2 * tid + 1; above_sh = e1; }
+      int run = incl - mine;
+      for (int w = 0; w < wave; ++w) run += wred_j[w];
+#pragma unroll
+      for (int u = 0; u < BPT; ++u) {
+        if (run < K && K <= run + cb[u]) { cut_sh = BPT * tid + u; above_sh = run; }
+        run += cb[u];
+      }
     }
     lds_barrier();
     const int cut = cut_sh, need = K - above_sh;  // `need` of the cut bucket's members belong to the top K
 #pragma unroll
     for (int r = 0; r < MG_REGK; ++r)
-      if (kreg[r] != 0u && bin_of(kreg[r]) == cut) {
+      if (r < rreg && kreg[r] != 0u && bin_of(kreg[r]) == cut) {
         const int i = atomicAdd(&lcount_sh, 1);
         if (i < MG_LIST) lkey[i] = kreg[r];
       }
@@ -1378,40 +1393,58 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   // pass 2 places the winners; the owner of a winner stores its key and position
   int base_above = 0, base_tie = 0;
   {
-    unsigned long long ma_r[MG_REGK], mt_r[MG_REGK];
+    // (round, wavefront) counts of winners / ties, packed: low half = above, high half = ties
 #pragma unroll
     for (int r = 0; r < MG_REGK; ++r) {
-      const uint32_t key = kreg[r];
-      const bool above = (key != 0u) && (take_all || key > tau), tie = (key != 0u) && !take_all && key == tau;
-      ma_r[r] = __builtin_amdgcn_ballot_w64(above);
-      mt_r[r] = __builtin_amdgcn_ballot_w64(tie);
+      unsigned long long ma = 0ull, mt = 0ull;
+      if (r < rreg) {
+        const uint32_t key = kreg[r];
+        const bool above = (key != 0u) && (take_all || key > tau), tie = (key != 0u) && !take_all && key == tau;
+        ma = __builtin_amdgcn_ballot_w64(above);
+        mt = __builtin_amdgcn_ballot_w64(tie);
+      }
       if (lane == 0) {
-        cnt_a[r * MG_WAVES + wave] = __popcll(ma_r[r]);
-        cnt_t[r * MG_WAVES + wave] = __popcll(mt_r[r]);
+        cnt_a[r * MG_WAVES + wave] = __popcll(ma);
+        cnt_t[r * MG_WAVES + wave] = __popcll(mt);
       }
     }
     lds_barrier();
-    if (wave == 0) {  // exclusive scan of the (round, wave) counts, 2 entries per lane
-      static_assert(MG_REGK * MG_WAVES == 128, "two entries per lane");
-      const int i0 = 2 * lane, i1 = 2 * lane + 1;
-      const int a0 = cnt_a[i0], a1 = cnt_a[i1], t0 = cnt_t[i0], t1 = cnt_t[i1];
-      const int ia = wave_incl_scan_i(a0 + a1), it = wave_incl_scan_i(t0 + t1);
-      cnt_a[i0] = ia - a0 - a1; cnt_t[i0] = it - t0 - t1;
-      cnt_a[i1] = ia - a1; cnt_t[i1] = it - t1;
+    if (wave == 0) {  // exclusive scan of the (round, wave) counts, EPL consecutive entries per lane
+      constexpr int EPL = MG_REGK * MG_WAVES / 64;
+      int a[EPL], t[EPL], sa = 0, st = 0;
+#pragma unroll
+      for (int i = 0; i < EPL; ++i) {
+        a[i] = cnt_a[lane * EPL + i];
+        t[i] = cnt_t[lane * EPL + i];
+        sa += a[i];
+        st += t[i];
+      }
+      const int ia = wave_incl_scan_i(sa), it = wave_incl_scan_i(st);
+      int ra = ia - sa, rt = it - st;
+#pragma unroll
+      for (int i = 0; i < EPL; ++i) {
+        cnt_a[lane * EPL + i] = ra;
+        cnt_t[lane * EPL + i] = rt;
+        ra += a[i];
+        rt += t[i];
+      }
       if (lane == 63) { tot_a_sh = ia; tot_t_sh = it; }
     }
     lds_barrier();
 #pragma unroll
     for (int r = 0; r < MG_REGK; ++r) {
-      const unsigned long long ma = ma_r[r], mt = mt_r[r];
-      const bool above = (ma >> lane) & 1ull, tie = (mt >> lane) & 1ull;
-      const int pa = cnt_a[r * MG_WAVES + wave] + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(ma >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)ma, 0u));
-      const int pt = cnt_t[r * MG_WAVES + wave] + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(mt >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mt, 0u));
-      if (above || (tie && pt < quota)) {
-        const int pos = pa + min(pt, quota);
-        if (pos < K) {
-          win_key[pos] = kreg[r];
-          win_idx[pos] = ireg[r];
+      if (r < rreg) {
+        const uint32_t key = kreg[r];
+        const bool above = (key != 0u) && (take_all || key > tau), tie = (key != 0u) && !take_all && key == tau;
+        const unsigned long long ma = __builtin_amdgcn_ballot_w64(above), mt = __builtin_amdgcn_ballot_w64(tie);
+        const int pa = cnt_a[r * MG_WAVES + wave] + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(ma >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)ma, 0u));
+        const int pt = cnt_t[r * MG_WAVES + wave] + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(mt >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mt, 0u));
+        if (above || (tie && pt < quota)) {
+          const int pos = pa + min(pt, quota);
+          if (pos < K) {
+            win_key[pos] = kreg[r];
+            win_idx[pos] = ireg[r];
+          }
         }
       }
     }
@@ -1581,7 +1614,7 @@ inline void fused_plan(int scheme, int NG, int B, int H_q, int H_kv, int max_S, 
   const int units = B * H_kv > 0 ? B * H_kv : 1;
   // two resident workgroups per CU on 256 CUs where a workgroup has eight wavefronts and a small score block,
   // one otherwise
-  const int wg_target = (G <= 4 && scheme != JF_SCHEME_K3V2) ? 512 : 256;
+  const int wg_target = 256;
   int target = wg_target / units;
   if (target < 1) target = 1;
   int L = (max_S + target - 1) / target;
@@ -1735,13 +1768,20 @@ extern "C" int jf_fused_scan_topk(int scheme, int group_size, const uint16_t* q,
     }
   }
   if (rc != JF_OK) return rc;
-  dim3 mgrid(B, H_q), mblock(MG_THREADS);
+  dim3 mgrid(B, H_q);
+  const bool big = (long long)p.n_splits * p.Kc > 8192;
+#define JF_MERGE(VB, NGG)                                                                                   \
+  do {                                                                                                      \
+    if (big) hipLaunchKernelGGL((fused_merge_kernel<VB, NGG, 1024, 32>), mgrid, dim3(1024), 0, st, p);      \
+    else hipLaunchKernelGGL((fused_merge_kernel<VB, NGG, 512, 16>), mgrid, dim3(512), 0, st, p);            \
+  } while (0)
   if (scheme == JF_SCHEME_K3V2) {
-    if (NGv == 2) hipLaunchKernelGGL((fused_merge_kernel<2, 2>), mgrid, mblock, 0, st, p);
-    else hipLaunchKernelGGL((fused_merge_kernel<2, 1>), mgrid, mblock, 0, st, p);
+    if (NGv == 2) JF_MERGE(2, 2);
+    else JF_MERGE(2, 1);
   } else {
-    hipLaunchKernelGGL((fused_merge_kernel<4, 1>), mgrid, mblock, 0, st, p);
+    JF_MERGE(4, 1);
   }
+#undef JF_MERGE
   JF_CHECK_LAUNCH();
   return JF_OK;
 }
