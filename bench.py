@@ -71,6 +71,11 @@ def main() -> int:
     ap.add_argument("--paged", action="store_true", help="random block table instead of the identity mapping")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--graph", action="store_true", help="replay the step from a HIP graph (roofline timing stays eager)")
+    ap.add_argument("--handoff", dest="handoff", action="store_true", default=None,
+                    help="include the pinned hand-off and the CPU correction per layer (default for c4 and c5, "
+                         "whose definition is end to end)")
+    ap.add_argument("--no-handoff", dest="handoff", action="store_false")
+    ap.add_argument("--cpu-threads", type=int, default=16, help="CPU correction threads (hand-off mode)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run a plain 1 GiB device copy 10 times and exit (reference for the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -94,16 +99,29 @@ def main() -> int:
         torch.cuda.synchronize()
         print(json.dumps({"calibrate_copy_bytes_read": 1 << 30, "calibrate_copy_bytes_written": 1 << 30, "launches": 10}))
         return 0
-    w = workloads.build(args.workload, n_layers=args.layers)
+    handoff = args.handoff if args.handoff is not None else args.workload in ("c4", "c5")
+    if handoff and args.graph:
+        print("bench.py: --graph and the hand-off mode are exclusive", file=sys.stderr)
+        return 2
+    n_shadow = 4 if handoff else 0   # distinct host shadows, cycled over the layers (a layer's shadow is 2*H_kv*slots*256 B)
+    w = workloads.build(args.workload, n_layers=args.layers, keep_shadow=n_shadow)
     n_layers = len(w.layers)
     o_new = torch.zeros(w.B, w.H_q, 128, dtype=torch.bfloat16, device="cuda")
     out = torch.empty_like(o_new)
+    ctxs = []
+    if handoff:
+        ops.set_cpu_attn_threads(args.cpu_threads)
+        ctxs = [ops.CpuTopkHandoff(w.B, w.H_q, w.H_kv, w.top_k, ksh, vsh, w.attn_scale) for ksh, vsh in w.shadows]
 
     def step():
-        for lay in w.layers:
+        for li, lay in enumerate(w.layers):
             o_hat, slots, o_old, W, idx = ops.fused_attn_topk(
                 w.scheme, w.q, lay.k_data, lay.k_scales, lay.v_data, lay.v_scales, w.block_table, w.seq_lens,
                 w.S, w.H_q, w.H_kv, 16, w.top_k, w.attn_scale)
+            if ctxs:
+                h = ctxs[li % len(ctxs)]
+                h.submit(w.q, slots)
+                h.wait(o_new)
             ops.blend_unnorm_into(o_hat, o_old, W, o_new, out)
 
     for _ in range(args.warmup):
@@ -168,13 +186,17 @@ def main() -> int:
         "dtype": "u8 codes; int8/bf16 MFMA, fp32 softmax", "data": "synthetic",
         "config": {"workload": f"{args.workload}: B{w.B} Hq{w.H_q} Hkv{w.H_kv} D128 S{w.S} {w.scheme} g{w.group} "
                                f"top_k{w.top_k} x{n_layers} layers, {'paged (random)' if args.paged else 'identity'} block table",
-                   "packed_bytes_per_layer": bytes_layer, "launch": "hip-graph" if graph is not None else "eager"},
+                   "packed_bytes_per_layer": bytes_layer, "launch": "hip-graph" if graph is not None else "eager",
+                   "handoff": (f"pinned D2H of slots + CPU correction on {ops.get_cpu_attn_threads()} threads + H2D, every layer"
+                               if handoff else "not in the timed region (GPU path only)")},
         "roofline": {"bound": "hbm", "kernel": "fused_scan_kernel", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
                      "kernel_us": round(scan_us, 2), "launches_timed": launches.value},
     }
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(w)
+    for h in ctxs:
+        h.close()
     print(json.dumps(res))
     return 0
 

@@ -239,6 +239,89 @@ static void topk_attn_row(const uint16_t* q, const uint16_t* k_shadow, const uin
   for (int i = 0; i < D; ++i) out[i] = f32_to_bf16(o[i]);
 }
 
+#if defined(__x86_64__)
+// AVX2 + FMA form of the same row (selected at run time when the host supports it): eight fp32 lanes per
+// step, the rows of the next slots requested ahead of their use (the gather is DRAM-latency bound).
+__attribute__((target("avx2,fma"))) static inline __m256 bf16x8_to_f32(const uint16_t* p) {
+  return _mm256_castsi256_ps(_mm256_slli_epi32(_mm256_cvtepu16_epi32(_mm_loadu_si128(reinterpret_cast<const __m128i*>(p))), 16));
+}
+__attribute__((target("avx2,fma"))) static void topk_attn_row_avx2(const uint16_t* q, const uint16_t* k_shadow,
+                                                                   const uint16_t* v_shadow, int64_t num_slots,
+                                                                   const int64_t* head_map, const int64_t* slots, int K,
+                                                                   int H_kv, float scale, uint16_t* out, float* score_buf) {
+  constexpr int AHEAD = 8;
+  __m256 qv[D / 8];
+  for (int i = 0; i < D / 8; ++i) qv[i] = bf16x8_to_f32(q + 8 * i);
+  auto row_of = [&](const uint16_t* base, int k) -> const uint16_t* {
+    const int64_t s = slots[k], h = head_map[k];
+    if (s < 0 || s >= num_slots || h < 0 || h >= H_kv) return nullptr;
+    return base + ((size_t)h * num_slots + s) * D;
+  };
+  auto prefetch_row = [](const uint16_t* r) {
+    if (r) {
+      for (int b = 0; b < D * 2; b += 64) _mm_prefetch(reinterpret_cast<const char*>(r) + b, _MM_HINT_T0);
+    }
+  };
+  for (int k = 0; k < K && k < AHEAD; ++k) prefetch_row(row_of(k_shadow, k));
+  float mx = -INFINITY;
+  bool any = false;
+  for (int k = 0; k < K; ++k) {
+    if (k + AHEAD < K) prefetch_row(row_of(k_shadow, k + AHEAD));
+    const uint16_t* kr = row_of(k_shadow, k);
+    if (!kr) {
+      score_buf[k] = -INFINITY;
+      continue;
+    }
+    any = true;
+    __m256 a0 = _mm256_setzero_ps(), a1 = _mm256_setzero_ps();
+    for (int i = 0; i < D / 8; i += 2) {
+      a0 = _mm256_fmadd_ps(qv[i], bf16x8_to_f32(kr + 8 * i), a0);
+      a1 = _mm256_fmadd_ps(qv[i + 1], bf16x8_to_f32(kr + 8 * i + 8), a1);
+    }
+    const __m256 a = _mm256_add_ps(a0, a1);
+    __m128 r = _mm_add_ps(_mm256_castps256_ps128(a), _mm256_extractf128_ps(a, 1));
+    r = _mm_add_ps(r, _mm_movehl_ps(r, r));
+    r = _mm_add_ss(r, _mm_shuffle_ps(r, r, 1));
+    const float sc = _mm_cvtss_f32(r) * scale;
+    score_buf[k] = sc;
+    if (sc > mx) mx = sc;
+  }
+  if (!any) {
+    memset(out, 0, D * sizeof(uint16_t));
+    return;
+  }
+  for (int k = 0; k < K && k < AHEAD; ++k) prefetch_row(row_of(v_shadow, k));
+  float den = 0.0f;
+  for (int k = 0; k < K; ++k) {
+    score_buf[k] = std::exp(score_buf[k] - mx);
+    den += score_buf[k];
+  }
+  if (!(den > 0.0f) || !std::isfinite(den)) {
+    memset(out, 0, D * sizeof(uint16_t));
+    return;
+  }
+  const float inv = 1.0f / den;
+  __m256 o[D / 8];
+  for (int i = 0; i < D / 8; ++i) o[i] = _mm256_setzero_ps();
+  for (int k = 0; k < K; ++k) {
+    if (k + AHEAD < K) prefetch_row(row_of(v_shadow, k + AHEAD));
+    const uint16_t* vr = row_of(v_shadow, k);
+    if (!vr) continue;
+    const __m256 w = _mm256_set1_ps(score_buf[k] * inv);
+    for (int i = 0; i < D / 8; ++i) o[i] = _mm256_fmadd_ps(w, bf16x8_to_f32(vr + 8 * i), o[i]);
+  }
+  float of[D];
+  for (int i = 0; i < D / 8; ++i) _mm256_storeu_ps(of + 8 * i, o[i]);
+  for (int i = 0; i < D; ++i) out[i] = f32_to_bf16(of[i]);
+}
+static bool host_has_avx2_fma() {
+  static const bool ok = __builtin_cpu_supports("avx2") && __builtin_cpu_supports("fma");
+  return ok;
+}
+#else
+static bool host_has_avx2_fma() { return false; }
+#endif
+
 struct CpuJob {
   const uint16_t *q, *k_shadow, *v_shadow;
   const int64_t *head_map, *ts_buf;
@@ -250,6 +333,14 @@ struct CpuJob {
 
 static void run_rows(const CpuJob& j, int64_t b, int64_t e) {
   std::vector<float> buf((size_t)j.K);
+#if defined(__x86_64__)
+  if (host_has_avx2_fma()) {
+    for (int64_t r = b; r < e; ++r)
+      topk_attn_row_avx2(j.q + r * D, j.k_shadow, j.v_shadow, j.num_slots, j.head_map + r * j.K, j.ts_buf + r * j.K, j.K,
+                         j.H_kv, j.scale, j.o_new + r * D, buf.data());
+    return;
+  }
+#endif
   for (int64_t r = b; r < e; ++r)
     topk_attn_row(j.q + r * D, j.k_shadow, j.v_shadow, j.num_slots, j.head_map + r * j.K, j.ts_buf + r * j.K, j.K, j.H_kv,
                   j.scale, j.o_new + r * D, buf.data());

@@ -54,7 +54,9 @@ class Workload:
 
 
 def build(name: str, n_layers: int | None = None, seed: int = 0, paged: bool = False, device: str = "cuda",
-          keep_shadow: bool = False) -> Workload:
+          keep_shadow: int = 0) -> Workload:
+    """keep_shadow: number of layers (the first ones) whose bf16 K/V are also kept on the host in the cache's
+    slot order, as the CPU correction's shadow."""
     B, Hq, Hkv, S, scheme, gs, top_k, layers = CONFIGS[name]
     if n_layers is not None:
         layers = n_layers
@@ -89,7 +91,7 @@ def build(name: str, n_layers: int | None = None, seed: int = 0, paged: bool = F
         else:
             ops.fused_quant_write_int4_sym_kv(k, v, slots, kd, ks, vd, vs, gs)
         caches.append(LayerCache(kd, ks, vd, vs))
-        if keep_shadow:
+        if len(shadows) < int(keep_shadow):
             ksh = torch.empty(Hkv, T, HEAD_DIM, dtype=torch.bfloat16)
             vsh = torch.empty(Hkv, T, HEAD_DIM, dtype=torch.bfloat16)
             ksh[:, slots.cpu()] = k.permute(1, 0, 2).cpu()
