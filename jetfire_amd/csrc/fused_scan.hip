@@ -87,12 +87,13 @@ struct K3Prep {
   int exp_w[NSET * 8];
 };
 
-template <int G>
+// Phase-A constants of the INT4 path: the int8-quantised query rows as MFMA A operand.  Row 4*head + kk holds
+// the head's values of 32-channel block kk and zeros elsewhere, so one accumulator register per block.
+template <int NSET>
 struct QInt8F {
-  int qe[G][16];
-  int qo[G][16];
-  float qs[G][4];
-  int sum8[G][4];
+  int8_t aop[NSET][16][4][2][16];  // [set][row = 4*head + block][k-block][MFMA][byte]
+  float qs[NSET * 4][4];           // query scale of (head, block)
+  int sum8[NSET * 4][4];           // 8 * sum of the int8 query over the block (the codes carry an offset of 8)
 };
 
 // LDS carve-up shared by the kernel and its launcher.
@@ -120,10 +121,10 @@ struct ScanLds {
   static constexpr int KST = 64 * KROW;
   static constexpr int WAVE_STAGE = (VST + WL > KST) ? (VST + WL) : KST;
   static constexpr int ACC_REGS = 8 + NG;                   // v4i accumulators per set: 8 channel tiles + NG weight sums
-  static constexpr int SPR = 1;                             // sets exchanged per round
+  static constexpr int XW = NW < 8 ? NW : 8;                // partial accumulator sets that reach the final sum
   static constexpr int XWAVE = ACC_REGS * (48 * 16 + 16 * 4);  // bytes one wavefront writes per set (rows 0..12 only)
-  static constexpr int RED = NW * SPR * XWAVE;
-  static constexpr int PREP = K3 ? (int)sizeof(K3Prep<NSET>) : (int)sizeof(QInt8F<G>);
+  static constexpr int RED = XW * XWAVE;
+  static constexpr int PREP = K3 ? (int)sizeof(K3Prep<NSET>) : (int)sizeof(QInt8F<NSET>);
   static constexpr int HIST = G * SEG * 256 * 4;
   static constexpr int AUX = ((PREP > HIST ? PREP : HIST) + 15) & ~15;
   __host__ __device__ static constexpr int stage_bytes() { return NW * WAVE_STAGE; }
@@ -265,7 +266,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   const uint8_t* ksb = reinterpret_cast<const uint8_t*>(p.k_scales + (size_t)hkv * p.num_slots * (K3 ? NG : 1));
   struct KBuf {
     v4u r[KLD];
-    uint32_t s[K3 ? 4 : 1];
+    uint32_t s[4];
   };
   const int t16 = lane & 15, lg = lane >> 4;
   auto issue_k = [&](int chunk) -> KBuf {
@@ -275,18 +276,13 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
       const uint32_t sb = (uint32_t)sbase[chunk * 4 + kl_page[i]];
       kbuf.r[i] = *reinterpret_cast<const v4u*>(kbase + (size_t)(sb * (uint32_t)KP + kl_off[i]));
     }
-    if constexpr (K3) {
+    constexpr int KNG = K3 ? NG : 1;  // key scales per row
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int sb = __builtin_amdgcn_readfirstlane(sbase[chunk * 4 + j]);  // first slot of the page (uniform)
-        const uint8_t* srow = ksb + (size_t)sb * (NG * 2) + t16 * (NG * 2);
-        if (NG == 2) kbuf.s[j] = *reinterpret_cast<const uint32_t*>(srow);
-        else kbuf.s[j] = *reinterpret_cast<const uint16_t*>(srow);
-      }
-    } else {
-      const int t = chunk * 64 + lane;
-      const uint32_t slot = (uint32_t)(sbase[t >> 4] + (t & 15));
-      kbuf.s[0] = *reinterpret_cast<const uint16_t*>(ksb + (size_t)(slot * 2u));
+    for (int j = 0; j < 4; ++j) {
+      const int sb = __builtin_amdgcn_readfirstlane(sbase[chunk * 4 + j]);  // first slot of the page (uniform)
+      const uint8_t* srow = ksb + (size_t)sb * (KNG * 2) + t16 * (KNG * 2);
+      if (KNG == 2) kbuf.s[j] = *reinterpret_cast<const uint32_t*>(srow);
+      else kbuf.s[j] = *reinterpret_cast<const uint16_t*>(srow);
     }
     return kbuf;
   };
@@ -367,29 +363,34 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
       prep->qsc[h][g] = ldexpf(p.attn_scale, e - 22);
     }
   } else {
-    // int8 quantisation of the G query rows per 32 channels (int8tc_qk_scores.cu:250-290), one element per thread
-    QInt8F<G>* qsh = reinterpret_cast<QInt8F<G>*>(aux);
+    // int8 quantisation of the query rows per 32 channels (int8tc_qk_scores.cu:250-290), one element per thread;
+    // heads past G are zero rows
+    QInt8F<NSET>* qsh = reinterpret_cast<QInt8F<NSET>*>(aux);
 #pragma unroll
     for (int it = 0; it < QPT; ++it) {
       const int i = it * NT + tid;
-      if (i < G * D) {  // uniform per wavefront: G * D is a multiple of 64
-        const int g = i >> 7, d = i & 127, kk = d >> 5;
+      if (i < QN) {  // uniform per wavefront: QN is a multiple of 64
+        const int h = i >> 7, d = i & 127, kk = d >> 5;
         const float x = qv[it];
         float a = fabsf(x);
 #pragma unroll
         for (int off = 16; off >= 1; off >>= 1) a = fmaxf(a, __shfl_xor(a, off));
-        const float s = fmaxf(a / 127.0f, 1e-12f);
-        const float inv = 1.0f / s;
+        const float sq = fmaxf(a / 127.0f, 1e-12f);
+        const float inv = 1.0f / sq;
         const int v = max(-128, min(127, (int)rintf(x * inv)));
         int sv = v;
 #pragma unroll
         for (int off = 16; off >= 1; off >>= 1) sv += __shfl_xor(sv, off);
-        const int j = d >> 3, e = d & 7;
-        int8_t* dst = (e & 1) ? reinterpret_cast<int8_t*>(&qsh->qo[g][j]) : reinterpret_cast<int8_t*>(&qsh->qe[g][j]);
-        dst[e >> 1] = (int8_t)v;
+        // channel d sits in MFMA d>>6, k-block (d>>4)&3; inside the k-block's 16 bytes the nibble spread of two
+        // packed dwords yields: even channels of bytes 0-3, odd channels of bytes 0-3, then the same for bytes 4-7
+        const int set = h >> 2, hh = h & 3, mi = d >> 6, kb = (d >> 4) & 3;
+        const int j2 = (d & 15) >> 1, odd = d & 1;
+        const int by = (j2 >> 2) * 8 + odd * 4 + (j2 & 3);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) qsh->aop[set][4 * hh + r][kb][mi][by] = (r == kk) ? (int8_t)v : (int8_t)0;
         if ((lane & 31) == 0) {
-          qsh->qs[g][kk] = s;
-          qsh->sum8[g][kk] = 8 * sv;
+          qsh->qs[h][kk] = sq;
+          qsh->sum8[h][kk] = 8 * sv;
         }
       }
     }
@@ -399,13 +400,6 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   if (clk && tid == 0) clk[7] = clock64();
 
   // ------------------------------------------------------------------ phase A
-  float mx[G], mn[G];
-#pragma unroll
-  for (int h = 0; h < G; ++h) {
-    mx[h] = -INFINITY;
-    mn[h] = INFINITY;
-  }
-
   if constexpr (K3) {
     // INT3 keys on v_mfma_i32_16x16x64_i8.  The bf16 query row is held exactly as a 23-bit fixed-point number
     // per (head, scale group), split into three balanced int8 limbs that sit in different A-operand rows
@@ -559,49 +553,94 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
       }
     }
   } else {
-    // INT4 keys, int8-Q model: lane = token, row read back from the staged chunk
-    const QInt8F<G>* qsh = reinterpret_cast<const QInt8F<G>*>(aux);
-    auto body = [&](int chunk, uint32_t ksw) {
-      uint32_t pk[16];
+    // INT4 keys, int8-Q model on v_mfma_i32_16x16x64_i8: exact nibble codes (offset 8 removed through the
+    // per-block constant), int32 block sums, the reference's four-term fp32 rescale in its order
+    // (int8tc_qk_scores.cu:455-468).  Lane (token, k-block lg) spreads the 16 channels 64*m + 16*lg .. +15 of
+    // both 64-channel spans m; its accumulator registers are the four 32-channel blocks of head lg.
+    const QInt8F<NSET>* qsh = reinterpret_cast<const QInt8F<NSET>*>(aux);
+    v4i Aop[NSET][2];
+    int sum8[NSET][4];
+    float qs[NSET][4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const v4u r = *reinterpret_cast<const v4u*>(kst + lane * KROW + 16 * i);
-        pk[4 * i] = r[0]; pk[4 * i + 1] = r[1]; pk[4 * i + 2] = r[2]; pk[4 * i + 3] = r[3];
+    for (int set = 0; set < NSET; ++set) {
+#pragma unroll
+      for (int mi = 0; mi < 2; ++mi) Aop[set][mi] = *reinterpret_cast<const v4i*>(&qsh->aop[set][t16][lg][mi][0]);
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+        sum8[set][kk] = qsh->sum8[set * 4 + lg][kk];
+        qs[set][kk] = qsh->qs[set * 4 + lg][kk];
       }
-      const float ks = bf16_to_f32((uint16_t)ksw);
-      const int tok = chunk * 64 + lane;
-      const bool valid = tok < n;
+    }
+    const uint8_t* krd = kst + t16 * KROW + lg * 8;
+    float mxl[NSET], mnl[NSET];
 #pragma unroll
-      for (int g = 0; g < G; ++g) {
-        float sacc = 0.0f;
+    for (int set = 0; set < NSET; ++set) {
+      mxl[set] = -INFINITY;
+      mnl[set] = INFINITY;
+    }
+    auto body = [&](int chunk, const uint32_t (&Sx)[4]) {
+      v2u Xj[4][2];
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
-          int acc = 0;
+      for (int j = 0; j < 4; ++j) {
+        const uint8_t* rp = krd + j * 16 * KROW;
+        Xj[j][0] = *reinterpret_cast<const v2u*>(rp);
+        Xj[j][1] = *reinterpret_cast<const v2u*>(rp + 32);
+      }
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-          for (int j = 4 * kk; j < 4 * kk + 4; ++j) {
-            acc = __builtin_amdgcn_sdot4((int)((pk[j] >> 4) & 0x0f0f0f0fu), qsh->qe[g][j], acc, false);
-            acc = __builtin_amdgcn_sdot4((int)(pk[j] & 0x0f0f0f0fu), qsh->qo[g][j], acc, false);
-          }
-          acc -= qsh->sum8[g][kk];
-          sacc = (kk == 0) ? ((float)acc * qsh->qs[g][0]) : __builtin_fmaf((float)acc, qsh->qs[g][kk], sacc);
+      for (int j = 0; j < 4; ++j) {
+        v4i Bm[2];
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi) {
+          const uint32_t x0 = Xj[j][mi][0], x1 = Xj[j][mi][1];
+          Bm[mi] = (v4i){(int)((x0 >> 4) & 0x0f0f0f0fu), (int)(x0 & 0x0f0f0f0fu), (int)((x1 >> 4) & 0x0f0f0f0fu), (int)(x1 & 0x0f0f0f0fu)};
         }
-        const float a = __fmul_rn(__fmul_rn(sacc, ks), p.attn_scale);
-        sc[g * L + tok] = valid ? a : -INFINITY;
-        mx[g] = fmaxf(mx[g], valid ? a : -INFINITY);
-        mn[g] = fminf(mn[g], valid ? a : INFINITY);
+        const float ks = bf16_to_f32((uint16_t)Sx[j]);
+        const int tok = chunk * 64 + 16 * j + t16;
+        const bool valid = tok < n;
+#pragma unroll
+        for (int set = 0; set < NSET; ++set) {
+          const v4i zero = {0, 0, 0, 0};
+          v4i Dq = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][0], Bm[0], zero, 0, 0, 0);
+          Dq = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][1], Bm[1], Dq, 0, 0, 0);
+          float sacc = (float)(Dq[0] - sum8[set][0]) * qs[set][0];
+#pragma unroll
+          for (int kk = 1; kk < 4; ++kk) sacc = __builtin_fmaf((float)(Dq[kk] - sum8[set][kk]), qs[set][kk], sacc);
+          const float a = __fmul_rn(__fmul_rn(sacc, ks), p.attn_scale);
+          const int h = set * 4 + lg;
+          if ((G % 4 == 0) || h < G) {
+            sc[h * L + tok] = valid ? a : -INFINITY;
+            mxl[set] = fmaxf(mxl[set], valid ? a : -INFINITY);
+            mnl[set] = fminf(mnl[set], valid ? a : INFINITY);
+          }
+        }
       }
     };
 #pragma unroll
     for (int it = 0; it < MAXIT; ++it) {
       const int chunk = wave + it * NW;
       if (chunk < nch_cover) {
+        set_wave_prio(3 - it);
         KBuf& cur = (it & 1) ? Kb : Ka;
         stash_k(cur);
         wave_lds_fence();
-        const uint32_t ksw = cur.s[0];
+        uint32_t Sc[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) Sc[j] = cur.s[j];
         if (it + 2 < MAXIT && chunk + 2 * NW < nch_cover) cur = issue_k(chunk + 2 * NW);
-        body(chunk, ksw);
+        body(chunk, Sc);
         wave_lds_fence();
+      }
+    }
+#pragma unroll
+    for (int set = 0; set < NSET; ++set) {
+      float a = mxl[set], c = -mnl[set];
+      JF_DPP_ROW_REDUCE(a, op_fmax, float, -INFINITY);
+      JF_DPP_ROW_REDUCE(c, op_fmax, float, -INFINITY);
+      const int h = set * 4 + lg;
+      if (t16 == 15 && h < G) {
+        red_f[wave][h] = a;
+        red_f[wave][G + h] = -c;
       }
     }
   }
@@ -655,17 +694,6 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     if (lane == 0) {
       vmax_sh[wave][0] = vm0;
       vmax_sh[wave][1] = vm1;
-    }
-  }
-  if constexpr (!K3) {
-#pragma unroll
-    for (int h = 0; h < G; ++h) {
-      const float v = wave_max(mx[h]);
-      const float u = -wave_max(-mn[h]);
-      if (lane == 0) {
-        red_f[wave][h] = v;
-        red_f[wave][G + h] = u;
-      }
     }
   }
   lds_barrier();  // phase A complete: the query constants are dead, their space becomes the histograms
@@ -927,8 +955,11 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     uint32_t* ck = p.cand_key + (part_base + (size_t)h * p.n_splits) * Kcap;
     int32_t* ci = p.cand_idx + (part_base + (size_t)h * p.n_splits) * Kcap;
     if (!exact_sh[h]) {
-      const uint32_t cut = (uint32_t)cut_sh[h];
-      const float ba = bin_a_sh[h], bb = bin_b_sh[h];
+      // bucket(s) <= cut  <=>  not (s * ba + bb >= cut + 1): the bucket is the floor of that value clamped to
+      // [0, 255]; with cut = 255 every position qualifies
+      const int cut = cut_sh[h];
+      const float thr = uniform_f((cut >= 255) ? INFINITY : (float)(cut + 1));
+      const float ba = uniform_f(bin_a_sh[h]), bb = uniform_f(bin_b_sh[h]);
       const int tb = seg * (L / SEG);
       const int te = min(n, (seg + 1) * (L / SEG));
       // the emitted total is at most Kcap by construction of the cut
@@ -945,18 +976,17 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
           const int t = t0 + 64 * u + lane;
-          const uint32_t bin = (uint32_t)__builtin_amdgcn_fmed3f(__builtin_fmaf(kk[u], ba, bb), 0.f, 255.f);
-          const bool above = (t < te) && (bin <= cut);
+          const bool above = (t < te) && !(__builtin_fmaf(kk[u], ba, bb) >= thr);
           const unsigned long long ma = __builtin_amdgcn_ballot_w64(above);
           const uint32_t pos = (uint32_t)count + __builtin_amdgcn_mbcnt_hi((uint32_t)(ma >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)ma, 0u));
-          if (above) {
+          if (above && pos < (uint32_t)Kcap) {  // the bound only matters for non-finite scores
             *reinterpret_cast<uint32_t*>(ckb + (size_t)(pos * 4u)) = score_key(kk[u]);
             *reinterpret_cast<int32_t*>(cib + (size_t)(pos * 4u)) = s0 + t;
           }
           count += __popcll(ma);
         }
       }
-      if (lane == 0 && seg == SEG - 1) p.cand_cnt[part_base + (size_t)h * p.n_splits] = count;
+      if (lane == 0 && seg == SEG - 1) p.cand_cnt[part_base + (size_t)h * p.n_splits] = min(Kcap, count);
     } else if (seg == 0) {
       // exact fallback: 8-bit radix select over the order-preserving keys (bits shared by every key skipped),
       // then the keys above the K-th and the lowest-position ties that fill the quota
@@ -1042,56 +1072,67 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   // rows that are used (0..12 of 16: lanes 0-47 whole registers, lanes 48-63 the first component), then each
   // output element sums its eight partials.  D layout: row r of a tile sits in lane 16*(r>>2) + column,
   // register r&3; rows are (limb, head), row 12 is the ones row.
-  constexpr int SPR = Lds::SPR;
-  v4i* xa = reinterpret_cast<v4i*>(smem);                                            // [wave][SPR][AR][48]
-  int* xb = reinterpret_cast<int*>(smem + (size_t)NW * SPR * AR * 48 * 16);   // [wave][SPR][AR][16]
+  constexpr int XW = Lds::XW;  // partial sets that reach the final sum
+  v4i* xa = reinterpret_cast<v4i*>(smem);                                  // [XW][AR][48]
+  int* xb = reinterpret_cast<int*>(smem + (size_t)XW * AR * 48 * 16);      // [XW][AR][16]
   float lfin = 0.f;
   if (tid < G) {
 #pragma unroll
     for (int w = 0; w < NW; ++w) lfin += lsum_sh[w][tid];
   }
 #pragma unroll
-  for (int round = 0; round < NSET / SPR; ++round) {
-    if (round > 0) lds_barrier();
-#pragma unroll
-    for (int sl = 0; sl < SPR; ++sl) {
-      const int set = round * SPR + sl;
+  for (int set = 0; set < NSET; ++set) {
+    if (set > 0) lds_barrier();
+    auto put = [&](int slot) {
 #pragma unroll
       for (int r = 0; r < AR; ++r) {
         const v4i v = (r < NTILE) ? acc[set][r < NTILE ? r : 0] : accw[set][r >= NTILE ? r - NTILE : 0];
-        if (lane < 48) xa[((size_t)(wave * SPR + sl) * AR + r) * 48 + lane] = v;
-        else xb[((wave * SPR + sl) * AR + r) * 16 + (lane - 48)] = v[0];
+        if (lane < 48) xa[((size_t)slot * AR + r) * 48 + lane] = v;
+        else xb[(slot * AR + r) * 16 + (lane - 48)] = v[0];
+      }
+    };
+    if (NW > XW) {  // sixteen wavefronts: the upper half hands its sums to the lower half first
+      if (wave >= XW) put(wave - XW);
+      lds_barrier();
+      if (wave < XW) {
+#pragma unroll
+        for (int r = 0; r < AR; ++r) {
+          v4i o = {0, 0, 0, 0};
+          if (lane < 48) o = xa[((size_t)wave * AR + r) * 48 + lane];
+          else o[0] = xb[(wave * AR + r) * 16 + (lane - 48)];
+          if (r < NTILE) acc[set][r < NTILE ? r : 0] += o;
+          else accw[set][r >= NTILE ? r - NTILE : 0] += o;
+        }
       }
     }
+    if (wave < XW) put(wave);
     lds_barrier();
-    for (int i = tid; i < SPR * 4 * D; i += NT) {
-      const int hl = i / D, d = i % D;
-      const int sl = hl >> 2, hh = hl & 3;
-      const int set = round * SPR + sl, h = set * 4 + hh;
+    // thread -> (tile, head, column): the 64 lanes of a wavefront read 64 different banks
+    for (int i = tid; i < 4 * D; i += NT) {
+      const int col = i & 15, hh = (i >> 4) & 3, tile = i >> 6;
+      const int h = set * 4 + hh;
       if (h >= G) continue;
-      int tile, col;
+      int d;
       if (K3) {
-        const int qc = d >> 5, rem = d & 31, kbyte = rem >> 2, e = rem & 3;
-        col = 2 * kbyte + ((e < 2) ? 1 : 0);
-        tile = 2 * qc + (e & 1);
+        const int e = ((col & 1) ? 0 : 2) + (tile & 1);
+        d = (tile >> 1) * 32 + (col >> 1) * 4 + e;
       } else {
-        const int qc = d >> 4, rem = d & 15, kbyte = rem >> 1;
-        col = 2 * kbyte + ((rem & 1) ? 0 : 1);
-        tile = qc;
+        d = tile * 16 + 2 * (col >> 1) + (1 - (col & 1));
       }
       const int g = (NG == 1) ? 0 : (d / (D / NG));
-      int i0 = 0, i1 = 0, i2 = 0, cs = 0, w0 = 0, w1 = 0, w2 = 0;  // |partial| < 2^22 per wavefront: no overflow
+      const int* xi = reinterpret_cast<const int*>(xa);
+      int i0 = 0, i1 = 0, i2 = 0, cs = 0, w0 = 0, w1 = 0, w2 = 0;  // |partial| < 2^23 per set: no overflow
 #pragma unroll
-      for (int w = 0; w < NW; ++w) {
-        const v4i* ta = xa + ((size_t)(w * SPR + sl) * AR + tile) * 48;
-        i0 += ta[col][hh];
-        i1 += ta[16 + col][hh];
-        i2 += ta[32 + col][hh];
-        cs += xb[((w * SPR + sl) * AR + tile) * 16 + col];
-        const v4i* wa = xa + ((size_t)(w * SPR + sl) * AR + NTILE + g) * 48;
-        w0 += wa[0][hh];
-        w1 += wa[16][hh];
-        w2 += wa[32][hh];
+      for (int w = 0; w < XW; ++w) {
+        const int* ta = xi + ((size_t)(w * AR + tile) * 48 + col) * 4 + hh;
+        i0 += ta[0];
+        i1 += ta[16 * 4];
+        i2 += ta[32 * 4];
+        cs += xb[(w * AR + tile) * 16 + col];
+        const int* wa = xi + ((size_t)(w * AR + NTILE + g) * 48) * 4 + hh;
+        w0 += wa[0];
+        w1 += wa[16 * 4];
+        w2 += wa[32 * 4];
       }
       const long long wsum = (long long)w2 * 65536ll + (long long)w1 * 256ll + (long long)w0 + 32896ll * 64ll * (long long)nch;
       const long long tot = (long long)i2 * 65536ll + (long long)i1 * 256ll + (long long)i0 + 32896ll * (long long)cs - (long long)VOFF * wsum;
