@@ -122,7 +122,7 @@ int jf_softmax_v_pre_corr(const float* scores, const float* softmax_m, const flo
  * The reference's own single-call form of this contract is int2_fused_attn_topk
  * (jetfire_vllm/kernels/int2_fused_attn_topk.py:5-10).  scheme: JF_SCHEME_K3V2 (group 64 or 128) or
  * JF_SCHEME_K4V4 (group 128).  top_k: power of two in [32, 1024] (the split entry points above take up
- * to 8192).  If scores is non-NULL the fp32 scores are also written (validation).
+ * to 8192); num_slots at most 2^25 (row offsets are 32-bit).  If scores is non-NULL the fp32 scores are also written (validation).
  * workspace: jf_fused_workspace_bytes() bytes of device memory. */
 size_t jf_fused_workspace_bytes(int scheme, int B, int H_q, int H_kv, int max_S, int top_k);
 int jf_fused_scan_topk(int scheme, int group_size,
@@ -141,11 +141,10 @@ int jf_fused_scan_topk(int scheme, int group_size,
  * launches); end synchronises them and returns the summed device time and the number of launches. */
 int jf_profile_scan_begin(int max_launches);
 int jf_profile_scan_end(double* total_ms, int* launches);
-/* Measurement aid: if device_buffer is non-NULL, every fused-scan workgroup stores ten int64 values
- * (s_memtime at start, after Q.K^T, after the statistics, after P.V, after the partial reduction and at
- * the end, three more inside the candidate selection, and the selection mode) at
- * device_buffer[((b * H_kv + hkv) * n_splits + split) * 10 ...], and every merge workgroup eight stamps
- * at device_buffer[B * H_kv * n_splits * 10 + (b * H_q + hq) * 8 ...].  NULL switches it off. */
+/* Measurement aid: if device_buffer is non-NULL, every fused-scan workgroup stores ten int64 s_memtime
+ * stamps of its phase boundaries at device_buffer[((b * H_kv + hkv) * n_splits + split) * 10 ...], and every
+ * merge workgroup eight at device_buffer[B * H_kv * n_splits * 10 + (b * H_q + hq) * 8 ...] (which stamp
+ * marks which boundary is internal to the kernels and may change).  NULL switches it off. */
 int jf_debug_phase_clock(void* device_buffer);
 
 /* ------------------------------------------------------------------ piece 4: merge

@@ -1,24 +1,28 @@
 // Fused decode scan + top-k for gfx950: one pass over the packed K and V of every (sequence, kv-head),
 // no (B, H_q, S) score tensor in HBM.
 //
-// Launch 1, fused_scan_kernel, grid (n_splits, H_kv, B), 512 threads (8 wavefronts).  A workgroup owns L
-// consecutive positions of one (sequence, kv-head) and all G query heads of that kv-head.  The page
-// table of the split is read once into LDS; every wavefront then streams 64-token chunks with the loads
-// of its next chunk in flight while it works on the current one (no workgroup barrier inside a phase):
-//   phase A  Q.K^T            scores[G][L] -> LDS (fp32), running max per head, V scales -> LDS
-//            INT3 keys: K-hat = bf16((code-4)*scale) built in registers, v_mfma_f32_16x16x32_bf16 with the
-//                       tokens on the N side; the four 16-token tiles of a chunk land one per 16-lane
-//                       group, so lane l ends up holding the G scores of token l.
-//            INT4 keys: int8-quantised Q, exact nibble codes, v_dot4_i32_i8, fp32 rescale (every step
-//                       is exactly reproducible, so it is bit-equal to the split-form kernel).
-//   phase B  P.V on v_mfma_i32_16x16x64_i8.  p = exp(s - m_split) is known exactly because phase A is
-//            complete, so w = p * v_scale is converted to 22-bit fixed point once (fma with 2^23), its
-//            three bytes are the A-operand rows (limb, head), and the int32 accumulators live for the whole
-//            split: every product is exact.  V codes are staged packed in wavefront-private LDS and
-//            transposed by ds_read_b64_tr_b4 (16 tokens of one channel per lane), then nibble-spread.
-//            sum_t w_t*(code - off) = sum_t w_t*code - off * sum_t w_t; a constant-ones row gives sum_t code.
-//   phase C  per-head radix select with the keys held in registers (bits shared by all keys of the split
-//            are skipped): the split's top-min(K, n) candidates (key, position), ascending position.
+// Launch 1, fused_scan_kernel, grid (n_splits, H_kv, B), 16 wavefronts per workgroup (8 where the register
+// budget does not allow 1024 threads).  A workgroup owns L consecutive positions of one (sequence, kv-head)
+// and all G query heads of that kv-head.  The page table of the split is read once into LDS.  Key and value
+// rows are fetched in 64-position chunks with 16-byte loads whose lane addresses are consecutive inside a
+// page, two chunks per wavefront in flight, staged in wavefront-private LDS and read back in the layout the
+// arithmetic wants; barriers order LDS traffic only, so prefetched rows stay in flight across them.
+//   phase A  Q.K^T on v_mfma_i32_16x16x64_i8, tokens on the N side, rows = (head, limb or block):
+//            INT3 keys: the bf16 query as exact 23-bit fixed point in three int8 limbs, codes spread from the
+//                       byte planes with shift/mask on dwords, a second contraction with the indicator of
+//                       codes +-3 reproduces the reference's bf16 rounding of the dequantised key.
+//            INT4 keys: int8-quantised Q, exact nibble codes, one accumulator row per 32-channel block, the
+//                       reference's fp32 rescale order (bit-equal to the split-form kernel).
+//            scores[G][L] -> LDS (fp32), running max / min per head.
+//   phase B  P.V on the same MFMA.  p = exp(s - m_split) is known exactly because phase A is complete, so
+//            w = p * v_scale is converted to 22-bit fixed point once (fma with 2^23), its three bytes are the
+//            A-operand rows (limb, head), and the int32 accumulators live for the whole split: every product
+//            is exact.  V codes are transposed by ds_read_b64_tr_b4, weight rows by ds_read_b64_tr_b8.
+//            The same pass drops every score into one of 256 linear buckets per (head, segment).
+//   phase C  from the bucket histograms: the smallest bucket range that holds the split's top min(K, n) scores
+//            and fits the candidate buffer; its positions are emitted as (key, position) in ascending
+//            position, one wavefront per (head, segment).  Heavily tied scores fall back to a radix select.
+//   exchange of the wavefronts' integer accumulators through LDS, exact int64 recombination -> partial o.
 // Launch 2, fused_merge_kernel, grid (B, H_q): selects the global top-k among the candidates (ties to
 // the lower position, ascending output), merges the split partials
 //   M = max m_i, l = sum l_i e^{m_i-M}, o_hat = sum o_i e^{m_i-M} / l
@@ -41,7 +45,7 @@ typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
 
 constexpr int FS_MAX_TOPK = 1024;      // winners cached in LDS by the merge kernel
-constexpr int FS_CAND_SLACK = 256;     // extra candidate slots per (row, split)
+constexpr int FS_CAND_SLACK = 256;     // extra candidate slots per (row, split): room for the whole cut bucket
 
 struct FusedParams {
   const uint16_t* q;
@@ -72,7 +76,7 @@ struct FusedParams {
   float* W;
   float* softmax_m;
   float* softmax_inv_z;
-  long long* phase_clock;  // optional: 6 s_memtime stamps per scan workgroup (measurement aid)
+  long long* phase_clock;  // optional: 10 s_memtime stamps per scan workgroup, 8 per merge workgroup (measurement aid)
 };
 
 // Phase-A constants of the INT3 path, built once per workgroup in LDS.
@@ -1653,16 +1657,26 @@ inline void fused_plan(int scheme, int NG, int B, int H_q, int H_kv, int max_S, 
                        int* kc_out) {
   const int G = H_q / H_kv;
   const int units = B * H_kv > 0 ? B * H_kv : 1;
-  // two resident workgroups per CU on 256 CUs where a workgroup has eight wavefronts and a small score block,
-  // one otherwise
-  const int wg_target = 256;
-  int target = wg_target / units;
-  if (target < 1) target = 1;
-  int L = (max_S + target - 1) / target;
-  L = (L + 255) / 256 * 256;
+  // One workgroup is resident per CU (256 CUs).  Among the split lengths that fit LDS pick the one that
+  // minimises (rounds of workgroups) x (split length + a fixed per-workgroup cost, in positions) plus a term
+  // for the merge kernel, whose work grows with the number of candidate lists; a launch whose workgroup
+  // count is just over a multiple of 256 pays a whole extra round.
   const int lmax = lmax_dispatch(scheme, G, NG);
-  if (L > lmax) L = lmax;
-  if (L < 256) L = 256;
+  constexpr int kCUs = 256, kFixed = 640;
+  int L = 256;
+  long best = -1;
+  for (int cand = 256; cand <= lmax; cand += 256) {
+    const long nsp = (max_S + cand - 1) / cand > 0 ? (max_S + cand - 1) / cand : 1;
+    if (nsp > MG_MAX_SPLITS && cand < lmax) continue;
+    const long rounds = (nsp * units + kCUs - 1) / kCUs;
+    const long kc = (top_k + FS_CAND_SLACK) < cand ? (top_k + FS_CAND_SLACK) : cand;
+    const long cost = rounds * (cand + kFixed) + nsp * kc / 5;  // + the merge kernel's pass over the candidates
+    if (best < 0 || cost <= best) {
+      best = cost;
+      L = cand;
+    }
+    if (cand >= max_S) break;
+  }
   int ns = (max_S + L - 1) / L;
   if (ns < 1) ns = 1;
   *L_out = L;
