@@ -128,10 +128,13 @@ struct ScanLds {
   static constexpr int XW = NW < 8 ? NW : 8;                // partial accumulator sets that reach the final sum
   static constexpr int XWAVE = ACC_REGS * (48 * 16 + 16 * 4);  // bytes one wavefront writes per set (rows 0..12 only)
   static constexpr int RED = XW * XWAVE;
+  // with one head set and enough staging space the exchange runs in the staging area while the score rows
+  // are still being read by the candidate emission
   static constexpr int PREP = K3 ? (int)sizeof(K3Prep<NSET>) : (int)sizeof(QInt8F<NSET>);
   static constexpr int HIST = G * SEG * 256 * 4;
   static constexpr int AUX = ((PREP > HIST ? PREP : HIST) + 15) & ~15;
   __host__ __device__ static constexpr int stage_bytes() { return NW * WAVE_STAGE; }
+  static constexpr bool XS = (NSET == 1) && (NW * WAVE_STAGE >= RED);
   __host__ __device__ static constexpr size_t per_position() { return (size_t)G * 4; }
   __host__ __device__ static size_t aux_offset(int L) { return (per_position() * L + (size_t)(L / 16) * 4 + 15) & ~(size_t)15; }
   __host__ __device__ static size_t total(int L) {
@@ -891,6 +894,68 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   lds_barrier();
   if (clk && tid == 0) clk[2] = clock64();
 
+  // ---- exchange of the integer accumulators: every wavefront stores the rows that are used (0..12 of 16:
+  // lanes 0-47 whole registers, lanes 48-63 the first component); with sixteen wavefronts the upper half hands
+  // its sums to the lower half first; then each output element sums the remaining partials.  D layout: row r
+  // of a tile sits in lane 16*(r>>2) + column, register r&3; rows are (limb, head), row 12 is the ones row.
+  constexpr int XW = Lds::XW;  // partial sets that reach the final sum
+  constexpr bool XS = Lds::XS;
+  uint8_t* xbase = XS ? stage : smem;
+  v4i* xa = reinterpret_cast<v4i*>(xbase);                              // [XW][AR][48]
+  int* xb = reinterpret_cast<int*>(xbase + (size_t)XW * AR * 48 * 16);  // [XW][AR][16]
+  auto put = [&](int set, int slot) {
+#pragma unroll
+    for (int r = 0; r < AR; ++r) {
+      const v4i v = (r < NTILE) ? acc[set][r < NTILE ? r : 0] : accw[set][r >= NTILE ? r - NTILE : 0];
+      if (lane < 48) xa[((size_t)slot * AR + r) * 48 + lane] = v;
+      else xb[(slot * AR + r) * 16 + (lane - 48)] = v[0];
+    }
+  };
+  auto take = [&](int set, int slot) {
+#pragma unroll
+    for (int r = 0; r < AR; ++r) {
+      v4i o = {0, 0, 0, 0};
+      if (lane < 48) o = xa[((size_t)slot * AR + r) * 48 + lane];
+      else o[0] = xb[(slot * AR + r) * 16 + (lane - 48)];
+      if (r < NTILE) acc[set][r < NTILE ? r : 0] += o;
+      else accw[set][r >= NTILE ? r - NTILE : 0] += o;
+    }
+  };
+  auto combine = [&](int set) {
+    // thread -> (tile, head, column): the 64 lanes of a wavefront read 64 different banks
+    for (int i = tid; i < 4 * D; i += NT) {
+      const int col = i & 15, hh = (i >> 4) & 3, tile = i >> 6;
+      const int h = set * 4 + hh;
+      if (h >= G) continue;
+      int d;
+      if (K3) {
+        const int e = ((col & 1) ? 0 : 2) + (tile & 1);
+        d = (tile >> 1) * 32 + (col >> 1) * 4 + e;
+      } else {
+        d = tile * 16 + 2 * (col >> 1) + (1 - (col & 1));
+      }
+      const int g = (NG == 1) ? 0 : (d / (D / NG));
+      const int* xi = reinterpret_cast<const int*>(xa);
+      int i0 = 0, i1 = 0, i2 = 0, cs = 0, w0 = 0, w1 = 0, w2 = 0;  // |partial| < 2^23 per set: no overflow
+#pragma unroll
+      for (int w = 0; w < XW; ++w) {
+        const int* ta = xi + ((size_t)(w * AR + tile) * 48 + col) * 4 + hh;
+        i0 += ta[0];
+        i1 += ta[16 * 4];
+        i2 += ta[32 * 4];
+        cs += xb[(w * AR + tile) * 16 + col];
+        const int* wa = xi + ((size_t)(w * AR + NTILE + g) * 48) * 4 + hh;
+        w0 += wa[0];
+        w1 += wa[16 * 4];
+        w2 += wa[32 * 4];
+      }
+      const long long wsum = (long long)w2 * 65536ll + (long long)w1 * 256ll + (long long)w0 + 32896ll * 64ll * (long long)nch;
+      const long long tot = (long long)i2 * 65536ll + (long long)i1 * 256ll + (long long)i0 + 32896ll * (long long)cs - (long long)VOFF * wsum;
+      p.part_o[(part_base + (size_t)h * p.n_splits) * D + d] = (float)ldexp((double)tot, -E[g]);
+    }
+  };
+  if (XS && NW > XW && wave >= XW) put(0, wave - XW);  // overlaps the cut search below
+
   // ------------------------------------------------------------------ phase C: candidates of the split
   // The merge kernel needs a superset of the split's top Kt = min(top_k, n) scores per head that fits the
   // candidate buffer (Kcap entries), in ascending position.  From the histograms: the smallest bucket index
@@ -953,6 +1018,10 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   }
   lds_barrier();
   if (clk && tid == 0) clk[6] = clock64();
+  if (XS && wave < XW) {
+    if (NW > XW) take(0, wave);
+    put(0, wave);
+  }
   for (int hs = wave; hs < G * SEG; hs += NW) {
     const int h = hs / SEG, seg = hs % SEG;
     const float* srow = sc + h * L;
@@ -994,7 +1063,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     } else if (seg == 0) {
       // exact fallback: 8-bit radix select over the order-preserving keys (bits shared by every key skipped),
       // then the keys above the K-th and the lowest-position ties that fill the quota
-      int* rh = reinterpret_cast<int*>(stage + wave * Lds::WAVE_STAGE);
+      int* rh = XS ? reinterpret_cast<int*>(aux) + h * 256 : reinterpret_cast<int*>(stage + wave * Lds::WAVE_STAGE);
       uint32_t T = 0;
       int quota = 0;
       uint32_t kmin = 0xffffffffu, kmax = 0u;
@@ -1072,75 +1141,26 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   lds_barrier();
   if (clk && tid == 0) clk[3] = clock64();
 
-  // ---- exchange of the integer accumulators (the score rows are dead by now): every wavefront stores the
-  // rows that are used (0..12 of 16: lanes 0-47 whole registers, lanes 48-63 the first component), then each
-  // output element sums its eight partials.  D layout: row r of a tile sits in lane 16*(r>>2) + column,
-  // register r&3; rows are (limb, head), row 12 is the ones row.
-  constexpr int XW = Lds::XW;  // partial sets that reach the final sum
-  v4i* xa = reinterpret_cast<v4i*>(smem);                                  // [XW][AR][48]
-  int* xb = reinterpret_cast<int*>(smem + (size_t)XW * AR * 48 * 16);      // [XW][AR][16]
   float lfin = 0.f;
   if (tid < G) {
 #pragma unroll
     for (int w = 0; w < NW; ++w) lfin += lsum_sh[w][tid];
   }
+  if (XS) {
+    combine(0);
+  } else {
+    // the score rows are dead by now: the exchange reuses their space, one head set at a time
 #pragma unroll
-  for (int set = 0; set < NSET; ++set) {
-    if (set > 0) lds_barrier();
-    auto put = [&](int slot) {
-#pragma unroll
-      for (int r = 0; r < AR; ++r) {
-        const v4i v = (r < NTILE) ? acc[set][r < NTILE ? r : 0] : accw[set][r >= NTILE ? r - NTILE : 0];
-        if (lane < 48) xa[((size_t)slot * AR + r) * 48 + lane] = v;
-        else xb[(slot * AR + r) * 16 + (lane - 48)] = v[0];
+    for (int set = 0; set < NSET; ++set) {
+      if (set > 0) lds_barrier();
+      if (NW > XW) {
+        if (wave >= XW) put(set, wave - XW);
+        lds_barrier();
+        if (wave < XW) take(set, wave);
       }
-    };
-    if (NW > XW) {  // sixteen wavefronts: the upper half hands its sums to the lower half first
-      if (wave >= XW) put(wave - XW);
+      if (wave < XW) put(set, wave);
       lds_barrier();
-      if (wave < XW) {
-#pragma unroll
-        for (int r = 0; r < AR; ++r) {
-          v4i o = {0, 0, 0, 0};
-          if (lane < 48) o = xa[((size_t)wave * AR + r) * 48 + lane];
-          else o[0] = xb[(wave * AR + r) * 16 + (lane - 48)];
-          if (r < NTILE) acc[set][r < NTILE ? r : 0] += o;
-          else accw[set][r >= NTILE ? r - NTILE : 0] += o;
-        }
-      }
-    }
-    if (wave < XW) put(wave);
-    lds_barrier();
-    // thread -> (tile, head, column): the 64 lanes of a wavefront read 64 different banks
-    for (int i = tid; i < 4 * D; i += NT) {
-      const int col = i & 15, hh = (i >> 4) & 3, tile = i >> 6;
-      const int h = set * 4 + hh;
-      if (h >= G) continue;
-      int d;
-      if (K3) {
-        const int e = ((col & 1) ? 0 : 2) + (tile & 1);
-        d = (tile >> 1) * 32 + (col >> 1) * 4 + e;
-      } else {
-        d = tile * 16 + 2 * (col >> 1) + (1 - (col & 1));
-      }
-      const int g = (NG == 1) ? 0 : (d / (D / NG));
-      const int* xi = reinterpret_cast<const int*>(xa);
-      int i0 = 0, i1 = 0, i2 = 0, cs = 0, w0 = 0, w1 = 0, w2 = 0;  // |partial| < 2^23 per set: no overflow
-#pragma unroll
-      for (int w = 0; w < XW; ++w) {
-        const int* ta = xi + ((size_t)(w * AR + tile) * 48 + col) * 4 + hh;
-        i0 += ta[0];
-        i1 += ta[16 * 4];
-        i2 += ta[32 * 4];
-        cs += xb[(w * AR + tile) * 16 + col];
-        const int* wa = xi + ((size_t)(w * AR + NTILE + g) * 48) * 4 + hh;
-        w0 += wa[0];
-        w1 += wa[16 * 4];
-        w2 += wa[32 * 4];
-      }
-      const long long wsum = (long long)w2 * 65536ll + (long long)w1 * 256ll + (long long)w0 + 32896ll * 64ll * (long long)nch;
-      const long long tot = (long long)i2 * 65536ll + (long long)i1 * 256ll + (long long)i0 + 32896ll * (long long)cs - (long long)VOFF * wsum;
-      p.part_o[(part_base + (size_t)h * p.n_splits) * D + d] = (float)ldexp((double)tot, -E[g]);
+      combine(set);
     }
   }
   if (tid < G) {
