@@ -1,0 +1,72 @@
+"""Parity of the fused decode step at the benchmark's full shapes (one layer), through properties that do
+not need the slow CPU oracle: the reference's own validation formulas evaluated with torch on the GPU
+(dequantised cache via the torch restatement of `unpack`, dense fp32 attention), exact top-k on the
+kernel's own scores, softmax statistics, and run-to-run determinism."""
+import pytest
+import torch
+
+from oracle import torch_cpu_path as T
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(w, lay, **kw):
+    from jetfire_amd import ops
+    return ops.fused_attn_topk(w.scheme, w.q, lay.k_data, lay.k_scales, lay.v_data, lay.v_scales, w.block_table,
+                               w.seq_lens, w.S, w.H_q, w.H_kv, 16, w.top_k, w.attn_scale, **kw)
+
+
+@pytest.mark.parametrize("name", ["c2", "c3", "c4"])
+def test_full_size_layer_properties(name):
+    from jetfire_amd import workloads
+    w = workloads.build(name, n_layers=1, paged=True)
+    lay = w.layers[0]
+    B, Hq, Hkv, S, K = w.B, w.H_q, w.H_kv, w.S, w.top_k
+    G = Hq // Hkv
+    kb, vb = (3, 2) if w.scheme == "k3v2" else (4, 4)
+    o_hat, slots, o_old, W, idx, m, iz, scores = _run(w, lay, return_scores=True, return_stats=True)
+    again = _run(w, lay, return_scores=True, return_stats=True)
+    for a, b in zip((o_hat, slots, o_old, W, idx, m, iz, scores), again):
+        assert torch.equal(a, b)                                   # deterministic
+
+    # --- top-k: exact on the kernel's own scores, ascending positions, slots through the block table
+    tv, _ = scores.topk(K, dim=-1)
+    got = scores.gather(-1, idx)
+    assert torch.equal(got.sort(dim=-1, descending=True).values, tv)
+    assert (idx[..., 1:] > idx[..., :-1]).all()
+    pos_slots = torch.gather(w.block_table, 1, (idx // 16).reshape(B, -1)).reshape(B, Hq, K) * 16 + idx % 16
+    assert torch.equal(slots, pos_slots)
+
+    # --- softmax statistics of those scores
+    assert torch.equal(m, scores.max(dim=-1).values)
+    z = (scores - m[..., None]).exp().sum(-1)
+    torch.testing.assert_close(iz, 1.0 / z, rtol=2e-5, atol=0)
+
+    # --- dense reference from the dequantised cache (per sequence, one kv-head at a time to bound memory)
+    pos = torch.arange(S, device="cuda")
+    max_sc = 0.0
+    for b in range(B):
+        sl = w.block_table[b, pos // 16] * 16 + pos % 16
+        for h in range(Hkv):
+            khat = T.unpack(lay.k_data[h, sl], lay.k_scales[h, sl], w.group, kb).float()      # (S, 128)
+            vhat = (T.unpack(lay.v_data[h, sl], lay.v_scales[h, sl], w.group, vb)).float()
+            # Stage B multiplies by the unrounded fp32 scale: redo the dequant without the bf16 rounding
+            vq = T.unpack(lay.v_data[h, sl], torch.ones_like(lay.v_scales[h, sl]), w.group, vb).float()
+            vexact = (vq.reshape(S, -1, w.group) * lay.v_scales[h, sl].float()[..., None]).reshape(S, 128)
+            qh = w.q[b, h * G:(h + 1) * G].float()
+            ref = (qh @ khat.T) * w.attn_scale                                                  # (G, S)
+            mine = scores[b, h * G:(h + 1) * G]
+            if w.scheme == "k3v2":      # same scoring model: bf16-rounded dequantised keys
+                torch.testing.assert_close(mine, ref, atol=3e-5, rtol=3e-5)
+            else:                       # int8-quantised query model: close to the dense model, not equal
+                assert (mine - ref).abs().max() < 0.05 * ref.abs().max()
+            max_sc = max(max_sc, float(mine.abs().max()))
+            p = torch.softmax(mine, dim=-1)
+            torch.testing.assert_close(o_hat[b, h * G:(h + 1) * G], p @ vexact, atol=4e-6, rtol=1e-4)
+            sel = idx[b, h * G:(h + 1) * G]
+            pw = p.gather(-1, sel)
+            torch.testing.assert_close(W[b, h * G:(h + 1) * G], pw.sum(-1), atol=4e-6, rtol=1e-4)
+            old = torch.einsum("gk,gkd->gd", pw, vexact[sel])
+            torch.testing.assert_close(o_old[b, h * G:(h + 1) * G], old, atol=4e-6, rtol=1e-4)
+            del khat, vhat, vq, vexact
+    assert max_sc > 0
