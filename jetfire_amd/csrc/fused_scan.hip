@@ -406,6 +406,43 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   if (wave + NW < nch_cover) Kb = issue_k(wave + NW);
   if (clk && tid == 0) clk[7] = clock64();
 
+  // ---- V stream, set-up (same scheme as the key stream)
+  uint8_t* vst = stage + wave * Lds::WAVE_STAGE;  // [64][VROW], this wavefront only
+  uint8_t* wl = vst + Lds::VST;                   // [NG][NSET][64 tokens][16]
+  constexpr int VLD = VP / 16;
+  uint32_t vl_page[VLD], vl_off[VLD], vl_lds[VLD];
+#pragma unroll
+  for (int i = 0; i < VLD; ++i) {
+    const int o = 1024 * i + 16 * lane;
+    vl_page[i] = (uint32_t)(o / (16 * VP));
+    vl_off[i] = (uint32_t)(o % (16 * VP));
+    vl_lds[i] = (uint32_t)((o / VP) * VROW + (o % VP));
+  }
+  struct VBuf {
+    v4u r[VLD];
+    uint32_t w;
+  };
+  auto issue_v = [&](int chunk) -> VBuf {
+    VBuf vbuf;
+#pragma unroll
+    for (int i = 0; i < VLD; ++i) {
+      const uint32_t sb = (uint32_t)sbase[chunk * 4 + vl_page[i]];
+      vbuf.r[i] = *reinterpret_cast<const v4u*>(vbase + (size_t)(sb * (uint32_t)VP + vl_off[i]));
+    }
+    const int t = chunk * 64 + lane;
+    const uint32_t slot = (uint32_t)(sbase[t >> 4] + (t & 15));
+    if (NG == 2) vbuf.w = *reinterpret_cast<const uint32_t*>(vsbase + (size_t)(slot * 4u));
+    else vbuf.w = (uint32_t) * reinterpret_cast<const uint16_t*>(vsbase + (size_t)(slot * 2u));
+    return vbuf;
+  };
+  // the first two V chunks are requested while the last key chunks are being worked on
+  VBuf Va = {}, Vb = {};
+  auto prefetch_v = [&](int it) {
+    if (it == MAXIT - 2 && wave < nch) Va = issue_v(wave);
+    if (it == MAXIT - 1 && wave + NW < nch) Vb = issue_v(wave + NW);
+  };
+
+
   // ------------------------------------------------------------------ phase A
   if constexpr (K3) {
     // INT3 keys on v_mfma_i32_16x16x64_i8.  The bf16 query row is held exactly as a 23-bit fixed-point number
@@ -533,6 +570,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
 #pragma unroll
     for (int it = 0; it < MAXIT; ++it) {
       const int chunk = wave + it * NW;
+      prefetch_v(it);
       if (chunk < nch_cover) {
         set_wave_prio(3 - it);  // wavefronts that are behind get the issue slots first
         KBuf& cur = (it & 1) ? Kb : Ka;
@@ -626,6 +664,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
 #pragma unroll
     for (int it = 0; it < MAXIT; ++it) {
       const int chunk = wave + it * NW;
+      prefetch_v(it);
       if (chunk < nch_cover) {
         set_wave_prio(3 - it);
         KBuf& cur = (it & 1) ? Kb : Ka;
@@ -651,39 +690,6 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
       }
     }
   }
-
-  // ---- V stream, set-up (same scheme as the key stream); its first two chunks start before the barrier
-  uint8_t* vst = stage + wave * Lds::WAVE_STAGE;  // [64][VROW], this wavefront only
-  uint8_t* wl = vst + Lds::VST;                   // [NG][NSET][64 tokens][16]
-  constexpr int VLD = VP / 16;
-  uint32_t vl_page[VLD], vl_off[VLD], vl_lds[VLD];
-#pragma unroll
-  for (int i = 0; i < VLD; ++i) {
-    const int o = 1024 * i + 16 * lane;
-    vl_page[i] = (uint32_t)(o / (16 * VP));
-    vl_off[i] = (uint32_t)(o % (16 * VP));
-    vl_lds[i] = (uint32_t)((o / VP) * VROW + (o % VP));
-  }
-  struct VBuf {
-    v4u r[VLD];
-    uint32_t w;
-  };
-  auto issue_v = [&](int chunk) -> VBuf {
-    VBuf vbuf;
-#pragma unroll
-    for (int i = 0; i < VLD; ++i) {
-      const uint32_t sb = (uint32_t)sbase[chunk * 4 + vl_page[i]];
-      vbuf.r[i] = *reinterpret_cast<const v4u*>(vbase + (size_t)(sb * (uint32_t)VP + vl_off[i]));
-    }
-    const int t = chunk * 64 + lane;
-    const uint32_t slot = (uint32_t)(sbase[t >> 4] + (t & 15));
-    if (NG == 2) vbuf.w = *reinterpret_cast<const uint32_t*>(vsbase + (size_t)(slot * 4u));
-    else vbuf.w = (uint32_t) * reinterpret_cast<const uint16_t*>(vsbase + (size_t)(slot * 2u));
-    return vbuf;
-  };
-  VBuf Va = {}, Vb = {};
-  if (wave < nch) Va = issue_v(wave);
-  if (wave + NW < nch) Vb = issue_v(wave + NW);
 
   if (clk && tid == 0) clk[9] = clock64();  // wavefront 0 finished its chunks
   if (clk && lane == 0) atomicMax(&tmax_sh, (unsigned long long)clock64());
