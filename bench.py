@@ -79,6 +79,8 @@ def main() -> int:
                          "whose definition is end to end)")
     ap.add_argument("--no-handoff", dest="handoff", action="store_false")
     ap.add_argument("--cpu-threads", type=int, default=16, help="CPU correction threads (hand-off mode)")
+    ap.add_argument("--split-len", type=int, default=0,
+                    help="measurement aid: force the fused scan's split length (0 = the library's planner)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run a plain 1 GiB device copy 10 times and exit (reference for the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -102,6 +104,8 @@ def main() -> int:
         torch.cuda.synchronize()
         print(json.dumps({"calibrate_copy_bytes_read": 1 << 30, "calibrate_copy_bytes_written": 1 << 30, "launches": 10}))
         return 0
+    if args.split_len:
+        _lib.check(lib.jf_debug_split_len(args.split_len))
     handoff = args.handoff if args.handoff is not None else args.workload in ("c4", "c5")
     if args.graph is None:
         args.graph = not handoff
@@ -192,6 +196,7 @@ def main() -> int:
         "config": {"workload": f"{args.workload}: B{w.B} Hq{w.H_q} Hkv{w.H_kv} D128 S{w.S} {w.scheme} g{w.group} "
                                f"top_k{w.top_k} x{n_layers} layers, {'paged (random)' if args.paged else 'identity'} block table",
                    "packed_bytes_per_layer": bytes_layer, "launch": "hip-graph" if graph is not None else "eager",
+                   **({"split_len_forced": args.split_len} if args.split_len else {}),
                    "handoff": (f"pinned D2H of slots + CPU correction on {ops.get_cpu_attn_threads()} threads + H2D, every layer"
                                if handoff else "not in the timed region (GPU path only)")},
         "roofline": {"bound": "hbm", "kernel": "fused_scan_kernel", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS,

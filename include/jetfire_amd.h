@@ -146,6 +146,10 @@ int jf_profile_scan_end(double* total_ms, int* launches);
  * merge workgroup eight at device_buffer[B * H_kv * n_splits * 10 + (b * H_q + hq) * 8 ...] (which stamp
  * marks which boundary is internal to the kernels and may change).  NULL switches it off. */
 int jf_debug_phase_clock(void* device_buffer);
+/* Test / measurement aid with no counterpart in the reference: a positive split_len (rounded up to a
+ * multiple of 256 and clamped to what fits the kernel's LDS) replaces the planner's choice of the split
+ * length in jf_fused_scan_topk and jf_fused_workspace_bytes; 0 restores the planner.  Process-wide. */
+int jf_debug_split_len(int split_len);
 
 /* ------------------------------------------------------------------ piece 4: merge
  * out = bf16_rne(fma(W, f32(o_new), o_hat) - o_old_unnorm).  Replaces blend_unnorm_into

@@ -68,6 +68,13 @@ struct FusedParams {
   uint32_t* cand_key;  // (B, H_q, NS, Kc)
   int32_t* cand_idx;   // (B, H_q, NS, Kc)
   int32_t* cand_cnt;   // (B, H_q, NS)
+  // two-stage merge (long contexts): `mg_parts` workgroups per row first reduce `mg_spp` consecutive
+  // candidate lists each to the row's top_k among them; the final merge then reads those lists
+  int mg_parts, mg_spp;
+  uint32_t k_magic;    // ceil(2^32 / top_k)
+  uint32_t* key2;      // (B, H_q, mg_parts, top_k)
+  int32_t* idx2;       // (B, H_q, mg_parts, top_k)
+  int32_t* cnt2;       // (B, H_q, mg_parts)
   // merge outputs
   int64_t* topk_idx;
   int64_t* topk_slots;
@@ -224,6 +231,20 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   long long* clk = p.phase_clock ? p.phase_clock + (((size_t)b * p.H_kv + hkv) * p.n_splits + split) * 10 : nullptr;
   if (clk && tid == 0) clk[0] = clock64();
 
+  // The page-table entry and the query elements of this thread do not depend on the sequence length: they
+  // are requested first, so their latency runs in parallel with the load of seq_lens[b] instead of after it.
+  const int nch_cover = (n_cover + 63) >> 6;
+  int64_t bt_mine = 0;  // LMAX / 16 <= NT: one entry per thread covers the split
+  if (tid < nch_cover * 4) bt_mine = bt[min((s0 >> 4) + tid, p.max_blocks - 1)];
+  constexpr int QN = NSET * 4 * D;               // elements of the padded query block (whole head sets)
+  constexpr int QPT = (QN + NT - 1) / NT;
+  float qv[QPT];
+#pragma unroll
+  for (int it = 0; it < QPT; ++it) {
+    const int i = it * NT + tid;
+    qv[it] = (i < G * D) ? bf16_to_f32(p.q[head0 * D + i]) : 0.f;
+  }
+
   if (n == 0) {  // nothing valid in this split: padding scores, empty partials
     if (p.scores)
       for (int i = tid; i < G * n_cover; i += NT)
@@ -237,24 +258,12 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     return;
   }
 
-  // Page table of the split: one entry per 16 positions of every 64-token chunk that is touched.  Pages past
-  // the last valid position repeat the last valid page, so every row address formed below is in bounds
-  // (those rows' scores are masked to -inf, their softmax weights are exactly zero).
-  const int nch_cover = (n_cover + 63) >> 6;
+  // Page table of the split: one entry per 16 positions of every 64-token chunk that is touched.  Table
+  // entries past the last valid position may hold anything: those pages read slot 0 instead, so every row
+  // address formed below is in bounds (those rows' scores are masked to -inf, their softmax weights are
+  // exactly zero).
   const int nch = (n + 63) >> 6;
-  {
-    const int last_page = (n - 1) >> 4;
-    for (int i = tid; i < nch_cover * 4; i += NT) sbase[i] = (int)(bt[(s0 >> 4) + min(i, last_page)] * BS);
-  }
-  // query elements of this thread (in flight while the page table arrives)
-  constexpr int QN = NSET * 4 * D;               // elements of the padded query block (whole head sets)
-  constexpr int QPT = (QN + NT - 1) / NT;
-  float qv[QPT];
-#pragma unroll
-  for (int it = 0; it < QPT; ++it) {
-    const int i = it * NT + tid;
-    qv[it] = (i < G * D) ? bf16_to_f32(p.q[head0 * D + i]) : 0.f;
-  }
+  if (tid < nch_cover * 4) sbase[tid] = (tid <= ((n - 1) >> 4)) ? (int)(bt_mine * BS) : 0;
   lds_barrier();
 
   // ---- key stream, set-up.  A chunk is 64 consecutive positions = 4 pages; its rows are fetched with
@@ -1195,7 +1204,12 @@ constexpr int MG_BT_LDS = 4096;    // block-table entries cached in LDS (65536 p
 // re-read from global memory in every pass.
 // Two shapes: 512 threads x 16 register-resident candidates each (up to 8192 candidates, the common case)
 // and 1024 x 32 for long contexts with wide top-k.
-template <int VBITS, int NG, int MG_THREADS, int MG_REGK>
+// PARTIAL = true is the first stage of the two-stage merge: blockIdx.z selects a run of mg_spp candidate
+// lists, steps 2 and 3 run on those alone and the winners (still in position order) are written out as one
+// new candidate list; the final merge (PARTIAL = false, mg_parts > 1) reads these lists instead of the
+// scan's.  The top K of a union is the top K of the parts' top K's, ties included: a candidate that a part
+// drops is beaten by K candidates of that part.
+template <int VBITS, int NG, int MG_THREADS, int MG_REGK, bool PARTIAL>
 __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) {
   constexpr int MG_WAVES = MG_THREADS / 64;
   constexpr int VP = D * VBITS / 8;
@@ -1225,29 +1239,36 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   const int b = blockIdx.x, hq = blockIdx.y, tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const size_t bh = (size_t)b * p.H_q + hq;
-  const int NS = p.n_splits, Kc = p.Kc, K = p.top_k;
+  const int NS = p.n_splits, K = p.top_k;
   const int hkv = hq / (p.H_q / p.H_kv);
-  const uint32_t* ck = p.cand_key + bh * NS * Kc;
-  const int32_t* ci = p.cand_idx + bh * NS * Kc;
-  const int32_t* cc = p.cand_cnt + bh * NS;
+  // candidate lists of this workgroup: NL lists of capacity Kc
+  const bool staged = !PARTIAL && p.mg_parts > 1;
+  const int part = PARTIAL ? (int)blockIdx.z : 0;
+  const int l0 = PARTIAL ? part * p.mg_spp : 0;
+  const int NL = PARTIAL ? min(p.mg_spp, NS - l0) : (staged ? p.mg_parts : NS);
+  const int Kc = staged ? K : p.Kc;
+  const uint32_t kc_magic = staged ? p.k_magic : p.kc_magic;
+  const uint32_t* ck = staged ? p.key2 + bh * p.mg_parts * K : p.cand_key + (bh * NS + l0) * Kc;
+  const int32_t* ci = staged ? p.idx2 + bh * p.mg_parts * K : p.cand_idx + (bh * NS + l0) * Kc;
+  const int32_t* cc = staged ? p.cnt2 + bh * p.mg_parts : p.cand_cnt + bh * NS + l0;
   const int64_t* bt = p.block_table + (size_t)b * p.max_blocks;
   int64_t* out_idx = p.topk_idx + bh * (size_t)K;
   int64_t* out_slot = p.topk_slots + bh * (size_t)K;
-  const int flat = NS * Kc;
+  const int flat = NL * Kc;
   const int rounds = (flat + MG_THREADS - 1) / MG_THREADS;
   const int nblk_lds = min(p.max_blocks, MG_BT_LDS);
 
-  long long* mclk = p.phase_clock ? p.phase_clock + (size_t)p.B * p.H_kv * p.n_splits * 10 + bh * 8 : nullptr;
+  long long* mclk = (p.phase_clock && !PARTIAL) ? p.phase_clock + (size_t)p.B * p.H_kv * p.n_splits * 10 + bh * 8 : nullptr;
   if (mclk && tid == 0) mclk[0] = clock64();
 
   // ---- everything that does not depend on anything else is requested first, in the order of its use
   float pm = -INFINITY, pl = 0.f;
   int my_cnt = 0;
-  if (tid < NS) {
+  if (!PARTIAL && tid < NS) {
     pm = p.part_m[bh * NS + tid];
     pl = p.part_l[bh * NS + tid];
-    my_cnt = cc[tid];
   }
+  if (tid < NL) my_cnt = cc[tid];
   const int rreg = min(rounds, MG_REGK);  // rounds whose candidates live in registers (uniform)
   uint32_t kreg[MG_REGK];
   int ireg[MG_REGK];
@@ -1261,7 +1282,7 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
     const int f = r * MG_THREADS + tid;
     ireg[r] = (r < rreg && f < flat) ? ci[f] : 0;
   }
-  if (tid < NS) cnt_sh[tid] = my_cnt;
+  if (tid < NL) cnt_sh[tid] = my_cnt;
   // o_hat: the thread groups of 128 take the splits round-robin (first terms requested now)
   constexpr int PO_PRE = 2, PO_GRP = MG_THREADS / D;
   float po[PO_PRE];
@@ -1270,36 +1291,37 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
 #pragma unroll
     for (int i = 0; i < PO_PRE; ++i) {
       const int sp = q4 + PO_GRP * i;
-      po[i] = (sp < NS) ? p.part_o[(bh * NS + sp) * D + d] : 0.f;
+      po[i] = (!PARTIAL && sp < NS) ? p.part_o[(bh * NS + sp) * D + d] : 0.f;
     }
   }
-  for (int i = tid; i < nblk_lds; i += MG_THREADS) bt_sh[i] = (int)bt[i];
+  if (!PARTIAL)
+    for (int i = tid; i < nblk_lds; i += MG_THREADS) bt_sh[i] = (int)bt[i];
   for (int i = tid; i < MG_BINS; i += MG_THREADS) hist[i] = 0;
   if (tid == 0) lcount_sh = 0;
 
   // ---- split statistics: M, coefficients e^{m_i - M}, l, o_hat
-  {
+  if (!PARTIAL) {
     const float v = wave_max(pm);
     if (lane == 0) wred_f[wave] = v;
   }
   lds_barrier();
   if (mclk && tid == 0) mclk[6] = clock64();
   float M = -INFINITY;
+  if (!PARTIAL) {
 #pragma unroll
-  for (int w = 0; w < MG_WAVES; ++w) M = fmaxf(M, wred_f[w]);
-  if (!isfinite(M)) M = 0.f;
-  const float coef = (pm == -INFINITY) ? 0.f : __expf(pm - M);
-  if (tid < NS) coef_sh[tid] = coef;
-  {
+    for (int w = 0; w < MG_WAVES; ++w) M = fmaxf(M, wred_f[w]);
+    if (!isfinite(M)) M = 0.f;
+    const float coef = (pm == -INFINITY) ? 0.f : __expf(pm - M);
+    if (tid < NS) coef_sh[tid] = coef;
     const float v = wave_sum(pl * coef);  // fixed reduction tree: deterministic
     lds_barrier();                      // wred_f was read above
     if (lane == 0) wred_f[wave] = v;
   }
   // candidates outside their list's count are not candidates: key 0 (no finite score maps to it)
   int total = 0;
-  for (int s2 = 0; s2 < NS; ++s2) total += cnt_sh[s2];
+  for (int s2 = 0; s2 < NL; ++s2) total += cnt_sh[s2];
   auto valid_f = [&](int f) -> bool {
-    const int s2 = (int)__umulhi((uint32_t)f, p.kc_magic);  // f / Kc, exact for f < 2^21
+    const int s2 = (int)__umulhi((uint32_t)f, kc_magic);  // f / Kc, exact for f < 2^21
     return f < flat && (f - s2 * Kc) < cnt_sh[s2];
   };
 #pragma unroll
@@ -1307,11 +1329,12 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
     if (r < rreg && !valid_f(r * MG_THREADS + tid)) kreg[r] = 0u;
   lds_barrier();
   if (mclk && tid == 0) mclk[7] = clock64();
-  float lsum = 0.f;
+  float inv_z = 0.f;
+  if (!PARTIAL) {
+    float lsum = 0.f;
 #pragma unroll
-  for (int w = 0; w < MG_WAVES; ++w) lsum += wred_f[w];
-  const float inv_z = (lsum > 0.f) ? 1.0f / lsum : 0.f;
-  {
+    for (int w = 0; w < MG_WAVES; ++w) lsum += wred_f[w];
+    inv_z = (lsum > 0.f) ? 1.0f / lsum : 0.f;
     // o_hat: four thread groups take every fourth split, then a fixed-order sum
     const int d = tid & (D - 1), q4 = tid >> 7;
     float o = 0.f;
@@ -1320,19 +1343,33 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
       const int sp = q4 + PO_GRP * i;
       if (sp < NS) o = __builtin_fmaf(po[i], coef_sh[sp], o);
     }
-    for (int sp = q4 + PO_GRP * PO_PRE; sp < NS; sp += PO_GRP) o = __builtin_fmaf(p.part_o[(bh * NS + sp) * D + d], coef_sh[sp], o);
-    red_sh[q4][d] = o;
-  }
-  lds_barrier();
-  if (tid < D) {
-    float o = red_sh[0][tid];
+    // the remaining splits eight at a time: the loads of a batch are in flight together, the sum keeps its order
+    constexpr int PO_B = 8;
+    for (int sp0 = q4 + PO_GRP * PO_PRE; sp0 < NS; sp0 += PO_GRP * PO_B) {
+      float v[PO_B];
 #pragma unroll
-    for (int q = 1; q < PO_GRP; ++q) o += red_sh[q][tid];  // fixed order
-    p.o_hat[bh * D + tid] = o * inv_z;
-  }
-  if (tid == 0 && p.softmax_m) {
-    p.softmax_m[bh] = M;
-    p.softmax_inv_z[bh] = inv_z;
+      for (int u = 0; u < PO_B; ++u) {
+        const int sp = sp0 + PO_GRP * u;
+        v[u] = (sp < NS) ? p.part_o[(bh * NS + sp) * D + d] : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < PO_B; ++u) {
+        const int sp = sp0 + PO_GRP * u;
+        if (sp < NS) o = __builtin_fmaf(v[u], coef_sh[sp], o);
+      }
+    }
+    red_sh[q4][d] = o;
+    lds_barrier();
+    if (tid < D) {
+      float o2 = red_sh[0][tid];
+#pragma unroll
+      for (int q = 1; q < PO_GRP; ++q) o2 += red_sh[q][tid];  // fixed order
+      p.o_hat[bh * D + tid] = o2 * inv_z;
+    }
+    if (tid == 0 && p.softmax_m) {
+      p.softmax_m[bh] = M;
+      p.softmax_inv_z[bh] = inv_z;
+    }
   }
   if (mclk && tid == 0) mclk[1] = clock64();
 
@@ -1555,6 +1592,15 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   }
   const int n_out = min(K, base_above + min(base_tie, quota));
   if (mclk && tid == 0) mclk[3] = clock64();
+  if (PARTIAL) {  // the winners become one candidate list of the final merge
+    const size_t lo = (bh * p.mg_parts + part) * (size_t)K;
+    for (int r = tid; r < n_out; r += MG_THREADS) {
+      p.key2[lo + r] = win_key[r];
+      p.idx2[lo + r] = win_idx[r];
+    }
+    if (tid == 0) p.cnt2[bh * p.mg_parts + part] = n_out;
+    return;
+  }
 
   // one thread per winner: position, paged slot, softmax weight
   for (int r = tid; r < K; r += MG_THREADS) {
@@ -1578,7 +1624,7 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
 
   // ---- pre-correction over the winners.  One winner row per DW lanes: lane (w_in, dwi) holds dword dwi of
   // the winner's packed V row (CPD codes) and accumulates its CPD channels; winners are visited in a fixed
-  // order, so the sums are run-to-run deterministic.  Four rows per lane are requested before any is used.
+  // order, so the sums are run-to-run deterministic.  UNR rows per lane are requested before any is used.
   const uint8_t* vbase = p.v_data + (size_t)hkv * p.num_slots * VP;
   const uint8_t* vsbase = reinterpret_cast<const uint8_t*>(p.v_scales + (size_t)hkv * p.num_slots * NG);
   const int dwi = lane % DW, w_in = lane / DW;
@@ -1587,7 +1633,7 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
 #pragma unroll
   for (int c = 0; c < CPD; ++c) acc[c] = 0.f;
   float accw = 0.f;
-  constexpr int UNR = 4;
+  constexpr int UNR = (256 / (MG_WAVES * WPI) > 0) ? 256 / (MG_WAVES * WPI) : 1;  // 256 winners per pass
   for (int k0 = wave * WPI; k0 < n_out; k0 += UNR * MG_WAVES * WPI) {
     uint32_t word[UNR];
     uint16_t sbits[UNR];
@@ -1614,17 +1660,43 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
       if (dwi == 0) accw += wv[u];
     }
   }
-  // reduce over the WPI winners of a wavefront instruction (lanes with equal dwi), then over wavefronts
+  // reduce over the WPI winners of a wavefront instruction (lanes with equal dwi): every exchange step halves
+  // the channels a lane is responsible for (the lane whose offset bit is clear keeps the lower half), so after
+  // log2(WPI) steps every lane holds the sums of CPD / WPI = 2 channels; then over wavefronts through LDS
+  {
+    int chan = dwi * CPD;
+    auto halve = [&](auto off_c, auto n_c) {
+      constexpr int OFF = decltype(off_c)::value, N = decltype(n_c)::value;
+      const bool upper = (lane & OFF) != 0;
 #pragma unroll
-  for (int off = DW; off < 64; off <<= 1) {
-#pragma unroll
-    for (int c = 0; c < CPD; ++c) acc[c] += __shfl_xor(acc[c], off);
-    accw += __shfl_xor(accw, off);
-  }
-  if (w_in == 0) {
-#pragma unroll
-    for (int c = 0; c < CPD; ++c) old_sh[wave][dwi * CPD + c] = acc[c];
-    if (dwi == 0) w_sh[wave] = accw;
+      for (int i = 0; i < N / 2; ++i) {
+        if constexpr (OFF == 32) {  // one half-wave swap serves both directions
+          const auto sw = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(uint32_t, acc[i]), __builtin_bit_cast(uint32_t, acc[i + N / 2]), false, false);
+          acc[i] = __builtin_bit_cast(float, (uint32_t)sw[0]) + __builtin_bit_cast(float, (uint32_t)sw[1]);
+        } else {
+          const float keep = upper ? acc[i + N / 2] : acc[i];
+          const int send = __builtin_bit_cast(int, upper ? acc[i] : acc[i + N / 2]);
+          // lane ^ 8: rotation by 8 inside the 16-lane row; lane ^ 16: swizzle inside 32 lanes
+          const int recv = (OFF == 8) ? dpp_mov<0x128, 0xf>(0, send) : __builtin_amdgcn_ds_swizzle(send, 0x401F);
+          acc[i] = keep + __builtin_bit_cast(float, recv);
+        }
+      }
+      chan += upper ? N / 2 : 0;
+    };
+    static_assert(DW == 8 || DW == 16, "V rows of 32 or 64 bytes");
+    if constexpr (DW == 8) {
+      halve(std::integral_constant<int, 8>{}, std::integral_constant<int, CPD>{});
+      halve(std::integral_constant<int, 16>{}, std::integral_constant<int, CPD / 2>{});
+      halve(std::integral_constant<int, 32>{}, std::integral_constant<int, CPD / 4>{});
+    } else {
+      halve(std::integral_constant<int, 16>{}, std::integral_constant<int, CPD>{});
+      halve(std::integral_constant<int, 32>{}, std::integral_constant<int, CPD / 2>{});
+    }
+    static_assert(CPD / WPI == 2, "two channels per lane after the exchange");
+    old_sh[wave][chan] = acc[0];
+    old_sh[wave][chan + 1] = acc[1];
+    const float wsum = wave_sum(accw);  // only the dwi == 0 lanes hold weights
+    if (lane == 0) w_sh[wave] = wsum;
   }
   lds_barrier();
   if (tid < D) {
@@ -1651,6 +1723,7 @@ struct ScanProfile {
 };
 ScanProfile g_prof;
 long long* g_phase_clock = nullptr;
+int g_force_split_len = 0;  // test / measurement aid: overrides the planner's split length when positive
 
 constexpr size_t LDS_BUDGET_2WG = 80 * 1024 - 512;    // two workgroups per CU (160 KB LDS)
 constexpr size_t LDS_BUDGET_1WG = 160 * 1024 - 1024;
@@ -1703,6 +1776,11 @@ inline void fused_plan(int scheme, int NG, int B, int H_q, int H_kv, int max_S, 
     }
     if (cand >= max_S) break;
   }
+  if (g_force_split_len > 0) {
+    L = (g_force_split_len + 255) / 256 * 256;
+    if (L > lmax) L = lmax;
+    while ((max_S + L - 1) / L > MG_MAX_SPLITS && L < lmax) L += 256;
+  }
   int ns = (max_S + L - 1) / L;
   if (ns < 1) ns = 1;
   *L_out = L;
@@ -1711,10 +1789,32 @@ inline void fused_plan(int scheme, int NG, int B, int H_q, int H_kv, int max_S, 
   *kc_out = cap < L ? cap : L;
 }
 
+// Two-stage merge when one workgroup per row would face more than 8192 candidates (what the 512-thread
+// shape keeps in registers): parts of at most 8192 candidates, enough of them for about two workgroups per
+// CU, at most 8192 / top_k so that the final merge keeps its candidates in registers too, and at least two
+// lists in every part.  parts == 1: single stage.
+constexpr int MG_REG_CANDS = 8192;
+inline void merge_plan(int rows, int ns, int kc, int top_k, int* parts_out, int* spp_out) {
+  *parts_out = 1;
+  *spp_out = ns;
+  if ((long long)ns * kc <= MG_REG_CANDS || ns < 4) return;
+  const int spp_max = MG_REG_CANDS / kc > 0 ? MG_REG_CANDS / kc : 1;
+  const int parts_min = (ns + spp_max - 1) / spp_max;
+  const int want = (512 + rows - 1) / (rows > 0 ? rows : 1);
+  int parts = parts_min > want ? parts_min : want;
+  const int cap = MG_REG_CANDS / top_k;
+  if (parts > cap) parts = cap;
+  if (parts > ns / 2) parts = ns / 2;
+  if (parts < 2) return;
+  const int spp = (ns + parts - 1) / parts;
+  *parts_out = (ns + spp - 1) / spp;
+  *spp_out = spp;
+}
+
 struct WsLayout {
-  size_t off_m, off_l, off_o, off_key, off_idx, off_cnt, total;
+  size_t off_m, off_l, off_o, off_key, off_idx, off_cnt, off_key2, off_idx2, off_cnt2, total;
 };
-inline WsLayout ws_layout(int B, int H_q, int ns, int kc) {
+inline WsLayout ws_layout(int B, int H_q, int ns, int kc, int parts, int top_k) {
   WsLayout w;
   const size_t rows = (size_t)B * H_q;
   size_t o = 0;
@@ -1725,6 +1825,12 @@ inline WsLayout ws_layout(int B, int H_q, int ns, int kc) {
   w.off_key = take(rows * ns * kc * 4);
   w.off_idx = take(rows * ns * kc * 4);
   w.off_cnt = take(rows * ns * 4);
+  w.off_key2 = w.off_idx2 = w.off_cnt2 = 0;
+  if (parts > 1) {
+    w.off_key2 = take(rows * parts * top_k * 4);
+    w.off_idx2 = take(rows * parts * top_k * 4);
+    w.off_cnt2 = take(rows * parts * 4);
+  }
   w.total = o + 256;
   return w;
 }
@@ -1763,7 +1869,9 @@ extern "C" size_t jf_fused_workspace_bytes(int scheme, int B, int H_q, int H_kv,
   for (int ng = 1; ng <= 2; ++ng) {
     int L, ns, kc;
     fused_plan(scheme, ng, B, H_q, H_kv, max_S, top_k, &L, &ns, &kc);
-    const size_t t = ws_layout(B, H_q, ns, kc).total;
+    int parts, spp;
+    merge_plan(B * H_q, ns, kc, top_k, &parts, &spp);
+    const size_t t = ws_layout(B, H_q, ns, kc, parts, top_k).total;
     if (t > worst) worst = t;
   }
   return worst;
@@ -1804,7 +1912,9 @@ extern "C" int jf_fused_scan_topk(int scheme, int group_size, const uint16_t* q,
   fused_plan(scheme, NGv, B, H_q, H_kv, max_S, top_k, &p.L, &p.n_splits, &p.Kc);
   p.kc_magic = (uint32_t)((0x100000000ull + (uint64_t)p.Kc - 1) / (uint64_t)p.Kc);
   JF_CHECK_ARG(p.n_splits <= MG_MAX_SPLITS, "fused_scan: too many splits (%d > %d)", p.n_splits, MG_MAX_SPLITS);
-  const WsLayout wl = ws_layout(B, H_q, p.n_splits, p.Kc);
+  merge_plan(B * H_q, p.n_splits, p.Kc, top_k, &p.mg_parts, &p.mg_spp);
+  p.k_magic = (uint32_t)((0x100000000ull + (uint64_t)top_k - 1) / (uint64_t)top_k);
+  const WsLayout wl = ws_layout(B, H_q, p.n_splits, p.Kc, p.mg_parts, top_k);
   JF_CHECK_ARG(workspace && workspace_bytes >= wl.total, "fused_scan: workspace too small (%zu < %zu)", workspace_bytes, wl.total);
   JF_CHECK_ARG(((uintptr_t)workspace & 255) == 0, "fused_scan: workspace must be 256-byte aligned");
   uint8_t* ws = reinterpret_cast<uint8_t*>(workspace);
@@ -1815,6 +1925,9 @@ extern "C" int jf_fused_scan_topk(int scheme, int group_size, const uint16_t* q,
   p.cand_key = reinterpret_cast<uint32_t*>(ws + wl.off_key);
   p.cand_idx = reinterpret_cast<int32_t*>(ws + wl.off_idx);
   p.cand_cnt = reinterpret_cast<int32_t*>(ws + wl.off_cnt);
+  p.key2 = reinterpret_cast<uint32_t*>(ws + wl.off_key2);
+  p.idx2 = reinterpret_cast<int32_t*>(ws + wl.off_idx2);
+  p.cnt2 = reinterpret_cast<int32_t*>(ws + wl.off_cnt2);
   p.topk_idx = topk_idx; p.topk_slots = topk_slots; p.o_hat = o_hat; p.o_old = o_old_unnorm; p.W = W;
   p.softmax_m = softmax_m; p.softmax_inv_z = softmax_inv_z;
   p.phase_clock = g_phase_clock;
@@ -1850,11 +1963,17 @@ extern "C" int jf_fused_scan_topk(int scheme, int group_size, const uint16_t* q,
   }
   if (rc != JF_OK) return rc;
   dim3 mgrid(B, H_q);
-  const bool big = (long long)p.n_splits * p.Kc > 8192;
-#define JF_MERGE(VB, NGG)                                                                                   \
-  do {                                                                                                      \
-    if (big) hipLaunchKernelGGL((fused_merge_kernel<VB, NGG, 1024, 32>), mgrid, dim3(1024), 0, st, p);      \
-    else hipLaunchKernelGGL((fused_merge_kernel<VB, NGG, 512, 16>), mgrid, dim3(512), 0, st, p);            \
+  if (p.mg_parts > 1) {  // first stage: every part's top_k, as new candidate lists
+    const dim3 pgrid(B, H_q, p.mg_parts);
+    if ((long long)p.mg_spp * p.Kc > MG_REG_CANDS) hipLaunchKernelGGL((fused_merge_kernel<4, 1, 1024, 32, true>), pgrid, dim3(1024), 0, st, p);
+    else hipLaunchKernelGGL((fused_merge_kernel<4, 1, 1024, 8, true>), pgrid, dim3(1024), 0, st, p);
+    JF_CHECK_LAUNCH();
+  }
+  const bool big = (p.mg_parts > 1 ? (long long)p.mg_parts * top_k : (long long)p.n_splits * p.Kc) > MG_REG_CANDS;
+#define JF_MERGE(VB, NGG)                                                                                     \
+  do {                                                                                                        \
+    if (big) hipLaunchKernelGGL((fused_merge_kernel<VB, NGG, 1024, 32, false>), mgrid, dim3(1024), 0, st, p); \
+    else hipLaunchKernelGGL((fused_merge_kernel<VB, NGG, 1024, 8, false>), mgrid, dim3(1024), 0, st, p);       \
   } while (0)
   if (scheme == JF_SCHEME_K3V2) {
     if (NGv == 2) JF_MERGE(2, 2);
@@ -1897,5 +2016,11 @@ extern "C" int jf_profile_scan_end(double* total_ms, int* launches) {
 
 extern "C" int jf_debug_phase_clock(void* device_buffer) {
   g_phase_clock = reinterpret_cast<long long*>(device_buffer);
+  return JF_OK;
+}
+
+extern "C" int jf_debug_split_len(int split_len) {
+  JF_CHECK_ARG(split_len >= 0, "debug_split_len: negative length");
+  g_force_split_len = split_len;
   return JF_OK;
 }
