@@ -86,15 +86,48 @@ def test_fused_scan_matches_oracle(scheme, B, Hq, Hkv, S, lens, K):
     check_against_oracle(scheme, c, S, K, out)
 
 
-def test_fused_scan_ties_go_to_the_lower_position():
+@pytest.mark.parametrize("scheme,S,lens,K,split_len", [
+    ("k3v2", 5000, [4987], 256, 256),      # 20 short splits: single-stage merge over many lists
+    ("k3v2", 10000, [9989], 256, 512),     # 20 lists of 512 candidates: two-stage merge
+    ("k4v4", 10000, [9000], 512, 768),     # two-stage, lists of top_k + 256 entries, empty tail splits
+    ("k4v4", 10000, [10000], 1024, 1280),  # widest top-k: parts limited to 8192 / top_k
+    ("k3v2", 3000, [3000], 64, 1024),      # longer than the planner would pick for this size
+])
+def test_fused_scan_with_forced_split_length(scheme, S, lens, K, split_len):
+    from jetfire_amd import _lib
+    lib = _lib.load()
+    kb, vb, gs = {"k3v2": (3, 2, 64), "k4v4": (4, 4, 128)}[scheme]
+    c = make_case(11 + S + K, 1, 8, 2, S, kb, vb, gs, lens=lens, extra_blocks=3)
+    d = to_device(c)
+    _lib.check(lib.jf_debug_split_len(split_len))
+    try:
+        out = run_fused(scheme, c, d, S, K)
+        forced = [t.clone() for t in out]
+    finally:
+        _lib.check(lib.jf_debug_split_len(0))
+    check_against_oracle(scheme, c, S, K, forced)
+    # the planner's own split length selects the same positions
+    again = run_fused(scheme, c, d, S, K)
+    assert torch.equal(forced[4], again[4]) and torch.equal(forced[1], again[1])
+
+
+@pytest.mark.parametrize("S,K,split_len", [(600, 64, 0), (10000, 256, 512)])
+def test_fused_scan_ties_go_to_the_lower_position(S, K, split_len):
     # identical keys in every slot -> every score of a head is equal: winners are positions 0..K-1
-    c = make_case(5, 1, 8, 2, 600, 3, 2, 64, ragged=False, shuffle=True)
+    # (the second case goes through the two-stage merge)
+    from jetfire_amd import _lib
+    lib = _lib.load()
+    c = make_case(5, 1, 8, 2, S, 3, 2, 64, ragged=False, shuffle=True)
     c["kd"][:] = c["kd"][:, :1]
     c["ks"][:] = c["ks"][:, :1]
     d = to_device(c)
-    out = run_fused("k3v2", c, d, 600, 64)
-    idx = out[4].cpu().numpy()
-    assert (idx == np.arange(64)[None, None, :]).all()
+    _lib.check(lib.jf_debug_split_len(split_len))
+    try:
+        out = run_fused("k3v2", c, d, S, K)
+        idx = out[4].cpu().numpy()
+    finally:
+        _lib.check(lib.jf_debug_split_len(0))
+    assert (idx == np.arange(K)[None, None, :]).all()
 
 
 def test_fused_scan_is_deterministic_and_matches_split_path():
