@@ -136,6 +136,13 @@ int jf_fused_scan_topk(int scheme, int group_size,
                        float* softmax_m, float* softmax_inv_z, float* scores,
                        void* workspace, size_t workspace_bytes, void* stream);
 
+/* Introspection with no counterpart in the reference: the launch geometry jf_fused_scan_topk uses for a
+ * shape.  split_len positions per scan workgroup, n_splits = ceil(max_S / split_len) workgroups per
+ * (sequence, kv-head), list_cap candidate slots per (row, split), merge_parts > 1 if the candidate lists are
+ * first reduced by that many workgroups per row.  Any output pointer may be NULL.  Needs no GPU. */
+int jf_fused_plan(int scheme, int group_size, int B, int H_q, int H_kv, int max_S, int top_k,
+                  int* split_len, int* n_splits, int* list_cap, int* merge_parts);
+
 /* Measurement aid with no counterpart in the reference: between begin and end, every launch of the fused
  * scan kernel is bracketed by a pair of HIP events recorded on the launch stream (at most max_launches
  * launches); end synchronises them and returns the summed device time and the number of launches. */

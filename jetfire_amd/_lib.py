@@ -34,6 +34,7 @@ SIGNATURES = {
     "jf_profile_scan_end": (I, [P, P]),
     "jf_debug_phase_clock": (I, [P]),
     "jf_debug_split_len": (I, [I]),
+    "jf_fused_plan": (I, [I, I, I, I, I, I, I, P, P, P, P]),
     "jf_blend_unnorm": (I, [P, P, P, P, P, I, I, I, P]),
     "jf_cpu_topk_attn": (I, [P, P, P, P, P, P, I, I, I, I, L, F, P]),
     "jf_set_cpu_attn_threads": (I, [I]),

@@ -1752,25 +1752,70 @@ inline int lmax_dispatch(int scheme, int G, int NG) {
   return 256;
 }
 
+// Estimated microseconds of the merge (fitted on MI355X): a fixed part per launch plus a part proportional to
+// the candidates one workgroup visits.
+constexpr double kMergeFixed = 8.5, kPartialFixed = 7.5, kPerCand = 0.0004, kPerCandBig = 0.001;
+constexpr int MG_REG_CANDS = 8192;  // candidates the common merge shape keeps in registers
+inline double merge_pass_us(double fixed, long cands) {
+  return cands <= MG_REG_CANDS ? fixed + kPerCand * (double)cands : fixed + 1.5 + kPerCandBig * (double)cands;
+}
+
+// Two-stage merge when one workgroup per row would face more than MG_REG_CANDS candidates: the number of
+// parts (at most MG_REG_CANDS / top_k, so that the final merge keeps its candidates in registers, and at least
+// two lists per part) with the smallest estimated time.  parts == 1: single stage.
+inline double merge_plan(int rows, int ns, int kc, int top_k, int* parts_out, int* spp_out) {
+  *parts_out = 1;
+  *spp_out = ns;
+  const double wide = 1.5 * (top_k > 256 ? (double)top_k / 256.0 - 1.0 : 0.0);  // slots and pre-correction of the winners
+  double best = merge_pass_us(kMergeFixed, (long)ns * kc) + wide;
+  if ((long long)ns * kc <= MG_REG_CANDS || ns < 4) return best;
+  int cap = MG_REG_CANDS / top_k;
+  if (cap > ns / 2) cap = ns / 2;
+  for (int parts = 2; parts <= cap; ++parts) {
+    const int spp = (ns + parts - 1) / parts;
+    if ((ns + spp - 1) / spp != parts) continue;  // the same spp as a smaller number of parts
+    const long wgs = (long)(rows > 0 ? rows : 1) * parts;
+    const double rounds = (double)((wgs + 511) / 512);  // two workgroups per CU
+    const double us = kPartialFixed + rounds * (merge_pass_us(kPartialFixed, (long)spp * kc) - kPartialFixed) +
+                      merge_pass_us(kMergeFixed, (long)parts * top_k) + wide;
+    if (us < best) {
+      best = us;
+      *parts_out = parts;
+      *spp_out = spp;
+    }
+  }
+  return best;
+}
+
 inline void fused_plan(int scheme, int NG, int B, int H_q, int H_kv, int max_S, int top_k, int* L_out, int* ns_out,
                        int* kc_out) {
   const int G = H_q / H_kv;
   const int units = B * H_kv > 0 ? B * H_kv : 1;
-  // One workgroup is resident per CU (256 CUs).  Among the split lengths that fit LDS pick the one that
-  // minimises (rounds of workgroups) x (split length + a fixed per-workgroup cost, in positions) plus a term
-  // for the merge kernel, whose work grows with the number of candidate lists; a launch whose workgroup
-  // count is just over a multiple of 256 pays a whole extra round.
+  const int rows = B * H_q > 0 ? B * H_q : 1;
+  // One scan workgroup is resident per CU (256 CUs).  Among the split lengths that fit LDS pick the one with
+  // the smallest estimated time of scan + merge.  The constants are microseconds fitted to measurements on
+  // MI355X: a scan workgroup costs a fixed part plus a part proportional to the 64-position chunks each of
+  // its wavefronts works through; a last, partly filled round of workgroups runs faster than a full one; the
+  // merge costs a fixed part per launch plus a part proportional to the candidates one workgroup visits.
   const int lmax = lmax_dispatch(scheme, G, NG);
-  constexpr int kCUs = 256, kFixed = 640;
+  const int nw = (G <= 4) ? 16 : 8;
+  constexpr int kCUs = 256;
+  constexpr double kScanFixed = 8.5;
+  const double per_chunk = (scheme == JF_SCHEME_K4V4) ? 6.6 : 5.9;  // one chunk per wavefront, all wavefronts
   int L = 256;
-  long best = -1;
+  double best = -1.0;
   for (int cand = 256; cand <= lmax; cand += 256) {
     const long nsp = (max_S + cand - 1) / cand > 0 ? (max_S + cand - 1) / cand : 1;
     if (nsp > MG_MAX_SPLITS && cand < lmax) continue;
-    const long rounds = (nsp * units + kCUs - 1) / kCUs;
-    const long kc = (top_k + FS_CAND_SLACK) < cand ? (top_k + FS_CAND_SLACK) : cand;
-    const long cost = rounds * (cand + kFixed) + nsp * kc / 5;  // + the merge kernel's pass over the candidates
-    if (best < 0 || cost <= best) {
+    const long nwg = nsp * units;
+    const long full = nwg / kCUs, rem = nwg % kCUs;
+    const double stream = per_chunk * (double)cand / (64.0 * nw);
+    double cost = (double)full * (kScanFixed + stream);
+    if (rem > 0) cost += kScanFixed + stream * (0.5 + 0.5 * (double)rem / kCUs);
+    const int kc = (top_k + FS_CAND_SLACK) < cand ? (top_k + FS_CAND_SLACK) : cand;
+    int parts, spp;
+    cost += merge_plan(rows, (int)nsp, kc, top_k, &parts, &spp);
+    if (best < 0.0 || cost <= best) {
       best = cost;
       L = cand;
     }
@@ -1787,28 +1832,6 @@ inline void fused_plan(int scheme, int NG, int B, int H_q, int H_kv, int max_S, 
   *ns_out = ns;
   const int cap = top_k + FS_CAND_SLACK;  // the split may emit a superset of its top-k (see phase C)
   *kc_out = cap < L ? cap : L;
-}
-
-// Two-stage merge when one workgroup per row would face more than 8192 candidates (what the 512-thread
-// shape keeps in registers): parts of at most 8192 candidates, enough of them for about two workgroups per
-// CU, at most 8192 / top_k so that the final merge keeps its candidates in registers too, and at least two
-// lists in every part.  parts == 1: single stage.
-constexpr int MG_REG_CANDS = 8192;
-inline void merge_plan(int rows, int ns, int kc, int top_k, int* parts_out, int* spp_out) {
-  *parts_out = 1;
-  *spp_out = ns;
-  if ((long long)ns * kc <= MG_REG_CANDS || ns < 4) return;
-  const int spp_max = MG_REG_CANDS / kc > 0 ? MG_REG_CANDS / kc : 1;
-  const int parts_min = (ns + spp_max - 1) / spp_max;
-  const int want = (512 + rows - 1) / (rows > 0 ? rows : 1);
-  int parts = parts_min > want ? parts_min : want;
-  const int cap = MG_REG_CANDS / top_k;
-  if (parts > cap) parts = cap;
-  if (parts > ns / 2) parts = ns / 2;
-  if (parts < 2) return;
-  const int spp = (ns + parts - 1) / parts;
-  *parts_out = (ns + spp - 1) / spp;
-  *spp_out = spp;
 }
 
 struct WsLayout {
@@ -1875,6 +1898,21 @@ extern "C" size_t jf_fused_workspace_bytes(int scheme, int B, int H_q, int H_kv,
     if (t > worst) worst = t;
   }
   return worst;
+}
+
+extern "C" int jf_fused_plan(int scheme, int group_size, int B, int H_q, int H_kv, int max_S, int top_k,
+                             int* split_len, int* n_splits, int* list_cap, int* merge_parts) {
+  JF_CHECK_ARG(scheme == JF_SCHEME_K3V2 || scheme == JF_SCHEME_K4V4, "fused_plan: unknown scheme %d", scheme);
+  JF_CHECK_ARG(B > 0 && H_q > 0 && H_kv > 0 && H_q % H_kv == 0 && max_S >= 0 && top_k > 0, "fused_plan: bad shape");
+  JF_CHECK_ARG(group_size == 64 || group_size == 128, "fused_plan: group_size must be 64 or 128");
+  int L, ns, kc, parts, spp;
+  fused_plan(scheme, scheme_ng(scheme, group_size), B, H_q, H_kv, max_S, top_k, &L, &ns, &kc);
+  merge_plan(B * H_q, ns, kc, top_k, &parts, &spp);
+  if (split_len) *split_len = L;
+  if (n_splits) *n_splits = ns;
+  if (list_cap) *list_cap = kc;
+  if (merge_parts) *merge_parts = parts;
+  return JF_OK;
 }
 
 extern "C" int jf_fused_scan_topk(int scheme, int group_size, const uint16_t* q, const uint8_t* k_data,
