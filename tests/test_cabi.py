@@ -113,3 +113,53 @@ def test_kernel_sets_mirror_the_reference_dispatch_protocol():
         k32.quant_write_k(None, None, None, None, object(), 64)
     with pytest.raises(ValueError):
         get_kernel_set("AsymInt2K4Level_SymInt2V")
+
+
+@pytest.mark.parametrize("scheme,gs,B,Hq,Hkv,S,K", [
+    (32, 64, 4, 32, 8, 32768, 256),       # the headline shape
+    (44, 128, 1, 32, 8, 131072, 512),     # long context, few rows: two-stage merge
+    (32, 64, 2, 32, 4, 65536, 512),
+    (32, 128, 1, 8, 8, 100, 32),
+    (44, 128, 64, 32, 8, 2048, 1024),
+    (44, 128, 1, 32, 8, 262144, 1024),
+    (32, 64, 1, 16, 1, 0, 64),
+])
+def test_fused_plan_geometry_is_consistent(scheme, gs, B, Hq, Hkv, S, K):
+    """Host logic of the fused launch (no GPU): the split grid covers max_S, stays inside the kernels' limits,
+    the two-stage merge keeps its final pass register-resident, and the workspace grows with it."""
+    import ctypes as C
+    from jetfire_amd import _lib
+    lib = _lib.load()
+    out = [C.c_int() for _ in range(4)]
+    _lib.check(lib.jf_fused_plan(scheme, gs, B, Hq, Hkv, S, K, *[C.byref(o) for o in out]))
+    L, ns, cap, parts = [o.value for o in out]
+    assert L % 256 == 0 and 256 <= L <= 4096
+    assert ns >= 1 and ns * L >= S and (ns - 1) * L < max(S, 1)
+    assert ns <= 256
+    assert cap == min(L, K + 256)
+    assert parts >= 1
+    if ns * cap <= 8192:
+        assert parts == 1
+    if parts > 1:
+        assert parts * K <= 8192 and parts * 2 <= ns
+    need = lib.jf_fused_workspace_bytes(scheme, B, Hq, Hkv, S, K)
+    rows = B * Hq
+    floor = rows * ns * (8 + 128 * 4 + cap * 8 + 4) + (rows * parts * (K * 8 + 4) if parts > 1 else 0)
+    assert need >= floor
+    # forcing a split length is honoured (rounded up to 256, clamped) and switched off again by 0
+    _lib.check(lib.jf_debug_split_len(300))
+    try:
+        _lib.check(lib.jf_fused_plan(scheme, gs, B, Hq, Hkv, S, K, C.byref(out[0]), None, None, None))
+        assert out[0].value == 512 or (S > 512 * 256 and out[0].value > 512)
+    finally:
+        _lib.check(lib.jf_debug_split_len(0))
+    _lib.check(lib.jf_fused_plan(scheme, gs, B, Hq, Hkv, S, K, C.byref(out[0]), None, None, None))
+    assert out[0].value == L
+
+
+def test_fused_plan_rejects_bad_shapes():
+    from jetfire_amd import _lib
+    lib = _lib.load()
+    assert lib.jf_fused_plan(7, 64, 1, 8, 2, 100, 32, None, None, None, None) != 0
+    assert lib.jf_fused_plan(32, 64, 1, 8, 3, 100, 32, None, None, None, None) != 0
+    assert lib.jf_fused_plan(32, 32, 1, 8, 2, 100, 32, None, None, None, None) != 0
