@@ -126,7 +126,11 @@ struct ScanLds {
   static constexpr int KP = K3 ? 48 : 64;
   static constexpr int KROW = K3 ? 48 : 80;     // LDS pitch of a staged key row (INT4: padded against bank conflicts)
   static constexpr int VP = K3 ? 32 : 64;
-  static constexpr int VROW = VP + 8;  // 16 consecutive rows hit 16 distinct bank pairs
+  // LDS pitch of a staged V row.  INT2 rows (32 bytes) are padded so that 16 consecutive rows hit 16 distinct
+  // bank pairs; INT4 rows (64 bytes) keep their pitch and swap their 16-byte quarters instead (quarter q of
+  // row r sits at q ^ ((r >> 2) & 3)), which has the same effect without the padding bytes.
+  static constexpr bool VSWZ = !K3;
+  static constexpr int VROW = VSWZ ? VP : VP + 8;
   static constexpr int VST = 64 * VROW;
   static constexpr int WL = NG * NSET * 64 * 16;  // per (group, set): one 16-byte weight row per token
   static constexpr int KST = 64 * KROW;
@@ -138,7 +142,10 @@ struct ScanLds {
   // with one head set and enough staging space the exchange runs in the staging area while the score rows
   // are still being read by the candidate emission
   static constexpr int PREP = K3 ? (int)sizeof(K3Prep<NSET>) : (int)sizeof(QInt8F<NSET>);
-  static constexpr int HIST = G * SEG * 256 * 4;
+  // selection histograms: 32-bit counters, or (INT4 scheme, where LDS is tighter) two 16-bit counters per
+  // word: a (head, segment) histogram counts at most LMAX / SEG <= 4096 positions
+  static constexpr bool H16 = !K3;
+  static constexpr int HIST = G * SEG * 256 * (H16 ? 2 : 4);
   static constexpr int AUX = ((PREP > HIST ? PREP : HIST) + 15) & ~15;
   __host__ __device__ static constexpr int stage_bytes() { return NW * WAVE_STAGE; }
   static constexpr bool XS = (NSET == 1) && (NW * WAVE_STAGE >= RED);
@@ -425,7 +432,8 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     const int o = 1024 * i + 16 * lane;
     vl_page[i] = (uint32_t)(o / (16 * VP));
     vl_off[i] = (uint32_t)(o % (16 * VP));
-    vl_lds[i] = (uint32_t)((o / VP) * VROW + (o % VP));
+    const int row = o / VP, q16 = (o % VP) / 16;
+    vl_lds[i] = Lds::VSWZ ? (uint32_t)(row * VROW + ((q16 ^ ((row >> 2) & 3)) * 16)) : (uint32_t)(row * VROW + (o % VP));
   }
   struct VBuf {
     v4u r[VLD];
@@ -725,7 +733,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
       const int h = i / n_cover, t = i - h * n_cover;
       p.scores[(head0 + h) * (size_t)p.max_S + s0 + t] = sc[h * L + t];
     }
-  for (int i = tid; i < G * SEG * 256; i += NT) hist[i] = 0;
+  for (int i = tid; i < Lds::HIST / 4; i += NT) hist[i] = 0;
   if (tid < G) {
     float m = red_f[0][tid], lo = red_f[0][G + tid];
 #pragma unroll
@@ -794,7 +802,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     float vsf[NG];
     vsf[0] = ldexpf(bf16_to_f32((uint16_t)(vsw & 0xffffu)), E[0]);
     if (NG == 2) vsf[NG - 1] = ldexpf(bf16_to_f32((uint16_t)(vsw >> 16)), E[NG - 1]);
-    int* hb = hist + ((SEG == 1) ? 0 : (chunk / seg_chunks) * 256);
+    int* hb = hist + ((SEG == 1) ? 0 : (chunk / seg_chunks) * (Lds::H16 ? 128 : 256));
     const bool tv = t < n;
     uint32_t bits[NSET * 4][NG];
 #pragma unroll
@@ -807,7 +815,11 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
 #pragma unroll
         for (int g = 0; g < NG; ++g) bits[h][g] = __builtin_bit_cast(uint32_t, __builtin_fmaf(pw, vsf[g], 8388608.0f));
         const uint32_t bin = (uint32_t)__builtin_amdgcn_fmed3f(__builtin_fmaf(s, bin_a[h], bin_b[h]), 0.f, 255.f);
-        if (tv) atomicAdd(hb + h * (SEG * 256) + (int)bin, 1);
+        if (Lds::H16) {
+          if (tv) atomicAdd(hb + ((h * (SEG * 256) + (int)bin) >> 1), (bin & 1u) ? 0x10000 : 1);
+        } else {
+          if (tv) atomicAdd(hb + h * (SEG * 256) + (int)bin, 1);
+        }
       } else {
 #pragma unroll
         for (int g = 0; g < NG; ++g) bits[h][g] = 0x4b000000u;
@@ -866,9 +878,10 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
         }
       }
     } else {
+      const int vx = 16 * ((lane >> 2) & 3);  // quarter swap of this lane's row
 #pragma unroll
       for (int qc = 0; qc < 8; ++qc) {
-        const v2i x = __builtin_amdgcn_ds_read_tr4_b64_v2i32((__attribute__((address_space(3))) v2i*)(vrow + 8 * qc));
+        const v2i x = __builtin_amdgcn_ds_read_tr4_b64_v2i32((__attribute__((address_space(3))) v2i*)(vrow + (Lds::VSWZ ? ((8 * qc) ^ vx) : 8 * qc)));
         const uint32_t x0 = (uint32_t)x[0], x1 = (uint32_t)x[1];
         const v4i Bv = {(int)(x0 & 0x0f0f0f0fu), (int)((x0 >> 4) & 0x0f0f0f0fu),
                         (int)(x1 & 0x0f0f0f0fu), (int)((x1 >> 4) & 0x0f0f0f0fu)};
@@ -883,9 +896,13 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   auto stash_v = [&](const VBuf& vbuf) {
 #pragma unroll
     for (int i = 0; i < VLD; ++i) {
-      v2u* dst = reinterpret_cast<v2u*>(vst + vl_lds[i]);
-      dst[0] = (v2u){vbuf.r[i][0], vbuf.r[i][1]};
-      dst[1] = (v2u){vbuf.r[i][2], vbuf.r[i][3]};
+      if (Lds::VSWZ) {
+        *reinterpret_cast<v4u*>(vst + vl_lds[i]) = vbuf.r[i];  // 16-byte aligned with the unpadded pitch
+      } else {
+        v2u* dst = reinterpret_cast<v2u*>(vst + vl_lds[i]);
+        dst[0] = (v2u){vbuf.r[i][0], vbuf.r[i][1]};
+        dst[1] = (v2u){vbuf.r[i][2], vbuf.r[i][3]};
+      }
     }
   };
 #pragma unroll
@@ -980,17 +997,27 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   const int Kcap = p.Kc;
   const int Kt = min(p.top_k, n);
   for (int h = wave; h < G; h += NW) {
-    const int* h0 = hist + h * (SEG * 256);
+    const int* h0 = hist + h * (SEG * 256) / (Lds::H16 ? 2 : 1);
     // lane l owns buckets 4l .. 4l+3 (ascending bucket = descending score) of every segment's histogram
     int cs[SEG][4], c[4], mine = 0;
+#pragma unroll
+    for (int sg = 0; sg < SEG; ++sg) {
+      if (Lds::H16) {
+        const uint32_t w0 = (uint32_t)h0[sg * 128 + 2 * lane], w1 = (uint32_t)h0[sg * 128 + 2 * lane + 1];
+        cs[sg][0] = (int)(w0 & 0xffffu);
+        cs[sg][1] = (int)(w0 >> 16);
+        cs[sg][2] = (int)(w1 & 0xffffu);
+        cs[sg][3] = (int)(w1 >> 16);
+      } else {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) cs[sg][u] = h0[sg * 256 + 4 * lane + u];
+      }
+    }
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       c[u] = 0;
 #pragma unroll
-      for (int sg = 0; sg < SEG; ++sg) {
-        cs[sg][u] = h0[sg * 256 + 4 * lane + u];
-        c[u] += cs[sg][u];
-      }
+      for (int sg = 0; sg < SEG; ++sg) c[u] += cs[sg][u];
       mine += c[u];
     }
     const int incl = wave_incl_scan_i(mine);
