@@ -60,7 +60,6 @@ struct FusedParams {
   float attn_scale;
   int top_k;
   int L, n_splits, Kc;
-  uint32_t kc_magic;  // ceil(2^32 / Kc)
   float* scores;  // optional (B, H_q, max_S)
   float* part_m;  // (B, H_q, NS)
   float* part_l;  // (B, H_q, NS)
@@ -71,7 +70,6 @@ struct FusedParams {
   // two-stage merge (long contexts): `mg_parts` workgroups per row first reduce `mg_spp` consecutive
   // candidate lists each to the row's top_k among them; the final merge then reads those lists
   int mg_parts, mg_spp;
-  uint32_t k_magic;    // ceil(2^32 / top_k)
   uint32_t* key2;      // (B, H_q, mg_parts, top_k)
   int32_t* idx2;       // (B, H_q, mg_parts, top_k)
   int32_t* cnt2;       // (B, H_q, mg_parts)
@@ -262,6 +260,8 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
       p.part_l[part_base + (size_t)tid * p.n_splits] = 0.f;
       p.cand_cnt[part_base + (size_t)tid * p.n_splits] = 0;
     }
+    for (int i = tid; i < G * p.Kc; i += NT)  // unused candidate slots hold key 0 (no score maps to it)
+      p.cand_key[(part_base + (size_t)(i / p.Kc) * p.n_splits) * p.Kc + (i % p.Kc)] = 0u;
     return;
   }
 
@@ -1079,6 +1079,10 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
       const int te = min(n, (seg + 1) * (L / SEG));
       // the emitted total is at most Kcap by construction of the cut
       int count = __builtin_amdgcn_readfirstlane(segoff_sh[h][seg]);
+      // unused slots hold key 0 (no score maps to it); the planned total is known, so the head's wavefronts
+      // share the padding and its stores leave before the emission's
+      const int etot = min(Kcap, __builtin_amdgcn_readfirstlane(segoff_sh[h][SEG]));
+      for (int i = etot + seg * 64 + lane; i < Kcap; i += SEG * 64) ck[i] = 0u;
       uint8_t* ckb = reinterpret_cast<uint8_t*>(ck);
       uint8_t* cib = reinterpret_cast<uint8_t*>(ci);
       for (int t0 = tb; t0 < te; t0 += 512) {
@@ -1101,7 +1105,10 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
           count += __popcll(ma);
         }
       }
-      if (lane == 0 && seg == SEG - 1) p.cand_cnt[part_base + (size_t)h * p.n_splits] = min(Kcap, count);
+      if (seg == SEG - 1) {
+        if (lane == 0) p.cand_cnt[part_base + (size_t)h * p.n_splits] = min(Kcap, count);
+        for (int i = count + lane; i < etot; i += 64) ck[i] = 0u;  // (only if a segment emitted less than planned)
+      }
     } else if (seg == 0) {
       // exact fallback: 8-bit radix select over the order-preserving keys (bits shared by every key skipped),
       // then the keys above the K-th and the lowest-position ties that fill the quota
@@ -1178,6 +1185,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
       }
       count += min(base_tie, quota);
       if (lane == 0) p.cand_cnt[part_base + (size_t)h * p.n_splits] = min(Kcap, count);
+      for (int i = count + lane; i < Kcap; i += 64) ck[i] = 0u;
     }
   }
   lds_barrier();
@@ -1253,14 +1261,14 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   __shared__ int win_idx[FS_MAX_TOPK];
   __shared__ int win_slot[FS_MAX_TOPK];
   __shared__ float win_w[FS_MAX_TOPK];
-  __shared__ int cnt_a[MG_REGK * MG_WAVES], cnt_t[MG_REGK * MG_WAVES];
+  __shared__ uint32_t cnt_a[MG_REGK / 4 * MG_WAVES];  // packed (winners, ties) per (group, wavefront)
   __shared__ float red_sh[MG_THREADS / D][D];
   __shared__ float old_sh[MG_WAVES][D];
   __shared__ float w_sh[MG_WAVES];
   __shared__ float wred_f[MG_WAVES];
   __shared__ uint32_t wred_u[MG_WAVES];
   __shared__ int wred_i[MG_WAVES], wred_j[MG_WAVES];
-  __shared__ int lcount_sh, cut_sh, above_sh, quota_sh, tot_a_sh, tot_t_sh;
+  __shared__ int lcount_sh, cut_sh, above_sh, quota_sh;
   __shared__ uint32_t tau_sh;
 
   const int b = blockIdx.x, hq = blockIdx.y, tid = threadIdx.x, lane = tid & 63;
@@ -1274,7 +1282,6 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   const int l0 = PARTIAL ? part * p.mg_spp : 0;
   const int NL = PARTIAL ? min(p.mg_spp, NS - l0) : (staged ? p.mg_parts : NS);
   const int Kc = staged ? K : p.Kc;
-  const uint32_t kc_magic = staged ? p.k_magic : p.kc_magic;
   const uint32_t* ck = staged ? p.key2 + bh * p.mg_parts * K : p.cand_key + (bh * NS + l0) * Kc;
   const int32_t* ci = staged ? p.idx2 + bh * p.mg_parts * K : p.cand_idx + (bh * NS + l0) * Kc;
   const int32_t* cc = staged ? p.cnt2 + bh * p.mg_parts : p.cand_cnt + bh * NS + l0;
@@ -1296,18 +1303,29 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
     pl = p.part_l[bh * NS + tid];
   }
   if (tid < NL) my_cnt = cc[tid];
-  const int rreg = min(rounds, MG_REGK);  // rounds whose candidates live in registers (uniform)
+  // The first MG_REGK * MG_THREADS candidates live in registers: group g = r / 4 of a thread holds the four
+  // consecutive candidates (g * MG_THREADS + tid) * 4 + (r % 4), fetched with one 16-byte load.  Candidate
+  // order = (group, thread, element).  Slots past a list's count hold key 0 (written by the producer).
+  static_assert(MG_REGK % 4 == 0, "register candidates come in groups of four");
+  constexpr int NGRP = MG_REGK / 4;
+  const int rreg = min((flat + 4 * MG_THREADS - 1) / (4 * MG_THREADS), NGRP) * 4;  // register slots in use (uniform)
   uint32_t kreg[MG_REGK];
   int ireg[MG_REGK];
 #pragma unroll
-  for (int r = 0; r < MG_REGK; ++r) {
-    const int f = r * MG_THREADS + tid;
-    kreg[r] = (r < rreg && f < flat) ? ck[f] : 0u;
+  for (int g = 0; g < NGRP; ++g) {
+    const int f4 = (g * MG_THREADS + tid) * 4;
+    v4u k4 = {0u, 0u, 0u, 0u};
+    if (4 * g < rreg && f4 < flat) k4 = *reinterpret_cast<const v4u*>(ck + f4);  // flat is a multiple of 4
+#pragma unroll
+    for (int j = 0; j < 4; ++j) kreg[4 * g + j] = k4[j];
   }
 #pragma unroll
-  for (int r = 0; r < MG_REGK; ++r) {
-    const int f = r * MG_THREADS + tid;
-    ireg[r] = (r < rreg && f < flat) ? ci[f] : 0;
+  for (int g = 0; g < NGRP; ++g) {
+    const int f4 = (g * MG_THREADS + tid) * 4;
+    v4i i4 = {0, 0, 0, 0};
+    if (4 * g < rreg && f4 < flat) i4 = *reinterpret_cast<const v4i*>(ci + f4);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) ireg[4 * g + j] = i4[j];
   }
   if (tid < NL) cnt_sh[tid] = my_cnt;
   // o_hat: the thread groups of 128 take the splits round-robin (first terms requested now)
@@ -1344,16 +1362,8 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
     lds_barrier();                      // wred_f was read above
     if (lane == 0) wred_f[wave] = v;
   }
-  // candidates outside their list's count are not candidates: key 0 (no finite score maps to it)
   int total = 0;
   for (int s2 = 0; s2 < NL; ++s2) total += cnt_sh[s2];
-  auto valid_f = [&](int f) -> bool {
-    const int s2 = (int)__umulhi((uint32_t)f, kc_magic);  // f / Kc, exact for f < 2^21
-    return f < flat && (f - s2 * Kc) < cnt_sh[s2];
-  };
-#pragma unroll
-  for (int r = 0; r < MG_REGK; ++r)
-    if (r < rreg && !valid_f(r * MG_THREADS + tid)) kreg[r] = 0u;
   lds_barrier();
   if (mclk && tid == 0) mclk[7] = clock64();
   float inv_z = 0.f;
@@ -1403,7 +1413,7 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   // key of candidate f in pass-over-all-candidates loops: registers first, global memory beyond
   auto key_of = [&](int r) -> uint32_t {
     const int f = r * MG_THREADS + tid;
-    return valid_f(f) ? ck[f] : 0u;
+    return (f < flat) ? ck[f] : 0u;
   };
   // number of candidates with key >= x (x > 0), identical in every thread
   auto count_ge = [&](uint32_t x) -> int {
@@ -1524,67 +1534,61 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   }
   if (mclk && tid == 0) mclk[2] = clock64();
 
-  // ---- ordered compaction: pass 1 stores every (round, wavefront) count, one scan turns them into offsets,
-  // pass 2 places the winners; the owner of a winner stores its key and position
+  // ---- ordered compaction.  Register candidates: every thread counts its winners and ties per group, a
+  // wavefront scan plus the wavefront totals in LDS give the thread's first place, and the thread places its
+  // (consecutive) candidates one after the other.  The owner of a winner stores its key and position.
   int base_above = 0, base_tie = 0;
   {
-    // (round, wavefront) counts of winners / ties, packed: low half = above, high half = ties
+    int cnt_g[NGRP];  // low half: winners, high half: ties of this thread in group g
+    int scan_g[NGRP];
 #pragma unroll
-    for (int r = 0; r < MG_REGK; ++r) {
-      unsigned long long ma = 0ull, mt = 0ull;
-      if (r < rreg) {
-        const uint32_t key = kreg[r];
-        const bool above = (key != 0u) && (take_all || key > tau), tie = (key != 0u) && !take_all && key == tau;
-        ma = __builtin_amdgcn_ballot_w64(above);
-        mt = __builtin_amdgcn_ballot_w64(tie);
-      }
-      if (lane == 0) {
-        cnt_a[r * MG_WAVES + wave] = __popcll(ma);
-        cnt_t[r * MG_WAVES + wave] = __popcll(mt);
-      }
-    }
-    lds_barrier();
-    if (wave == 0) {  // exclusive scan of the (round, wave) counts, EPL consecutive entries per lane
-      constexpr int EPL = MG_REGK * MG_WAVES / 64;
-      int a[EPL], t[EPL], sa = 0, st = 0;
+    for (int g = 0; g < NGRP; ++g) {
+      int c = 0;
+      if (4 * g < rreg) {
 #pragma unroll
-      for (int i = 0; i < EPL; ++i) {
-        a[i] = cnt_a[lane * EPL + i];
-        t[i] = cnt_t[lane * EPL + i];
-        sa += a[i];
-        st += t[i];
-      }
-      const int ia = wave_incl_scan_i(sa), it = wave_incl_scan_i(st);
-      int ra = ia - sa, rt = it - st;
-#pragma unroll
-      for (int i = 0; i < EPL; ++i) {
-        cnt_a[lane * EPL + i] = ra;
-        cnt_t[lane * EPL + i] = rt;
-        ra += a[i];
-        rt += t[i];
-      }
-      if (lane == 63) { tot_a_sh = ia; tot_t_sh = it; }
-    }
-    lds_barrier();
-#pragma unroll
-    for (int r = 0; r < MG_REGK; ++r) {
-      if (r < rreg) {
-        const uint32_t key = kreg[r];
-        const bool above = (key != 0u) && (take_all || key > tau), tie = (key != 0u) && !take_all && key == tau;
-        const unsigned long long ma = __builtin_amdgcn_ballot_w64(above), mt = __builtin_amdgcn_ballot_w64(tie);
-        const int pa = cnt_a[r * MG_WAVES + wave] + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(ma >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)ma, 0u));
-        const int pt = cnt_t[r * MG_WAVES + wave] + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(mt >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mt, 0u));
-        if (above || (tie && pt < quota)) {
-          const int pos = pa + min(pt, quota);
-          if (pos < K) {
-            win_key[pos] = kreg[r];
-            win_idx[pos] = ireg[r];
-          }
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t key = kreg[4 * g + j];
+          const bool above = (key != 0u) && (take_all || key > tau), tie = (key != 0u) && !take_all && key == tau;
+          c += (above ? 1 : 0) + (tie ? 0x10000 : 0);
         }
       }
+      cnt_g[g] = c;
+      scan_g[g] = wave_incl_scan_i(c);  // at most 4 * 64 per half: no carry between the halves
+      if (lane == 63) cnt_a[g * MG_WAVES + wave] = (uint32_t)scan_g[g];
     }
-    base_above = tot_a_sh;
-    base_tie = tot_t_sh;
+    lds_barrier();
+    uint32_t run = 0u;  // packed totals of the groups before g (each half stays below 2^16: at most 32768 candidates)
+#pragma unroll
+    for (int g = 0; g < NGRP; ++g) {
+      uint32_t before = 0u, all = 0u;
+#pragma unroll
+      for (int w = 0; w < MG_WAVES; ++w) {
+        const uint32_t t = cnt_a[g * MG_WAVES + w];
+        before += (w < wave) ? t : 0u;
+        all += t;
+      }
+      if (4 * g < rreg) {
+        const uint32_t start = run + before + (uint32_t)(scan_g[g] - cnt_g[g]);
+        int pa = (int)(start & 0xffffu), pt = (int)(start >> 16);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t key = kreg[4 * g + j];
+          const bool above = (key != 0u) && (take_all || key > tau), tie = (key != 0u) && !take_all && key == tau;
+          if (above || (tie && pt < quota)) {
+            const int pos = pa + min(pt, quota);
+            if (pos < K) {
+              win_key[pos] = key;
+              win_idx[pos] = ireg[4 * g + j];
+            }
+          }
+          pa += above ? 1 : 0;
+          pt += tie ? 1 : 0;
+        }
+      }
+      run += all;
+    }
+    base_above = (int)(run & 0xffffu);
+    base_tie = (int)(run >> 16);
     lds_barrier();
   }
   for (int r = MG_REGK; r < rounds; ++r) {  // candidates beyond the register-resident ones, one round at a time
@@ -1621,9 +1625,9 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   if (mclk && tid == 0) mclk[3] = clock64();
   if (PARTIAL) {  // the winners become one candidate list of the final merge
     const size_t lo = (bh * p.mg_parts + part) * (size_t)K;
-    for (int r = tid; r < n_out; r += MG_THREADS) {
-      p.key2[lo + r] = win_key[r];
-      p.idx2[lo + r] = win_idx[r];
+    for (int r = tid; r < K; r += MG_THREADS) {
+      p.key2[lo + r] = (r < n_out) ? win_key[r] : 0u;  // unused slots: key 0
+      if (r < n_out) p.idx2[lo + r] = win_idx[r];
     }
     if (tid == 0) p.cnt2[bh * p.mg_parts + part] = n_out;
     return;
@@ -1975,10 +1979,8 @@ extern "C" int jf_fused_scan_topk(int scheme, int group_size, const uint16_t* q,
   p.B = B; p.H_q = H_q; p.H_kv = H_kv; p.max_S = max_S; p.max_blocks = max_blocks; p.num_slots = num_slots;
   p.attn_scale = attn_scale; p.top_k = top_k;
   fused_plan(scheme, NGv, B, H_q, H_kv, max_S, top_k, &p.L, &p.n_splits, &p.Kc);
-  p.kc_magic = (uint32_t)((0x100000000ull + (uint64_t)p.Kc - 1) / (uint64_t)p.Kc);
   JF_CHECK_ARG(p.n_splits <= MG_MAX_SPLITS, "fused_scan: too many splits (%d > %d)", p.n_splits, MG_MAX_SPLITS);
   merge_plan(B * H_q, p.n_splits, p.Kc, top_k, &p.mg_parts, &p.mg_spp);
-  p.k_magic = (uint32_t)((0x100000000ull + (uint64_t)top_k - 1) / (uint64_t)top_k);
   const WsLayout wl = ws_layout(B, H_q, p.n_splits, p.Kc, p.mg_parts, top_k);
   JF_CHECK_ARG(workspace && workspace_bytes >= wl.total, "fused_scan: workspace too small (%zu < %zu)", workspace_bytes, wl.total);
   JF_CHECK_ARG(((uintptr_t)workspace & 255) == 0, "fused_scan: workspace must be 256-byte aligned");
