@@ -95,6 +95,8 @@ __device__ inline float dpp_f32(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
 }
 
+// Grid: x = blocks of 16 tokens, y = kv-head, z = tensor (K or V of the fused launch): no index arithmetic
+// beyond adds, and the 16 rows of a block leave as one contiguous run when their slots are consecutive.
 template <int NBITS>
 __global__ __launch_bounds__(256) void quant_write16_kernel(RowSrc s0, RowDst d0, RowSrc s1, RowDst d1,
                                                             const int64_t* __restrict__ slots, int64_t T,
@@ -102,15 +104,12 @@ __global__ __launch_bounds__(256) void quant_write16_kernel(RowSrc s0, RowDst d0
   constexpr int QMAX = (1 << (NBITS - 1)) - 1;
   constexpr int OFF = 1 << (NBITS - 1);
   const int l16 = threadIdx.x & 15;
-  const int64_t unit = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
-  const int64_t total = T * H_kv * n_tensors;
+  const int64_t tq = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+  const int h = blockIdx.y;
+  const int which = blockIdx.z;
   // rows past the end and masked rows still take part in the cross-lane steps (with zeros)
-  bool live = unit < total;
-  const int64_t uc = live ? unit : 0;
-  const int which = (int)(uc / (T * H_kv));
-  const int64_t rem = uc - (int64_t)which * T * H_kv;
-  const int64_t t = rem / H_kv;
-  const int h = (int)(rem - t * H_kv);
+  bool live = tq < T;
+  const int64_t t = live ? tq : 0;
   const int64_t slot = slots[t];
   live = live && slot >= 0;
   const RowSrc& s = which ? s1 : s0;
@@ -134,9 +133,20 @@ __global__ __launch_bounds__(256) void quant_write16_kernel(RowSrc s0, RowDst d0
   const float sraw = fmaxf(amax / (float)QMAX, 1e-8f);
   const uint16_t sb = f32_to_bf16(sraw);
   const float sf = bf16_to_f32(sb);
+  // code = clamp(rint(x / sf)).  x and sf are bf16 values (8 significant bits each), so the exact quotient is
+  // either exactly a half-integer or at least 1/2040 away from one (for |q| >= 1/2): rint of the fp32-rounded
+  // quotient equals rint of ANY value within a few ulp of the exact quotient, provided exact half-integers come
+  // out exact.  q0 = x * rcp(sf) is within 2 ulp; one correction with the exact residual r = x - sf * q0 (an
+  // fma) gives the exact quotient up to ~2^-45 relative, which rounds to the half-integer itself in a tie.
+  // One reciprocal per lane replaces eight correctly rounded divisions.
+  const float ry = __builtin_amdgcn_rcpf(sf);
   uint32_t c[8];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) c[i] = (uint32_t)((int)fminf(fmaxf(rintf(x[i] / sf), (float)-QMAX), (float)QMAX) + OFF);
+  for (int i = 0; i < 8; ++i) {
+    const float q0 = x[i] * ry;
+    const float q = __builtin_fmaf(__builtin_fmaf(-sf, q0, x[i]), ry, q0);
+    c[i] = (uint32_t)((int)fminf(fmaxf(rintf(q), (float)-QMAX), (float)QMAX) + OFF);
+  }
   uint8_t* drow = d.data + (int64_t)h * d.data_stride_h + slot * d.data_stride_slot;
   uint16_t* srow = d.scale + (int64_t)h * d.scale_stride_h + slot * d.scale_stride_slot;
   const int lpg = group_size >> 3;  // lanes per scale group
@@ -222,7 +232,7 @@ extern "C" int jf_quant_write_sym(const uint16_t* x, int64_t x_stride_t, int64_t
   const int64_t units = T * H_kv;
   hipStream_t st = (hipStream_t)stream;
   if (rows_16b_aligned(x, x_stride_t, x_stride_h)) {
-    dim3 grid16((unsigned)((units + 15) / 16)), block16(256);
+    dim3 grid16((unsigned)((T + 15) / 16), (unsigned)H_kv, 1), block16(256);
     if (nbits == 2) hipLaunchKernelGGL(quant_write16_kernel<2>, grid16, block16, 0, st, s, d, s, d, slots, T, H_kv, 1, group_size);
     else if (nbits == 3) hipLaunchKernelGGL(quant_write16_kernel<3>, grid16, block16, 0, st, s, d, s, d, slots, T, H_kv, 1, group_size);
     else hipLaunchKernelGGL(quant_write16_kernel<4>, grid16, block16, 0, st, s, d, s, d, slots, T, H_kv, 1, group_size);
@@ -256,7 +266,7 @@ extern "C" int jf_quant_write_int4_sym_kv(const uint16_t* key, int64_t k_stride_
   RowDst d1{v_data, v_data_stride_h, v_data_stride_slot, v_scale, v_scale_stride_h, v_scale_stride_slot};
   const int64_t units = T * H_kv * 2;
   if (rows_16b_aligned(key, k_stride_t, k_stride_h) && rows_16b_aligned(value, v_stride_t, v_stride_h)) {
-    dim3 grid16((unsigned)((units + 15) / 16)), block16(256);
+    dim3 grid16((unsigned)((T + 15) / 16), (unsigned)H_kv, 2), block16(256);
     hipLaunchKernelGGL(quant_write16_kernel<4>, grid16, block16, 0, (hipStream_t)stream, s0, d0, s1, d1, slots, T, H_kv, 2, group_size);
     JF_CHECK_LAUNCH();
     return JF_OK;

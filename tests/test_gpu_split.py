@@ -67,6 +67,44 @@ def test_pack_bit_exact_scatter_masked_and_strided(bits, gs):
     assert bool((data[:, T] == 0xA5).all())                       # the masked token wrote nothing
 
 
+@pytest.mark.parametrize("bits", (2, 3, 4))
+def test_pack_rounding_is_exact_for_every_mantissa_pair(bits):
+    """The pack kernel replaces the division by the scale with a reciprocal and one residual correction; this
+    sweeps every (group maximum, element) mantissa pair over the binades where the quotient can reach a code
+    boundary (ties included), at several magnitudes, and compares the bytes with the oracle's true division."""
+    gs = 64
+    qm = (1 << (bits - 1)) - 1
+    # elements: every bf16 value in [2^-5, 2), both signs, plus zero
+    mags = (np.arange(1 << 7, dtype=np.uint32)[None, :] | ((np.arange(122, 128, dtype=np.uint32)[:, None]) << 7)).reshape(-1)
+    elems = np.concatenate([mags, mags | 0x8000, [0]]).astype(np.uint16)
+    elems_f = O.bf16_bits_to_f32(elems)                                          # 1537 values, |x| < 2
+    rows = []
+    for e_a in (127, 128):                                                       # group maxima in [1, 4): scales in [1/qm, 4/qm)
+        for m_a in range(128):
+            a = O.bf16_bits_to_f32(np.array([(e_a << 7) | m_a], dtype=np.uint16))[0]
+            vals = elems_f[np.abs(elems_f) <= a]
+            pad = (-len(vals)) % (gs - 1)
+            vals = np.concatenate([vals, np.zeros(pad, np.float32)]).reshape(-1, gs - 1)
+            grp = np.concatenate([np.full((len(vals), 1), a, np.float32), vals], axis=1)   # (n, 64): maximum first
+            if len(grp) % 2:
+                grp = np.concatenate([grp, grp[:1]])
+            rows.append(grp.reshape(-1, 128))
+    base = np.concatenate(rows)                                                  # (T0, 128)
+    xs = [base * np.float32(sc) for sc in (1.0, 2.0 ** -9, 2.0 ** 11, 3.0)]      # x3: other scale mantissas after bf16 rounding
+    xn = O.bf16_round(np.concatenate(xs)).astype(np.float32)[:, None, :]         # (T, 1, 128)
+    T = xn.shape[0]
+    P = 128 * bits // 8
+    data = torch.zeros(1, T, P, dtype=torch.uint8, device="cuda")
+    scales = torch.zeros(1, T, 128 // gs, dtype=torch.bfloat16, device="cuda")
+    slots = torch.arange(T, dtype=torch.int64, device="cuda")
+    getattr(ops(), f"fused_quant_write_int{bits}_sym")(bf16_tensor(xn).cuda(), slots, data, scales, gs)
+    ref_d, ref_s = O.quantize_and_pack(xn, gs, bits)
+    assert np.array_equal(bf16_to_bits(scales)[0], ref_s[:, 0])
+    assert np.array_equal(data.cpu().numpy()[0], ref_d[:, 0])
+    codes = O.decode_codes(ref_d[:, 0], bits)
+    assert codes.min() == 1 and codes.max() == 2 * qm + 1                        # both ends of the code range occur
+
+
 def test_pack_int4_kv_single_launch_matches_two_launches():
     rng = np.random.default_rng(7)
     T, H = 70, 8
