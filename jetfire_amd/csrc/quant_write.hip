@@ -107,16 +107,17 @@ __global__ __launch_bounds__(256) void quant_write16_kernel(RowSrc s0, RowDst d0
   const int64_t tq = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
   const int h = blockIdx.y;
   const int which = blockIdx.z;
-  // rows past the end and masked rows still take part in the cross-lane steps (with zeros)
-  bool live = tq < T;
-  const int64_t t = live ? tq : 0;
+  // rows past the end still take part in the cross-lane steps (they re-read row 0); the row is requested
+  // without waiting for its slot, so the two loads are in flight together; masked rows (slot < 0) only skip
+  // the stores
+  const bool inside = tq < T;
+  const int64_t t = inside ? tq : 0;
   const int64_t slot = slots[t];
-  live = live && slot >= 0;
   const RowSrc& s = which ? s1 : s0;
   const RowDst& d = which ? d1 : d0;
   const uint16_t* xrow = s.x + t * s.stride_t + (int64_t)h * s.stride_h;
-  uint4 raw = make_uint4(0u, 0u, 0u, 0u);
-  if (live) raw = reinterpret_cast<const uint4*>(xrow)[l16];
+  const uint4 raw = reinterpret_cast<const uint4*>(xrow)[l16];
+  const bool live = inside && slot >= 0;
   float x[8];
   x[0] = bf16_to_f32((uint16_t)(raw.x & 0xffffu)); x[1] = bf16_to_f32((uint16_t)(raw.x >> 16));
   x[2] = bf16_to_f32((uint16_t)(raw.y & 0xffffu)); x[3] = bf16_to_f32((uint16_t)(raw.y >> 16));
