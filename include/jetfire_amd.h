@@ -179,10 +179,16 @@ int jf_get_cpu_attn_threads(void);
 /* Pinned hand-off context: replaces create_cpu_topk_submit_ctx / stream_submit_cpu_topk_attn /
  * stream_wait_cpu_topk_attn (jetfire_vllm/csrc/cpu_topk_attn.cpp:2054-2163, 2239, 2302) and the
  * pinned copies around them (jetfire_vllm/adapter/decode_path.py:2243-2267, 3107-3114).
- * submit: async D2H of q and topk_slots into pinned buffers, then a stream-ordered host function that
- *         starts the CPU correction on the worker pool and returns.
- * wait:   a stream-ordered host function that joins the CPU job, then async H2D of o_new into
- *         o_new_dev.  Only one job per context may be in flight. */
+ * submit: enqueues one small kernel on `stream` that copies q and topk_slots (both 16-byte aligned,
+ *         K even) into pinned host buffers and then raises a sequence flag in pinned memory; a
+ *         dispatcher thread of the context polls that flag and runs the CPU correction on the worker
+ *         pool as soon as the GPU has reached it.  Returns at once.
+ * wait:   blocks the calling host thread until the correction of the last submit has finished (as the
+ *         reference blocks on its future; JETFIRE_CPU_FUTURE_TIMEOUT_S, default 30 s, then
+ *         JF_ERR_TIMEOUT), then enqueues a small kernel on `stream` that brings o_new from the pinned
+ *         buffer into o_new_dev (16-byte aligned).  Not capturable into a HIP graph.
+ * One job per context may be in flight: a second submit before wait is rejected.  Leave two host cores
+ * to the caller and the dispatcher when sizing the worker pool (jf_set_cpu_attn_threads). */
 typedef struct jf_handoff jf_handoff;
 jf_handoff* jf_handoff_create(int B, int H_q, int H_kv, int K, int64_t num_slots,
                               const uint16_t* k_shadow_host, const uint16_t* v_shadow_host, float scale);

@@ -374,6 +374,13 @@ extern "C" int jf_cpu_topk_attn(const uint16_t* q, const uint16_t* k_shadow, con
 }
 
 // ------------------------------------------------------------------ pinned hand-off
+// submit: one small kernel, in stream order behind the merge, copies q and the winners' slots into pinned
+// host memory and then raises a sequence flag there (last workgroup, after a system-scope fence).  A
+// dispatcher thread of the context polls the flag while a submit is outstanding (it sleeps on a condition
+// variable otherwise), runs the correction on the worker pool and publishes the finished sequence number.
+// wait: the calling host thread waits for that number (the reference blocks on its future the same way,
+// decode_path.py:3082-3114) and then enqueues a small kernel that brings o_new from the pinned buffer to the
+// device.  No stream callbacks and no hipMemcpyAsync: on this runtime each costs tens of microseconds per layer.
 struct jf_handoff {
   int B, H_q, H_kv, K;
   int64_t num_slots;
@@ -382,37 +389,92 @@ struct jf_handoff {
   uint16_t* q_pin = nullptr;       // (B, H_q, D) bf16
   int64_t* ts_pin = nullptr;       // (B, H_q, K)
   uint16_t* o_pin = nullptr;       // (B, H_q, D) bf16
+  int64_t* flag_pin = nullptr;     // [0]: sequence number of the last published (q, slots)
+  unsigned* counter_dev = nullptr; // workgroups of the publish kernel that have finished
   std::vector<int64_t> head_map;   // (B, H_q, K)
   std::atomic<int64_t> submits{0};
-  std::atomic<int> in_flight{0};
+  std::atomic<int64_t> host_seq{0};  // submits enqueued by the host
+  std::atomic<int64_t> done_seq{0};  // corrections finished by the dispatcher
   std::atomic<int> failed{0};
+  std::atomic<int> stop{0};
+  std::mutex mu;
+  std::condition_variable cv;
+  std::thread dispatcher;
   double timeout_s = 30.0;         // JETFIRE_CPU_FUTURE_TIMEOUT_S in the reference (decode_path.py:3082-3098)
 };
 
-static void handoff_submit_cb(void* p) {
-  jf_handoff* h = static_cast<jf_handoff*>(p);
-  CpuJob j{h->q_pin, h->k_shadow, h->v_shadow, h->head_map.data(), h->ts_pin, h->o_pin,
-           h->B, h->H_q, h->K, h->H_kv, h->num_slots, h->scale};
-  // Never block inside a stream callback for long: the pool is single-flight, so wait our turn briefly.
-  int tries = 0;
-  while (!Pool::instance().start((int64_t)h->B * h->H_q, [j](int64_t b, int64_t e) { run_rows(j, b, e); })) {
-    std::this_thread::yield();
-    if (++tries > 1000000) { h->failed.store(1); return; }
+namespace {
+
+__global__ __launch_bounds__(256) void handoff_publish_kernel(const uint4* __restrict__ q_src, uint4* q_dst, int nq16,
+                                                              const uint4* __restrict__ s_src, uint4* s_dst, int ns16,
+                                                              unsigned* counter, int64_t* flag, int64_t seq) {
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < nq16 + ns16; i += gridDim.x * blockDim.x) {
+    if (i < nq16) q_dst[i] = q_src[i];
+    else s_dst[i - nq16] = s_src[i - nq16];
   }
-  h->submits.fetch_add(1, std::memory_order_relaxed);
-  h->in_flight.store(1, std::memory_order_release);
+  __threadfence_system();  // this thread's stores to host memory are ordered before the counter update
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const unsigned done = atomicAdd(counter, 1u);
+    if (done == gridDim.x - 1) {  // every workgroup's stores are out: raise the flag
+      *counter = 0u;
+      __threadfence_system();
+      __hip_atomic_store(flag, seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+  }
 }
 
-static void handoff_wait_cb(void* p) {
-  jf_handoff* h = static_cast<jf_handoff*>(p);
-  if (h->in_flight.load(std::memory_order_acquire) == 0) return;
-  if (!Pool::instance().join(h->timeout_s)) h->failed.store(1);
-  h->in_flight.store(0, std::memory_order_release);
+__global__ __launch_bounds__(256) void handoff_fetch_kernel(const uint4* __restrict__ src, uint4* dst, int n16) {
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += gridDim.x * blockDim.x) dst[i] = src[i];
 }
+
+inline void cpu_relax() {
+#if defined(__x86_64__)
+  _mm_pause();
+#endif
+}
+
+void handoff_dispatch(jf_handoff* h) {
+  int64_t seen = 0;
+  for (;;) {
+    {  // nothing outstanding: sleep until a submit (or the end)
+      std::unique_lock<std::mutex> lk(h->mu);
+      h->cv.wait(lk, [&] { return h->stop.load() || h->host_seq.load() > seen; });
+    }
+    if (h->stop.load()) return;
+    // a submit is in the stream: poll the flag the publish kernel raises
+    const auto t0 = std::chrono::steady_clock::now();
+    int64_t f = seen;
+    for (uint64_t spin = 0;; ++spin) {
+      f = __atomic_load_n(h->flag_pin, __ATOMIC_ACQUIRE);
+      if (f != seen || h->stop.load(std::memory_order_relaxed)) break;
+      cpu_relax();
+      if ((spin & 0xfff) == 0xfff) {
+        const double el = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+        if (el > h->timeout_s) { h->failed.store(1); break; }
+        if (el > 0.002) std::this_thread::sleep_for(std::chrono::microseconds(50));  // a long GPU queue: stop burning a core
+      }
+    }
+    if (h->stop.load()) return;
+    if (f == seen) {  // timed out: give up on the outstanding submits
+      seen = h->host_seq.load();
+      h->done_seq.store(seen, std::memory_order_release);
+      continue;
+    }
+    seen = f;
+    CpuJob j{h->q_pin, h->k_shadow, h->v_shadow, h->head_map.data(), h->ts_pin, h->o_pin,
+             h->B, h->H_q, h->K, h->H_kv, h->num_slots, h->scale};
+    if (!Pool::instance().run((int64_t)h->B * h->H_q, [j](int64_t b, int64_t e) { run_rows(j, b, e); })) h->failed.store(1);
+    h->submits.fetch_add(1, std::memory_order_relaxed);
+    h->done_seq.store(seen, std::memory_order_release);
+  }
+}
+
+}  // namespace
 
 extern "C" jf_handoff* jf_handoff_create(int B, int H_q, int H_kv, int K, int64_t num_slots,
                                          const uint16_t* k_shadow_host, const uint16_t* v_shadow_host, float scale) {
-  if (B <= 0 || H_q <= 0 || H_kv <= 0 || K <= 0 || num_slots <= 0 || H_q % H_kv != 0 || !k_shadow_host || !v_shadow_host) {
+  if (B <= 0 || H_q <= 0 || H_kv <= 0 || K <= 0 || K % 2 != 0 || num_slots <= 0 || H_q % H_kv != 0 || !k_shadow_host || !v_shadow_host) {
     set_error("handoff_create: bad arguments");
     return nullptr;
   }
@@ -426,35 +488,65 @@ extern "C" jf_handoff* jf_handoff_create(int B, int H_q, int H_kv, int K, int64_
   const size_t nq = (size_t)B * H_q * D * sizeof(uint16_t), nt = (size_t)B * H_q * K * sizeof(int64_t);
   if (hipHostMalloc((void**)&h->q_pin, nq, hipHostMallocDefault) != hipSuccess ||
       hipHostMalloc((void**)&h->ts_pin, nt, hipHostMallocDefault) != hipSuccess ||
-      hipHostMalloc((void**)&h->o_pin, nq, hipHostMallocDefault) != hipSuccess) {
-    set_error("handoff_create: hipHostMalloc failed");
+      hipHostMalloc((void**)&h->o_pin, nq, hipHostMallocDefault) != hipSuccess ||
+      hipHostMalloc((void**)&h->flag_pin, 64, hipHostMallocDefault) != hipSuccess ||
+      hipMalloc((void**)&h->counter_dev, 64) != hipSuccess || hipMemset(h->counter_dev, 0, 64) != hipSuccess) {
+    set_error("handoff_create: allocation failed");
     jf_handoff_destroy(h);
     return nullptr;
   }
+  h->flag_pin[0] = 0;
   const int G = H_q / H_kv;
   h->head_map.resize((size_t)B * H_q * K);
   for (int b = 0; b < B; ++b)
     for (int hq = 0; hq < H_q; ++hq)
       for (int k = 0; k < K; ++k) h->head_map[((size_t)b * H_q + hq) * K + k] = hq / G;  // decode_path.py:400-408
+  h->dispatcher = std::thread(handoff_dispatch, h);
   return h;
 }
 
 extern "C" int jf_handoff_submit(jf_handoff* h, const uint16_t* q_dev, const int64_t* topk_slots_dev, void* stream) {
   JF_CHECK_ARG(h && q_dev && topk_slots_dev, "handoff_submit: null argument");
+  JF_CHECK_ARG(((uintptr_t)q_dev & 15) == 0 && ((uintptr_t)topk_slots_dev & 15) == 0, "handoff_submit: q and topk_slots must be 16-byte aligned");
   if (h->failed.load()) { set_error("handoff: an earlier CPU correction job failed or timed out"); return JF_ERR_TIMEOUT; }
+  JF_CHECK_ARG(h->host_seq.load() == h->done_seq.load(), "handoff_submit: the previous submit has not been waited for");
   hipStream_t st = (hipStream_t)stream;
-  JF_CHECK_HIP(hipMemcpyAsync(h->q_pin, q_dev, (size_t)h->B * h->H_q * D * sizeof(uint16_t), hipMemcpyDeviceToHost, st));
-  JF_CHECK_HIP(hipMemcpyAsync(h->ts_pin, topk_slots_dev, (size_t)h->B * h->H_q * h->K * sizeof(int64_t), hipMemcpyDeviceToHost, st));
-  JF_CHECK_HIP(hipLaunchHostFunc(st, handoff_submit_cb, h));
+  const int nq16 = (int)((size_t)h->B * h->H_q * D * sizeof(uint16_t) / 16);
+  const int ns16 = (int)((size_t)h->B * h->H_q * h->K * sizeof(int64_t) / 16);
+  const int64_t seq = h->host_seq.load() + 1;
+  int blocks = (nq16 + ns16 + 255) / 256;
+  if (blocks > 32) blocks = 32;
+  hipLaunchKernelGGL(handoff_publish_kernel, dim3(blocks), dim3(256), 0, st, reinterpret_cast<const uint4*>(q_dev),
+                     reinterpret_cast<uint4*>(h->q_pin), nq16, reinterpret_cast<const uint4*>(topk_slots_dev),
+                     reinterpret_cast<uint4*>(h->ts_pin), ns16, h->counter_dev, h->flag_pin, seq);
+  JF_CHECK_HIP(hipGetLastError());
+  {
+    std::lock_guard<std::mutex> g(h->mu);
+    h->host_seq.store(seq);
+  }
+  h->cv.notify_one();
   return JF_OK;
 }
 
 extern "C" int jf_handoff_wait(jf_handoff* h, uint16_t* o_new_dev, void* stream) {
   JF_CHECK_ARG(h && o_new_dev, "handoff_wait: null argument");
+  JF_CHECK_ARG(((uintptr_t)o_new_dev & 15) == 0, "handoff_wait: o_new must be 16-byte aligned");
   hipStream_t st = (hipStream_t)stream;
-  JF_CHECK_HIP(hipLaunchHostFunc(st, handoff_wait_cb, h));
-  JF_CHECK_HIP(hipMemcpyAsync(o_new_dev, h->o_pin, (size_t)h->B * h->H_q * D * sizeof(uint16_t), hipMemcpyHostToDevice, st));
+  const int64_t want = h->host_seq.load();
+  const auto t0 = std::chrono::steady_clock::now();
+  for (uint64_t spin = 0; h->done_seq.load(std::memory_order_acquire) < want; ++spin) {
+    cpu_relax();
+    if ((spin & 0xfff) == 0xfff) {
+      const double el = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+      if (el > h->timeout_s + 1.0) { h->failed.store(1); break; }
+      if (el > 0.002) std::this_thread::sleep_for(std::chrono::microseconds(50));
+    }
+  }
   if (h->failed.load()) { set_error("handoff: CPU correction job failed or timed out"); return JF_ERR_TIMEOUT; }
+  const int n16 = (int)((size_t)h->B * h->H_q * D * sizeof(uint16_t) / 16);
+  hipLaunchKernelGGL(handoff_fetch_kernel, dim3((n16 + 255) / 256 < 8 ? (n16 + 255) / 256 : 8), dim3(256), 0, st,
+                     reinterpret_cast<const uint4*>(h->o_pin), reinterpret_cast<uint4*>(o_new_dev), n16);
+  JF_CHECK_HIP(hipGetLastError());
   return JF_OK;
 }
 
@@ -462,9 +554,16 @@ extern "C" int64_t jf_handoff_submit_count(const jf_handoff* h) { return h ? h->
 
 extern "C" void jf_handoff_destroy(jf_handoff* h) {
   if (!h) return;
-  if (h->in_flight.load(std::memory_order_acquire)) Pool::instance().join(h->timeout_s);
+  {
+    std::lock_guard<std::mutex> g(h->mu);
+    h->stop.store(1);
+  }
+  h->cv.notify_all();
+  if (h->dispatcher.joinable()) h->dispatcher.join();
   if (h->q_pin) (void)hipHostFree(h->q_pin);
   if (h->ts_pin) (void)hipHostFree(h->ts_pin);
   if (h->o_pin) (void)hipHostFree(h->o_pin);
+  if (h->flag_pin) (void)hipHostFree(h->flag_pin);
+  if (h->counter_dev) (void)hipFree(h->counter_dev);
   delete h;
 }
