@@ -60,6 +60,10 @@ class Pool {
     n_ = n;
     const int w = (int)workers_.size();
     active_ = w;
+    // rows are handed out in small chunks from a shared counter: a worker that loses its core for a while
+    // simply takes fewer of them
+    chunk_ = std::max<int64_t>(1, n / ((int64_t)w * 8));
+    next_.store(0, std::memory_order_relaxed);
     remaining_.store(w, std::memory_order_release);
     epoch_.fetch_add(1, std::memory_order_acq_rel);
     lk.unlock();
@@ -111,8 +115,11 @@ class Pool {
       const int n = std::atoi(e);
       if (n > 0) return n;
     }
+    // default: all cores but two (the thread that launches the GPU work and the hand-off's dispatcher spin
+    // while a layer is in flight; workers that share a core with them stretch every job)
     unsigned hc = std::thread::hardware_concurrency();
     if (hc == 0) hc = 1;
+    if (hc > 4) hc -= 2;
     return (int)(hc < 64 ? hc : 64);
   }
   void ensure_workers() {
@@ -139,20 +146,24 @@ class Pool {
   }
   void worker(int id, uint64_t seen) {
     for (;;) {
-      // spin briefly for the next epoch, then sleep
+      // spin for the next epoch for about half a millisecond (the gap between two layers of a decode step is
+      // shorter than a futex wake-up of the whole pool), then sleep
       bool got = false;
-      for (int spin = 0; spin < 4000; ++spin) {
+      const auto t0 = std::chrono::steady_clock::now();
+      for (uint32_t spin = 0;; ++spin) {
         if (epoch_.load(std::memory_order_acquire) != seen) { got = true; break; }
 #if defined(__x86_64__)
         _mm_pause();
 #endif
+        if ((spin & 0x3ff) == 0x3ff &&
+            std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() > 500e-6) break;
       }
       if (!got) {
         std::unique_lock<std::mutex> lk(mu_);
         cv_work_.wait(lk, [&] { return epoch_.load(std::memory_order_acquire) != seen; });
       }
       std::function<void(int64_t, int64_t)> fn;
-      int64_t n;
+      int64_t n, chunk;
       int w;
       {
         std::lock_guard<std::mutex> g(mu_);
@@ -161,11 +172,14 @@ class Pool {
         fn = fn_;
         n = n_;
         w = active_;
+        chunk = chunk_;
       }
       if (fn && id < w) {
-        const int64_t per = (n + w - 1) / w;
-        const int64_t b = (int64_t)id * per, e = std::min<int64_t>(n, b + per);
-        if (b < e) fn(b, e);
+        for (;;) {
+          const int64_t b = next_.fetch_add(chunk, std::memory_order_relaxed);
+          if (b >= n) break;
+          fn(b, std::min<int64_t>(n, b + chunk));
+        }
         if (remaining_.fetch_sub(1, std::memory_order_acq_rel) == 1) {
           std::lock_guard<std::mutex> g(mu_);
           cv_done_.notify_all();
@@ -178,7 +192,8 @@ class Pool {
   std::condition_variable cv_work_, cv_done_;
   std::vector<std::thread> workers_;
   std::function<void(int64_t, int64_t)> fn_;
-  int64_t n_ = 0;
+  int64_t n_ = 0, chunk_ = 1;
+  std::atomic<int64_t> next_{0};
   int active_ = 0;
   int override_ = 0;
   bool busy_ = false, stop_ = false;
@@ -332,7 +347,8 @@ struct CpuJob {
 };
 
 static void run_rows(const CpuJob& j, int64_t b, int64_t e) {
-  std::vector<float> buf((size_t)j.K);
+  static thread_local std::vector<float> buf;
+  if (buf.size() < (size_t)j.K) buf.resize((size_t)j.K);
 #if defined(__x86_64__)
   if (host_has_avx2_fma()) {
     for (int64_t r = b; r < e; ++r)
