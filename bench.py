@@ -101,10 +101,17 @@ def main() -> int:
     if args.calibrate_copy:
         src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").random_(0, 255)
         dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
         for _ in range(10):
             dst.copy_(src)
+        e1.record()
         torch.cuda.synchronize()
-        print(json.dumps({"calibrate_copy_bytes_read": 1 << 30, "calibrate_copy_bytes_written": 1 << 30, "launches": 10}))
+        us = e0.elapsed_time(e1) * 100.0       # per copy
+        print(json.dumps({"calibrate_copy_bytes_read": 1 << 30, "calibrate_copy_bytes_written": 1 << 30, "launches": 11,
+                          "us_per_copy": round(us, 1), "copy_read_plus_write_GBps": round(2 * (1 << 30) / us / 1e3, 1)}))
         return 0
     if args.split_len:
         _lib.check(lib.jf_debug_split_len(args.split_len))
