@@ -1229,7 +1229,7 @@ constexpr int MG_BT_LDS = 4096;    // block-table entries cached in LDS (65536 p
 // Launch 2: one workgroup per (sequence, query head).
 //   1. split statistics -> M, l, o_hat
 //   2. the K-th largest candidate key tau (and how many keys equal to tau still belong to the top K): the
-//      candidates are dropped into MG_BINS linear score buckets between the smallest candidate and M, a scan
+//      candidates are dropped into MG_BINS linear score buckets between the smallest and the largest, a scan
 //      finds the bucket that holds the K-th largest, and the few members of that bucket are ranked against
 //      each other (a bisection over the key range covers the case of more than MG_LIST members)
 //   3. ordered compaction of the winners (key > tau, or key == tau while the quota lasts; candidates are stored
@@ -1237,8 +1237,9 @@ constexpr int MG_BT_LDS = 4096;    // block-table entries cached in LDS (65536 p
 //   4. slots, softmax weights, and the pre-correction terms over the winners' V rows.
 // The first MG_REGK * MG_THREADS candidates stay in registers from a single load; anything beyond that is
 // re-read from global memory in every pass.
-// Two shapes: 512 threads x 16 register-resident candidates each (up to 8192 candidates, the common case)
-// and 1024 x 32 for long contexts with wide top-k.
+// Two shapes: 1024 threads x 8 register-resident candidates each (up to 8192 candidates, the common case;
+// the phases are chains of LDS round trips and barriers, so more, lighter threads beat fewer, heavier ones)
+// and 1024 x 32 for first-stage parts that exceed it.
 // PARTIAL = true is the first stage of the two-stage merge: blockIdx.z selects a run of mg_spp candidate
 // lists, steps 2 and 3 run on those alone and the winners (still in position order) are written out as one
 // new candidate list; the final merge (PARTIAL = false, mg_parts > 1) reads these lists instead of the
