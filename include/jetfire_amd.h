@@ -187,7 +187,8 @@ int jf_get_cpu_attn_threads(void);
  *         reference blocks on its future; JETFIRE_CPU_FUTURE_TIMEOUT_S, default 30 s, then
  *         JF_ERR_TIMEOUT), then enqueues a small kernel on `stream` that brings o_new from the pinned
  *         buffer into o_new_dev (16-byte aligned).  Not capturable into a HIP graph.
- * One job per context may be in flight: a second submit before wait is rejected.  Leave two host cores
+ * One job per context may be in flight: a submit while the previous correction still runs is rejected
+ * (JF_ERR_ARG); destroy waits for an outstanding one.  Leave two host cores
  * to the caller and the dispatcher when sizing the worker pool (jf_set_cpu_attn_threads). */
 typedef struct jf_handoff jf_handoff;
 jf_handoff* jf_handoff_create(int B, int H_q, int H_kv, int K, int64_t num_slots,

@@ -525,7 +525,7 @@ extern "C" int jf_handoff_submit(jf_handoff* h, const uint16_t* q_dev, const int
   JF_CHECK_ARG(h && q_dev && topk_slots_dev, "handoff_submit: null argument");
   JF_CHECK_ARG(((uintptr_t)q_dev & 15) == 0 && ((uintptr_t)topk_slots_dev & 15) == 0, "handoff_submit: q and topk_slots must be 16-byte aligned");
   if (h->failed.load()) { set_error("handoff: an earlier CPU correction job failed or timed out"); return JF_ERR_TIMEOUT; }
-  JF_CHECK_ARG(h->host_seq.load() == h->done_seq.load(), "handoff_submit: the previous submit has not been waited for");
+  JF_CHECK_ARG(h->host_seq.load() == h->done_seq.load(), "handoff_submit: the previous correction is still in flight (wait for it first)");
   hipStream_t st = (hipStream_t)stream;
   const int nq16 = (int)((size_t)h->B * h->H_q * D * sizeof(uint16_t) / 16);
   const int ns16 = (int)((size_t)h->B * h->H_q * h->K * sizeof(int64_t) / 16);
@@ -570,6 +570,14 @@ extern "C" int64_t jf_handoff_submit_count(const jf_handoff* h) { return h ? h->
 
 extern "C" void jf_handoff_destroy(jf_handoff* h) {
   if (!h) return;
+  // a submit that was never waited for: its kernel still writes the pinned buffers and its job reads them
+  if (h->dispatcher.joinable() && !h->failed.load()) {
+    const auto t0 = std::chrono::steady_clock::now();
+    while (h->done_seq.load(std::memory_order_acquire) < h->host_seq.load()) {
+      std::this_thread::sleep_for(std::chrono::microseconds(100));
+      if (std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() > h->timeout_s + 1.0) break;
+    }
+  }
   {
     std::lock_guard<std::mutex> g(h->mu);
     h->stop.store(1);

@@ -316,3 +316,28 @@ def test_split_pipeline_with_handoff(scheme, B, Hq, Hkv, lens, K):
     err = np.abs(got - r["out"])
     assert err.max() <= 2e-2 and err.mean() <= 1e-3               # the acceptance bar for attention outputs
     h.close()
+
+
+def test_handoff_protocol_edges():
+    """wait without a submit returns at once; closing a context with a submit that was never waited for lets
+    the job finish first."""
+    B, Hq, Hkv, K, S = 1, 8, 2, 32, 64
+    c = make_case(77, B, Hq, Hkv, S, 3, 2, 64)
+    d = to_device(c)
+    o = ops()
+    ksh, vsh = bf16_tensor(c["K"]), bf16_tensor(c["V"])
+    o.set_cpu_attn_threads(2)
+    scale = 128 ** -0.5
+    _, idx, slots = o.int3_qk_scores_topk(d["q"], d["kd"], d["ks"], d["bt"], d["lens"], S, Hq, Hkv, 16, scale, K)
+    o_new = torch.zeros(B, Hq, 128, dtype=torch.bfloat16, device="cuda")
+    h = o.CpuTopkHandoff(B, Hq, Hkv, K, ksh, vsh, scale)
+    h.wait(o_new)                                                 # nothing outstanding
+    h.submit(d["q"], slots)
+    h.wait(o_new)
+    torch.cuda.synchronize()
+    ref = O.cpu_topk_attn(c["q"], c["K"], c["V"], O.head_map(B, Hq, Hq // Hkv, K), slots.cpu().numpy(), scale)
+    np.testing.assert_allclose(bf16_to_f32(o_new), ref, atol=2e-3, rtol=6e-3)
+    assert h.submit_count == 1
+    h.submit(d["q"], slots)                                       # left outstanding on purpose
+    h.close()                                                     # must wait for the job, then free
+    torch.cuda.synchronize()
