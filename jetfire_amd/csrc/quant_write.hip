@@ -202,7 +202,8 @@ inline bool rows_16b_aligned(const void* x, int64_t stride_t, int64_t stride_h) 
 
 int check_common(const void* x, const int64_t* slots, int64_t T, int H_kv, int group_size,
                  int64_t data_stride_slot, int nbits, const void* data, const void* scale) {
-  JF_CHECK_ARG(T >= 0 && H_kv > 0, "quant_write: bad T=%lld H_kv=%d", (long long)T, H_kv);
+  JF_CHECK_ARG(T >= 0 && H_kv > 0 && H_kv <= 65535, "quant_write: bad T=%lld H_kv=%d", (long long)T, H_kv);
+  JF_CHECK_ARG(T <= (int64_t)16 * 0x7fffffff, "quant_write: T=%lld exceeds the launch grid", (long long)T);
   JF_CHECK_ARG(group_size == 32 || group_size == 64 || group_size == 128,
                "quant_write: group_size must be 32, 64 or 128 (got %d)", group_size);
   JF_CHECK_ARG(nbits == 2 || nbits == 3 || nbits == 4, "quant_write: nbits must be 2, 3 or 4 (got %d)", nbits);
