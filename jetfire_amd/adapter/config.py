@@ -1,0 +1,77 @@
+"""Runtime configuration of the adapter (the part of `jetfire_vllm/adapter/config.py:91-163` the decode path
+reads): quantisation scheme, group size, correction width, switches.  Values come from the environment
+variables the reference uses, and can be replaced programmatically with `set_jetfire_config`."""
+from __future__ import annotations
+
+import os
+from dataclasses import dataclass, replace
+
+
+@dataclass(frozen=True)
+class QuantScheme:
+    name: str
+    k_nbits: int
+    v_nbits: int
+    k_asymmetric: bool = False
+    v_asymmetric: bool = False
+    default_group_size: int = 128
+
+
+# the two schemes this library implements (jetfire_vllm/artifact.py:59 gives their group sizes)
+SCHEMES = {
+    "SymInt3K_SymInt2V": QuantScheme("SymInt3K_SymInt2V", 3, 2, default_group_size=64),
+    "SymInt4K_SymInt4V": QuantScheme("SymInt4K_SymInt4V", 4, 4, default_group_size=128),
+}
+
+
+@dataclass(frozen=True)
+class JetFireConfig:
+    scheme: QuantScheme = SCHEMES["SymInt3K_SymInt2V"]
+    group_size: int = 64
+    topk: int = 256
+    layer_stride: int = 1
+    use_custom_backend: bool = True
+    cpu_correction: bool = True
+    shadow_enabled: bool = True
+    max_batch_size: int = 0
+    cpu_attn_threads: int = 0          # 0: the pool's default (all cores but two)
+    debug_log: bool = False
+
+
+_CONFIG: JetFireConfig | None = None
+
+
+def _from_env() -> JetFireConfig:
+    name = os.environ.get("JETFIRE_QUANT_SCHEME", "SymInt3K_SymInt2V")
+    if name not in SCHEMES:
+        raise ValueError(f"JETFIRE_QUANT_SCHEME={name!r} is not one of {sorted(SCHEMES)}")
+    scheme = SCHEMES[name]
+    return JetFireConfig(
+        scheme=scheme,
+        group_size=int(os.environ.get("JETFIRE_GROUP_SIZE", scheme.default_group_size)),
+        topk=int(os.environ.get("JETFIRE_TOPK", 256)),
+        layer_stride=int(os.environ.get("JETFIRE_LAYER_STRIDE", 1)),
+        use_custom_backend=os.environ.get("JETFIRE_USE_CUSTOM_BACKEND", "1") == "1",
+        cpu_correction=os.environ.get("JETFIRE_CPU_CORRECTION", "1") == "1",
+        shadow_enabled=os.environ.get("JETFIRE_SHADOW", "1") == "1",
+        max_batch_size=int(os.environ.get("JETFIRE_MAX_BATCH_SIZE", 0)),
+        cpu_attn_threads=int(os.environ.get("JETFIRE_CPU_ATTN_THREADS", 0)),
+        debug_log=os.environ.get("JETFIRE_DEBUG", "0") == "1",
+    )
+
+
+def get_jetfire_config() -> JetFireConfig:
+    global _CONFIG
+    if _CONFIG is None:
+        _CONFIG = _from_env()
+    return _CONFIG
+
+
+def set_jetfire_config(**changes) -> JetFireConfig:
+    """Replace fields of the active configuration (`scheme` may be given by name).  Existing pool managers
+    keep the configuration they were created with: reset the global manager afterwards."""
+    global _CONFIG
+    if isinstance(changes.get("scheme"), str):
+        changes["scheme"] = SCHEMES[changes["scheme"]]
+    _CONFIG = replace(get_jetfire_config(), **changes)
+    return _CONFIG

@@ -1,0 +1,176 @@
+"""Adapter glue: top-k width selection, dispatcher gate, pool registry (CPU), and a multi-step decode through
+`mirror_kv` + `try_jetfire_decode` against the oracle (GPU)."""
+import types
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import jetfire_oracle as O
+from tests.helpers import bf16_tensor, bf16_to_bits, bf16_to_f32
+
+
+@pytest.fixture
+def adapter():
+    import jetfire_amd.adapter as A
+    from jetfire_amd.adapter import decode_path
+    A.reset_global_kv_pool_manager()
+    yield A
+    decode_path.reset_jetfire_decode_runtime_state()
+    A.reset_global_kv_pool_manager()
+    A.set_jetfire_config(scheme="SymInt3K_SymInt2V", group_size=64, topk=256, use_custom_backend=True,
+                         cpu_correction=True, layer_stride=1)
+
+
+def test_select_top_k_matches_the_reference_table(adapter):
+    from jetfire_amd.adapter.decode_path import FUSED_SUPPORTED_TOP_K, _get_head_map_cpu, _select_top_k
+    supported = (32, 64, 128, 256, 512, 1024)
+    for req in (16, 32, 100, 256, 300, 1024, 5000):
+        for n in (0, 1, 31, 32, 33, 255, 256, 257, 4096):
+            assert _select_top_k(req, n, supported) == O.select_top_k(req, n, supported), (req, n)
+    assert FUSED_SUPPORTED_TOP_K == supported
+    hm = _get_head_map_cpu(2, 8, 4, 5).numpy()
+    assert np.array_equal(hm, O.head_map(2, 8, 4, 5))
+
+
+def _meta(seq_lens, block_table, **kw):
+    d = dict(seq_lens=seq_lens, block_table=block_table, use_cascade=False, max_query_len=1,
+             num_actual_tokens=int(seq_lens.numel()), max_seq_len=int(seq_lens.max()) if seq_lens.numel() else 0)
+    d.update(kw)
+    return types.SimpleNamespace(**d)
+
+
+def test_dispatcher_gate_reasons(adapter):
+    from jetfire_amd.adapter.decode_path import _decode_unsupported
+    pool = adapter.get_global_kv_pool_manager()
+    impl = types.SimpleNamespace(attn_type=types.SimpleNamespace(name="DECODER"), scale=0.1)
+    layer = types.SimpleNamespace(layer_name="model.layers.0.attn", num_heads=8, num_kv_heads=2, head_size=128)
+    q = torch.zeros(2, 8 * 128)
+    meta = _meta(torch.tensor([5, 7], dtype=torch.int32), torch.zeros(2, 1, dtype=torch.int64))
+    gate = lambda **kw: _decode_unsupported(**{**dict(impl=impl, layer=layer, query=q.view(2, 8, 128), attn_metadata=meta), **kw})
+    assert gate() == "layer_config_missing"
+    pool.ensure_layer_config_from_layer(layer.layer_name, layer)
+    assert pool.get_layer_config(layer.layer_name) == adapter.JetFireLayerConfig(8, 2, 128)
+    assert gate() is None
+    assert gate(attn_metadata=None) == "profiling_run"
+    assert gate(impl=types.SimpleNamespace(attn_type=types.SimpleNamespace(name="ENCODER"))) == "attn_type"
+    assert gate(attn_metadata=_meta(meta.seq_lens, meta.block_table, use_cascade=True)) == "cascade"
+    assert gate(attn_metadata=_meta(meta.seq_lens, meta.block_table, max_query_len=4)) == "prefill_or_multi_query"
+    assert gate(attn_metadata=_meta(meta.seq_lens, meta.block_table, num_actual_tokens=3)) == "batch_mismatch"
+    assert gate(query=q.view(2, 8, 128)[:1]) == "empty_query"
+    assert gate(layer=types.SimpleNamespace()) == "layer_name_missing"
+    assert gate(query=torch.zeros(2, 8, 64)) == "head_dim_mismatch"
+    # a miss is counted under its reason and the entry returns None
+    out = torch.zeros(2, 8, 128)
+    assert adapter.try_jetfire_decode(impl=impl, layer=layer, query=q.view(2, 8, 128), attn_metadata=meta, output=out) is None
+    assert pool.get_stats()["decode_fallbacks"] == {"store_missing": 1} and pool.decode_attempts == 1
+
+
+def test_pool_registry_and_store_geometry(adapter):
+    adapter.set_jetfire_config(scheme="SymInt4K_SymInt4V", group_size=128, layer_stride=2)
+    adapter.reset_global_kv_pool_manager()
+    pool = adapter.get_global_kv_pool_manager()
+    assert (pool.config.k_nbits, pool.config.v_nbits, pool.config.group_size) == (4, 4, 128)
+    for i in range(3):
+        name = f"model.layers.{i}.attn"
+        pool.register_layer_config(name, num_query_heads=8, num_kv_heads=2, head_dim=128)
+        pool.register_layer_layout(name, num_blocks=6, block_size=16)
+    assert pool.ensure_all_layer_stores(device="cpu") == 2          # layer_stride 2: layers 0 and 2
+    store = pool.get_layer_store("model.layers.0.attn")
+    assert pool.get_layer_store("model.layers.1.attn") is None
+    assert store.k_data.shape == (2, 96, 64) and store.v_scales.shape == (2, 96, 1) and store.k_shadow.shape == (2, 96, 128)
+    assert store.scheme == "k4v4" and store.num_slots == 96
+    row = torch.tensor([4, 1, 3], dtype=torch.int64)
+    slots = store.sequence_slots(row, 20)
+    assert slots.tolist() == list(range(64, 80)) + [16, 17, 18, 19]
+    assert torch.equal(store.sequence_slots_fast(row, 20), slots)
+    assert not store.has_sequence(row, 20) and not store.fast_has_sequence(1)
+    with pytest.raises(ValueError):
+        store.sequence_slots(row, 0)
+    with pytest.raises(ValueError):
+        store.sequence_slots(torch.tensor([0, -1]), 20)
+    with pytest.raises(NotImplementedError):
+        adapter.JetFireInt4CacheStore(num_kv_heads=2, head_dim=128, group_size=64, num_blocks=1, block_size=16,
+                                      device="cpu", k_nbits=2, v_nbits=2, k_asymmetric=True, v_asymmetric=False)
+    pool.mirror_kv("model.layers.1.attn", torch.zeros(1, 2, 128), torch.zeros(1, 2, 128), torch.tensor([0]))
+    assert pool.skipped_layers == 1                                  # stride-skipped layer
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("scheme_name,scheme,gs,kb,vb", [("SymInt3K_SymInt2V", "k3v2", 64, 3, 2),
+                                                         ("SymInt4K_SymInt4V", "k4v4", 128, 4, 4)])
+def test_prefill_then_decode_steps_match_the_oracle(adapter, scheme_name, scheme, gs, kb, vb):
+    B, Hq, Hkv, D, bs = 3, 8, 2, 128, 16
+    lens0 = [300, 37, 512]
+    steps = 3
+    adapter.set_jetfire_config(scheme=scheme_name, group_size=gs, topk=64, layer_stride=1, cpu_attn_threads=4)
+    adapter.reset_global_kv_pool_manager()
+    pool = adapter.get_global_kv_pool_manager()
+    name = "model.layers.0.self_attn.attn"
+    layer = types.SimpleNamespace(layer_name=name, num_heads=Hq, num_kv_heads=Hkv, head_size=D)
+    impl = types.SimpleNamespace(attn_type=types.SimpleNamespace(name="DECODER"), scale=D ** -0.5)
+    rng = np.random.default_rng(5)
+    per_seq = (max(lens0) + steps + bs - 1) // bs
+    nblk = B * per_seq + 2
+    bt = rng.permutation(nblk)[:B * per_seq].reshape(B, per_seq).astype(np.int64)
+    pool.ensure_layer_config_from_layer(name, layer)
+    pool.register_layer_layout(name, num_blocks=nblk, block_size=bs)
+    bt_dev = torch.from_numpy(bt).cuda()
+
+    def slot_of(b, pos):
+        return int(bt[b, pos // bs]) * bs + pos % bs
+
+    def new_kv(n):
+        k = O.bf16_round(rng.standard_normal((n, Hkv, D)).astype(np.float32))
+        k[..., [3, 40, 77, 101]] *= 8
+        return O.bf16_round(k), O.bf16_round(rng.standard_normal((n, Hkv, D)).astype(np.float32))
+
+    # prefill: every sequence's tokens in one call, plus two padding tokens (slot -1) that must be ignored
+    toks = [(b, p) for b in range(B) for p in range(lens0[b])]
+    k_np, v_np = new_kv(len(toks) + 2)
+    slot_map = np.array([slot_of(b, p) for b, p in toks] + [-1, -1], dtype=np.int64)
+    pool.mirror_kv(name, bf16_tensor(k_np).cuda(), bf16_tensor(v_np).cuda(), torch.from_numpy(slot_map).cuda())
+    store = pool.get_layer_store(name)
+    Kfull = np.zeros((Hkv, nblk * bs, D), np.float32)
+    Vfull = np.zeros_like(Kfull)
+    Kfull[:, slot_map[:-2]] = k_np[:-2].transpose(1, 0, 2)
+    Vfull[:, slot_map[:-2]] = v_np[:-2].transpose(1, 0, 2)
+    lens = list(lens0)
+    for step in range(steps):
+        # append one token per sequence, then decode
+        k_np, v_np = new_kv(B)
+        slot_map = np.array([slot_of(b, lens[b]) for b in range(B)], dtype=np.int64)
+        pool.mirror_kv(name, bf16_tensor(k_np).cuda(), bf16_tensor(v_np).cuda(), torch.from_numpy(slot_map).cuda())
+        Kfull[:, slot_map] = k_np.transpose(1, 0, 2)
+        Vfull[:, slot_map] = v_np.transpose(1, 0, 2)
+        lens = [n + 1 for n in lens]
+        q_np = O.bf16_round((rng.standard_normal((B, Hq, D)) / np.sqrt(D)).astype(np.float32))
+        seq_lens = torch.tensor(lens, dtype=torch.int32, device="cuda")
+        meta = _meta(seq_lens, bt_dev)
+        out = torch.zeros(B + 1, Hq * D, dtype=torch.bfloat16, device="cuda")          # one spare row, as vLLM pads
+        got = adapter.try_jetfire_decode(impl=impl, layer=layer, query=bf16_tensor(q_np).cuda(), attn_metadata=meta, output=out)
+        assert got is out
+        torch.cuda.synchronize()
+        # the cache holds exactly what the oracle quantiser packs, the shadow the bf16 rows
+        filled = store.slot_filled.cpu().numpy()
+        ref_kd, ref_ks = O.quantize_and_pack(Kfull, gs, kb)
+        ref_vd, ref_vs = O.quantize_and_pack(Vfull, gs, vb)
+        assert np.array_equal(store.k_data.cpu().numpy()[:, filled], ref_kd[:, filled])
+        assert np.array_equal(bf16_to_bits(store.k_scales)[:, filled], ref_ks[:, filled])
+        assert np.array_equal(store.v_data.cpu().numpy()[:, filled], ref_vd[:, filled])
+        assert np.array_equal(bf16_to_f32(store.k_shadow)[:, filled], Kfull[:, filled])
+        r = O.decode_reference(q_np, ref_kd, ref_ks, ref_vd, ref_vs, bt, np.array(lens, np.int32), max(lens), Hq, Hkv, bs,
+                               D ** -0.5, 64, scheme, Kfull, Vfull)
+        res = bf16_to_f32(out[:B]).reshape(B, Hq, D)
+        np.testing.assert_allclose(res, r["out"], atol=6e-3, rtol=1.5e-2)                # validate_runtime.py:195
+        err = np.abs(res - r["out"])
+        assert err.max() <= 2e-2 and err.mean() <= 1e-3
+        assert float(out[B].float().abs().sum()) == 0.0
+    stats = pool.get_stats()
+    assert stats["decode_hits"] == steps and stats["decode_fallbacks"] == {}
+    assert stats["written_slots"] == sum(lens0) + 2 + steps * B
+    # a sequence whose rows were never written is reported, not computed
+    bad = _meta(torch.tensor([lens[0] + 5, lens[1], lens[2]], dtype=torch.int32, device="cuda"), bt_dev)
+    assert adapter.try_jetfire_decode(impl=impl, layer=layer, query=torch.zeros(B, Hq, D, dtype=torch.bfloat16, device="cuda"),
+                                      attn_metadata=bad, output=out) is None
+    assert pool.get_stats()["decode_fallbacks"] == {"store_incomplete": 1}
