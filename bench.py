@@ -81,6 +81,9 @@ def main() -> int:
     ap.add_argument("--cpu-threads", type=int, default=14,
                     help="CPU correction worker threads (hand-off mode); the box gives 16 cores, two stay free for "
                          "the launching thread and the hand-off's dispatcher")
+    ap.add_argument("--via-adapter", action="store_true",
+                    help="hand-off mode only: run every layer through jetfire_amd.adapter.try_jetfire_decode (pool "
+                         "manager, cache stores, dispatcher gate) instead of calling the operators directly")
     ap.add_argument("--split-len", type=int, default=0,
                     help="measurement aid: force the fused scan's split length (0 = the library's planner)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -127,11 +130,48 @@ def main() -> int:
     o_new = torch.zeros(w.B, w.H_q, 128, dtype=torch.bfloat16, device="cuda")
     out = torch.empty_like(o_new)
     ctxs = []
-    if handoff:
+    if args.via_adapter and not handoff:
+        print("bench.py: --via-adapter needs the hand-off mode", file=sys.stderr)
+        return 2
+    if handoff and not args.via_adapter:
         ops.set_cpu_attn_threads(args.cpu_threads)
         ctxs = [ops.CpuTopkHandoff(w.B, w.H_q, w.H_kv, w.top_k, ksh, vsh, w.attn_scale) for ksh, vsh in w.shadows]
+    adapter_layers = []
+    if args.via_adapter:
+        # Four cache stores (one per distinct host shadow) own the packed tensors of the first four layers; the
+        # layers of the step cycle over them.  The stores are filled from the workload's tensors (quantised by
+        # the same append kernels) instead of being re-appended token by token.
+        import types
+        import jetfire_amd.adapter as adapter
+        os.environ["JETFIRE_FAST_STORE_COMPLETE_CHECK"] = "1"
+        adapter.set_jetfire_config(scheme={"k3v2": "SymInt3K_SymInt2V", "k4v4": "SymInt4K_SymInt4V"}[w.scheme],
+                                   group_size=w.group, topk=w.top_k, cpu_attn_threads=args.cpu_threads)
+        adapter.reset_global_kv_pool_manager()
+        pool = adapter.get_global_kv_pool_manager()
+        impl = types.SimpleNamespace(attn_type=types.SimpleNamespace(name="DECODER"), scale=w.attn_scale)
+        meta = types.SimpleNamespace(seq_lens=w.seq_lens, block_table=w.block_table, use_cascade=False, max_query_len=1,
+                                     num_actual_tokens=w.B, max_seq_len=w.S)
+        num_blocks = w.layers[0].k_data.size(1) // 16
+        for i, (ksh, vsh) in enumerate(w.shadows):
+            name = f"model.layers.{i}.self_attn.attn"
+            pool.register_layer_config(name, num_query_heads=w.H_q, num_kv_heads=w.H_kv, head_dim=128)
+            pool.register_layer_layout(name, num_blocks=num_blocks, block_size=16)
+            st = pool.ensure_layer_store(name, device=torch.device("cuda"))
+            lay = w.layers[i]
+            st.k_data, st.k_scales, st.v_data, st.v_scales = lay.k_data, lay.k_scales.view_as(st.k_scales), lay.v_data, lay.v_scales.view_as(st.v_scales)
+            st.k_shadow, st.v_shadow = ksh, vsh
+            st.slot_filled.fill_(True)
+            st.written_count = w.S
+            adapter_layers.append(types.SimpleNamespace(layer_name=name, num_heads=w.H_q, num_kv_heads=w.H_kv, head_size=128))
+        n_layers_adapter = n_layers
 
     def step():
+        if adapter_layers:
+            for li in range(n_layers_adapter):
+                got = adapter.try_jetfire_decode(impl=impl, layer=adapter_layers[li % len(adapter_layers)], query=w.q,
+                                                 attn_metadata=meta, output=out)
+                assert got is not None, pool.get_stats()["decode_fallbacks"]
+            return
         for li, lay in enumerate(w.layers):
             o_hat, slots, o_old, W, idx = ops.fused_attn_topk(
                 w.scheme, w.q, lay.k_data, lay.k_scales, lay.v_data, lay.v_scales, w.block_table, w.seq_lens,
@@ -206,6 +246,7 @@ def main() -> int:
                                f"top_k{w.top_k} x{n_layers} layers, {'paged (random)' if args.paged else 'identity'} block table",
                    "packed_bytes_per_layer": bytes_layer, "launch": "hip-graph" if graph is not None else "eager",
                    **({"split_len_forced": args.split_len} if args.split_len else {}),
+                   **({"via": "jetfire_amd.adapter.try_jetfire_decode (4 cache stores cycled over the layers)"} if args.via_adapter else {}),
                    "handoff": (f"slots + q to pinned memory, CPU correction on {ops.get_cpu_attn_threads()} threads, o_new back, every layer"
                                if handoff else "not in the timed region (GPU path only)")},
         "roofline": {"bound": "hbm", "kernel": "fused_scan_kernel", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS,

@@ -9,6 +9,7 @@ hooks, CUDA-graph capture mode, release policy and debug correction modes are no
 from __future__ import annotations
 
 import math
+import os
 
 import torch
 
@@ -23,6 +24,7 @@ _TOPK_CLAMP_LOGGED: set = set()
 _HEAD_MAP_CACHE: dict = {}
 _HANDOFFS: dict = {}
 _O_NEW: dict = {}
+_SEQ_LENS_CACHE: dict = {}
 
 
 def _select_top_k(config_top_k: int, seq_len: int, supported: tuple) -> int | None:
@@ -86,6 +88,18 @@ def _decode_unsupported(*, impl, layer, query, attn_metadata) -> str | None:
     return None
 
 
+def _seq_lens_on_host(seq_lens: torch.Tensor) -> torch.Tensor:
+    """Host copy of the step's sequence lengths.  Every layer of a step passes the same tensor: the copy (a
+    device synchronisation) is made once per (storage, in-place version) and reused by the other layers."""
+    key = (seq_lens.data_ptr(), int(seq_lens.numel()), seq_lens._version, str(seq_lens.device))
+    hit = _SEQ_LENS_CACHE.get("k")
+    if hit is not None and hit[0] == key:
+        return hit[1]
+    host = seq_lens.to("cpu", dtype=torch.long)
+    _SEQ_LENS_CACHE["k"] = (key, host)
+    return host
+
+
 def _handoff_for(store, B: int, H_q: int, H_kv: int, K: int, scale: float):
     key = (id(store), B, H_q, K, float(scale))
     h = _HANDOFFS.get(key)
@@ -105,6 +119,7 @@ def reset_jetfire_decode_runtime_state() -> None:
     _HANDOFFS.clear()
     _O_NEW.clear()
     _HEAD_MAP_CACHE.clear()
+    _SEQ_LENS_CACHE.clear()
 
 
 def try_jetfire_decode(*, impl, layer, query, attn_metadata, output, key=None, value=None):
@@ -135,11 +150,15 @@ def _decode_batched(*, impl, layer, query, attn_metadata, output):
     store.flush_pending_writes()
 
     n_seqs = int(attn_metadata.seq_lens.numel())
-    seq_lens_cpu = attn_metadata.seq_lens.to("cpu", dtype=torch.long)
-    for i, n in enumerate(seq_lens_cpu.tolist()):
-        if n > 0 and not store.has_sequence(attn_metadata.block_table[i], int(n)):
-            pool.record_decode_fallback("store_incomplete")
-            return None
+    seq_lens_cpu = _seq_lens_on_host(attn_metadata.seq_lens)
+    if os.environ.get("JETFIRE_FAST_STORE_COMPLETE_CHECK", "0") == "1":
+        complete = store.fast_has_sequence(int(seq_lens_cpu.max().item()))      # host-side counter, no sync per sequence
+    else:
+        complete = all(n <= 0 or store.has_sequence(attn_metadata.block_table[i], int(n))
+                       for i, n in enumerate(seq_lens_cpu.tolist()))
+    if not complete:
+        pool.record_decode_fallback("store_incomplete")
+        return None
 
     H_q, H_kv, D = layer_cfg.num_query_heads, layer_cfg.num_kv_heads, layer_cfg.head_dim
     scale = float(getattr(impl, "scale", 1.0 / math.sqrt(D)))
