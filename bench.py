@@ -59,6 +59,117 @@ def cpu_baseline(w, budget_s: float = 20.0):
     }
 
 
+def _median_ms(fn, sync, n=10, warm=2):
+    import time
+    ts = []
+    for i in range(warm + n):
+        sync()
+        t0 = time.perf_counter()
+        fn()
+        sync()
+        if i >= warm:
+            ts.append((time.perf_counter() - t0) * 1e3)
+    ts.sort()
+    return ts[len(ts) // 2]
+
+
+def component_append(args):
+    """A prefill chunk of --tokens tokens appended to one layer's store at the workload's geometry: the
+    quantise-on-write kernels, the mirror kernel that stores the bf16 rows into the pinned host shadow, the
+    store's whole `write_slots` + `flush_pending_writes`, and beside it the serial host mirror the reference
+    falls back to (device-to-host copy of the permuted chunk + `index_copy_`, cache_store.py:744-759)."""
+    import torch
+    from jetfire_amd import ops, workloads
+    from jetfire_amd.adapter.cache_store import JetFireInt4CacheStore
+    _, _, Hkv, _, scheme, gs, _, _ = workloads.CONFIGS[args.workload]
+    T = int(args.tokens)
+    kb, vb = (3, 2) if scheme == "k3v2" else (4, 4)
+    nblk = 2 * ((T + 15) // 16)
+    store = JetFireInt4CacheStore(num_kv_heads=Hkv, head_dim=128, group_size=gs, num_blocks=nblk, block_size=16,
+                                  device="cuda", k_nbits=kb, v_nbits=vb)
+    g = torch.Generator().manual_seed(0)
+    key = torch.randn(T, Hkv, 128, generator=g).to(torch.bfloat16).cuda()
+    value = torch.randn(T, Hkv, 128, generator=g).to(torch.bfloat16).cuda()
+    blocks = torch.randperm(nblk, generator=g)[:(T + 15) // 16]
+    slots = (blocks[:, None] * 16 + torch.arange(16)[None, :]).reshape(-1)[:T].cuda()     # paged: runs of 16 slots
+    sync = torch.cuda.synchronize
+    quant_ms = _median_ms(lambda: store._quantise(key, value, slots), sync)
+    mirror_ms = _median_ms(lambda: store._mirror(key, value, slots), sync)
+
+    def whole():
+        store.write_slots(key=key, value=value, slot_mapping=slots)
+        store.flush_pending_writes()
+    whole_ms = _median_ms(whole, sync)
+    import time
+    sync()
+    t0 = time.perf_counter()
+    store.write_slots(key=key, value=value, slot_mapping=slots)
+    torch.cuda.current_stream().synchronize()            # what the model's stream waits for
+    main_ms = (time.perf_counter() - t0) * 1e3
+    store.flush_pending_writes()
+    slots_cpu = slots.cpu()
+
+    def serial_host():
+        k_host = key.permute(1, 0, 2).to("cpu")
+        v_host = value.permute(1, 0, 2).to("cpu")
+        store.k_shadow.index_copy_(1, slots_cpu, k_host)
+        store.v_shadow.index_copy_(1, slots_cpu, v_host)
+    serial_ms = _median_ms(serial_host, sync, n=5, warm=1)
+    bf16_bytes = 2 * T * Hkv * 256
+    return {"component": "append", "workload": args.workload, "tokens": T, "H_kv": Hkv, "scheme": scheme,
+            "quantise_write_ms": round(quant_ms, 4), "shadow_mirror_kernel_ms": round(mirror_ms, 3),
+            "shadow_mirror_GBps_over_pcie": round(bf16_bytes / mirror_ms / 1e6, 1),
+            "write_slots_plus_flush_ms": round(whole_ms, 3), "model_stream_busy_ms": round(main_ms, 3),
+            "serial_host_mirror_ms": round(serial_ms, 3), "bf16_bytes_mirrored": bf16_bytes}
+
+
+def component_cpu_correction(args):
+    """The CPU correction alone (cpu_topk_attn.cpp:854-956) at the workload's (B, Hq, K): slots redrawn for every
+    call over a shadow much larger than the last-level cache, so the gather comes from DRAM
+    (the method of the reference's bench/cpu_correction_microbench.py:150-158)."""
+    import time
+    import torch
+    from jetfire_amd import ops, workloads
+    B, Hq, Hkv, S, _, _, K, _ = workloads.CONFIGS[args.workload]
+    num_slots = B * S
+    g = torch.Generator().manual_seed(0)
+    k_shadow = torch.randn(Hkv, num_slots, 128, generator=g).to(torch.bfloat16)
+    v_shadow = torch.randn(Hkv, num_slots, 128, generator=g).to(torch.bfloat16)
+    q = (torch.randn(B, Hq, 128, generator=g) / 128 ** 0.5).to(torch.bfloat16)
+    head_map = (torch.arange(Hq) // (Hq // Hkv))[None, :, None].expand(B, Hq, K).contiguous()
+    o_new = torch.zeros(B, Hq, 128, dtype=torch.bfloat16)
+    ops.set_cpu_attn_threads(args.cpu_threads)
+    ts = []
+    for i in range(23):
+        base = (torch.arange(B) * S)[:, None, None]
+        slots = (torch.randint(0, S, (B, Hq, K), generator=g) + base).contiguous()
+        t0 = time.perf_counter()
+        ops.cpu_topk_attn(q, k_shadow, v_shadow, head_map, slots, o_new, 128 ** -0.5)
+        if i >= 3:
+            ts.append(time.perf_counter() - t0)
+    ts.sort()
+    med = ts[len(ts) // 2]
+    return {"component": "cpu-correction", "workload": args.workload, "B": B, "H_q": Hq, "top_k": K, "threads": args.cpu_threads,
+            "us_per_call": round(med * 1e6, 1), "min_us": round(ts[0] * 1e6, 1),
+            "gathered_GBps": round(B * Hq * K * 512 / med / 1e9, 1), "rows_gathered": B * Hq * K * 2}
+
+
+def component_pcie(args):
+    """Pinned host <-> device copy latency by size (the reference's bench/pcie_transfer_microbench.py:20-42), and
+    the hand-off's own transfer of the workload: one publish kernel down, one fetch kernel up."""
+    import torch
+    out = {"component": "pcie", "sizes": {}}
+    sync = torch.cuda.synchronize
+    for nbytes in (4 << 10, 32 << 10, 256 << 10, 2 << 20, 16 << 20, 128 << 20):
+        host = torch.empty(nbytes, dtype=torch.uint8, pin_memory=True)
+        dev = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+        d2h = _median_ms(lambda: host.copy_(dev, non_blocking=True), sync, n=20, warm=3)
+        h2d = _median_ms(lambda: dev.copy_(host, non_blocking=True), sync, n=20, warm=3)
+        out["sizes"][str(nbytes)] = {"d2h_us": round(d2h * 1e3, 1), "h2d_us": round(h2d * 1e3, 1),
+                                     "d2h_GBps": round(nbytes / d2h / 1e6, 2), "h2d_GBps": round(nbytes / h2d / 1e6, 2)}
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
@@ -86,6 +197,11 @@ def main() -> int:
                          "manager, cache stores, dispatcher gate) instead of calling the operators directly")
     ap.add_argument("--split-len", type=int, default=0,
                     help="measurement aid: force the fused scan's split length (0 = the library's planner)")
+    ap.add_argument("--component", default=None, choices=["append", "cpu-correction", "pcie"],
+                    help="time one component of the path at the workload's geometry, print its own JSON line and exit: "
+                         "append = quantise-on-write + shadow mirror of a prefill chunk (--tokens); cpu-correction = the "
+                         "CPU pool alone on freshly drawn random slots; pcie = pinned copy latency by size")
+    ap.add_argument("--tokens", type=int, default=32768, help="--component append: tokens in the prefill chunk")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run a plain 1 GiB device copy 10 times and exit (reference for the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -115,6 +231,10 @@ def main() -> int:
         us = e0.elapsed_time(e1) * 100.0       # per copy
         print(json.dumps({"calibrate_copy_bytes_read": 1 << 30, "calibrate_copy_bytes_written": 1 << 30, "launches": 11,
                           "us_per_copy": round(us, 1), "copy_read_plus_write_GBps": round(2 * (1 << 30) / us / 1e3, 1)}))
+        return 0
+    if args.component is not None:
+        print(json.dumps({"append": component_append, "cpu-correction": component_cpu_correction,
+                          "pcie": component_pcie}[args.component](args)))
         return 0
     if args.split_len:
         _lib.check(lib.jf_debug_split_len(args.split_len))

@@ -63,6 +63,29 @@ int jf_quant_write_int4_sym_kv(const uint16_t* key, int64_t k_stride_t, int64_t 
                                uint16_t* v_scale, int64_t v_scale_stride_h, int64_t v_scale_stride_slot,
                                int64_t num_slots, int group_size, void* stream);
 
+/* Mirror of appended rows into the bf16 host shadow the CPU correction reads: k_shadow[h, slots[t], :] =
+ * key[t, h, :], the same for V; slots[t] < 0 (padding) and slots[t] >= num_slots are skipped.  Replaces the
+ * reference's shadow mirror: the serial host copy + index_copy_ (jetfire_vllm/adapter/cache_store.py:686-759),
+ * the prefill pipeline's D2H into pinned staging buffers followed by a worker thread's scatter
+ * (cache_store.py:1224-1338) and the graph-mode decode append (staging copies + host callback,
+ * cache_store.py:531-642, jetfire_vllm/csrc/cpu_topk_attn.cpp:1611-1665).  Here the shadow is pinned host
+ * memory the GPU addresses and ONE kernel stores the rows to it across PCIe; the launch is asynchronous, can
+ * be captured in a HIP graph, and its rows are visible to the host when work enqueued after it on the same
+ * stream runs (the hand-off's publish kernel) or the stream / an event recorded after it has been waited for.
+ * key / value are (T, H_kv, 128) bf16 with element strides (last dim contiguous, rows 4-byte aligned);
+ * k_shadow / v_shadow are DEVICE-VISIBLE addresses (jf_host_buffer_device_pointer) of (H_kv, num_slots, 128)
+ * bf16 with element strides shadow_stride_h / shadow_stride_slot, rows 16-byte aligned. */
+int jf_shadow_write(const uint16_t* key, int64_t k_stride_t, int64_t k_stride_h,
+                    const uint16_t* value, int64_t v_stride_t, int64_t v_stride_h,
+                    const int64_t* slots, int64_t T, int H_kv,
+                    uint16_t* k_shadow, uint16_t* v_shadow, int64_t shadow_stride_h, int64_t shadow_stride_slot,
+                    int64_t num_slots, void* stream);
+
+/* Address under which the GPU reaches a pinned host buffer (hipHostMalloc, torch's pin_memory=True), or
+ * JF_ERR_ARG when host_ptr is pageable or device memory.  The reference allocates its mapped buffers itself
+ * (alloc_mapped_pinned_pair, jetfire_vllm/csrc/cpu_topk_attn.cpp:972-1023); here the caller owns them. */
+int jf_host_buffer_device_pointer(const void* host_ptr, void** device_ptr);
+
 /* ------------------------------------------------------------------ Stage A (split form)
  * scores[b, hq, s] for s < seq_len, -inf for seq_len <= s < max_S.
  * jf_int3_qk_scores replaces int3_qk_scores (jetfire_vllm/csrc/int3_qk_scores.cu:318-390):

@@ -18,6 +18,7 @@ LIB_PATH = os.path.join(PKG_DIR, "libjetfire_amd.so")
 
 SOURCES = (
     "quant_write.hip",
+    "shadow_write.hip",
     "qk_scores.hip",
     "topk.hip",
     "softmax_v.hip",

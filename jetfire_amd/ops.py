@@ -119,6 +119,44 @@ def fused_quant_write_int4_sym_kv(key_tok, value_tok, slot_idx, k_data, k_scales
         k_data.shape[1], int(group_size), _stream(key_tok)))
 
 
+def host_buffer_device_pointer(t: torch.Tensor) -> int:
+    """Address under which the GPU reaches the pinned host tensor `t`; raises for pageable memory."""
+    import ctypes
+    lib = _lib.load()
+    _check(not t.is_cuda, "expected a host tensor")
+    out = ctypes.c_void_p()
+    _lib.check(lib.jf_host_buffer_device_pointer(t.data_ptr(), ctypes.byref(out)))
+    return int(out.value)
+
+
+def shadow_write(key_tok, value_tok, slot_idx, k_shadow, v_shadow, *, k_shadow_dev: int | None = None,
+                 v_shadow_dev: int | None = None) -> None:
+    """Mirror the appended rows into the pinned bf16 host shadows `(H_kv, num_slots, 128)`:
+    `k_shadow[h, slot_idx[t]] = key_tok[t, h]` (cache_store.py:686-759,1224-1338 in one kernel launch on the
+    current stream; asynchronous).  `*_dev` are the shadows' device-visible addresses when the caller has
+    looked them up already."""
+    lib = _lib.load()
+    _check(key_tok.is_cuda and value_tok.is_cuda, "tokens must be on the GPU")
+    _check(key_tok.dtype == torch.bfloat16 and value_tok.dtype == torch.bfloat16, "tokens must be bf16")
+    _check(value_tok.shape == key_tok.shape and key_tok.dim() == 3 and key_tok.shape[2] == HEAD_DIM,
+           "key/value tokens must both be (T, H_kv, 128)")
+    _check(key_tok.stride(2) == 1 and value_tok.stride(2) == 1, "tokens must be contiguous in the last dimension")
+    T, H_kv, D = key_tok.shape
+    for s in (k_shadow, v_shadow):
+        _check(not s.is_cuda and s.dtype == torch.bfloat16 and s.dim() == 3 and s.shape[0] == H_kv and s.shape[2] == D
+               and s.stride(2) == 1, "shadow must be a (H_kv, num_slots, 128) bf16 host tensor")
+    _check(k_shadow.shape == v_shadow.shape and k_shadow.stride() == v_shadow.stride(), "K and V shadows must match")
+    _check(slot_idx.is_cuda and slot_idx.dtype == torch.int64 and slot_idx.shape == (T,), "slots must be (T,) int64")
+    slot_idx = slot_idx.contiguous()
+    kd = host_buffer_device_pointer(k_shadow) if k_shadow_dev is None else int(k_shadow_dev)
+    vd = host_buffer_device_pointer(v_shadow) if v_shadow_dev is None else int(v_shadow_dev)
+    _lib.check(lib.jf_shadow_write(
+        key_tok.data_ptr(), key_tok.stride(0), key_tok.stride(1),
+        value_tok.data_ptr(), value_tok.stride(0), value_tok.stride(1),
+        slot_idx.data_ptr(), T, H_kv, kd, vd, k_shadow.stride(0), k_shadow.stride(1), k_shadow.shape[1],
+        _stream(key_tok)))
+
+
 # --------------------------------------------------------------------------- Stage A
 
 

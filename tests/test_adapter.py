@@ -174,3 +174,131 @@ def test_prefill_then_decode_steps_match_the_oracle(adapter, scheme_name, scheme
     assert adapter.try_jetfire_decode(impl=impl, layer=layer, query=torch.zeros(B, Hq, D, dtype=torch.bfloat16, device="cuda"),
                                       attn_metadata=bad, output=out) is None
     assert pool.get_stats()["decode_fallbacks"] == {"store_incomplete": 1}
+
+
+# ----------------------------------------------------------------------------- shadow mirror (GPU)
+def _bits(t):
+    return t.contiguous().view(torch.int16)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("misalign", [0, 2])
+def test_shadow_write_matches_a_host_scatter(misalign):
+    """`ops.shadow_write` against the reference's serial mirror (permute + `index_copy_`, cache_store.py:744-759)
+    on strided token views (slices of one fused qkv activation), padding slots and a slot outside the shadow."""
+    from jetfire_amd import ops
+    T, Hq, Hkv, D, num_slots = 1000, 8, 4, 128, 2048
+    g = torch.Generator().manual_seed(11)
+    qkv = torch.randn(T, (Hq + 2 * Hkv) * D + 8, generator=g).to(torch.bfloat16)
+    qkv_dev = qkv.cuda()
+    lo = Hq * D + misalign                                  # misalign = 2 elements: rows only 4-byte aligned
+    key = qkv_dev[:, lo:lo + Hkv * D].view(T, Hkv, D)
+    value = qkv_dev[:, lo + Hkv * D:lo + 2 * Hkv * D].view(T, Hkv, D)
+    slots = torch.randperm(num_slots, generator=g)[:T].to(torch.int64)
+    slots[::37] = -1
+    slots[5] = num_slots + 3                                # never stored
+    k_shadow = torch.zeros(Hkv, num_slots, D, dtype=torch.bfloat16, pin_memory=True)
+    v_shadow = torch.zeros(Hkv, num_slots, D, dtype=torch.bfloat16, pin_memory=True)
+    ops.shadow_write(key, value, slots.cuda(), k_shadow, v_shadow)
+    torch.cuda.synchronize()
+    keep = (slots >= 0) & (slots < num_slots)
+    want_k = torch.zeros(Hkv, num_slots, D, dtype=torch.bfloat16)
+    want_v = torch.zeros_like(want_k)
+    want_k.index_copy_(1, slots[keep], qkv[:, lo:lo + Hkv * D].reshape(T, Hkv, D).permute(1, 0, 2)[:, keep].contiguous())
+    want_v.index_copy_(1, slots[keep], qkv[:, lo + Hkv * D:lo + 2 * Hkv * D].reshape(T, Hkv, D).permute(1, 0, 2)[:, keep].contiguous())
+    assert torch.equal(_bits(k_shadow), _bits(want_k))
+    assert torch.equal(_bits(v_shadow), _bits(want_v))
+
+
+@pytest.mark.gpu
+def test_shadow_write_rejects_pageable_memory_and_bad_shapes():
+    from jetfire_amd import ops
+    key = torch.zeros(4, 2, 128, dtype=torch.bfloat16, device="cuda")
+    slots = torch.arange(4, device="cuda")
+    pageable = torch.zeros(2, 64, 128, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="pinned|not known"):
+        ops.shadow_write(key, key, slots, pageable, pageable)
+    pinned = torch.zeros(3, 64, 128, dtype=torch.bfloat16, pin_memory=True)
+    with pytest.raises(RuntimeError, match="shadow must be"):
+        ops.shadow_write(key, key, slots, pinned, pinned)          # kv-head count differs
+    ok = torch.zeros(2, 64, 128, dtype=torch.bfloat16, pin_memory=True)
+    with pytest.raises(RuntimeError, match="slots"):
+        ops.shadow_write(key, key, slots[:3], ok, ok)
+    ops.shadow_write(key[:0], key[:0], slots[:0], ok, ok)          # empty append is a no-op
+    torch.cuda.synchronize()
+    assert float(ok.float().abs().sum()) == 0.0
+
+
+@pytest.mark.gpu
+def test_prefill_chunks_mirror_off_stream_until_flush():
+    """Chunks of >= JETFIRE_PIPELINE_MIN_TOKENS tokens go to the side stream and stay pending until
+    `flush_pending_writes`; afterwards the shadow holds every chunk, the later write of a slot winning."""
+    from jetfire_amd.adapter.cache_store import JetFireInt4CacheStore
+    Hkv, D, nblk, bs = 4, 128, 512, 16
+    store = JetFireInt4CacheStore(num_kv_heads=Hkv, head_dim=D, group_size=64, num_blocks=nblk, block_size=bs,
+                                  device="cuda", k_nbits=3, v_nbits=2)
+    g = torch.Generator().manual_seed(3)
+    want_k = torch.zeros(Hkv, nblk * bs, D, dtype=torch.bfloat16)
+    want_v = torch.zeros_like(want_k)
+    perm = torch.randperm(nblk * bs, generator=g)
+    chunks = [(0, 4096), (4096, 6144), (6144, 6200), (100, 300)]            # the last one rewrites slots of the first
+    for i, (a, b) in enumerate(chunks):
+        k = torch.randn(b - a, Hkv, D, generator=g).to(torch.bfloat16)
+        v = torch.randn(b - a, Hkv, D, generator=g).to(torch.bfloat16)
+        slots = perm[a:b].clone()
+        assert store.write_slots(key=k.cuda(), value=v.cuda(), slot_mapping=slots.cuda()) == b - a
+        want_k.index_copy_(1, slots, k.permute(1, 0, 2).contiguous())
+        want_v.index_copy_(1, slots, v.permute(1, 0, 2).contiguous())
+    assert len(store._pending_mirrors) == 3                                  # the 56-token chunk stayed on the stream
+    store.flush_pending_writes()
+    torch.cuda.current_stream().synchronize()                                # the small chunk ran on this stream
+    assert store._pending_mirrors == []
+    assert torch.equal(_bits(store.k_shadow), _bits(want_k))
+    assert torch.equal(_bits(store.v_shadow), _bits(want_v))
+    filled = torch.zeros(nblk * bs, dtype=torch.bool)
+    filled[perm[:6200]] = True
+    assert torch.equal(store.slot_filled.cpu(), filled)
+    assert store.written_count == sum(b - a for a, b in chunks)
+
+
+@pytest.mark.gpu
+def test_decode_append_replays_from_a_hip_graph():
+    """`write_slots_graph` (cache_store.py:531-642) captured once and replayed with new tokens and slots in the
+    same static buffers: every replay lands in the INT cache and in the shadow; eager work in between."""
+    from jetfire_amd.adapter.cache_store import JetFireInt4CacheStore
+    Hkv, D, nblk, bs, Bmax = 2, 128, 8, 16, 4
+    store = JetFireInt4CacheStore(num_kv_heads=Hkv, head_dim=D, group_size=128, num_blocks=nblk, block_size=bs,
+                                  device="cuda", k_nbits=4, v_nbits=4)
+    eager = JetFireInt4CacheStore(num_kv_heads=Hkv, head_dim=D, group_size=128, num_blocks=nblk, block_size=bs,
+                                  device="cuda", k_nbits=4, v_nbits=4)
+    key = torch.zeros(Bmax, Hkv, D, dtype=torch.bfloat16, device="cuda")
+    value = torch.zeros_like(key)
+    slots = torch.full((Bmax,), -1, dtype=torch.int64, device="cuda")
+    with pytest.raises(RuntimeError, match="max_batch_size"):
+        store.write_slots_graph(key=key, value=value, slot_mapping=slots, max_batch_size=2)
+    store.warmup_graph_append(Bmax)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        store.write_slots_graph(key=key, value=value, slot_mapping=slots, max_batch_size=Bmax)   # warm-up, all padding
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        store.write_slots_graph(key=key, value=value, slot_mapping=slots, max_batch_size=Bmax)
+    g = torch.Generator().manual_seed(9)
+    for step in range(4):
+        k = torch.randn(Bmax, Hkv, D, generator=g).to(torch.bfloat16)
+        v = torch.randn(Bmax, Hkv, D, generator=g).to(torch.bfloat16)
+        s = torch.tensor([step, 16 + step, -1 if step % 2 else 40 + step, 100 + step], dtype=torch.int64)
+        key.copy_(k.cuda()); value.copy_(v.cuda()); slots.copy_(s.cuda())
+        graph.replay()
+        eager.write_slots(key=k.cuda(), value=v.cuda(), slot_mapping=s.cuda())
+        torch.cuda.synchronize()
+        for name in ("k_data", "k_scales", "v_data", "v_scales"):
+            a, b = getattr(store, name), getattr(eager, name)
+            assert torch.equal(a.view(torch.uint8) if a.dtype == torch.uint8 else _bits(a),
+                               b.view(torch.uint8) if b.dtype == torch.uint8 else _bits(b)), (step, name)
+        assert torch.equal(_bits(store.k_shadow), _bits(eager.k_shadow)), step
+        assert torch.equal(_bits(store.v_shadow), _bits(eager.v_shadow)), step
+        keep = s >= 0
+        assert torch.equal(_bits(store.k_shadow[:, s[keep]]), _bits(k.permute(1, 0, 2)[:, keep].contiguous())), step
