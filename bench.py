@@ -138,7 +138,8 @@ def component_cpu_correction(args):
     q = (torch.randn(B, Hq, 128, generator=g) / 128 ** 0.5).to(torch.bfloat16)
     head_map = (torch.arange(Hq) // (Hq // Hkv))[None, :, None].expand(B, Hq, K).contiguous()
     o_new = torch.zeros(B, Hq, 128, dtype=torch.bfloat16)
-    ops.set_cpu_attn_threads(args.cpu_threads)
+    threads = args.cpu_threads or 14
+    ops.set_cpu_attn_threads(threads)
     ts = []
     for i in range(23):
         base = (torch.arange(B) * S)[:, None, None]
@@ -149,7 +150,7 @@ def component_cpu_correction(args):
             ts.append(time.perf_counter() - t0)
     ts.sort()
     med = ts[len(ts) // 2]
-    return {"component": "cpu-correction", "workload": args.workload, "B": B, "H_q": Hq, "top_k": K, "threads": args.cpu_threads,
+    return {"component": "cpu-correction", "workload": args.workload, "B": B, "H_q": Hq, "top_k": K, "threads": threads,
             "us_per_call": round(med * 1e6, 1), "min_us": round(ts[0] * 1e6, 1),
             "gathered_GBps": round(B * Hq * K * 512 / med / 1e9, 1), "rows_gathered": B * Hq * K * 2}
 
@@ -189,9 +190,11 @@ def main() -> int:
                     help="include the pinned hand-off and the CPU correction per layer (default for c4 and c5, "
                          "whose definition is end to end)")
     ap.add_argument("--no-handoff", dest="handoff", action="store_false")
-    ap.add_argument("--cpu-threads", type=int, default=14,
-                    help="CPU correction worker threads (hand-off mode); the box gives 16 cores, two stay free for "
-                         "the launching thread and the hand-off's dispatcher")
+    ap.add_argument("--cpu-threads", type=int, default=None,
+                    help="CPU correction worker threads (hand-off mode); default 14 of the box's 16 cores with the "
+                         "host-blocking wait (two stay free for the launching thread and the hand-off's dispatcher), 11 "
+                         "with --graph, where the runtime's own threads are busy too: one worker too many and a "
+                         "descheduled worker stretches every job to a scheduler time slice")
     ap.add_argument("--via-adapter", action="store_true",
                     help="hand-off mode only: run every layer through jetfire_amd.adapter.try_jetfire_decode (pool "
                          "manager, cache stores, dispatcher gate) instead of calling the operators directly")
@@ -239,10 +242,12 @@ def main() -> int:
     if args.split_len:
         _lib.check(lib.jf_debug_split_len(args.split_len))
     handoff = args.handoff if args.handoff is not None else args.workload in ("c4", "c5")
+    if args.cpu_threads is None:
+        args.cpu_threads = 11 if (handoff and args.graph) else 14
     if args.graph is None:
         args.graph = not handoff
-    if handoff and args.graph:
-        print("bench.py: --graph and the hand-off mode are exclusive", file=sys.stderr)
+    if handoff and args.graph and args.via_adapter:
+        print("bench.py: --graph with the hand-off goes through the operators, not the adapter", file=sys.stderr)
         return 2
     n_shadow = 4 if handoff else 0   # distinct host shadows, cycled over the layers (a layer's shadow is 2*H_kv*slots*256 B)
     w = workloads.build(args.workload, n_layers=args.layers, keep_shadow=n_shadow)
@@ -298,8 +303,12 @@ def main() -> int:
                 w.S, w.H_q, w.H_kv, 16, w.top_k, w.attn_scale)
             if ctxs:
                 h = ctxs[li % len(ctxs)]
-                h.submit(w.q, slots)
-                h.wait(o_new)
+                if args.graph:      # kernels only: the publish kernel and a device-side wait
+                    h.stream_submit(w.q, slots)
+                    h.stream_wait(o_new)
+                else:
+                    h.submit(w.q, slots)
+                    h.wait(o_new)
             ops.blend_unnorm_into(o_hat, o_old, W, o_new, out)
 
     for _ in range(args.warmup):
@@ -333,6 +342,9 @@ def main() -> int:
             step()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    for h in ctxs:
+        if args.graph:
+            h.check_status()
     if graph is None:
         _lib.check(lib.jf_profile_scan_end(ctypes.byref(total_ms), ctypes.byref(launches)))
     else:   # kernel time from a separate eager pass
@@ -368,6 +380,7 @@ def main() -> int:
                    **({"split_len_forced": args.split_len} if args.split_len else {}),
                    **({"via": "jetfire_amd.adapter.try_jetfire_decode (4 cache stores cycled over the layers)"} if args.via_adapter else {}),
                    "handoff": (f"slots + q to pinned memory, CPU correction on {ops.get_cpu_attn_threads()} threads, o_new back, every layer"
+                               + (" (device-side wait, whole step in one graph)" if args.graph else " (host-blocking wait)")
                                if handoff else "not in the timed region (GPU path only)")},
         "roofline": {"bound": "hbm", "kernel": "fused_scan_kernel", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,

@@ -221,6 +221,30 @@ int jf_handoff_wait(jf_handoff* h, uint16_t* o_new_dev, void* stream);
 int64_t jf_handoff_submit_count(const jf_handoff* h);
 void jf_handoff_destroy(jf_handoff* h);
 
+/* Stream mode of the same context: the graph-capturable pair.  Replaces the reference's host-callback
+ * submit / join (graph_submit_callback / graph_join_callback and stream_write_value64 / stream_wait_value64,
+ * jetfire_vllm/csrc/cpu_topk_attn.cpp:1805-2016, 1293-1344) without any host callback or stream memory
+ * operation: both calls only enqueue kernels, so a captured graph replays them with no host code in between.
+ * stream_submit: the publish kernel of jf_handoff_submit, except that the sequence number comes from a counter
+ *         in device memory which the kernel advances itself; from the first call on the dispatcher thread polls
+ *         the pinned flag continuously (with sleeps that lengthen while the GPU is silent).
+ * stream_wait: one workgroup whose first lane polls the pinned "finished" word until the correction of the
+ *         device's current sequence number is done, then copies o_new into o_new_dev.  The wait is bounded
+ *         (min(JETFIRE_CPU_FUTURE_TIMEOUT_S, 10 s); jf_handoff_set_device_wait_limit_us): at the limit the
+ *         kernel raises a status word, writes zeros to o_new_dev and ends; every later wait of the context
+ *         falls through at once.  jf_handoff_status reports it (JF_ERR_TIMEOUT) after the stream has been
+ *         synchronised; jf_handoff_stream_submit refuses a failed context.
+ * A context serves one mode: mixing the pairs is JF_ERR_ARG.  Calls of one context must be ordered on one
+ * stream (submit, wait, submit, ...).  Destroy a stream-mode context only when no graph that holds its kernels
+ * will be replayed again; destroy synchronises the device first. */
+int jf_handoff_stream_submit(jf_handoff* h, const uint16_t* q_dev, const int64_t* topk_slots_dev, void* stream);
+int jf_handoff_stream_wait(jf_handoff* h, uint16_t* o_new_dev, void* stream);
+int jf_handoff_status(jf_handoff* h);
+int jf_handoff_set_device_wait_limit_us(jf_handoff* h, int64_t us);
+/* Test aid: while on, the dispatcher ignores published flags (a correction that never finishes, without
+ * hanging anything: the device-side wait runs into its limit). */
+int jf_handoff_debug_pause(jf_handoff* h, int on);
+
 #ifdef __cplusplus
 }
 #endif

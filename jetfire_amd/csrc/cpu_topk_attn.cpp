@@ -405,8 +405,13 @@ struct jf_handoff {
   uint16_t* q_pin = nullptr;       // (B, H_q, D) bf16
   int64_t* ts_pin = nullptr;       // (B, H_q, K)
   uint16_t* o_pin = nullptr;       // (B, H_q, D) bf16
-  int64_t* flag_pin = nullptr;     // [0]: sequence number of the last published (q, slots)
-  unsigned* counter_dev = nullptr; // workgroups of the publish kernel that have finished
+  int64_t* flag_pin = nullptr;     // [0]: sequence number of the last published (q, slots); [8]: sequence number of
+                                   // the last finished correction; [16]: status raised by the device-side wait
+  unsigned* counter_dev = nullptr; // [0]: workgroups of the publish kernel that have finished; bytes 8..15: the
+                                   // device's own sequence counter (stream mode)
+  std::atomic<int> mode{0};        // 0 = not used yet, 1 = host-blocking wait, 2 = stream mode (device-side wait)
+  std::atomic<int> paused{0};      // test aid: the dispatcher ignores published flags
+  uint64_t device_wait_ticks = 0;  // bound of the device-side wait, in ticks of the 100 MHz wall clock
   std::vector<int64_t> head_map;   // (B, H_q, K)
   std::atomic<int64_t> submits{0};
   std::atomic<int64_t> host_seq{0};  // submits enqueued by the host
@@ -423,7 +428,8 @@ namespace {
 
 __global__ __launch_bounds__(256) void handoff_publish_kernel(const uint4* __restrict__ q_src, uint4* q_dst, int nq16,
                                                               const uint4* __restrict__ s_src, uint4* s_dst, int ns16,
-                                                              unsigned* counter, int64_t* flag, int64_t seq) {
+                                                              unsigned* counter, int64_t* flag, int64_t seq,
+                                                              int64_t* seq_dev) {
   for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < nq16 + ns16; i += gridDim.x * blockDim.x) {
     if (i < nq16) q_dst[i] = q_src[i];
     else s_dst[i - nq16] = s_src[i - nq16];
@@ -434,6 +440,10 @@ __global__ __launch_bounds__(256) void handoff_publish_kernel(const uint4* __res
     const unsigned done = atomicAdd(counter, 1u);
     if (done == gridDim.x - 1) {  // every workgroup's stores are out: raise the flag
       *counter = 0u;
+      if (seq_dev) {  // stream mode: the device numbers the submits itself, so a graph replay needs no new argument
+        seq = *seq_dev + 1;
+        *seq_dev = seq;
+      }
       __threadfence_system();
       __hip_atomic_store(flag, seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
     }
@@ -442,6 +452,35 @@ __global__ __launch_bounds__(256) void handoff_publish_kernel(const uint4* __res
 
 __global__ __launch_bounds__(256) void handoff_fetch_kernel(const uint4* __restrict__ src, uint4* dst, int n16) {
   for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += gridDim.x * blockDim.x) dst[i] = src[i];
+}
+
+// Stream mode: ONE workgroup.  Its first lane polls the finished-sequence word in pinned host memory until the
+// correction of the device's current sequence number is done or `limit_ticks` of the constant 100 MHz clock have
+// passed (then the status word is raised and o_new is zero-filled: the kernel always ends), the workgroup then
+// copies o_new to the device.
+__global__ __launch_bounds__(1024) void handoff_wait_fetch_kernel(const int64_t* done, const int64_t* seq_dev,
+                                                                  int64_t* status, uint64_t limit_ticks,
+                                                                  const uint4* __restrict__ src, uint4* dst, int n16) {
+  __shared__ int ok_sh;
+  if (threadIdx.x == 0) {
+    const int64_t want = *seq_dev;
+    const uint64_t t0 = wall_clock64();
+    // a context that has failed once does not wait again: every later launch falls through at once
+    int ok = __hip_atomic_load(status, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM) == 0;
+    while (ok && __hip_atomic_load(done, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM) < want) {
+      if (wall_clock64() - t0 > limit_ticks) {
+        ok = 0;
+        break;
+      }
+      __builtin_amdgcn_s_sleep(16);
+    }
+    if (!ok && __hip_atomic_load(status, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM) == 0)
+      __hip_atomic_store(status, (int64_t)1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    ok_sh = ok;
+  }
+  __syncthreads();
+  const bool ok = ok_sh != 0;
+  for (int i = threadIdx.x; i < n16; i += blockDim.x) dst[i] = ok ? src[i] : make_uint4(0u, 0u, 0u, 0u);
 }
 
 inline void cpu_relax() {
@@ -453,22 +492,24 @@ inline void cpu_relax() {
 void handoff_dispatch(jf_handoff* h) {
   int64_t seen = 0;
   for (;;) {
-    {  // nothing outstanding: sleep until a submit (or the end)
+    if (h->mode.load() != 2) {  // host mode with nothing outstanding: sleep until a submit (or the end)
       std::unique_lock<std::mutex> lk(h->mu);
-      h->cv.wait(lk, [&] { return h->stop.load() || h->host_seq.load() > seen; });
+      h->cv.wait(lk, [&] { return h->stop.load() || h->host_seq.load() > seen || h->mode.load() == 2; });
     }
     if (h->stop.load()) return;
-    // a submit is in the stream: poll the flag the publish kernel raises
+    const bool streaming = h->mode.load() == 2;
+    // poll the flag the publish kernel raises.  Stream mode: submits arrive from graph replays without any host
+    // call, so the thread keeps polling, with sleeps that lengthen while the GPU stays silent.
     const auto t0 = std::chrono::steady_clock::now();
     int64_t f = seen;
     for (uint64_t spin = 0;; ++spin) {
-      f = __atomic_load_n(h->flag_pin, __ATOMIC_ACQUIRE);
+      f = h->paused.load(std::memory_order_relaxed) ? seen : __atomic_load_n(h->flag_pin, __ATOMIC_ACQUIRE);
       if (f != seen || h->stop.load(std::memory_order_relaxed)) break;
       cpu_relax();
       if ((spin & 0xfff) == 0xfff) {
         const double el = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
-        if (el > h->timeout_s) { h->failed.store(1); break; }
-        if (el > 0.002) std::this_thread::sleep_for(std::chrono::microseconds(50));  // a long GPU queue: stop burning a core
+        if (!streaming && el > h->timeout_s) { h->failed.store(1); break; }
+        if (el > 0.002) std::this_thread::sleep_for(std::chrono::microseconds(streaming && el > 1.0 ? 200 : 50));
       }
     }
     if (h->stop.load()) return;
@@ -480,10 +521,19 @@ void handoff_dispatch(jf_handoff* h) {
     seen = f;
     CpuJob j{h->q_pin, h->k_shadow, h->v_shadow, h->head_map.data(), h->ts_pin, h->o_pin,
              h->B, h->H_q, h->K, h->H_kv, h->num_slots, h->scale};
-    if (!Pool::instance().run((int64_t)h->B * h->H_q, [j](int64_t b, int64_t e) { run_rows(j, b, e); })) h->failed.store(1);
+    if (!Pool::instance().run((int64_t)h->B * h->H_q, [j](int64_t b, int64_t e) { run_rows(j, b, e); })) {
+      h->failed.store(1);
+      __atomic_store_n(h->flag_pin + 16, (int64_t)2, __ATOMIC_RELEASE);
+    }
     h->submits.fetch_add(1, std::memory_order_relaxed);
     h->done_seq.store(seen, std::memory_order_release);
+    __atomic_store_n(h->flag_pin + 8, seen, __ATOMIC_RELEASE);  // what the device-side wait polls
   }
+}
+
+bool claim_mode(jf_handoff* h, int mode) {
+  int expected = 0;
+  return h->mode.compare_exchange_strong(expected, mode) || expected == mode;
 }
 
 }  // namespace
@@ -505,13 +555,14 @@ extern "C" jf_handoff* jf_handoff_create(int B, int H_q, int H_kv, int K, int64_
   if (hipHostMalloc((void**)&h->q_pin, nq, hipHostMallocDefault) != hipSuccess ||
       hipHostMalloc((void**)&h->ts_pin, nt, hipHostMallocDefault) != hipSuccess ||
       hipHostMalloc((void**)&h->o_pin, nq, hipHostMallocDefault) != hipSuccess ||
-      hipHostMalloc((void**)&h->flag_pin, 64, hipHostMallocDefault) != hipSuccess ||
+      hipHostMalloc((void**)&h->flag_pin, 256, hipHostMallocDefault) != hipSuccess ||
       hipMalloc((void**)&h->counter_dev, 64) != hipSuccess || hipMemset(h->counter_dev, 0, 64) != hipSuccess) {
     set_error("handoff_create: allocation failed");
     jf_handoff_destroy(h);
     return nullptr;
   }
-  h->flag_pin[0] = 0;
+  h->flag_pin[0] = h->flag_pin[8] = h->flag_pin[16] = 0;
+  h->device_wait_ticks = (uint64_t)((h->timeout_s < 10.0 ? h->timeout_s : 10.0) * 1e8);
   const int G = H_q / H_kv;
   h->head_map.resize((size_t)B * H_q * K);
   for (int b = 0; b < B; ++b)
@@ -525,6 +576,7 @@ extern "C" int jf_handoff_submit(jf_handoff* h, const uint16_t* q_dev, const int
   JF_CHECK_ARG(h && q_dev && topk_slots_dev, "handoff_submit: null argument");
   JF_CHECK_ARG(((uintptr_t)q_dev & 15) == 0 && ((uintptr_t)topk_slots_dev & 15) == 0, "handoff_submit: q and topk_slots must be 16-byte aligned");
   if (h->failed.load()) { set_error("handoff: an earlier CPU correction job failed or timed out"); return JF_ERR_TIMEOUT; }
+  JF_CHECK_ARG(claim_mode(h, 1), "handoff_submit: the context is in stream mode (use jf_handoff_stream_submit)");
   JF_CHECK_ARG(h->host_seq.load() == h->done_seq.load(), "handoff_submit: the previous correction is still in flight (wait for it first)");
   hipStream_t st = (hipStream_t)stream;
   const int nq16 = (int)((size_t)h->B * h->H_q * D * sizeof(uint16_t) / 16);
@@ -534,7 +586,7 @@ extern "C" int jf_handoff_submit(jf_handoff* h, const uint16_t* q_dev, const int
   if (blocks > 32) blocks = 32;
   hipLaunchKernelGGL(handoff_publish_kernel, dim3(blocks), dim3(256), 0, st, reinterpret_cast<const uint4*>(q_dev),
                      reinterpret_cast<uint4*>(h->q_pin), nq16, reinterpret_cast<const uint4*>(topk_slots_dev),
-                     reinterpret_cast<uint4*>(h->ts_pin), ns16, h->counter_dev, h->flag_pin, seq);
+                     reinterpret_cast<uint4*>(h->ts_pin), ns16, h->counter_dev, h->flag_pin, seq, (int64_t*)nullptr);
   JF_CHECK_HIP(hipGetLastError());
   {
     std::lock_guard<std::mutex> g(h->mu);
@@ -544,9 +596,66 @@ extern "C" int jf_handoff_submit(jf_handoff* h, const uint16_t* q_dev, const int
   return JF_OK;
 }
 
+extern "C" int jf_handoff_stream_submit(jf_handoff* h, const uint16_t* q_dev, const int64_t* topk_slots_dev, void* stream) {
+  JF_CHECK_ARG(h && q_dev && topk_slots_dev, "handoff_stream_submit: null argument");
+  JF_CHECK_ARG(((uintptr_t)q_dev & 15) == 0 && ((uintptr_t)topk_slots_dev & 15) == 0, "handoff_stream_submit: q and topk_slots must be 16-byte aligned");
+  if (h->failed.load() || __atomic_load_n(h->flag_pin + 16, __ATOMIC_ACQUIRE) != 0) {
+    set_error("handoff: an earlier CPU correction job failed or timed out");
+    return JF_ERR_TIMEOUT;
+  }
+  JF_CHECK_ARG(claim_mode(h, 2), "handoff_stream_submit: the context is in host mode (use jf_handoff_submit)");
+  {  // the dispatcher polls from now on
+    std::lock_guard<std::mutex> g(h->mu);
+  }
+  h->cv.notify_one();
+  const int nq16 = (int)((size_t)h->B * h->H_q * D * sizeof(uint16_t) / 16);
+  const int ns16 = (int)((size_t)h->B * h->H_q * h->K * sizeof(int64_t) / 16);
+  int blocks = (nq16 + ns16 + 255) / 256;
+  if (blocks > 32) blocks = 32;
+  hipLaunchKernelGGL(handoff_publish_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream,
+                     reinterpret_cast<const uint4*>(q_dev), reinterpret_cast<uint4*>(h->q_pin), nq16,
+                     reinterpret_cast<const uint4*>(topk_slots_dev), reinterpret_cast<uint4*>(h->ts_pin), ns16,
+                     h->counter_dev, h->flag_pin, (int64_t)0, reinterpret_cast<int64_t*>(h->counter_dev + 2));
+  JF_CHECK_HIP(hipGetLastError());
+  return JF_OK;
+}
+
+extern "C" int jf_handoff_stream_wait(jf_handoff* h, uint16_t* o_new_dev, void* stream) {
+  JF_CHECK_ARG(h && o_new_dev, "handoff_stream_wait: null argument");
+  JF_CHECK_ARG(((uintptr_t)o_new_dev & 15) == 0, "handoff_stream_wait: o_new must be 16-byte aligned");
+  JF_CHECK_ARG(h->mode.load() == 2, "handoff_stream_wait: no jf_handoff_stream_submit precedes it");
+  const int n16 = (int)((size_t)h->B * h->H_q * D * sizeof(uint16_t) / 16);
+  hipLaunchKernelGGL(handoff_wait_fetch_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, h->flag_pin + 8,
+                     reinterpret_cast<const int64_t*>(h->counter_dev + 2), h->flag_pin + 16, h->device_wait_ticks,
+                     reinterpret_cast<const uint4*>(h->o_pin), reinterpret_cast<uint4*>(o_new_dev), n16);
+  JF_CHECK_HIP(hipGetLastError());
+  return JF_OK;
+}
+
+extern "C" int jf_handoff_status(jf_handoff* h) {
+  JF_CHECK_ARG(h, "handoff_status: null argument");
+  const int64_t st = __atomic_load_n(h->flag_pin + 16, __ATOMIC_ACQUIRE);
+  if (st == 1) { set_error("handoff: the device-side wait for the CPU correction ran into its limit"); return JF_ERR_TIMEOUT; }
+  if (st != 0 || h->failed.load()) { set_error("handoff: a CPU correction job failed or timed out"); return JF_ERR_TIMEOUT; }
+  return JF_OK;
+}
+
+extern "C" int jf_handoff_set_device_wait_limit_us(jf_handoff* h, int64_t us) {
+  JF_CHECK_ARG(h && us > 0 && us <= 60000000, "handoff_set_device_wait_limit_us: limit must be in (0, 60 s]");
+  h->device_wait_ticks = (uint64_t)us * 100u;
+  return JF_OK;
+}
+
+extern "C" int jf_handoff_debug_pause(jf_handoff* h, int on) {
+  JF_CHECK_ARG(h, "handoff_debug_pause: null argument");
+  h->paused.store(on ? 1 : 0);
+  return JF_OK;
+}
+
 extern "C" int jf_handoff_wait(jf_handoff* h, uint16_t* o_new_dev, void* stream) {
   JF_CHECK_ARG(h && o_new_dev, "handoff_wait: null argument");
   JF_CHECK_ARG(((uintptr_t)o_new_dev & 15) == 0, "handoff_wait: o_new must be 16-byte aligned");
+  JF_CHECK_ARG(h->mode.load() != 2, "handoff_wait: the context is in stream mode (use jf_handoff_stream_wait)");
   hipStream_t st = (hipStream_t)stream;
   const int64_t want = h->host_seq.load();
   const auto t0 = std::chrono::steady_clock::now();
@@ -570,6 +679,8 @@ extern "C" int64_t jf_handoff_submit_count(const jf_handoff* h) { return h ? h->
 
 extern "C" void jf_handoff_destroy(jf_handoff* h) {
   if (!h) return;
+  // stream mode: kernels that poll or fill the pinned buffers may still be queued; they need the dispatcher alive
+  if (h->mode.load() == 2) (void)hipDeviceSynchronize();
   // a submit that was never waited for: its kernel still writes the pinned buffers and its job reads them
   if (h->dispatcher.joinable() && !h->failed.load()) {
     const auto t0 = std::chrono::steady_clock::now();

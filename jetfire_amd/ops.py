@@ -497,6 +497,32 @@ class CpuTopkHandoff:
                and o_new.shape == (B, H_q, HEAD_DIM), "o_new must be contiguous (B, H_q, 128) bf16 on the GPU")
         _lib.check(_lib.load().jf_handoff_wait(self._h, o_new.data_ptr(), _stream(o_new)))
 
+    def stream_submit(self, q, topk_slots) -> None:
+        """Graph-capturable submit (cpu_topk_attn.cpp:1805-1900 without the host callback): kernels only."""
+        B, H_q, K = self.shape
+        _check(q.is_cuda and q.dtype == torch.bfloat16 and q.is_contiguous() and q.shape == (B, H_q, HEAD_DIM),
+               "q must be contiguous (B, H_q, 128) bf16 on the GPU")
+        _check(topk_slots.is_cuda and topk_slots.dtype == torch.int64 and topk_slots.is_contiguous()
+               and topk_slots.shape == (B, H_q, K), "topk_slots must be contiguous (B, H_q, K) int64 on the GPU")
+        _lib.check(_lib.load().jf_handoff_stream_submit(self._h, q.data_ptr(), topk_slots.data_ptr(), _stream(q)))
+
+    def stream_wait(self, o_new) -> None:
+        """Graph-capturable join: a kernel waits (bounded) for the correction and brings o_new to the device."""
+        B, H_q, _ = self.shape
+        _check(o_new.is_cuda and o_new.dtype == torch.bfloat16 and o_new.is_contiguous()
+               and o_new.shape == (B, H_q, HEAD_DIM), "o_new must be contiguous (B, H_q, 128) bf16 on the GPU")
+        _lib.check(_lib.load().jf_handoff_stream_wait(self._h, o_new.data_ptr(), _stream(o_new)))
+
+    def check_status(self) -> None:
+        """Raises if a correction failed or a device-side wait ran into its limit (call after a synchronise)."""
+        _lib.check(_lib.load().jf_handoff_status(self._h))
+
+    def set_device_wait_limit_us(self, us: int) -> None:
+        _lib.check(_lib.load().jf_handoff_set_device_wait_limit_us(self._h, int(us)))
+
+    def debug_pause(self, on: bool) -> None:
+        _lib.check(_lib.load().jf_handoff_debug_pause(self._h, 1 if on else 0))
+
     @property
     def submit_count(self) -> int:
         return int(_lib.load().jf_handoff_submit_count(self._h))

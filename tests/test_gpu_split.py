@@ -341,3 +341,103 @@ def test_handoff_protocol_edges():
     h.submit(d["q"], slots)                                       # left outstanding on purpose
     h.close()                                                     # must wait for the job, then free
     torch.cuda.synchronize()
+
+
+def test_handoff_stream_mode_replays_from_a_hip_graph():
+    """The kernel-only submit / wait pair: eager calls, then a captured graph (publish, device-side wait, blend)
+    replayed with new queries and slots in the same buffers, eager work and synchronisations in between; every
+    result equals the host-blocking pair's on the same inputs."""
+    B, Hq, Hkv, K, S = 2, 8, 2, 32, 256
+    c = make_case(78, B, Hq, Hkv, S, 3, 2, 64, ragged=False)
+    o = ops()
+    ksh, vsh = bf16_tensor(c["K"]), bf16_tensor(c["V"])
+    o.set_cpu_attn_threads(2)
+    scale = 128 ** -0.5
+    rng = np.random.default_rng(1)
+    num_slots = ksh.shape[1]
+
+    def draw():
+        q = bf16_tensor(O.bf16_round((rng.standard_normal((B, Hq, 128)) / np.sqrt(128)).astype(np.float32))).cuda()
+        s = torch.from_numpy(np.stack([rng.choice(num_slots, K, replace=False) for _ in range(B * Hq)]).reshape(B, Hq, K)).cuda()
+        s[0, 0, :3] = -1                                          # padding entries are masked on the CPU side
+        return q, s
+
+    def host_pair(q, s):
+        h = o.CpuTopkHandoff(B, Hq, Hkv, K, ksh, vsh, scale)
+        out = torch.zeros(B, Hq, 128, dtype=torch.bfloat16, device="cuda")
+        h.submit(q, s)
+        h.wait(out)
+        torch.cuda.synchronize()
+        h.close()
+        return out
+
+    h = o.CpuTopkHandoff(B, Hq, Hkv, K, ksh, vsh, scale)
+    q_buf, s_buf = draw()
+    o_new = torch.zeros(B, Hq, 128, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(RuntimeError, match="stream_submit"):
+        h.stream_wait(o_new)                                      # nothing was submitted in this mode
+    for _ in range(2):                                            # eager
+        q, s = draw()
+        h.stream_submit(q, s)
+        h.stream_wait(o_new)
+        torch.cuda.synchronize()
+        h.check_status()
+        assert torch.equal(o_new.view(torch.int16), host_pair(q, s).view(torch.int16))
+    with pytest.raises(RuntimeError, match="stream mode"):
+        h.submit(q_buf, s_buf)                                    # one mode per context
+    o_hat = torch.randn(B, Hq, 128, device="cuda")
+    o_old = torch.randn(B, Hq, 128, device="cuda") * 0.1
+    W = torch.rand(B, Hq, device="cuda")
+    out = torch.zeros(B, Hq, 128, dtype=torch.bfloat16, device="cuda")
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        h.stream_submit(q_buf, s_buf)
+        h.stream_wait(o_new)
+        o.blend_unnorm_into(o_hat, o_old, W, o_new, out)
+    for step in range(4):
+        q, s = draw()
+        q_buf.copy_(q); s_buf.copy_(s)
+        graph.replay()
+        torch.cuda.synchronize()
+        h.check_status()
+        want_new = host_pair(q, s)
+        assert torch.equal(o_new.view(torch.int16), want_new.view(torch.int16)), step
+        want = torch.zeros_like(out)
+        o.blend_unnorm_into(o_hat, o_old, W, want_new, want)
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(torch.int16), want.view(torch.int16)), step
+    assert h.submit_count == 6
+    h.close()
+
+
+def test_handoff_stream_wait_is_bounded():
+    """A correction that never finishes (the dispatcher is told to ignore the flag): the device-side wait runs
+    into its limit, the kernel ends, o_new is zero, the status reports it, and later waits fall through."""
+    import time
+    B, Hq, Hkv, K = 1, 4, 2, 32
+    o = ops()
+    ksh = torch.zeros(Hkv, 64, 128, dtype=torch.bfloat16)
+    h = o.CpuTopkHandoff(B, Hq, Hkv, K, ksh, ksh, 0.1)
+    h.debug_pause(True)
+    h.set_device_wait_limit_us(20000)
+    q = torch.zeros(B, Hq, 128, dtype=torch.bfloat16, device="cuda")
+    s = torch.zeros(B, Hq, K, dtype=torch.int64, device="cuda")
+    o_new = torch.ones(B, Hq, 128, dtype=torch.bfloat16, device="cuda")
+    h.stream_submit(q, s)
+    h.stream_wait(o_new)
+    t0 = time.perf_counter()
+    torch.cuda.synchronize()
+    assert time.perf_counter() - t0 < 5.0
+    with pytest.raises(RuntimeError, match="limit"):
+        h.check_status()
+    assert float(o_new.float().abs().sum()) == 0.0
+    o_new.fill_(1)
+    h.stream_wait(o_new)                                          # falls through: no second 20 ms wait needed
+    torch.cuda.synchronize()
+    assert float(o_new.float().abs().sum()) == 0.0
+    with pytest.raises(RuntimeError, match="failed or timed out"):
+        h.stream_submit(q, s)
+    h.debug_pause(False)
+    h.close()
