@@ -138,7 +138,7 @@ def component_cpu_correction(args):
     q = (torch.randn(B, Hq, 128, generator=g) / 128 ** 0.5).to(torch.bfloat16)
     head_map = (torch.arange(Hq) // (Hq // Hkv))[None, :, None].expand(B, Hq, K).contiguous()
     o_new = torch.zeros(B, Hq, 128, dtype=torch.bfloat16)
-    threads = args.cpu_threads or 14
+    threads = args.cpu_threads
     ops.set_cpu_attn_threads(threads)
     ts = []
     for i in range(23):
@@ -183,18 +183,17 @@ def main() -> int:
     ap.add_argument("--paged", action="store_true", help="random block table instead of the identity mapping")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--graph", dest="graph", action="store_true", default=None,
-                    help="replay the step from a HIP graph (default without the hand-off; the roofline kernel timing "
-                         "comes from a separate eager pass)")
-    ap.add_argument("--eager", dest="graph", action="store_false", help="launch every kernel eagerly in the timed region")
+                    help="replay the step from a HIP graph (default; with the hand-off the graph holds the publish kernel "
+                         "and the device-side wait of every layer; the roofline kernel timing comes from a separate "
+                         "eager pass)")
+    ap.add_argument("--eager", dest="graph", action="store_false", help="launch every kernel eagerly in the timed region (with the hand-off: the host-blocking wait)")
     ap.add_argument("--handoff", dest="handoff", action="store_true", default=None,
                     help="include the pinned hand-off and the CPU correction per layer (default for c4 and c5, "
                          "whose definition is end to end)")
     ap.add_argument("--no-handoff", dest="handoff", action="store_false")
-    ap.add_argument("--cpu-threads", type=int, default=None,
-                    help="CPU correction worker threads (hand-off mode); default 14 of the box's 16 cores with the "
-                         "host-blocking wait (two stay free for the launching thread and the hand-off's dispatcher), 11 "
-                         "with --graph, where the runtime's own threads are busy too: one worker too many and a "
-                         "descheduled worker stretches every job to a scheduler time slice")
+    ap.add_argument("--cpu-threads", type=int, default=14,
+                    help="CPU correction worker threads (hand-off mode); the box gives 16 cores, two stay free for "
+                         "the launching thread and the hand-off's dispatcher / poller")
     ap.add_argument("--via-adapter", action="store_true",
                     help="hand-off mode only: run every layer through jetfire_amd.adapter.try_jetfire_decode (pool "
                          "manager, cache stores, dispatcher gate) instead of calling the operators directly")
@@ -242,10 +241,8 @@ def main() -> int:
     if args.split_len:
         _lib.check(lib.jf_debug_split_len(args.split_len))
     handoff = args.handoff if args.handoff is not None else args.workload in ("c4", "c5")
-    if args.cpu_threads is None:
-        args.cpu_threads = 11 if (handoff and args.graph) else 14
     if args.graph is None:
-        args.graph = not handoff
+        args.graph = not args.via_adapter
     if handoff and args.graph and args.via_adapter:
         print("bench.py: --graph with the hand-off goes through the operators, not the adapter", file=sys.stderr)
         return 2

@@ -226,8 +226,9 @@ void jf_handoff_destroy(jf_handoff* h);
  * jetfire_vllm/csrc/cpu_topk_attn.cpp:1805-2016, 1293-1344) without any host callback or stream memory
  * operation: both calls only enqueue kernels, so a captured graph replays them with no host code in between.
  * stream_submit: the publish kernel of jf_handoff_submit, except that the sequence number comes from a counter
- *         in device memory which the kernel advances itself; from the first call on the dispatcher thread polls
- *         the pinned flag continuously (with sleeps that lengthen while the GPU is silent).
+ *         in device memory which the kernel advances itself; from the first call on, ONE poller thread of the
+ *         process (shared by every stream-mode context: a model has one per layer and batch size) looks at the
+ *         context's pinned flag, with sleeps that lengthen while the GPU is silent, and runs the correction.
  * stream_wait: one workgroup whose first lane polls the pinned "finished" word until the correction of the
  *         device's current sequence number is done, then copies o_new into o_new_dev.  The wait is bounded
  *         (min(JETFIRE_CPU_FUTURE_TIMEOUT_S, 10 s); jf_handoff_set_device_wait_limit_us): at the limit the

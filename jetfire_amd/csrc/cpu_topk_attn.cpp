@@ -410,7 +410,9 @@ struct jf_handoff {
   unsigned* counter_dev = nullptr; // [0]: workgroups of the publish kernel that have finished; bytes 8..15: the
                                    // device's own sequence counter (stream mode)
   std::atomic<int> mode{0};        // 0 = not used yet, 1 = host-blocking wait, 2 = stream mode (device-side wait)
-  std::atomic<int> paused{0};      // test aid: the dispatcher ignores published flags
+  std::atomic<int> paused{0};      // test aid: published flags are ignored
+  int64_t stream_seen = 0;         // stream mode: last sequence number the shared poller has served
+  bool registered = false;         // stream mode: known to the shared poller
   uint64_t device_wait_ticks = 0;  // bound of the device-side wait, in ticks of the 100 MHz wall clock
   std::vector<int64_t> head_map;   // (B, H_q, K)
   std::atomic<int64_t> submits{0};
@@ -489,27 +491,32 @@ inline void cpu_relax() {
 #endif
 }
 
+bool run_correction(jf_handoff* h) {
+  CpuJob j{h->q_pin, h->k_shadow, h->v_shadow, h->head_map.data(), h->ts_pin, h->o_pin,
+           h->B, h->H_q, h->K, h->H_kv, h->num_slots, h->scale};
+  return Pool::instance().run((int64_t)h->B * h->H_q, [j](int64_t b, int64_t e) { run_rows(j, b, e); });
+}
+
+// Host mode: the context's own thread, asleep unless a submit is outstanding.
 void handoff_dispatch(jf_handoff* h) {
   int64_t seen = 0;
   for (;;) {
-    if (h->mode.load() != 2) {  // host mode with nothing outstanding: sleep until a submit (or the end)
+    {  // nothing outstanding: sleep until a submit (or the end)
       std::unique_lock<std::mutex> lk(h->mu);
-      h->cv.wait(lk, [&] { return h->stop.load() || h->host_seq.load() > seen || h->mode.load() == 2; });
+      h->cv.wait(lk, [&] { return h->stop.load() || h->host_seq.load() > seen; });
     }
     if (h->stop.load()) return;
-    const bool streaming = h->mode.load() == 2;
-    // poll the flag the publish kernel raises.  Stream mode: submits arrive from graph replays without any host
-    // call, so the thread keeps polling, with sleeps that lengthen while the GPU stays silent.
+    // a submit is in the stream: poll the flag the publish kernel raises
     const auto t0 = std::chrono::steady_clock::now();
     int64_t f = seen;
     for (uint64_t spin = 0;; ++spin) {
-      f = h->paused.load(std::memory_order_relaxed) ? seen : __atomic_load_n(h->flag_pin, __ATOMIC_ACQUIRE);
+      f = __atomic_load_n(h->flag_pin, __ATOMIC_ACQUIRE);
       if (f != seen || h->stop.load(std::memory_order_relaxed)) break;
       cpu_relax();
       if ((spin & 0xfff) == 0xfff) {
         const double el = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
-        if (!streaming && el > h->timeout_s) { h->failed.store(1); break; }
-        if (el > 0.002) std::this_thread::sleep_for(std::chrono::microseconds(streaming && el > 1.0 ? 200 : 50));
+        if (el > h->timeout_s) { h->failed.store(1); break; }
+        if (el > 0.002) std::this_thread::sleep_for(std::chrono::microseconds(50));  // a long GPU queue: stop burning a core
       }
     }
     if (h->stop.load()) return;
@@ -519,17 +526,82 @@ void handoff_dispatch(jf_handoff* h) {
       continue;
     }
     seen = f;
-    CpuJob j{h->q_pin, h->k_shadow, h->v_shadow, h->head_map.data(), h->ts_pin, h->o_pin,
-             h->B, h->H_q, h->K, h->H_kv, h->num_slots, h->scale};
-    if (!Pool::instance().run((int64_t)h->B * h->H_q, [j](int64_t b, int64_t e) { run_rows(j, b, e); })) {
-      h->failed.store(1);
-      __atomic_store_n(h->flag_pin + 16, (int64_t)2, __ATOMIC_RELEASE);
-    }
+    if (!run_correction(h)) h->failed.store(1);
     h->submits.fetch_add(1, std::memory_order_relaxed);
     h->done_seq.store(seen, std::memory_order_release);
-    __atomic_store_n(h->flag_pin + 8, seen, __ATOMIC_RELEASE);  // what the device-side wait polls
   }
 }
+
+// Stream mode: submits arrive from kernels (graph replays included) without any host call, so somebody has to
+// keep looking at the flags.  ONE thread of the process does that for every stream-mode context (a model has a
+// context per layer and batch size; a spinning thread each would eat the cores the correction needs): it walks
+// the registered contexts, serves a raised flag at once, and sleeps between walks, longer and longer, while the
+// GPU stays silent.  It is created on first use and lives until the process ends.
+struct StreamPoller {
+  std::mutex mu;
+  std::condition_variable cv;
+  std::vector<jf_handoff*> ctxs;
+
+  static StreamPoller& instance() {
+    static StreamPoller* p = [] {
+      StreamPoller* sp = new StreamPoller();
+      std::thread([sp] { sp->loop(); }).detach();
+      return sp;
+    }();
+    return *p;
+  }
+  void add(jf_handoff* h) {
+    {
+      std::lock_guard<std::mutex> g(mu);
+      ctxs.push_back(h);
+    }
+    cv.notify_one();
+  }
+  void remove(jf_handoff* h) {  // on return the poller does not touch h any more
+    std::lock_guard<std::mutex> g(mu);
+    for (size_t i = 0; i < ctxs.size(); ++i)
+      if (ctxs[i] == h) {
+        ctxs[i] = ctxs.back();
+        ctxs.pop_back();
+        break;
+      }
+  }
+  void loop() {
+    auto idle_since = std::chrono::steady_clock::now();
+    for (uint64_t walk = 0;; ++walk) {
+      bool served = false;
+      {
+        std::unique_lock<std::mutex> lk(mu);
+        if (ctxs.empty()) {
+          cv.wait(lk, [&] { return !ctxs.empty(); });
+          idle_since = std::chrono::steady_clock::now();
+        }
+        for (jf_handoff* h : ctxs) {
+          if (h->paused.load(std::memory_order_relaxed)) continue;
+          const int64_t f = __atomic_load_n(h->flag_pin, __ATOMIC_ACQUIRE);
+          if (f == h->stream_seen) continue;
+          h->stream_seen = f;
+          if (!run_correction(h)) {
+            h->failed.store(1);
+            __atomic_store_n(h->flag_pin + 16, (int64_t)2, __ATOMIC_RELEASE);
+          }
+          h->submits.fetch_add(1, std::memory_order_relaxed);
+          __atomic_store_n(h->flag_pin + 8, f, __ATOMIC_RELEASE);  // what the device-side wait polls
+          served = true;
+        }
+      }
+      if (served) {
+        idle_since = std::chrono::steady_clock::now();
+        continue;
+      }
+      cpu_relax();
+      if ((walk & 0x3ff) == 0x3ff) {
+        const double el = std::chrono::duration<double>(std::chrono::steady_clock::now() - idle_since).count();
+        if (el > 0.002) std::this_thread::sleep_for(std::chrono::microseconds(el > 1.0 ? 200 : 50));
+      }
+    }
+  }
+};
 
 bool claim_mode(jf_handoff* h, int mode) {
   int expected = 0;
@@ -604,10 +676,10 @@ extern "C" int jf_handoff_stream_submit(jf_handoff* h, const uint16_t* q_dev, co
     return JF_ERR_TIMEOUT;
   }
   JF_CHECK_ARG(claim_mode(h, 2), "handoff_stream_submit: the context is in host mode (use jf_handoff_submit)");
-  {  // the dispatcher polls from now on
-    std::lock_guard<std::mutex> g(h->mu);
+  if (!h->registered) {  // the shared poller looks at this context's flag from now on
+    h->registered = true;
+    StreamPoller::instance().add(h);
   }
-  h->cv.notify_one();
   const int nq16 = (int)((size_t)h->B * h->H_q * D * sizeof(uint16_t) / 16);
   const int ns16 = (int)((size_t)h->B * h->H_q * h->K * sizeof(int64_t) / 16);
   int blocks = (nq16 + ns16 + 255) / 256;
@@ -681,6 +753,7 @@ extern "C" void jf_handoff_destroy(jf_handoff* h) {
   if (!h) return;
   // stream mode: kernels that poll or fill the pinned buffers may still be queued; they need the dispatcher alive
   if (h->mode.load() == 2) (void)hipDeviceSynchronize();
+  if (h->registered) StreamPoller::instance().remove(h);
   // a submit that was never waited for: its kernel still writes the pinned buffers and its job reads them
   if (h->dispatcher.joinable() && !h->failed.load()) {
     const auto t0 = std::chrono::steady_clock::now();
