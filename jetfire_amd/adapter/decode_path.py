@@ -4,8 +4,14 @@ layer's attention for a batch of single-token queries over the quantised cache,
     fused scan + top-k  ->  pinned hand-off + CPU correction over the bf16 shadow  ->  blend into `output`.
 
 `try_jetfire_decode` returns `output` on success and None when a precondition fails (the caller then uses
-its native attention); every miss is recorded with the reference's reason string.  The reference's trace
-hooks, CUDA-graph capture mode, release policy and debug correction modes are not reproduced."""
+its native attention); every miss is recorded with the reference's reason string.
+
+Graph mode (`JETFIRE_DECODE_GRAPH=1`, `decode_path.py:634-646`): the hand-off uses the kernel-only submit /
+wait pair, nothing in the entry synchronises with the device, and the whole layer can be captured into a HIP
+graph and replayed; `warmup_graph_decode_submit_contexts` creates, before capture, whatever a capture may
+not allocate.  A miss while a graph is being captured raises instead of baking the caller's fall-back into
+the graph (`:698-706`).  The reference's trace hooks, release policy and debug correction modes are not
+reproduced."""
 from __future__ import annotations
 
 import math
@@ -54,13 +60,50 @@ def _get_head_map_cpu(B: int, H_q: int, num_groups: int, K: int) -> torch.Tensor
     return hm
 
 
+def _graph_mode_enabled() -> bool:
+    return os.environ.get("JETFIRE_DECODE_GRAPH", "0") == "1"
+
+
+def _graph_capture_active() -> bool:
+    return torch.cuda.is_available() and torch.cuda.is_current_stream_capturing()
+
+
+def _graph_context_batch_sizes(max_batch_size: int) -> list[int]:
+    """Batch sizes whose hand-off contexts must exist before capture: all of 1..max, or the sizes listed in
+    `JETFIRE_GRAPH_CAPTURE_SIZES` plus the maximum (`decode_path.py:668-695`)."""
+    if max_batch_size <= 0:
+        return []
+    raw = os.environ.get("JETFIRE_GRAPH_CAPTURE_SIZES", "").strip()
+    if not raw:
+        return list(range(1, max_batch_size + 1))
+    out = {max_batch_size}
+    for part in raw.replace(";", ",").split(","):
+        part = part.strip()
+        if not part:
+            continue
+        try:
+            value = int(part)
+        except ValueError:
+            raise RuntimeError("JETFIRE_GRAPH_CAPTURE_SIZES must be a comma-separated list of integers; "
+                               f"got {raw!r}") from None
+        if 1 <= value <= max_batch_size:
+            out.add(value)
+    return sorted(out)
+
+
+def _raise_graph_decode_miss(reason: str, *, layer_name: str) -> None:
+    raise RuntimeError("JetFire graph decode miss would fall back to native attention and poison the captured "
+                       f"graph. reason={reason} layer={layer_name}. Pre-create JetFire stores and graph submit "
+                       "contexts before the decode step is captured, or disable JETFIRE_DECODE_GRAPH.")
+
+
 def _decode_unsupported(*, impl, layer, query, attn_metadata) -> str | None:
     """Dispatcher gate: the reason string of a miss, or None."""
     pool = get_global_kv_pool_manager()
     if not pool.config.enabled:
         return "pool_disabled"
-    if query.is_cuda and torch.cuda.is_current_stream_capturing():
-        return "cuda_graph_capture"          # the hand-off blocks the host: not capturable
+    if query.is_cuda and torch.cuda.is_current_stream_capturing() and not _graph_mode_enabled():
+        return "cuda_graph_capture"          # the host-blocking hand-off cannot be captured
     if attn_metadata is None:
         return "profiling_run"
     attn_type = getattr(impl, "attn_type", None)
@@ -100,16 +143,64 @@ def _seq_lens_on_host(seq_lens: torch.Tensor) -> torch.Tensor:
     return host
 
 
-def _handoff_for(store, B: int, H_q: int, H_kv: int, K: int, scale: float):
-    key = (id(store), B, H_q, K, float(scale))
+def _handoff_for(store, B: int, H_q: int, H_kv: int, K: int, scale: float, *, stream_mode: bool = False,
+                 layer_name: str = "unknown_layer"):
+    # a context serves one of the two modes
+    key = (id(store), B, H_q, K, float(scale), bool(stream_mode))
     h = _HANDOFFS.get(key)
     if h is None:
+        if _graph_capture_active():        # pinned allocations and thread start-up are not capturable
+            _raise_graph_decode_miss("submit_context_missing", layer_name=layer_name)
         threads = get_jetfire_config().cpu_attn_threads
         if threads > 0:
             ops.set_cpu_attn_threads(threads)
         h = ops.CpuTopkHandoff(B, H_q, H_kv, K, store.k_shadow, store.v_shadow, scale)
         _HANDOFFS[key] = h
     return h
+
+
+def _o_new_for(n_seqs: int, H_q: int, D: int, device) -> torch.Tensor:
+    key = (n_seqs, H_q, torch.device(device))
+    o_new = _O_NEW.get(key)
+    if o_new is None:
+        o_new = _O_NEW[key] = torch.empty(n_seqs, H_q, D, dtype=torch.bfloat16, device=device)
+    return o_new
+
+
+def warmup_graph_decode_submit_contexts(*, max_batch_size: int, device=None, scale: float | None = None) -> dict:
+    """Create, before a decode step is captured, the graph-mode hand-off contexts (pinned buffers, poller
+    registration happens on first submit) of every mirrored layer for every captured batch size and every
+    correction width up to the configured one, the `o_new` buffers, and the stores' append state
+    (`decode_path.py:851-1015`).  `scale` is the attention scale the layers use (default head_dim ** -0.5)."""
+    if max_batch_size <= 0:
+        raise RuntimeError("JETFIRE_DECODE_GRAPH=1 requires JETFIRE_MAX_BATCH_SIZE>0 so decode host buffers and "
+                           "submit contexts have stable pointers before graph capture.")
+    cfg = get_jetfire_config()
+    if not cfg.cpu_correction:
+        raise RuntimeError("JETFIRE_DECODE_GRAPH=1 currently requires JETFIRE_CPU_CORRECTION=1.")
+    pool = get_global_kv_pool_manager()
+    if not pool.layer_stores:
+        raise RuntimeError("JETFIRE_DECODE_GRAPH=1 cannot warm submit contexts before JetFire layer stores exist.")
+    top_k = _select_top_k(cfg.topk, cfg.topk, FUSED_SUPPORTED_TOP_K)
+    if top_k is None:
+        raise RuntimeError(f"JETFIRE_TOPK={cfg.topk} is not supported by the active kernel set.")
+    widths = tuple(k for k in FUSED_SUPPORTED_TOP_K if k <= top_k) or (top_k,)
+    sizes = _graph_context_batch_sizes(int(max_batch_size))
+    created = 0
+    for name, store in pool.layer_stores.items():
+        layer_cfg = pool.get_layer_config(name)
+        if layer_cfg is None or store.scheme is None or not store.shadow_enabled:
+            continue
+        store.warmup_graph_append(int(max_batch_size))
+        sc = float(scale) if scale is not None else 1.0 / math.sqrt(layer_cfg.head_dim)
+        for n in sizes:
+            _o_new_for(n, layer_cfg.num_query_heads, layer_cfg.head_dim, device if device is not None else store.device)
+            for k in widths:
+                before = len(_HANDOFFS)
+                _handoff_for(store, n, layer_cfg.num_query_heads, layer_cfg.num_kv_heads, k, sc, stream_mode=True,
+                             layer_name=name)
+                created += len(_HANDOFFS) - before
+    return {"layers": len(pool.layer_stores), "batch_sizes": sizes, "top_k": list(widths), "contexts_created": created}
 
 
 def reset_jetfire_decode_runtime_state() -> None:
@@ -132,41 +223,49 @@ def _decode_batched(*, impl, layer, query, attn_metadata, output):
     pool.record_decode_attempt()
     layer_name = getattr(layer, "layer_name", "unknown_layer")
     pool.ensure_layer_config_from_layer(layer_name, layer)
+    graph_mode = _graph_mode_enabled()
+
+    def miss(reason: str):
+        pool.record_decode_fallback(reason)
+        if graph_mode and _graph_capture_active():
+            _raise_graph_decode_miss(reason, layer_name=layer_name)
+        return None
+
     reason = _decode_unsupported(impl=impl, layer=layer, query=query, attn_metadata=attn_metadata)
     if reason is not None:
-        pool.record_decode_fallback(reason)
-        return None
+        return miss(reason)
     if not get_jetfire_config().cpu_correction:
-        pool.record_decode_fallback("cpu_correction_disabled")
-        return None
+        return miss("cpu_correction_disabled")
     layer_cfg = pool.get_layer_config(layer_name)
     store = pool.get_layer_store(layer_name)
     if store is None:
-        pool.record_decode_fallback("store_missing")
-        return None
+        return miss("store_missing")
     if store.scheme is None or store.block_size != 16 or layer_cfg.head_dim != 128 or not store.shadow_enabled:
-        pool.record_decode_fallback("scheme_unsupported")
-        return None
+        return miss("scheme_unsupported")
     store.flush_pending_writes()
 
     n_seqs = int(attn_metadata.seq_lens.numel())
-    seq_lens_cpu = _seq_lens_on_host(attn_metadata.seq_lens)
-    if os.environ.get("JETFIRE_FAST_STORE_COMPLETE_CHECK", "0") == "1":
-        complete = store.fast_has_sequence(int(seq_lens_cpu.max().item()))      # host-side counter, no sync per sequence
-    else:
-        complete = all(n <= 0 or store.has_sequence(attn_metadata.block_table[i], int(n))
-                       for i, n in enumerate(seq_lens_cpu.tolist()))
-    if not complete:
-        pool.record_decode_fallback("store_incomplete")
-        return None
-
     H_q, H_kv, D = layer_cfg.num_query_heads, layer_cfg.num_kv_heads, layer_cfg.head_dim
     scale = float(getattr(impl, "scale", 1.0 / math.sqrt(D)))
-    max_S = int(getattr(attn_metadata, "max_seq_len", int(seq_lens_cpu.max().item())))
+    if graph_mode:
+        # no device-to-host copy of the lengths and no completeness check: they would block a capture; the
+        # caller guarantees that the stores hold the sequences (decode_path.py:1749-1755)
+        max_S = int(getattr(attn_metadata, "max_seq_len", 0) or 0)
+        if max_S <= 0:
+            return miss("max_seq_len_missing")
+    else:
+        seq_lens_cpu = _seq_lens_on_host(attn_metadata.seq_lens)
+        if os.environ.get("JETFIRE_FAST_STORE_COMPLETE_CHECK", "0") == "1":
+            complete = store.fast_has_sequence(int(seq_lens_cpu.max().item()))      # host-side counter, no sync per sequence
+        else:
+            complete = all(n <= 0 or store.has_sequence(attn_metadata.block_table[i], int(n))
+                           for i, n in enumerate(seq_lens_cpu.tolist()))
+        if not complete:
+            return miss("store_incomplete")
+        max_S = int(getattr(attn_metadata, "max_seq_len", int(seq_lens_cpu.max().item())))
     top_k = _select_top_k(pool.config.topk, max_S, FUSED_SUPPORTED_TOP_K)
     if top_k is None:
-        pool.record_decode_fallback("seq_len_too_short")
-        return None
+        return miss("seq_len_too_short")
 
     q_batch = query[:n_seqs].contiguous().view(n_seqs, H_q, D).to(torch.bfloat16)
     bt_batch = attn_metadata.block_table[:n_seqs].to(torch.int64).contiguous()
@@ -175,12 +274,14 @@ def _decode_batched(*, impl, layer, query, attn_metadata, output):
     o_hat, topk_slots, o_old, W, _ = ops.fused_attn_topk(
         store.scheme, q_batch, store.k_data, store.k_scales, store.v_data, store.v_scales, bt_batch, seq_lens_batch,
         max_S, H_q, H_kv, store.block_size, top_k, scale)
-    handoff = _handoff_for(store, n_seqs, H_q, H_kv, top_k, scale)
-    handoff.submit(q_batch, topk_slots)
-    o_new = _O_NEW.get((n_seqs, H_q, query.device))
-    if o_new is None:
-        o_new = _O_NEW[(n_seqs, H_q, query.device)] = torch.empty(n_seqs, H_q, D, dtype=torch.bfloat16, device=query.device)
-    handoff.wait(o_new)
+    handoff = _handoff_for(store, n_seqs, H_q, H_kv, top_k, scale, stream_mode=graph_mode, layer_name=layer_name)
+    o_new = _o_new_for(n_seqs, H_q, D, query.device)
+    if graph_mode:          # kernels only: nothing here waits for the CPU
+        handoff.stream_submit(q_batch, topk_slots)
+        handoff.stream_wait(o_new)
+    else:
+        handoff.submit(q_batch, topk_slots)
+        handoff.wait(o_new)
 
     out_view = output[:n_seqs].view(n_seqs, H_q, D)
     if out_view.dtype == torch.bfloat16 and out_view.is_contiguous():

@@ -122,7 +122,11 @@ class JetFireKVPoolManager:
             raise RuntimeError(f"JetFire layer config mismatch for {layer_name}: expected "
                                f"({config.num_kv_heads}, {config.head_dim}), got ({int(key.shape[1])}, {int(key.shape[2])})")
         store = self._get_or_create_store(layer_name=layer_name, device=key.device)
-        written = store.write_slots(key=key, value=value, slot_mapping=slot_mapping)
+        if key.is_cuda and torch.cuda.is_current_stream_capturing():
+            written = store.write_slots_graph(key=key, value=value, slot_mapping=slot_mapping,
+                                              max_batch_size=get_jetfire_config().max_batch_size)
+        else:
+            written = store.write_slots(key=key, value=value, slot_mapping=slot_mapping)
         if written > 0:
             self.token_counters[layer_name] = self.token_counters.get(layer_name, 0) + written
             self.written_slots += written

@@ -302,3 +302,111 @@ def test_decode_append_replays_from_a_hip_graph():
         assert torch.equal(_bits(store.v_shadow), _bits(eager.v_shadow)), step
         keep = s >= 0
         assert torch.equal(_bits(store.k_shadow[:, s[keep]]), _bits(k.permute(1, 0, 2)[:, keep].contiguous())), step
+
+
+@pytest.mark.gpu
+def test_graph_mode_decode_step_replays_against_the_oracle(adapter, monkeypatch):
+    """JETFIRE_DECODE_GRAPH=1: two layers' append + decode captured once into a HIP graph (quantise-on-write,
+    shadow mirror kernel, fused scan, merge, publish, device-side wait, blend) and replayed for three decode
+    steps with new tokens, slots, lengths and queries in the same buffers; every step is checked against the
+    oracle, and a miss during capture raises."""
+    monkeypatch.setenv("JETFIRE_DECODE_GRAPH", "1")
+    B, Hq, Hkv, D, bs, K, max_S = 2, 8, 2, 128, 16, 32, 160
+    gs, kb, vb, scheme = 64, 3, 2, "k3v2"
+    lens0 = [100, 70]
+    adapter.set_jetfire_config(scheme="SymInt3K_SymInt2V", group_size=gs, topk=K, layer_stride=1, cpu_attn_threads=2,
+                               max_batch_size=B)
+    adapter.reset_global_kv_pool_manager()
+    pool = adapter.get_global_kv_pool_manager()
+    names = [f"model.layers.{i}.self_attn.attn" for i in range(2)]
+    layers = [types.SimpleNamespace(layer_name=n, num_heads=Hq, num_kv_heads=Hkv, head_size=D) for n in names]
+    impl = types.SimpleNamespace(attn_type=types.SimpleNamespace(name="DECODER"), scale=D ** -0.5)
+    rng = np.random.default_rng(21)
+    per_seq = max_S // bs
+    nblk = B * per_seq + 1
+    bt = rng.permutation(nblk)[:B * per_seq].reshape(B, per_seq).astype(np.int64)
+    bt_dev = torch.from_numpy(bt).cuda()
+
+    def slot_of(b, pos):
+        return int(bt[b, pos // bs]) * bs + pos % bs
+
+    def new_kv(n):
+        k = O.bf16_round(rng.standard_normal((n, Hkv, D)).astype(np.float32))
+        k[..., [3, 40, 77, 101]] *= 8
+        return O.bf16_round(k), O.bf16_round(rng.standard_normal((n, Hkv, D)).astype(np.float32))
+
+    Kfull = [np.zeros((Hkv, nblk * bs, D), np.float32) for _ in names]
+    Vfull = [np.zeros((Hkv, nblk * bs, D), np.float32) for _ in names]
+    toks = [(b, p) for b in range(B) for p in range(lens0[b])]
+    slot_map = np.array([slot_of(b, p) for b, p in toks], dtype=np.int64)
+    for li, (name, layer) in enumerate(zip(names, layers)):
+        pool.ensure_layer_config_from_layer(name, layer)
+        pool.register_layer_layout(name, num_blocks=nblk, block_size=bs)
+        k_np, v_np = new_kv(len(toks))
+        pool.mirror_kv(name, bf16_tensor(k_np).cuda(), bf16_tensor(v_np).cuda(), torch.from_numpy(slot_map).cuda())
+        Kfull[li][:, slot_map] = k_np.transpose(1, 0, 2)
+        Vfull[li][:, slot_map] = v_np.transpose(1, 0, 2)
+    pool.flush_pending_writes()
+
+    # static buffers of the captured step
+    key_buf = [torch.zeros(B, Hkv, D, dtype=torch.bfloat16, device="cuda") for _ in names]
+    val_buf = [torch.zeros(B, Hkv, D, dtype=torch.bfloat16, device="cuda") for _ in names]
+    q_buf = [torch.zeros(B, Hq, D, dtype=torch.bfloat16, device="cuda") for _ in names]
+    out_buf = [torch.zeros(B, Hq * D, dtype=torch.bfloat16, device="cuda") for _ in names]
+    slot_buf = torch.full((B,), -1, dtype=torch.int64, device="cuda")
+    seq_lens = torch.tensor(lens0, dtype=torch.int32, device="cuda")
+    meta = _meta(seq_lens, bt_dev, max_seq_len=max_S)
+
+    def step():
+        for li, (name, layer) in enumerate(zip(names, layers)):
+            pool.mirror_kv(name, key_buf[li], val_buf[li], slot_buf)
+            got = adapter.try_jetfire_decode(impl=impl, layer=layer, query=q_buf[li], attn_metadata=meta, output=out_buf[li])
+            assert got is out_buf[li]
+
+    # a capture without the pre-created contexts must raise, not record a fall-back
+    probe = torch.cuda.CUDAGraph()
+    with pytest.raises(RuntimeError, match="submit_context_missing"):
+        with torch.cuda.graph(probe):
+            step()
+    del probe
+    info = adapter.warmup_graph_decode_submit_contexts(max_batch_size=B)
+    assert info["contexts_created"] == 2 * B and info["top_k"] == [32]
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()                                     # warm-up: all-padding append, decode of the prefill
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+
+    lens = list(lens0)
+    for it in range(3):
+        sm = np.array([slot_of(b, lens[b]) for b in range(B)], dtype=np.int64)
+        slot_buf.copy_(torch.from_numpy(sm).cuda())
+        lens = [n + 1 for n in lens]
+        seq_lens.copy_(torch.tensor(lens, dtype=torch.int32).cuda())
+        q_np = []
+        for li in range(len(names)):
+            k_np, v_np = new_kv(B)
+            key_buf[li].copy_(bf16_tensor(k_np).cuda()); val_buf[li].copy_(bf16_tensor(v_np).cuda())
+            Kfull[li][:, sm] = k_np.transpose(1, 0, 2)
+            Vfull[li][:, sm] = v_np.transpose(1, 0, 2)
+            q_np.append(O.bf16_round((rng.standard_normal((B, Hq, D)) / np.sqrt(D)).astype(np.float32)))
+            q_buf[li].copy_(bf16_tensor(q_np[li]).cuda())
+        graph.replay()
+        torch.cuda.synchronize()
+        for li, name in enumerate(names):
+            store = pool.get_layer_store(name)
+            assert np.array_equal(bf16_to_f32(store.k_shadow)[:, sm], Kfull[li][:, sm])
+            ref_kd, ref_ks = O.quantize_and_pack(Kfull[li], gs, kb)
+            ref_vd, ref_vs = O.quantize_and_pack(Vfull[li], gs, vb)
+            assert np.array_equal(store.k_data.cpu().numpy()[:, sm], ref_kd[:, sm])
+            r = O.decode_reference(q_np[li], ref_kd, ref_ks, ref_vd, ref_vs, bt, np.array(lens, np.int32), max(lens), Hq, Hkv,
+                                   bs, D ** -0.5, K, scheme, Kfull[li], Vfull[li])
+            res = bf16_to_f32(out_buf[li]).reshape(B, Hq, D)
+            np.testing.assert_allclose(res, r["out"], atol=6e-3, rtol=1.5e-2, err_msg=f"step {it} layer {li}")
+            err = np.abs(res - r["out"])
+            assert err.max() <= 2e-2 and err.mean() <= 1e-3
+    del graph
