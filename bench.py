@@ -300,12 +300,12 @@ def main() -> int:
                 w.S, w.H_q, w.H_kv, 16, w.top_k, w.attn_scale)
             if ctxs:
                 h = ctxs[li % len(ctxs)]
-                if args.graph:      # kernels only: the publish kernel and a device-side wait
+                if args.graph:      # kernels only: the publish kernel, then a device-side wait that also blends
                     h.stream_submit(w.q, slots)
-                    h.stream_wait(o_new)
-                else:
-                    h.submit(w.q, slots)
-                    h.wait(o_new)
+                    h.stream_wait_blend(o_hat, o_old, W, out)
+                    continue
+                h.submit(w.q, slots)
+                h.wait(o_new)
             ops.blend_unnorm_into(o_hat, o_old, W, o_new, out)
 
     for _ in range(args.warmup):

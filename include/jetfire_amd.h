@@ -203,7 +203,7 @@ int jf_get_cpu_attn_threads(void);
  * stream_wait_cpu_topk_attn (jetfire_vllm/csrc/cpu_topk_attn.cpp:2054-2163, 2239, 2302) and the
  * pinned copies around them (jetfire_vllm/adapter/decode_path.py:2243-2267, 3107-3114).
  * submit: enqueues one small kernel on `stream` that copies q and topk_slots (both 16-byte aligned,
- *         K even) into pinned host buffers and then raises a sequence flag in pinned memory; a
+ *         K a multiple of 4; the slots cross PCIe as 32-bit values) into pinned host buffers and then raises a sequence flag in pinned memory; a
  *         dispatcher thread of the context polls that flag and runs the CPU correction on the worker
  *         pool as soon as the GPU has reached it.  Returns at once.
  * wait:   blocks the calling host thread until the correction of the last submit has finished (as the
@@ -240,6 +240,11 @@ void jf_handoff_destroy(jf_handoff* h);
  * will be replayed again; destroy synchronises the device first. */
 int jf_handoff_stream_submit(jf_handoff* h, const uint16_t* q_dev, const int64_t* topk_slots_dev, void* stream);
 int jf_handoff_stream_wait(jf_handoff* h, uint16_t* o_new_dev, void* stream);
+/* stream_wait followed by the blend of jf_blend_unnorm in the same kernel: out = bf16(fma(W, o_new, o_hat) -
+ * o_old_unnorm) on the elements as they arrive (at the wait's limit o_new counts as zero).  o_new_dev may be
+ * NULL when the caller has no use for the correction itself. */
+int jf_handoff_stream_wait_blend(jf_handoff* h, const float* o_hat, const float* o_old_unnorm, const float* W,
+                                 uint16_t* out, uint16_t* o_new_dev, void* stream);
 int jf_handoff_status(jf_handoff* h);
 int jf_handoff_set_device_wait_limit_us(jf_handoff* h, int64_t us);
 /* Test aid: while on, the dispatcher ignores published flags (a correction that never finishes, without

@@ -47,6 +47,7 @@ SIGNATURES = {
     "jf_handoff_submit_count": (L, [P]),
     "jf_handoff_stream_submit": (I, [P, P, P, P]),
     "jf_handoff_stream_wait": (I, [P, P, P]),
+    "jf_handoff_stream_wait_blend": (I, [P, P, P, P, P, P, P]),
     "jf_handoff_status": (I, [P]),
     "jf_handoff_set_device_wait_limit_us": (I, [P, L]),
     "jf_handoff_debug_pause": (I, [P, I]),

@@ -276,15 +276,19 @@ def _decode_batched(*, impl, layer, query, attn_metadata, output):
         max_S, H_q, H_kv, store.block_size, top_k, scale)
     handoff = _handoff_for(store, n_seqs, H_q, H_kv, top_k, scale, stream_mode=graph_mode, layer_name=layer_name)
     o_new = _o_new_for(n_seqs, H_q, D, query.device)
+    out_view = output[:n_seqs].view(n_seqs, H_q, D)
+    direct = out_view.dtype == torch.bfloat16 and out_view.is_contiguous()
     if graph_mode:          # kernels only: nothing here waits for the CPU
         handoff.stream_submit(q_batch, topk_slots)
+        if direct:          # the device-side wait blends as the correction arrives
+            handoff.stream_wait_blend(o_hat, o_old, W, out_view)
+            pool.record_decode_hit()
+            return output
         handoff.stream_wait(o_new)
     else:
         handoff.submit(q_batch, topk_slots)
         handoff.wait(o_new)
-
-    out_view = output[:n_seqs].view(n_seqs, H_q, D)
-    if out_view.dtype == torch.bfloat16 and out_view.is_contiguous():
+    if direct:
         ops.blend_unnorm_into(o_hat, o_old, W, o_new, out_view)
     else:
         tmp = torch.empty(n_seqs, H_q, D, dtype=torch.bfloat16, device=query.device)

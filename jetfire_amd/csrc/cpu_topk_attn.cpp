@@ -205,15 +205,18 @@ class Pool {
 static inline float bf(uint16_t b) { return bf16_to_f32(b); }
 
 // One (sequence, query head) row.  fp32 accumulation in ascending channel / slot order.
+// SlotT: int64 (the operator's ts_buf) or int32 (the hand-off's own pinned buffer).  head_map == nullptr: every
+// slot of the row reads kv-head `fixed_h`.
+template <typename SlotT>
 static void topk_attn_row(const uint16_t* q, const uint16_t* k_shadow, const uint16_t* v_shadow, int64_t num_slots,
-                          const int64_t* head_map, const int64_t* slots, int K, int H_kv, float scale, uint16_t* out,
-                          float* score_buf) {
+                          const int64_t* head_map, int64_t fixed_h, const SlotT* slots, int K, int H_kv, float scale,
+                          uint16_t* out, float* score_buf) {
   float qf[D];
   for (int i = 0; i < D; ++i) qf[i] = bf(q[i]);
   float mx = -INFINITY;
   bool any = false;
   for (int k = 0; k < K; ++k) {
-    const int64_t s = slots[k], h = head_map[k];
+    const int64_t s = slots[k], h = head_map ? head_map[k] : fixed_h;
     if (s < 0 || s >= num_slots || h < 0 || h >= H_kv) {
       score_buf[k] = -INFINITY;
       continue;
@@ -245,7 +248,7 @@ static void topk_attn_row(const uint16_t* q, const uint16_t* k_shadow, const uin
   float o[D];
   for (int i = 0; i < D; ++i) o[i] = 0.0f;
   for (int k = 0; k < K; ++k) {
-    const int64_t s = slots[k], h = head_map[k];
+    const int64_t s = slots[k], h = head_map ? head_map[k] : fixed_h;
     if (s < 0 || s >= num_slots || h < 0 || h >= H_kv) continue;
     const uint16_t* vr = v_shadow + ((size_t)h * num_slots + s) * D;
     const float w = score_buf[k] * inv;
@@ -260,15 +263,17 @@ static void topk_attn_row(const uint16_t* q, const uint16_t* k_shadow, const uin
 __attribute__((target("avx2,fma"))) static inline __m256 bf16x8_to_f32(const uint16_t* p) {
   return _mm256_castsi256_ps(_mm256_slli_epi32(_mm256_cvtepu16_epi32(_mm_loadu_si128(reinterpret_cast<const __m128i*>(p))), 16));
 }
+template <typename SlotT>
 __attribute__((target("avx2,fma"))) static void topk_attn_row_avx2(const uint16_t* q, const uint16_t* k_shadow,
                                                                    const uint16_t* v_shadow, int64_t num_slots,
-                                                                   const int64_t* head_map, const int64_t* slots, int K,
-                                                                   int H_kv, float scale, uint16_t* out, float* score_buf) {
+                                                                   const int64_t* head_map, int64_t fixed_h,
+                                                                   const SlotT* slots, int K, int H_kv, float scale,
+                                                                   uint16_t* out, float* score_buf) {
   constexpr int AHEAD = 8;
   __m256 qv[D / 8];
   for (int i = 0; i < D / 8; ++i) qv[i] = bf16x8_to_f32(q + 8 * i);
   auto row_of = [&](const uint16_t* base, int k) -> const uint16_t* {
-    const int64_t s = slots[k], h = head_map[k];
+    const int64_t s = slots[k], h = head_map ? head_map[k] : fixed_h;
     if (s < 0 || s >= num_slots || h < 0 || h >= H_kv) return nullptr;
     return base + ((size_t)h * num_slots + s) * D;
   };
@@ -339,27 +344,35 @@ static bool host_has_avx2_fma() { return false; }
 
 struct CpuJob {
   const uint16_t *q, *k_shadow, *v_shadow;
-  const int64_t *head_map, *ts_buf;
+  const int64_t *head_map, *ts_buf;  // head_map may be null (kv-head = query head / (H_q / H_kv)); ts_buf or ts32
   uint16_t* o_new;
   int B, H_q, K, H_kv;
   int64_t num_slots;
   float scale;
+  const int32_t* ts32 = nullptr;     // 32-bit slots instead of ts_buf
 };
 
-static void run_rows(const CpuJob& j, int64_t b, int64_t e) {
-  static thread_local std::vector<float> buf;
-  if (buf.size() < (size_t)j.K) buf.resize((size_t)j.K);
+template <typename SlotT>
+static void run_rows_t(const CpuJob& j, const SlotT* ts, int64_t b, int64_t e, float* buf) {
+  const int G = j.H_q / j.H_kv;
 #if defined(__x86_64__)
   if (host_has_avx2_fma()) {
     for (int64_t r = b; r < e; ++r)
-      topk_attn_row_avx2(j.q + r * D, j.k_shadow, j.v_shadow, j.num_slots, j.head_map + r * j.K, j.ts_buf + r * j.K, j.K,
-                         j.H_kv, j.scale, j.o_new + r * D, buf.data());
+      topk_attn_row_avx2<SlotT>(j.q + r * D, j.k_shadow, j.v_shadow, j.num_slots, j.head_map ? j.head_map + r * j.K : nullptr,
+                                (r % j.H_q) / G, ts + r * j.K, j.K, j.H_kv, j.scale, j.o_new + r * D, buf);
     return;
   }
 #endif
   for (int64_t r = b; r < e; ++r)
-    topk_attn_row(j.q + r * D, j.k_shadow, j.v_shadow, j.num_slots, j.head_map + r * j.K, j.ts_buf + r * j.K, j.K, j.H_kv,
-                  j.scale, j.o_new + r * D, buf.data());
+    topk_attn_row<SlotT>(j.q + r * D, j.k_shadow, j.v_shadow, j.num_slots, j.head_map ? j.head_map + r * j.K : nullptr,
+                         (r % j.H_q) / G, ts + r * j.K, j.K, j.H_kv, j.scale, j.o_new + r * D, buf);
+}
+
+static void run_rows(const CpuJob& j, int64_t b, int64_t e) {
+  static thread_local std::vector<float> buf;
+  if (buf.size() < (size_t)j.K) buf.resize((size_t)j.K);
+  if (j.ts32) run_rows_t<int32_t>(j, j.ts32, b, e, buf.data());
+  else run_rows_t<int64_t>(j, j.ts_buf, b, e, buf.data());
 }
 
 }  // namespace jf
@@ -403,7 +416,7 @@ struct jf_handoff {
   const uint16_t *k_shadow, *v_shadow;
   float scale;
   uint16_t* q_pin = nullptr;       // (B, H_q, D) bf16
-  int64_t* ts_pin = nullptr;       // (B, H_q, K)
+  int32_t* ts_pin = nullptr;       // (B, H_q, K) slots, narrowed to 32 bits by the publish kernel (half the PCIe bytes)
   uint16_t* o_pin = nullptr;       // (B, H_q, D) bf16
   int64_t* flag_pin = nullptr;     // [0]: sequence number of the last published (q, slots); [8]: sequence number of
                                    // the last finished correction; [16]: status raised by the device-side wait
@@ -414,7 +427,6 @@ struct jf_handoff {
   int64_t stream_seen = 0;         // stream mode: last sequence number the shared poller has served
   bool registered = false;         // stream mode: known to the shared poller
   uint64_t device_wait_ticks = 0;  // bound of the device-side wait, in ticks of the 100 MHz wall clock
-  std::vector<int64_t> head_map;   // (B, H_q, K)
   std::atomic<int64_t> submits{0};
   std::atomic<int64_t> host_seq{0};  // submits enqueued by the host
   std::atomic<int64_t> done_seq{0};  // corrections finished by the dispatcher
@@ -432,9 +444,15 @@ __global__ __launch_bounds__(256) void handoff_publish_kernel(const uint4* __res
                                                               const uint4* __restrict__ s_src, uint4* s_dst, int ns16,
                                                               unsigned* counter, int64_t* flag, int64_t seq,
                                                               int64_t* seq_dev) {
+  // q: 16 bytes per item; slots: item i narrows four int64 slots (two 16-byte loads) to one 16-byte store
   for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < nq16 + ns16; i += gridDim.x * blockDim.x) {
-    if (i < nq16) q_dst[i] = q_src[i];
-    else s_dst[i - nq16] = s_src[i - nq16];
+    if (i < nq16) {
+      q_dst[i] = q_src[i];
+    } else {
+      const int j = i - nq16;
+      const uint4 a = s_src[2 * j], b = s_src[2 * j + 1];
+      s_dst[j] = make_uint4(a.x, a.z, b.x, b.z);  // low words: slots are < 2^31, -1 stays -1
+    }
   }
   __threadfence_system();  // this thread's stores to host memory are ordered before the counter update
   __syncthreads();
@@ -462,7 +480,10 @@ __global__ __launch_bounds__(256) void handoff_fetch_kernel(const uint4* __restr
 // copies o_new to the device.
 __global__ __launch_bounds__(1024) void handoff_wait_fetch_kernel(const int64_t* done, const int64_t* seq_dev,
                                                                   int64_t* status, uint64_t limit_ticks,
-                                                                  const uint4* __restrict__ src, uint4* dst, int n16) {
+                                                                  const uint4* __restrict__ src, uint4* dst, int n16,
+                                                                  const float* __restrict__ o_hat,
+                                                                  const float* __restrict__ o_old,
+                                                                  const float* __restrict__ W, uint4* out) {
   __shared__ int ok_sh;
   if (threadIdx.x == 0) {
     const int64_t want = *seq_dev;
@@ -482,7 +503,26 @@ __global__ __launch_bounds__(1024) void handoff_wait_fetch_kernel(const int64_t*
   }
   __syncthreads();
   const bool ok = ok_sh != 0;
-  for (int i = threadIdx.x; i < n16; i += blockDim.x) dst[i] = ok ? src[i] : make_uint4(0u, 0u, 0u, 0u);
+  for (int i = threadIdx.x; i < n16; i += blockDim.x) {
+    const uint4 v = ok ? src[i] : make_uint4(0u, 0u, 0u, 0u);
+    if (dst) dst[i] = v;
+    if (out) {  // the blend of jf_blend_unnorm on the eight elements this lane has just fetched
+      const float w = W[i >> 4];  // 16 lanes per 128-element row
+      const float4 h0 = reinterpret_cast<const float4*>(o_hat)[2 * i], h1 = reinterpret_cast<const float4*>(o_hat)[2 * i + 1];
+      const float4 d0 = reinterpret_cast<const float4*>(o_old)[2 * i], d1 = reinterpret_cast<const float4*>(o_old)[2 * i + 1];
+      const uint32_t n[4] = {v.x, v.y, v.z, v.w};
+      const float hh[8] = {h0.x, h0.y, h0.z, h0.w, h1.x, h1.y, h1.z, h1.w};
+      const float dd[8] = {d0.x, d0.y, d0.z, d0.w, d1.x, d1.y, d1.z, d1.w};
+      uint32_t r[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float lo = __builtin_fmaf(w, bf16_to_f32((uint16_t)(n[e] & 0xffffu)), hh[2 * e]) - dd[2 * e];
+        const float hi = __builtin_fmaf(w, bf16_to_f32((uint16_t)(n[e] >> 16)), hh[2 * e + 1]) - dd[2 * e + 1];
+        r[e] = (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+      }
+      out[i] = make_uint4(r[0], r[1], r[2], r[3]);
+    }
+  }
 }
 
 inline void cpu_relax() {
@@ -492,8 +532,9 @@ inline void cpu_relax() {
 }
 
 bool run_correction(jf_handoff* h) {
-  CpuJob j{h->q_pin, h->k_shadow, h->v_shadow, h->head_map.data(), h->ts_pin, h->o_pin,
-           h->B, h->H_q, h->K, h->H_kv, h->num_slots, h->scale};
+  // kv-head of a row = query head / (H_q / H_kv) (decode_path.py:400-408): no head map is read
+  CpuJob j{h->q_pin, h->k_shadow, h->v_shadow, nullptr, nullptr, h->o_pin,
+           h->B, h->H_q, h->K, h->H_kv, h->num_slots, h->scale, h->ts_pin};
   return Pool::instance().run((int64_t)h->B * h->H_q, [j](int64_t b, int64_t e) { run_rows(j, b, e); });
 }
 
@@ -612,7 +653,8 @@ bool claim_mode(jf_handoff* h, int mode) {
 
 extern "C" jf_handoff* jf_handoff_create(int B, int H_q, int H_kv, int K, int64_t num_slots,
                                          const uint16_t* k_shadow_host, const uint16_t* v_shadow_host, float scale) {
-  if (B <= 0 || H_q <= 0 || H_kv <= 0 || K <= 0 || K % 2 != 0 || num_slots <= 0 || H_q % H_kv != 0 || !k_shadow_host || !v_shadow_host) {
+  if (B <= 0 || H_q <= 0 || H_kv <= 0 || K <= 0 || K % 4 != 0 || num_slots <= 0 || num_slots > 0x7fffffffLL || H_q % H_kv != 0 ||
+      !k_shadow_host || !v_shadow_host) {
     set_error("handoff_create: bad arguments");
     return nullptr;
   }
@@ -623,7 +665,7 @@ extern "C" jf_handoff* jf_handoff_create(int B, int H_q, int H_kv, int K, int64_
     const double t = std::atof(e);
     if (t > 0) h->timeout_s = t;
   }
-  const size_t nq = (size_t)B * H_q * D * sizeof(uint16_t), nt = (size_t)B * H_q * K * sizeof(int64_t);
+  const size_t nq = (size_t)B * H_q * D * sizeof(uint16_t), nt = (size_t)B * H_q * K * sizeof(int32_t);
   if (hipHostMalloc((void**)&h->q_pin, nq, hipHostMallocDefault) != hipSuccess ||
       hipHostMalloc((void**)&h->ts_pin, nt, hipHostMallocDefault) != hipSuccess ||
       hipHostMalloc((void**)&h->o_pin, nq, hipHostMallocDefault) != hipSuccess ||
@@ -635,11 +677,6 @@ extern "C" jf_handoff* jf_handoff_create(int B, int H_q, int H_kv, int K, int64_
   }
   h->flag_pin[0] = h->flag_pin[8] = h->flag_pin[16] = 0;
   h->device_wait_ticks = (uint64_t)((h->timeout_s < 10.0 ? h->timeout_s : 10.0) * 1e8);
-  const int G = H_q / H_kv;
-  h->head_map.resize((size_t)B * H_q * K);
-  for (int b = 0; b < B; ++b)
-    for (int hq = 0; hq < H_q; ++hq)
-      for (int k = 0; k < K; ++k) h->head_map[((size_t)b * H_q + hq) * K + k] = hq / G;  // decode_path.py:400-408
   h->dispatcher = std::thread(handoff_dispatch, h);
   return h;
 }
@@ -652,7 +689,7 @@ extern "C" int jf_handoff_submit(jf_handoff* h, const uint16_t* q_dev, const int
   JF_CHECK_ARG(h->host_seq.load() == h->done_seq.load(), "handoff_submit: the previous correction is still in flight (wait for it first)");
   hipStream_t st = (hipStream_t)stream;
   const int nq16 = (int)((size_t)h->B * h->H_q * D * sizeof(uint16_t) / 16);
-  const int ns16 = (int)((size_t)h->B * h->H_q * h->K * sizeof(int64_t) / 16);
+  const int ns16 = (int)((size_t)h->B * h->H_q * h->K * sizeof(int32_t) / 16);
   const int64_t seq = h->host_seq.load() + 1;
   int blocks = (nq16 + ns16 + 255) / 256;
   if (blocks > 32) blocks = 32;
@@ -681,7 +718,7 @@ extern "C" int jf_handoff_stream_submit(jf_handoff* h, const uint16_t* q_dev, co
     StreamPoller::instance().add(h);
   }
   const int nq16 = (int)((size_t)h->B * h->H_q * D * sizeof(uint16_t) / 16);
-  const int ns16 = (int)((size_t)h->B * h->H_q * h->K * sizeof(int64_t) / 16);
+  const int ns16 = (int)((size_t)h->B * h->H_q * h->K * sizeof(int32_t) / 16);
   int blocks = (nq16 + ns16 + 255) / 256;
   if (blocks > 32) blocks = 32;
   hipLaunchKernelGGL(handoff_publish_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream,
@@ -699,7 +736,23 @@ extern "C" int jf_handoff_stream_wait(jf_handoff* h, uint16_t* o_new_dev, void* 
   const int n16 = (int)((size_t)h->B * h->H_q * D * sizeof(uint16_t) / 16);
   hipLaunchKernelGGL(handoff_wait_fetch_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, h->flag_pin + 8,
                      reinterpret_cast<const int64_t*>(h->counter_dev + 2), h->flag_pin + 16, h->device_wait_ticks,
-                     reinterpret_cast<const uint4*>(h->o_pin), reinterpret_cast<uint4*>(o_new_dev), n16);
+                     reinterpret_cast<const uint4*>(h->o_pin), reinterpret_cast<uint4*>(o_new_dev), n16,
+                     (const float*)nullptr, (const float*)nullptr, (const float*)nullptr, (uint4*)nullptr);
+  JF_CHECK_HIP(hipGetLastError());
+  return JF_OK;
+}
+
+extern "C" int jf_handoff_stream_wait_blend(jf_handoff* h, const float* o_hat, const float* o_old_unnorm, const float* W,
+                                            uint16_t* out, uint16_t* o_new_dev, void* stream) {
+  JF_CHECK_ARG(h && o_hat && o_old_unnorm && W && out, "handoff_stream_wait_blend: null argument");
+  JF_CHECK_ARG((((uintptr_t)o_hat | (uintptr_t)o_old_unnorm | (uintptr_t)out | (uintptr_t)o_new_dev) & 15) == 0,
+               "handoff_stream_wait_blend: tensors must be 16-byte aligned");
+  JF_CHECK_ARG(h->mode.load() == 2, "handoff_stream_wait_blend: no jf_handoff_stream_submit precedes it");
+  const int n16 = (int)((size_t)h->B * h->H_q * D * sizeof(uint16_t) / 16);
+  hipLaunchKernelGGL(handoff_wait_fetch_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, h->flag_pin + 8,
+                     reinterpret_cast<const int64_t*>(h->counter_dev + 2), h->flag_pin + 16, h->device_wait_ticks,
+                     reinterpret_cast<const uint4*>(h->o_pin), reinterpret_cast<uint4*>(o_new_dev), n16, o_hat,
+                     o_old_unnorm, W, reinterpret_cast<uint4*>(out));
   JF_CHECK_HIP(hipGetLastError());
   return JF_OK;
 }

@@ -513,6 +513,19 @@ class CpuTopkHandoff:
                and o_new.shape == (B, H_q, HEAD_DIM), "o_new must be contiguous (B, H_q, 128) bf16 on the GPU")
         _lib.check(_lib.load().jf_handoff_stream_wait(self._h, o_new.data_ptr(), _stream(o_new)))
 
+    def stream_wait_blend(self, o_hat, o_old_unnorm, W, out, o_new=None) -> None:
+        """`stream_wait` and `blend_unnorm_into` in one kernel: `out = bf16(fma(W, o_new, o_hat) - o_old_unnorm)`."""
+        B, H_q, _ = self.shape
+        for t in (o_hat, o_old_unnorm):
+            _check(t.is_cuda and t.dtype == torch.float32 and t.is_contiguous() and t.shape == (B, H_q, HEAD_DIM),
+                   "o_hat / o_old_unnorm must be contiguous (B, H_q, 128) fp32 on the GPU")
+        _check(W.is_cuda and W.dtype == torch.float32 and W.is_contiguous() and W.shape == (B, H_q), "W must be (B, H_q) fp32")
+        for t in (out,) + ((o_new,) if o_new is not None else ()):
+            _check(t.is_cuda and t.dtype == torch.bfloat16 and t.is_contiguous() and t.shape == (B, H_q, HEAD_DIM),
+                   "out / o_new must be contiguous (B, H_q, 128) bf16 on the GPU")
+        _lib.check(_lib.load().jf_handoff_stream_wait_blend(self._h, o_hat.data_ptr(), o_old_unnorm.data_ptr(), W.data_ptr(),
+                                                            out.data_ptr(), _ptr(o_new), _stream(out)))
+
     def check_status(self) -> None:
         """Raises if a correction failed or a device-side wait ran into its limit (call after a synchronise)."""
         _lib.check(_lib.load().jf_handoff_status(self._h))

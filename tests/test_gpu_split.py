@@ -344,7 +344,7 @@ def test_handoff_protocol_edges():
 
 
 def test_handoff_stream_mode_replays_from_a_hip_graph():
-    """The kernel-only submit / wait pair: eager calls, then a captured graph (publish, device-side wait, blend)
+    """The kernel-only submit / wait pair: eager calls, then a captured graph (publish, device-side wait + blend)
     replayed with new queries and slots in the same buffers, eager work and synchronisations in between; every
     result equals the host-blocking pair's on the same inputs."""
     B, Hq, Hkv, K, S = 2, 8, 2, 32, 256
@@ -394,8 +394,7 @@ def test_handoff_stream_mode_replays_from_a_hip_graph():
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph, stream=side):
         h.stream_submit(q_buf, s_buf)
-        h.stream_wait(o_new)
-        o.blend_unnorm_into(o_hat, o_old, W, o_new, out)
+        h.stream_wait_blend(o_hat, o_old, W, out, o_new)          # wait + fetch + blend in one kernel
     for step in range(4):
         q, s = draw()
         q_buf.copy_(q); s_buf.copy_(s)
