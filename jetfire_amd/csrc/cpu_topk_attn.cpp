@@ -33,9 +33,14 @@ void set_error(const char* fmt, ...) {
 }
 
 // ------------------------------------------------------------------ worker pool
-// One job at a time (like the reference's single-flight pool, jetfire_pool.h:270-305).  A job is a
-// range [0, n) of rows cut into contiguous shares, one per worker; the submitting thread either
-// blocks in run() or returns immediately from start() and later calls join().
+// One job at a time (like the reference's single-flight pool, jetfire_pool.h:270-305).  A job is a range
+// [0, n) of rows handed out in small chunks from a shared counter; the submitting thread either blocks in
+// run() or returns immediately from start() and later calls join().
+//
+// A job is finished when all of its ROWS are, not when every worker has checked in: a worker that has lost
+// its core (more busy threads than cores) or is still asleep takes no rows and holds nobody up; it only
+// matters while it sits on a claimed row.  The counter carries the job's epoch in its upper half, so a worker
+// that wakes up late with an old job in hand cannot claim rows of a newer one.
 class Pool {
  public:
   static Pool& instance() {
@@ -56,16 +61,16 @@ class Pool {
     std::unique_lock<std::mutex> lk(mu_);
     if (busy_) return false;
     busy_ = true;
-    fn_ = std::move(fn);
-    n_ = n;
+    const uint64_t e = epoch_.load(std::memory_order_relaxed) + 1;
+    Job& jb = jobs_[e & 1];
+    jb.fn = std::move(fn);
+    jb.n = n;
     const int w = (int)workers_.size();
-    active_ = w;
-    // rows are handed out in small chunks from a shared counter: a worker that loses its core for a while
-    // simply takes fewer of them
-    chunk_ = std::max<int64_t>(1, n / ((int64_t)w * 8));
-    next_.store(0, std::memory_order_relaxed);
-    remaining_.store(w, std::memory_order_release);
-    epoch_.fetch_add(1, std::memory_order_acq_rel);
+    jb.chunk = std::max<int64_t>(1, n / ((int64_t)w * 8));
+    n_ = n;
+    done_rows_.store(0, std::memory_order_relaxed);
+    next_.store(e << 32, std::memory_order_relaxed);
+    epoch_.store(e, std::memory_order_release);
     lk.unlock();
     cv_work_.notify_all();
     return true;
@@ -74,37 +79,38 @@ class Pool {
   bool join(double timeout_s) {
     const auto t0 = std::chrono::steady_clock::now();
     for (int spin = 0; spin < 20000; ++spin) {
-      if (remaining_.load(std::memory_order_acquire) == 0) break;
+      if (done_rows_.load(std::memory_order_acquire) >= n_) break;
 #if defined(__x86_64__)
       _mm_pause();
 #endif
     }
     std::unique_lock<std::mutex> lk(mu_);
-    while (remaining_.load(std::memory_order_acquire) != 0) {
+    while (done_rows_.load(std::memory_order_acquire) < n_) {
       if (timeout_s > 0) {
         const double el = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
         if (el > timeout_s) return false;
-        cv_done_.wait_for(lk, std::chrono::milliseconds(1));
-      } else {
-        cv_done_.wait_for(lk, std::chrono::milliseconds(1));
       }
+      cv_done_.wait_for(lk, std::chrono::milliseconds(1));
     }
     busy_ = false;
-    fn_ = nullptr;
     return true;
   }
   bool run(int64_t n, std::function<void(int64_t, int64_t)> fn) {
+    if (n <= 0) return true;
     while (!start(n, fn)) std::this_thread::yield();
     return join(0);
   }
 
  private:
+  struct Job {
+    std::function<void(int64_t, int64_t)> fn;
+    int64_t n = 0, chunk = 1;
+  };
   Pool() = default;
   ~Pool() {
     {
       std::lock_guard<std::mutex> g(mu_);
       stop_ = true;
-      epoch_.fetch_add(1, std::memory_order_acq_rel);
     }
     cv_work_.notify_all();
     for (auto& t : workers_) t.join();
@@ -133,7 +139,6 @@ class Pool {
     // resize: stop the old set, start a new one
     if (!workers_.empty()) {
       stop_ = true;
-      epoch_.fetch_add(1, std::memory_order_acq_rel);
       lk.unlock();
       cv_work_.notify_all();
       for (auto& t : workers_) t.join();
@@ -142,16 +147,16 @@ class Pool {
       stop_ = false;
     }
     const uint64_t e0 = epoch_.load(std::memory_order_acquire);
-    for (int i = 0; i < want; ++i) workers_.emplace_back([this, i, e0] { worker(i, e0); });
+    for (int i = 0; i < want; ++i) workers_.emplace_back([this, e0] { worker(e0); });
   }
-  void worker(int id, uint64_t seen) {
+  void worker(uint64_t seen) {
     for (;;) {
       // spin for the next epoch for about half a millisecond (the gap between two layers of a decode step is
       // shorter than a futex wake-up of the whole pool), then sleep
       bool got = false;
       const auto t0 = std::chrono::steady_clock::now();
       for (uint32_t spin = 0;; ++spin) {
-        if (epoch_.load(std::memory_order_acquire) != seen) { got = true; break; }
+        if (epoch_.load(std::memory_order_acquire) != seen || stop_flag()) { got = true; break; }
 #if defined(__x86_64__)
         _mm_pause();
 #endif
@@ -160,45 +165,46 @@ class Pool {
       }
       if (!got) {
         std::unique_lock<std::mutex> lk(mu_);
-        cv_work_.wait(lk, [&] { return epoch_.load(std::memory_order_acquire) != seen; });
+        cv_work_.wait(lk, [&] { return stop_ || epoch_.load(std::memory_order_acquire) != seen; });
       }
-      std::function<void(int64_t, int64_t)> fn;
-      int64_t n, chunk;
-      int w;
-      {
-        std::lock_guard<std::mutex> g(mu_);
-        seen = epoch_.load(std::memory_order_acquire);
-        if (stop_) return;
-        fn = fn_;
-        n = n_;
-        w = active_;
-        chunk = chunk_;
-      }
-      if (fn && id < w) {
-        for (;;) {
-          const int64_t b = next_.fetch_add(chunk, std::memory_order_relaxed);
-          if (b >= n) break;
-          fn(b, std::min<int64_t>(n, b + chunk));
-        }
-        if (remaining_.fetch_sub(1, std::memory_order_acq_rel) == 1) {
+      if (stop_flag()) return;
+      const uint64_t e = epoch_.load(std::memory_order_acquire);
+      seen = e;
+      // The job of epoch e stays in its slot at least until all its rows are done; the slot is only read after a
+      // claim on the counter of that very epoch has succeeded, i.e. while the job is certainly still current.
+      const Job& jb = jobs_[e & 1];
+      uint64_t v = next_.load(std::memory_order_acquire);
+      for (;;) {
+        if ((v >> 32) != (e & 0xffffffffu)) break;  // a newer job: this one is long finished
+        const int64_t b = (int64_t)(v & 0xffffffffu);
+        const int64_t n = jb.n, chunk = jb.chunk;
+        if (b >= n) break;
+        if (!next_.compare_exchange_weak(v, v + (uint64_t)chunk, std::memory_order_acq_rel, std::memory_order_acquire)) continue;
+        const int64_t end = std::min<int64_t>(n, b + chunk);
+        jb.fn(b, end);
+        if (done_rows_.fetch_add(end - b, std::memory_order_acq_rel) + (end - b) >= n) {
           std::lock_guard<std::mutex> g(mu_);
           cv_done_.notify_all();
+          break;
         }
+        v = next_.load(std::memory_order_acquire);
       }
     }
+  }
+  bool stop_flag() {
+    return __atomic_load_n(&stop_, __ATOMIC_ACQUIRE);
   }
 
   std::mutex mu_, cfg_mu_;
   std::condition_variable cv_work_, cv_done_;
   std::vector<std::thread> workers_;
-  std::function<void(int64_t, int64_t)> fn_;
-  int64_t n_ = 0, chunk_ = 1;
-  std::atomic<int64_t> next_{0};
-  int active_ = 0;
+  Job jobs_[2];
+  int64_t n_ = 0;
+  std::atomic<uint64_t> next_{0};       // (epoch << 32) | first unclaimed row
+  std::atomic<int64_t> done_rows_{0};
   int override_ = 0;
   bool busy_ = false, stop_ = false;
   std::atomic<uint64_t> epoch_{0};
-  std::atomic<int> remaining_{0};
 };
 
 // ------------------------------------------------------------------ row kernel
@@ -269,7 +275,9 @@ __attribute__((target("avx2,fma"))) static void topk_attn_row_avx2(const uint16_
                                                                    const int64_t* head_map, int64_t fixed_h,
                                                                    const SlotT* slots, int K, int H_kv, float scale,
                                                                    uint16_t* out, float* score_buf) {
-  constexpr int AHEAD = 8;
+  // rows requested ahead of their use: measured on a 16-core EPYC share, 8 rows leave the gather at 3/4 of the
+  // rate that 24 to 64 rows reach (110 against 148 us for 32768 row pairs on 14 threads)
+  constexpr int AHEAD = 32;
   __m256 qv[D / 8];
   for (int i = 0; i < D / 8; ++i) qv[i] = bf16x8_to_f32(q + 8 * i);
   auto row_of = [&](const uint16_t* base, int k) -> const uint16_t* {

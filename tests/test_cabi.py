@@ -78,6 +78,35 @@ def test_cpu_topk_attn_matches_oracle(threads, B, Hq, Hkv, K):
     assert (bf16_to_f32(out)[0, 1] == 0).all()
 
 
+def test_cpu_pool_survives_oversubscription_and_resizing():
+    """Many back-to-back jobs on far more workers than cores, with the pool resized in between: every job's
+    output equals the single-thread result bit for bit (a late worker must never touch a newer job's rows)."""
+    from jetfire_amd import ops
+    B, Hq, Hkv, K = 4, 16, 4, 64
+    c = make_case(91, B, Hq, Hkv, 512, 3, 2, 64, ragged=False)
+    rng = np.random.default_rng(3)
+    nslots = c["K"].shape[1]
+    hm = torch.from_numpy(O.head_map(B, Hq, Hq // Hkv, K))
+    ksh, vsh = bf16_tensor(c["K"]), bf16_tensor(c["V"])
+    cases = []
+    ops.set_cpu_attn_threads(1)
+    for i in range(6):
+        q = bf16_tensor(O.bf16_round((rng.standard_normal((B, Hq, 128)) / np.sqrt(128)).astype(np.float32)))
+        ts = torch.from_numpy(rng.integers(-1, nslots, size=(B, Hq, K)).astype(np.int64))
+        want = torch.zeros(B, Hq, 128, dtype=torch.bfloat16)
+        ops.cpu_topk_attn(q, ksh, vsh, hm, ts, want, 0.09)
+        cases.append((q, ts, want))
+    out = torch.zeros(B, Hq, 128, dtype=torch.bfloat16)
+    for threads in (33, 5, 64):
+        ops.set_cpu_attn_threads(threads)
+        for rep in range(60):
+            q, ts, want = cases[rep % len(cases)]
+            out.fill_(3.0)
+            ops.cpu_topk_attn(q, ksh, vsh, hm, ts, out, 0.09)
+            assert torch.equal(out.view(torch.int16), want.view(torch.int16)), (threads, rep)
+    ops.set_cpu_attn_threads(2)
+
+
 def test_cpu_topk_attn_single_slot_returns_the_value_row():
     from jetfire_amd import ops
     c = make_case(60, 1, 4, 2, 64, 3, 2, 64, ragged=False)
