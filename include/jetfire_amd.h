@@ -99,6 +99,14 @@ int jf_int3_qk_scores(const uint16_t* q, const uint8_t* k_data, const uint16_t* 
                       int B, int H_q, int H_kv, int max_S, int max_blocks, int64_t num_slots,
                       int n_scale_groups, int block_size, float attn_scale,
                       float* scores, void* stream);
+/* The bf16 model of jf_int3_qk_scores for any symmetric key width: k_nbits 2 replaces int2_qk_scores with an
+ * empty k_zp (jetfire_vllm/csrc/int2_qk_scores.cu:279-420: codes - 2, four per byte MSB first), 3 is
+ * jf_int3_qk_scores, 4 replaces int4_qk_scores (jetfire_vllm/csrc/int4_qk_scores.cu:280-420: nibbles - 8,
+ * (even << 4) | odd).  k_data (H_kv, num_slots, 16 * k_nbits), k_scales (H_kv, num_slots, n_scale_groups). */
+int jf_intn_qk_scores(int k_nbits, const uint16_t* q, const uint8_t* k_data, const uint16_t* k_scales,
+                      const int64_t* block_table, const int32_t* seq_lens, int B, int H_q, int H_kv,
+                      int max_S, int max_blocks, int64_t num_slots, int n_scale_groups, int block_size,
+                      float attn_scale, float* scores, void* stream);
 int jf_int8tc_qk_scores(const uint16_t* q, const uint8_t* k_data, const uint16_t* k_scales,
                         const int64_t* block_table, const int32_t* seq_lens,
                         int B, int H_q, int H_kv, int max_S, int max_blocks, int64_t num_slots,

@@ -66,6 +66,61 @@ __global__ __launch_bounds__(QK_THREADS) void int3_qk_scores_kernel(
   for (int g = 0; g < G; ++g) out[(size_t)g * max_S] = acc[g] * attn_scale;
 }
 
+// INT2 / INT4 keys with the same bf16 model (jetfire_vllm/csrc/int2_qk_scores.cu:66-79, int4_qk_scores.cu:68-80):
+//     score = (sum_d f32(q_d) * f32(bf16((code_d - 2^(bits-1)) * scale_g))) * attn_scale       fp32 accumulate
+// INT2 rows: 32 bytes, four codes per byte MSB first; INT4 rows: 64 bytes, (even << 4) | odd.
+template <int KBITS, int G, int NG>
+__global__ __launch_bounds__(QK_THREADS) void intn_qk_scores_kernel(
+    const uint16_t* __restrict__ q, const uint8_t* __restrict__ k_data, const uint16_t* __restrict__ k_scales,
+    const int64_t* __restrict__ block_table, const int32_t* __restrict__ seq_lens, float* __restrict__ scores,
+    int H_q, int H_kv, int max_S, int max_blocks, int64_t num_slots, int bs, float attn_scale) {
+  static_assert(KBITS == 2 || KBITS == 4, "planar INT3 rows have their own kernel");
+  constexpr int P = D * KBITS / 8, NDW = P / 4, OFF = 1 << (KBITS - 1);
+  __shared__ float qs[G][D];
+  const int b = blockIdx.z, hkv = blockIdx.y, tid = threadIdx.x;
+  for (int i = tid; i < G * D; i += QK_THREADS)
+    qs[i / D][i % D] = bf16_to_f32(q[((size_t)b * H_q + (size_t)hkv * G + i / D) * D + i % D]);
+  __syncthreads();
+  const int s = blockIdx.x * QK_THREADS + tid;
+  if (s >= max_S) return;
+  float* out = scores + ((size_t)b * H_q + (size_t)hkv * G) * max_S + s;
+  const int S = seq_lens[b];
+  if (s >= S) {
+#pragma unroll
+    for (int g = 0; g < G; ++g) out[(size_t)g * max_S] = -INFINITY;
+    return;
+  }
+  const int64_t slot = block_table[(size_t)b * max_blocks + s / bs] * bs + s % bs;
+  const uint32_t* row = reinterpret_cast<const uint32_t*>(k_data + ((size_t)hkv * num_slots + slot) * P);
+  uint32_t p[NDW];
+#pragma unroll
+  for (int i = 0; i < NDW; ++i) p[i] = row[i];
+  float sc[NG];
+#pragma unroll
+  for (int g = 0; g < NG; ++g) sc[g] = bf16_to_f32(k_scales[((size_t)hkv * num_slots + slot) * NG + g]);
+  float acc[G];
+#pragma unroll
+  for (int g = 0; g < G; ++g) acc[g] = 0.0f;
+#pragma unroll
+  for (int gi = 0; gi < 16; ++gi) {  // eight channels at a time
+    const float scale = sc[(gi * 8 * NG) / D];
+    float kv[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      int code;
+      if (KBITS == 4) code = (int)((p[gi] >> (8 * (j >> 1) + ((j & 1) ? 0 : 4))) & 15u);
+      else code = (int)((p[gi >> 1] >> (16 * (gi & 1) + 8 * (j >> 2) + (6 - 2 * (j & 3)))) & 3u);
+      kv[j] = bf16_to_f32(f32_to_bf16((float)(code - OFF) * scale));
+    }
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[g] = __builtin_fmaf(qs[g][gi * 8 + j], kv[j], acc[g]);
+  }
+#pragma unroll
+  for (int g = 0; g < G; ++g) out[(size_t)g * max_S] = acc[g] * attn_scale;
+}
+
 // q quantisation shared by the INT4 kernels: qi packed so that dword j of `qe` holds channels
 // 8j+{0,2,4,6} (the high nibbles of key dword j) and `qo` holds 8j+{1,3,5,7} (the low nibbles).
 template <int G>
@@ -211,6 +266,38 @@ extern "C" int jf_int3_qk_scores(const uint16_t* q, const uint8_t* k_data, const
       hipLaunchKernelGGL((int3_qk_scores_kernel<GG, 2>), grid, block, 0, st, q, k_data, k_scales, block_table, seq_lens,
                          scores, H_q, H_kv, max_S, max_blocks, num_slots, block_size, attn_scale);
   });
+  JF_CHECK_LAUNCH();
+  return JF_OK;
+}
+
+extern "C" int jf_intn_qk_scores(int k_nbits, const uint16_t* q, const uint8_t* k_data, const uint16_t* k_scales,
+                                 const int64_t* block_table, const int32_t* seq_lens, int B, int H_q, int H_kv,
+                                 int max_S, int max_blocks, int64_t num_slots, int n_scale_groups, int block_size,
+                                 float attn_scale, float* scores, void* stream) {
+  if (k_nbits == 3)
+    return jf_int3_qk_scores(q, k_data, k_scales, block_table, seq_lens, B, H_q, H_kv, max_S, max_blocks, num_slots,
+                             n_scale_groups, block_size, attn_scale, scores, stream);
+  JF_CHECK_ARG(k_nbits == 2 || k_nbits == 4, "intn_qk_scores: k_nbits must be 2, 3 or 4 (got %d)", k_nbits);
+  int rc = check_stage_a("intn_qk_scores", q, k_data, k_scales, block_table, seq_lens, scores, B, H_q, H_kv, max_S,
+                         max_blocks, num_slots, block_size);
+  if (rc != JF_OK) return rc;
+  JF_CHECK_ARG(n_scale_groups == 1 || n_scale_groups == 2, "intn_qk_scores supports K quant groups 1 or 2, got %d",
+               n_scale_groups);
+  if (B == 0 || max_S == 0) return JF_OK;
+  dim3 grid((unsigned)((max_S + QK_THREADS - 1) / QK_THREADS), (unsigned)H_kv, (unsigned)B), block(QK_THREADS);
+  hipStream_t st = (hipStream_t)stream;
+  const int G = H_q / H_kv;
+#define JF_INTN_LAUNCH(KB, NGV)                                                                                        \
+  hipLaunchKernelGGL((intn_qk_scores_kernel<KB, GG, NGV>), grid, block, 0, st, q, k_data, k_scales, block_table,      \
+                     seq_lens, scores, H_q, H_kv, max_S, max_blocks, num_slots, block_size, attn_scale)
+  JF_DISPATCH_G(G, {
+    if (k_nbits == 2) {
+      if (n_scale_groups == 1) JF_INTN_LAUNCH(2, 1); else JF_INTN_LAUNCH(2, 2);
+    } else {
+      if (n_scale_groups == 1) JF_INTN_LAUNCH(4, 1); else JF_INTN_LAUNCH(4, 2);
+    }
+  });
+#undef JF_INTN_LAUNCH
   JF_CHECK_LAUNCH();
   return JF_OK;
 }

@@ -56,6 +56,11 @@ __global__ __launch_bounds__(SV_THREADS) void softmax_stats_kernel(const float* 
 template <int NBITS>
 __device__ inline int v_code(const uint8_t* row, int d) {
   if (NBITS == 2) return (int)((row[d >> 2] >> ((3 - (d & 3)) * 2)) & 3) - 2;
+  if (NBITS == 3) {  // planar: codes 8w .. 8w+7 are the 24-bit word whose bytes sit at w, 16 + w, 32 + w (MSB first)
+    const int w = d >> 3;
+    const uint32_t word = ((uint32_t)row[w] << 16) | ((uint32_t)row[16 + w] << 8) | (uint32_t)row[32 + w];
+    return (int)((word >> (21 - 3 * (d & 7))) & 7u) - 4;
+  }
   return (int)((row[d >> 1] >> ((1 - (d & 1)) * 4)) & 15) - 8;
 }
 
@@ -83,10 +88,12 @@ __global__ __launch_bounds__(SV_THREADS) void weighted_v_split_kernel(
     const int64_t base_slot = bt[p0 / BS] * BS;
     __syncthreads();
     {
-      constexpr int DW = BS * P / 4 / SV_THREADS;  // dwords per thread
+      constexpr int NDW = BS * P / 4;  // dwords of a page (128, 192 or 256)
       const uint32_t* src = reinterpret_cast<const uint32_t*>(vbase + base_slot * P);
 #pragma unroll
-      for (int i = 0; i < DW; ++i) reinterpret_cast<uint32_t*>(vbuf)[tid + i * SV_THREADS] = src[tid + i * SV_THREADS];
+      for (int i = 0; i < (NDW + SV_THREADS - 1) / SV_THREADS; ++i)
+        if (NDW % SV_THREADS == 0 || tid + i * SV_THREADS < NDW)
+          reinterpret_cast<uint32_t*>(vbuf)[tid + i * SV_THREADS] = src[tid + i * SV_THREADS];
     }
     for (int i = tid; i < G * BS; i += SV_THREADS) {
       const int g = i / BS, j = i % BS;
@@ -204,7 +211,7 @@ extern "C" int jf_softmax_v_pre_corr(const float* scores, const float* softmax_m
   const int G = H_q / H_kv;
   JF_CHECK_ARG(G == 1 || G == 2 || G == 4 || G == 8 || G == 16, "softmax_v: GQA group %d not in {1,2,4,8,16}", G);
   JF_CHECK_ARG(block_size == 16, "wvs2 only supports block_size=16");
-  JF_CHECK_ARG(v_nbits == 2 || v_nbits == 4, "softmax_v: v_nbits must be 2 or 4 (got %d)", v_nbits);
+  JF_CHECK_ARG(v_nbits == 2 || v_nbits == 3 || v_nbits == 4, "softmax_v: v_nbits must be 2, 3 or 4 (got %d)", v_nbits);
   JF_CHECK_ARG(n_scale_groups == 1 || n_scale_groups == 2, "wvs2 requires num_groups=1 or 2 (got %d)", n_scale_groups);
   JF_CHECK_ARG((int64_t)max_blocks * block_size >= max_S, "softmax_v: block_table does not cover max_S");
   JF_CHECK_ARG((softmax_m == nullptr) == (softmax_inv_z == nullptr), "softmax_v: softmax_m and softmax_inv_z go together");
@@ -250,6 +257,8 @@ extern "C" int jf_softmax_v_pre_corr(const float* scores, const float* softmax_m
   }
   if (v_nbits == 2 && n_scale_groups == 1) { JF_SV_LAUNCH(2, 1) }
   else if (v_nbits == 2) { JF_SV_LAUNCH(2, 2) }
+  else if (v_nbits == 3 && n_scale_groups == 1) { JF_SV_LAUNCH(3, 1) }
+  else if (v_nbits == 3) { JF_SV_LAUNCH(3, 2) }
   else if (n_scale_groups == 1) { JF_SV_LAUNCH(4, 1) }
   else { JF_SV_LAUNCH(4, 2) }
   return JF_OK;

@@ -1,14 +1,12 @@
 """Per-quant-scheme kernel sets (jetfire_vllm/kernels/_dispatch/__init__.py:24-127).
 
-Only the two release schemes are provided: SymInt3K_SymInt2V and SymInt4K_SymInt4V."""
+The nine symmetric K/V pairs are provided; the asymmetric INT2-key schemes are not."""
 from __future__ import annotations
 
 import importlib
 
-_SCHEMES = {
-    "SymInt3K_SymInt2V": "jetfire_amd.kernels._dispatch.sym_int3_k_sym_int2_v:KERNELS",
-    "SymInt4K_SymInt4V": "jetfire_amd.kernels._dispatch.sym_int4_k_sym_int4_v:KERNELS",
-}
+_SCHEMES = {f"SymInt{k}K_SymInt{v}V": f"jetfire_amd.kernels._dispatch.sym_int{k}_k_sym_int{v}_v:KERNELS"
+            for k in (2, 3, 4) for v in (2, 3, 4)}
 
 
 def get_kernel_set(scheme_name: str):

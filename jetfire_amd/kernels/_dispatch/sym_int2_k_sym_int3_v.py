@@ -1,0 +1,4 @@
+"""KernelSet for SymInt2K_SymInt3V (jetfire_vllm/kernels/_dispatch/sym_int2_k_sym_int3_v.py)."""
+from ._sym import SymKernelSet
+
+KERNELS = SymKernelSet(2, 3)

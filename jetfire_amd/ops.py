@@ -192,6 +192,63 @@ def int3_qk_scores(q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_kv,
     return scores
 
 
+def _intn_qk_scores(nbits: int, name: str, q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_kv, block_size,
+                    attn_scale):
+    lib = _lib.load()
+    q, kd, ks, bt, sl = _stage_a_args(q, k_data, k_scales, block_table, seq_lens, H_q, H_kv, HEAD_DIM * nbits // 8)
+    ng = ks.size(2)
+    _check(ng in (1, 2), f"{name} currently supports K quant groups 1 or 2, got {ng}")
+    B = q.size(0)
+    scores = torch.empty((B, H_q, max_S), dtype=torch.float32, device=q.device)
+    _lib.check(lib.jf_intn_qk_scores(nbits, q.data_ptr(), kd.data_ptr(), ks.data_ptr(), bt.data_ptr(), sl.data_ptr(),
+                                     B, H_q, H_kv, int(max_S), bt.size(1), kd.size(1), ng, int(block_size),
+                                     float(attn_scale), scores.data_ptr(), _stream(q)))
+    return scores
+
+
+def _no_zero_point(k_zp, name: str) -> None:
+    if k_zp is not None and k_zp.numel() > 0:
+        raise NotImplementedError(f"{name}: asymmetric INT2 keys (k_zp) are outside this library's decode path")
+
+
+def int2_qk_scores(q, k_data, k_scales, k_zp, block_table, seq_lens, max_S, H_q, H_kv, block_size, attn_scale):
+    """int2_qk_scores.cu:279-420 for symmetric keys (`k_zp` empty or None) -> scores (B, H_q, max_S) fp32."""
+    _no_zero_point(k_zp, "int2_qk_scores")
+    return _intn_qk_scores(2, "int2_qk_scores", q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_kv, block_size,
+                           attn_scale)
+
+
+def int2_qk_scores_topk(q, k_data, k_scales, k_zp, block_table, seq_lens, max_S, H_q, H_kv, block_size, attn_scale,
+                        top_k) -> List[torch.Tensor]:
+    """int2_qk_scores.cu:583-660 -> [scores, topk_idx, topk_slots]."""
+    scores = int2_qk_scores(q, k_data, k_scales, k_zp, block_table, seq_lens, max_S, H_q, H_kv, block_size, attn_scale)
+    idx, slots, _, _ = _topk(scores, block_table, seq_lens, max_S, H_q, block_size, top_k, False, "int2_qk_scores_topk")
+    return [scores, idx, slots]
+
+
+def int4_qk_scores(q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_kv, block_size, attn_scale):
+    """int4_qk_scores.cu:280-420 (bf16 q times bf16-rounded INT4 keys) -> scores (B, H_q, max_S) fp32."""
+    return _intn_qk_scores(4, "int4_qk_scores", q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_kv, block_size,
+                           attn_scale)
+
+
+def int4_qk_scores_topk(q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_kv, block_size, attn_scale,
+                        top_k) -> List[torch.Tensor]:
+    """int4_qk_scores.cu:714-786 -> [scores, topk_idx, topk_slots]."""
+    scores = int4_qk_scores(q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_kv, block_size, attn_scale)
+    idx, slots, _, _ = _topk(scores, block_table, seq_lens, max_S, H_q, block_size, top_k, False, "int4_qk_scores_topk")
+    return [scores, idx, slots]
+
+
+def int4_qk_scores_topk_stats(q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_kv, block_size, attn_scale,
+                              top_k) -> List[torch.Tensor]:
+    """int4_qk_scores.cu:788-848 -> [scores, topk_idx, topk_slots, softmax_m, softmax_inv_z]."""
+    scores = int4_qk_scores(q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_kv, block_size, attn_scale)
+    idx, slots, m, iz = _topk(scores, block_table, seq_lens, max_S, H_q, block_size, top_k, True,
+                              "int4_qk_scores_topk_stats")
+    return [scores, idx, slots, m, iz]
+
+
 def int8tc_qk_scores(q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_kv, block_size, attn_scale):
     """int8tc_qk_scores.cu:1263-1331 -> scores (B, H_q, max_S) fp32."""
     lib = _lib.load()
@@ -319,6 +376,31 @@ def int2_softmax_v_with_pre_corr(scores, v_data, v_scales, block_table, seq_lens
 def int2_softmax_v(scores, v_data, v_scales, block_table, seq_lens, max_S, H_q, H_kv, block_size) -> torch.Tensor:
     return _softmax_v(scores, None, None, v_data, v_scales, block_table, seq_lens, None, max_S, H_q, H_kv, block_size,
                       32, 2)[0]
+
+
+def int3_softmax_v_with_pre_corr_wvs2(scores, v_data, v_scales, block_table, seq_lens, topk_idx, max_S, H_q, H_kv,
+                                      block_size, top_k) -> List[torch.Tensor]:
+    """int3_softmax_v.cu:752-860 (planar INT3 values) -> [o_hat, o_old_unnorm, W]."""
+    return _softmax_v(scores, None, None, v_data, v_scales, block_table, seq_lens, topk_idx, max_S, H_q, H_kv,
+                      block_size, top_k, 3)
+
+
+def int3_softmax_v_with_pre_corr_wvs2_inplace(scores, v_data, v_scales, block_table, seq_lens, topk_idx, weights,
+                                              o_hat, o_old_unnorm, W_out, max_S, H_q, H_kv, block_size, top_k) -> None:
+    """int3_softmax_v.cu:862-985: caller-owned outputs; `weights` is accepted and unused."""
+    _softmax_v(scores, None, None, v_data, v_scales, block_table, seq_lens, topk_idx, max_S, H_q, H_kv, block_size,
+               top_k, 3, outs=(o_hat, o_old_unnorm, W_out))
+
+
+def int3_softmax_v_with_pre_corr(scores, v_data, v_scales, block_table, seq_lens, topk_idx, max_S, H_q, H_kv,
+                                 block_size, top_k) -> List[torch.Tensor]:
+    return int3_softmax_v_with_pre_corr_wvs2(scores, v_data, v_scales, block_table, seq_lens, topk_idx, max_S, H_q,
+                                             H_kv, block_size, top_k)
+
+
+def int3_softmax_v(scores, v_data, v_scales, block_table, seq_lens, max_S, H_q, H_kv, block_size) -> torch.Tensor:
+    return _softmax_v(scores, None, None, v_data, v_scales, block_table, seq_lens, None, max_S, H_q, H_kv, block_size,
+                      32, 3)[0]
 
 
 def int4_softmax_v_with_pre_corr_wvs2_scores(scores, v_data, v_scales, block_table, seq_lens, topk_idx, max_S, H_q,

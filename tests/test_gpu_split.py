@@ -160,6 +160,36 @@ def test_int3_scores_and_topk(B, Hq, Hkv, S, gs):
 
 
 @pytest.mark.parametrize("B,Hq,Hkv,S", CASES_A)
+@pytest.mark.parametrize("kb,gs", [(2, 64), (2, 128), (4, 64), (4, 128)])
+def test_int2_and_int4_scores_with_the_bf16_model(B, Hq, Hkv, S, kb, gs):
+    """int2_qk_scores (symmetric keys, empty k_zp) and int4_qk_scores: bf16 q times bf16-rounded keys."""
+    c = make_case(13 + S + gs + kb, B, Hq, Hkv, S, kb, 2, gs)
+    d = to_device(c)
+    scale = 128 ** -0.5
+    K = 32 if S < 64 else 64
+    o = ops()
+    if kb == 2:
+        scores, idx, slots = o.int2_qk_scores_topk(d["q"], d["kd"], d["ks"], None, d["bt"], d["lens"], S, Hq, Hkv, 16, scale, K)
+        with pytest.raises(NotImplementedError):
+            o.int2_qk_scores(d["q"], d["kd"], d["ks"], d["ks"], d["bt"], d["lens"], S, Hq, Hkv, 16, scale)
+    else:
+        scores, idx, slots, m, iz = o.int4_qk_scores_topk_stats(d["q"], d["kd"], d["ks"], d["bt"], d["lens"], S, Hq, Hkv,
+                                                                16, scale, K)
+    ref = O.scores_bf16_model(c["q"], c["kd"], c["ks"], c["bt"], c["lens"], S, Hq, Hkv, 16, scale, kb, gs)
+    got = scores.cpu().numpy()
+    valid = np.isfinite(ref)
+    assert np.array_equal(np.isneginf(got), ~valid)
+    np.testing.assert_allclose(got[valid], ref[valid], atol=2e-5, rtol=2e-5)   # validate_runtime.py:147-148
+    ridx, rslots = O.topk_select(got, c["lens"], c["bt"], S, K)
+    assert np.array_equal(idx.cpu().numpy(), ridx)
+    assert np.array_equal(slots.cpu().numpy(), rslots)
+    if kb == 4:
+        rm, riz = O.softmax_stats(got, c["lens"], S)
+        np.testing.assert_allclose(m.cpu().numpy(), rm, rtol=0, atol=0)
+        np.testing.assert_allclose(iz.cpu().numpy(), riz, rtol=2e-5)
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,S", CASES_A)
 def test_int8tc_scores_bit_exact_topk_and_stats(B, Hq, Hkv, S):
     c = make_case(21 + S, B, Hq, Hkv, S, 4, 4, 128)
     d = to_device(c)
@@ -226,10 +256,11 @@ def test_unsupported_top_k_raises():
 # ------------------------------------------------------------------ Stage B + merge
 
 
-@pytest.mark.parametrize("scheme", ("k3v2", "k4v4", "k3v2_g128"))
+@pytest.mark.parametrize("scheme", ("k3v2", "k4v4", "k3v2_g128", "k3v3", "k3v3_g128"))
 @pytest.mark.parametrize("B,Hq,Hkv,lens", [(2, 8, 2, None), (3, 32, 4, [17, 257, 512]), (4, 8, 2, [0, 1, 9, 17])])
 def test_stage_b_outputs(scheme, B, Hq, Hkv, lens):
-    kb, vb, gs = {"k3v2": (3, 2, 64), "k4v4": (4, 4, 128), "k3v2_g128": (3, 2, 128)}[scheme]
+    kb, vb, gs = {"k3v2": (3, 2, 64), "k4v4": (4, 4, 128), "k3v2_g128": (3, 2, 128), "k3v3": (3, 3, 64),
+                  "k3v3_g128": (3, 3, 128)}[scheme]
     S = 512 if lens is None or max(lens) > 32 else 32
     c = make_case(31 + B, B, Hq, Hkv, S, kb, vb, gs, lens=lens)
     d = to_device(c)
@@ -242,7 +273,8 @@ def test_stage_b_outputs(scheme, B, Hq, Hkv, lens):
         ref_sc = O.scores_int8_model(c["q"], c["kd"], c["ks"], c["bt"], c["lens"], S, Hq, Hkv, 16, scale)
     ridx, _ = O.topk_select(ref_sc, c["lens"], c["bt"], S, K)
     sc_t, idx_t = torch.from_numpy(ref_sc).cuda(), torch.from_numpy(ridx).cuda()
-    fn = o.int2_softmax_v_with_pre_corr_wvs2 if vb == 2 else o.int4_softmax_v_with_pre_corr_wvs2_scores
+    fn = {2: o.int2_softmax_v_with_pre_corr_wvs2, 3: o.int3_softmax_v_with_pre_corr_wvs2,
+          4: o.int4_softmax_v_with_pre_corr_wvs2_scores}[vb]
     o_hat, o_old, W = fn(sc_t, d["vd"], d["vs"], d["bt"], d["lens"], idx_t, S, Hq, Hkv, 16, K)
     r_hat, r_old, r_W = O.softmax_v(ref_sc, c["vd"], c["vs"], c["bt"], c["lens"], ridx, S, Hq, Hkv, 16, vb, gs)
     np.testing.assert_allclose(o_hat.cpu().numpy(), r_hat, atol=3e-6, rtol=3e-6)     # validate_runtime.py:173-177
