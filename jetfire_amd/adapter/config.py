@@ -17,11 +17,11 @@ class QuantScheme:
     default_group_size: int = 128
 
 
-# the two schemes this library implements (jetfire_vllm/artifact.py:59 gives their group sizes)
-SCHEMES = {
-    "SymInt3K_SymInt2V": QuantScheme("SymInt3K_SymInt2V", 3, 2, default_group_size=64),
-    "SymInt4K_SymInt4V": QuantScheme("SymInt4K_SymInt4V", 4, 4, default_group_size=128),
-}
+# the nine symmetric schemes of jetfire_vllm/adapter/config.py:91-163 (the asymmetric INT2-key ones are not
+# implemented); jetfire_vllm/artifact.py:59 gives the group sizes of the two release schemes
+SCHEMES = {f"SymInt{k}K_SymInt{v}V": QuantScheme(f"SymInt{k}K_SymInt{v}V", k, v,
+                                                 default_group_size=64 if (k, v) == (3, 2) else 128)
+           for k in (2, 3, 4) for v in (2, 3, 4)}
 
 
 @dataclass(frozen=True)

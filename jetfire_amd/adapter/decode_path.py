@@ -23,8 +23,9 @@ from .. import ops
 from .config import get_jetfire_config
 from .kv_pool import get_global_kv_pool_manager
 
-# correction widths the fused kernels take (the split entry points go up to 8192)
+# correction widths the fused kernels take; the split entry points go up to 8192
 FUSED_SUPPORTED_TOP_K = (32, 64, 128, 256, 512, 1024)
+SPLIT_SUPPORTED_TOP_K = ops.SUPPORTED_TOP_K
 
 _TOPK_CLAMP_LOGGED: set = set()
 _HEAD_MAP_CACHE: dict = {}
@@ -181,16 +182,18 @@ def warmup_graph_decode_submit_contexts(*, max_batch_size: int, device=None, sca
     pool = get_global_kv_pool_manager()
     if not pool.layer_stores:
         raise RuntimeError("JETFIRE_DECODE_GRAPH=1 cannot warm submit contexts before JetFire layer stores exist.")
-    top_k = _select_top_k(cfg.topk, cfg.topk, FUSED_SUPPORTED_TOP_K)
-    if top_k is None:
-        raise RuntimeError(f"JETFIRE_TOPK={cfg.topk} is not supported by the active kernel set.")
-    widths = tuple(k for k in FUSED_SUPPORTED_TOP_K if k <= top_k) or (top_k,)
     sizes = _graph_context_batch_sizes(int(max_batch_size))
     created = 0
+    widths = ()
     for name, store in pool.layer_stores.items():
         layer_cfg = pool.get_layer_config(name)
-        if layer_cfg is None or store.scheme is None or not store.shadow_enabled:
+        if layer_cfg is None or not store.shadow_enabled:
             continue
+        supported = FUSED_SUPPORTED_TOP_K if store.scheme is not None else SPLIT_SUPPORTED_TOP_K
+        top_k = _select_top_k(cfg.topk, cfg.topk, supported)
+        if top_k is None:
+            raise RuntimeError(f"JETFIRE_TOPK={cfg.topk} is not supported by the active kernel set.")
+        widths = tuple(k for k in supported if k <= top_k) or (top_k,)
         store.warmup_graph_append(int(max_batch_size))
         sc = float(scale) if scale is not None else 1.0 / math.sqrt(layer_cfg.head_dim)
         for n in sizes:
@@ -211,6 +214,30 @@ def reset_jetfire_decode_runtime_state() -> None:
     _O_NEW.clear()
     _HEAD_MAP_CACHE.clear()
     _SEQ_LENS_CACHE.clear()
+
+
+def _split_stages(store, q, bt, sl, max_S: int, H_q: int, H_kv: int, top_k: int, scale: float):
+    """Stage A and Stage B as separate kernels, each side chosen by its bit width as the reference does
+    (`decode_path.py:2013-2131` Stage A, `:2695-2935` Stage B): the path of the schemes that have no fused kernel."""
+    bs = store.block_size
+    m = iz = None
+    kd, ks, vd, vs = store.k_data, store.k_scales, store.v_data, store.v_scales
+    if store.k_nbits == 4:
+        int8tc = (ks.shape[-1] == 1 and top_k >= 64 and os.environ.get("JETFIRE_USE_INT8_TC", "1") == "1")
+        stage_a = ops.int8tc_qk_scores_topk_stats if int8tc else ops.int4_qk_scores_topk_stats
+        scores, idx, slots, m, iz = stage_a(q, kd, ks, bt, sl, max_S, H_q, H_kv, bs, scale, top_k)
+    elif store.k_nbits == 3:
+        scores, idx, slots = ops.int3_qk_scores_topk(q, kd, ks, bt, sl, max_S, H_q, H_kv, bs, scale, top_k)
+    else:
+        scores, idx, slots = ops.int2_qk_scores_topk(q, kd, ks, None, bt, sl, max_S, H_q, H_kv, bs, scale, top_k)
+    if store.v_nbits == 4 and m is not None and vs.shape[-1] == 1:
+        o_hat, o_old, W = ops.int8tc_softmax_v_with_pre_corr_reg_stats(scores, m, iz, vd, vs, bt, sl, idx, max_S, H_q, H_kv,
+                                                                      bs, top_k)
+    else:
+        stage_b = {2: ops.int2_softmax_v_with_pre_corr_wvs2, 3: ops.int3_softmax_v_with_pre_corr_wvs2,
+                   4: ops.int4_softmax_v_with_pre_corr_wvs2_scores}[store.v_nbits]
+        o_hat, o_old, W = stage_b(scores, vd, vs, bt, sl, idx, max_S, H_q, H_kv, bs, top_k)
+    return o_hat, slots, o_old, W
 
 
 def try_jetfire_decode(*, impl, layer, query, attn_metadata, output, key=None, value=None):
@@ -240,7 +267,7 @@ def _decode_batched(*, impl, layer, query, attn_metadata, output):
     store = pool.get_layer_store(layer_name)
     if store is None:
         return miss("store_missing")
-    if store.scheme is None or store.block_size != 16 or layer_cfg.head_dim != 128 or not store.shadow_enabled:
+    if store.block_size != 16 or layer_cfg.head_dim != 128 or not store.shadow_enabled or store.k_scales.shape[-1] > 2:
         return miss("scheme_unsupported")
     store.flush_pending_writes()
 
@@ -263,7 +290,8 @@ def _decode_batched(*, impl, layer, query, attn_metadata, output):
         if not complete:
             return miss("store_incomplete")
         max_S = int(getattr(attn_metadata, "max_seq_len", int(seq_lens_cpu.max().item())))
-    top_k = _select_top_k(pool.config.topk, max_S, FUSED_SUPPORTED_TOP_K)
+    fused = store.scheme is not None and os.environ.get("JETFIRE_USE_FUSED_ATTN_TOPK", "1") == "1"
+    top_k = _select_top_k(pool.config.topk, max_S, FUSED_SUPPORTED_TOP_K if fused else SPLIT_SUPPORTED_TOP_K)
     if top_k is None:
         return miss("seq_len_too_short")
 
@@ -271,9 +299,12 @@ def _decode_batched(*, impl, layer, query, attn_metadata, output):
     bt_batch = attn_metadata.block_table[:n_seqs].to(torch.int64).contiguous()
     seq_lens_batch = attn_metadata.seq_lens.to(device=query.device, dtype=torch.int32).contiguous()
 
-    o_hat, topk_slots, o_old, W, _ = ops.fused_attn_topk(
-        store.scheme, q_batch, store.k_data, store.k_scales, store.v_data, store.v_scales, bt_batch, seq_lens_batch,
-        max_S, H_q, H_kv, store.block_size, top_k, scale)
+    if fused:
+        o_hat, topk_slots, o_old, W, _ = ops.fused_attn_topk(
+            store.scheme, q_batch, store.k_data, store.k_scales, store.v_data, store.v_scales, bt_batch, seq_lens_batch,
+            max_S, H_q, H_kv, store.block_size, top_k, scale)
+    else:
+        o_hat, topk_slots, o_old, W = _split_stages(store, q_batch, bt_batch, seq_lens_batch, max_S, H_q, H_kv, top_k, scale)
     handoff = _handoff_for(store, n_seqs, H_q, H_kv, top_k, scale, stream_mode=graph_mode, layer_name=layer_name)
     o_new = _o_new_for(n_seqs, H_q, D, query.device)
     out_view = output[:n_seqs].view(n_seqs, H_q, D)

@@ -530,19 +530,27 @@ def head_map(B: int, H_q: int, num_groups: int, K: int) -> np.ndarray:
 
 
 def decode_reference(q, k_data, k_scale_bits, v_data, v_scale_bits, block_table, seq_lens, max_S,
-                     H_q, H_kv, block_size, attn_scale, top_k, scheme: str, k_shadow=None, v_shadow=None):
+                     H_q, H_kv, block_size, attn_scale, top_k, scheme: str, k_shadow=None, v_shadow=None,
+                     group_size: int | None = None, k_model: str | None = None):
     """Whole per-layer decode step in the reference's order (decode_path.py:2081-2131,2785-2935,3126-3226).
-    scheme: "k3v2" (group 64) or "k4v4" (group 128).  Returns a dict of every intermediate."""
-    if scheme == "k3v2":
-        sc = scores_bf16_model(q, k_data, k_scale_bits, block_table, seq_lens, max_S, H_q, H_kv,
-                               block_size, attn_scale, 3, 64)
-        vb, vg = 2, 64
-    elif scheme == "k4v4":
+    scheme: "k<kb>v<vb>" with kb, vb in {2, 3, 4}; group_size defaults to 64 for "k3v2" and 128 otherwise
+    (jetfire_vllm/artifact.py:59).  k_model: "bf16" (bf16 q times bf16-rounded keys: the INT2 / INT3 / native
+    INT4 Stage A) or "int8" (INT4 keys with one scale per slot through the int8 tensor-core Stage A,
+    decode_path.py:2013-2024); default "int8" for 4-bit keys at group 128, else "bf16".
+    Returns a dict of every intermediate."""
+    kb, vb = int(scheme[1]), int(scheme[3])
+    if group_size is None:
+        group_size = 64 if scheme == "k3v2" else 128
+    if k_model is None:
+        k_model = "int8" if (kb == 4 and group_size == 128) else "bf16"
+    if k_model == "int8":
+        assert kb == 4 and group_size == 128
         sc = scores_int8_model(q, k_data, k_scale_bits, block_table, seq_lens, max_S, H_q, H_kv,
                                block_size, attn_scale)
-        vb, vg = 4, 128
     else:
-        raise ValueError(scheme)
+        sc = scores_bf16_model(q, k_data, k_scale_bits, block_table, seq_lens, max_S, H_q, H_kv,
+                               block_size, attn_scale, kb, group_size)
+    vg = group_size
     idx, slots = topk_select(sc, seq_lens, block_table, max_S, top_k, block_size)
     m, iz = softmax_stats(sc, seq_lens, max_S)
     o_hat, o_old, W = softmax_v(sc, v_data, v_scale_bits, block_table, seq_lens, idx, max_S, H_q, H_kv,

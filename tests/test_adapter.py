@@ -97,8 +97,12 @@ def test_pool_registry_and_store_geometry(adapter):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("scheme_name,scheme,gs,kb,vb", [("SymInt3K_SymInt2V", "k3v2", 64, 3, 2),
-                                                         ("SymInt4K_SymInt4V", "k4v4", 128, 4, 4)])
+@pytest.mark.parametrize("scheme_name,scheme,gs,kb,vb", [
+    ("SymInt3K_SymInt2V", "k3v2", 64, 3, 2), ("SymInt4K_SymInt4V", "k4v4", 128, 4, 4),      # fused kernels
+    # the pairs without a fused kernel run Stage A and Stage B as separate kernels chosen by bit width
+    ("SymInt2K_SymInt2V", "k2v2", 128, 2, 2), ("SymInt2K_SymInt3V", "k2v3", 128, 2, 3), ("SymInt2K_SymInt4V", "k2v4", 128, 2, 4),
+    ("SymInt3K_SymInt3V", "k3v3", 64, 3, 3), ("SymInt3K_SymInt4V", "k3v4", 128, 3, 4),
+    ("SymInt4K_SymInt2V", "k4v2", 128, 4, 2), ("SymInt4K_SymInt3V", "k4v3", 64, 4, 3)])
 def test_prefill_then_decode_steps_match_the_oracle(adapter, scheme_name, scheme, gs, kb, vb):
     B, Hq, Hkv, D, bs = 3, 8, 2, 128, 16
     lens0 = [300, 37, 512]
@@ -160,7 +164,7 @@ def test_prefill_then_decode_steps_match_the_oracle(adapter, scheme_name, scheme
         assert np.array_equal(store.v_data.cpu().numpy()[:, filled], ref_vd[:, filled])
         assert np.array_equal(bf16_to_f32(store.k_shadow)[:, filled], Kfull[:, filled])
         r = O.decode_reference(q_np, ref_kd, ref_ks, ref_vd, ref_vs, bt, np.array(lens, np.int32), max(lens), Hq, Hkv, bs,
-                               D ** -0.5, 64, scheme, Kfull, Vfull)
+                               D ** -0.5, 64, scheme, Kfull, Vfull, group_size=gs)
         res = bf16_to_f32(out[:B]).reshape(B, Hq, D)
         np.testing.assert_allclose(res, r["out"], atol=6e-3, rtol=1.5e-2)                # validate_runtime.py:195
         err = np.abs(res - r["out"])

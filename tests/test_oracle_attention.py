@@ -28,12 +28,13 @@ def make_case(seed, B, Hq, Hkv, S, kbits, vbits, gs, ragged=True, shuffle=True):
                 V=V.transpose(1, 0, 2).copy(), S=S, B=B, Hq=Hq, Hkv=Hkv)
 
 
-def test_bf16_score_model_one_hot_query_reads_one_dequantised_channel():
-    c = make_case(1, 2, 8, 2, 64, 3, 2, 64)
+@pytest.mark.parametrize("kbits,gs", [(3, 64), (2, 64), (2, 128), (4, 64), (4, 128)])
+def test_bf16_score_model_one_hot_query_reads_one_dequantised_channel(kbits, gs):
+    c = make_case(1, 2, 8, 2, 64, kbits, 2, gs)
     q = np.zeros_like(c["q"])
     q[:, :, 37] = 1.0
-    sc = O.scores_bf16_model(q, c["kd"], c["ks"], c["bt"], c["lens"], 64, 8, 2, 16, 0.5, 3, 64)
-    khat = O.unpack(c["kd"], c["ks"], 64, 3)
+    sc = O.scores_bf16_model(q, c["kd"], c["ks"], c["bt"], c["lens"], 64, 8, 2, 16, 0.5, kbits, gs)
+    khat = O.unpack(c["kd"], c["ks"], gs, kbits)
     slots = O.slots_from_block_table(c["bt"], 64)
     for b in range(2):
         S = c["lens"][b]
@@ -110,25 +111,26 @@ def test_radix_key_is_order_preserving():
     assert (np.diff(k) > 0).all()
 
 
-def test_softmax_v_invariants():
-    c = make_case(6, 2, 8, 2, 96, 3, 2, 64)
-    sc = O.scores_bf16_model(c["q"], c["kd"], c["ks"], c["bt"], c["lens"], 96, 8, 2, 16, 128 ** -0.5, 3, 64)
+@pytest.mark.parametrize("vbits,vg", [(2, 64), (3, 64), (3, 128), (4, 64)])
+def test_softmax_v_invariants(vbits, vg):
+    c = make_case(6, 2, 8, 2, 96, 3, vbits, vg)
+    sc = O.scores_bf16_model(c["q"], c["kd"], c["ks"], c["bt"], c["lens"], 96, 8, 2, 16, 128 ** -0.5, 3, vg)
     # K >= S: all positions selected -> W == 1, o_old == o_hat
     idx, _ = O.topk_select(sc, c["lens"], c["bt"], 96, 128)
-    o_hat, o_old, W = O.softmax_v(sc, c["vd"], c["vs"], c["bt"], c["lens"], idx, 96, 8, 2, 16, 2, 64)
+    o_hat, o_old, W = O.softmax_v(sc, c["vd"], c["vs"], c["bt"], c["lens"], idx, 96, 8, 2, 16, vbits, vg)
     np.testing.assert_allclose(W, 1.0, atol=1e-6)
     np.testing.assert_allclose(o_old, o_hat, atol=1e-6)
     # uniform scores: o_hat is the plain mean of the dequantised V rows
     flat = np.where(np.isfinite(sc), np.float32(0.25), sc)
-    o_hat, o_old, W = O.softmax_v(flat, c["vd"], c["vs"], c["bt"], c["lens"], None, 96, 8, 2, 16, 2, 64)
-    v0 = O.dequant(c["vd"], c["vs"], 2, 64, bf16=False)
+    o_hat, o_old, W = O.softmax_v(flat, c["vd"], c["vs"], c["bt"], c["lens"], None, 96, 8, 2, 16, vbits, vg)
+    v0 = O.dequant(c["vd"], c["vs"], vbits, vg, bf16=False)
     slots = O.slots_from_block_table(c["bt"], 96)
     for b in range(2):
         S = c["lens"][b]
         np.testing.assert_allclose(o_hat[b, 5], v0[1, slots[b, :S]].mean(0), atol=2e-6)
     # partial top-k: 0 <= W <= 1 and W equals the softmax mass of the winners
     idx, _ = O.topk_select(sc, c["lens"], c["bt"], 96, 32)
-    _, _, W = O.softmax_v(sc, c["vd"], c["vs"], c["bt"], c["lens"], idx, 96, 8, 2, 16, 2, 64)
+    _, _, W = O.softmax_v(sc, c["vd"], c["vs"], c["bt"], c["lens"], idx, 96, 8, 2, 16, vbits, vg)
     assert (W > 0).all() and (W < 1).all()
     p = np.exp(sc[0, 0, :96].astype(np.float64))
     p /= p.sum()
