@@ -52,6 +52,17 @@ int jf_quant_write_sym(const uint16_t* x, int64_t x_stride_t, int64_t x_stride_h
                        uint16_t* out_scale, int64_t scale_stride_h, int64_t scale_stride_slot,
                        int64_t num_slots, int group_size, int nbits, void* stream);
 
+/* Asymmetric INT2 keys over the full codebook.  Replaces fused_quant_write_int2_asym
+ * (jetfire_vllm/kernels/fused_quant_write.py:36-133,204-239; golden form quantize_and_pack_asym,
+ * kernels/intN_pack.py:110-169): per group scale = bf16(max((xmax - xmin) / 3, 1e-8)),
+ * zp = bf16(xmin + 2 * scale), code = clamp(rint((x - zp) / scale), -2, 1) + 2, INT2 wire format; out_zp is
+ * (H_kv, num_slots, NG) bf16 with element strides.  Token rows must be 16-byte aligned. */
+int jf_quant_write_int2_asym(const uint16_t* x, int64_t x_stride_t, int64_t x_stride_h, const int64_t* slots,
+                             int64_t T, int H_kv, uint8_t* out_data, int64_t data_stride_h, int64_t data_stride_slot,
+                             uint16_t* out_scale, int64_t scale_stride_h, int64_t scale_stride_slot,
+                             uint16_t* out_zp, int64_t zp_stride_h, int64_t zp_stride_slot,
+                             int64_t num_slots, int group_size, void* stream);
+
 /* K and V of an INT4/INT4 cache in one launch.  Replaces fused_quant_write_int4_sym_kv
  * (jetfire_vllm/kernels/fused_quant_write.py:552-617). */
 int jf_quant_write_int4_sym_kv(const uint16_t* key, int64_t k_stride_t, int64_t k_stride_h,
@@ -102,9 +113,11 @@ int jf_int3_qk_scores(const uint16_t* q, const uint8_t* k_data, const uint16_t* 
 /* The bf16 model of jf_int3_qk_scores for any symmetric key width: k_nbits 2 replaces int2_qk_scores with an
  * empty k_zp (jetfire_vllm/csrc/int2_qk_scores.cu:279-420: codes - 2, four per byte MSB first), 3 is
  * jf_int3_qk_scores, 4 replaces int4_qk_scores (jetfire_vllm/csrc/int4_qk_scores.cu:280-420: nibbles - 8,
- * (even << 4) | odd).  k_data (H_kv, num_slots, 16 * k_nbits), k_scales (H_kv, num_slots, n_scale_groups). */
+ * (even << 4) | odd).  k_data (H_kv, num_slots, 16 * k_nbits), k_scales (H_kv, num_slots, n_scale_groups).
+ * k_zp: NULL for symmetric keys; for the asymmetric INT2 keys (AsymInt2K4Level schemes) the zero-points
+ * (H_kv, num_slots, n_scale_groups) bf16: keys are bf16(fma(code - 2, scale, zp)). */
 int jf_intn_qk_scores(int k_nbits, const uint16_t* q, const uint8_t* k_data, const uint16_t* k_scales,
-                      const int64_t* block_table, const int32_t* seq_lens, int B, int H_q, int H_kv,
+                      const uint16_t* k_zp, const int64_t* block_table, const int32_t* seq_lens, int B, int H_q, int H_kv,
                       int max_S, int max_blocks, int64_t num_slots, int n_scale_groups, int block_size,
                       float attn_scale, float* scores, void* stream);
 int jf_int8tc_qk_scores(const uint16_t* q, const uint8_t* k_data, const uint16_t* k_scales,

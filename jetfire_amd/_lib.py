@@ -26,7 +26,8 @@ SIGNATURES = {
     "jf_shadow_write": (I, [P, L, L, P, L, L, P, L, I, P, P, L, L, L, P]),
     "jf_host_buffer_device_pointer": (I, [P, P]),
     "jf_int3_qk_scores": (I, [P, P, P, P, P, I, I, I, I, I, L, I, I, F, P, P]),
-    "jf_intn_qk_scores": (I, [I, P, P, P, P, P, I, I, I, I, I, L, I, I, F, P, P]),
+    "jf_intn_qk_scores": (I, [I, P, P, P, P, P, P, I, I, I, I, I, L, I, I, F, P, P]),
+    "jf_quant_write_int2_asym": (I, [P, L, L, P, L, I, P, L, L, P, L, L, P, L, L, L, I, P]),
     "jf_int8tc_qk_scores": (I, [P, P, P, P, P, I, I, I, I, I, L, I, F, P, P]),
     "jf_topk_slots": (I, [P, P, P, I, I, I, I, I, I, P, P, P, P, P]),
     "jf_softmax_v_workspace_bytes": (Z, [I, I, I]),

@@ -55,15 +55,16 @@ class JetFireLayerView:
 
 
 class JetFireInt4CacheStore:
-    """Quantised KV cache of one layer.  Independent K and V bit widths (2, 3 or 4), symmetric only."""
+    """Quantised KV cache of one layer.  Independent K and V bit widths (2, 3 or 4), symmetric, plus the
+    asymmetric INT2 keys (full four-level codebook with a zero-point per group, `k_zp`)."""
 
     def __init__(self, *, num_kv_heads: int, head_dim: int, group_size: int, num_blocks: int, block_size: int,
                  device, k_nbits: int, v_nbits: int, k_asymmetric: bool = False, v_asymmetric: bool = False,
                  shadow_enabled: bool = True) -> None:
         if head_dim % group_size != 0:
             raise ValueError(f"head_dim={head_dim} must be divisible by group_size={group_size}")
-        if k_asymmetric or v_asymmetric:
-            raise NotImplementedError("asymmetric (zero-point) schemes are outside this library's decode path")
+        if v_asymmetric or (k_asymmetric and int(k_nbits) != 2):
+            raise NotImplementedError("only INT2 keys have an asymmetric (zero-point) form in this library")
         if int(k_nbits) not in (2, 3, 4) or int(v_nbits) not in (2, 3, 4):
             raise ValueError(f"unsupported bit widths k={k_nbits} v={v_nbits}")
         self.num_kv_heads = int(num_kv_heads)
@@ -74,7 +75,7 @@ class JetFireInt4CacheStore:
         self.num_slots = self.num_blocks * self.block_size
         self.device = torch.device(device)
         self.k_nbits, self.v_nbits = int(k_nbits), int(v_nbits)
-        self.k_asymmetric = self.v_asymmetric = False
+        self.k_asymmetric, self.v_asymmetric = bool(k_asymmetric), False
         ng = self.head_dim // self.group_size
         dev = self.device
         # zero-initialised: positions past a sequence's end are never scored, but they are read
@@ -82,7 +83,8 @@ class JetFireInt4CacheStore:
         self.k_scales = torch.zeros(self.num_kv_heads, self.num_slots, ng, dtype=torch.bfloat16, device=dev)
         self.v_data = torch.zeros(self.num_kv_heads, self.num_slots, packed_dim(self.head_dim, self.v_nbits), dtype=torch.uint8, device=dev)
         self.v_scales = torch.zeros(self.num_kv_heads, self.num_slots, ng, dtype=torch.bfloat16, device=dev)
-        self.k_zp = self.v_zp = None
+        self.v_zp = None
+        self.k_zp = torch.zeros(self.num_kv_heads, self.num_slots, ng, dtype=torch.bfloat16, device=dev) if self.k_asymmetric else None
         # one spare entry at the end takes the marks of padding tokens (slot < 0), so that marking needs no mask
         self._slot_filled_buf = torch.zeros(self.num_slots + 1, dtype=torch.bool, device=dev)
         self.slot_filled = self._slot_filled_buf[:self.num_slots]
@@ -109,6 +111,8 @@ class JetFireInt4CacheStore:
     @property
     def scheme(self) -> str | None:
         """Name the fused decode kernels know this store by, or None (split kernels / unsupported)."""
+        if self.k_asymmetric:
+            return None
         if (self.k_nbits, self.v_nbits) == (3, 2) and self.group_size in (64, 128):
             return "k3v2"
         if (self.k_nbits, self.v_nbits) == (4, 4) and self.group_size == 128:
@@ -127,11 +131,14 @@ class JetFireInt4CacheStore:
         return n, slots, key_tok, value_tok
 
     def _quantise(self, key_tok, value_tok, slots) -> None:
-        if self.k_nbits == 4 and self.v_nbits == 4:
+        sym = {2: ops.fused_quant_write_int2_sym, 3: ops.fused_quant_write_int3_sym, 4: ops.fused_quant_write_int4_sym}
+        if self.k_asymmetric:
+            ops.fused_quant_write_int2_asym(key_tok, slots, self.k_data, self.k_scales, self.k_zp, self.group_size)
+            sym[self.v_nbits](value_tok, slots, self.v_data, self.v_scales, self.group_size)
+        elif self.k_nbits == 4 and self.v_nbits == 4:
             ops.fused_quant_write_int4_sym_kv(key_tok, value_tok, slots, self.k_data, self.k_scales, self.v_data,
                                               self.v_scales, self.group_size)
         else:
-            sym = {2: ops.fused_quant_write_int2_sym, 3: ops.fused_quant_write_int3_sym, 4: ops.fused_quant_write_int4_sym}
             sym[self.k_nbits](key_tok, slots, self.k_data, self.k_scales, self.group_size)
             sym[self.v_nbits](value_tok, slots, self.v_data, self.v_scales, self.group_size)
 
@@ -253,4 +260,5 @@ class JetFireInt4CacheStore:
         slots = self.sequence_slots(block_table_row, seq_len)
         return JetFireLayerView(k_data=self.k_data.index_select(1, slots), k_scales=self.k_scales.index_select(1, slots),
                                 v_data=self.v_data.index_select(1, slots), v_scales=self.v_scales.index_select(1, slots),
-                                seq_len=int(seq_len))
+                                seq_len=int(seq_len),
+                                k_zp=self.k_zp.index_select(1, slots) if self.k_zp is not None else None)

@@ -17,11 +17,15 @@ class QuantScheme:
     default_group_size: int = 128
 
 
-# the nine symmetric schemes of jetfire_vllm/adapter/config.py:91-163 (the asymmetric INT2-key ones are not
-# implemented); jetfire_vllm/artifact.py:59 gives the group sizes of the two release schemes
+# the schemes of jetfire_vllm/adapter/config.py:91-163 that have kernels there: the nine symmetric pairs and the
+# asymmetric INT2 keys; jetfire_vllm/artifact.py:59 gives the group sizes of the two release schemes
 SCHEMES = {f"SymInt{k}K_SymInt{v}V": QuantScheme(f"SymInt{k}K_SymInt{v}V", k, v,
                                                  default_group_size=64 if (k, v) == (3, 2) else 128)
            for k in (2, 3, 4) for v in (2, 3, 4)}
+# INT2 keys over the full four-level codebook with a zero-point per group, and their historical aliases
+for _v in (2, 3, 4):
+    SCHEMES[f"AsymInt2K4Level_SymInt{_v}V"] = QuantScheme(f"AsymInt2K4Level_SymInt{_v}V", 2, _v, k_asymmetric=True)
+    SCHEMES[f"AsymInt2K_SymInt{_v}V"] = SCHEMES[f"AsymInt2K4Level_SymInt{_v}V"]
 
 
 @dataclass(frozen=True)

@@ -229,7 +229,7 @@ def _split_stages(store, q, bt, sl, max_S: int, H_q: int, H_kv: int, top_k: int,
     elif store.k_nbits == 3:
         scores, idx, slots = ops.int3_qk_scores_topk(q, kd, ks, bt, sl, max_S, H_q, H_kv, bs, scale, top_k)
     else:
-        scores, idx, slots = ops.int2_qk_scores_topk(q, kd, ks, None, bt, sl, max_S, H_q, H_kv, bs, scale, top_k)
+        scores, idx, slots = ops.int2_qk_scores_topk(q, kd, ks, store.k_zp, bt, sl, max_S, H_q, H_kv, bs, scale, top_k)
     if store.v_nbits == 4 and m is not None and vs.shape[-1] == 1:
         o_hat, o_old, W = ops.int8tc_softmax_v_with_pre_corr_reg_stats(scores, m, iz, vd, vs, bt, sl, idx, max_S, H_q, H_kv,
                                                                       bs, top_k)

@@ -72,7 +72,7 @@ __global__ __launch_bounds__(QK_THREADS) void int3_qk_scores_kernel(
 template <int KBITS, int G, int NG>
 __global__ __launch_bounds__(QK_THREADS) void intn_qk_scores_kernel(
     const uint16_t* __restrict__ q, const uint8_t* __restrict__ k_data, const uint16_t* __restrict__ k_scales,
-    const int64_t* __restrict__ block_table, const int32_t* __restrict__ seq_lens, float* __restrict__ scores,
+    const uint16_t* __restrict__ k_zp, const int64_t* __restrict__ block_table, const int32_t* __restrict__ seq_lens, float* __restrict__ scores,
     int H_q, int H_kv, int max_S, int max_blocks, int64_t num_slots, int bs, float attn_scale) {
   static_assert(KBITS == 2 || KBITS == 4, "planar INT3 rows have their own kernel");
   constexpr int P = D * KBITS / 8, NDW = P / 4, OFF = 1 << (KBITS - 1);
@@ -95,22 +95,26 @@ __global__ __launch_bounds__(QK_THREADS) void intn_qk_scores_kernel(
   uint32_t p[NDW];
 #pragma unroll
   for (int i = 0; i < NDW; ++i) p[i] = row[i];
-  float sc[NG];
+  // asymmetric keys add a zero-point per group: bf16(fma(code - off, scale, zp)) (int2_qk_scores.cu:66-79)
+  float sc[NG], zp[NG];
 #pragma unroll
-  for (int g = 0; g < NG; ++g) sc[g] = bf16_to_f32(k_scales[((size_t)hkv * num_slots + slot) * NG + g]);
+  for (int g = 0; g < NG; ++g) {
+    sc[g] = bf16_to_f32(k_scales[((size_t)hkv * num_slots + slot) * NG + g]);
+    zp[g] = k_zp ? bf16_to_f32(k_zp[((size_t)hkv * num_slots + slot) * NG + g]) : 0.0f;
+  }
   float acc[G];
 #pragma unroll
   for (int g = 0; g < G; ++g) acc[g] = 0.0f;
 #pragma unroll
   for (int gi = 0; gi < 16; ++gi) {  // eight channels at a time
-    const float scale = sc[(gi * 8 * NG) / D];
+    const float scale = sc[(gi * 8 * NG) / D], zero = zp[(gi * 8 * NG) / D];
     float kv[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       int code;
       if (KBITS == 4) code = (int)((p[gi] >> (8 * (j >> 1) + ((j & 1) ? 0 : 4))) & 15u);
       else code = (int)((p[gi >> 1] >> (16 * (gi & 1) + 8 * (j >> 2) + (6 - 2 * (j & 3)))) & 3u);
-      kv[j] = bf16_to_f32(f32_to_bf16((float)(code - OFF) * scale));
+      kv[j] = bf16_to_f32(f32_to_bf16(__builtin_fmaf((float)(code - OFF), scale, zero)));
     }
 #pragma unroll
     for (int g = 0; g < G; ++g)
@@ -271,9 +275,10 @@ extern "C" int jf_int3_qk_scores(const uint16_t* q, const uint8_t* k_data, const
 }
 
 extern "C" int jf_intn_qk_scores(int k_nbits, const uint16_t* q, const uint8_t* k_data, const uint16_t* k_scales,
-                                 const int64_t* block_table, const int32_t* seq_lens, int B, int H_q, int H_kv,
+                                 const uint16_t* k_zp, const int64_t* block_table, const int32_t* seq_lens, int B, int H_q, int H_kv,
                                  int max_S, int max_blocks, int64_t num_slots, int n_scale_groups, int block_size,
                                  float attn_scale, float* scores, void* stream) {
+  JF_CHECK_ARG(k_zp == nullptr || k_nbits == 2, "intn_qk_scores: zero-points are only defined for INT2 keys");
   if (k_nbits == 3)
     return jf_int3_qk_scores(q, k_data, k_scales, block_table, seq_lens, B, H_q, H_kv, max_S, max_blocks, num_slots,
                              n_scale_groups, block_size, attn_scale, scores, stream);
@@ -288,7 +293,7 @@ extern "C" int jf_intn_qk_scores(int k_nbits, const uint16_t* q, const uint8_t* 
   hipStream_t st = (hipStream_t)stream;
   const int G = H_q / H_kv;
 #define JF_INTN_LAUNCH(KB, NGV)                                                                                        \
-  hipLaunchKernelGGL((intn_qk_scores_kernel<KB, GG, NGV>), grid, block, 0, st, q, k_data, k_scales, block_table,      \
+  hipLaunchKernelGGL((intn_qk_scores_kernel<KB, GG, NGV>), grid, block, 0, st, q, k_data, k_scales, k_zp, block_table, \
                      seq_lens, scores, H_q, H_kv, max_S, max_blocks, num_slots, block_size, attn_scale)
   JF_DISPATCH_G(G, {
     if (k_nbits == 2) {

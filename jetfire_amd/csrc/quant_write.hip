@@ -173,6 +173,57 @@ __global__ __launch_bounds__(256) void quant_write16_kernel(RowSrc s0, RowDst d0
   }
 }
 
+// Asymmetric INT2 keys over the full codebook (jetfire_vllm/kernels/intN_pack.py:110-169,
+// fused_quant_write.py:85-133): per group scale = bf16(max((xmax - xmin) / 3, 1e-8)),
+// zp = bf16(xmin + 2 * scale_f32), code = clamp(rint((x - zp) / scale), -2, 1) + 2.  Same lane layout as
+// quant_write16_kernel (sixteen lanes per row, eight channels per lane); the divisions are IEEE divisions:
+// the numerator x - zp is not a bf16 value, so the reciprocal shortcut of the symmetric kernel does not apply.
+__global__ __launch_bounds__(256) void quant_write16_int2_asym_kernel(RowSrc s, RowDst d, uint16_t* __restrict__ zp_out,
+                                                                      int64_t zp_stride_h, int64_t zp_stride_slot,
+                                                                      const int64_t* __restrict__ slots, int64_t T,
+                                                                      int group_size) {
+  const int l16 = threadIdx.x & 15;
+  const int64_t tq = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+  const int h = blockIdx.y;
+  const bool inside = tq < T;
+  const int64_t t = inside ? tq : 0;
+  const int64_t slot = slots[t];
+  const uint16_t* xrow = s.x + t * s.stride_t + (int64_t)h * s.stride_h;
+  const uint4 raw = reinterpret_cast<const uint4*>(xrow)[l16];
+  const bool live = inside && slot >= 0;
+  float x[8];
+  x[0] = bf16_to_f32((uint16_t)(raw.x & 0xffffu)); x[1] = bf16_to_f32((uint16_t)(raw.x >> 16));
+  x[2] = bf16_to_f32((uint16_t)(raw.y & 0xffffu)); x[3] = bf16_to_f32((uint16_t)(raw.y >> 16));
+  x[4] = bf16_to_f32((uint16_t)(raw.z & 0xffffu)); x[5] = bf16_to_f32((uint16_t)(raw.z >> 16));
+  x[6] = bf16_to_f32((uint16_t)(raw.w & 0xffffu)); x[7] = bf16_to_f32((uint16_t)(raw.w >> 16));
+  float xmax = x[0], xmin = x[0];
+#pragma unroll
+  for (int i = 1; i < 8; ++i) {
+    xmax = fmaxf(xmax, x[i]);
+    xmin = fminf(xmin, x[i]);
+  }
+  xmax = fmaxf(xmax, dpp_f32<0xB1>(xmax)); xmin = fminf(xmin, dpp_f32<0xB1>(xmin));
+  xmax = fmaxf(xmax, dpp_f32<0x4E>(xmax)); xmin = fminf(xmin, dpp_f32<0x4E>(xmin));
+  if (group_size >= 64) { xmax = fmaxf(xmax, dpp_f32<0x141>(xmax)); xmin = fminf(xmin, dpp_f32<0x141>(xmin)); }
+  if (group_size >= 128) { xmax = fmaxf(xmax, dpp_f32<0x140>(xmax)); xmin = fminf(xmin, dpp_f32<0x140>(xmin)); }
+  const float sraw = fmaxf((xmax - xmin) / 3.0f, 1e-8f);
+  const float zraw = xmin + 2.0f * sraw;
+  const uint16_t sb = f32_to_bf16(sraw), zb = f32_to_bf16(zraw);
+  const float sf = bf16_to_f32(sb), zf = bf16_to_f32(zb);
+  uint32_t c[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) c[i] = (uint32_t)((int)fminf(fmaxf(rintf((x[i] - zf) / sf), -2.0f), 1.0f) + 2);
+  uint8_t* drow = d.data + (int64_t)h * d.data_stride_h + slot * d.data_stride_slot;
+  const int lpg = group_size >> 3;
+  if (live && (l16 & (lpg - 1)) == 0) {
+    d.scale[(int64_t)h * d.scale_stride_h + slot * d.scale_stride_slot + l16 / lpg] = sb;
+    zp_out[(int64_t)h * zp_stride_h + slot * zp_stride_slot + l16 / lpg] = zb;
+  }
+  const uint32_t hw = ((c[0] << 6) | (c[1] << 4) | (c[2] << 2) | c[3]) | (((c[4] << 6) | (c[5] << 4) | (c[6] << 2) | c[7]) << 8);
+  const uint32_t nb = dpp_u32<0xB1>(hw);
+  if (live && (l16 & 1) == 0) reinterpret_cast<uint32_t*>(drow)[l16 >> 1] = hw | (nb << 16);
+}
+
 // units = T * H_kv * n_tensors (n_tensors = 2 for the fused K+V INT4 launch)
 template <int NBITS>
 __global__ __launch_bounds__(256) void quant_write_kernel(RowSrc s0, RowDst d0, RowSrc s1, RowDst d1,
@@ -275,6 +326,25 @@ extern "C" int jf_quant_write_int4_sym_kv(const uint16_t* key, int64_t k_stride_
   }
   dim3 grid((unsigned)((units + 3) / 4)), block(256);
   hipLaunchKernelGGL(quant_write_kernel<4>, grid, block, 0, (hipStream_t)stream, s0, d0, s1, d1, slots, T, H_kv, 2, group_size);
+  JF_CHECK_LAUNCH();
+  return JF_OK;
+}
+
+extern "C" int jf_quant_write_int2_asym(const uint16_t* x, int64_t x_stride_t, int64_t x_stride_h, const int64_t* slots,
+                                        int64_t T, int H_kv, uint8_t* out_data, int64_t data_stride_h,
+                                        int64_t data_stride_slot, uint16_t* out_scale, int64_t scale_stride_h,
+                                        int64_t scale_stride_slot, uint16_t* out_zp, int64_t zp_stride_h,
+                                        int64_t zp_stride_slot, int64_t num_slots, int group_size, void* stream) {
+  (void)num_slots;
+  int rc = check_common(x, slots, T, H_kv, group_size, data_stride_slot, 2, out_data, out_scale);
+  if (rc != JF_OK || T == 0) return rc;
+  JF_CHECK_ARG(out_zp, "quant_write_int2_asym: null zero-point tensor");
+  JF_CHECK_ARG(rows_16b_aligned(x, x_stride_t, x_stride_h), "quant_write_int2_asym: token rows must be 16-byte aligned");
+  RowSrc s{x, x_stride_t, x_stride_h};
+  RowDst d{out_data, data_stride_h, data_stride_slot, out_scale, scale_stride_h, scale_stride_slot};
+  dim3 grid((unsigned)((T + 15) / 16), (unsigned)H_kv, 1), block(256);
+  hipLaunchKernelGGL(quant_write16_int2_asym_kernel, grid, block, 0, (hipStream_t)stream, s, d, out_zp, zp_stride_h,
+                     zp_stride_slot, slots, T, group_size);
   JF_CHECK_LAUNCH();
   return JF_OK;
 }

@@ -89,6 +89,32 @@ def fused_quant_write_int4_sym(value_tok, slot_idx, v_data, v_scales, group_size
     _quant_write(value_tok, slot_idx, v_data, v_scales, group_size, 4)
 
 
+def fused_quant_write_int2_asym(key_tok, slots, out_data, out_scale, out_zp, group_size: int) -> None:
+    """fused_quant_write.py:204-239: asymmetric INT2 keys over the full codebook, in place."""
+    lib = _lib.load()
+    _check(key_tok.is_cuda and key_tok.dtype == torch.bfloat16 and key_tok.dim() == 3 and key_tok.shape[2] == HEAD_DIM,
+           "key_tok must be (T, H_kv, 128) bf16 on the GPU")
+    _check(key_tok.stride(2) == 1, "tokens must be contiguous in the last dimension")
+    T, H_kv, D = key_tok.shape
+    _check(D % group_size == 0, f"D={D} not divisible by gs={group_size}")
+    if out_scale.dim() == 2:
+        out_scale = out_scale.unsqueeze(-1)
+    if out_zp.dim() == 2:
+        out_zp = out_zp.unsqueeze(-1)
+    _check(out_data.dtype == torch.uint8 and out_data.shape[0] == H_kv and out_data.shape[2] == D // 4
+           and out_data.stride(2) == 1, "cache data must be (H_kv, num_slots, 32) uint8")
+    for t in (out_scale, out_zp):
+        _check(t.dtype == torch.bfloat16 and t.shape[0] == H_kv and t.shape[2] == D // group_size and t.stride(2) == 1,
+               "scales / zero-points must be (H_kv, num_slots, D / group_size) bf16")
+    _check(slots.is_cuda and slots.dtype == torch.int64 and slots.shape == (T,), "slots must be (T,) int64")
+    slots = slots.contiguous()
+    _lib.check(lib.jf_quant_write_int2_asym(
+        key_tok.data_ptr(), key_tok.stride(0), key_tok.stride(1), slots.data_ptr(), T, H_kv,
+        out_data.data_ptr(), out_data.stride(0), out_data.stride(1), out_scale.data_ptr(), out_scale.stride(0),
+        out_scale.stride(1), out_zp.data_ptr(), out_zp.stride(0), out_zp.stride(1), out_data.shape[1], int(group_size),
+        _stream(key_tok)))
+
+
 def fused_quant_write_int4_sym_kv(key_tok, value_tok, slot_idx, k_data, k_scales, v_data, v_scales,
                                   group_size: int) -> None:
     """fused_quant_write.py:552-617 (K and V in one launch)."""
@@ -193,29 +219,30 @@ def int3_qk_scores(q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_kv,
 
 
 def _intn_qk_scores(nbits: int, name: str, q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_kv, block_size,
-                    attn_scale):
+                    attn_scale, k_zp=None):
     lib = _lib.load()
     q, kd, ks, bt, sl = _stage_a_args(q, k_data, k_scales, block_table, seq_lens, H_q, H_kv, HEAD_DIM * nbits // 8)
     ng = ks.size(2)
     _check(ng in (1, 2), f"{name} currently supports K quant groups 1 or 2, got {ng}")
+    if k_zp is not None:
+        k_zp = (k_zp.unsqueeze(-1) if k_zp.dim() == 2 else k_zp).contiguous()
+        _check(k_zp.is_cuda and k_zp.dtype == torch.bfloat16 and k_zp.shape == ks.shape,
+               "k_zp must be bf16 with the shape of k_scales")
     B = q.size(0)
     scores = torch.empty((B, H_q, max_S), dtype=torch.float32, device=q.device)
-    _lib.check(lib.jf_intn_qk_scores(nbits, q.data_ptr(), kd.data_ptr(), ks.data_ptr(), bt.data_ptr(), sl.data_ptr(),
+    _lib.check(lib.jf_intn_qk_scores(nbits, q.data_ptr(), kd.data_ptr(), ks.data_ptr(), _ptr(k_zp), bt.data_ptr(), sl.data_ptr(),
                                      B, H_q, H_kv, int(max_S), bt.size(1), kd.size(1), ng, int(block_size),
                                      float(attn_scale), scores.data_ptr(), _stream(q)))
     return scores
 
 
-def _no_zero_point(k_zp, name: str) -> None:
-    if k_zp is not None and k_zp.numel() > 0:
-        raise NotImplementedError(f"{name}: asymmetric INT2 keys (k_zp) are outside this library's decode path")
-
-
 def int2_qk_scores(q, k_data, k_scales, k_zp, block_table, seq_lens, max_S, H_q, H_kv, block_size, attn_scale):
-    """int2_qk_scores.cu:279-420 for symmetric keys (`k_zp` empty or None) -> scores (B, H_q, max_S) fp32."""
-    _no_zero_point(k_zp, "int2_qk_scores")
+    """int2_qk_scores.cu:279-420 -> scores (B, H_q, max_S) fp32.  `k_zp` empty or None: symmetric keys; else the
+    zero-points of the asymmetric INT2 keys, shaped like `k_scales`."""
+    if k_zp is not None and k_zp.numel() == 0:
+        k_zp = None
     return _intn_qk_scores(2, "int2_qk_scores", q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_kv, block_size,
-                           attn_scale)
+                           attn_scale, k_zp)
 
 
 def int2_qk_scores_topk(q, k_data, k_scales, k_zp, block_table, seq_lens, max_S, H_q, H_kv, block_size, attn_scale,

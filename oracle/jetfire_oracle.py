@@ -171,6 +171,47 @@ def quantize_and_pack(x: np.ndarray, group_size: int = 128, nbits: int = 4):
     return pack_codes(codes, nbits), sbits
 
 
+def quantize_codes_asym(x: np.ndarray, group_size: int, nbits: int = 2):
+    """Golden asymmetric quantiser over the full codebook (intN_pack.py:110-169; the fused writer
+    fused_quant_write.py:85-133 uses the same formulas): per group
+        scale = bf16(max((xmax - xmin) / (2^n - 1), 1e-8)),  zp = bf16(xmin + 2^(n-1) * scale_f32),
+        q = clamp(rint((x - f32(zp)) / f32(scale)), -2^(n-1), 2^(n-1) - 1),  code = q + 2^(n-1).
+    All arithmetic is IEEE float32.  Returns (codes uint8 (..., D), scale bits, zp bits uint16 (..., D/gs))."""
+    x = np.asarray(x, dtype=np.float32)
+    lead, D = x.shape[:-1], x.shape[-1]
+    assert D % group_size == 0
+    ng = D // group_size
+    off = offset(nbits)
+    xg = x.reshape(*lead, ng, group_size)
+    xmax, xmin = xg.max(axis=-1), xg.min(axis=-1)
+    scale = np.maximum((xmax - xmin).astype(np.float32) / np.float32(2 * off - 1), np.float32(1e-8)).astype(np.float32)
+    zp = (xmin + (np.float32(off) * scale).astype(np.float32)).astype(np.float32)
+    sbits, zbits = f32_to_bf16_bits(scale), f32_to_bf16_bits(zp)
+    sf, zf = bf16_bits_to_f32(sbits)[..., None], bf16_bits_to_f32(zbits)[..., None]
+    with np.errstate(over="ignore", invalid="ignore"):
+        q = np.rint(((xg - zf).astype(np.float32) / sf).astype(np.float32))
+    q = np.clip(q, -off, off - 1).astype(np.int32) + off
+    return q.reshape(*lead, D).astype(np.uint8), sbits, zbits
+
+
+def quantize_and_pack_asym(x: np.ndarray, group_size: int = 128, nbits: int = 2):
+    """(data uint8 (..., packed_dim), scale bits, zp bits uint16 (..., D/gs))."""
+    codes, sbits, zbits = quantize_codes_asym(x, group_size, nbits)
+    return pack_codes(codes, nbits), sbits, zbits
+
+
+def dequant_asym_bf16(data, scale_bits, zp_bits, nbits: int, group_size: int) -> np.ndarray:
+    """bf16(fma(code - offset, f32(scale), f32(zp))): what the Stage A kernel feeds its matrix unit
+    (int2_qk_scores.cu:66-79: `float(q) * scale + zp` is one fused multiply-add under nvcc's default
+    contraction, then __float2bfloat16)."""
+    codes = decode_codes(data, nbits).astype(np.float32) - np.float32(offset(nbits))
+    shape = codes.shape
+    s = bf16_bits_to_f32(scale_bits).reshape(*shape[:-1], -1)[..., None]
+    z = bf16_bits_to_f32(zp_bits).reshape(*shape[:-1], -1)[..., None]
+    c = codes.reshape(*shape[:-1], -1, group_size)
+    return bf16_round(fmaf(c, np.broadcast_to(s, c.shape), np.broadcast_to(z, c.shape))).reshape(shape)
+
+
 def dequant(data, scale_bits, nbits: int, group_size: int, *, bf16: bool = True) -> np.ndarray:
     """(code - offset) * f32(scale); optionally rounded to bf16 (validate_runtime.py:35-43)."""
     codes = decode_codes(data, nbits).astype(np.float32) - np.float32(offset(nbits))
@@ -213,7 +254,7 @@ def slots_from_block_table(block_table: np.ndarray, max_S: int, block_size: int 
 
 
 def scores_bf16_model(q, k_data, k_scale_bits, block_table, seq_lens, max_S, H_q, H_kv,
-                      block_size, attn_scale, nbits: int, group_size: int) -> np.ndarray:
+                      block_size, attn_scale, nbits: int, group_size: int, k_zp_bits=None) -> np.ndarray:
     """scores[b,h,s] = f32(sum_d q_d * bf16(code_d*scale_g)) * attn_scale; -inf for s >= seq_len.
 
     int3_qk_scores.cu:90-99 (bf16 rounding of every dequantised K element),
@@ -225,7 +266,10 @@ def scores_bf16_model(q, k_data, k_scale_bits, block_table, seq_lens, max_S, H_q
     q = np.asarray(q, dtype=np.float32)
     B = q.shape[0]
     G = H_q // H_kv
-    khat = dequant(k_data, k_scale_bits, nbits, group_size, bf16=True).astype(np.float64)
+    if k_zp_bits is None:
+        khat = dequant(k_data, k_scale_bits, nbits, group_size, bf16=True).astype(np.float64)
+    else:   # asymmetric keys (int2_qk_scores.cu:66-79)
+        khat = dequant_asym_bf16(k_data, k_scale_bits, k_zp_bits, nbits, group_size).astype(np.float64)
     slots = slots_from_block_table(block_table, max_S, block_size)
     out = np.full((B, H_q, max_S), -np.inf, dtype=np.float32)
     for b in range(B):
@@ -531,7 +575,7 @@ def head_map(B: int, H_q: int, num_groups: int, K: int) -> np.ndarray:
 
 def decode_reference(q, k_data, k_scale_bits, v_data, v_scale_bits, block_table, seq_lens, max_S,
                      H_q, H_kv, block_size, attn_scale, top_k, scheme: str, k_shadow=None, v_shadow=None,
-                     group_size: int | None = None, k_model: str | None = None):
+                     group_size: int | None = None, k_model: str | None = None, k_zp_bits=None):
     """Whole per-layer decode step in the reference's order (decode_path.py:2081-2131,2785-2935,3126-3226).
     scheme: "k<kb>v<vb>" with kb, vb in {2, 3, 4}; group_size defaults to 64 for "k3v2" and 128 otherwise
     (jetfire_vllm/artifact.py:59).  k_model: "bf16" (bf16 q times bf16-rounded keys: the INT2 / INT3 / native
@@ -549,7 +593,7 @@ def decode_reference(q, k_data, k_scale_bits, v_data, v_scale_bits, block_table,
                                block_size, attn_scale)
     else:
         sc = scores_bf16_model(q, k_data, k_scale_bits, block_table, seq_lens, max_S, H_q, H_kv,
-                               block_size, attn_scale, kb, group_size)
+                               block_size, attn_scale, kb, group_size, k_zp_bits)
     vg = group_size
     idx, slots = topk_select(sc, seq_lens, block_table, max_S, top_k, block_size)
     m, iz = softmax_stats(sc, seq_lens, max_S)
@@ -573,6 +617,11 @@ PINNED_BY = {
                       "[1, 2^n-1], |xhat-x| <= scale/2 unless clamped; brute-force ties (.5 -> even); "
                       "amax not bf16-representable -> clamp",
     "scores_bf16_model": "one-hot q gives the dequantised channel; agreement with dense float64 einsum",
+    "quantize_codes_asym": "no vector in the reference's tests; pinned by what the formulas fix: the group minimum maps "
+                           "to code 0 and the maximum to code 2^n-1, scale and zp reproduce intN_pack.py:121's closed "
+                           "form on exactly representable inputs, |xhat - x| <= scale/2 + rounding of zp inside the "
+                           "range, a constant group gives scale 1e-8 clamped, and the asymmetric grid is never worse "
+                           "than the symmetric one by more than 5 % MSE (the reference's own self-test, intN_pack.py:375-403)",
     "scores_int8_model": "agreement with validator restatement scores_int8_model_dense (validate_runtime.py:46-58) "
                          "within fp32 rounding; one-hot q closed form",
     "topk_select": "brute-force sort on tiny inputs; S<K: every valid position once then -1 "

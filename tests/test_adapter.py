@@ -89,9 +89,13 @@ def test_pool_registry_and_store_geometry(adapter):
         store.sequence_slots(row, 0)
     with pytest.raises(ValueError):
         store.sequence_slots(torch.tensor([0, -1]), 20)
-    with pytest.raises(NotImplementedError):
-        adapter.JetFireInt4CacheStore(num_kv_heads=2, head_dim=128, group_size=64, num_blocks=1, block_size=16,
-                                      device="cpu", k_nbits=2, v_nbits=2, k_asymmetric=True, v_asymmetric=False)
+    asym = adapter.JetFireInt4CacheStore(num_kv_heads=2, head_dim=128, group_size=64, num_blocks=1, block_size=16,
+                                         device="cpu", k_nbits=2, v_nbits=2, k_asymmetric=True, v_asymmetric=False)
+    assert asym.k_zp.shape == asym.k_scales.shape == (2, 16, 2) and asym.scheme is None     # INT2 keys with zero-points
+    for kw in (dict(k_nbits=3, v_nbits=2, k_asymmetric=True), dict(k_nbits=2, v_nbits=2, v_asymmetric=True)):
+        with pytest.raises(NotImplementedError):
+            adapter.JetFireInt4CacheStore(num_kv_heads=2, head_dim=128, group_size=64, num_blocks=1, block_size=16,
+                                          device="cpu", **kw)
     pool.mirror_kv("model.layers.1.attn", torch.zeros(1, 2, 128), torch.zeros(1, 2, 128), torch.tensor([0]))
     assert pool.skipped_layers == 1                                  # stride-skipped layer
 
@@ -102,7 +106,9 @@ def test_pool_registry_and_store_geometry(adapter):
     # the pairs without a fused kernel run Stage A and Stage B as separate kernels chosen by bit width
     ("SymInt2K_SymInt2V", "k2v2", 128, 2, 2), ("SymInt2K_SymInt3V", "k2v3", 128, 2, 3), ("SymInt2K_SymInt4V", "k2v4", 128, 2, 4),
     ("SymInt3K_SymInt3V", "k3v3", 64, 3, 3), ("SymInt3K_SymInt4V", "k3v4", 128, 3, 4),
-    ("SymInt4K_SymInt2V", "k4v2", 128, 4, 2), ("SymInt4K_SymInt3V", "k4v3", 64, 4, 3)])
+    ("SymInt4K_SymInt2V", "k4v2", 128, 4, 2), ("SymInt4K_SymInt3V", "k4v3", 64, 4, 3),
+    # asymmetric INT2 keys (zero-point per group)
+    ("AsymInt2K4Level_SymInt2V", "k2v2", 128, 2, 2), ("AsymInt2K_SymInt4V", "k2v4", 64, 2, 4)])
 def test_prefill_then_decode_steps_match_the_oracle(adapter, scheme_name, scheme, gs, kb, vb):
     B, Hq, Hkv, D, bs = 3, 8, 2, 128, 16
     lens0 = [300, 37, 512]
@@ -157,14 +163,20 @@ def test_prefill_then_decode_steps_match_the_oracle(adapter, scheme_name, scheme
         torch.cuda.synchronize()
         # the cache holds exactly what the oracle quantiser packs, the shadow the bf16 rows
         filled = store.slot_filled.cpu().numpy()
-        ref_kd, ref_ks = O.quantize_and_pack(Kfull, gs, kb)
+        asym = scheme_name.startswith("Asym")
+        if asym:
+            ref_kd, ref_ks, ref_kz = O.quantize_and_pack_asym(Kfull, gs, kb)
+            assert np.array_equal(bf16_to_bits(store.k_zp)[:, filled], ref_kz[:, filled])
+        else:
+            ref_kd, ref_ks = O.quantize_and_pack(Kfull, gs, kb)
+            ref_kz = None
         ref_vd, ref_vs = O.quantize_and_pack(Vfull, gs, vb)
         assert np.array_equal(store.k_data.cpu().numpy()[:, filled], ref_kd[:, filled])
         assert np.array_equal(bf16_to_bits(store.k_scales)[:, filled], ref_ks[:, filled])
         assert np.array_equal(store.v_data.cpu().numpy()[:, filled], ref_vd[:, filled])
         assert np.array_equal(bf16_to_f32(store.k_shadow)[:, filled], Kfull[:, filled])
         r = O.decode_reference(q_np, ref_kd, ref_ks, ref_vd, ref_vs, bt, np.array(lens, np.int32), max(lens), Hq, Hkv, bs,
-                               D ** -0.5, 64, scheme, Kfull, Vfull, group_size=gs)
+                               D ** -0.5, 64, scheme, Kfull, Vfull, group_size=gs, k_zp_bits=ref_kz)
         res = bf16_to_f32(out[:B]).reshape(B, Hq, D)
         np.testing.assert_allclose(res, r["out"], atol=6e-3, rtol=1.5e-2)                # validate_runtime.py:195
         err = np.abs(res - r["out"])

@@ -105,6 +105,52 @@ def test_pack_rounding_is_exact_for_every_mantissa_pair(bits):
     assert codes.min() == 1 and codes.max() == 2 * qm + 1                        # both ends of the code range occur
 
 
+@pytest.mark.parametrize("gs", (32, 64, 128))
+def test_asymmetric_int2_pack_and_scores(gs):
+    """fused_quant_write_int2_asym bit-exact against the oracle's quantize_and_pack_asym (codes, scale and
+    zero-point bits; scattered, masked, strided), then int2_qk_scores with those zero-points against the
+    oracle's bf16(fma(code - 2, scale, zp)) model."""
+    rng = np.random.default_rng(40 + gs)
+    T, H, nslots = 203, 4, 256
+    wide = O.bf16_round((rng.standard_normal((T, H, 136)) * 1.3 + rng.standard_normal((T, H, 1))).astype(np.float32))
+    wide[3, 1, :128] = 0.25                                              # a constant row: the 1e-8 floor
+    x = wide[..., :128]
+    slots = rng.permutation(nslots)[:T].astype(np.int64)
+    slots[::29] = -1
+    keep = slots >= 0
+    data = torch.zeros(H, nslots, 32, dtype=torch.uint8, device="cuda")
+    sc = torch.zeros(H, nslots, 128 // gs, dtype=torch.bfloat16, device="cuda")
+    zp = torch.zeros_like(sc)
+    o = ops()
+    o.fused_quant_write_int2_asym(bf16_tensor(wide).cuda()[..., :128], torch.from_numpy(slots).cuda(), data, sc, zp, gs)
+    rd, rs, rz = O.quantize_and_pack_asym(x, gs, 2)
+    got_d, got_s, got_z = data.cpu().numpy(), bf16_to_bits(sc), bf16_to_bits(zp)
+    assert np.array_equal(got_d[:, slots[keep]].transpose(1, 0, 2), rd[keep])
+    assert np.array_equal(got_s[:, slots[keep]].transpose(1, 0, 2), rs[keep])
+    assert np.array_equal(got_z[:, slots[keep]].transpose(1, 0, 2), rz[keep])
+    untouched = np.setdiff1d(np.arange(nslots), slots[keep])
+    assert not got_d[:, untouched].any() and not got_s[:, untouched].any()
+    if gs == 32:
+        return                                                           # Stage A takes one or two scale groups per row
+    # scores over the rows just written: one sequence whose positions are the kept slots in order
+    order = np.sort(slots[keep])
+    S = (len(order) // 16) * 16
+    blocks = np.arange(nslots // 16, dtype=np.int64)[None, :]
+    lens = np.array([S - 5], np.int32)
+    Hq = 8
+    q = O.bf16_round((rng.standard_normal((1, Hq, 128)) / np.sqrt(128)).astype(np.float32))
+    scores = o.int2_qk_scores(bf16_tensor(q).cuda(), data, sc, zp, torch.from_numpy(blocks).cuda(),
+                              torch.from_numpy(lens).cuda(), S, Hq, H, 16, 0.11)
+    ref = O.scores_bf16_model(q, got_d, got_s, blocks, lens, S, Hq, H, 16, 0.11, 2, gs, k_zp_bits=got_z)
+    got = scores.cpu().numpy()
+    valid = np.isfinite(ref)
+    assert np.array_equal(np.isneginf(got), ~valid)
+    np.testing.assert_allclose(got[valid], ref[valid], atol=2e-5, rtol=2e-5)
+    # an unaligned token view is refused, not mis-read
+    with pytest.raises(RuntimeError, match="16-byte"):
+        o.fused_quant_write_int2_asym(bf16_tensor(wide).cuda()[..., 2:130], torch.from_numpy(slots).cuda(), data, sc, zp, gs)
+
+
 def test_pack_int4_kv_single_launch_matches_two_launches():
     rng = np.random.default_rng(7)
     T, H = 70, 8
@@ -170,8 +216,6 @@ def test_int2_and_int4_scores_with_the_bf16_model(B, Hq, Hkv, S, kb, gs):
     o = ops()
     if kb == 2:
         scores, idx, slots = o.int2_qk_scores_topk(d["q"], d["kd"], d["ks"], None, d["bt"], d["lens"], S, Hq, Hkv, 16, scale, K)
-        with pytest.raises(NotImplementedError):
-            o.int2_qk_scores(d["q"], d["kd"], d["ks"], d["ks"], d["bt"], d["lens"], S, Hq, Hkv, 16, scale)
     else:
         scores, idx, slots, m, iz = o.int4_qk_scores_topk_stats(d["q"], d["kd"], d["ks"], d["bt"], d["lens"], S, Hq, Hkv,
                                                                 16, scale, K)

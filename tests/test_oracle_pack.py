@@ -161,3 +161,47 @@ def test_fmaf_is_correctly_rounded():
         up = Fraction(float(np.nextafter(got[i], np.float32(np.inf))))
         dn = Fraction(float(np.nextafter(got[i], np.float32(-np.inf))))
         assert abs(g - exact) <= abs(up - exact) and abs(g - exact) <= abs(dn - exact)
+
+
+@pytest.mark.parametrize("gs", (32, 64, 128))
+def test_asymmetric_int2_quantiser_is_pinned_by_its_closed_form(gs):
+    """quantize_and_pack_asym (intN_pack.py:110-169) has no vector in the reference's tests; what the formulas
+    fix: scale = (max - min) / 3 and zp = min + 2 * scale on exactly representable inputs, the group minimum
+    maps to code 0 and the maximum to code 3, a point of the grid maps to itself, the error inside the range is
+    at most scale / 2 (+ the bf16 rounding of zp), a constant group takes the 1e-8 floor, and the reference's own
+    self-test (:375-403): the asymmetric grid is not worse than the symmetric one by more than 5 % MSE."""
+    # closed form: a group spanning [-1, 2] exactly: scale 1, zp 1, grid {-1, 0, 1, 2}
+    x = np.zeros((1, 128), np.float32)
+    x[0, ::4], x[0, 1::4], x[0, 2::4], x[0, 3::4] = -1.0, 0.0, 1.0, 2.0
+    codes, sb, zb = O.quantize_codes_asym(x, gs, 2)
+    assert (O.bf16_bits_to_f32(sb) == 1.0).all() and (O.bf16_bits_to_f32(zb) == 1.0).all()
+    assert np.array_equal(codes[0, :4], [0, 1, 2, 3])
+    # ties at .5 round to even: -0.5 -> q = rint(-1.5) = -2 -> code 0 ; 0.5 -> rint(-0.5) = -0 -> code 2
+    y = x.copy(); y[0, 5], y[0, 6] = -0.5, 0.5
+    cy, _, _ = O.quantize_codes_asym(y, gs, 2)
+    assert cy[0, 5] == 0 and cy[0, 6] == 2
+    rng = np.random.default_rng(gs)
+    x = O.bf16_round((rng.standard_normal((64, 128)) * 1.7 + rng.standard_normal((64, 1))).astype(np.float32))
+    codes, sb, zb = O.quantize_codes_asym(x, gs, 2)
+    xg, cg = x.reshape(64, -1, gs), codes.reshape(64, -1, gs)
+    assert codes.min() == 0 and codes.max() == 3
+    assert (cg[np.arange(64)[:, None], np.arange(128 // gs)[None, :], xg.argmin(-1)] == 0).all()
+    assert (cg[np.arange(64)[:, None], np.arange(128 // gs)[None, :], xg.argmax(-1)] == 3).all()
+    data, sb2, zb2 = O.quantize_and_pack_asym(x, gs, 2)
+    assert np.array_equal(sb, sb2) and np.array_equal(O.decode_codes(data, 2), codes)
+    sf, zf = O.bf16_bits_to_f32(sb)[..., None], O.bf16_bits_to_f32(zb)[..., None]
+    xhat = (cg.astype(np.float32) - 2) * sf + zf
+    inside = (xg >= zf - 2 * sf) & (xg <= zf + sf)
+    assert (np.abs(xhat - xg)[inside] <= sf.repeat(gs, -1)[inside] * 0.5 + 1e-6).all()
+    # the kernel's dequant (one fma, then bf16) stays within bf16 rounding of that grid
+    kd = O.dequant_asym_bf16(data, sb, zb, 2, gs).reshape(64, -1, gs)
+    assert (np.abs(kd - xhat) <= np.abs(xhat) * 2.0 ** -8 + 1e-30).all()
+    # a constant group: scale takes the floor, every element lands on one code
+    c = np.full((2, 128), 0.375, np.float32)
+    cc, cs, cz = O.quantize_codes_asym(c, gs, 2)
+    assert (O.bf16_bits_to_f32(cs) == O.bf16_round(np.float32(1e-8))).all() and len(np.unique(cc)) == 1
+    # the reference's self-test criterion
+    sd, ss = O.quantize_and_pack(x, gs, 2)
+    sym_mse = ((O.dequant(sd, ss, 2, gs, bf16=False) - x) ** 2).mean()
+    asym_mse = ((xhat.reshape(64, 128) - x) ** 2).mean()
+    assert asym_mse <= sym_mse * 1.05
