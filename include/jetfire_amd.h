@@ -34,6 +34,8 @@ extern "C" {
 
 #define JF_SCHEME_K3V2 32    /* INT3 keys, INT2 values  (SymInt3K_SymInt2V) */
 #define JF_SCHEME_K4V4 44    /* INT4 keys, INT4 values  (SymInt4K_SymInt4V) */
+#define JF_SCHEME_K3V4 34    /* INT3 keys, INT4 values  (SymInt3K_SymInt4V), group 128 */
+#define JF_SCHEME_K4V2 42    /* INT4 keys, INT2 values  (SymInt4K_SymInt2V), group 128 */
 
 const char* jf_last_error(void);
 const char* jf_version(void);
@@ -164,8 +166,9 @@ int jf_softmax_v_pre_corr(const float* scores, const float* softmax_m, const flo
  * reference's Stage A + Stage B pair produces (jetfire_vllm/adapter/decode_path.py:2081-2131,
  * 2785-2935): topk_idx, topk_slots, o_hat, o_old_unnorm, W, and optionally softmax_m / softmax_inv_z.
  * The reference's own single-call form of this contract is int2_fused_attn_topk
- * (jetfire_vllm/kernels/int2_fused_attn_topk.py:5-10).  scheme: JF_SCHEME_K3V2 (group 64 or 128) or
- * JF_SCHEME_K4V4 (group 128).  top_k: power of two in [32, 1024] (the split entry points above take up
+ * (jetfire_vllm/kernels/int2_fused_attn_topk.py:5-10).  scheme: JF_SCHEME_K3V2 (group 64 or 128), or
+ * JF_SCHEME_K4V4 / JF_SCHEME_K3V4 / JF_SCHEME_K4V2 (group 128): INT3 keys score with the bf16 model of
+ * jf_int3_qk_scores, INT4 keys with the int8-Q model of jf_int8tc_qk_scores.  top_k: power of two in [32, 1024] (the split entry points above take up
  * to 8192); num_slots at most 2^25 (row offsets are 32-bit).  If scores is non-NULL the fp32 scores are also written (validation).
  * workspace: jf_fused_workspace_bytes() bytes of device memory. */
 size_t jf_fused_workspace_bytes(int scheme, int B, int H_q, int H_kv, int max_S, int top_k);

@@ -115,8 +115,8 @@ class JetFireInt4CacheStore:
             return None
         if (self.k_nbits, self.v_nbits) == (3, 2) and self.group_size in (64, 128):
             return "k3v2"
-        if (self.k_nbits, self.v_nbits) == (4, 4) and self.group_size == 128:
-            return "k4v4"
+        if (self.k_nbits, self.v_nbits) in ((4, 4), (3, 4), (4, 2)) and self.group_size == 128:
+            return f"k{self.k_nbits}v{self.v_nbits}"
         return None
 
     # ------------------------------------------------------------------ append

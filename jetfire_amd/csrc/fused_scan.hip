@@ -113,7 +113,11 @@ struct QInt8F {
 // After the selection the whole block is reused for the exchange of the P.V accumulators.
 template <int SCHEME, int G, int NG>
 struct ScanLds {
-  static constexpr bool K3 = (SCHEME == JF_SCHEME_K3V2);
+  // SCHEME = 10 * key bits + value bits: the key side (staging, query constants, phase A) and the value side
+  // (staging, phase B) are chosen independently
+  static constexpr bool K3 = (SCHEME / 10 == 3);
+  static constexpr bool V2 = (SCHEME % 10 == 2);
+  static_assert((K3 || SCHEME / 10 == 4) && (V2 || SCHEME % 10 == 4), "keys are INT3 or INT4, values INT2 or INT4");
   static constexpr int NSET = (G + 3) / 4;
   // wavefronts per workgroup: sixteen where the register budget allows (128 VGPRs at 1024 threads), else eight
   static constexpr int NW = (G <= 4) ? 16 : 8;
@@ -123,11 +127,11 @@ struct ScanLds {
   static constexpr int SEG = (NW / G >= 4) ? 4 : ((NW / G >= 2) ? 2 : 1);
   static constexpr int KP = K3 ? 48 : 64;
   static constexpr int KROW = K3 ? 48 : 80;     // LDS pitch of a staged key row (INT4: padded against bank conflicts)
-  static constexpr int VP = K3 ? 32 : 64;
+  static constexpr int VP = V2 ? 32 : 64;
   // LDS pitch of a staged V row.  INT2 rows (32 bytes) are padded so that 16 consecutive rows hit 16 distinct
   // bank pairs; INT4 rows (64 bytes) keep their pitch and swap their 16-byte quarters instead (quarter q of
   // row r sits at q ^ ((r >> 2) & 3)), which has the same effect without the padding bytes.
-  static constexpr bool VSWZ = !K3;
+  static constexpr bool VSWZ = !V2;
   static constexpr int VROW = VSWZ ? VP : VP + 8;
   static constexpr int VST = 64 * VROW;
   static constexpr int WL = NG * NSET * 64 * 16;  // per (group, set): one 16-byte weight row per token
@@ -140,9 +144,9 @@ struct ScanLds {
   // with one head set and enough staging space the exchange runs in the staging area while the score rows
   // are still being read by the candidate emission
   static constexpr int PREP = K3 ? (int)sizeof(K3Prep<NSET>) : (int)sizeof(QInt8F<NSET>);
-  // selection histograms: 32-bit counters, or (INT4 scheme, where LDS is tighter) two 16-bit counters per
-  // word: a (head, segment) histogram counts at most LMAX / SEG <= 4096 positions
-  static constexpr bool H16 = !K3;
+  // selection histograms: 32-bit counters, or (any INT4 side, where the staging areas are larger and LDS is
+  // tighter) two 16-bit counters per word: a (head, segment) histogram counts at most LMAX / SEG <= 4096 positions
+  static constexpr bool H16 = !(K3 && V2);
   static constexpr int HIST = G * SEG * 256 * (H16 ? 2 : 4);
   static constexpr int AUX = ((PREP > HIST ? PREP : HIST) + 15) & ~15;
   __host__ __device__ static constexpr int stage_bytes() { return NW * WAVE_STAGE; }
@@ -189,13 +193,14 @@ template <int SCHEME, int G, int NG>
 __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kernel(FusedParams p) {
   using Lds = ScanLds<SCHEME, G, NG>;
   constexpr bool K3 = Lds::K3;
+  constexpr bool V2 = Lds::V2;
   constexpr int NSET = Lds::NSET;
   constexpr int SEG = Lds::SEG;
   constexpr int KP = Lds::KP;
   constexpr int KROW = Lds::KROW;
   constexpr int VP = Lds::VP;
   constexpr int VROW = Lds::VROW;
-  constexpr int VOFF = K3 ? 2 : 8;  // code offset of the V format
+  constexpr int VOFF = V2 ? 2 : 8;  // code offset of the V format
   constexpr int NTILE = 8;          // 8 MFMA column tiles of 16 channels
   constexpr int AR = Lds::ACC_REGS;
   constexpr float LOG2E = 1.44269504088896340736f;
@@ -861,7 +866,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     // the nibble spread of a transposed V dword yields tokens 0,2,4,6 | 1,3,5,7 | 8,10,12,14 | 9,11,13,15 of the
     // lane group's 16 tokens: token r sits in byte (r&8) | ((r&1)<<2) | ((r>>1)&3)
     const uint8_t* vrow = vst + lane * VROW;
-    if (K3) {
+    if (V2) {
 #pragma unroll
       for (int qc = 0; qc < 4; ++qc) {
         const v2i x = __builtin_amdgcn_ds_read_tr4_b64_v2i32((__attribute__((address_space(3))) v2i*)(vrow + 8 * qc));
@@ -960,7 +965,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
       const int h = set * 4 + hh;
       if (h >= G) continue;
       int d;
-      if (K3) {
+      if (V2) {
         const int e = ((col & 1) ? 0 : 2) + (tile & 1);
         d = (tile >> 1) * 32 + (col >> 1) * 4 + e;
       } else {
@@ -1780,6 +1785,10 @@ inline int lmax_dispatch(int scheme, int G, int NG) {
   JF_LMAX_CASE(JF_SCHEME_K3V2, 8, 2); JF_LMAX_CASE(JF_SCHEME_K3V2, 16, 2);
   JF_LMAX_CASE(JF_SCHEME_K4V4, 1, 1); JF_LMAX_CASE(JF_SCHEME_K4V4, 2, 1); JF_LMAX_CASE(JF_SCHEME_K4V4, 4, 1);
   JF_LMAX_CASE(JF_SCHEME_K4V4, 8, 1); JF_LMAX_CASE(JF_SCHEME_K4V4, 16, 1);
+  JF_LMAX_CASE(JF_SCHEME_K3V4, 1, 1); JF_LMAX_CASE(JF_SCHEME_K3V4, 2, 1); JF_LMAX_CASE(JF_SCHEME_K3V4, 4, 1);
+  JF_LMAX_CASE(JF_SCHEME_K3V4, 8, 1); JF_LMAX_CASE(JF_SCHEME_K3V4, 16, 1);
+  JF_LMAX_CASE(JF_SCHEME_K4V2, 1, 1); JF_LMAX_CASE(JF_SCHEME_K4V2, 2, 1); JF_LMAX_CASE(JF_SCHEME_K4V2, 4, 1);
+  JF_LMAX_CASE(JF_SCHEME_K4V2, 8, 1); JF_LMAX_CASE(JF_SCHEME_K4V2, 16, 1);
 #undef JF_LMAX_CASE
   return 256;
 }
@@ -1833,7 +1842,8 @@ inline void fused_plan(int scheme, int NG, int B, int H_q, int H_kv, int max_S, 
   const int nw = (G <= 4) ? 16 : 8;
   constexpr int kCUs = 256;
   constexpr double kScanFixed = 8.5;
-  const double per_chunk = (scheme == JF_SCHEME_K4V4) ? 6.6 : 5.9;  // one chunk per wavefront, all wavefronts
+  // one chunk per wavefront, all wavefronts; the mixed schemes are priced like the wider one
+  const double per_chunk = (scheme == JF_SCHEME_K3V2) ? 5.9 : 6.6;
   int L = 256;
   double best = -1.0;
   for (int cand = 256; cand <= lmax; cand += 256) {
@@ -1910,7 +1920,10 @@ int launch_scan(const FusedParams& p, hipStream_t st) {
   return JF_OK;
 }
 
-inline int scheme_ng(int scheme, int group_size) { return (scheme == JF_SCHEME_K4V4) ? 1 : D / group_size; }
+inline bool known_scheme(int scheme) {
+  return scheme == JF_SCHEME_K3V2 || scheme == JF_SCHEME_K4V4 || scheme == JF_SCHEME_K3V4 || scheme == JF_SCHEME_K4V2;
+}
+inline int scheme_ng(int scheme, int group_size) { return (scheme == JF_SCHEME_K3V2) ? D / group_size : 1; }
 
 }  // namespace
 }  // namespace jf
@@ -1934,7 +1947,7 @@ extern "C" size_t jf_fused_workspace_bytes(int scheme, int B, int H_q, int H_kv,
 
 extern "C" int jf_fused_plan(int scheme, int group_size, int B, int H_q, int H_kv, int max_S, int top_k,
                              int* split_len, int* n_splits, int* list_cap, int* merge_parts) {
-  JF_CHECK_ARG(scheme == JF_SCHEME_K3V2 || scheme == JF_SCHEME_K4V4, "fused_plan: unknown scheme %d", scheme);
+  JF_CHECK_ARG(known_scheme(scheme), "fused_plan: unknown scheme %d", scheme);
   JF_CHECK_ARG(B > 0 && H_q > 0 && H_kv > 0 && H_q % H_kv == 0 && max_S >= 0 && top_k > 0, "fused_plan: bad shape");
   JF_CHECK_ARG(group_size == 64 || group_size == 128, "fused_plan: group_size must be 64 or 128");
   int L, ns, kc, parts, spp;
@@ -1954,13 +1967,14 @@ extern "C" int jf_fused_scan_topk(int scheme, int group_size, const uint16_t* q,
                                   int top_k, int64_t* topk_idx, int64_t* topk_slots, float* o_hat,
                                   float* o_old_unnorm, float* W, float* softmax_m, float* softmax_inv_z, float* scores,
                                   void* workspace, size_t workspace_bytes, void* stream) {
-  JF_CHECK_ARG(scheme == JF_SCHEME_K3V2 || scheme == JF_SCHEME_K4V4, "fused_scan: unknown scheme %d", scheme);
+  JF_CHECK_ARG(known_scheme(scheme), "fused_scan: unknown scheme %d", scheme);
   JF_CHECK_ARG(B >= 0 && H_q > 0 && H_kv > 0 && max_S >= 0 && H_q % H_kv == 0, "fused_scan: bad shape");
   const int G = H_q / H_kv;
   JF_CHECK_ARG(G == 1 || G == 2 || G == 4 || G == 8 || G == 16, "fused_scan: GQA group %d not in {1,2,4,8,16}", G);
   JF_CHECK_ARG(block_size == 16, "fused_scan only supports block_size=16");
   JF_CHECK_ARG(group_size == 64 || group_size == 128, "fused_scan: group_size must be 64 or 128 (got %d)", group_size);
-  JF_CHECK_ARG(scheme != JF_SCHEME_K4V4 || group_size == 128, "fused_scan: the INT4 int8-Q path needs group_size 128");
+  JF_CHECK_ARG(scheme == JF_SCHEME_K3V2 || group_size == 128,
+               "fused_scan: the INT4 sides (int8-Q keys, INT4 values) need group_size 128");
   JF_CHECK_ARG(is_pow2(top_k) && top_k >= 32 && top_k <= FS_MAX_TOPK,
                "fused_scan: unsupported top_k=%d (supported: 32,64,128,256,512,1024; larger widths use the split-form operators)", top_k);
   JF_CHECK_ARG(max_S <= 262144, "fused_scan: max_S=%d exceeds supported limit (262144)", max_S);
@@ -2020,13 +2034,29 @@ extern "C" int jf_fused_scan_topk(int scheme, int group_size, const uint16_t* q,
         default: JF_FUSED_CASE(JF_SCHEME_K3V2, 16, 1); break;
       }
     }
-  } else {
+  } else if (scheme == JF_SCHEME_K4V4) {
     switch (G) {
       case 1: JF_FUSED_CASE(JF_SCHEME_K4V4, 1, 1); break;
       case 2: JF_FUSED_CASE(JF_SCHEME_K4V4, 2, 1); break;
       case 4: JF_FUSED_CASE(JF_SCHEME_K4V4, 4, 1); break;
       case 8: JF_FUSED_CASE(JF_SCHEME_K4V4, 8, 1); break;
       default: JF_FUSED_CASE(JF_SCHEME_K4V4, 16, 1); break;
+    }
+  } else if (scheme == JF_SCHEME_K3V4) {
+    switch (G) {
+      case 1: JF_FUSED_CASE(JF_SCHEME_K3V4, 1, 1); break;
+      case 2: JF_FUSED_CASE(JF_SCHEME_K3V4, 2, 1); break;
+      case 4: JF_FUSED_CASE(JF_SCHEME_K3V4, 4, 1); break;
+      case 8: JF_FUSED_CASE(JF_SCHEME_K3V4, 8, 1); break;
+      default: JF_FUSED_CASE(JF_SCHEME_K3V4, 16, 1); break;
+    }
+  } else {
+    switch (G) {
+      case 1: JF_FUSED_CASE(JF_SCHEME_K4V2, 1, 1); break;
+      case 2: JF_FUSED_CASE(JF_SCHEME_K4V2, 2, 1); break;
+      case 4: JF_FUSED_CASE(JF_SCHEME_K4V2, 4, 1); break;
+      case 8: JF_FUSED_CASE(JF_SCHEME_K4V2, 8, 1); break;
+      default: JF_FUSED_CASE(JF_SCHEME_K4V2, 16, 1); break;
     }
   }
   if (rc != JF_OK) return rc;
@@ -2043,7 +2073,7 @@ extern "C" int jf_fused_scan_topk(int scheme, int group_size, const uint16_t* q,
     if (big) hipLaunchKernelGGL((fused_merge_kernel<VB, NGG, 1024, 32, false>), mgrid, dim3(1024), 0, st, p); \
     else hipLaunchKernelGGL((fused_merge_kernel<VB, NGG, 1024, 8, false>), mgrid, dim3(1024), 0, st, p);       \
   } while (0)
-  if (scheme == JF_SCHEME_K3V2) {
+  if (scheme % 10 == 2) {  // INT2 values
     if (NGv == 2) JF_MERGE(2, 2);
     else JF_MERGE(2, 1);
   } else {

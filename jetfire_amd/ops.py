@@ -467,11 +467,12 @@ def fused_attn_topk(scheme: str, q, k_data, k_scales, v_data, v_scales, block_ta
     """One fused pass: -> (o_hat, topk_slots, o_old_unnorm, W, topk_idx[, softmax_m, softmax_inv_z][, scores]).
 
     The single-call contract is the one of the reference's int2_fused_attn_topk
-    (jetfire_vllm/kernels/int2_fused_attn_topk.py:5-10) extended to the K3V2 / K4V4 schemes."""
+    (jetfire_vllm/kernels/int2_fused_attn_topk.py:5-10) extended to INT3 / INT4 keys (INT4: the int8-Q scoring
+    model) with INT2 / INT4 values: "k3v2" (group 64 or 128), "k4v4", "k3v4", "k4v2" (group 128)."""
     lib = _lib.load()
-    scheme_id = {"k3v2": 32, "k4v4": 44}.get(scheme)
-    _check(scheme_id is not None, f"unknown scheme {scheme!r} (k3v2, k4v4)")
-    kp, vp = (48, 32) if scheme == "k3v2" else (64, 64)
+    scheme_id = {"k3v2": 32, "k4v4": 44, "k3v4": 34, "k4v2": 42}.get(scheme)
+    _check(scheme_id is not None, f"unknown scheme {scheme!r} (k3v2, k4v4, k3v4, k4v2)")
+    kp, vp = 16 * (scheme_id // 10), 16 * (scheme_id % 10)
     q, kd, ks, bt, sl = _stage_a_args(q, k_data, k_scales, block_table, seq_lens, H_q, H_kv, kp)
     _gpu(v_data, v_scales)
     _check(v_data.dtype == torch.uint8 and v_data.dim() == 3 and v_data.size(2) == vp, f"v_data last dim must be {vp}")

@@ -74,12 +74,20 @@ CASES = [
     ("k4v4", 1, 4, 2, 300, None, 64),                     # G=2
     ("k3v2", 1, 16, 1, 600, None, 64),                    # G=16
     ("k4v4", 1, 16, 1, 600, None, 64),
+    # the mixed pairs: the key side of one scheme with the value side of the other (group 128)
+    ("k3v4", 2, 8, 2, 512, None, 64), ("k4v2", 2, 8, 2, 512, None, 64),
+    ("k3v4", 3, 32, 4, 512, [17, 257, 512], 256), ("k4v2", 3, 32, 4, 512, [17, 257, 512], 256),
+    ("k3v4", 4, 8, 2, 32, [0, 1, 9, 17], 32), ("k4v2", 4, 8, 2, 32, [0, 1, 9, 17], 64),
+    ("k3v4", 1, 8, 2, 5000, [4987], 256), ("k4v2", 1, 8, 2, 5000, [4987], 512),
+    ("k3v4", 1, 4, 4, 300, None, 32), ("k4v2", 1, 4, 2, 300, None, 64),
+    ("k3v4", 1, 16, 1, 600, None, 64), ("k4v2", 1, 16, 1, 600, None, 64),
 ]
 
 
 @pytest.mark.parametrize("scheme,B,Hq,Hkv,S,lens,K", CASES)
 def test_fused_scan_matches_oracle(scheme, B, Hq, Hkv, S, lens, K):
-    kb, vb, gs = {"k3v2": (3, 2, 64), "k4v4": (4, 4, 128), "k3v2_g128": (3, 2, 128)}[scheme]
+    kb, vb, gs = {"k3v2": (3, 2, 64), "k4v4": (4, 4, 128), "k3v2_g128": (3, 2, 128), "k3v4": (3, 4, 128),
+                  "k4v2": (4, 2, 128)}[scheme]
     c = make_case(70 + S + Hq, B, Hq, Hkv, S, kb, vb, gs, lens=lens, extra_blocks=3)
     d = to_device(c)
     out = run_fused(scheme, c, d, S, K)
@@ -92,11 +100,12 @@ def test_fused_scan_matches_oracle(scheme, B, Hq, Hkv, S, lens, K):
     ("k4v4", 10000, [9000], 512, 768),     # two-stage, lists of top_k + 256 entries, empty tail splits
     ("k4v4", 10000, [10000], 1024, 1280),  # widest top-k: parts limited to 8192 / top_k
     ("k3v2", 3000, [3000], 64, 1024),      # longer than the planner would pick for this size
+    ("k3v4", 10000, [9989], 256, 512), ("k4v2", 10000, [9000], 512, 768),      # two-stage merges of the mixed pairs
 ])
 def test_fused_scan_with_forced_split_length(scheme, S, lens, K, split_len):
     from jetfire_amd import _lib
     lib = _lib.load()
-    kb, vb, gs = {"k3v2": (3, 2, 64), "k4v4": (4, 4, 128)}[scheme]
+    kb, vb, gs = {"k3v2": (3, 2, 64), "k4v4": (4, 4, 128), "k3v4": (3, 4, 128), "k4v2": (4, 2, 128)}[scheme]
     c = make_case(11 + S + K, 1, 8, 2, S, kb, vb, gs, lens=lens, extra_blocks=3)
     d = to_device(c)
     _lib.check(lib.jf_debug_split_len(split_len))
@@ -149,11 +158,12 @@ def test_fused_scan_is_deterministic_and_matches_split_path():
     ("k4v4", 2, 32, 8, 1024, None, 256),
     ("k3v2", 2, 32, 4, 768, [700, 768], 256),             # the TP2 70B local-head geometry
     ("k4v4", 4, 8, 2, 32, [0, 1, 9, 17], 64),
+    ("k3v4", 2, 32, 8, 1024, None, 256), ("k4v2", 2, 32, 4, 768, [700, 768], 256),
 ])
 def test_fused_decode_step_end_to_end(scheme, B, Hq, Hkv, S, lens, K):
     """scan+top-k -> pinned hand-off -> CPU correction -> merge, checked against the oracle's whole step and the
     acceptance bar for attention outputs (max-abs 2e-2, mean-abs 1e-3 in bf16)."""
-    kb, vb, gs = (3, 2, 64) if scheme == "k3v2" else (4, 4, 128)
+    kb, vb, gs = {"k3v2": (3, 2, 64), "k4v4": (4, 4, 128), "k3v4": (3, 4, 128), "k4v2": (4, 2, 128)}[scheme]
     c = make_case(80 + B + Hq, B, Hq, Hkv, S, kb, vb, gs, lens=lens)
     d = to_device(c)
     o = ops()
