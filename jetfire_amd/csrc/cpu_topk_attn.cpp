@@ -492,7 +492,27 @@ __global__ __launch_bounds__(1024) void handoff_wait_fetch_kernel(const int64_t*
                                                                   const float* __restrict__ o_hat,
                                                                   const float* __restrict__ o_old,
                                                                   const float* __restrict__ W, uint4* out) {
+  // Each lane owns up to U items per pass (item = eight bf16 elements).  What does not depend on the CPU -- the
+  // o_hat / o_old rows and W of the first pass -- is loaded before the wait, and the U reads from pinned host
+  // memory of a pass are issued together, so that one PCIe round trip covers them.
+  constexpr int U = 4;
   __shared__ int ok_sh;
+  float4 H[U][2], O[U][2];
+  float Wv[U];
+  auto load_gpu_side = [&](int base) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int i = base + (int)threadIdx.x + u * (int)blockDim.x;
+      if (out && i < n16) {
+        H[u][0] = reinterpret_cast<const float4*>(o_hat)[2 * i];
+        H[u][1] = reinterpret_cast<const float4*>(o_hat)[2 * i + 1];
+        O[u][0] = reinterpret_cast<const float4*>(o_old)[2 * i];
+        O[u][1] = reinterpret_cast<const float4*>(o_old)[2 * i + 1];
+        Wv[u] = W[i >> 4];  // 16 items per 128-element row
+      }
+    }
+  };
+  load_gpu_side(0);
   if (threadIdx.x == 0) {
     const int64_t want = *seq_dev;
     const uint64_t t0 = wall_clock64();
@@ -511,24 +531,32 @@ __global__ __launch_bounds__(1024) void handoff_wait_fetch_kernel(const int64_t*
   }
   __syncthreads();
   const bool ok = ok_sh != 0;
-  for (int i = threadIdx.x; i < n16; i += blockDim.x) {
-    const uint4 v = ok ? src[i] : make_uint4(0u, 0u, 0u, 0u);
-    if (dst) dst[i] = v;
-    if (out) {  // the blend of jf_blend_unnorm on the eight elements this lane has just fetched
-      const float w = W[i >> 4];  // 16 lanes per 128-element row
-      const float4 h0 = reinterpret_cast<const float4*>(o_hat)[2 * i], h1 = reinterpret_cast<const float4*>(o_hat)[2 * i + 1];
-      const float4 d0 = reinterpret_cast<const float4*>(o_old)[2 * i], d1 = reinterpret_cast<const float4*>(o_old)[2 * i + 1];
-      const uint32_t n[4] = {v.x, v.y, v.z, v.w};
-      const float hh[8] = {h0.x, h0.y, h0.z, h0.w, h1.x, h1.y, h1.z, h1.w};
-      const float dd[8] = {d0.x, d0.y, d0.z, d0.w, d1.x, d1.y, d1.z, d1.w};
-      uint32_t r[4];
+  for (int base = 0; base < n16; base += U * (int)blockDim.x) {
+    if (base > 0) load_gpu_side(base);
+    uint4 v[U];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const float lo = __builtin_fmaf(w, bf16_to_f32((uint16_t)(n[e] & 0xffffu)), hh[2 * e]) - dd[2 * e];
-        const float hi = __builtin_fmaf(w, bf16_to_f32((uint16_t)(n[e] >> 16)), hh[2 * e + 1]) - dd[2 * e + 1];
-        r[e] = (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+    for (int u = 0; u < U; ++u) {
+      const int i = base + (int)threadIdx.x + u * (int)blockDim.x;
+      v[u] = (ok && i < n16) ? src[i] : make_uint4(0u, 0u, 0u, 0u);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int i = base + (int)threadIdx.x + u * (int)blockDim.x;
+      if (i >= n16) continue;
+      if (dst) dst[i] = v[u];
+      if (out) {  // the blend of jf_blend_unnorm on the eight elements this lane has just fetched
+        const uint32_t n[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+        const float hh[8] = {H[u][0].x, H[u][0].y, H[u][0].z, H[u][0].w, H[u][1].x, H[u][1].y, H[u][1].z, H[u][1].w};
+        const float dd[8] = {O[u][0].x, O[u][0].y, O[u][0].z, O[u][0].w, O[u][1].x, O[u][1].y, O[u][1].z, O[u][1].w};
+        uint32_t r[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float lo = __builtin_fmaf(Wv[u], bf16_to_f32((uint16_t)(n[e] & 0xffffu)), hh[2 * e]) - dd[2 * e];
+          const float hi = __builtin_fmaf(Wv[u], bf16_to_f32((uint16_t)(n[e] >> 16)), hh[2 * e + 1]) - dd[2 * e + 1];
+          r[e] = (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+        }
+        out[i] = make_uint4(r[0], r[1], r[2], r[3]);
       }
-      out[i] = make_uint4(r[0], r[1], r[2], r[3]);
     }
   }
 }

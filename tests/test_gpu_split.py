@@ -487,6 +487,37 @@ def test_handoff_stream_mode_replays_from_a_hip_graph():
     h.close()
 
 
+def test_handoff_stream_wait_blend_more_rows_than_one_pass():
+    """288 rows: the wait + blend kernel (one workgroup, 4096 eight-element items per pass) takes a second pass."""
+    B, Hq, Hkv, K = 9, 32, 4, 32
+    o = ops()
+    rng = np.random.default_rng(5)
+    num_slots = 512
+    ksh = bf16_tensor(O.bf16_round(rng.standard_normal((Hkv, num_slots, 128)).astype(np.float32)))
+    vsh = bf16_tensor(O.bf16_round(rng.standard_normal((Hkv, num_slots, 128)).astype(np.float32)))
+    q = bf16_tensor(O.bf16_round((rng.standard_normal((B, Hq, 128)) / np.sqrt(128)).astype(np.float32))).cuda()
+    s = torch.from_numpy(rng.integers(0, num_slots, size=(B, Hq, K)).astype(np.int64)).cuda()
+    o.set_cpu_attn_threads(3)
+    o_hat = torch.randn(B, Hq, 128, device="cuda")
+    o_old = torch.randn(B, Hq, 128, device="cuda") * 0.1
+    W = torch.rand(B, Hq, device="cuda")
+    h = o.CpuTopkHandoff(B, Hq, Hkv, K, ksh, vsh, 0.1)
+    out = torch.zeros(B, Hq, 128, dtype=torch.bfloat16, device="cuda")
+    o_new = torch.zeros_like(out)
+    h.stream_submit(q, s)
+    h.stream_wait_blend(o_hat, o_old, W, out, o_new)
+    torch.cuda.synchronize()
+    h.check_status()
+    h.close()
+    want_new = torch.zeros(B, Hq, 128, dtype=torch.bfloat16)
+    o.cpu_topk_attn(q.cpu(), ksh, vsh, torch.from_numpy(O.head_map(B, Hq, Hq // Hkv, K)), s.cpu(), want_new, 0.1)
+    assert torch.equal(o_new.cpu().view(torch.int16), want_new.view(torch.int16))
+    want = torch.zeros_like(out)
+    o.blend_unnorm_into(o_hat, o_old, W, o_new, want)
+    torch.cuda.synchronize()
+    assert torch.equal(out.view(torch.int16), want.view(torch.int16))
+
+
 def test_handoff_stream_wait_is_bounded():
     """A correction that never finishes (the dispatcher is told to ignore the flag): the device-side wait runs
     into its limit, the kernel ends, o_new is zero, the status reports it, and later waits fall through."""
