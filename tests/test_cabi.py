@@ -140,8 +140,16 @@ def test_kernel_sets_mirror_the_reference_dispatch_protocol():
         k32.attn_with_scores()
     with pytest.raises(ValueError):
         k32.quant_write_k(None, None, None, None, object(), 64)
+    for k in (2, 3, 4):
+        for v in (2, 3, 4):
+            ks = get_kernel_set(f"SymInt{k}K_SymInt{v}V")
+            assert (ks.nbits_k, ks.nbits_v, ks.asymmetric_k) == (k, v, False)
+    a2 = get_kernel_set("AsymInt2K_SymInt3V")                       # historical alias of the 4-level scheme
+    assert a2 is get_kernel_set("AsymInt2K4Level_SymInt3V") and (a2.nbits_k, a2.nbits_v, a2.asymmetric_k) == (2, 3, True)
     with pytest.raises(ValueError):
-        get_kernel_set("AsymInt2K4Level_SymInt2V")
+        a2.quant_write_k(None, None, None, None, None, 64)          # zero-points are required
+    with pytest.raises(ValueError):
+        get_kernel_set("AsymInt3K_SymInt3V")                        # a placeholder in the reference too: no kernels
 
 
 @pytest.mark.parametrize("scheme,gs,B,Hq,Hkv,S,K", [
