@@ -1,0 +1,43 @@
+"""Seeded sweep of the fused scan over randomly drawn geometries (GQA group, batch, ragged lengths, correction
+width, forced split lengths, block-table permutations) for the four fused schemes, each case checked against
+the oracle exactly as the hand-picked cases are."""
+import numpy as np
+import pytest
+
+from tests.helpers import make_case, to_device
+from tests.test_gpu_fused import check_against_oracle, run_fused
+
+pytestmark = pytest.mark.gpu
+
+SCHEMES = {"k3v2": (3, 2, 64), "k3v2_g128": (3, 2, 128), "k4v4": (4, 4, 128), "k3v4": (3, 4, 128), "k4v2": (4, 2, 128)}
+
+
+def _draw(seed):
+    rng = np.random.default_rng(1000 + seed)
+    scheme = list(SCHEMES)[seed % len(SCHEMES)]
+    G = int(rng.choice([1, 2, 4, 8, 16]))
+    Hkv = int(rng.choice([1, 2, 4])) if G < 16 else 1
+    B = int(rng.integers(1, 4))
+    S = int(rng.choice([48, 200, 777, 1500, 2600, 4100]))
+    lens = [int(x) for x in rng.integers(0, S + 1, size=B)]
+    lens[int(rng.integers(0, B))] = S                       # at least one full-length row
+    K = int(rng.choice([32, 64, 128, 256, 512, 1024]))
+    split = int(rng.choice([0, 0, 256, 512, 1024]))
+    return scheme, B, G * Hkv, Hkv, S, lens, K, split
+
+
+@pytest.mark.parametrize("seed", range(64))
+def test_fused_scan_random_geometry(seed):
+    from jetfire_amd import _lib
+    scheme, B, Hq, Hkv, S, lens, K, split = _draw(seed)
+    kb, vb, gs = SCHEMES[scheme]
+    c = make_case(500 + seed, B, Hq, Hkv, S, kb, vb, gs, lens=lens, extra_blocks=int(seed % 4))
+    d = to_device(c)
+    lib = _lib.load()
+    print(f"case: {scheme} B={B} Hq={Hq} Hkv={Hkv} S={S} lens={lens} K={K} split={split}", flush=True)
+    _lib.check(lib.jf_debug_split_len(split))
+    try:
+        out = [t.clone() for t in run_fused(scheme, c, d, S, K)]
+    finally:
+        _lib.check(lib.jf_debug_split_len(0))
+    check_against_oracle(scheme, c, S, K, out)
