@@ -16,7 +16,7 @@ def _run(w, lay, **kw):
                                w.seq_lens, w.S, w.H_q, w.H_kv, 16, w.top_k, w.attn_scale, **kw)
 
 
-@pytest.mark.parametrize("name", ["c2", "c3", "c4"])
+@pytest.mark.parametrize("name", ["c1", "c2", "c3", "c4", "c5"])
 def test_full_size_layer_properties(name):
     from jetfire_amd import workloads
     w = workloads.build(name, n_layers=1, paged=True)
