@@ -70,3 +70,32 @@ def test_full_size_layer_properties(name):
             torch.testing.assert_close(o_old[b, h * G:(h + 1) * G], old, atol=4e-6, rtol=1e-4)
             del khat, vhat, vq, vexact
     assert max_sc > 0
+
+
+def test_c1_gpu_split_path_agrees_with_the_cpu_torch_path():
+    """C1 is the configuration the reference itself runs on a CPU (unpack -> einsum -> topk in torch, fp32 q times
+    bf16-rounded keys).  The split-form INT4 kernels with the same scoring model (int4_qk_scores, exact top-k,
+    int4_softmax_v) against the torch restatement of that CPU path on the full C1 shape: the same winners
+    wherever the margin exceeds accumulation noise, and the same attention output up to the bf16 rounding the
+    CPU path applies to the dequantised values."""
+    from jetfire_amd import ops, workloads
+    w = workloads.build("c1", n_layers=1, paged=False)
+    lay = w.layers[0]
+    S, K, Hq, Hkv = w.S, w.top_k, w.H_q, w.H_kv
+    scores, idx, slots, m, iz = ops.int4_qk_scores_topk_stats(w.q, lay.k_data, lay.k_scales, w.block_table, w.seq_lens, S,
+                                                             Hq, Hkv, 16, w.attn_scale, K)
+    o_hat, o_old, W = ops.int4_softmax_v_with_pre_corr_wvs2_scores(scores, lay.v_data, lay.v_scales, w.block_table,
+                                                                   w.seq_lens, idx, S, Hq, Hkv, 16, K)
+    def cpu(t):                                       # the sequence occupies slots [0, S) of the identity block table
+        t = t[:, :S].cpu()
+        return (t.unsqueeze(-1) if t.dim() == 2 else t).unsqueeze(0)
+    ref_o, ref_idx = T.decode_path(w.q.cpu(), cpu(lay.k_data), cpu(lay.k_scales), cpu(lay.v_data), cpu(lay.v_scales),
+                                   w.group, 4, 4, K)
+    sc = scores[0].cpu()
+    for h in range(Hq):
+        cut = sc[h].topk(K).values[-1]
+        clear = {int(i) for i in ref_idx[0, h].tolist() if sc[h, int(i)] > cut + 1e-4}
+        assert clear <= set(idx[0, h].cpu().tolist())
+        assert len(clear) >= K - 4                                        # almost every winner is clear of the cut
+    torch.testing.assert_close(o_hat.cpu(), ref_o.float(), atol=2e-3, rtol=2e-2)
+    assert float((o_hat.cpu() - ref_o.float()).abs().mean()) < 2e-4
