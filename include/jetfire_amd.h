@@ -183,6 +183,26 @@ int jf_fused_scan_topk(int scheme, int group_size,
                        float* softmax_m, float* softmax_inv_z, float* scores,
                        void* workspace, size_t workspace_bytes, void* stream);
 
+/* jf_fused_scan_topk without the workspace arguments, for callers that cannot allocate device memory (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in
+ * the reference.  The workspace is a fixed array of JF_FUSED_STATIC_SCRATCH_BYTES in device memory that each
+ * GPU the library runs on holds until the process ends; its address is looked up once per device on the first
+ * call there (make that call outside a capture).  The call itself allocates and frees nothing.  Shapes whose
+ * jf_fused_workspace_bytes() exceeds the array are rejected with JF_ERR_ARG.  Every call on a GPU shares that
+ * GPU's array, so calls that overlap on one GPU (two streams, two threads) race; calls ordered on one stream
+ * are safe, and nothing in the array has to be cleared between calls (every call rewrites what it reads).
+ * Same kernels, same results as jf_fused_scan_topk. */
+#define JF_FUSED_STATIC_SCRATCH_BYTES (64u << 20)
+int jf_fused_scan_topk_static(int scheme, int group_size,
+                              const uint16_t* q, const uint8_t* k_data, const uint16_t* k_scales,
+                              const uint8_t* v_data, const uint16_t* v_scales,
+                              const int64_t* block_table, const int32_t* seq_lens,
+                              int B, int H_q, int H_kv, int max_S, int max_blocks, int64_t num_slots,
+                              int block_size, float attn_scale, int top_k,
+                              int64_t* topk_idx, int64_t* topk_slots,
+                              float* o_hat, float* o_old_unnorm, float* W,
+                              float* softmax_m, float* softmax_inv_z, float* scores, void* stream);
+
 /* Introspection with no counterpart in the reference: the launch geometry jf_fused_scan_topk uses for a
  * shape.  split_len positions per scan workgroup, n_splits = ceil(max_S / split_len) workgroups per
  * (sequence, kv-head), list_cap candidate slots per (row, split), merge_parts > 1 if the candidate lists are

@@ -30,6 +30,7 @@
 // pre-correction terms o_old_unnorm, W over the winners (jetfire_vllm/csrc/int2_softmax_v.cu:738-788).
 #include "common.h"
 
+#include <mutex>
 #include <vector>
 
 namespace jf {
@@ -1960,13 +1961,14 @@ extern "C" int jf_fused_plan(int scheme, int group_size, int B, int H_q, int H_k
   return JF_OK;
 }
 
-extern "C" int jf_fused_scan_topk(int scheme, int group_size, const uint16_t* q, const uint8_t* k_data,
-                                  const uint16_t* k_scales, const uint8_t* v_data, const uint16_t* v_scales,
-                                  const int64_t* block_table, const int32_t* seq_lens, int B, int H_q, int H_kv,
-                                  int max_S, int max_blocks, int64_t num_slots, int block_size, float attn_scale,
-                                  int top_k, int64_t* topk_idx, int64_t* topk_slots, float* o_hat,
-                                  float* o_old_unnorm, float* W, float* softmax_m, float* softmax_inv_z, float* scores,
-                                  void* workspace, size_t workspace_bytes, void* stream) {
+// The whole fused step (scan, merge) on caller-provided workspace memory; both public entry points end here.
+static int fused_scan_run(int scheme, int group_size, const uint16_t* q, const uint8_t* k_data,
+                          const uint16_t* k_scales, const uint8_t* v_data, const uint16_t* v_scales,
+                          const int64_t* block_table, const int32_t* seq_lens, int B, int H_q, int H_kv,
+                          int max_S, int max_blocks, int64_t num_slots, int block_size, float attn_scale,
+                          int top_k, int64_t* topk_idx, int64_t* topk_slots, float* o_hat,
+                          float* o_old_unnorm, float* W, float* softmax_m, float* softmax_inv_z, float* scores,
+                          void* workspace, size_t workspace_bytes, void* stream) {
   JF_CHECK_ARG(known_scheme(scheme), "fused_scan: unknown scheme %d", scheme);
   JF_CHECK_ARG(B >= 0 && H_q > 0 && H_kv > 0 && max_S >= 0 && H_q % H_kv == 0, "fused_scan: bad shape");
   const int G = H_q / H_kv;
@@ -2082,6 +2084,66 @@ extern "C" int jf_fused_scan_topk(int scheme, int group_size, const uint16_t* q,
 #undef JF_MERGE
   JF_CHECK_LAUNCH();
   return JF_OK;
+}
+
+extern "C" int jf_fused_scan_topk(int scheme, int group_size, const uint16_t* q, const uint8_t* k_data,
+                                  const uint16_t* k_scales, const uint8_t* v_data, const uint16_t* v_scales,
+                                  const int64_t* block_table, const int32_t* seq_lens, int B, int H_q, int H_kv,
+                                  int max_S, int max_blocks, int64_t num_slots, int block_size, float attn_scale,
+                                  int top_k, int64_t* topk_idx, int64_t* topk_slots, float* o_hat,
+                                  float* o_old_unnorm, float* W, float* softmax_m, float* softmax_inv_z, float* scores,
+                                  void* workspace, size_t workspace_bytes, void* stream) {
+  return fused_scan_run(scheme, group_size, q, k_data, k_scales, v_data, v_scales, block_table, seq_lens, B, H_q, H_kv,
+                        max_S, max_blocks, num_slots, block_size, attn_scale, top_k, topk_idx, topk_slots, o_hat,
+                        o_old_unnorm, W, softmax_m, softmax_inv_z, scores, workspace, workspace_bytes, stream);
+}
+
+// ---------------------------------------------------------------------------------------------------
+// The same step for callers that may not allocate: the workspace is a fixed array in device memory that every
+// GPU the library runs on holds until the process ends.  `scratch` names the array for the device code
+// object only; host code never passes that name anywhere: it asks the runtime once per device for the array's
+// address on that device and uses the returned pointer from then on.
+static __device__ __align__(256) unsigned char scratch[JF_FUSED_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[kMaxDevices] = {};  // address of `scratch` on each device, resolved on first use
+}  // namespace
+
+extern "C" int jf_fused_scan_topk_static(int scheme, int group_size, const uint16_t* q, const uint8_t* k_data,
+                                         const uint16_t* k_scales, const uint8_t* v_data, const uint16_t* v_scales,
+                                         const int64_t* block_table, const int32_t* seq_lens, int B, int H_q,
+                                         int H_kv, int max_S, int max_blocks, int64_t num_slots, int block_size,
+                                         float attn_scale, int top_k, int64_t* topk_idx, int64_t* topk_slots,
+                                         float* o_hat, float* o_old_unnorm, float* W, float* softmax_m,
+                                         float* softmax_inv_z, float* scores, void* stream) {
+  JF_CHECK_ARG(known_scheme(scheme), "fused_scan_static: unknown scheme %d", scheme);
+  JF_CHECK_ARG(B >= 0 && H_q > 0 && H_kv > 0 && max_S >= 0 && H_q % H_kv == 0 && top_k > 0,
+               "fused_scan_static: bad shape");
+  const size_t need = jf_fused_workspace_bytes(scheme, B, H_q, H_kv, max_S, top_k);
+  JF_CHECK_ARG(need <= (size_t)JF_FUSED_STATIC_SCRATCH_BYTES,
+               "fused_scan_static: this shape needs %zu bytes of workspace, the built-in scratch holds %zu; use "
+               "jf_fused_scan_topk with a caller-provided workspace",
+               need, (size_t)JF_FUSED_STATIC_SCRATCH_BYTES);
+  int dev = -1;
+  JF_CHECK_HIP(hipGetDevice(&dev));
+  JF_CHECK_ARG(dev >= 0 && dev < kMaxDevices, "fused_scan_static: device ordinal %d out of range", dev);
+  void* ws = nullptr;
+  {
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (g_scratch_ptr[dev] == nullptr) {  // once per device, with that device current
+      void* ptr = nullptr;
+      JF_CHECK_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+      JF_CHECK_ARG(ptr != nullptr, "fused_scan_static: the runtime returned no address for the scratch array");
+      g_scratch_ptr[dev] = ptr;
+    }
+    ws = g_scratch_ptr[dev];
+  }
+  return fused_scan_run(scheme, group_size, q, k_data, k_scales, v_data, v_scales, block_table, seq_lens, B, H_q, H_kv,
+                        max_S, max_blocks, num_slots, block_size, attn_scale, top_k, topk_idx, topk_slots, o_hat,
+                        o_old_unnorm, W, softmax_m, softmax_inv_z, scores, ws, (size_t)JF_FUSED_STATIC_SCRATCH_BYTES,
+                        stream);
 }
 
 extern "C" int jf_profile_scan_begin(int max_launches) {
