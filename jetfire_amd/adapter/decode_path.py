@@ -14,8 +14,11 @@ the graph (`:698-706`).  The reference's trace hooks, release policy and debug c
 reproduced."""
 from __future__ import annotations
 
+import bisect
 import math
 import os
+import re
+import weakref
 
 import torch
 
@@ -29,26 +32,28 @@ SPLIT_SUPPORTED_TOP_K = ops.SUPPORTED_TOP_K
 
 _TOPK_CLAMP_LOGGED: set = set()
 _HEAD_MAP_CACHE: dict = {}
-_HANDOFFS: dict = {}
+_STORES_WITH_HANDOFFS: "weakref.WeakSet" = weakref.WeakSet()   # stores that carry hand-off contexts (`store._jf_handoffs`)
 _O_NEW: dict = {}
 _SEQ_LENS_CACHE: dict = {}
 
 
 def _select_top_k(config_top_k: int, seq_len: int, supported: tuple) -> int | None:
-    """Largest supported width <= the configured one that the context can fill; a context shorter than the
-    smallest width still runs with that width (unused lanes are padded with -1).  None for an empty sequence
-    or when no supported width is <= the configured one."""
-    requested, length = int(config_top_k), int(seq_len)
-    configured = [k for k in supported if 0 < k <= requested]
-    if not configured or length <= 0:
+    """Correction width for a step (contract of `decode_path.py:1156-1182`, table in
+    `tests/test_runtime_edge_cases.py:13-35`): the widest supported width that neither exceeds the configured
+    one nor the context length; a context shorter than every admissible width runs with the narrowest of them
+    (the kernels pad unused lanes with -1).  None for an empty context or when no width is admissible."""
+    want, have = int(config_top_k), int(seq_len)
+    widths = sorted(w for w in supported if 0 < w <= want)
+    if have <= 0 or not widths:
         return None
-    candidates = [k for k in configured if k <= length]
-    selected = max(candidates) if candidates else min(configured)
-    if selected != requested and (requested, selected) not in _TOPK_CLAMP_LOGGED:
-        _TOPK_CLAMP_LOGGED.add((requested, selected))
-        print(f"[jetfire] requested top_k={requested} clamped to kernel-supported top_k={selected}; "
+    fit = bisect.bisect_right(widths, have)          # widths[:fit] can be filled by the context
+    chosen = widths[fit - 1] if fit else widths[0]
+    note = (want, chosen, tuple(supported))
+    if chosen != want and note not in _TOPK_CLAMP_LOGGED:
+        _TOPK_CLAMP_LOGGED.add(note)
+        print(f"[jetfire] requested top_k={want} clamped to kernel-supported top_k={chosen}; "
               f"supported={tuple(supported)}.", flush=True)
-    return selected
+    return chosen
 
 
 def _get_head_map_cpu(B: int, H_q: int, num_groups: int, K: int) -> torch.Tensor:
@@ -70,66 +75,65 @@ def _graph_capture_active() -> bool:
 
 
 def _graph_context_batch_sizes(max_batch_size: int) -> list[int]:
-    """Batch sizes whose hand-off contexts must exist before capture: all of 1..max, or the sizes listed in
-    `JETFIRE_GRAPH_CAPTURE_SIZES` plus the maximum (`decode_path.py:668-695`)."""
-    if max_batch_size <= 0:
+    """Batch sizes that need a hand-off context before a capture (`decode_path.py:668-695`): every size up to
+    the maximum, unless `JETFIRE_GRAPH_CAPTURE_SIZES` lists the captured sizes (comma or semicolon separated;
+    sizes outside 1..max are ignored, the maximum is always included)."""
+    top = int(max_batch_size)
+    if top <= 0:
         return []
-    raw = os.environ.get("JETFIRE_GRAPH_CAPTURE_SIZES", "").strip()
-    if not raw:
-        return list(range(1, max_batch_size + 1))
-    out = {max_batch_size}
-    for part in raw.replace(";", ",").split(","):
-        part = part.strip()
-        if not part:
-            continue
-        try:
-            value = int(part)
-        except ValueError:
-            raise RuntimeError("JETFIRE_GRAPH_CAPTURE_SIZES must be a comma-separated list of integers; "
-                               f"got {raw!r}") from None
-        if 1 <= value <= max_batch_size:
-            out.add(value)
-    return sorted(out)
+    spec = os.environ.get("JETFIRE_GRAPH_CAPTURE_SIZES", "").strip()
+    if not spec:
+        return list(range(1, top + 1))
+    fields = [f for f in (piece.strip() for piece in re.split(r"[;,]", spec)) if f]
+    if any(re.fullmatch(r"[+-]?\d+", f) is None for f in fields):
+        raise RuntimeError(f"JETFIRE_GRAPH_CAPTURE_SIZES must be a comma-separated list of integers; got {spec!r}")
+    return sorted({top} | {n for n in map(int, fields) if 1 <= n <= top})
 
 
 def _raise_graph_decode_miss(reason: str, *, layer_name: str) -> None:
-    raise RuntimeError("JetFire graph decode miss would fall back to native attention and poison the captured "
-                       f"graph. reason={reason} layer={layer_name}. Pre-create JetFire stores and graph submit "
-                       "contexts before the decode step is captured, or disable JETFIRE_DECODE_GRAPH.")
+    """A miss during capture would record the caller's native attention into the graph: refuse instead
+    (`decode_path.py:698-706`).  `reason=` and `layer=` are what callers parse."""
+    raise RuntimeError(f"JetFire decode cannot miss while a HIP graph is being captured (the fall-back would be "
+                       f"recorded into the graph): reason={reason} layer={layer_name}. Create the layer stores and "
+                       f"call warmup_graph_decode_submit_contexts() before the capture, or unset JETFIRE_DECODE_GRAPH.")
 
 
 def _decode_unsupported(*, impl, layer, query, attn_metadata) -> str | None:
-    """Dispatcher gate: the reason string of a miss, or None."""
+    """Dispatcher gate (`decode_path.py:1667-1695`): the reference's reason string of the first failing
+    precondition, or None.  The preconditions are evaluated lazily, in the reference's order."""
     pool = get_global_kv_pool_manager()
-    if not pool.config.enabled:
-        return "pool_disabled"
-    if query.is_cuda and torch.cuda.is_current_stream_capturing() and not _graph_mode_enabled():
-        return "cuda_graph_capture"          # the host-blocking hand-off cannot be captured
-    if attn_metadata is None:
-        return "profiling_run"
-    attn_type = getattr(impl, "attn_type", None)
-    if attn_type is not None and getattr(attn_type, "name", str(attn_type)) != "DECODER":
-        return "attn_type"
-    if getattr(attn_metadata, "use_cascade", False):
-        return "cascade"
-    if int(getattr(attn_metadata, "max_query_len", 1)) != 1:
-        return "prefill_or_multi_query"
-    n_seqs = int(attn_metadata.seq_lens.numel())
-    if int(getattr(attn_metadata, "num_actual_tokens", n_seqs)) != n_seqs:
-        return "batch_mismatch"
-    if int(query.shape[0]) < n_seqs:
-        return "empty_query"
-    layer_name = getattr(layer, "layer_name", None)
-    if layer_name is None:
-        return "layer_name_missing"
-    layer_cfg = pool.get_layer_config(layer_name)
-    if layer_cfg is None:
-        return "layer_config_missing"
-    if int(query.shape[-1]) != layer_cfg.head_dim:
-        return "head_dim_mismatch"
-    if layer_cfg.head_dim % pool.config.group_size != 0:
-        return "group_size_mismatch"
-    return None
+    md = attn_metadata
+    state: dict = {}
+
+    def attn_type_name():
+        kind = getattr(impl, "attn_type", None)
+        return "DECODER" if kind is None else getattr(kind, "name", str(kind))
+
+    def n_seqs():
+        return int(md.seq_lens.numel())
+
+    def layer_cfg():
+        if "cfg" not in state:
+            state["cfg"] = pool.get_layer_config(getattr(layer, "layer_name", None))
+        return state["cfg"]
+
+    gate = (
+        ("pool_disabled", lambda: not pool.config.enabled),
+        # the host-blocking hand-off cannot be captured; graph mode uses the kernel-only pair
+        ("cuda_graph_capture", lambda: query.is_cuda and torch.cuda.is_current_stream_capturing()
+                                       and not _graph_mode_enabled()),
+        ("profiling_run", lambda: md is None),
+        ("attn_type", lambda: attn_type_name() != "DECODER"),
+        ("cascade", lambda: bool(getattr(md, "use_cascade", False))),
+        ("prefill_or_multi_query", lambda: int(getattr(md, "max_query_len", 1)) != 1),
+        ("batch_mismatch", lambda: int(getattr(md, "num_actual_tokens", n_seqs())) != n_seqs()),
+        ("empty_query", lambda: int(query.shape[0]) < n_seqs()),
+        ("layer_name_missing", lambda: getattr(layer, "layer_name", None) is None),
+        ("layer_config_missing", lambda: layer_cfg() is None),
+        ("head_dim_mismatch", lambda: int(query.shape[-1]) != layer_cfg().head_dim),
+        ("group_size_mismatch", lambda: layer_cfg().head_dim % pool.config.group_size != 0),
+    )
+    return next((reason for reason, fails in gate if fails()), None)
 
 
 def _seq_lens_on_host(seq_lens: torch.Tensor) -> torch.Tensor:
@@ -146,9 +150,12 @@ def _seq_lens_on_host(seq_lens: torch.Tensor) -> torch.Tensor:
 
 def _handoff_for(store, B: int, H_q: int, H_kv: int, K: int, scale: float, *, stream_mode: bool = False,
                  layer_name: str = "unknown_layer"):
-    # a context serves one of the two modes
-    key = (id(store), B, H_q, K, float(scale), bool(stream_mode))
-    h = _HANDOFFS.get(key)
+    """Hand-off context of (store, shape, mode).  The contexts live ON the store object, so a store that goes
+    away takes its contexts (pinned buffers, dispatcher thread, the pointers into its shadow) with it and a new
+    store can never be served a context that reads another store's shadow."""
+    cache = store.__dict__.setdefault("_jf_handoffs", {})
+    key = (B, H_q, K, float(scale), bool(stream_mode))      # a context serves one of the two modes
+    h = cache.get(key)
     if h is None:
         if _graph_capture_active():        # pinned allocations and thread start-up are not capturable
             _raise_graph_decode_miss("submit_context_missing", layer_name=layer_name)
@@ -156,8 +163,23 @@ def _handoff_for(store, B: int, H_q: int, H_kv: int, K: int, scale: float, *, st
         if threads > 0:
             ops.set_cpu_attn_threads(threads)
         h = ops.CpuTopkHandoff(B, H_q, H_kv, K, store.k_shadow, store.v_shadow, scale)
-        _HANDOFFS[key] = h
+        cache[key] = h
+        _STORES_WITH_HANDOFFS.add(store)
     return h
+
+
+def _all_handoffs():
+    return [h for store in list(_STORES_WITH_HANDOFFS) for h in store.__dict__.get("_jf_handoffs", {}).values()]
+
+
+def check_decode_handoffs() -> None:
+    """Raise if any hand-off context has failed: a CPU correction job that failed or timed out, or a
+    device-side wait that ran into its limit (from then on a graph replay blends zeros instead of the
+    correction, without any host call that could notice).  One load of a pinned status word per context, no
+    synchronisation: call it after the step's synchronise.  The decode entry, `flush_pending_writes` of the pool
+    and `reset_jetfire_decode_runtime_state` call it too."""
+    for h in _all_handoffs():
+        h.check_status()
 
 
 def _o_new_for(n_seqs: int, H_q: int, D: int, device) -> torch.Tensor:
@@ -199,18 +221,22 @@ def warmup_graph_decode_submit_contexts(*, max_batch_size: int, device=None, sca
         for n in sizes:
             _o_new_for(n, layer_cfg.num_query_heads, layer_cfg.head_dim, device if device is not None else store.device)
             for k in widths:
-                before = len(_HANDOFFS)
+                before = len(store.__dict__.get("_jf_handoffs", {}))
                 _handoff_for(store, n, layer_cfg.num_query_heads, layer_cfg.num_kv_heads, k, sc, stream_mode=True,
                              layer_name=name)
-                created += len(_HANDOFFS) - before
+                created += len(store._jf_handoffs) - before
     return {"layers": len(pool.layer_stores), "batch_sizes": sizes, "top_k": list(widths), "contexts_created": created}
 
 
-def reset_jetfire_decode_runtime_state() -> None:
-    """Close the cached hand-off contexts and scratch tensors (call before the stores they point at go away)."""
-    for h in _HANDOFFS.values():
-        h.close()
-    _HANDOFFS.clear()
+def reset_jetfire_decode_runtime_state(*, check: bool = False) -> None:
+    """Close every hand-off context and drop the scratch tensors (the pool manager calls this before it lets
+    go of its stores).  `check=True` first raises if a context has failed."""
+    if check:
+        check_decode_handoffs()
+    for store in list(_STORES_WITH_HANDOFFS):
+        for h in store.__dict__.pop("_jf_handoffs", {}).values():
+            h.close()
+    _STORES_WITH_HANDOFFS.clear()
     _O_NEW.clear()
     _HEAD_MAP_CACHE.clear()
     _SEQ_LENS_CACHE.clear()
@@ -270,6 +296,8 @@ def _decode_batched(*, impl, layer, query, attn_metadata, output):
     if store.block_size != 16 or layer_cfg.head_dim != 128 or not store.shadow_enabled or store.k_scales.shape[-1] > 2:
         return miss("scheme_unsupported")
     store.flush_pending_writes()
+    for h in store.__dict__.get("_jf_handoffs", {}).values():
+        h.check_status()                    # a failed context must not go on blending zeros silently
 
     n_seqs = int(attn_metadata.seq_lens.numel())
     H_q, H_kv, D = layer_cfg.num_query_heads, layer_cfg.num_kv_heads, layer_cfg.head_dim

@@ -134,6 +134,8 @@ class JetFireKVPoolManager:
     def flush_pending_writes(self) -> None:
         for store in self.layer_stores.values():
             store.flush_pending_writes()
+            for h in store.__dict__.get("_jf_handoffs", {}).values():
+                h.check_status()          # raises if a correction failed or a device-side wait hit its limit
 
     # ------------------------------------------------------------------ statistics
     def record_decode_attempt(self) -> None:
@@ -158,6 +160,8 @@ class JetFireKVPoolManager:
         }
 
     def reset_runtime_state(self, *, preserve_layouts: bool = True) -> None:
+        from .decode_path import reset_jetfire_decode_runtime_state
+        reset_jetfire_decode_runtime_state()      # the hand-off contexts point into the stores that go away now
         self.token_counters.clear()
         self.layer_stores.clear()
         if not preserve_layouts:
@@ -191,4 +195,6 @@ def get_global_kv_pool_manager() -> JetFireKVPoolManager:
 def reset_global_kv_pool_manager() -> None:
     """Drop the global manager (and its stores); the next `get_global_kv_pool_manager` reads the configuration again."""
     global _GLOBAL_MANAGER
+    from .decode_path import reset_jetfire_decode_runtime_state
+    reset_jetfire_decode_runtime_state()
     _GLOBAL_MANAGER = None

@@ -66,6 +66,68 @@ def test_dispatcher_gate_reasons(adapter):
     assert pool.get_stats()["decode_fallbacks"] == {"store_missing": 1} and pool.decode_attempts == 1
 
 
+def test_graph_capture_batch_sizes_and_miss_message(adapter, monkeypatch):
+    """`decode_path.py:668-706`: all sizes by default, the listed ones plus the maximum otherwise; a malformed
+    list and a miss during capture raise with the fields callers parse."""
+    from jetfire_amd.adapter.decode_path import _graph_context_batch_sizes, _raise_graph_decode_miss
+    monkeypatch.delenv("JETFIRE_GRAPH_CAPTURE_SIZES", raising=False)
+    assert _graph_context_batch_sizes(0) == [] and _graph_context_batch_sizes(-3) == []
+    assert _graph_context_batch_sizes(4) == [1, 2, 3, 4]
+    monkeypatch.setenv("JETFIRE_GRAPH_CAPTURE_SIZES", " 8; 2,2 ,, 64, 0 ,-1")
+    assert _graph_context_batch_sizes(16) == [2, 8, 16]
+    monkeypatch.setenv("JETFIRE_GRAPH_CAPTURE_SIZES", "1,two")
+    with pytest.raises(RuntimeError, match="comma-separated list of integers"):
+        _graph_context_batch_sizes(4)
+    with pytest.raises(RuntimeError, match=r"reason=store_missing layer=model\.layers\.3"):
+        _raise_graph_decode_miss("store_missing", layer_name="model.layers.3")
+
+
+def test_handoff_contexts_belong_to_their_store(adapter, monkeypatch):
+    """The cached hand-off contexts live on the store object: resetting the pool closes them, and a new store
+    (even one that reuses the old one's id) gets contexts that read ITS shadow."""
+    from jetfire_amd.adapter import decode_path
+    made, closed = [], []
+
+    class FakeHandoff:
+        def __init__(self, B, H_q, H_kv, K, k_shadow, v_shadow, scale):
+            self.k_ptr = k_shadow.data_ptr()
+            self.failed = False
+            made.append(self)
+
+        def check_status(self):
+            if self.failed:
+                raise RuntimeError("handoff: the device-side wait for the CPU correction ran into its limit")
+
+        def close(self):
+            closed.append(self)
+
+    monkeypatch.setattr(decode_path.ops, "CpuTopkHandoff", FakeHandoff)
+    pool = adapter.get_global_kv_pool_manager()
+    name = "model.layers.0.attn"
+    pool.register_layer_config(name, num_query_heads=8, num_kv_heads=2, head_dim=128)
+    pool.register_layer_layout(name, num_blocks=4, block_size=16)
+    store = pool.ensure_layer_store(name, device="cpu")
+    h1 = decode_path._handoff_for(store, 2, 8, 2, 32, 0.1, stream_mode=True)
+    assert decode_path._handoff_for(store, 2, 8, 2, 32, 0.1, stream_mode=True) is h1
+    assert decode_path._handoff_for(store, 2, 8, 2, 32, 0.1, stream_mode=False) is not h1
+    assert h1.k_ptr == store.k_shadow.data_ptr() and len(made) == 2
+    decode_path.check_decode_handoffs()
+    h1.failed = True
+    with pytest.raises(RuntimeError, match="ran into its limit"):
+        decode_path.check_decode_handoffs()
+    with pytest.raises(RuntimeError, match="ran into its limit"):
+        pool.flush_pending_writes()
+    h1.failed = False
+    pool.reset_runtime_state()                       # drops the stores: their contexts are closed first
+    assert len(closed) == 2 and not pool.layer_stores
+    del store
+    new_store = pool.ensure_layer_store(name, device="cpu")
+    h2 = decode_path._handoff_for(new_store, 2, 8, 2, 32, 0.1, stream_mode=True)
+    assert h2 is not h1 and h2.k_ptr == new_store.k_shadow.data_ptr()
+    adapter.reset_global_kv_pool_manager()
+    assert len(closed) == 3
+
+
 def test_pool_registry_and_store_geometry(adapter):
     adapter.set_jetfire_config(scheme="SymInt4K_SymInt4V", group_size=128, layer_stride=2)
     adapter.reset_global_kv_pool_manager()
@@ -426,3 +488,51 @@ def test_graph_mode_decode_step_replays_against_the_oracle(adapter, monkeypatch)
             err = np.abs(res - r["out"])
             assert err.max() <= 2e-2 and err.mean() <= 1e-3
     del graph
+
+
+@pytest.mark.gpu
+def test_graph_mode_reports_a_correction_that_never_arrives(adapter, monkeypatch):
+    """Graph mode makes no host call per step, so a device-side wait that runs into its limit (here: the
+    dispatcher is told to ignore the flag, limit 20 ms; every kernel ends normally) would blend zeros from then
+    on without anyone noticing: `check_decode_handoffs`, the pool's flush and the next decode call all raise."""
+    from jetfire_amd.adapter import decode_path
+    monkeypatch.setenv("JETFIRE_DECODE_GRAPH", "1")
+    B, Hq, Hkv, D, bs, K, max_S = 1, 8, 2, 128, 16, 32, 64
+    adapter.set_jetfire_config(scheme="SymInt3K_SymInt2V", group_size=64, topk=K, layer_stride=1, cpu_attn_threads=2,
+                               max_batch_size=B)
+    adapter.reset_global_kv_pool_manager()
+    pool = adapter.get_global_kv_pool_manager()
+    name = "model.layers.0.self_attn.attn"
+    layer = types.SimpleNamespace(layer_name=name, num_heads=Hq, num_kv_heads=Hkv, head_size=D)
+    impl = types.SimpleNamespace(attn_type=types.SimpleNamespace(name="DECODER"), scale=D ** -0.5)
+    pool.ensure_layer_config_from_layer(name, layer)
+    pool.register_layer_layout(name, num_blocks=max_S // bs, block_size=bs)
+    g = torch.Generator().manual_seed(5)
+    n = 40
+    k = torch.randn(n, Hkv, D, generator=g).to(torch.bfloat16).cuda()
+    v = torch.randn(n, Hkv, D, generator=g).to(torch.bfloat16).cuda()
+    pool.mirror_kv(name, k, v, torch.arange(n, dtype=torch.int64, device="cuda"))
+    pool.flush_pending_writes()
+    adapter.warmup_graph_decode_submit_contexts(max_batch_size=B)
+    store = pool.get_layer_store(name)
+    (h,) = store._jf_handoffs.values()
+    meta = _meta(torch.tensor([n], dtype=torch.int32, device="cuda"),
+                 torch.arange(max_S // bs, dtype=torch.int64, device="cuda").view(1, -1), max_seq_len=max_S)
+    q = (torch.randn(B, Hq, D, generator=g) / D ** 0.5).to(torch.bfloat16).cuda()
+    out = torch.zeros(B, Hq * D, dtype=torch.bfloat16, device="cuda")
+    assert adapter.try_jetfire_decode(impl=impl, layer=layer, query=q, attn_metadata=meta, output=out) is out
+    torch.cuda.synchronize()
+    decode_path.check_decode_handoffs()                       # a healthy step: nothing to report
+    good = out.clone()
+    h.debug_pause(True)
+    h.set_device_wait_limit_us(20000)
+    assert adapter.try_jetfire_decode(impl=impl, layer=layer, query=q, attn_metadata=meta, output=out) is out
+    torch.cuda.synchronize()
+    assert not torch.equal(out, good)                         # the correction is missing from this step's output
+    with pytest.raises(RuntimeError, match="limit"):
+        decode_path.check_decode_handoffs()
+    with pytest.raises(RuntimeError, match="limit"):
+        pool.flush_pending_writes()
+    with pytest.raises(RuntimeError, match="limit"):
+        adapter.try_jetfire_decode(impl=impl, layer=layer, query=q, attn_metadata=meta, output=out)
+    h.debug_pause(False)
