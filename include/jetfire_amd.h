@@ -231,6 +231,11 @@ int jf_debug_split_len(int split_len);
 int jf_blend_unnorm(const float* o_hat, const float* o_old_unnorm, const float* W,
                     const uint16_t* o_new, uint16_t* out, int B, int H_q, int D, void* stream);
 
+/* out = bf16_rne(fma(W, f32(o_new) - o_old, o_hat)) with a NORMALISED o_old: replaces blend / blend_into
+ * (jetfire_vllm/csrc/blend.cu:44-66, 68-190). */
+int jf_blend(const float* o_hat, const float* o_old, const float* W,
+             const uint16_t* o_new, uint16_t* out, int B, int H_q, int D, void* stream);
+
 /* ------------------------------------------------------------------ piece 4: CPU correction + hand-off
  * Exact softmax attention over the top-k slots from the host bf16 shadow.  Replaces cpu_topk_attn
  * (jetfire_vllm/csrc/cpu_topk_attn.cpp:854-956; row kernel :602-690): invalid slots (<0 or
@@ -294,6 +299,53 @@ int jf_handoff_set_device_wait_limit_us(jf_handoff* h, int64_t us);
 /* Test aid: while on, the dispatcher ignores published flags (a correction that never finishes, without
  * hanging anything: the device-side wait runs into its limit). */
 int jf_handoff_debug_pause(jf_handoff* h, int on);
+
+/* Row implementation of the CPU correction: 0 scalar (cpu_topk_attn.cpp:602-690), 1 AVX2+FMA, 2 AVX-512-BF16
+ * (vdpbf16ps row, jetfire_vllm/csrc/cpu_topk_attn.cpp:316-479).  The widest one the host supports is used unless
+ * JETFIRE_CPU_ATTN_ISA (scalar | avx2 | avx512bf16) or jf_set_cpu_attn_isa asks for a narrower one (-1: widest).
+ * An output row that comes out non-finite is recomputed by the scalar row and zeroed if it still is; the count
+ * of such rows is get_cpu_topk_sanitize_count (cpu_topk_attn.cpp:809-826, 2643). */
+int jf_set_cpu_attn_isa(int isa);
+int jf_get_cpu_attn_isa(void);
+int64_t jf_cpu_topk_sanitize_count(void);
+
+/* The reference's own submit-context interface (jetfire_vllm/csrc/cpu_topk_attn.cpp:2054-2163
+ * create_cpu_topk_submit_ctx, :2239 stream_submit_cpu_topk_attn, :2302 stream_wait_cpu_topk_attn): the caller owns
+ * pinned host buffers q (B, H_q, 128) bf16, head_map / ts_buf (B, H_q, K) int64 and o_new (B, H_q, 128) bf16 and
+ * fills q / ts_buf with its own stream-ordered copies (jetfire_vllm/adapter/decode_path.py:2243-2267); a context
+ * remembers the pointers.  stream_submit enqueues a one-lane kernel that raises the context's sequence flag in
+ * pinned memory, in stream order behind those copies; the shared poller thread then runs the correction into
+ * o_new and stores 1 to flag_host (nullable).  stream_wait enqueues the bounded device-side wait of
+ * jf_handoff_stream_wait (without a copy: the caller's own H2D copy of o_new follows it).  Both are kernels only
+ * and can be captured into a HIP graph.  Handles are positive integers, 0 on error; they stay valid until
+ * jf_clear_graph_contexts.  jf_submit_ctx_status: as jf_handoff_status. */
+int64_t jf_submit_ctx_create(const uint16_t* q_host, const uint16_t* k_shadow_host, const uint16_t* v_shadow_host,
+                             const int64_t* head_map_host, const int64_t* ts_buf_host, uint16_t* o_new_host,
+                             int B, int H_q, int K, int H_kv, int64_t num_slots, float scale, int64_t* flag_host);
+int jf_submit_ctx_stream_submit(int64_t ctx, void* stream);
+int jf_submit_ctx_stream_wait(int64_t ctx, void* stream);
+int jf_submit_ctx_status(int64_t ctx);
+/* stream_write_value64 / stream_wait_value64 (jetfire_vllm/csrc/cpu_topk_attn.cpp:1293-1344) as one-lane kernels:
+ * store `value` to a device-visible word with system scope / poll it until it equals `value`.  The wait is bounded
+ * by min(JETFIRE_CPU_FUTURE_TIMEOUT_S, 10 s); jf_stream_wait_timeouts counts waits that ran into the bound. */
+int jf_stream_write_value64(void* stream, int64_t* flag_device, int64_t value);
+int jf_stream_wait_value64(void* stream, const int64_t* flag_device, int64_t value);
+int64_t jf_stream_wait_timeouts(void);
+/* submit_cpu_topk_attn_async / wait_for_flag (jetfire_vllm/csrc/cpu_topk_attn.cpp:1184-1260): jf_cpu_topk_attn on an
+ * executor thread, returns at once; 1 is stored to `flag` when o_new is complete.  wait_for_flag spins, then sleeps in
+ * short steps, until the flag is non-zero (timeout_s <= 0: forever). */
+int jf_cpu_topk_attn_async(const uint16_t* q, const uint16_t* k_shadow, const uint16_t* v_shadow,
+                           const int64_t* head_map, const int64_t* ts_buf, uint16_t* o_new,
+                           int B, int H_q, int K, int H_kv, int64_t num_slots, float scale, int64_t* flag);
+int jf_wait_for_flag(const int64_t* flag, double timeout_s);
+/* graph_pool_warmup[_threads], get_graph_submit_count, reset_graph_runtime_state, clear_graph_contexts
+ * (jetfire_vllm/csrc/cpu_topk_attn.cpp:2620-2660): start (n_threads > 0: resize) the worker pool; number of
+ * stream-mode submits the poller has served; reset the counters; destroy every submit context (only when no
+ * graph that holds their kernels will be replayed again). */
+int jf_graph_pool_warmup(int n_threads);
+int64_t jf_graph_submit_count(void);
+int jf_reset_graph_runtime_state(void);
+int jf_clear_graph_contexts(void);
 
 #ifdef __cplusplus
 }

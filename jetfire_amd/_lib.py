@@ -55,6 +55,23 @@ SIGNATURES = {
     "jf_handoff_set_device_wait_limit_us": (I, [P, L]),
     "jf_handoff_debug_pause": (I, [P, I]),
     "jf_handoff_destroy": (None, [P]),
+    "jf_blend": (I, [P, P, P, P, P, I, I, I, P]),
+    "jf_set_cpu_attn_isa": (I, [I]),
+    "jf_get_cpu_attn_isa": (I, []),
+    "jf_cpu_topk_sanitize_count": (L, []),
+    "jf_submit_ctx_create": (L, [P, P, P, P, P, P, I, I, I, I, L, F, P]),
+    "jf_submit_ctx_stream_submit": (I, [L, P]),
+    "jf_submit_ctx_stream_wait": (I, [L, P]),
+    "jf_submit_ctx_status": (I, [L]),
+    "jf_stream_write_value64": (I, [P, P, L]),
+    "jf_stream_wait_value64": (I, [P, P, L]),
+    "jf_stream_wait_timeouts": (L, []),
+    "jf_cpu_topk_attn_async": (I, [P, P, P, P, P, P, I, I, I, I, L, F, P]),
+    "jf_wait_for_flag": (I, [P, C.c_double]),
+    "jf_graph_pool_warmup": (I, [I]),
+    "jf_graph_submit_count": (L, []),
+    "jf_reset_graph_runtime_state": (I, []),
+    "jf_clear_graph_contexts": (I, []),
 }
 
 _lib = None

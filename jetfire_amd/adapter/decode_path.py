@@ -18,6 +18,7 @@ import bisect
 import math
 import os
 import re
+import struct
 import weakref
 
 import torch
@@ -154,7 +155,9 @@ def _handoff_for(store, B: int, H_q: int, H_kv: int, K: int, scale: float, *, st
     away takes its contexts (pinned buffers, dispatcher thread, the pointers into its shadow) with it and a new
     store can never be served a context that reads another store's shadow."""
     cache = store.__dict__.setdefault("_jf_handoffs", {})
-    key = (B, H_q, K, float(scale), bool(stream_mode))      # a context serves one of the two modes
+    # a context serves one of the two modes; the scale is keyed as the fp32 value the kernels receive, so that
+    # 1 / sqrt(d) and d ** -0.5 (one ulp apart in double precision) name the same context
+    key = (B, H_q, K, struct.unpack("f", struct.pack("f", float(scale)))[0], bool(stream_mode))
     h = cache.get(key)
     if h is None:
         if _graph_capture_active():        # pinned allocations and thread start-up are not capturable
@@ -190,11 +193,14 @@ def _o_new_for(n_seqs: int, H_q: int, D: int, device) -> torch.Tensor:
     return o_new
 
 
-def warmup_graph_decode_submit_contexts(*, max_batch_size: int, device=None, scale: float | None = None) -> dict:
+def warmup_graph_decode_submit_contexts(*, max_batch_size: int, device=None, scale: float | None = None,
+                                        max_seq_len: int | None = None) -> dict:
     """Create, before a decode step is captured, the graph-mode hand-off contexts (pinned buffers, poller
     registration happens on first submit) of every mirrored layer for every captured batch size and every
     correction width up to the configured one, the `o_new` buffers, and the stores' append state
-    (`decode_path.py:851-1015`).  `scale` is the attention scale the layers use (default head_dim ** -0.5)."""
+    (`decode_path.py:851-1015`).  `scale` is the attention scale the layers use (default head_dim ** -0.5); with
+    `max_seq_len` the fused scan's workspace is sized for the longest context too (call this on the stream the
+    capture will use)."""
     if max_batch_size <= 0:
         raise RuntimeError("JETFIRE_DECODE_GRAPH=1 requires JETFIRE_MAX_BATCH_SIZE>0 so decode host buffers and "
                            "submit contexts have stable pointers before graph capture.")
@@ -217,6 +223,10 @@ def warmup_graph_decode_submit_contexts(*, max_batch_size: int, device=None, sca
             raise RuntimeError(f"JETFIRE_TOPK={cfg.topk} is not supported by the active kernel set.")
         widths = tuple(k for k in supported if k <= top_k) or (top_k,)
         store.warmup_graph_append(int(max_batch_size))
+        if max_seq_len and store.scheme is not None and store.device.type == "cuda":
+            # the scan's workspace of this stream, sized for the largest step, so that no capture has to grow it
+            ops.reserve_fused_workspace(store.scheme, int(max_batch_size), layer_cfg.num_query_heads,
+                                        layer_cfg.num_kv_heads, int(max_seq_len), top_k, store.device)
         sc = float(scale) if scale is not None else 1.0 / math.sqrt(layer_cfg.head_dim)
         for n in sizes:
             _o_new_for(n, layer_cfg.num_query_heads, layer_cfg.head_dim, device if device is not None else store.device)

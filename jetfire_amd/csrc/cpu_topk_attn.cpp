@@ -1,7 +1,10 @@
 // Host side of the hand-off: exact softmax attention over the top-k slots from the bf16 shadow
-// (restates the contract of jetfire_vllm/csrc/cpu_topk_attn.cpp:602-690,854-956), a persistent
-// worker pool (spin, then sleep on a condition variable), and the stream-ordered pinned hand-off
-// (submit: D2H q + slots -> host function starts the CPU job; wait: host function joins -> H2D o_new).
+// (restates the contract of jetfire_vllm/csrc/cpu_topk_attn.cpp:602-690,854-956; AVX2+FMA and AVX-512-BF16 rows
+// selected at run time, :316-479), a persistent worker pool (spin, then sleep on a condition variable), and the
+// pinned hand-off: a small kernel stores q and the winners' slots into pinned host memory and raises a flag
+// there, a host thread that polls the flag runs the correction, and the result comes back either after a
+// host-blocking wait or through a kernel that waits on the device (graph-capturable).  No hipMemcpyAsync and
+// no stream callbacks anywhere.
 #include <hip/hip_runtime.h>
 
 #include <atomic>
@@ -75,7 +78,8 @@ class Pool {
     cv_work_.notify_all();
     return true;
   }
-  // Wait for the job started with start().  timeout_s <= 0: wait forever.
+  // Wait for the job started with start().  timeout_s <= 0: wait forever.  On a timeout the job is withdrawn
+  // (no further rows can be claimed, rows in flight are waited for) and the pool is free again.
   bool join(double timeout_s) {
     const auto t0 = std::chrono::steady_clock::now();
     for (int spin = 0; spin < 20000; ++spin) {
@@ -88,7 +92,18 @@ class Pool {
     while (done_rows_.load(std::memory_order_acquire) < n_) {
       if (timeout_s > 0) {
         const double el = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
-        if (el > timeout_s) return false;
+        if (el > timeout_s) {
+          // withdraw: a counter value of a later epoch stops every claim; then let the rows in flight drain
+          const uint64_t e = epoch_.load(std::memory_order_relaxed) + 1;
+          next_.store(e << 32, std::memory_order_release);
+          epoch_.store(e, std::memory_order_release);
+          jobs_[e & 1].n = 0;
+          lk.unlock();
+          while (active_.load(std::memory_order_acquire) != 0) std::this_thread::sleep_for(std::chrono::microseconds(50));
+          lk.lock();
+          busy_ = false;
+          return false;
+        }
       }
       cv_done_.wait_for(lk, std::chrono::milliseconds(1));
     }
@@ -129,6 +144,8 @@ class Pool {
     return (int)(hc < 64 ? hc : 64);
   }
   void ensure_workers() {
+    // one resize at a time: a second submitter must not join the same thread objects
+    std::lock_guard<std::mutex> rg(resize_mu_);
     int want;
     {
       std::lock_guard<std::mutex> g(cfg_mu_);
@@ -149,10 +166,19 @@ class Pool {
     const uint64_t e0 = epoch_.load(std::memory_order_acquire);
     for (int i = 0; i < want; ++i) workers_.emplace_back([this, e0] { worker(e0); });
   }
+  static double spin_seconds() {
+    // how long an idle worker spins for the next job before it sleeps: the gap between two layers of a decode
+    // step (and between two steps of a running decode loop) is shorter than a futex wake-up of the whole pool,
+    // which costs the first job after it several hundred microseconds (JETFIRE_POOL_SPIN_US, default 2000)
+    static const double s = [] {
+      const char* e = std::getenv("JETFIRE_POOL_SPIN_US");
+      const double us = e ? std::atof(e) : 2000.0;
+      return (us >= 0.0 && us <= 1e6 ? us : 2000.0) * 1e-6;
+    }();
+    return s;
+  }
   void worker(uint64_t seen) {
     for (;;) {
-      // spin for the next epoch for about half a millisecond (the gap between two layers of a decode step is
-      // shorter than a futex wake-up of the whole pool), then sleep
       bool got = false;
       const auto t0 = std::chrono::steady_clock::now();
       for (uint32_t spin = 0;; ++spin) {
@@ -161,7 +187,7 @@ class Pool {
         _mm_pause();
 #endif
         if ((spin & 0x3ff) == 0x3ff &&
-            std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() > 500e-6) break;
+            std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() > spin_seconds()) break;
       }
       if (!got) {
         std::unique_lock<std::mutex> lk(mu_);
@@ -181,7 +207,9 @@ class Pool {
         if (b >= n) break;
         if (!next_.compare_exchange_weak(v, v + (uint64_t)chunk, std::memory_order_acq_rel, std::memory_order_acquire)) continue;
         const int64_t end = std::min<int64_t>(n, b + chunk);
+        active_.fetch_add(1, std::memory_order_acq_rel);
         jb.fn(b, end);
+        active_.fetch_sub(1, std::memory_order_acq_rel);
         if (done_rows_.fetch_add(end - b, std::memory_order_acq_rel) + (end - b) >= n) {
           std::lock_guard<std::mutex> g(mu_);
           cv_done_.notify_all();
@@ -195,7 +223,8 @@ class Pool {
     return __atomic_load_n(&stop_, __ATOMIC_ACQUIRE);
   }
 
-  std::mutex mu_, cfg_mu_;
+  std::mutex mu_, cfg_mu_, resize_mu_;
+  std::atomic<int> active_{0};          // workers inside a job function
   std::condition_variable cv_work_, cv_done_;
   std::vector<std::thread> workers_;
   Job jobs_[2];
@@ -346,9 +375,121 @@ static bool host_has_avx2_fma() {
   static const bool ok = __builtin_cpu_supports("avx2") && __builtin_cpu_supports("fma");
   return ok;
 }
+
+// AVX-512-BF16 form (jetfire_vllm/csrc/cpu_topk_attn.cpp:316-479): the K dot products run on vdpbf16ps, which
+// multiplies the bf16 operands directly (four instructions per 128-channel row, pairs of products summed in
+// fp32); V is accumulated in eight 16-lane fp32 registers and converted with vcvtneps2bf16.  Rows are
+// requested 32 slots ahead like the AVX2 form (the gather is DRAM-latency bound on this host; the reference's
+// packing of the V rows into a contiguous buffer trades that latency for a second pass over 256 bytes per slot).
+#define JF_AVX512BF16_TARGET __attribute__((target("avx512f,avx512bw,avx512vl,avx512dq,avx512bf16")))
+template <typename SlotT>
+JF_AVX512BF16_TARGET static void topk_attn_row_avx512bf16(const uint16_t* q, const uint16_t* k_shadow,
+                                                          const uint16_t* v_shadow, int64_t num_slots,
+                                                          const int64_t* head_map, int64_t fixed_h,
+                                                          const SlotT* slots, int K, int H_kv, float scale,
+                                                          uint16_t* out, float* score_buf) {
+  constexpr int AHEAD = 32;
+  __m512bh qv[4];
+  for (int i = 0; i < 4; ++i) qv[i] = (__m512bh)_mm512_loadu_si512(reinterpret_cast<const void*>(q + 32 * i));
+  auto row_of = [&](const uint16_t* base, int k) -> const uint16_t* {
+    const int64_t s = slots[k], h = head_map ? head_map[k] : fixed_h;
+    if (s < 0 || s >= num_slots || h < 0 || h >= H_kv) return nullptr;
+    return base + ((size_t)h * num_slots + s) * D;
+  };
+  auto prefetch_row = [](const uint16_t* r) {
+    if (r) {
+      for (int b = 0; b < D * 2; b += 64) _mm_prefetch(reinterpret_cast<const char*>(r) + b, _MM_HINT_T0);
+    }
+  };
+  for (int k = 0; k < K && k < AHEAD; ++k) prefetch_row(row_of(k_shadow, k));
+  float mx = -INFINITY;
+  bool any = false;
+  for (int k = 0; k < K; ++k) {
+    if (k + AHEAD < K) prefetch_row(row_of(k_shadow, k + AHEAD));
+    const uint16_t* kr = row_of(k_shadow, k);
+    if (!kr) {
+      score_buf[k] = -INFINITY;
+      continue;
+    }
+    any = true;
+    __m512 acc = _mm512_setzero_ps();
+    for (int i = 0; i < 4; ++i)
+      acc = _mm512_dpbf16_ps(acc, qv[i], (__m512bh)_mm512_loadu_si512(reinterpret_cast<const void*>(kr + 32 * i)));
+    const float sc = _mm512_reduce_add_ps(acc) * scale;
+    score_buf[k] = sc;
+    if (sc > mx) mx = sc;
+  }
+  if (!any) {
+    memset(out, 0, D * sizeof(uint16_t));
+    return;
+  }
+  for (int k = 0; k < K && k < AHEAD; ++k) prefetch_row(row_of(v_shadow, k));
+  float den = 0.0f;
+  for (int k = 0; k < K; ++k) {
+    score_buf[k] = std::exp(score_buf[k] - mx);
+    den += score_buf[k];
+  }
+  if (!(den > 0.0f) || !std::isfinite(den)) {
+    memset(out, 0, D * sizeof(uint16_t));
+    return;
+  }
+  const float inv = 1.0f / den;
+  __m512 o[D / 16];
+  for (int i = 0; i < D / 16; ++i) o[i] = _mm512_setzero_ps();
+  for (int k = 0; k < K; ++k) {
+    if (k + AHEAD < K) prefetch_row(row_of(v_shadow, k + AHEAD));
+    const uint16_t* vr = row_of(v_shadow, k);
+    if (!vr) continue;
+    const __m512 w = _mm512_set1_ps(score_buf[k] * inv);
+    for (int i = 0; i < D / 16; ++i) {
+      const __m512i u = _mm512_slli_epi32(_mm512_cvtepu16_epi32(_mm256_loadu_si256(reinterpret_cast<const __m256i*>(vr + 16 * i))), 16);
+      o[i] = _mm512_fmadd_ps(w, _mm512_castsi512_ps(u), o[i]);
+    }
+  }
+  for (int i = 0; i < D / 16; ++i)
+    _mm256_storeu_si256(reinterpret_cast<__m256i*>(out + 16 * i), (__m256i)_mm512_cvtneps_pbh(o[i]));
+}
+static bool host_has_avx512bf16() {
+  static const bool ok = __builtin_cpu_supports("avx512f") && __builtin_cpu_supports("avx512bw") &&
+                        __builtin_cpu_supports("avx512vl") && __builtin_cpu_supports("avx512dq") &&
+                        __builtin_cpu_supports("avx512bf16");
+  return ok;
+}
 #else
 static bool host_has_avx2_fma() { return false; }
+static bool host_has_avx512bf16() { return false; }
 #endif
+
+// Row implementation in use: 0 scalar, 1 AVX2+FMA, 2 AVX-512-BF16.  The widest the host supports, unless
+// JETFIRE_CPU_ATTN_ISA (scalar | avx2 | avx512bf16) or jf_set_cpu_attn_isa asks for a narrower one.
+static std::atomic<int> g_isa_override{-1};
+static int resolve_isa() {
+  int best = host_has_avx512bf16() ? 2 : (host_has_avx2_fma() ? 1 : 0);
+  int want = g_isa_override.load(std::memory_order_relaxed);
+  if (want < 0) {
+    static const int env = [] {
+      const char* e = std::getenv("JETFIRE_CPU_ATTN_ISA");
+      if (!e) return -1;
+      if (!strcmp(e, "scalar")) return 0;
+      if (!strcmp(e, "avx2")) return 1;
+      if (!strcmp(e, "avx512bf16")) return 2;
+      return -1;
+    }();
+    want = env;
+  }
+  if (want >= 0 && want < best) best = want;
+  return best;
+}
+
+// Rows whose output came out non-finite (jetfire_vllm/csrc/cpu_topk_attn.cpp:809-826, 839-846): a vector row
+// is recomputed by the scalar row, and a row that is still non-finite is zeroed, so that one bad correction
+// cannot poison the layers after it.  The counter is what get_cpu_topk_sanitize_count reports.
+static std::atomic<int64_t> g_sanitize_count{0};
+static inline bool bf16_row_has_nonfinite(const uint16_t* r) {
+  for (int i = 0; i < D; ++i)
+    if ((r[i] & 0x7f80u) == 0x7f80u) return true;
+  return false;
+}
 
 struct CpuJob {
   const uint16_t *q, *k_shadow, *v_shadow;
@@ -363,17 +504,24 @@ struct CpuJob {
 template <typename SlotT>
 static void run_rows_t(const CpuJob& j, const SlotT* ts, int64_t b, int64_t e, float* buf) {
   const int G = j.H_q / j.H_kv;
+  const int isa = resolve_isa();
+  for (int64_t r = b; r < e; ++r) {
+    const uint16_t* q = j.q + r * D;
+    const int64_t* hm = j.head_map ? j.head_map + r * j.K : nullptr;
+    const int64_t fixed_h = (r % j.H_q) / G;
+    uint16_t* out = j.o_new + r * D;
 #if defined(__x86_64__)
-  if (host_has_avx2_fma()) {
-    for (int64_t r = b; r < e; ++r)
-      topk_attn_row_avx2<SlotT>(j.q + r * D, j.k_shadow, j.v_shadow, j.num_slots, j.head_map ? j.head_map + r * j.K : nullptr,
-                                (r % j.H_q) / G, ts + r * j.K, j.K, j.H_kv, j.scale, j.o_new + r * D, buf);
-    return;
-  }
+    if (isa == 2) topk_attn_row_avx512bf16<SlotT>(q, j.k_shadow, j.v_shadow, j.num_slots, hm, fixed_h, ts + r * j.K, j.K, j.H_kv, j.scale, out, buf);
+    else if (isa == 1) topk_attn_row_avx2<SlotT>(q, j.k_shadow, j.v_shadow, j.num_slots, hm, fixed_h, ts + r * j.K, j.K, j.H_kv, j.scale, out, buf);
+    else
 #endif
-  for (int64_t r = b; r < e; ++r)
-    topk_attn_row<SlotT>(j.q + r * D, j.k_shadow, j.v_shadow, j.num_slots, j.head_map ? j.head_map + r * j.K : nullptr,
-                         (r % j.H_q) / G, ts + r * j.K, j.K, j.H_kv, j.scale, j.o_new + r * D, buf);
+      topk_attn_row<SlotT>(q, j.k_shadow, j.v_shadow, j.num_slots, hm, fixed_h, ts + r * j.K, j.K, j.H_kv, j.scale, out, buf);
+    if (bf16_row_has_nonfinite(out)) {
+      g_sanitize_count.fetch_add(1, std::memory_order_acq_rel);
+      if (isa != 0) topk_attn_row<SlotT>(q, j.k_shadow, j.v_shadow, j.num_slots, hm, fixed_h, ts + r * j.K, j.K, j.H_kv, j.scale, out, buf);
+      if (isa == 0 || bf16_row_has_nonfinite(out)) memset(out, 0, D * sizeof(uint16_t));
+    }
+  }
 }
 
 static void run_rows(const CpuJob& j, int64_t b, int64_t e) {
@@ -395,6 +543,14 @@ extern "C" int jf_set_cpu_attn_threads(int n) {
   return JF_OK;
 }
 extern "C" int jf_get_cpu_attn_threads(void) { return Pool::instance().threads(); }
+
+extern "C" int jf_set_cpu_attn_isa(int isa) {
+  JF_CHECK_ARG(isa >= -1 && isa <= 2, "set_cpu_attn_isa: isa must be -1 (widest), 0 (scalar), 1 (avx2) or 2 (avx512bf16)");
+  g_isa_override.store(isa);
+  return JF_OK;
+}
+extern "C" int jf_get_cpu_attn_isa(void) { return resolve_isa(); }
+extern "C" int64_t jf_cpu_topk_sanitize_count(void) { return g_sanitize_count.load(); }
 
 extern "C" int jf_cpu_topk_attn(const uint16_t* q, const uint16_t* k_shadow, const uint16_t* v_shadow,
                                 const int64_t* head_map, const int64_t* ts_buf, uint16_t* o_new, int B, int H_q, int K,
@@ -444,6 +600,13 @@ struct jf_handoff {
   std::condition_variable cv;
   std::thread dispatcher;
   double timeout_s = 30.0;         // JETFIRE_CPU_FUTURE_TIMEOUT_S in the reference (decode_path.py:3082-3098)
+  // submit contexts over the caller's own pinned buffers (jf_submit_ctx_create): nothing is copied by a kernel,
+  // the correction reads q / head_map / slots from and writes o_new to these, then raises ext_flag
+  const uint16_t* ext_q = nullptr;
+  const int64_t* ext_head_map = nullptr;
+  const int64_t* ext_ts = nullptr;
+  uint16_t* ext_o = nullptr;
+  int64_t* ext_flag = nullptr;
 };
 
 namespace {
@@ -567,11 +730,47 @@ inline void cpu_relax() {
 #endif
 }
 
+std::atomic<int64_t> g_graph_submits{0};   // stream-mode submits served by the poller (get_graph_submit_count)
+
 bool run_correction(jf_handoff* h) {
+  if (h->ext_q) {  // the caller's buffers, its head map and 64-bit slots
+    CpuJob j{h->ext_q, h->k_shadow, h->v_shadow, h->ext_head_map, h->ext_ts, h->ext_o,
+             h->B, h->H_q, h->K, h->H_kv, h->num_slots, h->scale};
+    const bool ok = Pool::instance().run((int64_t)h->B * h->H_q, [j](int64_t b, int64_t e) { run_rows(j, b, e); });
+    std::atomic_thread_fence(std::memory_order_release);
+    if (h->ext_flag) __atomic_store_n(h->ext_flag, (int64_t)1, __ATOMIC_RELEASE);
+    return ok;
+  }
   // kv-head of a row = query head / (H_q / H_kv) (decode_path.py:400-408): no head map is read
   CpuJob j{h->q_pin, h->k_shadow, h->v_shadow, nullptr, nullptr, h->o_pin,
            h->B, h->H_q, h->K, h->H_kv, h->num_slots, h->scale, h->ts_pin};
   return Pool::instance().run((int64_t)h->B * h->H_q, [j](int64_t b, int64_t e) { run_rows(j, b, e); });
+}
+
+// Raises the sequence flag of a context whose buffers the caller fills itself (stream-ordered behind its copies).
+__global__ void handoff_signal_kernel(int64_t* flag, int64_t* seq_dev) {
+  const int64_t seq = *seq_dev + 1;
+  *seq_dev = seq;
+  __threadfence_system();
+  __hip_atomic_store(flag, seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+// Stream value operations as kernels (the reference uses cuStreamWriteValue64 / cuStreamWaitValue64,
+// jetfire_vllm/csrc/cpu_topk_attn.cpp:1293-1344): one lane writes, or polls until the word equals `value` or the
+// limit has passed (then *timeouts is incremented: every kernel ends).
+__global__ void stream_write_value64_kernel(int64_t* p, int64_t value) {
+  __threadfence_system();
+  __hip_atomic_store(p, value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+__global__ void stream_wait_value64_kernel(const int64_t* p, int64_t value, uint64_t limit_ticks, int64_t* timeouts) {
+  const uint64_t t0 = wall_clock64();
+  while (__hip_atomic_load(p, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM) != value) {
+    if (wall_clock64() - t0 > limit_ticks) {
+      __hip_atomic_fetch_add(timeouts, (int64_t)1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      break;
+    }
+    __builtin_amdgcn_s_sleep(16);
+  }
 }
 
 // Host mode: the context's own thread, asleep unless a submit is outstanding.
@@ -663,6 +862,7 @@ struct StreamPoller {
             __atomic_store_n(h->flag_pin + 16, (int64_t)2, __ATOMIC_RELEASE);
           }
           h->submits.fetch_add(1, std::memory_order_relaxed);
+          g_graph_submits.fetch_add(1, std::memory_order_relaxed);
           __atomic_store_n(h->flag_pin + 8, f, __ATOMIC_RELEASE);  // what the device-side wait polls
           served = true;
         }
@@ -674,7 +874,9 @@ struct StreamPoller {
       cpu_relax();
       if ((walk & 0x3ff) == 0x3ff) {
         const double el = std::chrono::duration<double>(std::chrono::steady_clock::now() - idle_since).count();
-        if (el > 0.002) std::this_thread::sleep_for(std::chrono::microseconds(el > 1.0 ? 200 : 50));
+        // a decode loop raises a flag every few hundred microseconds; only a GPU that has been silent for a while
+        // (no step in flight) is worth sleeping on: a sleep costs the next submit its wake-up latency
+        if (el > 0.05) std::this_thread::sleep_for(std::chrono::microseconds(el > 1.0 ? 200 : 50));
       }
     }
   }
@@ -863,4 +1065,207 @@ extern "C" void jf_handoff_destroy(jf_handoff* h) {
   if (h->flag_pin) (void)hipHostFree(h->flag_pin);
   if (h->counter_dev) (void)hipFree(h->counter_dev);
   delete h;
+}
+
+// ------------------------------------------------------------------ submit contexts, the reference's way
+// create_cpu_topk_submit_ctx / stream_submit_cpu_topk_attn / stream_wait_cpu_topk_attn
+// (jetfire_vllm/csrc/cpu_topk_attn.cpp:2054-2163, 2239, 2302): the caller owns the pinned q / slots / o_new
+// buffers and fills them with its own stream-ordered copies; a context only remembers the pointers.  Contexts
+// are integer handles that live until clear_graph_contexts.
+namespace {
+std::mutex g_ctx_mu;
+std::vector<jf_handoff*> g_ctxs;             // handle = index + 1
+int64_t* g_wait_timeouts = nullptr;          // pinned counter of stream_wait_value64 waits that hit their limit
+
+jf_handoff* ctx_of(int64_t handle) {
+  std::lock_guard<std::mutex> g(g_ctx_mu);
+  if (handle <= 0 || handle > (int64_t)g_ctxs.size()) return nullptr;
+  return g_ctxs[(size_t)handle - 1];
+}
+double future_timeout_s() {
+  double t = 30.0;
+  if (const char* e = std::getenv("JETFIRE_CPU_FUTURE_TIMEOUT_S")) {
+    const double v = std::atof(e);
+    if (v > 0) t = v;
+  }
+  return t;
+}
+
+// submit_cpu_topk_attn_async (cpu_topk_attn.cpp:1184-1205): one executor thread takes the jobs in order
+struct AsyncExecutor {
+  std::mutex mu;
+  std::condition_variable cv;
+  std::vector<std::pair<CpuJob, int64_t*>> queue;
+  bool started = false;
+  static AsyncExecutor& instance() {
+    static AsyncExecutor* e = new AsyncExecutor();
+    return *e;
+  }
+  void submit(const CpuJob& j, int64_t* flag) {
+    {
+      std::lock_guard<std::mutex> g(mu);
+      if (!started) {
+        started = true;
+        std::thread([this] { loop(); }).detach();
+      }
+      queue.emplace_back(j, flag);
+    }
+    cv.notify_one();
+  }
+  void loop() {
+    for (;;) {
+      std::pair<CpuJob, int64_t*> item;
+      {
+        std::unique_lock<std::mutex> lk(mu);
+        cv.wait(lk, [&] { return !queue.empty(); });
+        item = queue.front();
+        queue.erase(queue.begin());
+      }
+      const CpuJob j = item.first;
+      Pool::instance().run((int64_t)j.B * j.H_q, [j](int64_t b, int64_t e) { run_rows(j, b, e); });
+      std::atomic_thread_fence(std::memory_order_release);
+      __atomic_store_n(item.second, (int64_t)1, __ATOMIC_RELEASE);
+    }
+  }
+};
+}  // namespace
+
+extern "C" int64_t jf_submit_ctx_create(const uint16_t* q_host, const uint16_t* k_shadow_host, const uint16_t* v_shadow_host,
+                                        const int64_t* head_map_host, const int64_t* ts_buf_host, uint16_t* o_new_host,
+                                        int B, int H_q, int K, int H_kv, int64_t num_slots, float scale,
+                                        int64_t* flag_host) {
+  if (!q_host || !k_shadow_host || !v_shadow_host || !head_map_host || !ts_buf_host || !o_new_host || B <= 0 || H_q <= 0 ||
+      K <= 0 || H_kv <= 0 || num_slots <= 0) {
+    set_error("submit_ctx_create: bad arguments");
+    return 0;
+  }
+  jf_handoff* h = new jf_handoff();
+  h->B = B; h->H_q = H_q; h->H_kv = H_kv; h->K = K; h->num_slots = num_slots;
+  h->k_shadow = k_shadow_host; h->v_shadow = v_shadow_host; h->scale = scale;
+  h->ext_q = q_host; h->ext_head_map = head_map_host; h->ext_ts = ts_buf_host; h->ext_o = o_new_host; h->ext_flag = flag_host;
+  h->timeout_s = future_timeout_s();
+  if (hipHostMalloc((void**)&h->flag_pin, 256, hipHostMallocDefault) != hipSuccess ||
+      hipMalloc((void**)&h->counter_dev, 64) != hipSuccess || hipMemset(h->counter_dev, 0, 64) != hipSuccess) {
+    set_error("submit_ctx_create: allocation failed");
+    jf_handoff_destroy(h);
+    return 0;
+  }
+  h->flag_pin[0] = h->flag_pin[8] = h->flag_pin[16] = 0;
+  h->device_wait_ticks = (uint64_t)((h->timeout_s < 10.0 ? h->timeout_s : 10.0) * 1e8);
+  h->mode.store(2);
+  std::lock_guard<std::mutex> g(g_ctx_mu);
+  g_ctxs.push_back(h);
+  return (int64_t)g_ctxs.size();
+}
+
+extern "C" int jf_submit_ctx_stream_submit(int64_t ctx, void* stream) {
+  jf_handoff* h = ctx_of(ctx);
+  if (!h || !h->ext_q) { set_error("stream_submit_cpu_topk_attn: unknown context handle %lld", (long long)ctx); return JF_ERR_STATE; }
+  if (h->failed.load() || __atomic_load_n(h->flag_pin + 16, __ATOMIC_ACQUIRE) != 0) {
+    set_error("handoff: an earlier CPU correction job failed or timed out");
+    return JF_ERR_TIMEOUT;
+  }
+  if (!h->registered) {
+    h->registered = true;
+    StreamPoller::instance().add(h);
+  }
+  hipLaunchKernelGGL(handoff_signal_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, h->flag_pin,
+                     reinterpret_cast<int64_t*>(h->counter_dev + 2));
+  JF_CHECK_HIP(hipGetLastError());
+  return JF_OK;
+}
+
+extern "C" int jf_submit_ctx_stream_wait(int64_t ctx, void* stream) {
+  jf_handoff* h = ctx_of(ctx);
+  if (!h || !h->ext_q) { set_error("stream_wait_cpu_topk_attn: unknown context handle %lld", (long long)ctx); return JF_ERR_STATE; }
+  hipLaunchKernelGGL(handoff_wait_fetch_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, h->flag_pin + 8,
+                     reinterpret_cast<const int64_t*>(h->counter_dev + 2), h->flag_pin + 16, h->device_wait_ticks,
+                     (const uint4*)nullptr, (uint4*)nullptr, 0, (const float*)nullptr, (const float*)nullptr,
+                     (const float*)nullptr, (uint4*)nullptr);
+  JF_CHECK_HIP(hipGetLastError());
+  return JF_OK;
+}
+
+extern "C" int jf_submit_ctx_status(int64_t ctx) {
+  jf_handoff* h = ctx_of(ctx);
+  if (!h) { set_error("submit_ctx_status: unknown context handle %lld", (long long)ctx); return JF_ERR_STATE; }
+  return jf_handoff_status(h);
+}
+
+extern "C" int jf_stream_write_value64(void* stream, int64_t* flag_device, int64_t value) {
+  JF_CHECK_ARG(flag_device, "stream_write_value64: null flag");
+  hipLaunchKernelGGL(stream_write_value64_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, flag_device, value);
+  JF_CHECK_HIP(hipGetLastError());
+  return JF_OK;
+}
+
+extern "C" int jf_stream_wait_value64(void* stream, const int64_t* flag_device, int64_t value) {
+  JF_CHECK_ARG(flag_device, "stream_wait_value64: null flag");
+  {
+    std::lock_guard<std::mutex> g(g_ctx_mu);
+    if (!g_wait_timeouts) {
+      JF_CHECK_HIP(hipHostMalloc((void**)&g_wait_timeouts, 64, hipHostMallocDefault));
+      *g_wait_timeouts = 0;
+    }
+  }
+  const double t = future_timeout_s();
+  hipLaunchKernelGGL(stream_wait_value64_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, flag_device, value,
+                     (uint64_t)((t < 10.0 ? t : 10.0) * 1e8), g_wait_timeouts);
+  JF_CHECK_HIP(hipGetLastError());
+  return JF_OK;
+}
+
+extern "C" int64_t jf_stream_wait_timeouts(void) {
+  std::lock_guard<std::mutex> g(g_ctx_mu);
+  return g_wait_timeouts ? __atomic_load_n(g_wait_timeouts, __ATOMIC_ACQUIRE) : 0;
+}
+
+extern "C" int jf_cpu_topk_attn_async(const uint16_t* q, const uint16_t* k_shadow, const uint16_t* v_shadow,
+                                      const int64_t* head_map, const int64_t* ts_buf, uint16_t* o_new, int B, int H_q, int K,
+                                      int H_kv, int64_t num_slots, float scale, int64_t* flag) {
+  JF_CHECK_ARG(B > 0 && H_q > 0 && K > 0 && H_kv > 0 && num_slots > 0, "submit_cpu_topk_attn_async: bad shape");
+  JF_CHECK_ARG(q && k_shadow && v_shadow && head_map && ts_buf && o_new && flag, "submit_cpu_topk_attn_async: null pointer");
+  CpuJob j{q, k_shadow, v_shadow, head_map, ts_buf, o_new, B, H_q, K, H_kv, num_slots, scale};
+  AsyncExecutor::instance().submit(j, flag);
+  return JF_OK;
+}
+
+extern "C" int jf_wait_for_flag(const int64_t* flag, double timeout_s) {
+  JF_CHECK_ARG(flag, "wait_for_flag: null flag");
+  const auto t0 = std::chrono::steady_clock::now();
+  for (uint64_t spin = 0; __atomic_load_n(flag, __ATOMIC_ACQUIRE) == 0; ++spin) {
+    cpu_relax();
+    if ((spin & 0xfff) == 0xfff) {
+      const double el = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+      if (timeout_s > 0 && el > timeout_s) { set_error("wait_for_flag: timed out after %.1f s", el); return JF_ERR_TIMEOUT; }
+      if (el > 0.002) std::this_thread::sleep_for(std::chrono::microseconds(50));
+    }
+  }
+  return JF_OK;
+}
+
+extern "C" int jf_graph_pool_warmup(int n_threads) {
+  if (n_threads > 0) Pool::instance().set_threads(n_threads);
+  return Pool::instance().run(1, [](int64_t, int64_t) {}) ? JF_OK : JF_ERR_TIMEOUT;  // starts (or resizes) the workers
+}
+
+extern "C" int64_t jf_graph_submit_count(void) { return g_graph_submits.load(); }
+
+extern "C" int jf_reset_graph_runtime_state(void) {
+  g_graph_submits.store(0);
+  g_sanitize_count.store(0);
+  std::lock_guard<std::mutex> g(g_ctx_mu);
+  if (g_wait_timeouts) __atomic_store_n(g_wait_timeouts, (int64_t)0, __ATOMIC_RELEASE);
+  return JF_OK;
+}
+
+extern "C" int jf_clear_graph_contexts(void) {
+  std::vector<jf_handoff*> old;
+  {
+    std::lock_guard<std::mutex> g(g_ctx_mu);
+    old.swap(g_ctxs);
+  }
+  for (jf_handoff* h : old) jf_handoff_destroy(h);
+  g_graph_submits.store(0);
+  return JF_OK;
 }

@@ -17,6 +17,7 @@ HEAD_DIM = 128
 SUPPORTED_TOP_K = (32, 64, 128, 256, 512, 1024, 2048, 4096, 8192)
 
 _workspaces: dict = {}
+_retired_workspaces: list = []   # superseded buffers, kept because captured graphs may still point at them
 
 
 def _check(cond: bool, msg: str) -> None:
@@ -33,13 +34,25 @@ def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
 
 
 def _workspace(device: torch.device, nbytes: int, tag: str) -> torch.Tensor:
-    """Per-(device, stream, tag) scratch buffer that only grows; safe under stream ordering."""
+    """Per-(device, stream, tag) scratch buffer that only grows; safe under stream ordering.  A buffer that is
+    replaced by a larger one is kept alive: a HIP graph captured earlier on the stream has its address baked into
+    its kernels, and the allocator must not hand that memory to anyone else while the graph can be replayed."""
     key = (device, torch.cuda.current_stream(device).cuda_stream, tag)
     buf = _workspaces.get(key)
     if buf is None or buf.numel() < nbytes:
+        if buf is not None:
+            _retired_workspaces.append(buf)
         buf = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
         _workspaces[key] = buf
     return buf
+
+
+def reserve_fused_workspace(scheme: str, B: int, H_q: int, H_kv: int, max_S: int, top_k: int, device) -> int:
+    """Size the current stream's fused-scan workspace for a shape ahead of time (before a graph capture, so that
+    no capture or later eager call has to grow it).  Returns the size in bytes."""
+    scheme_id = {"k3v2": 32, "k4v4": 44, "k3v4": 34, "k4v2": 42}[scheme]
+    need = int(_lib.load().jf_fused_workspace_bytes(scheme_id, int(B), int(H_q), int(H_kv), int(max_S), int(top_k)))
+    return int(_workspace(torch.device(device), need, "fused").numel())
 
 
 def _gpu(*ts: torch.Tensor) -> None:
@@ -538,6 +551,59 @@ def blend_unnorm(o_hat, o_old_unnorm, W, o_new) -> torch.Tensor:
     return out
 
 
+def _blend_args(name, o_hat, o_old, W, o_new, out):
+    _check(o_hat.is_cuda and o_old.is_cuda and W.is_cuda and o_new.is_cuda and (out is None or out.is_cuda),
+           f"{name}: all tensors must be on the GPU")
+    _check(o_hat.dtype == torch.float32 and o_old.dtype == torch.float32 and W.dtype == torch.float32,
+           "o_hat / o_old / W must be fp32")
+    _check(o_new.dtype == torch.bfloat16 and (out is None or out.dtype == torch.bfloat16), "o_new / out must be bf16")
+    _check(o_hat.dim() == 3 and o_old.dim() == 3 and o_new.dim() == 3, "o_hat/o_old/o_new must be 3D (B, H_q, D)")
+    _check(W.dim() == 2, "W must be 2D (B, H_q)")
+    hc, oc, wc, nc = o_hat.contiguous(), o_old.contiguous(), W.contiguous(), o_new.contiguous()
+    _check(oc.shape == hc.shape, "o_old shape mismatch")
+    _check(nc.shape == hc.shape, "o_new shape mismatch")
+    _check(wc.shape == hc.shape[:2], "W shape mismatch")
+    if out is not None:
+        _check(out.is_contiguous(), "out must be contiguous")
+        _check(out.shape == hc.shape, "out shape mismatch")
+    return hc, oc, wc, nc
+
+
+def blend_into(o_hat, o_old, W, o_new, out) -> None:
+    """blend.cu:130-190: out = bf16(o_hat + W * (o_new - o_old)) with a normalised o_old, into `out`."""
+    hc, oc, wc, nc = _blend_args("blend_into", o_hat, o_old, W, o_new, out)
+    B, H_q, D = hc.shape
+    _lib.check(_lib.load().jf_blend(hc.data_ptr(), oc.data_ptr(), wc.data_ptr(), nc.data_ptr(), out.data_ptr(), B, H_q, D,
+                                    _stream(out)))
+
+
+def blend(o_hat, o_old, W, o_new) -> torch.Tensor:
+    """blend.cu:68-128: as blend_into, returning a new (B, H_q, D) bf16 tensor."""
+    hc, oc, wc, nc = _blend_args("blend", o_hat, o_old, W, o_new, None)
+    out = torch.empty(hc.shape, dtype=torch.bfloat16, device=hc.device)
+    B, H_q, D = hc.shape
+    _lib.check(_lib.load().jf_blend(hc.data_ptr(), oc.data_ptr(), wc.data_ptr(), nc.data_ptr(), out.data_ptr(), B, H_q, D,
+                                    _stream(out)))
+    return out
+
+
+def _flag_ptr(flag, name: str) -> int:
+    _check(isinstance(flag, torch.Tensor) and not flag.is_cuda and flag.numel() == 1 and flag.dtype == torch.int64,
+           f"{name} must be a 1-element int64 CPU tensor")
+    return flag.data_ptr()
+
+
+def wait_and_blend_unnorm_into(done_flag, o_hat, o_old_unnorm, W, o_new, out) -> None:
+    """blend.cu:292-377: the calling thread waits until the CPU correction has stored 1 to `done_flag`, then
+    launches blend_unnorm_into on the current stream (o_new is the device view of the mapped pinned buffer the
+    correction wrote)."""
+    ptr = _flag_ptr(done_flag, "done_flag")
+    _check(o_hat.is_cuda and o_old_unnorm.is_cuda and W.is_cuda and o_new.is_cuda and out.is_cuda,
+           "wait_and_blend_unnorm_into: all device tensors must be on the GPU")
+    _lib.check(_lib.load().jf_wait_for_flag(ptr, 0.0))
+    blend_unnorm_into(o_hat, o_old_unnorm, W, o_new, out)
+
+
 # --------------------------------------------------------------------------- CPU correction
 
 
@@ -572,6 +638,160 @@ def set_cpu_attn_threads(n: int) -> None:
 
 def get_cpu_attn_threads() -> int:
     return int(_lib.load().jf_get_cpu_attn_threads())
+
+
+class _DeviceView:
+    """Zero-copy device tensor over pinned host memory (the GPU addresses it across PCIe)."""
+
+    def __init__(self, ptr: int, shape, dtype: torch.dtype, owner):
+        typestr = {torch.bfloat16: "<u2", torch.float16: "<f2", torch.float32: "<f4", torch.int64: "<i8",
+                   torch.int32: "<i4", torch.uint8: "|u1", torch.int16: "<i2"}[dtype]
+        self.__cuda_array_interface__ = {"shape": tuple(int(x) for x in shape), "typestr": typestr, "data": (int(ptr), False),
+                                         "version": 2, "strides": None}
+        self._owner = owner
+
+
+def alloc_mapped_pinned_pair(shape, dtype):
+    """cpu_topk_attn.cpp:972-1023 -> (host_tensor, device_tensor) over the same pinned host memory: what the CPU
+    stores through the host tensor the GPU reads through the device tensor, with no copy."""
+    shape = tuple(int(x) for x in shape)
+    _check(len(shape) > 0 and all(x > 0 for x in shape), "alloc_mapped_pinned_pair: empty shape")
+    host = torch.zeros(shape, dtype=dtype, pin_memory=True)
+    dev_ptr = host_buffer_device_pointer(host)
+    if dtype == torch.bfloat16:      # the array interface has no bf16: view 16-bit words, then reinterpret
+        dev = torch.as_tensor(_DeviceView(dev_ptr, shape, torch.int16, host), device="cuda").view(torch.bfloat16)
+    else:
+        dev = torch.as_tensor(_DeviceView(dev_ptr, shape, dtype, host), device="cuda")
+    _check(dev.data_ptr() == dev_ptr, "alloc_mapped_pinned_pair: the device view does not alias the host buffer")
+    dev._jf_host = host              # the view borrows: keep the owner alive with it
+    return host, dev
+
+
+def _cpu_job_args(name, q, k_shadow, v_shadow, head_map, ts_buf, o_new):
+    for t in (q, k_shadow, v_shadow, head_map, ts_buf, o_new):
+        _check(not t.is_cuda, f"{name}: all tensors must be CPU")
+    _check(q.dtype == torch.bfloat16 and k_shadow.dtype == torch.bfloat16 and v_shadow.dtype == torch.bfloat16
+           and o_new.dtype == torch.bfloat16, "q / shadows / o_new must be bf16")
+    _check(head_map.dtype == torch.int64 and ts_buf.dtype == torch.int64, "head_map / ts_buf must be int64")
+    _check(q.dim() == 3 and q.size(2) == HEAD_DIM and k_shadow.dim() == 3 and k_shadow.size(2) == HEAD_DIM,
+           "q must be (B, H_q, 128) and shadows (H_kv, num_slots, 128)")
+    _check(v_shadow.shape == k_shadow.shape, "k_shadow / v_shadow shape mismatch")
+    _check(head_map.shape == ts_buf.shape and ts_buf.dim() == 3 and ts_buf.shape[:2] == q.shape[:2],
+           "head_map / ts_buf must be (B, H_q, K)")
+    _check(o_new.shape == q.shape, "o_new must be (B, H_q, 128)")
+    for t in (q, k_shadow, v_shadow, head_map, ts_buf, o_new):
+        _check(t.is_contiguous(), f"{name}: tensors must be contiguous")
+
+
+_ASYNC_KEEP: list = []      # tensors of asynchronous jobs in flight (released by wait_for_flag)
+_CTX_KEEP: dict = {}        # context handle -> the tensors it points at
+
+
+def submit_cpu_topk_attn_async(q, k_shadow, v_shadow, head_map, ts_buf, o_new, scale, flag) -> None:
+    """cpu_topk_attn.cpp:1184-1205: cpu_topk_attn on the library's executor thread; returns at once, 1 is stored to
+    `flag` (1-element int64 CPU tensor) when o_new is complete."""
+    _cpu_job_args("submit_cpu_topk_attn_async", q, k_shadow, v_shadow, head_map, ts_buf, o_new)
+    fp = _flag_ptr(flag, "flag")
+    B, H_q, _ = q.shape
+    _ASYNC_KEEP.append((flag, q, k_shadow, v_shadow, head_map, ts_buf, o_new))
+    _lib.check(_lib.load().jf_cpu_topk_attn_async(q.data_ptr(), k_shadow.data_ptr(), v_shadow.data_ptr(), head_map.data_ptr(),
+                                                  ts_buf.data_ptr(), o_new.data_ptr(), B, H_q, ts_buf.size(2),
+                                                  k_shadow.size(0), k_shadow.size(1), float(scale), fp))
+
+
+def wait_for_flag(flag) -> None:
+    """cpu_topk_attn.cpp:1217-1260: block until `flag` reads non-zero."""
+    fp = _flag_ptr(flag, "flag")
+    _lib.check(_lib.load().jf_wait_for_flag(fp, 0.0))
+    _ASYNC_KEEP[:] = [k for k in _ASYNC_KEEP if k[0].data_ptr() != fp]
+
+
+def persistent_worker_warmup() -> None:
+    _lib.check(_lib.load().jf_graph_pool_warmup(0))
+
+
+def create_cpu_topk_submit_ctx(q, k_shadow, v_shadow, head_map, ts_buf, o_new, scale, flag_host) -> int:
+    """cpu_topk_attn.cpp:2054-2163 -> opaque int handle for stream_submit_cpu_topk_attn / stream_wait_cpu_topk_attn.
+    All tensors are CPU (pinned q / ts_buf / o_new that the caller fills and reads with its own stream-ordered
+    copies); `flag_host` is the host half of an alloc_mapped_pinned_pair and receives 1 when a correction is done."""
+    _cpu_job_args("create_cpu_topk_submit_ctx", q, k_shadow, v_shadow, head_map, ts_buf, o_new)
+    fp = _flag_ptr(flag_host, "flag_host")
+    B, H_q, _ = q.shape
+    lib = _lib.load()
+    h = int(lib.jf_submit_ctx_create(q.data_ptr(), k_shadow.data_ptr(), v_shadow.data_ptr(), head_map.data_ptr(),
+                                     ts_buf.data_ptr(), o_new.data_ptr(), B, H_q, ts_buf.size(2), k_shadow.size(0),
+                                     k_shadow.size(1), float(scale), fp))
+    if h <= 0:
+        raise RuntimeError(lib.jf_last_error().decode())
+    _CTX_KEEP[h] = (q, k_shadow, v_shadow, head_map, ts_buf, o_new, flag_host)
+    return h
+
+
+def stream_submit_cpu_topk_attn(stream_id: int, ctx_handle: int) -> None:
+    """cpu_topk_attn.cpp:2239: start the context's CPU correction in stream order (graph-capturable: a kernel)."""
+    _lib.check(_lib.load().jf_submit_ctx_stream_submit(int(ctx_handle), int(stream_id)))
+
+
+def stream_wait_cpu_topk_attn(stream_id: int, ctx_handle: int) -> None:
+    """cpu_topk_attn.cpp:2302: make the stream wait for the context's correction (graph-capturable: a kernel with a
+    bounded device-side wait; check_cpu_topk_submit_ctx reports a wait that ran into its limit)."""
+    _lib.check(_lib.load().jf_submit_ctx_stream_wait(int(ctx_handle), int(stream_id)))
+
+
+def check_cpu_topk_submit_ctx(ctx_handle: int) -> None:
+    _lib.check(_lib.load().jf_submit_ctx_status(int(ctx_handle)))
+
+
+def _flag_dev_ptr(flag_device) -> int:
+    _check(isinstance(flag_device, torch.Tensor) and flag_device.is_cuda and flag_device.dtype == torch.int64
+           and flag_device.numel() >= 1, "flag_device must be the int64 device tensor of an alloc_mapped_pinned_pair")
+    return flag_device.data_ptr()
+
+
+def stream_write_value64(stream_id: int, flag_device, value: int) -> None:
+    """cpu_topk_attn.cpp:1293-1318"""
+    _lib.check(_lib.load().jf_stream_write_value64(int(stream_id), _flag_dev_ptr(flag_device), int(value)))
+
+
+def stream_wait_value64(stream_id: int, flag_device, value: int) -> None:
+    """cpu_topk_attn.cpp:1320-1344 (EQ)"""
+    _lib.check(_lib.load().jf_stream_wait_value64(int(stream_id), _flag_dev_ptr(flag_device), int(value)))
+
+
+def graph_pool_warmup() -> None:
+    _lib.check(_lib.load().jf_graph_pool_warmup(0))
+
+
+def graph_pool_warmup_threads(n_threads: int) -> None:
+    _check(int(n_threads) > 0, "graph_pool_warmup_threads: n_threads must be positive")
+    _lib.check(_lib.load().jf_graph_pool_warmup(int(n_threads)))
+
+
+def get_graph_submit_count() -> int:
+    return int(_lib.load().jf_graph_submit_count())
+
+
+def get_cpu_topk_sanitize_count() -> int:
+    return int(_lib.load().jf_cpu_topk_sanitize_count())
+
+
+def reset_graph_runtime_state() -> None:
+    _lib.check(_lib.load().jf_reset_graph_runtime_state())
+
+
+def clear_graph_contexts() -> None:
+    _lib.check(_lib.load().jf_clear_graph_contexts())
+    _CTX_KEEP.clear()
+
+
+def set_cpu_attn_isa(name) -> None:
+    """Row implementation of the CPU correction: None / "widest", "scalar", "avx2", "avx512bf16"."""
+    code = {None: -1, "widest": -1, "scalar": 0, "avx2": 1, "avx512bf16": 2}[name]
+    _lib.check(_lib.load().jf_set_cpu_attn_isa(code))
+
+
+def get_cpu_attn_isa() -> str:
+    return ("scalar", "avx2", "avx512bf16")[int(_lib.load().jf_get_cpu_attn_isa())]
 
 
 class CpuTopkHandoff:

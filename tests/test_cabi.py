@@ -54,10 +54,29 @@ def test_product_package_never_imports_the_oracle():
                 assert "oracle" not in src.lower() or f == "build.py", f"{f} mentions the oracle"
 
 
+def _host_isas():
+    from jetfire_amd import ops
+    ops.set_cpu_attn_isa(None)
+    widest = ops.get_cpu_attn_isa()
+    return ("scalar", "avx2", "avx512bf16")[:("scalar", "avx2", "avx512bf16").index(widest) + 1]
+
+
+@pytest.fixture
+def widest_isa_afterwards():
+    yield
+    from jetfire_amd import ops
+    ops.set_cpu_attn_isa(None)
+
+
+@pytest.mark.parametrize("isa", ("scalar", "avx2", "avx512bf16"))
 @pytest.mark.parametrize("threads", (1, 3))
 @pytest.mark.parametrize("B,Hq,Hkv,K", [(2, 8, 2, 32), (1, 32, 4, 256), (3, 4, 4, 7)])
-def test_cpu_topk_attn_matches_oracle(threads, B, Hq, Hkv, K):
+def test_cpu_topk_attn_matches_oracle(threads, B, Hq, Hkv, K, isa, widest_isa_afterwards):
     from jetfire_amd import ops
+    if isa not in _host_isas():
+        pytest.skip(f"this host has no {isa}")
+    ops.set_cpu_attn_isa(isa)
+    assert ops.get_cpu_attn_isa() == isa
     c = make_case(50 + K, B, Hq, Hkv, 256, 3, 2, 64, ragged=False)
     rng = np.random.default_rng(K)
     nslots = c["K"].shape[1]
@@ -76,6 +95,80 @@ def test_cpu_topk_attn_matches_oracle(threads, B, Hq, Hkv, K):
     ref = O.cpu_topk_attn(c["q"], c["K"], c["V"], hm, ts, 128 ** -0.5)
     np.testing.assert_allclose(bf16_to_f32(out), ref, atol=2e-3, rtol=6e-3)    # scripts/validate_runtime.py:187-191
     assert (bf16_to_f32(out)[0, 1] == 0).all()
+
+
+@pytest.mark.parametrize("isa", ("scalar", "avx2", "avx512bf16"))
+def test_cpu_topk_attn_sanitises_non_finite_rows(isa, widest_isa_afterwards):
+    """jetfire_vllm/csrc/cpu_topk_attn.cpp:809-826,839-846: a row whose output is not finite (here: an infinite V
+    element among its slots) is recomputed by the scalar row and zeroed when it still is; such rows are counted
+    and every other row is untouched."""
+    from jetfire_amd import ops
+    if isa not in _host_isas():
+        pytest.skip(f"this host has no {isa}")
+    ops.set_cpu_attn_isa(isa)
+    B, Hq, Hkv, K = 2, 8, 2, 16
+    c = make_case(77, B, Hq, Hkv, 128, 3, 2, 64, ragged=False)
+    rng = np.random.default_rng(5)
+    nslots = c["K"].shape[1]
+    ts = rng.integers(0, nslots, size=(B, Hq, K)).astype(np.int64)
+    hm = O.head_map(B, Hq, Hq // Hkv, K)
+    V = c["V"].copy()
+    bad_slot = int(ts[1, 5, 3])
+    V[5 // (Hq // Hkv), bad_slot, 17] = np.inf
+    poisoned = {(b, h) for b in range(B) for h in range(Hq) if h // (Hq // Hkv) == 5 // (Hq // Hkv) and bad_slot in ts[b, h]}
+    assert (1, 5) in poisoned
+    ops.reset_graph_runtime_state()
+    out = torch.full((B, Hq, 128), 7.0, dtype=torch.bfloat16)
+    ops.cpu_topk_attn(bf16_tensor(c["q"]), bf16_tensor(c["K"]), bf16_tensor(V), torch.from_numpy(hm), torch.from_numpy(ts), out,
+                      128 ** -0.5)
+    assert ops.get_cpu_topk_sanitize_count() == len(poisoned)
+    got = bf16_to_f32(out)
+    assert np.isfinite(got).all()
+    ref = O.cpu_topk_attn(c["q"], c["K"], c["V"], hm, ts, 128 ** -0.5)
+    for b in range(B):
+        for h in range(Hq):
+            if (b, h) in poisoned:
+                assert (got[b, h] == 0).all()
+            else:
+                np.testing.assert_allclose(got[b, h], ref[b, h], atol=2e-3, rtol=6e-3)
+    ops.reset_graph_runtime_state()
+    assert ops.get_cpu_topk_sanitize_count() == 0
+
+
+def test_async_submit_and_wait_for_flag_match_the_synchronous_call():
+    """submit_cpu_topk_attn_async / wait_for_flag (jetfire_vllm/csrc/cpu_topk_attn.cpp:1184-1260)."""
+    from jetfire_amd.kernels.cpu_topk_attn import load_cpu_topk_attn_ext
+    ext = load_cpu_topk_attn_ext()
+    for name in ("cpu_topk_attn", "alloc_mapped_pinned_pair", "submit_cpu_topk_attn_async", "wait_for_flag",
+                 "create_cpu_topk_submit_ctx", "stream_submit_cpu_topk_attn", "stream_wait_cpu_topk_attn",
+                 "stream_write_value64", "stream_wait_value64", "graph_pool_warmup", "graph_pool_warmup_threads",
+                 "get_graph_submit_count", "get_cpu_topk_sanitize_count", "reset_graph_runtime_state",
+                 "clear_graph_contexts", "set_cpu_attn_threads", "get_cpu_attn_threads"):
+        assert callable(getattr(ext, name)), name
+    from jetfire_amd.kernels.blend import load_blend_ext
+    for name in ("blend", "blend_into", "blend_unnorm_into", "wait_and_blend_unnorm_into"):
+        assert callable(getattr(load_blend_ext(), name)), name
+    B, Hq, Hkv, K = 2, 8, 2, 32
+    c = make_case(31, B, Hq, Hkv, 256, 3, 2, 64, ragged=False)
+    rng = np.random.default_rng(9)
+    ts = torch.from_numpy(rng.integers(-1, c["K"].shape[1], size=(B, Hq, K)).astype(np.int64))
+    hm = torch.from_numpy(O.head_map(B, Hq, Hq // Hkv, K))
+    q, ksh, vsh = bf16_tensor(c["q"]), bf16_tensor(c["K"]), bf16_tensor(c["V"])
+    ext.graph_pool_warmup_threads(3)
+    assert ext.get_cpu_attn_threads() == 3
+    want = torch.zeros(B, Hq, 128, dtype=torch.bfloat16)
+    ext.cpu_topk_attn(q, ksh, vsh, hm, ts, want, 0.09)
+    for rep in range(3):
+        got = torch.full((B, Hq, 128), 5.0, dtype=torch.bfloat16)
+        flag = torch.zeros(1, dtype=torch.int64)
+        ext.submit_cpu_topk_attn_async(q, ksh, vsh, hm, ts, got, 0.09, flag)
+        ext.wait_for_flag(flag)
+        assert int(flag[0]) == 1 and torch.equal(got.view(torch.int16), want.view(torch.int16))
+    with pytest.raises(RuntimeError, match="flag must be"):
+        ext.wait_for_flag(torch.zeros(2, dtype=torch.int64))
+    with pytest.raises(RuntimeError, match="unknown context handle"):
+        ext.stream_submit_cpu_topk_attn(0, 12345)
+    ext.set_cpu_attn_threads(2)
 
 
 def test_cpu_pool_survives_oversubscription_and_resizing():
