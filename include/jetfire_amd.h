@@ -147,8 +147,8 @@ int jf_topk_slots(const float* scores, const int32_t* seq_lens, const int64_t* b
  * Replaces int2_softmax_v_with_pre_corr_wvs2 (jetfire_vllm/csrc/int2_softmax_v.cu:792-901) for
  * v_nbits == 2 and int4_softmax_v_with_pre_corr_wvs2_scores (jetfire_vllm/csrc/int4_softmax_v.cu:
  * 2203-2235) for v_nbits == 4.  softmax_m / softmax_inv_z may be NULL (computed internally), or the
- * Stage-A statistics (then this is int8tc_softmax_v_with_pre_corr_reg_stats' contract with exact fp32
- * weights, jetfire_vllm/csrc/int8tc_softmax_v_fused.cu:1591-1734).  topk_idx may be NULL (o_hat only).
+ * Stage-A statistics (int4_softmax_v_with_pre_corr_wvs2_scores; the int8-weight form of
+ * int8tc_softmax_v_with_pre_corr_reg_stats is jf_softmax_v_int8_tiles below).  topk_idx may be NULL (o_hat only).
  * Split partials are reduced in a fixed order, so the result is run-to-run deterministic.
  * workspace: jf_softmax_v_workspace_bytes() bytes of device memory. */
 size_t jf_softmax_v_workspace_bytes(int B, int H_q, int max_S);
@@ -159,6 +159,21 @@ int jf_softmax_v_pre_corr(const float* scores, const float* softmax_m, const flo
                           int block_size, int top_k, int v_nbits, int n_scale_groups,
                           float* o_hat, float* o_old_unnorm, float* W,
                           void* workspace, size_t workspace_bytes, void* stream);
+
+/* INT4 values with int8-quantised softmax weights: replaces int8tc_softmax_v_with_pre_corr_reg_stats
+ * (jetfire_vllm/csrc/int8tc_softmax_v_fused.cu:1017-1401 kernel, :1591-1734 launcher) with its arithmetic: eight
+ * ranges of ceil(max_S / 8) positions, tiles of two pages starting at the page of a range's first position, per
+ * tile and row rs = max|p * v_scale| / 127, pq = clamp(rint(p * v_scale / rs), -127, 127), o_hat += f32(sum pq *
+ * (nibble - 8)) * rs (:1203-1236, 1298-1311); o_old_unnorm and W with exact fp32 weights (:1340-1400).  Needs the
+ * Stage-A statistics and one V scale per token (group 128).  The ranges' partial sums are added in ascending order
+ * (the reference adds them with atomics).  workspace: jf_softmax_v_workspace_bytes() bytes. */
+int jf_softmax_v_int8_tiles(const float* scores, const float* softmax_m, const float* softmax_inv_z,
+                            const uint8_t* v_data, const uint16_t* v_scales,
+                            const int64_t* block_table, const int32_t* seq_lens, const int64_t* topk_idx,
+                            int B, int H_q, int H_kv, int max_S, int max_blocks, int64_t num_slots,
+                            int block_size, int top_k,
+                            float* o_hat, float* o_old_unnorm, float* W,
+                            void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------ pieces 2+3: fused decode scan + top-k
  * One pass over the packed K and V of every (sequence, kv-head): Q.K^T for the GQA group, softmax

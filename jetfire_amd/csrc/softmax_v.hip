@@ -118,6 +118,96 @@ __global__ __launch_bounds__(SV_THREADS) void weighted_v_split_kernel(
     partial[(((size_t)b * H_q + (size_t)hkv * G + g) * n_splits + split) * D + tid] = acc[g];
 }
 
+// INT4 values with int8-quantised weights, the arithmetic of the reference's register-MMA Stage B
+// (jetfire_vllm/csrc/int8tc_softmax_v_fused.cu:1049-1052 split geometry, :1178 tile origin, :1203-1236 weight
+// quantisation, :1298-1311 accumulation): the sequence is cut into TQ_SPLITS ranges of ceil(max_S / TQ_SPLITS)
+// positions; a range is walked in tiles of two pages that start at the page holding its first position; per tile
+// and query head
+//     pv_t = exp(score_t - m) * inv_z * f32(v_scale_t)   (0 outside the range)
+//     rs   = max_t |pv_t| / 127,  pq_t = clamp(rint(pv_t * (1 / rs)), -127, 127)   (rs == 0: pq = 0)
+//     o_hat[d] += f32(sum_t pq_t * (nibble_t,d - 8)) * rs
+// with an exact int32 sum per tile and an fp32 running sum over the tiles in ascending order.
+// grid (TQ_SPLITS, H_kv, B); thread = output channel d; the 32-lane quarters of the workgroup take the heads in turn.
+constexpr int TQ_SPLITS = 8;
+constexpr int TQ_TILE = 2 * BS;
+template <int G>
+__global__ __launch_bounds__(SV_THREADS) void tile_quantised_v_split_kernel(
+    const float* __restrict__ scores, const float* __restrict__ softmax_m, const float* __restrict__ softmax_inv_z,
+    const uint8_t* __restrict__ v_data, const uint16_t* __restrict__ v_scales, const int64_t* __restrict__ block_table,
+    const int32_t* __restrict__ seq_lens, float* __restrict__ partial, int H_q, int H_kv, int max_S, int max_blocks,
+    int64_t num_slots) {
+  constexpr int P = D / 2;
+  __shared__ __align__(16) uint8_t vbuf[TQ_TILE * P];
+  __shared__ int pq[G][TQ_TILE];
+  __shared__ float rs_sh[G];
+  const int split = blockIdx.x, hkv = blockIdx.y, b = blockIdx.z, tid = threadIdx.x;
+  const int S = max(0, min(max_S, seq_lens[b]));
+  const int chunk = (max_S + TQ_SPLITS - 1) / TQ_SPLITS;
+  const int s_start = split * chunk, s_end = min(s_start + chunk, S);
+  float acc[G];
+#pragma unroll
+  for (int g = 0; g < G; ++g) acc[g] = 0.0f;
+  const uint8_t* vbase = v_data + (size_t)hkv * num_slots * P;
+  const uint16_t* sbase = v_scales + (size_t)hkv * num_slots;
+  const int64_t* bt = block_table + (size_t)b * max_blocks;
+  const int q32 = tid >> 5, l32 = tid & 31;
+  for (int t0 = (s_start / BS) * BS; t0 < s_end; t0 += TQ_TILE) {
+    __syncthreads();
+    // the two pages of the tile (a page past the table or the sequence contributes zero weights; its codes are not read)
+    int64_t base_slot[2];
+#pragma unroll
+    for (int pg = 0; pg < 2; ++pg) {
+      const int blk = t0 / BS + pg;
+      const int64_t e = (blk < max_blocks && blk * BS < s_end) ? bt[blk] : -1;
+      base_slot[pg] = (e >= 0 && (e + 1) * BS <= num_slots) ? e * BS : -1;
+    }
+    {
+      constexpr int NDW = BS * P / 4;  // 256 dwords per page
+#pragma unroll
+      for (int pg = 0; pg < 2; ++pg) {
+        const uint32_t* src = reinterpret_cast<const uint32_t*>(vbase + (base_slot[pg] < 0 ? 0 : base_slot[pg]) * P);
+#pragma unroll
+        for (int i = 0; i < NDW / SV_THREADS; ++i)
+          reinterpret_cast<uint32_t*>(vbuf)[pg * NDW + tid + i * SV_THREADS] = base_slot[pg] < 0 ? 0x88888888u : src[tid + i * SV_THREADS];
+      }
+    }
+    for (int g = q32; g < G; g += SV_THREADS / 32) {
+      const size_t bh = (size_t)b * H_q + (size_t)hkv * G + g;
+      const int pos = t0 + l32;
+      const int64_t bs = base_slot[l32 / BS];
+      float pv = 0.0f;
+      if (pos >= s_start && pos < s_end && bs >= 0) {
+        const float pr = __expf(scores[bh * (size_t)max_S + pos] - softmax_m[bh]) * softmax_inv_z[bh];
+        pv = pr * bf16_to_f32(sbase[bs + (l32 % BS)]);
+      }
+      float a = fabsf(pv);
+#pragma unroll
+      for (int o = 16; o > 0; o >>= 1) a = fmaxf(a, __shfl_xor(a, o, 32));
+      const float row_scale = a / 127.0f;
+      const float inv_scale = (row_scale > 0.0f) ? (1.0f / row_scale) : 0.0f;
+      int qv = (int)rintf(pv * inv_scale);
+      qv = max(-127, min(127, qv));
+      pq[g][l32] = qv;
+      if (l32 == 0) rs_sh[g] = row_scale;
+    }
+    __syncthreads();
+    int dot[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) dot[g] = 0;
+#pragma unroll 8
+    for (int j = 0; j < TQ_TILE; ++j) {
+      const int c = v_code<4>(vbuf + j * P, tid);
+#pragma unroll
+      for (int g = 0; g < G; ++g) dot[g] += pq[g][j] * c;
+    }
+#pragma unroll
+    for (int g = 0; g < G; ++g) acc[g] += (float)dot[g] * rs_sh[g];
+  }
+#pragma unroll
+  for (int g = 0; g < G; ++g)
+    partial[(((size_t)b * H_q + (size_t)hkv * G + g) * TQ_SPLITS + split) * D + tid] = acc[g];
+}
+
 // grid (B, H_q); adds split partials in order, then the top-k pre-correction.
 template <int NBITS, int NG>
 __global__ __launch_bounds__(SV_THREADS) void combine_precorr_kernel(
@@ -197,8 +287,9 @@ using namespace jf;
 extern "C" size_t jf_softmax_v_workspace_bytes(int B, int H_q, int max_S) {
   if (B <= 0 || H_q <= 0) return 256;
   // partials for the largest split count any H_kv can produce, plus the two statistics rows
-  const size_t max_splits = (size_t)((max_S + 63) / 64 < 2048 ? (max_S + 63) / 64 : 2048);
-  return ((size_t)B * H_q * (max_splits > 0 ? max_splits : 1) * D + 2 * (size_t)B * H_q) * sizeof(float) + 256;
+  size_t max_splits = (size_t)((max_S + 63) / 64 < 2048 ? (max_S + 63) / 64 : 2048);
+  if (max_splits < (size_t)TQ_SPLITS) max_splits = TQ_SPLITS;  // the tile-quantised form always uses TQ_SPLITS ranges
+  return ((size_t)B * H_q * max_splits * D + 2 * (size_t)B * H_q) * sizeof(float) + 256;
 }
 
 extern "C" int jf_softmax_v_pre_corr(const float* scores, const float* softmax_m, const float* softmax_inv_z,
@@ -261,5 +352,39 @@ extern "C" int jf_softmax_v_pre_corr(const float* scores, const float* softmax_m
   else if (v_nbits == 3) { JF_SV_LAUNCH(3, 2) }
   else if (n_scale_groups == 1) { JF_SV_LAUNCH(4, 1) }
   else { JF_SV_LAUNCH(4, 2) }
+  return JF_OK;
+}
+
+extern "C" int jf_softmax_v_int8_tiles(const float* scores, const float* softmax_m, const float* softmax_inv_z,
+                                       const uint8_t* v_data, const uint16_t* v_scales, const int64_t* block_table,
+                                       const int32_t* seq_lens, const int64_t* topk_idx, int B, int H_q, int H_kv,
+                                       int max_S, int max_blocks, int64_t num_slots, int block_size, int top_k,
+                                       float* o_hat, float* o_old_unnorm, float* W, void* workspace,
+                                       size_t workspace_bytes, void* stream) {
+  JF_CHECK_ARG(B >= 0 && H_q > 0 && H_kv > 0 && max_S >= 0 && H_q % H_kv == 0, "int8tc_softmax_v: bad shape");
+  const int G = H_q / H_kv;
+  JF_CHECK_ARG(G == 1 || G == 2 || G == 4 || G == 8 || G == 16, "int8tc_softmax_v requires H_q/H_kv in {1,2,4,8,16} (got %d)", G);
+  JF_CHECK_ARG(block_size == 16, "int8tc_softmax_v only supports block_size=16");
+  JF_CHECK_ARG((int64_t)max_blocks * block_size >= max_S, "int8tc_softmax_v: block_table does not cover max_S");
+  JF_CHECK_ARG(topk_idx == nullptr || top_k > 0, "int8tc_softmax_v: top_k must be positive");
+  if (B == 0) return JF_OK;
+  JF_CHECK_ARG(scores && softmax_m && softmax_inv_z && v_data && v_scales && block_table && seq_lens && o_hat,
+               "int8tc_softmax_v: null pointer (the Stage-A statistics are required)");
+  JF_CHECK_ARG(topk_idx == nullptr || (o_old_unnorm && W), "int8tc_softmax_v: o_old_unnorm / W required with topk_idx");
+  JF_CHECK_ARG(workspace && workspace_bytes >= jf_softmax_v_workspace_bytes(B, H_q, max_S) &&
+                   workspace_bytes >= (size_t)B * H_q * TQ_SPLITS * D * sizeof(float),
+               "int8tc_softmax_v: workspace too small");
+  hipStream_t st = (hipStream_t)stream;
+  float* partial = reinterpret_cast<float*>(workspace);
+  dim3 grid(TQ_SPLITS, H_kv, B), block(SV_THREADS);
+  JF_DISPATCH_G2(G, {
+    hipLaunchKernelGGL((tile_quantised_v_split_kernel<GG>), grid, block, 0, st, scores, softmax_m, softmax_inv_z, v_data,
+                       v_scales, block_table, seq_lens, partial, H_q, H_kv, max_S, max_blocks, num_slots);
+  });
+  JF_CHECK_LAUNCH();
+  hipLaunchKernelGGL((combine_precorr_kernel<4, 1>), dim3(B, H_q), block, 0, st, partial, scores, softmax_m, softmax_inv_z,
+                     v_data, v_scales, block_table, seq_lens, topk_idx, o_hat, o_old_unnorm, W, H_q, H_kv, max_S, max_blocks,
+                     num_slots, TQ_SPLITS, top_k);
+  JF_CHECK_LAUNCH();
   return JF_OK;
 }

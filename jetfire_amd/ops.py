@@ -352,7 +352,7 @@ def int8tc_qk_scores_topk_stats(q, k_data, k_scales, block_table, seq_lens, max_
 
 
 def _softmax_v(scores, m, iz, v_data, v_scales, block_table, seq_lens, topk_idx, max_S, H_q, H_kv, block_size, top_k,
-               nbits: int, outs=None):
+               nbits: int, outs=None, int8_tiles: bool = False):
     lib = _lib.load()
     _gpu(scores, v_data, v_scales, block_table, seq_lens)
     _check(scores.dtype == torch.float32 and scores.dim() == 3, "scores must be (B, H_q, max_S) fp32")
@@ -385,6 +385,12 @@ def _softmax_v(scores, m, iz, v_data, v_scales, block_table, seq_lens, topk_idx,
     ws = _workspace(dev, need, "softmax_v")
     if m is not None:
         m, iz = m.contiguous(), iz.contiguous()
+    if int8_tiles:
+        _lib.check(lib.jf_softmax_v_int8_tiles(
+            sc.data_ptr(), _ptr(m), _ptr(iz), vd.data_ptr(), vs.data_ptr(), bt.data_ptr(), sl.data_ptr(), _ptr(topk_idx),
+            B, H_q, H_kv, int(max_S), bt.size(1), vd.size(1), int(block_size), int(top_k),
+            o_hat.data_ptr(), o_old.data_ptr(), W.data_ptr(), ws.data_ptr(), ws.numel(), _stream(sc)))
+        return [o_hat, o_old, W]
     _lib.check(lib.jf_softmax_v_pre_corr(
         sc.data_ptr(), _ptr(m), _ptr(iz), vd.data_ptr(), vs.data_ptr(), bt.data_ptr(), sl.data_ptr(), _ptr(topk_idx),
         B, H_q, H_kv, int(max_S), bt.size(1), vd.size(1), int(block_size), int(top_k), nbits, ng,
@@ -458,17 +464,16 @@ def int4_softmax_v_with_pre_corr_wvs2(scores, v_data, v_scales, block_table, seq
 
 def int8tc_softmax_v_with_pre_corr_reg_stats(scores, softmax_m, softmax_inv_z, v_data, v_scales, block_table, seq_lens,
                                              topk_idx, max_S, H_q, H_kv, block_size, top_k) -> List[torch.Tensor]:
-    """int8tc_softmax_v_fused.cu:1591-1734 -> [o_hat, o_old_unnorm, W].
-
-    The reference quantises P*v_scale to int8 per 32-token tile (an extra approximation it tolerates at 3e-3,
-    scripts/validate_runtime.py:173-176); this implementation keeps the weights in fp32, i.e. it returns the dense
-    quantity that approximation targets, and uses the Stage-A statistics it is handed."""
+    """int8tc_softmax_v_fused.cu:1591-1734 -> [o_hat, o_old_unnorm, W], with the reference's arithmetic: P * v_scale
+    quantised to int8 per 32-position tile and row (:1203-1236), int32 tile sums scaled back in fp32 (:1298-1311),
+    exact fp32 weights for o_old_unnorm and W (:1340-1400).  Uses the Stage-A statistics it is handed."""
+    _check(softmax_m is not None and softmax_inv_z is not None, "int8tc_softmax_v requires the Stage-A statistics")
     _check(softmax_m.dtype == torch.float32 and softmax_inv_z.dtype == torch.float32, "softmax stats must be fp32")
     vs = v_scales.unsqueeze(-1) if v_scales.dim() == 2 else v_scales
     _check(vs.size(2) == 1, "int8tc_softmax_v requires one V scale per token (group 128)")
     _check(H_q // H_kv <= 16, "int8tc_softmax_v requires H_q/H_kv <= 16")
     return _softmax_v(scores, softmax_m, softmax_inv_z, v_data, v_scales, block_table, seq_lens, topk_idx, max_S, H_q,
-                      H_kv, block_size, top_k, 4)
+                      H_kv, block_size, top_k, 4, int8_tiles=True)
 
 
 # --------------------------------------------------------------------------- fused scan

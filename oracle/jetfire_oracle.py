@@ -461,7 +461,8 @@ def softmax_v_int8_tiles(scores, softmax_m, softmax_inv_z, v_data, v_scale_bits,
                          topk_idx, max_S, H_q, H_kv, block_size, splits: int = 8):
     """INT4 V with int8-quantised P (int8tc_softmax_v_fused.cu:1203-1236,1298-1311;
     validate_runtime_edges.py:146-164).  The sequence is cut into `splits` ranges of
-    ceil(max_S/splits) positions; inside each range, per 32-position tile and per row:
+    ceil(max_S/splits) positions (:1049-1052); a range is walked in tiles of two pages starting at the page of
+    its first position (:1178); per tile and per row:
       pv = p * f32(v_scale); rs = amax|pv| / 127; pq = clamp(rint(pv / rs), -127, 127) (0 if rs == 0)
       o_hat += f32(sum_t pq_t * (nibble - 8)) * rs
     o_old_unnorm and W use the exact fp32 weights.
@@ -492,8 +493,11 @@ def softmax_v_int8_tiles(scores, softmax_m, softmax_inv_z, v_data, v_scale_bits,
             acc = np.zeros(D, dtype=np.float64)
             for s0 in range(0, S, chunk):
                 s1 = min(s0 + chunk, S)
-                for t0 in range(s0, s1, 32):
-                    t1 = min(t0 + 32, s1)
+                # tiles are pairs of pages counted from the page that holds s0 (int8tc_softmax_v_fused.cu:1052,1178);
+                # positions of a tile outside [s0, s1) carry zero weight (:1218)
+                origin = (s0 // block_size) * block_size
+                for tile0 in range(origin, s1, 2 * block_size):
+                    t0, t1 = max(tile0, s0), min(tile0 + 2 * block_size, s1)
                     pv = (p[t0:t1] * vs[t0:t1]).astype(np.float32)
                     amax = np.abs(pv).max() if t1 > t0 else np.float32(0)
                     rs = np.float32(amax) / np.float32(127.0)

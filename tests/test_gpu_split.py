@@ -324,15 +324,38 @@ def test_stage_b_outputs(scheme, B, Hq, Hkv, lens):
     np.testing.assert_allclose(o_hat.cpu().numpy(), r_hat, atol=3e-6, rtol=3e-6)     # validate_runtime.py:173-177
     np.testing.assert_allclose(o_old.cpu().numpy(), r_old, atol=3e-6, rtol=3e-6)
     np.testing.assert_allclose(W.cpu().numpy(), r_W, atol=3e-6, rtol=3e-6)
-    if vb == 4:                                                   # the variant that is handed Stage-A statistics
+    if vb == 4:                                                   # the int8-weight variant, handed Stage-A statistics
         m, iz = O.softmax_stats(ref_sc, c["lens"], S)
         o2 = o.int8tc_softmax_v_with_pre_corr_reg_stats(sc_t, torch.from_numpy(m).cuda(), torch.from_numpy(iz).cuda(),
                                                         d["vd"], d["vs"], d["bt"], d["lens"], idx_t, S, Hq, Hkv, 16, K)
-        np.testing.assert_allclose(o2[0].cpu().numpy(), r_hat, atol=3e-6, rtol=3e-6)
-        if lens is None:   # long rows: within the reference's own int8-P tolerance (validate_runtime.py:173-176);
-            # on short peaked rows the int8-P approximation itself strays further (validate_runtime_edges.py:146-152)
-            t_hat, _, _ = O.softmax_v_int8_tiles(ref_sc, m, iz, c["vd"], c["vs"], c["bt"], c["lens"], ridx, S, Hq, Hkv, 16)
-            np.testing.assert_allclose(o2[0].cpu().numpy(), t_hat, atol=3e-3)
+        # the reference's own tile arithmetic, at the tolerance its validator uses for it
+        # (scripts/validate_runtime_edges.py:146-171); the pre-correction terms use exact fp32 weights
+        t_hat, t_old, t_W = O.softmax_v_int8_tiles(ref_sc, m, iz, c["vd"], c["vs"], c["bt"], c["lens"], ridx, S, Hq, Hkv, 16)
+        np.testing.assert_allclose(o2[0].cpu().numpy(), t_hat, atol=3e-6, rtol=3e-6)
+        np.testing.assert_allclose(o2[1].cpu().numpy(), t_old, atol=3e-6, rtol=3e-6)
+        np.testing.assert_allclose(o2[2].cpu().numpy(), t_W, atol=3e-6, rtol=3e-6)
+        if lens is None:   # long rows: the approximation stays within the reference's int8-P tolerance of the dense
+            # result (validate_runtime.py:173-176); on short peaked rows it strays further (validate_runtime_edges.py:146-152)
+            np.testing.assert_allclose(o2[0].cpu().numpy(), r_hat, atol=3e-3)
+
+
+@pytest.mark.parametrize("S,lens", [(1000, [1000, 333]), (72, [72, 5]), (256, [256, 0])])
+def test_int8_tile_stage_b_on_ranges_that_do_not_start_on_a_page(S, lens):
+    """ceil(S / 8) is not a multiple of 16 here: tiles start at the page holding a range's first position and the
+    positions of that page before the range carry no weight (int8tc_softmax_v_fused.cu:1052,1178,1218)."""
+    B, Hq, Hkv, K = 2, 8, 2, 64
+    c = make_case(5 + S, B, Hq, Hkv, S, 4, 4, 128, lens=lens)
+    d = to_device(c)
+    o = ops()
+    ref_sc = O.scores_int8_model(c["q"], c["kd"], c["ks"], c["bt"], c["lens"], S, Hq, Hkv, 16, 128 ** -0.5)
+    ridx, _ = O.topk_select(ref_sc, c["lens"], c["bt"], S, K)
+    m, iz = O.softmax_stats(ref_sc, c["lens"], S)
+    got = o.int8tc_softmax_v_with_pre_corr_reg_stats(torch.from_numpy(ref_sc).cuda(), torch.from_numpy(m).cuda(),
+                                                     torch.from_numpy(iz).cuda(), d["vd"], d["vs"], d["bt"], d["lens"],
+                                                     torch.from_numpy(ridx).cuda(), S, Hq, Hkv, 16, K)
+    want = O.softmax_v_int8_tiles(ref_sc, m, iz, c["vd"], c["vs"], c["bt"], c["lens"], ridx, S, Hq, Hkv, 16)
+    for g, w in zip(got, want):
+        np.testing.assert_allclose(g.cpu().numpy(), w, atol=3e-6, rtol=3e-6)
 
 
 def test_blend_bit_exact():

@@ -160,6 +160,67 @@ def test_int8_tile_model_tracks_dense_model():
     np.testing.assert_allclose(t[2], d[2], atol=3e-6, rtol=3e-6)
 
 
+def test_int8_tile_model_equals_the_validators_restatement_on_aligned_contexts():
+    """scripts/validate_runtime_edges.py:146-164 models the tile arithmetic for contexts that are multiples of 256
+    (eight ranges aligned to the 32-position tiles) as: reshape(P * v_scale) to (..., 32), scale = amax / 127,
+    round(weighted / scale).clamp(+-127) * scale, then a dense contraction with the V codes.  Restated here with
+    numpy and compared with the oracle's tile walk."""
+    B, Hq, Hkv, S = 2, 4, 2, 512
+    c = make_case(18, B, Hq, Hkv, S, 4, 4, 128, ragged=False)
+    sc = O.scores_int8_model(c["q"], c["kd"], c["ks"], c["bt"], c["lens"], S, Hq, Hkv, 16, 128 ** -0.5)
+    m, iz = O.softmax_stats(sc, c["lens"], S)
+    got, _, _ = O.softmax_v_int8_tiles(sc, m, iz, c["vd"], c["vs"], c["bt"], c["lens"], None, S, Hq, Hkv, 16)
+    slots = O.slots_from_block_table(c["bt"], S, 16)
+    codes = O.decode_codes(c["vd"], 4).astype(np.float64) - 8
+    vs = O.bf16_bits_to_f32(c["vs"]).reshape(Hkv, -1)
+    for b in range(B):
+        for h in range(Hq):
+            hk = h // (Hq // Hkv)
+            p = (np.exp((sc[b, h] - m[b, h]).astype(np.float64)) * float(iz[b, h])).astype(np.float32)
+            weighted = (p * vs[hk, slots[b]]).astype(np.float32).reshape(-1, 32)
+            amax = np.abs(weighted).max(-1, keepdims=True)
+            tile_scale = (amax / np.float32(127)).astype(np.float32)
+            inverse = np.where(tile_scale > 0, np.float32(1) / np.where(tile_scale > 0, tile_scale, 1), 0).astype(np.float32)
+            qw = (np.clip(np.rint((weighted * inverse).astype(np.float32)), -127, 127) * tile_scale).reshape(-1)
+            want = qw.astype(np.float64) @ codes[hk, slots[b]]
+            np.testing.assert_allclose(got[b, h], want, atol=3e-6, rtol=3e-6)
+
+
+def test_int8_tile_model_tile_origin_on_unaligned_ranges():
+    """Brute force where ceil(S / 8) = 25 is not a page multiple: every range's tiles are page pairs counted from
+    the page of its first position (int8tc_softmax_v_fused.cu:1052,1178), restricted to the range (:1218).  The
+    range [25, 50) is therefore TWO tiles, [25, 48) and [48, 50), not the single tile a walk in steps of 32 from
+    position 25 would make; the two give different sums because each tile has its own scale."""
+    S, Hq, Hkv = 200, 1, 1
+    c = make_case(19, 1, Hq, Hkv, S, 4, 4, 128, ragged=False)
+    rng = np.random.default_rng(4)
+    sc = rng.standard_normal((1, 1, S)).astype(np.float32) * 2
+    m, iz = O.softmax_stats(sc, c["lens"], S)
+    got, _, _ = O.softmax_v_int8_tiles(sc, m, iz, c["vd"], c["vs"], c["bt"], c["lens"], None, S, Hq, Hkv, 16)
+    slots = O.slots_from_block_table(c["bt"], S, 16)[0]
+    codes = O.decode_codes(c["vd"], 4).astype(np.float64)[0] - 8
+    vs = O.bf16_bits_to_f32(c["vs"]).reshape(Hkv, -1)[0]
+    p = (np.exp((sc[0, 0] - m[0, 0]).astype(np.float64)) * float(iz[0, 0])).astype(np.float32)
+
+    def walk(origin_of):
+        total = np.zeros(128)
+        for r in range(8):
+            s0, s1 = 25 * r, min(25 * r + 25, S)
+            for tile0 in range(origin_of(s0), s1, 32):
+                pos = [t for t in range(tile0, tile0 + 32) if s0 <= t < s1]
+                if not pos:
+                    continue
+                pv = (p[pos] * vs[slots[pos]]).astype(np.float32)
+                rs = np.float32(np.abs(pv).max() / np.float32(127))
+                if rs > 0:
+                    pq = np.clip(np.rint(pv * (np.float32(1) / rs)), -127, 127)
+                    total += (pq @ codes[slots[pos]]) * float(rs)
+        return total
+
+    np.testing.assert_allclose(got[0, 0], walk(lambda s0: (s0 // 16) * 16), atol=1e-6)
+    assert np.abs(got[0, 0] - walk(lambda s0: s0)).max() > 1e-5     # the other tiling is a different function
+
+
 def test_cpu_correction_special_cases():
     c = make_case(9, 2, 8, 2, 64, 3, 2, 64, ragged=False)
     hm = O.head_map(2, 8, 4, 1)
