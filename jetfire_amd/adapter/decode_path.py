@@ -10,8 +10,8 @@ Graph mode (`JETFIRE_DECODE_GRAPH=1`, `decode_path.py:634-646`): the hand-off us
 wait pair, nothing in the entry synchronises with the device, and the whole layer can be captured into a HIP
 graph and replayed; `warmup_graph_decode_submit_contexts` creates, before capture, whatever a capture may
 not allocate.  A miss while a graph is being captured raises instead of baking the caller's fall-back into
-the graph (`:698-706`).  The reference's trace hooks, release policy and debug correction modes are not
-reproduced."""
+the graph (`:698-706`).  With `JETFIRE_RELEASE_GRAPH_POLICY=1` the kernels of a step are the ones the release
+policy names (`release_policy.py`).  The reference's trace hooks and debug correction modes are not reproduced."""
 from __future__ import annotations
 
 import bisect
@@ -24,6 +24,7 @@ import weakref
 import torch
 
 from .. import ops
+from . import release_policy
 from .config import get_jetfire_config
 from .kv_pool import get_global_kv_pool_manager
 
@@ -252,26 +253,41 @@ def reset_jetfire_decode_runtime_state(*, check: bool = False) -> None:
     _SEQ_LENS_CACHE.clear()
 
 
-def _split_stages(store, q, bt, sl, max_S: int, H_q: int, H_kv: int, top_k: int, scale: float):
-    """Stage A and Stage B as separate kernels, each side chosen by its bit width as the reference does
+def _split_stages(store, q, bt, sl, max_S: int, H_q: int, H_kv: int, top_k: int, scale: float, plan=None):
+    """Stage A and Stage B as separate kernels.  With a release plan (`release_policy.plan_release_graph`) the two
+    operators are the ones the plan names; otherwise each side is chosen by its bit width as the reference does
     (`decode_path.py:2013-2131` Stage A, `:2695-2935` Stage B): the path of the schemes that have no fused kernel."""
     bs = store.block_size
-    m = iz = None
     kd, ks, vd, vs = store.k_data, store.k_scales, store.v_data, store.v_scales
-    if store.k_nbits == 4:
-        int8tc = (ks.shape[-1] == 1 and top_k >= 64 and os.environ.get("JETFIRE_USE_INT8_TC", "1") == "1")
-        stage_a = ops.int8tc_qk_scores_topk_stats if int8tc else ops.int4_qk_scores_topk_stats
-        scores, idx, slots, m, iz = stage_a(q, kd, ks, bt, sl, max_S, H_q, H_kv, bs, scale, top_k)
-    elif store.k_nbits == 3:
-        scores, idx, slots = ops.int3_qk_scores_topk(q, kd, ks, bt, sl, max_S, H_q, H_kv, bs, scale, top_k)
+    if plan is not None:
+        a_name, b_name = plan.operators()
+        if a_name is None or b_name is None:
+            raise RuntimeError(f"release plan {plan.stage_a} / {plan.stage_b} has no kernel in this library")
     else:
-        scores, idx, slots = ops.int2_qk_scores_topk(q, kd, ks, store.k_zp, bt, sl, max_S, H_q, H_kv, bs, scale, top_k)
-    if store.v_nbits == 4 and m is not None and vs.shape[-1] == 1:
-        o_hat, o_old, W = ops.int8tc_softmax_v_with_pre_corr_reg_stats(scores, m, iz, vd, vs, bt, sl, idx, max_S, H_q, H_kv,
-                                                                      bs, top_k)
+        if store.k_nbits == 4:
+            int8tc = (ks.shape[-1] == 1 and top_k >= 64 and os.environ.get("JETFIRE_USE_INT8_TC", "1") == "1")
+            a_name = "int8tc_qk_scores_topk_stats" if int8tc else "int4_qk_scores_topk_stats"
+        else:
+            a_name = f"int{store.k_nbits}_qk_scores_topk"
+        if store.v_nbits == 4 and store.k_nbits == 4 and vs.shape[-1] == 1:
+            b_name = "int8tc_softmax_v_with_pre_corr_reg_stats" if q.shape[0] > 1 else "int4_softmax_v_with_pre_corr_wvs2_scores"
+        else:
+            b_name = {2: "int2_softmax_v_with_pre_corr_wvs2", 3: "int3_softmax_v_with_pre_corr_wvs2",
+                      4: "int4_softmax_v_with_pre_corr_wvs2_scores"}[store.v_nbits]
+    stage_a, stage_b = getattr(ops, a_name), getattr(ops, b_name)
+    m = iz = None
+    if a_name == "int2_qk_scores_topk":
+        scores, idx, slots = stage_a(q, kd, ks, store.k_zp, bt, sl, max_S, H_q, H_kv, bs, scale, top_k)
     else:
-        stage_b = {2: ops.int2_softmax_v_with_pre_corr_wvs2, 3: ops.int3_softmax_v_with_pre_corr_wvs2,
-                   4: ops.int4_softmax_v_with_pre_corr_wvs2_scores}[store.v_nbits]
+        res = stage_a(q, kd, ks, bt, sl, max_S, H_q, H_kv, bs, scale, top_k)
+        scores, idx, slots = res[:3]
+        if len(res) == 5:
+            m, iz = res[3], res[4]
+    if b_name == "int8tc_softmax_v_with_pre_corr_reg_stats":
+        if m is None:
+            raise RuntimeError("the int8-weight Stage B needs the statistics of the int8 Stage A")
+        o_hat, o_old, W = stage_b(scores, m, iz, vd, vs, bt, sl, idx, max_S, H_q, H_kv, bs, top_k)
+    else:
         o_hat, o_old, W = stage_b(scores, vd, vs, bt, sl, idx, max_S, H_q, H_kv, bs, top_k)
     return o_hat, slots, o_old, W
 
@@ -328,10 +344,22 @@ def _decode_batched(*, impl, layer, query, attn_metadata, output):
         if not complete:
             return miss("store_incomplete")
         max_S = int(getattr(attn_metadata, "max_seq_len", int(seq_lens_cpu.max().item())))
-    fused = store.scheme is not None and os.environ.get("JETFIRE_USE_FUSED_ATTN_TOPK", "1") == "1"
+    # Under the release policy (JETFIRE_RELEASE_GRAPH_POLICY=1) the step runs the two kernels the policy names for
+    # this cell, through the split operators; otherwise the fused scan where it covers the scheme.
+    release = release_policy.release_policy_enabled() and not store.k_asymmetric
+    if release:
+        release_policy.validate_release_environment()
+    fused = (not release and store.scheme is not None and os.environ.get("JETFIRE_USE_FUSED_ATTN_TOPK", "1") == "1")
     top_k = _select_top_k(pool.config.topk, max_S, FUSED_SUPPORTED_TOP_K if fused else SPLIT_SUPPORTED_TOP_K)
     if top_k is None:
         return miss("seq_len_too_short")
+    plan = None
+    if release:
+        plan = release_policy.plan_release_graph(
+            mode=f"SymInt{store.k_nbits}K_SymInt{store.v_nbits}V", group_size=store.group_size, top_k=top_k, head_dim=D,
+            num_query_heads=H_q, num_kv_heads=H_kv,
+            max_graph_batch=max(n_seqs, int(get_jetfire_config().max_batch_size or 0)),
+            require_ready=release_policy.release_require_ready())
 
     q_batch = query[:n_seqs].contiguous().view(n_seqs, H_q, D).to(torch.bfloat16)
     bt_batch = attn_metadata.block_table[:n_seqs].to(torch.int64).contiguous()
@@ -342,7 +370,8 @@ def _decode_batched(*, impl, layer, query, attn_metadata, output):
             store.scheme, q_batch, store.k_data, store.k_scales, store.v_data, store.v_scales, bt_batch, seq_lens_batch,
             max_S, H_q, H_kv, store.block_size, top_k, scale)
     else:
-        o_hat, topk_slots, o_old, W = _split_stages(store, q_batch, bt_batch, seq_lens_batch, max_S, H_q, H_kv, top_k, scale)
+        o_hat, topk_slots, o_old, W = _split_stages(store, q_batch, bt_batch, seq_lens_batch, max_S, H_q, H_kv, top_k, scale,
+                                                    plan=plan)
     handoff = _handoff_for(store, n_seqs, H_q, H_kv, top_k, scale, stream_mode=graph_mode, layer_name=layer_name)
     o_new = _o_new_for(n_seqs, H_q, D, query.device)
     out_view = output[:n_seqs].view(n_seqs, H_q, D)

@@ -536,3 +536,56 @@ def test_graph_mode_reports_a_correction_that_never_arrives(adapter, monkeypatch
     with pytest.raises(RuntimeError, match="limit"):
         adapter.try_jetfire_decode(impl=impl, layer=layer, query=q, attn_metadata=meta, output=out)
     h.debug_pause(False)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("scheme_name,gs", [("SymInt3K_SymInt2V", 64), ("SymInt4K_SymInt4V", 128)])
+def test_release_policy_selects_the_named_split_kernels(adapter, monkeypatch, scheme_name, gs):
+    """JETFIRE_RELEASE_GRAPH_POLICY=1: the step runs the Stage A / Stage B operators the plan names (recorded by
+    wrapping them), gives the fused path's result within the stage tolerances, and an experimental switch raises."""
+    from jetfire_amd import ops as jops
+    from jetfire_amd.adapter import release_policy
+    for name in list(__import__("os").environ):
+        if name.startswith("JETFIRE_"):
+            monkeypatch.delenv(name)
+    B, Hq, Hkv, D, bs, K, max_S = 2, 8, 2, 128, 16, 64, 256
+    adapter.set_jetfire_config(scheme=scheme_name, group_size=gs, topk=K, layer_stride=1, cpu_attn_threads=2, max_batch_size=B)
+    adapter.reset_global_kv_pool_manager()
+    pool = adapter.get_global_kv_pool_manager()
+    name = "model.layers.0.self_attn.attn"
+    layer = types.SimpleNamespace(layer_name=name, num_heads=Hq, num_kv_heads=Hkv, head_size=D)
+    impl = types.SimpleNamespace(attn_type=types.SimpleNamespace(name="DECODER"), scale=D ** -0.5)
+    pool.ensure_layer_config_from_layer(name, layer)
+    per_seq = max_S // bs
+    pool.register_layer_layout(name, num_blocks=B * per_seq, block_size=bs)
+    g = torch.Generator().manual_seed(11)
+    lens = [200, 131]
+    bt = torch.arange(B * per_seq, dtype=torch.int64).view(B, per_seq).cuda()
+    slots = torch.cat([bt[b, p // bs].cpu() * bs + p % bs for b in range(B) for p in [torch.arange(lens[b])]]).cuda()
+    n = int(slots.numel())
+    pool.mirror_kv(name, torch.randn(n, Hkv, D, generator=g).to(torch.bfloat16).cuda(),
+                   torch.randn(n, Hkv, D, generator=g).to(torch.bfloat16).cuda(), slots)
+    pool.flush_pending_writes()
+    meta = _meta(torch.tensor(lens, dtype=torch.int32, device="cuda"), bt, max_seq_len=max(lens))
+    q = (torch.randn(B, Hq, D, generator=g) / D ** 0.5).to(torch.bfloat16).cuda()
+    fused_out = torch.zeros(B, Hq * D, dtype=torch.bfloat16, device="cuda")
+    assert adapter.try_jetfire_decode(impl=impl, layer=layer, query=q, attn_metadata=meta, output=fused_out) is fused_out
+    torch.cuda.synchronize()
+    store = pool.get_layer_store(name)
+    plan = release_policy.plan_release_graph(mode=scheme_name, group_size=gs, top_k=K, max_graph_batch=B)
+    called = []
+    for op_name in plan.operators():
+        real = getattr(jops, op_name)
+        monkeypatch.setattr(jops, op_name, (lambda f, nm: (lambda *a, **k: (called.append(nm), f(*a, **k))[1]))(real, op_name))
+    monkeypatch.setenv("JETFIRE_RELEASE_GRAPH_POLICY", "1")
+    monkeypatch.setenv("JETFIRE_RELEASE_REQUIRE_READY", "1")
+    out = torch.zeros_like(fused_out)
+    assert adapter.try_jetfire_decode(impl=impl, layer=layer, query=q, attn_metadata=meta, output=out) is out
+    torch.cuda.synchronize()
+    assert called == list(plan.operators())
+    err = (out.float() - fused_out.float()).abs()
+    assert float(err.max()) <= 2e-2 and float(err.mean()) <= 1e-3
+    monkeypatch.setenv("JETFIRE_USE_FUSED_ATTN_TOPK", "1")
+    with pytest.raises(release_policy.ReleasePolicyError, match="JETFIRE_USE_FUSED_ATTN_TOPK"):
+        adapter.try_jetfire_decode(impl=impl, layer=layer, query=q, attn_metadata=meta, output=out)
+    assert store.scheme is not None
