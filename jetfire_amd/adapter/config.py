@@ -37,6 +37,7 @@ class JetFireConfig:
     use_custom_backend: bool = True
     cpu_correction: bool = True
     shadow_enabled: bool = True
+    skip_native_kv: bool = True         # the serving engine keeps no KV cache of its own (JETFIRE_SKIP_NATIVE_KV)
     max_batch_size: int = 0
     cpu_attn_threads: int = 0          # 0: the pool's default (all cores but two)
     debug_log: bool = False
@@ -58,6 +59,7 @@ def _from_env() -> JetFireConfig:
         use_custom_backend=os.environ.get("JETFIRE_USE_CUSTOM_BACKEND", "1") == "1",
         cpu_correction=os.environ.get("JETFIRE_CPU_CORRECTION", "1") == "1",
         shadow_enabled=os.environ.get("JETFIRE_SHADOW", "1") == "1",
+        skip_native_kv=os.environ.get("JETFIRE_SKIP_NATIVE_KV", "1") == "1",
         max_batch_size=int(os.environ.get("JETFIRE_MAX_BATCH_SIZE", 0)),
         cpu_attn_threads=int(os.environ.get("JETFIRE_CPU_ATTN_THREADS", 0)),
         debug_log=os.environ.get("JETFIRE_DEBUG", "0") == "1",

@@ -1,0 +1,52 @@
+"""Attention-backend shim (`jetfire_vllm/adapter/jetfire_backend.py:135-209`): the two methods a serving
+engine's attention implementation calls per layer, `do_kv_cache_update` (append: quantise-on-write + shadow mirror)
+and `forward` (decode through `try_jetfire_decode`, anything else through the engine's own implementation).
+
+The reference derives its class from vLLM's FlashAttentionImpl; here the engine's implementation class is a
+parameter, so the shim does not import a serving engine: `make_jetfire_attention_impl(FlashAttentionImpl)` gives
+the drop-in class.  Prefill attention is the engine's own (outside this library's decode path)."""
+from __future__ import annotations
+
+from .config import get_jetfire_config
+from .decode_path import try_jetfire_decode
+from .kv_pool import get_global_kv_pool_manager
+
+_FALLBACK_HELP = (
+    "JetFire decode fell back to the native attention, but with JETFIRE_SKIP_NATIVE_KV=1 the engine keeps no KV "
+    "cache of its own, so the fall-back would produce garbage.\nRecent decode_fallbacks: {fallbacks}\n"
+    "Common causes:\n"
+    "  - seq_len_too_short: empty sequence or unsupported JETFIRE_TOPK (use a positive supported correction width)\n"
+    "  - cpu_correction_disabled: set JETFIRE_CPU_CORRECTION=1 (default) or JETFIRE_SKIP_NATIVE_KV=0\n"
+    "  - store_missing: the layer is not mirrored (JETFIRE_LAYER_STRIDE must be 1 when skip_native_kv=1)")
+
+
+def make_jetfire_attention_impl(native_impl_cls):
+    """Subclass of the engine's attention implementation with JetFire's append and decode."""
+
+    class JetFireAttentionImpl(native_impl_cls):
+        def forward(self, layer, query, key, value, kv_cache, attn_metadata, output=None, output_scale=None,
+                    output_block_scale=None):
+            if output is not None:
+                done = try_jetfire_decode(impl=self, layer=layer, query=query, key=key, value=value,
+                                          attn_metadata=attn_metadata, output=output)
+                if done is not None:
+                    return done
+            kind = getattr(getattr(self, "attn_type", None), "name", "DECODER")
+            decode_step = attn_metadata is not None and int(getattr(attn_metadata, "max_query_len", 1)) == 1
+            if get_jetfire_config().skip_native_kv and decode_step and kind == "DECODER":
+                # (the profiling pass, attn_metadata None, may fall through: its output is discarded; so may
+                # prefill, which attends over the tokens it is handed)
+                raise RuntimeError(_FALLBACK_HELP.format(fallbacks=get_global_kv_pool_manager().decode_fallbacks))
+            return super().forward(layer, query, key, value, kv_cache, attn_metadata, output=output,
+                                   output_scale=output_scale, output_block_scale=output_block_scale)
+
+        def do_kv_cache_update(self, layer, key, value, kv_cache, slot_mapping) -> None:
+            pool = get_global_kv_pool_manager()
+            name = getattr(layer, "layer_name", "unknown_layer")
+            pool.ensure_layer_config_from_layer(name, layer)
+            pool.mirror_kv(layer_name=name, key=key, value=value, slot_mapping=slot_mapping)
+            if not get_jetfire_config().skip_native_kv:
+                super().do_kv_cache_update(layer, key, value, kv_cache, slot_mapping)
+
+    JetFireAttentionImpl.__qualname__ = f"JetFireAttentionImpl[{native_impl_cls.__name__}]"
+    return JetFireAttentionImpl

@@ -19,7 +19,7 @@ def adapter():
     decode_path.reset_jetfire_decode_runtime_state()
     A.reset_global_kv_pool_manager()
     A.set_jetfire_config(scheme="SymInt3K_SymInt2V", group_size=64, topk=256, use_custom_backend=True,
-                         cpu_correction=True, layer_stride=1)
+                         cpu_correction=True, layer_stride=1, skip_native_kv=True)
 
 
 def test_select_top_k_matches_the_reference_table(adapter):
@@ -589,3 +589,93 @@ def test_release_policy_selects_the_named_split_kernels(adapter, monkeypatch, sc
     with pytest.raises(release_policy.ReleasePolicyError, match="JETFIRE_USE_FUSED_ATTN_TOPK"):
         adapter.try_jetfire_decode(impl=impl, layer=layer, query=q, attn_metadata=meta, output=out)
     assert store.scheme is not None
+
+
+class _NativeImpl:
+    """Stand-in for the serving engine's attention implementation: records what reaches it."""
+
+    def __init__(self):
+        self.attn_type = types.SimpleNamespace(name="DECODER")
+        self.scale = 128 ** -0.5
+        self.native_forward = 0
+        self.native_updates = 0
+
+    def forward(self, layer, query, key, value, kv_cache, attn_metadata, output=None, output_scale=None,
+                output_block_scale=None):
+        self.native_forward += 1
+        return "native"
+
+    def do_kv_cache_update(self, layer, key, value, kv_cache, slot_mapping):
+        self.native_updates += 1
+
+
+def test_backend_shim_routes_appends_and_fallbacks(adapter):
+    """`jetfire_backend.py:135-209`: appends always reach the pool (and the engine's own cache only when it keeps
+    one); a decode miss with no native cache raises with the recorded reasons; the profiling pass and prefill
+    fall through to the engine's implementation."""
+    from jetfire_amd.adapter.jetfire_backend import make_jetfire_attention_impl
+    Impl = make_jetfire_attention_impl(_NativeImpl)
+    impl = Impl()
+    layer = types.SimpleNamespace(layer_name="model.layers.0.attn", num_heads=8, num_kv_heads=2, head_size=128)
+    pool = adapter.get_global_kv_pool_manager()
+    pool.register_layer_layout(layer.layer_name, num_blocks=2, block_size=16)
+    k = torch.zeros(3, 2, 128, dtype=torch.bfloat16)
+    seen = []
+    pool.mirror_kv = lambda **kw: seen.append(sorted(kw))
+    adapter.set_jetfire_config(skip_native_kv=True)
+    impl.do_kv_cache_update(layer, k, k, None, torch.arange(3))
+    assert seen == [["key", "layer_name", "slot_mapping", "value"]] and impl.native_updates == 0
+    assert pool.get_layer_config(layer.layer_name) == adapter.JetFireLayerConfig(8, 2, 128)
+    adapter.set_jetfire_config(skip_native_kv=False)
+    impl.do_kv_cache_update(layer, k, k, None, torch.arange(3))
+    assert len(seen) == 2 and impl.native_updates == 1
+    q = torch.zeros(2, 8, 128, dtype=torch.bfloat16)
+    out = torch.zeros(2, 8 * 128, dtype=torch.bfloat16)
+    meta = _meta(torch.tensor([5, 7], dtype=torch.int32), torch.zeros(2, 1, dtype=torch.int64))
+    assert impl.forward(layer, q, None, None, None, meta, output=out) == "native"        # store missing, native cache kept
+    assert pool.decode_fallbacks.get("store_missing") == 1
+    adapter.set_jetfire_config(skip_native_kv=True)
+    with pytest.raises(RuntimeError, match="store_missing"):
+        impl.forward(layer, q, None, None, None, meta, output=out)
+    assert impl.forward(layer, q, None, None, None, None, output=out) == "native"        # profiling pass
+    prefill = _meta(meta.seq_lens, meta.block_table, max_query_len=4)
+    assert impl.forward(layer, q, None, None, None, prefill, output=out) == "native"     # prefill is the engine's
+    assert impl.native_forward == 3
+
+
+@pytest.mark.gpu
+def test_backend_shim_appends_and_decodes_on_the_gpu(adapter):
+    from jetfire_amd.adapter.jetfire_backend import make_jetfire_attention_impl
+    B, Hq, Hkv, D, bs, K, max_S = 2, 8, 2, 128, 16, 32, 128
+    adapter.set_jetfire_config(scheme="SymInt3K_SymInt2V", group_size=64, topk=K, layer_stride=1, cpu_attn_threads=2,
+                               skip_native_kv=True)
+    adapter.reset_global_kv_pool_manager()
+    pool = adapter.get_global_kv_pool_manager()
+    impl = make_jetfire_attention_impl(_NativeImpl)()
+    layer = types.SimpleNamespace(layer_name="model.layers.0.self_attn.attn", num_heads=Hq, num_kv_heads=Hkv, head_size=D)
+    per_seq = max_S // bs
+    pool.register_layer_layout(layer.layer_name, num_blocks=B * per_seq, block_size=bs)
+    rng = np.random.default_rng(13)
+    lens = [90, 47]
+    bt = np.arange(B * per_seq, dtype=np.int64).reshape(B, per_seq)
+    slots = np.concatenate([bt[b, np.arange(lens[b]) // bs] * bs + np.arange(lens[b]) % bs for b in range(B)])
+    n = len(slots)
+    k_np = O.bf16_round(rng.standard_normal((n, Hkv, D)).astype(np.float32))
+    v_np = O.bf16_round(rng.standard_normal((n, Hkv, D)).astype(np.float32))
+    impl.do_kv_cache_update(layer, bf16_tensor(k_np).cuda(), bf16_tensor(v_np).cuda(), None, torch.from_numpy(slots).cuda())
+    q_np = O.bf16_round((rng.standard_normal((B, Hq, D)) / np.sqrt(D)).astype(np.float32))
+    out = torch.zeros(B, Hq * D, dtype=torch.bfloat16, device="cuda")
+    meta = _meta(torch.tensor(lens, dtype=torch.int32, device="cuda"), torch.from_numpy(bt).cuda(), max_seq_len=max(lens))
+    got = impl.forward(layer, bf16_tensor(q_np).cuda(), None, None, None, meta, output=out)
+    torch.cuda.synchronize()
+    assert got is out and impl.native_forward == 0 and pool.decode_hits == 1
+    Kfull = np.zeros((Hkv, B * max_S, D), np.float32)
+    Vfull = np.zeros((Hkv, B * max_S, D), np.float32)
+    Kfull[:, slots] = k_np.transpose(1, 0, 2)
+    Vfull[:, slots] = v_np.transpose(1, 0, 2)
+    kd, ks = O.quantize_and_pack(Kfull, 64, 3)
+    vd, vs = O.quantize_and_pack(Vfull, 64, 2)
+    r = O.decode_reference(q_np, kd, ks, vd, vs, bt, np.array(lens, np.int32), max(lens), Hq, Hkv, bs, D ** -0.5, K, "k3v2",
+                           Kfull, Vfull)
+    res = bf16_to_f32(out).reshape(B, Hq, D)
+    np.testing.assert_allclose(res, r["out"], atol=6e-3, rtol=1.5e-2)
