@@ -30,6 +30,7 @@
 // pre-correction terms o_old_unnorm, W over the winners (jetfire_vllm/csrc/int2_softmax_v.cu:738-788).
 #include "common.h"
 
+#include <atomic>
 #include <mutex>
 #include <vector>
 
@@ -1757,11 +1758,28 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
 struct ScanProfile {
   std::vector<hipEvent_t> ev;
   int used = 0;
-  bool armed = false;
+  std::atomic<bool> armed{false};
 };
+// Process-wide measurement / test switches, reachable from the public debug entry points: the event list has its
+// own lock, the two scalars are atomics (a launch reads each once).
 ScanProfile g_prof;
-long long* g_phase_clock = nullptr;
-int g_force_split_len = 0;  // test / measurement aid: overrides the planner's split length when positive
+std::mutex g_prof_mu;
+std::atomic<long long*> g_phase_clock{nullptr};
+std::atomic<int> g_force_split_len{0};  // test / measurement aid: overrides the planner's split length when positive
+
+// Compute units of the current device (the planner balances workgroups over them); 256, the MI355X count, when
+// no device can be asked (planning on a host without a GPU).
+int device_cus() {
+  static const int cus = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+      return n;
+    (void)hipGetLastError();
+    return 256;
+  }();
+  return cus;
+}
 
 constexpr size_t LDS_BUDGET_2WG = 80 * 1024 - 512;    // two workgroups per CU (160 KB LDS)
 constexpr size_t LDS_BUDGET_1WG = 160 * 1024 - 1024;
@@ -1841,7 +1859,7 @@ inline void fused_plan(int scheme, int NG, int B, int H_q, int H_kv, int max_S, 
   // merge costs a fixed part per launch plus a part proportional to the candidates one workgroup visits.
   const int lmax = lmax_dispatch(scheme, G, NG);
   const int nw = (G <= 4) ? 16 : 8;
-  constexpr int kCUs = 256;
+  const int kCUs = device_cus();
   constexpr double kScanFixed = 8.5;
   // one chunk per wavefront, all wavefronts; the mixed schemes are priced like the wider one
   const double per_chunk = (scheme == JF_SCHEME_K3V2) ? 5.9 : 6.6;
@@ -1864,8 +1882,8 @@ inline void fused_plan(int scheme, int NG, int B, int H_q, int H_kv, int max_S, 
     }
     if (cand >= max_S) break;
   }
-  if (g_force_split_len > 0) {
-    L = (g_force_split_len + 255) / 256 * 256;
+  if (const int forced = g_force_split_len.load(std::memory_order_relaxed); forced > 0) {
+    L = (forced + 255) / 256 * 256;
     if (L > lmax) L = lmax;
     while ((max_S + L - 1) / L > MG_MAX_SPLITS && L < lmax) L += 256;
   }
@@ -1905,12 +1923,23 @@ template <int SCHEME, int G, int NG>
 int launch_scan(const FusedParams& p, hipStream_t st) {
   const size_t smem = ScanLds<SCHEME, G, NG>::total(p.L);
   auto kern = fused_scan_kernel<SCHEME, G, NG>;
-  static size_t attr_smem = 0;  // per instantiation: raise the dynamic-LDS limit only when it grows
-  if (smem > attr_smem) {
-    JF_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    attr_smem = smem;
+  // per instantiation: raise the dynamic-LDS limit only when it grows (launches may come from several threads)
+  static std::mutex attr_mu;
+  static size_t attr_smem = 0;
+  {
+    std::lock_guard<std::mutex> lock(attr_mu);
+    if (smem > attr_smem) {
+      JF_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+      attr_smem = smem;
+    }
   }
-  const bool prof = g_prof.armed && g_prof.used + 2 <= (int)g_prof.ev.size();
+  std::unique_lock<std::mutex> plock(g_prof_mu, std::defer_lock);
+  bool prof = false;
+  if (g_prof.armed) {  // (read without the lock: arming happens-before the launches a benchmark times)
+    plock.lock();
+    prof = g_prof.armed && g_prof.used + 2 <= (int)g_prof.ev.size();
+    if (!prof) plock.unlock();
+  }
   if (prof) JF_CHECK_HIP(hipEventRecord(g_prof.ev[g_prof.used], st));
   hipLaunchKernelGGL(kern, dim3(p.n_splits, p.H_kv, p.B), dim3(ScanLds<SCHEME, G, NG>::NT), smem, st, p);
   JF_CHECK_LAUNCH();
@@ -2014,7 +2043,7 @@ static int fused_scan_run(int scheme, int group_size, const uint16_t* q, const u
   p.cnt2 = reinterpret_cast<int32_t*>(ws + wl.off_cnt2);
   p.topk_idx = topk_idx; p.topk_slots = topk_slots; p.o_hat = o_hat; p.o_old = o_old_unnorm; p.W = W;
   p.softmax_m = softmax_m; p.softmax_inv_z = softmax_inv_z;
-  p.phase_clock = g_phase_clock;
+  p.phase_clock = g_phase_clock.load(std::memory_order_relaxed);
   hipStream_t st = (hipStream_t)stream;
   int rc = JF_OK;
 #define JF_FUSED_CASE(SCH, GG, NGG) rc = launch_scan<SCH, GG, NGG>(p, st)
@@ -2148,6 +2177,7 @@ extern "C" int jf_fused_scan_topk_static(int scheme, int group_size, const uint1
 
 extern "C" int jf_profile_scan_begin(int max_launches) {
   JF_CHECK_ARG(max_launches > 0 && max_launches <= (1 << 20), "profile_scan_begin: bad max_launches=%d", max_launches);
+  std::lock_guard<std::mutex> lock(g_prof_mu);
   for (hipEvent_t e : g_prof.ev) (void)hipEventDestroy(e);
   g_prof.ev.assign((size_t)max_launches * 2, nullptr);
   for (auto& e : g_prof.ev) JF_CHECK_HIP(hipEventCreate(&e));
@@ -2158,6 +2188,7 @@ extern "C" int jf_profile_scan_begin(int max_launches) {
 
 extern "C" int jf_profile_scan_end(double* total_ms, int* launches) {
   JF_CHECK_ARG(total_ms && launches, "profile_scan_end: null output");
+  std::lock_guard<std::mutex> lock(g_prof_mu);
   g_prof.armed = false;
   double tot = 0.0;
   for (int i = 0; i + 1 < g_prof.used; i += 2) {
@@ -2175,12 +2206,12 @@ extern "C" int jf_profile_scan_end(double* total_ms, int* launches) {
 }
 
 extern "C" int jf_debug_phase_clock(void* device_buffer) {
-  g_phase_clock = reinterpret_cast<long long*>(device_buffer);
+  g_phase_clock.store(reinterpret_cast<long long*>(device_buffer));
   return JF_OK;
 }
 
 extern "C" int jf_debug_split_len(int split_len) {
   JF_CHECK_ARG(split_len >= 0, "debug_split_len: negative length");
-  g_force_split_len = split_len;
+  g_force_split_len.store(split_len);
   return JF_OK;
 }
