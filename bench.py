@@ -60,6 +60,31 @@ def cpu_baseline(w, target_s: float = 10.0, budget_s: float = 25.0):
     }
 
 
+def cpu_baseline_c1(target_s: float = 4.0):
+    """The whole of configuration C1 (B1, 32 query / 8 kv heads, 4096 positions, K4V4, top-k 64: the reference's own
+    CPU-runnable case) through the torch CPU path: median seconds per layer pass."""
+    import torch
+    from jetfire_amd import workloads
+    from oracle import torch_cpu_path as T
+    w = workloads.build("c1")
+    lay = w.layers[0]
+    kd, ks = lay.k_data.cpu().unsqueeze(0), lay.k_scales.cpu().unsqueeze(0)
+    vd, vs = lay.v_data.cpu().unsqueeze(0), lay.v_scales.cpu().unsqueeze(0)
+    q = w.q.cpu()
+    T.decode_path(q, kd, ks, vd, vs, w.group, 4, 4, w.top_k)
+    times = []
+    t_start = time.perf_counter()
+    while len(times) < 5 or time.perf_counter() - t_start < target_s:
+        t0 = time.perf_counter()
+        T.decode_path(q, kd, ks, vd, vs, w.group, 4, 4, w.top_k)
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    return {"workload": "c1: B1 Hq32 Hkv8 S4096 k4v4 g128 top_k64, one layer, whole configuration",
+            "value": round(w.packed_bytes_per_layer / med / 1e9, 4), "unit": "GB/s", "ms_per_layer": round(med * 1e3, 3),
+            "runs": len(times), "cores": torch.get_num_threads()}
+
+
 def _median_ms(fn, sync, n=10, warm=2):
     import time
     ts = []
@@ -172,13 +197,121 @@ def component_pcie(args):
     return out
 
 
+def component_split(args):
+    """The split-form operators (one per reference kernel: Stage A scores + top-k, Stage B) at the workload's
+    shape, a few layers, eagerly: wall time per layer, and a launch sequence for a kernel trace."""
+    import torch
+    from jetfire_amd import ops, workloads
+    w = workloads.build(args.workload, n_layers=args.layers or 4)
+    sync = torch.cuda.synchronize
+
+    def layer(lay):
+        if w.scheme == "k3v2":
+            scores, idx, slots = ops.int3_qk_scores_topk(w.q, lay.k_data, lay.k_scales, w.block_table, w.seq_lens, w.S, w.H_q,
+                                                         w.H_kv, 16, w.attn_scale, w.top_k)
+            return ops.int2_softmax_v_with_pre_corr_wvs2(scores, lay.v_data, lay.v_scales, w.block_table, w.seq_lens, idx,
+                                                         w.S, w.H_q, w.H_kv, 16, w.top_k)
+        scores, idx, slots, m, iz = ops.int8tc_qk_scores_topk_stats(w.q, lay.k_data, lay.k_scales, w.block_table, w.seq_lens,
+                                                                    w.S, w.H_q, w.H_kv, 16, w.attn_scale, w.top_k)
+        fn = ops.int8tc_softmax_v_with_pre_corr_reg_stats if w.B > 1 else None
+        if fn is not None:
+            return fn(scores, m, iz, lay.v_data, lay.v_scales, w.block_table, w.seq_lens, idx, w.S, w.H_q, w.H_kv, 16, w.top_k)
+        return ops.int4_softmax_v_with_pre_corr_wvs2_scores(scores, lay.v_data, lay.v_scales, w.block_table, w.seq_lens, idx,
+                                                            w.S, w.H_q, w.H_kv, 16, w.top_k)
+
+    def step():
+        for lay in w.layers:
+            layer(lay)
+    ms = _median_ms(step, sync, n=5, warm=2)
+    return {"component": "split", "workload": args.workload, "layers": len(w.layers),
+            "us_per_layer": round(ms * 1e3 / len(w.layers), 1),
+            "packed_GBps": round(w.packed_bytes_per_layer * len(w.layers) / ms / 1e6, 1)}
+
+
+def measure_gpu_path(name: str, steps: int, warmup: int, lib):
+    """One more workload inside the same run: the GPU path (scan + merge + blend per layer, replayed from a HIP
+    graph) timed like the main one, the scan kernel timed with HIP events in a separate eager pass."""
+    import torch
+    from jetfire_amd import _lib, ops, workloads
+    w = workloads.build(name)
+    n_layers = len(w.layers)
+    o_new = torch.zeros(w.B, w.H_q, 128, dtype=torch.bfloat16, device="cuda")
+    out = torch.empty_like(o_new)
+
+    def step():
+        for lay in w.layers:
+            o_hat, slots, o_old, W, idx = ops.fused_attn_topk(w.scheme, w.q, lay.k_data, lay.k_scales, lay.v_data, lay.v_scales,
+                                                              w.block_table, w.seq_lens, w.S, w.H_q, w.H_kv, 16, w.top_k,
+                                                              w.attn_scale)
+            ops.blend_unnorm_into(o_hat, o_old, W, o_new, out)
+    for _ in range(max(1, warmup)):
+        step()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        step()
+    torch.cuda.current_stream().wait_stream(s)
+    with torch.cuda.graph(graph, stream=s):
+        step()
+    graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        graph.replay()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) / steps * 1e3
+    total_ms, launches = ctypes.c_double(0.0), ctypes.c_int(0)
+    _lib.check(lib.jf_profile_scan_begin(n_layers * 3))
+    for _ in range(3):
+        step()
+    torch.cuda.synchronize()
+    _lib.check(lib.jf_profile_scan_end(ctypes.byref(total_ms), ctypes.byref(launches)))
+    scan_us = total_ms.value / max(1, launches.value) * 1e3
+    achieved = w.packed_bytes_per_layer / (scan_us * 1e-6) / 1e9
+    rec = {"workload": f"{name}: B{w.B} Hq{w.H_q} Hkv{w.H_kv} D128 S{w.S} {w.scheme} g{w.group} top_k{w.top_k} x{n_layers} layers",
+           "packed_bytes_per_layer": w.packed_bytes_per_layer, "steps": steps, "ms_per_step": round(ms_per_step, 4),
+           "us_per_layer": round(ms_per_step * 1e3 / n_layers, 2),
+           "value": round(w.packed_bytes_per_layer * n_layers / (ms_per_step * 1e-3) / 1e9, 2), "unit": "GB/s",
+           "roofline": {"bound": "hbm", "kernel": "fused_scan_kernel", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS,
+                        "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "kernel_us": round(scan_us, 2),
+                        "launches_timed": launches.value, **profile_counters(w.scheme, name)}}
+    del graph, w
+    torch.cuda.empty_cache()
+    return rec
+
+
+def profile_counters(scheme: str, workload: str):
+    """Counter-derived figures of the scan kernel for this workload, from the committed rocprofv3 summaries (they
+    cannot be collected from inside a benchmark process): HBM traffic per launch, MFMA and VALU busy shares."""
+    out = {"traffic": None}
+    tpath = os.path.join(ROOT, "profiles", f"fused_scan_{scheme}_{workload}_traffic.json")
+    cpath = os.path.join(ROOT, "profiles", f"decode_kernels_{workload}_sq_counters.json")
+    try:
+        out["traffic"] = json.load(open(tpath)).get("traffic_bytes_per_launch")
+        out["traffic_source"] = os.path.relpath(tpath, ROOT)
+    except Exception:
+        pass
+    try:
+        c = json.load(open(cpath))["fused_scan_kernel"]
+        out["mfma_busy_pct"] = c.get("mfma_busy_pct")
+        out["valu_issue_pct"] = c.get("valu_issue_pct")
+        out["counters_source"] = os.path.relpath(cpath, ROOT)
+    except Exception:
+        pass
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4", "c5"],
-                    help="c2: Llama-3.1-8B B4 S32768 K3V2 k256 x32 layers (the headline); c3: B1 S131072 K4V4 k512; "
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c2k4", "c3", "c4", "c5"],
+                    help="c1: B1 S4096 K4V4 k64, one layer (the reference's CPU-runnable case); "
+                         "c2: Llama-3.1-8B B4 S32768 K3V2 k256 x32 layers (the headline); c2k4: the c2 shape with K4V4; "
+                         "c3: B1 S131072 K4V4 k512; "
                          "c4: Qwen3-30B-A3B B4 GQA8 K3V2 x48; c5: Llama-3.3-70B TP2 shard B2 S65536 K3V2 x80")
     ap.add_argument("--layers", type=int, default=None, help="override the number of distinct layer caches")
     ap.add_argument("--paged", action="store_true", help="random block table instead of the identity mapping")
@@ -200,7 +333,12 @@ def main() -> int:
                          "manager, cache stores, dispatcher gate) instead of calling the operators directly")
     ap.add_argument("--split-len", type=int, default=0,
                     help="measurement aid: force the fused scan's split length (0 = the library's planner)")
-    ap.add_argument("--component", default=None, choices=["append", "cpu-correction", "pcie"],
+    ap.add_argument("--no-extras", action="store_true",
+                    help="default run only: skip the K4V4 records (c2k4 and c3, a few layers fewer would not change them) "
+                         "that the c2 line carries besides its own figures")
+    ap.add_argument("--calibrate-read", action="store_true",
+                    help="stream 1 GiB with a kernel that only reads (10 times) and exit: the read-stream ceiling")
+    ap.add_argument("--component", default=None, choices=["append", "cpu-correction", "pcie", "split"],
                     help="time one component of the path at the workload's geometry, print its own JSON line and exit: "
                          "append = quantise-on-write + shadow mirror of a prefill chunk (--tokens); cpu-correction = the "
                          "CPU pool alone on freshly drawn random slots; pcie = pinned copy latency by size")
@@ -235,9 +373,25 @@ def main() -> int:
         print(json.dumps({"calibrate_copy_bytes_read": 1 << 30, "calibrate_copy_bytes_written": 1 << 30, "launches": 11,
                           "us_per_copy": round(us, 1), "copy_read_plus_write_GBps": round(2 * (1 << 30) / us / 1e3, 1)}))
         return 0
+    if args.calibrate_read:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").random_(0, 255)
+        sink = torch.zeros(4, dtype=torch.uint8, device="cuda")
+        st = torch.cuda.current_stream().cuda_stream
+        _lib.check(lib.jf_calibrate_stream_read(src.data_ptr(), src.numel(), sink.data_ptr(), st))
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(10):
+            _lib.check(lib.jf_calibrate_stream_read(src.data_ptr(), src.numel(), sink.data_ptr(), st))
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 100.0
+        print(json.dumps({"calibrate_read_bytes": 1 << 30, "launches": 11, "us_per_pass": round(us, 1),
+                          "read_GBps": round((1 << 30) / us / 1e3, 1), "frac_of_8TBps": round((1 << 30) / us / 1e3 / HBM_PEAK_GBPS, 4)}))
+        return 0
     if args.component is not None:
         print(json.dumps({"append": component_append, "cpu-correction": component_cpu_correction,
-                          "pcie": component_pcie}[args.component](args)))
+                          "pcie": component_pcie, "split": component_split}[args.component](args)))
         return 0
     if args.split_len:
         _lib.check(lib.jf_debug_split_len(args.split_len))
@@ -357,13 +511,7 @@ def main() -> int:
     value = bytes_layer * n_layers / (ms_per_step * 1e-3) / 1e9
     scan_us = total_ms.value / max(1, launches.value) * 1e3
     achieved = bytes_layer / (scan_us * 1e-6) / 1e9 if scan_us > 0 else 0.0
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", f"fused_scan_{w.scheme}_{args.workload}_traffic.json")
-    if os.path.exists(tpath):
-        try:
-            traffic = json.load(open(tpath)).get("traffic_bytes_per_launch")
-        except Exception:
-            traffic = None
+    counters = profile_counters(w.scheme, args.workload)
 
     res = {
         "metric": "decode-scan HBM GB/s on packed KV (fused scan + top-k + merge, all layers of one decode step)",
@@ -381,13 +529,22 @@ def main() -> int:
                                + (" (device-side wait, whole step in one graph)" if args.graph else " (host-blocking wait)")
                                if handoff else "not in the timed region (GPU path only)")},
         "roofline": {"bound": "hbm", "kernel": "fused_scan_kernel", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
-                     "kernel_us": round(scan_us, 2), "launches_timed": launches.value},
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "kernel_us": round(scan_us, 2),
+                     "launches_timed": launches.value, **counters},
     }
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(w)
+        res["cpu_baseline"]["c1"] = cpu_baseline_c1()
     for h in ctxs:
         h.close()
+    default_run = (args.workload == "c2" and not handoff and not args.no_extras and args.layers is None
+                   and not args.paged and not args.split_len and graph is not None)
+    if default_run:
+        # the metric is quoted for K3V2 and K4V4: the K4V4 figures of the same run
+        del graph
+        w.layers.clear()
+        torch.cuda.empty_cache()
+        res["k4v4"] = [measure_gpu_path(name, max(3, args.steps // 2), 1, lib) for name in ("c2k4", "c3")]
     print(json.dumps(res))
     return 0
 

@@ -230,6 +230,10 @@ int jf_fused_plan(int scheme, int group_size, int B, int H_q, int H_kv, int max_
  * launches); end synchronises them and returns the summed device time and the number of launches. */
 int jf_profile_scan_begin(int max_launches);
 int jf_profile_scan_end(double* total_ms, int* launches);
+/* Measurement aid with no counterpart in the reference: one kernel that streams `bytes` bytes from src with 16-byte
+ * loads and writes nothing (sink: 4 bytes of device memory, may be NULL).  Its rate is the read-stream ceiling of
+ * this machine, the figure the scan's achieved bandwidth is put beside. */
+int jf_calibrate_stream_read(const void* src, size_t bytes, void* sink, void* stream);
 /* Measurement aid: if device_buffer is non-NULL, every fused-scan workgroup stores ten int64 s_memtime
  * stamps of its phase boundaries at device_buffer[((b * H_kv + hkv) * n_splits + split) * 10 ...], and every
  * merge workgroup eight at device_buffer[B * H_kv * n_splits * 10 + (b * H_q + hq) * 8 ...] (which stamp

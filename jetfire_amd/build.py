@@ -24,6 +24,7 @@ SOURCES = (
     "softmax_v.hip",
     "fused_scan.hip",
     "blend.hip",
+    "calibrate.hip",
     "cpu_topk_attn.cpp",
 )
 

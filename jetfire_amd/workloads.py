@@ -17,6 +17,7 @@ BLOCK = 16
 CONFIGS = {
     "c1": (1, 32, 8, 4096, "k4v4", 128, 64, 1),
     "c2": (4, 32, 8, 32768, "k3v2", 64, 256, 32),
+    "c2k4": (4, 32, 8, 32768, "k4v4", 128, 256, 32),     # the c2 shape with INT4 keys and values (the metric's "K4V4 at 32k")
     "c3": (1, 32, 8, 131072, "k4v4", 128, 512, 32),
     "c4": (4, 32, 4, 32768, "k3v2", 64, 256, 48),
     "c5": (2, 32, 4, 65536, "k3v2", 64, 512, 80),

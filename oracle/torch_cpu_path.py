@@ -45,3 +45,29 @@ def decode_path(q, k_data, k_scales, v_data, v_scales, group_size: int, k_nbits:
     o_hat = torch.einsum("bhgs,bhsd->bhgd", probs, vhat).reshape(B, Hq, D)
     idx = scores.topk(min(top_k, scores.shape[-1]), dim=-1).indices.reshape(B, Hq, -1)
     return o_hat, idx
+
+
+def int8_q_scores(q: torch.Tensor, k_data: torch.Tensor, k_scales: torch.Tensor, attn_scale: float) -> torch.Tensor:
+    """The int8-quantised-query scoring model of the reference's INT4 Stage A
+    (jetfire_vllm/csrc/int8tc_qk_scores.cu:250-290 query quantisation, :435-469 rescale order), restated with torch
+    so that it can run on the GPU at full context lengths:
+        qs_kk = max(amax_{32 channels}|q| / 127, 1e-12), qi = clamp(rint(q * (1 / qs_kk)), -128, 127)
+        acc_kk = sum_{32} qi * (nibble - 8)                      exact integers
+        s = fma(acc_3, qs_3, fma(acc_2, qs_2, fma(acc_1, qs_1, acc_0 * qs_0)));  score = (s * k_scale) * attn_scale
+    q (G, 128) bf16 (the query heads of one kv-head), k_data (S, 64) uint8, k_scales (S,) or (S, 1) bf16 -> (G, S) fp32.
+    The query is quantised on the host (IEEE division); every fused multiply-add is evaluated in float64, where the
+    product is exact, and rounded once to fp32."""
+    dev = k_data.device
+    qf = q.detach().float().cpu().reshape(-1, 4, 32)
+    qs = torch.clamp(qf.abs().amax(-1) / 127.0, min=1e-12)                       # (G, 4) fp32
+    inv = 1.0 / qs
+    qi = torch.clamp(torch.round(qf * inv[..., None]), -128, 127)                # (G, 4, 32), round half to even
+    d = k_data.to(torch.int32)
+    codes = (torch.stack([(d >> 4) & 0xF, d & 0xF], dim=-1).reshape(d.shape[0], 4, 32) - 8).float()   # (S, 4, 32)
+    acc = torch.einsum("skd,gkd->gsk", codes, qi.to(dev))                        # integers below 2^24: exact in fp32
+    qs64 = qs.to(dev).double()
+    s = (acc[..., 0].double() * qs64[:, None, 0]).float()
+    for kk in range(1, 4):
+        s = (acc[..., kk].double() * qs64[:, None, kk] + s.double()).float()
+    ks = k_scales.reshape(-1).float()
+    return (s * ks[None, :]) * torch.tensor(attn_scale, dtype=torch.float32, device=dev)

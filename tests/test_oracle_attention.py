@@ -295,3 +295,22 @@ def test_torch_cpu_path_agrees_with_the_numpy_oracle(kbits, vbits, gs):
     p /= p.sum(-1, keepdims=True)
     want = np.einsum("hs,hsd->hd", p, vhat[np.arange(Hq) // (Hq // Hkv)][:, :S].astype(np.float64))
     np.testing.assert_allclose(o_hat[0].numpy(), want, atol=2e-5, rtol=1e-4)
+
+
+def test_torch_int8_q_restatement_is_bit_equal_to_the_oracle():
+    """oracle/torch_cpu_path.int8_q_scores (used on the GPU at full context lengths) against scores_int8_model."""
+    import torch
+    from oracle import torch_cpu_path as T
+    from tests.helpers import bf16_tensor, bits_to_bf16
+    B, Hq, Hkv, S = 2, 8, 2, 300
+    c = make_case(23, B, Hq, Hkv, S, 4, 4, 128, ragged=True)
+    ref = O.scores_int8_model(c["q"], c["kd"], c["ks"], c["bt"], c["lens"], S, Hq, Hkv, 16, 128 ** -0.5)
+    slots = O.slots_from_block_table(c["bt"], S, 16)
+    G = Hq // Hkv
+    for b in range(B):
+        n = int(c["lens"][b])
+        for h in range(Hkv):
+            sl = torch.from_numpy(slots[b, :n])
+            got = T.int8_q_scores(bf16_tensor(c["q"][b, h * G:(h + 1) * G]), torch.from_numpy(c["kd"][h])[sl],
+                                  bits_to_bf16(c["ks"][h])[sl], 128 ** -0.5).numpy()
+            assert np.array_equal(got.view(np.uint32), ref[b, h * G:(h + 1) * G, :n].view(np.uint32))
