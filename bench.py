@@ -240,10 +240,8 @@ def measure_gpu_path(name: str, steps: int, warmup: int, lib):
 
     def step():
         for lay in w.layers:
-            o_hat, slots, o_old, W, idx = ops.fused_attn_topk(w.scheme, w.q, lay.k_data, lay.k_scales, lay.v_data, lay.v_scales,
-                                                              w.block_table, w.seq_lens, w.S, w.H_q, w.H_kv, 16, w.top_k,
-                                                              w.attn_scale)
-            ops.blend_unnorm_into(o_hat, o_old, W, o_new, out)
+            ops.fused_attn_topk(w.scheme, w.q, lay.k_data, lay.k_scales, lay.v_data, lay.v_scales, w.block_table,
+                                w.seq_lens, w.S, w.H_q, w.H_kv, 16, w.top_k, w.attn_scale, blend=(o_new, out))
     for _ in range(max(1, warmup)):
         step()
     torch.cuda.synchronize()
@@ -333,6 +331,8 @@ def main() -> int:
                          "manager, cache stores, dispatcher gate) instead of calling the operators directly")
     ap.add_argument("--split-len", type=int, default=0,
                     help="measurement aid: force the fused scan's split length (0 = the library's planner)")
+    ap.add_argument("--separate-blend", action="store_true",
+                    help="GPU-only path: launch the blend as its own kernel instead of the merge kernel's epilogue")
     ap.add_argument("--no-extras", action="store_true",
                     help="default run only: skip the K4V4 records (c2k4 and c3, a few layers fewer would not change them) "
                          "that the c2 line carries besides its own figures")
@@ -452,7 +452,9 @@ def main() -> int:
         for li, lay in enumerate(w.layers):
             o_hat, slots, o_old, W, idx = ops.fused_attn_topk(
                 w.scheme, w.q, lay.k_data, lay.k_scales, lay.v_data, lay.v_scales, w.block_table, w.seq_lens,
-                w.S, w.H_q, w.H_kv, 16, w.top_k, w.attn_scale)
+                w.S, w.H_q, w.H_kv, 16, w.top_k, w.attn_scale, blend=None if (ctxs or args.separate_blend) else (o_new, out))
+            if not ctxs and not args.separate_blend:
+                continue            # the merge kernel has written `out` (o_new is known up front without a hand-off)
             if ctxs:
                 h = ctxs[li % len(ctxs)]
                 if args.graph:      # kernels only: the publish kernel, then a device-side wait that also blends

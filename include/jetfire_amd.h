@@ -198,6 +198,22 @@ int jf_fused_scan_topk(int scheme, int group_size,
                        float* softmax_m, float* softmax_inv_z, float* scores,
                        void* workspace, size_t workspace_bytes, void* stream);
 
+/* jf_fused_scan_topk followed by the blend of jf_blend_unnorm (jetfire_vllm/csrc/blend.cu:202-226) inside the
+ * merge kernel, for callers that hold the correction term already when the step is enqueued (a path without CPU
+ * correction passes zeros): out = bf16(fma(W, o_new, o_hat) - o_old_unnorm), o_new and out (B, H_q, 128) bf16.
+ * Every other output is written as by jf_fused_scan_topk; out is bit-equal to the separate blend. */
+int jf_fused_scan_topk_blend(int scheme, int group_size,
+                             const uint16_t* q, const uint8_t* k_data, const uint16_t* k_scales,
+                             const uint8_t* v_data, const uint16_t* v_scales,
+                             const int64_t* block_table, const int32_t* seq_lens,
+                             int B, int H_q, int H_kv, int max_S, int max_blocks, int64_t num_slots,
+                             int block_size, float attn_scale, int top_k,
+                             int64_t* topk_idx, int64_t* topk_slots,
+                             float* o_hat, float* o_old_unnorm, float* W,
+                             float* softmax_m, float* softmax_inv_z, float* scores,
+                             const uint16_t* o_new, uint16_t* out,
+                             void* workspace, size_t workspace_bytes, void* stream);
+
 /* jf_fused_scan_topk without the workspace arguments, for callers that cannot allocate device memory (code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in
  * the reference.  The workspace is a fixed array of JF_FUSED_STATIC_SCRATCH_BYTES in device memory that each

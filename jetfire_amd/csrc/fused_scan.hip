@@ -83,6 +83,9 @@ struct FusedParams {
   float* W;
   float* softmax_m;
   float* softmax_inv_z;
+  // optional merge epilogue: out = bf16(fma(W, o_new, o_hat) - o_old_unnorm), both (B, H_q, D) bf16
+  const uint16_t* blend_o_new;
+  uint16_t* blend_out;
   long long* phase_clock;  // optional: 10 s_memtime stamps per scan workgroup, 8 per merge workgroup (measurement aid)
 };
 
@@ -1311,6 +1314,8 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
     pl = p.part_l[bh * NS + tid];
   }
   if (tid < NL) my_cnt = cc[tid];
+  float blend_new = 0.f, blend_hat = 0.f;
+  if (!PARTIAL && p.blend_out && tid < D) blend_new = bf16_to_f32(p.blend_o_new[bh * D + tid]);
   // The first MG_REGK * MG_THREADS candidates live in registers: group g = r / 4 of a thread holds the four
   // consecutive candidates (g * MG_THREADS + tid) * 4 + (r % 4), fetched with one 16-byte load.  Candidate
   // order = (group, thread, element).  Slots past a list's count hold key 0 (written by the producer).
@@ -1409,7 +1414,8 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
       float o2 = red_sh[0][tid];
 #pragma unroll
       for (int q = 1; q < PO_GRP; ++q) o2 += red_sh[q][tid];  // fixed order
-      p.o_hat[bh * D + tid] = o2 * inv_z;
+      blend_hat = o2 * inv_z;
+      p.o_hat[bh * D + tid] = blend_hat;
     }
     if (tid == 0 && p.softmax_m) {
       p.softmax_m[bh] = M;
@@ -1743,12 +1749,12 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
 #pragma unroll
     for (int w = 0; w < MG_WAVES; ++w) o += old_sh[w][tid];  // fixed order
     p.o_old[bh * D + tid] = o;
-  }
-  if (tid == 0) {
-    float o = 0.f;
+    float wt = 0.f;
 #pragma unroll
-    for (int w = 0; w < MG_WAVES; ++w) o += w_sh[w];
-    p.W[bh] = o;
+    for (int w = 0; w < MG_WAVES; ++w) wt += w_sh[w];  // fixed order: the same value in every thread
+    if (tid == 0) p.W[bh] = wt;
+    // the blend of jetfire_vllm/csrc/blend.cu:202-226 for callers that hold o_new already
+    if (p.blend_out) p.blend_out[bh * D + tid] = f32_to_bf16(__builtin_fmaf(wt, blend_new, blend_hat) - o);
   }
   if (mclk && tid == 0) mclk[5] = clock64();
 }
@@ -1997,8 +2003,10 @@ static int fused_scan_run(int scheme, int group_size, const uint16_t* q, const u
                           int max_S, int max_blocks, int64_t num_slots, int block_size, float attn_scale,
                           int top_k, int64_t* topk_idx, int64_t* topk_slots, float* o_hat,
                           float* o_old_unnorm, float* W, float* softmax_m, float* softmax_inv_z, float* scores,
-                          void* workspace, size_t workspace_bytes, void* stream) {
+                          const uint16_t* blend_o_new, uint16_t* blend_out, void* workspace, size_t workspace_bytes,
+                          void* stream) {
   JF_CHECK_ARG(known_scheme(scheme), "fused_scan: unknown scheme %d", scheme);
+  JF_CHECK_ARG((blend_o_new == nullptr) == (blend_out == nullptr), "fused_scan: o_new and out go together");
   JF_CHECK_ARG(B >= 0 && H_q > 0 && H_kv > 0 && max_S >= 0 && H_q % H_kv == 0, "fused_scan: bad shape");
   const int G = H_q / H_kv;
   JF_CHECK_ARG(G == 1 || G == 2 || G == 4 || G == 8 || G == 16, "fused_scan: GQA group %d not in {1,2,4,8,16}", G);
@@ -2043,6 +2051,7 @@ static int fused_scan_run(int scheme, int group_size, const uint16_t* q, const u
   p.cnt2 = reinterpret_cast<int32_t*>(ws + wl.off_cnt2);
   p.topk_idx = topk_idx; p.topk_slots = topk_slots; p.o_hat = o_hat; p.o_old = o_old_unnorm; p.W = W;
   p.softmax_m = softmax_m; p.softmax_inv_z = softmax_inv_z;
+  p.blend_o_new = blend_o_new; p.blend_out = blend_out;
   p.phase_clock = g_phase_clock.load(std::memory_order_relaxed);
   hipStream_t st = (hipStream_t)stream;
   int rc = JF_OK;
@@ -2124,7 +2133,22 @@ extern "C" int jf_fused_scan_topk(int scheme, int group_size, const uint16_t* q,
                                   void* workspace, size_t workspace_bytes, void* stream) {
   return fused_scan_run(scheme, group_size, q, k_data, k_scales, v_data, v_scales, block_table, seq_lens, B, H_q, H_kv,
                         max_S, max_blocks, num_slots, block_size, attn_scale, top_k, topk_idx, topk_slots, o_hat,
-                        o_old_unnorm, W, softmax_m, softmax_inv_z, scores, workspace, workspace_bytes, stream);
+                        o_old_unnorm, W, softmax_m, softmax_inv_z, scores, nullptr, nullptr, workspace, workspace_bytes,
+                        stream);
+}
+
+extern "C" int jf_fused_scan_topk_blend(int scheme, int group_size, const uint16_t* q, const uint8_t* k_data,
+                                        const uint16_t* k_scales, const uint8_t* v_data, const uint16_t* v_scales,
+                                        const int64_t* block_table, const int32_t* seq_lens, int B, int H_q, int H_kv,
+                                        int max_S, int max_blocks, int64_t num_slots, int block_size, float attn_scale,
+                                        int top_k, int64_t* topk_idx, int64_t* topk_slots, float* o_hat,
+                                        float* o_old_unnorm, float* W, float* softmax_m, float* softmax_inv_z,
+                                        float* scores, const uint16_t* o_new, uint16_t* out, void* workspace,
+                                        size_t workspace_bytes, void* stream) {
+  JF_CHECK_ARG(B == 0 || (o_new && out), "fused_scan_blend: null o_new / out");
+  return fused_scan_run(scheme, group_size, q, k_data, k_scales, v_data, v_scales, block_table, seq_lens, B, H_q, H_kv,
+                        max_S, max_blocks, num_slots, block_size, attn_scale, top_k, topk_idx, topk_slots, o_hat,
+                        o_old_unnorm, W, softmax_m, softmax_inv_z, scores, o_new, out, workspace, workspace_bytes, stream);
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -2171,8 +2195,8 @@ extern "C" int jf_fused_scan_topk_static(int scheme, int group_size, const uint1
   }
   return fused_scan_run(scheme, group_size, q, k_data, k_scales, v_data, v_scales, block_table, seq_lens, B, H_q, H_kv,
                         max_S, max_blocks, num_slots, block_size, attn_scale, top_k, topk_idx, topk_slots, o_hat,
-                        o_old_unnorm, W, softmax_m, softmax_inv_z, scores, ws, (size_t)JF_FUSED_STATIC_SCRATCH_BYTES,
-                        stream);
+                        o_old_unnorm, W, softmax_m, softmax_inv_z, scores, nullptr, nullptr, ws,
+                        (size_t)JF_FUSED_STATIC_SCRATCH_BYTES, stream);
 }
 
 extern "C" int jf_profile_scan_begin(int max_launches) {

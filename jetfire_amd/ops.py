@@ -481,8 +481,12 @@ def int8tc_softmax_v_with_pre_corr_reg_stats(scores, softmax_m, softmax_inv_z, v
 
 def fused_attn_topk(scheme: str, q, k_data, k_scales, v_data, v_scales, block_table, seq_lens, max_S, H_q, H_kv,
                     block_size, top_k, attn_scale, group_size: Optional[int] = None, return_scores: bool = False,
-                    return_stats: bool = False):
+                    return_stats: bool = False, blend=None):
     """One fused pass: -> (o_hat, topk_slots, o_old_unnorm, W, topk_idx[, softmax_m, softmax_inv_z][, scores]).
+
+    blend=(o_new, out), both (B, H_q, 128) bf16 on the GPU: the merge kernel also writes
+    out = bf16(fma(W, o_new, o_hat) - o_old_unnorm), bit-equal to blend_unnorm_into (for callers that hold o_new
+    when the step is enqueued).
 
     The single-call contract is the one of the reference's int2_fused_attn_topk
     (jetfire_vllm/kernels/int2_fused_attn_topk.py:5-10) extended to INT3 / INT4 keys (INT4: the int8-Q scoring
@@ -515,11 +519,21 @@ def fused_attn_topk(scheme: str, q, k_data, k_scales, v_data, v_scales, block_ta
     scores = torch.empty((B, H_q, max_S), dtype=torch.float32, device=dev) if return_scores else None
     need = lib.jf_fused_workspace_bytes(scheme_id, B, H_q, H_kv, int(max_S), int(top_k))
     ws = _workspace(dev, need, "fused")
-    _lib.check(lib.jf_fused_scan_topk(
-        scheme_id, gs, q.data_ptr(), kd.data_ptr(), ks.data_ptr(), vd.data_ptr(), vs.data_ptr(), bt.data_ptr(),
-        sl.data_ptr(), B, H_q, H_kv, int(max_S), bt.size(1), kd.size(1), int(block_size), float(attn_scale), int(top_k),
-        idx.data_ptr(), slots.data_ptr(), o_hat.data_ptr(), o_old.data_ptr(), W.data_ptr(), _ptr(m), _ptr(iz),
-        _ptr(scores), ws.data_ptr(), ws.numel(), _stream(q)))
+    head = (scheme_id, gs, q.data_ptr(), kd.data_ptr(), ks.data_ptr(), vd.data_ptr(), vs.data_ptr(), bt.data_ptr(),
+            sl.data_ptr(), B, H_q, H_kv, int(max_S), bt.size(1), kd.size(1), int(block_size), float(attn_scale), int(top_k),
+            idx.data_ptr(), slots.data_ptr(), o_hat.data_ptr(), o_old.data_ptr(), W.data_ptr(), _ptr(m), _ptr(iz),
+            _ptr(scores))
+    if blend is None:
+        _lib.check(lib.jf_fused_scan_topk(*head, ws.data_ptr(), ws.numel(), _stream(q)))
+    else:
+        o_new, out = blend
+        _gpu(o_new, out)
+        _check(o_new.dtype == torch.bfloat16 and out.dtype == torch.bfloat16, "o_new / out must be bf16")
+        _check(tuple(o_new.shape) == (B, H_q, HEAD_DIM) and tuple(out.shape) == (B, H_q, HEAD_DIM),
+               "o_new / out must be (B, H_q, 128)")
+        _check(o_new.is_contiguous() and out.is_contiguous(), "o_new / out must be contiguous")
+        _lib.check(lib.jf_fused_scan_topk_blend(*head, o_new.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(),
+                                                _stream(q)))
     out = [o_hat, slots, o_old, W, idx]
     if return_stats:
         out += [m, iz]

@@ -153,6 +153,39 @@ def test_fused_scan_is_deterministic_and_matches_split_path():
     np.testing.assert_allclose(a[0].cpu().numpy(), o_hat.cpu().numpy(), atol=3e-6, rtol=2e-5)
 
 
+@pytest.mark.parametrize("scheme,B,Hq,Hkv,S,lens,K,split_len", [
+    ("k3v2", 2, 32, 8, 2048, None, 256, 0),
+    ("k4v4", 3, 32, 4, 512, [0, 257, 512], 256, 0),       # a zero-length row: out = bf16(0 + 0 * o_new - 0)
+    ("k4v4", 1, 8, 2, 10000, [9000], 512, 768),           # two-stage merge: the epilogue runs in the final stage only
+])
+def test_fused_blend_epilogue_equals_the_separate_blend(scheme, B, Hq, Hkv, S, lens, K, split_len):
+    """jf_fused_scan_topk_blend: the merge kernel's `out` is bit-equal to jf_blend_unnorm on its other outputs,
+    and those are what jf_fused_scan_topk writes."""
+    from jetfire_amd import _lib
+    kb, vb, gs = {"k3v2": (3, 2, 64), "k4v4": (4, 4, 128)}[scheme]
+    c = make_case(91 + S, B, Hq, Hkv, S, kb, vb, gs, lens=lens, extra_blocks=2)
+    d = to_device(c)
+    o = ops()
+    g = torch.Generator(device="cuda").manual_seed(5)
+    o_new = torch.randn(B, Hq, 128, generator=g, device="cuda").to(torch.bfloat16)
+    out = torch.full_like(o_new, 7.0)
+    lib = _lib.load()
+    _lib.check(lib.jf_debug_split_len(split_len))
+    try:
+        plain = o.fused_attn_topk(scheme, d["q"], d["kd"], d["ks"], d["vd"], d["vs"], d["bt"], d["lens"], S, Hq, Hkv, 16, K, SCALE)
+        fused = o.fused_attn_topk(scheme, d["q"], d["kd"], d["ks"], d["vd"], d["vs"], d["bt"], d["lens"], S, Hq, Hkv, 16, K, SCALE,
+                                  blend=(o_new, out))
+    finally:
+        _lib.check(lib.jf_debug_split_len(0))
+    for x, y in zip(plain, fused):
+        assert torch.equal(x, y)
+    ref = o.blend_unnorm(fused[0], fused[2], fused[3], o_new)
+    assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
+    with pytest.raises(RuntimeError, match="bf16"):
+        o.fused_attn_topk(scheme, d["q"], d["kd"], d["ks"], d["vd"], d["vs"], d["bt"], d["lens"], S, Hq, Hkv, 16, K, SCALE,
+                          blend=(o_new.float(), out))
+
+
 @pytest.mark.parametrize("scheme,B,Hq,Hkv,S,lens,K", [
     ("k3v2", 2, 32, 8, 1024, None, 256),
     ("k4v4", 2, 32, 8, 1024, None, 256),
