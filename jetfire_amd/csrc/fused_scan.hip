@@ -115,7 +115,7 @@ struct QInt8F {
 //   sbase  [L/16] first slot of every 16-position page
 //   aux    phase A: query constants (K3Prep / QInt8F); afterwards: selection histograms [G][SEG][256]
 //   stage  one private staging area per wavefront: key rows in phase A, V rows + weight rows in phase B
-// After the selection the whole block is reused for the exchange of the P.V accumulators.
+// After phase B the staging area holds the sum of the wavefronts' P.V accumulators.
 template <int SCHEME, int G, int NG>
 struct ScanLds {
   // SCHEME = 10 * key bits + value bits: the key side (staging, query constants, phase A) and the value side
@@ -143,11 +143,9 @@ struct ScanLds {
   static constexpr int KST = 64 * KROW;
   static constexpr int WAVE_STAGE = (VST + WL > KST) ? (VST + WL) : KST;
   static constexpr int ACC_REGS = 8 + NG;                   // v4i accumulators per set: 8 channel tiles + NG weight sums
-  static constexpr int XW = NW < 8 ? NW : 8;                // partial accumulator sets that reach the final sum
-  static constexpr int XWAVE = ACC_REGS * (48 * 16 + 16 * 4);  // bytes one wavefront writes per set (rows 0..12 only)
-  static constexpr int RED = XW * XWAVE;
-  // with one head set and enough staging space the exchange runs in the staging area while the score rows
-  // are still being read by the candidate emission
+  // sum of the wavefronts' accumulators: one int per (set, accumulator register, component, lane), in the staging
+  // area (dead after phase B), followed by one kilobyte per wavefront for the exact selection's histogram
+  static constexpr int XACC = NSET * ACC_REGS * 4 * 64 * 4;
   static constexpr int PREP = K3 ? (int)sizeof(K3Prep<NSET>) : (int)sizeof(QInt8F<NSET>);
   // selection histograms: 32-bit counters, or (any INT4 side, where the staging areas are larger and LDS is
   // tighter) two 16-bit counters per word: a (head, segment) histogram counts at most LMAX / SEG <= 4096 positions
@@ -155,12 +153,11 @@ struct ScanLds {
   static constexpr int HIST = G * SEG * 256 * (H16 ? 2 : 4);
   static constexpr int AUX = ((PREP > HIST ? PREP : HIST) + 15) & ~15;
   __host__ __device__ static constexpr int stage_bytes() { return NW * WAVE_STAGE; }
-  static constexpr bool XS = (NSET == 1) && (NW * WAVE_STAGE >= RED);
+  static_assert(NW * WAVE_STAGE >= XACC + NW * 1024, "the staging area must hold the accumulator sums and the selection scratch");
   __host__ __device__ static constexpr size_t per_position() { return (size_t)G * 4; }
   __host__ __device__ static size_t aux_offset(int L) { return (per_position() * L + (size_t)(L / 16) * 4 + 15) & ~(size_t)15; }
   __host__ __device__ static size_t total(int L) {
-    const size_t t = aux_offset(L) + AUX + stage_bytes() + 64;
-    return t > (size_t)RED + 64 ? t : (size_t)RED + 64;
+    return aux_offset(L) + AUX + stage_bytes() + 64;
   }
 };
 
@@ -875,11 +872,10 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
 #pragma unroll
       for (int qc = 0; qc < 4; ++qc) {
         const v2i x = __builtin_amdgcn_ds_read_tr4_b64_v2i32((__attribute__((address_space(3))) v2i*)(vrow + 8 * qc));
-        const uint32_t x0 = (uint32_t)x[0], x1 = (uint32_t)x[1];
-        const v4i Ba = {(int)((x0 >> 2) & 0x03030303u), (int)((x0 >> 6) & 0x03030303u),
-                        (int)((x1 >> 2) & 0x03030303u), (int)((x1 >> 6) & 0x03030303u)};
-        const v4i Bb = {(int)(x0 & 0x03030303u), (int)((x0 >> 4) & 0x03030303u),
-                        (int)(x1 & 0x03030303u), (int)((x1 >> 4) & 0x03030303u)};
+        const uint32_t x0 = (uint32_t)x[0], x1 = (uint32_t)x[1], y0 = x0 >> 4, y1 = x1 >> 4;
+        // the upper code of every nibble stays where it is: tile 2*qc accumulates 4 * code (undone in `combine`)
+        const v4i Ba = {(int)(x0 & 0x0c0c0c0cu), (int)(y0 & 0x0c0c0c0cu), (int)(x1 & 0x0c0c0c0cu), (int)(y1 & 0x0c0c0c0cu)};
+        const v4i Bb = {(int)(x0 & 0x03030303u), (int)(y0 & 0x03030303u), (int)(x1 & 0x03030303u), (int)(y1 & 0x03030303u)};
         const int g = (NG == 1) ? 0 : (qc >> 1);
 #pragma unroll
         for (int set = 0; set < NSET; ++set) {
@@ -936,35 +932,24 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   lds_barrier();
   if (clk && tid == 0) clk[2] = clock64();
 
-  // ---- exchange of the integer accumulators: every wavefront stores the rows that are used (0..12 of 16:
-  // lanes 0-47 whole registers, lanes 48-63 the first component); with sixteen wavefronts the upper half hands
-  // its sums to the lower half first; then each output element sums the remaining partials.  D layout: row r
-  // of a tile sits in lane 16*(r>>2) + column, register r&3; rows are (limb, head), row 12 is the ones row.
-  constexpr int XW = Lds::XW;  // partial sets that reach the final sum
-  constexpr bool XS = Lds::XS;
-  uint8_t* xbase = XS ? stage : smem;
-  v4i* xa = reinterpret_cast<v4i*>(xbase);                              // [XW][AR][48]
-  int* xb = reinterpret_cast<int*>(xbase + (size_t)XW * AR * 48 * 16);  // [XW][AR][16]
-  auto put = [&](int set, int slot) {
+  // ---- sum of the integer accumulators over the wavefronts: LDS integer atomics into one array in the staging
+  // area (dead now: every wavefront has passed the barrier above), zeroed here, filled after the cut search while
+  // the candidates are emitted, read by `combine` at the end.  Integer sums: exact and independent of the order.
+  // D layout: row r of a tile sits in lane 16*(r>>2) + column, register r&3; rows are (limb, head), row 12 is the
+  // ones row.  Element (set, register r, component c, lane l) lives at xacc[((set*AR + r)*4 + c)*64 + l].
+  int* xacc = reinterpret_cast<int*>(stage);
+  for (int i = tid; i < Lds::XACC / 4; i += NT) xacc[i] = 0;
+  auto add_acc = [&](int set) {
 #pragma unroll
     for (int r = 0; r < AR; ++r) {
       const v4i v = (r < NTILE) ? acc[set][r < NTILE ? r : 0] : accw[set][r >= NTILE ? r - NTILE : 0];
-      if (lane < 48) xa[((size_t)slot * AR + r) * 48 + lane] = v;
-      else xb[(slot * AR + r) * 16 + (lane - 48)] = v[0];
-    }
-  };
-  auto take = [&](int set, int slot) {
+      int* dst = xacc + ((set * AR + r) * 4) * 64 + lane;
 #pragma unroll
-    for (int r = 0; r < AR; ++r) {
-      v4i o = {0, 0, 0, 0};
-      if (lane < 48) o = xa[((size_t)slot * AR + r) * 48 + lane];
-      else o[0] = xb[(slot * AR + r) * 16 + (lane - 48)];
-      if (r < NTILE) acc[set][r < NTILE ? r : 0] += o;
-      else accw[set][r >= NTILE ? r - NTILE : 0] += o;
+      for (int c = 0; c < 4; ++c) atomicAdd(dst + c * 64, v[c]);
     }
   };
   auto combine = [&](int set) {
-    // thread -> (tile, head, column): the 64 lanes of a wavefront read 64 different banks
+    // thread -> (tile, head, column)
     for (int i = tid; i < 4 * D; i += NT) {
       const int col = i & 15, hh = (i >> 4) & 3, tile = i >> 6;
       const int h = set * 4 + hh;
@@ -977,26 +962,21 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
         d = tile * 16 + 2 * (col >> 1) + (1 - (col & 1));
       }
       const int g = (NG == 1) ? 0 : (d / (D / NG));
-      const int* xi = reinterpret_cast<const int*>(xa);
-      int i0 = 0, i1 = 0, i2 = 0, cs = 0, w0 = 0, w1 = 0, w2 = 0;  // |partial| < 2^23 per set: no overflow
-#pragma unroll
-      for (int w = 0; w < XW; ++w) {
-        const int* ta = xi + ((size_t)(w * AR + tile) * 48 + col) * 4 + hh;
-        i0 += ta[0];
-        i1 += ta[16 * 4];
-        i2 += ta[32 * 4];
-        cs += xb[(w * AR + tile) * 16 + col];
-        const int* wa = xi + ((size_t)(w * AR + NTILE + g) * 48) * 4 + hh;
-        w0 += wa[0];
-        w1 += wa[16 * 4];
-        w2 += wa[32 * 4];
+      const int* ta = xacc + ((set * AR + tile) * 4) * 64;          // limb l of head hh: component hh, lane 16*l + col
+      const int* wa = xacc + ((set * AR + NTILE + g) * 4) * 64;    // weight sums: any column of the all-ones tile
+      int i0 = ta[hh * 64 + col], i1 = ta[hh * 64 + 16 + col], i2 = ta[hh * 64 + 32 + col], cs = ta[48 + col];
+      if (V2 && !(tile & 1)) {  // even INT2 tiles hold four times their sums (exact multiples)
+        i0 >>= 2;
+        i1 >>= 2;
+        i2 >>= 2;
+        cs >>= 2;
       }
+      const int w0 = wa[hh * 64], w1 = wa[hh * 64 + 16], w2 = wa[hh * 64 + 32];   // |sum| < 2^24: no overflow
       const long long wsum = (long long)w2 * 65536ll + (long long)w1 * 256ll + (long long)w0 + 32896ll * 64ll * (long long)nch;
       const long long tot = (long long)i2 * 65536ll + (long long)i1 * 256ll + (long long)i0 + 32896ll * (long long)cs - (long long)VOFF * wsum;
       p.part_o[(part_base + (size_t)h * p.n_splits) * D + d] = (float)ldexp((double)tot, -E[g]);
     }
   };
-  if (XS && NW > XW && wave >= XW) put(0, wave - XW);  // overlaps the cut search below
 
   // ------------------------------------------------------------------ phase C: candidates of the split
   // The merge kernel needs a superset of the split's top Kt = min(top_k, n) scores per head that fits the
@@ -1070,10 +1050,8 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   }
   lds_barrier();
   if (clk && tid == 0) clk[6] = clock64();
-  if (XS && wave < XW) {
-    if (NW > XW) take(0, wave);
-    put(0, wave);
-  }
+#pragma unroll
+  for (int set = 0; set < NSET; ++set) add_acc(set);
   for (int hs = wave; hs < G * SEG; hs += NW) {
     const int h = hs / SEG, seg = hs % SEG;
     const float* srow = sc + h * L;
@@ -1122,7 +1100,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     } else if (seg == 0) {
       // exact fallback: 8-bit radix select over the order-preserving keys (bits shared by every key skipped),
       // then the keys above the K-th and the lowest-position ties that fill the quota
-      int* rh = XS ? reinterpret_cast<int*>(aux) + h * 256 : reinterpret_cast<int*>(stage + wave * Lds::WAVE_STAGE);
+      int* rh = reinterpret_cast<int*>(stage + Lds::XACC + wave * 1024);
       uint32_t T = 0;
       int quota = 0;
       uint32_t kmin = 0xffffffffu, kmax = 0u;
@@ -1206,23 +1184,8 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
 #pragma unroll
     for (int w = 0; w < NW; ++w) lfin += lsum_sh[w][tid];
   }
-  if (XS) {
-    combine(0);
-  } else {
-    // the score rows are dead by now: the exchange reuses their space, one head set at a time
 #pragma unroll
-    for (int set = 0; set < NSET; ++set) {
-      if (set > 0) lds_barrier();
-      if (NW > XW) {
-        if (wave >= XW) put(set, wave - XW);
-        lds_barrier();
-        if (wave < XW) take(set, wave);
-      }
-      if (wave < XW) put(set, wave);
-      lds_barrier();
-      combine(set);
-    }
-  }
+  for (int set = 0; set < NSET; ++set) combine(set);
   if (tid < G) {
     p.part_m[part_base + (size_t)tid * p.n_splits] = m_sh[tid];
     p.part_l[part_base + (size_t)tid * p.n_splits] = lfin;
