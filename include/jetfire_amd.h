@@ -214,6 +214,37 @@ int jf_fused_scan_topk_blend(int scheme, int group_size,
                              const uint16_t* o_new, uint16_t* out,
                              void* workspace, size_t workspace_bytes, void* stream);
 
+/* Stage A alone and Stage B alone on the kernels of the fused step, for callers that keep the reference's two-call
+ * structure (jetfire_vllm/adapter/decode_path.py:2081-2131 then :2804-2935): the same results as the split entry
+ * points above for the shapes the fused step supports (head_dim 128, block_size 16, H_q/H_kv in {1,2,4,8,16},
+ * top_k <= 1024, num_slots <= 2^25), at a fraction of their time.  workspace: jf_fused_workspace_bytes(format, ...).
+ *
+ * jf_stage_a_topk replaces int3_qk_scores / int3_qk_scores_topk (jetfire_vllm/csrc/int3_qk_scores.cu:640-655;
+ * key_format JF_SCHEME_K3V2: INT3 keys, bf16 model, group 64 or 128) and int8tc_qk_scores / _topk / _topk_stats
+ * (jetfire_vllm/csrc/int8tc_qk_scores.cu:2774-2798; key_format JF_SCHEME_K4V4: INT4 keys, int8-Q model, group 128).
+ * scores (B, H_q, max_S) may be NULL (not written); softmax_m / softmax_inv_z may be NULL.  top_k == 0: scores alone
+ * (topk_idx, topk_slots and the workspace are then unused). */
+int jf_stage_a_topk(int key_format, int group_size,
+                    const uint16_t* q, const uint8_t* k_data, const uint16_t* k_scales,
+                    const int64_t* block_table, const int32_t* seq_lens,
+                    int B, int H_q, int H_kv, int max_S, int max_blocks, int64_t num_slots,
+                    int block_size, float attn_scale, int top_k,
+                    float* scores, int64_t* topk_idx, int64_t* topk_slots,
+                    float* softmax_m, float* softmax_inv_z,
+                    void* workspace, size_t workspace_bytes, void* stream);
+/* jf_stage_b_softmax_v replaces int2_softmax_v_with_pre_corr_wvs2 (jetfire_vllm/csrc/int2_softmax_v.cu:792-901;
+ * value_format JF_SCHEME_K3V2: INT2 values, group 64 or 128) and int4_softmax_v_with_pre_corr_wvs2_scores
+ * (jetfire_vllm/csrc/int4_softmax_v.cu:2203-2235; value_format JF_SCHEME_K4V4: INT4 values, group 128), with exact
+ * fp32 softmax weights computed from `scores`.  topk_idx (B, H_q, top_k), ascending and -1 padded, may be NULL
+ * (o_hat only; o_old_unnorm and W are then zero). */
+int jf_stage_b_softmax_v(int value_format, int group_size,
+                         const float* scores, const uint8_t* v_data, const uint16_t* v_scales,
+                         const int64_t* block_table, const int32_t* seq_lens, const int64_t* topk_idx,
+                         int B, int H_q, int H_kv, int max_S, int max_blocks, int64_t num_slots,
+                         int block_size, int top_k,
+                         float* o_hat, float* o_old_unnorm, float* W,
+                         void* workspace, size_t workspace_bytes, void* stream);
+
 /* jf_fused_scan_topk without the workspace arguments, for callers that cannot allocate device memory (code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in
  * the reference.  The workspace is a fixed array of JF_FUSED_STATIC_SCRATCH_BYTES in device memory that each

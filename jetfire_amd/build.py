@@ -23,6 +23,8 @@ SOURCES = (
     "topk.hip",
     "softmax_v.hip",
     "fused_scan.hip",
+    "fused_stage_a.hip",
+    "fused_stage_b.hip",
     "blend.hip",
     "calibrate.hip",
     "cpu_topk_attn.cpp",

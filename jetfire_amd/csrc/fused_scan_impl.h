@@ -1,0 +1,2123 @@
+// Fused decode scan + top-k for gfx950: one pass over the packed K and V of every (sequence, kv-head),
+// no (B, H_q, S) score tensor in HBM.
+//
+// Launch 1, fused_scan_kernel, grid (n_splits, H_kv, B), 16 wavefronts per workgroup (8 where the register
+// budget does not allow 1024 threads).  A workgroup owns L consecutive positions of one (sequence, kv-head)
+// and all G query heads of that kv-head.  The page table of the split is read once into LDS.  Key and value
+// rows are fetched in 64-position chunks with 16-byte loads whose lane addresses are consecutive inside a
+// page, two chunks per wavefront in flight, staged in wavefront-private LDS and read back in the layout the
+// arithmetic wants; barriers order LDS traffic only, so prefetched rows stay in flight across them.
+//   phase A  Q.K^T on v_mfma_i32_16x16x64_i8, tokens on the N side, rows = (head, limb or block):
+//            INT3 keys: the bf16 query as exact 23-bit fixed point in three int8 limbs, codes spread from the
+//                       byte planes with shift/mask on dwords, a second contraction with the indicator of
+//                       codes +-3 reproduces the reference's bf16 rounding of the dequantised key.
+//            INT4 keys: int8-quantised Q, exact nibble codes, one accumulator row per 32-channel block, the
+//                       reference's fp32 rescale order (bit-equal to the split-form kernel).
+//            scores[G][L] -> LDS (fp32), running max / min per head.
+//   phase B  P.V on the same MFMA.  p = exp(s - m_split) is known exactly because phase A is complete, so
+//            w = p * v_scale is converted to 22-bit fixed point once (fma with 2^23), its three bytes are the
+//            A-operand rows (limb, head), and the int32 accumulators live for the whole split: every product
+//            is exact.  V codes are transposed by ds_read_b64_tr_b4, weight rows by ds_read_b64_tr_b8.
+//            The same pass drops every score into one of 256 linear buckets per (head, segment).
+//   phase C  from the bucket histograms: the smallest bucket range that holds the split's top min(K, n) scores
+//            and fits the candidate buffer; its positions are emitted as (key, position) in ascending
+//            position, one wavefront per (head, segment).  Heavily tied scores fall back to a radix select.
+//   exchange of the wavefronts' integer accumulators through LDS, exact int64 recombination -> partial o.
+// Launch 2, fused_merge_kernel, grid (B, H_q): selects the global top-k among the candidates (ties to
+// the lower position, ascending output), merges the split partials
+//   M = max m_i, l = sum l_i e^{m_i-M}, o_hat = sum o_i e^{m_i-M} / l
+// (the split-KV combine of jetfire_vllm/csrc/fused_decode_wmma.cu:1226-1253), and computes the
+// pre-correction terms o_old_unnorm, W over the winners (jetfire_vllm/csrc/int2_softmax_v.cu:738-788).
+//
+// This header holds the kernels, the launch planner and the launcher; it is included by the translation units that
+// instantiate them (fused_scan.hip and the stage-wise forms), each for its own set of template arguments.
+#pragma once
+#include "common.h"
+
+#include <atomic>
+#include <mutex>
+#include <vector>
+
+namespace jf {
+
+// Process-wide measurement / test switches shared by those translation units (defined in fused_scan.hip),
+// reachable from the public debug entry points: the event list has its own lock, the two scalars are atomics
+// (a launch reads each once).
+// Optional measurement hook: when armed, every fused_scan_kernel launch is bracketed by a pair of HIP
+// events on its own stream, so a benchmark can read the kernel's device time without a profiler.
+struct ScanProfile {
+  std::vector<hipEvent_t> ev;
+  int used = 0;
+  std::atomic<bool> armed{false};
+};
+extern ScanProfile g_prof;
+extern std::mutex g_prof_mu;
+extern std::atomic<long long*> g_phase_clock;
+extern std::atomic<int> g_force_split_len;  // test / measurement aid: overrides the planner's split length when positive
+// Compute units of the current device (the planner balances workgroups over them); 256, the MI355X count, when
+// no device can be asked (planning on a host without a GPU).
+int device_cus();
+
+namespace {
+
+
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef unsigned v2u __attribute__((ext_vector_type(2)));
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+
+// Forms of the step (template argument MODE of both kernels):
+//   FS_FULL     Stage A + Stage B + top-k in one pass (keys and values streamed once, scores never in HBM)
+//   FS_STAGE_A  Stage A alone: scores (optionally written out), top-k, softmax statistics; no value stream
+//   FS_STAGE_B  Stage B alone: scores and winners are inputs; value stream, o_hat and the pre-correction terms
+constexpr int FS_FULL = 0, FS_STAGE_A = 1, FS_STAGE_B = 2;
+
+constexpr int FS_MAX_TOPK = 1024;      // winners cached in LDS by the merge kernel
+constexpr int FS_CAND_SLACK = 256;     // extra candidate slots per (row, split): room for the whole cut bucket
+
+struct FusedParams {
+  const uint16_t* q;
+  const uint8_t* k_data;
+  const uint16_t* k_scales;
+  const uint8_t* v_data;
+  const uint16_t* v_scales;
+  const int64_t* block_table;
+  const int32_t* seq_lens;
+  int B, H_q, H_kv, max_S, max_blocks;
+  int64_t num_slots;
+  float attn_scale;
+  int top_k;
+  int L, n_splits, Kc;
+  float* scores;  // optional (B, H_q, max_S)
+  const float* scores_in;  // FS_STAGE_B: the scores (B, H_q, max_S)
+  int scores_only;         // FS_STAGE_A: stop after writing `scores`
+  float* part_m;  // (B, H_q, NS)
+  float* part_l;  // (B, H_q, NS)
+  float* part_o;  // (B, H_q, NS, D)
+  uint32_t* cand_key;  // (B, H_q, NS, Kc)
+  int32_t* cand_idx;   // (B, H_q, NS, Kc)
+  int32_t* cand_cnt;   // (B, H_q, NS)
+  // two-stage merge (long contexts): `mg_parts` workgroups per row first reduce `mg_spp` consecutive
+  // candidate lists each to the row's top_k among them; the final merge then reads those lists
+  int mg_parts, mg_spp;
+  uint32_t* key2;      // (B, H_q, mg_parts, top_k)
+  int32_t* idx2;       // (B, H_q, mg_parts, top_k)
+  int32_t* cnt2;       // (B, H_q, mg_parts)
+  // merge outputs
+  int64_t* topk_idx;
+  int64_t* topk_slots;
+  float* o_hat;
+  float* o_old;
+  float* W;
+  float* softmax_m;
+  float* softmax_inv_z;
+  // optional merge epilogue: out = bf16(fma(W, o_new, o_hat) - o_old_unnorm), both (B, H_q, D) bf16
+  const uint16_t* blend_o_new;
+  uint16_t* blend_out;
+  long long* phase_clock;  // optional: 10 s_memtime stamps per scan workgroup, 8 per merge workgroup (measurement aid)
+};
+
+// Phase-A constants of the INT3 path, built once per workgroup in LDS.
+template <int NSET>
+struct K3Prep {
+  int8_t aop[NSET][16][4][2][16];  // A operand bytes: [set][row = 4*head + limb][k-block][MFMA][byte]
+  int sq4[NSET * 4][2];            // 4 * sum of the fixed-point query over the scale group
+  float qsc[NSET * 4][2];          // 2^(e-22) * attn_scale of the (head, group)
+  float eps[128];                  // 256 * (bf16(3s) - 3s) / s for s = 1 + m/128
+  float amax_w[NSET * 8];          // per 64-channel half row: |q| maximum, fixed-point sum, exponent
+  int sum_w[NSET * 8];
+  int exp_w[NSET * 8];
+};
+
+// Phase-A constants of the INT4 path: the int8-quantised query rows as MFMA A operand.  Row 4*head + kk holds
+// the head's values of 32-channel block kk and zeros elsewhere, so one accumulator register per block.
+template <int NSET>
+struct QInt8F {
+  int8_t aop[NSET][16][4][2][16];  // [set][row = 4*head + block][k-block][MFMA][byte]
+  float qs[NSET * 4][4];           // query scale of (head, block)
+  int sum8[NSET * 4][4];           // 8 * sum of the int8 query over the block (the codes carry an offset of 8)
+};
+
+// LDS carve-up shared by the kernel and its launcher.
+//   sc     [G][L] fp32 scores of the split
+//   sbase  [L/16] first slot of every 16-position page
+//   aux    phase A: query constants (K3Prep / QInt8F); afterwards: selection histograms [G][SEG][256]
+//   stage  one private staging area per wavefront: key rows in phase A, V rows + weight rows in phase B
+// After phase B the staging area holds the sum of the wavefronts' P.V accumulators.
+template <int SCHEME, int G, int NG>
+struct ScanLds {
+  // SCHEME = 10 * key bits + value bits: the key side (staging, query constants, phase A) and the value side
+  // (staging, phase B) are chosen independently
+  static constexpr bool K3 = (SCHEME / 10 == 3);
+  static constexpr bool V2 = (SCHEME % 10 == 2);
+  static_assert((K3 || SCHEME / 10 == 4) && (V2 || SCHEME % 10 == 4), "keys are INT3 or INT4, values INT2 or INT4");
+  static constexpr int NSET = (G + 3) / 4;
+  // wavefronts per workgroup: sixteen where the register budget allows (128 VGPRs at 1024 threads), else eight
+  static constexpr int NW = (G <= 4) ? 16 : 8;
+  static constexpr int NT = NW * 64;
+  static constexpr int LMAX = NW * 256;  // four 64-position chunks per wavefront
+  // emission segments per head (one wavefront each)
+  static constexpr int SEG = (NW / G >= 4) ? 4 : ((NW / G >= 2) ? 2 : 1);
+  static constexpr int KP = K3 ? 48 : 64;
+  static constexpr int KROW = K3 ? 48 : 80;     // LDS pitch of a staged key row (INT4: padded against bank conflicts)
+  static constexpr int VP = V2 ? 32 : 64;
+  // LDS pitch of a staged V row.  INT2 rows (32 bytes) are padded so that 16 consecutive rows hit 16 distinct
+  // bank pairs; INT4 rows (64 bytes) keep their pitch and swap their 16-byte quarters instead (quarter q of
+  // row r sits at q ^ ((r >> 2) & 3)), which has the same effect without the padding bytes.
+  static constexpr bool VSWZ = !V2;
+  static constexpr int VROW = VSWZ ? VP : VP + 8;
+  static constexpr int VST = 64 * VROW;
+  static constexpr int WL = NG * NSET * 64 * 16;  // per (group, set): one 16-byte weight row per token
+  static constexpr int KST = 64 * KROW;
+  static constexpr int WAVE_STAGE = (VST + WL > KST) ? (VST + WL) : KST;
+  static constexpr int ACC_REGS = 8 + NG;                   // v4i accumulators per set: 8 channel tiles + NG weight sums
+  // sum of the wavefronts' accumulators: one int per (set, accumulator register, component, lane), in the staging
+  // area (dead after phase B), followed by one kilobyte per wavefront for the exact selection's histogram
+  static constexpr int XACC = NSET * ACC_REGS * 4 * 64 * 4;
+  static constexpr int PREP = K3 ? (int)sizeof(K3Prep<NSET>) : (int)sizeof(QInt8F<NSET>);
+  // selection histograms: 32-bit counters, or (any INT4 side, where the staging areas are larger and LDS is
+  // tighter) two 16-bit counters per word: a (head, segment) histogram counts at most LMAX / SEG <= 4096 positions
+  static constexpr bool H16 = !(K3 && V2);
+  static constexpr int HIST = G * SEG * 256 * (H16 ? 2 : 4);
+  static constexpr int AUX = ((PREP > HIST ? PREP : HIST) + 15) & ~15;
+  __host__ __device__ static constexpr int stage_bytes() { return NW * WAVE_STAGE; }
+  static_assert(NW * WAVE_STAGE >= XACC + NW * 1024, "the staging area must hold the accumulator sums and the selection scratch");
+  __host__ __device__ static constexpr size_t per_position() { return (size_t)G * 4; }
+  __host__ __device__ static size_t aux_offset(int L) { return (per_position() * L + (size_t)(L / 16) * 4 + 15) & ~(size_t)15; }
+  __host__ __device__ static size_t total(int L) {
+    return aux_offset(L) + AUX + stage_bytes() + 64;
+  }
+};
+
+__device__ inline float key_to_score(uint32_t key) {
+  const uint32_t u = (key & 0x80000000u) ? (key & 0x7fffffffu) : ~key;
+  return __builtin_bit_cast(float, u);
+}
+
+// Orders this wavefront's earlier LDS writes before its later LDS reads (the LDS pipe executes one
+// wavefront's instructions in order; this only stops the compiler from moving them).
+__device__ inline void wave_lds_fence() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Workgroup barrier that orders LDS traffic only: unlike __syncthreads() it does not wait for global loads
+// that are still in flight (the prefetched key / value rows), which no other wavefront consumes.
+__device__ inline void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// s_setprio takes an immediate; `p` is a compile-time constant after unrolling
+__device__ inline void set_wave_prio(int p) {
+  if (p >= 3) __builtin_amdgcn_s_setprio(3);
+  else if (p == 2) __builtin_amdgcn_s_setprio(2);
+  else if (p == 1) __builtin_amdgcn_s_setprio(1);
+  else __builtin_amdgcn_s_setprio(0);
+}
+
+__device__ inline float uniform_f(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, v)));
+}
+
+// ---------------------------------------------------------------------------------------------------
+template <int MODE, int SCHEME, int G, int NG>
+__global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kernel(FusedParams p) {
+  using Lds = ScanLds<SCHEME, G, NG>;
+  constexpr bool HAS_K = (MODE != FS_STAGE_B);     // key stream and phase A
+  constexpr bool HAS_V = (MODE != FS_STAGE_A);     // value stream and the P.V part of phase B
+  constexpr bool HAS_TOPK = (MODE != FS_STAGE_B);  // histograms and phase C
+  constexpr bool K3 = Lds::K3;
+  constexpr bool V2 = Lds::V2;
+  constexpr int NSET = Lds::NSET;
+  constexpr int SEG = Lds::SEG;
+  constexpr int KP = Lds::KP;
+  constexpr int KROW = Lds::KROW;
+  constexpr int VP = Lds::VP;
+  constexpr int VROW = Lds::VROW;
+  constexpr int VOFF = V2 ? 2 : 8;  // code offset of the V format
+  constexpr int NTILE = 8;          // 8 MFMA column tiles of 16 channels
+  constexpr int AR = Lds::ACC_REGS;
+  constexpr float LOG2E = 1.44269504088896340736f;
+  constexpr int NW = Lds::NW, NT = Lds::NT;
+  constexpr int MAXIT = Lds::LMAX / 64 / NW;  // chunks per wavefront
+
+  extern __shared__ __align__(16) uint8_t smem[];
+  const int L = p.L;
+  float* sc = reinterpret_cast<float*>(smem);                     // [G][L]
+  int* sbase = reinterpret_cast<int*>(smem + (size_t)G * L * 4);  // [L/16] first slot of each page
+  uint8_t* aux = smem + Lds::aux_offset(L);
+  uint8_t* stage = aux + Lds::AUX;
+  int* hist = reinterpret_cast<int*>(aux);  // [G][SEG][256], valid after phase A
+  __shared__ float red_f[NW][2 * G];
+  __shared__ uint32_t vmax_sh[NW][2];
+  __shared__ float m_sh[G], bin_a_sh[G], bin_b_sh[G], lsum_sh[NW][G];
+  __shared__ int e_sh[2];
+  __shared__ int cut_sh[G], segoff_sh[G][SEG + 1], exact_sh[G];
+  __shared__ unsigned long long tmax_sh;
+  if (threadIdx.x == 0) tmax_sh = 0ull;
+
+  const int split = blockIdx.x, hkv = blockIdx.y, b = blockIdx.z;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: keeps wave-derived addresses in SGPRs
+  const int S = max(0, min(p.max_S, p.seq_lens[b]));
+  const int s0 = split * L;
+  const int s1 = min(s0 + L, S);
+  const int n = max(0, s1 - s0);
+  const int s_cover = min(s0 + L, p.max_S);
+  const int n_cover = max(0, s_cover - s0);
+  const int64_t* bt = p.block_table + (size_t)b * p.max_blocks;
+  const size_t head0 = (size_t)b * p.H_q + (size_t)hkv * G;
+  const size_t part_base = head0 * p.n_splits + split;  // + h * n_splits
+  const uint8_t* kbase = p.k_data + (size_t)hkv * p.num_slots * KP;
+  const uint8_t* vbase = p.v_data + (size_t)hkv * p.num_slots * VP;
+  const uint8_t* vsbase = reinterpret_cast<const uint8_t*>(p.v_scales + (size_t)hkv * p.num_slots * NG);
+
+  long long* clk = p.phase_clock ? p.phase_clock + (((size_t)b * p.H_kv + hkv) * p.n_splits + split) * 10 : nullptr;
+  if (clk && tid == 0) clk[0] = clock64();
+
+  // The page-table entry and the query elements of this thread do not depend on the sequence length: they
+  // are requested first, so their latency runs in parallel with the load of seq_lens[b] instead of after it.
+  const int nch_cover = (n_cover + 63) >> 6;
+  int64_t bt_mine = 0;  // LMAX / 16 <= NT: one entry per thread covers the split
+  if (tid < nch_cover * 4) bt_mine = bt[min((s0 >> 4) + tid, p.max_blocks - 1)];
+  constexpr int QN = NSET * 4 * D;               // elements of the padded query block (whole head sets)
+  constexpr int QPT = (QN + NT - 1) / NT;
+  float qv[QPT];
+#pragma unroll
+  for (int it = 0; it < QPT; ++it) {
+    const int i = it * NT + tid;
+    qv[it] = (i < G * D) ? bf16_to_f32(p.q[head0 * D + i]) : 0.f;
+  }
+
+  if (n == 0) {  // nothing valid in this split: padding scores, empty partials
+    if (p.scores)
+      for (int i = tid; i < G * n_cover; i += NT)
+        p.scores[(head0 + i / n_cover) * (size_t)p.max_S + s0 + (i % n_cover)] = -INFINITY;
+    if constexpr (MODE == FS_STAGE_A)
+      if (p.scores_only) return;
+    for (int i = tid; i < G * D; i += NT) p.part_o[(part_base + (size_t)(i / D) * p.n_splits) * D + (i % D)] = 0.f;
+    if (tid < G) {
+      p.part_m[part_base + (size_t)tid * p.n_splits] = -INFINITY;
+      p.part_l[part_base + (size_t)tid * p.n_splits] = 0.f;
+      p.cand_cnt[part_base + (size_t)tid * p.n_splits] = 0;
+    }
+    for (int i = tid; i < G * p.Kc; i += NT)  // unused candidate slots hold key 0 (no score maps to it)
+      p.cand_key[(part_base + (size_t)(i / p.Kc) * p.n_splits) * p.Kc + (i % p.Kc)] = 0u;
+    return;
+  }
+
+  // Page table of the split: one entry per 16 positions of every 64-token chunk that is touched.  Table
+  // entries past the last valid position may hold anything: those pages read slot 0 instead, so every row
+  // address formed below is in bounds (those rows' scores are masked to -inf, their softmax weights are
+  // exactly zero).
+  const int nch = (n + 63) >> 6;
+  if (tid < nch_cover * 4) sbase[tid] = (tid <= ((n - 1) >> 4)) ? (int)(bt_mine * BS) : 0;
+  lds_barrier();
+
+  // ---- key stream, set-up.  A chunk is 64 consecutive positions = 4 pages; its rows are fetched with
+  // 16-byte loads whose lane addresses are consecutive inside a page, staged in this wavefront's LDS area
+  // in position order, and read back in the layout the arithmetic wants.
+  uint8_t* kst = stage + wave * Lds::WAVE_STAGE;
+  constexpr int KLD = KP / 16;  // 16-byte loads per lane and chunk
+  uint32_t kl_page[KLD], kl_off[KLD], kl_lds[KLD];
+#pragma unroll
+  for (int i = 0; i < KLD; ++i) {
+    const int o = 1024 * i + 16 * lane;  // byte offset inside the chunk's 64 rows
+    kl_page[i] = (uint32_t)(o / (16 * KP));
+    kl_off[i] = (uint32_t)(o % (16 * KP));
+    kl_lds[i] = (uint32_t)((o / KP) * KROW + (o % KP));
+  }
+  const uint8_t* ksb = reinterpret_cast<const uint8_t*>(p.k_scales + (size_t)hkv * p.num_slots * (K3 ? NG : 1));
+  struct KBuf {
+    v4u r[KLD];
+    uint32_t s[4];
+  };
+  const int t16 = lane & 15, lg = lane >> 4;
+  auto issue_k = [&](int chunk) -> KBuf {
+    KBuf kbuf;
+#pragma unroll
+    for (int i = 0; i < KLD; ++i) {
+      const uint32_t sb = (uint32_t)sbase[chunk * 4 + kl_page[i]];
+      kbuf.r[i] = *reinterpret_cast<const v4u*>(kbase + (size_t)(sb * (uint32_t)KP + kl_off[i]));
+    }
+    constexpr int KNG = K3 ? NG : 1;  // key scales per row
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int sb = __builtin_amdgcn_readfirstlane(sbase[chunk * 4 + j]);  // first slot of the page (uniform)
+      const uint8_t* srow = ksb + (size_t)sb * (KNG * 2) + t16 * (KNG * 2);
+      if (KNG == 2) kbuf.s[j] = *reinterpret_cast<const uint32_t*>(srow);
+      else kbuf.s[j] = *reinterpret_cast<const uint16_t*>(srow);
+    }
+    return kbuf;
+  };
+  auto stash_k = [&](const KBuf& kbuf) {
+#pragma unroll
+    for (int i = 0; i < KLD; ++i) *reinterpret_cast<v4u*>(kst + kl_lds[i]) = kbuf.r[i];
+  };
+  // first two chunks of this wavefront and the V scales of the split start now, before the query set-up
+  KBuf Ka = {}, Kb = {};
+  if (HAS_K && wave < nch_cover) Ka = issue_k(wave);
+  constexpr int VSPT = Lds::LMAX / NT;
+  uint32_t vsw[VSPT];
+#pragma unroll
+  for (int i = 0; i < VSPT; ++i) {
+    const int t = tid + i * NT;
+    vsw[i] = 0u;
+    if (HAS_V && t < n) {
+      const uint32_t slot = (uint32_t)(sbase[t >> 4] + (t & 15));
+      if (NG == 2) vsw[i] = *reinterpret_cast<const uint32_t*>(vsbase + (size_t)(slot * 4u));
+      else vsw[i] = (uint32_t) * reinterpret_cast<const uint16_t*>(vsbase + (size_t)(slot * 2u));
+    }
+  }
+
+  if constexpr (!HAS_K) {
+    // the scores are an input: no query constants
+  } else if constexpr (K3) {
+    // Query rows -> 23-bit fixed point per (head, scale group), three balanced int8 limbs, written in the
+    // byte order of the MFMA A operand.  One element per thread; group statistics by wavefront reductions.
+    K3Prep<NSET>* prep = reinterpret_cast<K3Prep<NSET>*>(aux);
+    if (tid < 128) {
+      const float sm = 1.0f + (float)tid * (1.0f / 128.0f);
+      const float t3 = 3.0f * sm;  // exact in fp32
+      prep->eps[tid] = 256.0f * ((bf16_to_f32(f32_to_bf16(t3)) - t3) / sm);
+    }
+#pragma unroll
+    for (int it = 0; it < QPT; ++it) {
+      const int c = it * NW + wave;  // 64-channel half row of this wavefront
+      if (c * 64 < QN) {             // uniform per wavefront
+        const float am = wave_max(fabsf(qv[it]));
+        if (lane == 0) prep->amax_w[c] = am;
+      }
+    }
+    lds_barrier();
+#pragma unroll
+    for (int it = 0; it < QPT; ++it) {
+      const int i = it * NT + tid, h = i >> 7, d = i & 127;
+      const float x = qv[it];
+      const int c = it * NW + wave;
+      if (c * 64 >= QN) continue;
+      const float amax = (NG == 2) ? prep->amax_w[c] : fmaxf(prep->amax_w[c & ~1], prep->amax_w[c | 1]);
+      int e = 0;
+      if (amax > 0.f && isfinite(amax)) (void)frexpf(amax, &e);  // amax = f * 2^e, f in [0.5, 1)
+      const int qf = (int)rintf(ldexpf(x, 22 - e));
+      const int s = wave_sum_i(qf);
+      if (lane == 0) {
+        prep->sum_w[c] = s;
+        prep->exp_w[c] = e;
+      }
+      const int l0 = (int)(int8_t)(qf & 255);
+      const int r1 = (qf - l0) >> 8;
+      const int l1 = (int)(int8_t)(r1 & 255);
+      const int l2 = (r1 - l1) >> 8;
+      const int set = h >> 2, hh = h & 3;
+      // channel d of the key row sits in byte 4*(d&3) + ((d>>3)&3) of a 16-byte k-block (the order the plane
+      // spread produces); with two scale groups MFMA g covers group g only (see the lane swap in phase A)
+      const int mi = (NG == 2) ? (d >> 6) : ((d >> 2) & 1);
+      const int kb = (NG == 2) ? (((d >> 5) & 1) + 2 * ((d >> 2) & 1)) : (d >> 5);
+      const int by = 4 * (d & 3) + ((d >> 3) & 3);
+      prep->aop[set][4 * hh + 0][kb][mi][by] = (int8_t)l0;
+      prep->aop[set][4 * hh + 1][kb][mi][by] = (int8_t)l1;
+      prep->aop[set][4 * hh + 2][kb][mi][by] = (int8_t)l2;
+      prep->aop[set][4 * hh + 3][kb][mi][by] = 0;
+    }
+    lds_barrier();
+    if (tid < NSET * 4 * NG) {
+      const int h = tid / NG, g = tid % NG;
+      const int sum = (NG == 2) ? prep->sum_w[2 * h + g] : prep->sum_w[2 * h] + prep->sum_w[2 * h + 1];
+      const int e = prep->exp_w[2 * h + ((NG == 2) ? g : 0)];
+      prep->sq4[h][g] = 4 * sum;
+      prep->qsc[h][g] = ldexpf(p.attn_scale, e - 22);
+    }
+  } else {
+    // int8 quantisation of the query rows per 32 channels (int8tc_qk_scores.cu:250-290), one element per thread;
+    // heads past G are zero rows
+    QInt8F<NSET>* qsh = reinterpret_cast<QInt8F<NSET>*>(aux);
+#pragma unroll
+    for (int it = 0; it < QPT; ++it) {
+      const int i = it * NT + tid;
+      if (i < QN) {  // uniform per wavefront: QN is a multiple of 64
+        const int h = i >> 7, d = i & 127, kk = d >> 5;
+        const float x = qv[it];
+        float a = fabsf(x);
+#pragma unroll
+        for (int off = 16; off >= 1; off >>= 1) a = fmaxf(a, __shfl_xor(a, off));
+        const float sq = fmaxf(a / 127.0f, 1e-12f);
+        const float inv = 1.0f / sq;
+        const int v = max(-128, min(127, (int)rintf(x * inv)));
+        int sv = v;
+#pragma unroll
+        for (int off = 16; off >= 1; off >>= 1) sv += __shfl_xor(sv, off);
+        // channel d sits in MFMA d>>6, k-block (d>>4)&3; inside the k-block's 16 bytes the nibble spread of two
+        // packed dwords yields: even channels of bytes 0-3, odd channels of bytes 0-3, then the same for bytes 4-7
+        const int set = h >> 2, hh = h & 3, mi = d >> 6, kb = (d >> 4) & 3;
+        const int j2 = (d & 15) >> 1, odd = d & 1;
+        const int by = (j2 >> 2) * 8 + odd * 4 + (j2 & 3);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) qsh->aop[set][4 * hh + r][kb][mi][by] = (r == kk) ? (int8_t)v : (int8_t)0;
+        if ((lane & 31) == 0) {
+          qsh->qs[h][kk] = sq;
+          qsh->sum8[h][kk] = 8 * sv;
+        }
+      }
+    }
+  }
+  lds_barrier();
+  if (HAS_K && wave + NW < nch_cover) Kb = issue_k(wave + NW);
+  if (clk && tid == 0) clk[7] = clock64();
+
+  // ---- V stream, set-up (same scheme as the key stream)
+  uint8_t* vst = stage + wave * Lds::WAVE_STAGE;  // [64][VROW], this wavefront only
+  uint8_t* wl = vst + Lds::VST;                   // [NG][NSET][64 tokens][16]
+  constexpr int VLD = VP / 16;
+  uint32_t vl_page[VLD], vl_off[VLD], vl_lds[VLD];
+#pragma unroll
+  for (int i = 0; i < VLD; ++i) {
+    const int o = 1024 * i + 16 * lane;
+    vl_page[i] = (uint32_t)(o / (16 * VP));
+    vl_off[i] = (uint32_t)(o % (16 * VP));
+    const int row = o / VP, q16 = (o % VP) / 16;
+    vl_lds[i] = Lds::VSWZ ? (uint32_t)(row * VROW + ((q16 ^ ((row >> 2) & 3)) * 16)) : (uint32_t)(row * VROW + (o % VP));
+  }
+  struct VBuf {
+    v4u r[VLD];
+    uint32_t w;
+  };
+  auto issue_v = [&](int chunk) -> VBuf {
+    VBuf vbuf;
+#pragma unroll
+    for (int i = 0; i < VLD; ++i) {
+      const uint32_t sb = (uint32_t)sbase[chunk * 4 + vl_page[i]];
+      vbuf.r[i] = *reinterpret_cast<const v4u*>(vbase + (size_t)(sb * (uint32_t)VP + vl_off[i]));
+    }
+    const int t = chunk * 64 + lane;
+    const uint32_t slot = (uint32_t)(sbase[t >> 4] + (t & 15));
+    if (NG == 2) vbuf.w = *reinterpret_cast<const uint32_t*>(vsbase + (size_t)(slot * 4u));
+    else vbuf.w = (uint32_t) * reinterpret_cast<const uint16_t*>(vsbase + (size_t)(slot * 2u));
+    return vbuf;
+  };
+  // the first two V chunks are requested while the last key chunks are being worked on
+  VBuf Va = {}, Vb = {};
+  auto prefetch_v = [&](int it) {
+    if constexpr (MODE == FS_FULL) {
+      if (it == MAXIT - 2 && wave < nch) Va = issue_v(wave);
+      if (it == MAXIT - 1 && wave + NW < nch) Vb = issue_v(wave + NW);
+    }
+  };
+  if constexpr (MODE == FS_STAGE_B) {  // nothing to wait for: the value stream starts at once
+    if (wave < nch) Va = issue_v(wave);
+    if (wave + NW < nch) Vb = issue_v(wave + NW);
+  }
+
+
+  // ------------------------------------------------------------------ phase A
+  if constexpr (!HAS_K) {
+    // the split's scores come from the caller's (B, H_q, max_S) tensor: -> LDS, running maximum per head;
+    // positions past the sequence (and the rest of the last chunk) become -inf
+#pragma unroll
+    for (int h = 0; h < G; ++h) {
+      const float* srow = p.scores_in + (head0 + h) * (size_t)p.max_S + s0;
+      float mx = -INFINITY;
+      for (int t = tid; t < nch * 64; t += NT) {
+        const float v = (t < n) ? srow[t] : -INFINITY;
+        sc[h * L + t] = v;
+        mx = fmaxf(mx, v);
+      }
+      mx = wave_max(mx);
+      if (lane == 0) {
+        red_f[wave][h] = mx;
+        red_f[wave][G + h] = mx;  // (the minimum only shapes the selection buckets, which this form does not use)
+      }
+    }
+  } else if constexpr (K3) {
+    // INT3 keys on v_mfma_i32_16x16x64_i8.  The bf16 query row is held exactly as a 23-bit fixed-point number
+    // per (head, scale group), split into three balanced int8 limbs that sit in different A-operand rows
+    // (row = 4*head + limb), so one MFMA yields the three integer partial sums of a (token, head) in the
+    // registers of one lane.  K codes are spread from the three byte planes to one byte per code with
+    // shift/mask on whole dwords (4 codes per VALU operation) and used unsigned; the -4 offset is removed with
+    // the per-row constant 4*sum(q).  Lane (token, k-block lg) holds channels 32*lg .. 32*lg+31, i.e. lanes
+    // 0-31 hold scale group 0 and lanes 32-63 group 1; one v_permlane32_swap per dword regroups them so that
+    // each MFMA contracts over exactly one scale group.  The reference rounds every dequantised key to bf16
+    // (int3_qk_scores.cu:90-99); only codes +-3 are inexact, so that rounding is reproduced by a second
+    // contraction with the indicator (+1 for code 7, -1 for code 1, byte LUT through v_perm_b32) weighted by
+    // eps = (bf16(3s) - 3s) / s, which depends on the 7 mantissa bits of the scale only (128-entry table).
+    const K3Prep<NSET>* prep = reinterpret_cast<const K3Prep<NSET>*>(aux);
+    v4i Aop[NSET][2];
+    int sq4[NSET][NG];
+    float qsc[NSET][NG];
+#pragma unroll
+    for (int set = 0; set < NSET; ++set) {
+#pragma unroll
+      for (int mi = 0; mi < 2; ++mi) Aop[set][mi] = *reinterpret_cast<const v4i*>(&prep->aop[set][t16][lg][mi][0]);
+#pragma unroll
+      for (int g = 0; g < NG; ++g) {
+        sq4[set][g] = prep->sq4[set * 4 + lg][g];
+        qsc[set][g] = prep->qsc[set * 4 + lg][g];
+      }
+    }
+    const uint8_t* krd = kst + t16 * KROW + lg * 4;  // this lane's plane dwords of token t16 of a page
+    float mxl[NSET], mnl[NSET];
+#pragma unroll
+    for (int set = 0; set < NSET; ++set) {
+      mxl[set] = -INFINITY;
+      mnl[set] = INFINITY;
+    }
+    auto body = [&](int chunk, const uint32_t (&Sx)[4]) {
+      // all LDS reads of the chunk first (plane dwords of the four pages, rounding coefficients), then arithmetic
+      uint32_t Pj[4][3];
+      float sgj[4][NG], egj[4][NG];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint8_t* rp = krd + j * 16 * KROW;
+        Pj[j][0] = *reinterpret_cast<const uint32_t*>(rp);
+        Pj[j][1] = *reinterpret_cast<const uint32_t*>(rp + 16);
+        Pj[j][2] = *reinterpret_cast<const uint32_t*>(rp + 32);
+        const uint32_t sw = Sx[j];
+        sgj[j][0] = bf16_to_f32((uint16_t)(sw & 0xffffu));
+        egj[j][0] = prep->eps[sw & 0x7fu];
+        if (NG == 2) {
+          sgj[j][NG - 1] = bf16_to_f32((uint16_t)(sw >> 16));
+          egj[j][NG - 1] = prep->eps[(sw >> 16) & 0x7fu];
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t P0 = Pj[j][0], P1 = Pj[j][1], P2 = Pj[j][2];
+        v4i Bc[2], Br[2];
+        Bc[0][0] = (int)((P0 >> 5) & 0x07070707u);
+        Bc[0][1] = (int)((P0 >> 2) & 0x07070707u);
+        Bc[0][2] = (int)(((P0 << 1) & 0x06060606u) | ((P1 >> 7) & 0x01010101u));
+        Bc[0][3] = (int)((P1 >> 4) & 0x07070707u);
+        Bc[1][0] = (int)((P1 >> 1) & 0x07070707u);
+        Bc[1][1] = (int)(((P1 << 2) & 0x04040404u) | ((P2 >> 6) & 0x03030303u));
+        Bc[1][2] = (int)((P2 >> 3) & 0x07070707u);
+        Bc[1][3] = (int)(P2 & 0x07070707u);
+        if (NG == 2) {
+          // Bc[0] <- lanes 0-31 keep their first half, lanes 32-63 receive the second half of lane-32;
+          // Bc[1] <- lanes 0-31 receive the first half of lane+32, lanes 32-63 keep their second half
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const auto sw = __builtin_amdgcn_permlane32_swap((uint32_t)Bc[0][e], (uint32_t)Bc[1][e], false, false);
+            Bc[0][e] = (int)sw[0];
+            Bc[1][e] = (int)sw[1];
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            Br[u][e] = (int)__builtin_amdgcn_perm(0x01000000u, 0x0000ff00u, (uint32_t)Bc[u][e]);
+        // per-token scales (both groups) and the rounding coefficient
+        float sg[NG], eg[NG];
+#pragma unroll
+        for (int g = 0; g < NG; ++g) {
+          sg[g] = sgj[j][g];
+          eg[g] = egj[j][g];
+        }
+        const int tok = chunk * 64 + 16 * j + t16;
+        const bool valid = tok < n;
+#pragma unroll
+        for (int set = 0; set < NSET; ++set) {
+          float score = 0.f;
+          const v4i zero = {0, 0, 0, 0};
+          if (NG == 2) {
+#pragma unroll
+            for (int g = 0; g < NG; ++g) {
+              const v4i Dc = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][g], Bc[g], zero, 0, 0, 0);
+              const v4i Dr = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][g], Br[g], zero, 0, 0, 0);
+              const int xc = (((Dc[2] << 8) + Dc[1]) << 8) + Dc[0] - sq4[set][g];
+              const int xr = (Dr[2] << 8) + Dr[1];
+              const float v = __builtin_fmaf(eg[g], (float)xr, (float)xc);
+              score = __builtin_fmaf(v, sg[g] * qsc[set][g], score);
+            }
+          } else {
+            v4i Dc = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][0], Bc[0], zero, 0, 0, 0);
+            v4i Dr = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][0], Br[0], zero, 0, 0, 0);
+            Dc = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][1], Bc[1], Dc, 0, 0, 0);
+            Dr = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][1], Br[1], Dr, 0, 0, 0);
+            const int xc = (((Dc[2] << 8) + Dc[1]) << 8) + Dc[0] - sq4[set][0];
+            const int xr = (Dr[2] << 8) + Dr[1];
+            const float v = __builtin_fmaf(eg[0], (float)xr, (float)xc);
+            score = __builtin_fmaf(v, sg[0] * qsc[set][0], score);
+          }
+          const int h = set * 4 + lg;
+          if ((G % 4 == 0) || h < G) {
+            sc[h * L + tok] = valid ? score : -INFINITY;
+            mxl[set] = fmaxf(mxl[set], valid ? score : -INFINITY);
+            mnl[set] = fminf(mnl[set], valid ? score : INFINITY);
+          }
+        }
+      }
+    };
+    // at most Lds::LMAX / 64 / NW chunks per wavefront: straight-line code, so that the wait for a chunk's
+    // loads leaves the loads of the following chunks in flight
+#pragma unroll
+    for (int it = 0; it < MAXIT; ++it) {
+      const int chunk = wave + it * NW;
+      prefetch_v(it);
+      if (chunk < nch_cover) {
+        set_wave_prio(3 - it);  // wavefronts that are behind get the issue slots first
+        KBuf& cur = (it & 1) ? Kb : Ka;
+        stash_k(cur);
+        wave_lds_fence();
+        uint32_t Sc[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) Sc[j] = cur.s[j];
+        if (it + 2 < MAXIT && chunk + 2 * NW < nch_cover) cur = issue_k(chunk + 2 * NW);
+        body(chunk, Sc);
+        wave_lds_fence();
+      }
+    }
+    // lanes of 16-lane row lg hold the running extrema of head set*4 + lg: reduce inside the rows (lane 15 of
+    // a row ends up with the row's result) and publish them
+#pragma unroll
+    for (int set = 0; set < NSET; ++set) {
+      float a = mxl[set], c = -mnl[set];
+      JF_DPP_ROW_REDUCE(a, op_fmax, float, -INFINITY);
+      JF_DPP_ROW_REDUCE(c, op_fmax, float, -INFINITY);
+      const int h = set * 4 + lg;
+      if (t16 == 15 && h < G) {
+        red_f[wave][h] = a;
+        red_f[wave][G + h] = -c;
+      }
+    }
+  } else {
+    // INT4 keys, int8-Q model on v_mfma_i32_16x16x64_i8: exact nibble codes (offset 8 removed through the
+    // per-block constant), int32 block sums, the reference's four-term fp32 rescale in its order
+    // (int8tc_qk_scores.cu:455-468).  Lane (token, k-block lg) spreads the 16 channels 64*m + 16*lg .. +15 of
+    // both 64-channel spans m; its accumulator registers are the four 32-channel blocks of head lg.
+    const QInt8F<NSET>* qsh = reinterpret_cast<const QInt8F<NSET>*>(aux);
+    v4i Aop[NSET][2];
+    int sum8[NSET][4];
+    float qs[NSET][4];
+#pragma unroll
+    for (int set = 0; set < NSET; ++set) {
+#pragma unroll
+      for (int mi = 0; mi < 2; ++mi) Aop[set][mi] = *reinterpret_cast<const v4i*>(&qsh->aop[set][t16][lg][mi][0]);
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+        sum8[set][kk] = qsh->sum8[set * 4 + lg][kk];
+        qs[set][kk] = qsh->qs[set * 4 + lg][kk];
+      }
+    }
+    const uint8_t* krd = kst + t16 * KROW + lg * 8;
+    float mxl[NSET], mnl[NSET];
+#pragma unroll
+    for (int set = 0; set < NSET; ++set) {
+      mxl[set] = -INFINITY;
+      mnl[set] = INFINITY;
+    }
+    auto body = [&](int chunk, const uint32_t (&Sx)[4]) {
+      v2u Xj[4][2];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint8_t* rp = krd + j * 16 * KROW;
+        Xj[j][0] = *reinterpret_cast<const v2u*>(rp);
+        Xj[j][1] = *reinterpret_cast<const v2u*>(rp + 32);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        v4i Bm[2];
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi) {
+          const uint32_t x0 = Xj[j][mi][0], x1 = Xj[j][mi][1];
+          Bm[mi] = (v4i){(int)((x0 >> 4) & 0x0f0f0f0fu), (int)(x0 & 0x0f0f0f0fu), (int)((x1 >> 4) & 0x0f0f0f0fu), (int)(x1 & 0x0f0f0f0fu)};
+        }
+        const float ks = bf16_to_f32((uint16_t)Sx[j]);
+        const int tok = chunk * 64 + 16 * j + t16;
+        const bool valid = tok < n;
+#pragma unroll
+        for (int set = 0; set < NSET; ++set) {
+          const v4i zero = {0, 0, 0, 0};
+          v4i Dq = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][0], Bm[0], zero, 0, 0, 0);
+          Dq = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][1], Bm[1], Dq, 0, 0, 0);
+          float sacc = (float)(Dq[0] - sum8[set][0]) * qs[set][0];
+#pragma unroll
+          for (int kk = 1; kk < 4; ++kk) sacc = __builtin_fmaf((float)(Dq[kk] - sum8[set][kk]), qs[set][kk], sacc);
+          const float a = __fmul_rn(__fmul_rn(sacc, ks), p.attn_scale);
+          const int h = set * 4 + lg;
+          if ((G % 4 == 0) || h < G) {
+            sc[h * L + tok] = valid ? a : -INFINITY;
+            mxl[set] = fmaxf(mxl[set], valid ? a : -INFINITY);
+            mnl[set] = fminf(mnl[set], valid ? a : INFINITY);
+          }
+        }
+      }
+    };
+#pragma unroll
+    for (int it = 0; it < MAXIT; ++it) {
+      const int chunk = wave + it * NW;
+      prefetch_v(it);
+      if (chunk < nch_cover) {
+        set_wave_prio(3 - it);
+        KBuf& cur = (it & 1) ? Kb : Ka;
+        stash_k(cur);
+        wave_lds_fence();
+        uint32_t Sc[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) Sc[j] = cur.s[j];
+        if (it + 2 < MAXIT && chunk + 2 * NW < nch_cover) cur = issue_k(chunk + 2 * NW);
+        body(chunk, Sc);
+        wave_lds_fence();
+      }
+    }
+#pragma unroll
+    for (int set = 0; set < NSET; ++set) {
+      float a = mxl[set], c = -mnl[set];
+      JF_DPP_ROW_REDUCE(a, op_fmax, float, -INFINITY);
+      JF_DPP_ROW_REDUCE(c, op_fmax, float, -INFINITY);
+      const int h = set * 4 + lg;
+      if (t16 == 15 && h < G) {
+        red_f[wave][h] = a;
+        red_f[wave][G + h] = -c;
+      }
+    }
+  }
+
+  if (clk && tid == 0) clk[9] = clock64();  // wavefront 0 finished its chunks
+  if (clk && lane == 0) atomicMax(&tmax_sh, (unsigned long long)clock64());
+  __builtin_amdgcn_s_setprio(0);
+  // split extrema per head; fixed-point exponent of the V scales; selection buckets
+  if constexpr (HAS_V) {
+    uint32_t vm0 = 0u, vm1 = 0u;
+#pragma unroll
+    for (int i = 0; i < VSPT; ++i) {
+      vm0 = max(vm0, vsw[i] & 0x7fffu);
+      vm1 = max(vm1, (vsw[i] >> 16) & 0x7fffu);
+    }
+    vm0 = wave_max_u(vm0);
+    vm1 = wave_max_u(vm1);
+    if (lane == 0) {
+      vmax_sh[wave][0] = vm0;
+      vmax_sh[wave][1] = vm1;
+    }
+  }
+  lds_barrier();  // phase A complete: the query constants are dead, their space becomes the histograms
+  if (clk && tid == 0) { clk[8] = clock64(); clk[5] = (long long)tmax_sh; }
+  if (p.scores)  // validation output
+    for (int i = tid; i < G * n_cover; i += NT) {
+      const int h = i / n_cover, t = i - h * n_cover;
+      p.scores[(head0 + h) * (size_t)p.max_S + s0 + t] = sc[h * L + t];
+    }
+  if constexpr (MODE == FS_STAGE_A)
+    if (p.scores_only) return;
+  if constexpr (HAS_TOPK)
+    for (int i = tid; i < Lds::HIST / 4; i += NT) hist[i] = 0;
+  if (tid < G) {
+    float m = red_f[0][tid], lo = red_f[0][G + tid];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) {
+      m = fmaxf(m, red_f[w][tid]);
+      lo = fminf(lo, red_f[w][G + tid]);
+    }
+    m_sh[tid] = m;
+    // bucket of a score: min(255, (m - s) * 255 / (m - lo)), bucket 0 = largest; monotone in s
+    const float range = m - lo;
+    const float iw = (range > 0.f && isfinite(range)) ? 254.99f / range : 0.f;
+    bin_a_sh[tid] = -iw;
+    bin_b_sh[tid] = isfinite(m) ? m * iw : 0.f;
+  }
+  if (HAS_V && tid >= 64 && tid < 64 + NG) {
+    const int g = tid - 64;
+    uint32_t vb = vmax_sh[0][g];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) vb = max(vb, vmax_sh[w][g]);
+    const float v = bf16_to_f32((uint16_t)vb);
+    int e = 0;
+    if (v > 0.f && isfinite(v)) (void)frexpf(v, &e);  // v = f * 2^e, f in [0.5, 1)
+    e_sh[g] = 22 - e;                                 // v * 2^E in [2^21, 2^22)
+  }
+  lds_barrier();
+  if (clk && tid == 0) clk[1] = clock64();
+
+  // ------------------------------------------------------------------ phase B: P.V on v_mfma_i32_16x16x64_i8
+  // p = exp(s - m_split) is known exactly because phase A is complete, so w = p * v_scale is converted to
+  // 22-bit fixed point once (fma with 2^23); its three bytes, balanced around zero, are rows (limb, head) of
+  // the A operand.  Lane = token builds one 16-byte row per scale group (limb-major, then a constant 1 that
+  // becomes the all-ones row), and ds_read_b64_tr_b8 turns 8 token rows into the per-row byte runs the MFMA
+  // wants.  V codes are staged packed in wavefront-private LDS and transposed by ds_read_b64_tr_b4 (16
+  // tokens of one channel pair per lane), then spread.  sum_t w_t*(code - off) = sum_t w_t*code - off*sum_t w_t:
+  // the ones row gives sum_t code (needed because the limbs are balanced), a ones B tile gives sum_t w_t.
+  // Every accumulation is an exact integer.  The same pass drops every score into one of 256 linear buckets
+  // per (head, half of the split) for the candidate selection.
+  int E[NG];
+#pragma unroll
+  for (int g = 0; g < NG; ++g) E[g] = HAS_V ? __builtin_amdgcn_readfirstlane(e_sh[g]) : 0;
+  v4i acc[NSET][NTILE], accw[NSET][NG];
+#pragma unroll
+  for (int set = 0; set < NSET; ++set) {
+#pragma unroll
+    for (int t = 0; t < NTILE; ++t) acc[set][t] = (v4i){0, 0, 0, 0};
+#pragma unroll
+    for (int g = 0; g < NG; ++g) accw[set][g] = (v4i){0, 0, 0, 0};
+  }
+  float lsum[G], nml[G], bin_a[G], bin_b[G];
+#pragma unroll
+  for (int h = 0; h < G; ++h) {
+    lsum[h] = 0.f;
+    nml[h] = uniform_f(-(m_sh[h] * LOG2E));
+    bin_a[h] = uniform_f(bin_a_sh[h]);
+    bin_b[h] = uniform_f(bin_b_sh[h]);
+  }
+  const int r16 = lane & 15, kb4 = lane >> 4;
+  // transposed weight read: 16-lane group kb4 fetches the rows of tokens 16*kb4 .. +15; the lane pair (2j, 2j+1)
+  // supplies the two halves of the row that must land in byte j, i.e. of the token whose byte position in the
+  // V operand (see below) is j
+  const int tr_tok = (((r16 >> 1) & 3) << 1) | ((r16 >> 3) & 1);
+  const uint8_t* wrow = wl + (kb4 * 16 + tr_tok) * 16 + (r16 & 1) * 8;
+  const int seg_chunks = L / 64 / SEG;  // chunks per emission segment
+  auto body_v = [&](int chunk, uint32_t vsw) {
+    const int t = chunk * 64 + lane;
+    float vsf[NG];
+    vsf[0] = ldexpf(bf16_to_f32((uint16_t)(vsw & 0xffffu)), E[0]);
+    if (NG == 2) vsf[NG - 1] = ldexpf(bf16_to_f32((uint16_t)(vsw >> 16)), E[NG - 1]);
+    int* hb = hist + ((SEG == 1) ? 0 : (chunk / seg_chunks) * (Lds::H16 ? 128 : 256));
+    const bool tv = t < n;
+    uint32_t bits[NSET * 4][NG];
+#pragma unroll
+    for (int h = 0; h < NSET * 4; ++h) {
+      if (h < G) {
+        const float s = sc[h * L + t];
+        // masked positions hold -inf: their weight is exactly zero
+        const float pw = __builtin_amdgcn_exp2f(__builtin_fmaf(s, LOG2E, nml[h]));
+        lsum[h] += pw;
+#pragma unroll
+        for (int g = 0; g < NG; ++g) bits[h][g] = __builtin_bit_cast(uint32_t, __builtin_fmaf(pw, vsf[g], 8388608.0f));
+        if constexpr (HAS_TOPK) {
+          const uint32_t bin = (uint32_t)__builtin_amdgcn_fmed3f(__builtin_fmaf(s, bin_a[h], bin_b[h]), 0.f, 255.f);
+          if (Lds::H16) {
+            if (tv) atomicAdd(hb + ((h * (SEG * 256) + (int)bin) >> 1), (bin & 1u) ? 0x10000 : 1);
+          } else {
+            if (tv) atomicAdd(hb + h * (SEG * 256) + (int)bin, 1);
+          }
+        }
+      } else {
+#pragma unroll
+        for (int g = 0; g < NG; ++g) bits[h][g] = 0x4b000000u;
+      }
+    }
+    if constexpr (!HAS_V) return;  // Stage A alone: the weights' sums and the selection buckets were all
+#pragma unroll
+    for (int g = 0; g < NG; ++g)
+#pragma unroll
+      for (int set = 0; set < NSET; ++set) {
+        const uint32_t h0 = bits[set * 4 + 0][g], h1 = bits[set * 4 + 1][g], h2 = bits[set * 4 + 2][g], h3 = bits[set * 4 + 3][g];
+        const uint32_t T01 = __builtin_amdgcn_perm(h1, h0, 0x05010400u);  // h0.b0 h1.b0 h0.b1 h1.b1
+        const uint32_t U01 = __builtin_amdgcn_perm(h1, h0, 0x0c0c0602u);  // h0.b2 h1.b2 0 0
+        const uint32_t T23 = __builtin_amdgcn_perm(h3, h2, 0x05010400u);
+        const uint32_t U23 = __builtin_amdgcn_perm(h3, h2, 0x0c0c0602u);
+        v4i row;
+        row[0] = (int)(__builtin_amdgcn_perm(T23, T01, 0x05040100u) ^ 0x80808080u);  // limb 0 of heads 0..3, balanced
+        row[1] = (int)(__builtin_amdgcn_perm(T23, T01, 0x07060302u) ^ 0x80808080u);  // limb 1
+        row[2] = (int)(U01 | (U23 << 16));                                           // limb 2 (< 128)
+        row[3] = 1;                                                                  // row 12: ones; 13..15: zero
+        *reinterpret_cast<v4i*>(wl + ((g * NSET + set) * 64 + lane) * 16) = row;
+      }
+    wave_lds_fence();
+    v4i A[NG][NSET];
+#pragma unroll
+    for (int g = 0; g < NG; ++g)
+#pragma unroll
+      for (int set = 0; set < NSET; ++set) {
+        const uint8_t* src = wrow + (g * NSET + set) * 1024;
+        const v2i x0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i*)(src));
+        const v2i x1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i*)(src + 128));
+        A[g][set] = (v4i){x0[0], x0[1], x1[0], x1[1]};
+      }
+    const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
+#pragma unroll
+    for (int g = 0; g < NG; ++g)
+#pragma unroll
+      for (int set = 0; set < NSET; ++set)
+        accw[set][g] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[g][set], ones, accw[set][g], 0, 0, 0);
+    // the nibble spread of a transposed V dword yields tokens 0,2,4,6 | 1,3,5,7 | 8,10,12,14 | 9,11,13,15 of the
+    // lane group's 16 tokens: token r sits in byte (r&8) | ((r&1)<<2) | ((r>>1)&3)
+    const uint8_t* vrow = vst + lane * VROW;
+    if (V2) {
+#pragma unroll
+      for (int qc = 0; qc < 4; ++qc) {
+        const v2i x = __builtin_amdgcn_ds_read_tr4_b64_v2i32((__attribute__((address_space(3))) v2i*)(vrow + 8 * qc));
+        const uint32_t x0 = (uint32_t)x[0], x1 = (uint32_t)x[1], y0 = x0 >> 4, y1 = x1 >> 4;
+        // the upper code of every nibble stays where it is: tile 2*qc accumulates 4 * code (undone in `combine`)
+        const v4i Ba = {(int)(x0 & 0x0c0c0c0cu), (int)(y0 & 0x0c0c0c0cu), (int)(x1 & 0x0c0c0c0cu), (int)(y1 & 0x0c0c0c0cu)};
+        const v4i Bb = {(int)(x0 & 0x03030303u), (int)(y0 & 0x03030303u), (int)(x1 & 0x03030303u), (int)(y1 & 0x03030303u)};
+        const int g = (NG == 1) ? 0 : (qc >> 1);
+#pragma unroll
+        for (int set = 0; set < NSET; ++set) {
+          acc[set][2 * qc] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[g][set], Ba, acc[set][2 * qc], 0, 0, 0);
+          acc[set][2 * qc + 1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[g][set], Bb, acc[set][2 * qc + 1], 0, 0, 0);
+        }
+      }
+    } else {
+      const int vx = 16 * ((lane >> 2) & 3);  // quarter swap of this lane's row
+#pragma unroll
+      for (int qc = 0; qc < 8; ++qc) {
+        const v2i x = __builtin_amdgcn_ds_read_tr4_b64_v2i32((__attribute__((address_space(3))) v2i*)(vrow + (Lds::VSWZ ? ((8 * qc) ^ vx) : 8 * qc)));
+        const uint32_t x0 = (uint32_t)x[0], x1 = (uint32_t)x[1];
+        const v4i Bv = {(int)(x0 & 0x0f0f0f0fu), (int)((x0 >> 4) & 0x0f0f0f0fu),
+                        (int)(x1 & 0x0f0f0f0fu), (int)((x1 >> 4) & 0x0f0f0f0fu)};
+        const int g = (NG == 1) ? 0 : (qc >> 2);
+#pragma unroll
+        for (int set = 0; set < NSET; ++set)
+          acc[set][qc] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[g][set], Bv, acc[set][qc], 0, 0, 0);
+      }
+    }
+    wave_lds_fence();
+  };
+  auto stash_v = [&](const VBuf& vbuf) {
+#pragma unroll
+    for (int i = 0; i < VLD; ++i) {
+      if (Lds::VSWZ) {
+        *reinterpret_cast<v4u*>(vst + vl_lds[i]) = vbuf.r[i];  // 16-byte aligned with the unpadded pitch
+      } else {
+        v2u* dst = reinterpret_cast<v2u*>(vst + vl_lds[i]);
+        dst[0] = (v2u){vbuf.r[i][0], vbuf.r[i][1]};
+        dst[1] = (v2u){vbuf.r[i][2], vbuf.r[i][3]};
+      }
+    }
+  };
+#pragma unroll
+  for (int it = 0; it < MAXIT; ++it) {
+    const int chunk = wave + it * NW;
+    if (chunk < nch) {
+      set_wave_prio(3 - it);
+      uint32_t vw = 0u;
+      if constexpr (HAS_V) {
+        VBuf& cur = (it & 1) ? Vb : Va;
+        stash_v(cur);
+        vw = cur.w;
+        if (it + 2 < MAXIT && chunk + 2 * NW < nch) cur = issue_v(chunk + 2 * NW);
+      }
+      body_v(chunk, vw);
+    }
+  }
+  __builtin_amdgcn_s_setprio(0);
+#pragma unroll
+  for (int h = 0; h < G; ++h) {
+    const float ls = wave_sum(lsum[h]);
+    if (lane == 0) lsum_sh[wave][h] = ls;  // summed in wavefront order below: run-to-run deterministic
+  }
+  lds_barrier();
+  if (clk && tid == 0) clk[2] = clock64();
+
+  // ---- sum of the integer accumulators over the wavefronts: LDS integer atomics into one array in the staging
+  // area (dead now: every wavefront has passed the barrier above), zeroed here, filled after the cut search while
+  // the candidates are emitted, read by `combine` at the end.  Integer sums: exact and independent of the order.
+  // D layout: row r of a tile sits in lane 16*(r>>2) + column, register r&3; rows are (limb, head), row 12 is the
+  // ones row.  Element (set, register r, component c, lane l) lives at xacc[((set*AR + r)*4 + c)*64 + l].
+  int* xacc = reinterpret_cast<int*>(stage);
+  if constexpr (HAS_V)
+    for (int i = tid; i < Lds::XACC / 4; i += NT) xacc[i] = 0;
+  auto add_acc = [&](int set) {
+#pragma unroll
+    for (int r = 0; r < AR; ++r) {
+      const v4i v = (r < NTILE) ? acc[set][r < NTILE ? r : 0] : accw[set][r >= NTILE ? r - NTILE : 0];
+      int* dst = xacc + ((set * AR + r) * 4) * 64 + lane;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) atomicAdd(dst + c * 64, v[c]);
+    }
+  };
+  auto combine = [&](int set) {
+    // thread -> (tile, head, column)
+    for (int i = tid; i < 4 * D; i += NT) {
+      const int col = i & 15, hh = (i >> 4) & 3, tile = i >> 6;
+      const int h = set * 4 + hh;
+      if (h >= G) continue;
+      int d;
+      if (V2) {
+        const int e = ((col & 1) ? 0 : 2) + (tile & 1);
+        d = (tile >> 1) * 32 + (col >> 1) * 4 + e;
+      } else {
+        d = tile * 16 + 2 * (col >> 1) + (1 - (col & 1));
+      }
+      const int g = (NG == 1) ? 0 : (d / (D / NG));
+      const int* ta = xacc + ((set * AR + tile) * 4) * 64;          // limb l of head hh: component hh, lane 16*l + col
+      const int* wa = xacc + ((set * AR + NTILE + g) * 4) * 64;    // weight sums: any column of the all-ones tile
+      int i0 = ta[hh * 64 + col], i1 = ta[hh * 64 + 16 + col], i2 = ta[hh * 64 + 32 + col], cs = ta[48 + col];
+      if (V2 && !(tile & 1)) {  // even INT2 tiles hold four times their sums (exact multiples)
+        i0 >>= 2;
+        i1 >>= 2;
+        i2 >>= 2;
+        cs >>= 2;
+      }
+      const int w0 = wa[hh * 64], w1 = wa[hh * 64 + 16], w2 = wa[hh * 64 + 32];   // |sum| < 2^24: no overflow
+      const long long wsum = (long long)w2 * 65536ll + (long long)w1 * 256ll + (long long)w0 + 32896ll * 64ll * (long long)nch;
+      const long long tot = (long long)i2 * 65536ll + (long long)i1 * 256ll + (long long)i0 + 32896ll * (long long)cs - (long long)VOFF * wsum;
+      p.part_o[(part_base + (size_t)h * p.n_splits) * D + d] = (float)ldexp((double)tot, -E[g]);
+    }
+  };
+
+  // ------------------------------------------------------------------ phase C: candidates of the split
+  // The merge kernel needs a superset of the split's top Kt = min(top_k, n) scores per head that fits the
+  // candidate buffer (Kcap entries), in ascending position.  From the histograms: the smallest bucket index
+  // `cut` with count(bucket <= cut) >= Kt.  If that count fits, every position whose bucket is <= cut is
+  // emitted, one wavefront per (head, half of the split), the second half starting where the first one's count
+  // ends.  Otherwise (heavily tied scores) one wavefront falls back to an exact radix select over the keys.
+  const int Kcap = p.Kc;
+  const int Kt = min(p.top_k, n);
+  for (int h = wave; HAS_TOPK && h < G; h += NW) {
+    const int* h0 = hist + h * (SEG * 256) / (Lds::H16 ? 2 : 1);
+    // lane l owns buckets 4l .. 4l+3 (ascending bucket = descending score) of every segment's histogram
+    int cs[SEG][4], c[4], mine = 0;
+#pragma unroll
+    for (int sg = 0; sg < SEG; ++sg) {
+      if (Lds::H16) {
+        const uint32_t w0 = (uint32_t)h0[sg * 128 + 2 * lane], w1 = (uint32_t)h0[sg * 128 + 2 * lane + 1];
+        cs[sg][0] = (int)(w0 & 0xffffu);
+        cs[sg][1] = (int)(w0 >> 16);
+        cs[sg][2] = (int)(w1 & 0xffffu);
+        cs[sg][3] = (int)(w1 >> 16);
+      } else {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) cs[sg][u] = h0[sg * 256 + 4 * lane + u];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      c[u] = 0;
+#pragma unroll
+      for (int sg = 0; sg < SEG; ++sg) c[u] += cs[sg][u];
+      mine += c[u];
+    }
+    const int incl = wave_incl_scan_i(mine);
+    int run = incl - mine;
+    int cut = -1, tot = 0;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int before = run;
+      run += c[u];
+      if (cut < 0 && before < Kt && run >= Kt) {
+        cut = 4 * lane + u;
+        tot = run;
+      }
+    }
+    const unsigned long long who = __ballot(cut >= 0);
+    bool ok = false;
+    if (who != 0ull) {
+      const int src = __ffsll((long long)who) - 1;
+      cut = __builtin_amdgcn_readlane(cut, src);
+      tot = __builtin_amdgcn_readlane(tot, src);
+      ok = tot <= Kcap;
+    }
+    if (!ok) cut = 255;
+    // entries every segment emits: its histogram summed over the buckets <= cut
+    int off = 0;
+#pragma unroll
+    for (int sg = 0; sg < SEG; ++sg) {
+      int part = 0;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) part += (4 * lane + u <= cut) ? cs[sg][u] : 0;
+      part = wave_sum_i(part);
+      if (lane == 0) segoff_sh[h][sg] = off;
+      off += part;
+    }
+    if (lane == 0) {
+      segoff_sh[h][SEG] = off;
+      cut_sh[h] = cut;
+      exact_sh[h] = ok ? 0 : 1;
+    }
+  }
+  lds_barrier();
+  if (clk && tid == 0) clk[6] = clock64();
+#pragma unroll
+  for (int set = 0; set < NSET; ++set)
+    if constexpr (HAS_V) add_acc(set);
+  for (int hs = wave; HAS_TOPK && hs < G * SEG; hs += NW) {
+    const int h = hs / SEG, seg = hs % SEG;
+    const float* srow = sc + h * L;
+    uint32_t* ck = p.cand_key + (part_base + (size_t)h * p.n_splits) * Kcap;
+    int32_t* ci = p.cand_idx + (part_base + (size_t)h * p.n_splits) * Kcap;
+    if (!exact_sh[h]) {
+      // bucket(s) <= cut  <=>  not (s * ba + bb >= cut + 1): the bucket is the floor of that value clamped to
+      // [0, 255]; with cut = 255 every position qualifies
+      const int cut = cut_sh[h];
+      const float thr = uniform_f((cut >= 255) ? INFINITY : (float)(cut + 1));
+      const float ba = uniform_f(bin_a_sh[h]), bb = uniform_f(bin_b_sh[h]);
+      const int tb = seg * (L / SEG);
+      const int te = min(n, (seg + 1) * (L / SEG));
+      // the emitted total is at most Kcap by construction of the cut
+      int count = __builtin_amdgcn_readfirstlane(segoff_sh[h][seg]);
+      // unused slots hold key 0 (no score maps to it); the planned total is known, so the head's wavefronts
+      // share the padding and its stores leave before the emission's
+      const int etot = min(Kcap, __builtin_amdgcn_readfirstlane(segoff_sh[h][SEG]));
+      for (int i = etot + seg * 64 + lane; i < Kcap; i += SEG * 64) ck[i] = 0u;
+      uint8_t* ckb = reinterpret_cast<uint8_t*>(ck);
+      uint8_t* cib = reinterpret_cast<uint8_t*>(ci);
+      for (int t0 = tb; t0 < te; t0 += 512) {
+        float kk[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int t = t0 + 64 * u + lane;
+          kk[u] = (t < te) ? srow[t] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int t = t0 + 64 * u + lane;
+          const bool above = (t < te) && !(__builtin_fmaf(kk[u], ba, bb) >= thr);
+          const unsigned long long ma = __builtin_amdgcn_ballot_w64(above);
+          const uint32_t pos = (uint32_t)count + __builtin_amdgcn_mbcnt_hi((uint32_t)(ma >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)ma, 0u));
+          if (above && pos < (uint32_t)Kcap) {  // the bound only matters for non-finite scores
+            *reinterpret_cast<uint32_t*>(ckb + (size_t)(pos * 4u)) = score_key(kk[u]);
+            *reinterpret_cast<int32_t*>(cib + (size_t)(pos * 4u)) = s0 + t;
+          }
+          count += __popcll(ma);
+        }
+      }
+      if (seg == SEG - 1) {
+        if (lane == 0) p.cand_cnt[part_base + (size_t)h * p.n_splits] = min(Kcap, count);
+        for (int i = count + lane; i < etot; i += 64) ck[i] = 0u;  // (only if a segment emitted less than planned)
+      }
+    } else if (seg == 0) {
+      // exact fallback: 8-bit radix select over the order-preserving keys (bits shared by every key skipped),
+      // then the keys above the K-th and the lowest-position ties that fill the quota
+      int* rh = reinterpret_cast<int*>(stage + Lds::XACC + wave * 1024);
+      uint32_t T = 0;
+      int quota = 0;
+      uint32_t kmin = 0xffffffffu, kmax = 0u;
+      for (int t = lane; t < n; t += 64) {
+        const uint32_t k = score_key(srow[t]);
+        kmin = min(kmin, k);
+        kmax = max(kmax, k);
+      }
+      kmin = wave_min_u(kmin);
+      kmax = wave_max_u(kmax);
+      const uint32_t diff = kmin ^ kmax;
+      if (diff == 0u) {  // every key equal: the lowest positions win
+        T = kmax;
+        quota = Kt;
+      } else {
+        int bits_left = 32 - __clz((int)diff);  // number of low bits that vary
+        uint32_t prefix = (bits_left == 32) ? 0u : (kmax >> bits_left);
+        int k_rem = Kt;
+        while (bits_left > 0) {
+          const int nb = min(8, bits_left);
+          const int shift = bits_left - nb;
+          const uint32_t dmask = (1u << nb) - 1u;
+          for (int i = lane; i < 256; i += 64) rh[i] = 0;
+          const bool first = (bits_left == 32);
+          const int hi_shift = first ? 0 : bits_left;
+          for (int t0 = 0; t0 < n; t0 += 64) {
+            const int t = t0 + lane;
+            const uint32_t k = (t < n) ? score_key(srow[t]) : 0u;
+            const bool inpre = (t < n) && (first || ((k >> hi_shift) == prefix));
+            if (inpre) atomicAdd(&rh[(int)((k >> shift) & dmask)], 1);
+          }
+          // lane l owns bins 255-4l .. 252-4l (descending), so a prefix scan over lanes counts the bins above
+          const int c3 = rh[255 - 4 * lane], c2 = rh[254 - 4 * lane], c1 = rh[253 - 4 * lane], c0 = rh[252 - 4 * lane];
+          const int mine = c0 + c1 + c2 + c3;
+          const int e3 = wave_incl_scan_i(mine) - mine;  // keys in bins above 255-4l
+          const int e2 = e3 + c3, e1 = e2 + c2, e0 = e1 + c1;
+          int cut = -1, above = 0;
+          if (e3 < k_rem && k_rem <= e3 + c3) { cut = 255 - 4 * lane; above = e3; }
+          else if (e2 < k_rem && k_rem <= e2 + c2) { cut = 254 - 4 * lane; above = e2; }
+          else if (e1 < k_rem && k_rem <= e1 + c1) { cut = 253 - 4 * lane; above = e1; }
+          else if (e0 < k_rem && k_rem <= e0 + c0) { cut = 252 - 4 * lane; above = e0; }
+          const unsigned long long who = __ballot(cut >= 0);
+          const int src = __ffsll((long long)who) - 1;
+          cut = __builtin_amdgcn_readlane(cut, src);
+          above = __builtin_amdgcn_readlane(above, src);
+          prefix = (prefix << nb) | (uint32_t)cut;
+          k_rem -= above;
+          bits_left = shift;
+        }
+        T = prefix;
+        quota = k_rem;
+      }
+      int count = 0, base_tie = 0;
+      for (int t0 = 0; t0 < n; t0 += 64) {
+        const int t = t0 + lane;
+        const uint32_t k = (t < n) ? score_key(srow[t]) : 0u;
+        const bool above = (t < n) && (k > T), tie = (t < n) && (k == T);
+        const unsigned long long ma = __ballot(above), mt = __ballot(tie);
+        const int pa = count + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(ma >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)ma, 0u));
+        const int pt = base_tie + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(mt >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mt, 0u));
+        if (above || (tie && pt < quota)) {
+          const int pos = pa + min(pt, quota);
+          if (pos < Kcap) {
+            ck[pos] = k;
+            ci[pos] = s0 + t;
+          }
+        }
+        count += __popcll(ma);
+        base_tie += __popcll(mt);
+      }
+      count += min(base_tie, quota);
+      if (lane == 0) p.cand_cnt[part_base + (size_t)h * p.n_splits] = min(Kcap, count);
+      for (int i = count + lane; i < Kcap; i += 64) ck[i] = 0u;
+    }
+  }
+  lds_barrier();
+  if (clk && tid == 0) clk[3] = clock64();
+
+  float lfin = 0.f;
+  if (tid < G) {
+#pragma unroll
+    for (int w = 0; w < NW; ++w) lfin += lsum_sh[w][tid];
+  }
+#pragma unroll
+  for (int set = 0; set < NSET; ++set)
+    if constexpr (HAS_V) combine(set);
+  if (tid < G) {
+    p.part_m[part_base + (size_t)tid * p.n_splits] = m_sh[tid];
+    p.part_l[part_base + (size_t)tid * p.n_splits] = lfin;
+  }
+  if (clk && tid == 0) clk[4] = clock64();
+}
+
+// ---------------------------------------------------------------------------------------------------
+constexpr int MG_MAX_SPLITS = 256;
+constexpr int MG_BINS = 1024;      // linear score buckets of the threshold search
+constexpr int MG_LIST = 1024;      // members of the cut bucket resolved by rank counting
+constexpr int MG_BT_LDS = 4096;    // block-table entries cached in LDS (65536 positions)
+
+// Launch 2: one workgroup per (sequence, query head).
+//   1. split statistics -> M, l, o_hat
+//   2. the K-th largest candidate key tau (and how many keys equal to tau still belong to the top K): the
+//      candidates are dropped into MG_BINS linear score buckets between the smallest and the largest, a scan
+//      finds the bucket that holds the K-th largest, and the few members of that bucket are ranked against
+//      each other (a bisection over the key range covers the case of more than MG_LIST members)
+//   3. ordered compaction of the winners (key > tau, or key == tau while the quota lasts; candidates are stored
+//      in position order, so ties resolve to the lower position and the output is ascending)
+//   4. slots, softmax weights, and the pre-correction terms over the winners' V rows.
+// The first MG_REGK * MG_THREADS candidates stay in registers from a single load; anything beyond that is
+// re-read from global memory in every pass.
+// Two shapes: 1024 threads x 8 register-resident candidates each (up to 8192 candidates, the common case;
+// the phases are chains of LDS round trips and barriers, so more, lighter threads beat fewer, heavier ones)
+// and 1024 x 32 for first-stage parts that exceed it.
+// PARTIAL = true is the first stage of the two-stage merge: blockIdx.z selects a run of mg_spp candidate
+// lists, steps 2 and 3 run on those alone and the winners (still in position order) are written out as one
+// new candidate list; the final merge (PARTIAL = false, mg_parts > 1) reads these lists instead of the
+// scan's.  The top K of a union is the top K of the parts' top K's, ties included: a candidate that a part
+// drops is beaten by K candidates of that part.
+template <int MODE, int VBITS, int NG, int MG_THREADS, int MG_REGK, bool PARTIAL>
+__global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) {
+  static_assert(!(PARTIAL && MODE == FS_STAGE_B), "Stage B alone selects nothing");
+  constexpr int MG_WAVES = MG_THREADS / 64;
+  constexpr int VP = D * VBITS / 8;
+  constexpr int VOFF = 1 << (VBITS - 1);
+  constexpr int DW = VP / 4;            // dwords per V row
+  constexpr int CPD = 32 / VBITS;       // codes per dword
+  constexpr int WPI = 64 / DW;          // winners per wavefront instruction
+  __shared__ int hist[MG_BINS];
+  __shared__ uint32_t lkey[MG_LIST];
+  __shared__ float coef_sh[MG_MAX_SPLITS];
+  __shared__ int cnt_sh[MG_MAX_SPLITS];
+  __shared__ int bt_sh[MG_BT_LDS];
+  __shared__ uint32_t win_key[FS_MAX_TOPK];
+  __shared__ int win_idx[FS_MAX_TOPK];
+  __shared__ int win_slot[FS_MAX_TOPK];
+  __shared__ float win_w[FS_MAX_TOPK];
+  __shared__ uint32_t cnt_a[MG_REGK / 4 * MG_WAVES];  // packed (winners, ties) per (group, wavefront)
+  __shared__ float red_sh[MG_THREADS / D][D];
+  __shared__ float old_sh[MG_WAVES][D];
+  __shared__ float w_sh[MG_WAVES];
+  __shared__ float wred_f[MG_WAVES];
+  __shared__ uint32_t wred_u[MG_WAVES];
+  __shared__ int wred_i[MG_WAVES], wred_j[MG_WAVES];
+  __shared__ int lcount_sh, cut_sh, above_sh, quota_sh;
+  __shared__ uint32_t tau_sh;
+
+  const int b = blockIdx.x, hq = blockIdx.y, tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const size_t bh = (size_t)b * p.H_q + hq;
+  const int NS = p.n_splits, K = p.top_k;
+  const int hkv = hq / (p.H_q / p.H_kv);
+  // candidate lists of this workgroup: NL lists of capacity Kc
+  const bool staged = !PARTIAL && p.mg_parts > 1;
+  const int part = PARTIAL ? (int)blockIdx.z : 0;
+  const int l0 = PARTIAL ? part * p.mg_spp : 0;
+  // (Stage B alone: the winners are an input, there are no candidate lists)
+  const int NL = (MODE == FS_STAGE_B) ? 0 : (PARTIAL ? min(p.mg_spp, NS - l0) : (staged ? p.mg_parts : NS));
+  const int Kc = staged ? K : p.Kc;
+  const uint32_t* ck = staged ? p.key2 + bh * p.mg_parts * K : p.cand_key + (bh * NS + l0) * Kc;
+  const int32_t* ci = staged ? p.idx2 + bh * p.mg_parts * K : p.cand_idx + (bh * NS + l0) * Kc;
+  const int32_t* cc = staged ? p.cnt2 + bh * p.mg_parts : p.cand_cnt + bh * NS + l0;
+  const int64_t* bt = p.block_table + (size_t)b * p.max_blocks;
+  int64_t* out_idx = p.topk_idx + bh * (size_t)K;
+  int64_t* out_slot = p.topk_slots + bh * (size_t)K;
+  const int flat = NL * Kc;
+  const int rounds = (flat + MG_THREADS - 1) / MG_THREADS;
+  const int nblk_lds = min(p.max_blocks, MG_BT_LDS);
+
+  long long* mclk = (p.phase_clock && !PARTIAL) ? p.phase_clock + (size_t)p.B * p.H_kv * p.n_splits * 10 + bh * 8 : nullptr;
+  if (mclk && tid == 0) mclk[0] = clock64();
+
+  // ---- everything that does not depend on anything else is requested first, in the order of its use
+  float pm = -INFINITY, pl = 0.f;
+  int my_cnt = 0;
+  if (!PARTIAL && tid < NS) {
+    pm = p.part_m[bh * NS + tid];
+    pl = p.part_l[bh * NS + tid];
+  }
+  if (tid < NL) my_cnt = cc[tid];
+  float blend_new = 0.f, blend_hat = 0.f;
+  if (MODE == FS_FULL && !PARTIAL && p.blend_out && tid < D) blend_new = bf16_to_f32(p.blend_o_new[bh * D + tid]);
+  // The first MG_REGK * MG_THREADS candidates live in registers: group g = r / 4 of a thread holds the four
+  // consecutive candidates (g * MG_THREADS + tid) * 4 + (r % 4), fetched with one 16-byte load.  Candidate
+  // order = (group, thread, element).  Slots past a list's count hold key 0 (written by the producer).
+  static_assert(MG_REGK % 4 == 0, "register candidates come in groups of four");
+  constexpr int NGRP = MG_REGK / 4;
+  const int rreg = min((flat + 4 * MG_THREADS - 1) / (4 * MG_THREADS), NGRP) * 4;  // register slots in use (uniform)
+  uint32_t kreg[MG_REGK];
+  int ireg[MG_REGK];
+#pragma unroll
+  for (int g = 0; g < NGRP; ++g) {
+    const int f4 = (g * MG_THREADS + tid) * 4;
+    v4u k4 = {0u, 0u, 0u, 0u};
+    if (4 * g < rreg && f4 < flat) k4 = *reinterpret_cast<const v4u*>(ck + f4);  // flat is a multiple of 4
+#pragma unroll
+    for (int j = 0; j < 4; ++j) kreg[4 * g + j] = k4[j];
+  }
+#pragma unroll
+  for (int g = 0; g < NGRP; ++g) {
+    const int f4 = (g * MG_THREADS + tid) * 4;
+    v4i i4 = {0, 0, 0, 0};
+    if (4 * g < rreg && f4 < flat) i4 = *reinterpret_cast<const v4i*>(ci + f4);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) ireg[4 * g + j] = i4[j];
+  }
+  if (tid < NL) cnt_sh[tid] = my_cnt;
+  // o_hat: the thread groups of 128 take the splits round-robin (first terms requested now)
+  constexpr int PO_PRE = 2, PO_GRP = MG_THREADS / D;
+  float po[PO_PRE];
+  {
+    const int d = tid & (D - 1), q4 = tid >> 7;
+#pragma unroll
+    for (int i = 0; i < PO_PRE; ++i) {
+      const int sp = q4 + PO_GRP * i;
+      po[i] = (MODE != FS_STAGE_A && !PARTIAL && sp < NS) ? p.part_o[(bh * NS + sp) * D + d] : 0.f;
+    }
+  }
+  if (!PARTIAL)
+    for (int i = tid; i < nblk_lds; i += MG_THREADS) bt_sh[i] = (int)bt[i];
+  for (int i = tid; i < MG_BINS; i += MG_THREADS) hist[i] = 0;
+  if (tid == 0) lcount_sh = 0;
+
+  // ---- split statistics: M, coefficients e^{m_i - M}, l, o_hat
+  if (!PARTIAL) {
+    const float v = wave_max(pm);
+    if (lane == 0) wred_f[wave] = v;
+  }
+  lds_barrier();
+  if (mclk && tid == 0) mclk[6] = clock64();
+  float M = -INFINITY;
+  if (!PARTIAL) {
+#pragma unroll
+    for (int w = 0; w < MG_WAVES; ++w) M = fmaxf(M, wred_f[w]);
+    if (!isfinite(M)) M = 0.f;
+    const float coef = (pm == -INFINITY) ? 0.f : __expf(pm - M);
+    if (tid < NS) coef_sh[tid] = coef;
+    const float v = wave_sum(pl * coef);  // fixed reduction tree: deterministic
+    lds_barrier();                      // wred_f was read above
+    if (lane == 0) wred_f[wave] = v;
+  }
+  int total = 0;
+  for (int s2 = 0; s2 < NL; ++s2) total += cnt_sh[s2];
+  lds_barrier();
+  if (mclk && tid == 0) mclk[7] = clock64();
+  float inv_z = 0.f;
+  if (!PARTIAL) {
+    float lsum = 0.f;
+#pragma unroll
+    for (int w = 0; w < MG_WAVES; ++w) lsum += wred_f[w];
+    inv_z = (lsum > 0.f) ? 1.0f / lsum : 0.f;
+    if (tid == 0 && p.softmax_m) {
+      p.softmax_m[bh] = M;
+      p.softmax_inv_z[bh] = inv_z;
+    }
+  }
+  if constexpr (!PARTIAL && MODE != FS_STAGE_A) {
+    // o_hat: four thread groups take every fourth split, then a fixed-order sum
+    const int d = tid & (D - 1), q4 = tid >> 7;
+    float o = 0.f;
+#pragma unroll
+    for (int i = 0; i < PO_PRE; ++i) {
+      const int sp = q4 + PO_GRP * i;
+      if (sp < NS) o = __builtin_fmaf(po[i], coef_sh[sp], o);
+    }
+    // the remaining splits eight at a time: the loads of a batch are in flight together, the sum keeps its order
+    constexpr int PO_B = 8;
+    for (int sp0 = q4 + PO_GRP * PO_PRE; sp0 < NS; sp0 += PO_GRP * PO_B) {
+      float v[PO_B];
+#pragma unroll
+      for (int u = 0; u < PO_B; ++u) {
+        const int sp = sp0 + PO_GRP * u;
+        v[u] = (sp < NS) ? p.part_o[(bh * NS + sp) * D + d] : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < PO_B; ++u) {
+        const int sp = sp0 + PO_GRP * u;
+        if (sp < NS) o = __builtin_fmaf(v[u], coef_sh[sp], o);
+      }
+    }
+    red_sh[q4][d] = o;
+    lds_barrier();
+    if (tid < D) {
+      float o2 = red_sh[0][tid];
+#pragma unroll
+      for (int q = 1; q < PO_GRP; ++q) o2 += red_sh[q][tid];  // fixed order
+      blend_hat = o2 * inv_z;
+      p.o_hat[bh * D + tid] = blend_hat;
+    }
+  }
+  if (mclk && tid == 0) mclk[1] = clock64();
+
+  // key of candidate f in pass-over-all-candidates loops: registers first, global memory beyond
+  auto key_of = [&](int r) -> uint32_t {
+    const int f = r * MG_THREADS + tid;
+    return (f < flat) ? ck[f] : 0u;
+  };
+  // number of candidates with key >= x (x > 0), identical in every thread
+  auto count_ge = [&](uint32_t x) -> int {
+    int c = 0;
+#pragma unroll
+    for (int r = 0; r < MG_REGK; ++r)
+      if (r < rreg) c += __popcll(__builtin_amdgcn_ballot_w64(kreg[r] >= x));
+    for (int r = MG_REGK; r < rounds; ++r) c += __popcll(__builtin_amdgcn_ballot_w64(key_of(r) >= x));
+    lds_barrier();
+    if (lane == 0) wred_i[wave] = c;
+    lds_barrier();
+    int t = 0;
+#pragma unroll
+    for (int w = 0; w < MG_WAVES; ++w) t += wred_i[w];
+    return t;
+  };
+
+  uint32_t tau = 0;
+  int quota = 0;
+  const bool take_all = (total <= K);
+  if (!take_all) {
+    // range of the candidate keys
+    uint32_t kmin = 0xffffffffu, kmax = 0u;
+#pragma unroll
+    for (int r = 0; r < MG_REGK; ++r)
+      if (r < rreg && kreg[r] != 0u) { kmin = min(kmin, kreg[r]); kmax = max(kmax, kreg[r]); }
+    for (int r = MG_REGK; r < rounds; ++r) {
+      const uint32_t k = key_of(r);
+      if (k != 0u) { kmin = min(kmin, k); kmax = max(kmax, k); }
+    }
+    kmin = wave_min_u(kmin);
+    kmax = wave_max_u(kmax);
+    if (lane == 0) { wred_u[wave] = kmin; wred_i[wave] = (int)kmax; }
+    lds_barrier();
+#pragma unroll
+    for (int w = 0; w < MG_WAVES; ++w) { kmin = min(kmin, wred_u[w]); kmax = max(kmax, (uint32_t)wred_i[w]); }
+    const float hi = key_to_score(kmax), lo = key_to_score(kmin);
+    const float range = hi - lo;
+    const float iw = (range > 0.f && isfinite(range)) ? ((float)MG_BINS - 0.01f) / range : 0.f;
+    const float ba = -iw, bb = isfinite(hi) ? hi * iw : 0.f;
+    auto bin_of = [&](uint32_t k) -> int {
+      return (int)__builtin_amdgcn_fmed3f(__builtin_fmaf(key_to_score(k), ba, bb), 0.f, (float)(MG_BINS - 1));
+    };
+#pragma unroll
+    for (int r = 0; r < MG_REGK; ++r)
+      if (r < rreg && kreg[r] != 0u) atomicAdd(&hist[bin_of(kreg[r])], 1);
+    for (int r = MG_REGK; r < rounds; ++r) {
+      const uint32_t k = key_of(r);
+      if (k != 0u) atomicAdd(&hist[bin_of(k)], 1);
+    }
+    lds_barrier();
+    {
+      // thread t owns buckets BPT*t .. BPT*t + BPT-1 (bucket 0 = largest scores): which bucket holds the K-th largest
+      constexpr int BPT = MG_BINS / MG_THREADS;
+      int cb[BPT], mine = 0;
+#pragma unroll
+      for (int u = 0; u < BPT; ++u) {
+        cb[u] = hist[BPT * tid + u];
+        mine += cb[u];
+      }
+      const int incl = wave_incl_scan_i(mine);
+      if (lane == 63) wred_j[wave] = incl;
+      lds_barrier();
+      int run = incl - mine;
+      for (int w = 0; w < wave; ++w) run += wred_j[w];
+#pragma unroll
+      for (int u = 0; u < BPT; ++u) {
+        if (run < K && K <= run + cb[u]) { cut_sh = BPT * tid + u; above_sh = run; }
+        run += cb[u];
+      }
+    }
+    lds_barrier();
+    const int cut = cut_sh, need = K - above_sh;  // `need` of the cut bucket's members belong to the top K
+#pragma unroll
+    for (int r = 0; r < MG_REGK; ++r)
+      if (r < rreg && kreg[r] != 0u && bin_of(kreg[r]) == cut) {
+        const int i = atomicAdd(&lcount_sh, 1);
+        if (i < MG_LIST) lkey[i] = kreg[r];
+      }
+    for (int r = MG_REGK; r < rounds; ++r) {
+      const uint32_t k = key_of(r);
+      if (k != 0u && bin_of(k) == cut) {
+        const int i = atomicAdd(&lcount_sh, 1);
+        if (i < MG_LIST) lkey[i] = k;
+      }
+    }
+    lds_barrier();
+    const int m = lcount_sh;
+    if (m <= MG_LIST) {
+      // rank counting: the member with fewer than `need` larger members and at least `need` members >= it
+      for (int i = tid; i < m; i += MG_THREADS) {
+        const uint32_t k = lkey[i];
+        int gt = 0, ge = 0;
+        for (int j = 0; j < m; ++j) {
+          const uint32_t o = lkey[j];
+          gt += (o > k) ? 1 : 0;
+          ge += (o >= k) ? 1 : 0;
+        }
+        if (gt < need && need <= ge) {  // every thread that gets here writes the same pair
+          tau_sh = k;
+          quota_sh = need - gt;
+        }
+      }
+      lds_barrier();
+      tau = tau_sh;
+      quota = quota_sh;
+    } else {
+      // bisection over the key range: largest x with count(key >= x) >= K
+      uint32_t lo_k = kmin, hi_k = kmax;  // invariant: count_ge(lo_k) >= K
+      while (lo_k < hi_k) {
+        const uint32_t mid = lo_k + (hi_k - lo_k + 1u) / 2u;
+        if (count_ge(mid) >= K) lo_k = mid;
+        else hi_k = mid - 1u;
+      }
+      tau = lo_k;
+      quota = K - ((tau == 0xffffffffu) ? 0 : count_ge(tau + 1u));
+    }
+  }
+  if (mclk && tid == 0) mclk[2] = clock64();
+
+  // ---- ordered compaction.  Register candidates: every thread counts its winners and ties per group, a
+  // wavefront scan plus the wavefront totals in LDS give the thread's first place, and the thread places its
+  // (consecutive) candidates one after the other.  The owner of a winner stores its key and position.
+  int base_above = 0, base_tie = 0;
+  {
+    int cnt_g[NGRP];  // low half: winners, high half: ties of this thread in group g
+    int scan_g[NGRP];
+#pragma unroll
+    for (int g = 0; g < NGRP; ++g) {
+      int c = 0;
+      if (4 * g < rreg) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t key = kreg[4 * g + j];
+          const bool above = (key != 0u) && (take_all || key > tau), tie = (key != 0u) && !take_all && key == tau;
+          c += (above ? 1 : 0) + (tie ? 0x10000 : 0);
+        }
+      }
+      cnt_g[g] = c;
+      scan_g[g] = wave_incl_scan_i(c);  // at most 4 * 64 per half: no carry between the halves
+      if (lane == 63) cnt_a[g * MG_WAVES + wave] = (uint32_t)scan_g[g];
+    }
+    lds_barrier();
+    uint32_t run = 0u;  // packed totals of the groups before g (each half stays below 2^16: at most 32768 candidates)
+#pragma unroll
+    for (int g = 0; g < NGRP; ++g) {
+      uint32_t before = 0u, all = 0u;
+#pragma unroll
+      for (int w = 0; w < MG_WAVES; ++w) {
+        const uint32_t t = cnt_a[g * MG_WAVES + w];
+        before += (w < wave) ? t : 0u;
+        all += t;
+      }
+      if (4 * g < rreg) {
+        const uint32_t start = run + before + (uint32_t)(scan_g[g] - cnt_g[g]);
+        int pa = (int)(start & 0xffffu), pt = (int)(start >> 16);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t key = kreg[4 * g + j];
+          const bool above = (key != 0u) && (take_all || key > tau), tie = (key != 0u) && !take_all && key == tau;
+          if (above || (tie && pt < quota)) {
+            const int pos = pa + min(pt, quota);
+            if (pos < K) {
+              win_key[pos] = key;
+              win_idx[pos] = ireg[4 * g + j];
+            }
+          }
+          pa += above ? 1 : 0;
+          pt += tie ? 1 : 0;
+        }
+      }
+      run += all;
+    }
+    base_above = (int)(run & 0xffffu);
+    base_tie = (int)(run >> 16);
+    lds_barrier();
+  }
+  for (int r = MG_REGK; r < rounds; ++r) {  // candidates beyond the register-resident ones, one round at a time
+    const int f = r * MG_THREADS + tid;
+    const uint32_t key = key_of(r);
+    const bool above = (key != 0u) && (take_all || key > tau), tie = (key != 0u) && !take_all && key == tau;
+    const unsigned long long ma = __builtin_amdgcn_ballot_w64(above), mt = __builtin_amdgcn_ballot_w64(tie);
+    if (lane == 0) {
+      wred_i[wave] = __popcll(ma);
+      wred_j[wave] = __popcll(mt);
+    }
+    lds_barrier();
+    int pa = base_above + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(ma >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)ma, 0u));
+    int pt = base_tie + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(mt >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mt, 0u));
+    int tot_a = 0, tot_t = 0;
+#pragma unroll
+    for (int w = 0; w < MG_WAVES; ++w) {
+      if (w < wave) { pa += wred_i[w]; pt += wred_j[w]; }
+      tot_a += wred_i[w];
+      tot_t += wred_j[w];
+    }
+    if (above || (tie && pt < quota)) {
+      const int pos = pa + min(pt, quota);
+      if (pos < K) {
+        win_key[pos] = key;
+        win_idx[pos] = ci[f];
+      }
+    }
+    base_above += tot_a;
+    base_tie += tot_t;
+    lds_barrier();
+  }
+  int n_out = min(K, base_above + min(base_tie, quota));
+  if constexpr (MODE == FS_STAGE_B) {
+    // the winners are given (ascending positions, -1 padded, possibly none at all): their keys come from the
+    // caller's score tensor
+    n_out = p.topk_idx ? K : 0;
+    const int64_t s_len = max(0, min(p.max_S, p.seq_lens[b]));
+    for (int r = tid; r < n_out; r += MG_THREADS) {
+      const int64_t pos = p.topk_idx[bh * (size_t)K + r];
+      const bool ok = pos >= 0 && pos < s_len;
+      win_idx[r] = ok ? (int)pos : -1;
+      win_key[r] = ok ? score_key(p.scores_in[bh * (size_t)p.max_S + pos]) : 0u;
+    }
+    lds_barrier();
+  }
+  if (mclk && tid == 0) mclk[3] = clock64();
+  if (PARTIAL) {  // the winners become one candidate list of the final merge
+    const size_t lo = (bh * p.mg_parts + part) * (size_t)K;
+    for (int r = tid; r < K; r += MG_THREADS) {
+      p.key2[lo + r] = (r < n_out) ? win_key[r] : 0u;  // unused slots: key 0
+      if (r < n_out) p.idx2[lo + r] = win_idx[r];
+    }
+    if (tid == 0) p.cnt2[bh * p.mg_parts + part] = n_out;
+    return;
+  }
+
+  // one thread per winner: position, paged slot, softmax weight
+  for (int r = tid; r < K; r += MG_THREADS) {
+    int64_t position = -1, slot = -1;
+    int wslot = -1;
+    float ww = 0.f;
+    if (r < n_out && win_idx[r] >= 0) {
+      position = win_idx[r];
+      const int blk = (int)(position / BS);
+      if (blk < p.max_blocks) slot = (int64_t)((blk < nblk_lds) ? (int64_t)bt_sh[blk] : bt[blk]) * BS + (position % BS);
+      wslot = (slot >= 0 && slot < p.num_slots) ? (int)slot : -1;
+      ww = __expf(key_to_score(win_key[r]) - M) * inv_z;
+    }
+    if constexpr (MODE != FS_STAGE_B) {
+      out_idx[r] = position;
+      out_slot[r] = slot;
+    }
+    win_slot[r] = wslot;
+    win_w[r] = ww;
+  }
+  if constexpr (MODE == FS_STAGE_A) return;  // Stage A alone ends with the winners and the statistics
+  lds_barrier();
+  if (mclk && tid == 0) mclk[4] = clock64();
+
+  // ---- pre-correction over the winners.  One winner row per DW lanes: lane (w_in, dwi) holds dword dwi of
+  // the winner's packed V row (CPD codes) and accumulates its CPD channels; winners are visited in a fixed
+  // order, so the sums are run-to-run deterministic.  UNR rows per lane are requested before any is used.
+  const uint8_t* vbase = p.v_data + (size_t)hkv * p.num_slots * VP;
+  const uint8_t* vsbase = reinterpret_cast<const uint8_t*>(p.v_scales + (size_t)hkv * p.num_slots * NG);
+  const int dwi = lane % DW, w_in = lane / DW;
+  const int g_of_lane = (NG == 1) ? 0 : ((dwi * CPD) / (D / NG));
+  float acc[CPD];
+#pragma unroll
+  for (int c = 0; c < CPD; ++c) acc[c] = 0.f;
+  float accw = 0.f;
+  constexpr int UNR = (256 / (MG_WAVES * WPI) > 0) ? 256 / (MG_WAVES * WPI) : 1;  // 256 winners per pass
+  for (int k0 = wave * WPI; k0 < n_out; k0 += UNR * MG_WAVES * WPI) {
+    uint32_t word[UNR];
+    uint16_t sbits[UNR];
+    float wv[UNR];
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      const int k = k0 + u * MG_WAVES * WPI + w_in;
+      const int slot = (k < n_out) ? win_slot[k] : -1;
+      wv[u] = (slot >= 0) ? win_w[k] : 0.f;
+      const uint32_t sl = (uint32_t)max(slot, 0);
+      word[u] = *reinterpret_cast<const uint32_t*>(vbase + (size_t)(sl * (uint32_t)VP) + dwi * 4);
+      sbits[u] = *reinterpret_cast<const uint16_t*>(vsbase + (size_t)(sl * (uint32_t)(NG * 2)) + g_of_lane * 2);
+    }
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      const float ws = wv[u] * bf16_to_f32(sbits[u]);  // zero for padding rows
+      // byte `byte` of the dword holds its codes MSB first; channel of code c in the dword = dwi*CPD + c
+#pragma unroll
+      for (int c = 0; c < CPD; ++c) {
+        const int byte = c / (8 / VBITS), inb = c % (8 / VBITS);
+        const int code = (int)((word[u] >> (8 * byte + (8 - VBITS * (inb + 1)))) & ((1u << VBITS) - 1u)) - VOFF;
+        acc[c] = __builtin_fmaf(ws, (float)code, acc[c]);
+      }
+      if (dwi == 0) accw += wv[u];
+    }
+  }
+  // reduce over the WPI winners of a wavefront instruction (lanes with equal dwi): every exchange step halves
+  // the channels a lane is responsible for (the lane whose offset bit is clear keeps the lower half), so after
+  // log2(WPI) steps every lane holds the sums of CPD / WPI = 2 channels; then over wavefronts through LDS
+  {
+    int chan = dwi * CPD;
+    auto halve = [&](auto off_c, auto n_c) {
+      constexpr int OFF = decltype(off_c)::value, N = decltype(n_c)::value;
+      const bool upper = (lane & OFF) != 0;
+#pragma unroll
+      for (int i = 0; i < N / 2; ++i) {
+        if constexpr (OFF == 32) {  // one half-wave swap serves both directions
+          const auto sw = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(uint32_t, acc[i]), __builtin_bit_cast(uint32_t, acc[i + N / 2]), false, false);
+          acc[i] = __builtin_bit_cast(float, (uint32_t)sw[0]) + __builtin_bit_cast(float, (uint32_t)sw[1]);
+        } else {
+          const float keep = upper ? acc[i + N / 2] : acc[i];
+          const int send = __builtin_bit_cast(int, upper ? acc[i] : acc[i + N / 2]);
+          // lane ^ 8: rotation by 8 inside the 16-lane row; lane ^ 16: swizzle inside 32 lanes
+          const int recv = (OFF == 8) ? dpp_mov<0x128, 0xf>(0, send) : __builtin_amdgcn_ds_swizzle(send, 0x401F);
+          acc[i] = keep + __builtin_bit_cast(float, recv);
+        }
+      }
+      chan += upper ? N / 2 : 0;
+    };
+    static_assert(DW == 8 || DW == 16, "V rows of 32 or 64 bytes");
+    if constexpr (DW == 8) {
+      halve(std::integral_constant<int, 8>{}, std::integral_constant<int, CPD>{});
+      halve(std::integral_constant<int, 16>{}, std::integral_constant<int, CPD / 2>{});
+      halve(std::integral_constant<int, 32>{}, std::integral_constant<int, CPD / 4>{});
+    } else {
+      halve(std::integral_constant<int, 16>{}, std::integral_constant<int, CPD>{});
+      halve(std::integral_constant<int, 32>{}, std::integral_constant<int, CPD / 2>{});
+    }
+    static_assert(CPD / WPI == 2, "two channels per lane after the exchange");
+    old_sh[wave][chan] = acc[0];
+    old_sh[wave][chan + 1] = acc[1];
+    const float wsum = wave_sum(accw);  // only the dwi == 0 lanes hold weights
+    if (lane == 0) w_sh[wave] = wsum;
+  }
+  lds_barrier();
+  if (tid < D) {
+    float o = 0.f;
+#pragma unroll
+    for (int w = 0; w < MG_WAVES; ++w) o += old_sh[w][tid];  // fixed order
+    p.o_old[bh * D + tid] = o;
+    float wt = 0.f;
+#pragma unroll
+    for (int w = 0; w < MG_WAVES; ++w) wt += w_sh[w];  // fixed order: the same value in every thread
+    if (tid == 0) p.W[bh] = wt;
+    // the blend of jetfire_vllm/csrc/blend.cu:202-226 for callers that hold o_new already
+    if (MODE == FS_FULL && p.blend_out) p.blend_out[bh * D + tid] = f32_to_bf16(__builtin_fmaf(wt, blend_new, blend_hat) - o);
+  }
+  if (mclk && tid == 0) mclk[5] = clock64();
+}
+
+constexpr size_t LDS_BUDGET_2WG = 80 * 1024 - 512;    // two workgroups per CU (160 KB LDS)
+constexpr size_t LDS_BUDGET_1WG = 160 * 1024 - 1024;
+
+template <int SCHEME, int G, int NG>
+int lmax_for() {
+  using Lds = ScanLds<SCHEME, G, NG>;
+  const size_t budget = (G <= 4 && Lds::NW == 8) ? LDS_BUDGET_2WG : LDS_BUDGET_1WG;
+  const size_t fixed = Lds::AUX + Lds::stage_bytes() + 64 + 832;  // + static LDS of the kernel
+  long lm = (long)((budget - fixed) / (Lds::per_position() + 1));  // +1: page table (4 bytes per 16 positions)
+  lm = lm / 256 * 256;
+  if (lm > Lds::LMAX) lm = Lds::LMAX;
+  if (lm < 256) lm = 256;
+  return (int)lm;
+}
+
+inline int lmax_dispatch(int scheme, int G, int NG) {
+#define JF_LMAX_CASE(SCH, GG, NGG) if (scheme == SCH && G == GG && NG == NGG) return lmax_for<SCH, GG, NGG>()
+  JF_LMAX_CASE(JF_SCHEME_K3V2, 1, 1); JF_LMAX_CASE(JF_SCHEME_K3V2, 2, 1); JF_LMAX_CASE(JF_SCHEME_K3V2, 4, 1);
+  JF_LMAX_CASE(JF_SCHEME_K3V2, 8, 1); JF_LMAX_CASE(JF_SCHEME_K3V2, 16, 1);
+  JF_LMAX_CASE(JF_SCHEME_K3V2, 1, 2); JF_LMAX_CASE(JF_SCHEME_K3V2, 2, 2); JF_LMAX_CASE(JF_SCHEME_K3V2, 4, 2);
+  JF_LMAX_CASE(JF_SCHEME_K3V2, 8, 2); JF_LMAX_CASE(JF_SCHEME_K3V2, 16, 2);
+  JF_LMAX_CASE(JF_SCHEME_K4V4, 1, 1); JF_LMAX_CASE(JF_SCHEME_K4V4, 2, 1); JF_LMAX_CASE(JF_SCHEME_K4V4, 4, 1);
+  JF_LMAX_CASE(JF_SCHEME_K4V4, 8, 1); JF_LMAX_CASE(JF_SCHEME_K4V4, 16, 1);
+  JF_LMAX_CASE(JF_SCHEME_K3V4, 1, 1); JF_LMAX_CASE(JF_SCHEME_K3V4, 2, 1); JF_LMAX_CASE(JF_SCHEME_K3V4, 4, 1);
+  JF_LMAX_CASE(JF_SCHEME_K3V4, 8, 1); JF_LMAX_CASE(JF_SCHEME_K3V4, 16, 1);
+  JF_LMAX_CASE(JF_SCHEME_K4V2, 1, 1); JF_LMAX_CASE(JF_SCHEME_K4V2, 2, 1); JF_LMAX_CASE(JF_SCHEME_K4V2, 4, 1);
+  JF_LMAX_CASE(JF_SCHEME_K4V2, 8, 1); JF_LMAX_CASE(JF_SCHEME_K4V2, 16, 1);
+#undef JF_LMAX_CASE
+  return 256;
+}
+
+// Estimated microseconds of the merge (fitted on MI355X): a fixed part per launch plus a part proportional to
+// the candidates one workgroup visits.
+constexpr double kMergeFixed = 8.5, kPartialFixed = 7.5, kPerCand = 0.0004, kPerCandBig = 0.001;
+constexpr int MG_REG_CANDS = 8192;  // candidates the common merge shape keeps in registers
+inline double merge_pass_us(double fixed, long cands) {
+  return cands <= MG_REG_CANDS ? fixed + kPerCand * (double)cands : fixed + 1.5 + kPerCandBig * (double)cands;
+}
+
+// Two-stage merge when one workgroup per row would face more than MG_REG_CANDS candidates: the number of
+// parts (at most MG_REG_CANDS / top_k, so that the final merge keeps its candidates in registers, and at least
+// two lists per part) with the smallest estimated time.  parts == 1: single stage.
+inline double merge_plan(int rows, int ns, int kc, int top_k, int* parts_out, int* spp_out) {
+  *parts_out = 1;
+  *spp_out = ns;
+  const double wide = 1.5 * (top_k > 256 ? (double)top_k / 256.0 - 1.0 : 0.0);  // slots and pre-correction of the winners
+  double best = merge_pass_us(kMergeFixed, (long)ns * kc) + wide;
+  if ((long long)ns * kc <= MG_REG_CANDS || ns < 4) return best;
+  int cap = MG_REG_CANDS / top_k;
+  if (cap > ns / 2) cap = ns / 2;
+  for (int parts = 2; parts <= cap; ++parts) {
+    const int spp = (ns + parts - 1) / parts;
+    if ((ns + spp - 1) / spp != parts) continue;  // the same spp as a smaller number of parts
+    const long wgs = (long)(rows > 0 ? rows : 1) * parts;
+    const double rounds = (double)((wgs + 511) / 512);  // two workgroups per CU
+    const double us = kPartialFixed + rounds * (merge_pass_us(kPartialFixed, (long)spp * kc) - kPartialFixed) +
+                      merge_pass_us(kMergeFixed, (long)parts * top_k) + wide;
+    if (us < best) {
+      best = us;
+      *parts_out = parts;
+      *spp_out = spp;
+    }
+  }
+  return best;
+}
+
+inline void fused_plan(int scheme, int NG, int B, int H_q, int H_kv, int max_S, int top_k, int* L_out, int* ns_out,
+                       int* kc_out) {
+  const int G = H_q / H_kv;
+  const int units = B * H_kv > 0 ? B * H_kv : 1;
+  const int rows = B * H_q > 0 ? B * H_q : 1;
+  // One scan workgroup is resident per CU (256 CUs).  Among the split lengths that fit LDS pick the one with
+  // the smallest estimated time of scan + merge.  The constants are microseconds fitted to measurements on
+  // MI355X: a scan workgroup costs a fixed part plus a part proportional to the 64-position chunks each of
+  // its wavefronts works through; a last, partly filled round of workgroups runs faster than a full one; the
+  // merge costs a fixed part per launch plus a part proportional to the candidates one workgroup visits.
+  const int lmax = lmax_dispatch(scheme, G, NG);
+  const int nw = (G <= 4) ? 16 : 8;
+  const int kCUs = device_cus();
+  constexpr double kScanFixed = 8.5;
+  // one chunk per wavefront, all wavefronts; the mixed schemes are priced like the wider one
+  const double per_chunk = (scheme == JF_SCHEME_K3V2) ? 5.9 : 6.6;
+  int L = 256;
+  double best = -1.0;
+  for (int cand = 256; cand <= lmax; cand += 256) {
+    const long nsp = (max_S + cand - 1) / cand > 0 ? (max_S + cand - 1) / cand : 1;
+    if (nsp > MG_MAX_SPLITS && cand < lmax) continue;
+    const long nwg = nsp * units;
+    const long full = nwg / kCUs, rem = nwg % kCUs;
+    const double stream = per_chunk * (double)cand / (64.0 * nw);
+    double cost = (double)full * (kScanFixed + stream);
+    if (rem > 0) cost += kScanFixed + stream * (0.5 + 0.5 * (double)rem / kCUs);
+    const int kc = (top_k + FS_CAND_SLACK) < cand ? (top_k + FS_CAND_SLACK) : cand;
+    int parts, spp;
+    cost += merge_plan(rows, (int)nsp, kc, top_k, &parts, &spp);
+    if (best < 0.0 || cost <= best) {
+      best = cost;
+      L = cand;
+    }
+    if (cand >= max_S) break;
+  }
+  if (const int forced = g_force_split_len.load(std::memory_order_relaxed); forced > 0) {
+    L = (forced + 255) / 256 * 256;
+    if (L > lmax) L = lmax;
+    while ((max_S + L - 1) / L > MG_MAX_SPLITS && L < lmax) L += 256;
+  }
+  int ns = (max_S + L - 1) / L;
+  if (ns < 1) ns = 1;
+  *L_out = L;
+  *ns_out = ns;
+  const int cap = top_k + FS_CAND_SLACK;  // the split may emit a superset of its top-k (see phase C)
+  *kc_out = cap < L ? cap : L;
+}
+
+struct WsLayout {
+  size_t off_m, off_l, off_o, off_key, off_idx, off_cnt, off_key2, off_idx2, off_cnt2, total;
+};
+inline WsLayout ws_layout(int B, int H_q, int ns, int kc, int parts, int top_k) {
+  WsLayout w;
+  const size_t rows = (size_t)B * H_q;
+  size_t o = 0;
+  auto take = [&](size_t bytes) { size_t r = o; o += (bytes + 255) / 256 * 256; return r; };
+  w.off_m = take(rows * ns * 4);
+  w.off_l = take(rows * ns * 4);
+  w.off_o = take(rows * ns * D * 4);
+  w.off_key = take(rows * ns * kc * 4);
+  w.off_idx = take(rows * ns * kc * 4);
+  w.off_cnt = take(rows * ns * 4);
+  w.off_key2 = w.off_idx2 = w.off_cnt2 = 0;
+  if (parts > 1) {
+    w.off_key2 = take(rows * parts * top_k * 4);
+    w.off_idx2 = take(rows * parts * top_k * 4);
+    w.off_cnt2 = take(rows * parts * 4);
+  }
+  w.total = o + 256;
+  return w;
+}
+
+template <int MODE, int SCHEME, int G, int NG>
+int launch_scan(const FusedParams& p, hipStream_t st) {
+  const size_t smem = ScanLds<SCHEME, G, NG>::total(p.L);
+  auto kern = fused_scan_kernel<MODE, SCHEME, G, NG>;
+  // per instantiation: raise the dynamic-LDS limit only when it grows (launches may come from several threads)
+  static std::mutex attr_mu;
+  static size_t attr_smem = 0;
+  {
+    std::lock_guard<std::mutex> lock(attr_mu);
+    if (smem > attr_smem) {
+      JF_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+      attr_smem = smem;
+    }
+  }
+  std::unique_lock<std::mutex> plock(g_prof_mu, std::defer_lock);
+  bool prof = false;
+  if (g_prof.armed) {  // (read without the lock: arming happens-before the launches a benchmark times)
+    plock.lock();
+    prof = g_prof.armed && g_prof.used + 2 <= (int)g_prof.ev.size();
+    if (!prof) plock.unlock();
+  }
+  if (prof) JF_CHECK_HIP(hipEventRecord(g_prof.ev[g_prof.used], st));
+  hipLaunchKernelGGL(kern, dim3(p.n_splits, p.H_kv, p.B), dim3(ScanLds<SCHEME, G, NG>::NT), smem, st, p);
+  JF_CHECK_LAUNCH();
+  if (prof) {
+    JF_CHECK_HIP(hipEventRecord(g_prof.ev[g_prof.used + 1], st));
+    g_prof.used += 2;
+  }
+  return JF_OK;
+}
+
+inline bool known_scheme(int scheme) {
+  return scheme == JF_SCHEME_K3V2 || scheme == JF_SCHEME_K4V4 || scheme == JF_SCHEME_K3V4 || scheme == JF_SCHEME_K4V2;
+}
+inline int scheme_ng(int scheme, int group_size) { return (scheme == JF_SCHEME_K3V2) ? D / group_size : 1; }
+
+
+// The whole step on caller-provided workspace memory; every public entry point of the fused forms ends here.
+// MODE FS_FULL: all arguments as in jf_fused_scan_topk.  FS_STAGE_A: the value side, o_hat, o_old_unnorm, W are
+// unused; top_k == 0 asks for the scores alone (then nothing but `scores` is written and no workspace is needed).
+// FS_STAGE_B: q and the key side are unused, `scores_in` and `topk_idx` are inputs (topk_idx may be NULL: o_hat only,
+// zeros for the pre-correction terms), topk_slots is unused.
+template <int MODE>
+static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_t* k_data,
+                     const uint16_t* k_scales, const uint8_t* v_data, const uint16_t* v_scales,
+                     const int64_t* block_table, const int32_t* seq_lens, int B, int H_q, int H_kv,
+                     int max_S, int max_blocks, int64_t num_slots, int block_size, float attn_scale,
+                     int top_k, int64_t* topk_idx, int64_t* topk_slots, float* o_hat,
+                     float* o_old_unnorm, float* W, float* softmax_m, float* softmax_inv_z, float* scores,
+                     const float* scores_in, const uint16_t* blend_o_new, uint16_t* blend_out, void* workspace,
+                     size_t workspace_bytes, void* stream) {
+  JF_CHECK_ARG(known_scheme(scheme), "fused_scan: unknown scheme %d", scheme);
+  JF_CHECK_ARG(MODE == FS_FULL || scheme == JF_SCHEME_K3V2 || scheme == JF_SCHEME_K4V4,
+               "fused_scan: the stage-wise forms take the K3V2 or K4V4 side formats");
+  JF_CHECK_ARG((blend_o_new == nullptr) == (blend_out == nullptr), "fused_scan: o_new and out go together");
+  JF_CHECK_ARG(B >= 0 && H_q > 0 && H_kv > 0 && max_S >= 0 && H_q % H_kv == 0, "fused_scan: bad shape");
+  const int G = H_q / H_kv;
+  JF_CHECK_ARG(G == 1 || G == 2 || G == 4 || G == 8 || G == 16, "fused_scan: GQA group %d not in {1,2,4,8,16}", G);
+  JF_CHECK_ARG(block_size == 16, "fused_scan only supports block_size=16");
+  JF_CHECK_ARG(group_size == 64 || group_size == 128, "fused_scan: group_size must be 64 or 128 (got %d)", group_size);
+  JF_CHECK_ARG(scheme == JF_SCHEME_K3V2 || group_size == 128,
+               "fused_scan: the INT4 sides (int8-Q keys, INT4 values) need group_size 128");
+  const bool scores_only = (MODE == FS_STAGE_A) && top_k == 0;
+  if (scores_only) top_k = 32;  // (any valid width: the plan depends on it, the kernel stops before using it)
+  JF_CHECK_ARG(is_pow2(top_k) && top_k >= 32 && top_k <= FS_MAX_TOPK,
+               "fused_scan: unsupported top_k=%d (supported: 32,64,128,256,512,1024; larger widths use the split-form operators)", top_k);
+  JF_CHECK_ARG(max_S <= 262144, "fused_scan: max_S=%d exceeds supported limit (262144)", max_S);
+  JF_CHECK_ARG((int64_t)max_blocks * block_size >= max_S, "fused_scan: block_table does not cover max_S");
+  JF_CHECK_ARG(num_slots > 0 && num_slots <= (1ll << 25), "fused_scan: num_slots out of range (at most 2^25: row offsets are 32-bit)");
+  JF_CHECK_ARG((softmax_m == nullptr) == (softmax_inv_z == nullptr), "fused_scan: softmax_m and softmax_inv_z go together");
+  if (B == 0) return JF_OK;
+  JF_CHECK_ARG(block_table && seq_lens, "fused_scan: null input");
+  if (MODE != FS_STAGE_B) {
+    JF_CHECK_ARG(q && k_data && k_scales, "fused_scan: null input");
+    JF_CHECK_ARG(((uintptr_t)k_data & 15) == 0 && ((uintptr_t)q & 15) == 0, "fused_scan: q and k_data must be 16-byte aligned");
+    JF_CHECK_ARG(scores_only ? scores != nullptr : (topk_idx && topk_slots), "fused_scan: null output");
+  }
+  if (MODE != FS_STAGE_A) {
+    JF_CHECK_ARG(v_data && v_scales, "fused_scan: null input");
+    JF_CHECK_ARG(((uintptr_t)v_data & 15) == 0 && ((uintptr_t)v_scales & 3) == 0,
+                 "fused_scan: v_data must be 16-byte aligned, v_scales 4-byte aligned");
+    JF_CHECK_ARG(o_hat && o_old_unnorm && W, "fused_scan: null output");
+  }
+  if (MODE == FS_STAGE_B) JF_CHECK_ARG(scores_in != nullptr, "fused_scan: null scores");
+  const int NGv = scheme_ng(scheme, group_size);
+  FusedParams p;
+  p.q = q; p.k_data = k_data; p.k_scales = k_scales; p.v_data = v_data; p.v_scales = v_scales;
+  p.block_table = block_table; p.seq_lens = seq_lens;
+  p.B = B; p.H_q = H_q; p.H_kv = H_kv; p.max_S = max_S; p.max_blocks = max_blocks; p.num_slots = num_slots;
+  p.attn_scale = attn_scale; p.top_k = top_k;
+  fused_plan(scheme, NGv, B, H_q, H_kv, max_S, top_k, &p.L, &p.n_splits, &p.Kc);
+  JF_CHECK_ARG(p.n_splits <= MG_MAX_SPLITS, "fused_scan: too many splits (%d > %d)", p.n_splits, MG_MAX_SPLITS);
+  merge_plan(B * H_q, p.n_splits, p.Kc, top_k, &p.mg_parts, &p.mg_spp);
+  if (MODE == FS_STAGE_B) { p.mg_parts = 1; p.mg_spp = p.n_splits; }
+  const WsLayout wl = ws_layout(B, H_q, p.n_splits, p.Kc, p.mg_parts, top_k);
+  if (!scores_only) {
+    JF_CHECK_ARG(workspace && workspace_bytes >= wl.total, "fused_scan: workspace too small (%zu < %zu)", workspace_bytes, wl.total);
+    JF_CHECK_ARG(((uintptr_t)workspace & 255) == 0, "fused_scan: workspace must be 256-byte aligned");
+  }
+  uint8_t* ws = reinterpret_cast<uint8_t*>(workspace);
+  p.scores = (MODE == FS_STAGE_B) ? nullptr : scores;
+  p.scores_in = scores_in;
+  p.scores_only = scores_only ? 1 : 0;
+  p.part_m = reinterpret_cast<float*>(ws + wl.off_m);
+  p.part_l = reinterpret_cast<float*>(ws + wl.off_l);
+  p.part_o = reinterpret_cast<float*>(ws + wl.off_o);
+  p.cand_key = reinterpret_cast<uint32_t*>(ws + wl.off_key);
+  p.cand_idx = reinterpret_cast<int32_t*>(ws + wl.off_idx);
+  p.cand_cnt = reinterpret_cast<int32_t*>(ws + wl.off_cnt);
+  p.key2 = reinterpret_cast<uint32_t*>(ws + wl.off_key2);
+  p.idx2 = reinterpret_cast<int32_t*>(ws + wl.off_idx2);
+  p.cnt2 = reinterpret_cast<int32_t*>(ws + wl.off_cnt2);
+  p.topk_idx = topk_idx; p.topk_slots = topk_slots; p.o_hat = o_hat; p.o_old = o_old_unnorm; p.W = W;
+  p.softmax_m = softmax_m; p.softmax_inv_z = softmax_inv_z;
+  p.blend_o_new = blend_o_new; p.blend_out = blend_out;
+  p.phase_clock = g_phase_clock.load(std::memory_order_relaxed);
+  hipStream_t st = (hipStream_t)stream;
+  int rc = JF_OK;
+#define JF_FUSED_CASE(SCH, GG, NGG) rc = launch_scan<MODE, SCH, GG, NGG>(p, st)
+#define JF_FUSED_BY_G(SCH, NGG)                        \
+  switch (G) {                                         \
+    case 1: JF_FUSED_CASE(SCH, 1, NGG); break;         \
+    case 2: JF_FUSED_CASE(SCH, 2, NGG); break;         \
+    case 4: JF_FUSED_CASE(SCH, 4, NGG); break;         \
+    case 8: JF_FUSED_CASE(SCH, 8, NGG); break;         \
+    default: JF_FUSED_CASE(SCH, 16, NGG); break;       \
+  }
+  if (scheme == JF_SCHEME_K3V2) {
+    if (NGv == 2) JF_FUSED_BY_G(JF_SCHEME_K3V2, 2) else JF_FUSED_BY_G(JF_SCHEME_K3V2, 1)
+  } else if (scheme == JF_SCHEME_K4V4) {
+    JF_FUSED_BY_G(JF_SCHEME_K4V4, 1)
+  } else if constexpr (MODE == FS_FULL) {  // the mixed pairs exist in the one-pass form only
+    if (scheme == JF_SCHEME_K3V4) JF_FUSED_BY_G(JF_SCHEME_K3V4, 1) else JF_FUSED_BY_G(JF_SCHEME_K4V2, 1)
+  }
+#undef JF_FUSED_BY_G
+#undef JF_FUSED_CASE
+  if (rc != JF_OK || scores_only) return rc;
+  dim3 mgrid(B, H_q);
+  if (p.mg_parts > 1) {  // first stage: every part's top_k, as new candidate lists (the same kernel for every form)
+    const dim3 pgrid(B, H_q, p.mg_parts);
+    if ((long long)p.mg_spp * p.Kc > MG_REG_CANDS) hipLaunchKernelGGL((fused_merge_kernel<FS_FULL, 4, 1, 1024, 32, true>), pgrid, dim3(1024), 0, st, p);
+    else hipLaunchKernelGGL((fused_merge_kernel<FS_FULL, 4, 1, 1024, 8, true>), pgrid, dim3(1024), 0, st, p);
+    JF_CHECK_LAUNCH();
+  }
+  const bool big = (MODE != FS_STAGE_B) &&
+                   (p.mg_parts > 1 ? (long long)p.mg_parts * top_k : (long long)p.n_splits * p.Kc) > MG_REG_CANDS;
+#define JF_MERGE(VB, NGG)                                                                                            \
+  do {                                                                                                               \
+    if (big) hipLaunchKernelGGL((fused_merge_kernel<MODE, VB, NGG, 1024, 32, false>), mgrid, dim3(1024), 0, st, p); \
+    else hipLaunchKernelGGL((fused_merge_kernel<MODE, VB, NGG, 1024, 8, false>), mgrid, dim3(1024), 0, st, p);       \
+  } while (0)
+  if constexpr (MODE == FS_STAGE_A) {  // no value rows are read: one instantiation serves every format
+    JF_MERGE(4, 1);
+  } else if (scheme % 10 == 2) {  // INT2 values
+    if (NGv == 2) JF_MERGE(2, 2);
+    else JF_MERGE(2, 1);
+  } else {
+    JF_MERGE(4, 1);
+  }
+#undef JF_MERGE
+  JF_CHECK_LAUNCH();
+  return JF_OK;
+}
+
+}  // namespace
+}  // namespace jf

@@ -127,7 +127,10 @@ __global__ __launch_bounds__(SV_THREADS) void weighted_v_split_kernel(
 //     rs   = max_t |pv_t| / 127,  pq_t = clamp(rint(pv_t * (1 / rs)), -127, 127)   (rs == 0: pq = 0)
 //     o_hat[d] += f32(sum_t pq_t * (nibble_t,d - 8)) * rs
 // with an exact int32 sum per tile and an fp32 running sum over the tiles in ascending order.
-// grid (TQ_SPLITS, H_kv, B); thread = output channel d; the 32-lane quarters of the workgroup take the heads in turn.
+// grid (TQ_SPLITS * sub_count, H_kv, B); thread = output channel d; the 32-lane quarters of the workgroup take the heads
+// in turn.  A range's tiles are dealt out in runs to `sub_count` workgroups (the tiles themselves, and with them every
+// quantisation step, stay those of the reference's eight ranges; only the association of the fp32 sum over tiles
+// changes, at the 1e-7 level), so that a long context fills the chip.
 constexpr int TQ_SPLITS = 8;
 constexpr int TQ_TILE = 2 * BS;
 template <int G>
@@ -135,12 +138,13 @@ __global__ __launch_bounds__(SV_THREADS) void tile_quantised_v_split_kernel(
     const float* __restrict__ scores, const float* __restrict__ softmax_m, const float* __restrict__ softmax_inv_z,
     const uint8_t* __restrict__ v_data, const uint16_t* __restrict__ v_scales, const int64_t* __restrict__ block_table,
     const int32_t* __restrict__ seq_lens, float* __restrict__ partial, int H_q, int H_kv, int max_S, int max_blocks,
-    int64_t num_slots) {
+    int64_t num_slots, int sub_count) {
   constexpr int P = D / 2;
   __shared__ __align__(16) uint8_t vbuf[TQ_TILE * P];
   __shared__ int pq[G][TQ_TILE];
   __shared__ float rs_sh[G];
-  const int split = blockIdx.x, hkv = blockIdx.y, b = blockIdx.z, tid = threadIdx.x;
+  const int split = blockIdx.x / sub_count, sub = blockIdx.x % sub_count;
+  const int hkv = blockIdx.y, b = blockIdx.z, tid = threadIdx.x;
   const int S = max(0, min(max_S, seq_lens[b]));
   const int chunk = (max_S + TQ_SPLITS - 1) / TQ_SPLITS;
   const int s_start = split * chunk, s_end = min(s_start + chunk, S);
@@ -151,7 +155,12 @@ __global__ __launch_bounds__(SV_THREADS) void tile_quantised_v_split_kernel(
   const uint16_t* sbase = v_scales + (size_t)hkv * num_slots;
   const int64_t* bt = block_table + (size_t)b * max_blocks;
   const int q32 = tid >> 5, l32 = tid & 31;
-  for (int t0 = (s_start / BS) * BS; t0 < s_end; t0 += TQ_TILE) {
+  const int t_first = (s_start / BS) * BS;
+  const int n_tiles = (s_end > t_first) ? (s_end - t_first + TQ_TILE - 1) / TQ_TILE : 0;
+  const int per_sub = (n_tiles + sub_count - 1) / sub_count;
+  const int tile_end = min(n_tiles, (sub + 1) * per_sub);
+  for (int tile = sub * per_sub; tile < tile_end; ++tile) {
+    const int t0 = t_first + tile * TQ_TILE;
     __syncthreads();
     // the two pages of the tile (a page past the table or the sequence contributes zero weights; its codes are not read)
     int64_t base_slot[2];
@@ -205,7 +214,7 @@ __global__ __launch_bounds__(SV_THREADS) void tile_quantised_v_split_kernel(
   }
 #pragma unroll
   for (int g = 0; g < G; ++g)
-    partial[(((size_t)b * H_q + (size_t)hkv * G + g) * TQ_SPLITS + split) * D + tid] = acc[g];
+    partial[(((size_t)b * H_q + (size_t)hkv * G + g) * (TQ_SPLITS * sub_count) + blockIdx.x) * D + tid] = acc[g];
 }
 
 // grid (B, H_q); adds split partials in order, then the top-k pre-correction.
@@ -376,15 +385,21 @@ extern "C" int jf_softmax_v_int8_tiles(const float* scores, const float* softmax
                "int8tc_softmax_v: workspace too small");
   hipStream_t st = (hipStream_t)stream;
   float* partial = reinterpret_cast<float*>(workspace);
-  dim3 grid(TQ_SPLITS, H_kv, B), block(SV_THREADS);
+  // runs of at least four tiles per workgroup, at most sixteen workgroups per range (8 * sub_count <= max_S / 128
+  // partial rows: inside the workspace, which holds max(8, max_S / 64))
+  const int tiles_per_range = ((max_S + TQ_SPLITS - 1) / TQ_SPLITS + TQ_TILE - 1) / TQ_TILE + 1;
+  int sub_count = tiles_per_range / 4;
+  sub_count = sub_count < 1 ? 1 : (sub_count > 16 ? 16 : sub_count);
+  while (sub_count > 1 && (size_t)TQ_SPLITS * sub_count > (size_t)(max_S + 63) / 64) --sub_count;
+  dim3 grid(TQ_SPLITS * sub_count, H_kv, B), block(SV_THREADS);
   JF_DISPATCH_G2(G, {
     hipLaunchKernelGGL((tile_quantised_v_split_kernel<GG>), grid, block, 0, st, scores, softmax_m, softmax_inv_z, v_data,
-                       v_scales, block_table, seq_lens, partial, H_q, H_kv, max_S, max_blocks, num_slots);
+                       v_scales, block_table, seq_lens, partial, H_q, H_kv, max_S, max_blocks, num_slots, sub_count);
   });
   JF_CHECK_LAUNCH();
   hipLaunchKernelGGL((combine_precorr_kernel<4, 1>), dim3(B, H_q), block, 0, st, partial, scores, softmax_m, softmax_inv_z,
                      v_data, v_scales, block_table, seq_lens, topk_idx, o_hat, o_old_unnorm, W, H_q, H_kv, max_S, max_blocks,
-                     num_slots, TQ_SPLITS, top_k);
+                     num_slots, TQ_SPLITS * sub_count, top_k);
   JF_CHECK_LAUNCH();
   return JF_OK;
 }

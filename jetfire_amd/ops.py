@@ -7,6 +7,7 @@ Tensors are only used for device memory and the current stream; all arithmetic i
 """
 from __future__ import annotations
 
+import os
 from typing import List, Optional
 
 import torch
@@ -197,6 +198,57 @@ def shadow_write(key_tok, value_tok, slot_idx, k_shadow, v_shadow, *, k_shadow_d
 
 
 # --------------------------------------------------------------------------- Stage A
+#
+# The reference's Stage A and Stage B operators come in two implementations here: "fast" (default) runs them on the
+# kernels of the fused step wherever its shape limits allow (jf_stage_a_topk / jf_stage_b_softmax_v), "simple" is one
+# plain kernel per reference kernel (every width, group layout and top_k up to 8192; also the second implementation
+# the parity tests compare against).  JETFIRE_SPLIT_IMPL=simple or set_split_impl("simple") forces the latter.
+
+_split_impl = os.environ.get("JETFIRE_SPLIT_IMPL", "fast").strip().lower() or "fast"
+
+
+def set_split_impl(name: str) -> str:
+    """Select the implementation of the Stage A / Stage B operators ("fast" or "simple"); returns the previous one."""
+    global _split_impl
+    _check(name in ("fast", "simple"), "split implementation must be 'fast' or 'simple'")
+    prev, _split_impl = _split_impl, name
+    return prev
+
+
+def get_split_impl() -> str:
+    return _split_impl
+
+
+def _fast_shape(H_q, H_kv, block_size, max_S, num_slots, top_k=None) -> bool:
+    return (_split_impl == "fast" and H_kv > 0 and H_q % H_kv == 0 and H_q // H_kv in (1, 2, 4, 8, 16)
+            and int(block_size) == 16 and 0 < int(max_S) <= 262144 and 0 < int(num_slots) <= (1 << 25)
+            and (top_k is None or int(top_k) in (32, 64, 128, 256, 512, 1024)))
+
+
+def _stage_a_fast(fmt: int, q, kd, ks, bt, sl, max_S, H_q, H_kv, attn_scale, top_k, stats: bool):
+    """jf_stage_a_topk: -> (scores, idx, slots, m, iz); top_k None: scores alone."""
+    lib = _lib.load()
+    B, dev = q.size(0), q.device
+    scores = torch.empty((B, H_q, max_S), dtype=torch.float32, device=dev)
+    idx = slots = m = iz = ws = None
+    if top_k is not None:
+        idx = torch.empty((B, H_q, top_k), dtype=torch.int64, device=dev)
+        slots = torch.empty((B, H_q, top_k), dtype=torch.int64, device=dev)
+        if stats:
+            m = torch.empty((B, H_q), dtype=torch.float32, device=dev)
+            iz = torch.empty((B, H_q), dtype=torch.float32, device=dev)
+        ws = _workspace(dev, lib.jf_fused_workspace_bytes(fmt, B, H_q, H_kv, int(max_S), int(top_k)), "fused")
+    _lib.check(lib.jf_stage_a_topk(
+        fmt, HEAD_DIM // ks.size(2), q.data_ptr(), kd.data_ptr(), ks.data_ptr(), bt.data_ptr(), sl.data_ptr(), B, H_q, H_kv,
+        int(max_S), bt.size(1), kd.size(1), 16, float(attn_scale), 0 if top_k is None else int(top_k), scores.data_ptr(),
+        _ptr(idx), _ptr(slots), _ptr(m), _ptr(iz), _ptr(ws), 0 if ws is None else ws.numel(), _stream(q)))
+    return scores, idx, slots, m, iz
+
+
+def _check_top_k(top_k, name: str, minimum: int = 32) -> None:
+    _check(int(top_k) in SUPPORTED_TOP_K and int(top_k) >= minimum,
+           f"{name}: unsupported radix-select top_k={top_k} (supported: "
+           f"{','.join(str(k) for k in SUPPORTED_TOP_K if k >= minimum)})")
 
 
 def _stage_a_args(q, k_data, k_scales, block_table, seq_lens, H_q, H_kv, packed):
@@ -224,6 +276,8 @@ def int3_qk_scores(q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_kv,
     ng = ks.size(2)
     _check(ng in (1, 2), f"int3_qk_scores currently supports K quant groups 1 or 2, got {ng}")
     B = q.size(0)
+    if _fast_shape(H_q, H_kv, block_size, max_S, kd.size(1)):
+        return _stage_a_fast(32, q, kd, ks, bt, sl, max_S, H_q, H_kv, attn_scale, None, False)[0]
     scores = torch.empty((B, H_q, max_S), dtype=torch.float32, device=q.device)
     _lib.check(lib.jf_int3_qk_scores(q.data_ptr(), kd.data_ptr(), ks.data_ptr(), bt.data_ptr(), sl.data_ptr(),
                                      B, H_q, H_kv, int(max_S), bt.size(1), kd.size(1), ng, int(block_size),
@@ -296,6 +350,8 @@ def int8tc_qk_scores(q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_k
         _check(k_scales.size(2) == 1, "int8tc_qk_scores needs one K scale per token (group 128)")
     q, kd, ks, bt, sl = _stage_a_args(q, k_data, k_scales, block_table, seq_lens, H_q, H_kv, 64)
     B = q.size(0)
+    if _fast_shape(H_q, H_kv, block_size, max_S, kd.size(1)):
+        return _stage_a_fast(44, q, kd, ks, bt, sl, max_S, H_q, H_kv, attn_scale, None, False)[0]
     scores = torch.empty((B, H_q, max_S), dtype=torch.float32, device=q.device)
     _lib.check(lib.jf_int8tc_qk_scores(q.data_ptr(), kd.data_ptr(), ks.data_ptr(), bt.data_ptr(), sl.data_ptr(),
                                        B, H_q, H_kv, int(max_S), bt.size(1), kd.size(1), int(block_size),
@@ -305,9 +361,7 @@ def int8tc_qk_scores(q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_k
 
 def _topk(scores, block_table, seq_lens, max_S, H_q, block_size, top_k, stats: bool, name: str, minimum: int = 32):
     lib = _lib.load()
-    _check(int(top_k) in SUPPORTED_TOP_K and int(top_k) >= minimum,
-           f"{name}: unsupported radix-select top_k={top_k} (supported: "
-           f"{','.join(str(k) for k in SUPPORTED_TOP_K if k >= minimum)})")
+    _check_top_k(top_k, name, minimum)
     _check(max_S <= 262144, f"{name}: max_S={max_S} exceeds supported limit (262144).")
     B = scores.size(0)
     bt, sl = block_table.contiguous(), seq_lens.contiguous()
@@ -326,6 +380,10 @@ def _topk(scores, block_table, seq_lens, max_S, H_q, block_size, top_k, stats: b
 def int3_qk_scores_topk(q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_kv, block_size, attn_scale,
                         top_k) -> List[torch.Tensor]:
     """int3_qk_scores.cu:562-633 -> [scores, topk_idx, topk_slots]."""
+    if _fast_shape(H_q, H_kv, block_size, max_S, k_data.size(1) if k_data.dim() == 3 else 0, top_k):
+        q_, kd, ks, bt, sl = _stage_a_args(q, k_data, k_scales, block_table, seq_lens, H_q, H_kv, 48)
+        _check(ks.size(2) in (1, 2), f"int3_qk_scores currently supports K quant groups 1 or 2, got {ks.size(2)}")
+        return list(_stage_a_fast(32, q_, kd, ks, bt, sl, max_S, H_q, H_kv, attn_scale, int(top_k), False)[:3])
     scores = int3_qk_scores(q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_kv, block_size, attn_scale)
     idx, slots, _, _ = _topk(scores, block_table, seq_lens, max_S, H_q, block_size, top_k, False, "int3_qk_scores_topk")
     return [scores, idx, slots]
@@ -334,6 +392,10 @@ def int3_qk_scores_topk(q, k_data, k_scales, block_table, seq_lens, max_S, H_q, 
 def int8tc_qk_scores_topk(q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_kv, block_size, attn_scale,
                           top_k) -> List[torch.Tensor]:
     """int8tc_qk_scores.cu:2345-2424 -> [scores, topk_idx, topk_slots]."""
+    if _fast_shape(H_q, H_kv, block_size, max_S, k_data.size(1) if k_data.dim() == 3 else 0, top_k):
+        _check(k_scales.dim() == 2 or k_scales.size(2) == 1, "int8tc_qk_scores needs one K scale per token (group 128)")
+        q_, kd, ks, bt, sl = _stage_a_args(q, k_data, k_scales, block_table, seq_lens, H_q, H_kv, 64)
+        return list(_stage_a_fast(44, q_, kd, ks, bt, sl, max_S, H_q, H_kv, attn_scale, int(top_k), False)[:3])
     scores = int8tc_qk_scores(q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_kv, block_size, attn_scale)
     idx, slots, _, _ = _topk(scores, block_table, seq_lens, max_S, H_q, block_size, top_k, False, "int8tc_qk_scores_topk")
     return [scores, idx, slots]
@@ -342,6 +404,11 @@ def int8tc_qk_scores_topk(q, k_data, k_scales, block_table, seq_lens, max_S, H_q
 def int8tc_qk_scores_topk_stats(q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_kv, block_size, attn_scale,
                                 top_k) -> List[torch.Tensor]:
     """int8tc_qk_scores.cu:2426-2482 -> [scores, topk_idx, topk_slots, softmax_m, softmax_inv_z]."""
+    _check_top_k(top_k, "int8tc_qk_scores_topk_stats", 64)
+    if _fast_shape(H_q, H_kv, block_size, max_S, k_data.size(1) if k_data.dim() == 3 else 0, top_k):
+        _check(k_scales.dim() == 2 or k_scales.size(2) == 1, "int8tc_qk_scores needs one K scale per token (group 128)")
+        q_, kd, ks, bt, sl = _stage_a_args(q, k_data, k_scales, block_table, seq_lens, H_q, H_kv, 64)
+        return list(_stage_a_fast(44, q_, kd, ks, bt, sl, max_S, H_q, H_kv, attn_scale, int(top_k), True))
     scores = int8tc_qk_scores(q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_kv, block_size, attn_scale)
     idx, slots, m, iz = _topk(scores, block_table, seq_lens, max_S, H_q, block_size, top_k, True,
                               "int8tc_qk_scores_topk_stats", minimum=64)
@@ -381,6 +448,16 @@ def _softmax_v(scores, m, iz, v_data, v_scales, block_table, seq_lens, topk_idx,
         o_hat, o_old, W = outs
         for t in outs:
             _check(t.is_cuda and t.dtype == torch.float32 and t.is_contiguous(), "output buffers must be contiguous fp32")
+    if (not int8_tiles and m is None and nbits in (2, 4) and (nbits == 2 or ng == 1) and vd.size(0) == H_kv
+            and _fast_shape(H_q, H_kv, block_size, max_S, vd.size(1), top_k if topk_idx is not None else None)):
+        fmt = 32 if nbits == 2 else 44
+        k_eff = int(top_k) if topk_idx is not None else 32
+        ws = _workspace(dev, lib.jf_fused_workspace_bytes(fmt, B, H_q, H_kv, int(max_S), k_eff), "fused")
+        _lib.check(lib.jf_stage_b_softmax_v(
+            fmt, HEAD_DIM // ng, sc.data_ptr(), vd.data_ptr(), vs.data_ptr(), bt.data_ptr(), sl.data_ptr(), _ptr(topk_idx),
+            B, H_q, H_kv, int(max_S), bt.size(1), vd.size(1), 16, k_eff, o_hat.data_ptr(), o_old.data_ptr(), W.data_ptr(),
+            ws.data_ptr(), ws.numel(), _stream(sc)))
+        return [o_hat, o_old, W]
     need = lib.jf_softmax_v_workspace_bytes(B, H_q, int(max_S))
     ws = _workspace(dev, need, "softmax_v")
     if m is not None:

@@ -181,6 +181,15 @@ def test_pack_rejects_bad_arguments():
 # ------------------------------------------------------------------ Stage A + top-k
 
 
+@pytest.fixture(params=["fast", "simple"])
+def impl(request):
+    """Both implementations of the Stage A / Stage B operators: on the kernels of the fused step, and one plain
+    kernel per reference kernel."""
+    prev = ops().set_split_impl(request.param)
+    yield request.param
+    ops().set_split_impl(prev)
+
+
 CASES_A = [  # (B, Hq, Hkv, S)
     (2, 8, 2, 512), (3, 32, 8, 300), (2, 32, 4, 272), (1, 8, 2, 17),
 ]
@@ -188,7 +197,7 @@ CASES_A = [  # (B, Hq, Hkv, S)
 
 @pytest.mark.parametrize("B,Hq,Hkv,S", CASES_A)
 @pytest.mark.parametrize("gs", (64, 128))
-def test_int3_scores_and_topk(B, Hq, Hkv, S, gs):
+def test_int3_scores_and_topk(B, Hq, Hkv, S, gs, impl):
     c = make_case(11 + S + gs, B, Hq, Hkv, S, 3, 2, gs)
     d = to_device(c)
     scale = 128 ** -0.5
@@ -203,6 +212,8 @@ def test_int3_scores_and_topk(B, Hq, Hkv, S, gs):
     ridx, rslots = O.topk_select(got, c["lens"], c["bt"], S, K)
     assert np.array_equal(idx.cpu().numpy(), ridx)
     assert np.array_equal(slots.cpu().numpy(), rslots)
+    alone = ops().int3_qk_scores(d["q"], d["kd"], d["ks"], d["bt"], d["lens"], S, Hq, Hkv, 16, scale)
+    assert torch.equal(alone, scores)                            # the scores-only operator: the same kernel arithmetic
 
 
 @pytest.mark.parametrize("B,Hq,Hkv,S", CASES_A)
@@ -234,7 +245,7 @@ def test_int2_and_int4_scores_with_the_bf16_model(B, Hq, Hkv, S, kb, gs):
 
 
 @pytest.mark.parametrize("B,Hq,Hkv,S", CASES_A)
-def test_int8tc_scores_bit_exact_topk_and_stats(B, Hq, Hkv, S):
+def test_int8tc_scores_bit_exact_topk_and_stats(B, Hq, Hkv, S, impl):
     c = make_case(21 + S, B, Hq, Hkv, S, 4, 4, 128)
     d = to_device(c)
     scale = 128 ** -0.5
@@ -250,6 +261,10 @@ def test_int8tc_scores_bit_exact_topk_and_stats(B, Hq, Hkv, S):
     rm, riz = O.softmax_stats(ref, c["lens"], S)
     np.testing.assert_allclose(m.cpu().numpy(), rm, atol=0, rtol=0)
     np.testing.assert_allclose(iz.cpu().numpy(), riz, rtol=1e-5)
+    alone = ops().int8tc_qk_scores(d["q"], d["kd"], d["ks"], d["bt"], d["lens"], S, Hq, Hkv, 16, scale)
+    assert torch.equal(alone, scores)
+    three = ops().int8tc_qk_scores_topk(d["q"], d["kd"], d["ks"], d["bt"], d["lens"], S, Hq, Hkv, 16, scale, K)
+    assert torch.equal(three[1], idx) and torch.equal(three[2], slots)
 
 
 def test_topk_ties_short_rows_and_zero_length():
@@ -302,7 +317,7 @@ def test_unsupported_top_k_raises():
 
 @pytest.mark.parametrize("scheme", ("k3v2", "k4v4", "k3v2_g128", "k3v3", "k3v3_g128"))
 @pytest.mark.parametrize("B,Hq,Hkv,lens", [(2, 8, 2, None), (3, 32, 4, [17, 257, 512]), (4, 8, 2, [0, 1, 9, 17])])
-def test_stage_b_outputs(scheme, B, Hq, Hkv, lens):
+def test_stage_b_outputs(scheme, B, Hq, Hkv, lens, impl):
     kb, vb, gs = {"k3v2": (3, 2, 64), "k4v4": (4, 4, 128), "k3v2_g128": (3, 2, 128), "k3v3": (3, 3, 64),
                   "k3v3_g128": (3, 3, 128)}[scheme]
     S = 512 if lens is None or max(lens) > 32 else 32
@@ -324,6 +339,19 @@ def test_stage_b_outputs(scheme, B, Hq, Hkv, lens):
     np.testing.assert_allclose(o_hat.cpu().numpy(), r_hat, atol=3e-6, rtol=3e-6)     # validate_runtime.py:173-177
     np.testing.assert_allclose(o_old.cpu().numpy(), r_old, atol=3e-6, rtol=3e-6)
     np.testing.assert_allclose(W.cpu().numpy(), r_W, atol=3e-6, rtol=3e-6)
+    if vb != 3:                                                   # without winners: o_hat alone
+        plain = {2: o.int2_softmax_v, 4: None}[vb]
+        if plain is not None:
+            only = plain(sc_t, d["vd"], d["vs"], d["bt"], d["lens"], S, Hq, Hkv, 16)
+            np.testing.assert_allclose(only.cpu().numpy(), r_hat, atol=3e-6, rtol=3e-6)
+        padded = idx_t.clone()
+        padded[:, :, K // 2:] = -1                                # half of the winners dropped: -1 entries carry no weight
+        h_idx = ridx.copy()
+        h_idx[:, :, K // 2:] = -1
+        _, p_old, p_W = fn(sc_t, d["vd"], d["vs"], d["bt"], d["lens"], padded, S, Hq, Hkv, 16, K)
+        _, q_old, q_W = O.softmax_v(ref_sc, c["vd"], c["vs"], c["bt"], c["lens"], h_idx, S, Hq, Hkv, 16, vb, gs)
+        np.testing.assert_allclose(p_old.cpu().numpy(), q_old, atol=3e-6, rtol=3e-6)
+        np.testing.assert_allclose(p_W.cpu().numpy(), q_W, atol=3e-6, rtol=3e-6)
     if vb == 4:                                                   # the int8-weight variant, handed Stage-A statistics
         m, iz = O.softmax_stats(ref_sc, c["lens"], S)
         o2 = o.int8tc_softmax_v_with_pre_corr_reg_stats(sc_t, torch.from_numpy(m).cuda(), torch.from_numpy(iz).cuda(),
