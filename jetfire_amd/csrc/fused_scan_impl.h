@@ -94,6 +94,8 @@ struct FusedParams {
   int L, n_splits, Kc;
   float* scores;  // optional (B, H_q, max_S)
   const float* scores_in;  // FS_STAGE_B: the scores (B, H_q, max_S)
+  const float* stats_m;    // FS_STAGE_B merge, optional: softmax statistics (B, H_q) that replace the ones derived
+  const float* stats_iz;   //   from the split partials (pre-correction terms alone: n_splits == 0, o_hat == NULL)
   int scores_only;         // FS_STAGE_A: stop after writing `scores`
   float* part_m;  // (B, H_q, NS)
   float* part_l;  // (B, H_q, NS)
@@ -1430,6 +1432,12 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
       p.softmax_inv_z[bh] = inv_z;
     }
   }
+  if constexpr (MODE == FS_STAGE_B) {
+    if (p.stats_m) {  // (uniform) the caller's statistics
+      M = p.stats_m[bh];
+      inv_z = p.stats_iz[bh];
+    }
+  }
   if constexpr (!PARTIAL && MODE != FS_STAGE_A) {
     // o_hat: four thread groups take every fourth split, then a fixed-order sum
     const int d = tid & (D - 1), q4 = tid >> 7;
@@ -1461,7 +1469,7 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
 #pragma unroll
       for (int q = 1; q < PO_GRP; ++q) o2 += red_sh[q][tid];  // fixed order
       blend_hat = o2 * inv_z;
-      p.o_hat[bh * D + tid] = blend_hat;
+      if (MODE != FS_STAGE_B || p.o_hat) p.o_hat[bh * D + tid] = blend_hat;
     }
   }
   if (mclk && tid == 0) mclk[1] = clock64();
@@ -2057,6 +2065,7 @@ static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_
   uint8_t* ws = reinterpret_cast<uint8_t*>(workspace);
   p.scores = (MODE == FS_STAGE_B) ? nullptr : scores;
   p.scores_in = scores_in;
+  p.stats_m = p.stats_iz = nullptr;
   p.scores_only = scores_only ? 1 : 0;
   p.part_m = reinterpret_cast<float*>(ws + wl.off_m);
   p.part_l = reinterpret_cast<float*>(ws + wl.off_l);
@@ -2115,6 +2124,27 @@ static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_
     JF_MERGE(4, 1);
   }
 #undef JF_MERGE
+  JF_CHECK_LAUNCH();
+  return JF_OK;
+}
+
+// The pre-correction terms alone (Stage B merge kernel with the caller's softmax statistics):
+//   W = sum_j p_j, o_old_unnorm = sum_j p_j * Vhat_j over the given winners, p_j = exp(score_j - m) * inv_z.
+template <int VBITS, int NG>
+static int launch_precorr_given_stats(const float* scores, const float* softmax_m, const float* softmax_inv_z,
+                                      const uint8_t* v_data, const uint16_t* v_scales, const int64_t* block_table,
+                                      const int32_t* seq_lens, const int64_t* topk_idx, int B, int H_q, int H_kv,
+                                      int max_S, int max_blocks, int64_t num_slots, int top_k, float* o_old_unnorm,
+                                      float* W, hipStream_t st) {
+  FusedParams p = {};
+  p.v_data = v_data; p.v_scales = v_scales; p.block_table = block_table; p.seq_lens = seq_lens;
+  p.B = B; p.H_q = H_q; p.H_kv = H_kv; p.max_S = max_S; p.max_blocks = max_blocks; p.num_slots = num_slots;
+  p.top_k = top_k;
+  p.n_splits = 0; p.mg_parts = 1; p.mg_spp = 0; p.Kc = 0;
+  p.scores_in = scores; p.stats_m = softmax_m; p.stats_iz = softmax_inv_z;
+  p.topk_idx = const_cast<int64_t*>(topk_idx);
+  p.o_old = o_old_unnorm; p.W = W;
+  hipLaunchKernelGGL((fused_merge_kernel<FS_STAGE_B, VBITS, NG, 1024, 8, false>), dim3(B, H_q), dim3(1024), 0, st, p);
   JF_CHECK_LAUNCH();
   return JF_OK;
 }

@@ -19,3 +19,13 @@ extern "C" int jf_stage_b_softmax_v(int value_format, int group_size, const floa
                                const_cast<int64_t*>(topk_idx), nullptr, o_hat, o_old_unnorm, W, nullptr, nullptr, nullptr,
                                scores, nullptr, nullptr, workspace, workspace_bytes, stream);
 }
+
+int jf::precorr_int4_given_stats(const float* scores, const float* softmax_m, const float* softmax_inv_z,
+                                 const uint8_t* v_data, const uint16_t* v_scales, const int64_t* block_table,
+                                 const int32_t* seq_lens, const int64_t* topk_idx, int B, int H_q, int H_kv, int max_S,
+                                 int max_blocks, int64_t num_slots, int top_k, float* o_old_unnorm, float* W,
+                                 void* stream) {
+  return launch_precorr_given_stats<4, 1>(scores, softmax_m, softmax_inv_z, v_data, v_scales, block_table, seq_lens,
+                                          topk_idx, B, H_q, H_kv, max_S, max_blocks, num_slots, top_k, o_old_unnorm, W,
+                                          (hipStream_t)stream);
+}

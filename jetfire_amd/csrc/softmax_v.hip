@@ -234,7 +234,13 @@ __global__ __launch_bounds__(SV_THREADS) void combine_precorr_kernel(
   const size_t bh = (size_t)b * H_q + hq;
   const int hkv = hq / (H_q / H_kv);
   float acc = 0.0f;
-  for (int s = 0; s < n_splits; ++s) acc += partial[(bh * n_splits + s) * D + tid];
+  for (int s0 = 0; s0 < n_splits; s0 += 8) {  // eight loads in flight, the sum keeps its order
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = (s0 + u < n_splits) ? partial[(bh * n_splits + s0 + u) * D + tid] : 0.0f;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) acc += v[u];
+  }
   o_hat[bh * D + tid] = acc;
   if (topk_idx == nullptr) return;
   const int S = max(0, min(max_S, seq_lens[b]));
@@ -397,9 +403,15 @@ extern "C" int jf_softmax_v_int8_tiles(const float* scores, const float* softmax
                        v_scales, block_table, seq_lens, partial, H_q, H_kv, max_S, max_blocks, num_slots, sub_count);
   });
   JF_CHECK_LAUNCH();
+  // the pre-correction terms run on the merge kernel of the fused step where its limits allow (the same
+  // formula, p_j = exp(score_j - m) * inv_z with the caller's statistics), else in the combine kernel
+  const bool fast_precorr = topk_idx != nullptr && top_k <= 1024 && num_slots <= (1ll << 25) && ((uintptr_t)v_data & 3) == 0;
   hipLaunchKernelGGL((combine_precorr_kernel<4, 1>), dim3(B, H_q), block, 0, st, partial, scores, softmax_m, softmax_inv_z,
-                     v_data, v_scales, block_table, seq_lens, topk_idx, o_hat, o_old_unnorm, W, H_q, H_kv, max_S, max_blocks,
-                     num_slots, TQ_SPLITS * sub_count, top_k);
+                     v_data, v_scales, block_table, seq_lens, fast_precorr ? nullptr : topk_idx, o_hat, o_old_unnorm, W, H_q,
+                     H_kv, max_S, max_blocks, num_slots, TQ_SPLITS * sub_count, top_k);
   JF_CHECK_LAUNCH();
+  if (fast_precorr)
+    return precorr_int4_given_stats(scores, softmax_m, softmax_inv_z, v_data, v_scales, block_table, seq_lens, topk_idx, B,
+                                    H_q, H_kv, max_S, max_blocks, num_slots, top_k, o_old_unnorm, W, stream);
   return JF_OK;
 }
