@@ -110,3 +110,29 @@ def test_c1_gpu_split_path_agrees_with_the_cpu_torch_path():
         assert len(clear) >= K - 4                                        # almost every winner is clear of the cut
     torch.testing.assert_close(o_hat.cpu(), ref_o.float(), atol=2e-3, rtol=2e-2)
     assert float((o_hat.cpu() - ref_o.float()).abs().mean()) < 2e-4
+
+
+@pytest.mark.parametrize("name", ["c2", "c3", "c4"])
+def test_two_call_form_equals_the_one_pass_form_at_full_size(name):
+    """The reference-named Stage A and Stage B operators run on the same kernels as the one-pass form (without the
+    other stage): scores, winners, slots and statistics come out bit-equal, and so do o_hat, o_old_unnorm and W
+    (exact integer accumulation, the same split geometry)."""
+    from jetfire_amd import ops, workloads
+    w = workloads.build(name, n_layers=1, paged=True)
+    lay = w.layers[0]
+    S, K, Hq, Hkv = w.S, w.top_k, w.H_q, w.H_kv
+    assert ops.get_split_impl() == "fast"
+    o_hat, slots, o_old, W, idx, m, iz, scores = _run(w, lay, return_scores=True, return_stats=True)
+    if w.scheme == "k3v2":
+        sc2, idx2, slots2 = ops.int3_qk_scores_topk(w.q, lay.k_data, lay.k_scales, w.block_table, w.seq_lens, S, Hq, Hkv, 16,
+                                                    w.attn_scale, K)
+        stage_b = ops.int2_softmax_v_with_pre_corr_wvs2
+    else:
+        sc2, idx2, slots2, m2, iz2 = ops.int8tc_qk_scores_topk_stats(w.q, lay.k_data, lay.k_scales, w.block_table,
+                                                                     w.seq_lens, S, Hq, Hkv, 16, w.attn_scale, K)
+        assert torch.equal(m2, m) and torch.equal(iz2, iz)
+        stage_b = ops.int4_softmax_v_with_pre_corr_wvs2_scores
+    assert torch.equal(sc2.view(torch.int32), scores.view(torch.int32))
+    assert torch.equal(idx2, idx) and torch.equal(slots2, slots)
+    o_hat2, o_old2, W2 = stage_b(sc2, lay.v_data, lay.v_scales, w.block_table, w.seq_lens, idx2, S, Hq, Hkv, 16, K)
+    assert torch.equal(o_hat2, o_hat) and torch.equal(o_old2, o_old) and torch.equal(W2, W)
