@@ -290,6 +290,13 @@ int jf_debug_phase_clock(void* device_buffer);
  * multiple of 256 and clamped to what fits the kernel's LDS) replaces the planner's choice of the split
  * length in jf_fused_scan_topk and jf_fused_workspace_bytes; 0 restores the planner.  Process-wide. */
 int jf_debug_split_len(int split_len);
+/* Test aids for the CPU pool, no counterpart in the reference.  jf_debug_pool_stall: the worker that claims `row` of
+ * the next correction job sleeps `microseconds` before it computes the row (one shot), as if it had lost its core.
+ * jf_debug_pool_wait_stragglers(0): jf_cpu_topk_attn returns as soon as every row is committed, like the hand-off
+ * jobs do, instead of also waiting for workers that are still inside a row (the caller must then keep its tensors
+ * alive); 1 restores the default. */
+int jf_debug_pool_stall(int64_t row, int microseconds);
+int jf_debug_pool_wait_stragglers(int on);
 
 /* ------------------------------------------------------------------ piece 4: merge
  * out = bf16_rne(fma(W, f32(o_new), o_hat) - o_old_unnorm).  Replaces blend_unnorm_into

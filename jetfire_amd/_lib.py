@@ -44,6 +44,8 @@ SIGNATURES = {
     "jf_profile_scan_end": (I, [P, P]),
     "jf_debug_phase_clock": (I, [P]),
     "jf_debug_split_len": (I, [I]),
+    "jf_debug_pool_stall": (I, [L, I]),
+    "jf_debug_pool_wait_stragglers": (I, [I]),
     "jf_fused_plan": (I, [I, I, I, I, I, I, I, P, P, P, P]),
     "jf_blend_unnorm": (I, [P, P, P, P, P, I, I, I, P]),
     "jf_cpu_topk_attn": (I, [P, P, P, P, P, P, I, I, I, I, L, F, P]),

@@ -14,6 +14,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <functional>
+#include <memory>
 #include <mutex>
 #include <thread>
 #include <vector>
@@ -44,6 +45,31 @@ void set_error(const char* fmt, ...) {
 // its core (more busy threads than cores) or is still asleep takes no rows and holds nobody up; it only
 // matters while it sits on a claimed row.  The counter carries the job's epoch in its upper half, so a worker
 // that wakes up late with an old job in hand cannot claim rows of a newer one.
+struct CpuJob {
+  const uint16_t *q, *k_shadow, *v_shadow;
+  const int64_t *head_map, *ts_buf;  // head_map may be null (kv-head = query head / (H_q / H_kv)); ts_buf or ts32
+  uint16_t* o_new;
+  int B, H_q, K, H_kv;
+  int64_t num_slots;
+  float scale;
+  const int32_t* ts32 = nullptr;     // 32-bit slots instead of ts_buf
+};
+// One row (sequence, query head) of the job into `out` (128 bf16 values of the caller's choosing).
+static void compute_row(const CpuJob& j, int64_t r, uint16_t* out);
+
+// Test aid: the worker that claims this row of the next job sleeps first (one shot); see jf_debug_pool_stall.
+static std::atomic<int64_t> g_stall_row{-1};
+static std::atomic<int> g_stall_us{0};
+// Whether a synchronous call returns only after every worker has left its rows (default; the caller may free its
+// tensors right after the call).  Jobs over buffers that outlive them (the hand-off contexts) never wait.
+static std::atomic<int> g_wait_stragglers{1};
+
+// Backup copies of straggling rows: a worker that finds no unclaimed row left waits a grace period
+// (JETFIRE_POOL_BACKUP_US, default 30; negative: never) and then recomputes rows that are claimed but not yet
+// committed.  Every row is computed into a buffer of the worker and committed by the first one to finish
+// (compare-and-swap on the row's epoch tag, then the copy to o_new, then the count), so a worker that has lost its
+// core in the middle of a row (a scheduler time slice is milliseconds, a row ten microseconds) delays the job by
+// the grace period instead of by its absence, and whatever it does when it comes back is discarded.
 class Pool {
  public:
   static Pool& instance() {
@@ -58,15 +84,27 @@ class Pool {
     std::lock_guard<std::mutex> g(cfg_mu_);
     override_ = n;
   }
-  // Start fn(begin, end) over [0, n) asynchronously.  Returns false if a job is already in flight.
-  bool start(int64_t n, std::function<void(int64_t, int64_t)> fn) {
+  // Start the rows [0, n) of `job` asynchronously.  Returns false if a job is already in flight.
+  bool start(const CpuJob& job, int64_t n) {
     ensure_workers();
     std::unique_lock<std::mutex> lk(mu_);
     if (busy_) return false;
+    if (n > tag_cap_) {  // grow the tags only while no worker can be looking at them
+      lk.unlock();
+      quiesce();
+      lk.lock();
+      if (busy_) return false;
+      int64_t cap = tag_cap_ > 0 ? tag_cap_ : 1024;
+      while (cap < n) cap *= 2;
+      tags_.reset(new std::atomic<uint64_t>[(size_t)cap]);
+      const uint64_t now = epoch_.load(std::memory_order_relaxed);
+      for (int64_t i = 0; i < cap; ++i) tags_[i].store(now, std::memory_order_relaxed);
+      tag_cap_ = cap;
+    }
     busy_ = true;
     const uint64_t e = epoch_.load(std::memory_order_relaxed) + 1;
     Job& jb = jobs_[e & 1];
-    jb.fn = std::move(fn);
+    jb.cj = job;
     jb.n = n;
     const int w = (int)workers_.size();
     jb.chunk = std::max<int64_t>(1, n / ((int64_t)w * 8));
@@ -79,8 +117,8 @@ class Pool {
     return true;
   }
   // Wait for the job started with start().  timeout_s <= 0: wait forever.  On a timeout the job is withdrawn
-  // (no further rows can be claimed, rows in flight are waited for) and the pool is free again.
-  bool join(double timeout_s) {
+  // (no further rows can be claimed or committed, rows in flight are waited for) and the pool is free again.
+  bool join(double timeout_s, bool wait_stragglers) {
     const auto t0 = std::chrono::steady_clock::now();
     for (int spin = 0; spin < 20000; ++spin) {
       if (done_rows_.load(std::memory_order_acquire) >= n_) break;
@@ -93,13 +131,14 @@ class Pool {
       if (timeout_s > 0) {
         const double el = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
         if (el > timeout_s) {
-          // withdraw: a counter value of a later epoch stops every claim; then let the rows in flight drain
+          // withdraw: a counter value of a later epoch stops every claim and every commit; then let the rows in
+          // flight drain
           const uint64_t e = epoch_.load(std::memory_order_relaxed) + 1;
           next_.store(e << 32, std::memory_order_release);
-          epoch_.store(e, std::memory_order_release);
           jobs_[e & 1].n = 0;
+          epoch_.store(e, std::memory_order_release);
           lk.unlock();
-          while (active_.load(std::memory_order_acquire) != 0) std::this_thread::sleep_for(std::chrono::microseconds(50));
+          quiesce();
           lk.lock();
           busy_ = false;
           return false;
@@ -107,18 +146,28 @@ class Pool {
       }
       cv_done_.wait_for(lk, std::chrono::milliseconds(1));
     }
+    lk.unlock();
+    if (wait_stragglers) quiesce();
+    lk.lock();
     busy_ = false;
     return true;
   }
-  bool run(int64_t n, std::function<void(int64_t, int64_t)> fn) {
+  // `persistent`: the job's buffers outlive it (a straggler may still read them after the call has returned).
+  bool run(const CpuJob& job, int64_t n, bool persistent) {
     if (n <= 0) return true;
-    while (!start(n, fn)) std::this_thread::yield();
-    return join(0);
+    while (!start(job, n)) std::this_thread::yield();
+    return join(0, !persistent && g_wait_stragglers.load(std::memory_order_relaxed) != 0);
+  }
+  // Starts (or resizes) the workers without running anything.
+  void warm() { ensure_workers(); }
+  // Returns when no worker is inside a row.
+  void quiesce() {
+    while (active_.load(std::memory_order_acquire) != 0) std::this_thread::sleep_for(std::chrono::microseconds(20));
   }
 
  private:
   struct Job {
-    std::function<void(int64_t, int64_t)> fn;
+    CpuJob cj{};
     int64_t n = 0, chunk = 1;
   };
   Pool() = default;
@@ -164,7 +213,7 @@ class Pool {
       stop_ = false;
     }
     const uint64_t e0 = epoch_.load(std::memory_order_acquire);
-    for (int i = 0; i < want; ++i) workers_.emplace_back([this, e0] { worker(e0); });
+    for (int i = 0; i < want; ++i) workers_.emplace_back([this, e0, i] { worker(e0, i); });
   }
   static double spin_seconds() {
     // how long an idle worker spins for the next job before it sleeps: the gap between two layers of a decode
@@ -177,7 +226,40 @@ class Pool {
     }();
     return s;
   }
-  void worker(uint64_t seen) {
+  static double backup_seconds() {
+    static const double s = [] {
+      const char* e = std::getenv("JETFIRE_POOL_BACKUP_US");
+      const double us = e ? std::atof(e) : 30.0;
+      return (us <= 1e6 ? us : 30.0) * 1e-6;  // negative: no backup copies
+    }();
+    return s;
+  }
+  // Computes row r of the job of epoch e and commits it unless somebody else has.
+  void do_row(const Job& jb, uint64_t e, int64_t r, bool claimed) {
+    uint16_t local[D];
+    active_.fetch_add(1, std::memory_order_acq_rel);
+    if (claimed) {
+      int64_t sr = g_stall_row.load(std::memory_order_relaxed);
+      if (sr == r && g_stall_row.compare_exchange_strong(sr, -1))
+        std::this_thread::sleep_for(std::chrono::microseconds(g_stall_us.load(std::memory_order_relaxed)));
+    }
+    compute_row(jb.cj, r, local);
+    // the row's tag holds the epoch of the last job that committed it: a tag below e means that the job of epoch e
+    // is still current and the row is open; the worker that moves it to e owns the row's output
+    uint64_t old = tags_[r].load(std::memory_order_acquire);
+    while (old < e) {
+      if (tags_[r].compare_exchange_weak(old, e, std::memory_order_acq_rel, std::memory_order_acquire)) {
+        memcpy(jb.cj.o_new + r * D, local, sizeof(local));
+        if (done_rows_.fetch_add(1, std::memory_order_acq_rel) + 1 >= jb.n) {
+          std::lock_guard<std::mutex> g(mu_);
+          cv_done_.notify_all();
+        }
+        break;
+      }
+    }
+    active_.fetch_sub(1, std::memory_order_acq_rel);
+  }
+  void worker(uint64_t seen, int index) {
     for (;;) {
       bool got = false;
       const auto t0 = std::chrono::steady_clock::now();
@@ -196,26 +278,44 @@ class Pool {
       if (stop_flag()) return;
       const uint64_t e = epoch_.load(std::memory_order_acquire);
       seen = e;
-      // The job of epoch e stays in its slot at least until all its rows are done; the slot is only read after a
-      // claim on the counter of that very epoch has succeeded, i.e. while the job is certainly still current.
-      const Job& jb = jobs_[e & 1];
+      // A private copy of the job: its slot is rewritten by the job after next at the earliest, so the copy is
+      // whole if the epoch has moved by at most one since it was read.
+      const Job jb = jobs_[e & 1];
+      if (epoch_.load(std::memory_order_acquire) - e > 1) continue;
       uint64_t v = next_.load(std::memory_order_acquire);
       for (;;) {
-        if ((v >> 32) != (e & 0xffffffffu)) break;  // a newer job: this one is long finished
+        if ((v >> 32) != (e & 0xffffffffu)) break;  // a newer job: this one is finished or withdrawn
         const int64_t b = (int64_t)(v & 0xffffffffu);
-        const int64_t n = jb.n, chunk = jb.chunk;
-        if (b >= n) break;
-        if (!next_.compare_exchange_weak(v, v + (uint64_t)chunk, std::memory_order_acq_rel, std::memory_order_acquire)) continue;
-        const int64_t end = std::min<int64_t>(n, b + chunk);
-        active_.fetch_add(1, std::memory_order_acq_rel);
-        jb.fn(b, end);
-        active_.fetch_sub(1, std::memory_order_acq_rel);
-        if (done_rows_.fetch_add(end - b, std::memory_order_acq_rel) + (end - b) >= n) {
-          std::lock_guard<std::mutex> g(mu_);
-          cv_done_.notify_all();
-          break;
-        }
+        if (b >= jb.n) break;
+        if (!next_.compare_exchange_weak(v, v + (uint64_t)jb.chunk, std::memory_order_acq_rel, std::memory_order_acquire)) continue;
+        const int64_t end = std::min<int64_t>(jb.n, b + jb.chunk);
+        for (int64_t r = b; r < end; ++r) do_row(jb, e, r, true);
         v = next_.load(std::memory_order_acquire);
+      }
+      // no unclaimed row left: after the grace period, back up rows that are still open
+      const double grace = backup_seconds();
+      if (grace < 0.0 || jb.n <= 0) continue;
+      const auto t_idle = std::chrono::steady_clock::now();
+      bool waited = false;
+      while (done_rows_.load(std::memory_order_acquire) < jb.n && epoch_.load(std::memory_order_acquire) == e &&
+             !stop_flag()) {
+        if (!waited) {
+          if (std::chrono::duration<double>(std::chrono::steady_clock::now() - t_idle).count() < grace) {
+#if defined(__x86_64__)
+            _mm_pause();
+#endif
+            continue;
+          }
+          waited = true;
+        }
+        int64_t open = -1;
+        const int64_t first = ((int64_t)index * 7919) % jb.n;  // idle workers start their search at different rows
+        for (int64_t k = 0; k < jb.n; ++k) {
+          const int64_t r = first + k < jb.n ? first + k : first + k - jb.n;
+          if (tags_[r].load(std::memory_order_acquire) < e) { open = r; break; }
+        }
+        if (open < 0) break;
+        do_row(jb, e, open, false);
       }
     }
   }
@@ -224,13 +324,15 @@ class Pool {
   }
 
   std::mutex mu_, cfg_mu_, resize_mu_;
-  std::atomic<int> active_{0};          // workers inside a job function
+  std::atomic<int> active_{0};          // workers inside a row
   std::condition_variable cv_work_, cv_done_;
   std::vector<std::thread> workers_;
   Job jobs_[2];
   int64_t n_ = 0;
   std::atomic<uint64_t> next_{0};       // (epoch << 32) | first unclaimed row
-  std::atomic<int64_t> done_rows_{0};
+  std::atomic<int64_t> done_rows_{0};   // committed rows of the current job
+  std::unique_ptr<std::atomic<uint64_t>[]> tags_;  // per row: epoch of the last job that committed it
+  int64_t tag_cap_ = 0;
   int override_ = 0;
   bool busy_ = false, stop_ = false;
   std::atomic<uint64_t> epoch_{0};
@@ -491,44 +593,31 @@ static inline bool bf16_row_has_nonfinite(const uint16_t* r) {
   return false;
 }
 
-struct CpuJob {
-  const uint16_t *q, *k_shadow, *v_shadow;
-  const int64_t *head_map, *ts_buf;  // head_map may be null (kv-head = query head / (H_q / H_kv)); ts_buf or ts32
-  uint16_t* o_new;
-  int B, H_q, K, H_kv;
-  int64_t num_slots;
-  float scale;
-  const int32_t* ts32 = nullptr;     // 32-bit slots instead of ts_buf
-};
-
 template <typename SlotT>
-static void run_rows_t(const CpuJob& j, const SlotT* ts, int64_t b, int64_t e, float* buf) {
+static void compute_row_t(const CpuJob& j, const SlotT* ts, int64_t r, uint16_t* out, float* buf) {
   const int G = j.H_q / j.H_kv;
   const int isa = resolve_isa();
-  for (int64_t r = b; r < e; ++r) {
-    const uint16_t* q = j.q + r * D;
-    const int64_t* hm = j.head_map ? j.head_map + r * j.K : nullptr;
-    const int64_t fixed_h = (r % j.H_q) / G;
-    uint16_t* out = j.o_new + r * D;
+  const uint16_t* q = j.q + r * D;
+  const int64_t* hm = j.head_map ? j.head_map + r * j.K : nullptr;
+  const int64_t fixed_h = (r % j.H_q) / G;
 #if defined(__x86_64__)
-    if (isa == 2) topk_attn_row_avx512bf16<SlotT>(q, j.k_shadow, j.v_shadow, j.num_slots, hm, fixed_h, ts + r * j.K, j.K, j.H_kv, j.scale, out, buf);
-    else if (isa == 1) topk_attn_row_avx2<SlotT>(q, j.k_shadow, j.v_shadow, j.num_slots, hm, fixed_h, ts + r * j.K, j.K, j.H_kv, j.scale, out, buf);
-    else
+  if (isa == 2) topk_attn_row_avx512bf16<SlotT>(q, j.k_shadow, j.v_shadow, j.num_slots, hm, fixed_h, ts + r * j.K, j.K, j.H_kv, j.scale, out, buf);
+  else if (isa == 1) topk_attn_row_avx2<SlotT>(q, j.k_shadow, j.v_shadow, j.num_slots, hm, fixed_h, ts + r * j.K, j.K, j.H_kv, j.scale, out, buf);
+  else
 #endif
-      topk_attn_row<SlotT>(q, j.k_shadow, j.v_shadow, j.num_slots, hm, fixed_h, ts + r * j.K, j.K, j.H_kv, j.scale, out, buf);
-    if (bf16_row_has_nonfinite(out)) {
-      g_sanitize_count.fetch_add(1, std::memory_order_acq_rel);
-      if (isa != 0) topk_attn_row<SlotT>(q, j.k_shadow, j.v_shadow, j.num_slots, hm, fixed_h, ts + r * j.K, j.K, j.H_kv, j.scale, out, buf);
-      if (isa == 0 || bf16_row_has_nonfinite(out)) memset(out, 0, D * sizeof(uint16_t));
-    }
+    topk_attn_row<SlotT>(q, j.k_shadow, j.v_shadow, j.num_slots, hm, fixed_h, ts + r * j.K, j.K, j.H_kv, j.scale, out, buf);
+  if (bf16_row_has_nonfinite(out)) {
+    g_sanitize_count.fetch_add(1, std::memory_order_acq_rel);
+    if (isa != 0) topk_attn_row<SlotT>(q, j.k_shadow, j.v_shadow, j.num_slots, hm, fixed_h, ts + r * j.K, j.K, j.H_kv, j.scale, out, buf);
+    if (isa == 0 || bf16_row_has_nonfinite(out)) memset(out, 0, D * sizeof(uint16_t));
   }
 }
 
-static void run_rows(const CpuJob& j, int64_t b, int64_t e) {
+static void compute_row(const CpuJob& j, int64_t r, uint16_t* out) {
   static thread_local std::vector<float> buf;
   if (buf.size() < (size_t)j.K) buf.resize((size_t)j.K);
-  if (j.ts32) run_rows_t<int32_t>(j, j.ts32, b, e, buf.data());
-  else run_rows_t<int64_t>(j, j.ts_buf, b, e, buf.data());
+  if (j.ts32) compute_row_t<int32_t>(j, j.ts32, r, out, buf.data());
+  else compute_row_t<int64_t>(j, j.ts_buf, r, out, buf.data());
 }
 
 }  // namespace jf
@@ -552,6 +641,18 @@ extern "C" int jf_set_cpu_attn_isa(int isa) {
 extern "C" int jf_get_cpu_attn_isa(void) { return resolve_isa(); }
 extern "C" int64_t jf_cpu_topk_sanitize_count(void) { return g_sanitize_count.load(); }
 
+extern "C" int jf_debug_pool_stall(int64_t row, int microseconds) {
+  JF_CHECK_ARG(microseconds >= 0 && microseconds <= 10000000, "debug_pool_stall: bad duration");
+  g_stall_us.store(microseconds);
+  g_stall_row.store(row);
+  return JF_OK;
+}
+extern "C" int jf_debug_pool_wait_stragglers(int on) {
+  g_wait_stragglers.store(on ? 1 : 0);
+  if (on) Pool::instance().quiesce();
+  return JF_OK;
+}
+
 extern "C" int jf_cpu_topk_attn(const uint16_t* q, const uint16_t* k_shadow, const uint16_t* v_shadow,
                                 const int64_t* head_map, const int64_t* ts_buf, uint16_t* o_new, int B, int H_q, int K,
                                 int H_kv, int64_t num_slots, float scale, int64_t* done_flag) {
@@ -559,7 +660,7 @@ extern "C" int jf_cpu_topk_attn(const uint16_t* q, const uint16_t* k_shadow, con
   if (B > 0) {
     JF_CHECK_ARG(q && k_shadow && v_shadow && head_map && ts_buf && o_new, "cpu_topk_attn: null pointer");
     CpuJob j{q, k_shadow, v_shadow, head_map, ts_buf, o_new, B, H_q, K, H_kv, num_slots, scale};
-    Pool::instance().run((int64_t)B * H_q, [j](int64_t b, int64_t e) { run_rows(j, b, e); });
+    Pool::instance().run(j, (int64_t)B * H_q, false);
   }
   std::atomic_thread_fence(std::memory_order_release);
   if (done_flag) reinterpret_cast<std::atomic<int64_t>*>(done_flag)->store(1, std::memory_order_release);
@@ -736,7 +837,7 @@ bool run_correction(jf_handoff* h) {
   if (h->ext_q) {  // the caller's buffers, its head map and 64-bit slots
     CpuJob j{h->ext_q, h->k_shadow, h->v_shadow, h->ext_head_map, h->ext_ts, h->ext_o,
              h->B, h->H_q, h->K, h->H_kv, h->num_slots, h->scale};
-    const bool ok = Pool::instance().run((int64_t)h->B * h->H_q, [j](int64_t b, int64_t e) { run_rows(j, b, e); });
+    const bool ok = Pool::instance().run(j, (int64_t)h->B * h->H_q, true);  // the context's buffers outlive the job
     std::atomic_thread_fence(std::memory_order_release);
     if (h->ext_flag) __atomic_store_n(h->ext_flag, (int64_t)1, __ATOMIC_RELEASE);
     return ok;
@@ -744,7 +845,7 @@ bool run_correction(jf_handoff* h) {
   // kv-head of a row = query head / (H_q / H_kv) (decode_path.py:400-408): no head map is read
   CpuJob j{h->q_pin, h->k_shadow, h->v_shadow, nullptr, nullptr, h->o_pin,
            h->B, h->H_q, h->K, h->H_kv, h->num_slots, h->scale, h->ts_pin};
-  return Pool::instance().run((int64_t)h->B * h->H_q, [j](int64_t b, int64_t e) { run_rows(j, b, e); });
+  return Pool::instance().run(j, (int64_t)h->B * h->H_q, true);
 }
 
 // Raises the sequence flag of a context whose buffers the caller fills itself (stream-ordered behind its copies).
@@ -1041,6 +1142,7 @@ extern "C" int jf_handoff_wait(jf_handoff* h, uint16_t* o_new_dev, void* stream)
 extern "C" int64_t jf_handoff_submit_count(const jf_handoff* h) { return h ? h->submits.load() : -1; }
 
 extern "C" void jf_handoff_destroy(jf_handoff* h) {
+  Pool::instance().quiesce();  // a straggling worker may still be reading a finished job's buffers
   if (!h) return;
   // stream mode: kernels that poll or fill the pinned buffers may still be queued; they need the dispatcher alive
   if (h->mode.load() == 2) (void)hipDeviceSynchronize();
@@ -1122,7 +1224,7 @@ struct AsyncExecutor {
         queue.erase(queue.begin());
       }
       const CpuJob j = item.first;
-      Pool::instance().run((int64_t)j.B * j.H_q, [j](int64_t b, int64_t e) { run_rows(j, b, e); });
+      Pool::instance().run(j, (int64_t)j.B * j.H_q, false);
       std::atomic_thread_fence(std::memory_order_release);
       __atomic_store_n(item.second, (int64_t)1, __ATOMIC_RELEASE);
     }
@@ -1246,12 +1348,14 @@ extern "C" int jf_wait_for_flag(const int64_t* flag, double timeout_s) {
 
 extern "C" int jf_graph_pool_warmup(int n_threads) {
   if (n_threads > 0) Pool::instance().set_threads(n_threads);
-  return Pool::instance().run(1, [](int64_t, int64_t) {}) ? JF_OK : JF_ERR_TIMEOUT;  // starts (or resizes) the workers
+  Pool::instance().warm();  // starts (or resizes) the workers
+  return JF_OK;
 }
 
 extern "C" int64_t jf_graph_submit_count(void) { return g_graph_submits.load(); }
 
 extern "C" int jf_reset_graph_runtime_state(void) {
+  Pool::instance().quiesce();  // a straggling worker may still be reading a finished job's buffers
   g_graph_submits.store(0);
   g_sanitize_count.store(0);
   std::lock_guard<std::mutex> g(g_ctx_mu);
@@ -1260,6 +1364,7 @@ extern "C" int jf_reset_graph_runtime_state(void) {
 }
 
 extern "C" int jf_clear_graph_contexts(void) {
+  Pool::instance().quiesce();  // a straggling worker may still be reading a finished job's buffers
   std::vector<jf_handoff*> old;
   {
     std::lock_guard<std::mutex> g(g_ctx_mu);

@@ -200,6 +200,61 @@ def test_cpu_pool_survives_oversubscription_and_resizing():
     ops.set_cpu_attn_threads(2)
 
 
+def test_cpu_pool_backs_up_a_row_whose_worker_has_stalled():
+    """A worker that stalls inside a row (as if it had lost its core) must not hold the job: an idle worker recomputes
+    the row after the grace period and commits it; what the stalled worker produces later is discarded, also when a
+    newer job has reused the buffers by then."""
+    import time
+    from jetfire_amd import _lib, ops
+    lib = _lib.load()
+    B, Hq, Hkv, K = 2, 16, 4, 64
+    c = make_case(92, B, Hq, Hkv, 512, 3, 2, 64, ragged=False)
+    rng = np.random.default_rng(4)
+    nslots = c["K"].shape[1]
+    hm = torch.from_numpy(O.head_map(B, Hq, Hq // Hkv, K))
+    ksh, vsh = bf16_tensor(c["K"]), bf16_tensor(c["V"])
+    ops.set_cpu_attn_threads(4)
+
+    def case():
+        q = bf16_tensor(O.bf16_round((rng.standard_normal((B, Hq, 128)) / np.sqrt(128)).astype(np.float32)))
+        ts = torch.from_numpy(rng.integers(-1, nslots, size=(B, Hq, K)).astype(np.int64))
+        return q, ts
+    q1, ts1 = case()
+    q2, ts2 = case()
+    want1, want2 = torch.zeros(B, Hq, 128, dtype=torch.bfloat16), torch.zeros(B, Hq, 128, dtype=torch.bfloat16)
+    ops.cpu_topk_attn(q1, ksh, vsh, hm, ts1, want1, 0.09)
+    ops.cpu_topk_attn(q2, ksh, vsh, hm, ts2, want2, 0.09)
+    assert not torch.equal(want1, want2)
+    q, ts, out = q1.clone(), ts1.clone(), torch.zeros(B, Hq, 128, dtype=torch.bfloat16)
+    stall_s = 0.6
+    _lib.check(lib.jf_debug_pool_wait_stragglers(0))
+    try:
+        _lib.check(lib.jf_debug_pool_stall(5, int(stall_s * 1e6)))
+        t0 = time.perf_counter()
+        ops.cpu_topk_attn(q, ksh, vsh, hm, ts, out, 0.09)
+        took = time.perf_counter() - t0
+        assert took < stall_s / 2, took                       # the job did not wait for the stalled worker
+        assert torch.equal(out.view(torch.int16), want1.view(torch.int16))
+        # a newer job over the same buffers while the stalled worker is still asleep on the old one
+        q.copy_(q2)
+        ts.copy_(ts2)
+        ops.cpu_topk_attn(q, ksh, vsh, hm, ts, out, 0.09)
+        assert torch.equal(out.view(torch.int16), want2.view(torch.int16))
+        time.sleep(stall_s + 0.2)                             # the stalled worker wakes up, finishes, and must write nothing
+        assert torch.equal(out.view(torch.int16), want2.view(torch.int16))
+        ops.cpu_topk_attn(q, ksh, vsh, hm, ts, out, 0.09)     # and the pool is whole again
+        assert torch.equal(out.view(torch.int16), want2.view(torch.int16))
+    finally:
+        _lib.check(lib.jf_debug_pool_wait_stragglers(1))
+    # default behaviour of the synchronous call: it returns only when no worker is inside a row any more
+    _lib.check(lib.jf_debug_pool_stall(3, 200000))
+    t0 = time.perf_counter()
+    ops.cpu_topk_attn(q, ksh, vsh, hm, ts, out, 0.09)
+    assert time.perf_counter() - t0 >= 0.19
+    assert torch.equal(out.view(torch.int16), want2.view(torch.int16))
+    ops.set_cpu_attn_threads(2)
+
+
 def test_cpu_topk_attn_single_slot_returns_the_value_row():
     from jetfire_amd import ops
     c = make_case(60, 1, 4, 2, 64, 3, 2, 64, ragged=False)
