@@ -1007,8 +1007,8 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   if (clk && tid == 0) clk[2] = clock64();
 
   // ---- sum of the integer accumulators over the wavefronts: LDS integer atomics into one array in the staging
-  // area (dead now: every wavefront has passed the barrier above), zeroed here, filled after the cut search while
-  // the candidates are emitted, read by `combine` at the end.  Integer sums: exact and independent of the order.
+  // area (dead now: every wavefront has passed the barrier above), zeroed here, filled while the cut is searched,
+  // read by `combine` after the candidates have been emitted.  Integer sums: exact and independent of the order.
   // D layout: row r of a tile sits in lane 16*(r>>2) + column, register r&3; rows are (limb, head), row 12 is the
   // ones row.  Element (set, register r, component c, lane l) lives at xacc[((set*AR + r)*4 + c)*64 + l].
   int* xacc = reinterpret_cast<int*>(stage);
@@ -1061,6 +1061,11 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   // ends.  Otherwise (heavily tied scores) one wavefront falls back to an exact radix select over the keys.
   const int Kcap = p.Kc;
   const int Kt = min(p.top_k, n);
+  if constexpr (HAS_V) {  // the accumulator sums go first: they run in the LDS pipe while the cut is searched
+    lds_barrier();        // (the array is zero everywhere)
+#pragma unroll
+    for (int set = 0; set < NSET; ++set) add_acc(set);
+  }
   for (int h = wave; HAS_TOPK && h < G; h += NW) {
     const int* h0 = hist + h * (SEG * 256) / (Lds::H16 ? 2 : 1);
     // lane l owns buckets 4l .. 4l+3 (ascending bucket = descending score) of every segment's histogram
@@ -1125,9 +1130,6 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   }
   lds_barrier();
   if (clk && tid == 0) clk[6] = clock64();
-#pragma unroll
-  for (int set = 0; set < NSET; ++set)
-    if constexpr (HAS_V) add_acc(set);
   for (int hs = wave; HAS_TOPK && hs < G * SEG; hs += NW) {
     const int h = hs / SEG, seg = hs % SEG;
     const float* srow = sc + h * L;
@@ -1252,9 +1254,10 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
       for (int i = count + lane; i < Kcap; i += 64) ck[i] = 0u;
     }
   }
-  lds_barrier();
   if (clk && tid == 0) clk[3] = clock64();
 
+  // (no barrier: the accumulator sums were complete before the emission started, and nothing below reads what the
+  // emission wrote)
   float lfin = 0.f;
   if (tid < G) {
 #pragma unroll
