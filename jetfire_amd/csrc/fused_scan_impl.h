@@ -1321,7 +1321,8 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   __shared__ float old_sh[MG_WAVES][D];
   __shared__ float w_sh[MG_WAVES];
   __shared__ float wred_f[MG_WAVES];
-  __shared__ uint32_t wred_u[MG_WAVES];
+  __shared__ uint32_t wred_u[MG_WAVES], wred_k[MG_WAVES];
+  __shared__ float wred_g[MG_WAVES];
   __shared__ int wred_i[MG_WAVES], wred_j[MG_WAVES];
   __shared__ int lcount_sh, cut_sh, above_sh, quota_sh;
   __shared__ uint32_t tau_sh;
@@ -1402,13 +1403,48 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   for (int i = tid; i < MG_BINS; i += MG_THREADS) hist[i] = 0;
   if (tid == 0) lcount_sh = 0;
 
-  // ---- split statistics: M, coefficients e^{m_i - M}, l, o_hat
+  // key of candidate f in pass-over-all-candidates loops: registers first, global memory beyond
+  auto key_of = [&](int r) -> uint32_t {
+    const int f = r * MG_THREADS + tid;
+    return (f < flat) ? ck[f] : 0u;
+  };
+  // number of candidates with key >= x (x > 0), identical in every thread
+  auto count_ge = [&](uint32_t x) -> int {
+    int c = 0;
+#pragma unroll
+    for (int r = 0; r < MG_REGK; ++r)
+      if (r < rreg) c += __popcll(__builtin_amdgcn_ballot_w64(kreg[r] >= x));
+    for (int r = MG_REGK; r < rounds; ++r) c += __popcll(__builtin_amdgcn_ballot_w64(key_of(r) >= x));
+    lds_barrier();
+    if (lane == 0) wred_i[wave] = c;
+    lds_barrier();
+    int t = 0;
+#pragma unroll
+    for (int w = 0; w < MG_WAVES; ++w) t += wred_i[w];
+    return t;
+  };
+
+  // The split statistics (M, coefficients e^{m_i - M}, l, o_hat) and the threshold search (range of the candidate
+  // keys, bucket histogram, bucket scan) do not depend on each other: their steps share the barrier intervals.
+  // ---- interval 1: per-wavefront maximum of the split maxima and range of the candidate keys
   if (!PARTIAL) {
     const float v = wave_max(pm);
     if (lane == 0) wred_f[wave] = v;
   }
+  uint32_t kmin = 0xffffffffu, kmax = 0u;
+#pragma unroll
+  for (int r = 0; r < MG_REGK; ++r)
+    if (r < rreg && kreg[r] != 0u) { kmin = min(kmin, kreg[r]); kmax = max(kmax, kreg[r]); }
+  for (int r = MG_REGK; r < rounds; ++r) {
+    const uint32_t k = key_of(r);
+    if (k != 0u) { kmin = min(kmin, k); kmax = max(kmax, k); }
+  }
+  kmin = wave_min_u(kmin);
+  kmax = wave_max_u(kmax);
+  if (lane == 0) { wred_u[wave] = kmin; wred_k[wave] = kmax; }
   lds_barrier();
   if (mclk && tid == 0) mclk[6] = clock64();
+  // ---- interval 2: M, the coefficients, per-wavefront sums of l; the candidates drop into MG_BINS linear buckets
   float M = -INFINITY;
   if (!PARTIAL) {
 #pragma unroll
@@ -1417,18 +1453,37 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
     const float coef = (pm == -INFINITY) ? 0.f : __expf(pm - M);
     if (tid < NS) coef_sh[tid] = coef;
     const float v = wave_sum(pl * coef);  // fixed reduction tree: deterministic
-    lds_barrier();                      // wred_f was read above
-    if (lane == 0) wred_f[wave] = v;
+    if (lane == 0) wred_g[wave] = v;
   }
   int total = 0;
   for (int s2 = 0; s2 < NL; ++s2) total += cnt_sh[s2];
+#pragma unroll
+  for (int w = 0; w < MG_WAVES; ++w) { kmin = min(kmin, wred_u[w]); kmax = max(kmax, wred_k[w]); }
+  const float hi = key_to_score(kmax), lo = key_to_score(kmin);
+  const float range = hi - lo;
+  const float iw = (range > 0.f && isfinite(range)) ? ((float)MG_BINS - 0.01f) / range : 0.f;
+  const float ba = -iw, bb = isfinite(hi) ? hi * iw : 0.f;
+  auto bin_of = [&](uint32_t k) -> int {
+    return (int)__builtin_amdgcn_fmed3f(__builtin_fmaf(key_to_score(k), ba, bb), 0.f, (float)(MG_BINS - 1));
+  };
+  const bool take_all = (total <= K);  // (uniform) every candidate wins: no threshold
+  if (!take_all) {
+#pragma unroll
+    for (int r = 0; r < MG_REGK; ++r)
+      if (r < rreg && kreg[r] != 0u) atomicAdd(&hist[bin_of(kreg[r])], 1);
+    for (int r = MG_REGK; r < rounds; ++r) {
+      const uint32_t k = key_of(r);
+      if (k != 0u) atomicAdd(&hist[bin_of(k)], 1);
+    }
+  }
   lds_barrier();
   if (mclk && tid == 0) mclk[7] = clock64();
+  // ---- interval 3: 1/l, the partial sums of o_hat; first half of the bucket scan
   float inv_z = 0.f;
   if (!PARTIAL) {
     float lsum = 0.f;
 #pragma unroll
-    for (int w = 0; w < MG_WAVES; ++w) lsum += wred_f[w];
+    for (int w = 0; w < MG_WAVES; ++w) lsum += wred_g[w];
     inv_z = (lsum > 0.f) ? 1.0f / lsum : 0.f;
     if (tid == 0 && p.softmax_m) {
       p.softmax_m[bh] = M;
@@ -1441,6 +1496,16 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
       inv_z = p.stats_iz[bh];
     }
   }
+  // thread t owns buckets BPT*t .. BPT*t + BPT-1 (bucket 0 = largest scores): which bucket holds the K-th largest
+  constexpr int BPT = MG_BINS / MG_THREADS;
+  int cb[BPT], mine = 0;
+#pragma unroll
+  for (int u = 0; u < BPT; ++u) {
+    cb[u] = hist[BPT * tid + u];
+    mine += cb[u];
+  }
+  const int incl = wave_incl_scan_i(mine);
+  if (lane == 63) wred_j[wave] = incl;
   if constexpr (!PARTIAL && MODE != FS_STAGE_A) {
     // o_hat: four thread groups take every fourth split, then a fixed-order sum
     const int d = tid & (D - 1), q4 = tid >> 7;
@@ -1466,7 +1531,10 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
       }
     }
     red_sh[q4][d] = o;
-    lds_barrier();
+  }
+  lds_barrier();
+  // ---- interval 4: o_hat; the bucket of the K-th largest candidate
+  if constexpr (!PARTIAL && MODE != FS_STAGE_A) {
     if (tid < D) {
       float o2 = red_sh[0][tid];
 #pragma unroll
@@ -1477,73 +1545,10 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   }
   if (mclk && tid == 0) mclk[1] = clock64();
 
-  // key of candidate f in pass-over-all-candidates loops: registers first, global memory beyond
-  auto key_of = [&](int r) -> uint32_t {
-    const int f = r * MG_THREADS + tid;
-    return (f < flat) ? ck[f] : 0u;
-  };
-  // number of candidates with key >= x (x > 0), identical in every thread
-  auto count_ge = [&](uint32_t x) -> int {
-    int c = 0;
-#pragma unroll
-    for (int r = 0; r < MG_REGK; ++r)
-      if (r < rreg) c += __popcll(__builtin_amdgcn_ballot_w64(kreg[r] >= x));
-    for (int r = MG_REGK; r < rounds; ++r) c += __popcll(__builtin_amdgcn_ballot_w64(key_of(r) >= x));
-    lds_barrier();
-    if (lane == 0) wred_i[wave] = c;
-    lds_barrier();
-    int t = 0;
-#pragma unroll
-    for (int w = 0; w < MG_WAVES; ++w) t += wred_i[w];
-    return t;
-  };
-
   uint32_t tau = 0;
   int quota = 0;
-  const bool take_all = (total <= K);
   if (!take_all) {
-    // range of the candidate keys
-    uint32_t kmin = 0xffffffffu, kmax = 0u;
-#pragma unroll
-    for (int r = 0; r < MG_REGK; ++r)
-      if (r < rreg && kreg[r] != 0u) { kmin = min(kmin, kreg[r]); kmax = max(kmax, kreg[r]); }
-    for (int r = MG_REGK; r < rounds; ++r) {
-      const uint32_t k = key_of(r);
-      if (k != 0u) { kmin = min(kmin, k); kmax = max(kmax, k); }
-    }
-    kmin = wave_min_u(kmin);
-    kmax = wave_max_u(kmax);
-    if (lane == 0) { wred_u[wave] = kmin; wred_i[wave] = (int)kmax; }
-    lds_barrier();
-#pragma unroll
-    for (int w = 0; w < MG_WAVES; ++w) { kmin = min(kmin, wred_u[w]); kmax = max(kmax, (uint32_t)wred_i[w]); }
-    const float hi = key_to_score(kmax), lo = key_to_score(kmin);
-    const float range = hi - lo;
-    const float iw = (range > 0.f && isfinite(range)) ? ((float)MG_BINS - 0.01f) / range : 0.f;
-    const float ba = -iw, bb = isfinite(hi) ? hi * iw : 0.f;
-    auto bin_of = [&](uint32_t k) -> int {
-      return (int)__builtin_amdgcn_fmed3f(__builtin_fmaf(key_to_score(k), ba, bb), 0.f, (float)(MG_BINS - 1));
-    };
-#pragma unroll
-    for (int r = 0; r < MG_REGK; ++r)
-      if (r < rreg && kreg[r] != 0u) atomicAdd(&hist[bin_of(kreg[r])], 1);
-    for (int r = MG_REGK; r < rounds; ++r) {
-      const uint32_t k = key_of(r);
-      if (k != 0u) atomicAdd(&hist[bin_of(k)], 1);
-    }
-    lds_barrier();
     {
-      // thread t owns buckets BPT*t .. BPT*t + BPT-1 (bucket 0 = largest scores): which bucket holds the K-th largest
-      constexpr int BPT = MG_BINS / MG_THREADS;
-      int cb[BPT], mine = 0;
-#pragma unroll
-      for (int u = 0; u < BPT; ++u) {
-        cb[u] = hist[BPT * tid + u];
-        mine += cb[u];
-      }
-      const int incl = wave_incl_scan_i(mine);
-      if (lane == 63) wred_j[wave] = incl;
-      lds_barrier();
       int run = incl - mine;
       for (int w = 0; w < wave; ++w) run += wred_j[w];
 #pragma unroll
