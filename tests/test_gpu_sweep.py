@@ -41,3 +41,40 @@ def test_fused_scan_random_geometry(seed):
     finally:
         _lib.check(lib.jf_debug_split_len(0))
     check_against_oracle(scheme, c, S, K, out)
+
+
+@pytest.mark.parametrize("seed", range(0, 64, 2))
+def test_two_call_form_random_geometry(seed):
+    """The same draw through the reference-named Stage A and Stage B operators (run on the kernels of the one-pass
+    form without the other stage): every output bit-equal to the one-pass form's, which the test above pins to the
+    oracle."""
+    import torch
+    from jetfire_amd import _lib, ops
+    scheme, B, Hq, Hkv, S, lens, K, split = _draw(seed)
+    if scheme in ("k3v4", "k4v2"):
+        scheme = "k3v2" if seed % 4 == 0 else "k4v4"        # the stage-wise forms take the K3V2 and K4V4 side formats
+    if scheme == "k4v4" and K < 64:
+        K = 64                                              # int8tc_qk_scores_topk_stats starts at 64
+    kb, vb, gs = SCHEMES[scheme]
+    c = make_case(500 + seed, B, Hq, Hkv, S, kb, vb, gs, lens=lens, extra_blocks=int(seed % 4))
+    d = to_device(c)
+    lib = _lib.load()
+    print(f"case: {scheme} B={B} Hq={Hq} Hkv={Hkv} S={S} lens={lens} K={K} split={split}", flush=True)
+    assert ops.get_split_impl() == "fast"
+    _lib.check(lib.jf_debug_split_len(split))
+    try:
+        o_hat, slots, o_old, W, idx, m, iz, scores = [t.clone() for t in run_fused(scheme, c, d, S, K)]
+        args = (d["q"], d["kd"], d["ks"], d["bt"], d["lens"], S, Hq, Hkv, 16, 128 ** -0.5, K)
+        if kb == 3:
+            sc2, idx2, slots2 = ops.int3_qk_scores_topk(*args)
+            stage_b = ops.int2_softmax_v_with_pre_corr_wvs2
+        else:
+            sc2, idx2, slots2, m2, iz2 = ops.int8tc_qk_scores_topk_stats(*args)
+            assert torch.equal(m2, m) and torch.equal(iz2, iz)
+            stage_b = ops.int4_softmax_v_with_pre_corr_wvs2_scores
+        assert torch.equal(sc2.view(torch.int32), scores.view(torch.int32))
+        assert torch.equal(idx2, idx) and torch.equal(slots2, slots)
+        o_hat2, o_old2, W2 = stage_b(sc2, d["vd"], d["vs"], d["bt"], d["lens"], idx2, S, Hq, Hkv, 16, K)
+    finally:
+        _lib.check(lib.jf_debug_split_len(0))
+    assert torch.equal(o_hat2, o_hat) and torch.equal(o_old2, o_old) and torch.equal(W2, W)
