@@ -232,6 +232,14 @@ int jf_stage_a_topk(int key_format, int group_size,
                     float* scores, int64_t* topk_idx, int64_t* topk_slots,
                     float* softmax_m, float* softmax_inv_z,
                     void* workspace, size_t workspace_bytes, void* stream);
+/* jf_topk_slots on the kernels of the fused step (top_k <= 1024): the same outputs as jf_topk_slots, i.e.
+ * topk_slots_kernel_v5 / topk_slots_stats_kernel_v5 (jetfire_vllm/csrc/int3_qk_scores.cu:426-554,
+ * jetfire_vllm/csrc/int8tc_qk_scores.cu:1678-1823).  workspace: jf_topk_slots_fast_workspace_bytes(). */
+size_t jf_topk_slots_fast_workspace_bytes(int B, int H_q, int max_S, int top_k);
+int jf_topk_slots_fast(const float* scores, const int32_t* seq_lens, const int64_t* block_table,
+                       int B, int H_q, int max_S, int max_blocks, int block_size, int top_k,
+                       int64_t* topk_idx, int64_t* topk_slots, float* softmax_m, float* softmax_inv_z,
+                       void* workspace, size_t workspace_bytes, void* stream);
 /* jf_stage_b_softmax_v replaces int2_softmax_v_with_pre_corr_wvs2 (jetfire_vllm/csrc/int2_softmax_v.cu:792-901;
  * value_format JF_SCHEME_K3V2: INT2 values, group 64 or 128) and int4_softmax_v_with_pre_corr_wvs2_scores
  * (jetfire_vllm/csrc/int4_softmax_v.cu:2203-2235; value_format JF_SCHEME_K4V4: INT4 values, group 128), with exact

@@ -74,7 +74,9 @@ typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
 //   FS_FULL     Stage A + Stage B + top-k in one pass (keys and values streamed once, scores never in HBM)
 //   FS_STAGE_A  Stage A alone: scores (optionally written out), top-k, softmax statistics; no value stream
 //   FS_STAGE_B  Stage B alone: scores and winners are inputs; value stream, o_hat and the pre-correction terms
-constexpr int FS_FULL = 0, FS_STAGE_A = 1, FS_STAGE_B = 2;
+//   FS_TOPK     selection alone: scores are an input; top-k, slots and softmax statistics (scan kernel only; its
+//               merge is the FS_STAGE_A one)
+constexpr int FS_FULL = 0, FS_STAGE_A = 1, FS_STAGE_B = 2, FS_TOPK = 3;
 
 constexpr int FS_MAX_TOPK = 1024;      // winners cached in LDS by the merge kernel
 constexpr int FS_CAND_SLACK = 256;     // extra candidate slots per (row, split): room for the whole cut bucket
@@ -228,9 +230,9 @@ __device__ inline float uniform_f(float v) {
 template <int MODE, int SCHEME, int G, int NG>
 __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kernel(FusedParams p) {
   using Lds = ScanLds<SCHEME, G, NG>;
-  constexpr bool HAS_K = (MODE != FS_STAGE_B);     // key stream and phase A
-  constexpr bool HAS_V = (MODE != FS_STAGE_A);     // value stream and the P.V part of phase B
-  constexpr bool HAS_TOPK = (MODE != FS_STAGE_B);  // histograms and phase C
+  constexpr bool HAS_K = (MODE == FS_FULL || MODE == FS_STAGE_A);  // key stream and phase A
+  constexpr bool HAS_V = (MODE == FS_FULL || MODE == FS_STAGE_B);  // value stream and the P.V part of phase B
+  constexpr bool HAS_TOPK = (MODE != FS_STAGE_B);                  // histograms and phase C
   constexpr bool K3 = Lds::K3;
   constexpr bool V2 = Lds::V2;
   constexpr int NSET = Lds::NSET;
@@ -521,16 +523,18 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
 #pragma unroll
     for (int h = 0; h < G; ++h) {
       const float* srow = p.scores_in + (head0 + h) * (size_t)p.max_S + s0;
-      float mx = -INFINITY;
+      float mx = -INFINITY, mn = INFINITY;
       for (int t = tid; t < nch * 64; t += NT) {
         const float v = (t < n) ? srow[t] : -INFINITY;
         sc[h * L + t] = v;
         mx = fmaxf(mx, v);
+        mn = fminf(mn, (t < n) ? v : INFINITY);
       }
       mx = wave_max(mx);
+      mn = -wave_max(-mn);
       if (lane == 0) {
         red_f[wave][h] = mx;
-        red_f[wave][G + h] = mx;  // (the minimum only shapes the selection buckets, which this form does not use)
+        red_f[wave][G + h] = mn;  // (the minimum shapes the selection buckets)
       }
     }
   } else if constexpr (K3) {
@@ -2025,6 +2029,8 @@ static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_
   JF_CHECK_ARG(known_scheme(scheme), "fused_scan: unknown scheme %d", scheme);
   JF_CHECK_ARG(MODE == FS_FULL || scheme == JF_SCHEME_K3V2 || scheme == JF_SCHEME_K4V4,
                "fused_scan: the stage-wise forms take the K3V2 or K4V4 side formats");
+  constexpr bool HAS_K = (MODE == FS_FULL || MODE == FS_STAGE_A), HAS_V = (MODE == FS_FULL || MODE == FS_STAGE_B);
+  JF_CHECK_ARG(MODE != FS_TOPK || scheme == JF_SCHEME_K4V4, "fused_scan: the selection-only form uses the K4V4 layout");
   JF_CHECK_ARG((blend_o_new == nullptr) == (blend_out == nullptr), "fused_scan: o_new and out go together");
   JF_CHECK_ARG(B >= 0 && H_q > 0 && H_kv > 0 && max_S >= 0 && H_q % H_kv == 0, "fused_scan: bad shape");
   const int G = H_q / H_kv;
@@ -2043,18 +2049,18 @@ static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_
   JF_CHECK_ARG((softmax_m == nullptr) == (softmax_inv_z == nullptr), "fused_scan: softmax_m and softmax_inv_z go together");
   if (B == 0) return JF_OK;
   JF_CHECK_ARG(block_table && seq_lens, "fused_scan: null input");
-  if (MODE != FS_STAGE_B) {
+  if (HAS_K) {
     JF_CHECK_ARG(q && k_data && k_scales, "fused_scan: null input");
     JF_CHECK_ARG(((uintptr_t)k_data & 15) == 0 && ((uintptr_t)q & 15) == 0, "fused_scan: q and k_data must be 16-byte aligned");
-    JF_CHECK_ARG(scores_only ? scores != nullptr : (topk_idx && topk_slots), "fused_scan: null output");
   }
-  if (MODE != FS_STAGE_A) {
+  if (MODE != FS_STAGE_B) JF_CHECK_ARG(scores_only ? scores != nullptr : (topk_idx && topk_slots), "fused_scan: null output");
+  if (HAS_V) {
     JF_CHECK_ARG(v_data && v_scales, "fused_scan: null input");
     JF_CHECK_ARG(((uintptr_t)v_data & 15) == 0 && ((uintptr_t)v_scales & 3) == 0,
                  "fused_scan: v_data must be 16-byte aligned, v_scales 4-byte aligned");
     JF_CHECK_ARG(o_hat && o_old_unnorm && W, "fused_scan: null output");
   }
-  if (MODE == FS_STAGE_B) JF_CHECK_ARG(scores_in != nullptr, "fused_scan: null scores");
+  if (!HAS_K) JF_CHECK_ARG(scores_in != nullptr, "fused_scan: null scores");
   const int NGv = scheme_ng(scheme, group_size);
   FusedParams p;
   p.q = q; p.k_data = k_data; p.k_scales = k_scales; p.v_data = v_data; p.v_scales = v_scales;
@@ -2071,7 +2077,7 @@ static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_
     JF_CHECK_ARG(((uintptr_t)workspace & 255) == 0, "fused_scan: workspace must be 256-byte aligned");
   }
   uint8_t* ws = reinterpret_cast<uint8_t*>(workspace);
-  p.scores = (MODE == FS_STAGE_B) ? nullptr : scores;
+  p.scores = HAS_K ? scores : nullptr;
   p.scores_in = scores_in;
   p.stats_m = p.stats_iz = nullptr;
   p.scores_only = scores_only ? 1 : 0;
@@ -2099,7 +2105,9 @@ static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_
     case 8: JF_FUSED_CASE(SCH, 8, NGG); break;         \
     default: JF_FUSED_CASE(SCH, 16, NGG); break;       \
   }
-  if (scheme == JF_SCHEME_K3V2) {
+  if constexpr (MODE == FS_TOPK) {
+    JF_FUSED_BY_G(JF_SCHEME_K4V4, 1)
+  } else if (scheme == JF_SCHEME_K3V2) {
     if (NGv == 2) JF_FUSED_BY_G(JF_SCHEME_K3V2, 2) else JF_FUSED_BY_G(JF_SCHEME_K3V2, 1)
   } else if (scheme == JF_SCHEME_K4V4) {
     JF_FUSED_BY_G(JF_SCHEME_K4V4, 1)
@@ -2123,8 +2131,9 @@ static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_
     if (big) hipLaunchKernelGGL((fused_merge_kernel<MODE, VB, NGG, 1024, 32, false>), mgrid, dim3(1024), 0, st, p); \
     else hipLaunchKernelGGL((fused_merge_kernel<MODE, VB, NGG, 1024, 8, false>), mgrid, dim3(1024), 0, st, p);       \
   } while (0)
-  if constexpr (MODE == FS_STAGE_A) {  // no value rows are read: one instantiation serves every format
-    JF_MERGE(4, 1);
+  if constexpr (MODE == FS_STAGE_A || MODE == FS_TOPK) {  // no value rows are read: one instantiation serves every format
+    if (big) hipLaunchKernelGGL((fused_merge_kernel<FS_STAGE_A, 4, 1, 1024, 32, false>), mgrid, dim3(1024), 0, st, p);
+    else hipLaunchKernelGGL((fused_merge_kernel<FS_STAGE_A, 4, 1, 1024, 8, false>), mgrid, dim3(1024), 0, st, p);
   } else if (scheme % 10 == 2) {  // INT2 values
     if (NGv == 2) JF_MERGE(2, 2);
     else JF_MERGE(2, 1);

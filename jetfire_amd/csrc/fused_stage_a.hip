@@ -20,3 +20,24 @@ extern "C" int jf_stage_a_topk(int key_format, int group_size, const uint16_t* q
                                topk_slots, nullptr, nullptr, nullptr, softmax_m, softmax_inv_z, scores, nullptr, nullptr,
                                nullptr, workspace, workspace_bytes, stream);
 }
+
+// The selection alone (scores are an input): the fast form of jf_topk_slots for top_k <= 1024.  The rows are grouped
+// four (or two, or one) to a workgroup; nothing else depends on the grouping.
+extern "C" int jf_topk_slots_fast(const float* scores, const int32_t* seq_lens, const int64_t* block_table, int B, int H_q,
+                                  int max_S, int max_blocks, int block_size, int top_k, int64_t* topk_idx,
+                                  int64_t* topk_slots, float* softmax_m, float* softmax_inv_z, void* workspace,
+                                  size_t workspace_bytes, void* stream) {
+  JF_CHECK_ARG(H_q > 0 && top_k > 0, "topk_slots_fast: bad shape");
+  const int G = (H_q % 4 == 0) ? 4 : ((H_q % 2 == 0) ? 2 : 1);
+  return fused_run<FS_TOPK>(JF_SCHEME_K4V4, 128, nullptr, nullptr, nullptr, nullptr, nullptr, block_table, seq_lens, B, H_q,
+                            H_q / G, max_S, max_blocks, (int64_t)1 << 25, block_size, 0.0f, top_k, topk_idx, topk_slots,
+                            nullptr, nullptr, nullptr, softmax_m, softmax_inv_z, nullptr, scores, nullptr, nullptr,
+                            workspace, workspace_bytes, stream);
+}
+
+// Workspace of jf_topk_slots_fast (the grouping is its own).
+extern "C" size_t jf_topk_slots_fast_workspace_bytes(int B, int H_q, int max_S, int top_k) {
+  if (H_q <= 0) return 256;
+  const int G = (H_q % 4 == 0) ? 4 : ((H_q % 2 == 0) ? 2 : 1);
+  return jf_fused_workspace_bytes(JF_SCHEME_K4V4, B, H_q, H_q / G, max_S, top_k);
+}

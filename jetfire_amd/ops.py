@@ -371,6 +371,13 @@ def _topk(scores, block_table, seq_lens, max_S, H_q, block_size, top_k, stats: b
     if stats:
         m = torch.empty((B, H_q), dtype=torch.float32, device=scores.device)
         iz = torch.empty((B, H_q), dtype=torch.float32, device=scores.device)
+    if _split_impl == "fast" and int(top_k) <= 1024 and int(block_size) == 16 and max_S > 0 and B > 0:
+        sc = scores.contiguous()
+        ws = _workspace(scores.device, lib.jf_topk_slots_fast_workspace_bytes(B, H_q, int(max_S), int(top_k)), "fused")
+        _lib.check(lib.jf_topk_slots_fast(sc.data_ptr(), sl.data_ptr(), bt.data_ptr(), B, H_q, int(max_S), bt.size(1), 16,
+                                          int(top_k), idx.data_ptr(), slots.data_ptr(), _ptr(m), _ptr(iz), ws.data_ptr(),
+                                          ws.numel(), _stream(scores)))
+        return idx, slots, m, iz
     _lib.check(lib.jf_topk_slots(scores.data_ptr(), sl.data_ptr(), bt.data_ptr(), B, H_q, int(max_S), bt.size(1),
                                  int(block_size), int(top_k), idx.data_ptr(), slots.data_ptr(), _ptr(m), _ptr(iz),
                                  _stream(scores)))

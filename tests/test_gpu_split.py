@@ -218,7 +218,7 @@ def test_int3_scores_and_topk(B, Hq, Hkv, S, gs, impl):
 
 @pytest.mark.parametrize("B,Hq,Hkv,S", CASES_A)
 @pytest.mark.parametrize("kb,gs", [(2, 64), (2, 128), (4, 64), (4, 128)])
-def test_int2_and_int4_scores_with_the_bf16_model(B, Hq, Hkv, S, kb, gs):
+def test_int2_and_int4_scores_with_the_bf16_model(B, Hq, Hkv, S, kb, gs, impl):
     """int2_qk_scores (symmetric keys, empty k_zp) and int4_qk_scores: bf16 q times bf16-rounded keys."""
     c = make_case(13 + S + gs + kb, B, Hq, Hkv, S, kb, 2, gs)
     d = to_device(c)
@@ -267,7 +267,7 @@ def test_int8tc_scores_bit_exact_topk_and_stats(B, Hq, Hkv, S, impl):
     assert torch.equal(three[1], idx) and torch.equal(three[2], slots)
 
 
-def test_topk_ties_short_rows_and_zero_length():
+def test_topk_ties_short_rows_and_zero_length(impl):
     rng = np.random.default_rng(3)
     B, Hq, S, K = 4, 4, 96, 32
     sc = rng.integers(-2, 3, size=(B, Hq, S)).astype(np.float32)            # heavy ties
@@ -286,9 +286,15 @@ def test_topk_ties_short_rows_and_zero_length():
     ridx, rslots = O.topk_select(sc, lens, bt, S, K)
     assert np.array_equal(idx.cpu().numpy(), ridx)
     assert np.array_equal(slots.cpu().numpy(), rslots)
+    # the operator-level selection (either implementation), with the statistics
+    idx2, slots2, m2, iz2 = ops()._topk(t, bt_t, lens_t, S, Hq, 16, K, True, "t")
+    assert np.array_equal(idx2.cpu().numpy(), ridx) and np.array_equal(slots2.cpu().numpy(), rslots)
+    rm, riz = O.softmax_stats(sc, lens, S)
+    np.testing.assert_allclose(m2.cpu().numpy(), rm, rtol=0, atol=0)
+    np.testing.assert_allclose(iz2.cpu().numpy(), riz, rtol=2e-5)
 
 
-def test_topk_large_row_and_k():
+def test_topk_large_row_and_k(impl):
     rng = np.random.default_rng(4)
     B, Hq, S, K = 1, 2, 40000, 512
     sc = (rng.standard_normal((B, Hq, S)) * 0.15).astype(np.float32)
