@@ -36,6 +36,8 @@ extern "C" {
 #define JF_SCHEME_K4V4 44    /* INT4 keys, INT4 values  (SymInt4K_SymInt4V) */
 #define JF_SCHEME_K3V4 34    /* INT3 keys, INT4 values  (SymInt3K_SymInt4V), group 128 */
 #define JF_SCHEME_K4V2 42    /* INT4 keys, INT2 values  (SymInt4K_SymInt2V), group 128 */
+#define JF_SCHEME_K2V2 22    /* INT2 keys, INT2 values  (SymInt2K_SymInt2V), group 64 or 128 */
+#define JF_SCHEME_K2V4 24    /* INT2 keys, INT4 values  (SymInt2K_SymInt4V), group 128 */
 
 const char* jf_last_error(void);
 const char* jf_version(void);
@@ -182,8 +184,9 @@ int jf_softmax_v_int8_tiles(const float* scores, const float* softmax_m, const f
  * 2785-2935): topk_idx, topk_slots, o_hat, o_old_unnorm, W, and optionally softmax_m / softmax_inv_z.
  * The reference's own single-call form of this contract is int2_fused_attn_topk
  * (jetfire_vllm/kernels/int2_fused_attn_topk.py:5-10).  scheme: JF_SCHEME_K3V2 (group 64 or 128), or
- * JF_SCHEME_K4V4 / JF_SCHEME_K3V4 / JF_SCHEME_K4V2 (group 128): INT3 keys score with the bf16 model of
- * jf_int3_qk_scores, INT4 keys with the int8-Q model of jf_int8tc_qk_scores.  top_k: power of two in [32, 1024] (the split entry points above take up
+ * JF_SCHEME_K4V4 / JF_SCHEME_K3V4 / JF_SCHEME_K4V2 (group 128), JF_SCHEME_K2V2 (group 64 or 128), JF_SCHEME_K2V4 (group
+ * 128): INT3 and symmetric INT2 keys score with the bf16 model of jf_int3_qk_scores / jf_intn_qk_scores
+ * (jetfire_vllm/csrc/int2_qk_scores.cu:66-79), INT4 keys with the int8-Q model of jf_int8tc_qk_scores.  top_k: power of two in [32, 1024] (the split entry points above take up
  * to 8192); num_slots at most 2^25 (row offsets are 32-bit).  If scores is non-NULL the fp32 scores are also written (validation).
  * workspace: jf_fused_workspace_bytes() bytes of device memory. */
 size_t jf_fused_workspace_bytes(int scheme, int B, int H_q, int H_kv, int max_S, int top_k);
@@ -220,7 +223,8 @@ int jf_fused_scan_topk_blend(int scheme, int group_size,
  * top_k <= 1024, num_slots <= 2^25), at a fraction of their time.  workspace: jf_fused_workspace_bytes(format, ...).
  *
  * jf_stage_a_topk replaces int3_qk_scores / int3_qk_scores_topk (jetfire_vllm/csrc/int3_qk_scores.cu:640-655;
- * key_format JF_SCHEME_K3V2: INT3 keys, bf16 model, group 64 or 128) and int8tc_qk_scores / _topk / _topk_stats
+ * key_format JF_SCHEME_K3V2: INT3 keys, bf16 model, group 64 or 128), int2_qk_scores / int2_qk_scores_topk with
+ * symmetric keys (jetfire_vllm/csrc/int2_qk_scores.cu:663-680; key_format JF_SCHEME_K2V2) and int8tc_qk_scores / _topk / _topk_stats
  * (jetfire_vllm/csrc/int8tc_qk_scores.cu:2774-2798; key_format JF_SCHEME_K4V4: INT4 keys, int8-Q model, group 128).
  * scores (B, H_q, max_S) may be NULL (not written); softmax_m / softmax_inv_z may be NULL.  top_k == 0: scores alone
  * (topk_idx, topk_slots and the workspace are then unused). */

@@ -157,8 +157,10 @@ struct ScanLds {
   // SCHEME = 10 * key bits + value bits: the key side (staging, query constants, phase A) and the value side
   // (staging, phase B) are chosen independently
   static constexpr bool K3 = (SCHEME / 10 == 3);
+  static constexpr bool K2 = (SCHEME / 10 == 2);
+  static constexpr bool KLIMB = K2 || K3;  // keys with the bf16 model: fixed-point query limbs against integer codes
   static constexpr bool V2 = (SCHEME % 10 == 2);
-  static_assert((K3 || SCHEME / 10 == 4) && (V2 || SCHEME % 10 == 4), "keys are INT3 or INT4, values INT2 or INT4");
+  static_assert((KLIMB || SCHEME / 10 == 4) && (V2 || SCHEME % 10 == 4), "keys are INT2, INT3 or INT4, values INT2 or INT4");
   static constexpr int NSET = (G + 3) / 4;
   // wavefronts per workgroup: sixteen where the register budget allows (128 VGPRs at 1024 threads), else eight
   static constexpr int NW = (G <= 4) ? 16 : 8;
@@ -166,8 +168,8 @@ struct ScanLds {
   static constexpr int LMAX = NW * 256;  // four 64-position chunks per wavefront
   // emission segments per head (one wavefront each)
   static constexpr int SEG = (NW / G >= 4) ? 4 : ((NW / G >= 2) ? 2 : 1);
-  static constexpr int KP = K3 ? 48 : 64;
-  static constexpr int KROW = K3 ? 48 : 80;     // LDS pitch of a staged key row (INT4: padded against bank conflicts)
+  static constexpr int KP = K2 ? 32 : (K3 ? 48 : 64);
+  static constexpr int KROW = K2 ? 40 : (K3 ? 48 : 80);  // LDS pitch of a staged key row (INT2, INT4: padded against bank conflicts)
   static constexpr int VP = V2 ? 32 : 64;
   // LDS pitch of a staged V row.  INT2 rows (32 bytes) are padded so that 16 consecutive rows hit 16 distinct
   // bank pairs; INT4 rows (64 bytes) keep their pitch and swap their 16-byte quarters instead (quarter q of
@@ -182,10 +184,10 @@ struct ScanLds {
   // sum of the wavefronts' accumulators: one int per (set, accumulator register, component, lane), in the staging
   // area (dead after phase B), followed by one kilobyte per wavefront for the exact selection's histogram
   static constexpr int XACC = NSET * ACC_REGS * 4 * 64 * 4;
-  static constexpr int PREP = K3 ? (int)sizeof(K3Prep<NSET>) : (int)sizeof(QInt8F<NSET>);
+  static constexpr int PREP = KLIMB ? (int)sizeof(K3Prep<NSET>) : (int)sizeof(QInt8F<NSET>);
   // selection histograms: 32-bit counters, or (any INT4 side, where the staging areas are larger and LDS is
   // tighter) two 16-bit counters per word: a (head, segment) histogram counts at most LMAX / SEG <= 4096 positions
-  static constexpr bool H16 = !(K3 && V2);
+  static constexpr bool H16 = !(KLIMB && V2);
   static constexpr int HIST = G * SEG * 256 * (H16 ? 2 : 4);
   static constexpr int AUX = ((PREP > HIST ? PREP : HIST) + 15) & ~15;
   __host__ __device__ static constexpr int stage_bytes() { return NW * WAVE_STAGE; }
@@ -233,7 +235,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   constexpr bool HAS_K = (MODE == FS_FULL || MODE == FS_STAGE_A);  // key stream and phase A
   constexpr bool HAS_V = (MODE == FS_FULL || MODE == FS_STAGE_B);  // value stream and the P.V part of phase B
   constexpr bool HAS_TOPK = (MODE != FS_STAGE_B);                  // histograms and phase C
-  constexpr bool K3 = Lds::K3;
+  constexpr bool K3 = Lds::K3, KLIMB = Lds::KLIMB;
   constexpr bool V2 = Lds::V2;
   constexpr int NSET = Lds::NSET;
   constexpr int SEG = Lds::SEG;
@@ -334,7 +336,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     kl_off[i] = (uint32_t)(o % (16 * KP));
     kl_lds[i] = (uint32_t)((o / KP) * KROW + (o % KP));
   }
-  const uint8_t* ksb = reinterpret_cast<const uint8_t*>(p.k_scales + (size_t)hkv * p.num_slots * (K3 ? NG : 1));
+  const uint8_t* ksb = reinterpret_cast<const uint8_t*>(p.k_scales + (size_t)hkv * p.num_slots * (KLIMB ? NG : 1));
   struct KBuf {
     v4u r[KLD];
     uint32_t s[4];
@@ -347,7 +349,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
       const uint32_t sb = (uint32_t)sbase[chunk * 4 + kl_page[i]];
       kbuf.r[i] = *reinterpret_cast<const v4u*>(kbase + (size_t)(sb * (uint32_t)KP + kl_off[i]));
     }
-    constexpr int KNG = K3 ? NG : 1;  // key scales per row
+    constexpr int KNG = KLIMB ? NG : 1;  // key scales per row
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int sb = __builtin_amdgcn_readfirstlane(sbase[chunk * 4 + j]);  // first slot of the page (uniform)
@@ -379,11 +381,11 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
 
   if constexpr (!HAS_K) {
     // the scores are an input: no query constants
-  } else if constexpr (K3) {
+  } else if constexpr (KLIMB) {
     // Query rows -> 23-bit fixed point per (head, scale group), three balanced int8 limbs, written in the
     // byte order of the MFMA A operand.  One element per thread; group statistics by wavefront reductions.
     K3Prep<NSET>* prep = reinterpret_cast<K3Prep<NSET>*>(aux);
-    if (tid < 128) {
+    if (K3 && tid < 128) {
       const float sm = 1.0f + (float)tid * (1.0f / 128.0f);
       const float t3 = 3.0f * sm;  // exact in fp32
       prep->eps[tid] = 256.0f * ((bf16_to_f32(f32_to_bf16(t3)) - t3) / sm);
@@ -417,11 +419,13 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
       const int l1 = (int)(int8_t)(r1 & 255);
       const int l2 = (r1 - l1) >> 8;
       const int set = h >> 2, hh = h & 3;
-      // channel d of the key row sits in byte 4*(d&3) + ((d>>3)&3) of a 16-byte k-block (the order the plane
-      // spread produces); with two scale groups MFMA g covers group g only (see the lane swap in phase A)
-      const int mi = (NG == 2) ? (d >> 6) : ((d >> 2) & 1);
-      const int kb = (NG == 2) ? (((d >> 5) & 1) + 2 * ((d >> 2) & 1)) : (d >> 5);
-      const int by = 4 * (d & 3) + ((d >> 3) & 3);
+      // A lane of phase A spreads the 32 channels 32*lg .. 32*lg+31 of its token into two 16-byte operands u = 0, 1
+      // (dword e, byte b).  INT3 (plane spread): channel 8b + 4u + e; INT2 (four codes per byte): channel 16u + 4b + e.
+      // With two scale groups MFMA g covers group g only (see the lane swap in phase A).
+      const int u = K3 ? ((d >> 2) & 1) : ((d >> 4) & 1);
+      const int mi = (NG == 2) ? (d >> 6) : u;
+      const int kb = (NG == 2) ? (((d >> 5) & 1) + 2 * u) : (d >> 5);
+      const int by = 4 * (d & 3) + (K3 ? ((d >> 3) & 3) : ((d >> 2) & 3));
       prep->aop[set][4 * hh + 0][kb][mi][by] = (int8_t)l0;
       prep->aop[set][4 * hh + 1][kb][mi][by] = (int8_t)l1;
       prep->aop[set][4 * hh + 2][kb][mi][by] = (int8_t)l2;
@@ -432,7 +436,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
       const int h = tid / NG, g = tid % NG;
       const int sum = (NG == 2) ? prep->sum_w[2 * h + g] : prep->sum_w[2 * h] + prep->sum_w[2 * h + 1];
       const int e = prep->exp_w[2 * h + ((NG == 2) ? g : 0)];
-      prep->sq4[h][g] = 4 * sum;
+      prep->sq4[h][g] = (K3 ? 4 : 2) * sum;  // the codes are used unsigned: offset 4 (INT3) or 2 (INT2)
       prep->qsc[h][g] = ldexpf(p.attn_scale, e - 22);
     }
   } else {
@@ -537,7 +541,9 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
         red_f[wave][G + h] = mn;  // (the minimum shapes the selection buckets)
       }
     }
-  } else if constexpr (K3) {
+  } else if constexpr (KLIMB) {
+    // INT2 keys: the same scheme without the second contraction: (code - 2) * scale is exact in bf16 for every code,
+    // so the reference's rounding (int2_qk_scores.cu:66-79) changes nothing; the codes sit four to a byte, MSB first.
     // INT3 keys on v_mfma_i32_16x16x64_i8.  The bf16 query row is held exactly as a 23-bit fixed-point number
     // per (head, scale group), split into three balanced int8 limbs that sit in different A-operand rows
     // (row = 4*head + limb), so one MFMA yields the three integer partial sums of a (token, head) in the
@@ -563,7 +569,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
         qsc[set][g] = prep->qsc[set * 4 + lg][g];
       }
     }
-    const uint8_t* krd = kst + t16 * KROW + lg * 4;  // this lane's plane dwords of token t16 of a page
+    const uint8_t* krd = kst + t16 * KROW + lg * (K3 ? 4 : 8);  // this lane's plane dwords (INT2: its 8 bytes) of token t16 of a page
     float mxl[NSET], mnl[NSET];
 #pragma unroll
     for (int set = 0; set < NSET; ++set) {
@@ -577,15 +583,22 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const uint8_t* rp = krd + j * 16 * KROW;
-        Pj[j][0] = *reinterpret_cast<const uint32_t*>(rp);
-        Pj[j][1] = *reinterpret_cast<const uint32_t*>(rp + 16);
-        Pj[j][2] = *reinterpret_cast<const uint32_t*>(rp + 32);
+        if constexpr (K3) {
+          Pj[j][0] = *reinterpret_cast<const uint32_t*>(rp);
+          Pj[j][1] = *reinterpret_cast<const uint32_t*>(rp + 16);
+          Pj[j][2] = *reinterpret_cast<const uint32_t*>(rp + 32);
+        } else {
+          const v2u x = *reinterpret_cast<const v2u*>(rp);
+          Pj[j][0] = x[0];
+          Pj[j][1] = x[1];
+          Pj[j][2] = 0u;
+        }
         const uint32_t sw = Sx[j];
         sgj[j][0] = bf16_to_f32((uint16_t)(sw & 0xffffu));
-        egj[j][0] = prep->eps[sw & 0x7fu];
+        egj[j][0] = K3 ? prep->eps[sw & 0x7fu] : 0.f;
         if (NG == 2) {
           sgj[j][NG - 1] = bf16_to_f32((uint16_t)(sw >> 16));
-          egj[j][NG - 1] = prep->eps[(sw >> 16) & 0x7fu];
+          egj[j][NG - 1] = K3 ? prep->eps[(sw >> 16) & 0x7fu] : 0.f;
         }
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -593,14 +606,20 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
       for (int j = 0; j < 4; ++j) {
         const uint32_t P0 = Pj[j][0], P1 = Pj[j][1], P2 = Pj[j][2];
         v4i Bc[2], Br[2];
-        Bc[0][0] = (int)((P0 >> 5) & 0x07070707u);
-        Bc[0][1] = (int)((P0 >> 2) & 0x07070707u);
-        Bc[0][2] = (int)(((P0 << 1) & 0x06060606u) | ((P1 >> 7) & 0x01010101u));
-        Bc[0][3] = (int)((P1 >> 4) & 0x07070707u);
-        Bc[1][0] = (int)((P1 >> 1) & 0x07070707u);
-        Bc[1][1] = (int)(((P1 << 2) & 0x04040404u) | ((P2 >> 6) & 0x03030303u));
-        Bc[1][2] = (int)((P2 >> 3) & 0x07070707u);
-        Bc[1][3] = (int)(P2 & 0x07070707u);
+        if constexpr (K3) {
+          Bc[0][0] = (int)((P0 >> 5) & 0x07070707u);
+          Bc[0][1] = (int)((P0 >> 2) & 0x07070707u);
+          Bc[0][2] = (int)(((P0 << 1) & 0x06060606u) | ((P1 >> 7) & 0x01010101u));
+          Bc[0][3] = (int)((P1 >> 4) & 0x07070707u);
+          Bc[1][0] = (int)((P1 >> 1) & 0x07070707u);
+          Bc[1][1] = (int)(((P1 << 2) & 0x04040404u) | ((P2 >> 6) & 0x03030303u));
+          Bc[1][2] = (int)((P2 >> 3) & 0x07070707u);
+          Bc[1][3] = (int)(P2 & 0x07070707u);
+        } else {  // four codes per byte, MSB first: dword e of operand u holds code e of each of the four bytes
+          (void)P2;
+          Bc[0] = (v4i){(int)((P0 >> 6) & 0x03030303u), (int)((P0 >> 4) & 0x03030303u), (int)((P0 >> 2) & 0x03030303u), (int)(P0 & 0x03030303u)};
+          Bc[1] = (v4i){(int)((P1 >> 6) & 0x03030303u), (int)((P1 >> 4) & 0x03030303u), (int)((P1 >> 2) & 0x03030303u), (int)(P1 & 0x03030303u)};
+        }
         if (NG == 2) {
           // Bc[0] <- lanes 0-31 keep their first half, lanes 32-63 receive the second half of lane-32;
           // Bc[1] <- lanes 0-31 receive the first half of lane+32, lanes 32-63 keep their second half
@@ -611,11 +630,13 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
             Bc[1][e] = (int)sw[1];
           }
         }
+        if constexpr (K3) {
 #pragma unroll
-        for (int u = 0; u < 2; ++u)
+          for (int u = 0; u < 2; ++u)
 #pragma unroll
-          for (int e = 0; e < 4; ++e)
-            Br[u][e] = (int)__builtin_amdgcn_perm(0x01000000u, 0x0000ff00u, (uint32_t)Bc[u][e]);
+            for (int e = 0; e < 4; ++e)
+              Br[u][e] = (int)__builtin_amdgcn_perm(0x01000000u, 0x0000ff00u, (uint32_t)Bc[u][e]);
+        }
         // per-token scales (both groups) and the rounding coefficient
         float sg[NG], eg[NG];
 #pragma unroll
@@ -633,20 +654,26 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
 #pragma unroll
             for (int g = 0; g < NG; ++g) {
               const v4i Dc = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][g], Bc[g], zero, 0, 0, 0);
-              const v4i Dr = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][g], Br[g], zero, 0, 0, 0);
               const int xc = (((Dc[2] << 8) + Dc[1]) << 8) + Dc[0] - sq4[set][g];
-              const int xr = (Dr[2] << 8) + Dr[1];
-              const float v = __builtin_fmaf(eg[g], (float)xr, (float)xc);
+              float v = (float)xc;
+              if constexpr (K3) {
+                const v4i Dr = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][g], Br[g], zero, 0, 0, 0);
+                const int xr = (Dr[2] << 8) + Dr[1];
+                v = __builtin_fmaf(eg[g], (float)xr, v);
+              }
               score = __builtin_fmaf(v, sg[g] * qsc[set][g], score);
             }
           } else {
             v4i Dc = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][0], Bc[0], zero, 0, 0, 0);
-            v4i Dr = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][0], Br[0], zero, 0, 0, 0);
             Dc = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][1], Bc[1], Dc, 0, 0, 0);
-            Dr = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][1], Br[1], Dr, 0, 0, 0);
             const int xc = (((Dc[2] << 8) + Dc[1]) << 8) + Dc[0] - sq4[set][0];
-            const int xr = (Dr[2] << 8) + Dr[1];
-            const float v = __builtin_fmaf(eg[0], (float)xr, (float)xc);
+            float v = (float)xc;
+            if constexpr (K3) {
+              v4i Dr = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][0], Br[0], zero, 0, 0, 0);
+              Dr = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][1], Br[1], Dr, 0, 0, 0);
+              const int xr = (Dr[2] << 8) + Dr[1];
+              v = __builtin_fmaf(eg[0], (float)xr, v);
+            }
             score = __builtin_fmaf(v, sg[0] * qsc[set][0], score);
           }
           const int h = set * 4 + lg;
@@ -1864,6 +1891,12 @@ inline int lmax_dispatch(int scheme, int G, int NG) {
   JF_LMAX_CASE(JF_SCHEME_K3V4, 8, 1); JF_LMAX_CASE(JF_SCHEME_K3V4, 16, 1);
   JF_LMAX_CASE(JF_SCHEME_K4V2, 1, 1); JF_LMAX_CASE(JF_SCHEME_K4V2, 2, 1); JF_LMAX_CASE(JF_SCHEME_K4V2, 4, 1);
   JF_LMAX_CASE(JF_SCHEME_K4V2, 8, 1); JF_LMAX_CASE(JF_SCHEME_K4V2, 16, 1);
+  JF_LMAX_CASE(JF_SCHEME_K2V2, 1, 1); JF_LMAX_CASE(JF_SCHEME_K2V2, 2, 1); JF_LMAX_CASE(JF_SCHEME_K2V2, 4, 1);
+  JF_LMAX_CASE(JF_SCHEME_K2V2, 8, 1); JF_LMAX_CASE(JF_SCHEME_K2V2, 16, 1);
+  JF_LMAX_CASE(JF_SCHEME_K2V2, 1, 2); JF_LMAX_CASE(JF_SCHEME_K2V2, 2, 2); JF_LMAX_CASE(JF_SCHEME_K2V2, 4, 2);
+  JF_LMAX_CASE(JF_SCHEME_K2V2, 8, 2); JF_LMAX_CASE(JF_SCHEME_K2V2, 16, 2);
+  JF_LMAX_CASE(JF_SCHEME_K2V4, 1, 1); JF_LMAX_CASE(JF_SCHEME_K2V4, 2, 1); JF_LMAX_CASE(JF_SCHEME_K2V4, 4, 1);
+  JF_LMAX_CASE(JF_SCHEME_K2V4, 8, 1); JF_LMAX_CASE(JF_SCHEME_K2V4, 16, 1);
 #undef JF_LMAX_CASE
   return 256;
 }
@@ -1918,7 +1951,7 @@ inline void fused_plan(int scheme, int NG, int B, int H_q, int H_kv, int max_S, 
   const int kCUs = device_cus();
   constexpr double kScanFixed = 8.5;
   // one chunk per wavefront, all wavefronts; the mixed schemes are priced like the wider one
-  const double per_chunk = (scheme == JF_SCHEME_K3V2) ? 5.9 : 6.6;
+  const double per_chunk = (scheme == JF_SCHEME_K3V2 || scheme == JF_SCHEME_K2V2) ? 5.9 : 6.6;
   int L = 256;
   double best = -1.0;
   for (int cand = 256; cand <= lmax; cand += 256) {
@@ -2007,9 +2040,12 @@ int launch_scan(const FusedParams& p, hipStream_t st) {
 }
 
 inline bool known_scheme(int scheme) {
-  return scheme == JF_SCHEME_K3V2 || scheme == JF_SCHEME_K4V4 || scheme == JF_SCHEME_K3V4 || scheme == JF_SCHEME_K4V2;
+  return scheme == JF_SCHEME_K3V2 || scheme == JF_SCHEME_K4V4 || scheme == JF_SCHEME_K3V4 || scheme == JF_SCHEME_K4V2 ||
+         scheme == JF_SCHEME_K2V2 || scheme == JF_SCHEME_K2V4;
 }
-inline int scheme_ng(int scheme, int group_size) { return (scheme == JF_SCHEME_K3V2) ? D / group_size : 1; }
+// scale groups per row: the schemes without an INT4 side may use 64-channel groups
+inline bool scheme_any_group(int scheme) { return scheme == JF_SCHEME_K3V2 || scheme == JF_SCHEME_K2V2; }
+inline int scheme_ng(int scheme, int group_size) { return scheme_any_group(scheme) ? D / group_size : 1; }
 
 
 // The whole step on caller-provided workspace memory; every public entry point of the fused forms ends here.
@@ -2027,8 +2063,9 @@ static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_
                      const float* scores_in, const uint16_t* blend_o_new, uint16_t* blend_out, void* workspace,
                      size_t workspace_bytes, void* stream) {
   JF_CHECK_ARG(known_scheme(scheme), "fused_scan: unknown scheme %d", scheme);
-  JF_CHECK_ARG(MODE == FS_FULL || scheme == JF_SCHEME_K3V2 || scheme == JF_SCHEME_K4V4,
-               "fused_scan: the stage-wise forms take the K3V2 or K4V4 side formats");
+  JF_CHECK_ARG(MODE == FS_FULL || scheme == JF_SCHEME_K3V2 || scheme == JF_SCHEME_K4V4 ||
+                   (MODE == FS_STAGE_A && scheme == JF_SCHEME_K2V2),
+               "fused_scan: the stage-wise forms take the K3V2 or K4V4 side formats (Stage A also K2V2)");
   constexpr bool HAS_K = (MODE == FS_FULL || MODE == FS_STAGE_A), HAS_V = (MODE == FS_FULL || MODE == FS_STAGE_B);
   JF_CHECK_ARG(MODE != FS_TOPK || scheme == JF_SCHEME_K4V4, "fused_scan: the selection-only form uses the K4V4 layout");
   JF_CHECK_ARG((blend_o_new == nullptr) == (blend_out == nullptr), "fused_scan: o_new and out go together");
@@ -2037,7 +2074,7 @@ static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_
   JF_CHECK_ARG(G == 1 || G == 2 || G == 4 || G == 8 || G == 16, "fused_scan: GQA group %d not in {1,2,4,8,16}", G);
   JF_CHECK_ARG(block_size == 16, "fused_scan only supports block_size=16");
   JF_CHECK_ARG(group_size == 64 || group_size == 128, "fused_scan: group_size must be 64 or 128 (got %d)", group_size);
-  JF_CHECK_ARG(scheme == JF_SCHEME_K3V2 || group_size == 128,
+  JF_CHECK_ARG(scheme_any_group(scheme) || group_size == 128,
                "fused_scan: the INT4 sides (int8-Q keys, INT4 values) need group_size 128");
   const bool scores_only = (MODE == FS_STAGE_A) && top_k == 0;
   if (scores_only) top_k = 32;  // (any valid width: the plan depends on it, the kernel stops before using it)
@@ -2111,8 +2148,14 @@ static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_
     if (NGv == 2) JF_FUSED_BY_G(JF_SCHEME_K3V2, 2) else JF_FUSED_BY_G(JF_SCHEME_K3V2, 1)
   } else if (scheme == JF_SCHEME_K4V4) {
     JF_FUSED_BY_G(JF_SCHEME_K4V4, 1)
-  } else if constexpr (MODE == FS_FULL) {  // the mixed pairs exist in the one-pass form only
-    if (scheme == JF_SCHEME_K3V4) JF_FUSED_BY_G(JF_SCHEME_K3V4, 1) else JF_FUSED_BY_G(JF_SCHEME_K4V2, 1)
+  } else if constexpr (MODE == FS_FULL || MODE == FS_STAGE_A) {
+    if (scheme == JF_SCHEME_K2V2) {
+      if (NGv == 2) JF_FUSED_BY_G(JF_SCHEME_K2V2, 2) else JF_FUSED_BY_G(JF_SCHEME_K2V2, 1)
+    } else if constexpr (MODE == FS_FULL) {  // the mixed pairs exist in the one-pass form only
+      if (scheme == JF_SCHEME_K3V4) JF_FUSED_BY_G(JF_SCHEME_K3V4, 1)
+      else if (scheme == JF_SCHEME_K4V2) JF_FUSED_BY_G(JF_SCHEME_K4V2, 1)
+      else JF_FUSED_BY_G(JF_SCHEME_K2V4, 1)
+    }
   }
 #undef JF_FUSED_BY_G
 #undef JF_FUSED_CASE

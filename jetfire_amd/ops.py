@@ -291,6 +291,8 @@ def _intn_qk_scores(nbits: int, name: str, q, k_data, k_scales, block_table, seq
     q, kd, ks, bt, sl = _stage_a_args(q, k_data, k_scales, block_table, seq_lens, H_q, H_kv, HEAD_DIM * nbits // 8)
     ng = ks.size(2)
     _check(ng in (1, 2), f"{name} currently supports K quant groups 1 or 2, got {ng}")
+    if nbits == 2 and k_zp is None and _fast_shape(H_q, H_kv, block_size, max_S, kd.size(1)):
+        return _stage_a_fast(22, q, kd, ks, bt, sl, max_S, H_q, H_kv, attn_scale, None, False)[0]
     if k_zp is not None:
         k_zp = (k_zp.unsqueeze(-1) if k_zp.dim() == 2 else k_zp).contiguous()
         _check(k_zp.is_cuda and k_zp.dtype == torch.bfloat16 and k_zp.shape == ks.shape,
@@ -315,6 +317,11 @@ def int2_qk_scores(q, k_data, k_scales, k_zp, block_table, seq_lens, max_S, H_q,
 def int2_qk_scores_topk(q, k_data, k_scales, k_zp, block_table, seq_lens, max_S, H_q, H_kv, block_size, attn_scale,
                         top_k) -> List[torch.Tensor]:
     """int2_qk_scores.cu:583-660 -> [scores, topk_idx, topk_slots]."""
+    symmetric = k_zp is None or k_zp.numel() == 0
+    if symmetric and _fast_shape(H_q, H_kv, block_size, max_S, k_data.size(1) if k_data.dim() == 3 else 0, top_k):
+        q_, kd, ks, bt, sl = _stage_a_args(q, k_data, k_scales, block_table, seq_lens, H_q, H_kv, 32)
+        _check(ks.size(2) in (1, 2), f"int2_qk_scores currently supports K quant groups 1 or 2, got {ks.size(2)}")
+        return list(_stage_a_fast(22, q_, kd, ks, bt, sl, max_S, H_q, H_kv, attn_scale, int(top_k), False)[:3])
     scores = int2_qk_scores(q, k_data, k_scales, k_zp, block_table, seq_lens, max_S, H_q, H_kv, block_size, attn_scale)
     idx, slots, _, _ = _topk(scores, block_table, seq_lens, max_S, H_q, block_size, top_k, False, "int2_qk_scores_topk")
     return [scores, idx, slots]
@@ -574,10 +581,11 @@ def fused_attn_topk(scheme: str, q, k_data, k_scales, v_data, v_scales, block_ta
 
     The single-call contract is the one of the reference's int2_fused_attn_topk
     (jetfire_vllm/kernels/int2_fused_attn_topk.py:5-10) extended to INT3 / INT4 keys (INT4: the int8-Q scoring
-    model) with INT2 / INT4 values: "k3v2" (group 64 or 128), "k4v4", "k3v4", "k4v2" (group 128)."""
+    model) and symmetric INT2 keys with INT2 / INT4 values: "k3v2", "k2v2" (group 64 or 128), "k4v4", "k3v4", "k4v2",
+    "k2v4" (group 128)."""
     lib = _lib.load()
-    scheme_id = {"k3v2": 32, "k4v4": 44, "k3v4": 34, "k4v2": 42}.get(scheme)
-    _check(scheme_id is not None, f"unknown scheme {scheme!r} (k3v2, k4v4, k3v4, k4v2)")
+    scheme_id = {"k3v2": 32, "k4v4": 44, "k3v4": 34, "k4v2": 42, "k2v2": 22, "k2v4": 24}.get(scheme)
+    _check(scheme_id is not None, f"unknown scheme {scheme!r} (k3v2, k4v4, k3v4, k4v2, k2v2, k2v4)")
     kp, vp = 16 * (scheme_id // 10), 16 * (scheme_id % 10)
     q, kd, ks, bt, sl = _stage_a_args(q, k_data, k_scales, block_table, seq_lens, H_q, H_kv, kp)
     _gpu(v_data, v_scales)

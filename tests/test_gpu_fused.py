@@ -27,8 +27,8 @@ def check_against_oracle(scheme, c, S, K, out):
     o_hat, slots, o_old, W, idx, m, iz, scores = [t.cpu().numpy() for t in out]
     kb, vb, gs = c["kbits"], c["vbits"], c["gs"]
     Hq, Hkv = c["Hq"], c["Hkv"]
-    if kb == 3:
-        ref_sc = O.scores_bf16_model(c["q"], c["kd"], c["ks"], c["bt"], c["lens"], S, Hq, Hkv, 16, SCALE, 3, gs)
+    if kb in (2, 3):
+        ref_sc = O.scores_bf16_model(c["q"], c["kd"], c["ks"], c["bt"], c["lens"], S, Hq, Hkv, 16, SCALE, kb, gs)
         valid = np.isfinite(ref_sc)
         assert np.array_equal(np.isneginf(scores), ~valid)
         np.testing.assert_allclose(scores[valid], ref_sc[valid], atol=2e-5, rtol=2e-5)
@@ -81,13 +81,18 @@ CASES = [
     ("k3v4", 1, 8, 2, 5000, [4987], 256), ("k4v2", 1, 8, 2, 5000, [4987], 512),
     ("k3v4", 1, 4, 4, 300, None, 32), ("k4v2", 1, 4, 2, 300, None, 64),
     ("k3v4", 1, 16, 1, 600, None, 64), ("k4v2", 1, 16, 1, 600, None, 64),
+    # symmetric INT2 keys (bf16 model, exact for every code)
+    ("k2v2", 2, 8, 2, 512, None, 64), ("k2v2_g128", 2, 8, 2, 700, None, 128), ("k2v4", 2, 8, 2, 512, None, 64),
+    ("k2v2", 3, 32, 4, 512, [17, 257, 512], 256), ("k2v4", 3, 32, 4, 512, [17, 257, 512], 256),
+    ("k2v2", 4, 8, 2, 32, [0, 1, 9, 17], 32), ("k2v2", 1, 8, 2, 5000, [4987], 256), ("k2v4", 1, 8, 2, 5000, [4987], 512),
+    ("k2v2", 1, 4, 4, 300, None, 32), ("k2v4", 1, 4, 2, 300, None, 64), ("k2v2", 1, 16, 1, 600, None, 64),
 ]
 
 
 @pytest.mark.parametrize("scheme,B,Hq,Hkv,S,lens,K", CASES)
 def test_fused_scan_matches_oracle(scheme, B, Hq, Hkv, S, lens, K):
     kb, vb, gs = {"k3v2": (3, 2, 64), "k4v4": (4, 4, 128), "k3v2_g128": (3, 2, 128), "k3v4": (3, 4, 128),
-                  "k4v2": (4, 2, 128)}[scheme]
+                  "k4v2": (4, 2, 128), "k2v2": (2, 2, 64), "k2v2_g128": (2, 2, 128), "k2v4": (2, 4, 128)}[scheme]
     c = make_case(70 + S + Hq, B, Hq, Hkv, S, kb, vb, gs, lens=lens, extra_blocks=3)
     d = to_device(c)
     out = run_fused(scheme, c, d, S, K)

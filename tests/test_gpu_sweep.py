@@ -9,7 +9,8 @@ from tests.test_gpu_fused import check_against_oracle, run_fused
 
 pytestmark = pytest.mark.gpu
 
-SCHEMES = {"k3v2": (3, 2, 64), "k3v2_g128": (3, 2, 128), "k4v4": (4, 4, 128), "k3v4": (3, 4, 128), "k4v2": (4, 2, 128)}
+SCHEMES = {"k3v2": (3, 2, 64), "k3v2_g128": (3, 2, 128), "k4v4": (4, 4, 128), "k3v4": (3, 4, 128), "k4v2": (4, 2, 128),
+           "k2v2": (2, 2, 64), "k2v2_g128": (2, 2, 128), "k2v4": (2, 4, 128)}
 
 
 def _draw(seed):
@@ -26,7 +27,7 @@ def _draw(seed):
     return scheme, B, G * Hkv, Hkv, S, lens, K, split
 
 
-@pytest.mark.parametrize("seed", range(64))
+@pytest.mark.parametrize("seed", range(80))
 def test_fused_scan_random_geometry(seed):
     from jetfire_amd import _lib
     scheme, B, Hq, Hkv, S, lens, K, split = _draw(seed)
@@ -51,8 +52,8 @@ def test_two_call_form_random_geometry(seed):
     import torch
     from jetfire_amd import _lib, ops
     scheme, B, Hq, Hkv, S, lens, K, split = _draw(seed)
-    if scheme in ("k3v4", "k4v2"):
-        scheme = "k3v2" if seed % 4 == 0 else "k4v4"        # the stage-wise forms take the K3V2 and K4V4 side formats
+    if scheme in ("k3v4", "k4v2", "k2v2", "k2v2_g128", "k2v4"):
+        scheme = "k3v2" if seed % 4 == 0 else "k4v4"        # the two operator pairs below are those of K3V2 and K4V4
     if scheme == "k4v4" and K < 64:
         K = 64                                              # int8tc_qk_scores_topk_stats starts at 64
     kb, vb, gs = SCHEMES[scheme]
