@@ -11,6 +11,8 @@
 //            INT3 keys: the bf16 query as exact 23-bit fixed point in three int8 limbs, codes spread from the
 //                       byte planes with shift/mask on dwords, a second contraction with the indicator of
 //                       codes +-3 reproduces the reference's bf16 rounding of the dequantised key.
+//            INT2 keys: the same limbs against the four-codes-per-byte rows; no second contraction, every
+//                       dequantised INT2 key is exact in bf16.
 //            INT4 keys: int8-quantised Q, exact nibble codes, one accumulator row per 32-channel block, the
 //                       reference's fp32 rescale order (bit-equal to the split-form kernel).
 //            scores[G][L] -> LDS (fp32), running max / min per head.
@@ -22,12 +24,16 @@
 //   phase C  from the bucket histograms: the smallest bucket range that holds the split's top min(K, n) scores
 //            and fits the candidate buffer; its positions are emitted as (key, position) in ascending
 //            position, one wavefront per (head, segment).  Heavily tied scores fall back to a radix select.
-//   exchange of the wavefronts' integer accumulators through LDS, exact int64 recombination -> partial o.
+//   sum of the wavefronts' integer accumulators with LDS integer atomics (while the cut is searched), exact
+//   int64 recombination -> partial o.
 // Launch 2, fused_merge_kernel, grid (B, H_q): selects the global top-k among the candidates (ties to
 // the lower position, ascending output), merges the split partials
 //   M = max m_i, l = sum l_i e^{m_i-M}, o_hat = sum o_i e^{m_i-M} / l
 // (the split-KV combine of jetfire_vllm/csrc/fused_decode_wmma.cu:1226-1253), and computes the
 // pre-correction terms o_old_unnorm, W over the winners (jetfire_vllm/csrc/int2_softmax_v.cu:738-788).
+// Both kernels take a template argument MODE: the whole step, or one stage alone (Stage A: scores written out,
+// top-k, statistics; Stage B: scores and winners given, value stream; selection alone), for callers that keep the
+// reference's separate operators.
 //
 // This header holds the kernels, the launch planner and the launcher; it is included by the translation units that
 // instantiate them (fused_scan.hip and the stage-wise forms), each for its own set of template arguments.
