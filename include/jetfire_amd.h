@@ -381,6 +381,9 @@ int jf_handoff_stream_wait_blend(jf_handoff* h, const float* o_hat, const float*
                                  uint16_t* out, uint16_t* o_new_dev, void* stream);
 int jf_handoff_status(jf_handoff* h);
 int jf_handoff_set_device_wait_limit_us(jf_handoff* h, int64_t us);
+/* on != 0: jf_handoff_stream_wait_blend writes zero for every non-finite output element, the graph-mode guard of
+ * _sanitize_decode_output_if_needed (jetfire_vllm/adapter/decode_path.py:1133-1149) folded into the blend. */
+int jf_handoff_set_output_sanitize(jf_handoff* h, int on);
 /* Test aid: while on, the dispatcher ignores published flags (a correction that never finishes, without
  * hanging anything: the device-side wait runs into its limit). */
 int jf_handoff_debug_pause(jf_handoff* h, int on);

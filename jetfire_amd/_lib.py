@@ -62,6 +62,7 @@ SIGNATURES = {
     "jf_handoff_stream_wait_blend": (I, [P, P, P, P, P, P, P]),
     "jf_handoff_status": (I, [P]),
     "jf_handoff_set_device_wait_limit_us": (I, [P, L]),
+    "jf_handoff_set_output_sanitize": (I, [P, I]),
     "jf_handoff_debug_pause": (I, [P, I]),
     "jf_handoff_destroy": (None, [P]),
     "jf_blend": (I, [P, P, P, P, P, I, I, I, P]),

@@ -167,9 +167,17 @@ def _handoff_for(store, B: int, H_q: int, H_kv: int, K: int, scale: float, *, st
         if threads > 0:
             ops.set_cpu_attn_threads(threads)
         h = ops.CpuTopkHandoff(B, H_q, H_kv, K, store.k_shadow, store.v_shadow, scale)
+        if stream_mode and _sanitize_output_enabled():   # the graph-mode guard, inside the blending wait kernel
+            h.set_output_sanitize(True)
         cache[key] = h
         _STORES_WITH_HANDOFFS.add(store)
     return h
+
+
+def _sanitize_output_enabled() -> bool:
+    """decode_path.py:1142: non-finite decode outputs become zero in graph mode unless JETFIRE_SANITIZE_DECODE_OUTPUT=0
+    (a NaN that enters the next layer poisons q, k and v of every later step of a replayed graph)."""
+    return os.environ.get("JETFIRE_SANITIZE_DECODE_OUTPUT", "1") != "0"
 
 
 def _all_handoffs():
@@ -392,5 +400,7 @@ def _decode_batched(*, impl, layer, query, attn_metadata, output):
         tmp = torch.empty(n_seqs, H_q, D, dtype=torch.bfloat16, device=query.device)
         ops.blend_unnorm_into(o_hat, o_old, W, o_new, tmp)
         out_view.copy_(tmp.to(out_view.dtype))
+    if graph_mode and _sanitize_output_enabled():   # (decode_path.py:1133-1149)
+        torch.nan_to_num(out_view, nan=0.0, posinf=0.0, neginf=0.0, out=out_view)
     pool.record_decode_hit()
     return output

@@ -689,6 +689,7 @@ struct jf_handoff {
                                    // device's own sequence counter (stream mode)
   std::atomic<int> mode{0};        // 0 = not used yet, 1 = host-blocking wait, 2 = stream mode (device-side wait)
   std::atomic<int> paused{0};      // test aid: published flags are ignored
+  std::atomic<int> sanitize{0};    // stream_wait_blend writes zero for non-finite outputs
   int64_t stream_seen = 0;         // stream mode: last sequence number the shared poller has served
   bool registered = false;         // stream mode: known to the shared poller
   uint64_t device_wait_ticks = 0;  // bound of the device-side wait, in ticks of the 100 MHz wall clock
@@ -755,7 +756,7 @@ __global__ __launch_bounds__(1024) void handoff_wait_fetch_kernel(const int64_t*
                                                                   const uint4* __restrict__ src, uint4* dst, int n16,
                                                                   const float* __restrict__ o_hat,
                                                                   const float* __restrict__ o_old,
-                                                                  const float* __restrict__ W, uint4* out) {
+                                                                  const float* __restrict__ W, uint4* out, int sanitize) {
   // Each lane owns up to U items per pass (item = eight bf16 elements).  What does not depend on the CPU -- the
   // o_hat / o_old rows and W of the first pass -- is loaded before the wait, and the U reads from pinned host
   // memory of a pass are issued together, so that one PCIe round trip covers them.
@@ -815,8 +816,12 @@ __global__ __launch_bounds__(1024) void handoff_wait_fetch_kernel(const int64_t*
         uint32_t r[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          const float lo = __builtin_fmaf(Wv[u], bf16_to_f32((uint16_t)(n[e] & 0xffffu)), hh[2 * e]) - dd[2 * e];
-          const float hi = __builtin_fmaf(Wv[u], bf16_to_f32((uint16_t)(n[e] >> 16)), hh[2 * e + 1]) - dd[2 * e + 1];
+          float lo = __builtin_fmaf(Wv[u], bf16_to_f32((uint16_t)(n[e] & 0xffffu)), hh[2 * e]) - dd[2 * e];
+          float hi = __builtin_fmaf(Wv[u], bf16_to_f32((uint16_t)(n[e] >> 16)), hh[2 * e + 1]) - dd[2 * e + 1];
+          if (sanitize) {  // non-finite outputs become zero (decode_path.py:1133-1149)
+            lo = isfinite(lo) ? lo : 0.0f;
+            hi = isfinite(hi) ? hi : 0.0f;
+          }
           r[e] = (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
         }
         out[i] = make_uint4(r[0], r[1], r[2], r[3]);
@@ -1076,8 +1081,14 @@ extern "C" int jf_handoff_stream_wait(jf_handoff* h, uint16_t* o_new_dev, void* 
   hipLaunchKernelGGL(handoff_wait_fetch_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, h->flag_pin + 8,
                      reinterpret_cast<const int64_t*>(h->counter_dev + 2), h->flag_pin + 16, h->device_wait_ticks,
                      reinterpret_cast<const uint4*>(h->o_pin), reinterpret_cast<uint4*>(o_new_dev), n16,
-                     (const float*)nullptr, (const float*)nullptr, (const float*)nullptr, (uint4*)nullptr);
+                     (const float*)nullptr, (const float*)nullptr, (const float*)nullptr, (uint4*)nullptr, 0);
   JF_CHECK_HIP(hipGetLastError());
+  return JF_OK;
+}
+
+extern "C" int jf_handoff_set_output_sanitize(jf_handoff* h, int on) {
+  JF_CHECK_ARG(h, "handoff_set_output_sanitize: null argument");
+  h->sanitize.store(on ? 1 : 0);
   return JF_OK;
 }
 
@@ -1091,7 +1102,7 @@ extern "C" int jf_handoff_stream_wait_blend(jf_handoff* h, const float* o_hat, c
   hipLaunchKernelGGL(handoff_wait_fetch_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, h->flag_pin + 8,
                      reinterpret_cast<const int64_t*>(h->counter_dev + 2), h->flag_pin + 16, h->device_wait_ticks,
                      reinterpret_cast<const uint4*>(h->o_pin), reinterpret_cast<uint4*>(o_new_dev), n16, o_hat,
-                     o_old_unnorm, W, reinterpret_cast<uint4*>(out));
+                     o_old_unnorm, W, reinterpret_cast<uint4*>(out), h->sanitize.load());
   JF_CHECK_HIP(hipGetLastError());
   return JF_OK;
 }
@@ -1283,7 +1294,7 @@ extern "C" int jf_submit_ctx_stream_wait(int64_t ctx, void* stream) {
   hipLaunchKernelGGL(handoff_wait_fetch_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, h->flag_pin + 8,
                      reinterpret_cast<const int64_t*>(h->counter_dev + 2), h->flag_pin + 16, h->device_wait_ticks,
                      (const uint4*)nullptr, (uint4*)nullptr, 0, (const float*)nullptr, (const float*)nullptr,
-                     (const float*)nullptr, (uint4*)nullptr);
+                     (const float*)nullptr, (uint4*)nullptr, 0);
   JF_CHECK_HIP(hipGetLastError());
   return JF_OK;
 }

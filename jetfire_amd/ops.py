@@ -967,6 +967,10 @@ class CpuTopkHandoff:
         _lib.check(_lib.load().jf_handoff_stream_wait_blend(self._h, o_hat.data_ptr(), o_old_unnorm.data_ptr(), W.data_ptr(),
                                                             out.data_ptr(), _ptr(o_new), _stream(out)))
 
+    def set_output_sanitize(self, on: bool) -> None:
+        """stream_wait_blend writes zero for non-finite outputs (decode_path.py:1133-1149)."""
+        _lib.check(_lib.load().jf_handoff_set_output_sanitize(self._h, 1 if on else 0))
+
     def check_status(self) -> None:
         """Raises if a correction failed or a device-side wait ran into its limit (call after a synchronise)."""
         _lib.check(_lib.load().jf_handoff_status(self._h))

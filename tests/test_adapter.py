@@ -94,6 +94,9 @@ def test_handoff_contexts_belong_to_their_store(adapter, monkeypatch):
             self.failed = False
             made.append(self)
 
+        def set_output_sanitize(self, on):
+            self.sanitize = bool(on)
+
         def check_status(self):
             if self.failed:
                 raise RuntimeError("handoff: the device-side wait for the CPU correction ran into its limit")
@@ -111,6 +114,7 @@ def test_handoff_contexts_belong_to_their_store(adapter, monkeypatch):
     assert decode_path._handoff_for(store, 2, 8, 2, 32, 0.1, stream_mode=True) is h1
     assert decode_path._handoff_for(store, 2, 8, 2, 32, 0.1, stream_mode=False) is not h1
     assert h1.k_ptr == store.k_shadow.data_ptr() and len(made) == 2
+    assert h1.sanitize and not hasattr(made[1], "sanitize")      # the graph-mode guard is set on stream-mode contexts only
     decode_path.check_decode_handoffs()
     h1.failed = True
     with pytest.raises(RuntimeError, match="ran into its limit"):

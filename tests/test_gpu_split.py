@@ -575,6 +575,44 @@ def test_handoff_stream_wait_blend_more_rows_than_one_pass():
     assert torch.equal(out.view(torch.int16), want.view(torch.int16))
 
 
+def test_handoff_stream_wait_blend_can_zero_non_finite_outputs():
+    """The graph-mode guard of the reference (decode_path.py:1133-1149) inside the blending wait kernel: with the option
+    set, non-finite outputs come out as zero and every other element is the plain blend; without it they pass."""
+    B, Hq, Hkv, K = 2, 8, 2, 32
+    o = ops()
+    rng = np.random.default_rng(6)
+    num_slots = 256
+    ksh = bf16_tensor(O.bf16_round(rng.standard_normal((Hkv, num_slots, 128)).astype(np.float32)))
+    vsh = bf16_tensor(O.bf16_round(rng.standard_normal((Hkv, num_slots, 128)).astype(np.float32)))
+    q = bf16_tensor(O.bf16_round((rng.standard_normal((B, Hq, 128)) / np.sqrt(128)).astype(np.float32))).cuda()
+    s = torch.from_numpy(rng.integers(0, num_slots, size=(B, Hq, K)).astype(np.int64)).cuda()
+    o.set_cpu_attn_threads(2)
+    o_hat = torch.randn(B, Hq, 128, device="cuda")
+    o_old = torch.randn(B, Hq, 128, device="cuda") * 0.1
+    W = torch.rand(B, Hq, device="cuda")
+    o_hat[0, 1, 5] = float("nan")
+    o_hat[1, 7, 127] = float("inf")
+    o_old[1, 0, 0] = float("inf")
+    outs = []
+    for on in (False, True):
+        h = o.CpuTopkHandoff(B, Hq, Hkv, K, ksh, vsh, 0.1)
+        h.set_output_sanitize(on)
+        out = torch.zeros(B, Hq, 128, dtype=torch.bfloat16, device="cuda")
+        o_new = torch.zeros_like(out)
+        h.stream_submit(q, s)
+        h.stream_wait_blend(o_hat, o_old, W, out, o_new)
+        torch.cuda.synchronize()
+        h.check_status()
+        h.close()
+        outs.append((out, o_new))
+    plain = o.blend_unnorm(o_hat, o_old, W, outs[0][1])
+    assert torch.equal(outs[0][0].view(torch.int16), plain.view(torch.int16))
+    assert not torch.isfinite(outs[0][0].float()).all()
+    clean = torch.nan_to_num(plain.float(), nan=0.0, posinf=0.0, neginf=0.0).to(torch.bfloat16)
+    assert torch.equal(outs[1][0].view(torch.int16), clean.view(torch.int16))
+    assert torch.isfinite(outs[1][0].float()).all()
+
+
 def test_handoff_stream_wait_is_bounded():
     """A correction that never finishes (the dispatcher is told to ignore the flag): the device-side wait runs
     into its limit, the kernel ends, o_new is zero, the status reports it, and later waits fall through."""
