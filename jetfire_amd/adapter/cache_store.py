@@ -113,9 +113,9 @@ class JetFireInt4CacheStore:
         """Name the fused decode kernels know this store by, or None (split kernels / unsupported)."""
         if self.k_asymmetric:
             return None
-        if (self.k_nbits, self.v_nbits) in ((3, 2), (2, 2)) and self.group_size in (64, 128):
-            return f"k{self.k_nbits}v2"
-        if (self.k_nbits, self.v_nbits) in ((4, 4), (3, 4), (4, 2), (2, 4)) and self.group_size == 128:
+        if self.k_nbits not in (2, 3, 4) or self.v_nbits not in (2, 3, 4):
+            return None
+        if self.group_size == 128 or (self.group_size == 64 and 4 not in (self.k_nbits, self.v_nbits)):
             return f"k{self.k_nbits}v{self.v_nbits}"
         return None
 

@@ -166,7 +166,8 @@ struct ScanLds {
   static constexpr bool K2 = (SCHEME / 10 == 2);
   static constexpr bool KLIMB = K2 || K3;  // keys with the bf16 model: fixed-point query limbs against integer codes
   static constexpr bool V2 = (SCHEME % 10 == 2);
-  static_assert((KLIMB || SCHEME / 10 == 4) && (V2 || SCHEME % 10 == 4), "keys are INT2, INT3 or INT4, values INT2 or INT4");
+  static constexpr bool V3 = (SCHEME % 10 == 3);
+  static_assert((KLIMB || SCHEME / 10 == 4) && (V2 || V3 || SCHEME % 10 == 4), "keys and values are INT2, INT3 or INT4");
   static constexpr int NSET = (G + 3) / 4;
   // wavefronts per workgroup: sixteen where the register budget allows (128 VGPRs at 1024 threads), else eight
   static constexpr int NW = (G <= 4) ? 16 : 8;
@@ -176,12 +177,14 @@ struct ScanLds {
   static constexpr int SEG = (NW / G >= 4) ? 4 : ((NW / G >= 2) ? 2 : 1);
   static constexpr int KP = K2 ? 32 : (K3 ? 48 : 64);
   static constexpr int KROW = K2 ? 40 : (K3 ? 48 : 80);  // LDS pitch of a staged key row (INT2, INT4: padded against bank conflicts)
-  static constexpr int VP = V2 ? 32 : 64;
+  static constexpr int VP = V2 ? 32 : (V3 ? 48 : 64);
   // LDS pitch of a staged V row.  INT2 rows (32 bytes) are padded so that 16 consecutive rows hit 16 distinct
-  // bank pairs; INT4 rows (64 bytes) keep their pitch and swap their 16-byte quarters instead (quarter q of
-  // row r sits at q ^ ((r >> 2) & 3)), which has the same effect without the padding bytes.
-  static constexpr bool VSWZ = !V2;
-  static constexpr int VROW = VSWZ ? VP : VP + 8;
+  // bank pairs; INT4 rows (64 bytes) keep their pitch and swap their 16-byte quarters instead (quarter q of row r
+  // sits at q ^ ((r >> 2) & 3)), which has the same effect without the padding bytes.  INT3 rows (48 bytes: 16
+  // consecutive rows already hit distinct bank pairs) swap the 8-byte halves of every plane in rows 16..31 and
+  // 48..63, so that the two 16-row groups one 8-byte read serves in a cycle do not meet either.
+  static constexpr bool VSWZ = !(V2 || V3);
+  static constexpr int VROW = (VSWZ || V3) ? VP : VP + 8;
   static constexpr int VST = 64 * VROW;
   static constexpr int WL = NG * NSET * 64 * 16;  // per (group, set): one 16-byte weight row per token
   static constexpr int KST = 64 * KROW;
@@ -242,14 +245,14 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   constexpr bool HAS_V = (MODE == FS_FULL || MODE == FS_STAGE_B);  // value stream and the P.V part of phase B
   constexpr bool HAS_TOPK = (MODE != FS_STAGE_B);                  // histograms and phase C
   constexpr bool K3 = Lds::K3, KLIMB = Lds::KLIMB;
-  constexpr bool V2 = Lds::V2;
+  constexpr bool V2 = Lds::V2, V3 = Lds::V3;
   constexpr int NSET = Lds::NSET;
   constexpr int SEG = Lds::SEG;
   constexpr int KP = Lds::KP;
   constexpr int KROW = Lds::KROW;
   constexpr int VP = Lds::VP;
   constexpr int VROW = Lds::VROW;
-  constexpr int VOFF = V2 ? 2 : 8;  // code offset of the V format
+  constexpr int VOFF = V2 ? 2 : (V3 ? 4 : 8);  // code offset of the V format
   constexpr int NTILE = 8;          // 8 MFMA column tiles of 16 channels
   constexpr int AR = Lds::ACC_REGS;
   constexpr float LOG2E = 1.44269504088896340736f;
@@ -493,7 +496,8 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     vl_page[i] = (uint32_t)(o / (16 * VP));
     vl_off[i] = (uint32_t)(o % (16 * VP));
     const int row = o / VP, q16 = (o % VP) / 16;
-    vl_lds[i] = Lds::VSWZ ? (uint32_t)(row * VROW + ((q16 ^ ((row >> 2) & 3)) * 16)) : (uint32_t)(row * VROW + (o % VP));
+    vl_lds[i] = Lds::VSWZ ? (uint32_t)(row * VROW + ((q16 ^ ((row >> 2) & 3)) * 16))
+                          : (uint32_t)(row * VROW + (o % VP) + (V3 ? 8 * ((row >> 4) & 1) : 0));  // (INT3: first half's place)
   }
   struct VBuf {
     v4u r[VLD];
@@ -991,6 +995,46 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
           acc[set][2 * qc + 1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[g][set], Bb, acc[set][2 * qc + 1], 0, 0, 0);
         }
       }
+    } else if (V3) {
+      // Planar INT3: bytes j of the three 16-byte planes form the 24-bit word of channels 8j .. 8j+7, code i at
+      // bits 23-3i .. 21-3i.  A transposed read of one plane's 8-byte half hands lane c the nibble c of 16 tokens:
+      // odd lanes the high nibbles of byte c >> 1, even lanes the low ones.  With one exchange inside the lane
+      // pair (the odd lane needs its partner's plane-0 nibble, the even lane its partner's plane-2 nibble) the odd
+      // lane holds what codes 0..3 of the word are made of and the even lane what codes 4..7 are made of, in the
+      // same three positions: a = [c0 c0 c0 c1], b = [c1 c1 c2 c2], c = [c2 c3 c3 c3] (msb first).
+      const bool odd = (lane & 1) != 0;
+      const int hsw = 8 * ((lane >> 4) & 1);  // rows 16..31, 48..63 keep their plane halves swapped
+#pragma unroll
+      for (int w = 0; w < 2; ++w) {
+        const uint8_t* src = vrow + (w ? 8 - hsw : hsw);
+        const v2i x0 = __builtin_amdgcn_ds_read_tr4_b64_v2i32((__attribute__((address_space(3))) v2i*)(src));
+        const v2i x1 = __builtin_amdgcn_ds_read_tr4_b64_v2i32((__attribute__((address_space(3))) v2i*)(src + 16));
+        const v2i x2 = __builtin_amdgcn_ds_read_tr4_b64_v2i32((__attribute__((address_space(3))) v2i*)(src + 32));
+        v4i Bc[4];
+#pragma unroll
+        for (int hw = 0; hw < 2; ++hw) {  // tokens 0..7 and 8..15 of the lane group, one nibble each
+          const int send = odd ? x2[hw] : x0[hw];
+          const uint32_t b = (uint32_t)dpp_mov<0xb1, 0xf>(0, send);  // quad_perm [1,0,3,2]: the pair partner's value
+          const uint32_t a = (uint32_t)(odd ? x0[hw] : x1[hw]), c = (uint32_t)(odd ? x1[hw] : x2[hw]);
+          // per nibble (bit 3 of the two middle codes is cleared by the byte masks below)
+          const uint32_t n1 = ((b >> 2) & 0x33333333u) | ((a << 2) & ~0x33333333u);
+          const uint32_t n2 = ((c >> 3) & 0x11111111u) | ((b << 1) & ~0x11111111u);
+          Bc[0][2 * hw] = (int)((a >> 1) & 0x07070707u);
+          Bc[0][2 * hw + 1] = (int)((a >> 5) & 0x07070707u);
+          Bc[1][2 * hw] = (int)(n1 & 0x07070707u);
+          Bc[1][2 * hw + 1] = (int)((n1 >> 4) & 0x07070707u);
+          Bc[2][2 * hw] = (int)(n2 & 0x07070707u);
+          Bc[2][2 * hw + 1] = (int)((n2 >> 4) & 0x07070707u);
+          Bc[3][2 * hw] = (int)(c & 0x07070707u);
+          Bc[3][2 * hw + 1] = (int)((c >> 4) & 0x07070707u);
+        }
+        const int g = (NG == 1) ? 0 : w;
+#pragma unroll
+        for (int m = 0; m < 4; ++m)
+#pragma unroll
+          for (int set = 0; set < NSET; ++set)
+            acc[set][4 * w + m] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[g][set], Bc[m], acc[set][4 * w + m], 0, 0, 0);
+      }
     } else {
       const int vx = 16 * ((lane >> 2) & 3);  // quarter swap of this lane's row
 #pragma unroll
@@ -1013,9 +1057,8 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
       if (Lds::VSWZ) {
         *reinterpret_cast<v4u*>(vst + vl_lds[i]) = vbuf.r[i];  // 16-byte aligned with the unpadded pitch
       } else {
-        v2u* dst = reinterpret_cast<v2u*>(vst + vl_lds[i]);
-        dst[0] = (v2u){vbuf.r[i][0], vbuf.r[i][1]};
-        dst[1] = (v2u){vbuf.r[i][2], vbuf.r[i][3]};
+        *reinterpret_cast<v2u*>(vst + vl_lds[i]) = (v2u){vbuf.r[i][0], vbuf.r[i][1]};
+        *reinterpret_cast<v2u*>(vst + (V3 ? (vl_lds[i] ^ 8u) : (vl_lds[i] + 8u))) = (v2u){vbuf.r[i][2], vbuf.r[i][3]};
       }
     }
   };
@@ -1070,6 +1113,8 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
       if (V2) {
         const int e = ((col & 1) ? 0 : 2) + (tile & 1);
         d = (tile >> 1) * 32 + (col >> 1) * 4 + e;
+      } else if (V3) {  // tile = 4 * (64-channel half) + code within the lane's four; odd columns hold codes 0..3
+        d = (tile >> 2) * 64 + (col >> 1) * 8 + ((col & 1) ? 0 : 4) + (tile & 3);
       } else {
         d = tile * 16 + 2 * (col >> 1) + (1 - (col & 1));
       }
@@ -1341,8 +1386,10 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   constexpr int MG_WAVES = MG_THREADS / 64;
   constexpr int VP = D * VBITS / 8;
   constexpr int VOFF = 1 << (VBITS - 1);
-  constexpr int DW = VP / 4;            // dwords per V row
-  constexpr int CPD = 32 / VBITS;       // codes per dword
+  // lanes per winner row and codes per lane: a dword of the row each (INT2, INT4), or (INT3, planar) two bytes of
+  // each of the three planes = 16 codes
+  constexpr int DW = (VBITS == 3) ? 8 : VP / 4;
+  constexpr int CPD = (VBITS == 3) ? 16 : 32 / VBITS;
   constexpr int WPI = 64 / DW;          // winners per wavefront instruction
   __shared__ int hist[MG_BINS];
   __shared__ uint32_t lkey[MG_LIST];
@@ -1791,7 +1838,7 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   float accw = 0.f;
   constexpr int UNR = (256 / (MG_WAVES * WPI) > 0) ? 256 / (MG_WAVES * WPI) : 1;  // 256 winners per pass
   for (int k0 = wave * WPI; k0 < n_out; k0 += UNR * MG_WAVES * WPI) {
-    uint32_t word[UNR];
+    uint32_t word[UNR], word_b[UNR];  // (word_b: INT3 only)
     uint16_t sbits[UNR];
     float wv[UNR];
 #pragma unroll
@@ -1800,7 +1847,16 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
       const int slot = (k < n_out) ? win_slot[k] : -1;
       wv[u] = (slot >= 0) ? win_w[k] : 0.f;
       const uint32_t sl = (uint32_t)max(slot, 0);
-      word[u] = *reinterpret_cast<const uint32_t*>(vbase + (size_t)(sl * (uint32_t)VP) + dwi * 4);
+      if constexpr (VBITS == 3) {  // bytes 2*dwi, 2*dwi+1 of every plane -> the 24-bit words of two 8-code groups
+        const uint8_t* row = vbase + (size_t)(sl * (uint32_t)VP) + dwi * 2;
+        const uint32_t h0 = *reinterpret_cast<const uint16_t*>(row), h1 = *reinterpret_cast<const uint16_t*>(row + 16),
+                       h2 = *reinterpret_cast<const uint16_t*>(row + 32);
+        word[u] = ((h0 & 0xffu) << 16) | ((h1 & 0xffu) << 8) | (h2 & 0xffu);
+        word_b[u] = ((h0 >> 8) << 16) | ((h1 >> 8) << 8) | (h2 >> 8);
+      } else {
+        word[u] = *reinterpret_cast<const uint32_t*>(vbase + (size_t)(sl * (uint32_t)VP) + dwi * 4);
+        word_b[u] = 0;
+      }
       sbits[u] = *reinterpret_cast<const uint16_t*>(vsbase + (size_t)(sl * (uint32_t)(NG * 2)) + g_of_lane * 2);
     }
 #pragma unroll
@@ -1809,8 +1865,13 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
       // byte `byte` of the dword holds its codes MSB first; channel of code c in the dword = dwi*CPD + c
 #pragma unroll
       for (int c = 0; c < CPD; ++c) {
-        const int byte = c / (8 / VBITS), inb = c % (8 / VBITS);
-        const int code = (int)((word[u] >> (8 * byte + (8 - VBITS * (inb + 1)))) & ((1u << VBITS) - 1u)) - VOFF;
+        int code;
+        if constexpr (VBITS == 3) {
+          code = (int)((((c < 8) ? word[u] : word_b[u]) >> (21 - 3 * (c & 7))) & 7u) - VOFF;
+        } else {
+          const int byte = c / (8 / VBITS), inb = c % (8 / VBITS);
+          code = (int)((word[u] >> (8 * byte + (8 - VBITS * (inb + 1)))) & ((1u << VBITS) - 1u)) - VOFF;
+        }
         acc[c] = __builtin_fmaf(ws, (float)code, acc[c]);
       }
       if (dwi == 0) accw += wv[u];
@@ -1839,7 +1900,7 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
       }
       chan += upper ? N / 2 : 0;
     };
-    static_assert(DW == 8 || DW == 16, "V rows of 32 or 64 bytes");
+    static_assert(DW == 8 || DW == 16, "eight or sixteen lanes per V row");
     if constexpr (DW == 8) {
       halve(std::integral_constant<int, 8>{}, std::integral_constant<int, CPD>{});
       halve(std::integral_constant<int, 16>{}, std::integral_constant<int, CPD / 2>{});
@@ -1903,6 +1964,13 @@ inline int lmax_dispatch(int scheme, int G, int NG) {
   JF_LMAX_CASE(JF_SCHEME_K2V2, 8, 2); JF_LMAX_CASE(JF_SCHEME_K2V2, 16, 2);
   JF_LMAX_CASE(JF_SCHEME_K2V4, 1, 1); JF_LMAX_CASE(JF_SCHEME_K2V4, 2, 1); JF_LMAX_CASE(JF_SCHEME_K2V4, 4, 1);
   JF_LMAX_CASE(JF_SCHEME_K2V4, 8, 1); JF_LMAX_CASE(JF_SCHEME_K2V4, 16, 1);
+#define JF_LMAX_ALL_G(SCH, NGG)                                                                      \
+  JF_LMAX_CASE(SCH, 1, NGG); JF_LMAX_CASE(SCH, 2, NGG); JF_LMAX_CASE(SCH, 4, NGG); JF_LMAX_CASE(SCH, 8, NGG); \
+  JF_LMAX_CASE(SCH, 16, NGG)
+  JF_LMAX_ALL_G(JF_SCHEME_K2V3, 1); JF_LMAX_ALL_G(JF_SCHEME_K2V3, 2);
+  JF_LMAX_ALL_G(JF_SCHEME_K3V3, 1); JF_LMAX_ALL_G(JF_SCHEME_K3V3, 2);
+  JF_LMAX_ALL_G(JF_SCHEME_K4V3, 1);
+#undef JF_LMAX_ALL_G
 #undef JF_LMAX_CASE
   return 256;
 }
@@ -1957,7 +2025,7 @@ inline void fused_plan(int scheme, int NG, int B, int H_q, int H_kv, int max_S, 
   const int kCUs = device_cus();
   constexpr double kScanFixed = 8.5;
   // one chunk per wavefront, all wavefronts; the mixed schemes are priced like the wider one
-  const double per_chunk = (scheme == JF_SCHEME_K3V2 || scheme == JF_SCHEME_K2V2) ? 5.9 : 6.6;
+  const double per_chunk = (scheme == JF_SCHEME_K3V2 || scheme == JF_SCHEME_K2V2) ? 5.9 : 6.6;  // (INT3 values: as INT4)
   int L = 256;
   double best = -1.0;
   for (int cand = 256; cand <= lmax; cand += 256) {
@@ -2047,10 +2115,13 @@ int launch_scan(const FusedParams& p, hipStream_t st) {
 
 inline bool known_scheme(int scheme) {
   return scheme == JF_SCHEME_K3V2 || scheme == JF_SCHEME_K4V4 || scheme == JF_SCHEME_K3V4 || scheme == JF_SCHEME_K4V2 ||
-         scheme == JF_SCHEME_K2V2 || scheme == JF_SCHEME_K2V4;
+         scheme == JF_SCHEME_K2V2 || scheme == JF_SCHEME_K2V4 || scheme == JF_SCHEME_K2V3 || scheme == JF_SCHEME_K3V3 ||
+         scheme == JF_SCHEME_K4V3;
 }
 // scale groups per row: the schemes without an INT4 side may use 64-channel groups
-inline bool scheme_any_group(int scheme) { return scheme == JF_SCHEME_K3V2 || scheme == JF_SCHEME_K2V2; }
+inline bool scheme_any_group(int scheme) {
+  return scheme == JF_SCHEME_K3V2 || scheme == JF_SCHEME_K2V2 || scheme == JF_SCHEME_K2V3 || scheme == JF_SCHEME_K3V3;
+}
 inline int scheme_ng(int scheme, int group_size) { return scheme_any_group(scheme) ? D / group_size : 1; }
 
 
@@ -2070,8 +2141,8 @@ static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_
                      size_t workspace_bytes, void* stream) {
   JF_CHECK_ARG(known_scheme(scheme), "fused_scan: unknown scheme %d", scheme);
   JF_CHECK_ARG(MODE == FS_FULL || scheme == JF_SCHEME_K3V2 || scheme == JF_SCHEME_K4V4 ||
-                   (MODE == FS_STAGE_A && scheme == JF_SCHEME_K2V2),
-               "fused_scan: the stage-wise forms take the K3V2 or K4V4 side formats (Stage A also K2V2)");
+                   (MODE == FS_STAGE_A && scheme == JF_SCHEME_K2V2) || (MODE == FS_STAGE_B && scheme == JF_SCHEME_K3V3),
+               "fused_scan: the stage-wise forms take the K3V2 or K4V4 side formats (Stage A also K2V2, Stage B also K3V3)");
   constexpr bool HAS_K = (MODE == FS_FULL || MODE == FS_STAGE_A), HAS_V = (MODE == FS_FULL || MODE == FS_STAGE_B);
   JF_CHECK_ARG(MODE != FS_TOPK || scheme == JF_SCHEME_K4V4, "fused_scan: the selection-only form uses the K4V4 layout");
   JF_CHECK_ARG((blend_o_new == nullptr) == (blend_out == nullptr), "fused_scan: o_new and out go together");
@@ -2154,13 +2225,20 @@ static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_
     if (NGv == 2) JF_FUSED_BY_G(JF_SCHEME_K3V2, 2) else JF_FUSED_BY_G(JF_SCHEME_K3V2, 1)
   } else if (scheme == JF_SCHEME_K4V4) {
     JF_FUSED_BY_G(JF_SCHEME_K4V4, 1)
+  } else if (MODE != FS_STAGE_A && scheme == JF_SCHEME_K3V3) {
+    if constexpr (MODE != FS_STAGE_A) {
+      if (NGv == 2) JF_FUSED_BY_G(JF_SCHEME_K3V3, 2) else JF_FUSED_BY_G(JF_SCHEME_K3V3, 1)
+    }
   } else if constexpr (MODE == FS_FULL || MODE == FS_STAGE_A) {
     if (scheme == JF_SCHEME_K2V2) {
       if (NGv == 2) JF_FUSED_BY_G(JF_SCHEME_K2V2, 2) else JF_FUSED_BY_G(JF_SCHEME_K2V2, 1)
     } else if constexpr (MODE == FS_FULL) {  // the mixed pairs exist in the one-pass form only
       if (scheme == JF_SCHEME_K3V4) JF_FUSED_BY_G(JF_SCHEME_K3V4, 1)
       else if (scheme == JF_SCHEME_K4V2) JF_FUSED_BY_G(JF_SCHEME_K4V2, 1)
-      else JF_FUSED_BY_G(JF_SCHEME_K2V4, 1)
+      else if (scheme == JF_SCHEME_K2V4) JF_FUSED_BY_G(JF_SCHEME_K2V4, 1)
+      else if (scheme == JF_SCHEME_K4V3) JF_FUSED_BY_G(JF_SCHEME_K4V3, 1)
+      else if (NGv == 2) JF_FUSED_BY_G(JF_SCHEME_K2V3, 2)
+      else JF_FUSED_BY_G(JF_SCHEME_K2V3, 1)
     }
   }
 #undef JF_FUSED_BY_G
@@ -2186,6 +2264,9 @@ static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_
   } else if (scheme % 10 == 2) {  // INT2 values
     if (NGv == 2) JF_MERGE(2, 2);
     else JF_MERGE(2, 1);
+  } else if (scheme % 10 == 3) {  // INT3 values
+    if (NGv == 2) JF_MERGE(3, 2);
+    else JF_MERGE(3, 1);
   } else {
     JF_MERGE(4, 1);
   }

@@ -48,10 +48,14 @@ def _workspace(device: torch.device, nbytes: int, tag: str) -> torch.Tensor:
     return buf
 
 
+# the nine symmetric (key bits, value bits) pairs of the fused step: name -> 10 * key bits + value bits
+FUSED_SCHEMES = {f"k{kb}v{vb}": 10 * kb + vb for kb in (2, 3, 4) for vb in (2, 3, 4)}
+
+
 def reserve_fused_workspace(scheme: str, B: int, H_q: int, H_kv: int, max_S: int, top_k: int, device) -> int:
     """Size the current stream's fused-scan workspace for a shape ahead of time (before a graph capture, so that
     no capture or later eager call has to grow it).  Returns the size in bytes."""
-    scheme_id = {"k3v2": 32, "k4v4": 44, "k3v4": 34, "k4v2": 42}[scheme]
+    scheme_id = FUSED_SCHEMES[scheme]
     need = int(_lib.load().jf_fused_workspace_bytes(scheme_id, int(B), int(H_q), int(H_kv), int(max_S), int(top_k)))
     return int(_workspace(torch.device(device), need, "fused").numel())
 
@@ -462,9 +466,9 @@ def _softmax_v(scores, m, iz, v_data, v_scales, block_table, seq_lens, topk_idx,
         o_hat, o_old, W = outs
         for t in outs:
             _check(t.is_cuda and t.dtype == torch.float32 and t.is_contiguous(), "output buffers must be contiguous fp32")
-    if (not int8_tiles and m is None and nbits in (2, 4) and (nbits == 2 or ng == 1) and vd.size(0) == H_kv
+    if (not int8_tiles and m is None and nbits in (2, 3, 4) and (nbits != 4 or ng == 1) and vd.size(0) == H_kv
             and _fast_shape(H_q, H_kv, block_size, max_S, vd.size(1), top_k if topk_idx is not None else None)):
-        fmt = 32 if nbits == 2 else 44
+        fmt = {2: 32, 3: 33, 4: 44}[nbits]
         k_eff = int(top_k) if topk_idx is not None else 32
         ws = _workspace(dev, lib.jf_fused_workspace_bytes(fmt, B, H_q, H_kv, int(max_S), k_eff), "fused")
         _lib.check(lib.jf_stage_b_softmax_v(
@@ -581,11 +585,11 @@ def fused_attn_topk(scheme: str, q, k_data, k_scales, v_data, v_scales, block_ta
 
     The single-call contract is the one of the reference's int2_fused_attn_topk
     (jetfire_vllm/kernels/int2_fused_attn_topk.py:5-10) extended to INT3 / INT4 keys (INT4: the int8-Q scoring
-    model) and symmetric INT2 keys with INT2 / INT4 values: "k3v2", "k2v2" (group 64 or 128), "k4v4", "k3v4", "k4v2",
-    "k2v4" (group 128)."""
+    model), symmetric INT2 keys, and INT2 / INT3 / INT4 values: "k{2,3,4}v{2,3,4}"; pairs without an INT4 side take
+    group 64 or 128, the others group 128."""
     lib = _lib.load()
-    scheme_id = {"k3v2": 32, "k4v4": 44, "k3v4": 34, "k4v2": 42, "k2v2": 22, "k2v4": 24}.get(scheme)
-    _check(scheme_id is not None, f"unknown scheme {scheme!r} (k3v2, k4v4, k3v4, k4v2, k2v2, k2v4)")
+    scheme_id = FUSED_SCHEMES.get(scheme)
+    _check(scheme_id is not None, f"unknown scheme {scheme!r} ({', '.join(sorted(FUSED_SCHEMES))})")
     kp, vp = 16 * (scheme_id // 10), 16 * (scheme_id % 10)
     q, kd, ks, bt, sl = _stage_a_args(q, k_data, k_scales, block_table, seq_lens, H_q, H_kv, kp)
     _gpu(v_data, v_scales)

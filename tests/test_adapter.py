@@ -169,7 +169,8 @@ def test_pool_registry_and_store_geometry(adapter):
 @pytest.mark.gpu
 @pytest.mark.parametrize("scheme_name,scheme,gs,kb,vb", [
     ("SymInt3K_SymInt2V", "k3v2", 64, 3, 2), ("SymInt4K_SymInt4V", "k4v4", 128, 4, 4),      # fused kernels
-    # the pairs without a fused kernel run Stage A and Stage B as separate kernels chosen by bit width
+    # the other pairs: fused where the group size allows (an INT4 side needs group 128), else Stage A and Stage B as
+    # separate kernels chosen by bit width
     ("SymInt2K_SymInt2V", "k2v2", 128, 2, 2), ("SymInt2K_SymInt3V", "k2v3", 128, 2, 3), ("SymInt2K_SymInt4V", "k2v4", 128, 2, 4),
     ("SymInt3K_SymInt3V", "k3v3", 64, 3, 3), ("SymInt3K_SymInt4V", "k3v4", 128, 3, 4),
     ("SymInt4K_SymInt2V", "k4v2", 128, 4, 2), ("SymInt4K_SymInt3V", "k4v3", 64, 4, 3),

@@ -86,13 +86,23 @@ CASES = [
     ("k2v2", 3, 32, 4, 512, [17, 257, 512], 256), ("k2v4", 3, 32, 4, 512, [17, 257, 512], 256),
     ("k2v2", 4, 8, 2, 32, [0, 1, 9, 17], 32), ("k2v2", 1, 8, 2, 5000, [4987], 256), ("k2v4", 1, 8, 2, 5000, [4987], 512),
     ("k2v2", 1, 4, 4, 300, None, 32), ("k2v4", 1, 4, 2, 300, None, 64), ("k2v2", 1, 16, 1, 600, None, 64),
+    # planar INT3 values with every key format
+    ("k3v3", 2, 8, 2, 512, None, 64), ("k3v3_g128", 2, 8, 2, 700, None, 128), ("k2v3", 2, 8, 2, 512, None, 64),
+    ("k2v3_g128", 2, 8, 2, 700, None, 128), ("k4v3", 2, 8, 2, 512, None, 64),
+    ("k3v3", 3, 32, 4, 512, [17, 257, 512], 256), ("k4v3", 3, 32, 4, 512, [17, 257, 512], 256),
+    ("k2v3", 3, 32, 4, 512, [17, 257, 512], 256),
+    ("k3v3", 4, 8, 2, 32, [0, 1, 9, 17], 32), ("k4v3", 4, 8, 2, 32, [0, 1, 9, 17], 64),
+    ("k3v3", 1, 8, 2, 5000, [4987], 256), ("k4v3", 1, 8, 2, 5000, [4987], 512), ("k2v3", 1, 8, 2, 5000, [4987], 1024),
+    ("k3v3", 1, 4, 4, 300, None, 32), ("k4v3", 1, 4, 2, 300, None, 64), ("k3v3_g128", 1, 16, 1, 600, None, 64),
+    ("k2v3", 1, 16, 1, 600, None, 64),
 ]
+SCHEME_GEOMETRY = {f"k{kb}v{vb}": (kb, vb, 128 if 4 in (kb, vb) else 64) for kb in (2, 3, 4) for vb in (2, 3, 4)}
+SCHEME_GEOMETRY.update({f"k{kb}v{vb}_g128": (kb, vb, 128) for kb in (2, 3) for vb in (2, 3)})
 
 
 @pytest.mark.parametrize("scheme,B,Hq,Hkv,S,lens,K", CASES)
 def test_fused_scan_matches_oracle(scheme, B, Hq, Hkv, S, lens, K):
-    kb, vb, gs = {"k3v2": (3, 2, 64), "k4v4": (4, 4, 128), "k3v2_g128": (3, 2, 128), "k3v4": (3, 4, 128),
-                  "k4v2": (4, 2, 128), "k2v2": (2, 2, 64), "k2v2_g128": (2, 2, 128), "k2v4": (2, 4, 128)}[scheme]
+    kb, vb, gs = SCHEME_GEOMETRY[scheme]
     c = make_case(70 + S + Hq, B, Hq, Hkv, S, kb, vb, gs, lens=lens, extra_blocks=3)
     d = to_device(c)
     out = run_fused(scheme, c, d, S, K)

@@ -1,5 +1,5 @@
 """Seeded sweep of the fused scan over randomly drawn geometries (GQA group, batch, ragged lengths, correction
-width, forced split lengths, block-table permutations) for the four fused schemes, each case checked against
+width, forced split lengths, block-table permutations) for the fused schemes, each case checked against
 the oracle exactly as the hand-picked cases are."""
 import numpy as np
 import pytest
@@ -10,7 +10,8 @@ from tests.test_gpu_fused import check_against_oracle, run_fused
 pytestmark = pytest.mark.gpu
 
 SCHEMES = {"k3v2": (3, 2, 64), "k3v2_g128": (3, 2, 128), "k4v4": (4, 4, 128), "k3v4": (3, 4, 128), "k4v2": (4, 2, 128),
-           "k2v2": (2, 2, 64), "k2v2_g128": (2, 2, 128), "k2v4": (2, 4, 128)}
+           "k2v2": (2, 2, 64), "k2v2_g128": (2, 2, 128), "k2v4": (2, 4, 128),
+           "k3v3": (3, 3, 64), "k3v3_g128": (3, 3, 128), "k2v3": (2, 3, 64), "k4v3": (4, 3, 128)}
 
 
 def _draw(seed):
@@ -27,7 +28,7 @@ def _draw(seed):
     return scheme, B, G * Hkv, Hkv, S, lens, K, split
 
 
-@pytest.mark.parametrize("seed", range(80))
+@pytest.mark.parametrize("seed", range(96))
 def test_fused_scan_random_geometry(seed):
     from jetfire_amd import _lib
     scheme, B, Hq, Hkv, S, lens, K, split = _draw(seed)
@@ -52,8 +53,8 @@ def test_two_call_form_random_geometry(seed):
     import torch
     from jetfire_amd import _lib, ops
     scheme, B, Hq, Hkv, S, lens, K, split = _draw(seed)
-    if scheme in ("k3v4", "k4v2", "k2v2", "k2v2_g128", "k2v4"):
-        scheme = "k3v2" if seed % 4 == 0 else "k4v4"        # the two operator pairs below are those of K3V2 and K4V4
+    if scheme not in ("k3v2", "k3v2_g128", "k4v4", "k3v3", "k3v3_g128"):   # the operator pairs below: K3V2, K3V3, K4V4
+        scheme = "k3v2" if seed % 4 == 0 else "k4v4"
     if scheme == "k4v4" and K < 64:
         K = 64                                              # int8tc_qk_scores_topk_stats starts at 64
     kb, vb, gs = SCHEMES[scheme]
@@ -68,7 +69,7 @@ def test_two_call_form_random_geometry(seed):
         args = (d["q"], d["kd"], d["ks"], d["bt"], d["lens"], S, Hq, Hkv, 16, 128 ** -0.5, K)
         if kb == 3:
             sc2, idx2, slots2 = ops.int3_qk_scores_topk(*args)
-            stage_b = ops.int2_softmax_v_with_pre_corr_wvs2
+            stage_b = ops.int2_softmax_v_with_pre_corr_wvs2 if vb == 2 else ops.int3_softmax_v_with_pre_corr_wvs2
         else:
             sc2, idx2, slots2, m2, iz2 = ops.int8tc_qk_scores_topk_stats(*args)
             assert torch.equal(m2, m) and torch.equal(iz2, iz)
