@@ -29,7 +29,7 @@ from .config import get_jetfire_config
 from .kv_pool import get_global_kv_pool_manager
 
 # correction widths the fused kernels take; the split entry points go up to 8192
-FUSED_SUPPORTED_TOP_K = (32, 64, 128, 256, 512, 1024)
+FUSED_SUPPORTED_TOP_K = (32, 64, 128, 256, 512, 1024, 2048)
 SPLIT_SUPPORTED_TOP_K = ops.SUPPORTED_TOP_K
 
 _TOPK_CLAMP_LOGGED: set = set()
@@ -226,13 +226,14 @@ def warmup_graph_decode_submit_contexts(*, max_batch_size: int, device=None, sca
         layer_cfg = pool.get_layer_config(name)
         if layer_cfg is None or not store.shadow_enabled:
             continue
-        supported = FUSED_SUPPORTED_TOP_K if store.scheme is not None else SPLIT_SUPPORTED_TOP_K
+        supported = SPLIT_SUPPORTED_TOP_K       # (widths beyond the fused form's run the stage-wise kernels)
         top_k = _select_top_k(cfg.topk, cfg.topk, supported)
         if top_k is None:
             raise RuntimeError(f"JETFIRE_TOPK={cfg.topk} is not supported by the active kernel set.")
         widths = tuple(k for k in supported if k <= top_k) or (top_k,)
         store.warmup_graph_append(int(max_batch_size))
-        if max_seq_len and store.scheme is not None and store.device.type == "cuda":
+        if (max_seq_len and store.scheme is not None and top_k in FUSED_SUPPORTED_TOP_K
+                and store.device.type == "cuda"):
             # the scan's workspace of this stream, sized for the largest step, so that no capture has to grow it
             ops.reserve_fused_workspace(store.scheme, int(max_batch_size), layer_cfg.num_query_heads,
                                         layer_cfg.num_kv_heads, int(max_seq_len), top_k, store.device)
@@ -357,10 +358,12 @@ def _decode_batched(*, impl, layer, query, attn_metadata, output):
     release = release_policy.release_policy_enabled() and not store.k_asymmetric
     if release:
         release_policy.validate_release_environment()
-    fused = (not release and store.scheme is not None and os.environ.get("JETFIRE_USE_FUSED_ATTN_TOPK", "1") == "1")
-    top_k = _select_top_k(pool.config.topk, max_S, FUSED_SUPPORTED_TOP_K if fused else SPLIT_SUPPORTED_TOP_K)
+    top_k = _select_top_k(pool.config.topk, max_S, SPLIT_SUPPORTED_TOP_K)
     if top_k is None:
         return miss("seq_len_too_short")
+    # the fused scan where it covers the scheme and the width; wider corrections run the stage-wise kernels
+    fused = (not release and store.scheme is not None and top_k in FUSED_SUPPORTED_TOP_K
+             and os.environ.get("JETFIRE_USE_FUSED_ATTN_TOPK", "1") == "1")
     plan = None
     if release:
         plan = release_policy.plan_release_graph(

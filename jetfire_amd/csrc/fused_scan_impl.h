@@ -84,7 +84,7 @@ typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
 //               merge is the FS_STAGE_A one)
 constexpr int FS_FULL = 0, FS_STAGE_A = 1, FS_STAGE_B = 2, FS_TOPK = 3;
 
-constexpr int FS_MAX_TOPK = 1024;      // winners cached in LDS by the merge kernel
+constexpr int FS_MAX_TOPK = 2048;      // winners cached in LDS by the merge kernel
 constexpr int FS_CAND_SLACK = 256;     // extra candidate slots per (row, split): room for the whole cut bucket
 
 struct FusedParams {
@@ -1396,10 +1396,10 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   __shared__ float coef_sh[MG_MAX_SPLITS];
   __shared__ int cnt_sh[MG_MAX_SPLITS];
   __shared__ int bt_sh[MG_BT_LDS];
+  // winners: key and position while they are selected; the thread that turns winner r into its softmax weight and
+  // paged slot overwrites the two entries in place (weight bits over the key, slot over the position)
   __shared__ uint32_t win_key[FS_MAX_TOPK];
   __shared__ int win_idx[FS_MAX_TOPK];
-  __shared__ int win_slot[FS_MAX_TOPK];
-  __shared__ float win_w[FS_MAX_TOPK];
   __shared__ uint32_t cnt_a[MG_REGK / 4 * MG_WAVES];  // packed (winners, ties) per (group, wavefront)
   __shared__ float red_sh[MG_THREADS / D][D];
   __shared__ float old_sh[MG_WAVES][D];
@@ -1818,8 +1818,8 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
       out_idx[r] = position;
       out_slot[r] = slot;
     }
-    win_slot[r] = wslot;
-    win_w[r] = ww;
+    win_idx[r] = wslot;
+    win_key[r] = __builtin_bit_cast(uint32_t, ww);
   }
   if constexpr (MODE == FS_STAGE_A) return;  // Stage A alone ends with the winners and the statistics
   lds_barrier();
@@ -1844,8 +1844,8 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
 #pragma unroll
     for (int u = 0; u < UNR; ++u) {
       const int k = k0 + u * MG_WAVES * WPI + w_in;
-      const int slot = (k < n_out) ? win_slot[k] : -1;
-      wv[u] = (slot >= 0) ? win_w[k] : 0.f;
+      const int slot = (k < n_out) ? win_idx[k] : -1;
+      wv[u] = (slot >= 0) ? __builtin_bit_cast(float, win_key[k]) : 0.f;
       const uint32_t sl = (uint32_t)max(slot, 0);
       if constexpr (VBITS == 3) {  // bytes 2*dwi, 2*dwi+1 of every plane -> the 24-bit words of two 8-code groups
         const uint8_t* row = vbase + (size_t)(sl * (uint32_t)VP) + dwi * 2;
@@ -2156,7 +2156,7 @@ static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_
   const bool scores_only = (MODE == FS_STAGE_A) && top_k == 0;
   if (scores_only) top_k = 32;  // (any valid width: the plan depends on it, the kernel stops before using it)
   JF_CHECK_ARG(is_pow2(top_k) && top_k >= 32 && top_k <= FS_MAX_TOPK,
-               "fused_scan: unsupported top_k=%d (supported: 32,64,128,256,512,1024; larger widths use the split-form operators)", top_k);
+               "fused_scan: unsupported top_k=%d (supported: 32,64,128,256,512,1024,2048; larger widths use the split-form operators)", top_k);
   JF_CHECK_ARG(max_S <= 262144, "fused_scan: max_S=%d exceeds supported limit (262144)", max_S);
   JF_CHECK_ARG((int64_t)max_blocks * block_size >= max_S, "fused_scan: block_table does not cover max_S");
   JF_CHECK_ARG(num_slots > 0 && num_slots <= (1ll << 25), "fused_scan: num_slots out of range (at most 2^25: row offsets are 32-bit)");

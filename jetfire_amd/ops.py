@@ -16,6 +16,7 @@ from . import _lib
 
 HEAD_DIM = 128
 SUPPORTED_TOP_K = (32, 64, 128, 256, 512, 1024, 2048, 4096, 8192)
+FUSED_TOP_K = (32, 64, 128, 256, 512, 1024, 2048)      # widths of the one-pass form and of the fast stage-wise forms
 
 _workspaces: dict = {}
 _retired_workspaces: list = []   # superseded buffers, kept because captured graphs may still point at them
@@ -226,7 +227,7 @@ def get_split_impl() -> str:
 def _fast_shape(H_q, H_kv, block_size, max_S, num_slots, top_k=None) -> bool:
     return (_split_impl == "fast" and H_kv > 0 and H_q % H_kv == 0 and H_q // H_kv in (1, 2, 4, 8, 16)
             and int(block_size) == 16 and 0 < int(max_S) <= 262144 and 0 < int(num_slots) <= (1 << 25)
-            and (top_k is None or int(top_k) in (32, 64, 128, 256, 512, 1024)))
+            and (top_k is None or int(top_k) in FUSED_TOP_K))
 
 
 def _stage_a_fast(fmt: int, q, kd, ks, bt, sl, max_S, H_q, H_kv, attn_scale, top_k, stats: bool):
@@ -382,7 +383,7 @@ def _topk(scores, block_table, seq_lens, max_S, H_q, block_size, top_k, stats: b
     if stats:
         m = torch.empty((B, H_q), dtype=torch.float32, device=scores.device)
         iz = torch.empty((B, H_q), dtype=torch.float32, device=scores.device)
-    if _split_impl == "fast" and int(top_k) <= 1024 and int(block_size) == 16 and max_S > 0 and B > 0:
+    if _split_impl == "fast" and int(top_k) <= FUSED_TOP_K[-1] and int(block_size) == 16 and max_S > 0 and B > 0:
         sc = scores.contiguous()
         ws = _workspace(scores.device, lib.jf_topk_slots_fast_workspace_bytes(B, H_q, int(max_S), int(top_k)), "fused")
         _lib.check(lib.jf_topk_slots_fast(sc.data_ptr(), sl.data_ptr(), bt.data_ptr(), B, H_q, int(max_S), bt.size(1), 16,

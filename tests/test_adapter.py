@@ -28,7 +28,7 @@ def test_select_top_k_matches_the_reference_table(adapter):
     for req in (16, 32, 100, 256, 300, 1024, 5000):
         for n in (0, 1, 31, 32, 33, 255, 256, 257, 4096):
             assert _select_top_k(req, n, supported) == O.select_top_k(req, n, supported), (req, n)
-    assert FUSED_SUPPORTED_TOP_K == supported
+    assert FUSED_SUPPORTED_TOP_K == supported + (2048,)
     hm = _get_head_map_cpu(2, 8, 4, 5).numpy()
     assert np.array_equal(hm, O.head_map(2, 8, 4, 5))
 

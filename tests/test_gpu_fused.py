@@ -95,6 +95,9 @@ CASES = [
     ("k3v3", 1, 8, 2, 5000, [4987], 256), ("k4v3", 1, 8, 2, 5000, [4987], 512), ("k2v3", 1, 8, 2, 5000, [4987], 1024),
     ("k3v3", 1, 4, 4, 300, None, 32), ("k4v3", 1, 4, 2, 300, None, 64), ("k3v3_g128", 1, 16, 1, 600, None, 64),
     ("k2v3", 1, 16, 1, 600, None, 64),
+    # the widest correction of the fused form
+    ("k3v2", 1, 8, 2, 5000, [4987], 2048), ("k4v4", 2, 8, 2, 3000, [1000, 3000], 2048),
+    ("k3v3", 1, 32, 4, 6000, None, 2048), ("k2v4", 2, 4, 4, 2048, [2048, 2047], 2048),
 ]
 SCHEME_GEOMETRY = {f"k{kb}v{vb}": (kb, vb, 128 if 4 in (kb, vb) else 64) for kb in (2, 3, 4) for vb in (2, 3, 4)}
 SCHEME_GEOMETRY.update({f"k{kb}v{vb}_g128": (kb, vb, 128) for kb in (2, 3) for vb in (2, 3)})
@@ -116,6 +119,8 @@ def test_fused_scan_matches_oracle(scheme, B, Hq, Hkv, S, lens, K):
     ("k4v4", 10000, [10000], 1024, 1280),  # widest top-k: parts limited to 8192 / top_k
     ("k3v2", 3000, [3000], 64, 1024),      # longer than the planner would pick for this size
     ("k3v4", 10000, [9989], 256, 512), ("k4v2", 10000, [9000], 512, 768),      # two-stage merges of the mixed pairs
+    ("k3v2", 20000, [19989], 2048, 512),   # every position a candidate, 40 lists: two-stage merge at the widest correction
+    ("k4v4", 40000, [39000], 2048, 0),     # the planner's own split: lists of 2304 entries, first stage beyond the registers
 ])
 def test_fused_scan_with_forced_split_length(scheme, S, lens, K, split_len):
     from jetfire_amd import _lib
