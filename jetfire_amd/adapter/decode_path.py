@@ -363,7 +363,7 @@ def _decode_batched(*, impl, layer, query, attn_metadata, output):
         return miss("seq_len_too_short")
     # the fused scan where it covers the scheme and the width; wider corrections run the stage-wise kernels
     fused = (not release and store.scheme is not None and top_k in FUSED_SUPPORTED_TOP_K
-             and os.environ.get("JETFIRE_USE_FUSED_ATTN_TOPK", "1") == "1")
+             and int(store.k_data.shape[1]) <= ops.FUSED_MAX_SLOTS and os.environ.get("JETFIRE_USE_FUSED_ATTN_TOPK", "1") == "1")
     plan = None
     if release:
         plan = release_policy.plan_release_graph(

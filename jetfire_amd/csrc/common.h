@@ -117,7 +117,7 @@ __device__ inline int wave_incl_scan_i(int v) {
 inline bool is_pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
 
 // Pre-correction terms of INT4 values (one scale per row) over given winners with given softmax statistics, on the
-// merge kernel of the fused step (fused_stage_b.hip); top_k <= 1024, num_slots <= 2^25.
+// merge kernel of the fused step (fused_stage_b.hip); top_k <= 2048, num_slots <= 2^26.
 int precorr_int4_given_stats(const float* scores, const float* softmax_m, const float* softmax_inv_z,
                              const uint8_t* v_data, const uint16_t* v_scales, const int64_t* block_table,
                              const int32_t* seq_lens, const int64_t* topk_idx, int B, int H_q, int H_kv, int max_S,

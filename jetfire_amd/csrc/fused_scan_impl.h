@@ -85,6 +85,7 @@ typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
 constexpr int FS_FULL = 0, FS_STAGE_A = 1, FS_STAGE_B = 2, FS_TOPK = 3;
 
 constexpr int FS_MAX_TOPK = 2048;      // winners cached in LDS by the merge kernel
+constexpr long long FS_MAX_SLOTS = 1ll << 26;  // slots per kv-head tensor: 64-byte rows, 32-bit row offsets (4 GB)
 constexpr int FS_CAND_SLACK = 256;     // extra candidate slots per (row, split): room for the whole cut bucket
 
 struct FusedParams {
@@ -2159,7 +2160,8 @@ static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_
                "fused_scan: unsupported top_k=%d (supported: 32,64,128,256,512,1024,2048; larger widths use the split-form operators)", top_k);
   JF_CHECK_ARG(max_S <= 262144, "fused_scan: max_S=%d exceeds supported limit (262144)", max_S);
   JF_CHECK_ARG((int64_t)max_blocks * block_size >= max_S, "fused_scan: block_table does not cover max_S");
-  JF_CHECK_ARG(num_slots > 0 && num_slots <= (1ll << 25), "fused_scan: num_slots out of range (at most 2^25: row offsets are 32-bit)");
+  // (a row's byte offset inside one kv-head's tensor is formed in 32 bits: rows of at most 64 bytes)
+  JF_CHECK_ARG(num_slots > 0 && num_slots <= FS_MAX_SLOTS, "fused_scan: num_slots out of range (at most 2^26: row offsets are 32-bit)");
   JF_CHECK_ARG((softmax_m == nullptr) == (softmax_inv_z == nullptr), "fused_scan: softmax_m and softmax_inv_z go together");
   if (B == 0) return JF_OK;
   JF_CHECK_ARG(block_table && seq_lens, "fused_scan: null input");

@@ -405,7 +405,7 @@ extern "C" int jf_softmax_v_int8_tiles(const float* scores, const float* softmax
   JF_CHECK_LAUNCH();
   // the pre-correction terms run on the merge kernel of the fused step where its limits allow (the same
   // formula, p_j = exp(score_j - m) * inv_z with the caller's statistics), else in the combine kernel
-  const bool fast_precorr = topk_idx != nullptr && top_k <= 2048 && num_slots <= (1ll << 25) && ((uintptr_t)v_data & 3) == 0;
+  const bool fast_precorr = topk_idx != nullptr && top_k <= 2048 && num_slots <= (1ll << 26) && ((uintptr_t)v_data & 3) == 0;
   hipLaunchKernelGGL((combine_precorr_kernel<4, 1>), dim3(B, H_q), block, 0, st, partial, scores, softmax_m, softmax_inv_z,
                      v_data, v_scales, block_table, seq_lens, fast_precorr ? nullptr : topk_idx, o_hat, o_old_unnorm, W, H_q,
                      H_kv, max_S, max_blocks, num_slots, TQ_SPLITS * sub_count, top_k);

@@ -17,6 +17,7 @@ from . import _lib
 HEAD_DIM = 128
 SUPPORTED_TOP_K = (32, 64, 128, 256, 512, 1024, 2048, 4096, 8192)
 FUSED_TOP_K = (32, 64, 128, 256, 512, 1024, 2048)      # widths of the one-pass form and of the fast stage-wise forms
+FUSED_MAX_SLOTS = 1 << 26                               # slots per kv-head tensor those forms address (4 GB of 64-byte rows)
 
 _workspaces: dict = {}
 _retired_workspaces: list = []   # superseded buffers, kept because captured graphs may still point at them
@@ -226,7 +227,7 @@ def get_split_impl() -> str:
 
 def _fast_shape(H_q, H_kv, block_size, max_S, num_slots, top_k=None) -> bool:
     return (_split_impl == "fast" and H_kv > 0 and H_q % H_kv == 0 and H_q // H_kv in (1, 2, 4, 8, 16)
-            and int(block_size) == 16 and 0 < int(max_S) <= 262144 and 0 < int(num_slots) <= (1 << 25)
+            and int(block_size) == 16 and 0 < int(max_S) <= 262144 and 0 < int(num_slots) <= FUSED_MAX_SLOTS
             and (top_k is None or int(top_k) in FUSED_TOP_K))
 
 

@@ -278,6 +278,46 @@ def test_fused_step_replays_from_a_hip_graph():
             assert torch.equal(got, want)
 
 
+@pytest.mark.parametrize("scheme,kb,vb,gs", [("k4v4", 4, 4, 128), ("k3v2", 3, 2, 64)])
+def test_fused_scan_addresses_the_top_of_a_4gb_pool(scheme, kb, vb, gs):
+    """The largest pool the fused form addresses: 2^26 slots per kv-head (4 GB of 64-byte rows).  A small case whose
+    pages sit in the last blocks of such a pool gives the outputs of the same case in a small pool, bit for bit,
+    with the slots shifted; one slot more is rejected."""
+    o = ops()
+    S, K, Hq, Hkv = 700, 64, 4, 1
+    c = make_case(77, 2, Hq, Hkv, S, kb, vb, gs, extra_blocks=2)
+    d = to_device(c)
+    small = o.fused_attn_topk(scheme, d["q"], d["kd"], d["ks"], d["vd"], d["vs"], d["bt"], d["lens"], S, Hq, Hkv, 16, K,
+                              SCALE, return_scores=True, return_stats=True)
+    n_small = d["kd"].size(1)
+    n_big = 1 << 26
+    shift = n_big - n_small                                   # (a multiple of 16: whole blocks)
+    big = {}
+    for name in ("kd", "ks", "vd", "vs"):
+        t = torch.zeros((Hkv, n_big) + tuple(d[name].shape[2:]), dtype=d[name].dtype, device="cuda")
+        t[:, shift:] = d[name]
+        big[name] = t
+    bt_big = d["bt"] + shift // 16
+    out = o.fused_attn_topk(scheme, d["q"], big["kd"], big["ks"], big["vd"], big["vs"], bt_big, d["lens"], S, Hq, Hkv, 16,
+                            K, SCALE, return_scores=True, return_stats=True)
+    for i, (a, b) in enumerate(zip(out, small)):
+        if i == 1:                                            # topk_slots
+            assert torch.equal(a, torch.where(b >= 0, b + shift, b))
+        else:
+            assert torch.equal(a, b)
+    # one block more is refused before anything is launched (the argument check alone sees the slot count)
+    from jetfire_amd import _lib
+    lib = _lib.load()
+    idx, slots, o_hat, o_old, W = out[4], out[1], out[0], out[2], out[3]
+    ws = torch.empty(lib.jf_fused_workspace_bytes(10 * kb + vb, 2, Hq, Hkv, S, K), dtype=torch.uint8, device="cuda")
+    rc = lib.jf_fused_scan_topk(10 * kb + vb, gs, d["q"].data_ptr(), big["kd"].data_ptr(), big["ks"].data_ptr(),
+                                big["vd"].data_ptr(), big["vs"].data_ptr(), bt_big.data_ptr(), d["lens"].data_ptr(), 2, Hq,
+                                Hkv, S, bt_big.size(1), n_big + 16, 16, SCALE, K, idx.data_ptr(), slots.data_ptr(),
+                                o_hat.data_ptr(), o_old.data_ptr(), W.data_ptr(), None, None, None, ws.data_ptr(),
+                                ws.numel(), None)
+    assert rc != 0 and "num_slots" in lib.jf_last_error().decode()
+
+
 def test_fused_scan_rejects_unsupported_arguments():
     c = make_case(9, 1, 8, 2, 64, 3, 2, 64)
     d = to_device(c)
