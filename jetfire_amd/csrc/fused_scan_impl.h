@@ -1361,6 +1361,7 @@ constexpr int MG_MAX_SPLITS = 256;
 constexpr int MG_BINS = 1024;      // linear score buckets of the threshold search
 constexpr int MG_LIST = 1024;      // members of the cut bucket resolved by rank counting
 constexpr int MG_BT_LDS = 4096;    // block-table entries cached in LDS (65536 positions)
+constexpr int MG_LIGHT_THREADS = 256, MG_LIGHT_REGK = 16, MG_LIGHT_TOPK = 512;  // the light shape of the merge
 
 // Launch 2: one workgroup per (sequence, query head).
 //   1. split statistics -> M, l, o_hat
@@ -1392,19 +1393,28 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   constexpr int DW = (VBITS == 3) ? 8 : VP / 4;
   constexpr int CPD = (VBITS == 3) ? 16 : 32 / VBITS;
   constexpr int WPI = 64 / DW;          // winners per wavefront instruction
+  // The floating-point sums (o_hat over the splits, the pre-correction terms over the winners) are organised
+  // as if eight thread groups of 128 and sixteen wavefronts were at work, whatever MG_THREADS is: a smaller
+  // workgroup takes several of those roles one after the other, so every shape of this kernel adds the same
+  // numbers in the same order and the results do not depend on which shape the launcher picks.
+  constexpr int VGRP = 8, VWAVES = 16;
+  static_assert(MG_THREADS % D == 0 && VGRP % (MG_THREADS / D) == 0 && VWAVES % MG_WAVES == 0, "whole roles per thread group / wavefront");
+  // the light shape (many rows per launch, few candidates per row) trades table sizes for workgroups per CU
+  constexpr int MG_BT = (MG_THREADS >= 1024) ? MG_BT_LDS : 1024;  // block-table entries cached in LDS
+  constexpr int MG_WIN = (MG_THREADS >= 1024) ? FS_MAX_TOPK : 512;  // widest correction of this shape
   __shared__ int hist[MG_BINS];
   __shared__ uint32_t lkey[MG_LIST];
   __shared__ float coef_sh[MG_MAX_SPLITS];
   __shared__ int cnt_sh[MG_MAX_SPLITS];
-  __shared__ int bt_sh[MG_BT_LDS];
+  __shared__ int bt_sh[MG_BT];
   // winners: key and position while they are selected; the thread that turns winner r into its softmax weight and
   // paged slot overwrites the two entries in place (weight bits over the key, slot over the position)
-  __shared__ uint32_t win_key[FS_MAX_TOPK];
-  __shared__ int win_idx[FS_MAX_TOPK];
+  __shared__ uint32_t win_key[MG_WIN];
+  __shared__ int win_idx[MG_WIN];
   __shared__ uint32_t cnt_a[MG_REGK / 4 * MG_WAVES];  // packed (winners, ties) per (group, wavefront)
-  __shared__ float red_sh[MG_THREADS / D][D];
-  __shared__ float old_sh[MG_WAVES][D];
-  __shared__ float w_sh[MG_WAVES];
+  __shared__ float red_sh[VGRP][D];
+  __shared__ float old_sh[VWAVES][D];
+  __shared__ float w_sh[VWAVES];
   __shared__ float wred_f[MG_WAVES];
   __shared__ uint32_t wred_u[MG_WAVES], wred_k[MG_WAVES];
   __shared__ float wred_g[MG_WAVES];
@@ -1432,7 +1442,7 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   int64_t* out_slot = p.topk_slots + bh * (size_t)K;
   const int flat = NL * Kc;
   const int rounds = (flat + MG_THREADS - 1) / MG_THREADS;
-  const int nblk_lds = min(p.max_blocks, MG_BT_LDS);
+  const int nblk_lds = min(p.max_blocks, MG_BT);
 
   long long* mclk = (p.phase_clock && !PARTIAL) ? p.phase_clock + (size_t)p.B * p.H_kv * p.n_splits * 10 + bh * 8 : nullptr;
   if (mclk && tid == 0) mclk[0] = clock64();
@@ -1479,7 +1489,7 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
     const int d = tid & (D - 1), q4 = tid >> 7;
 #pragma unroll
     for (int i = 0; i < PO_PRE; ++i) {
-      const int sp = q4 + PO_GRP * i;
+      const int sp = q4 + VGRP * i;
       po[i] = (MODE != FS_STAGE_A && !PARTIAL && sp < NS) ? p.part_o[(bh * NS + sp) * D + d] : 0.f;
     }
   }
@@ -1592,30 +1602,32 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   const int incl = wave_incl_scan_i(mine);
   if (lane == 63) wred_j[wave] = incl;
   if constexpr (!PARTIAL && MODE != FS_STAGE_A) {
-    // o_hat: four thread groups take every fourth split, then a fixed-order sum
+    // o_hat: group vg of the eight takes every eighth split, then a fixed-order sum
     const int d = tid & (D - 1), q4 = tid >> 7;
-    float o = 0.f;
+    for (int vg = q4; vg < VGRP; vg += PO_GRP) {
+      float o = 0.f;
 #pragma unroll
-    for (int i = 0; i < PO_PRE; ++i) {
-      const int sp = q4 + PO_GRP * i;
-      if (sp < NS) o = __builtin_fmaf(po[i], coef_sh[sp], o);
-    }
-    // the remaining splits eight at a time: the loads of a batch are in flight together, the sum keeps its order
-    constexpr int PO_B = 8;
-    for (int sp0 = q4 + PO_GRP * PO_PRE; sp0 < NS; sp0 += PO_GRP * PO_B) {
-      float v[PO_B];
-#pragma unroll
-      for (int u = 0; u < PO_B; ++u) {
-        const int sp = sp0 + PO_GRP * u;
-        v[u] = (sp < NS) ? p.part_o[(bh * NS + sp) * D + d] : 0.f;
+      for (int i = 0; i < PO_PRE; ++i) {
+        const int sp = vg + VGRP * i;
+        if (sp < NS) o = __builtin_fmaf((vg == q4) ? po[i] : p.part_o[(bh * NS + sp) * D + d], coef_sh[sp], o);
       }
+      // the remaining splits eight at a time: the loads of a batch are in flight together, the sum keeps its order
+      constexpr int PO_B = 8;
+      for (int sp0 = vg + VGRP * PO_PRE; sp0 < NS; sp0 += VGRP * PO_B) {
+        float v[PO_B];
 #pragma unroll
-      for (int u = 0; u < PO_B; ++u) {
-        const int sp = sp0 + PO_GRP * u;
-        if (sp < NS) o = __builtin_fmaf(v[u], coef_sh[sp], o);
+        for (int u = 0; u < PO_B; ++u) {
+          const int sp = sp0 + VGRP * u;
+          v[u] = (sp < NS) ? p.part_o[(bh * NS + sp) * D + d] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < PO_B; ++u) {
+          const int sp = sp0 + VGRP * u;
+          if (sp < NS) o = __builtin_fmaf(v[u], coef_sh[sp], o);
+        }
       }
+      red_sh[vg][d] = o;
     }
-    red_sh[q4][d] = o;
   }
   lds_barrier();
   // ---- interval 4: o_hat; the bucket of the K-th largest candidate
@@ -1623,7 +1635,7 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
     if (tid < D) {
       float o2 = red_sh[0][tid];
 #pragma unroll
-      for (int q = 1; q < PO_GRP; ++q) o2 += red_sh[q][tid];  // fixed order
+      for (int q = 1; q < VGRP; ++q) o2 += red_sh[q][tid];  // fixed order
       blend_hat = o2 * inv_z;
       if (MODE != FS_STAGE_B || p.o_hat) p.o_hat[bh * D + tid] = blend_hat;
     }
@@ -1833,18 +1845,19 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   const uint8_t* vsbase = reinterpret_cast<const uint8_t*>(p.v_scales + (size_t)hkv * p.num_slots * NG);
   const int dwi = lane % DW, w_in = lane / DW;
   const int g_of_lane = (NG == 1) ? 0 : ((dwi * CPD) / (D / NG));
+  constexpr int UNR = (256 / (VWAVES * WPI) > 0) ? 256 / (VWAVES * WPI) : 1;  // 256 winners per pass
+  for (int vw = wave; vw < VWAVES; vw += MG_WAVES) {  // (one turn unless the workgroup has fewer than sixteen wavefronts)
   float acc[CPD];
 #pragma unroll
   for (int c = 0; c < CPD; ++c) acc[c] = 0.f;
   float accw = 0.f;
-  constexpr int UNR = (256 / (MG_WAVES * WPI) > 0) ? 256 / (MG_WAVES * WPI) : 1;  // 256 winners per pass
-  for (int k0 = wave * WPI; k0 < n_out; k0 += UNR * MG_WAVES * WPI) {
+  for (int k0 = vw * WPI; k0 < n_out; k0 += UNR * VWAVES * WPI) {
     uint32_t word[UNR], word_b[UNR];  // (word_b: INT3 only)
     uint16_t sbits[UNR];
     float wv[UNR];
 #pragma unroll
     for (int u = 0; u < UNR; ++u) {
-      const int k = k0 + u * MG_WAVES * WPI + w_in;
+      const int k = k0 + u * VWAVES * WPI + w_in;
       const int slot = (k < n_out) ? win_idx[k] : -1;
       wv[u] = (slot >= 0) ? __builtin_bit_cast(float, win_key[k]) : 0.f;
       const uint32_t sl = (uint32_t)max(slot, 0);
@@ -1911,20 +1924,21 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
       halve(std::integral_constant<int, 32>{}, std::integral_constant<int, CPD / 2>{});
     }
     static_assert(CPD / WPI == 2, "two channels per lane after the exchange");
-    old_sh[wave][chan] = acc[0];
-    old_sh[wave][chan + 1] = acc[1];
+    old_sh[vw][chan] = acc[0];
+    old_sh[vw][chan + 1] = acc[1];
     const float wsum = wave_sum(accw);  // only the dwi == 0 lanes hold weights
-    if (lane == 0) w_sh[wave] = wsum;
+    if (lane == 0) w_sh[vw] = wsum;
+  }
   }
   lds_barrier();
   if (tid < D) {
     float o = 0.f;
 #pragma unroll
-    for (int w = 0; w < MG_WAVES; ++w) o += old_sh[w][tid];  // fixed order
+    for (int w = 0; w < VWAVES; ++w) o += old_sh[w][tid];  // fixed order
     p.o_old[bh * D + tid] = o;
     float wt = 0.f;
 #pragma unroll
-    for (int w = 0; w < MG_WAVES; ++w) wt += w_sh[w];  // fixed order: the same value in every thread
+    for (int w = 0; w < VWAVES; ++w) wt += w_sh[w];  // fixed order: the same value in every thread
     if (tid == 0) p.W[bh] = wt;
     // the blend of jetfire_vllm/csrc/blend.cu:202-226 for callers that hold o_new already
     if (MODE == FS_FULL && p.blend_out) p.blend_out[bh * D + tid] = f32_to_bf16(__builtin_fmaf(wt, blend_new, blend_hat) - o);
@@ -2255,10 +2269,19 @@ static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_
   }
   const bool big = (MODE != FS_STAGE_B) &&
                    (p.mg_parts > 1 ? (long long)p.mg_parts * top_k : (long long)p.n_splits * p.Kc) > MG_REG_CANDS;
+  // Many rows with few candidates each (large batches of short or medium sequences): four wavefronts per row and
+  // small tables, so that five rows share a CU instead of one (measured from 257 rows up: 42.5 against 47.5 us per
+  // layer at 384 rows of 2048 candidates, 38 against 57 at 1024 rows of 512).  Same results (see VGRP / VWAVES in
+  // the kernel).
+  const bool light = (MODE == FS_FULL) && !big && p.mg_parts == 1 && top_k <= MG_LIGHT_TOPK &&
+                     (long long)B * H_q > (long long)device_cus() && (long long)p.n_splits * p.Kc <= MG_LIGHT_THREADS * MG_LIGHT_REGK;
 #define JF_MERGE(VB, NGG)                                                                                            \
   do {                                                                                                               \
     if (big) hipLaunchKernelGGL((fused_merge_kernel<MODE, VB, NGG, 1024, 32, false>), mgrid, dim3(1024), 0, st, p); \
-    else hipLaunchKernelGGL((fused_merge_kernel<MODE, VB, NGG, 1024, 8, false>), mgrid, dim3(1024), 0, st, p);       \
+    else if (light) {                                                                                                \
+      if constexpr (MODE == FS_FULL)                                                                                 \
+        hipLaunchKernelGGL((fused_merge_kernel<FS_FULL, VB, NGG, MG_LIGHT_THREADS, MG_LIGHT_REGK, false>), mgrid, dim3(MG_LIGHT_THREADS), 0, st, p); \
+    } else hipLaunchKernelGGL((fused_merge_kernel<MODE, VB, NGG, 1024, 8, false>), mgrid, dim3(1024), 0, st, p);       \
   } while (0)
   if constexpr (MODE == FS_STAGE_A || MODE == FS_TOPK) {  // no value rows are read: one instantiation serves every format
     if (big) hipLaunchKernelGGL((fused_merge_kernel<FS_STAGE_A, 4, 1, 1024, 32, false>), mgrid, dim3(1024), 0, st, p);

@@ -278,6 +278,35 @@ def test_fused_step_replays_from_a_hip_graph():
             assert torch.equal(got, want)
 
 
+@pytest.mark.parametrize("scheme,S,K,split_len", [("k3v2", 300, 64, 256), ("k4v4", 1500, 256, 512), ("k3v3", 700, 512, 256),
+                                                  ("k2v4", 5000, 128, 1024)])
+def test_many_rows_take_the_light_merge_with_identical_results(scheme, S, K, split_len):
+    """More than two rows per CU with few candidates each run the merge with four wavefronts per row; its sums are
+    arranged like the sixteen-wavefront shape's, so a batch gives bit for bit what its halves give alone (those are
+    small enough for the regular shape), and the oracle's values.  (The split length is pinned: the planner's own
+    choice depends on the batch size.)"""
+    from jetfire_amd import _lib
+    lib = _lib.load()
+    kb, vb, gs = SCHEME_GEOMETRY[scheme]
+    B, Hq, Hkv = 20, 32, 8                                    # 640 rows
+    lens = [S - 7 * b for b in range(B)]
+    c = make_case(300 + S, B, Hq, Hkv, S, kb, vb, gs, lens=lens)
+    d = to_device(c)
+    _lib.check(lib.jf_debug_split_len(split_len))
+    try:
+        whole = [t.clone() for t in run_fused(scheme, c, d, S, K)]
+        for lo, hi in ((0, 10), (10, 20)):
+            part = ops().fused_attn_topk(scheme, d["q"][lo:hi].contiguous(), d["kd"], d["ks"], d["vd"], d["vs"],
+                                         d["bt"][lo:hi].contiguous(), d["lens"][lo:hi].contiguous(), S, Hq, Hkv, 16, K,
+                                         SCALE, return_scores=True, return_stats=True)
+            for a, b in zip(whole, part):
+                assert torch.equal(a[lo:hi], b)
+    finally:
+        _lib.check(lib.jf_debug_split_len(0))
+    if S <= 1500:
+        check_against_oracle(scheme, c, S, K, whole)
+
+
 @pytest.mark.parametrize("scheme,kb,vb,gs", [("k4v4", 4, 4, 128), ("k3v2", 3, 2, 64)])
 def test_fused_scan_addresses_the_top_of_a_4gb_pool(scheme, kb, vb, gs):
     """The largest pool the fused form addresses: 2^26 slots per kv-head (4 GB of 64-byte rows).  A small case whose
