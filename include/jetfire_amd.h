@@ -41,6 +41,10 @@ extern "C" {
 #define JF_SCHEME_K2V3 23    /* INT2 keys, INT3 values  (SymInt2K_SymInt3V), group 64 or 128 */
 #define JF_SCHEME_K3V3 33    /* INT3 keys, INT3 values  (SymInt3K_SymInt3V), group 64 or 128 */
 #define JF_SCHEME_K4V3 43    /* INT4 keys, INT3 values  (SymInt4K_SymInt3V), group 128 */
+/* asymmetric INT2 keys (four levels, a zero-point per group: k_zp), key digit 1 */
+#define JF_SCHEME_A2V2 12    /* (AsymInt2K4Level_SymInt2V), group 64 or 128 */
+#define JF_SCHEME_A2V3 13    /* (AsymInt2K4Level_SymInt3V), group 64 or 128 */
+#define JF_SCHEME_A2V4 14    /* (AsymInt2K4Level_SymInt4V), group 128 */
 
 const char* jf_last_error(void);
 const char* jf_version(void);
@@ -222,6 +226,24 @@ int jf_fused_scan_topk_blend(int scheme, int group_size,
                              const uint16_t* o_new, uint16_t* out,
                              void* workspace, size_t workspace_bytes, void* stream);
 
+/* The fused step for the asymmetric INT2 keys (the reference's kernel sets
+ * jetfire_vllm/kernels/_dispatch/int2_asym_k_sym_v.py, int2_asym_k_sym_int3_v.py, int2_asym_k_sym_int4_v.py): scheme
+ * JF_SCHEME_A2V2 / JF_SCHEME_A2V3 (group 64 or 128) or JF_SCHEME_A2V4 (group 128); k_zp (H_kv, num_slots, 128/group)
+ * bf16 holds the zero-points; keys score with khat = bf16(fma(code - 2, scale, zp))
+ * (jetfire_vllm/csrc/int2_qk_scores.cu:66-79).  o_new / out as in jf_fused_scan_topk_blend, or both NULL (no blend).
+ * Everything else as jf_fused_scan_topk. */
+int jf_fused_scan_topk_asym(int scheme, int group_size,
+                            const uint16_t* q, const uint8_t* k_data, const uint16_t* k_scales, const uint16_t* k_zp,
+                            const uint8_t* v_data, const uint16_t* v_scales,
+                            const int64_t* block_table, const int32_t* seq_lens,
+                            int B, int H_q, int H_kv, int max_S, int max_blocks, int64_t num_slots,
+                            int block_size, float attn_scale, int top_k,
+                            int64_t* topk_idx, int64_t* topk_slots,
+                            float* o_hat, float* o_old_unnorm, float* W,
+                            float* softmax_m, float* softmax_inv_z, float* scores,
+                            const uint16_t* o_new, uint16_t* out,
+                            void* workspace, size_t workspace_bytes, void* stream);
+
 /* Stage A alone and Stage B alone on the kernels of the fused step, for callers that keep the reference's two-call
  * structure (jetfire_vllm/adapter/decode_path.py:2081-2131 then :2804-2935): the same results as the split entry
  * points above for the shapes the fused step supports (head_dim 128, block_size 16, H_q/H_kv in {1,2,4,8,16},
@@ -241,6 +263,17 @@ int jf_stage_a_topk(int key_format, int group_size,
                     float* scores, int64_t* topk_idx, int64_t* topk_slots,
                     float* softmax_m, float* softmax_inv_z,
                     void* workspace, size_t workspace_bytes, void* stream);
+/* jf_stage_a_topk for the asymmetric INT2 keys: int2_qk_scores / int2_qk_scores_topk with k_zp
+ * (jetfire_vllm/csrc/int2_qk_scores.cu:66-79, 663-680); group 64 or 128; workspace:
+ * jf_fused_workspace_bytes(JF_SCHEME_A2V2, ...). */
+int jf_stage_a_topk_asym(int group_size,
+                         const uint16_t* q, const uint8_t* k_data, const uint16_t* k_scales, const uint16_t* k_zp,
+                         const int64_t* block_table, const int32_t* seq_lens,
+                         int B, int H_q, int H_kv, int max_S, int max_blocks, int64_t num_slots,
+                         int block_size, float attn_scale, int top_k,
+                         float* scores, int64_t* topk_idx, int64_t* topk_slots,
+                         float* softmax_m, float* softmax_inv_z,
+                         void* workspace, size_t workspace_bytes, void* stream);
 /* jf_topk_slots on the kernels of the fused step (top_k <= 2048): the same outputs as jf_topk_slots, i.e.
  * topk_slots_kernel_v5 / topk_slots_stats_kernel_v5 (jetfire_vllm/csrc/int3_qk_scores.cu:426-554,
  * jetfire_vllm/csrc/int8tc_qk_scores.cu:1678-1823).  workspace: jf_topk_slots_fast_workspace_bytes(). */

@@ -37,6 +37,8 @@ SIGNATURES = {
     "jf_fused_scan_topk": (I, [I, I, P, P, P, P, P, P, P, I, I, I, I, I, L, I, F, I, P, P, P, P, P, P, P, P, P, Z, P]),
     "jf_fused_scan_topk_blend": (I, [I, I, P, P, P, P, P, P, P, I, I, I, I, I, L, I, F, I, P, P, P, P, P, P, P, P, P, P, P, Z, P]),
     "jf_stage_a_topk": (I, [I, I, P, P, P, P, P, I, I, I, I, I, L, I, F, I, P, P, P, P, P, P, Z, P]),
+    "jf_stage_a_topk_asym": (I, [I, P, P, P, P, P, P, I, I, I, I, I, L, I, F, I, P, P, P, P, P, P, Z, P]),
+    "jf_fused_scan_topk_asym": (I, [I, I, P, P, P, P, P, P, P, P, I, I, I, I, I, L, I, F, I, P, P, P, P, P, P, P, P, P, P, P, Z, P]),
     "jf_topk_slots_fast_workspace_bytes": (Z, [I, I, I, I]),
     "jf_topk_slots_fast": (I, [P, P, P, I, I, I, I, I, I, P, P, P, P, P, Z, P]),
     "jf_stage_b_softmax_v": (I, [I, I, P, P, P, P, P, P, I, I, I, I, I, L, I, I, P, P, P, P, Z, P]),

@@ -111,12 +111,10 @@ class JetFireInt4CacheStore:
     @property
     def scheme(self) -> str | None:
         """Name the fused decode kernels know this store by, or None (split kernels / unsupported)."""
-        if self.k_asymmetric:
-            return None
-        if self.k_nbits not in (2, 3, 4) or self.v_nbits not in (2, 3, 4):
+        if self.k_nbits not in (2, 3, 4) or self.v_nbits not in (2, 3, 4) or (self.k_asymmetric and self.k_nbits != 2):
             return None
         if self.group_size == 128 or (self.group_size == 64 and 4 not in (self.k_nbits, self.v_nbits)):
-            return f"k{self.k_nbits}v{self.v_nbits}"
+            return f"a2v{self.v_nbits}" if self.k_asymmetric else f"k{self.k_nbits}v{self.v_nbits}"
         return None
 
     # ------------------------------------------------------------------ append

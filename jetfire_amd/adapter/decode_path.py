@@ -379,7 +379,7 @@ def _decode_batched(*, impl, layer, query, attn_metadata, output):
     if fused:
         o_hat, topk_slots, o_old, W, _ = ops.fused_attn_topk(
             store.scheme, q_batch, store.k_data, store.k_scales, store.v_data, store.v_scales, bt_batch, seq_lens_batch,
-            max_S, H_q, H_kv, store.block_size, top_k, scale)
+            max_S, H_q, H_kv, store.block_size, top_k, scale, k_zp=store.k_zp if store.k_asymmetric else None)
     else:
         o_hat, topk_slots, o_old, W = _split_stages(store, q_batch, bt_batch, seq_lens_batch, max_S, H_q, H_kv, top_k, scale,
                                                     plan=plan)

@@ -60,7 +60,7 @@ extern "C" int jf_fused_scan_topk(int scheme, int group_size, const uint16_t* q,
                                   int top_k, int64_t* topk_idx, int64_t* topk_slots, float* o_hat,
                                   float* o_old_unnorm, float* W, float* softmax_m, float* softmax_inv_z, float* scores,
                                   void* workspace, size_t workspace_bytes, void* stream) {
-  return fused_run<FS_FULL>(scheme, group_size, q, k_data, k_scales, v_data, v_scales, block_table, seq_lens, B, H_q,
+  return fused_run<FS_FULL>(scheme, group_size, q, k_data, k_scales, nullptr, v_data, v_scales, block_table, seq_lens, B, H_q,
                             H_kv, max_S, max_blocks, num_slots, block_size, attn_scale, top_k, topk_idx, topk_slots,
                             o_hat, o_old_unnorm, W, softmax_m, softmax_inv_z, scores, nullptr, nullptr, nullptr, workspace,
                             workspace_bytes, stream);
@@ -75,7 +75,24 @@ extern "C" int jf_fused_scan_topk_blend(int scheme, int group_size, const uint16
                                         float* scores, const uint16_t* o_new, uint16_t* out, void* workspace,
                                         size_t workspace_bytes, void* stream) {
   JF_CHECK_ARG(B == 0 || (o_new && out), "fused_scan_blend: null o_new / out");
-  return fused_run<FS_FULL>(scheme, group_size, q, k_data, k_scales, v_data, v_scales, block_table, seq_lens, B, H_q,
+  return fused_run<FS_FULL>(scheme, group_size, q, k_data, k_scales, nullptr, v_data, v_scales, block_table, seq_lens, B, H_q,
+                            H_kv, max_S, max_blocks, num_slots, block_size, attn_scale, top_k, topk_idx, topk_slots,
+                            o_hat, o_old_unnorm, W, softmax_m, softmax_inv_z, scores, nullptr, o_new, out, workspace,
+                            workspace_bytes, stream);
+}
+
+// Asymmetric INT2 keys: the same step with the zero-points of the key groups (and, optionally, the blend).
+extern "C" int jf_fused_scan_topk_asym(int scheme, int group_size, const uint16_t* q, const uint8_t* k_data,
+                                       const uint16_t* k_scales, const uint16_t* k_zp, const uint8_t* v_data,
+                                       const uint16_t* v_scales, const int64_t* block_table, const int32_t* seq_lens, int B,
+                                       int H_q, int H_kv, int max_S, int max_blocks, int64_t num_slots, int block_size,
+                                       float attn_scale, int top_k, int64_t* topk_idx, int64_t* topk_slots, float* o_hat,
+                                       float* o_old_unnorm, float* W, float* softmax_m, float* softmax_inv_z,
+                                       float* scores, const uint16_t* o_new, uint16_t* out, void* workspace,
+                                       size_t workspace_bytes, void* stream) {
+  JF_CHECK_ARG(scheme_has_zp(scheme), "fused_scan_asym: scheme must be JF_SCHEME_A2V2, JF_SCHEME_A2V3 or JF_SCHEME_A2V4");
+  JF_CHECK_ARG(B == 0 || k_zp != nullptr, "fused_scan_asym: null k_zp");
+  return fused_run<FS_FULL>(scheme, group_size, q, k_data, k_scales, k_zp, v_data, v_scales, block_table, seq_lens, B, H_q,
                             H_kv, max_S, max_blocks, num_slots, block_size, attn_scale, top_k, topk_idx, topk_slots,
                             o_hat, o_old_unnorm, W, softmax_m, softmax_inv_z, scores, nullptr, o_new, out, workspace,
                             workspace_bytes, stream);
@@ -123,7 +140,7 @@ extern "C" int jf_fused_scan_topk_static(int scheme, int group_size, const uint1
     }
     ws = g_scratch_ptr[dev];
   }
-  return fused_run<FS_FULL>(scheme, group_size, q, k_data, k_scales, v_data, v_scales, block_table, seq_lens, B, H_q,
+  return fused_run<FS_FULL>(scheme, group_size, q, k_data, k_scales, nullptr, v_data, v_scales, block_table, seq_lens, B, H_q,
                             H_kv, max_S, max_blocks, num_slots, block_size, attn_scale, top_k, topk_idx, topk_slots,
                             o_hat, o_old_unnorm, W, softmax_m, softmax_inv_z, scores, nullptr, nullptr, nullptr, ws,
                             (size_t)JF_FUSED_STATIC_SCRATCH_BYTES, stream);

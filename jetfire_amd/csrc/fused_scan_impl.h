@@ -92,6 +92,7 @@ struct FusedParams {
   const uint16_t* q;
   const uint8_t* k_data;
   const uint16_t* k_scales;
+  const uint16_t* k_zp;  // asymmetric INT2 keys only: zero-points, shaped like k_scales
   const uint8_t* v_data;
   const uint16_t* v_scales;
   const int64_t* block_table;
@@ -161,10 +162,11 @@ struct QInt8F {
 // After phase B the staging area holds the sum of the wavefronts' P.V accumulators.
 template <int SCHEME, int G, int NG>
 struct ScanLds {
-  // SCHEME = 10 * key bits + value bits: the key side (staging, query constants, phase A) and the value side
+  // SCHEME = 10 * key bits + value bits (key digit 1: asymmetric INT2): the key side (staging, query constants, phase A) and the value side
   // (staging, phase B) are chosen independently
   static constexpr bool K3 = (SCHEME / 10 == 3);
-  static constexpr bool K2 = (SCHEME / 10 == 2);
+  static constexpr bool KA = (SCHEME / 10 == 1);        // INT2 keys with a zero-point per group (four levels)
+  static constexpr bool K2 = (SCHEME / 10 == 2) || KA;  // four codes per byte
   static constexpr bool KLIMB = K2 || K3;  // keys with the bf16 model: fixed-point query limbs against integer codes
   static constexpr bool V2 = (SCHEME % 10 == 2);
   static constexpr bool V3 = (SCHEME % 10 == 3);
@@ -245,7 +247,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   constexpr bool HAS_K = (MODE == FS_FULL || MODE == FS_STAGE_A);  // key stream and phase A
   constexpr bool HAS_V = (MODE == FS_FULL || MODE == FS_STAGE_B);  // value stream and the P.V part of phase B
   constexpr bool HAS_TOPK = (MODE != FS_STAGE_B);                  // histograms and phase C
-  constexpr bool K3 = Lds::K3, KLIMB = Lds::KLIMB;
+  constexpr bool K3 = Lds::K3, KLIMB = Lds::KLIMB, KA = Lds::KA;
   constexpr bool V2 = Lds::V2, V3 = Lds::V3;
   constexpr int NSET = Lds::NSET;
   constexpr int SEG = Lds::SEG;
@@ -347,9 +349,11 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     kl_lds[i] = (uint32_t)((o / KP) * KROW + (o % KP));
   }
   const uint8_t* ksb = reinterpret_cast<const uint8_t*>(p.k_scales + (size_t)hkv * p.num_slots * (KLIMB ? NG : 1));
+  const uint8_t* kzb = KA ? reinterpret_cast<const uint8_t*>(p.k_zp + (size_t)hkv * p.num_slots * NG) : nullptr;
   struct KBuf {
     v4u r[KLD];
     uint32_t s[4];
+    uint32_t z[KA ? 4 : 1];  // zero-points of the asymmetric keys, packed like the scales
   };
   const int t16 = lane & 15, lg = lane >> 4;
   auto issue_k = [&](int chunk) -> KBuf {
@@ -366,6 +370,11 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
       const uint8_t* srow = ksb + (size_t)sb * (KNG * 2) + t16 * (KNG * 2);
       if (KNG == 2) kbuf.s[j] = *reinterpret_cast<const uint32_t*>(srow);
       else kbuf.s[j] = *reinterpret_cast<const uint16_t*>(srow);
+      if constexpr (KA) {
+        const uint8_t* zrow = kzb + (size_t)sb * (KNG * 2) + t16 * (KNG * 2);
+        if (KNG == 2) kbuf.z[j] = *reinterpret_cast<const uint32_t*>(zrow);
+        else kbuf.z[j] = *reinterpret_cast<const uint16_t*>(zrow);
+      }
     }
     return kbuf;
   };
@@ -587,7 +596,14 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
       mxl[set] = -INFINITY;
       mnl[set] = INFINITY;
     }
-    auto body = [&](int chunk, const uint32_t (&Sx)[4]) {
+    float sumq[NSET][NG];  // fixed-point sum of the query over the scale group (asymmetric keys)
+#pragma unroll
+    for (int set = 0; set < NSET; ++set)
+#pragma unroll
+      for (int g = 0; g < NG; ++g) sumq[set][g] = (float)(sq4[set][g] / 2);
+    (void)sumq;
+    auto body = [&](int chunk, const uint32_t (&Sx)[4], const uint32_t (&Zx)[4]) {
+      (void)Zx;
       // all LDS reads of the chunk first (plane dwords of the four pages, rounding coefficients), then arithmetic
       uint32_t Pj[4][3];
       float sgj[4][NG], egj[4][NG];
@@ -640,6 +656,75 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
             Bc[0][e] = (int)sw[0];
             Bc[1][e] = (int)sw[1];
           }
+        }
+        if constexpr (KA) {
+          // Four levels per group: khat(code) = bf16(fma(code - 2, scale, zp)) (int2_qk_scores.cu:66-79) is any function
+          // of the code's two bits b1 b0, so with the indicator bytes x0 = b0, x1 = b1, x01 = b0 & b1
+          //   khat = v0 + (v1 - v0) x0 + (v2 - v0) x1 + (v3 - v2 - v1 + v0) x01,   v_c = khat(c),
+          // and q . khat is four exact fixed-point sums (the query's own, and the three contractions with the
+          // indicators) combined in fp32 with coefficients that are exact differences of bf16 values.
+          v4i X0[2], X1[2], X01[2];
+#pragma unroll
+          for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const uint32_t c = (uint32_t)Bc[u][e];
+              const uint32_t b0 = c & 0x01010101u, b1 = (c >> 1) & 0x01010101u;
+              X0[u][e] = (int)b0;
+              X1[u][e] = (int)b1;
+              X01[u][e] = (int)(b0 & b1);
+            }
+          float coef[NG][4];
+#pragma unroll
+          for (int g = 0; g < NG; ++g) {
+            const float sc_g = sgj[j][g];
+            const float zp_g = bf16_to_f32((uint16_t)((g == 0) ? (Zx[j] & 0xffffu) : (Zx[j] >> 16)));
+            float v[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) v[c] = bf16_to_f32(f32_to_bf16(__builtin_fmaf((float)(c - 2), sc_g, zp_g)));
+            coef[g][0] = v[0];
+            coef[g][1] = v[1] - v[0];
+            coef[g][2] = v[2] - v[0];
+            coef[g][3] = (v[3] - v[2]) - (v[1] - v[0]);
+          }
+          const int tok = chunk * 64 + 16 * j + t16;
+          const bool valid = tok < n;
+#pragma unroll
+          for (int set = 0; set < NSET; ++set) {
+            const v4i zero = {0, 0, 0, 0};
+            float score = 0.f;
+#pragma unroll
+            for (int g = 0; g < NG; ++g) {
+              v4i D0, D1, D01;
+              if (NG == 2) {
+                D0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][g], X0[g], zero, 0, 0, 0);
+                D1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][g], X1[g], zero, 0, 0, 0);
+                D01 = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][g], X01[g], zero, 0, 0, 0);
+              } else {
+                D0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][0], X0[0], zero, 0, 0, 0);
+                D0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][1], X0[1], D0, 0, 0, 0);
+                D1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][0], X1[0], zero, 0, 0, 0);
+                D1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][1], X1[1], D1, 0, 0, 0);
+                D01 = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][0], X01[0], zero, 0, 0, 0);
+                D01 = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][1], X01[1], D01, 0, 0, 0);
+              }
+              const float s0f = (float)((((D0[2] << 8) + D0[1]) << 8) + D0[0]);
+              const float s1f = (float)((((D1[2] << 8) + D1[1]) << 8) + D1[0]);
+              const float s01f = (float)((((D01[2] << 8) + D01[1]) << 8) + D01[0]);
+              float v = coef[g][0] * sumq[set][g];
+              v = __builtin_fmaf(coef[g][1], s0f, v);
+              v = __builtin_fmaf(coef[g][2], s1f, v);
+              v = __builtin_fmaf(coef[g][3], s01f, v);
+              score = __builtin_fmaf(v, qsc[set][g], score);
+            }
+            const int h = set * 4 + lg;
+            if ((G % 4 == 0) || h < G) {
+              sc[h * L + tok] = valid ? score : -INFINITY;
+              mxl[set] = fmaxf(mxl[set], valid ? score : -INFINITY);
+              mnl[set] = fminf(mnl[set], valid ? score : INFINITY);
+            }
+          }
+          continue;
         }
         if constexpr (K3) {
 #pragma unroll
@@ -707,11 +792,14 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
         KBuf& cur = (it & 1) ? Kb : Ka;
         stash_k(cur);
         wave_lds_fence();
-        uint32_t Sc[4];
+        uint32_t Sc[4], Zc[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) Sc[j] = cur.s[j];
+        for (int j = 0; j < 4; ++j) {
+          Sc[j] = cur.s[j];
+          Zc[j] = KA ? cur.z[KA ? j : 0] : 0u;
+        }
         if (it + 2 < MAXIT && chunk + 2 * NW < nch_cover) cur = issue_k(chunk + 2 * NW);
-        body(chunk, Sc);
+        body(chunk, Sc, Zc);
         wave_lds_fence();
       }
     }
@@ -1985,6 +2073,9 @@ inline int lmax_dispatch(int scheme, int G, int NG) {
   JF_LMAX_ALL_G(JF_SCHEME_K2V3, 1); JF_LMAX_ALL_G(JF_SCHEME_K2V3, 2);
   JF_LMAX_ALL_G(JF_SCHEME_K3V3, 1); JF_LMAX_ALL_G(JF_SCHEME_K3V3, 2);
   JF_LMAX_ALL_G(JF_SCHEME_K4V3, 1);
+  JF_LMAX_ALL_G(JF_SCHEME_A2V2, 1); JF_LMAX_ALL_G(JF_SCHEME_A2V2, 2);
+  JF_LMAX_ALL_G(JF_SCHEME_A2V3, 1); JF_LMAX_ALL_G(JF_SCHEME_A2V3, 2);
+  JF_LMAX_ALL_G(JF_SCHEME_A2V4, 1);
 #undef JF_LMAX_ALL_G
 #undef JF_LMAX_CASE
   return 256;
@@ -2040,7 +2131,7 @@ inline void fused_plan(int scheme, int NG, int B, int H_q, int H_kv, int max_S, 
   const int kCUs = device_cus();
   constexpr double kScanFixed = 8.5;
   // one chunk per wavefront, all wavefronts; the mixed schemes are priced like the wider one
-  const double per_chunk = (scheme == JF_SCHEME_K3V2 || scheme == JF_SCHEME_K2V2) ? 5.9 : 6.6;  // (INT3 values: as INT4)
+  const double per_chunk = (scheme == JF_SCHEME_K3V2 || scheme == JF_SCHEME_K2V2) ? 5.9 : 6.6;  // (INT3 values, asymmetric keys: as INT4)
   int L = 256;
   double best = -1.0;
   for (int cand = 256; cand <= lmax; cand += 256) {
@@ -2128,14 +2219,18 @@ int launch_scan(const FusedParams& p, hipStream_t st) {
   return JF_OK;
 }
 
+inline bool scheme_has_zp(int scheme) {  // asymmetric INT2 keys
+  return scheme == JF_SCHEME_A2V2 || scheme == JF_SCHEME_A2V3 || scheme == JF_SCHEME_A2V4;
+}
 inline bool known_scheme(int scheme) {
   return scheme == JF_SCHEME_K3V2 || scheme == JF_SCHEME_K4V4 || scheme == JF_SCHEME_K3V4 || scheme == JF_SCHEME_K4V2 ||
          scheme == JF_SCHEME_K2V2 || scheme == JF_SCHEME_K2V4 || scheme == JF_SCHEME_K2V3 || scheme == JF_SCHEME_K3V3 ||
-         scheme == JF_SCHEME_K4V3;
+         scheme == JF_SCHEME_K4V3 || scheme_has_zp(scheme);
 }
 // scale groups per row: the schemes without an INT4 side may use 64-channel groups
 inline bool scheme_any_group(int scheme) {
-  return scheme == JF_SCHEME_K3V2 || scheme == JF_SCHEME_K2V2 || scheme == JF_SCHEME_K2V3 || scheme == JF_SCHEME_K3V3;
+  return scheme == JF_SCHEME_K3V2 || scheme == JF_SCHEME_K2V2 || scheme == JF_SCHEME_K2V3 || scheme == JF_SCHEME_K3V3 ||
+         scheme == JF_SCHEME_A2V2 || scheme == JF_SCHEME_A2V3;
 }
 inline int scheme_ng(int scheme, int group_size) { return scheme_any_group(scheme) ? D / group_size : 1; }
 
@@ -2147,7 +2242,7 @@ inline int scheme_ng(int scheme, int group_size) { return scheme_any_group(schem
 // zeros for the pre-correction terms), topk_slots is unused.
 template <int MODE>
 static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_t* k_data,
-                     const uint16_t* k_scales, const uint8_t* v_data, const uint16_t* v_scales,
+                     const uint16_t* k_scales, const uint16_t* k_zp, const uint8_t* v_data, const uint16_t* v_scales,
                      const int64_t* block_table, const int32_t* seq_lens, int B, int H_q, int H_kv,
                      int max_S, int max_blocks, int64_t num_slots, int block_size, float attn_scale,
                      int top_k, int64_t* topk_idx, int64_t* topk_slots, float* o_hat,
@@ -2156,8 +2251,11 @@ static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_
                      size_t workspace_bytes, void* stream) {
   JF_CHECK_ARG(known_scheme(scheme), "fused_scan: unknown scheme %d", scheme);
   JF_CHECK_ARG(MODE == FS_FULL || scheme == JF_SCHEME_K3V2 || scheme == JF_SCHEME_K4V4 ||
-                   (MODE == FS_STAGE_A && scheme == JF_SCHEME_K2V2) || (MODE == FS_STAGE_B && scheme == JF_SCHEME_K3V3),
-               "fused_scan: the stage-wise forms take the K3V2 or K4V4 side formats (Stage A also K2V2, Stage B also K3V3)");
+                   (MODE == FS_STAGE_A && (scheme == JF_SCHEME_K2V2 || scheme == JF_SCHEME_A2V2)) ||
+                   (MODE == FS_STAGE_B && scheme == JF_SCHEME_K3V3),
+               "fused_scan: the stage-wise forms take the K3V2 or K4V4 side formats (Stage A also K2V2 and A2V2, Stage B also K3V3)");
+  JF_CHECK_ARG(!(MODE == FS_FULL || MODE == FS_STAGE_A) || scheme_has_zp(scheme) == (k_zp != nullptr) || B == 0,
+               "fused_scan: zero-points go with the asymmetric INT2 key formats, and only with them");
   constexpr bool HAS_K = (MODE == FS_FULL || MODE == FS_STAGE_A), HAS_V = (MODE == FS_FULL || MODE == FS_STAGE_B);
   JF_CHECK_ARG(MODE != FS_TOPK || scheme == JF_SCHEME_K4V4, "fused_scan: the selection-only form uses the K4V4 layout");
   JF_CHECK_ARG((blend_o_new == nullptr) == (blend_out == nullptr), "fused_scan: o_new and out go together");
@@ -2182,6 +2280,7 @@ static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_
   if (HAS_K) {
     JF_CHECK_ARG(q && k_data && k_scales, "fused_scan: null input");
     JF_CHECK_ARG(((uintptr_t)k_data & 15) == 0 && ((uintptr_t)q & 15) == 0, "fused_scan: q and k_data must be 16-byte aligned");
+    JF_CHECK_ARG(((uintptr_t)k_scales & 3) == 0 && ((uintptr_t)k_zp & 3) == 0, "fused_scan: k_scales and k_zp must be 4-byte aligned");
   }
   if (MODE != FS_STAGE_B) JF_CHECK_ARG(scores_only ? scores != nullptr : (topk_idx && topk_slots), "fused_scan: null output");
   if (HAS_V) {
@@ -2193,7 +2292,7 @@ static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_
   if (!HAS_K) JF_CHECK_ARG(scores_in != nullptr, "fused_scan: null scores");
   const int NGv = scheme_ng(scheme, group_size);
   FusedParams p;
-  p.q = q; p.k_data = k_data; p.k_scales = k_scales; p.v_data = v_data; p.v_scales = v_scales;
+  p.q = q; p.k_data = k_data; p.k_scales = k_scales; p.k_zp = k_zp; p.v_data = v_data; p.v_scales = v_scales;
   p.block_table = block_table; p.seq_lens = seq_lens;
   p.B = B; p.H_q = H_q; p.H_kv = H_kv; p.max_S = max_S; p.max_blocks = max_blocks; p.num_slots = num_slots;
   p.attn_scale = attn_scale; p.top_k = top_k;
@@ -2248,11 +2347,17 @@ static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_
   } else if constexpr (MODE == FS_FULL || MODE == FS_STAGE_A) {
     if (scheme == JF_SCHEME_K2V2) {
       if (NGv == 2) JF_FUSED_BY_G(JF_SCHEME_K2V2, 2) else JF_FUSED_BY_G(JF_SCHEME_K2V2, 1)
+    } else if (scheme == JF_SCHEME_A2V2) {
+      if (NGv == 2) JF_FUSED_BY_G(JF_SCHEME_A2V2, 2) else JF_FUSED_BY_G(JF_SCHEME_A2V2, 1)
     } else if constexpr (MODE == FS_FULL) {  // the mixed pairs exist in the one-pass form only
       if (scheme == JF_SCHEME_K3V4) JF_FUSED_BY_G(JF_SCHEME_K3V4, 1)
       else if (scheme == JF_SCHEME_K4V2) JF_FUSED_BY_G(JF_SCHEME_K4V2, 1)
       else if (scheme == JF_SCHEME_K2V4) JF_FUSED_BY_G(JF_SCHEME_K2V4, 1)
       else if (scheme == JF_SCHEME_K4V3) JF_FUSED_BY_G(JF_SCHEME_K4V3, 1)
+      else if (scheme == JF_SCHEME_A2V4) JF_FUSED_BY_G(JF_SCHEME_A2V4, 1)
+      else if (scheme == JF_SCHEME_A2V3) {
+        if (NGv == 2) JF_FUSED_BY_G(JF_SCHEME_A2V3, 2) else JF_FUSED_BY_G(JF_SCHEME_A2V3, 1)
+      }
       else if (NGv == 2) JF_FUSED_BY_G(JF_SCHEME_K2V3, 2)
       else JF_FUSED_BY_G(JF_SCHEME_K2V3, 1)
     }

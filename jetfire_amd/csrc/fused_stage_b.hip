@@ -16,7 +16,7 @@ extern "C" int jf_stage_b_softmax_v(int value_format, int group_size, const floa
   JF_CHECK_ARG(value_format == JF_SCHEME_K3V2 || value_format == JF_SCHEME_K3V3 || value_format == JF_SCHEME_K4V4,
                "stage_b_softmax_v: value_format must be JF_SCHEME_K3V2 (INT2 values), JF_SCHEME_K3V3 (INT3 values) or "
                "JF_SCHEME_K4V4 (INT4 values)");
-  return fused_run<FS_STAGE_B>(value_format, group_size, nullptr, nullptr, nullptr, v_data, v_scales, block_table,
+  return fused_run<FS_STAGE_B>(value_format, group_size, nullptr, nullptr, nullptr, nullptr, v_data, v_scales, block_table,
                                seq_lens, B, H_q, H_kv, max_S, max_blocks, num_slots, block_size, 0.0f, top_k,
                                const_cast<int64_t*>(topk_idx), nullptr, o_hat, o_old_unnorm, W, nullptr, nullptr, nullptr,
                                scores, nullptr, nullptr, workspace, workspace_bytes, stream);

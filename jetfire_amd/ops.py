@@ -52,6 +52,8 @@ def _workspace(device: torch.device, nbytes: int, tag: str) -> torch.Tensor:
 
 # the nine symmetric (key bits, value bits) pairs of the fused step: name -> 10 * key bits + value bits
 FUSED_SCHEMES = {f"k{kb}v{vb}": 10 * kb + vb for kb in (2, 3, 4) for vb in (2, 3, 4)}
+# and the asymmetric INT2 keys (four levels, zero-points in k_zp): key digit 1
+FUSED_SCHEMES.update({f"a2v{vb}": 10 + vb for vb in (2, 3, 4)})
 
 
 def reserve_fused_workspace(scheme: str, B: int, H_q: int, H_kv: int, max_S: int, top_k: int, device) -> int:
@@ -231,7 +233,7 @@ def _fast_shape(H_q, H_kv, block_size, max_S, num_slots, top_k=None) -> bool:
             and (top_k is None or int(top_k) in FUSED_TOP_K))
 
 
-def _stage_a_fast(fmt: int, q, kd, ks, bt, sl, max_S, H_q, H_kv, attn_scale, top_k, stats: bool):
+def _stage_a_fast(fmt: int, q, kd, ks, bt, sl, max_S, H_q, H_kv, attn_scale, top_k, stats: bool, k_zp=None):
     """jf_stage_a_topk: -> (scores, idx, slots, m, iz); top_k None: scores alone."""
     lib = _lib.load()
     B, dev = q.size(0), q.device
@@ -244,10 +246,14 @@ def _stage_a_fast(fmt: int, q, kd, ks, bt, sl, max_S, H_q, H_kv, attn_scale, top
             m = torch.empty((B, H_q), dtype=torch.float32, device=dev)
             iz = torch.empty((B, H_q), dtype=torch.float32, device=dev)
         ws = _workspace(dev, lib.jf_fused_workspace_bytes(fmt, B, H_q, H_kv, int(max_S), int(top_k)), "fused")
-    _lib.check(lib.jf_stage_a_topk(
-        fmt, HEAD_DIM // ks.size(2), q.data_ptr(), kd.data_ptr(), ks.data_ptr(), bt.data_ptr(), sl.data_ptr(), B, H_q, H_kv,
-        int(max_S), bt.size(1), kd.size(1), 16, float(attn_scale), 0 if top_k is None else int(top_k), scores.data_ptr(),
-        _ptr(idx), _ptr(slots), _ptr(m), _ptr(iz), _ptr(ws), 0 if ws is None else ws.numel(), _stream(q)))
+    tail = (bt.data_ptr(), sl.data_ptr(), B, H_q, H_kv, int(max_S), bt.size(1), kd.size(1), 16, float(attn_scale),
+            0 if top_k is None else int(top_k), scores.data_ptr(), _ptr(idx), _ptr(slots), _ptr(m), _ptr(iz), _ptr(ws),
+            0 if ws is None else ws.numel(), _stream(q))
+    if k_zp is None:
+        _lib.check(lib.jf_stage_a_topk(fmt, HEAD_DIM // ks.size(2), q.data_ptr(), kd.data_ptr(), ks.data_ptr(), *tail))
+    else:       # asymmetric INT2 keys (fmt 12)
+        _lib.check(lib.jf_stage_a_topk_asym(HEAD_DIM // ks.size(2), q.data_ptr(), kd.data_ptr(), ks.data_ptr(),
+                                            k_zp.data_ptr(), *tail))
     return scores, idx, slots, m, iz
 
 
@@ -297,12 +303,13 @@ def _intn_qk_scores(nbits: int, name: str, q, k_data, k_scales, block_table, seq
     q, kd, ks, bt, sl = _stage_a_args(q, k_data, k_scales, block_table, seq_lens, H_q, H_kv, HEAD_DIM * nbits // 8)
     ng = ks.size(2)
     _check(ng in (1, 2), f"{name} currently supports K quant groups 1 or 2, got {ng}")
-    if nbits == 2 and k_zp is None and _fast_shape(H_q, H_kv, block_size, max_S, kd.size(1)):
-        return _stage_a_fast(22, q, kd, ks, bt, sl, max_S, H_q, H_kv, attn_scale, None, False)[0]
     if k_zp is not None:
         k_zp = (k_zp.unsqueeze(-1) if k_zp.dim() == 2 else k_zp).contiguous()
         _check(k_zp.is_cuda and k_zp.dtype == torch.bfloat16 and k_zp.shape == ks.shape,
                "k_zp must be bf16 with the shape of k_scales")
+    if nbits == 2 and _fast_shape(H_q, H_kv, block_size, max_S, kd.size(1)):
+        return _stage_a_fast(22 if k_zp is None else 12, q, kd, ks, bt, sl, max_S, H_q, H_kv, attn_scale, None, False,
+                             k_zp=k_zp)[0]
     B = q.size(0)
     scores = torch.empty((B, H_q, max_S), dtype=torch.float32, device=q.device)
     _lib.check(lib.jf_intn_qk_scores(nbits, q.data_ptr(), kd.data_ptr(), ks.data_ptr(), _ptr(k_zp), bt.data_ptr(), sl.data_ptr(),
@@ -323,11 +330,17 @@ def int2_qk_scores(q, k_data, k_scales, k_zp, block_table, seq_lens, max_S, H_q,
 def int2_qk_scores_topk(q, k_data, k_scales, k_zp, block_table, seq_lens, max_S, H_q, H_kv, block_size, attn_scale,
                         top_k) -> List[torch.Tensor]:
     """int2_qk_scores.cu:583-660 -> [scores, topk_idx, topk_slots]."""
-    symmetric = k_zp is None or k_zp.numel() == 0
-    if symmetric and _fast_shape(H_q, H_kv, block_size, max_S, k_data.size(1) if k_data.dim() == 3 else 0, top_k):
+    if k_zp is not None and k_zp.numel() == 0:
+        k_zp = None
+    if _fast_shape(H_q, H_kv, block_size, max_S, k_data.size(1) if k_data.dim() == 3 else 0, top_k):
         q_, kd, ks, bt, sl = _stage_a_args(q, k_data, k_scales, block_table, seq_lens, H_q, H_kv, 32)
         _check(ks.size(2) in (1, 2), f"int2_qk_scores currently supports K quant groups 1 or 2, got {ks.size(2)}")
-        return list(_stage_a_fast(22, q_, kd, ks, bt, sl, max_S, H_q, H_kv, attn_scale, int(top_k), False)[:3])
+        if k_zp is not None:
+            k_zp = (k_zp.unsqueeze(-1) if k_zp.dim() == 2 else k_zp).contiguous()
+            _check(k_zp.is_cuda and k_zp.dtype == torch.bfloat16 and k_zp.shape == ks.shape,
+                   "k_zp must be bf16 with the shape of k_scales")
+        return list(_stage_a_fast(22 if k_zp is None else 12, q_, kd, ks, bt, sl, max_S, H_q, H_kv, attn_scale, int(top_k),
+                                  False, k_zp=k_zp)[:3])
     scores = int2_qk_scores(q, k_data, k_scales, k_zp, block_table, seq_lens, max_S, H_q, H_kv, block_size, attn_scale)
     idx, slots, _, _ = _topk(scores, block_table, seq_lens, max_S, H_q, block_size, top_k, False, "int2_qk_scores_topk")
     return [scores, idx, slots]
@@ -578,7 +591,7 @@ def int8tc_softmax_v_with_pre_corr_reg_stats(scores, softmax_m, softmax_inv_z, v
 
 def fused_attn_topk(scheme: str, q, k_data, k_scales, v_data, v_scales, block_table, seq_lens, max_S, H_q, H_kv,
                     block_size, top_k, attn_scale, group_size: Optional[int] = None, return_scores: bool = False,
-                    return_stats: bool = False, blend=None):
+                    return_stats: bool = False, blend=None, k_zp=None):
     """One fused pass: -> (o_hat, topk_slots, o_old_unnorm, W, topk_idx[, softmax_m, softmax_inv_z][, scores]).
 
     blend=(o_new, out), both (B, H_q, 128) bf16 on the GPU: the merge kernel also writes
@@ -588,12 +601,19 @@ def fused_attn_topk(scheme: str, q, k_data, k_scales, v_data, v_scales, block_ta
     The single-call contract is the one of the reference's int2_fused_attn_topk
     (jetfire_vllm/kernels/int2_fused_attn_topk.py:5-10) extended to INT3 / INT4 keys (INT4: the int8-Q scoring
     model), symmetric INT2 keys, and INT2 / INT3 / INT4 values: "k{2,3,4}v{2,3,4}"; pairs without an INT4 side take
-    group 64 or 128, the others group 128."""
+    group 64 or 128, the others group 128.  "a2v{2,3,4}": asymmetric INT2 keys, whose zero-points come in `k_zp`
+    (shaped like k_scales), the reference's int2_asym_k_* kernel sets."""
     lib = _lib.load()
     scheme_id = FUSED_SCHEMES.get(scheme)
     _check(scheme_id is not None, f"unknown scheme {scheme!r} ({', '.join(sorted(FUSED_SCHEMES))})")
-    kp, vp = 16 * (scheme_id // 10), 16 * (scheme_id % 10)
+    asym = scheme_id // 10 == 1
+    kp, vp = (32 if asym else 16 * (scheme_id // 10)), 16 * (scheme_id % 10)
     q, kd, ks, bt, sl = _stage_a_args(q, k_data, k_scales, block_table, seq_lens, H_q, H_kv, kp)
+    _check(asym == (k_zp is not None), "k_zp goes with the a2v* schemes, and only with them")
+    if asym:
+        k_zp = (k_zp.unsqueeze(-1) if k_zp.dim() == 2 else k_zp).contiguous()
+        _check(k_zp.is_cuda and k_zp.dtype == torch.bfloat16 and k_zp.shape == ks.shape,
+               "k_zp must be bf16 with the shape of k_scales")
     _gpu(v_data, v_scales)
     _check(v_data.dtype == torch.uint8 and v_data.dim() == 3 and v_data.size(2) == vp, f"v_data last dim must be {vp}")
     _check(v_scales.dtype == torch.bfloat16, "v_scales must be bf16")
@@ -617,12 +637,15 @@ def fused_attn_topk(scheme: str, q, k_data, k_scales, v_data, v_scales, block_ta
     scores = torch.empty((B, H_q, max_S), dtype=torch.float32, device=dev) if return_scores else None
     need = lib.jf_fused_workspace_bytes(scheme_id, B, H_q, H_kv, int(max_S), int(top_k))
     ws = _workspace(dev, need, "fused")
-    head = (scheme_id, gs, q.data_ptr(), kd.data_ptr(), ks.data_ptr(), vd.data_ptr(), vs.data_ptr(), bt.data_ptr(),
+    head = (scheme_id, gs, q.data_ptr(), kd.data_ptr(), ks.data_ptr(), *((k_zp.data_ptr(),) if asym else ()),
+            vd.data_ptr(), vs.data_ptr(), bt.data_ptr(),
             sl.data_ptr(), B, H_q, H_kv, int(max_S), bt.size(1), kd.size(1), int(block_size), float(attn_scale), int(top_k),
             idx.data_ptr(), slots.data_ptr(), o_hat.data_ptr(), o_old.data_ptr(), W.data_ptr(), _ptr(m), _ptr(iz),
             _ptr(scores))
-    if blend is None:
+    if blend is None and not asym:
         _lib.check(lib.jf_fused_scan_topk(*head, ws.data_ptr(), ws.numel(), _stream(q)))
+    elif blend is None:
+        _lib.check(lib.jf_fused_scan_topk_asym(*head, None, None, ws.data_ptr(), ws.numel(), _stream(q)))
     else:
         o_new, out = blend
         _gpu(o_new, out)
@@ -630,8 +653,8 @@ def fused_attn_topk(scheme: str, q, k_data, k_scales, v_data, v_scales, block_ta
         _check(tuple(o_new.shape) == (B, H_q, HEAD_DIM) and tuple(out.shape) == (B, H_q, HEAD_DIM),
                "o_new / out must be (B, H_q, 128)")
         _check(o_new.is_contiguous() and out.is_contiguous(), "o_new / out must be contiguous")
-        _lib.check(lib.jf_fused_scan_topk_blend(*head, o_new.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(),
-                                                _stream(q)))
+        entry = lib.jf_fused_scan_topk_asym if asym else lib.jf_fused_scan_topk_blend
+        _lib.check(entry(*head, o_new.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(), _stream(q)))
     out = [o_hat, slots, o_old, W, idx]
     if return_stats:
         out += [m, iz]

@@ -157,7 +157,7 @@ def test_pool_registry_and_store_geometry(adapter):
         store.sequence_slots(torch.tensor([0, -1]), 20)
     asym = adapter.JetFireInt4CacheStore(num_kv_heads=2, head_dim=128, group_size=64, num_blocks=1, block_size=16,
                                          device="cpu", k_nbits=2, v_nbits=2, k_asymmetric=True, v_asymmetric=False)
-    assert asym.k_zp.shape == asym.k_scales.shape == (2, 16, 2) and asym.scheme is None     # INT2 keys with zero-points
+    assert asym.k_zp.shape == asym.k_scales.shape == (2, 16, 2) and asym.scheme == "a2v2"    # INT2 keys with zero-points
     for kw in (dict(k_nbits=3, v_nbits=2, k_asymmetric=True), dict(k_nbits=2, v_nbits=2, v_asymmetric=True)):
         with pytest.raises(NotImplementedError):
             adapter.JetFireInt4CacheStore(num_kv_heads=2, head_dim=128, group_size=64, num_blocks=1, block_size=16,

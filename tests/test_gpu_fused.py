@@ -20,7 +20,7 @@ def ops():
 def run_fused(scheme, c, d, S, K):
     o = ops()
     return o.fused_attn_topk(scheme.split("_")[0], d["q"], d["kd"], d["ks"], d["vd"], d["vs"], d["bt"], d["lens"], S,
-                             c["Hq"], c["Hkv"], 16, K, SCALE, return_scores=True, return_stats=True)
+                             c["Hq"], c["Hkv"], 16, K, SCALE, return_scores=True, return_stats=True, k_zp=d.get("kz"))
 
 
 def check_against_oracle(scheme, c, S, K, out):
@@ -28,7 +28,8 @@ def check_against_oracle(scheme, c, S, K, out):
     kb, vb, gs = c["kbits"], c["vbits"], c["gs"]
     Hq, Hkv = c["Hq"], c["Hkv"]
     if kb in (2, 3):
-        ref_sc = O.scores_bf16_model(c["q"], c["kd"], c["ks"], c["bt"], c["lens"], S, Hq, Hkv, 16, SCALE, kb, gs)
+        ref_sc = O.scores_bf16_model(c["q"], c["kd"], c["ks"], c["bt"], c["lens"], S, Hq, Hkv, 16, SCALE, kb, gs,
+                                     k_zp_bits=c.get("kzp"))
         valid = np.isfinite(ref_sc)
         assert np.array_equal(np.isneginf(scores), ~valid)
         np.testing.assert_allclose(scores[valid], ref_sc[valid], atol=2e-5, rtol=2e-5)
@@ -98,15 +99,25 @@ CASES = [
     # the widest correction of the fused form
     ("k3v2", 1, 8, 2, 5000, [4987], 2048), ("k4v4", 2, 8, 2, 3000, [1000, 3000], 2048),
     ("k3v3", 1, 32, 4, 6000, None, 2048), ("k2v4", 2, 4, 4, 2048, [2048, 2047], 2048),
+    # asymmetric INT2 keys (a zero-point per group) with every value format
+    ("a2v2", 2, 8, 2, 512, None, 64), ("a2v2_g128", 2, 8, 2, 700, None, 128), ("a2v3", 2, 8, 2, 512, None, 64),
+    ("a2v3_g128", 2, 8, 2, 700, None, 128), ("a2v4", 2, 8, 2, 512, None, 64),
+    ("a2v2", 3, 32, 4, 512, [17, 257, 512], 256), ("a2v4", 3, 32, 4, 512, [17, 257, 512], 256),
+    ("a2v2", 4, 8, 2, 32, [0, 1, 9, 17], 32), ("a2v3", 1, 8, 2, 5000, [4987], 256), ("a2v4", 1, 8, 2, 5000, [4987], 1024),
+    ("a2v2", 1, 4, 4, 300, None, 32), ("a2v4", 1, 4, 2, 300, None, 64), ("a2v2_g128", 1, 16, 1, 600, None, 64),
+    ("a2v3", 1, 16, 1, 600, None, 64),
 ]
 SCHEME_GEOMETRY = {f"k{kb}v{vb}": (kb, vb, 128 if 4 in (kb, vb) else 64) for kb in (2, 3, 4) for vb in (2, 3, 4)}
 SCHEME_GEOMETRY.update({f"k{kb}v{vb}_g128": (kb, vb, 128) for kb in (2, 3) for vb in (2, 3)})
+# asymmetric INT2 keys
+SCHEME_GEOMETRY.update({"a2v2": (2, 2, 64), "a2v2_g128": (2, 2, 128), "a2v3": (2, 3, 64), "a2v3_g128": (2, 3, 128),
+                        "a2v4": (2, 4, 128)})
 
 
 @pytest.mark.parametrize("scheme,B,Hq,Hkv,S,lens,K", CASES)
 def test_fused_scan_matches_oracle(scheme, B, Hq, Hkv, S, lens, K):
     kb, vb, gs = SCHEME_GEOMETRY[scheme]
-    c = make_case(70 + S + Hq, B, Hq, Hkv, S, kb, vb, gs, lens=lens, extra_blocks=3)
+    c = make_case(70 + S + Hq, B, Hq, Hkv, S, kb, vb, gs, lens=lens, extra_blocks=3, k_asym=scheme.startswith("a"))
     d = to_device(c)
     out = run_fused(scheme, c, d, S, K)
     check_against_oracle(scheme, c, S, K, out)

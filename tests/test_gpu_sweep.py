@@ -11,7 +11,8 @@ pytestmark = pytest.mark.gpu
 
 SCHEMES = {"k3v2": (3, 2, 64), "k3v2_g128": (3, 2, 128), "k4v4": (4, 4, 128), "k3v4": (3, 4, 128), "k4v2": (4, 2, 128),
            "k2v2": (2, 2, 64), "k2v2_g128": (2, 2, 128), "k2v4": (2, 4, 128),
-           "k3v3": (3, 3, 64), "k3v3_g128": (3, 3, 128), "k2v3": (2, 3, 64), "k4v3": (4, 3, 128)}
+           "k3v3": (3, 3, 64), "k3v3_g128": (3, 3, 128), "k2v3": (2, 3, 64), "k4v3": (4, 3, 128),
+           "a2v2": (2, 2, 64), "a2v2_g128": (2, 2, 128), "a2v3": (2, 3, 64), "a2v4": (2, 4, 128)}
 
 
 def _draw(seed):
@@ -28,12 +29,13 @@ def _draw(seed):
     return scheme, B, G * Hkv, Hkv, S, lens, K, split
 
 
-@pytest.mark.parametrize("seed", range(96))
+@pytest.mark.parametrize("seed", range(128))
 def test_fused_scan_random_geometry(seed):
     from jetfire_amd import _lib
     scheme, B, Hq, Hkv, S, lens, K, split = _draw(seed)
     kb, vb, gs = SCHEMES[scheme]
-    c = make_case(500 + seed, B, Hq, Hkv, S, kb, vb, gs, lens=lens, extra_blocks=int(seed % 4))
+    c = make_case(500 + seed, B, Hq, Hkv, S, kb, vb, gs, lens=lens, extra_blocks=int(seed % 4),
+                  k_asym=scheme.startswith("a"))
     d = to_device(c)
     lib = _lib.load()
     print(f"case: {scheme} B={B} Hq={Hq} Hkv={Hkv} S={S} lens={lens} K={K} split={split}", flush=True)
