@@ -16,7 +16,11 @@ CSRC = os.path.join(PKG_DIR, "csrc")
 OBJ_DIR = os.path.join(PKG_DIR, "build")
 LIB_PATH = os.path.join(PKG_DIR, "libjetfire_amd.so")
 
-SOURCES = (
+SOURCES = (     # (the long compilations first: the pool starts them together)
+    "fused_full_a.hip",
+    "fused_full_b.hip",
+    "fused_full_c.hip",
+    "fused_full_d.hip",
     "quant_write.hip",
     "shadow_write.hip",
     "qk_scores.hip",

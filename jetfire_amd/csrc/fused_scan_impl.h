@@ -63,6 +63,12 @@ extern std::atomic<int> g_force_split_len;  // test / measurement aid: overrides
 // Compute units of the current device (the planner balances workgroups over them); 256, the MI355X count, when
 // no device can be asked (planning on a host without a GPU).
 int device_cus();
+// The one-pass scan kernels are instantiated in four translation units (fused_full_*.hip), one per family of
+// schemes, so that they compile side by side; `params` points to the launcher's FusedParams.
+int launch_full_scan_a(int scheme, int G, int NG, const void* params, void* stream);  // K3V2, K4V4, K3V4, K4V2
+int launch_full_scan_b(int scheme, int G, int NG, const void* params, void* stream);  // K2V2, K2V3, K2V4
+int launch_full_scan_c(int scheme, int G, int NG, const void* params, void* stream);  // K3V3, K4V3
+int launch_full_scan_d(int scheme, int G, int NG, const void* params, void* stream);  // A2V2, A2V3, A2V4
 
 namespace {
 
@@ -2219,6 +2225,20 @@ int launch_scan(const FusedParams& p, hipStream_t st) {
   return JF_OK;
 }
 
+// One scheme of the one-pass form: the GQA group picks the instantiation.
+template <int SCHEME, int NG>
+int launch_full_by_group(int G, const void* params, void* stream) {
+  const FusedParams& p = *static_cast<const FusedParams*>(params);
+  hipStream_t st = (hipStream_t)stream;
+  switch (G) {
+    case 1: return launch_scan<FS_FULL, SCHEME, 1, NG>(p, st);
+    case 2: return launch_scan<FS_FULL, SCHEME, 2, NG>(p, st);
+    case 4: return launch_scan<FS_FULL, SCHEME, 4, NG>(p, st);
+    case 8: return launch_scan<FS_FULL, SCHEME, 8, NG>(p, st);
+    default: return launch_scan<FS_FULL, SCHEME, 16, NG>(p, st);
+  }
+}
+
 inline bool scheme_has_zp(int scheme) {  // asymmetric INT2 keys
   return scheme == JF_SCHEME_A2V2 || scheme == JF_SCHEME_A2V3 || scheme == JF_SCHEME_A2V4;
 }
@@ -2334,33 +2354,23 @@ static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_
     case 8: JF_FUSED_CASE(SCH, 8, NGG); break;         \
     default: JF_FUSED_CASE(SCH, 16, NGG); break;       \
   }
-  if constexpr (MODE == FS_TOPK) {
+  if constexpr (MODE == FS_FULL) {  // (instantiated elsewhere, by family)
+    if (scheme_has_zp(scheme)) rc = launch_full_scan_d(scheme, G, NGv, &p, stream);
+    else if (scheme / 10 == 2) rc = launch_full_scan_b(scheme, G, NGv, &p, stream);
+    else if (scheme == JF_SCHEME_K3V3 || scheme == JF_SCHEME_K4V3) rc = launch_full_scan_c(scheme, G, NGv, &p, stream);
+    else rc = launch_full_scan_a(scheme, G, NGv, &p, stream);
+  } else if constexpr (MODE == FS_TOPK) {
     JF_FUSED_BY_G(JF_SCHEME_K4V4, 1)
   } else if (scheme == JF_SCHEME_K3V2) {
     if (NGv == 2) JF_FUSED_BY_G(JF_SCHEME_K3V2, 2) else JF_FUSED_BY_G(JF_SCHEME_K3V2, 1)
   } else if (scheme == JF_SCHEME_K4V4) {
     JF_FUSED_BY_G(JF_SCHEME_K4V4, 1)
-  } else if (MODE != FS_STAGE_A && scheme == JF_SCHEME_K3V3) {
-    if constexpr (MODE != FS_STAGE_A) {
-      if (NGv == 2) JF_FUSED_BY_G(JF_SCHEME_K3V3, 2) else JF_FUSED_BY_G(JF_SCHEME_K3V3, 1)
-    }
-  } else if constexpr (MODE == FS_FULL || MODE == FS_STAGE_A) {
-    if (scheme == JF_SCHEME_K2V2) {
-      if (NGv == 2) JF_FUSED_BY_G(JF_SCHEME_K2V2, 2) else JF_FUSED_BY_G(JF_SCHEME_K2V2, 1)
-    } else if (scheme == JF_SCHEME_A2V2) {
-      if (NGv == 2) JF_FUSED_BY_G(JF_SCHEME_A2V2, 2) else JF_FUSED_BY_G(JF_SCHEME_A2V2, 1)
-    } else if constexpr (MODE == FS_FULL) {  // the mixed pairs exist in the one-pass form only
-      if (scheme == JF_SCHEME_K3V4) JF_FUSED_BY_G(JF_SCHEME_K3V4, 1)
-      else if (scheme == JF_SCHEME_K4V2) JF_FUSED_BY_G(JF_SCHEME_K4V2, 1)
-      else if (scheme == JF_SCHEME_K2V4) JF_FUSED_BY_G(JF_SCHEME_K2V4, 1)
-      else if (scheme == JF_SCHEME_K4V3) JF_FUSED_BY_G(JF_SCHEME_K4V3, 1)
-      else if (scheme == JF_SCHEME_A2V4) JF_FUSED_BY_G(JF_SCHEME_A2V4, 1)
-      else if (scheme == JF_SCHEME_A2V3) {
-        if (NGv == 2) JF_FUSED_BY_G(JF_SCHEME_A2V3, 2) else JF_FUSED_BY_G(JF_SCHEME_A2V3, 1)
-      }
-      else if (NGv == 2) JF_FUSED_BY_G(JF_SCHEME_K2V3, 2)
-      else JF_FUSED_BY_G(JF_SCHEME_K2V3, 1)
-    }
+  } else if constexpr (MODE == FS_STAGE_B) {
+    if (NGv == 2) JF_FUSED_BY_G(JF_SCHEME_K3V3, 2) else JF_FUSED_BY_G(JF_SCHEME_K3V3, 1)
+  } else if (scheme == JF_SCHEME_K2V2) {  // (Stage A)
+    if (NGv == 2) JF_FUSED_BY_G(JF_SCHEME_K2V2, 2) else JF_FUSED_BY_G(JF_SCHEME_K2V2, 1)
+  } else {
+    if (NGv == 2) JF_FUSED_BY_G(JF_SCHEME_A2V2, 2) else JF_FUSED_BY_G(JF_SCHEME_A2V2, 1)
   }
 #undef JF_FUSED_BY_G
 #undef JF_FUSED_CASE
