@@ -175,7 +175,8 @@ def test_pool_registry_and_store_geometry(adapter):
     ("SymInt3K_SymInt3V", "k3v3", 64, 3, 3), ("SymInt3K_SymInt4V", "k3v4", 128, 3, 4),
     ("SymInt4K_SymInt2V", "k4v2", 128, 4, 2), ("SymInt4K_SymInt3V", "k4v3", 64, 4, 3),
     # asymmetric INT2 keys (zero-point per group)
-    ("AsymInt2K4Level_SymInt2V", "k2v2", 128, 2, 2), ("AsymInt2K_SymInt4V", "k2v4", 64, 2, 4)])
+    ("AsymInt2K4Level_SymInt2V", "k2v2", 128, 2, 2), ("AsymInt2K_SymInt4V", "k2v4", 64, 2, 4),
+    ("AsymInt2K4Level_SymInt3V", "k2v3", 64, 2, 3), ("AsymInt2K4Level_SymInt4V", "k2v4", 128, 2, 4)])
 def test_prefill_then_decode_steps_match_the_oracle(adapter, scheme_name, scheme, gs, kb, vb):
     B, Hq, Hkv, D, bs = 3, 8, 2, 128, 16
     lens0 = [300, 37, 512]
