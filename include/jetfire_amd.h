@@ -34,17 +34,17 @@ extern "C" {
 
 #define JF_SCHEME_K3V2 32    /* INT3 keys, INT2 values  (SymInt3K_SymInt2V) */
 #define JF_SCHEME_K4V4 44    /* INT4 keys, INT4 values  (SymInt4K_SymInt4V) */
-#define JF_SCHEME_K3V4 34    /* INT3 keys, INT4 values  (SymInt3K_SymInt4V), group 128 */
+#define JF_SCHEME_K3V4 34    /* INT3 keys, INT4 values  (SymInt3K_SymInt4V), group 64 or 128 */
 #define JF_SCHEME_K4V2 42    /* INT4 keys, INT2 values  (SymInt4K_SymInt2V), group 128 */
 #define JF_SCHEME_K2V2 22    /* INT2 keys, INT2 values  (SymInt2K_SymInt2V), group 64 or 128 */
-#define JF_SCHEME_K2V4 24    /* INT2 keys, INT4 values  (SymInt2K_SymInt4V), group 128 */
+#define JF_SCHEME_K2V4 24    /* INT2 keys, INT4 values  (SymInt2K_SymInt4V), group 64 or 128 */
 #define JF_SCHEME_K2V3 23    /* INT2 keys, INT3 values  (SymInt2K_SymInt3V), group 64 or 128 */
 #define JF_SCHEME_K3V3 33    /* INT3 keys, INT3 values  (SymInt3K_SymInt3V), group 64 or 128 */
 #define JF_SCHEME_K4V3 43    /* INT4 keys, INT3 values  (SymInt4K_SymInt3V), group 128 */
 /* asymmetric INT2 keys (four levels, a zero-point per group: k_zp), key digit 1 */
 #define JF_SCHEME_A2V2 12    /* (AsymInt2K4Level_SymInt2V), group 64 or 128 */
 #define JF_SCHEME_A2V3 13    /* (AsymInt2K4Level_SymInt3V), group 64 or 128 */
-#define JF_SCHEME_A2V4 14    /* (AsymInt2K4Level_SymInt4V), group 128 */
+#define JF_SCHEME_A2V4 14    /* (AsymInt2K4Level_SymInt4V), group 64 or 128 */
 
 const char* jf_last_error(void);
 const char* jf_version(void);
@@ -191,8 +191,8 @@ int jf_softmax_v_int8_tiles(const float* scores, const float* softmax_m, const f
  * 2785-2935): topk_idx, topk_slots, o_hat, o_old_unnorm, W, and optionally softmax_m / softmax_inv_z.
  * The reference's own single-call form of this contract is int2_fused_attn_topk
  * (jetfire_vllm/kernels/int2_fused_attn_topk.py:5-10).  scheme: any of the nine symmetric pairs JF_SCHEME_K{2,3,4}V{2,3,4}
- * (the reference's kernel sets jetfire_vllm/kernels/_dispatch/sym_int*_k_sym_int*_v.py); pairs without an INT4 side take
- * group 64 or 128, the others group 128.  INT3 and symmetric INT2 keys score with the bf16 model of
+ * (the reference's kernel sets jetfire_vllm/kernels/_dispatch/sym_int*_k_sym_int*_v.py); pairs with INT4 keys (one key
+ * scale per row) take group 128, the others group 64 or 128.  INT3 and symmetric INT2 keys score with the bf16 model of
  * jf_int3_qk_scores / jf_intn_qk_scores (jetfire_vllm/csrc/int2_qk_scores.cu:66-79), INT4 keys with the int8-Q model
  * of jf_int8tc_qk_scores; INT3 values are the planar rows of jetfire_vllm/csrc/int3_softmax_v.cu:43,282-284.
  * top_k: power of two in [32, 2048] (the split entry points above take up to 8192); num_slots at most 2^26 (row
@@ -228,7 +228,7 @@ int jf_fused_scan_topk_blend(int scheme, int group_size,
 
 /* The fused step for the asymmetric INT2 keys (the reference's kernel sets
  * jetfire_vllm/kernels/_dispatch/int2_asym_k_sym_v.py, int2_asym_k_sym_int3_v.py, int2_asym_k_sym_int4_v.py): scheme
- * JF_SCHEME_A2V2 / JF_SCHEME_A2V3 (group 64 or 128) or JF_SCHEME_A2V4 (group 128); k_zp (H_kv, num_slots, 128/group)
+ * JF_SCHEME_A2V2 / JF_SCHEME_A2V3 / JF_SCHEME_A2V4 (group 64 or 128); k_zp (H_kv, num_slots, 128/group)
  * bf16 holds the zero-points; keys score with khat = bf16(fma(code - 2, scale, zp))
  * (jetfire_vllm/csrc/int2_qk_scores.cu:66-79).  o_new / out as in jf_fused_scan_topk_blend, or both NULL (no blend).
  * Everything else as jf_fused_scan_topk. */
@@ -286,7 +286,8 @@ int jf_topk_slots_fast(const float* scores, const int32_t* seq_lens, const int64
  * value_format JF_SCHEME_K3V2: INT2 values, group 64 or 128), int3_softmax_v_with_pre_corr_wvs2
  * (jetfire_vllm/csrc/int3_softmax_v.cu:752-860; value_format JF_SCHEME_K3V3: INT3 values, group 64 or 128) and
  * int4_softmax_v_with_pre_corr_wvs2_scores
- * (jetfire_vllm/csrc/int4_softmax_v.cu:2203-2235; value_format JF_SCHEME_K4V4: INT4 values, group 128), with exact
+ * (jetfire_vllm/csrc/int4_softmax_v.cu:2203-2235; value_format JF_SCHEME_K4V4: INT4 values, group 128, or
+ * JF_SCHEME_K3V4: INT4 values, group 64 or 128), with exact
  * fp32 softmax weights computed from `scores`.  topk_idx (B, H_q, top_k), ascending and -1 padded, may be NULL
  * (o_hat only; o_old_unnorm and W are then zero). */
 int jf_stage_b_softmax_v(int value_format, int group_size,

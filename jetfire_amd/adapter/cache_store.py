@@ -113,7 +113,7 @@ class JetFireInt4CacheStore:
         """Name the fused decode kernels know this store by, or None (split kernels / unsupported)."""
         if self.k_nbits not in (2, 3, 4) or self.v_nbits not in (2, 3, 4) or (self.k_asymmetric and self.k_nbits != 2):
             return None
-        if self.group_size == 128 or (self.group_size == 64 and 4 not in (self.k_nbits, self.v_nbits)):
+        if self.group_size == 128 or (self.group_size == 64 and self.k_nbits != 4):     # (INT4 keys: one scale per row)
             return f"a2v{self.v_nbits}" if self.k_asymmetric else f"k{self.k_nbits}v{self.v_nbits}"
         return None
 

@@ -7,7 +7,9 @@ int jf::launch_full_scan_a(int scheme, int G, int NG, const void* params, void* 
     return NG == 2 ? launch_full_by_group<JF_SCHEME_K3V2, 2>(G, params, stream)
                    : launch_full_by_group<JF_SCHEME_K3V2, 1>(G, params, stream);
   if (scheme == JF_SCHEME_K4V4) return launch_full_by_group<JF_SCHEME_K4V4, 1>(G, params, stream);
-  if (scheme == JF_SCHEME_K3V4) return launch_full_by_group<JF_SCHEME_K3V4, 1>(G, params, stream);
+  if (scheme == JF_SCHEME_K3V4)
+    return NG == 2 ? launch_full_by_group<JF_SCHEME_K3V4, 2>(G, params, stream)
+                   : launch_full_by_group<JF_SCHEME_K3V4, 1>(G, params, stream);
   if (scheme == JF_SCHEME_K4V2) return launch_full_by_group<JF_SCHEME_K4V2, 1>(G, params, stream);
   JF_CHECK_ARG(false, "fused_scan: scheme %d is not in this family", scheme);
   return JF_ERR_ARG;

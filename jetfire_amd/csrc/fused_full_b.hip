@@ -9,7 +9,9 @@ int jf::launch_full_scan_b(int scheme, int G, int NG, const void* params, void* 
   if (scheme == JF_SCHEME_K2V3)
     return NG == 2 ? launch_full_by_group<JF_SCHEME_K2V3, 2>(G, params, stream)
                    : launch_full_by_group<JF_SCHEME_K2V3, 1>(G, params, stream);
-  if (scheme == JF_SCHEME_K2V4) return launch_full_by_group<JF_SCHEME_K2V4, 1>(G, params, stream);
+  if (scheme == JF_SCHEME_K2V4)
+    return NG == 2 ? launch_full_by_group<JF_SCHEME_K2V4, 2>(G, params, stream)
+                   : launch_full_by_group<JF_SCHEME_K2V4, 1>(G, params, stream);
   JF_CHECK_ARG(false, "fused_scan: scheme %d is not in this family", scheme);
   return JF_ERR_ARG;
 }

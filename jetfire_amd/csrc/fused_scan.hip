@@ -27,7 +27,7 @@ extern "C" size_t jf_fused_workspace_bytes(int scheme, int B, int H_q, int H_kv,
   if (B <= 0 || H_q <= 0 || H_kv <= 0 || H_q % H_kv != 0 || max_S < 0 || top_k <= 0) return 256;
   // the split length depends on the group size only through the LDS budget; size for the worst case
   size_t worst = 0;
-  for (int ng = 1; ng <= 2; ++ng) {
+  for (int ng = 1; ng <= (scheme_any_group(scheme) ? 2 : 1); ++ng) {
     int L, ns, kc;
     fused_plan(scheme, ng, B, H_q, H_kv, max_S, top_k, &L, &ns, &kc);
     int parts, spp;

@@ -2082,6 +2082,7 @@ inline int lmax_dispatch(int scheme, int G, int NG) {
   JF_LMAX_ALL_G(JF_SCHEME_A2V2, 1); JF_LMAX_ALL_G(JF_SCHEME_A2V2, 2);
   JF_LMAX_ALL_G(JF_SCHEME_A2V3, 1); JF_LMAX_ALL_G(JF_SCHEME_A2V3, 2);
   JF_LMAX_ALL_G(JF_SCHEME_A2V4, 1);
+  JF_LMAX_ALL_G(JF_SCHEME_K3V4, 2); JF_LMAX_ALL_G(JF_SCHEME_K2V4, 2); JF_LMAX_ALL_G(JF_SCHEME_A2V4, 2);
 #undef JF_LMAX_ALL_G
 #undef JF_LMAX_CASE
   return 256;
@@ -2247,11 +2248,9 @@ inline bool known_scheme(int scheme) {
          scheme == JF_SCHEME_K2V2 || scheme == JF_SCHEME_K2V4 || scheme == JF_SCHEME_K2V3 || scheme == JF_SCHEME_K3V3 ||
          scheme == JF_SCHEME_K4V3 || scheme_has_zp(scheme);
 }
-// scale groups per row: the schemes without an INT4 side may use 64-channel groups
-inline bool scheme_any_group(int scheme) {
-  return scheme == JF_SCHEME_K3V2 || scheme == JF_SCHEME_K2V2 || scheme == JF_SCHEME_K2V3 || scheme == JF_SCHEME_K3V3 ||
-         scheme == JF_SCHEME_A2V2 || scheme == JF_SCHEME_A2V3;
-}
+// scale groups per row: every scheme but those with INT4 keys (int8-Q model: one key scale per row) may use
+// 64-channel groups
+inline bool scheme_any_group(int scheme) { return known_scheme(scheme) && scheme / 10 != 4; }
 inline int scheme_ng(int scheme, int group_size) { return scheme_any_group(scheme) ? D / group_size : 1; }
 
 
@@ -2272,7 +2271,7 @@ static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_
   JF_CHECK_ARG(known_scheme(scheme), "fused_scan: unknown scheme %d", scheme);
   JF_CHECK_ARG(MODE == FS_FULL || scheme == JF_SCHEME_K3V2 || scheme == JF_SCHEME_K4V4 ||
                    (MODE == FS_STAGE_A && (scheme == JF_SCHEME_K2V2 || scheme == JF_SCHEME_A2V2)) ||
-                   (MODE == FS_STAGE_B && scheme == JF_SCHEME_K3V3),
+                   (MODE == FS_STAGE_B && (scheme == JF_SCHEME_K3V3 || scheme == JF_SCHEME_K3V4)),
                "fused_scan: the stage-wise forms take the K3V2 or K4V4 side formats (Stage A also K2V2 and A2V2, Stage B also K3V3)");
   JF_CHECK_ARG(!(MODE == FS_FULL || MODE == FS_STAGE_A) || scheme_has_zp(scheme) == (k_zp != nullptr) || B == 0,
                "fused_scan: zero-points go with the asymmetric INT2 key formats, and only with them");
@@ -2366,7 +2365,9 @@ static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_
   } else if (scheme == JF_SCHEME_K4V4) {
     JF_FUSED_BY_G(JF_SCHEME_K4V4, 1)
   } else if constexpr (MODE == FS_STAGE_B) {
-    if (NGv == 2) JF_FUSED_BY_G(JF_SCHEME_K3V3, 2) else JF_FUSED_BY_G(JF_SCHEME_K3V3, 1)
+    if (scheme == JF_SCHEME_K3V4) {  // INT4 values with either group size (one group: the K4V4 instantiation)
+      if (NGv == 2) JF_FUSED_BY_G(JF_SCHEME_K3V4, 2) else JF_FUSED_BY_G(JF_SCHEME_K4V4, 1)
+    } else if (NGv == 2) JF_FUSED_BY_G(JF_SCHEME_K3V3, 2) else JF_FUSED_BY_G(JF_SCHEME_K3V3, 1)
   } else if (scheme == JF_SCHEME_K2V2) {  // (Stage A)
     if (NGv == 2) JF_FUSED_BY_G(JF_SCHEME_K2V2, 2) else JF_FUSED_BY_G(JF_SCHEME_K2V2, 1)
   } else {
@@ -2408,7 +2409,8 @@ static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_
     if (NGv == 2) JF_MERGE(3, 2);
     else JF_MERGE(3, 1);
   } else {
-    JF_MERGE(4, 1);
+    if (NGv == 2) JF_MERGE(4, 2);
+    else JF_MERGE(4, 1);
   }
 #undef JF_MERGE
   JF_CHECK_LAUNCH();

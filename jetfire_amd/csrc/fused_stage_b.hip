@@ -13,9 +13,10 @@ extern "C" int jf_stage_b_softmax_v(int value_format, int group_size, const floa
                                     const int64_t* topk_idx, int B, int H_q, int H_kv, int max_S, int max_blocks,
                                     int64_t num_slots, int block_size, int top_k, float* o_hat, float* o_old_unnorm,
                                     float* W, void* workspace, size_t workspace_bytes, void* stream) {
-  JF_CHECK_ARG(value_format == JF_SCHEME_K3V2 || value_format == JF_SCHEME_K3V3 || value_format == JF_SCHEME_K4V4,
-               "stage_b_softmax_v: value_format must be JF_SCHEME_K3V2 (INT2 values), JF_SCHEME_K3V3 (INT3 values) or "
-               "JF_SCHEME_K4V4 (INT4 values)");
+  JF_CHECK_ARG(value_format == JF_SCHEME_K3V2 || value_format == JF_SCHEME_K3V3 || value_format == JF_SCHEME_K4V4 ||
+                   value_format == JF_SCHEME_K3V4,
+               "stage_b_softmax_v: value_format must be JF_SCHEME_K3V2 (INT2 values), JF_SCHEME_K3V3 (INT3 values), "
+               "JF_SCHEME_K4V4 (INT4 values, group 128) or JF_SCHEME_K3V4 (INT4 values, group 64 or 128)");
   return fused_run<FS_STAGE_B>(value_format, group_size, nullptr, nullptr, nullptr, nullptr, v_data, v_scales, block_table,
                                seq_lens, B, H_q, H_kv, max_S, max_blocks, num_slots, block_size, 0.0f, top_k,
                                const_cast<int64_t*>(topk_idx), nullptr, o_hat, o_old_unnorm, W, nullptr, nullptr, nullptr,

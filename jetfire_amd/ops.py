@@ -481,9 +481,9 @@ def _softmax_v(scores, m, iz, v_data, v_scales, block_table, seq_lens, topk_idx,
         o_hat, o_old, W = outs
         for t in outs:
             _check(t.is_cuda and t.dtype == torch.float32 and t.is_contiguous(), "output buffers must be contiguous fp32")
-    if (not int8_tiles and m is None and nbits in (2, 3, 4) and (nbits != 4 or ng == 1) and vd.size(0) == H_kv
+    if (not int8_tiles and m is None and nbits in (2, 3, 4) and vd.size(0) == H_kv
             and _fast_shape(H_q, H_kv, block_size, max_S, vd.size(1), top_k if topk_idx is not None else None)):
-        fmt = {2: 32, 3: 33, 4: 44}[nbits]
+        fmt = {2: 32, 3: 33, 4: 44 if ng == 1 else 34}[nbits]      # (value side of the tag; 34: INT4 values, two groups)
         k_eff = int(top_k) if topk_idx is not None else 32
         ws = _workspace(dev, lib.jf_fused_workspace_bytes(fmt, B, H_q, H_kv, int(max_S), k_eff), "fused")
         _lib.check(lib.jf_stage_b_softmax_v(
@@ -600,8 +600,8 @@ def fused_attn_topk(scheme: str, q, k_data, k_scales, v_data, v_scales, block_ta
 
     The single-call contract is the one of the reference's int2_fused_attn_topk
     (jetfire_vllm/kernels/int2_fused_attn_topk.py:5-10) extended to INT3 / INT4 keys (INT4: the int8-Q scoring
-    model), symmetric INT2 keys, and INT2 / INT3 / INT4 values: "k{2,3,4}v{2,3,4}"; pairs without an INT4 side take
-    group 64 or 128, the others group 128.  "a2v{2,3,4}": asymmetric INT2 keys, whose zero-points come in `k_zp`
+    model), symmetric INT2 keys, and INT2 / INT3 / INT4 values: "k{2,3,4}v{2,3,4}"; pairs with INT4 keys take
+    group 128, the others group 64 or 128.  "a2v{2,3,4}": asymmetric INT2 keys, whose zero-points come in `k_zp`
     (shaped like k_scales), the reference's int2_asym_k_* kernel sets."""
     lib = _lib.load()
     scheme_id = FUSED_SCHEMES.get(scheme)

@@ -106,10 +106,14 @@ CASES = [
     ("a2v2", 4, 8, 2, 32, [0, 1, 9, 17], 32), ("a2v3", 1, 8, 2, 5000, [4987], 256), ("a2v4", 1, 8, 2, 5000, [4987], 1024),
     ("a2v2", 1, 4, 4, 300, None, 32), ("a2v4", 1, 4, 2, 300, None, 64), ("a2v2_g128", 1, 16, 1, 600, None, 64),
     ("a2v3", 1, 16, 1, 600, None, 64),
+    # INT4 values with 64-channel groups (keys other than INT4)
+    ("k3v4_g64", 2, 8, 2, 512, None, 64), ("k2v4_g64", 3, 32, 4, 512, [17, 257, 512], 256), ("a2v4_g64", 1, 8, 2, 5000, [4987], 256),
+    ("k3v4_g64", 1, 16, 1, 600, None, 64), ("k2v4_g64", 1, 4, 4, 300, None, 32), ("a2v4_g64", 1, 4, 2, 300, None, 64),
 ]
 SCHEME_GEOMETRY = {f"k{kb}v{vb}": (kb, vb, 128 if 4 in (kb, vb) else 64) for kb in (2, 3, 4) for vb in (2, 3, 4)}
 SCHEME_GEOMETRY.update({f"k{kb}v{vb}_g128": (kb, vb, 128) for kb in (2, 3) for vb in (2, 3)})
 # asymmetric INT2 keys
+SCHEME_GEOMETRY.update({"k3v4_g64": (3, 4, 64), "k2v4_g64": (2, 4, 64), "a2v4_g64": (2, 4, 64)})   # INT4 values, two scale groups
 SCHEME_GEOMETRY.update({"a2v2": (2, 2, 64), "a2v2_g128": (2, 2, 128), "a2v3": (2, 3, 64), "a2v3_g128": (2, 3, 128),
                         "a2v4": (2, 4, 128)})
 

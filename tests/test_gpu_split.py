@@ -321,11 +321,11 @@ def test_unsupported_top_k_raises():
 # ------------------------------------------------------------------ Stage B + merge
 
 
-@pytest.mark.parametrize("scheme", ("k3v2", "k4v4", "k3v2_g128", "k3v3", "k3v3_g128"))
+@pytest.mark.parametrize("scheme", ("k3v2", "k4v4", "k3v2_g128", "k3v3", "k3v3_g128", "k3v4_g64"))
 @pytest.mark.parametrize("B,Hq,Hkv,lens", [(2, 8, 2, None), (3, 32, 4, [17, 257, 512]), (4, 8, 2, [0, 1, 9, 17])])
 def test_stage_b_outputs(scheme, B, Hq, Hkv, lens, impl):
     kb, vb, gs = {"k3v2": (3, 2, 64), "k4v4": (4, 4, 128), "k3v2_g128": (3, 2, 128), "k3v3": (3, 3, 64),
-                  "k3v3_g128": (3, 3, 128)}[scheme]
+                  "k3v3_g128": (3, 3, 128), "k3v4_g64": (3, 4, 64)}[scheme]
     S = 512 if lens is None or max(lens) > 32 else 32
     c = make_case(31 + B, B, Hq, Hkv, S, kb, vb, gs, lens=lens)
     d = to_device(c)
@@ -358,7 +358,7 @@ def test_stage_b_outputs(scheme, B, Hq, Hkv, lens, impl):
         _, q_old, q_W = O.softmax_v(ref_sc, c["vd"], c["vs"], c["bt"], c["lens"], h_idx, S, Hq, Hkv, 16, vb, gs)
         np.testing.assert_allclose(p_old.cpu().numpy(), q_old, atol=3e-6, rtol=3e-6)
         np.testing.assert_allclose(p_W.cpu().numpy(), q_W, atol=3e-6, rtol=3e-6)
-    if vb == 4:                                                   # the int8-weight variant, handed Stage-A statistics
+    if vb == 4 and gs == 128:                                     # the int8-weight variant, handed Stage-A statistics
         m, iz = O.softmax_stats(ref_sc, c["lens"], S)
         o2 = o.int8tc_softmax_v_with_pre_corr_reg_stats(sc_t, torch.from_numpy(m).cuda(), torch.from_numpy(iz).cuda(),
                                                         d["vd"], d["vs"], d["bt"], d["lens"], idx_t, S, Hq, Hkv, 16, K)
