@@ -246,7 +246,7 @@ int jf_fused_scan_topk_asym(int scheme, int group_size,
 
 /* Stage A alone and Stage B alone on the kernels of the fused step, for callers that keep the reference's two-call
  * structure (jetfire_vllm/adapter/decode_path.py:2081-2131 then :2804-2935): the same results as the split entry
- * points above for the shapes the fused step supports (head_dim 128, block_size 16, H_q/H_kv in {1,2,4,8,16},
+ * points above for the shapes the fused step supports (head_dim 128, block_size 16, H_q/H_kv from 1 to 16,
  * top_k <= 2048, num_slots <= 2^26), at a fraction of their time.  workspace: jf_fused_workspace_bytes(format, ...).
  *
  * jf_stage_a_topk replaces int3_qk_scores / int3_qk_scores_topk (jetfire_vllm/csrc/int3_qk_scores.cu:640-655;

@@ -104,6 +104,7 @@ struct FusedParams {
   const int64_t* block_table;
   const int32_t* seq_lens;
   int B, H_q, H_kv, max_S, max_blocks;
+  int g_act;  // query heads per kv-head (H_q / H_kv); the kernel's G is this rounded up to 1, 2, 4, 8 or 16
   int64_t num_slots;
   float attn_scale;
   int top_k;
@@ -293,7 +294,10 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   const int s_cover = min(s0 + L, p.max_S);
   const int n_cover = max(0, s_cover - s0);
   const int64_t* bt = p.block_table + (size_t)b * p.max_blocks;
-  const size_t head0 = (size_t)b * p.H_q + (size_t)hkv * G;
+  // GA query heads belong to this kv-head; the template's G may be larger (the next of 1, 2, 4, 8, 16): the heads
+  // past GA are zero query rows whose arithmetic runs along and whose results are never stored
+  const int GA = p.g_act;
+  const size_t head0 = (size_t)b * p.H_q + (size_t)hkv * GA;
   const size_t part_base = head0 * p.n_splits + split;  // + h * n_splits
   const uint8_t* kbase = p.k_data + (size_t)hkv * p.num_slots * KP;
   const uint8_t* vbase = p.v_data + (size_t)hkv * p.num_slots * VP;
@@ -313,22 +317,22 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
 #pragma unroll
   for (int it = 0; it < QPT; ++it) {
     const int i = it * NT + tid;
-    qv[it] = (i < G * D) ? bf16_to_f32(p.q[head0 * D + i]) : 0.f;
+    qv[it] = (i < GA * D) ? bf16_to_f32(p.q[head0 * D + i]) : 0.f;
   }
 
   if (n == 0) {  // nothing valid in this split: padding scores, empty partials
     if (p.scores)
-      for (int i = tid; i < G * n_cover; i += NT)
+      for (int i = tid; i < GA * n_cover; i += NT)
         p.scores[(head0 + i / n_cover) * (size_t)p.max_S + s0 + (i % n_cover)] = -INFINITY;
     if constexpr (MODE == FS_STAGE_A)
       if (p.scores_only) return;
-    for (int i = tid; i < G * D; i += NT) p.part_o[(part_base + (size_t)(i / D) * p.n_splits) * D + (i % D)] = 0.f;
-    if (tid < G) {
+    for (int i = tid; i < GA * D; i += NT) p.part_o[(part_base + (size_t)(i / D) * p.n_splits) * D + (i % D)] = 0.f;
+    if (tid < GA) {
       p.part_m[part_base + (size_t)tid * p.n_splits] = -INFINITY;
       p.part_l[part_base + (size_t)tid * p.n_splits] = 0.f;
       p.cand_cnt[part_base + (size_t)tid * p.n_splits] = 0;
     }
-    for (int i = tid; i < G * p.Kc; i += NT)  // unused candidate slots hold key 0 (no score maps to it)
+    for (int i = tid; i < GA * p.Kc; i += NT)  // unused candidate slots hold key 0 (no score maps to it)
       p.cand_key[(part_base + (size_t)(i / p.Kc) * p.n_splits) * p.Kc + (i % p.Kc)] = 0u;
     return;
   }
@@ -552,7 +556,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     // positions past the sequence (and the rest of the last chunk) become -inf
 #pragma unroll
     for (int h = 0; h < G; ++h) {
-      const float* srow = p.scores_in + (head0 + h) * (size_t)p.max_S + s0;
+      const float* srow = p.scores_in + (head0 + min(h, GA - 1)) * (size_t)p.max_S + s0;  // (past GA: a copy, unused)
       float mx = -INFINITY, mn = INFINITY;
       for (int t = tid; t < nch * 64; t += NT) {
         const float v = (t < n) ? srow[t] : -INFINITY;
@@ -937,7 +941,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   lds_barrier();  // phase A complete: the query constants are dead, their space becomes the histograms
   if (clk && tid == 0) { clk[8] = clock64(); clk[5] = (long long)tmax_sh; }
   if (p.scores)  // validation output
-    for (int i = tid; i < G * n_cover; i += NT) {
+    for (int i = tid; i < GA * n_cover; i += NT) {
       const int h = i / n_cover, t = i - h * n_cover;
       p.scores[(head0 + h) * (size_t)p.max_S + s0 + t] = sc[h * L + t];
     }
@@ -1203,7 +1207,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     for (int i = tid; i < 4 * D; i += NT) {
       const int col = i & 15, hh = (i >> 4) & 3, tile = i >> 6;
       const int h = set * 4 + hh;
-      if (h >= G) continue;
+      if (h >= GA) continue;
       int d;
       if (V2) {
         const int e = ((col & 1) ? 0 : 2) + (tile & 1);
@@ -1243,7 +1247,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
 #pragma unroll
     for (int set = 0; set < NSET; ++set) add_acc(set);
   }
-  for (int h = wave; HAS_TOPK && h < G; h += NW) {
+  for (int h = wave; HAS_TOPK && h < GA; h += NW) {
     const int* h0 = hist + h * (SEG * 256) / (Lds::H16 ? 2 : 1);
     // lane l owns buckets 4l .. 4l+3 (ascending bucket = descending score) of every segment's histogram
     int cs[SEG][4], c[4], mine = 0;
@@ -1309,6 +1313,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   if (clk && tid == 0) clk[6] = clock64();
   for (int hs = wave; HAS_TOPK && hs < G * SEG; hs += NW) {
     const int h = hs / SEG, seg = hs % SEG;
+    if (h >= GA) continue;
     const float* srow = sc + h * L;
     uint32_t* ck = p.cand_key + (part_base + (size_t)h * p.n_splits) * Kcap;
     int32_t* ci = p.cand_idx + (part_base + (size_t)h * p.n_splits) * Kcap;
@@ -1443,7 +1448,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
 #pragma unroll
   for (int set = 0; set < NSET; ++set)
     if constexpr (HAS_V) combine(set);
-  if (tid < G) {
+  if (tid < GA) {
     p.part_m[part_base + (size_t)tid * p.n_splits] = m_sh[tid];
     p.part_l[part_base + (size_t)tid * p.n_splits] = lfin;
   }
@@ -2123,9 +2128,11 @@ inline double merge_plan(int rows, int ns, int kc, int top_k, int* parts_out, in
   return best;
 }
 
+inline int padded_group(int g) { return g <= 2 ? g : (g <= 4 ? 4 : (g <= 8 ? 8 : 16)); }
+
 inline void fused_plan(int scheme, int NG, int B, int H_q, int H_kv, int max_S, int top_k, int* L_out, int* ns_out,
                        int* kc_out) {
-  const int G = H_q / H_kv;
+  const int G = padded_group(H_q / H_kv);
   const int units = B * H_kv > 0 ? B * H_kv : 1;
   const int rows = B * H_q > 0 ? B * H_q : 1;
   // One scan workgroup is resident per CU (256 CUs).  Among the split lengths that fit LDS pick the one with
@@ -2279,8 +2286,9 @@ static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_
   JF_CHECK_ARG(MODE != FS_TOPK || scheme == JF_SCHEME_K4V4, "fused_scan: the selection-only form uses the K4V4 layout");
   JF_CHECK_ARG((blend_o_new == nullptr) == (blend_out == nullptr), "fused_scan: o_new and out go together");
   JF_CHECK_ARG(B >= 0 && H_q > 0 && H_kv > 0 && max_S >= 0 && H_q % H_kv == 0, "fused_scan: bad shape");
-  const int G = H_q / H_kv;
-  JF_CHECK_ARG(G == 1 || G == 2 || G == 4 || G == 8 || G == 16, "fused_scan: GQA group %d not in {1,2,4,8,16}", G);
+  const int g_act = H_q / H_kv;
+  JF_CHECK_ARG(g_act >= 1 && g_act <= 16, "fused_scan: GQA group %d not in 1..16", g_act);
+  const int G = padded_group(g_act);  // the kernels come for 1, 2, 4, 8 and 16 query heads per kv-head
   JF_CHECK_ARG(block_size == 16, "fused_scan only supports block_size=16");
   JF_CHECK_ARG(group_size == 64 || group_size == 128, "fused_scan: group_size must be 64 or 128 (got %d)", group_size);
   JF_CHECK_ARG(scheme_any_group(scheme) || group_size == 128,
@@ -2314,6 +2322,7 @@ static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_
   p.q = q; p.k_data = k_data; p.k_scales = k_scales; p.k_zp = k_zp; p.v_data = v_data; p.v_scales = v_scales;
   p.block_table = block_table; p.seq_lens = seq_lens;
   p.B = B; p.H_q = H_q; p.H_kv = H_kv; p.max_S = max_S; p.max_blocks = max_blocks; p.num_slots = num_slots;
+  p.g_act = g_act;
   p.attn_scale = attn_scale; p.top_k = top_k;
   fused_plan(scheme, NGv, B, H_q, H_kv, max_S, top_k, &p.L, &p.n_splits, &p.Kc);
   JF_CHECK_ARG(p.n_splits <= MG_MAX_SPLITS, "fused_scan: too many splits (%d > %d)", p.n_splits, MG_MAX_SPLITS);

@@ -19,19 +19,20 @@ template <int G, int NG>
 __global__ __launch_bounds__(QK_THREADS) void int3_qk_scores_kernel(
     const uint16_t* __restrict__ q, const uint8_t* __restrict__ k_data, const uint16_t* __restrict__ k_scales,
     const int64_t* __restrict__ block_table, const int32_t* __restrict__ seq_lens, float* __restrict__ scores,
-    int H_q, int H_kv, int max_S, int max_blocks, int64_t num_slots, int bs, float attn_scale) {
+    int H_q, int H_kv, int max_S, int max_blocks, int64_t num_slots, int bs, float attn_scale, int ga) {
   __shared__ float qs[G][D];
   const int b = blockIdx.z, hkv = blockIdx.y, tid = threadIdx.x;
-  for (int i = tid; i < G * D; i += QK_THREADS)
-    qs[i / D][i % D] = bf16_to_f32(q[((size_t)b * H_q + (size_t)hkv * G + i / D) * D + i % D]);
+  for (int i = tid; i < G * D; i += QK_THREADS)  // (rows past ga: zero query rows whose scores are never stored)
+    qs[i / D][i % D] = (i < ga * D) ? bf16_to_f32(q[((size_t)b * H_q + (size_t)hkv * ga + i / D) * D + i % D]) : 0.f;
   __syncthreads();
   const int s = blockIdx.x * QK_THREADS + tid;
   if (s >= max_S) return;
-  float* out = scores + ((size_t)b * H_q + (size_t)hkv * G) * max_S + s;
+  float* out = scores + ((size_t)b * H_q + (size_t)hkv * ga) * max_S + s;
   const int S = seq_lens[b];
   if (s >= S) {
 #pragma unroll
-    for (int g = 0; g < G; ++g) out[(size_t)g * max_S] = -INFINITY;
+    for (int g = 0; g < G; ++g)
+      if (g < ga) out[(size_t)g * max_S] = -INFINITY;
     return;
   }
   const int64_t slot = block_table[(size_t)b * max_blocks + s / bs] * bs + s % bs;
@@ -63,7 +64,8 @@ __global__ __launch_bounds__(QK_THREADS) void int3_qk_scores_kernel(
       for (int j = 0; j < 8; ++j) acc[g] = __builtin_fmaf(qs[g][gi * 8 + j], kv[j], acc[g]);
   }
 #pragma unroll
-  for (int g = 0; g < G; ++g) out[(size_t)g * max_S] = acc[g] * attn_scale;
+  for (int g = 0; g < G; ++g)
+    if (g < ga) out[(size_t)g * max_S] = acc[g] * attn_scale;
 }
 
 // INT2 / INT4 keys with the same bf16 model (jetfire_vllm/csrc/int2_qk_scores.cu:66-79, int4_qk_scores.cu:68-80):
@@ -73,21 +75,22 @@ template <int KBITS, int G, int NG>
 __global__ __launch_bounds__(QK_THREADS) void intn_qk_scores_kernel(
     const uint16_t* __restrict__ q, const uint8_t* __restrict__ k_data, const uint16_t* __restrict__ k_scales,
     const uint16_t* __restrict__ k_zp, const int64_t* __restrict__ block_table, const int32_t* __restrict__ seq_lens, float* __restrict__ scores,
-    int H_q, int H_kv, int max_S, int max_blocks, int64_t num_slots, int bs, float attn_scale) {
+    int H_q, int H_kv, int max_S, int max_blocks, int64_t num_slots, int bs, float attn_scale, int ga) {
   static_assert(KBITS == 2 || KBITS == 4, "planar INT3 rows have their own kernel");
   constexpr int P = D * KBITS / 8, NDW = P / 4, OFF = 1 << (KBITS - 1);
   __shared__ float qs[G][D];
   const int b = blockIdx.z, hkv = blockIdx.y, tid = threadIdx.x;
-  for (int i = tid; i < G * D; i += QK_THREADS)
-    qs[i / D][i % D] = bf16_to_f32(q[((size_t)b * H_q + (size_t)hkv * G + i / D) * D + i % D]);
+  for (int i = tid; i < G * D; i += QK_THREADS)  // (rows past ga: zero query rows whose scores are never stored)
+    qs[i / D][i % D] = (i < ga * D) ? bf16_to_f32(q[((size_t)b * H_q + (size_t)hkv * ga + i / D) * D + i % D]) : 0.f;
   __syncthreads();
   const int s = blockIdx.x * QK_THREADS + tid;
   if (s >= max_S) return;
-  float* out = scores + ((size_t)b * H_q + (size_t)hkv * G) * max_S + s;
+  float* out = scores + ((size_t)b * H_q + (size_t)hkv * ga) * max_S + s;
   const int S = seq_lens[b];
   if (s >= S) {
 #pragma unroll
-    for (int g = 0; g < G; ++g) out[(size_t)g * max_S] = -INFINITY;
+    for (int g = 0; g < G; ++g)
+      if (g < ga) out[(size_t)g * max_S] = -INFINITY;
     return;
   }
   const int64_t slot = block_table[(size_t)b * max_blocks + s / bs] * bs + s % bs;
@@ -122,7 +125,8 @@ __global__ __launch_bounds__(QK_THREADS) void intn_qk_scores_kernel(
       for (int j = 0; j < 8; ++j) acc[g] = __builtin_fmaf(qs[g][gi * 8 + j], kv[j], acc[g]);
   }
 #pragma unroll
-  for (int g = 0; g < G; ++g) out[(size_t)g * max_S] = acc[g] * attn_scale;
+  for (int g = 0; g < G; ++g)
+    if (g < ga) out[(size_t)g * max_S] = acc[g] * attn_scale;
 }
 
 // q quantisation shared by the INT4 kernels: qi packed so that dword j of `qe` holds channels
@@ -137,12 +141,12 @@ struct QInt8 {
 
 template <int G>
 __device__ inline void quantize_query_int8(const uint16_t* __restrict__ qrow0, QInt8<G>& sh, float* scratch, int tid,
-                                           int nthreads) {
-  // scratch: G*4 floats
+                                           int nthreads, int ga) {
+  // scratch: G*4 floats.  Rows past ga (the group padded to the kernel's G) are zero rows: nothing is read for them.
   for (int i = tid; i < G * 4; i += nthreads) {
     const int g = i >> 2, kk = i & 3;
     float amax = 0.0f;
-    for (int d = 0; d < 32; ++d) amax = fmaxf(amax, fabsf(bf16_to_f32(qrow0[(size_t)g * D + kk * 32 + d])));
+    for (int d = 0; d < 32 && g < ga; ++d) amax = fmaxf(amax, fabsf(bf16_to_f32(qrow0[(size_t)g * D + kk * 32 + d])));
     const float s = fmaxf(amax / 127.0f, 1e-12f);
     sh.qs[g][kk] = s;
     scratch[i] = 1.0f / s;
@@ -154,7 +158,7 @@ __device__ inline void quantize_query_int8(const uint16_t* __restrict__ qrow0, Q
     int v[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      const float f = bf16_to_f32(qrow0[(size_t)g * D + 8 * j + e]);
+      const float f = (g < ga) ? bf16_to_f32(qrow0[(size_t)g * D + 8 * j + e]) : 0.f;
       v[e] = max(-128, min(127, (int)rintf(f * inv)));
     }
     sh.qe[g][j] = (v[0] & 255) | ((v[2] & 255) << 8) | ((v[4] & 255) << 16) | ((v[6] & 255) << 24);
@@ -178,18 +182,19 @@ template <int G>
 __global__ __launch_bounds__(QK_THREADS) void int8tc_qk_scores_kernel(
     const uint16_t* __restrict__ q, const uint8_t* __restrict__ k_data, const uint16_t* __restrict__ k_scales,
     const int64_t* __restrict__ block_table, const int32_t* __restrict__ seq_lens, float* __restrict__ scores,
-    int H_q, int H_kv, int max_S, int max_blocks, int64_t num_slots, int bs, float attn_scale) {
+    int H_q, int H_kv, int max_S, int max_blocks, int64_t num_slots, int bs, float attn_scale, int ga) {
   __shared__ QInt8<G> sh;
   __shared__ float scratch[G * 4];
   const int b = blockIdx.z, hkv = blockIdx.y, tid = threadIdx.x;
-  quantize_query_int8<G>(q + ((size_t)b * H_q + (size_t)hkv * G) * D, sh, scratch, tid, QK_THREADS);
+  quantize_query_int8<G>(q + ((size_t)b * H_q + (size_t)hkv * ga) * D, sh, scratch, tid, QK_THREADS, ga);
   const int s = blockIdx.x * QK_THREADS + tid;
   if (s >= max_S) return;
-  float* out = scores + ((size_t)b * H_q + (size_t)hkv * G) * max_S + s;
+  float* out = scores + ((size_t)b * H_q + (size_t)hkv * ga) * max_S + s;
   const int S = seq_lens[b];
   if (s >= S) {
 #pragma unroll
-    for (int g = 0; g < G; ++g) out[(size_t)g * max_S] = -INFINITY;
+    for (int g = 0; g < G; ++g)
+      if (g < ga) out[(size_t)g * max_S] = -INFINITY;
     return;
   }
   const int64_t slot = block_table[(size_t)b * max_blocks + s / bs] * bs + s % bs;
@@ -216,7 +221,7 @@ __global__ __launch_bounds__(QK_THREADS) void int8tc_qk_scores_kernel(
       acc -= sh.sum8[g][kk];
       sacc = (kk == 0) ? ((float)acc * sh.qs[g][0]) : __builtin_fmaf((float)acc, sh.qs[g][kk], sacc);
     }
-    out[(size_t)g * max_S] = __fmul_rn(__fmul_rn(sacc, ks), attn_scale);
+    if (g < ga) out[(size_t)g * max_S] = __fmul_rn(__fmul_rn(sacc, ks), attn_scale);
   }
 }
 
@@ -225,7 +230,7 @@ int check_stage_a(const char* name, const void* q, const void* kd, const void* k
   JF_CHECK_ARG(B >= 0 && H_q > 0 && H_kv > 0 && max_S >= 0, "%s: bad shape", name);
   JF_CHECK_ARG(H_q % H_kv == 0, "%s: H_q must be divisible by H_kv", name);
   const int G = H_q / H_kv;
-  JF_CHECK_ARG(G == 1 || G == 2 || G == 4 || G == 8 || G == 16, "%s: GQA group %d not in {1,2,4,8,16}", name, G);
+  JF_CHECK_ARG(G >= 1 && G <= 16, "%s: GQA group %d not in 1..16", name, G);
   JF_CHECK_ARG(bs > 0 && (int64_t)max_blocks * bs >= max_S, "%s: block_table (%d blocks of %d) does not cover max_S=%d",
                name, max_blocks, bs, max_S);
   JF_CHECK_ARG(num_slots > 0, "%s: num_slots must be positive", name);
@@ -240,8 +245,10 @@ int check_stage_a(const char* name, const void* q, const void* kd, const void* k
 
 using namespace jf;
 
+// The kernels come for 1, 2, 4, 8 and 16 query heads per kv-head; other group sizes run the next larger one with
+// the actual size as an argument (zero query rows past it, nothing stored for them).
 #define JF_DISPATCH_G(G, ...)                      \
-  switch (G) {                                     \
+  switch ((G) <= 2 ? (G) : ((G) <= 4 ? 4 : ((G) <= 8 ? 8 : 16))) {  \
     case 1: { constexpr int GG = 1; __VA_ARGS__; } break;  \
     case 2: { constexpr int GG = 2; __VA_ARGS__; } break;  \
     case 4: { constexpr int GG = 4; __VA_ARGS__; } break;  \
@@ -265,10 +272,10 @@ extern "C" int jf_int3_qk_scores(const uint16_t* q, const uint8_t* k_data, const
   JF_DISPATCH_G(G, {
     if (n_scale_groups == 1)
       hipLaunchKernelGGL((int3_qk_scores_kernel<GG, 1>), grid, block, 0, st, q, k_data, k_scales, block_table, seq_lens,
-                         scores, H_q, H_kv, max_S, max_blocks, num_slots, block_size, attn_scale);
+                         scores, H_q, H_kv, max_S, max_blocks, num_slots, block_size, attn_scale, G);
     else
       hipLaunchKernelGGL((int3_qk_scores_kernel<GG, 2>), grid, block, 0, st, q, k_data, k_scales, block_table, seq_lens,
-                         scores, H_q, H_kv, max_S, max_blocks, num_slots, block_size, attn_scale);
+                         scores, H_q, H_kv, max_S, max_blocks, num_slots, block_size, attn_scale, G);
   });
   JF_CHECK_LAUNCH();
   return JF_OK;
@@ -294,7 +301,7 @@ extern "C" int jf_intn_qk_scores(int k_nbits, const uint16_t* q, const uint8_t* 
   const int G = H_q / H_kv;
 #define JF_INTN_LAUNCH(KB, NGV)                                                                                        \
   hipLaunchKernelGGL((intn_qk_scores_kernel<KB, GG, NGV>), grid, block, 0, st, q, k_data, k_scales, k_zp, block_table, \
-                     seq_lens, scores, H_q, H_kv, max_S, max_blocks, num_slots, block_size, attn_scale)
+                     seq_lens, scores, H_q, H_kv, max_S, max_blocks, num_slots, block_size, attn_scale, G)
   JF_DISPATCH_G(G, {
     if (k_nbits == 2) {
       if (n_scale_groups == 1) JF_INTN_LAUNCH(2, 1); else JF_INTN_LAUNCH(2, 2);
@@ -320,7 +327,7 @@ extern "C" int jf_int8tc_qk_scores(const uint16_t* q, const uint8_t* k_data, con
   const int G = H_q / H_kv;
   JF_DISPATCH_G(G, {
     hipLaunchKernelGGL((int8tc_qk_scores_kernel<GG>), grid, block, 0, st, q, k_data, k_scales, block_table, seq_lens,
-                       scores, H_q, H_kv, max_S, max_blocks, num_slots, block_size, attn_scale);
+                       scores, H_q, H_kv, max_S, max_blocks, num_slots, block_size, attn_scale, G);
   });
   JF_CHECK_LAUNCH();
   return JF_OK;

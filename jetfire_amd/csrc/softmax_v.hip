@@ -70,7 +70,8 @@ __global__ __launch_bounds__(SV_THREADS) void weighted_v_split_kernel(
     const float* __restrict__ scores, const float* __restrict__ softmax_m, const float* __restrict__ softmax_inv_z,
     const uint8_t* __restrict__ v_data, const uint16_t* __restrict__ v_scales, const int64_t* __restrict__ block_table,
     const int32_t* __restrict__ seq_lens, float* __restrict__ partial, int H_q, int H_kv, int max_S, int max_blocks,
-    int64_t num_slots, int chunk, int n_splits) {
+    int64_t num_slots, int chunk, int n_splits, int ga) {
+  // ga: the query heads that belong to a kv-head; G is ga rounded up to a kernel size, the heads past ga carry no weight
   constexpr int P = D * NBITS / 8;
   __shared__ __align__(16) uint8_t vbuf[BS * P];
   __shared__ float wsbuf[G][BS][NG];
@@ -98,12 +99,13 @@ __global__ __launch_bounds__(SV_THREADS) void weighted_v_split_kernel(
     for (int i = tid; i < G * BS; i += SV_THREADS) {
       const int g = i / BS, j = i % BS;
       const int p = p0 + j;
-      const size_t bh = (size_t)b * H_q + (size_t)hkv * G + g;
+      const size_t bh = (size_t)b * H_q + (size_t)hkv * ga + g;
+      const bool live = p < s1 && g < ga;
       float w = 0.0f;
-      if (p < s1) w = __expf(scores[bh * (size_t)max_S + p] - softmax_m[bh]) * softmax_inv_z[bh];
+      if (live) w = __expf(scores[bh * (size_t)max_S + p] - softmax_m[bh]) * softmax_inv_z[bh];
 #pragma unroll
       for (int k = 0; k < NG; ++k)
-        wsbuf[g][j][k] = (p < s1) ? w * bf16_to_f32(sbase[(size_t)(base_slot + j) * NG + k]) : 0.0f;
+        wsbuf[g][j][k] = live ? w * bf16_to_f32(sbase[(size_t)(base_slot + j) * NG + k]) : 0.0f;
     }
     __syncthreads();
 #pragma unroll
@@ -115,7 +117,7 @@ __global__ __launch_bounds__(SV_THREADS) void weighted_v_split_kernel(
   }
 #pragma unroll
   for (int g = 0; g < G; ++g)
-    partial[(((size_t)b * H_q + (size_t)hkv * G + g) * n_splits + split) * D + tid] = acc[g];
+    if (g < ga) partial[(((size_t)b * H_q + (size_t)hkv * ga + g) * n_splits + split) * D + tid] = acc[g];
 }
 
 // INT4 values with int8-quantised weights, the arithmetic of the reference's register-MMA Stage B
@@ -138,7 +140,7 @@ __global__ __launch_bounds__(SV_THREADS) void tile_quantised_v_split_kernel(
     const float* __restrict__ scores, const float* __restrict__ softmax_m, const float* __restrict__ softmax_inv_z,
     const uint8_t* __restrict__ v_data, const uint16_t* __restrict__ v_scales, const int64_t* __restrict__ block_table,
     const int32_t* __restrict__ seq_lens, float* __restrict__ partial, int H_q, int H_kv, int max_S, int max_blocks,
-    int64_t num_slots, int sub_count) {
+    int64_t num_slots, int sub_count, int ga) {
   constexpr int P = D / 2;
   __shared__ __align__(16) uint8_t vbuf[TQ_TILE * P];
   __shared__ int pq[G][TQ_TILE];
@@ -181,11 +183,11 @@ __global__ __launch_bounds__(SV_THREADS) void tile_quantised_v_split_kernel(
       }
     }
     for (int g = q32; g < G; g += SV_THREADS / 32) {
-      const size_t bh = (size_t)b * H_q + (size_t)hkv * G + g;
+      const size_t bh = (size_t)b * H_q + (size_t)hkv * ga + g;
       const int pos = t0 + l32;
       const int64_t bs = base_slot[l32 / BS];
       float pv = 0.0f;
-      if (pos >= s_start && pos < s_end && bs >= 0) {
+      if (pos >= s_start && pos < s_end && bs >= 0 && g < ga) {
         const float pr = __expf(scores[bh * (size_t)max_S + pos] - softmax_m[bh]) * softmax_inv_z[bh];
         pv = pr * bf16_to_f32(sbase[bs + (l32 % BS)]);
       }
@@ -214,7 +216,8 @@ __global__ __launch_bounds__(SV_THREADS) void tile_quantised_v_split_kernel(
   }
 #pragma unroll
   for (int g = 0; g < G; ++g)
-    partial[(((size_t)b * H_q + (size_t)hkv * G + g) * (TQ_SPLITS * sub_count) + blockIdx.x) * D + tid] = acc[g];
+    if (g < ga)
+      partial[(((size_t)b * H_q + (size_t)hkv * ga + g) * (TQ_SPLITS * sub_count) + blockIdx.x) * D + tid] = acc[g];
 }
 
 // grid (B, H_q); adds split partials in order, then the top-k pre-correction.
@@ -315,7 +318,7 @@ extern "C" int jf_softmax_v_pre_corr(const float* scores, const float* softmax_m
                                      void* workspace, size_t workspace_bytes, void* stream) {
   JF_CHECK_ARG(B >= 0 && H_q > 0 && H_kv > 0 && max_S >= 0 && H_q % H_kv == 0, "softmax_v: bad shape");
   const int G = H_q / H_kv;
-  JF_CHECK_ARG(G == 1 || G == 2 || G == 4 || G == 8 || G == 16, "softmax_v: GQA group %d not in {1,2,4,8,16}", G);
+  JF_CHECK_ARG(G >= 1 && G <= 16, "softmax_v: GQA group %d not in 1..16", G);
   JF_CHECK_ARG(block_size == 16, "wvs2 only supports block_size=16");
   JF_CHECK_ARG(v_nbits == 2 || v_nbits == 3 || v_nbits == 4, "softmax_v: v_nbits must be 2, 3 or 4 (got %d)", v_nbits);
   JF_CHECK_ARG(n_scale_groups == 1 || n_scale_groups == 2, "wvs2 requires num_groups=1 or 2 (got %d)", n_scale_groups);
@@ -346,7 +349,7 @@ extern "C" int jf_softmax_v_pre_corr(const float* scores, const float* softmax_m
   JF_DISPATCH_G2(G, {                                                                                                    \
     hipLaunchKernelGGL((weighted_v_split_kernel<NB, GG, NGC>), grid, block, 0, st, scores, softmax_m, softmax_inv_z,     \
                        v_data, v_scales, block_table, seq_lens, partial, H_q, H_kv, max_S, max_blocks, num_slots, chunk, \
-                       n_splits);                                                                                        \
+                       n_splits, G);                                                                                     \
   });                                                                                                                    \
   JF_CHECK_LAUNCH();                                                                                                     \
   hipLaunchKernelGGL((combine_precorr_kernel<NB, NGC>), dim3(B, H_q), block, 0, st, partial, scores, softmax_m,          \
@@ -354,7 +357,7 @@ extern "C" int jf_softmax_v_pre_corr(const float* scores, const float* softmax_m
                      max_S, max_blocks, num_slots, n_splits, top_k);                                                     \
   JF_CHECK_LAUNCH();
 #define JF_DISPATCH_G2(G, ...)                               \
-  switch (G) {                                               \
+  switch ((G) <= 2 ? (G) : ((G) <= 4 ? 4 : ((G) <= 8 ? 8 : 16))) {  /* the next kernel size; the kernels take G itself too */ \
     case 1: { constexpr int GG = 1; __VA_ARGS__; } break;    \
     case 2: { constexpr int GG = 2; __VA_ARGS__; } break;    \
     case 4: { constexpr int GG = 4; __VA_ARGS__; } break;    \
@@ -378,7 +381,7 @@ extern "C" int jf_softmax_v_int8_tiles(const float* scores, const float* softmax
                                        size_t workspace_bytes, void* stream) {
   JF_CHECK_ARG(B >= 0 && H_q > 0 && H_kv > 0 && max_S >= 0 && H_q % H_kv == 0, "int8tc_softmax_v: bad shape");
   const int G = H_q / H_kv;
-  JF_CHECK_ARG(G == 1 || G == 2 || G == 4 || G == 8 || G == 16, "int8tc_softmax_v requires H_q/H_kv in {1,2,4,8,16} (got %d)", G);
+  JF_CHECK_ARG(G >= 1 && G <= 16, "int8tc_softmax_v requires H_q/H_kv in 1..16 (got %d)", G);
   JF_CHECK_ARG(block_size == 16, "int8tc_softmax_v only supports block_size=16");
   JF_CHECK_ARG((int64_t)max_blocks * block_size >= max_S, "int8tc_softmax_v: block_table does not cover max_S");
   JF_CHECK_ARG(topk_idx == nullptr || top_k > 0, "int8tc_softmax_v: top_k must be positive");
@@ -400,7 +403,7 @@ extern "C" int jf_softmax_v_int8_tiles(const float* scores, const float* softmax
   dim3 grid(TQ_SPLITS * sub_count, H_kv, B), block(SV_THREADS);
   JF_DISPATCH_G2(G, {
     hipLaunchKernelGGL((tile_quantised_v_split_kernel<GG>), grid, block, 0, st, scores, softmax_m, softmax_inv_z, v_data,
-                       v_scales, block_table, seq_lens, partial, H_q, H_kv, max_S, max_blocks, num_slots, sub_count);
+                       v_scales, block_table, seq_lens, partial, H_q, H_kv, max_S, max_blocks, num_slots, sub_count, G);
   });
   JF_CHECK_LAUNCH();
   // the pre-correction terms run on the merge kernel of the fused step where its limits allow (the same

@@ -228,7 +228,7 @@ def get_split_impl() -> str:
 
 
 def _fast_shape(H_q, H_kv, block_size, max_S, num_slots, top_k=None) -> bool:
-    return (_split_impl == "fast" and H_kv > 0 and H_q % H_kv == 0 and H_q // H_kv in (1, 2, 4, 8, 16)
+    return (_split_impl == "fast" and H_kv > 0 and H_q % H_kv == 0 and 1 <= H_q // H_kv <= 16
             and int(block_size) == 16 and 0 < int(max_S) <= 262144 and 0 < int(num_slots) <= FUSED_MAX_SLOTS
             and (top_k is None or int(top_k) in FUSED_TOP_K))
 

@@ -109,6 +109,10 @@ CASES = [
     # INT4 values with 64-channel groups (keys other than INT4)
     ("k3v4_g64", 2, 8, 2, 512, None, 64), ("k2v4_g64", 3, 32, 4, 512, [17, 257, 512], 256), ("a2v4_g64", 1, 8, 2, 5000, [4987], 256),
     ("k3v4_g64", 1, 16, 1, 600, None, 64), ("k2v4_g64", 1, 4, 4, 300, None, 32), ("a2v4_g64", 1, 4, 2, 300, None, 64),
+    # query heads per kv-head that are not a power of two (28/4, 24/8, 40/8, 48/8, 12/1 ...): the next larger kernel
+    ("k3v2", 2, 28, 4, 700, [700, 650], 64), ("k4v4", 2, 24, 8, 512, None, 64), ("k3v3", 1, 40, 8, 900, None, 128),
+    ("a2v2", 2, 12, 2, 512, [17, 512], 32), ("k2v4", 1, 12, 1, 600, None, 64), ("k4v2", 1, 9, 1, 300, None, 32),
+    ("k3v2", 3, 21, 3, 32, [0, 9, 17], 32), ("k4v4", 1, 7, 1, 5000, [4987], 256),
 ]
 SCHEME_GEOMETRY = {f"k{kb}v{vb}": (kb, vb, 128 if 4 in (kb, vb) else 64) for kb in (2, 3, 4) for vb in (2, 3, 4)}
 SCHEME_GEOMETRY.update({f"k{kb}v{vb}_g128": (kb, vb, 128) for kb in (2, 3) for vb in (2, 3)})

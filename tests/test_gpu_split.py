@@ -192,6 +192,7 @@ def impl(request):
 
 CASES_A = [  # (B, Hq, Hkv, S)
     (2, 8, 2, 512), (3, 32, 8, 300), (2, 32, 4, 272), (1, 8, 2, 17),
+    (2, 28, 4, 300), (1, 24, 8, 272), (2, 12, 1, 200),          # 7, 3 and 12 query heads per kv-head
 ]
 
 
@@ -322,7 +323,8 @@ def test_unsupported_top_k_raises():
 
 
 @pytest.mark.parametrize("scheme", ("k3v2", "k4v4", "k3v2_g128", "k3v3", "k3v3_g128", "k3v4_g64"))
-@pytest.mark.parametrize("B,Hq,Hkv,lens", [(2, 8, 2, None), (3, 32, 4, [17, 257, 512]), (4, 8, 2, [0, 1, 9, 17])])
+@pytest.mark.parametrize("B,Hq,Hkv,lens", [(2, 8, 2, None), (3, 32, 4, [17, 257, 512]), (4, 8, 2, [0, 1, 9, 17]),
+                                           (2, 28, 4, [400, 512]), (2, 10, 2, None)])      # 7 and 5 heads per kv-head
 def test_stage_b_outputs(scheme, B, Hq, Hkv, lens, impl):
     kb, vb, gs = {"k3v2": (3, 2, 64), "k4v4": (4, 4, 128), "k3v2_g128": (3, 2, 128), "k3v3": (3, 3, 64),
                   "k3v3_g128": (3, 3, 128), "k3v4_g64": (3, 4, 64)}[scheme]

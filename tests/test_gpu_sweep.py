@@ -19,8 +19,8 @@ SCHEMES = {"k3v2": (3, 2, 64), "k3v2_g128": (3, 2, 128), "k4v4": (4, 4, 128), "k
 def _draw(seed):
     rng = np.random.default_rng(1000 + seed)
     scheme = list(SCHEMES)[seed % len(SCHEMES)]
-    G = int(rng.choice([1, 2, 4, 8, 16]))
-    Hkv = int(rng.choice([1, 2, 4])) if G < 16 else 1
+    G = int(rng.choice([1, 2, 4, 8, 16, 3, 5, 6, 7, 12]))
+    Hkv = int(rng.choice([1, 2, 4])) if G < 12 else 1
     B = int(rng.integers(1, 4))
     S = int(rng.choice([48, 200, 777, 1500, 2600, 4100]))
     lens = [int(x) for x in rng.integers(0, S + 1, size=B)]
