@@ -597,6 +597,52 @@ def test_release_policy_selects_the_named_split_kernels(adapter, monkeypatch, sc
     assert store.scheme is not None
 
 
+@pytest.mark.gpu
+def test_corrections_wider_than_the_fused_form_run_the_split_operators(adapter, monkeypatch):
+    """JETFIRE_TOPK=4096 on a fused scheme: the width is kept (not clamped to the fused form's 2048) and the step
+    runs Stage A and Stage B as separate operators; with nearly every position corrected the output is the exact
+    attention over the bf16 shadow."""
+    from jetfire_amd import ops as jops
+    for name in list(__import__("os").environ):
+        if name.startswith("JETFIRE_"):
+            monkeypatch.delenv(name)
+    B, Hq, Hkv, D, bs, K = 1, 8, 2, 128, 16, 4096
+    S = 4100                                       # (the four uncorrected positions keep their INT2 values)
+    adapter.set_jetfire_config(scheme="SymInt3K_SymInt2V", group_size=64, topk=K, layer_stride=1, cpu_attn_threads=4)
+    adapter.reset_global_kv_pool_manager()
+    pool = adapter.get_global_kv_pool_manager()
+    name = "model.layers.0.self_attn.attn"
+    layer = types.SimpleNamespace(layer_name=name, num_heads=Hq, num_kv_heads=Hkv, head_size=D)
+    impl = types.SimpleNamespace(attn_type=types.SimpleNamespace(name="DECODER"), scale=D ** -0.5)
+    pool.ensure_layer_config_from_layer(name, layer)
+    per_seq = (S + bs - 1) // bs
+    pool.register_layer_layout(name, num_blocks=per_seq, block_size=bs)
+    g = torch.Generator().manual_seed(3)
+    bt = torch.arange(per_seq, dtype=torch.int64).view(1, per_seq).cuda()
+    k = torch.randn(S, Hkv, D, generator=g).to(torch.bfloat16).cuda()
+    v = torch.randn(S, Hkv, D, generator=g).to(torch.bfloat16).cuda()
+    pool.mirror_kv(name, k, v, torch.arange(S, dtype=torch.int64).cuda())
+    pool.flush_pending_writes()
+    meta = _meta(torch.tensor([S], dtype=torch.int32, device="cuda"), bt, max_seq_len=S)
+    q = (torch.randn(B, Hq, D, generator=g) / D ** 0.5).to(torch.bfloat16).cuda()
+    called = []
+    for op_name in ("fused_attn_topk", "int3_qk_scores_topk", "int2_softmax_v_with_pre_corr_wvs2"):
+        real = getattr(jops, op_name)
+        monkeypatch.setattr(jops, op_name, (lambda f, nm: (lambda *a, **kw: (called.append((nm, a, kw)), f(*a, **kw))[1]))(real, op_name))
+    out = torch.zeros(B, Hq * D, dtype=torch.bfloat16, device="cuda")
+    assert adapter.try_jetfire_decode(impl=impl, layer=layer, query=q, attn_metadata=meta, output=out) is out
+    torch.cuda.synchronize()
+    names = [c[0] for c in called]
+    assert "fused_attn_topk" not in names and "int3_qk_scores_topk" in names
+    stage_a = next(c for c in called if c[0] == "int3_qk_scores_topk")
+    assert int(stage_a[1][-1]) == K                                   # the configured width reaches Stage A
+    G = Hq // Hkv
+    att = torch.softmax(torch.einsum("hd,shd->hs", q[0].float(), k.float().repeat_interleave(G, dim=1)) * D ** -0.5, dim=-1)
+    ref = torch.einsum("hs,shd->hd", att, v.float().repeat_interleave(G, dim=1))
+    err = (out.view(Hq, D).float() - ref).abs()
+    assert float(err.max()) <= 2e-2 and float(err.mean()) <= 1e-3
+
+
 class _NativeImpl:
     """Stand-in for the serving engine's attention implementation: records what reaches it."""
 
