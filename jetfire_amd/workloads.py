@@ -22,7 +22,19 @@ CONFIGS = {
     "c4": (4, 32, 4, 32768, "k3v2", 64, 256, 48),
     "c5": (2, 32, 4, 65536, "k3v2", 64, 512, 80),
 }
-BYTES_PER_TOKEN_HEAD = {"k3v2": {64: 88, 128: 84}, "k4v4": {128: 132, 64: 136}}
+
+
+def scheme_bits(scheme: str):
+    """"k3v2" -> (3, 2, False); "a2v4" (asymmetric INT2 keys with zero-points) -> (2, 4, True)."""
+    return int(scheme[1]), int(scheme[3]), scheme[0] == "a"
+
+
+def bytes_per_token_head(scheme: str, group: int) -> int:
+    """Packed codes plus bf16 scales (and zero-points) of one token of one kv-head, K and V together."""
+    kb, vb, asym = scheme_bits(scheme)
+    ng = HEAD_DIM // group
+    return 16 * kb + 16 * vb + 2 * ng * (3 if asym else 2)
+
 
 
 @dataclass
@@ -31,6 +43,7 @@ class LayerCache:
     k_scales: torch.Tensor
     v_data: torch.Tensor
     v_scales: torch.Tensor
+    k_zp: torch.Tensor | None = None        # asymmetric INT2 keys only
 
 
 @dataclass
@@ -51,7 +64,7 @@ class Workload:
 
     @property
     def packed_bytes_per_layer(self) -> int:
-        return self.B * self.H_kv * self.S * BYTES_PER_TOKEN_HEAD[self.scheme][self.group]
+        return self.B * self.H_kv * self.S * bytes_per_token_head(self.scheme, self.group)
 
 
 def build(name: str, n_layers: int | None = None, seed: int = 0, paged: bool = False, device: str = "cuda",
@@ -75,7 +88,8 @@ def build(name: str, n_layers: int | None = None, seed: int = 0, paged: bool = F
     block_table = perm.reshape(B, S // BLOCK).to(torch.int64).to(dev)
     pos = torch.arange(S, device=dev)
     slots = (block_table[:, pos // BLOCK] * BLOCK + pos % BLOCK).reshape(-1)      # token t = b*S + pos
-    kb, vb = (3, 2) if scheme == "k3v2" else (4, 4)
+    kb, vb, asym = scheme_bits(scheme)
+    sym_writer = {2: ops.fused_quant_write_int2_sym, 3: ops.fused_quant_write_int3_sym, 4: ops.fused_quant_write_int4_sym}
     caches = []
     shadows = []
     for _ in range(layers):
@@ -86,12 +100,17 @@ def build(name: str, n_layers: int | None = None, seed: int = 0, paged: bool = F
         ks = torch.empty(Hkv, T, HEAD_DIM // gs, dtype=torch.bfloat16, device=dev)
         vd = torch.empty(Hkv, T, HEAD_DIM * vb // 8, dtype=torch.uint8, device=dev)
         vs = torch.empty(Hkv, T, HEAD_DIM // gs, dtype=torch.bfloat16, device=dev)
-        if scheme == "k3v2":
-            ops.fused_quant_write_int3_sym(k, slots, kd, ks, gs)
-            ops.fused_quant_write_int2_sym(v, slots, vd, vs, gs)
-        else:
+        kz = None
+        if scheme == "k4v4":
             ops.fused_quant_write_int4_sym_kv(k, v, slots, kd, ks, vd, vs, gs)
-        caches.append(LayerCache(kd, ks, vd, vs))
+        else:
+            if asym:
+                kz = torch.empty_like(ks)
+                ops.fused_quant_write_int2_asym(k, slots, kd, ks, kz, gs)
+            else:
+                sym_writer[kb](k, slots, kd, ks, gs)
+            sym_writer[vb](v, slots, vd, vs, gs)
+        caches.append(LayerCache(kd, ks, vd, vs, kz))
         if len(shadows) < int(keep_shadow):
             ksh = torch.empty(Hkv, T, HEAD_DIM, dtype=torch.bfloat16)
             vsh = torch.empty(Hkv, T, HEAD_DIM, dtype=torch.bfloat16)

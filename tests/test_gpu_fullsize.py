@@ -14,17 +14,15 @@ pytestmark = pytest.mark.gpu
 def _run(w, lay, **kw):
     from jetfire_amd import ops
     return ops.fused_attn_topk(w.scheme, w.q, lay.k_data, lay.k_scales, lay.v_data, lay.v_scales, w.block_table,
-                               w.seq_lens, w.S, w.H_q, w.H_kv, 16, w.top_k, w.attn_scale, **kw)
+                               w.seq_lens, w.S, w.H_q, w.H_kv, 16, w.top_k, w.attn_scale, k_zp=lay.k_zp, **kw)
 
 
-@pytest.mark.parametrize("name", ["c1", "c2", "c3", "c4", "c5"])
-def test_full_size_layer_properties(name):
+def _check_layer_properties(w):
     from jetfire_amd import workloads
-    w = workloads.build(name, n_layers=1, paged=True)
     lay = w.layers[0]
     B, Hq, Hkv, S, K = w.B, w.H_q, w.H_kv, w.S, w.top_k
     G = Hq // Hkv
-    kb, vb = (3, 2) if w.scheme == "k3v2" else (4, 4)
+    kb, vb, asym = workloads.scheme_bits(w.scheme)
     o_hat, slots, o_old, W, idx, m, iz, scores = _run(w, lay, return_scores=True, return_stats=True)
     again = _run(w, lay, return_scores=True, return_stats=True)
     for a, b in zip((o_hat, slots, o_old, W, idx, m, iz, scores), again):
@@ -49,15 +47,20 @@ def test_full_size_layer_properties(name):
     for b in range(B):
         sl = w.block_table[b, pos // 16] * 16 + pos % 16
         for h in range(Hkv):
-            khat = T.unpack(lay.k_data[h, sl], lay.k_scales[h, sl], w.group, kb).float()      # (S, 128)
-            vhat = (T.unpack(lay.v_data[h, sl], lay.v_scales[h, sl], w.group, vb)).float()
+            if asym:    # khat = bf16(fma(code - 2, scale, zp)); (code - 2) * scale is exact in fp32, so mul + add is the fma
+                codes = T.unpack(lay.k_data[h, sl], torch.ones_like(lay.k_scales[h, sl]), w.group, kb).float()
+                kf = (codes.reshape(S, -1, w.group) * lay.k_scales[h, sl].float()[..., None]
+                      + lay.k_zp[h, sl].float()[..., None])
+                khat = kf.to(torch.bfloat16).float().reshape(S, 128)
+            else:
+                khat = T.unpack(lay.k_data[h, sl], lay.k_scales[h, sl], w.group, kb).float()      # (S, 128)
             # Stage B multiplies by the unrounded fp32 scale: redo the dequant without the bf16 rounding
             vq = T.unpack(lay.v_data[h, sl], torch.ones_like(lay.v_scales[h, sl]), w.group, vb).float()
             vexact = (vq.reshape(S, -1, w.group) * lay.v_scales[h, sl].float()[..., None]).reshape(S, 128)
             qh = w.q[b, h * G:(h + 1) * G].float()
             ref = (qh @ khat.T) * w.attn_scale                                                  # (G, S)
             mine = scores[b, h * G:(h + 1) * G]
-            if w.scheme == "k3v2":      # same scoring model: bf16-rounded dequantised keys
+            if kb != 4:                 # same scoring model: bf16-rounded dequantised keys
                 torch.testing.assert_close(mine, ref, atol=3e-5, rtol=3e-5)
                 # every winner of the reference scores that is clear of the cut by more than the score tolerance
                 # must be among the kernel's winners (near-ties at the cut may differ legitimately)
@@ -79,8 +82,35 @@ def test_full_size_layer_properties(name):
             torch.testing.assert_close(W[b, h * G:(h + 1) * G], pw.sum(-1), atol=4e-6, rtol=1e-4)
             old = torch.einsum("gk,gkd->gd", pw, vexact[sel])
             torch.testing.assert_close(o_old[b, h * G:(h + 1) * G], old, atol=4e-6, rtol=1e-4)
-            del khat, vhat, vq, vexact
+            del khat, vq, vexact
     assert max_sc > 0
+
+
+@pytest.mark.parametrize("name", ["c1", "c2", "c3", "c4", "c5"])
+def test_full_size_layer_properties(name):
+    from jetfire_amd import workloads
+    _check_layer_properties(workloads.build(name, n_layers=1, paged=True))
+
+
+@pytest.mark.parametrize("scheme,gs,Hq,Hkv", [
+    ("k3v3", 64, 8, 2), ("k2v3", 128, 8, 2), ("k4v3", 128, 16, 2), ("k2v2", 64, 8, 2), ("k3v4", 64, 8, 2), ("k2v4", 128, 4, 2),
+    ("a2v2", 64, 8, 2), ("a2v3", 128, 8, 2), ("a2v4", 64, 16, 2), ("k4v2", 128, 14, 2), ("k3v2", 64, 6, 2)])
+def test_full_length_splits_of_the_other_schemes(scheme, gs, Hq, Hkv):
+    """The same properties for the schemes the benchmark shapes do not use, at the longest split a workgroup takes
+    (4096 positions: the full LDS layout, four chunks per wavefront), on a paged cache; the last two rows have 7 and
+    3 query heads per kv-head."""
+    from jetfire_amd import _lib, workloads
+    lib = _lib.load()
+    workloads.CONFIGS["other"] = (2, Hq, Hkv, 16384, scheme, gs, 256, 1)
+    try:
+        w = workloads.build("other", n_layers=1, paged=True)
+    finally:
+        del workloads.CONFIGS["other"]
+    _lib.check(lib.jf_debug_split_len(4096))
+    try:
+        _check_layer_properties(w)
+    finally:
+        _lib.check(lib.jf_debug_split_len(0))
 
 
 def test_c1_gpu_split_path_agrees_with_the_cpu_torch_path():
