@@ -33,7 +33,8 @@ def cpu_baseline(w, target_s: float = 10.0, budget_s: float = 25.0):
     import torch
     from oracle import torch_cpu_path as T
     S, Hkv, gs = w.S, w.H_kv, w.group
-    kb, vb = (3, 2) if w.scheme == "k3v2" else (4, 4)
+    from jetfire_amd import workloads
+    kb, vb, _ = workloads.scheme_bits(w.scheme)
     lay = w.layers[0]
     # sequence 0 occupies slots [0, S) with the identity block table
     kd = lay.k_data[:, :S].cpu().unsqueeze(0)
@@ -241,7 +242,7 @@ def measure_gpu_path(name: str, steps: int, warmup: int, lib):
     def step():
         for lay in w.layers:
             ops.fused_attn_topk(w.scheme, w.q, lay.k_data, lay.k_scales, lay.v_data, lay.v_scales, w.block_table,
-                                w.seq_lens, w.S, w.H_q, w.H_kv, 16, w.top_k, w.attn_scale, blend=(o_new, out))
+                                w.seq_lens, w.S, w.H_q, w.H_kv, 16, w.top_k, w.attn_scale, blend=(o_new, out), k_zp=lay.k_zp)
     for _ in range(max(1, warmup)):
         step()
     torch.cuda.synchronize()
@@ -311,6 +312,10 @@ def main() -> int:
                          "c2: Llama-3.1-8B B4 S32768 K3V2 k256 x32 layers (the headline); c2k4: the c2 shape with K4V4; "
                          "c3: B1 S131072 K4V4 k512; "
                          "c4: Qwen3-30B-A3B B4 GQA8 K3V2 x48; c5: Llama-3.3-70B TP2 shard B2 S65536 K3V2 x80")
+    ap.add_argument("--scheme", default=None,
+                    help="run the workload's shape with another quantisation scheme: k{2,3,4}v{2,3,4}, or a2v{2,3,4} for "
+                         "the asymmetric INT2 keys (GPU path only; no CPU baseline, no extra workloads)")
+    ap.add_argument("--group", type=int, default=None, choices=[64, 128], help="with --scheme: the quantisation group size")
     ap.add_argument("--layers", type=int, default=None, help="override the number of distinct layer caches")
     ap.add_argument("--paged", action="store_true", help="random block table instead of the identity mapping")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -393,6 +398,14 @@ def main() -> int:
         print(json.dumps({"append": component_append, "cpu-correction": component_cpu_correction,
                           "pcie": component_pcie, "split": component_split}[args.component](args)))
         return 0
+    if args.scheme or args.group:
+        if args.via_adapter or args.scheme not in (None, *ops.FUSED_SCHEMES):
+            print("bench.py: --scheme takes one of " + ", ".join(sorted(ops.FUSED_SCHEMES)) + " and excludes --via-adapter",
+                  file=sys.stderr)
+            return 2
+        B_, Hq_, Hkv_, S_, sch_, gs_, K_, L_ = workloads.CONFIGS[args.workload]
+        workloads.CONFIGS[args.workload] = (B_, Hq_, Hkv_, S_, args.scheme or sch_, args.group or gs_, K_, L_)
+        args.no_cpu_baseline = args.no_extras = True
     if args.split_len:
         _lib.check(lib.jf_debug_split_len(args.split_len))
     handoff = args.handoff if args.handoff is not None else args.workload in ("c4", "c5")
@@ -452,7 +465,8 @@ def main() -> int:
         for li, lay in enumerate(w.layers):
             o_hat, slots, o_old, W, idx = ops.fused_attn_topk(
                 w.scheme, w.q, lay.k_data, lay.k_scales, lay.v_data, lay.v_scales, w.block_table, w.seq_lens,
-                w.S, w.H_q, w.H_kv, 16, w.top_k, w.attn_scale, blend=None if (ctxs or args.separate_blend) else (o_new, out))
+                w.S, w.H_q, w.H_kv, 16, w.top_k, w.attn_scale, blend=None if (ctxs or args.separate_blend) else (o_new, out),
+                k_zp=lay.k_zp)
             if not ctxs and not args.separate_blend:
                 continue            # the merge kernel has written `out` (o_new is known up front without a hand-off)
             if ctxs:
