@@ -45,6 +45,11 @@ extern "C" {
 #define JF_SCHEME_A2V2 12    /* (AsymInt2K4Level_SymInt2V), group 64 or 128 */
 #define JF_SCHEME_A2V3 13    /* (AsymInt2K4Level_SymInt3V), group 64 or 128 */
 #define JF_SCHEME_A2V4 14    /* (AsymInt2K4Level_SymInt4V), group 64 or 128 */
+/* INT4 keys scored with the bf16 model of int4_qk_scores (jetfire_vllm/csrc/int4_qk_scores.cu:68-80) instead of the
+ * int8-Q model: what the reference runs for INT4 keys with 64-channel groups (decode_path.py:2016-2022); key digit 5 */
+#define JF_SCHEME_B4V2 52    /* (SymInt4K_SymInt2V), group 64 or 128 */
+#define JF_SCHEME_B4V3 53    /* (SymInt4K_SymInt3V), group 64 or 128 */
+#define JF_SCHEME_B4V4 54    /* (SymInt4K_SymInt4V), group 64 or 128 */
 
 const char* jf_last_error(void);
 const char* jf_version(void);

@@ -113,9 +113,13 @@ class JetFireInt4CacheStore:
         """Name the fused decode kernels know this store by, or None (split kernels / unsupported)."""
         if self.k_nbits not in (2, 3, 4) or self.v_nbits not in (2, 3, 4) or (self.k_asymmetric and self.k_nbits != 2):
             return None
-        if self.group_size == 128 or (self.group_size == 64 and self.k_nbits != 4):     # (INT4 keys: one scale per row)
-            return f"a2v{self.v_nbits}" if self.k_asymmetric else f"k{self.k_nbits}v{self.v_nbits}"
-        return None
+        if self.group_size not in (64, 128):
+            return None
+        if self.k_asymmetric:
+            return f"a2v{self.v_nbits}"
+        if self.k_nbits == 4 and self.group_size == 64:      # two key scales per row: the bf16 model, as the reference
+            return f"b4v{self.v_nbits}"                       # (jetfire_vllm/adapter/decode_path.py:2016-2022)
+        return f"k{self.k_nbits}v{self.v_nbits}"
 
     # ------------------------------------------------------------------ append
     def _prepare(self, key, value, slot_mapping):

@@ -21,6 +21,7 @@ SOURCES = (     # (the long compilations first: the pool starts them together)
     "fused_full_b.hip",
     "fused_full_c.hip",
     "fused_full_d.hip",
+    "fused_full_e.hip",
     "quant_write.hip",
     "shadow_write.hip",
     "qk_scores.hip",

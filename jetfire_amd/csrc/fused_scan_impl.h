@@ -69,6 +69,7 @@ int launch_full_scan_a(int scheme, int G, int NG, const void* params, void* stre
 int launch_full_scan_b(int scheme, int G, int NG, const void* params, void* stream);  // K2V2, K2V3, K2V4
 int launch_full_scan_c(int scheme, int G, int NG, const void* params, void* stream);  // K3V3, K4V3
 int launch_full_scan_d(int scheme, int G, int NG, const void* params, void* stream);  // A2V2, A2V3, A2V4
+int launch_full_scan_e(int scheme, int G, int NG, const void* params, void* stream);  // B4V2, B4V3, B4V4
 
 namespace {
 
@@ -146,7 +147,7 @@ struct K3Prep {
   int8_t aop[NSET][16][4][2][16];  // A operand bytes: [set][row = 4*head + limb][k-block][MFMA][byte]
   int sq4[NSET * 4][2];            // 4 * sum of the fixed-point query over the scale group
   float qsc[NSET * 4][2];          // 2^(e-22) * attn_scale of the (head, group)
-  float eps[128];                  // 256 * (bf16(3s) - 3s) / s for s = 1 + m/128
+  float eps[3][128];               // 256 * (bf16(c s) - c s) / s for s = 1 + m/128; INT3: c = 3; INT4: c = 3, 5, 7
   float amax_w[NSET * 8];          // per 64-channel half row: |q| maximum, fixed-point sum, exponent
   int sum_w[NSET * 8];
   int exp_w[NSET * 8];
@@ -169,12 +170,13 @@ struct QInt8F {
 // After phase B the staging area holds the sum of the wavefronts' P.V accumulators.
 template <int SCHEME, int G, int NG>
 struct ScanLds {
-  // SCHEME = 10 * key bits + value bits (key digit 1: asymmetric INT2): the key side (staging, query constants, phase A) and the value side
+  // SCHEME = 10 * key bits + value bits (key digit 1: asymmetric INT2; 5: INT4 with the bf16 model): the key side (staging, query constants, phase A) and the value side
   // (staging, phase B) are chosen independently
   static constexpr bool K3 = (SCHEME / 10 == 3);
   static constexpr bool KA = (SCHEME / 10 == 1);        // INT2 keys with a zero-point per group (four levels)
   static constexpr bool K2 = (SCHEME / 10 == 2) || KA;  // four codes per byte
-  static constexpr bool KLIMB = K2 || K3;  // keys with the bf16 model: fixed-point query limbs against integer codes
+  static constexpr bool KB4 = (SCHEME / 10 == 5);       // INT4 keys scored with the bf16 model (any group size)
+  static constexpr bool KLIMB = K2 || K3 || KB4;  // keys with the bf16 model: fixed-point query limbs against integer codes
   static constexpr bool V2 = (SCHEME % 10 == 2);
   static constexpr bool V3 = (SCHEME % 10 == 3);
   static_assert((KLIMB || SCHEME / 10 == 4) && (V2 || V3 || SCHEME % 10 == 4), "keys and values are INT2, INT3 or INT4");
@@ -254,7 +256,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   constexpr bool HAS_K = (MODE == FS_FULL || MODE == FS_STAGE_A);  // key stream and phase A
   constexpr bool HAS_V = (MODE == FS_FULL || MODE == FS_STAGE_B);  // value stream and the P.V part of phase B
   constexpr bool HAS_TOPK = (MODE != FS_STAGE_B);                  // histograms and phase C
-  constexpr bool K3 = Lds::K3, KLIMB = Lds::KLIMB, KA = Lds::KA;
+  constexpr bool K3 = Lds::K3, KLIMB = Lds::KLIMB, KA = Lds::KA, KB4 = Lds::KB4;
   constexpr bool V2 = Lds::V2, V3 = Lds::V3;
   constexpr int NSET = Lds::NSET;
   constexpr int SEG = Lds::SEG;
@@ -414,10 +416,13 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     // Query rows -> 23-bit fixed point per (head, scale group), three balanced int8 limbs, written in the
     // byte order of the MFMA A operand.  One element per thread; group statistics by wavefront reductions.
     K3Prep<NSET>* prep = reinterpret_cast<K3Prep<NSET>*>(aux);
-    if (K3 && tid < 128) {
+    if ((K3 || KB4) && tid < 128) {
       const float sm = 1.0f + (float)tid * (1.0f / 128.0f);
-      const float t3 = 3.0f * sm;  // exact in fp32
-      prep->eps[tid] = 256.0f * ((bf16_to_f32(f32_to_bf16(t3)) - t3) / sm);
+#pragma unroll
+      for (int i = 0; i < (KB4 ? 3 : 1); ++i) {
+        const float t = (float)(3 + 2 * i) * sm;  // 3 s, 5 s, 7 s: exact in fp32
+        prep->eps[i][tid] = 256.0f * ((bf16_to_f32(f32_to_bf16(t)) - t) / sm);
+      }
     }
 #pragma unroll
     for (int it = 0; it < QPT; ++it) {
@@ -449,12 +454,14 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
       const int l2 = (r1 - l1) >> 8;
       const int set = h >> 2, hh = h & 3;
       // A lane of phase A spreads the 32 channels 32*lg .. 32*lg+31 of its token into two 16-byte operands u = 0, 1
-      // (dword e, byte b).  INT3 (plane spread): channel 8b + 4u + e; INT2 (four codes per byte): channel 16u + 4b + e.
+      // (dword e, byte b).  INT3 (plane spread): channel 8b + 4u + e; INT2 (four codes per byte): channel 16u + 4b + e;
+      // INT4 (nibble spread of the lane's four dwords): channel 16u + 8(e >> 1) + 2b + (e & 1).
       // With two scale groups MFMA g covers group g only (see the lane swap in phase A).
       const int u = K3 ? ((d >> 2) & 1) : ((d >> 4) & 1);
       const int mi = (NG == 2) ? (d >> 6) : u;
       const int kb = (NG == 2) ? (((d >> 5) & 1) + 2 * u) : (d >> 5);
-      const int by = 4 * (d & 3) + (K3 ? ((d >> 3) & 3) : ((d >> 2) & 3));
+      const int by = KB4 ? (4 * (2 * ((d >> 3) & 1) + (d & 1)) + ((d >> 1) & 3))
+                         : (4 * (d & 3) + (K3 ? ((d >> 3) & 3) : ((d >> 2) & 3)));
       prep->aop[set][4 * hh + 0][kb][mi][by] = (int8_t)l0;
       prep->aop[set][4 * hh + 1][kb][mi][by] = (int8_t)l1;
       prep->aop[set][4 * hh + 2][kb][mi][by] = (int8_t)l2;
@@ -465,7 +472,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
       const int h = tid / NG, g = tid % NG;
       const int sum = (NG == 2) ? prep->sum_w[2 * h + g] : prep->sum_w[2 * h] + prep->sum_w[2 * h + 1];
       const int e = prep->exp_w[2 * h + ((NG == 2) ? g : 0)];
-      prep->sq4[h][g] = (K3 ? 4 : 2) * sum;  // the codes are used unsigned: offset 4 (INT3) or 2 (INT2)
+      prep->sq4[h][g] = (KB4 ? 8 : (K3 ? 4 : 2)) * sum;  // the codes are used unsigned: offset 8 (INT4), 4 (INT3) or 2 (INT2)
       prep->qsc[h][g] = ldexpf(p.attn_scale, e - 22);
     }
   } else {
@@ -599,7 +606,8 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
         qsc[set][g] = prep->qsc[set * 4 + lg][g];
       }
     }
-    const uint8_t* krd = kst + t16 * KROW + lg * (K3 ? 4 : 8);  // this lane's plane dwords (INT2: its 8 bytes) of token t16 of a page
+    // this lane's plane dwords (INT2: its 8 bytes, INT4: its 16 bytes) of token t16 of a page
+    const uint8_t* krd = kst + t16 * KROW + lg * (K3 ? 4 : (KB4 ? 16 : 8));
     float mxl[NSET], mnl[NSET];
 #pragma unroll
     for (int set = 0; set < NSET; ++set) {
@@ -615,7 +623,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     auto body = [&](int chunk, const uint32_t (&Sx)[4], const uint32_t (&Zx)[4]) {
       (void)Zx;
       // all LDS reads of the chunk first (plane dwords of the four pages, rounding coefficients), then arithmetic
-      uint32_t Pj[4][3];
+      uint32_t Pj[4][KB4 ? 4 : 3];
       float sgj[4][NG], egj[4][NG];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
@@ -624,6 +632,10 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
           Pj[j][0] = *reinterpret_cast<const uint32_t*>(rp);
           Pj[j][1] = *reinterpret_cast<const uint32_t*>(rp + 16);
           Pj[j][2] = *reinterpret_cast<const uint32_t*>(rp + 32);
+        } else if constexpr (KB4) {
+          const v4u x = *reinterpret_cast<const v4u*>(rp);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) Pj[j][KB4 ? i : 0] = x[i];
         } else {
           const v2u x = *reinterpret_cast<const v2u*>(rp);
           Pj[j][0] = x[0];
@@ -632,10 +644,10 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
         }
         const uint32_t sw = Sx[j];
         sgj[j][0] = bf16_to_f32((uint16_t)(sw & 0xffffu));
-        egj[j][0] = K3 ? prep->eps[sw & 0x7fu] : 0.f;
+        egj[j][0] = K3 ? prep->eps[0][sw & 0x7fu] : 0.f;  // (INT4: three coefficients, read where they are used)
         if (NG == 2) {
           sgj[j][NG - 1] = bf16_to_f32((uint16_t)(sw >> 16));
-          egj[j][NG - 1] = K3 ? prep->eps[(sw >> 16) & 0x7fu] : 0.f;
+          egj[j][NG - 1] = K3 ? prep->eps[0][(sw >> 16) & 0x7fu] : 0.f;
         }
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -643,7 +655,11 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
       for (int j = 0; j < 4; ++j) {
         const uint32_t P0 = Pj[j][0], P1 = Pj[j][1], P2 = Pj[j][2];
         v4i Bc[2], Br[2];
-        if constexpr (K3) {
+        if constexpr (KB4) {  // two codes per byte, the even channel in the high nibble
+          const uint32_t P3 = Pj[j][KB4 ? 3 : 0];
+          Bc[0] = (v4i){(int)((P0 >> 4) & 0x0f0f0f0fu), (int)(P0 & 0x0f0f0f0fu), (int)((P1 >> 4) & 0x0f0f0f0fu), (int)(P1 & 0x0f0f0f0fu)};
+          Bc[1] = (v4i){(int)((P2 >> 4) & 0x0f0f0f0fu), (int)(P2 & 0x0f0f0f0fu), (int)((P3 >> 4) & 0x0f0f0f0fu), (int)(P3 & 0x0f0f0f0fu)};
+        } else if constexpr (K3) {
           Bc[0][0] = (int)((P0 >> 5) & 0x07070707u);
           Bc[0][1] = (int)((P0 >> 2) & 0x07070707u);
           Bc[0][2] = (int)(((P0 << 1) & 0x06060606u) | ((P1 >> 7) & 0x01010101u));
@@ -666,6 +682,75 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
             Bc[0][e] = (int)sw[0];
             Bc[1][e] = (int)sw[1];
           }
+        }
+        if constexpr (KB4) {
+          // khat = bf16((u - 8) s) for the unsigned nibble u: exact for |u - 8| in {0, 1, 2, 4, 8}; for 3, 5, 7 (and 6 =
+          // 2 * 3) the rounding is eps_c(s) * s with the sign of the code, eps_c a function of the scale's mantissa
+          // alone.  So next to the code contraction there are three with the signed indicators r3 = [c = +-3] +
+          // 2 [c = +-6], r5 = [c = +-5], r7 = [c = +-7], made by byte look-ups: one table for the codes >= 0 (u >= 8,
+          // selector u - 8 = c) and one for the codes < 0 (selector u = c + 8), chosen per byte by bit 3 of u.
+          const int tok = chunk * 64 + 16 * j + t16;
+          const bool valid = tok < n;
+          float acc_s[NSET][NG];
+#pragma unroll
+          for (int set = 0; set < NSET; ++set)
+#pragma unroll
+            for (int g = 0; g < NG; ++g) {
+              const v4i zero = {0, 0, 0, 0};
+              v4i Dc;
+              if (NG == 2) {
+                Dc = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][g], Bc[g], zero, 0, 0, 0);
+              } else {
+                Dc = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][0], Bc[0], zero, 0, 0, 0);
+                Dc = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][1], Bc[1], Dc, 0, 0, 0);
+              }
+              acc_s[set][g] = (float)((((Dc[2] << 8) + Dc[1]) << 8) + Dc[0] - sq4[set][g]);
+            }
+#pragma unroll
+          for (int c = 0; c < 3; ++c) {  // c = 0, 1, 2: the indicators of +-3 (and +-6), +-5, +-7
+            const uint32_t pos_hi = (c == 0) ? 0x00020000u : ((c == 1) ? 0x00000100u : 0x01000000u);  // selectors 4..7
+            const uint32_t pos_lo = (c == 0) ? 0x01000000u : 0u;                                       // selectors 0..3
+            const uint32_t neg_hi = (c == 0) ? 0x0000ff00u : 0u;
+            const uint32_t neg_lo = (c == 0) ? 0x00fe0000u : ((c == 1) ? 0xff000000u : 0x0000ff00u);
+            v4i Bi[2];
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                const uint32_t x = (uint32_t)Bc[u][e], sel = x & 0x07070707u;
+                const uint32_t t = (x >> 3) & 0x01010101u, hm = (t << 8) - t;  // 0xff in the bytes whose code is >= 0
+                const uint32_t rp_ = __builtin_amdgcn_perm(pos_hi, pos_lo, sel), rn_ = __builtin_amdgcn_perm(neg_hi, neg_lo, sel);
+                Bi[u][e] = (int)((rp_ & hm) | (rn_ & ~hm));
+              }
+#pragma unroll
+            for (int set = 0; set < NSET; ++set)
+#pragma unroll
+              for (int g = 0; g < NG; ++g) {
+                const v4i zero = {0, 0, 0, 0};
+                v4i Dr;
+                if (NG == 2) {
+                  Dr = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][g], Bi[g], zero, 0, 0, 0);
+                } else {
+                  Dr = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][0], Bi[0], zero, 0, 0, 0);
+                  Dr = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][1], Bi[1], Dr, 0, 0, 0);
+                }
+                const float ec = prep->eps[c][((g == 0) ? Sx[j] : (Sx[j] >> 16)) & 0x7fu];
+                acc_s[set][g] = __builtin_fmaf(ec, (float)((Dr[2] << 8) + Dr[1]), acc_s[set][g]);
+              }
+          }
+#pragma unroll
+          for (int set = 0; set < NSET; ++set) {
+            float score = 0.f;
+#pragma unroll
+            for (int g = 0; g < NG; ++g) score = __builtin_fmaf(acc_s[set][g], sgj[j][g] * qsc[set][g], score);
+            const int h = set * 4 + lg;
+            if ((G % 4 == 0) || h < G) {
+              sc[h * L + tok] = valid ? score : -INFINITY;
+              mxl[set] = fmaxf(mxl[set], valid ? score : -INFINITY);
+              mnl[set] = fminf(mnl[set], valid ? score : INFINITY);
+            }
+          }
+          continue;
         }
         if constexpr (KA) {
           // Four levels per group: khat(code) = bf16(fma(code - 2, scale, zp)) (int2_qk_scores.cu:66-79) is any function
@@ -2088,6 +2173,8 @@ inline int lmax_dispatch(int scheme, int G, int NG) {
   JF_LMAX_ALL_G(JF_SCHEME_A2V3, 1); JF_LMAX_ALL_G(JF_SCHEME_A2V3, 2);
   JF_LMAX_ALL_G(JF_SCHEME_A2V4, 1);
   JF_LMAX_ALL_G(JF_SCHEME_K3V4, 2); JF_LMAX_ALL_G(JF_SCHEME_K2V4, 2); JF_LMAX_ALL_G(JF_SCHEME_A2V4, 2);
+  JF_LMAX_ALL_G(JF_SCHEME_B4V2, 1); JF_LMAX_ALL_G(JF_SCHEME_B4V2, 2); JF_LMAX_ALL_G(JF_SCHEME_B4V3, 1);
+  JF_LMAX_ALL_G(JF_SCHEME_B4V3, 2); JF_LMAX_ALL_G(JF_SCHEME_B4V4, 1); JF_LMAX_ALL_G(JF_SCHEME_B4V4, 2);
 #undef JF_LMAX_ALL_G
 #undef JF_LMAX_CASE
   return 256;
@@ -2253,7 +2340,8 @@ inline bool scheme_has_zp(int scheme) {  // asymmetric INT2 keys
 inline bool known_scheme(int scheme) {
   return scheme == JF_SCHEME_K3V2 || scheme == JF_SCHEME_K4V4 || scheme == JF_SCHEME_K3V4 || scheme == JF_SCHEME_K4V2 ||
          scheme == JF_SCHEME_K2V2 || scheme == JF_SCHEME_K2V4 || scheme == JF_SCHEME_K2V3 || scheme == JF_SCHEME_K3V3 ||
-         scheme == JF_SCHEME_K4V3 || scheme_has_zp(scheme);
+         scheme == JF_SCHEME_K4V3 || scheme_has_zp(scheme) || scheme == JF_SCHEME_B4V2 || scheme == JF_SCHEME_B4V3 ||
+         scheme == JF_SCHEME_B4V4;
 }
 // scale groups per row: every scheme but those with INT4 keys (int8-Q model: one key scale per row) may use
 // 64-channel groups
@@ -2277,7 +2365,7 @@ static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_
                      size_t workspace_bytes, void* stream) {
   JF_CHECK_ARG(known_scheme(scheme), "fused_scan: unknown scheme %d", scheme);
   JF_CHECK_ARG(MODE == FS_FULL || scheme == JF_SCHEME_K3V2 || scheme == JF_SCHEME_K4V4 ||
-                   (MODE == FS_STAGE_A && (scheme == JF_SCHEME_K2V2 || scheme == JF_SCHEME_A2V2)) ||
+                   (MODE == FS_STAGE_A && (scheme == JF_SCHEME_K2V2 || scheme == JF_SCHEME_A2V2 || scheme == JF_SCHEME_B4V2)) ||
                    (MODE == FS_STAGE_B && (scheme == JF_SCHEME_K3V3 || scheme == JF_SCHEME_K3V4)),
                "fused_scan: the stage-wise forms take the K3V2 or K4V4 side formats (Stage A also K2V2 and A2V2, Stage B also K3V3)");
   JF_CHECK_ARG(!(MODE == FS_FULL || MODE == FS_STAGE_A) || scheme_has_zp(scheme) == (k_zp != nullptr) || B == 0,
@@ -2364,6 +2452,7 @@ static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_
   }
   if constexpr (MODE == FS_FULL) {  // (instantiated elsewhere, by family)
     if (scheme_has_zp(scheme)) rc = launch_full_scan_d(scheme, G, NGv, &p, stream);
+    else if (scheme / 10 == 5) rc = launch_full_scan_e(scheme, G, NGv, &p, stream);
     else if (scheme / 10 == 2) rc = launch_full_scan_b(scheme, G, NGv, &p, stream);
     else if (scheme == JF_SCHEME_K3V3 || scheme == JF_SCHEME_K4V3) rc = launch_full_scan_c(scheme, G, NGv, &p, stream);
     else rc = launch_full_scan_a(scheme, G, NGv, &p, stream);
@@ -2379,6 +2468,8 @@ static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_
     } else if (NGv == 2) JF_FUSED_BY_G(JF_SCHEME_K3V3, 2) else JF_FUSED_BY_G(JF_SCHEME_K3V3, 1)
   } else if (scheme == JF_SCHEME_K2V2) {  // (Stage A)
     if (NGv == 2) JF_FUSED_BY_G(JF_SCHEME_K2V2, 2) else JF_FUSED_BY_G(JF_SCHEME_K2V2, 1)
+  } else if (scheme == JF_SCHEME_B4V2) {
+    if (NGv == 2) JF_FUSED_BY_G(JF_SCHEME_B4V2, 2) else JF_FUSED_BY_G(JF_SCHEME_B4V2, 1)
   } else {
     if (NGv == 2) JF_FUSED_BY_G(JF_SCHEME_A2V2, 2) else JF_FUSED_BY_G(JF_SCHEME_A2V2, 1)
   }

@@ -12,9 +12,10 @@ extern "C" int jf_stage_a_topk(int key_format, int group_size, const uint16_t* q
                                float attn_scale, int top_k, float* scores, int64_t* topk_idx, int64_t* topk_slots,
                                float* softmax_m, float* softmax_inv_z, void* workspace, size_t workspace_bytes,
                                void* stream) {
-  JF_CHECK_ARG(key_format == JF_SCHEME_K3V2 || key_format == JF_SCHEME_K4V4 || key_format == JF_SCHEME_K2V2,
+  JF_CHECK_ARG(key_format == JF_SCHEME_K3V2 || key_format == JF_SCHEME_K4V4 || key_format == JF_SCHEME_K2V2 ||
+                   key_format == JF_SCHEME_B4V2,
                "stage_a_topk: key_format must be JF_SCHEME_K3V2 (INT3 keys, bf16 model), JF_SCHEME_K2V2 (symmetric INT2 keys, "
-               "bf16 model) or JF_SCHEME_K4V4 (INT4 keys, int8-Q model)");
+               "bf16 model), JF_SCHEME_B4V2 (INT4 keys, bf16 model) or JF_SCHEME_K4V4 (INT4 keys, int8-Q model)");
   JF_CHECK_ARG(top_k >= 0, "stage_a_topk: negative top_k");
   return fused_run<FS_STAGE_A>(key_format, group_size, q, k_data, k_scales, nullptr, nullptr, nullptr, block_table, seq_lens,
                                B, H_q, H_kv, max_S, max_blocks, num_slots, block_size, attn_scale, top_k, topk_idx,

@@ -54,6 +54,8 @@ def _workspace(device: torch.device, nbytes: int, tag: str) -> torch.Tensor:
 FUSED_SCHEMES = {f"k{kb}v{vb}": 10 * kb + vb for kb in (2, 3, 4) for vb in (2, 3, 4)}
 # and the asymmetric INT2 keys (four levels, zero-points in k_zp): key digit 1
 FUSED_SCHEMES.update({f"a2v{vb}": 10 + vb for vb in (2, 3, 4)})
+# and INT4 keys scored with the bf16 model (what the reference runs for INT4 keys with 64-channel groups): key digit 5
+FUSED_SCHEMES.update({f"b4v{vb}": 50 + vb for vb in (2, 3, 4)})
 
 
 def reserve_fused_workspace(scheme: str, B: int, H_q: int, H_kv: int, max_S: int, top_k: int, device) -> int:
@@ -307,9 +309,9 @@ def _intn_qk_scores(nbits: int, name: str, q, k_data, k_scales, block_table, seq
         k_zp = (k_zp.unsqueeze(-1) if k_zp.dim() == 2 else k_zp).contiguous()
         _check(k_zp.is_cuda and k_zp.dtype == torch.bfloat16 and k_zp.shape == ks.shape,
                "k_zp must be bf16 with the shape of k_scales")
-    if nbits == 2 and _fast_shape(H_q, H_kv, block_size, max_S, kd.size(1)):
-        return _stage_a_fast(22 if k_zp is None else 12, q, kd, ks, bt, sl, max_S, H_q, H_kv, attn_scale, None, False,
-                             k_zp=k_zp)[0]
+    if _fast_shape(H_q, H_kv, block_size, max_S, kd.size(1)):       # (INT4 keys: the bf16 model, tag 52)
+        fmt = 52 if nbits == 4 else (22 if k_zp is None else 12)
+        return _stage_a_fast(fmt, q, kd, ks, bt, sl, max_S, H_q, H_kv, attn_scale, None, False, k_zp=k_zp)[0]
     B = q.size(0)
     scores = torch.empty((B, H_q, max_S), dtype=torch.float32, device=q.device)
     _lib.check(lib.jf_intn_qk_scores(nbits, q.data_ptr(), kd.data_ptr(), ks.data_ptr(), _ptr(k_zp), bt.data_ptr(), sl.data_ptr(),
@@ -355,6 +357,10 @@ def int4_qk_scores(q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_kv,
 def int4_qk_scores_topk(q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_kv, block_size, attn_scale,
                         top_k) -> List[torch.Tensor]:
     """int4_qk_scores.cu:714-786 -> [scores, topk_idx, topk_slots]."""
+    if _fast_shape(H_q, H_kv, block_size, max_S, k_data.size(1) if k_data.dim() == 3 else 0, top_k):
+        q_, kd, ks, bt, sl = _stage_a_args(q, k_data, k_scales, block_table, seq_lens, H_q, H_kv, 64)
+        _check(ks.size(2) in (1, 2), f"int4_qk_scores currently supports K quant groups 1 or 2, got {ks.size(2)}")
+        return list(_stage_a_fast(52, q_, kd, ks, bt, sl, max_S, H_q, H_kv, attn_scale, int(top_k), False)[:3])
     scores = int4_qk_scores(q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_kv, block_size, attn_scale)
     idx, slots, _, _ = _topk(scores, block_table, seq_lens, max_S, H_q, block_size, top_k, False, "int4_qk_scores_topk")
     return [scores, idx, slots]
@@ -363,6 +369,10 @@ def int4_qk_scores_topk(q, k_data, k_scales, block_table, seq_lens, max_S, H_q, 
 def int4_qk_scores_topk_stats(q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_kv, block_size, attn_scale,
                               top_k) -> List[torch.Tensor]:
     """int4_qk_scores.cu:788-848 -> [scores, topk_idx, topk_slots, softmax_m, softmax_inv_z]."""
+    if _fast_shape(H_q, H_kv, block_size, max_S, k_data.size(1) if k_data.dim() == 3 else 0, top_k):
+        q_, kd, ks, bt, sl = _stage_a_args(q, k_data, k_scales, block_table, seq_lens, H_q, H_kv, 64)
+        _check(ks.size(2) in (1, 2), f"int4_qk_scores currently supports K quant groups 1 or 2, got {ks.size(2)}")
+        return list(_stage_a_fast(52, q_, kd, ks, bt, sl, max_S, H_q, H_kv, attn_scale, int(top_k), True))
     scores = int4_qk_scores(q, k_data, k_scales, block_table, seq_lens, max_S, H_q, H_kv, block_size, attn_scale)
     idx, slots, m, iz = _topk(scores, block_table, seq_lens, max_S, H_q, block_size, top_k, True,
                               "int4_qk_scores_topk_stats")
@@ -602,12 +612,13 @@ def fused_attn_topk(scheme: str, q, k_data, k_scales, v_data, v_scales, block_ta
     (jetfire_vllm/kernels/int2_fused_attn_topk.py:5-10) extended to INT3 / INT4 keys (INT4: the int8-Q scoring
     model), symmetric INT2 keys, and INT2 / INT3 / INT4 values: "k{2,3,4}v{2,3,4}"; pairs with INT4 keys take
     group 128, the others group 64 or 128.  "a2v{2,3,4}": asymmetric INT2 keys, whose zero-points come in `k_zp`
-    (shaped like k_scales), the reference's int2_asym_k_* kernel sets."""
+    (shaped like k_scales), the reference's int2_asym_k_* kernel sets.  "b4v{2,3,4}": INT4 keys scored with the bf16 model
+    of int4_qk_scores (group 64 or 128), what the reference runs for INT4 keys with 64-channel groups."""
     lib = _lib.load()
     scheme_id = FUSED_SCHEMES.get(scheme)
     _check(scheme_id is not None, f"unknown scheme {scheme!r} ({', '.join(sorted(FUSED_SCHEMES))})")
     asym = scheme_id // 10 == 1
-    kp, vp = (32 if asym else 16 * (scheme_id // 10)), 16 * (scheme_id % 10)
+    kp, vp = {1: 32, 5: 64}.get(scheme_id // 10, 16 * (scheme_id // 10)), 16 * (scheme_id % 10)
     q, kd, ks, bt, sl = _stage_a_args(q, k_data, k_scales, block_table, seq_lens, H_q, H_kv, kp)
     _check(asym == (k_zp is not None), "k_zp goes with the a2v* schemes, and only with them")
     if asym:

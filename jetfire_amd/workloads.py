@@ -25,7 +25,8 @@ CONFIGS = {
 
 
 def scheme_bits(scheme: str):
-    """"k3v2" -> (3, 2, False); "a2v4" (asymmetric INT2 keys with zero-points) -> (2, 4, True)."""
+    """"k3v2" -> (3, 2, False); "a2v4" (asymmetric INT2 keys with zero-points) -> (2, 4, True); "b4v4" (INT4 keys
+    scored with the bf16 model: the same cache as "k4v4") -> (4, 4, False)."""
     return int(scheme[1]), int(scheme[3]), scheme[0] == "a"
 
 

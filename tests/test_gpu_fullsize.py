@@ -60,7 +60,7 @@ def _check_layer_properties(w):
             qh = w.q[b, h * G:(h + 1) * G].float()
             ref = (qh @ khat.T) * w.attn_scale                                                  # (G, S)
             mine = scores[b, h * G:(h + 1) * G]
-            if kb != 4:                 # same scoring model: bf16-rounded dequantised keys
+            if kb != 4 or w.scheme[0] == "b":   # same scoring model: bf16-rounded dequantised keys
                 torch.testing.assert_close(mine, ref, atol=3e-5, rtol=3e-5)
                 # every winner of the reference scores that is clear of the cut by more than the score tolerance
                 # must be among the kernel's winners (near-ties at the cut may differ legitimately)
@@ -94,7 +94,8 @@ def test_full_size_layer_properties(name):
 
 @pytest.mark.parametrize("scheme,gs,Hq,Hkv", [
     ("k3v3", 64, 8, 2), ("k2v3", 128, 8, 2), ("k4v3", 128, 16, 2), ("k2v2", 64, 8, 2), ("k3v4", 64, 8, 2), ("k2v4", 128, 4, 2),
-    ("a2v2", 64, 8, 2), ("a2v3", 128, 8, 2), ("a2v4", 64, 16, 2), ("k4v2", 128, 14, 2), ("k3v2", 64, 6, 2)])
+    ("a2v2", 64, 8, 2), ("a2v3", 128, 8, 2), ("a2v4", 64, 16, 2), ("b4v4", 64, 8, 2), ("b4v3", 128, 16, 2),
+    ("k4v2", 128, 14, 2), ("k3v2", 64, 6, 2)])
 def test_full_length_splits_of_the_other_schemes(scheme, gs, Hq, Hkv):
     """The same properties for the schemes the benchmark shapes do not use, at the longest split a workgroup takes
     (4096 positions: the full LDS layout, four chunks per wavefront), on a paged cache; the last two rows have 7 and

@@ -27,7 +27,7 @@ def check_against_oracle(scheme, c, S, K, out):
     o_hat, slots, o_old, W, idx, m, iz, scores = [t.cpu().numpy() for t in out]
     kb, vb, gs = c["kbits"], c["vbits"], c["gs"]
     Hq, Hkv = c["Hq"], c["Hkv"]
-    if kb in (2, 3):
+    if kb in (2, 3) or scheme.startswith("b"):
         ref_sc = O.scores_bf16_model(c["q"], c["kd"], c["ks"], c["bt"], c["lens"], S, Hq, Hkv, 16, SCALE, kb, gs,
                                      k_zp_bits=c.get("kzp"))
         valid = np.isfinite(ref_sc)
@@ -109,6 +109,12 @@ CASES = [
     # INT4 values with 64-channel groups (keys other than INT4)
     ("k3v4_g64", 2, 8, 2, 512, None, 64), ("k2v4_g64", 3, 32, 4, 512, [17, 257, 512], 256), ("a2v4_g64", 1, 8, 2, 5000, [4987], 256),
     ("k3v4_g64", 1, 16, 1, 600, None, 64), ("k2v4_g64", 1, 4, 4, 300, None, 32), ("a2v4_g64", 1, 4, 2, 300, None, 64),
+    # INT4 keys scored with the bf16 model (any group size)
+    ("b4v4", 2, 8, 2, 512, None, 64), ("b4v4_g128", 2, 8, 2, 700, None, 128), ("b4v2", 2, 8, 2, 512, None, 64),
+    ("b4v2_g128", 3, 32, 4, 512, [17, 257, 512], 256), ("b4v3", 3, 32, 4, 512, [17, 257, 512], 256),
+    ("b4v4", 4, 8, 2, 32, [0, 1, 9, 17], 32), ("b4v3", 1, 8, 2, 5000, [4987], 256), ("b4v4", 1, 8, 2, 5000, [4987], 1024),
+    ("b4v2", 1, 4, 4, 300, None, 32), ("b4v4_g128", 1, 4, 2, 300, None, 64), ("b4v4", 1, 16, 1, 600, None, 64),
+    ("b4v4", 2, 28, 4, 700, [700, 650], 64),
     # query heads per kv-head that are not a power of two (28/4, 24/8, 40/8, 48/8, 12/1 ...): the next larger kernel
     ("k3v2", 2, 28, 4, 700, [700, 650], 64), ("k4v4", 2, 24, 8, 512, None, 64), ("k3v3", 1, 40, 8, 900, None, 128),
     ("a2v2", 2, 12, 2, 512, [17, 512], 32), ("k2v4", 1, 12, 1, 600, None, 64), ("k4v2", 1, 9, 1, 300, None, 32),
@@ -116,6 +122,8 @@ CASES = [
 ]
 SCHEME_GEOMETRY = {f"k{kb}v{vb}": (kb, vb, 128 if 4 in (kb, vb) else 64) for kb in (2, 3, 4) for vb in (2, 3, 4)}
 SCHEME_GEOMETRY.update({f"k{kb}v{vb}_g128": (kb, vb, 128) for kb in (2, 3) for vb in (2, 3)})
+# INT4 keys with the bf16 scoring model
+SCHEME_GEOMETRY.update({"b4v2": (4, 2, 64), "b4v2_g128": (4, 2, 128), "b4v3": (4, 3, 64), "b4v4": (4, 4, 64), "b4v4_g128": (4, 4, 128)})
 # asymmetric INT2 keys
 SCHEME_GEOMETRY.update({"k3v4_g64": (3, 4, 64), "k2v4_g64": (2, 4, 64), "a2v4_g64": (2, 4, 64)})   # INT4 values, two scale groups
 SCHEME_GEOMETRY.update({"a2v2": (2, 2, 64), "a2v2_g128": (2, 2, 128), "a2v3": (2, 3, 64), "a2v3_g128": (2, 3, 128),

@@ -13,7 +13,7 @@ SCHEMES = {"k3v2": (3, 2, 64), "k3v2_g128": (3, 2, 128), "k4v4": (4, 4, 128), "k
            "k2v2": (2, 2, 64), "k2v2_g128": (2, 2, 128), "k2v4": (2, 4, 128),
            "k3v3": (3, 3, 64), "k3v3_g128": (3, 3, 128), "k2v3": (2, 3, 64), "k4v3": (4, 3, 128),
            "a2v2": (2, 2, 64), "a2v2_g128": (2, 2, 128), "a2v3": (2, 3, 64), "a2v4": (2, 4, 128),
-           "k3v4_g64": (3, 4, 64), "a2v4_g64": (2, 4, 64)}
+           "k3v4_g64": (3, 4, 64), "a2v4_g64": (2, 4, 64), "b4v4": (4, 4, 64), "b4v2_g128": (4, 2, 128)}
 
 
 def _draw(seed):
@@ -30,7 +30,7 @@ def _draw(seed):
     return scheme, B, G * Hkv, Hkv, S, lens, K, split
 
 
-@pytest.mark.parametrize("seed", range(144))
+@pytest.mark.parametrize("seed", range(160))
 def test_fused_scan_random_geometry(seed):
     from jetfire_amd import _lib
     scheme, B, Hq, Hkv, S, lens, K, split = _draw(seed)
