@@ -200,7 +200,7 @@ int jf_softmax_v_int8_tiles(const float* scores, const float* softmax_m, const f
  * scale per row) take group 128, the others group 64 or 128.  INT3 and symmetric INT2 keys score with the bf16 model of
  * jf_int3_qk_scores / jf_intn_qk_scores (jetfire_vllm/csrc/int2_qk_scores.cu:66-79), INT4 keys with the int8-Q model
  * of jf_int8tc_qk_scores; INT3 values are the planar rows of jetfire_vllm/csrc/int3_softmax_v.cu:43,282-284.
- * top_k: power of two in [32, 2048] (the split entry points above take up to 8192); num_slots at most 2^26 (row
+ * top_k: power of two in [32, 8192]; num_slots at most 2^26 (row
  * offsets are 32-bit).  If scores is non-NULL the fp32 scores are also written (validation).
  * workspace: jf_fused_workspace_bytes() bytes of device memory. */
 size_t jf_fused_workspace_bytes(int scheme, int B, int H_q, int H_kv, int max_S, int top_k);
@@ -252,7 +252,7 @@ int jf_fused_scan_topk_asym(int scheme, int group_size,
 /* Stage A alone and Stage B alone on the kernels of the fused step, for callers that keep the reference's two-call
  * structure (jetfire_vllm/adapter/decode_path.py:2081-2131 then :2804-2935): the same results as the split entry
  * points above for the shapes the fused step supports (head_dim 128, block_size 16, H_q/H_kv from 1 to 16,
- * top_k <= 2048, num_slots <= 2^26), at a fraction of their time.  workspace: jf_fused_workspace_bytes(format, ...).
+ * num_slots <= 2^26), at a fraction of their time.  workspace: jf_fused_workspace_bytes(format, ...).
  *
  * jf_stage_a_topk replaces int3_qk_scores / int3_qk_scores_topk (jetfire_vllm/csrc/int3_qk_scores.cu:640-655;
  * key_format JF_SCHEME_K3V2: INT3 keys, bf16 model, group 64 or 128), int2_qk_scores / int2_qk_scores_topk with
@@ -279,7 +279,7 @@ int jf_stage_a_topk_asym(int group_size,
                          float* scores, int64_t* topk_idx, int64_t* topk_slots,
                          float* softmax_m, float* softmax_inv_z,
                          void* workspace, size_t workspace_bytes, void* stream);
-/* jf_topk_slots on the kernels of the fused step (top_k <= 2048): the same outputs as jf_topk_slots, i.e.
+/* jf_topk_slots on the kernels of the fused step: the same outputs as jf_topk_slots, i.e.
  * topk_slots_kernel_v5 / topk_slots_stats_kernel_v5 (jetfire_vllm/csrc/int3_qk_scores.cu:426-554,
  * jetfire_vllm/csrc/int8tc_qk_scores.cu:1678-1823).  workspace: jf_topk_slots_fast_workspace_bytes(). */
 size_t jf_topk_slots_fast_workspace_bytes(int B, int H_q, int max_S, int top_k);

@@ -28,8 +28,8 @@ from . import release_policy
 from .config import get_jetfire_config
 from .kv_pool import get_global_kv_pool_manager
 
-# correction widths the fused kernels take; the split entry points go up to 8192
-FUSED_SUPPORTED_TOP_K = (32, 64, 128, 256, 512, 1024, 2048)
+# correction widths the fused kernels take (all the split entry points take)
+FUSED_SUPPORTED_TOP_K = ops.FUSED_TOP_K
 SPLIT_SUPPORTED_TOP_K = ops.SUPPORTED_TOP_K
 
 _TOPK_CLAMP_LOGGED: set = set()

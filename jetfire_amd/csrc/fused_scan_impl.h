@@ -91,7 +91,8 @@ typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
 //               merge is the FS_STAGE_A one)
 constexpr int FS_FULL = 0, FS_STAGE_A = 1, FS_STAGE_B = 2, FS_TOPK = 3;
 
-constexpr int FS_MAX_TOPK = 2048;      // winners cached in LDS by the merge kernel
+constexpr int FS_MAX_TOPK = 8192;      // widest correction
+constexpr int FS_LDS_TOPK = 2048;      // winners the merge kernel keeps in static LDS; wider ones go to dynamic LDS
 constexpr long long FS_MAX_SLOTS = 1ll << 26;  // slots per kv-head tensor: 64-byte rows, 32-bit row offsets (4 GB)
 constexpr int FS_CAND_SLACK = 256;     // extra candidate slots per (row, split): room for the whole cut bucket
 
@@ -1566,7 +1567,7 @@ constexpr int MG_LIGHT_THREADS = 256, MG_LIGHT_REGK = 16, MG_LIGHT_TOPK = 512;  
 // new candidate list; the final merge (PARTIAL = false, mg_parts > 1) reads these lists instead of the
 // scan's.  The top K of a union is the top K of the parts' top K's, ties included: a candidate that a part
 // drops is beaten by K candidates of that part.
-template <int MODE, int VBITS, int NG, int MG_THREADS, int MG_REGK, bool PARTIAL>
+template <int MODE, int VBITS, int NG, int MG_THREADS, int MG_REGK, bool PARTIAL, bool WIDE = false>
 __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) {
   static_assert(!(PARTIAL && MODE == FS_STAGE_B), "Stage B alone selects nothing");
   constexpr int MG_WAVES = MG_THREADS / 64;
@@ -1585,7 +1586,7 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   static_assert(MG_THREADS % D == 0 && VGRP % (MG_THREADS / D) == 0 && VWAVES % MG_WAVES == 0, "whole roles per thread group / wavefront");
   // the light shape (many rows per launch, few candidates per row) trades table sizes for workgroups per CU
   constexpr int MG_BT = (MG_THREADS >= 1024) ? MG_BT_LDS : 1024;  // block-table entries cached in LDS
-  constexpr int MG_WIN = (MG_THREADS >= 1024) ? FS_MAX_TOPK : 512;  // widest correction of this shape
+  constexpr int MG_WIN = (MG_THREADS >= 1024) ? FS_LDS_TOPK : 512;  // widest correction of this shape (WIDE: any)
   __shared__ int hist[MG_BINS];
   __shared__ uint32_t lkey[MG_LIST];
   __shared__ float coef_sh[MG_MAX_SPLITS];
@@ -1593,8 +1594,12 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   __shared__ int bt_sh[MG_BT];
   // winners: key and position while they are selected; the thread that turns winner r into its softmax weight and
   // paged slot overwrites the two entries in place (weight bits over the key, slot over the position)
-  __shared__ uint32_t win_key[MG_WIN];
-  __shared__ int win_idx[MG_WIN];
+  // (WIDE, corrections beyond FS_LDS_TOPK: the two arrays are the launch's dynamic LDS, top_k entries each)
+  __shared__ uint32_t win_key_s[WIDE ? 1 : MG_WIN];
+  __shared__ int win_idx_s[WIDE ? 1 : MG_WIN];
+  extern __shared__ __align__(16) uint32_t win_dyn[];
+  uint32_t* const win_key = WIDE ? win_dyn : win_key_s;
+  int* const win_idx = WIDE ? reinterpret_cast<int*>(win_dyn + p.top_k) : win_idx_s;
   __shared__ uint32_t cnt_a[MG_REGK / 4 * MG_WAVES];  // packed (winners, ties) per (group, wavefront)
   __shared__ float red_sh[VGRP][D];
   __shared__ float old_sh[VWAVES][D];
@@ -2349,6 +2354,24 @@ inline bool scheme_any_group(int scheme) { return known_scheme(scheme) && scheme
 inline int scheme_ng(int scheme, int group_size) { return scheme_any_group(scheme) ? D / group_size : 1; }
 
 
+// A merge kernel whose winners live in dynamic LDS (corrections wider than FS_LDS_TOPK): 8 bytes per winner; the
+// dynamic-LDS limit of the instantiation is raised once.
+template <void (*KERN)(FusedParams)>
+int launch_wide_merge(dim3 grid, const FusedParams& p, hipStream_t st) {
+  static std::mutex mu;
+  static bool raised = false;
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    if (!raised) {
+      JF_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(KERN), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       FS_MAX_TOPK * 8));
+      raised = true;
+    }
+  }
+  hipLaunchKernelGGL(KERN, grid, dim3(1024), (size_t)p.top_k * 8, st, p);
+  return JF_OK;
+}
+
 // The whole step on caller-provided workspace memory; every public entry point of the fused forms ends here.
 // MODE FS_FULL: all arguments as in jf_fused_scan_topk.  FS_STAGE_A: the value side, o_hat, o_old_unnorm, W are
 // unused; top_k == 0 asks for the scores alone (then nothing but `scores` is written and no workspace is needed).
@@ -2384,7 +2407,7 @@ static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_
   const bool scores_only = (MODE == FS_STAGE_A) && top_k == 0;
   if (scores_only) top_k = 32;  // (any valid width: the plan depends on it, the kernel stops before using it)
   JF_CHECK_ARG(is_pow2(top_k) && top_k >= 32 && top_k <= FS_MAX_TOPK,
-               "fused_scan: unsupported top_k=%d (supported: 32,64,128,256,512,1024,2048; larger widths use the split-form operators)", top_k);
+               "fused_scan: unsupported top_k=%d (supported: the powers of two from 32 to 8192)", top_k);
   JF_CHECK_ARG(max_S <= 262144, "fused_scan: max_S=%d exceeds supported limit (262144)", max_S);
   JF_CHECK_ARG((int64_t)max_blocks * block_size >= max_S, "fused_scan: block_table does not cover max_S");
   // (a row's byte offset inside one kv-head's tensor is formed in 32 bits: rows of at most 64 bytes)
@@ -2477,10 +2500,13 @@ static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_
 #undef JF_FUSED_CASE
   if (rc != JF_OK || scores_only) return rc;
   dim3 mgrid(B, H_q);
+  const bool wide = top_k > FS_LDS_TOPK;  // the winners' arrays do not fit the kernels' static LDS
   if (p.mg_parts > 1) {  // first stage: every part's top_k, as new candidate lists (the same kernel for every form)
     const dim3 pgrid(B, H_q, p.mg_parts);
-    if ((long long)p.mg_spp * p.Kc > MG_REG_CANDS) hipLaunchKernelGGL((fused_merge_kernel<FS_FULL, 4, 1, 1024, 32, true>), pgrid, dim3(1024), 0, st, p);
+    if (wide) rc = launch_wide_merge<fused_merge_kernel<FS_FULL, 4, 1, 1024, 32, true, true>>(pgrid, p, st);
+    else if ((long long)p.mg_spp * p.Kc > MG_REG_CANDS) hipLaunchKernelGGL((fused_merge_kernel<FS_FULL, 4, 1, 1024, 32, true>), pgrid, dim3(1024), 0, st, p);
     else hipLaunchKernelGGL((fused_merge_kernel<FS_FULL, 4, 1, 1024, 8, true>), pgrid, dim3(1024), 0, st, p);
+    if (rc != JF_OK) return rc;
     JF_CHECK_LAUNCH();
   }
   const bool big = (MODE != FS_STAGE_B) &&
@@ -2493,14 +2519,18 @@ static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_
                      (long long)B * H_q > (long long)device_cus() && (long long)p.n_splits * p.Kc <= MG_LIGHT_THREADS * MG_LIGHT_REGK;
 #define JF_MERGE(VB, NGG)                                                                                            \
   do {                                                                                                               \
-    if (big) hipLaunchKernelGGL((fused_merge_kernel<MODE, VB, NGG, 1024, 32, false>), mgrid, dim3(1024), 0, st, p); \
+    if (wide) {                                                                                                      \
+      if constexpr (MODE == FS_STAGE_B) rc = launch_wide_merge<fused_merge_kernel<MODE, VB, NGG, 1024, 8, false, true>>(mgrid, p, st); \
+      else rc = launch_wide_merge<fused_merge_kernel<MODE, VB, NGG, 1024, 32, false, true>>(mgrid, p, st);            \
+    } else if (big) hipLaunchKernelGGL((fused_merge_kernel<MODE, VB, NGG, 1024, 32, false>), mgrid, dim3(1024), 0, st, p); \
     else if (light) {                                                                                                \
       if constexpr (MODE == FS_FULL)                                                                                 \
         hipLaunchKernelGGL((fused_merge_kernel<FS_FULL, VB, NGG, MG_LIGHT_THREADS, MG_LIGHT_REGK, false>), mgrid, dim3(MG_LIGHT_THREADS), 0, st, p); \
     } else hipLaunchKernelGGL((fused_merge_kernel<MODE, VB, NGG, 1024, 8, false>), mgrid, dim3(1024), 0, st, p);       \
   } while (0)
   if constexpr (MODE == FS_STAGE_A || MODE == FS_TOPK) {  // no value rows are read: one instantiation serves every format
-    if (big) hipLaunchKernelGGL((fused_merge_kernel<FS_STAGE_A, 4, 1, 1024, 32, false>), mgrid, dim3(1024), 0, st, p);
+    if (wide) rc = launch_wide_merge<fused_merge_kernel<FS_STAGE_A, 4, 1, 1024, 32, false, true>>(mgrid, p, st);
+    else if (big) hipLaunchKernelGGL((fused_merge_kernel<FS_STAGE_A, 4, 1, 1024, 32, false>), mgrid, dim3(1024), 0, st, p);
     else hipLaunchKernelGGL((fused_merge_kernel<FS_STAGE_A, 4, 1, 1024, 8, false>), mgrid, dim3(1024), 0, st, p);
   } else if (scheme % 10 == 2) {  // INT2 values
     if (NGv == 2) JF_MERGE(2, 2);
@@ -2513,6 +2543,7 @@ static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_
     else JF_MERGE(4, 1);
   }
 #undef JF_MERGE
+  if (rc != JF_OK) return rc;
   JF_CHECK_LAUNCH();
   return JF_OK;
 }

@@ -39,7 +39,7 @@ extern "C" int jf_stage_a_topk_asym(int group_size, const uint16_t* q, const uin
                                nullptr, nullptr, workspace, workspace_bytes, stream);
 }
 
-// The selection alone (scores are an input): the fast form of jf_topk_slots for top_k <= 2048.  The rows are grouped
+// The selection alone (scores are an input): the fast form of jf_topk_slots.  The rows are grouped
 // four (or two, or one) to a workgroup; nothing else depends on the grouping.
 extern "C" int jf_topk_slots_fast(const float* scores, const int32_t* seq_lens, const int64_t* block_table, int B, int H_q,
                                   int max_S, int max_blocks, int block_size, int top_k, int64_t* topk_idx,

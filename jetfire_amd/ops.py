@@ -16,7 +16,7 @@ from . import _lib
 
 HEAD_DIM = 128
 SUPPORTED_TOP_K = (32, 64, 128, 256, 512, 1024, 2048, 4096, 8192)
-FUSED_TOP_K = (32, 64, 128, 256, 512, 1024, 2048)      # widths of the one-pass form and of the fast stage-wise forms
+FUSED_TOP_K = SUPPORTED_TOP_K                           # widths of the one-pass form and of the fast stage-wise forms
 FUSED_MAX_SLOTS = 1 << 26                               # slots per kv-head tensor those forms address (4 GB of 64-byte rows)
 
 _workspaces: dict = {}

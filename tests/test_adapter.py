@@ -28,7 +28,7 @@ def test_select_top_k_matches_the_reference_table(adapter):
     for req in (16, 32, 100, 256, 300, 1024, 5000):
         for n in (0, 1, 31, 32, 33, 255, 256, 257, 4096):
             assert _select_top_k(req, n, supported) == O.select_top_k(req, n, supported), (req, n)
-    assert FUSED_SUPPORTED_TOP_K == supported + (2048,)
+    assert FUSED_SUPPORTED_TOP_K == supported + (2048, 4096, 8192)
     hm = _get_head_map_cpu(2, 8, 4, 5).numpy()
     assert np.array_equal(hm, O.head_map(2, 8, 4, 5))
 
@@ -598,10 +598,9 @@ def test_release_policy_selects_the_named_split_kernels(adapter, monkeypatch, sc
 
 
 @pytest.mark.gpu
-def test_corrections_wider_than_the_fused_form_run_the_split_operators(adapter, monkeypatch):
-    """JETFIRE_TOPK=4096 on a fused scheme: the width is kept (not clamped to the fused form's 2048) and the step
-    runs Stage A and Stage B as separate operators; with nearly every position corrected the output is the exact
-    attention over the bf16 shadow."""
+def test_a_wide_correction_keeps_its_width(adapter, monkeypatch):
+    """JETFIRE_TOPK=4096: the width reaches the fused step unclamped; with nearly every position corrected the output
+    is the exact attention over the bf16 shadow."""
     from jetfire_amd import ops as jops
     for name in list(__import__("os").environ):
         if name.startswith("JETFIRE_"):
@@ -633,9 +632,8 @@ def test_corrections_wider_than_the_fused_form_run_the_split_operators(adapter, 
     assert adapter.try_jetfire_decode(impl=impl, layer=layer, query=q, attn_metadata=meta, output=out) is out
     torch.cuda.synchronize()
     names = [c[0] for c in called]
-    assert "fused_attn_topk" not in names and "int3_qk_scores_topk" in names
-    stage_a = next(c for c in called if c[0] == "int3_qk_scores_topk")
-    assert int(stage_a[1][-1]) == K                                   # the configured width reaches Stage A
+    assert names == ["fused_attn_topk"]
+    assert int(called[0][1][12]) == K                                 # the configured width reaches the fused step
     G = Hq // Hkv
     att = torch.softmax(torch.einsum("hd,shd->hs", q[0].float(), k.float().repeat_interleave(G, dim=1)) * D ** -0.5, dim=-1)
     ref = torch.einsum("hs,shd->hd", att, v.float().repeat_interleave(G, dim=1))

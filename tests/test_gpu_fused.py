@@ -96,7 +96,9 @@ CASES = [
     ("k3v3", 1, 8, 2, 5000, [4987], 256), ("k4v3", 1, 8, 2, 5000, [4987], 512), ("k2v3", 1, 8, 2, 5000, [4987], 1024),
     ("k3v3", 1, 4, 4, 300, None, 32), ("k4v3", 1, 4, 2, 300, None, 64), ("k3v3_g128", 1, 16, 1, 600, None, 64),
     ("k2v3", 1, 16, 1, 600, None, 64),
-    # the widest correction of the fused form
+    # wide corrections: the merge kernels keep the winners in dynamic LDS beyond 2048
+    ("k3v2", 1, 8, 2, 9000, [8987], 4096), ("k4v4", 2, 4, 2, 9000, [5000, 9000], 8192), ("k3v3", 1, 8, 1, 4200, None, 4096),
+    ("a2v2", 1, 4, 4, 8192, None, 8192), ("k2v4", 1, 28, 4, 6000, None, 4096),
     ("k3v2", 1, 8, 2, 5000, [4987], 2048), ("k4v4", 2, 8, 2, 3000, [1000, 3000], 2048),
     ("k3v3", 1, 32, 4, 6000, None, 2048), ("k2v4", 2, 4, 4, 2048, [2048, 2047], 2048),
     # asymmetric INT2 keys (a zero-point per group) with every value format
@@ -148,6 +150,8 @@ def test_fused_scan_matches_oracle(scheme, B, Hq, Hkv, S, lens, K):
     ("k3v4", 10000, [9989], 256, 512), ("k4v2", 10000, [9000], 512, 768),      # two-stage merges of the mixed pairs
     ("k3v2", 20000, [19989], 2048, 512),   # every position a candidate, 40 lists: two-stage merge at the widest correction
     ("k4v4", 40000, [39000], 2048, 0),     # the planner's own split: lists of 2304 entries, first stage beyond the registers
+    ("k3v2", 40000, [39990], 4096, 0),     # every position a candidate; two-stage merge whose parts exceed the registers
+    ("k4v4", 20000, [19000], 8192, 1024),  # single stage over every position, most candidates re-read from global memory
 ])
 def test_fused_scan_with_forced_split_length(scheme, S, lens, K, split_len):
     from jetfire_amd import _lib

@@ -25,7 +25,7 @@ def _draw(seed):
     S = int(rng.choice([48, 200, 777, 1500, 2600, 4100]))
     lens = [int(x) for x in rng.integers(0, S + 1, size=B)]
     lens[int(rng.integers(0, B))] = S                       # at least one full-length row
-    K = int(rng.choice([32, 64, 128, 256, 512, 1024, 2048]))
+    K = int(rng.choice([32, 64, 128, 256, 512, 1024, 2048, 4096]))
     split = int(rng.choice([0, 0, 256, 512, 1024]))
     return scheme, B, G * Hkv, Hkv, S, lens, K, split
 
