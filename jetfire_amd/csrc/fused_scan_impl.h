@@ -2202,7 +2202,8 @@ inline double merge_plan(int rows, int ns, int kc, int top_k, int* parts_out, in
   const double wide = 1.5 * (top_k > 256 ? (double)top_k / 256.0 - 1.0 : 0.0);  // slots and pre-correction of the winners
   double best = merge_pass_us(kMergeFixed, (long)ns * kc) + wide;
   if ((long long)ns * kc <= MG_REG_CANDS || ns < 4) return best;
-  int cap = MG_REG_CANDS / top_k;
+  // (wide corrections run the 32-register shape throughout: its 32768 candidates bound the final merge)
+  int cap = (top_k > FS_LDS_TOPK ? 4 * MG_REG_CANDS : MG_REG_CANDS) / top_k;
   if (cap > ns / 2) cap = ns / 2;
   for (int parts = 2; parts <= cap; ++parts) {
     const int spp = (ns + parts - 1) / parts;
