@@ -19,6 +19,9 @@
 #include <thread>
 #include <vector>
 
+#include <pthread.h>
+#include <sched.h>
+
 #if defined(__x86_64__)
 #include <immintrin.h>
 #endif
@@ -259,7 +262,35 @@ class Pool {
     }
     active_.fetch_sub(1, std::memory_order_acq_rel);
   }
+  // JETFIRE_CPU_ATTN_PIN=1 (jetfire_vllm/csrc/cpu_topk_attn.cpp:895-905, jetfire_pool.h:141-149): worker i stays on
+  // one core.  The reference binds it to core i; here it is the i-th core the process may run on (the same core
+  // when every core is allowed, and still a valid one inside a restricted cpu set).  More workers than allowed
+  // cores: the surplus stays unpinned.
+  static bool pin_workers() {
+    static const bool on = [] {
+      const char* e = std::getenv("JETFIRE_CPU_ATTN_PIN");
+      return e != nullptr && std::atoi(e) == 1;
+    }();
+    return on;
+  }
+  static void pin_to_allowed_core(int index) {
+    cpu_set_t allowed;
+    CPU_ZERO(&allowed);
+    if (sched_getaffinity(0, sizeof(allowed), &allowed) != 0) return;
+    int seen = 0;
+    for (int c = 0; c < CPU_SETSIZE; ++c) {
+      if (!CPU_ISSET(c, &allowed)) continue;
+      if (seen++ == index) {
+        cpu_set_t one;
+        CPU_ZERO(&one);
+        CPU_SET(c, &one);
+        (void)pthread_setaffinity_np(pthread_self(), sizeof(one), &one);
+        return;
+      }
+    }
+  }
   void worker(uint64_t seen, int index) {
+    if (pin_workers()) pin_to_allowed_core(index);
     for (;;) {
       bool got = false;
       const auto t0 = std::chrono::steady_clock::now();

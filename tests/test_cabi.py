@@ -255,6 +255,52 @@ def test_cpu_pool_backs_up_a_row_whose_worker_has_stalled():
     ops.set_cpu_attn_threads(2)
 
 
+def test_cpu_pool_pins_its_workers_on_request():
+    """JETFIRE_CPU_ATTN_PIN=1 (read once per process, so a child process): every worker ends up on one core of the
+    set the process may use, each on a different one, and the rows come out as without the switch."""
+    import os
+    import subprocess
+    import sys
+    code = r"""
+import os, sys, glob, numpy as np, torch
+sys.path.insert(0, %r)
+from jetfire_amd import ops
+from oracle import jetfire_oracle as O
+from tests.helpers import bf16_tensor, make_case
+B, Hq, Hkv, K = 2, 8, 2, 32
+c = make_case(5, B, Hq, Hkv, 256, 3, 2, 64, ragged=False)
+rng = np.random.default_rng(1)
+hm = torch.from_numpy(O.head_map(B, Hq, Hq // Hkv, K))
+q = bf16_tensor(O.bf16_round((rng.standard_normal((B, Hq, 128)) / np.sqrt(128)).astype(np.float32)))
+ts = torch.from_numpy(rng.integers(-1, c["K"].shape[1], size=(B, Hq, K)).astype(np.int64))
+out = torch.zeros(B, Hq, 128, dtype=torch.bfloat16)
+ops.set_cpu_attn_threads(3)
+ops.cpu_topk_attn(q, bf16_tensor(c["K"]), bf16_tensor(c["V"]), hm, ts, out, 0.09)
+import time
+time.sleep(0.5)            # (a short job can end before the last worker thread has run its first instruction)
+masks = []
+for t in glob.glob("/proc/self/task/*/status"):
+    txt = open(t).read()
+    allowed = [l.split(":")[1].strip() for l in txt.splitlines() if l.startswith("Cpus_allowed_list")][0]
+    masks.append(allowed)
+print("MASKS", ";".join(sorted(masks)))
+print("SUM", float(out.float().abs().sum()))
+""" % os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    runs = {}
+    for pin in ("0", "1"):
+        env = dict(os.environ, JETFIRE_CPU_ATTN_PIN=pin)
+        res = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=300)
+        assert res.returncode == 0, res.stderr[-2000:]
+        lines = dict(l.split(" ", 1) for l in res.stdout.splitlines() if l.startswith(("MASKS", "SUM")))
+        runs[pin] = lines
+    assert runs["0"]["SUM"] == runs["1"]["SUM"]
+    allowed = sorted(os.sched_getaffinity(0))
+    single = [m for m in runs["1"]["MASKS"].split(";") if m.isdigit()]       # threads bound to exactly one core
+    if len(allowed) >= 3:
+        assert sorted(int(m) for m in single) == allowed[:3], (single, allowed)
+    assert not [m for m in runs["0"]["MASKS"].split(";") if m.isdigit()] or len(allowed) == 1
+
+
 def test_cpu_topk_attn_single_slot_returns_the_value_row():
     from jetfire_amd import ops
     c = make_case(60, 1, 4, 2, 64, 3, 2, 64, ragged=False)
