@@ -90,6 +90,16 @@ int jf_quant_write_int4_sym_kv(const uint16_t* key, int64_t k_stride_t, int64_t 
                                uint16_t* v_scale, int64_t v_scale_stride_h, int64_t v_scale_stride_slot,
                                int64_t num_slots, int group_size, void* stream);
 
+/* Dequantise packed rows back to bf16.  Replaces unpack (jetfire_vllm/kernels/intN_pack.py:227-311):
+ * out[r, c] = bf16(f32(code - 2^(nbits-1)) * f32(scale[r, c / group_size])); when zps is not NULL the
+ * rounded product is widened, f32(zp) added and the sum rounded to bf16 again (:251-256).  data is
+ * (rows, 128 * nbits / 8) uint8 with a row stride in bytes; scales / zps are (rows, 128 / group_size) bf16 and
+ * out is (rows, 128) bf16, their row strides in elements.  nbits in {2,3,4}; group_size a power of two in
+ * 8..128; output rows 16-byte aligned, INT4 data rows 4-byte and INT2 data rows 2-byte aligned. */
+int jf_unpack(const uint8_t* data, int64_t data_stride_row, const uint16_t* scales, int64_t scale_stride_row,
+              const uint16_t* zps, int64_t zp_stride_row, int64_t rows, int group_size, int nbits,
+              uint16_t* out, int64_t out_stride_row, void* stream);
+
 /* Mirror of appended rows into the bf16 host shadow the CPU correction reads: k_shadow[h, slots[t], :] =
  * key[t, h, :], the same for V; slots[t] < 0 (padding) and slots[t] >= num_slots are skipped.  Replaces the
  * reference's shadow mirror: the serial host copy + index_copy_ (jetfire_vllm/adapter/cache_store.py:686-759),

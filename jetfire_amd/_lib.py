@@ -28,6 +28,7 @@ SIGNATURES = {
     "jf_int3_qk_scores": (I, [P, P, P, P, P, I, I, I, I, I, L, I, I, F, P, P]),
     "jf_intn_qk_scores": (I, [I, P, P, P, P, P, P, I, I, I, I, I, L, I, I, F, P, P]),
     "jf_quant_write_int2_asym": (I, [P, L, L, P, L, I, P, L, L, P, L, L, P, L, L, L, I, P]),
+    "jf_unpack": (I, [P, L, P, L, P, L, L, I, I, P, L, P]),
     "jf_int8tc_qk_scores": (I, [P, P, P, P, P, I, I, I, I, I, L, I, F, P, P]),
     "jf_topk_slots": (I, [P, P, P, I, I, I, I, I, I, P, P, P, P, P]),
     "jf_softmax_v_workspace_bytes": (Z, [I, I, I]),

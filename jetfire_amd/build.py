@@ -23,6 +23,7 @@ SOURCES = (     # (the long compilations first: the pool starts them together)
     "fused_full_d.hip",
     "fused_full_e.hip",
     "quant_write.hip",
+    "unpack.hip",
     "shadow_write.hip",
     "qk_scores.hip",
     "topk.hip",

@@ -169,6 +169,70 @@ def fused_quant_write_int4_sym_kv(key_tok, value_tok, slot_idx, k_data, k_scales
         k_data.shape[1], int(group_size), _stream(key_tok)))
 
 
+def packed_dim(head_dim: int, nbits: int) -> int:
+    """intN_pack.py:35-44: bytes of one packed row."""
+    _check(nbits in (2, 3, 4), f"Unsupported nbits={nbits}")
+    _check(head_dim % 8 == 0, f"head_dim={head_dim} must be a multiple of 8")
+    return head_dim * nbits // 8
+
+
+def _rows_for_pack(x, name: str):
+    _check(x.is_cuda and x.dtype == torch.bfloat16, f"{name}: x must be bf16 on the GPU")
+    _check(x.dim() >= 1 and x.shape[-1] == HEAD_DIM, f"{name}: the last dimension must be {HEAD_DIM}")
+    return x.reshape(-1, 1, HEAD_DIM), tuple(x.shape[:-1])
+
+
+def quantize_and_pack(x, group_size: int = 128, nbits: int = 4):
+    """intN_pack.py:60-107 on the GPU: (..., 128) bf16 -> data (..., 128 * nbits / 8) uint8, scales
+    (..., 128 / group_size) bf16.  The rows go through the cache writer with the identity slot mapping."""
+    _check(nbits in (2, 3, 4), f"Unsupported nbits={nbits}")
+    rows, lead = _rows_for_pack(x, "quantize_and_pack")
+    n = rows.shape[0]
+    data = torch.empty(1, n, HEAD_DIM * nbits // 8, dtype=torch.uint8, device=x.device)
+    scales = torch.empty(1, n, HEAD_DIM // group_size, dtype=torch.bfloat16, device=x.device)
+    if n:
+        _quant_write(rows, torch.arange(n, dtype=torch.int64, device=x.device), data, scales, group_size, nbits)
+    return data.view(*lead, data.shape[-1]), scales.view(*lead, scales.shape[-1])
+
+
+def quantize_and_pack_asym(x, group_size: int = 128, nbits: int = 2):
+    """intN_pack.py:110-169 on the GPU, for the one width whose zero-point form has kernels (INT2):
+    returns data, scales, zps."""
+    if nbits != 2:
+        raise NotImplementedError("only INT2 has an asymmetric (zero-point) form in this library")
+    rows, lead = _rows_for_pack(x, "quantize_and_pack_asym")
+    n = rows.shape[0]
+    data = torch.empty(1, n, HEAD_DIM // 4, dtype=torch.uint8, device=x.device)
+    scales = torch.empty(1, n, HEAD_DIM // group_size, dtype=torch.bfloat16, device=x.device)
+    zps = torch.empty_like(scales)
+    if n:
+        fused_quant_write_int2_asym(rows, torch.arange(n, dtype=torch.int64, device=x.device), data, scales, zps,
+                                    group_size)
+    return data.view(*lead, data.shape[-1]), scales.view(*lead, scales.shape[-1]), zps.view(*lead, zps.shape[-1])
+
+
+def unpack(data, scales, group_size: int = 128, nbits: int = 4, zps=None):
+    """intN_pack.py:227-256 on the GPU: packed rows -> dequantised (..., 128) bf16."""
+    lib = _lib.load()
+    _check(nbits in (2, 3, 4), f"Unsupported nbits={nbits}")
+    _check(data.is_cuda and data.dtype == torch.uint8 and data.shape[-1] == HEAD_DIM * nbits // 8,
+           f"unpack: data must be (..., {HEAD_DIM * nbits // 8}) uint8 on the GPU")
+    ng = HEAD_DIM // group_size
+    lead = tuple(data.shape[:-1])
+    for t, name in ((scales, "scales"), (zps, "zps")):
+        if t is not None:
+            _check(t.is_cuda and t.dtype == torch.bfloat16 and tuple(t.shape) == lead + (ng,),
+                   f"unpack: {name} must be {lead + (ng,)} bf16 on the GPU")
+    d2 = data.reshape(-1, data.shape[-1]).contiguous()
+    s2 = scales.reshape(-1, ng).contiguous()
+    z2 = zps.reshape(-1, ng).contiguous() if zps is not None else None
+    out = torch.empty(d2.shape[0], HEAD_DIM, dtype=torch.bfloat16, device=data.device)
+    _lib.check(lib.jf_unpack(d2.data_ptr(), d2.stride(0), s2.data_ptr(), s2.stride(0), _ptr(z2),
+                             z2.stride(0) if z2 is not None else 0, d2.shape[0], int(group_size), nbits,
+                             out.data_ptr(), out.stride(0), _stream(data)))
+    return out.view(*lead, HEAD_DIM)
+
+
 def host_buffer_device_pointer(t: torch.Tensor) -> int:
     """Address under which the GPU reaches the pinned host tensor `t`; raises for pageable memory."""
     import ctypes

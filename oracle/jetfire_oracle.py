@@ -221,9 +221,16 @@ def dequant(data, scale_bits, nbits: int, group_size: int, *, bf16: bool = True)
     return bf16_round(out) if bf16 else out
 
 
-def unpack(data, scale_bits, group_size: int = 128, nbits: int = 4) -> np.ndarray:
-    """intN_pack.py:227-311: dequantised values rounded to the scale dtype (bf16)."""
-    return dequant(data, scale_bits, nbits, group_size, bf16=True)
+def unpack(data, scale_bits, group_size: int = 128, nbits: int = 4, zp_bits=None) -> np.ndarray:
+    """intN_pack.py:227-311: dequantised values rounded to the scale dtype (bf16).  With zero-points the
+    rounded product is widened, the zero-point added in fp32 and the sum rounded again (:251-256): two
+    roundings, unlike the fused multiply-add of the Stage A kernel (dequant_asym_bf16)."""
+    out = dequant(data, scale_bits, nbits, group_size, bf16=True)
+    if zp_bits is None:
+        return out
+    z = bf16_bits_to_f32(zp_bits).reshape(*out.shape[:-1], -1)
+    z = np.repeat(z, group_size, axis=-1).astype(np.float32)
+    return bf16_round((out.astype(np.float32) + z).astype(np.float32))
 
 
 def write_cache(x, slots, data, scale_bits, group_size: int, nbits: int) -> None:

@@ -151,6 +151,87 @@ def test_asymmetric_int2_pack_and_scores(gs):
         o.fused_quant_write_int2_asym(bf16_tensor(wide).cuda()[..., 2:130], torch.from_numpy(slots).cuda(), data, sc, zp, gs)
 
 
+@pytest.mark.parametrize("gs", (32, 64, 128))
+@pytest.mark.parametrize("bits", (2, 3, 4))
+def test_whole_tensor_quantise_and_unpack_match_the_oracle(bits, gs):
+    """The reference's tensor-level API (kernels/intN_pack.py:60-107,227-311) through the loader module of its
+    name: packed bytes, scale bits and the dequantised bf16 values bit-exact against the oracle, for a
+    tensor with several leading dimensions, an odd row count and rows that hit the clamp."""
+    from jetfire_amd.kernels import intN_pack as P
+    rng = np.random.default_rng(100 * bits + gs)
+    x = O.bf16_round((rng.standard_normal((3, 5, 7, 128)) * np.exp(rng.standard_normal((3, 5, 7, 1)))).astype(np.float32))
+    x[0, 0, 0] = 0.0
+    x[1, 2, 3, ::2] = 0.5                                   # exact halves of the scale: round-half-even ties
+    xd = bf16_tensor(x).cuda()
+    data, scales = P.quantize_and_pack(xd, group_size=gs, nbits=bits)
+    rd, rs = O.quantize_and_pack(x, gs, bits)
+    assert data.shape == (3, 5, 7, P.packed_dim(128, bits)) and scales.shape == (3, 5, 7, 128 // gs)
+    assert np.array_equal(data.cpu().numpy(), rd) and np.array_equal(bf16_to_bits(scales), rs)
+    back = P.unpack(data, scales, group_size=gs, nbits=bits)
+    assert back.shape == x.shape and back.dtype == torch.bfloat16
+    assert np.array_equal(bf16_to_bits(back), O.f32_to_bf16_bits(O.unpack(rd, rs, gs, bits)))
+    # rows that are a slice of a wider tensor (part of one kv-head of a cache)
+    cache = torch.zeros(4, 40, P.packed_dim(128, bits), dtype=torch.uint8, device="cuda")
+    cache[2, :35] = data.view(-1, data.shape[-1])[:35]
+    sc = torch.ones(4, 40, 128 // gs, dtype=torch.bfloat16, device="cuda")
+    sc[2, :35] = scales.view(-1, scales.shape[-1])[:35]
+    part = P.unpack(cache[2, 3:35], sc[2, 3:35], group_size=gs, nbits=bits)
+    assert torch.equal(part, back.view(-1, 128)[3:35])
+    # nothing to do
+    e_d, e_s = P.quantize_and_pack(xd[:0], group_size=gs, nbits=bits)
+    assert e_d.shape == (0, 5, 7, P.packed_dim(128, bits)) and P.unpack(e_d, e_s, gs, bits).shape == (0, 5, 7, 128)
+
+
+@pytest.mark.parametrize("gs", (32, 64, 128))
+def test_whole_tensor_asymmetric_int2_and_unpack_with_zero_points(gs):
+    from jetfire_amd.kernels import fused_quantize as FQ, intN_pack as P
+    rng = np.random.default_rng(300 + gs)
+    x = O.bf16_round((rng.standard_normal((11, 3, 128)) * 0.7 + rng.standard_normal((11, 3, 1))).astype(np.float32))
+    xd = bf16_tensor(x).cuda()
+    data, scales, zps = P.quantize_and_pack_asym(xd, group_size=gs, nbits=2)
+    rd, rs, rz = O.quantize_and_pack_asym(x, gs, 2)
+    assert np.array_equal(data.cpu().numpy(), rd)
+    assert np.array_equal(bf16_to_bits(scales), rs) and np.array_equal(bf16_to_bits(zps), rz)
+    back = P.unpack(data, scales, group_size=gs, nbits=2, zps=zps)
+    assert np.array_equal(bf16_to_bits(back), O.f32_to_bf16_bits(O.unpack(rd, rs, gs, 2, zp_bits=rz)))
+    # the one-launch names of the reference (kernels/fused_quantize.py:214-284) are the same functions
+    d2, s2, z2 = FQ.fused_quantize_and_pack_int2_asym(xd, gs)
+    assert torch.equal(d2, data) and torch.equal(s2, scales) and torch.equal(z2, zps)
+    d3, s3 = FQ.fused_quantize_and_pack_int2(xd, gs)
+    rd3, rs3 = O.quantize_and_pack(x, gs, 2)
+    assert np.array_equal(d3.cpu().numpy(), rd3) and np.array_equal(bf16_to_bits(s3), rs3)
+    with pytest.raises(NotImplementedError):
+        P.quantize_and_pack_asym(xd, group_size=gs, nbits=4)
+
+
+@pytest.mark.parametrize("bits", (3, 4))
+def test_unpack_with_zero_points_of_wider_codes_rounds_twice(bits):
+    """Zero-points over INT3 / INT4 codes have no writer here, but unpack takes them as the reference does;
+    with 3- and 4-bit codes the product needs more than bf16's 8 bits, so the two roundings show."""
+    from jetfire_amd.kernels import intN_pack as P
+    rng = np.random.default_rng(50 + bits)
+    codes = rng.integers(0, 1 << bits, size=(97, 128)).astype(np.uint8)
+    data = O.pack_codes(codes, bits)
+    sb = O.f32_to_bf16_bits((np.exp(rng.standard_normal((97, 2))) * (1 + 2.0 ** -7)).astype(np.float32))
+    zb = O.f32_to_bf16_bits(rng.standard_normal((97, 2)).astype(np.float32))
+    got = P.unpack(torch.from_numpy(data).cuda(), bits_to_bf16(sb).cuda(), 64, bits, zps=bits_to_bf16(zb).cuda())
+    assert np.array_equal(bf16_to_bits(got), O.f32_to_bf16_bits(O.unpack(data, sb, 64, bits, zp_bits=zb)))
+
+
+def test_unpack_refuses_what_it_cannot_read():
+    from jetfire_amd.kernels import intN_pack as P
+    d = torch.zeros(4, 64, dtype=torch.uint8, device="cuda")
+    s = torch.ones(4, 1, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(RuntimeError, match="data must be"):
+        P.unpack(d, s, 128, 3)
+    with pytest.raises(RuntimeError, match="scales must be"):
+        P.unpack(d, s, 64, 4)
+    with pytest.raises(RuntimeError, match="Unsupported nbits"):
+        P.unpack(d, s, 128, 8)
+    with pytest.raises(RuntimeError, match="bf16"):
+        P.quantize_and_pack(torch.zeros(2, 128, device="cuda"), 128, 4)
+
+
 def test_pack_int4_kv_single_launch_matches_two_launches():
     rng = np.random.default_rng(7)
     T, H = 70, 8

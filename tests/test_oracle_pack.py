@@ -205,3 +205,24 @@ def test_asymmetric_int2_quantiser_is_pinned_by_its_closed_form(gs):
     sym_mse = ((O.dequant(sd, ss, 2, gs, bf16=False) - x) ** 2).mean()
     asym_mse = ((xhat.reshape(64, 128) - x) ** 2).mean()
     assert asym_mse <= sym_mse * 1.05
+
+
+def test_unpack_with_zero_points_rounds_twice():
+    """intN_pack.py:251-256 rounds the product to bf16 before the zero-point is added.  Hand-worked case
+    that a single rounding (or a fused multiply-add) fails: code 3 at scale 1 + 2^-7 is 3.0234375, a tie
+    between the bf16 neighbours 3.015625 and 3.03125 that goes to the even one, 3.03125; adding the
+    zero-point -2^-7 gives 3.0234375 again -> 3.03125.  One rounding of 3.0234375 - 0.0078125 = 3.015625
+    would give 3.015625."""
+    codes = np.full((1, 128), 3 + 8, dtype=np.uint8)
+    data = O.pack_codes(codes, 4)
+    sbits = O.f32_to_bf16_bits(np.array([[1.0 + 2.0 ** -7]], dtype=np.float32))
+    zbits = O.f32_to_bf16_bits(np.array([[-(2.0 ** -7)]], dtype=np.float32))
+    assert O.bf16_bits_to_f32(sbits)[0, 0] == 1.0 + 2.0 ** -7      # representable: the case is what it says
+    out = O.unpack(data, sbits, 128, 4, zp_bits=zbits)
+    assert (out == np.float32(3.03125)).all()
+    # plain codebook check: scale 1, zero-point 0.5 shifts the INT2 grid -2..1 to -1.5..1.5
+    c2 = np.tile(np.arange(4, dtype=np.uint8), 32).reshape(1, 128)
+    out = O.unpack(O.pack_codes(c2, 2), O.f32_to_bf16_bits(np.ones((1, 2), np.float32)), 64, 2,
+                   zp_bits=O.f32_to_bf16_bits(np.array([[0.5, -0.5]], np.float32)))
+    assert np.array_equal(out[0, :4], np.array([-1.5, -0.5, 0.5, 1.5], np.float32))
+    assert np.array_equal(out[0, 64:68], np.array([-2.5, -1.5, -0.5, 0.5], np.float32))
