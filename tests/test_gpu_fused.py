@@ -171,6 +171,31 @@ def test_fused_scan_with_forced_split_length(scheme, S, lens, K, split_len):
     assert torch.equal(forced[4], again[4]) and torch.equal(forced[1], again[1])
 
 
+@pytest.mark.parametrize("gs", (128, 64))
+def test_int2_single_call_names_of_the_reference(gs):
+    """int2_fused_attn_topk and int2_fused_attn_topk_v1 (jetfire_vllm/csrc/int2_fused_attn_topk.cu:403-417,
+    int2_fused_attn_topk_v1.cu:581-595): the reference's argument order with the zero-points fourth, four
+    tensors back; scale tensors without the trailing group axis, as the reference passes them at group 128."""
+    from jetfire_amd.kernels.int2_fused_attn_topk import load_int2_fused_attn_topk_ext
+    from jetfire_amd.kernels.int2_fused_attn_topk_v1 import load_int2_fused_attn_topk_v1_ext
+    scheme = "a2v2_g128" if gs == 128 else "a2v2"
+    S, K = 700, 128
+    c = make_case(91 + gs, 2, 8, 2, S, 2, 2, gs, lens=[333, 700], extra_blocks=3, k_asym=True)
+    d = to_device(c)
+    full = run_fused(scheme, c, d, S, K)
+    check_against_oracle(scheme, c, S, K, full)
+    sq = (lambda t: t.squeeze(-1)) if gs == 128 else (lambda t: t)
+    for fn in (load_int2_fused_attn_topk_ext().int2_fused_attn_topk,
+               load_int2_fused_attn_topk_v1_ext().int2_fused_attn_topk_v1):
+        got = fn(d["q"], d["kd"], sq(d["ks"]), sq(d["kz"]), d["vd"], sq(d["vs"]), d["bt"], d["lens"], S, c["Hq"], c["Hkv"],
+                 16, K, SCALE)
+        assert len(got) == 4
+        for a, b in zip(got, full[:4]):
+            assert torch.equal(a, b)
+    with pytest.raises(RuntimeError, match="top_k"):
+        fn(d["q"], d["kd"], d["ks"], d["kz"], d["vd"], d["vs"], d["bt"], d["lens"], S, c["Hq"], c["Hkv"], 16, 96, SCALE)
+
+
 @pytest.mark.parametrize("S,K,split_len", [(600, 64, 0), (10000, 256, 512)])
 def test_fused_scan_ties_go_to_the_lower_position(S, K, split_len):
     # identical keys in every slot -> every score of a head is equal: winners are positions 0..K-1
