@@ -41,6 +41,7 @@
 #include "common.h"
 
 #include <atomic>
+#include <type_traits>
 #include <mutex>
 #include <vector>
 
@@ -238,6 +239,14 @@ __device__ inline void wave_lds_fence() {
 // that are still in flight (the prefetched key / value rows), which no other wavefront consumes.
 __device__ inline void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
+// A copy the compiler cannot see through: the source register is dead afterwards, so a load issued next can
+// write it directly instead of a temporary that is moved into place (after a wait) at the end of the block.
+__device__ inline uint32_t reg_copy(uint32_t v) {
+  uint32_t r;
+  asm volatile("v_mov_b32 %0, %1" : "=v"(r) : "v"(v));
+  return r;
+}
+
 // s_setprio takes an immediate; `p` is a compile-time constant after unrolling
 __device__ inline void set_wave_prio(int p) {
   if (p >= 3) __builtin_amdgcn_s_setprio(3);
@@ -312,16 +321,15 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   // The page-table entry and the query elements of this thread do not depend on the sequence length: they
   // are requested first, so their latency runs in parallel with the load of seq_lens[b] instead of after it.
   const int nch_cover = (n_cover + 63) >> 6;
-  int64_t bt_mine = 0;  // LMAX / 16 <= NT: one entry per thread covers the split
-  if (tid < nch_cover * 4) bt_mine = bt[min((s0 >> 4) + tid, p.max_blocks - 1)];
+  // (both unconditional, on clamped indices: under a condition the compiler waits for each load inside its branch,
+  // one cold miss after the other)
+  const int64_t bt_mine = bt[min((s0 >> 4) + tid, p.max_blocks - 1)];  // LMAX / 16 <= NT: one entry per thread covers the split
   constexpr int QN = NSET * 4 * D;               // elements of the padded query block (whole head sets)
   constexpr int QPT = (QN + NT - 1) / NT;
-  float qv[QPT];
+  uint16_t qraw[QPT];
 #pragma unroll
-  for (int it = 0; it < QPT; ++it) {
-    const int i = it * NT + tid;
-    qv[it] = (i < GA * D) ? bf16_to_f32(p.q[head0 * D + i]) : 0.f;
-  }
+  for (int it = 0; it < QPT; ++it) qraw[it] = HAS_K ? p.q[head0 * D + min(it * NT + tid, GA * D - 1)] : (uint16_t)0;
+  auto q_elem = [&](int it) -> float { return (it * NT + tid < GA * D) ? bf16_to_f32(qraw[it]) : 0.f; };
 
   if (n == 0) {  // nothing valid in this split: padding scores, empty partials
     if (p.scores)
@@ -371,12 +379,8 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   const int t16 = lane & 15, lg = lane >> 4;
   auto issue_k = [&](int chunk) -> KBuf {
     KBuf kbuf;
-#pragma unroll
-    for (int i = 0; i < KLD; ++i) {
-      const uint32_t sb = (uint32_t)sbase[chunk * 4 + kl_page[i]];
-      kbuf.r[i] = *reinterpret_cast<const v4u*>(kbase + (size_t)(sb * (uint32_t)KP + kl_off[i]));
-    }
     constexpr int KNG = KLIMB ? NG : 1;  // key scales per row
+    // (the scales first: they are copied out of the buffer one chunk earlier than the rows are, and loads return in order)
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int sb = __builtin_amdgcn_readfirstlane(sbase[chunk * 4 + j]);  // first slot of the page (uniform)
@@ -389,6 +393,11 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
         else kbuf.z[j] = *reinterpret_cast<const uint16_t*>(zrow);
       }
     }
+#pragma unroll
+    for (int i = 0; i < KLD; ++i) {
+      const uint32_t sb = (uint32_t)sbase[chunk * 4 + kl_page[i]];
+      kbuf.r[i] = *reinterpret_cast<const v4u*>(kbase + (size_t)(sb * (uint32_t)KP + kl_off[i]));
+    }
     return kbuf;
   };
   auto stash_k = [&](const KBuf& kbuf) {
@@ -397,17 +406,24 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   };
   // first two chunks of this wavefront and the V scales of the split start now, before the query set-up
   KBuf Ka = {}, Kb = {};
-  if (HAS_K && wave < nch_cover) Ka = issue_k(wave);
+  // (every wavefront requests, on a clamped chunk if it has none of its own: the number of loads in flight at each
+  // later wait is then the same on every path, and the compiler's waits leave the younger loads in flight)
+  if constexpr (HAS_K) Ka = issue_k(min(wave, nch_cover - 1));
   constexpr int VSPT = Lds::LMAX / NT;
-  uint32_t vsw[VSPT];
+  // (positions past the split's end read the scale of its last row again: straight-line code whose loads leave
+  // together, and the only use of these values is their maximum)
+  uint32_t vsw[VSPT], vs_slot[VSPT];
 #pragma unroll
   for (int i = 0; i < VSPT; ++i) {
-    const int t = tid + i * NT;
+    const int t = min(tid + i * NT, n - 1);
+    vs_slot[i] = HAS_V ? (uint32_t)(sbase[t >> 4] + (t & 15)) : 0u;
+  }
+#pragma unroll
+  for (int i = 0; i < VSPT; ++i) {
     vsw[i] = 0u;
-    if (HAS_V && t < n) {
-      const uint32_t slot = (uint32_t)(sbase[t >> 4] + (t & 15));
-      if (NG == 2) vsw[i] = *reinterpret_cast<const uint32_t*>(vsbase + (size_t)(slot * 4u));
-      else vsw[i] = (uint32_t) * reinterpret_cast<const uint16_t*>(vsbase + (size_t)(slot * 2u));
+    if constexpr (HAS_V) {
+      if (NG == 2) vsw[i] = *reinterpret_cast<const uint32_t*>(vsbase + (size_t)(vs_slot[i] * 4u));
+      else vsw[i] = (uint32_t) * reinterpret_cast<const uint16_t*>(vsbase + (size_t)(vs_slot[i] * 2u));
     }
   }
 
@@ -429,7 +445,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     for (int it = 0; it < QPT; ++it) {
       const int c = it * NW + wave;  // 64-channel half row of this wavefront
       if (c * 64 < QN) {             // uniform per wavefront
-        const float am = wave_max(fabsf(qv[it]));
+        const float am = wave_max(fabsf(q_elem(it)));
         if (lane == 0) prep->amax_w[c] = am;
       }
     }
@@ -437,7 +453,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
 #pragma unroll
     for (int it = 0; it < QPT; ++it) {
       const int i = it * NT + tid, h = i >> 7, d = i & 127;
-      const float x = qv[it];
+      const float x = q_elem(it);
       const int c = it * NW + wave;
       if (c * 64 >= QN) continue;
       const float amax = (NG == 2) ? prep->amax_w[c] : fmaxf(prep->amax_w[c & ~1], prep->amax_w[c | 1]);
@@ -485,7 +501,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
       const int i = it * NT + tid;
       if (i < QN) {  // uniform per wavefront: QN is a multiple of 64
         const int h = i >> 7, d = i & 127, kk = d >> 5;
-        const float x = qv[it];
+        const float x = q_elem(it);
         float a = fabsf(x);
 #pragma unroll
         for (int off = 16; off >= 1; off >>= 1) a = fmaxf(a, __shfl_xor(a, off));
@@ -510,7 +526,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     }
   }
   lds_barrier();
-  if (HAS_K && wave + NW < nch_cover) Kb = issue_k(wave + NW);
+  if constexpr (HAS_K) Kb = issue_k(min(wave + NW, nch_cover - 1));
   if (clk && tid == 0) clk[7] = clock64();
 
   // ---- V stream, set-up (same scheme as the key stream)
@@ -546,15 +562,22 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   };
   // the first two V chunks are requested while the last key chunks are being worked on
   VBuf Va = {}, Vb = {};
+  bool va_requested = false, vb_requested = false;  // (uniform per wavefront)
   auto prefetch_v = [&](int it) {
     if constexpr (MODE == FS_FULL) {
-      if (it == MAXIT - 2 && wave < nch) Va = issue_v(wave);
-      if (it == MAXIT - 1 && wave + NW < nch) Vb = issue_v(wave + NW);
+      if (it == MAXIT - 2) {
+        Va = issue_v(min(wave, nch - 1));
+        va_requested = true;
+      }
+      if (it == MAXIT - 1) {
+        Vb = issue_v(min(wave + NW, nch - 1));
+        vb_requested = true;
+      }
     }
   };
   if constexpr (MODE == FS_STAGE_B) {  // nothing to wait for: the value stream starts at once
-    if (wave < nch) Va = issue_v(wave);
-    if (wave + NW < nch) Vb = issue_v(wave + NW);
+    Va = issue_v(min(wave, nch - 1));
+    Vb = issue_v(min(wave + NW, nch - 1));
   }
 
 
@@ -879,8 +902,10 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     };
     // at most Lds::LMAX / 64 / NW chunks per wavefront: straight-line code, so that the wait for a chunk's
     // loads leaves the loads of the following chunks in flight
-#pragma unroll
-    for (int it = 0; it < MAXIT; ++it) {
+    // (step it + 1 sits inside step it's block, and the chunk two ahead is requested unconditionally, clamped: no
+    // two paths with different numbers of loads in flight meet before a wait)
+    auto key_step = [&](auto self, auto it_tag) -> void {
+      constexpr int it = decltype(it_tag)::value;
       const int chunk = wave + it * NW;
       prefetch_v(it);
       if (chunk < nch_cover) {
@@ -891,14 +916,16 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
         uint32_t Sc[4], Zc[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          Sc[j] = cur.s[j];
-          Zc[j] = KA ? cur.z[KA ? j : 0] : 0u;
+          Sc[j] = reg_copy(cur.s[j]);
+          Zc[j] = KA ? reg_copy(cur.z[KA ? j : 0]) : 0u;
         }
-        if (it + 2 < MAXIT && chunk + 2 * NW < nch_cover) cur = issue_k(chunk + 2 * NW);
+        if constexpr (it + 2 < MAXIT) cur = issue_k(min(chunk + 2 * NW, nch_cover - 1));
         body(chunk, Sc, Zc);
         wave_lds_fence();
+        if constexpr (it + 1 < MAXIT) self(self, std::integral_constant<int, it + 1>{});
       }
-    }
+    };
+    key_step(key_step, std::integral_constant<int, 0>{});
     // lanes of 16-lane row lg hold the running extrema of head set*4 + lg: reduce inside the rows (lane 15 of
     // a row ends up with the row's result) and publish them
 #pragma unroll
@@ -976,8 +1003,8 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
         }
       }
     };
-#pragma unroll
-    for (int it = 0; it < MAXIT; ++it) {
+    auto key_step = [&](auto self, auto it_tag) -> void {  // (nested, as for the other key formats)
+      constexpr int it = decltype(it_tag)::value;
       const int chunk = wave + it * NW;
       prefetch_v(it);
       if (chunk < nch_cover) {
@@ -987,12 +1014,14 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
         wave_lds_fence();
         uint32_t Sc[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) Sc[j] = cur.s[j];
-        if (it + 2 < MAXIT && chunk + 2 * NW < nch_cover) cur = issue_k(chunk + 2 * NW);
+        for (int j = 0; j < 4; ++j) Sc[j] = reg_copy(cur.s[j]);
+        if constexpr (it + 2 < MAXIT) cur = issue_k(min(chunk + 2 * NW, nch_cover - 1));
         body(chunk, Sc);
         wave_lds_fence();
+        if constexpr (it + 1 < MAXIT) self(self, std::integral_constant<int, it + 1>{});
       }
-    }
+    };
+    key_step(key_step, std::integral_constant<int, 0>{});
 #pragma unroll
     for (int set = 0; set < NSET; ++set) {
       float a = mxl[set], c = -mnl[set];
@@ -1247,8 +1276,12 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
       }
     }
   };
-#pragma unroll
-  for (int it = 0; it < MAXIT; ++it) {
+  if constexpr (MODE == FS_FULL) {  // (wavefronts that left the key stream before its last two steps)
+    if (!va_requested) Va = issue_v(min(wave, nch - 1));
+    if (!vb_requested) Vb = issue_v(min(wave + NW, nch - 1));
+  }
+  auto value_step = [&](auto self, auto it_tag) -> void {  // (nested like the key stream's steps)
+    constexpr int it = decltype(it_tag)::value;
     const int chunk = wave + it * NW;
     if (chunk < nch) {
       set_wave_prio(3 - it);
@@ -1256,12 +1289,14 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
       if constexpr (HAS_V) {
         VBuf& cur = (it & 1) ? Vb : Va;
         stash_v(cur);
-        vw = cur.w;
-        if (it + 2 < MAXIT && chunk + 2 * NW < nch) cur = issue_v(chunk + 2 * NW);
+        vw = reg_copy(cur.w);
+        if constexpr (it + 2 < MAXIT) cur = issue_v(min(chunk + 2 * NW, nch - 1));
       }
       body_v(chunk, vw);
+      if constexpr (it + 1 < MAXIT) self(self, std::integral_constant<int, it + 1>{});
     }
-  }
+  };
+  value_step(value_step, std::integral_constant<int, 0>{});
   __builtin_amdgcn_s_setprio(0);
 #pragma unroll
   for (int h = 0; h < G; ++h) {
@@ -1636,16 +1671,26 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   long long* mclk = (p.phase_clock && !PARTIAL) ? p.phase_clock + (size_t)p.B * p.H_kv * p.n_splits * 10 + bh * 8 : nullptr;
   if (mclk && tid == 0) mclk[0] = clock64();
 
-  // ---- everything that does not depend on anything else is requested first, in the order of its use
+  // ---- everything that does not depend on anything else is requested first, in the order of its use.  Every load
+  // is unconditional, on a clamped index, and its mask is applied further down: under a condition the compiler waits
+  // for a load inside its branch, and these loads (first touches of what other XCDs wrote) would cost one round trip
+  // after the other instead of one for all.
+  constexpr bool HAS_LISTS = (MODE != FS_STAGE_B);
   float pm = -INFINITY, pl = 0.f;
   int my_cnt = 0;
-  if (!PARTIAL && tid < NS) {
-    pm = p.part_m[bh * NS + tid];
-    pl = p.part_l[bh * NS + tid];
+  // (given statistics, jf_stage_b_softmax_v: no partial results at all, NS = 0 and the pointers are null; those
+  // loads then read the page table, which every caller of this kernel passes, and every one of them is masked)
+  const bool has_parts = NS > 0;
+  const float* dummy_f = reinterpret_cast<const float*>(bt);
+  if constexpr (!PARTIAL) {
+    pm = *(has_parts ? p.part_m + bh * NS + min(tid, NS - 1) : dummy_f);
+    pl = *(has_parts ? p.part_l + bh * NS + min(tid, NS - 1) : dummy_f);
   }
-  if (tid < NL) my_cnt = cc[tid];
+  if constexpr (HAS_LISTS) my_cnt = cc[min(tid, NL - 1)];
+  uint16_t blend_raw = 0;
   float blend_new = 0.f, blend_hat = 0.f;
-  if (MODE == FS_FULL && !PARTIAL && p.blend_out && tid < D) blend_new = bf16_to_f32(p.blend_o_new[bh * D + tid]);
+  if constexpr (MODE == FS_FULL && !PARTIAL)  // (no blend: any readable address)
+    blend_raw = *(p.blend_out ? p.blend_o_new + bh * D + (tid & (D - 1)) : reinterpret_cast<const uint16_t*>(ck));
   // The first MG_REGK * MG_THREADS candidates live in registers: group g = r / 4 of a thread holds the four
   // consecutive candidates (g * MG_THREADS + tid) * 4 + (r % 4), fetched with one 16-byte load.  Candidate
   // order = (group, thread, element).  Slots past a list's count hold key 0 (written by the producer).
@@ -1654,23 +1699,19 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   const int rreg = min((flat + 4 * MG_THREADS - 1) / (4 * MG_THREADS), NGRP) * 4;  // register slots in use (uniform)
   uint32_t kreg[MG_REGK];
   int ireg[MG_REGK];
+  v4u k4[NGRP];
+  v4i i4[NGRP];
 #pragma unroll
   for (int g = 0; g < NGRP; ++g) {
-    const int f4 = (g * MG_THREADS + tid) * 4;
-    v4u k4 = {0u, 0u, 0u, 0u};
-    if (4 * g < rreg && f4 < flat) k4 = *reinterpret_cast<const v4u*>(ck + f4);  // flat is a multiple of 4
-#pragma unroll
-    for (int j = 0; j < 4; ++j) kreg[4 * g + j] = k4[j];
+    k4[g] = (v4u){0u, 0u, 0u, 0u};
+    if constexpr (HAS_LISTS)  // (a group past the end reads the last four again; flat is a multiple of 4)
+      k4[g] = *reinterpret_cast<const v4u*>(ck + min((g * MG_THREADS + tid) * 4, flat - 4));
   }
 #pragma unroll
   for (int g = 0; g < NGRP; ++g) {
-    const int f4 = (g * MG_THREADS + tid) * 4;
-    v4i i4 = {0, 0, 0, 0};
-    if (4 * g < rreg && f4 < flat) i4 = *reinterpret_cast<const v4i*>(ci + f4);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) ireg[4 * g + j] = i4[j];
+    i4[g] = (v4i){0, 0, 0, 0};
+    if constexpr (HAS_LISTS) i4[g] = *reinterpret_cast<const v4i*>(ci + min((g * MG_THREADS + tid) * 4, flat - 4));
   }
-  if (tid < NL) cnt_sh[tid] = my_cnt;
   // o_hat: the thread groups of 128 take the splits round-robin (first terms requested now)
   constexpr int PO_PRE = 2, PO_GRP = MG_THREADS / D;
   float po[PO_PRE];
@@ -1678,14 +1719,42 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
     const int d = tid & (D - 1), q4 = tid >> 7;
 #pragma unroll
     for (int i = 0; i < PO_PRE; ++i) {
-      const int sp = q4 + VGRP * i;
-      po[i] = (MODE != FS_STAGE_A && !PARTIAL && sp < NS) ? p.part_o[(bh * NS + sp) * D + d] : 0.f;
+      po[i] = 0.f;
+      if constexpr (MODE != FS_STAGE_A && !PARTIAL)
+        po[i] = *(has_parts ? p.part_o + (bh * NS + min(q4 + VGRP * i, NS - 1)) * D + d : dummy_f);
     }
   }
-  if (!PARTIAL)
-    for (int i = tid; i < nblk_lds; i += MG_THREADS) bt_sh[i] = (int)bt[i];
+  constexpr int BTPT = (MG_BT + MG_THREADS - 1) / MG_THREADS;  // page-table entries per thread (stored to LDS below)
+  int bt_mine[BTPT];
+#pragma unroll
+  for (int i = 0; i < BTPT; ++i) {
+    bt_mine[i] = 0;
+    if constexpr (!PARTIAL) bt_mine[i] = (int)bt[min(tid + i * MG_THREADS, p.max_blocks - 1)];
+  }
   for (int i = tid; i < MG_BINS; i += MG_THREADS) hist[i] = 0;
   if (tid == 0) lcount_sh = 0;
+  // the masks of the loads above
+  if (tid >= NS) {
+    pm = -INFINITY;
+    pl = 0.f;
+  }
+  if (tid >= NL) my_cnt = 0;
+  if (MODE == FS_FULL && !PARTIAL && p.blend_out && tid < D) blend_new = bf16_to_f32(blend_raw);
+#pragma unroll
+  for (int g = 0; g < NGRP; ++g) {
+    const bool in = (g * MG_THREADS + tid) * 4 < flat;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      kreg[4 * g + j] = in ? k4[g][j] : 0u;
+      ireg[4 * g + j] = in ? i4[g][j] : 0;
+    }
+  }
+  if (tid < NL) cnt_sh[tid] = my_cnt;
+  if constexpr (!PARTIAL) {
+#pragma unroll
+    for (int i = 0; i < BTPT; ++i)
+      if (tid + i * MG_THREADS < nblk_lds) bt_sh[tid + i * MG_THREADS] = bt_mine[i];
+  }
 
   // key of candidate f in pass-over-all-candidates loops: registers first, global memory beyond
   auto key_of = [&](int r) -> uint32_t {
