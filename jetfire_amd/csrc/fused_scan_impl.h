@@ -247,6 +247,16 @@ __device__ inline uint32_t reg_copy(uint32_t v) {
   return r;
 }
 
+// (hi * 256 + mid) * 256 + lo as two v_lshl_add_u32.  Written as plain shifts and adds the compiler re-associates
+// it into two shifts and a three-operand add, one instruction more, in the innermost loop of the key stream; the
+// empty statement makes the intermediate opaque.  (The instructions themselves stay the compiler's: it alone knows
+// how long after an MFMA its results may be read.)
+__device__ inline int join_limbs(int hi, int mid, int lo) {
+  int t = (hi << 8) + mid;
+  asm("" : "+v"(t));
+  return (t << 8) + lo;
+}
+
 // s_setprio takes an immediate; `p` is a compile-time constant after unrolling
 __device__ inline void set_wave_prio(int p) {
   if (p >= 3) __builtin_amdgcn_s_setprio(3);
@@ -728,7 +738,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
                 Dc = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][0], Bc[0], zero, 0, 0, 0);
                 Dc = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][1], Bc[1], Dc, 0, 0, 0);
               }
-              acc_s[set][g] = (float)((((Dc[2] << 8) + Dc[1]) << 8) + Dc[0] - sq4[set][g]);
+              acc_s[set][g] = (float)join_limbs(Dc[2], Dc[1], Dc[0] - sq4[set][g]);
             }
 #pragma unroll
           for (int c = 0; c < 3; ++c) {  // c = 0, 1, 2: the indicators of +-3 (and +-6), +-5, +-7
@@ -827,9 +837,9 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
                 D01 = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][0], X01[0], zero, 0, 0, 0);
                 D01 = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][1], X01[1], D01, 0, 0, 0);
               }
-              const float s0f = (float)((((D0[2] << 8) + D0[1]) << 8) + D0[0]);
-              const float s1f = (float)((((D1[2] << 8) + D1[1]) << 8) + D1[0]);
-              const float s01f = (float)((((D01[2] << 8) + D01[1]) << 8) + D01[0]);
+              const float s0f = (float)join_limbs(D0[2], D0[1], D0[0]);
+              const float s1f = (float)join_limbs(D1[2], D1[1], D1[0]);
+              const float s01f = (float)join_limbs(D01[2], D01[1], D01[0]);
               float v = coef[g][0] * sumq[set][g];
               v = __builtin_fmaf(coef[g][1], s0f, v);
               v = __builtin_fmaf(coef[g][2], s1f, v);
@@ -869,7 +879,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
 #pragma unroll
             for (int g = 0; g < NG; ++g) {
               const v4i Dc = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][g], Bc[g], zero, 0, 0, 0);
-              const int xc = (((Dc[2] << 8) + Dc[1]) << 8) + Dc[0] - sq4[set][g];
+              const int xc = join_limbs(Dc[2], Dc[1], Dc[0] - sq4[set][g]);
               float v = (float)xc;
               if constexpr (K3) {
                 const v4i Dr = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][g], Br[g], zero, 0, 0, 0);
@@ -881,7 +891,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
           } else {
             v4i Dc = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][0], Bc[0], zero, 0, 0, 0);
             Dc = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][1], Bc[1], Dc, 0, 0, 0);
-            const int xc = (((Dc[2] << 8) + Dc[1]) << 8) + Dc[0] - sq4[set][0];
+            const int xc = join_limbs(Dc[2], Dc[1], Dc[0] - sq4[set][0]);
             float v = (float)xc;
             if constexpr (K3) {
               v4i Dr = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][0], Br[0], zero, 0, 0, 0);
