@@ -724,7 +724,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
           // 2 [c = +-6], r5 = [c = +-5], r7 = [c = +-7], made by byte look-ups: one table for the codes >= 0 (u >= 8,
           // selector u - 8 = c) and one for the codes < 0 (selector u = c + 8), chosen per byte by bit 3 of u.
           const int tok = chunk * 64 + 16 * j + t16;
-          const bool valid = tok < n;
+          const bool valid = t16 < n - chunk * 64 - 16 * j;  // (tok < n, with the uniform part on one side)
           float acc_s[NSET][NG];
 #pragma unroll
           for (int set = 0; set < NSET; ++set)
@@ -817,7 +817,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
             coef[g][3] = (v[3] - v[2]) - (v[1] - v[0]);
           }
           const int tok = chunk * 64 + 16 * j + t16;
-          const bool valid = tok < n;
+          const bool valid = t16 < n - chunk * 64 - 16 * j;  // (tok < n, with the uniform part on one side)
 #pragma unroll
           for (int set = 0; set < NSET; ++set) {
             const v4i zero = {0, 0, 0, 0};
@@ -870,7 +870,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
           eg[g] = egj[j][g];
         }
         const int tok = chunk * 64 + 16 * j + t16;
-        const bool valid = tok < n;
+        const bool valid = t16 < n - chunk * 64 - 16 * j;  // (tok < n, with the uniform part on one side)
 #pragma unroll
         for (int set = 0; set < NSET; ++set) {
           float score = 0.f;
@@ -994,7 +994,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
         }
         const float ks = bf16_to_f32((uint16_t)Sx[j]);
         const int tok = chunk * 64 + 16 * j + t16;
-        const bool valid = tok < n;
+        const bool valid = t16 < n - chunk * 64 - 16 * j;  // (tok < n, with the uniform part on one side)
 #pragma unroll
         for (int set = 0; set < NSET; ++set) {
           const v4i zero = {0, 0, 0, 0};
