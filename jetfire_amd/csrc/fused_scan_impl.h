@@ -1130,6 +1130,16 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     bin_a[h] = uniform_f(bin_a_sh[h]);
     bin_b[h] = uniform_f(bin_b_sh[h]);
   }
+  // The bucket of a score is fma(s, a, b) clamped to [0, 255] with a and b uniform: an instruction takes one scalar
+  // operand only, and left alone the compiler copies b (and 255.0, and the increment) into a vector register again
+  // for every head of every chunk.  Copies it cannot see through stay in their registers through the stream.
+  float bin_bv[G], clamp_hi = 255.f;
+#pragma unroll
+  for (int h = 0; h < G; ++h) {
+    bin_bv[h] = bin_b[h];
+    asm volatile("" : "+v"(bin_bv[h]));
+  }
+  asm volatile("" : "+v"(clamp_hi));
   const int r16 = lane & 15, kb4 = lane >> 4;
   // transposed weight read: 16-lane group kb4 fetches the rows of tokens 16*kb4 .. +15; the lane pair (2j, 2j+1)
   // supplies the two halves of the row that must land in byte j, i.e. of the token whose byte position in the
@@ -1144,6 +1154,8 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     if (NG == 2) vsf[NG - 1] = ldexpf(bf16_to_f32((uint16_t)(vsw >> 16)), E[NG - 1]);
     int* hb = hist + ((SEG == 1) ? 0 : (chunk / seg_chunks) * (Lds::H16 ? 128 : 256));
     const bool tv = t < n;
+    const int inc = tv ? 1 : 0;
+    (void)inc;
     uint32_t bits[NSET * 4][NG];
 #pragma unroll
     for (int h = 0; h < NSET * 4; ++h) {
@@ -1155,12 +1167,11 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
 #pragma unroll
         for (int g = 0; g < NG; ++g) bits[h][g] = __builtin_bit_cast(uint32_t, __builtin_fmaf(pw, vsf[g], 8388608.0f));
         if constexpr (HAS_TOPK) {
-          const uint32_t bin = (uint32_t)__builtin_amdgcn_fmed3f(__builtin_fmaf(s, bin_a[h], bin_b[h]), 0.f, 255.f);
-          if (Lds::H16) {
-            if (tv) atomicAdd(hb + ((h * (SEG * 256) + (int)bin) >> 1), (bin & 1u) ? 0x10000 : 1);
-          } else {
-            if (tv) atomicAdd(hb + h * (SEG * 256) + (int)bin, 1);
-          }
+          // (positions past the end add zero instead of branching around the add: their score is -inf or, with a
+          // degenerate range, gives a NaN, and either clamps to a bucket inside the table)
+          const uint32_t bin = (uint32_t)__builtin_amdgcn_fmed3f(__builtin_fmaf(s, bin_a[h], bin_bv[h]), 0.f, clamp_hi);
+          if (Lds::H16) atomicAdd(hb + ((h * (SEG * 256) + (int)bin) >> 1), inc << ((bin & 1u) << 4));
+          else atomicAdd(hb + h * (SEG * 256) + (int)bin, inc);
         }
       } else {
 #pragma unroll
@@ -1453,7 +1464,9 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
       // [0, 255]; with cut = 255 every position qualifies
       const int cut = cut_sh[h];
       const float thr = uniform_f((cut >= 255) ? INFINITY : (float)(cut + 1));
-      const float ba = uniform_f(bin_a_sh[h]), bb = uniform_f(bin_b_sh[h]);
+      const float ba = uniform_f(bin_a_sh[h]);
+      float bb = uniform_f(bin_b_sh[h]);
+      asm volatile("" : "+v"(bb));  // (kept in a vector register: the multiply-add takes one scalar operand only)
       const int tb = seg * (L / SEG);
       const int te = min(n, (seg + 1) * (L / SEG));
       // the emitted total is at most Kcap by construction of the cut
@@ -1464,17 +1477,19 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
       for (int i = etot + seg * 64 + lane; i < Kcap; i += SEG * 64) ck[i] = 0u;
       uint8_t* ckb = reinterpret_cast<uint8_t*>(ck);
       uint8_t* cib = reinterpret_cast<uint8_t*>(ci);
-      for (int t0 = tb; t0 < te; t0 += 512) {
+      // eight groups of 64 positions at a time; whole batches run without the per-position end test
+      auto emit_batch = [&](int t0, auto checked_tag) {
+        constexpr bool CHECKED = decltype(checked_tag)::value;
         float kk[8];
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
           const int t = t0 + 64 * u + lane;
-          kk[u] = (t < te) ? srow[t] : 0.f;
+          kk[u] = (!CHECKED || t < te) ? srow[t] : 0.f;
         }
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
           const int t = t0 + 64 * u + lane;
-          const bool above = (t < te) && !(__builtin_fmaf(kk[u], ba, bb) >= thr);
+          const bool above = (!CHECKED || t < te) && !(__builtin_fmaf(kk[u], ba, bb) >= thr);
           const unsigned long long ma = __builtin_amdgcn_ballot_w64(above);
           const uint32_t pos = (uint32_t)count + __builtin_amdgcn_mbcnt_hi((uint32_t)(ma >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)ma, 0u));
           if (above && pos < (uint32_t)Kcap) {  // the bound only matters for non-finite scores
@@ -1483,7 +1498,10 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
           }
           count += __popcll(ma);
         }
-      }
+      };
+      int t0 = tb;
+      for (; t0 + 512 <= te; t0 += 512) emit_batch(t0, std::integral_constant<bool, false>{});
+      if (t0 < te) emit_batch(t0, std::integral_constant<bool, true>{});
       if (seg == SEG - 1) {
         if (lane == 0) p.cand_cnt[part_base + (size_t)h * p.n_splits] = min(Kcap, count);
         for (int i = count + lane; i < etot; i += 64) ck[i] = 0u;  // (only if a segment emitted less than planned)
