@@ -79,6 +79,7 @@ typedef int v2i __attribute__((ext_vector_type(2)));
 typedef unsigned v2u __attribute__((ext_vector_type(2)));
 typedef unsigned v4u __attribute__((ext_vector_type(4)));
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v3i __attribute__((ext_vector_type(3)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef float v2f __attribute__((ext_vector_type(2)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
@@ -1188,12 +1189,11 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
         const uint32_t U01 = __builtin_amdgcn_perm(h1, h0, 0x0c0c0602u);  // h0.b2 h1.b2 0 0
         const uint32_t T23 = __builtin_amdgcn_perm(h3, h2, 0x05010400u);
         const uint32_t U23 = __builtin_amdgcn_perm(h3, h2, 0x0c0c0602u);
-        v4i row;
+        v3i row;  // (the fourth dword of the row, the constant 1 of the ones row, was written before the stream)
         row[0] = (int)(__builtin_amdgcn_perm(T23, T01, 0x05040100u) ^ 0x80808080u);  // limb 0 of heads 0..3, balanced
         row[1] = (int)(__builtin_amdgcn_perm(T23, T01, 0x07060302u) ^ 0x80808080u);  // limb 1
         row[2] = (int)(U01 | (U23 << 16));                                           // limb 2 (< 128)
-        row[3] = 1;                                                                  // row 12: ones; 13..15: zero
-        *reinterpret_cast<v4i*>(wl + ((g * NSET + set) * 64 + lane) * 16) = row;
+        *reinterpret_cast<v3i*>(wl + ((g * NSET + set) * 64 + lane) * 16) = row;
       }
     wave_lds_fence();
     v4i A[NG][NSET];
@@ -1297,6 +1297,13 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
       }
     }
   };
+  if constexpr (HAS_V) {
+    // fourth dword of every weight row: row 12 of the A operand is all ones, rows 13..15 are zero.  Constant, so it
+    // is stored once (this wavefront's staging area held key rows until now) and the stream stores 12 bytes per row.
+#pragma unroll
+    for (int i = 0; i < NG * NSET; ++i) *reinterpret_cast<int*>(wl + (i * 64 + lane) * 16 + 12) = 1;
+    wave_lds_fence();
+  }
   if constexpr (MODE == FS_FULL) {  // (wavefronts that left the key stream before its last two steps)
     if (!va_requested) Va = issue_v(min(wave, nch - 1));
     if (!vb_requested) Vb = issue_v(min(wave + NW, nch - 1));
