@@ -150,7 +150,6 @@ struct K3Prep {
   int8_t aop[NSET][16][4][2][16];  // A operand bytes: [set][row = 4*head + limb][k-block][MFMA][byte]
   int sq4[NSET * 4][2];            // 4 * sum of the fixed-point query over the scale group
   float qsc[NSET * 4][2];          // 2^(e-22) * attn_scale of the (head, group)
-  float eps[3][128];               // 256 * (bf16(c s) - c s) / s for s = 1 + m/128; INT3: c = 3; INT4: c = 3, 5, 7
   float amax_w[NSET * 8];          // per 64-channel half row: |q| maximum, fixed-point sum, exponent
   int sum_w[NSET * 8];
   int exp_w[NSET * 8];
@@ -304,6 +303,9 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   __shared__ float m_sh[G], bin_a_sh[G], bin_b_sh[G], lsum_sh[NW][G];
   __shared__ int e_sh[2];
   __shared__ int cut_sh[G], segoff_sh[G][SEG + 1], exact_sh[G];
+  // rounding coefficients 256 * (bf16(c s) - c s) / s for s = 1 + m/128 (INT3: c = 3; INT4, bf16 model: c = 3, 5, 7).
+  // Static, so that a look-up's address is the index plus a constant the instruction carries.
+  __shared__ float eps_sh[KB4 ? 3 : 1][128];
   __shared__ unsigned long long tmax_sh;
   if (threadIdx.x == 0) tmax_sh = 0ull;
 
@@ -449,7 +451,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
 #pragma unroll
       for (int i = 0; i < (KB4 ? 3 : 1); ++i) {
         const float t = (float)(3 + 2 * i) * sm;  // 3 s, 5 s, 7 s: exact in fp32
-        prep->eps[i][tid] = 256.0f * ((bf16_to_f32(f32_to_bf16(t)) - t) / sm);
+        eps_sh[i][tid] = 256.0f * ((bf16_to_f32(f32_to_bf16(t)) - t) / sm);
       }
     }
 #pragma unroll
@@ -679,10 +681,10 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
         }
         const uint32_t sw = Sx[j];
         sgj[j][0] = bf16_to_f32((uint16_t)(sw & 0xffffu));
-        egj[j][0] = K3 ? prep->eps[0][sw & 0x7fu] : 0.f;  // (INT4: three coefficients, read where they are used)
+        egj[j][0] = K3 ? eps_sh[0][sw & 0x7fu] : 0.f;  // (INT4: three coefficients, read where they are used)
         if (NG == 2) {
           sgj[j][NG - 1] = bf16_to_f32((uint16_t)(sw >> 16));
-          egj[j][NG - 1] = K3 ? prep->eps[0][(sw >> 16) & 0x7fu] : 0.f;
+          egj[j][NG - 1] = K3 ? eps_sh[0][(sw >> 16) & 0x7fu] : 0.f;
         }
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -769,7 +771,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
                   Dr = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][0], Bi[0], zero, 0, 0, 0);
                   Dr = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][1], Bi[1], Dr, 0, 0, 0);
                 }
-                const float ec = prep->eps[c][((g == 0) ? Sx[j] : (Sx[j] >> 16)) & 0x7fu];
+                const float ec = eps_sh[c][((g == 0) ? Sx[j] : (Sx[j] >> 16)) & 0x7fu];
                 acc_s[set][g] = __builtin_fmaf(ec, (float)((Dr[2] << 8) + Dr[1]), acc_s[set][g]);
               }
           }
@@ -2246,7 +2248,7 @@ template <int SCHEME, int G, int NG>
 int lmax_for() {
   using Lds = ScanLds<SCHEME, G, NG>;
   const size_t budget = (G <= 4 && Lds::NW == 8) ? LDS_BUDGET_2WG : LDS_BUDGET_1WG;
-  const size_t fixed = Lds::AUX + Lds::stage_bytes() + 64 + 832;  // + static LDS of the kernel
+  const size_t fixed = Lds::AUX + Lds::stage_bytes() + 64 + 832 + (Lds::KB4 ? 1536 : (Lds::K3 ? 512 : 0));  // + static LDS of the kernel (incl. the rounding tables)
   long lm = (long)((budget - fixed) / (Lds::per_position() + 1));  // +1: page table (4 bytes per 16 positions)
   lm = lm / 256 * 256;
   if (lm > Lds::LMAX) lm = Lds::LMAX;
