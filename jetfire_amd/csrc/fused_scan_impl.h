@@ -1719,15 +1719,6 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   // loads then read the page table, which every caller of this kernel passes, and every one of them is masked)
   const bool has_parts = NS > 0;
   const float* dummy_f = reinterpret_cast<const float*>(bt);
-  if constexpr (!PARTIAL) {
-    pm = *(has_parts ? p.part_m + bh * NS + min(tid, NS - 1) : dummy_f);
-    pl = *(has_parts ? p.part_l + bh * NS + min(tid, NS - 1) : dummy_f);
-  }
-  if constexpr (HAS_LISTS) my_cnt = cc[min(tid, NL - 1)];
-  uint16_t blend_raw = 0;
-  float blend_new = 0.f, blend_hat = 0.f;
-  if constexpr (MODE == FS_FULL && !PARTIAL)  // (no blend: any readable address)
-    blend_raw = *(p.blend_out ? p.blend_o_new + bh * D + (tid & (D - 1)) : reinterpret_cast<const uint16_t*>(ck));
   // The first MG_REGK * MG_THREADS candidates live in registers: group g = r / 4 of a thread holds the four
   // consecutive candidates (g * MG_THREADS + tid) * 4 + (r % 4), fetched with one 16-byte load.  Candidate
   // order = (group, thread, element).  Slots past a list's count hold key 0 (written by the producer).
@@ -1738,17 +1729,27 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   int ireg[MG_REGK];
   v4u k4[NGRP];
   v4i i4[NGRP];
+  // what the first barrier interval needs goes first (loads return in order): the split maxima, the list counts,
+  // the candidate keys
+  if constexpr (!PARTIAL) pm = *(has_parts ? p.part_m + bh * NS + min(tid, NS - 1) : dummy_f);
+  if constexpr (HAS_LISTS) my_cnt = cc[min(tid, NL - 1)];
 #pragma unroll
   for (int g = 0; g < NGRP; ++g) {
     k4[g] = (v4u){0u, 0u, 0u, 0u};
-    if constexpr (HAS_LISTS)  // (a group past the end reads the last four again; flat is a multiple of 4)
-      k4[g] = *reinterpret_cast<const v4u*>(ck + min((g * MG_THREADS + tid) * 4, flat - 4));
+    if constexpr (HAS_LISTS)  // (flat is a multiple of 4; groups past the end are not requested)
+      if (g == 0 || 4 * g < rreg) k4[g] = *reinterpret_cast<const v4u*>(ck + min((g * MG_THREADS + tid) * 4, flat - 4));
   }
+  if constexpr (!PARTIAL) pl = *(has_parts ? p.part_l + bh * NS + min(tid, NS - 1) : dummy_f);
 #pragma unroll
   for (int g = 0; g < NGRP; ++g) {
     i4[g] = (v4i){0, 0, 0, 0};
-    if constexpr (HAS_LISTS) i4[g] = *reinterpret_cast<const v4i*>(ci + min((g * MG_THREADS + tid) * 4, flat - 4));
+    if constexpr (HAS_LISTS)
+      if (g == 0 || 4 * g < rreg) i4[g] = *reinterpret_cast<const v4i*>(ci + min((g * MG_THREADS + tid) * 4, flat - 4));
   }
+  uint16_t blend_raw = 0;
+  float blend_new = 0.f, blend_hat = 0.f;
+  if constexpr (MODE == FS_FULL && !PARTIAL)  // (no blend: any readable address)
+    blend_raw = *(p.blend_out ? p.blend_o_new + bh * D + (tid & (D - 1)) : reinterpret_cast<const uint16_t*>(ck));
   // o_hat: the thread groups of 128 take the splits round-robin (first terms requested now)
   constexpr int PO_PRE = 2, PO_GRP = MG_THREADS / D;
   float po[PO_PRE];
@@ -1761,37 +1762,29 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
         po[i] = *(has_parts ? p.part_o + (bh * NS + min(q4 + VGRP * i, NS - 1)) * D + d : dummy_f);
     }
   }
-  constexpr int BTPT = (MG_BT + MG_THREADS - 1) / MG_THREADS;  // page-table entries per thread (stored to LDS below)
+  // page-table entries for the table in LDS: stored after the first barrier, so that the wait for them (the
+  // youngest loads) is not part of the first interval
+  constexpr int BTPT = (MG_BT + MG_THREADS - 1) / MG_THREADS;
   int bt_mine[BTPT];
 #pragma unroll
   for (int i = 0; i < BTPT; ++i) {
     bt_mine[i] = 0;
-    if constexpr (!PARTIAL) bt_mine[i] = (int)bt[min(tid + i * MG_THREADS, p.max_blocks - 1)];
+    // (the low half of the 64-bit entry only: the unused half of a wider load is a register the compiler hands out
+    // again at once, and writing it has to wait for the load)
+    if constexpr (!PARTIAL) bt_mine[i] = reinterpret_cast<const int*>(bt)[2 * min(tid + i * MG_THREADS, p.max_blocks - 1)];
   }
   for (int i = tid; i < MG_BINS; i += MG_THREADS) hist[i] = 0;
   if (tid == 0) lcount_sh = 0;
-  // the masks of the loads above
-  if (tid >= NS) {
-    pm = -INFINITY;
-    pl = 0.f;
-  }
+  // the masks of the loads the first interval uses (the others follow its barrier)
+  if (tid >= NS) pm = -INFINITY;
   if (tid >= NL) my_cnt = 0;
-  if (MODE == FS_FULL && !PARTIAL && p.blend_out && tid < D) blend_new = bf16_to_f32(blend_raw);
 #pragma unroll
   for (int g = 0; g < NGRP; ++g) {
     const bool in = (g * MG_THREADS + tid) * 4 < flat;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      kreg[4 * g + j] = in ? k4[g][j] : 0u;
-      ireg[4 * g + j] = in ? i4[g][j] : 0;
-    }
+    for (int j = 0; j < 4; ++j) kreg[4 * g + j] = in ? k4[g][j] : 0u;
   }
   if (tid < NL) cnt_sh[tid] = my_cnt;
-  if constexpr (!PARTIAL) {
-#pragma unroll
-    for (int i = 0; i < BTPT; ++i)
-      if (tid + i * MG_THREADS < nblk_lds) bt_sh[tid + i * MG_THREADS] = bt_mine[i];
-  }
 
   // key of candidate f in pass-over-all-candidates loops: registers first, global memory beyond
   auto key_of = [&](int r) -> uint32_t {
@@ -1834,6 +1827,19 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   if (lane == 0) { wred_u[wave] = kmin; wred_k[wave] = kmax; }
   lds_barrier();
   if (mclk && tid == 0) mclk[6] = clock64();
+  if (tid >= NS) pl = 0.f;
+  if (MODE == FS_FULL && !PARTIAL && p.blend_out && tid < D) blend_new = bf16_to_f32(blend_raw);
+#pragma unroll
+  for (int g = 0; g < NGRP; ++g) {
+    const bool in = (g * MG_THREADS + tid) * 4 < flat;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) ireg[4 * g + j] = in ? i4[g][j] : 0;
+  }
+  if constexpr (!PARTIAL) {  // (first read long after the next barrier)
+#pragma unroll
+    for (int i = 0; i < BTPT; ++i)
+      if (tid + i * MG_THREADS < nblk_lds) bt_sh[tid + i * MG_THREADS] = bt_mine[i];
+  }
   // ---- interval 2: M, the coefficients, per-wavefront sums of l; the candidates drop into MG_BINS linear buckets
   float M = -INFINITY;
   if (!PARTIAL) {
