@@ -959,7 +959,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     // both 64-channel spans m; its accumulator registers are the four 32-channel blocks of head lg.
     const QInt8F<NSET>* qsh = reinterpret_cast<const QInt8F<NSET>*>(aux);
     v4i Aop[NSET][2];
-    int sum8[NSET][4];
+    v4i nsum8[NSET];  // minus the block sums: the accumulators' initial values
     float qs[NSET][4];
 #pragma unroll
     for (int set = 0; set < NSET; ++set) {
@@ -967,7 +967,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
       for (int mi = 0; mi < 2; ++mi) Aop[set][mi] = *reinterpret_cast<const v4i*>(&qsh->aop[set][t16][lg][mi][0]);
 #pragma unroll
       for (int kk = 0; kk < 4; ++kk) {
-        sum8[set][kk] = qsh->sum8[set * 4 + lg][kk];
+        nsum8[set][kk] = -qsh->sum8[set * 4 + lg][kk];
         qs[set][kk] = qsh->qs[set * 4 + lg][kk];
       }
     }
@@ -1000,12 +1000,13 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
         const bool valid = t16 < n - chunk * 64 - 16 * j;  // (tok < n, with the uniform part on one side)
 #pragma unroll
         for (int set = 0; set < NSET; ++set) {
-          const v4i zero = {0, 0, 0, 0};
-          v4i Dq = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][0], Bm[0], zero, 0, 0, 0);
+          // (the -8 * sum of the block's query values, the codes being used unsigned, enters as the accumulator's
+          // initial value: exact, and four subtractions per token and head less)
+          v4i Dq = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][0], Bm[0], nsum8[set], 0, 0, 0);
           Dq = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][1], Bm[1], Dq, 0, 0, 0);
-          float sacc = (float)(Dq[0] - sum8[set][0]) * qs[set][0];
+          float sacc = (float)Dq[0] * qs[set][0];
 #pragma unroll
-          for (int kk = 1; kk < 4; ++kk) sacc = __builtin_fmaf((float)(Dq[kk] - sum8[set][kk]), qs[set][kk], sacc);
+          for (int kk = 1; kk < 4; ++kk) sacc = __builtin_fmaf((float)Dq[kk], qs[set][kk], sacc);
           const float a = __fmul_rn(__fmul_rn(sacc, ks), p.attn_scale);
           const int h = set * 4 + lg;
           if ((G % 4 == 0) || h < G) {
