@@ -1144,6 +1144,8 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     asm volatile("" : "+v"(bin_bv[h]));
   }
   asm volatile("" : "+v"(clamp_hi));
+  v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};  // all-ones B tile of the weight sums (kept, like the above)
+  asm volatile("" : "+v"(ones));
   const int r16 = lane & 15, kb4 = lane >> 4;
   // transposed weight read: 16-lane group kb4 fetches the rows of tokens 16*kb4 .. +15; the lane pair (2j, 2j+1)
   // supplies the two halves of the row that must land in byte j, i.e. of the token whose byte position in the
@@ -1209,7 +1211,6 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
         const v2i x1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i*)(src + 128));
         A[g][set] = (v4i){x0[0], x0[1], x1[0], x1[1]};
       }
-    const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
 #pragma unroll
     for (int g = 0; g < NG; ++g)
 #pragma unroll
