@@ -874,6 +874,37 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
         }
         const int tok = chunk * 64 + 16 * j + t16;
         const bool valid = t16 < n - chunk * 64 - 16 * j;  // (tok < n, with the uniform part on one side)
+        if constexpr (NG == 2 && NSET >= 2) {
+          // Two head sets: with two wavefronts per SIMD little else hides the wait for an MFMA's results, so all of a
+          // token group's products are issued first and read afterwards.
+          const v4i zero = {0, 0, 0, 0};
+          v4i Dc_all[NSET][NG], Dr_all[NSET][NG];
+#pragma unroll
+          for (int set = 0; set < NSET; ++set)
+#pragma unroll
+            for (int g = 0; g < NG; ++g) {
+              Dc_all[set][g] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][g], Bc[g], zero, 0, 0, 0);
+              Dr_all[set][g] = K3 ? __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][g], Br[g], zero, 0, 0, 0) : zero;
+            }
+#pragma unroll
+          for (int set = 0; set < NSET; ++set) {
+            float score = 0.f;
+#pragma unroll
+            for (int g = 0; g < NG; ++g) {
+              const int xc = join_limbs(Dc_all[set][g][2], Dc_all[set][g][1], Dc_all[set][g][0] - sq4[set][g]);
+              float v = (float)xc;
+              if constexpr (K3) v = __builtin_fmaf(eg[g], (float)((Dr_all[set][g][2] << 8) + Dr_all[set][g][1]), v);
+              score = __builtin_fmaf(v, sg[g] * qsc[set][g], score);
+            }
+            const int h = set * 4 + lg;
+            if ((G % 4 == 0) || h < G) {
+              sc[h * L + tok] = valid ? score : -INFINITY;
+              mxl[set] = fmaxf(mxl[set], valid ? score : -INFINITY);
+              mnl[set] = fminf(mnl[set], valid ? score : INFINITY);
+            }
+          }
+          continue;
+        }
 #pragma unroll
         for (int set = 0; set < NSET; ++set) {
           float score = 0.f;
