@@ -58,7 +58,8 @@ def hipcc() -> str:
 
 def _compile(src: str) -> str:
     obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
-    cmd = [hipcc(), *COMMON_FLAGS, "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj]
+    extra = os.environ.get("JETFIRE_BUILD_FLAGS", "").split()   # e.g. -DNAME for a measurement variant
+    cmd = [hipcc(), *COMMON_FLAGS, *extra, "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"hipcc failed on {src}:\n{res.stdout}\n{res.stderr}")

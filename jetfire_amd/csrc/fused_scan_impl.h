@@ -409,7 +409,9 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
 #pragma unroll
     for (int i = 0; i < KLD; ++i) {
       const uint32_t sb = (uint32_t)sbase[chunk * 4 + kl_page[i]];
-      kbuf.r[i] = *reinterpret_cast<const v4u*>(kbase + (size_t)(sb * (uint32_t)KP + kl_off[i]));
+      // (streaming hint: a key row is read exactly once; measured 0.6 - 2 us per launch against plain loads.  The
+      // value rows keep the default policy: the merge kernel gathers the winners' rows again.)
+      kbuf.r[i] = __builtin_nontemporal_load(reinterpret_cast<const v4u*>(kbase + (size_t)(sb * (uint32_t)KP + kl_off[i])));
     }
     return kbuf;
   };
@@ -556,9 +558,10 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     vl_lds[i] = Lds::VSWZ ? (uint32_t)(row * VROW + ((q16 ^ ((row >> 2) & 3)) * 16))
                           : (uint32_t)(row * VROW + (o % VP) + (V3 ? 8 * ((row >> 4) & 1) : 0));  // (INT3: first half's place)
   }
+  // (the V scales of a chunk are not fetched again: position chunk * 64 + lane of step `it` is tid + it * NT, whose
+  // scale word this thread has held in vsw[it] since the set-up)
   struct VBuf {
     v4u r[VLD];
-    uint32_t w;
   };
   auto issue_v = [&](int chunk) -> VBuf {
     VBuf vbuf;
@@ -567,10 +570,6 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
       const uint32_t sb = (uint32_t)sbase[chunk * 4 + vl_page[i]];
       vbuf.r[i] = *reinterpret_cast<const v4u*>(vbase + (size_t)(sb * (uint32_t)VP + vl_off[i]));
     }
-    const int t = chunk * 64 + lane;
-    const uint32_t slot = (uint32_t)(sbase[t >> 4] + (t & 15));
-    if (NG == 2) vbuf.w = *reinterpret_cast<const uint32_t*>(vsbase + (size_t)(slot * 4u));
-    else vbuf.w = (uint32_t) * reinterpret_cast<const uint16_t*>(vsbase + (size_t)(slot * 2u));
     return vbuf;
   };
   // the first two V chunks are requested while the last key chunks are being worked on
@@ -593,6 +592,48 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     Vb = issue_v(min(wave + NW, nch - 1));
   }
 
+
+  // A chunk the sequence ends in (0 < n_local < 64 valid rows; uniform): the staged rows past the end and their
+  // scale words become copies of the last valid row, so the stream's arithmetic runs without a validity select per
+  // score (a copy of a valid score changes neither extremum), and `mask_tail` afterwards stores -inf over what those
+  // positions produced.  A chunk past the end (n_local <= 0) is not worked through at all.
+  auto clone_last_row = [&](int n_local, uint32_t (&Sx)[4], uint32_t (&Zx)[4]) {
+    const int last = n_local - 1, jl = last >> 4;
+    uint32_t sl = Sx[0], zl = Zx[0];
+#pragma unroll
+    for (int j = 1; j < 4; ++j) {
+      sl = (jl == j) ? Sx[j] : sl;
+      zl = (jl == j) ? Zx[j] : zl;
+    }
+    sl = (uint32_t)__builtin_amdgcn_readlane((int)sl, last & 15);
+    zl = (uint32_t)__builtin_amdgcn_readlane((int)zl, last & 15);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const bool past = 16 * j + (lane & 15) >= n_local;
+      Sx[j] = past ? sl : Sx[j];
+      Zx[j] = past ? zl : Zx[j];
+    }
+    constexpr int RDW = KP / 4;  // dwords per staged row
+    const uint8_t* src = kst + last * KROW;
+    for (int i = lane; i < (64 - n_local) * RDW; i += 64) {
+      const int r = n_local + i / RDW, dw = i % RDW;
+      *reinterpret_cast<uint32_t*>(kst + r * KROW + 4 * dw) = *reinterpret_cast<const uint32_t*>(src + 4 * dw);
+    }
+    wave_lds_fence();
+  };
+  auto mask_tail = [&](int chunk, int n_local) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int tl = 16 * j + (lane & 15);
+      if (tl >= n_local) {
+#pragma unroll
+        for (int set = 0; set < NSET; ++set) {
+          const int h = set * 4 + (lane >> 4);
+          if ((G % 4 == 0) || h < G) sc[h * L + chunk * 64 + tl] = -INFINITY;
+        }
+      }
+    }
+  };
 
   // ------------------------------------------------------------------ phase A
   if constexpr (!HAS_K) {
@@ -657,6 +698,13 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
 #pragma unroll
       for (int g = 0; g < NG; ++g) sumq[set][g] = (float)(sq4[set][g] / 2);
     (void)sumq;
+    // (the offset term -sq4 of the limb-0 sum enters as the accumulator's initial value: exact, and one subtraction
+    // per token, head and group less)
+    v4i Cin[NSET][NG];
+#pragma unroll
+    for (int set = 0; set < NSET; ++set)
+#pragma unroll
+      for (int g = 0; g < NG; ++g) Cin[set][g] = (v4i){-sq4[set][g], 0, 0, 0};
     auto body = [&](int chunk, const uint32_t (&Sx)[4], const uint32_t (&Zx)[4]) {
       (void)Zx;
       // all LDS reads of the chunk first (plane dwords of the four pages, rounding coefficients), then arithmetic
@@ -727,7 +775,6 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
           // 2 [c = +-6], r5 = [c = +-5], r7 = [c = +-7], made by byte look-ups: one table for the codes >= 0 (u >= 8,
           // selector u - 8 = c) and one for the codes < 0 (selector u = c + 8), chosen per byte by bit 3 of u.
           const int tok = chunk * 64 + 16 * j + t16;
-          const bool valid = t16 < n - chunk * 64 - 16 * j;  // (tok < n, with the uniform part on one side)
           float acc_s[NSET][NG];
 #pragma unroll
           for (int set = 0; set < NSET; ++set)
@@ -736,12 +783,13 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
               const v4i zero = {0, 0, 0, 0};
               v4i Dc;
               if (NG == 2) {
-                Dc = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][g], Bc[g], zero, 0, 0, 0);
+                Dc = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][g], Bc[g], Cin[set][g], 0, 0, 0);
               } else {
-                Dc = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][0], Bc[0], zero, 0, 0, 0);
+                Dc = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][0], Bc[0], Cin[set][0], 0, 0, 0);
                 Dc = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][1], Bc[1], Dc, 0, 0, 0);
               }
-              acc_s[set][g] = (float)join_limbs(Dc[2], Dc[1], Dc[0] - sq4[set][g]);
+              (void)zero;
+              acc_s[set][g] = (float)join_limbs(Dc[2], Dc[1], Dc[0]);
             }
 #pragma unroll
           for (int c = 0; c < 3; ++c) {  // c = 0, 1, 2: the indicators of +-3 (and +-6), +-5, +-7
@@ -782,9 +830,9 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
             for (int g = 0; g < NG; ++g) score = __builtin_fmaf(acc_s[set][g], sgj[j][g] * qsc[set][g], score);
             const int h = set * 4 + lg;
             if ((G % 4 == 0) || h < G) {
-              sc[h * L + tok] = valid ? score : -INFINITY;
-              mxl[set] = fmaxf(mxl[set], valid ? score : -INFINITY);
-              mnl[set] = fminf(mnl[set], valid ? score : INFINITY);
+              sc[h * L + tok] = score;
+              mxl[set] = fmaxf(mxl[set], score);
+              mnl[set] = fminf(mnl[set], score);
             }
           }
           continue;
@@ -820,7 +868,6 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
             coef[g][3] = (v[3] - v[2]) - (v[1] - v[0]);
           }
           const int tok = chunk * 64 + 16 * j + t16;
-          const bool valid = t16 < n - chunk * 64 - 16 * j;  // (tok < n, with the uniform part on one side)
 #pragma unroll
           for (int set = 0; set < NSET; ++set) {
             const v4i zero = {0, 0, 0, 0};
@@ -851,9 +898,9 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
             }
             const int h = set * 4 + lg;
             if ((G % 4 == 0) || h < G) {
-              sc[h * L + tok] = valid ? score : -INFINITY;
-              mxl[set] = fmaxf(mxl[set], valid ? score : -INFINITY);
-              mnl[set] = fminf(mnl[set], valid ? score : INFINITY);
+              sc[h * L + tok] = score;
+              mxl[set] = fmaxf(mxl[set], score);
+              mnl[set] = fminf(mnl[set], score);
             }
           }
           continue;
@@ -873,7 +920,6 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
           eg[g] = egj[j][g];
         }
         const int tok = chunk * 64 + 16 * j + t16;
-        const bool valid = t16 < n - chunk * 64 - 16 * j;  // (tok < n, with the uniform part on one side)
         if constexpr (NG == 2 && NSET >= 2) {
           // Two head sets: with two wavefronts per SIMD little else hides the wait for an MFMA's results, so all of a
           // token group's products are issued first and read afterwards.
@@ -883,7 +929,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
           for (int set = 0; set < NSET; ++set)
 #pragma unroll
             for (int g = 0; g < NG; ++g) {
-              Dc_all[set][g] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][g], Bc[g], zero, 0, 0, 0);
+              Dc_all[set][g] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][g], Bc[g], Cin[set][g], 0, 0, 0);
               Dr_all[set][g] = K3 ? __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][g], Br[g], zero, 0, 0, 0) : zero;
             }
 #pragma unroll
@@ -891,16 +937,16 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
             float score = 0.f;
 #pragma unroll
             for (int g = 0; g < NG; ++g) {
-              const int xc = join_limbs(Dc_all[set][g][2], Dc_all[set][g][1], Dc_all[set][g][0] - sq4[set][g]);
+              const int xc = join_limbs(Dc_all[set][g][2], Dc_all[set][g][1], Dc_all[set][g][0]);
               float v = (float)xc;
               if constexpr (K3) v = __builtin_fmaf(eg[g], (float)((Dr_all[set][g][2] << 8) + Dr_all[set][g][1]), v);
               score = __builtin_fmaf(v, sg[g] * qsc[set][g], score);
             }
             const int h = set * 4 + lg;
             if ((G % 4 == 0) || h < G) {
-              sc[h * L + tok] = valid ? score : -INFINITY;
-              mxl[set] = fmaxf(mxl[set], valid ? score : -INFINITY);
-              mnl[set] = fminf(mnl[set], valid ? score : INFINITY);
+              sc[h * L + tok] = score;
+              mxl[set] = fmaxf(mxl[set], score);
+              mnl[set] = fminf(mnl[set], score);
             }
           }
           continue;
@@ -912,8 +958,8 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
           if (NG == 2) {
 #pragma unroll
             for (int g = 0; g < NG; ++g) {
-              const v4i Dc = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][g], Bc[g], zero, 0, 0, 0);
-              const int xc = join_limbs(Dc[2], Dc[1], Dc[0] - sq4[set][g]);
+              const v4i Dc = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][g], Bc[g], Cin[set][g], 0, 0, 0);
+              const int xc = join_limbs(Dc[2], Dc[1], Dc[0]);
               float v = (float)xc;
               if constexpr (K3) {
                 const v4i Dr = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][g], Br[g], zero, 0, 0, 0);
@@ -923,9 +969,9 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
               score = __builtin_fmaf(v, sg[g] * qsc[set][g], score);
             }
           } else {
-            v4i Dc = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][0], Bc[0], zero, 0, 0, 0);
+            v4i Dc = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][0], Bc[0], Cin[set][0], 0, 0, 0);
             Dc = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][1], Bc[1], Dc, 0, 0, 0);
-            const int xc = join_limbs(Dc[2], Dc[1], Dc[0] - sq4[set][0]);
+            const int xc = join_limbs(Dc[2], Dc[1], Dc[0]);
             float v = (float)xc;
             if constexpr (K3) {
               v4i Dr = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aop[set][0], Br[0], zero, 0, 0, 0);
@@ -937,9 +983,9 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
           }
           const int h = set * 4 + lg;
           if ((G % 4 == 0) || h < G) {
-            sc[h * L + tok] = valid ? score : -INFINITY;
-            mxl[set] = fmaxf(mxl[set], valid ? score : -INFINITY);
-            mnl[set] = fminf(mnl[set], valid ? score : INFINITY);
+            sc[h * L + tok] = score;
+            mxl[set] = fmaxf(mxl[set], score);
+            mnl[set] = fminf(mnl[set], score);
           }
         }
       }
@@ -964,7 +1010,12 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
           Zc[j] = KA ? reg_copy(cur.z[KA ? j : 0]) : 0u;
         }
         if constexpr (it + 2 < MAXIT) cur = issue_k(min(chunk + 2 * NW, nch_cover - 1));
-        body(chunk, Sc, Zc);
+        const int n_local = n - chunk * 64;  // (uniform)
+        if (n_local > 0) {
+          if (n_local < 64) clone_last_row(n_local, Sc, Zc);
+          body(chunk, Sc, Zc);
+        }
+        if (n_local < 64) mask_tail(chunk, n_local);
         wave_lds_fence();
         if constexpr (it + 1 < MAXIT) self(self, std::integral_constant<int, it + 1>{});
       }
@@ -1028,7 +1079,6 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
         }
         const float ks = bf16_to_f32((uint16_t)Sx[j]);
         const int tok = chunk * 64 + 16 * j + t16;
-        const bool valid = t16 < n - chunk * 64 - 16 * j;  // (tok < n, with the uniform part on one side)
 #pragma unroll
         for (int set = 0; set < NSET; ++set) {
           // (the -8 * sum of the block's query values, the codes being used unsigned, enters as the accumulator's
@@ -1041,9 +1091,9 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
           const float a = __fmul_rn(__fmul_rn(sacc, ks), p.attn_scale);
           const int h = set * 4 + lg;
           if ((G % 4 == 0) || h < G) {
-            sc[h * L + tok] = valid ? a : -INFINITY;
-            mxl[set] = fmaxf(mxl[set], valid ? a : -INFINITY);
-            mnl[set] = fminf(mnl[set], valid ? a : INFINITY);
+            sc[h * L + tok] = a;
+            mxl[set] = fmaxf(mxl[set], a);
+            mnl[set] = fminf(mnl[set], a);
           }
         }
       }
@@ -1057,11 +1107,16 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
         KBuf& cur = (it & 1) ? Kb : Ka;
         stash_k(cur);
         wave_lds_fence();
-        uint32_t Sc[4];
+        uint32_t Sc[4], Zc[4] = {0u, 0u, 0u, 0u};
 #pragma unroll
         for (int j = 0; j < 4; ++j) Sc[j] = reg_copy(cur.s[j]);
         if constexpr (it + 2 < MAXIT) cur = issue_k(min(chunk + 2 * NW, nch_cover - 1));
-        body(chunk, Sc);
+        const int n_local = n - chunk * 64;  // (uniform)
+        if (n_local > 0) {
+          if (n_local < 64) clone_last_row(n_local, Sc, Zc);
+          body(chunk, Sc);
+        }
+        if (n_local < 64) mask_tail(chunk, n_local);
         wave_lds_fence();
         if constexpr (it + 1 < MAXIT) self(self, std::integral_constant<int, it + 1>{});
       }
@@ -1352,7 +1407,8 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
       if constexpr (HAS_V) {
         VBuf& cur = (it & 1) ? Vb : Va;
         stash_v(cur);
-        vw = reg_copy(cur.w);
+        static_assert(VSPT == MAXIT, "one V scale word per thread and step");
+        vw = vsw[it];
         if constexpr (it + 2 < MAXIT) cur = issue_v(min(chunk + 2 * NW, nch - 1));
       }
       body_v(chunk, vw);
