@@ -262,11 +262,11 @@ def measure_gpu_path(name: str, steps: int, warmup: int, lib):
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) / steps * 1e3
     total_ms, launches = ctypes.c_double(0.0), ctypes.c_int(0)
-    _lib.check(lib.jf_profile_scan_begin(n_layers * 3))
+    _lib.check(_lib.debug_hook("jf_profile_scan_begin")(n_layers * 3))
     for _ in range(3):
         step()
     torch.cuda.synchronize()
-    _lib.check(lib.jf_profile_scan_end(ctypes.byref(total_ms), ctypes.byref(launches)))
+    _lib.check(_lib.debug_hook("jf_profile_scan_end")(ctypes.byref(total_ms), ctypes.byref(launches)))
     scan_us = total_ms.value / max(1, launches.value) * 1e3
     achieved = w.packed_bytes_per_layer / (scan_us * 1e-6) / 1e9
     rec = {"workload": f"{name}: B{w.B} Hq{w.H_q} Hkv{w.H_kv} D128 S{w.S} {w.scheme} g{w.group} top_k{w.top_k} x{n_layers} layers",
@@ -382,12 +382,12 @@ def main() -> int:
         src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").random_(0, 255)
         sink = torch.zeros(4, dtype=torch.uint8, device="cuda")
         st = torch.cuda.current_stream().cuda_stream
-        _lib.check(lib.jf_calibrate_stream_read(src.data_ptr(), src.numel(), sink.data_ptr(), st))
+        _lib.check(_lib.debug_hook("jf_calibrate_stream_read")(src.data_ptr(), src.numel(), sink.data_ptr(), st))
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         for _ in range(10):
-            _lib.check(lib.jf_calibrate_stream_read(src.data_ptr(), src.numel(), sink.data_ptr(), st))
+            _lib.check(_lib.debug_hook("jf_calibrate_stream_read")(src.data_ptr(), src.numel(), sink.data_ptr(), st))
         e1.record()
         torch.cuda.synchronize()
         us = e0.elapsed_time(e1) * 100.0
@@ -407,7 +407,7 @@ def main() -> int:
         workloads.CONFIGS[args.workload] = (B_, Hq_, Hkv_, S_, args.scheme or sch_, args.group or gs_, K_, L_)
         args.no_cpu_baseline = args.no_extras = True
     if args.split_len:
-        _lib.check(lib.jf_debug_split_len(args.split_len))
+        _lib.check(_lib.debug_hook("jf_debug_split_len")(args.split_len))
     handoff = args.handoff if args.handoff is not None else args.workload in ("c4", "c5")
     if args.graph is None:
         args.graph = not args.via_adapter
@@ -500,7 +500,7 @@ def main() -> int:
     total_ms = ctypes.c_double(0.0)
     launches = ctypes.c_int(0)
     if graph is None:
-        _lib.check(lib.jf_profile_scan_begin(args.steps * n_layers))
+        _lib.check(_lib.debug_hook("jf_profile_scan_begin")(args.steps * n_layers))
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
@@ -514,13 +514,13 @@ def main() -> int:
         if args.graph:
             h.check_status()
     if graph is None:
-        _lib.check(lib.jf_profile_scan_end(ctypes.byref(total_ms), ctypes.byref(launches)))
+        _lib.check(_lib.debug_hook("jf_profile_scan_end")(ctypes.byref(total_ms), ctypes.byref(launches)))
     else:   # kernel time from a separate eager pass
-        _lib.check(lib.jf_profile_scan_begin(n_layers * 3))
+        _lib.check(_lib.debug_hook("jf_profile_scan_begin")(n_layers * 3))
         for _ in range(3):
             step()
         torch.cuda.synchronize()
-        _lib.check(lib.jf_profile_scan_end(ctypes.byref(total_ms), ctypes.byref(launches)))
+        _lib.check(_lib.debug_hook("jf_profile_scan_end")(ctypes.byref(total_ms), ctypes.byref(launches)))
 
     ms_per_step = elapsed / args.steps * 1e3
     bytes_layer = w.packed_bytes_per_layer

@@ -340,31 +340,8 @@ int jf_fused_scan_topk_static(int scheme, int group_size,
 int jf_fused_plan(int scheme, int group_size, int B, int H_q, int H_kv, int max_S, int top_k,
                   int* split_len, int* n_splits, int* list_cap, int* merge_parts);
 
-/* Measurement aid with no counterpart in the reference: between begin and end, every launch of the fused
- * scan kernel is bracketed by a pair of HIP events recorded on the launch stream (at most max_launches
- * launches); end synchronises them and returns the summed device time and the number of launches. */
-int jf_profile_scan_begin(int max_launches);
-int jf_profile_scan_end(double* total_ms, int* launches);
-/* Measurement aid with no counterpart in the reference: one kernel that streams `bytes` bytes from src with 16-byte
- * loads and writes nothing (sink: 4 bytes of device memory, may be NULL).  Its rate is the read-stream ceiling of
- * this machine, the figure the scan's achieved bandwidth is put beside. */
-int jf_calibrate_stream_read(const void* src, size_t bytes, void* sink, void* stream);
-/* Measurement aid: if device_buffer is non-NULL, every fused-scan workgroup stores ten int64 s_memtime
- * stamps of its phase boundaries at device_buffer[((b * H_kv + hkv) * n_splits + split) * 10 ...], and every
- * merge workgroup eight at device_buffer[B * H_kv * n_splits * 10 + (b * H_q + hq) * 8 ...] (which stamp
- * marks which boundary is internal to the kernels and may change).  NULL switches it off. */
-int jf_debug_phase_clock(void* device_buffer);
-/* Test / measurement aid with no counterpart in the reference: a positive split_len (rounded up to a
- * multiple of 256 and clamped to what fits the kernel's LDS) replaces the planner's choice of the split
- * length in jf_fused_scan_topk and jf_fused_workspace_bytes; 0 restores the planner.  Process-wide. */
-int jf_debug_split_len(int split_len);
-/* Test aids for the CPU pool, no counterpart in the reference.  jf_debug_pool_stall: the worker that claims `row` of
- * the next correction job sleeps `microseconds` before it computes the row (one shot), as if it had lost its core.
- * jf_debug_pool_wait_stragglers(0): jf_cpu_topk_attn returns as soon as every row is committed, like the hand-off
- * jobs do, instead of also waiting for workers that are still inside a row (the caller must then keep its tensors
- * alive); 1 restores the default. */
-int jf_debug_pool_stall(int64_t row, int microseconds);
-int jf_debug_pool_wait_stragglers(int on);
+/* Measurement and test hooks (kernel timing by HIP events, phase stamps, a forced split length, pool stalls ...)
+ * are declared in jetfire_amd_debug.h and exist only in a library built with -DJF_DEBUG_HOOKS. */
 
 /* ------------------------------------------------------------------ piece 4: merge
  * out = bf16_rne(fma(W, f32(o_new), o_hat) - o_old_unnorm).  Replaces blend_unnorm_into
@@ -440,9 +417,6 @@ int jf_handoff_set_device_wait_limit_us(jf_handoff* h, int64_t us);
 /* on != 0: jf_handoff_stream_wait_blend writes zero for every non-finite output element, the graph-mode guard of
  * _sanitize_decode_output_if_needed (jetfire_vllm/adapter/decode_path.py:1133-1149) folded into the blend. */
 int jf_handoff_set_output_sanitize(jf_handoff* h, int on);
-/* Test aid: while on, the dispatcher ignores published flags (a correction that never finishes, without
- * hanging anything: the device-side wait runs into its limit). */
-int jf_handoff_debug_pause(jf_handoff* h, int on);
 
 /* Row implementation of the CPU correction: 0 scalar (cpu_topk_attn.cpp:602-690), 1 AVX2+FMA, 2 AVX-512-BF16
  * (vdpbf16ps row, jetfire_vllm/csrc/cpu_topk_attn.cpp:316-479).  The widest one the host supports is used unless
@@ -490,6 +464,28 @@ int jf_graph_pool_warmup(int n_threads);
 int64_t jf_graph_submit_count(void);
 int jf_reset_graph_runtime_state(void);
 int jf_clear_graph_contexts(void);
+/* get_shadow_append_count (jetfire_vllm/csrc/cpu_topk_attn.cpp:2353-2355; read by jetfire_get_graph_stats,
+ * jetfire_vllm/adapter/decode_path.py:1017-1023): launches of the shadow mirror kernel that have run on the current
+ * device, replays from a HIP graph included (the reference counts its graph-mode append callbacks).  reset != 0
+ * zeroes the counter after reading it.  Copies one word from the device: call it outside graph capture. */
+int jf_shadow_append_count(int64_t* count, int reset);
+/* reset_graph_submit_count (jetfire_vllm/csrc/cpu_topk_attn.cpp:2436-2470; called by reset_jetfire_graph_stats,
+ * jetfire_vllm/adapter/decode_path.py:1041-1045): zeroes the submit, shadow-append and sanitise counters and the
+ * timing statistics below. */
+int jf_reset_graph_submit_count(void);
+/* get_graph_timing_stats (jetfire_vllm/csrc/cpu_topk_attn.cpp:2361-2434) as an array of JF_GRAPH_TIMING_FIELDS
+ * doubles: [0] topk_jobs (corrections run for hand-off contexts), [1] topk_done_avg_us, [2] topk_done_max_us (their
+ * duration on the worker pool), [3] shadow_append_jobs, [4] join_jobs (host-blocking jf_handoff_wait calls),
+ * [5] join_wait_avg_us, [6] join_wait_max_us, [7] pool_workers, [8] pool_done_count (jobs the pool has finished).
+ * This library has no host callbacks, so the reference's submit-callback times and "last call" words do not exist. */
+#define JF_GRAPH_TIMING_FIELDS 9
+int jf_graph_timing_stats(double* out, int n);
+/* No counterpart in the reference (its graph submit callback runs on a host thread and wakes the pool itself):
+ * jf_pool_wake brings sleeping workers of the correction pool back to spinning for the next job; jf_pool_doorbell
+ * enqueues a one-lane kernel on `stream` (capturable) that has the poller thread do the same when the GPU reaches
+ * it - put it at the head of a decode step so that the first layer's correction does not pay the pool's wake-up. */
+int jf_pool_wake(void);
+int jf_pool_doorbell(void* stream);
 
 #ifdef __cplusplus
 }

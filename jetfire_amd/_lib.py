@@ -44,13 +44,6 @@ SIGNATURES = {
     "jf_topk_slots_fast": (I, [P, P, P, I, I, I, I, I, I, P, P, P, P, P, Z, P]),
     "jf_stage_b_softmax_v": (I, [I, I, P, P, P, P, P, P, I, I, I, I, I, L, I, I, P, P, P, P, Z, P]),
     "jf_fused_scan_topk_static": (I, [I, I, P, P, P, P, P, P, P, I, I, I, I, I, L, I, F, I, P, P, P, P, P, P, P, P, P]),
-    "jf_calibrate_stream_read": (I, [P, Z, P, P]),
-    "jf_profile_scan_begin": (I, [I]),
-    "jf_profile_scan_end": (I, [P, P]),
-    "jf_debug_phase_clock": (I, [P]),
-    "jf_debug_split_len": (I, [I]),
-    "jf_debug_pool_stall": (I, [L, I]),
-    "jf_debug_pool_wait_stragglers": (I, [I]),
     "jf_fused_plan": (I, [I, I, I, I, I, I, I, P, P, P, P]),
     "jf_blend_unnorm": (I, [P, P, P, P, P, I, I, I, P]),
     "jf_cpu_topk_attn": (I, [P, P, P, P, P, P, I, I, I, I, L, F, P]),
@@ -66,7 +59,6 @@ SIGNATURES = {
     "jf_handoff_status": (I, [P]),
     "jf_handoff_set_device_wait_limit_us": (I, [P, L]),
     "jf_handoff_set_output_sanitize": (I, [P, I]),
-    "jf_handoff_debug_pause": (I, [P, I]),
     "jf_handoff_destroy": (None, [P]),
     "jf_blend": (I, [P, P, P, P, P, I, I, I, P]),
     "jf_set_cpu_attn_isa": (I, [I]),
@@ -85,6 +77,23 @@ SIGNATURES = {
     "jf_graph_submit_count": (L, []),
     "jf_reset_graph_runtime_state": (I, []),
     "jf_clear_graph_contexts": (I, []),
+    "jf_shadow_append_count": (I, [P, I]),
+    "jf_reset_graph_submit_count": (I, []),
+    "jf_graph_timing_stats": (I, [P, I]),
+    "jf_pool_wake": (I, []),
+    "jf_pool_doorbell": (I, [P]),
+}
+
+# the measurement / test hooks of include/jetfire_amd_debug.h: present only in a library built with -DJF_DEBUG_HOOKS
+DEBUG_SIGNATURES = {
+    "jf_calibrate_stream_read": (I, [P, Z, P, P]),
+    "jf_profile_scan_begin": (I, [I]),
+    "jf_profile_scan_end": (I, [P, P]),
+    "jf_debug_phase_clock": (I, [P]),
+    "jf_debug_split_len": (I, [I]),
+    "jf_debug_pool_stall": (I, [L, I]),
+    "jf_debug_pool_wait_stragglers": (I, [I]),
+    "jf_handoff_debug_pause": (I, [P, I]),
 }
 
 _lib = None
@@ -104,8 +113,26 @@ def load() -> C.CDLL:
         fn = getattr(lib, name)
         fn.restype = res
         fn.argtypes = args
+    for name, (res, args) in DEBUG_SIGNATURES.items():
+        fn = getattr(lib, name, None)
+        if fn is not None:
+            fn.restype = res
+            fn.argtypes = args
     _lib = lib
     return lib
+
+
+def has_debug_hooks() -> bool:
+    """Whether the loaded library was built with -DJF_DEBUG_HOOKS (tests and bench.py need that build)."""
+    return load().jf_version().decode().endswith("+debug-hooks")
+
+
+def debug_hook(name: str):
+    """A hook of include/jetfire_amd_debug.h, or a RuntimeError that says which build has it."""
+    fn = getattr(load(), name, None) if name in DEBUG_SIGNATURES else None
+    if fn is None or not has_debug_hooks():
+        raise RuntimeError(f"{name} is a measurement / test hook: rebuild with `python -m jetfire_amd.build --debug-hooks`")
+    return fn
 
 
 def check(rc: int) -> None:

@@ -46,23 +46,46 @@ class JetFireConfig:
 _CONFIG: JetFireConfig | None = None
 
 
+def _env(name: str, default, *aliases: str):
+    """The reference's variable `name` (jetfire_vllm/adapter/config.py:306-388); `aliases` are names earlier versions
+    of this adapter read, still honoured when the reference's own name is not set."""
+    for n in (name, *aliases):
+        if n in os.environ:
+            return os.environ[n]
+    return default
+
+
 def _from_env() -> JetFireConfig:
-    name = os.environ.get("JETFIRE_QUANT_SCHEME", "SymInt3K_SymInt2V")
+    name = _env("JETFIRE_MODE", "SymInt3K_SymInt2V", "JETFIRE_QUANT_SCHEME")
     if name not in SCHEMES:
-        raise ValueError(f"JETFIRE_QUANT_SCHEME={name!r} is not one of {sorted(SCHEMES)}")
+        raise ValueError(f"JETFIRE_MODE={name!r} is not a known quant scheme. Available: {sorted(SCHEMES)}")
     scheme = SCHEMES[name]
+    use_custom = os.environ.get("JETFIRE_USE_CUSTOM_BACKEND", "1") == "1"
+    cpu_corr = os.environ.get("JETFIRE_CPU_CORRECTION", "1") == "1"
+    skip_native = os.environ.get("JETFIRE_SKIP_NATIVE_KV", "1") == "1"
+    shadow = os.environ.get("JETFIRE_SHADOW", "1") == "1"
+    stride = int(_env("JETFIRE_MIRROR_LAYER_STRIDE", 1, "JETFIRE_LAYER_STRIDE"))
+    if use_custom:  # the reference's invariants (jetfire_vllm/adapter/config.py:337-358)
+        if not cpu_corr and skip_native and shadow:
+            raise ValueError("JETFIRE_CPU_CORRECTION=0 + JETFIRE_SKIP_NATIVE_KV=1 with shadow on is unsupported (decode "
+                             "would have nowhere to go). Either enable CPU correction (default) or also set "
+                             "JETFIRE_SHADOW=0 for a prefill-only configuration.")
+        if stride > 1 and skip_native:
+            raise ValueError(f"JETFIRE_MIRROR_LAYER_STRIDE={stride} skips some layers, which fall back to the native "
+                             "attention, but JETFIRE_SKIP_NATIVE_KV=1 has freed the native KV cache. Set "
+                             "JETFIRE_SKIP_NATIVE_KV=0 for this ablation.")
     return JetFireConfig(
         scheme=scheme,
         group_size=int(os.environ.get("JETFIRE_GROUP_SIZE", scheme.default_group_size)),
         topk=int(os.environ.get("JETFIRE_TOPK", 256)),
-        layer_stride=int(os.environ.get("JETFIRE_LAYER_STRIDE", 1)),
-        use_custom_backend=os.environ.get("JETFIRE_USE_CUSTOM_BACKEND", "1") == "1",
-        cpu_correction=os.environ.get("JETFIRE_CPU_CORRECTION", "1") == "1",
-        shadow_enabled=os.environ.get("JETFIRE_SHADOW", "1") == "1",
-        skip_native_kv=os.environ.get("JETFIRE_SKIP_NATIVE_KV", "1") == "1",
+        layer_stride=stride,
+        use_custom_backend=use_custom,
+        cpu_correction=cpu_corr,
+        shadow_enabled=shadow,
+        skip_native_kv=skip_native,
         max_batch_size=int(os.environ.get("JETFIRE_MAX_BATCH_SIZE", 0)),
         cpu_attn_threads=int(os.environ.get("JETFIRE_CPU_ATTN_THREADS", 0)),
-        debug_log=os.environ.get("JETFIRE_DEBUG", "0") == "1",
+        debug_log=_env("JETFIRE_DEBUG_LOG", "0", "JETFIRE_DEBUG") == "1",
     )
 
 
@@ -81,3 +104,9 @@ def set_jetfire_config(**changes) -> JetFireConfig:
         changes["scheme"] = SCHEMES[changes["scheme"]]
     _CONFIG = replace(get_jetfire_config(), **changes)
     return _CONFIG
+
+
+def reset_jetfire_config() -> None:
+    """Re-read the environment on the next `get_jetfire_config()` (jetfire_vllm/adapter/config.py:393-396)."""
+    global _CONFIG
+    _CONFIG = None

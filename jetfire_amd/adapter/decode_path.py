@@ -355,21 +355,32 @@ def _decode_batched(*, impl, layer, query, attn_metadata, output):
         max_S = int(getattr(attn_metadata, "max_seq_len", int(seq_lens_cpu.max().item())))
     # Under the release policy (JETFIRE_RELEASE_GRAPH_POLICY=1) the step runs the two kernels the policy names for
     # this cell, through the split operators; otherwise the fused scan where it covers the scheme.
-    release = release_policy.release_policy_enabled() and not store.k_asymmetric
+    # (every store goes through the policy, as in the reference, `decode_path.py:1857-1868`: a mode outside the
+    # release set raises there instead of falling through to another path silently)
+    release = release_policy.release_policy_enabled()
     if release:
         release_policy.validate_release_environment()
     top_k = _select_top_k(pool.config.topk, max_S, SPLIT_SUPPORTED_TOP_K)
     if top_k is None:
         return miss("seq_len_too_short")
     # the fused scan where it covers the scheme and the width; wider corrections run the stage-wise kernels
-    fused = (not release and store.scheme is not None and top_k in FUSED_SUPPORTED_TOP_K
+    # The scoring model of INT4 keys with one scale per row depends on the width and on JETFIRE_USE_INT8_TC, as in
+    # the reference (`decode_path.py:2012-2022`): the int8-quantised-query model from top_k 64 up, else the bf16 model.
+    scheme = store.scheme
+    if scheme is not None and scheme.startswith("k4") and (
+            top_k < 64 or os.environ.get("JETFIRE_USE_INT8_TC", "1") != "1"):
+        scheme = "b4" + scheme[2:]
+    fused = (not release and scheme is not None and top_k in FUSED_SUPPORTED_TOP_K
              and int(store.k_data.shape[1]) <= ops.FUSED_MAX_SLOTS and os.environ.get("JETFIRE_USE_FUSED_ATTN_TOPK", "1") == "1")
     plan = None
     if release:
+        mode = (f"AsymInt2K4Level_SymInt{store.v_nbits}V" if store.k_asymmetric
+                else f"SymInt{store.k_nbits}K_SymInt{store.v_nbits}V")
+        cfg_max_B = int(get_jetfire_config().max_batch_size or 0)
         plan = release_policy.plan_release_graph(
-            mode=f"SymInt{store.k_nbits}K_SymInt{store.v_nbits}V", group_size=store.group_size, top_k=top_k, head_dim=D,
+            mode=mode, group_size=store.group_size, top_k=top_k, head_dim=D,
             num_query_heads=H_q, num_kv_heads=H_kv,
-            max_graph_batch=max(n_seqs, int(get_jetfire_config().max_batch_size or 0)),
+            max_graph_batch=cfg_max_B if cfg_max_B > 0 else n_seqs,
             require_ready=release_policy.release_require_ready())
 
     q_batch = query[:n_seqs].contiguous().view(n_seqs, H_q, D).to(torch.bfloat16)
@@ -378,7 +389,7 @@ def _decode_batched(*, impl, layer, query, attn_metadata, output):
 
     if fused:
         o_hat, topk_slots, o_old, W, _ = ops.fused_attn_topk(
-            store.scheme, q_batch, store.k_data, store.k_scales, store.v_data, store.v_scales, bt_batch, seq_lens_batch,
+            scheme, q_batch, store.k_data, store.k_scales, store.v_data, store.v_scales, bt_batch, seq_lens_batch,
             max_S, H_q, H_kv, store.block_size, top_k, scale, k_zp=store.k_zp if store.k_asymmetric else None)
     else:
         o_hat, topk_slots, o_old, W = _split_stages(store, q_batch, bt_batch, seq_lens_batch, max_S, H_q, H_kv, top_k, scale,

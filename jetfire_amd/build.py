@@ -1,11 +1,13 @@
 """Builds libjetfire_amd.so (HIP kernels + C ABI) for gfx950 with hipcc, in-tree.
 
 `python -m jetfire_amd.build` compiles every source under jetfire_amd/csrc and links the shared
-library next to the package.  Nothing here needs a GPU: hipcc cross-compiles.
+library next to the package; `--debug-hooks` adds the measurement / test entry points the tests and bench.py use.
+Nothing here needs a GPU: hipcc cross-compiles.
 """
 from __future__ import annotations
 
 import concurrent.futures
+import hashlib
 import os
 import shutil
 import subprocess
@@ -56,9 +58,30 @@ def hipcc() -> str:
     return exe
 
 
-def _compile(src: str) -> str:
-    obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
+def _extra_flags(debug_hooks: bool) -> list:
     extra = os.environ.get("JETFIRE_BUILD_FLAGS", "").split()   # e.g. -DNAME for a measurement variant
+    if debug_hooks or os.environ.get("JETFIRE_DEBUG_HOOKS", "0") == "1":
+        extra.append("-DJF_DEBUG_HOOKS")                         # the hooks of include/jetfire_amd_debug.h
+    return extra
+
+
+def build_id(extra: list) -> str:
+    """Digest of everything the library is made from (sources, headers, flags): jf_version() carries it, so a
+    measurement can name the exact code it ran."""
+    h = hashlib.sha256()
+    names = sorted(os.listdir(CSRC)) + ["../../include/jetfire_amd.h", "../../include/jetfire_amd_debug.h"]
+    for name in names:
+        path = os.path.join(CSRC, name)
+        if os.path.isfile(path):
+            h.update(name.encode())
+            with open(path, "rb") as f:
+                h.update(f.read())
+    h.update(" ".join(COMMON_FLAGS + sorted(extra)).encode())
+    return h.hexdigest()[:12]
+
+
+def _compile(src: str, extra: list) -> str:
+    obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
     cmd = [hipcc(), *COMMON_FLAGS, *extra, "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
@@ -70,11 +93,15 @@ def _compile(src: str) -> str:
     return obj
 
 
-def build_library(verbose: bool = True) -> str:
-    """Compile all sources (always, even when a library is already there) and link the .so."""
+def build_library(verbose: bool = True, debug_hooks: bool = False) -> str:
+    """Compile all sources (always, even when a library is already there) and link the .so.  `debug_hooks` (or
+    JETFIRE_DEBUG_HOOKS=1) compiles the measurement / test entry points of include/jetfire_amd_debug.h in: the tests
+    and bench.py need them, a product build leaves them out."""
     os.makedirs(OBJ_DIR, exist_ok=True)
+    extra = _extra_flags(debug_hooks)
+    extra = extra + [f'-DJF_BUILD_ID="{build_id(extra)}"']
     with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as ex:
-        objs = list(ex.map(_compile, SOURCES))
+        objs = list(ex.map(lambda src: _compile(src, extra), SOURCES))
     tmp = LIB_PATH + ".tmp"
     cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", tmp, "-lpthread"]
     res = subprocess.run(cmd, capture_output=True, text=True)
@@ -87,4 +114,4 @@ def build_library(verbose: bool = True) -> str:
 
 
 if __name__ == "__main__":
-    build_library()
+    build_library(debug_hooks="--debug-hooks" in sys.argv[1:])

@@ -4,6 +4,8 @@
 // reference.
 #include "common.h"
 
+#ifdef JF_DEBUG_HOOKS
+
 namespace jf {
 namespace {
 typedef unsigned v4u __attribute__((ext_vector_type(4)));
@@ -41,3 +43,4 @@ extern "C" int jf_calibrate_stream_read(const void* src, size_t bytes, void* sin
   JF_CHECK_LAUNCH();
   return JF_OK;
 }
+#endif  // JF_DEBUG_HOOKS

@@ -6,6 +6,9 @@
 #include <stdarg.h>
 #include <math.h>
 #include "../../include/jetfire_amd.h"
+#ifdef JF_DEBUG_HOOKS
+#include "../../include/jetfire_amd_debug.h"
+#endif
 
 namespace jf {
 

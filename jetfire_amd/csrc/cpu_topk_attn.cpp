@@ -60,9 +60,11 @@ struct CpuJob {
 // One row (sequence, query head) of the job into `out` (128 bf16 values of the caller's choosing).
 static void compute_row(const CpuJob& j, int64_t r, uint16_t* out);
 
+#ifdef JF_DEBUG_HOOKS
 // Test aid: the worker that claims this row of the next job sleeps first (one shot); see jf_debug_pool_stall.
 static std::atomic<int64_t> g_stall_row{-1};
 static std::atomic<int> g_stall_us{0};
+#endif
 // Whether a synchronous call returns only after every worker has left its rows (default; the caller may free its
 // tensors right after the call).  Jobs over buffers that outlive them (the hand-off contexts) never wait.
 static std::atomic<int> g_wait_stragglers{1};
@@ -163,7 +165,20 @@ class Pool {
   }
   // Starts (or resizes) the workers without running anything.
   void warm() { ensure_workers(); }
-  // Returns when no worker is inside a row.
+  // Sleeping workers go back to spinning for the next job (for JETFIRE_POOL_SPIN_US): called when a decode step
+  // is known to be on its way, so that its first layer does not pay the wake-up of the whole pool.
+  void wake() {
+    ensure_workers();
+    wake_gen_.fetch_add(1, std::memory_order_acq_rel);
+    { std::lock_guard<std::mutex> g(mu_); }
+    cv_work_.notify_all();
+  }
+  int64_t jobs_done() const { return jobs_done_.load(std::memory_order_relaxed); }
+  int worker_count() {
+    std::lock_guard<std::mutex> g(mu_);
+    return (int)workers_.size();
+  }
+  // Returns when no worker is inside a job (between its first claim and its last look at the rows).
   void quiesce() {
     while (active_.load(std::memory_order_acquire) != 0) std::this_thread::sleep_for(std::chrono::microseconds(20));
   }
@@ -237,30 +252,37 @@ class Pool {
     }();
     return s;
   }
-  // Computes row r of the job of epoch e and commits it unless somebody else has.
+  // Computes row r of the job of epoch e and commits it unless somebody else has.  The caller (worker) holds
+  // `active_` raised from before it claims a row or scans the tags until it has left the job, so quiesce() also
+  // waits for a worker that sits between a claim and its row.
   void do_row(const Job& jb, uint64_t e, int64_t r, bool claimed) {
     uint16_t local[D];
-    active_.fetch_add(1, std::memory_order_acq_rel);
+#ifdef JF_DEBUG_HOOKS
     if (claimed) {
       int64_t sr = g_stall_row.load(std::memory_order_relaxed);
       if (sr == r && g_stall_row.compare_exchange_strong(sr, -1))
         std::this_thread::sleep_for(std::chrono::microseconds(g_stall_us.load(std::memory_order_relaxed)));
     }
+#else
+    (void)claimed;
+#endif
     compute_row(jb.cj, r, local);
     // the row's tag holds the epoch of the last job that committed it: a tag below e means that the job of epoch e
     // is still current and the row is open; the worker that moves it to e owns the row's output
     uint64_t old = tags_[r].load(std::memory_order_acquire);
-    while (old < e) {
+    // (a job that has been withdrawn, or followed by a newer one, commits nothing: its output buffer and the row
+    // count now belong to somebody else)
+    while (old < e && epoch_.load(std::memory_order_acquire) == e) {
       if (tags_[r].compare_exchange_weak(old, e, std::memory_order_acq_rel, std::memory_order_acquire)) {
         memcpy(jb.cj.o_new + r * D, local, sizeof(local));
         if (done_rows_.fetch_add(1, std::memory_order_acq_rel) + 1 >= jb.n) {
+          jobs_done_.fetch_add(1, std::memory_order_relaxed);
           std::lock_guard<std::mutex> g(mu_);
           cv_done_.notify_all();
         }
         break;
       }
     }
-    active_.fetch_sub(1, std::memory_order_acq_rel);
   }
   // JETFIRE_CPU_ATTN_PIN=1 (jetfire_vllm/csrc/cpu_topk_attn.cpp:895-905, jetfire_pool.h:141-149): worker i stays on
   // one core.  The reference binds it to core i; here it is the i-th core the process may run on (the same core
@@ -304,11 +326,21 @@ class Pool {
       }
       if (!got) {
         std::unique_lock<std::mutex> lk(mu_);
-        cv_work_.wait(lk, [&] { return stop_ || epoch_.load(std::memory_order_acquire) != seen; });
+        const uint64_t wg = wake_gen_.load(std::memory_order_acquire);
+        cv_work_.wait(lk, [&] {
+          return stop_ || epoch_.load(std::memory_order_acquire) != seen || wake_gen_.load(std::memory_order_acquire) != wg;
+        });
       }
       if (stop_flag()) return;
       const uint64_t e = epoch_.load(std::memory_order_acquire);
+      if (e == seen) continue;  // woken ahead of a job (wake()): back to spinning for it
       seen = e;
+      // from here until this worker has left the job it counts as active: quiesce() waits for it
+      struct ActiveScope {
+        std::atomic<int>& a;
+        explicit ActiveScope(std::atomic<int>& x) : a(x) { a.fetch_add(1, std::memory_order_acq_rel); }
+        ~ActiveScope() { a.fetch_sub(1, std::memory_order_acq_rel); }
+      } in_job(active_);
       // A private copy of the job: its slot is rewritten by the job after next at the earliest, so the copy is
       // whole if the epoch has moved by at most one since it was read.
       const Job jb = jobs_[e & 1];
@@ -355,7 +387,9 @@ class Pool {
   }
 
   std::mutex mu_, cfg_mu_, resize_mu_;
-  std::atomic<int> active_{0};          // workers inside a row
+  std::atomic<int> active_{0};          // workers inside a job (from before their first claim until they leave it)
+  std::atomic<uint64_t> wake_gen_{0};   // bumped by wake()
+  std::atomic<int64_t> jobs_done_{0};   // jobs whose last row has been committed
   std::condition_variable cv_work_, cv_done_;
   std::vector<std::thread> workers_;
   Job jobs_[2];
@@ -656,7 +690,17 @@ static void compute_row(const CpuJob& j, int64_t r, uint16_t* out) {
 using namespace jf;
 
 extern "C" const char* jf_last_error(void) { return g_err; }
-extern "C" const char* jf_version(void) { return "jetfire_amd 0.1 (gfx950)"; }
+#ifndef JF_BUILD_ID
+#define JF_BUILD_ID "unknown"
+#endif
+#ifdef JF_DEBUG_HOOKS
+#define JF_HOOKS_TAG " +debug-hooks"
+#else
+#define JF_HOOKS_TAG ""
+#endif
+// "jetfire_amd <release> (gfx950) build <id>[ +debug-hooks]": the id is a digest of the sources and flags the library
+// was built from (jetfire_amd/build.py), so a measurement can be tied to the exact code that ran
+extern "C" const char* jf_version(void) { return "jetfire_amd 0.3 (gfx950) build " JF_BUILD_ID JF_HOOKS_TAG; }
 
 extern "C" int jf_set_cpu_attn_threads(int n) {
   Pool::instance().set_threads(n);
@@ -672,6 +716,7 @@ extern "C" int jf_set_cpu_attn_isa(int isa) {
 extern "C" int jf_get_cpu_attn_isa(void) { return resolve_isa(); }
 extern "C" int64_t jf_cpu_topk_sanitize_count(void) { return g_sanitize_count.load(); }
 
+#ifdef JF_DEBUG_HOOKS
 extern "C" int jf_debug_pool_stall(int64_t row, int microseconds) {
   JF_CHECK_ARG(microseconds >= 0 && microseconds <= 10000000, "debug_pool_stall: bad duration");
   g_stall_us.store(microseconds);
@@ -683,6 +728,7 @@ extern "C" int jf_debug_pool_wait_stragglers(int on) {
   if (on) Pool::instance().quiesce();
   return JF_OK;
 }
+#endif  // JF_DEBUG_HOOKS
 
 extern "C" int jf_cpu_topk_attn(const uint16_t* q, const uint16_t* k_shadow, const uint16_t* v_shadow,
                                 const int64_t* head_map, const int64_t* ts_buf, uint16_t* o_new, int B, int H_q, int K,
@@ -868,6 +914,25 @@ inline void cpu_relax() {
 }
 
 std::atomic<int64_t> g_graph_submits{0};   // stream-mode submits served by the poller (get_graph_submit_count)
+// what get_graph_timing_stats reports (jetfire_vllm/csrc/cpu_topk_attn.cpp:2361-2434): the corrections the poller ran
+// and the host-blocking joins, count / total / longest in nanoseconds
+std::atomic<int64_t> g_topk_jobs{0}, g_topk_ns{0}, g_topk_max_ns{0};
+std::atomic<int64_t> g_join_jobs{0}, g_join_ns{0}, g_join_max_ns{0};
+inline void stat_add(std::atomic<int64_t>& n, std::atomic<int64_t>& tot, std::atomic<int64_t>& mx, int64_t dt) {
+  n.fetch_add(1, std::memory_order_relaxed);
+  tot.fetch_add(dt, std::memory_order_relaxed);
+  int64_t cur = mx.load(std::memory_order_relaxed);
+  while (dt > cur && !mx.compare_exchange_weak(cur, dt, std::memory_order_relaxed)) {}
+}
+inline int64_t steady_ns() {
+  return std::chrono::duration_cast<std::chrono::nanoseconds>(std::chrono::steady_clock::now().time_since_epoch()).count();
+}
+// Doorbell of the pool: a word in pinned host memory that a one-lane kernel at the head of a decode step (or of its
+// HIP graph) bumps; the poller thread sees the change and wakes the pool's workers ahead of the first layer's job.
+int64_t* g_doorbell_pin = nullptr;   // [0]: the word the kernel bumps
+int64_t* g_doorbell_dev = nullptr;   // the same word as the device sees it
+int64_t g_doorbell_seen = 0;         // (poller thread only)
+std::mutex g_doorbell_mu;
 
 bool run_correction(jf_handoff* h) {
   if (h->ext_q) {  // the caller's buffers, its head map and 64-bit slots
@@ -939,7 +1004,9 @@ void handoff_dispatch(jf_handoff* h) {
       continue;
     }
     seen = f;
+    const int64_t t_job = steady_ns();
     if (!run_correction(h)) h->failed.store(1);
+    stat_add(g_topk_jobs, g_topk_ns, g_topk_max_ns, steady_ns() - t_job);
     h->submits.fetch_add(1, std::memory_order_relaxed);
     h->done_seq.store(seen, std::memory_order_release);
   }
@@ -985,8 +1052,8 @@ struct StreamPoller {
       bool served = false;
       {
         std::unique_lock<std::mutex> lk(mu);
-        if (ctxs.empty()) {
-          cv.wait(lk, [&] { return !ctxs.empty(); });
+        if (ctxs.empty() && __atomic_load_n(&g_doorbell_pin, __ATOMIC_ACQUIRE) == nullptr) {
+          cv.wait(lk, [&] { return !ctxs.empty() || __atomic_load_n(&g_doorbell_pin, __ATOMIC_ACQUIRE) != nullptr; });
           idle_since = std::chrono::steady_clock::now();
         }
         for (jf_handoff* h : ctxs) {
@@ -994,6 +1061,7 @@ struct StreamPoller {
           const int64_t f = __atomic_load_n(h->flag_pin, __ATOMIC_ACQUIRE);
           if (f == h->stream_seen) continue;
           h->stream_seen = f;
+          const int64_t t_job = steady_ns();
           if (!run_correction(h)) {
             h->failed.store(1);
             __atomic_store_n(h->flag_pin + 16, (int64_t)2, __ATOMIC_RELEASE);
@@ -1001,6 +1069,15 @@ struct StreamPoller {
           h->submits.fetch_add(1, std::memory_order_relaxed);
           g_graph_submits.fetch_add(1, std::memory_order_relaxed);
           __atomic_store_n(h->flag_pin + 8, f, __ATOMIC_RELEASE);  // what the device-side wait polls
+          stat_add(g_topk_jobs, g_topk_ns, g_topk_max_ns, steady_ns() - t_job);
+          served = true;
+        }
+      }
+      if (int64_t* db = __atomic_load_n(&g_doorbell_pin, __ATOMIC_ACQUIRE)) {
+        const int64_t v = __atomic_load_n(db, __ATOMIC_ACQUIRE);
+        if (v != g_doorbell_seen) {  // a step is on its way: have the workers spinning when its first job arrives
+          g_doorbell_seen = v;
+          Pool::instance().wake();
           served = true;
         }
       }
@@ -1152,11 +1229,13 @@ extern "C" int jf_handoff_set_device_wait_limit_us(jf_handoff* h, int64_t us) {
   return JF_OK;
 }
 
+#ifdef JF_DEBUG_HOOKS
 extern "C" int jf_handoff_debug_pause(jf_handoff* h, int on) {
   JF_CHECK_ARG(h, "handoff_debug_pause: null argument");
   h->paused.store(on ? 1 : 0);
   return JF_OK;
 }
+#endif  // JF_DEBUG_HOOKS
 
 extern "C" int jf_handoff_wait(jf_handoff* h, uint16_t* o_new_dev, void* stream) {
   JF_CHECK_ARG(h && o_new_dev, "handoff_wait: null argument");
@@ -1173,6 +1252,8 @@ extern "C" int jf_handoff_wait(jf_handoff* h, uint16_t* o_new_dev, void* stream)
       if (el > 0.002) std::this_thread::sleep_for(std::chrono::microseconds(50));
     }
   }
+  stat_add(g_join_jobs, g_join_ns, g_join_max_ns,
+           std::chrono::duration_cast<std::chrono::nanoseconds>(std::chrono::steady_clock::now() - t0).count());
   if (h->failed.load()) { set_error("handoff: CPU correction job failed or timed out"); return JF_ERR_TIMEOUT; }
   const int n16 = (int)((size_t)h->B * h->H_q * D * sizeof(uint16_t) / 16);
   hipLaunchKernelGGL(handoff_fetch_kernel, dim3((n16 + 255) / 256 < 8 ? (n16 + 255) / 256 : 8), dim3(256), 0, st,
@@ -1395,6 +1476,60 @@ extern "C" int jf_graph_pool_warmup(int n_threads) {
 }
 
 extern "C" int64_t jf_graph_submit_count(void) { return g_graph_submits.load(); }
+
+extern "C" int jf_graph_timing_stats(double* out, int n) {
+  JF_CHECK_ARG(out && n >= JF_GRAPH_TIMING_FIELDS, "graph_timing_stats: room for %d values needed", JF_GRAPH_TIMING_FIELDS);
+  const int64_t jobs = g_topk_jobs.load(), joins = g_join_jobs.load();
+  int64_t appends = 0;
+  (void)jf_shadow_append_count(&appends, 0);
+  out[0] = (double)jobs;
+  out[1] = jobs > 0 ? (double)g_topk_ns.load() / (double)jobs / 1000.0 : 0.0;
+  out[2] = (double)g_topk_max_ns.load() / 1000.0;
+  out[3] = (double)appends;
+  out[4] = (double)joins;
+  out[5] = joins > 0 ? (double)g_join_ns.load() / (double)joins / 1000.0 : 0.0;
+  out[6] = (double)g_join_max_ns.load() / 1000.0;
+  out[7] = (double)Pool::instance().worker_count();
+  out[8] = (double)Pool::instance().jobs_done();
+  return JF_OK;
+}
+
+extern "C" int jf_reset_graph_submit_count(void) {
+  g_graph_submits.store(0);
+  g_sanitize_count.store(0);
+  for (std::atomic<int64_t>* c : {&g_topk_jobs, &g_topk_ns, &g_topk_max_ns, &g_join_jobs, &g_join_ns, &g_join_max_ns}) c->store(0);
+  int64_t unused = 0;
+  return jf_shadow_append_count(&unused, 1);
+}
+
+// One lane bumps the doorbell word (system scope: the poller thread reads it from host memory).
+__global__ void pool_doorbell_kernel(int64_t* word) {
+  __hip_atomic_fetch_add(word, (int64_t)1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+extern "C" int jf_pool_wake(void) {
+  Pool::instance().wake();
+  return JF_OK;
+}
+
+extern "C" int jf_pool_doorbell(void* stream) {
+  {
+    std::lock_guard<std::mutex> g(g_doorbell_mu);
+    if (g_doorbell_dev == nullptr) {  // once per process: the word, its device address, the poller
+      int64_t* pin = nullptr;
+      JF_CHECK_HIP(hipHostMalloc(reinterpret_cast<void**>(&pin), 64, hipHostMallocMapped));
+      memset(pin, 0, 64);
+      void* dev = nullptr;
+      JF_CHECK_HIP(hipHostGetDevicePointer(&dev, pin, 0));
+      g_doorbell_dev = reinterpret_cast<int64_t*>(dev);
+      __atomic_store_n(&g_doorbell_pin, pin, __ATOMIC_RELEASE);
+      StreamPoller::instance().cv.notify_one();
+    }
+  }
+  hipLaunchKernelGGL(pool_doorbell_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, g_doorbell_dev);
+  JF_CHECK_LAUNCH();
+  return JF_OK;
+}
 
 extern "C" int jf_reset_graph_runtime_state(void) {
   Pool::instance().quiesce();  // a straggling worker may still be reading a finished job's buffers

@@ -3,10 +3,12 @@
 #include "fused_scan_impl.h"
 
 namespace jf {
+#ifdef JF_DEBUG_HOOKS
 ScanProfile g_prof;
 std::mutex g_prof_mu;
 std::atomic<long long*> g_phase_clock{nullptr};
 std::atomic<int> g_force_split_len{0};
+#endif
 
 int device_cus() {
   static const int cus = [] {
@@ -119,6 +121,8 @@ extern "C" int jf_fused_scan_topk_static(int scheme, int group_size, const uint1
                                          float* o_hat, float* o_old_unnorm, float* W, float* softmax_m,
                                          float* softmax_inv_z, float* scores, void* stream) {
   JF_CHECK_ARG(known_scheme(scheme), "fused_scan_static: unknown scheme %d", scheme);
+  JF_CHECK_ARG(!scheme_has_zp(scheme),
+               "fused_scan_static: the asymmetric INT2 key formats need their zero-points: use jf_fused_scan_topk_asym");
   JF_CHECK_ARG(B >= 0 && H_q > 0 && H_kv > 0 && max_S >= 0 && H_q % H_kv == 0 && top_k > 0,
                "fused_scan_static: bad shape");
   const size_t need = jf_fused_workspace_bytes(scheme, B, H_q, H_kv, max_S, top_k);
@@ -146,6 +150,7 @@ extern "C" int jf_fused_scan_topk_static(int scheme, int group_size, const uint1
                             (size_t)JF_FUSED_STATIC_SCRATCH_BYTES, stream);
 }
 
+#ifdef JF_DEBUG_HOOKS
 extern "C" int jf_profile_scan_begin(int max_launches) {
   JF_CHECK_ARG(max_launches > 0 && max_launches <= (1 << 20), "profile_scan_begin: bad max_launches=%d", max_launches);
   std::lock_guard<std::mutex> lock(g_prof_mu);
@@ -186,3 +191,4 @@ extern "C" int jf_debug_split_len(int split_len) {
   g_force_split_len.store(split_len);
   return JF_OK;
 }
+#endif  // JF_DEBUG_HOOKS

@@ -47,9 +47,10 @@
 
 namespace jf {
 
+#ifdef JF_DEBUG_HOOKS
 // Process-wide measurement / test switches shared by those translation units (defined in fused_scan.hip),
-// reachable from the public debug entry points: the event list has its own lock, the two scalars are atomics
-// (a launch reads each once).
+// reachable from the debug entry points of jetfire_amd_debug.h; a library built without JF_DEBUG_HOOKS has none of
+// them.  The event list has its own lock, the two scalars are atomics (a launch reads each once).
 // Optional measurement hook: when armed, every fused_scan_kernel launch is bracketed by a pair of HIP
 // events on its own stream, so a benchmark can read the kernel's device time without a profiler.
 struct ScanProfile {
@@ -61,6 +62,10 @@ extern ScanProfile g_prof;
 extern std::mutex g_prof_mu;
 extern std::atomic<long long*> g_phase_clock;
 extern std::atomic<int> g_force_split_len;  // test / measurement aid: overrides the planner's split length when positive
+constexpr bool kDebugHooks = true;
+#else
+constexpr bool kDebugHooks = false;
+#endif
 // Compute units of the current device (the planner balances workgroups over them); 256, the MI355X count, when
 // no device can be asked (planning on a host without a GPU).
 int device_cus();
@@ -328,7 +333,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   const uint8_t* vbase = p.v_data + (size_t)hkv * p.num_slots * VP;
   const uint8_t* vsbase = reinterpret_cast<const uint8_t*>(p.v_scales + (size_t)hkv * p.num_slots * NG);
 
-  long long* clk = p.phase_clock ? p.phase_clock + (((size_t)b * p.H_kv + hkv) * p.n_splits + split) * 10 : nullptr;
+  long long* clk = (kDebugHooks && p.phase_clock) ? p.phase_clock + (((size_t)b * p.H_kv + hkv) * p.n_splits + split) * 10 : nullptr;
   if (clk && tid == 0) clk[0] = clock64();
 
   // The page-table entry and the query elements of this thread do not depend on the sequence length: they
@@ -1794,7 +1799,7 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   const int rounds = (flat + MG_THREADS - 1) / MG_THREADS;
   const int nblk_lds = min(p.max_blocks, MG_BT);
 
-  long long* mclk = (p.phase_clock && !PARTIAL) ? p.phase_clock + (size_t)p.B * p.H_kv * p.n_splits * 10 + bh * 8 : nullptr;
+  long long* mclk = (kDebugHooks && p.phase_clock && !PARTIAL) ? p.phase_clock + (size_t)p.B * p.H_kv * p.n_splits * 10 + bh * 8 : nullptr;
   if (mclk && tid == 0) mclk[0] = clock64();
 
   // ---- everything that does not depend on anything else is requested first, in the order of its use.  Every load
@@ -2459,11 +2464,13 @@ inline void fused_plan(int scheme, int NG, int B, int H_q, int H_kv, int max_S, 
     }
     if (cand >= max_S) break;
   }
+#ifdef JF_DEBUG_HOOKS
   if (const int forced = g_force_split_len.load(std::memory_order_relaxed); forced > 0) {
     L = (forced + 255) / 256 * 256;
     if (L > lmax) L = lmax;
     while ((max_S + L - 1) / L > MG_MAX_SPLITS && L < lmax) L += 256;
   }
+#endif
   int ns = (max_S + L - 1) / L;
   if (ns < 1) ns = 1;
   *L_out = L;
@@ -2510,6 +2517,7 @@ int launch_scan(const FusedParams& p, hipStream_t st) {
       attr_smem = smem;
     }
   }
+#ifdef JF_DEBUG_HOOKS
   std::unique_lock<std::mutex> plock(g_prof_mu, std::defer_lock);
   bool prof = false;
   if (g_prof.armed) {  // (read without the lock: arming happens-before the launches a benchmark times)
@@ -2518,12 +2526,15 @@ int launch_scan(const FusedParams& p, hipStream_t st) {
     if (!prof) plock.unlock();
   }
   if (prof) JF_CHECK_HIP(hipEventRecord(g_prof.ev[g_prof.used], st));
+#endif
   hipLaunchKernelGGL(kern, dim3(p.n_splits, p.H_kv, p.B), dim3(ScanLds<SCHEME, G, NG>::NT), smem, st, p);
   JF_CHECK_LAUNCH();
+#ifdef JF_DEBUG_HOOKS
   if (prof) {
     JF_CHECK_HIP(hipEventRecord(g_prof.ev[g_prof.used + 1], st));
     g_prof.used += 2;
   }
+#endif
   return JF_OK;
 }
 
@@ -2663,7 +2674,11 @@ static int fused_run(int scheme, int group_size, const uint16_t* q, const uint8_
   p.topk_idx = topk_idx; p.topk_slots = topk_slots; p.o_hat = o_hat; p.o_old = o_old_unnorm; p.W = W;
   p.softmax_m = softmax_m; p.softmax_inv_z = softmax_inv_z;
   p.blend_o_new = blend_o_new; p.blend_out = blend_out;
+#ifdef JF_DEBUG_HOOKS
   p.phase_clock = g_phase_clock.load(std::memory_order_relaxed);
+#else
+  p.phase_clock = nullptr;
+#endif
   hipStream_t st = (hipStream_t)stream;
   int rc = JF_OK;
 #define JF_FUSED_CASE(SCH, GG, NGG) rc = launch_scan<MODE, SCH, GG, NGG>(p, st)

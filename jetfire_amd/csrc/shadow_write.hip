@@ -17,12 +17,17 @@ struct MirrorSrc {
 
 // LPR lanes own one row: 16 lanes x 16 bytes, or 64 lanes x 4 bytes for rows that are only 4-byte aligned.
 // Grid: x = blocks of 256 / LPR tokens, y = kv-head, z = tensor (K, V).
+// Mirror launches that have run on this device, replays from a HIP graph included (the reference counts its
+// graph-mode append callbacks, jetfire_vllm/csrc/cpu_topk_attn.cpp:1611-1616); device code only.
+__device__ unsigned long long shadow_appends;
+
 template <int LPR>
 __global__ __launch_bounds__(256) void shadow_write_kernel(MirrorSrc k, MirrorSrc v, uint16_t* __restrict__ k_shadow,
                                                            uint16_t* __restrict__ v_shadow, int64_t stride_h,
                                                            int64_t stride_slot, const int64_t* __restrict__ slots,
                                                            int64_t T, int64_t num_slots) {
   constexpr int RPB = 256 / LPR;
+  if ((blockIdx.x | blockIdx.y | blockIdx.z | threadIdx.x) == 0) atomicAdd(&shadow_appends, 1ull);
   const int l = threadIdx.x % LPR;
   const int64_t t = (int64_t)blockIdx.x * RPB + threadIdx.x / LPR;
   if (t >= T) return;
@@ -98,5 +103,17 @@ extern "C" int jf_shadow_write(const uint16_t* key, int64_t k_stride_t, int64_t 
                        shadow_stride_slot, slots, T, num_slots);
   }
   JF_CHECK_LAUNCH();
+  return JF_OK;
+}
+
+extern "C" int jf_shadow_append_count(int64_t* count, int reset) {
+  JF_CHECK_ARG(count, "shadow_append_count: null output");
+  unsigned long long v = 0;
+  JF_CHECK_HIP(hipMemcpyFromSymbol(&v, HIP_SYMBOL(shadow_appends), sizeof(v)));
+  *count = (int64_t)v;
+  if (reset) {
+    const unsigned long long zero = 0;
+    JF_CHECK_HIP(hipMemcpyToSymbol(HIP_SYMBOL(shadow_appends), &zero, sizeof(zero)));
+  }
   return JF_OK;
 }

@@ -9,7 +9,7 @@ _NAMES = (
     "set_cpu_attn_threads", "get_cpu_attn_threads", "stream_write_value64", "stream_wait_value64",
     "create_cpu_topk_submit_ctx", "stream_submit_cpu_topk_attn", "stream_wait_cpu_topk_attn", "graph_pool_warmup",
     "graph_pool_warmup_threads", "get_graph_submit_count", "get_cpu_topk_sanitize_count", "reset_graph_runtime_state",
-    "clear_graph_contexts",
+    "clear_graph_contexts", "get_shadow_append_count", "reset_graph_submit_count", "get_graph_timing_stats",
 )
 
 
@@ -21,4 +21,6 @@ def load_cpu_topk_attn_ext():
     ext.check_cpu_topk_submit_ctx = ops.check_cpu_topk_submit_ctx
     ext.set_cpu_attn_isa = ops.set_cpu_attn_isa
     ext.get_cpu_attn_isa = ops.get_cpu_attn_isa
+    ext.pool_wake = ops.pool_wake
+    ext.pool_doorbell = ops.pool_doorbell
     return ext

@@ -15,4 +15,5 @@ def load_softmax_v_ext():
     _lib.load()
     return SimpleNamespace(
         int4_softmax_v_with_pre_corr_wvs2_scores=ops.int4_softmax_v_with_pre_corr_wvs2_scores,
-        int4_softmax_v_with_pre_corr_wvs2=ops.int4_softmax_v_with_pre_corr_wvs2)
+        int4_softmax_v_with_pre_corr_wvs2=ops.int4_softmax_v_with_pre_corr_wvs2,
+        int4_softmax_v_with_pre_corr_wvs2_inplace=ops.int4_softmax_v_with_pre_corr_wvs2_inplace)

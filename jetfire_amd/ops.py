@@ -7,6 +7,7 @@ Tensors are only used for device memory and the current stream; all arithmetic i
 """
 from __future__ import annotations
 
+import ctypes
 import os
 from typing import List, Optional
 
@@ -646,6 +647,14 @@ def int4_softmax_v_with_pre_corr_wvs2(scores, v_data, v_scales, block_table, seq
                                                     H_q, H_kv, block_size, top_k)
 
 
+def int4_softmax_v_with_pre_corr_wvs2_inplace(scores, v_data, v_scales, block_table, seq_lens, topk_idx, weights,
+                                              o_hat, o_old_unnorm, W_out, max_S, H_q, H_kv, block_size, top_k) -> None:
+    """int4_softmax_v.cu:927-1040 (what graph mode looks up under JETFIRE_GRAPH_STAGEB_INPLACE,
+    jetfire_vllm/adapter/decode_path.py:2872-2919): caller-owned outputs; `weights` is accepted and unused."""
+    _softmax_v(scores, None, None, v_data, v_scales, block_table, seq_lens, topk_idx, max_S, H_q, H_kv, block_size,
+               top_k, 4, outs=(o_hat, o_old_unnorm, W_out))
+
+
 def int8tc_softmax_v_with_pre_corr_reg_stats(scores, softmax_m, softmax_inv_z, v_data, v_scales, block_table, seq_lens,
                                              topk_idx, max_S, H_q, H_kv, block_size, top_k) -> List[torch.Tensor]:
     """int8tc_softmax_v_fused.cu:1591-1734 -> [o_hat, o_old_unnorm, W], with the reference's arithmetic: P * v_scale
@@ -990,6 +999,47 @@ def get_cpu_topk_sanitize_count() -> int:
     return int(_lib.load().jf_cpu_topk_sanitize_count())
 
 
+def get_shadow_append_count() -> int:
+    """Mirror-kernel launches that have run on the current device, graph replays included
+    (jetfire_vllm/csrc/cpu_topk_attn.cpp:2353-2355)."""
+    n = ctypes.c_int64(0)
+    _lib.check(_lib.load().jf_shadow_append_count(ctypes.byref(n), 0))
+    return int(n.value)
+
+
+def reset_graph_submit_count() -> None:
+    """Zero the submit / shadow-append / sanitise counters and the timing statistics
+    (jetfire_vllm/csrc/cpu_topk_attn.cpp:2436-2470)."""
+    _lib.check(_lib.load().jf_reset_graph_submit_count())
+
+
+_TIMING_FIELDS = ("topk_jobs", "topk_done_avg_us", "topk_done_max_us", "shadow_append_jobs", "join_jobs",
+                  "join_wait_avg_us", "join_wait_max_us", "pool_workers", "pool_done_count")
+
+
+def get_graph_timing_stats() -> dict:
+    """The counters this library keeps under the reference's key names
+    (jetfire_vllm/csrc/cpu_topk_attn.cpp:2361-2434): counts are ints, times floats in microseconds."""
+    buf = (ctypes.c_double * len(_TIMING_FIELDS))()
+    _lib.check(_lib.load().jf_graph_timing_stats(buf, len(_TIMING_FIELDS)))
+    out = {k: (float(v) if k.endswith("_us") else int(v)) for k, v in zip(_TIMING_FIELDS, buf)}
+    out["pool_initialized"] = out["pool_workers"] > 0
+    return out
+
+
+def pool_wake() -> None:
+    """Sleeping workers of the correction pool go back to spinning for the next job (call at the start of a decode
+    step issued from the host)."""
+    _lib.check(_lib.load().jf_pool_wake())
+
+
+def pool_doorbell(stream_id: Optional[int] = None) -> None:
+    """The same from the GPU's side: a one-lane kernel on the stream (capturable; put it at the head of a decode
+    step's graph) that has the poller thread wake the pool when the GPU reaches it."""
+    st = torch.cuda.current_stream().cuda_stream if stream_id is None else int(stream_id)
+    _lib.check(_lib.load().jf_pool_doorbell(st))
+
+
 def reset_graph_runtime_state() -> None:
     _lib.check(_lib.load().jf_reset_graph_runtime_state())
 
@@ -1083,7 +1133,7 @@ class CpuTopkHandoff:
         _lib.check(_lib.load().jf_handoff_set_device_wait_limit_us(self._h, int(us)))
 
     def debug_pause(self, on: bool) -> None:
-        _lib.check(_lib.load().jf_handoff_debug_pause(self._h, 1 if on else 0))
+        _lib.check(_lib.debug_hook("jf_handoff_debug_pause")(self._h, 1 if on else 0))
 
     @property
     def submit_count(self) -> int:

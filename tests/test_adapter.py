@@ -729,3 +729,122 @@ def test_backend_shim_appends_and_decodes_on_the_gpu(adapter):
                            Kfull, Vfull)
     res = bf16_to_f32(out).reshape(B, Hq, D)
     np.testing.assert_allclose(res, r["out"], atol=6e-3, rtol=1.5e-2)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("top_k,int8_tc,k_model", [(32, "1", "bf16"), (64, "0", "bf16"), (64, "1", "int8")])
+def test_int4_keys_take_the_reference_scoring_model_for_the_width(adapter, monkeypatch, top_k, int8_tc, k_model):
+    """INT4 keys with one scale per row are scored with the int8-quantised-query model only from top_k 64 up and
+    with JETFIRE_USE_INT8_TC=1 (`jetfire_vllm/adapter/decode_path.py:2012-2022`); otherwise with the bf16 model of
+    `int4_qk_scores`.  The fused path must follow: the winners equal the oracle's under that model."""
+    monkeypatch.setenv("JETFIRE_USE_INT8_TC", int8_tc)
+    B, Hq, Hkv, D, bs, max_S = 2, 8, 2, 128, 16, 256
+    adapter.set_jetfire_config(scheme="SymInt4K_SymInt4V", group_size=128, topk=top_k, layer_stride=1, cpu_attn_threads=2)
+    adapter.reset_global_kv_pool_manager()
+    pool = adapter.get_global_kv_pool_manager()
+    name = "model.layers.0.self_attn.attn"
+    layer = types.SimpleNamespace(layer_name=name, num_heads=Hq, num_kv_heads=Hkv, head_size=D)
+    impl = types.SimpleNamespace(attn_type=types.SimpleNamespace(name="DECODER"), scale=D ** -0.5)
+    pool.ensure_layer_config_from_layer(name, layer)
+    per_seq = max_S // bs
+    pool.register_layer_layout(name, num_blocks=B * per_seq, block_size=bs)
+    rng = np.random.default_rng(29)
+    lens = [230, 117]
+    bt = np.arange(B * per_seq, dtype=np.int64).reshape(B, per_seq)
+    slots = np.concatenate([bt[b, np.arange(lens[b]) // bs] * bs + np.arange(lens[b]) % bs for b in range(B)])
+    n = len(slots)
+    k_np = O.bf16_round(rng.standard_normal((n, Hkv, D)).astype(np.float32))
+    v_np = O.bf16_round(rng.standard_normal((n, Hkv, D)).astype(np.float32))
+    pool.mirror_kv(name, bf16_tensor(k_np).cuda(), bf16_tensor(v_np).cuda(), torch.from_numpy(slots).cuda())
+    pool.flush_pending_writes()
+    q_np = O.bf16_round((rng.standard_normal((B, Hq, D)) / np.sqrt(D)).astype(np.float32))
+    out = torch.zeros(B, Hq * D, dtype=torch.bfloat16, device="cuda")
+    meta = _meta(torch.tensor(lens, dtype=torch.int32, device="cuda"), torch.from_numpy(bt).cuda(), max_seq_len=max(lens))
+    from jetfire_amd import ops as jops
+    seen = []
+    real = jops.fused_attn_topk
+    monkeypatch.setattr(jops, "fused_attn_topk", lambda scheme, *a, **k: (seen.append(scheme), real(scheme, *a, **k))[1])
+    assert adapter.try_jetfire_decode(impl=impl, layer=layer, query=bf16_tensor(q_np).cuda(), attn_metadata=meta,
+                                      output=out) is out
+    torch.cuda.synchronize()
+    assert seen == [("b4v4" if k_model == "bf16" else "k4v4")]
+    Kfull = np.zeros((Hkv, B * max_S, D), np.float32)
+    Vfull = np.zeros((Hkv, B * max_S, D), np.float32)
+    Kfull[:, slots] = k_np.transpose(1, 0, 2)
+    Vfull[:, slots] = v_np.transpose(1, 0, 2)
+    kd, ks = O.quantize_and_pack(Kfull, 128, 4)
+    vd, vs = O.quantize_and_pack(Vfull, 128, 4)
+    r = O.decode_reference(q_np, kd, ks, vd, vs, bt, np.array(lens, np.int32), max(lens), Hq, Hkv, bs, D ** -0.5, top_k,
+                           "k4v4", Kfull, Vfull, group_size=128, k_model=k_model)
+    res = bf16_to_f32(out).reshape(B, Hq, D)
+    np.testing.assert_allclose(res, r["out"], atol=6e-3, rtol=1.5e-2)
+    err = np.abs(res - r["out"])
+    assert err.max() <= 2e-2 and err.mean() <= 1e-3
+
+
+@pytest.mark.gpu
+def test_release_policy_refuses_a_store_outside_the_release_modes(adapter, monkeypatch):
+    """Under JETFIRE_RELEASE_GRAPH_POLICY=1 every store is planned (`decode_path.py:1857-1868`): asymmetric INT2 keys
+    are outside the release modes and raise instead of running another path silently."""
+    from jetfire_amd.adapter import release_policy
+    for name in list(__import__("os").environ):
+        if name.startswith("JETFIRE_"):
+            monkeypatch.delenv(name)
+    B, Hq, Hkv, D, bs, K, max_S = 1, 8, 2, 128, 16, 64, 128
+    adapter.set_jetfire_config(scheme="AsymInt2K4Level_SymInt2V", group_size=64, topk=K, layer_stride=1,
+                               cpu_attn_threads=2, max_batch_size=0)
+    adapter.reset_global_kv_pool_manager()
+    pool = adapter.get_global_kv_pool_manager()
+    name = "model.layers.0.self_attn.attn"
+    layer = types.SimpleNamespace(layer_name=name, num_heads=Hq, num_kv_heads=Hkv, head_size=D)
+    impl = types.SimpleNamespace(attn_type=types.SimpleNamespace(name="DECODER"), scale=D ** -0.5)
+    pool.ensure_layer_config_from_layer(name, layer)
+    pool.register_layer_layout(name, num_blocks=max_S // bs, block_size=bs)
+    g = torch.Generator().manual_seed(3)
+    n = 100
+    pool.mirror_kv(name, torch.randn(n, Hkv, D, generator=g).to(torch.bfloat16).cuda(),
+                   torch.randn(n, Hkv, D, generator=g).to(torch.bfloat16).cuda(), torch.arange(n).cuda())
+    pool.flush_pending_writes()
+    meta = _meta(torch.tensor([n], dtype=torch.int32, device="cuda"), torch.arange(max_S // bs).view(1, -1).cuda(),
+                 max_seq_len=n)
+    q = torch.zeros(B, Hq, D, dtype=torch.bfloat16, device="cuda")
+    out = torch.zeros(B, Hq * D, dtype=torch.bfloat16, device="cuda")
+    assert adapter.try_jetfire_decode(impl=impl, layer=layer, query=q, attn_metadata=meta, output=out) is out
+    monkeypatch.setenv("JETFIRE_RELEASE_GRAPH_POLICY", "1")
+    with pytest.raises(release_policy.ReleasePolicyError, match="mode"):
+        adapter.try_jetfire_decode(impl=impl, layer=layer, query=q, attn_metadata=meta, output=out)
+
+
+@pytest.mark.gpu
+def test_backend_shim_defers_a_prefill_append_until_its_attention_is_enqueued(adapter, monkeypatch):
+    """JETFIRE_DEFER_PREFILL_KV_MIRROR=force (`jetfire_backend.py:32-63,196-209`): `do_kv_cache_update` parks a large
+    chunk on the layer, the engine's prefill `forward` runs, then the append happens; small chunks are never parked."""
+    from jetfire_amd.adapter.jetfire_backend import make_jetfire_attention_impl
+    monkeypatch.setenv("JETFIRE_DEFER_PREFILL_KV_MIRROR", "force")
+    B, Hq, Hkv, D, bs = 1, 8, 2, 128, 16
+    adapter.set_jetfire_config(scheme="SymInt3K_SymInt2V", group_size=64, topk=32, layer_stride=1, cpu_attn_threads=2,
+                               skip_native_kv=True)
+    adapter.reset_global_kv_pool_manager()
+    pool = adapter.get_global_kv_pool_manager()
+    impl = make_jetfire_attention_impl(_NativeImpl)()
+    layer = types.SimpleNamespace(layer_name="model.layers.0.self_attn.attn", num_heads=Hq, num_kv_heads=Hkv, head_size=D)
+    pool.register_layer_layout(layer.layer_name, num_blocks=16, block_size=bs)
+    k = torch.randn(96, Hkv, D).to(torch.bfloat16).cuda()
+    slots = torch.arange(96).cuda()
+    impl.do_kv_cache_update(layer, k, k, None, slots)
+    assert hasattr(layer, "_jetfire_deferred_kv_mirror")
+    store = pool.get_layer_store(layer.layer_name)
+    assert store is None or int(store.slot_filled.sum()) == 0
+    prefill = _meta(torch.tensor([96], dtype=torch.int32, device="cuda"), torch.arange(16).view(1, -1).cuda(),
+                    max_query_len=96)
+    out = torch.zeros(96, Hq * D, dtype=torch.bfloat16, device="cuda")
+    assert impl.forward(layer, torch.zeros(96, Hq, D, dtype=torch.bfloat16, device="cuda"), k, k, None, prefill,
+                        output=out) == "native"
+    assert not hasattr(layer, "_jetfire_deferred_kv_mirror")
+    pool.flush_pending_writes()
+    torch.cuda.synchronize()
+    store = pool.get_layer_store(layer.layer_name)
+    assert int(store.slot_filled.sum()) == 96
+    small = torch.randn(4, Hkv, D).to(torch.bfloat16).cuda()
+    impl.do_kv_cache_update(layer, small, small, None, torch.arange(96, 100).cuda())
+    assert not hasattr(layer, "_jetfire_deferred_kv_mirror")

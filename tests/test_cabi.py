@@ -13,8 +13,8 @@ from tests.helpers import bf16_tensor, bf16_to_f32, make_case
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def header_symbols():
-    text = open(os.path.join(ROOT, "include", "jetfire_amd.h")).read()
+def header_symbols(name="jetfire_amd.h"):
+    text = open(os.path.join(ROOT, "include", name)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(jf_[a-z0-9_]+)\s*\(", text)))
 
@@ -29,6 +29,23 @@ def test_library_exports_every_declared_symbol():
         assert n in _lib.SIGNATURES, f"{n} has no ctypes signature"
     assert set(_lib.SIGNATURES) == set(names)
     assert b"gfx950" in lib.jf_version()
+
+
+def test_debug_hooks_live_in_their_own_header_and_only_in_a_hooks_build():
+    """The product header declares no measurement / test hook; a library exports the hooks of
+    include/jetfire_amd_debug.h exactly when its version string says it was built with them."""
+    from jetfire_amd import _lib
+    lib = _lib.load()
+    product, hooks = header_symbols(), header_symbols("jetfire_amd_debug.h")
+    assert not [n for n in product if "debug" in n or "profile" in n or "calibrate" in n]
+    assert set(hooks) == set(_lib.DEBUG_SIGNATURES) and not set(hooks) & set(product)
+    built_with = lib.jf_version().decode().endswith("+debug-hooks")
+    assert built_with == _lib.has_debug_hooks()
+    for n in hooks:
+        assert hasattr(lib, n) == built_with, f"{n}: exported={hasattr(lib, n)}, hooks build={built_with}"
+    if not built_with:
+        with pytest.raises(RuntimeError, match="--debug-hooks"):
+            _lib.debug_hook("jf_debug_split_len")
 
 
 def test_every_declaration_cites_the_reference_interface_it_replaces():
@@ -227,9 +244,9 @@ def test_cpu_pool_backs_up_a_row_whose_worker_has_stalled():
     assert not torch.equal(want1, want2)
     q, ts, out = q1.clone(), ts1.clone(), torch.zeros(B, Hq, 128, dtype=torch.bfloat16)
     stall_s = 0.6
-    _lib.check(lib.jf_debug_pool_wait_stragglers(0))
+    _lib.check(_lib.debug_hook("jf_debug_pool_wait_stragglers")(0))
     try:
-        _lib.check(lib.jf_debug_pool_stall(5, int(stall_s * 1e6)))
+        _lib.check(_lib.debug_hook("jf_debug_pool_stall")(5, int(stall_s * 1e6)))
         t0 = time.perf_counter()
         ops.cpu_topk_attn(q, ksh, vsh, hm, ts, out, 0.09)
         took = time.perf_counter() - t0
@@ -245,9 +262,9 @@ def test_cpu_pool_backs_up_a_row_whose_worker_has_stalled():
         ops.cpu_topk_attn(q, ksh, vsh, hm, ts, out, 0.09)     # and the pool is whole again
         assert torch.equal(out.view(torch.int16), want2.view(torch.int16))
     finally:
-        _lib.check(lib.jf_debug_pool_wait_stragglers(1))
+        _lib.check(_lib.debug_hook("jf_debug_pool_wait_stragglers")(1))
     # default behaviour of the synchronous call: it returns only when no worker is inside a row any more
-    _lib.check(lib.jf_debug_pool_stall(3, 200000))
+    _lib.check(_lib.debug_hook("jf_debug_pool_stall")(3, 200000))
     t0 = time.perf_counter()
     ops.cpu_topk_attn(q, ksh, vsh, hm, ts, out, 0.09)
     assert time.perf_counter() - t0 >= 0.19
@@ -378,12 +395,12 @@ def test_fused_plan_geometry_is_consistent(scheme, gs, B, Hq, Hkv, S, K):
     floor = rows * ns * (8 + 128 * 4 + cap * 8 + 4) + (rows * parts * (K * 8 + 4) if parts > 1 else 0)
     assert need >= floor
     # forcing a split length is honoured (rounded up to 256, clamped) and switched off again by 0
-    _lib.check(lib.jf_debug_split_len(300))
+    _lib.check(_lib.debug_hook("jf_debug_split_len")(300))
     try:
         _lib.check(lib.jf_fused_plan(scheme, gs, B, Hq, Hkv, S, K, C.byref(out[0]), None, None, None))
         assert out[0].value == 512 or (S > 512 * 256 and out[0].value > 512)
     finally:
-        _lib.check(lib.jf_debug_split_len(0))
+        _lib.check(_lib.debug_hook("jf_debug_split_len")(0))
     _lib.check(lib.jf_fused_plan(scheme, gs, B, Hq, Hkv, S, K, C.byref(out[0]), None, None, None))
     assert out[0].value == L
 
@@ -394,3 +411,52 @@ def test_fused_plan_rejects_bad_shapes():
     assert lib.jf_fused_plan(7, 64, 1, 8, 2, 100, 32, None, None, None, None) != 0
     assert lib.jf_fused_plan(32, 64, 1, 8, 3, 100, 32, None, None, None, None) != 0
     assert lib.jf_fused_plan(32, 32, 1, 8, 2, 100, 32, None, None, None, None) != 0
+
+
+def test_adapter_reads_the_reference_environment_names(monkeypatch):
+    """`jetfire_vllm/adapter/config.py:306-388`: JETFIRE_MODE, JETFIRE_MIRROR_LAYER_STRIDE, JETFIRE_DEBUG_LOG (the names
+    this adapter used before stay as aliases), and the two invariants that protect a freed native KV cache."""
+    from jetfire_amd.adapter import config
+    for n in list(os.environ):
+        if n.startswith("JETFIRE_"):
+            monkeypatch.delenv(n)
+    config.reset_jetfire_config()
+    try:
+        monkeypatch.setenv("JETFIRE_MODE", "SymInt4K_SymInt4V")
+        monkeypatch.setenv("JETFIRE_QUANT_SCHEME", "SymInt2K_SymInt2V")      # the reference's name wins
+        monkeypatch.setenv("JETFIRE_DEBUG_LOG", "1")
+        cfg = config.get_jetfire_config()
+        assert cfg.scheme.name == "SymInt4K_SymInt4V" and cfg.debug_log and cfg.layer_stride == 1
+        config.reset_jetfire_config()
+        monkeypatch.delenv("JETFIRE_MODE")
+        assert config.get_jetfire_config().scheme.name == "SymInt2K_SymInt2V"   # alias alone still works
+        config.reset_jetfire_config()
+        monkeypatch.setenv("JETFIRE_MIRROR_LAYER_STRIDE", "2")
+        with pytest.raises(ValueError, match="JETFIRE_MIRROR_LAYER_STRIDE=2"):
+            config.get_jetfire_config()
+        monkeypatch.setenv("JETFIRE_SKIP_NATIVE_KV", "0")
+        assert config.get_jetfire_config().layer_stride == 2
+        config.reset_jetfire_config()
+        monkeypatch.delenv("JETFIRE_MIRROR_LAYER_STRIDE")
+        monkeypatch.setenv("JETFIRE_LAYER_STRIDE", "3")
+        assert config.get_jetfire_config().layer_stride == 3
+        config.reset_jetfire_config()
+        monkeypatch.setenv("JETFIRE_SKIP_NATIVE_KV", "1")
+        monkeypatch.delenv("JETFIRE_LAYER_STRIDE")
+        monkeypatch.setenv("JETFIRE_CPU_CORRECTION", "0")
+        with pytest.raises(ValueError, match="JETFIRE_CPU_CORRECTION=0"):
+            config.get_jetfire_config()
+        monkeypatch.setenv("JETFIRE_MODE", "NoSuchMode")
+        with pytest.raises(ValueError, match="JETFIRE_MODE='NoSuchMode'"):
+            config.get_jetfire_config()
+    finally:
+        config.reset_jetfire_config()
+
+
+def test_pool_wake_needs_no_gpu():
+    from jetfire_amd import ops
+    ops.set_cpu_attn_threads(2)
+    ops.pool_wake()
+    ops.pool_wake()
+    assert ops.get_cpu_attn_threads() == 2
+    ops.set_cpu_attn_threads(0)

@@ -161,3 +161,73 @@ def test_blend_forms_agree():
     assert (got.float() - unnorm.float()).abs().max() <= 0.02 * (1 + want.abs().max())
     with pytest.raises(RuntimeError, match="o_old shape mismatch"):
         blend.blend(o_hat, o_old[:, :4], W, o_new)
+
+
+def test_graph_statistics_carry_the_reference_names():
+    """What `jetfire_get_graph_stats` / `reset_jetfire_graph_stats` call on the extension module
+    (`jetfire_vllm/adapter/decode_path.py:1017-1045`): get_shadow_append_count, get_graph_timing_stats,
+    reset_graph_submit_count, next to the counters that were already there."""
+    from jetfire_amd import ops
+    cpu, _, _, _ = _exts()
+    cpu.reset_graph_submit_count()
+    assert cpu.get_shadow_append_count() == 0 and cpu.get_graph_submit_count() == 0
+    Hkv, n = 2, 40
+    k = torch.randn(n, Hkv, 128).to(torch.bfloat16).cuda()
+    ksh = torch.zeros(Hkv, 64, 128, dtype=torch.bfloat16, pin_memory=True)
+    vsh = torch.zeros_like(ksh).pin_memory()
+    for _ in range(3):
+        ops.shadow_write(k, k, torch.arange(n).cuda(), ksh, vsh)
+    torch.cuda.synchronize()
+    assert cpu.get_shadow_append_count() == 3
+    assert torch.equal(ksh[:, :n].view(torch.int16), k.cpu().transpose(0, 1).contiguous().view(torch.int16))
+    st = cpu.get_graph_timing_stats()
+    for key in ("topk_jobs", "topk_done_avg_us", "topk_done_max_us", "shadow_append_jobs", "join_jobs",
+                "join_wait_avg_us", "join_wait_max_us", "pool_workers", "pool_done_count", "pool_initialized"):
+        assert key in st
+    assert st["shadow_append_jobs"] == 3 and isinstance(st["topk_done_avg_us"], float)
+    cpu.reset_graph_submit_count()
+    assert cpu.get_shadow_append_count() == 0 and cpu.get_graph_timing_stats()["topk_jobs"] == 0
+
+
+def test_handoff_jobs_show_up_in_the_timing_statistics_and_the_doorbell_wakes_the_pool():
+    from jetfire_amd import ops
+    cpu, _, _, _ = _exts()
+    B, Hq, Hkv, S, K = 1, 8, 2, 256, 32
+    c = make_case(5, B, Hq, Hkv, S, 3, 2, 64)
+    d = to_device(c)
+    cpu.graph_pool_warmup_threads(2)
+    cpu.reset_graph_submit_count()
+    h = ops.CpuTopkHandoff(B, Hq, Hkv, K, bf16_tensor(c["K"]), bf16_tensor(c["V"]), SCALE)
+    slots = torch.arange(K, dtype=torch.int64).repeat(B, Hq, 1).cuda()
+    o_new = torch.empty(B, Hq, 128, dtype=torch.bfloat16, device="cuda")
+    cpu.pool_doorbell()                       # head of a step: a kernel, then the poller wakes the workers
+    h.stream_submit(d["q"], slots)
+    h.stream_wait(o_new)
+    torch.cuda.synchronize()
+    h.check_status()
+    st = cpu.get_graph_timing_stats()
+    assert st["topk_jobs"] == 1 and st["topk_done_max_us"] > 0 and st["pool_done_count"] >= 1 and st["pool_workers"] == 2
+    h.close()
+    cpu.pool_wake()                           # the host-side form: no error with or without sleeping workers
+
+
+def test_int4_stage_b_writes_caller_owned_buffers():
+    """`int4_softmax_v_with_pre_corr_wvs2_inplace`, the name graph mode looks up
+    (`jetfire_vllm/adapter/decode_path.py:2872-2919`): same numbers as the allocating form."""
+    from jetfire_amd.kernels.int4_split import load_softmax_v_ext
+    from jetfire_amd.kernels.int8tc_qk_scores import load_int8tc_qk_scores_ext
+    B, Hq, Hkv, S, K = 2, 8, 2, 384, 64
+    c = make_case(31, B, Hq, Hkv, S, 4, 4, 128)
+    d = to_device(c)
+    sa, sb = load_int8tc_qk_scores_ext(), load_softmax_v_ext()
+    scores, idx, _ = sa.int8tc_qk_scores_topk(d["q"], d["kd"], d["ks"], d["bt"], d["lens"], S, Hq, Hkv, 16, SCALE, K)[:3]
+    ref = sb.int4_softmax_v_with_pre_corr_wvs2_scores(scores, d["vd"], d["vs"], d["bt"], d["lens"], idx, S, Hq, Hkv, 16, K)
+    o_hat = torch.full((B, Hq, 128), float("nan"), device="cuda")
+    o_old = torch.full((B, Hq, 128), float("nan"), device="cuda")
+    W = torch.full((B, Hq), float("nan"), device="cuda")
+    weights = torch.empty(B, Hq, S, device="cuda")
+    assert sb.int4_softmax_v_with_pre_corr_wvs2_inplace(scores, d["vd"], d["vs"], d["bt"], d["lens"], idx, weights, o_hat,
+                                                        o_old, W, S, Hq, Hkv, 16, K) is None
+    torch.cuda.synchronize()
+    for a, b in zip(ref, (o_hat, o_old, W)):
+        assert torch.equal(a, b)

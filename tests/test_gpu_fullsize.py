@@ -107,11 +107,11 @@ def test_full_length_splits_of_the_other_schemes(scheme, gs, Hq, Hkv):
         w = workloads.build("other", n_layers=1, paged=True)
     finally:
         del workloads.CONFIGS["other"]
-    _lib.check(lib.jf_debug_split_len(4096))
+    _lib.check(_lib.debug_hook("jf_debug_split_len")(4096))
     try:
         _check_layer_properties(w)
     finally:
-        _lib.check(lib.jf_debug_split_len(0))
+        _lib.check(_lib.debug_hook("jf_debug_split_len")(0))
 
 
 def test_c1_gpu_split_path_agrees_with_the_cpu_torch_path():

@@ -159,12 +159,12 @@ def test_fused_scan_with_forced_split_length(scheme, S, lens, K, split_len):
     kb, vb, gs = {"k3v2": (3, 2, 64), "k4v4": (4, 4, 128), "k3v4": (3, 4, 128), "k4v2": (4, 2, 128)}[scheme]
     c = make_case(11 + S + K, 1, 8, 2, S, kb, vb, gs, lens=lens, extra_blocks=3)
     d = to_device(c)
-    _lib.check(lib.jf_debug_split_len(split_len))
+    _lib.check(_lib.debug_hook("jf_debug_split_len")(split_len))
     try:
         out = run_fused(scheme, c, d, S, K)
         forced = [t.clone() for t in out]
     finally:
-        _lib.check(lib.jf_debug_split_len(0))
+        _lib.check(_lib.debug_hook("jf_debug_split_len")(0))
     check_against_oracle(scheme, c, S, K, forced)
     # the planner's own split length selects the same positions
     again = run_fused(scheme, c, d, S, K)
@@ -206,12 +206,12 @@ def test_fused_scan_ties_go_to_the_lower_position(S, K, split_len):
     c["kd"][:] = c["kd"][:, :1]
     c["ks"][:] = c["ks"][:, :1]
     d = to_device(c)
-    _lib.check(lib.jf_debug_split_len(split_len))
+    _lib.check(_lib.debug_hook("jf_debug_split_len")(split_len))
     try:
         out = run_fused("k3v2", c, d, S, K)
         idx = out[4].cpu().numpy()
     finally:
-        _lib.check(lib.jf_debug_split_len(0))
+        _lib.check(_lib.debug_hook("jf_debug_split_len")(0))
     assert (idx == np.arange(K)[None, None, :]).all()
 
 
@@ -246,13 +246,13 @@ def test_fused_blend_epilogue_equals_the_separate_blend(scheme, B, Hq, Hkv, S, l
     o_new = torch.randn(B, Hq, 128, generator=g, device="cuda").to(torch.bfloat16)
     out = torch.full_like(o_new, 7.0)
     lib = _lib.load()
-    _lib.check(lib.jf_debug_split_len(split_len))
+    _lib.check(_lib.debug_hook("jf_debug_split_len")(split_len))
     try:
         plain = o.fused_attn_topk(scheme, d["q"], d["kd"], d["ks"], d["vd"], d["vs"], d["bt"], d["lens"], S, Hq, Hkv, 16, K, SCALE)
         fused = o.fused_attn_topk(scheme, d["q"], d["kd"], d["ks"], d["vd"], d["vs"], d["bt"], d["lens"], S, Hq, Hkv, 16, K, SCALE,
                                   blend=(o_new, out))
     finally:
-        _lib.check(lib.jf_debug_split_len(0))
+        _lib.check(_lib.debug_hook("jf_debug_split_len")(0))
     for x, y in zip(plain, fused):
         assert torch.equal(x, y)
     ref = o.blend_unnorm(fused[0], fused[2], fused[3], o_new)
@@ -348,7 +348,7 @@ def test_many_rows_take_the_light_merge_with_identical_results(scheme, S, K, spl
     lens = [S - 7 * b for b in range(B)]
     c = make_case(300 + S, B, Hq, Hkv, S, kb, vb, gs, lens=lens)
     d = to_device(c)
-    _lib.check(lib.jf_debug_split_len(split_len))
+    _lib.check(_lib.debug_hook("jf_debug_split_len")(split_len))
     try:
         whole = [t.clone() for t in run_fused(scheme, c, d, S, K)]
         for lo, hi in ((0, 10), (10, 20)):
@@ -358,7 +358,7 @@ def test_many_rows_take_the_light_merge_with_identical_results(scheme, S, K, spl
             for a, b in zip(whole, part):
                 assert torch.equal(a[lo:hi], b)
     finally:
-        _lib.check(lib.jf_debug_split_len(0))
+        _lib.check(_lib.debug_hook("jf_debug_split_len")(0))
     if S <= 1500:
         check_against_oracle(scheme, c, S, K, whole)
 

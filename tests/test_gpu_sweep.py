@@ -40,11 +40,11 @@ def test_fused_scan_random_geometry(seed):
     d = to_device(c)
     lib = _lib.load()
     print(f"case: {scheme} B={B} Hq={Hq} Hkv={Hkv} S={S} lens={lens} K={K} split={split}", flush=True)
-    _lib.check(lib.jf_debug_split_len(split))
+    _lib.check(_lib.debug_hook("jf_debug_split_len")(split))
     try:
         out = [t.clone() for t in run_fused(scheme, c, d, S, K)]
     finally:
-        _lib.check(lib.jf_debug_split_len(0))
+        _lib.check(_lib.debug_hook("jf_debug_split_len")(0))
     check_against_oracle(scheme, c, S, K, out)
 
 
@@ -66,7 +66,7 @@ def test_two_call_form_random_geometry(seed):
     lib = _lib.load()
     print(f"case: {scheme} B={B} Hq={Hq} Hkv={Hkv} S={S} lens={lens} K={K} split={split}", flush=True)
     assert ops.get_split_impl() == "fast"
-    _lib.check(lib.jf_debug_split_len(split))
+    _lib.check(_lib.debug_hook("jf_debug_split_len")(split))
     try:
         o_hat, slots, o_old, W, idx, m, iz, scores = [t.clone() for t in run_fused(scheme, c, d, S, K)]
         args = (d["q"], d["kd"], d["ks"], d["bt"], d["lens"], S, Hq, Hkv, 16, 128 ** -0.5, K)
@@ -81,5 +81,5 @@ def test_two_call_form_random_geometry(seed):
         assert torch.equal(idx2, idx) and torch.equal(slots2, slots)
         o_hat2, o_old2, W2 = stage_b(sc2, d["vd"], d["vs"], d["bt"], d["lens"], idx2, S, Hq, Hkv, 16, K)
     finally:
-        _lib.check(lib.jf_debug_split_len(0))
+        _lib.check(_lib.debug_hook("jf_debug_split_len")(0))
     assert torch.equal(o_hat2, o_hat) and torch.equal(o_old2, o_old) and torch.equal(W2, W)

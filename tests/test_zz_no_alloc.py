@@ -54,10 +54,15 @@ def _compare(scheme, seed, B, Hq, Hkv, S, K, lens=None):
     ws = torch.empty(need, dtype=torch.uint8, device="cuda")
     ref, got = _outputs(B, Hq, K, S, "cuda"), _outputs(B, Hq, K, S, "cuda")
     _lib.check(_call(lib, False, scheme, gs, c, d, S, K, ref, ws))
-    before = torch.cuda.memory_allocated()
+    # a first call resolves the array's address and sizes the kernel's LDS; the call after it must leave both torch's
+    # allocator and the device's free memory (hipMalloc / hipHostMalloc made behind torch's back) where they were
     _lib.check(_call(lib, True, scheme, gs, c, d, S, K, got))
-    assert torch.cuda.memory_allocated() == before
     torch.cuda.synchronize()
+    before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
+    _lib.check(_call(lib, True, scheme, gs, c, d, S, K, got))
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] == free_before, "the static entry point changed the device's free memory"
     for name in ref:
         a, b = ref[name].cpu().numpy(), got[name].cpu().numpy()
         assert np.array_equal(a.view(np.uint8), b.view(np.uint8)), f"{scheme}: {name} differs"
@@ -81,3 +86,13 @@ def test_static_scratch_entry_rejects_shapes_beyond_its_array():
                                        SCALE, K, nul, nul, nul, nul, nul, nul, nul, nul, nul)
     assert rc != 0
     assert b"built-in scratch" in lib.jf_last_error()
+
+
+def test_static_scratch_entry_names_the_entry_point_for_zero_point_schemes():
+    from jetfire_amd import _lib
+    lib = _lib.load()
+    nul = C.c_void_p(0)
+    rc = lib.jf_fused_scan_topk_static(12, 64, nul, nul, nul, nul, nul, nul, nul, 1, 8, 2, 256, 16, 1024, 16,
+                                       SCALE, 32, nul, nul, nul, nul, nul, nul, nul, nul, nul)
+    assert rc != 0
+    assert b"jf_fused_scan_topk_asym" in lib.jf_last_error()
