@@ -281,6 +281,75 @@ def measure_gpu_path(name: str, steps: int, warmup: int, lib):
     return rec
 
 
+def measure_e2e(name: str, steps: int, cpu_threads: int):
+    """Configuration C4 / C5 end to end inside the default run: per layer the fused scan + merge, the publish kernel
+    (slots + q to pinned memory), the CPU correction on the host's worker pool and the device-side wait that fetches
+    o_new and blends, the whole step replayed from ONE HIP graph whose first node is the pool's doorbell.  Wall time
+    per layer, and what the device-side waits themselves measured (their waiting time, 100 MHz clock)."""
+    import torch
+    from jetfire_amd import _lib, ops, workloads
+    w = workloads.build(name, keep_shadow=4)
+    n_layers = len(w.layers)
+    ops.set_cpu_attn_threads(cpu_threads)
+    ctxs = [ops.CpuTopkHandoff(w.B, w.H_q, w.H_kv, w.top_k, ksh, vsh, w.attn_scale) for ksh, vsh in w.shadows]
+    out = torch.empty(w.B, w.H_q, 128, dtype=torch.bfloat16, device="cuda")
+    cap = 4096
+    log = torch.zeros(cap + 1, dtype=torch.int64, device="cuda")
+    _lib.check(_lib.debug_hook("jf_debug_wait_log")(log.data_ptr(), cap))
+
+    def step():
+        ops.pool_doorbell()
+        for li, lay in enumerate(w.layers):
+            o_hat, slots, o_old, W, _ = ops.fused_attn_topk(w.scheme, w.q, lay.k_data, lay.k_scales, lay.v_data, lay.v_scales,
+                                                            w.block_table, w.seq_lens, w.S, w.H_q, w.H_kv, 16, w.top_k,
+                                                            w.attn_scale)
+            h = ctxs[li % len(ctxs)]
+            h.stream_submit(w.q, slots)
+            h.stream_wait_blend(o_hat, o_old, W, out)
+    try:
+        step()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        s = torch.cuda.Stream()
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            step()
+        torch.cuda.current_stream().wait_stream(s)
+        with torch.cuda.graph(graph, stream=s):
+            step()
+        graph.replay()
+        torch.cuda.synchronize()
+        time.sleep(0.02)                      # the pool goes to sleep, as between two decode steps of a served model
+        log.zero_()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+        for h in ctxs:
+            h.check_status()
+        rec_n = int(log[0].item())
+        waits = (log[1:1 + min(rec_n, cap)].cpu().numpy() / 100.0)      # microseconds
+        waits.sort()
+        us_layer = elapsed / steps / n_layers * 1e6
+        return {"workload": f"{name}: B{w.B} Hq{w.H_q} Hkv{w.H_kv} D128 S{w.S} {w.scheme} g{w.group} top_k{w.top_k} x{n_layers} "
+                            "layers, scan + merge + pinned hand-off + CPU correction + device-side wait and blend, one HIP "
+                            "graph per step with the pool's doorbell at its head",
+                "steps": steps, "us_per_layer": round(us_layer, 2), "ms_per_step": round(elapsed / steps * 1e3, 3),
+                "cpu_threads": ops.get_cpu_attn_threads(),
+                "value": round(w.packed_bytes_per_layer / us_layer / 1e3, 2), "unit": "GB/s",
+                "wait_kernel_us": {"launches": rec_n, "median": round(float(waits[len(waits) // 2]), 1) if len(waits) else None,
+                                   "p99": round(float(waits[int(len(waits) * 0.99)]), 1) if len(waits) else None,
+                                   "max": round(float(waits[-1]), 1) if len(waits) else None,
+                                   "clock": "device-side, 100 MHz"}}
+    finally:
+        _lib.check(_lib.debug_hook("jf_debug_wait_log")(None, 0))
+        torch.cuda.synchronize()
+        for h in ctxs:
+            h.close()
+
+
 def profile_counters(scheme: str, workload: str):
     """Counter-derived figures of the scan kernel for this workload, from the committed rocprofv3 summaries (they
     cannot be collected from inside a benchmark process): HBM traffic per launch, MFMA and VALU busy shares."""
@@ -462,6 +531,8 @@ def main() -> int:
                                                  attn_metadata=meta, output=out)
                 assert got is not None, pool.get_stats()["decode_fallbacks"]
             return
+        if ctxs:
+            ops.pool_doorbell() if args.graph else ops.pool_wake()   # the pool spins when the first layer's job arrives
         for li, lay in enumerate(w.layers):
             o_hat, slots, o_old, W, idx = ops.fused_attn_topk(
                 w.scheme, w.q, lay.k_data, lay.k_scales, lay.v_data, lay.v_scales, w.block_table, w.seq_lens,
@@ -561,6 +632,8 @@ def main() -> int:
         w.layers.clear()
         torch.cuda.empty_cache()
         res["k4v4"] = [measure_gpu_path(name, max(3, args.steps // 2), 1, lib) for name in ("c2k4", "c3")]
+        # C4 is defined end to end (hand-off + CPU correction + merge): its figure of the same run
+        res["e2e"] = measure_e2e("c4", min(10, max(3, args.steps // 2)), args.cpu_threads)
     print(json.dumps(res))
     return 0
 

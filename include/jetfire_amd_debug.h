@@ -39,6 +39,12 @@ int jf_debug_split_len(int split_len);
  * alive); 1 restores the default. */
 int jf_debug_pool_stall(int64_t row, int microseconds);
 int jf_debug_pool_wait_stragglers(int on);
+/* Measurement aid: device_buffer (capacity + 1 int64 words of device memory, zeroed by the caller) makes every
+ * device-side wait launched from now on (jf_handoff_stream_wait[_blend], jf_submit_ctx_stream_wait; a graph captured
+ * from now on keeps the pointer) add one to word 0 and store the time it waited, in ticks of the 100 MHz clock, to
+ * word 1 + (n mod capacity).  NULL switches it off for later launches; the buffer must outlive every graph that
+ * holds it. */
+int jf_debug_wait_log(void* device_buffer, int capacity);
 /* Test aid: while on, the dispatcher ignores published flags of the context (a correction that never finishes,
  * without hanging anything: the device-side wait runs into its limit). */
 int jf_handoff_debug_pause(jf_handoff* h, int on);

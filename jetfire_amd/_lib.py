@@ -94,6 +94,7 @@ DEBUG_SIGNATURES = {
     "jf_debug_pool_stall": (I, [L, I]),
     "jf_debug_pool_wait_stragglers": (I, [I]),
     "jf_handoff_debug_pause": (I, [P, I]),
+    "jf_debug_wait_log": (I, [P, I]),
 }
 
 _lib = None

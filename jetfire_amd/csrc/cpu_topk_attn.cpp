@@ -833,7 +833,8 @@ __global__ __launch_bounds__(1024) void handoff_wait_fetch_kernel(const int64_t*
                                                                   const uint4* __restrict__ src, uint4* dst, int n16,
                                                                   const float* __restrict__ o_hat,
                                                                   const float* __restrict__ o_old,
-                                                                  const float* __restrict__ W, uint4* out, int sanitize) {
+                                                                  const float* __restrict__ W, uint4* out, int sanitize,
+                                                                  int64_t* wait_log, int wait_log_cap) {
   // Each lane owns up to U items per pass (item = eight bf16 elements).  What does not depend on the CPU -- the
   // o_hat / o_old rows and W of the first pass -- is loaded before the wait, and the U reads from pinned host
   // memory of a pass are issued together, so that one PCIe round trip covers them.
@@ -869,6 +870,10 @@ __global__ __launch_bounds__(1024) void handoff_wait_fetch_kernel(const int64_t*
     }
     if (!ok && __hip_atomic_load(status, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM) == 0)
       __hip_atomic_store(status, (int64_t)1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    if (wait_log) {  // measurement aid: how long this launch waited, in ticks of the 100 MHz clock
+      const unsigned long long slot = atomicAdd(reinterpret_cast<unsigned long long*>(wait_log), 1ull);
+      wait_log[1 + (int64_t)(slot % (unsigned long long)wait_log_cap)] = (int64_t)(wall_clock64() - t0);
+    }
     ok_sh = ok;
   }
   __syncthreads();
@@ -929,6 +934,9 @@ inline int64_t steady_ns() {
 }
 // Doorbell of the pool: a word in pinned host memory that a one-lane kernel at the head of a decode step (or of its
 // HIP graph) bumps; the poller thread sees the change and wakes the pool's workers ahead of the first layer's job.
+// measurement aid (jf_debug_wait_log): device buffer the device-side waits record their waiting times in
+std::atomic<int64_t*> g_wait_log{nullptr};
+std::atomic<int> g_wait_log_cap{0};
 int64_t* g_doorbell_pin = nullptr;   // [0]: the word the kernel bumps
 int64_t* g_doorbell_dev = nullptr;   // the same word as the device sees it
 int64_t g_doorbell_seen = 0;         // (poller thread only)
@@ -1189,7 +1197,8 @@ extern "C" int jf_handoff_stream_wait(jf_handoff* h, uint16_t* o_new_dev, void* 
   hipLaunchKernelGGL(handoff_wait_fetch_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, h->flag_pin + 8,
                      reinterpret_cast<const int64_t*>(h->counter_dev + 2), h->flag_pin + 16, h->device_wait_ticks,
                      reinterpret_cast<const uint4*>(h->o_pin), reinterpret_cast<uint4*>(o_new_dev), n16,
-                     (const float*)nullptr, (const float*)nullptr, (const float*)nullptr, (uint4*)nullptr, 0);
+                     (const float*)nullptr, (const float*)nullptr, (const float*)nullptr, (uint4*)nullptr, 0,
+                     g_wait_log.load(), g_wait_log_cap.load());
   JF_CHECK_HIP(hipGetLastError());
   return JF_OK;
 }
@@ -1210,7 +1219,7 @@ extern "C" int jf_handoff_stream_wait_blend(jf_handoff* h, const float* o_hat, c
   hipLaunchKernelGGL(handoff_wait_fetch_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, h->flag_pin + 8,
                      reinterpret_cast<const int64_t*>(h->counter_dev + 2), h->flag_pin + 16, h->device_wait_ticks,
                      reinterpret_cast<const uint4*>(h->o_pin), reinterpret_cast<uint4*>(o_new_dev), n16, o_hat,
-                     o_old_unnorm, W, reinterpret_cast<uint4*>(out), h->sanitize.load());
+                     o_old_unnorm, W, reinterpret_cast<uint4*>(out), h->sanitize.load(), g_wait_log.load(), g_wait_log_cap.load());
   JF_CHECK_HIP(hipGetLastError());
   return JF_OK;
 }
@@ -1230,6 +1239,13 @@ extern "C" int jf_handoff_set_device_wait_limit_us(jf_handoff* h, int64_t us) {
 }
 
 #ifdef JF_DEBUG_HOOKS
+extern "C" int jf_debug_wait_log(void* device_buffer, int capacity) {
+  JF_CHECK_ARG(device_buffer == nullptr || capacity > 0, "debug_wait_log: capacity must be positive");
+  g_wait_log_cap.store(device_buffer ? capacity : 0);
+  g_wait_log.store(reinterpret_cast<int64_t*>(device_buffer));
+  return JF_OK;
+}
+
 extern "C" int jf_handoff_debug_pause(jf_handoff* h, int on) {
   JF_CHECK_ARG(h, "handoff_debug_pause: null argument");
   h->paused.store(on ? 1 : 0);
@@ -1406,7 +1422,7 @@ extern "C" int jf_submit_ctx_stream_wait(int64_t ctx, void* stream) {
   hipLaunchKernelGGL(handoff_wait_fetch_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, h->flag_pin + 8,
                      reinterpret_cast<const int64_t*>(h->counter_dev + 2), h->flag_pin + 16, h->device_wait_ticks,
                      (const uint4*)nullptr, (uint4*)nullptr, 0, (const float*)nullptr, (const float*)nullptr,
-                     (const float*)nullptr, (uint4*)nullptr, 0);
+                     (const float*)nullptr, (uint4*)nullptr, 0, g_wait_log.load(), g_wait_log_cap.load());
   JF_CHECK_HIP(hipGetLastError());
   return JF_OK;
 }
