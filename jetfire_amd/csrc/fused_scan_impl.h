@@ -63,7 +63,15 @@ extern std::mutex g_prof_mu;
 extern std::atomic<long long*> g_phase_clock;
 extern std::atomic<int> g_force_split_len;  // test / measurement aid: overrides the planner's split length when positive
 constexpr bool kDebugHooks = true;
+// clock of the phase stamps: the wavefront's own cycle counter, or (JF_STAMP_WALL_CLOCK) the constant 100 MHz counter
+// that every XCD shares, for comparing workgroups on different XCDs (their cycle counters run at different rates)
+#ifdef JF_STAMP_WALL_CLOCK
+#define JF_CLK() ((long long)wall_clock64())
 #else
+#define JF_CLK() clock64()
+#endif
+#else
+#define JF_CLK() 0ll
 constexpr bool kDebugHooks = false;
 #endif
 // Compute units of the current device (the planner balances workgroups over them); 256, the MI355X count, when
@@ -78,7 +86,6 @@ int launch_full_scan_d(int scheme, int G, int NG, const void* params, void* stre
 int launch_full_scan_e(int scheme, int G, int NG, const void* params, void* stream);  // B4V2, B4V3, B4V4
 
 namespace {
-
 
 typedef int v2i __attribute__((ext_vector_type(2)));
 typedef unsigned v2u __attribute__((ext_vector_type(2)));
@@ -208,6 +215,11 @@ struct ScanLds {
   static constexpr int WL = NG * NSET * 64 * 16;  // per (group, set): one 16-byte weight row per token
   static constexpr int KST = 64 * KROW;
   static constexpr int WAVE_STAGE = (VST + WL > KST) ? (VST + WL) : KST;
+  // INT3 / symmetric INT2 keys: the scale word of a token is loaded once (lane = token) and turned into the floats
+  // phase A multiplies by -- the group scales and the rounding coefficients -- in a table behind the staged key rows,
+  // 8 * NG bytes per token, instead of by every one of the four lanes that handle the token's heads
+  static constexpr int SCT = 8 * NG;
+  static constexpr bool SPREP = (K3 || (K2 && !KA)) && (WAVE_STAGE >= KST + 64 * SCT);
   static constexpr int ACC_REGS = 8 + NG;                   // v4i accumulators per set: 8 channel tiles + NG weight sums
   // sum of the wavefronts' accumulators: one int per (set, accumulator register, component, lane), in the staging
   // area (dead after phase B), followed by one kilobyte per wavefront for the exact selection's histogram
@@ -334,7 +346,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   const uint8_t* vsbase = reinterpret_cast<const uint8_t*>(p.v_scales + (size_t)hkv * p.num_slots * NG);
 
   long long* clk = (kDebugHooks && p.phase_clock) ? p.phase_clock + (((size_t)b * p.H_kv + hkv) * p.n_splits + split) * 10 : nullptr;
-  if (clk && tid == 0) clk[0] = clock64();
+  if (clk && tid == 0) clk[0] = JF_CLK();
 
   // The page-table entry and the query elements of this thread do not depend on the sequence length: they
   // are requested first, so their latency runs in parallel with the load of seq_lens[b] instead of after it.
@@ -389,9 +401,10 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   }
   const uint8_t* ksb = reinterpret_cast<const uint8_t*>(p.k_scales + (size_t)hkv * p.num_slots * (KLIMB ? NG : 1));
   const uint8_t* kzb = KA ? reinterpret_cast<const uint8_t*>(p.k_zp + (size_t)hkv * p.num_slots * NG) : nullptr;
+  constexpr bool SPREP = HAS_K && Lds::SPREP;
   struct KBuf {
     v4u r[KLD];
-    uint32_t s[4];
+    uint32_t s[SPREP ? 1 : 4];   // scale words: of the lane's token (SPREP), or of token t16 of each of the four pages
     uint32_t z[KA ? 4 : 1];  // zero-points of the asymmetric keys, packed like the scales
   };
   const int t16 = lane & 15, lg = lane >> 4;
@@ -399,12 +412,18 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     KBuf kbuf;
     constexpr int KNG = KLIMB ? NG : 1;  // key scales per row
     // (the scales first: they are copied out of the buffer one chunk earlier than the rows are, and loads return in order)
+    if constexpr (SPREP) {
+      const int tl = chunk * 64 + lane;
+      const uint32_t slot = (uint32_t)(sbase[tl >> 4] + (tl & 15));
+      if (KNG == 2) kbuf.s[0] = *reinterpret_cast<const uint32_t*>(ksb + (size_t)(slot * 4u));
+      else kbuf.s[0] = (uint32_t) * reinterpret_cast<const uint16_t*>(ksb + (size_t)(slot * 2u));
+    }
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < (SPREP ? 0 : 4); ++j) {
       const int sb = __builtin_amdgcn_readfirstlane(sbase[chunk * 4 + j]);  // first slot of the page (uniform)
       const uint8_t* srow = ksb + (size_t)sb * (KNG * 2) + t16 * (KNG * 2);
-      if (KNG == 2) kbuf.s[j] = *reinterpret_cast<const uint32_t*>(srow);
-      else kbuf.s[j] = *reinterpret_cast<const uint16_t*>(srow);
+      if (KNG == 2) kbuf.s[SPREP ? 0 : j] = *reinterpret_cast<const uint32_t*>(srow);
+      else kbuf.s[SPREP ? 0 : j] = *reinterpret_cast<const uint16_t*>(srow);
       if constexpr (KA) {
         const uint8_t* zrow = kzb + (size_t)sb * (KNG * 2) + t16 * (KNG * 2);
         if (KNG == 2) kbuf.z[j] = *reinterpret_cast<const uint32_t*>(zrow);
@@ -547,7 +566,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   }
   lds_barrier();
   if constexpr (HAS_K) Kb = issue_k(min(wave + NW, nch_cover - 1));
-  if (clk && tid == 0) clk[7] = clock64();
+  if (clk && tid == 0) clk[7] = JF_CLK();
 
   // ---- V stream, set-up (same scheme as the key stream)
   uint8_t* vst = stage + wave * Lds::WAVE_STAGE;  // [64][VROW], this wavefront only
@@ -604,19 +623,24 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   // positions produced.  A chunk past the end (n_local <= 0) is not worked through at all.
   auto clone_last_row = [&](int n_local, uint32_t (&Sx)[4], uint32_t (&Zx)[4]) {
     const int last = n_local - 1, jl = last >> 4;
-    uint32_t sl = Sx[0], zl = Zx[0];
+    if constexpr (SPREP) {  // one scale word per lane (= token): Sx[0]
+      const uint32_t sl = (uint32_t)__builtin_amdgcn_readlane((int)Sx[0], last);
+      Sx[0] = (lane >= n_local) ? sl : Sx[0];
+    } else {
+      uint32_t sl = Sx[0], zl = Zx[0];
 #pragma unroll
-    for (int j = 1; j < 4; ++j) {
-      sl = (jl == j) ? Sx[j] : sl;
-      zl = (jl == j) ? Zx[j] : zl;
-    }
-    sl = (uint32_t)__builtin_amdgcn_readlane((int)sl, last & 15);
-    zl = (uint32_t)__builtin_amdgcn_readlane((int)zl, last & 15);
+      for (int j = 1; j < 4; ++j) {
+        sl = (jl == j) ? Sx[j] : sl;
+        zl = (jl == j) ? Zx[j] : zl;
+      }
+      sl = (uint32_t)__builtin_amdgcn_readlane((int)sl, last & 15);
+      zl = (uint32_t)__builtin_amdgcn_readlane((int)zl, last & 15);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const bool past = 16 * j + (lane & 15) >= n_local;
-      Sx[j] = past ? sl : Sx[j];
-      Zx[j] = past ? zl : Zx[j];
+      for (int j = 0; j < 4; ++j) {
+        const bool past = 16 * j + (lane & 15) >= n_local;
+        Sx[j] = past ? sl : Sx[j];
+        Zx[j] = past ? zl : Zx[j];
+      }
     }
     constexpr int RDW = KP / 4;  // dwords per staged row
     const uint8_t* src = kst + last * KROW;
@@ -732,12 +756,27 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
           Pj[j][1] = x[1];
           Pj[j][2] = 0u;
         }
-        const uint32_t sw = Sx[j];
-        sgj[j][0] = bf16_to_f32((uint16_t)(sw & 0xffffu));
-        egj[j][0] = K3 ? eps_sh[0][sw & 0x7fu] : 0.f;  // (INT4: three coefficients, read where they are used)
-        if (NG == 2) {
-          sgj[j][NG - 1] = bf16_to_f32((uint16_t)(sw >> 16));
-          egj[j][NG - 1] = K3 ? eps_sh[0][(sw >> 16) & 0x7fu] : 0.f;
+        if constexpr (SPREP) {  // the token's entry of the table the wavefront has just written
+          const uint8_t* sp = kst + Lds::KST + (16 * j + t16) * Lds::SCT;
+          if (NG == 2) {
+            const v4f x = *reinterpret_cast<const v4f*>(sp);
+            sgj[j][0] = x[0];
+            sgj[j][NG - 1] = x[1];
+            egj[j][0] = x[2];
+            egj[j][NG - 1] = x[3];
+          } else {
+            const v2f x = *reinterpret_cast<const v2f*>(sp);
+            sgj[j][0] = x[0];
+            egj[j][0] = x[1];
+          }
+        } else {
+          const uint32_t sw = Sx[j];
+          sgj[j][0] = bf16_to_f32((uint16_t)(sw & 0xffffu));
+          egj[j][0] = K3 ? eps_sh[0][sw & 0x7fu] : 0.f;  // (INT4: three coefficients, read where they are used)
+          if (NG == 2) {
+            sgj[j][NG - 1] = bf16_to_f32((uint16_t)(sw >> 16));
+            egj[j][NG - 1] = K3 ? eps_sh[0][(sw >> 16) & 0x7fu] : 0.f;
+          }
         }
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -1008,16 +1047,30 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
         KBuf& cur = (it & 1) ? Kb : Ka;
         stash_k(cur);
         wave_lds_fence();
-        uint32_t Sc[4], Zc[4];
+        uint32_t Sc[4] = {0u, 0u, 0u, 0u}, Zc[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          Sc[j] = reg_copy(cur.s[j]);
+          if (!SPREP || j == 0) Sc[j] = reg_copy(cur.s[SPREP ? 0 : j]);
           Zc[j] = KA ? reg_copy(cur.z[KA ? j : 0]) : 0u;
         }
         if constexpr (it + 2 < MAXIT) cur = issue_k(min(chunk + 2 * NW, nch_cover - 1));
         const int n_local = n - chunk * 64;  // (uniform)
         if (n_local > 0) {
           if (n_local < 64) clone_last_row(n_local, Sc, Zc);
+          if constexpr (SPREP) {  // lane = token: scales and rounding coefficients of the chunk -> table
+            const uint32_t sw = Sc[0];
+            uint8_t* sp = kst + Lds::KST + lane * Lds::SCT;
+            const float s0f = bf16_to_f32((uint16_t)(sw & 0xffffu));
+            const float e0f = K3 ? eps_sh[0][sw & 0x7fu] : 0.f;
+            if (NG == 2) {
+              const float s1f = bf16_to_f32((uint16_t)(sw >> 16));
+              const float e1f = K3 ? eps_sh[0][(sw >> 16) & 0x7fu] : 0.f;
+              *reinterpret_cast<v4f*>(sp) = (v4f){s0f, s1f, e0f, e1f};
+            } else {
+              *reinterpret_cast<v2f*>(sp) = (v2f){s0f, e0f};
+            }
+            wave_lds_fence();
+          }
           body(chunk, Sc, Zc);
         }
         if (n_local < 64) mask_tail(chunk, n_local);
@@ -1140,8 +1193,8 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     }
   }
 
-  if (clk && tid == 0) clk[9] = clock64();  // wavefront 0 finished its chunks
-  if (clk && lane == 0) atomicMax(&tmax_sh, (unsigned long long)clock64());
+  if (clk && tid == 0) clk[9] = JF_CLK();  // wavefront 0 finished its chunks
+  if (clk && lane == 0) atomicMax(&tmax_sh, (unsigned long long)JF_CLK());
   __builtin_amdgcn_s_setprio(0);
   // split extrema per head; fixed-point exponent of the V scales; selection buckets
   if constexpr (HAS_V) {
@@ -1159,7 +1212,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     }
   }
   lds_barrier();  // phase A complete: the query constants are dead, their space becomes the histograms
-  if (clk && tid == 0) { clk[8] = clock64(); clk[5] = (long long)tmax_sh; }
+  if (clk && tid == 0) { clk[8] = JF_CLK(); clk[5] = (long long)tmax_sh; }
   if (p.scores)  // validation output
     for (int i = tid; i < GA * n_cover; i += NT) {
       const int h = i / n_cover, t = i - h * n_cover;
@@ -1194,7 +1247,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     e_sh[g] = 22 - e;                                 // v * 2^E in [2^21, 2^22)
   }
   lds_barrier();
-  if (clk && tid == 0) clk[1] = clock64();
+  if (clk && tid == 0) clk[1] = JF_CLK();
 
   // ------------------------------------------------------------------ phase B: P.V on v_mfma_i32_16x16x64_i8
   // p = exp(s - m_split) is known exactly because phase A is complete, so w = p * v_scale is converted to
@@ -1428,7 +1481,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     if (lane == 0) lsum_sh[wave][h] = ls;  // summed in wavefront order below: run-to-run deterministic
   }
   lds_barrier();
-  if (clk && tid == 0) clk[2] = clock64();
+  if (clk && tid == 0) clk[2] = JF_CLK();
 
   // ---- sum of the integer accumulators over the wavefronts: LDS integer atomics into one array in the staging
   // area (dead now: every wavefront has passed the barrier above), zeroed here, filled while the cut is searched,
@@ -1555,7 +1608,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     }
   }
   lds_barrier();
-  if (clk && tid == 0) clk[6] = clock64();
+  if (clk && tid == 0) clk[6] = JF_CLK();
   for (int hs = wave; HAS_TOPK && hs < G * SEG; hs += NW) {
     const int h = hs / SEG, seg = hs % SEG;
     if (h >= GA) continue;
@@ -1688,7 +1741,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
       for (int i = count + lane; i < Kcap; i += 64) ck[i] = 0u;
     }
   }
-  if (clk && tid == 0) clk[3] = clock64();
+  if (clk && tid == 0) clk[3] = JF_CLK();
 
   // (no barrier: the accumulator sums were complete before the emission started, and nothing below reads what the
   // emission wrote)
@@ -1704,7 +1757,7 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     p.part_m[part_base + (size_t)tid * p.n_splits] = m_sh[tid];
     p.part_l[part_base + (size_t)tid * p.n_splits] = lfin;
   }
-  if (clk && tid == 0) clk[4] = clock64();
+  if (clk && tid == 0) clk[4] = JF_CLK();
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -1800,7 +1853,7 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   const int nblk_lds = min(p.max_blocks, MG_BT);
 
   long long* mclk = (kDebugHooks && p.phase_clock && !PARTIAL) ? p.phase_clock + (size_t)p.B * p.H_kv * p.n_splits * 10 + bh * 8 : nullptr;
-  if (mclk && tid == 0) mclk[0] = clock64();
+  if (mclk && tid == 0) mclk[0] = JF_CLK();
 
   // ---- everything that does not depend on anything else is requested first, in the order of its use.  Every load
   // is unconditional, on a clamped index, and its mask is applied further down: under a condition the compiler waits
@@ -1920,7 +1973,7 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   kmax = wave_max_u(kmax);
   if (lane == 0) { wred_u[wave] = kmin; wred_k[wave] = kmax; }
   lds_barrier();
-  if (mclk && tid == 0) mclk[6] = clock64();
+  if (mclk && tid == 0) mclk[6] = JF_CLK();
   if (tid >= NS) pl = 0.f;
   if (MODE == FS_FULL && !PARTIAL && p.blend_out && tid < D) blend_new = bf16_to_f32(blend_raw);
 #pragma unroll
@@ -1967,7 +2020,7 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
     }
   }
   lds_barrier();
-  if (mclk && tid == 0) mclk[7] = clock64();
+  if (mclk && tid == 0) mclk[7] = JF_CLK();
   // ---- interval 3: 1/l, the partial sums of o_hat; first half of the bucket scan
   float inv_z = 0.f;
   if (!PARTIAL) {
@@ -2035,7 +2088,7 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
       if (MODE != FS_STAGE_B || p.o_hat) p.o_hat[bh * D + tid] = blend_hat;
     }
   }
-  if (mclk && tid == 0) mclk[1] = clock64();
+  if (mclk && tid == 0) mclk[1] = JF_CLK();
 
   uint32_t tau = 0;
   int quota = 0;
@@ -2096,7 +2149,7 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
       quota = K - ((tau == 0xffffffffu) ? 0 : count_ge(tau + 1u));
     }
   }
-  if (mclk && tid == 0) mclk[2] = clock64();
+  if (mclk && tid == 0) mclk[2] = JF_CLK();
 
   // ---- ordered compaction.  Register candidates: every thread counts its winners and ties per group, a
   // wavefront scan plus the wavefront totals in LDS give the thread's first place, and the thread places its
@@ -2199,7 +2252,7 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
     }
     lds_barrier();
   }
-  if (mclk && tid == 0) mclk[3] = clock64();
+  if (mclk && tid == 0) mclk[3] = JF_CLK();
   if (PARTIAL) {  // the winners become one candidate list of the final merge
     const size_t lo = (bh * p.mg_parts + part) * (size_t)K;
     for (int r = tid; r < K; r += MG_THREADS) {
@@ -2231,7 +2284,7 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   }
   if constexpr (MODE == FS_STAGE_A) return;  // Stage A alone ends with the winners and the statistics
   lds_barrier();
-  if (mclk && tid == 0) mclk[4] = clock64();
+  if (mclk && tid == 0) mclk[4] = JF_CLK();
 
   // ---- pre-correction over the winners.  One winner row per DW lanes: lane (w_in, dwi) holds dword dwi of
   // the winner's packed V row (CPD codes) and accumulates its CPD channels; winners are visited in a fixed
@@ -2338,7 +2391,7 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
     // the blend of jetfire_vllm/csrc/blend.cu:202-226 for callers that hold o_new already
     if (MODE == FS_FULL && p.blend_out) p.blend_out[bh * D + tid] = f32_to_bf16(__builtin_fmaf(wt, blend_new, blend_hat) - o);
   }
-  if (mclk && tid == 0) mclk[5] = clock64();
+  if (mclk && tid == 0) mclk[5] = JF_CLK();
 }
 
 constexpr size_t LDS_BUDGET_2WG = 80 * 1024 - 512;    // two workgroups per CU (160 KB LDS)
