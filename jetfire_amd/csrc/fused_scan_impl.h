@@ -319,7 +319,6 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   __shared__ uint32_t vmax_sh[NW][2];
   __shared__ float m_sh[G], bin_a_sh[G], bin_b_sh[G], lsum_sh[NW][G];
   __shared__ int e_sh[2];
-  __shared__ int cut_sh[G], segoff_sh[G][SEG + 1], exact_sh[G];
   // rounding coefficients 256 * (bf16(c s) - c s) / s for s = 1 + m/128 (INT3: c = 3; INT4, bf16 model: c = 3, 5, 7).
   // Static, so that a look-up's address is the index plus a constant the instruction carries.
   __shared__ float eps_sh[KB4 ? 3 : 1][128];
@@ -465,7 +464,6 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
       else vsw[i] = (uint32_t) * reinterpret_cast<const uint16_t*>(vsbase + (size_t)(vs_slot[i] * 2u));
     }
   }
-
   if constexpr (!HAS_K) {
     // the scores are an input: no query constants
   } else if constexpr (KLIMB) {
@@ -1252,11 +1250,11 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   // ------------------------------------------------------------------ phase B: P.V on v_mfma_i32_16x16x64_i8
   // p = exp(s - m_split) is known exactly because phase A is complete, so w = p * v_scale is converted to
   // 22-bit fixed point once (fma with 2^23); its three bytes, balanced around zero, are rows (limb, head) of
-  // the A operand.  Lane = token builds one 16-byte row per scale group (limb-major, then a constant 1 that
-  // becomes the all-ones row), and ds_read_b64_tr_b8 turns 8 token rows into the per-row byte runs the MFMA
+  // the A operand.  Lane = token stores the four heads' converted words as one 16-byte row per scale group (head-major;
+  // the word's top byte is the constant 75 and becomes a constant row), and ds_read_b64_tr_b8 turns 8 token rows into the per-row byte runs the MFMA
   // wants.  V codes are staged packed in wavefront-private LDS and transposed by ds_read_b64_tr_b4 (16
   // tokens of one channel pair per lane), then spread.  sum_t w_t*(code - off) = sum_t w_t*code - off*sum_t w_t:
-  // the ones row gives sum_t code (needed because the limbs are balanced), a ones B tile gives sum_t w_t.
+  // the constant row gives 75 * sum_t code (needed because the limbs are balanced), a ones B tile gives sum_t w_t.
   // Every accumulation is an exact integer.  The same pass drops every score into one of 256 linear buckets
   // per (head, half of the split) for the candidate selection.
   int E[NG];
@@ -1333,16 +1331,13 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     for (int g = 0; g < NG; ++g)
 #pragma unroll
       for (int set = 0; set < NSET; ++set) {
-        const uint32_t h0 = bits[set * 4 + 0][g], h1 = bits[set * 4 + 1][g], h2 = bits[set * 4 + 2][g], h3 = bits[set * 4 + 3][g];
-        const uint32_t T01 = __builtin_amdgcn_perm(h1, h0, 0x05010400u);  // h0.b0 h1.b0 h0.b1 h1.b1
-        const uint32_t U01 = __builtin_amdgcn_perm(h1, h0, 0x0c0c0602u);  // h0.b2 h1.b2 0 0
-        const uint32_t T23 = __builtin_amdgcn_perm(h3, h2, 0x05010400u);
-        const uint32_t U23 = __builtin_amdgcn_perm(h3, h2, 0x0c0c0602u);
-        v3i row;  // (the fourth dword of the row, the constant 1 of the ones row, was written before the stream)
-        row[0] = (int)(__builtin_amdgcn_perm(T23, T01, 0x05040100u) ^ 0x80808080u);  // limb 0 of heads 0..3, balanced
-        row[1] = (int)(__builtin_amdgcn_perm(T23, T01, 0x07060302u) ^ 0x80808080u);  // limb 1
-        row[2] = (int)(U01 | (U23 << 16));                                           // limb 2 (< 128)
-        *reinterpret_cast<v3i*>(wl + ((g * NSET + set) * 64 + lane) * 16) = row;
+        // one 16-byte row per token: byte 4h + l = limb l of head h (limbs 0 and 1 balanced around zero, limb 2 < 128),
+        // byte 4h + 3 = 75, the exponent byte of the fixed-point conversion, which serves as the constant row that
+        // yields the code sums
+        v4i row;
+#pragma unroll
+        for (int hh = 0; hh < 4; ++hh) row[hh] = (int)(bits[set * 4 + hh][g] ^ 0x00008080u);
+        *reinterpret_cast<v4i*>(wl + ((g * NSET + set) * 64 + lane) * 16) = row;
       }
     wave_lds_fence();
     v4i A[NG][NSET];
@@ -1445,13 +1440,6 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
       }
     }
   };
-  if constexpr (HAS_V) {
-    // fourth dword of every weight row: row 12 of the A operand is all ones, rows 13..15 are zero.  Constant, so it
-    // is stored once (this wavefront's staging area held key rows until now) and the stream stores 12 bytes per row.
-#pragma unroll
-    for (int i = 0; i < NG * NSET; ++i) *reinterpret_cast<int*>(wl + (i * 64 + lane) * 16 + 12) = 1;
-    wave_lds_fence();
-  }
   if constexpr (MODE == FS_FULL) {  // (wavefronts that left the key stream before its last two steps)
     if (!va_requested) Va = issue_v(min(wave, nch - 1));
     if (!vb_requested) Vb = issue_v(min(wave + NW, nch - 1));
@@ -1480,24 +1468,34 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     const float ls = wave_sum(lsum[h]);
     if (lane == 0) lsum_sh[wave][h] = ls;  // summed in wavefront order below: run-to-run deterministic
   }
+  if constexpr (HAS_V) {
+    // The accumulator sums below live at the start of the staging area: each wavefront clears what lies in its own
+    // part (it is done with it), so the array is zero behind the barrier.
+    const int z0 = wave * Lds::WAVE_STAGE;
+    const int z1 = min(z0 + Lds::WAVE_STAGE, Lds::XACC);
+    for (int o = z0 + lane * 16; o < z1; o += 1024) *reinterpret_cast<v4i*>(stage + o) = (v4i){0, 0, 0, 0};
+  }
   lds_barrier();
   if (clk && tid == 0) clk[2] = JF_CLK();
 
-  // ---- sum of the integer accumulators over the wavefronts: LDS integer atomics into one array in the staging
-  // area (dead now: every wavefront has passed the barrier above), zeroed here, filled while the cut is searched,
-  // read by `combine` after the candidates have been emitted.  Integer sums: exact and independent of the order.
-  // D layout: row r of a tile sits in lane 16*(r>>2) + column, register r&3; rows are (limb, head), row 12 is the
-  // ones row.  Element (set, register r, component c, lane l) lives at xacc[((set*AR + r)*4 + c)*64 + l].
+  // ---- sum of the integer accumulators over the wavefronts: LDS integer atomics into one array at the start of
+  // the staging area (cleared before the barrier above), read by `combine` after the candidates have been emitted.
+  // Integer sums: exact and independent of the order.  The atomics return nothing, so a wavefront issues them a few
+  // at a time along the comparisons of its first emission blocks: they drain in the LDS pipe while the vector ALU
+  // works.
+  // D layout: row r of a tile sits in lane 16*(r>>2) + column, register r&3; row 4*head + l is limb l for l < 3 and
+  // the constant row (75 * sum of codes) for l = 3.  Item j = (register i = j >> 2 of set i / AR, component j & 3)
+  // lives at xacc[j * 64 + lane].
   int* xacc = reinterpret_cast<int*>(stage);
-  if constexpr (HAS_V)
-    for (int i = tid; i < Lds::XACC / 4; i += NT) xacc[i] = 0;
-  auto add_acc = [&](int set) {
+  constexpr int ACC_TOTAL = NSET * AR, ACC_HALF = (ACC_TOTAL + 1) / 2;
+  bool acc_issued = false;  // (uniform) this wavefront's sums are on their way
+  auto add_acc_range = [&](const int first, const int last) {  // (constants once the caller's loop is unrolled)
 #pragma unroll
-    for (int r = 0; r < AR; ++r) {
+    for (int j = 0; j < ACC_TOTAL * 4; ++j) {
+      if (j < first || j >= last) continue;
+      const int i = j >> 2, c = j & 3, set = i / AR, r = i % AR;
       const v4i v = (r < NTILE) ? acc[set][r < NTILE ? r : 0] : accw[set][r >= NTILE ? r - NTILE : 0];
-      int* dst = xacc + ((set * AR + r) * 4) * 64 + lane;
-#pragma unroll
-      for (int c = 0; c < 4; ++c) atomicAdd(dst + c * 64, v[c]);
+      atomicAdd(xacc + j * 64 + lane, v[c]);
     }
   };
   auto combine = [&](int set) {
@@ -1516,16 +1514,16 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
         d = tile * 16 + 2 * (col >> 1) + (1 - (col & 1));
       }
       const int g = (NG == 1) ? 0 : (d / (D / NG));
-      const int* ta = xacc + ((set * AR + tile) * 4) * 64;          // limb l of head hh: component hh, lane 16*l + col
-      const int* wa = xacc + ((set * AR + NTILE + g) * 4) * 64;    // weight sums: any column of the all-ones tile
-      int i0 = ta[hh * 64 + col], i1 = ta[hh * 64 + 16 + col], i2 = ta[hh * 64 + 32 + col], cs = ta[48 + col];
+      const int* ta = xacc + ((set * AR + tile) * 4) * 64 + 16 * hh + col;   // row 4*hh + l of the tile: component l, lane 16*hh + col
+      const int* wa = xacc + ((set * AR + NTILE + g) * 4) * 64 + 16 * hh;    // weight sums: any column of the all-ones tile
+      int i0 = ta[0], i1 = ta[64], i2 = ta[128], cs = ta[192] / 75;          // (row 4*hh + 3 holds 75 * sum of the codes)
       if (V2 && !(tile & 1)) {  // even INT2 tiles hold four times their sums (exact multiples)
         i0 >>= 2;
         i1 >>= 2;
         i2 >>= 2;
         cs >>= 2;
       }
-      const int w0 = wa[hh * 64], w1 = wa[hh * 64 + 16], w2 = wa[hh * 64 + 32];   // |sum| < 2^24: no overflow
+      const int w0 = wa[0], w1 = wa[64], w2 = wa[128];   // |sum| < 2^24: no overflow
       const long long wsum = (long long)w2 * 65536ll + (long long)w1 * 256ll + (long long)w0 + 32896ll * 64ll * (long long)nch;
       const long long tot = (long long)i2 * 65536ll + (long long)i1 * 256ll + (long long)i0 + 32896ll * (long long)cs - (long long)VOFF * wsum;
       p.part_o[(part_base + (size_t)h * p.n_splits) * D + d] = (float)ldexp((double)tot, -E[g]);
@@ -1536,19 +1534,21 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   // The merge kernel needs a superset of the split's top Kt = min(top_k, n) scores per head that fits the
   // candidate buffer (Kcap entries), in ascending position.  From the histograms: the smallest bucket index
   // `cut` with count(bucket <= cut) >= Kt.  If that count fits, every position whose bucket is <= cut is
-  // emitted, one wavefront per (head, half of the split), the second half starting where the first one's count
-  // ends.  Otherwise (heavily tied scores) one wavefront falls back to an exact radix select over the keys.
+  // emitted, one wavefront per (head, segment of the split), each segment starting where the counts of the segments
+  // before it end.  Otherwise (heavily tied scores) one wavefront falls back to an exact radix select over the keys.
   const int Kcap = p.Kc;
   const int Kt = min(p.top_k, n);
-  if constexpr (HAS_V) {  // the accumulator sums go first: they run in the LDS pipe while the cut is searched
-    lds_barrier();        // (the array is zero everywhere)
-#pragma unroll
-    for (int set = 0; set < NSET; ++set) add_acc(set);
-  }
-  for (int h = wave; HAS_TOPK && h < GA; h += NW) {
+  for (int hs = wave; HAS_TOPK && hs < G * SEG; hs += NW) {
+    const int h = hs / SEG, seg = hs % SEG;
+    if (h >= GA) continue;
+    // Every wavefront of a head searches the cut itself (same histograms, same result): no exchange, no barrier
+    // between the search and the emission.
+    const float ba = uniform_f(bin_a_sh[h]);
+    float bb = uniform_f(bin_b_sh[h]);
+    asm volatile("" : "+v"(bb));  // (kept in a vector register: the multiply-add takes one scalar operand only)
     const int* h0 = hist + h * (SEG * 256) / (Lds::H16 ? 2 : 1);
     // lane l owns buckets 4l .. 4l+3 (ascending bucket = descending score) of every segment's histogram
-    int cs[SEG][4], c[4], mine = 0;
+    int cs[SEG][4], c[4], mine;
 #pragma unroll
     for (int sg = 0; sg < SEG; ++sg) {
       if (Lds::H16) {
@@ -1558,106 +1558,143 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
         cs[sg][2] = (int)(w1 & 0xffffu);
         cs[sg][3] = (int)(w1 >> 16);
       } else {
+        const v4i x = *reinterpret_cast<const v4i*>(h0 + sg * 256 + 4 * lane);
 #pragma unroll
-        for (int u = 0; u < 4; ++u) cs[sg][u] = h0[sg * 256 + 4 * lane + u];
+        for (int u = 0; u < 4; ++u) cs[sg][u] = x[u];
       }
     }
+    // c[u]: the bucket's count over all segments; cum[u]: over the segments before this wavefront's
+    int cum[4] = {0, 0, 0, 0};
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      c[u] = 0;
-#pragma unroll
-      for (int sg = 0; sg < SEG; ++sg) c[u] += cs[sg][u];
-      mine += c[u];
-    }
-    const int incl = wave_incl_scan_i(mine);
-    int run = incl - mine;
-    int cut = -1, tot = 0;
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int before = run;
-      run += c[u];
-      if (cut < 0 && before < Kt && run >= Kt) {
-        cut = 4 * lane + u;
-        tot = run;
-      }
-    }
-    const unsigned long long who = __ballot(cut >= 0);
-    bool ok = false;
-    if (who != 0ull) {
-      const int src = __ffsll((long long)who) - 1;
-      cut = __builtin_amdgcn_readlane(cut, src);
-      tot = __builtin_amdgcn_readlane(tot, src);
-      ok = tot <= Kcap;
-    }
-    if (!ok) cut = 255;
-    // entries every segment emits: its histogram summed over the buckets <= cut
-    int off = 0;
+    for (int u = 0; u < 4; ++u) c[u] = 0;
 #pragma unroll
     for (int sg = 0; sg < SEG; ++sg) {
-      int part = 0;
+      if (sg == seg) {  // (uniform)
 #pragma unroll
-      for (int u = 0; u < 4; ++u) part += (4 * lane + u <= cut) ? cs[sg][u] : 0;
-      part = wave_sum_i(part);
-      if (lane == 0) segoff_sh[h][sg] = off;
-      off += part;
+        for (int u = 0; u < 4; ++u) cum[u] = c[u];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) c[u] += cs[sg][u];
     }
-    if (lane == 0) {
-      segoff_sh[h][SEG] = off;
-      cut_sh[h] = cut;
-      exact_sh[h] = ok ? 0 : 1;
+    mine = (c[0] + c[1]) + (c[2] + c[3]);
+    const int cumt = (cum[0] + cum[1]) + (cum[2] + cum[3]);
+    // one scan for both: the totals in the low half, the earlier segments' in the high half (each sum <= 4096)
+    const int packed = mine | (cumt << 16);
+    const int incl = wave_incl_scan_i(packed);
+    // the first lane whose inclusive total reaches Kt holds the cut bucket; the rest is scalar arithmetic on that
+    // lane's four counts
+    const unsigned long long who = __ballot((incl & 0xffff) >= Kt);
+    bool ok = false;
+    int cut = 255, tot = 0, before_me = 0;
+    if (who != 0ull) {
+      const int src = __ffsll((long long)who) - 1;
+      const int ex = __builtin_amdgcn_readlane(incl - packed, src);  // exclusive sums at that lane
+      int run = ex & 0xffff;
+      before_me = ex >> 16;
+      bool found = false;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int cu = __builtin_amdgcn_readlane(c[u], src), mu = __builtin_amdgcn_readlane(cum[u], src);
+        if (!found) {
+          run += cu;
+          before_me += mu;
+          if (run >= Kt) {
+            found = true;
+            cut = 4 * src + u;
+            tot = run;
+          }
+        }
+      }
+      ok = tot <= Kcap;
     }
-  }
-  lds_barrier();
-  if (clk && tid == 0) clk[6] = JF_CLK();
-  for (int hs = wave; HAS_TOPK && hs < G * SEG; hs += NW) {
-    const int h = hs / SEG, seg = hs % SEG;
-    if (h >= GA) continue;
+    if (clk && tid == 0) clk[6] = JF_CLK();
     const float* srow = sc + h * L;
     uint32_t* ck = p.cand_key + (part_base + (size_t)h * p.n_splits) * Kcap;
     int32_t* ci = p.cand_idx + (part_base + (size_t)h * p.n_splits) * Kcap;
-    if (!exact_sh[h]) {
+    if (ok) {
       // bucket(s) <= cut  <=>  not (s * ba + bb >= cut + 1): the bucket is the floor of that value clamped to
       // [0, 255]; with cut = 255 every position qualifies
-      const int cut = cut_sh[h];
       const float thr = uniform_f((cut >= 255) ? INFINITY : (float)(cut + 1));
-      const float ba = uniform_f(bin_a_sh[h]);
-      float bb = uniform_f(bin_b_sh[h]);
-      asm volatile("" : "+v"(bb));  // (kept in a vector register: the multiply-add takes one scalar operand only)
       const int tb = seg * (L / SEG);
       const int te = min(n, (seg + 1) * (L / SEG));
       // the emitted total is at most Kcap by construction of the cut
-      int count = __builtin_amdgcn_readfirstlane(segoff_sh[h][seg]);
+      int count = __builtin_amdgcn_readfirstlane(before_me);
       // unused slots hold key 0 (no score maps to it); the planned total is known, so the head's wavefronts
       // share the padding and its stores leave before the emission's
-      const int etot = min(Kcap, __builtin_amdgcn_readfirstlane(segoff_sh[h][SEG]));
+      const int etot = min(Kcap, tot);
       for (int i = etot + seg * 64 + lane; i < Kcap; i += SEG * 64) ck[i] = 0u;
-      uint8_t* ckb = reinterpret_cast<uint8_t*>(ck);
-      uint8_t* cib = reinterpret_cast<uint8_t*>(ci);
-      // eight groups of 64 positions at a time; whole batches run without the per-position end test
-      auto emit_batch = [&](int t0, auto checked_tag) {
-        constexpr bool CHECKED = decltype(checked_tag)::value;
-        float kk[8];
+      // Blocks of 1024 positions, 16 consecutive ones per lane: the lane's candidates are consecutive in the output,
+      // so a block costs one comparison per position, one wavefront scan of the lanes' counts, and a loop over the
+      // few set bits of every lane.  The lane reads its four 16-byte quads starting at quad (lane >> 2) & 3 (the
+      // four lanes that share a bank group then read different banks) and rotates its bit mask back afterwards.
+      const int rot4 = ((lane >> 2) & 3) * 4;
+      auto emit_block = [&](int t0, auto acc_tag) {
+        constexpr int ACCSEL = decltype(acc_tag)::value;  // accumulator sums issued along the comparisons: -1 none, 0 / 1 a half, 2 all
+        constexpr int A_LO = (ACCSEL == 1) ? ACC_HALF * 4 : 0;
+        constexpr int A_HI = (ACCSEL < 0) ? 0 : ((ACCSEL == 0) ? ACC_HALF * 4 : ACC_TOTAL * 4);
+        constexpr int PER = (A_HI - A_LO + 15) / 16;      // a few behind every comparison: the LDS queue never fills
+        const int lt = t0 + 16 * lane;                    // first position of this lane
+        const float* lp = srow + lt;
+        v4f x[4];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          const int t = t0 + 64 * u + lane;
-          kk[u] = (!CHECKED || t < te) ? srow[t] : 0.f;
-        }
+        for (int q = 0; q < 4; ++q) x[q] = *reinterpret_cast<const v4f*>(lp + ((4 * q + rot4) & 15));
+        uint32_t ge = 0u;  // bit 4q + e set: element e of quad register q falls behind the cut (not emitted)
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          const int t = t0 + 64 * u + lane;
-          const bool above = (!CHECKED || t < te) && !(__builtin_fmaf(kk[u], ba, bb) >= thr);
-          const unsigned long long ma = __builtin_amdgcn_ballot_w64(above);
-          const uint32_t pos = (uint32_t)count + __builtin_amdgcn_mbcnt_hi((uint32_t)(ma >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)ma, 0u));
-          if (above && pos < (uint32_t)Kcap) {  // the bound only matters for non-finite scores
-            *reinterpret_cast<uint32_t*>(ckb + (size_t)(pos * 4u)) = score_key(kk[u]);
-            *reinterpret_cast<int32_t*>(cib + (size_t)(pos * 4u)) = s0 + t;
+        for (int bi = 15; bi >= 0; --bi) {
+          // ge = 2 * ge + [value >= thr]: the comparison's lane mask is the carry of one add
+          const unsigned long long c = __builtin_amdgcn_ballot_w64(__builtin_fmaf(x[bi >> 2][bi & 3], ba, bb) >= thr);
+          // (the two wait states between a vector instruction's scalar result and a vector instruction that reads it
+          // are the compiler's job everywhere else; it does not look inside an asm statement)
+          asm("s_nop 1\n\tv_addc_co_u32_e64 %0, vcc, %1, %1, %2" : "=v"(ge) : "v"(ge), "s"(c) : "vcc");
+          if constexpr (HAS_V && PER > 0) {
+            const int lo = A_LO + (15 - bi) * PER;
+            if (lo < A_HI) {
+              add_acc_range(lo, (lo + PER < A_HI) ? lo + PER : A_HI);
+              __builtin_amdgcn_sched_barrier(0);
+            }
           }
-          count += __popcll(ma);
+        }
+        // register bit b is position (b + rot4) mod 16 of the lane's run
+        uint32_t m2 = ~ge & 0xffffu;
+        m2 |= m2 << 16;
+        uint32_t mask = (m2 >> (16 - rot4)) & 0xffffu;
+        const int nvalid = max(0, min(16, te - lt));
+        mask &= (1u << nvalid) - 1u;
+        const int mine = __popc(mask);
+        const int incl = wave_incl_scan_i(mine);
+        uint32_t o = (uint32_t)(count + incl - mine);
+        count += __builtin_amdgcn_readlane(incl, 63);
+        // (the score of the next set bit is requested before the current one is stored: one LDS latency per lane run,
+        // not one per candidate)
+        int i = (mask != 0u) ? __ffs((int)mask) - 1 : 0;
+        float sco = lp[i];
+        while (mask != 0u) {
+          mask &= mask - 1u;
+          const int i_next = (mask != 0u) ? __ffs((int)mask) - 1 : 0;
+          const float s_next = lp[i_next];
+          if (o < (uint32_t)Kcap) {  // the bound only matters for non-finite scores
+            ck[o] = score_key(sco);
+            ci[o] = s0 + lt + i;
+          }
+          ++o;
+          i = i_next;
+          sco = s_next;
         }
       };
+      constexpr std::integral_constant<int, -1> plain{};
       int t0 = tb;
-      for (; t0 + 512 <= te; t0 += 512) emit_batch(t0, std::integral_constant<bool, false>{});
-      if (t0 < te) emit_batch(t0, std::integral_constant<bool, true>{});
+      if (HAS_V && !acc_issued && te > tb) {  // the first block (or the first two) of this wavefront carry the sums
+        if (te - tb > 1024) {
+          emit_block(tb, std::integral_constant<int, 0>{});
+          emit_block(tb + 1024, std::integral_constant<int, 1>{});
+          t0 = tb + 2048;
+        } else {
+          emit_block(tb, std::integral_constant<int, 2>{});
+          t0 = tb + 1024;
+        }
+        acc_issued = true;
+      }
+      for (; t0 < te; t0 += 1024) emit_block(t0, plain);
       if (seg == SEG - 1) {
         if (lane == 0) p.cand_cnt[part_base + (size_t)h * p.n_splits] = min(Kcap, count);
         for (int i = count + lane; i < etot; i += 64) ck[i] = 0u;  // (only if a segment emitted less than planned)
@@ -1743,8 +1780,10 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   }
   if (clk && tid == 0) clk[3] = JF_CLK();
 
-  // (no barrier: the accumulator sums were complete before the emission started, and nothing below reads what the
-  // emission wrote)
+  if constexpr (HAS_V) {  // whatever the emission did not carry (no batch of this wavefront, a short split, the exact selection)
+    if (!acc_issued) add_acc_range(0, ACC_TOTAL * 4);
+    lds_barrier();
+  }
   float lfin = 0.f;
   if (tid < G) {
 #pragma unroll
