@@ -470,38 +470,19 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     // Query rows -> 23-bit fixed point per (head, scale group), three balanced int8 limbs, written in the
     // byte order of the MFMA A operand.  One element per thread; group statistics by wavefront reductions.
     K3Prep<NSET>* prep = reinterpret_cast<K3Prep<NSET>*>(aux);
-    if ((K3 || KB4) && tid < 128) {
-      const float sm = 1.0f + (float)tid * (1.0f / 128.0f);
+    // (the rounding table is built by two wavefronts that have no query rows to prepare, where there are such)
+    constexpr int EPS_T0 = (QN / 64 <= NW - 2) ? NT - 128 : 0;
+    if ((K3 || KB4) && tid >= EPS_T0 && tid < EPS_T0 + 128) {
+      const int m = tid - EPS_T0;
+      const float sm = 1.0f + (float)m * (1.0f / 128.0f);
 #pragma unroll
       for (int i = 0; i < (KB4 ? 3 : 1); ++i) {
         const float t = (float)(3 + 2 * i) * sm;  // 3 s, 5 s, 7 s: exact in fp32
-        eps_sh[i][tid] = 256.0f * ((bf16_to_f32(f32_to_bf16(t)) - t) / sm);
+        eps_sh[i][m] = 256.0f * ((bf16_to_f32(f32_to_bf16(t)) - t) / sm);
       }
     }
-#pragma unroll
-    for (int it = 0; it < QPT; ++it) {
-      const int c = it * NW + wave;  // 64-channel half row of this wavefront
-      if (c * 64 < QN) {             // uniform per wavefront
-        const float am = wave_max(fabsf(q_elem(it)));
-        if (lane == 0) prep->amax_w[c] = am;
-      }
-    }
-    lds_barrier();
-#pragma unroll
-    for (int it = 0; it < QPT; ++it) {
-      const int i = it * NT + tid, h = i >> 7, d = i & 127;
-      const float x = q_elem(it);
-      const int c = it * NW + wave;
-      if (c * 64 >= QN) continue;
-      const float amax = (NG == 2) ? prep->amax_w[c] : fmaxf(prep->amax_w[c & ~1], prep->amax_w[c | 1]);
-      int e = 0;
-      if (amax > 0.f && isfinite(amax)) (void)frexpf(amax, &e);  // amax = f * 2^e, f in [0.5, 1)
-      const int qf = (int)rintf(ldexpf(x, 22 - e));
-      const int s = wave_sum_i(qf);
-      if (lane == 0) {
-        prep->sum_w[c] = s;
-        prep->exp_w[c] = e;
-      }
+    // stores the three limbs of element (h, d) in the byte order of the MFMA A operand
+    auto put_limbs = [&](int h, int d, int qf) {
       const int l0 = (int)(int8_t)(qf & 255);
       const int r1 = (qf - l0) >> 8;
       const int l1 = (int)(int8_t)(r1 & 255);
@@ -520,14 +501,60 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
       prep->aop[set][4 * hh + 1][kb][mi][by] = (int8_t)l1;
       prep->aop[set][4 * hh + 2][kb][mi][by] = (int8_t)l2;
       prep->aop[set][4 * hh + 3][kb][mi][by] = 0;
-    }
-    lds_barrier();
-    if (tid < NSET * 4 * NG) {
-      const int h = tid / NG, g = tid % NG;
-      const int sum = (NG == 2) ? prep->sum_w[2 * h + g] : prep->sum_w[2 * h] + prep->sum_w[2 * h + 1];
-      const int e = prep->exp_w[2 * h + ((NG == 2) ? g : 0)];
-      prep->sq4[h][g] = (KB4 ? 8 : (K3 ? 4 : 2)) * sum;  // the codes are used unsigned: offset 8 (INT4), 4 (INT3) or 2 (INT2)
-      prep->qsc[h][g] = ldexpf(p.attn_scale, e - 22);
+    };
+    constexpr int CODE_OFF4 = KB4 ? 8 : (K3 ? 4 : 2);  // the codes are used unsigned: offset 8 (INT4), 4 (INT3) or 2 (INT2)
+    if constexpr (NG == 2) {
+      // a wavefront's 64 elements are one scale group of one head: its statistics never leave the wavefront
+#pragma unroll
+      for (int it = 0; it < QPT; ++it) {
+        const int c = it * NW + wave;  // 64-channel half row of this wavefront
+        if (c * 64 >= QN) continue;    // uniform per wavefront
+        const int i = it * NT + tid, h = i >> 7, d = i & 127;
+        const float x = q_elem(it);
+        const float amax = wave_max(fabsf(x));
+        int e = 0;
+        if (amax > 0.f && isfinite(amax)) (void)frexpf(amax, &e);  // amax = f * 2^e, f in [0.5, 1)
+        const int qf = (int)rintf(ldexpf(x, 22 - e));
+        const int sum = wave_sum_i(qf);
+        put_limbs(h, d, qf);
+        if (lane == 0) {
+          prep->sq4[h][c & 1] = CODE_OFF4 * sum;
+          prep->qsc[h][c & 1] = ldexpf(p.attn_scale, e - 22);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int it = 0; it < QPT; ++it) {
+        const int c = it * NW + wave;  // 64-channel half row of this wavefront
+        if (c * 64 < QN) {             // uniform per wavefront
+          const float am = wave_max(fabsf(q_elem(it)));
+          if (lane == 0) prep->amax_w[c] = am;
+        }
+      }
+      lds_barrier();
+#pragma unroll
+      for (int it = 0; it < QPT; ++it) {
+        const int i = it * NT + tid, h = i >> 7, d = i & 127;
+        const float x = q_elem(it);
+        const int c = it * NW + wave;
+        if (c * 64 >= QN) continue;
+        const float amax = fmaxf(prep->amax_w[c & ~1], prep->amax_w[c | 1]);
+        int e = 0;
+        if (amax > 0.f && isfinite(amax)) (void)frexpf(amax, &e);  // amax = f * 2^e, f in [0.5, 1)
+        const int qf = (int)rintf(ldexpf(x, 22 - e));
+        const int s = wave_sum_i(qf);
+        if (lane == 0) {
+          prep->sum_w[c] = s;
+          prep->exp_w[c] = e;
+        }
+        put_limbs(h, d, qf);
+      }
+      lds_barrier();
+      if (tid < NSET * 4) {
+        const int h = tid;
+        prep->sq4[h][0] = CODE_OFF4 * (prep->sum_w[2 * h] + prep->sum_w[2 * h + 1]);
+        prep->qsc[h][0] = ldexpf(p.attn_scale, prep->exp_w[2 * h] - 22);
+      }
     }
   } else {
     // int8 quantisation of the query rows per 32 channels (int8tc_qk_scores.cu:250-290), one element per thread;
