@@ -1826,6 +1826,38 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
   if (clk && tid == 0) clk[4] = JF_CLK();
 }
 
+// Reductions over one value per wavefront (at most sixteen, in LDS): lane w of the first 16-lane row takes
+// wavefront w's value, the row reduces on the DPP network and the result is read from lane 15 -- a handful of
+// instructions instead of a loop over the sixteen entries in every thread.  Integer and min/max only: the result
+// does not depend on the order.
+template <int NWV>
+__device__ inline float waves_max_f(const float* arr, int lane) {
+  float v = (lane < NWV) ? arr[lane] : -INFINITY;
+  JF_DPP_ROW_REDUCE(v, op_fmax, float, -INFINITY);
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 15));
+}
+template <int NWV>
+__device__ inline uint32_t waves_max_u(const uint32_t* arr, int lane) {
+  uint32_t v = (lane < NWV) ? arr[lane] : 0u;
+  JF_DPP_ROW_REDUCE(v, op_umax, uint32_t, 0u);
+  return (uint32_t)__builtin_amdgcn_readlane((int)v, 15);
+}
+template <int NWV>
+__device__ inline uint32_t waves_min_u(const uint32_t* arr, int lane) {
+  uint32_t v = (lane < NWV) ? arr[lane] : 0xffffffffu;
+  JF_DPP_ROW_REDUCE(v, op_umin, uint32_t, 0xffffffffu);
+  return (uint32_t)__builtin_amdgcn_readlane((int)v, 15);
+}
+// sum of the entries before wavefront `wave` (uniform) and of all entries
+template <int NWV>
+__device__ inline void waves_prefix_i(const int* arr, int lane, int wave, int* before, int* all) {
+  const int own = (lane < NWV) ? arr[lane] : 0;
+  int v = own;
+  JF_DPP_ROW_REDUCE(v, op_iadd, int, 0);  // inclusive scan inside the row
+  *before = __builtin_amdgcn_readlane(v - own, wave);
+  *all = __builtin_amdgcn_readlane(v, 15);
+}
+
 // ---------------------------------------------------------------------------------------------------
 constexpr int MG_MAX_SPLITS = 256;
 constexpr int MG_BINS = 1024;      // linear score buckets of the threshold search
@@ -1857,7 +1889,6 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   static_assert(!(PARTIAL && MODE == FS_STAGE_B), "Stage B alone selects nothing");
   constexpr int MG_WAVES = MG_THREADS / 64;
   constexpr int VP = D * VBITS / 8;
-  constexpr int VOFF = 1 << (VBITS - 1);
   // lanes per winner row and codes per lane: a dword of the row each (INT2, INT4), or (INT3, planar) two bytes of
   // each of the three planes = 16 codes
   constexpr int DW = (VBITS == 3) ? 8 : VP / 4;
@@ -2014,9 +2045,8 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
     lds_barrier();
     if (lane == 0) wred_i[wave] = c;
     lds_barrier();
-    int t = 0;
-#pragma unroll
-    for (int w = 0; w < MG_WAVES; ++w) t += wred_i[w];
+    int before, t;
+    waves_prefix_i<MG_WAVES>(wred_i, lane, 0, &before, &t);
     return t;
   };
 
@@ -2056,8 +2086,7 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   // ---- interval 2: M, the coefficients, per-wavefront sums of l; the candidates drop into MG_BINS linear buckets
   float M = -INFINITY;
   if (!PARTIAL) {
-#pragma unroll
-    for (int w = 0; w < MG_WAVES; ++w) M = fmaxf(M, wred_f[w]);
+    M = waves_max_f<MG_WAVES>(wred_f, lane);
     if (!isfinite(M)) M = 0.f;
     const float coef = (pm == -INFINITY) ? 0.f : __expf(pm - M);
     if (tid < NS) coef_sh[tid] = coef;
@@ -2066,8 +2095,8 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   }
   int total = 0;
   for (int s2 = 0; s2 < NL; ++s2) total += cnt_sh[s2];
-#pragma unroll
-  for (int w = 0; w < MG_WAVES; ++w) { kmin = min(kmin, wred_u[w]); kmax = max(kmax, wred_k[w]); }
+  kmin = waves_min_u<MG_WAVES>(wred_u, lane);
+  kmax = waves_max_u<MG_WAVES>(wred_k, lane);
   const float hi = key_to_score(kmax), lo = key_to_score(kmin);
   const float range = hi - lo;
   const float iw = (range > 0.f && isfinite(range)) ? ((float)MG_BINS - 0.01f) / range : 0.f;
@@ -2160,8 +2189,9 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
   int quota = 0;
   if (!take_all) {
     {
-      int run = incl - mine;
-      for (int w = 0; w < wave; ++w) run += wred_j[w];
+      int run, all_waves;
+      waves_prefix_i<MG_WAVES>(wred_j, lane, wave, &run, &all_waves);
+      run += incl - mine;
 #pragma unroll
       for (int u = 0; u < BPT; ++u) {
         if (run < K && K <= run + cb[u]) { cut_sh = BPT * tid + u; above_sh = run; }
@@ -2243,13 +2273,9 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
     uint32_t run = 0u;  // packed totals of the groups before g (each half stays below 2^16: at most 32768 candidates)
 #pragma unroll
     for (int g = 0; g < NGRP; ++g) {
-      uint32_t before = 0u, all = 0u;
-#pragma unroll
-      for (int w = 0; w < MG_WAVES; ++w) {
-        const uint32_t t = cnt_a[g * MG_WAVES + w];
-        before += (w < wave) ? t : 0u;
-        all += t;
-      }
+      int before_i, all_i;  // (packed pairs: each half stays below 2^16, so the halves never carry into each other)
+      waves_prefix_i<MG_WAVES>(reinterpret_cast<const int*>(cnt_a) + g * MG_WAVES, lane, wave, &before_i, &all_i);
+      const uint32_t before = (uint32_t)before_i, all = (uint32_t)all_i;
       if (4 * g < rreg) {
         const uint32_t start = run + before + (uint32_t)(scan_g[g] - cnt_g[g]);
         int pa = (int)(start & 0xffffu), pt = (int)(start >> 16);
@@ -2390,16 +2416,22 @@ __global__ __launch_bounds__(MG_THREADS) void fused_merge_kernel(FusedParams p) 
 #pragma unroll
     for (int u = 0; u < UNR; ++u) {
       const float ws = wv[u] * bf16_to_f32(sbits[u]);  // zero for padding rows
-      // byte `byte` of the dword holds its codes MSB first; channel of code c in the dword = dwi*CPD + c
+      // byte `byte` of the dword holds its codes MSB first; channel of code c in the dword = dwi*CPD + c.
+      // code - VOFF is the code with its top bit flipped, read as a two's complement field: one signed bit-field
+      // extract per code after one exclusive-or per word.
+      constexpr uint32_t FLIP = (VBITS == 3) ? 0x00924924u : ((VBITS == 2) ? 0xaaaaaaaau : 0x88888888u);
+      const uint32_t xa = word[u] ^ FLIP, xb = word_b[u] ^ FLIP;
 #pragma unroll
       for (int c = 0; c < CPD; ++c) {
-        int code;
+        int sh;
         if constexpr (VBITS == 3) {
-          code = (int)((((c < 8) ? word[u] : word_b[u]) >> (21 - 3 * (c & 7))) & 7u) - VOFF;
+          sh = 21 - 3 * (c & 7);
         } else {
           const int byte = c / (8 / VBITS), inb = c % (8 / VBITS);
-          code = (int)((word[u] >> (8 * byte + (8 - VBITS * (inb + 1)))) & ((1u << VBITS) - 1u)) - VOFF;
+          sh = 8 * byte + (8 - VBITS * (inb + 1));
         }
+        const uint32_t x = (VBITS == 3 && c >= 8) ? xb : xa;
+        const int code = (int)(x << (32 - VBITS - sh)) >> (32 - VBITS);
         acc[c] = __builtin_fmaf(ws, (float)code, acc[c]);
       }
       if (dwi == 0) accw += wv[u];
