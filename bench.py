@@ -350,22 +350,39 @@ def measure_e2e(name: str, steps: int, cpu_threads: int):
             h.close()
 
 
+def lib_version() -> str:
+    """jf_version() of the loaded library: it carries a digest of the sources, headers and flags it was built from."""
+    from jetfire_amd import _lib
+    return _lib.load().jf_version().decode()
+
+
 def profile_counters(scheme: str, workload: str):
     """Counter-derived figures of the scan kernel for this workload, from the committed rocprofv3 summaries (they
-    cannot be collected from inside a benchmark process): HBM traffic per launch, MFMA and VALU busy shares."""
+    cannot be collected from inside a benchmark process): HBM traffic per launch, MFMA and VALU busy shares.  A summary
+    names the library build it was taken with; figures of another build than the loaded one are not reported
+    (`traffic` stays null and `*_stale` says which build the summary belongs to)."""
     out = {"traffic": None}
+    have = lib_version()
     tpath = os.path.join(ROOT, "profiles", f"fused_scan_{scheme}_{workload}_traffic.json")
     cpath = os.path.join(ROOT, "profiles", f"decode_kernels_{workload}_sq_counters.json")
     try:
-        out["traffic"] = json.load(open(tpath)).get("traffic_bytes_per_launch")
-        out["traffic_source"] = os.path.relpath(tpath, ROOT)
+        t = json.load(open(tpath))
+        if t.get("lib_version") == have:
+            out["traffic"] = t.get("traffic_bytes_per_launch")
+            out["traffic_source"] = os.path.relpath(tpath, ROOT)
+        else:
+            out["traffic_stale"] = f"{os.path.relpath(tpath, ROOT)} was taken with {t.get('lib_version', 'an unnamed build')}"
     except Exception:
         pass
     try:
-        c = json.load(open(cpath))["fused_scan_kernel"]
-        out["mfma_busy_pct"] = c.get("mfma_busy_pct")
-        out["valu_issue_pct"] = c.get("valu_issue_pct")
-        out["counters_source"] = os.path.relpath(cpath, ROOT)
+        cj = json.load(open(cpath))
+        if cj.get("lib_version") == have:
+            c = cj["fused_scan_kernel"]
+            out["mfma_busy_pct"] = c.get("mfma_busy_pct")
+            out["valu_issue_pct"] = c.get("valu_issue_pct")
+            out["counters_source"] = os.path.relpath(cpath, ROOT)
+        else:
+            out["counters_stale"] = f"{os.path.relpath(cpath, ROOT)} was taken with {cj.get('lib_version', 'an unnamed build')}"
     except Exception:
         pass
     return out
@@ -606,7 +623,7 @@ def main() -> int:
         "ms_per_step": round(ms_per_step, 4), "us_per_layer": round(ms_per_step * 1e3 / n_layers, 2),
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "u8 codes; int8/bf16 MFMA, fp32 softmax", "data": "synthetic",
+        "dtype": "u8 codes; int8/bf16 MFMA, fp32 softmax", "data": "synthetic", "lib_version": lib_version(),
         "config": {"workload": f"{args.workload}: B{w.B} Hq{w.H_q} Hkv{w.H_kv} D128 S{w.S} {w.scheme} g{w.group} "
                                f"top_k{w.top_k} x{n_layers} layers, {'paged (random)' if args.paged else 'identity'} block table",
                    "packed_bytes_per_layer": bytes_layer, "launch": "hip-graph" if graph is not None else "eager",

@@ -17,15 +17,17 @@
 //                       reference's fp32 rescale order (bit-equal to the split-form kernel).
 //            scores[G][L] -> LDS (fp32), running max / min per head.
 //   phase B  P.V on the same MFMA.  p = exp(s - m_split) is known exactly because phase A is complete, so
-//            w = p * v_scale is converted to 22-bit fixed point once (fma with 2^23), its three bytes are the
-//            A-operand rows (limb, head), and the int32 accumulators live for the whole split: every product
-//            is exact.  V codes are transposed by ds_read_b64_tr_b4, weight rows by ds_read_b64_tr_b8.
+//            w = p * v_scale is converted to 22-bit fixed point once (fma with 2^23), the four bytes of the
+//            converted word are the A-operand rows (head, limb 0..2 and the constant exponent byte), and the
+//            int32 accumulators live for the whole split: every product is exact.  V codes are transposed by
+//            ds_read_b64_tr_b4, weight rows by ds_read_b64_tr_b8.
 //            The same pass drops every score into one of 256 linear buckets per (head, segment).
-//   phase C  from the bucket histograms: the smallest bucket range that holds the split's top min(K, n) scores
-//            and fits the candidate buffer; its positions are emitted as (key, position) in ascending
-//            position, one wavefront per (head, segment).  Heavily tied scores fall back to a radix select.
-//   sum of the wavefronts' integer accumulators with LDS integer atomics (while the cut is searched), exact
-//   int64 recombination -> partial o.
+//   phase C  one wavefront per (head, segment): from the bucket histograms the smallest bucket range that holds
+//            the split's top min(K, n) scores and fits the candidate buffer (every wavefront of a head finds it
+//            itself); its positions are emitted as (key, position) in ascending position, sixteen consecutive
+//            scores per lane and block.  Heavily tied scores fall back to a radix select.
+//   sum of the wavefronts' integer accumulators with LDS integer atomics (issued along the emission's
+//   comparisons), exact int64 recombination -> partial o.
 // Launch 2, fused_merge_kernel, grid (B, H_q): selects the global top-k among the candidates (ties to
 // the lower position, ascending output), merges the split partials
 //   M = max m_i, l = sum l_i e^{m_i-M}, o_hat = sum o_i e^{m_i-M} / l
