@@ -460,3 +460,47 @@ def test_pool_wake_needs_no_gpu():
     ops.pool_wake()
     assert ops.get_cpu_attn_threads() == 2
     ops.set_cpu_attn_threads(0)
+
+
+def test_bench_reports_counter_figures_only_for_the_loaded_build(monkeypatch, tmp_path):
+    """bench.py takes `traffic` and the busy shares from the committed rocprofv3 summaries; a summary names the
+    library build it was taken with, and one of another build is not reported."""
+    import json
+    import bench
+    from jetfire_amd import _lib
+
+    have = _lib.load().jf_version().decode()
+    assert bench.lib_version() == have and "build" in have
+    prof = tmp_path / "profiles"
+    prof.mkdir()
+    monkeypatch.setattr(bench, "ROOT", str(tmp_path))
+
+    def write(version):
+        (prof / "fused_scan_k3v2_c2_traffic.json").write_text(json.dumps(
+            {"traffic_bytes_per_launch": 123, "lib_version": version}))
+        (prof / "decode_kernels_c2_sq_counters.json").write_text(json.dumps(
+            {"fused_scan_kernel": {"mfma_busy_pct": 1.0, "valu_issue_pct": 2.0}, "lib_version": version}))
+
+    write(have)
+    out = bench.profile_counters("k3v2", "c2")
+    assert out["traffic"] == 123 and out["mfma_busy_pct"] == 1.0 and "traffic_stale" not in out
+    write("jetfire_amd 0.3 (gfx950) build 000000000000")
+    out = bench.profile_counters("k3v2", "c2")
+    assert out["traffic"] is None and "mfma_busy_pct" not in out
+    assert "000000000000" in out["traffic_stale"] and "000000000000" in out["counters_stale"]
+    # no summary at all: null, nothing claimed
+    assert bench.profile_counters("k3v2", "nowhere") == {"traffic": None}
+
+
+def test_committed_counter_summaries_belong_to_the_sources_in_the_tree():
+    """The summaries under profiles/ name a build digest; it must be the digest of the sources, headers and flags the
+    library is built from here, so that the default bench line can report them."""
+    import glob
+    import json
+    from jetfire_amd import build
+
+    want = build.build_id(["-DJF_DEBUG_HOOKS"])
+    files = sorted(glob.glob(os.path.join(ROOT, "profiles", "*.json")))
+    assert files
+    for f in files:
+        assert f"build {want}" in json.load(open(f)).get("lib_version", ""), f
