@@ -5,14 +5,14 @@ INT3/INT2 and INT4/INT4 schemes, without any dependence on vLLM: the `impl`, `la
 arguments are read through the same attributes the reference reads."""
 from .cache_store import JetFireInt4CacheStore, JetFireLayerView
 from .config import JetFireConfig, get_jetfire_config, set_jetfire_config
-from .decode_path import (check_decode_handoffs, reset_jetfire_decode_runtime_state, try_jetfire_decode,
-                          warmup_graph_decode_submit_contexts)
+from .decode_path import (check_decode_handoffs, jetfire_get_profile, reset_jetfire_decode_runtime_state,
+                          try_jetfire_decode, warmup_graph_decode_submit_contexts)
 from .kv_pool import (JetFireKVPoolConfig, JetFireKVPoolManager, JetFireLayerConfig, JetFireLayerLayout,
                       get_global_kv_pool_manager, reset_global_kv_pool_manager)
 
 __all__ = [
     "JetFireInt4CacheStore", "JetFireLayerView", "JetFireConfig", "get_jetfire_config", "set_jetfire_config",
-    "try_jetfire_decode", "warmup_graph_decode_submit_contexts", "check_decode_handoffs",
+    "try_jetfire_decode", "warmup_graph_decode_submit_contexts", "check_decode_handoffs", "jetfire_get_profile",
     "reset_jetfire_decode_runtime_state", "JetFireKVPoolConfig", "JetFireKVPoolManager", "JetFireLayerConfig", "JetFireLayerLayout",
     "get_global_kv_pool_manager", "reset_global_kv_pool_manager",
 ]

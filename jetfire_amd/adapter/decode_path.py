@@ -11,14 +11,19 @@ wait pair, nothing in the entry synchronises with the device, and the whole laye
 graph and replayed; `warmup_graph_decode_submit_contexts` creates, before capture, whatever a capture may
 not allocate.  A miss while a graph is being captured raises instead of baking the caller's fall-back into
 the graph (`:698-706`).  With `JETFIRE_RELEASE_GRAPH_POLICY=1` the kernels of a step are the ones the release
-policy names (`release_policy.py`).  The reference's trace hooks and debug correction modes are not reproduced."""
+policy names (`release_policy.py`).  Every stage runs inside a named profiler range (`_timer`, the reference's
+`decode_path.py:60-85`: on ROCm `torch.cuda.nvtx` emits roctx ranges, which `rocprofv3 --marker-trace` shows on the
+timeline); `JETFIRE_PROFILE_DECODE=1` additionally synchronises around each stage and accumulates its wall time for
+`jetfire_get_profile()`.  The reference's step-trace files and debug correction modes are not reproduced."""
 from __future__ import annotations
 
 import bisect
+import contextlib
 import math
 import os
 import re
 import struct
+import time
 import weakref
 
 import torch
@@ -37,6 +42,39 @@ _HEAD_MAP_CACHE: dict = {}
 _STORES_WITH_HANDOFFS: "weakref.WeakSet" = weakref.WeakSet()   # stores that carry hand-off contexts (`store._jf_handoffs`)
 _O_NEW: dict = {}
 _SEQ_LENS_CACHE: dict = {}
+_PROFILE_ACCUM: dict = {}
+
+
+@contextlib.contextmanager
+def _timer(name: str):
+    """Named profiler range around one stage of the decode entry (`decode_path.py:60-85`; the stage names are the
+    reference's where the stage exists there).  The range is always emitted -- pushing one costs next to nothing when
+    no profiler listens -- except while a graph is being captured, where it would mark the capture, not the replays.
+    With JETFIRE_PROFILE_DECODE=1 (never in graph mode: it synchronises) the stage's wall time is accumulated."""
+    capturing = _graph_capture_active()
+    if not capturing:
+        torch.cuda.nvtx.range_push(name)
+    try:
+        if capturing or os.environ.get("JETFIRE_PROFILE_DECODE", "0") != "1":
+            yield
+            return
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        try:
+            yield
+        finally:
+            torch.cuda.synchronize()
+            _PROFILE_ACCUM.setdefault(name, []).append((time.perf_counter() - t0) * 1e3)
+    finally:
+        if not capturing:
+            torch.cuda.nvtx.range_pop()
+
+
+def jetfire_get_profile() -> dict:
+    """Milliseconds per stage accumulated since the last call (`decode_path.py:82-85`)."""
+    out = {k: list(v) for k, v in _PROFILE_ACCUM.items()}
+    _PROFILE_ACCUM.clear()
+    return out
 
 
 def _select_top_k(config_top_k: int, seq_len: int, supported: tuple) -> int | None:
@@ -303,7 +341,8 @@ def _split_stages(store, q, bt, sl, max_S: int, H_q: int, H_kv: int, top_k: int,
 
 def try_jetfire_decode(*, impl, layer, query, attn_metadata, output, key=None, value=None):
     """Production decode entry: `output` on success, None if a precondition fails."""
-    return _decode_batched(impl=impl, layer=layer, query=query, attn_metadata=attn_metadata, output=output)
+    with _timer("D_total"):
+        return _decode_batched(impl=impl, layer=layer, query=query, attn_metadata=attn_metadata, output=output)
 
 
 def _decode_batched(*, impl, layer, query, attn_metadata, output):
@@ -383,38 +422,46 @@ def _decode_batched(*, impl, layer, query, attn_metadata, output):
             max_graph_batch=cfg_max_B if cfg_max_B > 0 else n_seqs,
             require_ready=release_policy.release_require_ready())
 
-    q_batch = query[:n_seqs].contiguous().view(n_seqs, H_q, D).to(torch.bfloat16)
-    bt_batch = attn_metadata.block_table[:n_seqs].to(torch.int64).contiguous()
-    seq_lens_batch = attn_metadata.seq_lens.to(device=query.device, dtype=torch.int32).contiguous()
+    with _timer("V2_00_prep"):
+        q_batch = query[:n_seqs].contiguous().view(n_seqs, H_q, D).to(torch.bfloat16)
+        bt_batch = attn_metadata.block_table[:n_seqs].to(torch.int64).contiguous()
+        seq_lens_batch = attn_metadata.seq_lens.to(device=query.device, dtype=torch.int32).contiguous()
 
-    if fused:
-        o_hat, topk_slots, o_old, W, _ = ops.fused_attn_topk(
-            scheme, q_batch, store.k_data, store.k_scales, store.v_data, store.v_scales, bt_batch, seq_lens_batch,
-            max_S, H_q, H_kv, store.block_size, top_k, scale, k_zp=store.k_zp if store.k_asymmetric else None)
-    else:
-        o_hat, topk_slots, o_old, W = _split_stages(store, q_batch, bt_batch, seq_lens_batch, max_S, H_q, H_kv, top_k, scale,
-                                                    plan=plan)
+    with _timer("V2_01_attn"):          # Stage A + Stage B of the reference, one pass here where the scheme allows
+        if fused:
+            o_hat, topk_slots, o_old, W, _ = ops.fused_attn_topk(
+                scheme, q_batch, store.k_data, store.k_scales, store.v_data, store.v_scales, bt_batch, seq_lens_batch,
+                max_S, H_q, H_kv, store.block_size, top_k, scale, k_zp=store.k_zp if store.k_asymmetric else None)
+        else:
+            o_hat, topk_slots, o_old, W = _split_stages(store, q_batch, bt_batch, seq_lens_batch, max_S, H_q, H_kv, top_k,
+                                                        scale, plan=plan)
     handoff = _handoff_for(store, n_seqs, H_q, H_kv, top_k, scale, stream_mode=graph_mode, layer_name=layer_name)
     o_new = _o_new_for(n_seqs, H_q, D, query.device)
     out_view = output[:n_seqs].view(n_seqs, H_q, D)
     direct = out_view.dtype == torch.bfloat16 and out_view.is_contiguous()
     if graph_mode:          # kernels only: nothing here waits for the CPU
-        handoff.stream_submit(q_batch, topk_slots)
+        with _timer("V2_02c_tpe_submit"):
+            handoff.stream_submit(q_batch, topk_slots)
         if direct:          # the device-side wait blends as the correction arrives
-            handoff.stream_wait_blend(o_hat, o_old, W, out_view)
+            with _timer("V2_04_05_fused"):
+                handoff.stream_wait_blend(o_hat, o_old, W, out_view)
             pool.record_decode_hit()
             return output
-        handoff.stream_wait(o_new)
+        with _timer("V2_04_join"):
+            handoff.stream_wait(o_new)
     else:
-        handoff.submit(q_batch, topk_slots)
-        handoff.wait(o_new)
-    if direct:
-        ops.blend_unnorm_into(o_hat, o_old, W, o_new, out_view)
-    else:
-        tmp = torch.empty(n_seqs, H_q, D, dtype=torch.bfloat16, device=query.device)
-        ops.blend_unnorm_into(o_hat, o_old, W, o_new, tmp)
-        out_view.copy_(tmp.to(out_view.dtype))
-    if graph_mode and _sanitize_output_enabled():   # (decode_path.py:1133-1149)
-        torch.nan_to_num(out_view, nan=0.0, posinf=0.0, neginf=0.0, out=out_view)
+        with _timer("V2_02c_tpe_submit"):
+            handoff.submit(q_batch, topk_slots)
+        with _timer("V2_04_join"):
+            handoff.wait(o_new)
+    with _timer("V2_05_post_corr"):
+        if direct:
+            ops.blend_unnorm_into(o_hat, o_old, W, o_new, out_view)
+        else:
+            tmp = torch.empty(n_seqs, H_q, D, dtype=torch.bfloat16, device=query.device)
+            ops.blend_unnorm_into(o_hat, o_old, W, o_new, tmp)
+            out_view.copy_(tmp.to(out_view.dtype))
+        if graph_mode and _sanitize_output_enabled():   # (decode_path.py:1133-1149)
+            torch.nan_to_num(out_view, nan=0.0, posinf=0.0, neginf=0.0, out=out_view)
     pool.record_decode_hit()
     return output

@@ -848,3 +848,39 @@ def test_backend_shim_defers_a_prefill_append_until_its_attention_is_enqueued(ad
     small = torch.randn(4, Hkv, D).to(torch.bfloat16).cuda()
     impl.do_kv_cache_update(layer, small, small, None, torch.arange(96, 100).cuda())
     assert not hasattr(layer, "_jetfire_deferred_kv_mirror")
+
+
+@pytest.mark.gpu
+def test_decode_entry_reports_its_stages_under_profile_decode(adapter, monkeypatch):
+    """JETFIRE_PROFILE_DECODE=1 (`decode_path.py:60-85`): every stage of the decode entry is a named profiler range
+    and its wall time is accumulated under the reference's stage names; without the switch nothing is accumulated."""
+    B, Hq, Hkv, D, bs, K, max_S = 1, 8, 2, 128, 16, 32, 128
+    adapter.set_jetfire_config(scheme="SymInt3K_SymInt2V", group_size=64, topk=K, layer_stride=1, cpu_attn_threads=2)
+    adapter.reset_global_kv_pool_manager()
+    pool = adapter.get_global_kv_pool_manager()
+    name = "model.layers.0.self_attn.attn"
+    layer = types.SimpleNamespace(layer_name=name, num_heads=Hq, num_kv_heads=Hkv, head_size=D)
+    impl = types.SimpleNamespace(attn_type=types.SimpleNamespace(name="DECODER"), scale=D ** -0.5)
+    pool.ensure_layer_config_from_layer(name, layer)
+    pool.register_layer_layout(name, num_blocks=max_S // bs, block_size=bs)
+    g = torch.Generator().manual_seed(5)
+    n = 100
+    pool.mirror_kv(name, torch.randn(n, Hkv, D, generator=g).to(torch.bfloat16).cuda(),
+                   torch.randn(n, Hkv, D, generator=g).to(torch.bfloat16).cuda(), torch.arange(n).cuda())
+    pool.flush_pending_writes()
+    meta = _meta(torch.tensor([n], dtype=torch.int32, device="cuda"), torch.arange(max_S // bs).view(1, -1).cuda(),
+                 max_seq_len=n)
+    q = torch.randn(B, Hq, D, generator=g).to(torch.bfloat16).cuda()
+    out = torch.zeros(B, Hq * D, dtype=torch.bfloat16, device="cuda")
+    adapter.jetfire_get_profile()
+    assert adapter.try_jetfire_decode(impl=impl, layer=layer, query=q, attn_metadata=meta, output=out) is out
+    assert adapter.jetfire_get_profile() == {}
+    plain = out.clone()
+    monkeypatch.setenv("JETFIRE_PROFILE_DECODE", "1")
+    assert adapter.try_jetfire_decode(impl=impl, layer=layer, query=q, attn_metadata=meta, output=out) is out
+    prof = adapter.jetfire_get_profile()
+    assert {"D_total", "V2_00_prep", "V2_01_attn", "V2_02c_tpe_submit", "V2_04_join", "V2_05_post_corr"} <= set(prof)
+    assert all(len(v) == 1 and v[0] > 0.0 for v in prof.values())
+    assert prof["D_total"][0] >= prof["V2_01_attn"][0]
+    assert adapter.jetfire_get_profile() == {}          # reading clears
+    assert torch.equal(out, plain)                      # the ranges change nothing
