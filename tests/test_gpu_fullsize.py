@@ -169,17 +169,19 @@ def test_two_call_form_equals_the_one_pass_form_at_full_size(name):
     assert torch.equal(o_hat2, o_hat) and torch.equal(o_old2, o_old) and torch.equal(W2, W)
 
 
-def test_c4_end_to_end_with_handoff_matches_the_oracle_on_sampled_units():
-    """Configuration C4 at its full shape (B4, 32 query / 4 kv heads, 32768 positions, K3V2, top-k 256, paged), one
-    layer, the whole step: fused scan + merge, pinned hand-off, CPU correction from the bf16 host shadow, device-side
-    wait and blend.  The oracle's `decode_reference` (numpy) is run on two sampled (sequence, kv-head) units - all
-    eight query heads of each over the full context - and the blended output must match it within the acceptance
-    bounds (2e-2 max-abs, 1e-3 mean-abs in bf16) and the reference's own blend tolerance."""
+@pytest.mark.parametrize("name,units", [("c4", ((0, 1), (3, 2))), ("c5", ((0, 1), (1, 2)))])
+def test_end_to_end_with_handoff_matches_the_oracle_on_sampled_units(name, units):
+    """Configurations C4 (B4, 32 query / 4 kv heads, 32768 positions, top-k 256) and C5 (B2, 65536 positions, top-k
+    512) at their full shapes, K3V2, paged, one layer, the whole step: fused scan + merge, pinned hand-off, CPU
+    correction from the bf16 host shadow, device-side wait and blend.  The oracle's `decode_reference` (numpy) is run
+    on two sampled (sequence, kv-head) units - all eight query heads of each over the full context - and the blended
+    output must match it within the acceptance bounds (2e-2 max-abs, 1e-3 mean-abs in bf16) and the reference's own
+    blend tolerance."""
     import numpy as np
     from jetfire_amd import ops, workloads
     from oracle import jetfire_oracle as O
     from tests.helpers import bf16_to_bits, bf16_to_f32
-    w = workloads.build("c4", n_layers=1, paged=True, keep_shadow=1)
+    w = workloads.build(name, n_layers=1, paged=True, keep_shadow=1)
     lay = w.layers[0]
     ksh, vsh = w.shadows[0]
     B, Hq, Hkv, S, K = w.B, w.H_q, w.H_kv, w.S, w.top_k
@@ -198,7 +200,7 @@ def test_c4_end_to_end_with_handoff_matches_the_oracle_on_sampled_units():
         h.close()
     res = bf16_to_f32(out)
     bt = w.block_table.cpu().numpy()
-    for b, kvh in ((0, 1), (3, 2)):
+    for b, kvh in units:
         hs = slice(kvh * G, (kvh + 1) * G)
         r = O.decode_reference(
             bf16_to_f32(w.q[b:b + 1, hs]), lay.k_data[kvh:kvh + 1].cpu().numpy(), bf16_to_bits(lay.k_scales[kvh:kvh + 1]),
