@@ -17,7 +17,7 @@
 //                       reference's fp32 rescale order (bit-equal to the split-form kernel).
 //            scores[G][L] -> LDS (fp32), running max / min per head.
 //   phase B  P.V on the same MFMA.  p = exp(s - m_split) is known exactly because phase A is complete, so
-//            w = p * v_scale is converted to 22-bit fixed point once (fma with 2^23), the four bytes of the
+//            w = p * v_scale is converted to 23-bit fixed point once (fma with 2^23), the four bytes of the
 //            converted word are the A-operand rows (head, limb 0..2 and the constant exponent byte), and the
 //            int32 accumulators live for the whole split: every product is exact.  V codes are transposed by
 //            ds_read_b64_tr_b4, weight rows by ds_read_b64_tr_b8.
@@ -1271,14 +1271,15 @@ __global__ __launch_bounds__((ScanLds<SCHEME, G, NG>::NT)) void fused_scan_kerne
     const float v = bf16_to_f32((uint16_t)vb);
     int e = 0;
     if (v > 0.f && isfinite(v)) (void)frexpf(v, &e);  // v = f * 2^e, f in [0.5, 1)
-    e_sh[g] = 22 - e;                                 // v * 2^E in [2^21, 2^22)
+    e_sh[g] = 23 - e;                                 // v * 2^E in [2^22, 2^23): the weights use all 23 mantissa bits
   }
   lds_barrier();
   if (clk && tid == 0) clk[1] = JF_CLK();
 
   // ------------------------------------------------------------------ phase B: P.V on v_mfma_i32_16x16x64_i8
   // p = exp(s - m_split) is known exactly because phase A is complete, so w = p * v_scale is converted to
-  // 22-bit fixed point once (fma with 2^23); its three bytes, balanced around zero, are rows (limb, head) of
+  // 23-bit fixed point once (fma with 2^23: p <= 1 and the largest V scale below 2^e keep the sum below 2^24, where
+  // floats are integers); its three bytes, the lower two balanced around zero, are rows (limb, head) of
   // the A operand.  Lane = token stores the four heads' converted words as one 16-byte row per scale group (head-major;
   // the word's top byte is the constant 75 and becomes a constant row), and ds_read_b64_tr_b8 turns 8 token rows into the per-row byte runs the MFMA
   // wants.  V codes are staged packed in wavefront-private LDS and transposed by ds_read_b64_tr_b4 (16

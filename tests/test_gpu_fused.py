@@ -23,7 +23,7 @@ def run_fused(scheme, c, d, S, K):
                              c["Hq"], c["Hkv"], 16, K, SCALE, return_scores=True, return_stats=True, k_zp=d.get("kz"))
 
 
-def check_against_oracle(scheme, c, S, K, out):
+def check_against_oracle(scheme, c, S, K, out, atol_out=3e-6):
     o_hat, slots, o_old, W, idx, m, iz, scores = [t.cpu().numpy() for t in out]
     kb, vb, gs = c["kbits"], c["vbits"], c["gs"]
     Hq, Hkv = c["Hq"], c["Hkv"]
@@ -54,9 +54,9 @@ def check_against_oracle(scheme, c, S, K, out):
     np.testing.assert_allclose(m, rm, atol=1e-7)
     np.testing.assert_allclose(iz, riz, rtol=2e-5)
     r_hat, r_old, r_W = O.softmax_v(scores, c["vd"], c["vs"], c["bt"], c["lens"], idx, S, Hq, Hkv, 16, vb, gs)
-    np.testing.assert_allclose(o_hat, r_hat, atol=3e-6, rtol=2e-5)
-    np.testing.assert_allclose(o_old, r_old, atol=3e-6, rtol=2e-5)
-    np.testing.assert_allclose(W, r_W, atol=3e-6, rtol=2e-5)
+    np.testing.assert_allclose(o_hat, r_hat, atol=atol_out, rtol=2e-5)
+    np.testing.assert_allclose(o_old, r_old, atol=atol_out, rtol=2e-5)
+    np.testing.assert_allclose(W, r_W, atol=atol_out, rtol=2e-5)
     return ref_sc
 
 
@@ -169,6 +169,39 @@ def test_fused_scan_with_forced_split_length(scheme, S, lens, K, split_len):
     # the planner's own split length selects the same positions
     again = run_fused(scheme, c, d, S, K)
     assert torch.equal(forced[4], again[4]) and torch.equal(forced[1], again[1])
+
+
+@pytest.mark.parametrize("mode", ("zero_query", "few_values", "one_huge_many_tiny"))
+@pytest.mark.parametrize("scheme,G,Hkv,S,K,split_len", [
+    ("k3v2", 4, 2, 3000, 256, 0), ("k3v2", 8, 1, 2100, 2048, 512), ("k3v2", 16, 1, 2100, 2048, 512),
+    ("k4v4", 4, 2, 5000, 64, 1024), ("k2v2", 8, 1, 9000, 512, 0), ("a2v2", 4, 2, 3000, 256, 0),
+])
+def test_fused_scan_on_degenerate_queries(scheme, G, Hkv, S, K, split_len, mode):
+    """Queries that stress the fixed-point arithmetic and the selection: all zero (every score equal: the exact
+    selection and its ties), a few distinct values (massive ties at the cut), and one huge element among many tiny ones
+    per 64-channel group (the tiny ones keep few bits of the group's shared exponent; the softmax is peaked, so the
+    23-bit weights are coarse against the sum of the weights).  Scores stay within 2e-5 and the top-k exact; o_hat,
+    o_old and W within 6e-6 (on random queries: 3e-6; the measured worst case here is 4.4e-6 on isolated elements)."""
+    from jetfire_amd import _lib
+    lib = _lib.load()
+    kb, vb, gs = {"k3v2": (3, 2, 64), "k4v4": (4, 4, 128), "k2v2": (2, 2, 64), "a2v2": (2, 2, 64)}[scheme]
+    c = make_case(4242, 2, G * Hkv, Hkv, S, kb, vb, gs, lens=[S, S - 37], extra_blocks=1, k_asym=scheme.startswith("a"))
+    q = c["q"]
+    if mode == "zero_query":
+        q[...] = 0
+    elif mode == "few_values":
+        q[...] = np.sign(q) * 0.5 * (np.abs(q) > 1.0)
+    else:
+        q[...] = torch.tensor(q * 0.01).to(torch.bfloat16).float().numpy()
+        q[:, :, 5] = 8.0
+        q[:, :, 70] = -8.0
+    d = to_device(c)
+    _lib.check(_lib.debug_hook("jf_debug_split_len")(split_len))
+    try:
+        out = [t.clone() for t in run_fused(scheme, c, d, S, K)]
+    finally:
+        _lib.check(_lib.debug_hook("jf_debug_split_len")(0))
+    check_against_oracle(scheme, c, S, K, out, atol_out=6e-6)
 
 
 @pytest.mark.parametrize("gs", (128, 64))
