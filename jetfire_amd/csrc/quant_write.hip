@@ -104,20 +104,25 @@ __global__ __launch_bounds__(256) void quant_write16_kernel(RowSrc s0, RowDst d0
   constexpr int QMAX = (1 << (NBITS - 1)) - 1;
   constexpr int OFF = 1 << (NBITS - 1);
   const int l16 = threadIdx.x & 15;
-  const int64_t tq = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+  const uint32_t r = threadIdx.x >> 4;
+  const int64_t t0 = (int64_t)blockIdx.x * 16;  // first token of the block (uniform: its products stay on the scalar unit)
   const int h = blockIdx.y;
   const int which = blockIdx.z;
-  // rows past the end still take part in the cross-lane steps (they re-read row 0); the row is requested
-  // without waiting for its slot, so the two loads are in flight together; masked rows (slot < 0) only skip
-  // the stores
-  const bool inside = tq < T;
-  const int64_t t = inside ? tq : 0;
-  const int64_t slot = slots[t];
+  // rows past the end still take part in the cross-lane steps (they re-read the block's first row); the row is
+  // requested without waiting for its slot, so the two loads are in flight together; masked rows (slot < 0) only
+  // skip the stores
+  const bool inside = t0 + r < T;
+  const uint32_t re = inside ? r : 0u;
+  const int64_t slot = slots[t0 + re];
   const RowSrc& s = which ? s1 : s0;
   const RowDst& d = which ? d1 : d0;
-  const uint16_t* xrow = s.x + t * s.stride_t + (int64_t)h * s.stride_h;
+  // (the launcher takes this kernel only when the strides fit 32 bits: per-thread products are one 32 x 32 -> 64
+  // multiply-add instead of a 64 x 64 multiplication)
+  const uint16_t* xrow = s.x + t0 * s.stride_t + (int64_t)h * s.stride_h + (uint64_t)re * (uint32_t)s.stride_t;
   const uint4 raw = reinterpret_cast<const uint4*>(xrow)[l16];
-  const bool live = inside && slot >= 0;
+  // (a slot index takes 32 bits: negative = masked row; anything beyond 2^32 cannot be a row of a cache and is
+  // skipped like a masked row)
+  const bool live = inside && (uint64_t)slot < ((uint64_t)1 << 32);
   float x[8];
   x[0] = bf16_to_f32((uint16_t)(raw.x & 0xffffu)); x[1] = bf16_to_f32((uint16_t)(raw.x >> 16));
   x[2] = bf16_to_f32((uint16_t)(raw.y & 0xffffu)); x[3] = bf16_to_f32((uint16_t)(raw.y >> 16));
@@ -131,7 +136,13 @@ __global__ __launch_bounds__(256) void quant_write16_kernel(RowSrc s0, RowDst d0
   amax = fmaxf(amax, dpp_f32<0x4E>(amax));   // quad_perm [2,3,0,1]
   if (group_size >= 64) amax = fmaxf(amax, dpp_f32<0x141>(amax));   // row_half_mirror: lane i <-> 7 - i
   if (group_size >= 128) amax = fmaxf(amax, dpp_f32<0x140>(amax));  // row_mirror: lane i <-> 15 - i
-  const float sraw = fmaxf(amax / (float)QMAX, 1e-8f);
+  // scale = bf16(max(amax / QMAX, 1e-8)).  amax is a bf16 value M * 2^e with an 8-bit M, so the exact quotient by 3
+  // or 7 is either an 8-bit value itself or has a binary tail of k/3 (k/7) of the unit it is cut at: at least 1/6
+  // (1/14) of a bf16 ulp away from every bf16 rounding boundary.  The product with the fp32 reciprocal is within one
+  // fp32 ulp of the quotient, i.e. rounds to the same bf16 value as the correctly rounded division (the floor 1e-8
+  // is not within an fp32 ulp of a boundary either); checked for every mantissa by the tests.
+  constexpr float RQ = 1.0f / (float)QMAX;
+  const float sraw = fmaxf(amax * RQ, 1e-8f);
   const uint16_t sb = f32_to_bf16(sraw);
   const float sf = bf16_to_f32(sb);
   // code = clamp(rint(x / sf)).  x and sf are bf16 values (8 significant bits each), so the exact quotient is
@@ -139,19 +150,24 @@ __global__ __launch_bounds__(256) void quant_write16_kernel(RowSrc s0, RowDst d0
   // quotient equals rint of ANY value within a few ulp of the exact quotient, provided exact half-integers come
   // out exact.  q0 = x * rcp(sf) is within 2 ulp; one correction with the exact residual r = x - sf * q0 (an
   // fma) gives the exact quotient up to ~2^-45 relative, which rounds to the half-integer itself in a tie.
-  // One reciprocal per lane replaces eight correctly rounded divisions.
+  // One reciprocal per lane replaces eight correctly rounded divisions.  The clamp comes before the rounding (the
+  // bounds are integers: same result), and the rounding is the addition of 1.5 * 2^23 + OFF, whose sum has a unit
+  // in the last place of one: round-to-nearest-even like rint, and the code sits in the sum's low bits.
   const float ry = __builtin_amdgcn_rcpf(sf);
   uint32_t c[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     const float q0 = x[i] * ry;
     const float q = __builtin_fmaf(__builtin_fmaf(-sf, q0, x[i]), ry, q0);
-    c[i] = (uint32_t)((int)fminf(fmaxf(rintf(q), (float)-QMAX), (float)QMAX) + OFF);
+    const float qc = fminf(fmaxf(q, (float)-QMAX), (float)QMAX);
+    c[i] = __builtin_bit_cast(uint32_t, qc + (12582912.0f + (float)OFF)) & (uint32_t)(2 * OFF - 1);
   }
-  uint8_t* drow = d.data + (int64_t)h * d.data_stride_h + slot * d.data_stride_slot;
-  uint16_t* srow = d.scale + (int64_t)h * d.scale_stride_h + slot * d.scale_stride_slot;
-  const int lpg = group_size >> 3;  // lanes per scale group
-  if (live && (l16 & (lpg - 1)) == 0) srow[l16 / lpg] = sb;
+  const uint64_t so = (uint64_t)(uint32_t)slot;
+  uint8_t* drow = d.data + (int64_t)h * d.data_stride_h + so * (uint32_t)d.data_stride_slot;
+  uint16_t* srow = d.scale + (int64_t)h * d.scale_stride_h + so * (uint32_t)d.scale_stride_slot;
+  const int lpg = group_size >> 3;  // lanes per scale group: 4, 8 or 16
+  const int lpg_shift = (group_size >= 128) ? 4 : ((group_size >= 64) ? 3 : 2);
+  if (live && (l16 & (lpg - 1)) == 0) srow[l16 >> lpg_shift] = sb;
   if (NBITS == 4) {
     // byte j of the lane's dword = (c[2j] << 4) | c[2j+1]
     const uint32_t v = ((c[0] << 4) | c[1]) | (((c[2] << 4) | c[3]) << 8) | (((c[4] << 4) | c[5]) << 16) | (((c[6] << 4) | c[7]) << 24);
@@ -250,6 +266,12 @@ __global__ __launch_bounds__(256) void quant_write_kernel(RowSrc s0, RowDst d0, 
 inline bool rows_16b_aligned(const void* x, int64_t stride_t, int64_t stride_h) {
   return ((uintptr_t)x & 15) == 0 && stride_t % 8 == 0 && stride_h % 8 == 0;
 }
+// what quant_write16_kernel multiplies per thread with 32-bit operands
+inline bool strides_fit_32(int64_t x_stride_t, int64_t data_stride_slot, int64_t scale_stride_slot) {
+  const int64_t lim = (int64_t)1 << 32;
+  return x_stride_t >= 0 && x_stride_t < lim && data_stride_slot >= 0 && data_stride_slot < lim &&
+         scale_stride_slot >= 0 && scale_stride_slot < lim;
+}
 
 int check_common(const void* x, const int64_t* slots, int64_t T, int H_kv, int group_size,
                  int64_t data_stride_slot, int nbits, const void* data, const void* scale) {
@@ -284,7 +306,7 @@ extern "C" int jf_quant_write_sym(const uint16_t* x, int64_t x_stride_t, int64_t
   RowDst d{out_data, data_stride_h, data_stride_slot, out_scale, scale_stride_h, scale_stride_slot};
   const int64_t units = T * H_kv;
   hipStream_t st = (hipStream_t)stream;
-  if (rows_16b_aligned(x, x_stride_t, x_stride_h)) {
+  if (rows_16b_aligned(x, x_stride_t, x_stride_h) && strides_fit_32(x_stride_t, data_stride_slot, scale_stride_slot)) {
     dim3 grid16((unsigned)((T + 15) / 16), (unsigned)H_kv, 1), block16(256);
     if (nbits == 2) hipLaunchKernelGGL(quant_write16_kernel<2>, grid16, block16, 0, st, s, d, s, d, slots, T, H_kv, 1, group_size);
     else if (nbits == 3) hipLaunchKernelGGL(quant_write16_kernel<3>, grid16, block16, 0, st, s, d, s, d, slots, T, H_kv, 1, group_size);
@@ -318,7 +340,9 @@ extern "C" int jf_quant_write_int4_sym_kv(const uint16_t* key, int64_t k_stride_
   RowDst d0{k_data, k_data_stride_h, k_data_stride_slot, k_scale, k_scale_stride_h, k_scale_stride_slot};
   RowDst d1{v_data, v_data_stride_h, v_data_stride_slot, v_scale, v_scale_stride_h, v_scale_stride_slot};
   const int64_t units = T * H_kv * 2;
-  if (rows_16b_aligned(key, k_stride_t, k_stride_h) && rows_16b_aligned(value, v_stride_t, v_stride_h)) {
+  if (rows_16b_aligned(key, k_stride_t, k_stride_h) && rows_16b_aligned(value, v_stride_t, v_stride_h) &&
+      strides_fit_32(k_stride_t, k_data_stride_slot, k_scale_stride_slot) &&
+      strides_fit_32(v_stride_t, v_data_stride_slot, v_scale_stride_slot)) {
     dim3 grid16((unsigned)((T + 15) / 16), (unsigned)H_kv, 2), block16(256);
     hipLaunchKernelGGL(quant_write16_kernel<4>, grid16, block16, 0, (hipStream_t)stream, s0, d0, s1, d1, slots, T, H_kv, 2, group_size);
     JF_CHECK_LAUNCH();
