@@ -151,8 +151,11 @@ __global__ __launch_bounds__(256) void quant_write16_kernel(RowSrc s0, RowDst d0
   // out exact.  q0 = x * rcp(sf) is within 2 ulp; one correction with the exact residual r = x - sf * q0 (an
   // fma) gives the exact quotient up to ~2^-45 relative, which rounds to the half-integer itself in a tie.
   // One reciprocal per lane replaces eight correctly rounded divisions.  The clamp comes before the rounding (the
-  // bounds are integers: same result), and the rounding is the addition of 1.5 * 2^23 + OFF, whose sum has a unit
-  // in the last place of one: round-to-nearest-even like rint, and the code sits in the sum's low bits.
+  // bounds are integers: same result), and the rounding is the addition of 2^23 + OFF: the sum lies in
+  // [2^23 + 1, 2^23 + 2 OFF - 1], where floats are the integers, so the addition rounds to nearest-even like rint
+  // and leaves code = rint(q) + OFF in the low bits of the sum's pattern 0x4B000000 | code.  The pattern's own bits
+  // start at bit 24: the packing below shifts and merges the patterns as they are and only ever keeps bits that
+  // the codes alone reach.
   const float ry = __builtin_amdgcn_rcpf(sf);
   uint32_t c[8];
 #pragma unroll
@@ -160,7 +163,7 @@ __global__ __launch_bounds__(256) void quant_write16_kernel(RowSrc s0, RowDst d0
     const float q0 = x[i] * ry;
     const float q = __builtin_fmaf(__builtin_fmaf(-sf, q0, x[i]), ry, q0);
     const float qc = fminf(fmaxf(q, (float)-QMAX), (float)QMAX);
-    c[i] = __builtin_bit_cast(uint32_t, qc + (12582912.0f + (float)OFF)) & (uint32_t)(2 * OFF - 1);
+    c[i] = __builtin_bit_cast(uint32_t, qc + (8388608.0f + (float)OFF));
   }
   const uint64_t so = (uint64_t)(uint32_t)slot;
   uint8_t* drow = d.data + (int64_t)h * d.data_stride_h + so * (uint32_t)d.data_stride_slot;
@@ -169,16 +172,20 @@ __global__ __launch_bounds__(256) void quant_write16_kernel(RowSrc s0, RowDst d0
   const int lpg_shift = (group_size >= 128) ? 4 : ((group_size >= 64) ? 3 : 2);
   if (live && (l16 & (lpg - 1)) == 0) srow[l16 >> lpg_shift] = sb;
   if (NBITS == 4) {
-    // byte j of the lane's dword = (c[2j] << 4) | c[2j+1]
-    const uint32_t v = ((c[0] << 4) | c[1]) | (((c[2] << 4) | c[3]) << 8) | (((c[4] << 4) | c[5]) << 16) | (((c[6] << 4) | c[7]) << 24);
+    // byte j of the lane's dword = (c[2j] << 4) | c[2j+1]: the low byte of each merged pair (v_perm_b32 gathers them)
+    const uint32_t p0 = (c[0] << 4) | c[1], p1 = (c[2] << 4) | c[3], p2 = (c[4] << 4) | c[5], p3 = (c[6] << 4) | c[7];
+    const uint32_t v = __builtin_amdgcn_perm(p1, p0, 0x0c0c0400u) | __builtin_amdgcn_perm(p3, p2, 0x04000c0cu);
     if (live) reinterpret_cast<uint32_t*>(drow)[l16] = v;
   } else if (NBITS == 2) {
-    // the lane's 8 codes are two bytes, four codes each MSB first; lane pairs share a dword
-    const uint32_t hw = ((c[0] << 6) | (c[1] << 4) | (c[2] << 2) | c[3]) | (((c[4] << 6) | (c[5] << 4) | (c[6] << 2) | c[7]) << 8);
+    // the lane's 8 codes are two bytes, four codes each MSB first (the low bytes of the two merged quadruples);
+    // lane pairs share a dword
+    const uint32_t pa = (c[0] << 6) | (c[1] << 4) | (c[2] << 2) | c[3], pb = (c[4] << 6) | (c[5] << 4) | (c[6] << 2) | c[7];
+    const uint32_t hw = __builtin_amdgcn_perm(pb, pa, 0x0c0c0400u);
     const uint32_t nb = dpp_u32<0xB1>(hw);  // neighbour inside the lane pair
     if (live && (l16 & 1) == 0) reinterpret_cast<uint32_t*>(drow)[l16 >> 1] = hw | (nb << 16);
   } else {
-    // INT3 planar: the lane's 8 codes are the 24-bit word l16, MSB first; plane p holds byte p of every word.
+    // INT3 planar: the lane's 8 codes are the 24-bit word l16, MSB first (bits 0..23 of w; what lies above is the
+    // patterns' own bits and is never extracted); plane p holds byte p of every word.
     // Lane (4j + p), p < 3, assembles dword j of plane p from the four words of its quad.
     const uint32_t w = (c[0] << 21) | (c[1] << 18) | (c[2] << 15) | (c[3] << 12) | (c[4] << 9) | (c[5] << 6) | (c[6] << 3) | c[7];
     const uint32_t w0 = dpp_u32<0x00>(w), w1 = dpp_u32<0x55>(w), w2 = dpp_u32<0xAA>(w), w3 = dpp_u32<0xFF>(w);  // quad broadcasts
